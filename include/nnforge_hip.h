@@ -1,0 +1,179 @@
+/*
+ * nnforge_hip.h - C ABI of the gfx950 (MI355X) inference kernels behind nnForge's layer_tester surface.
+ *
+ * Every entry point is extern "C", takes plain pointers and sizes, never throws and never
+ * synchronises unless its name says so. Return value: 0 = success, > 0 = a hipError_t reported by
+ * the HIP runtime, < 0 = one of the NNF_HIP_E* codes below. nnf_hip_error_string() explains both.
+ *
+ * Tensor layout is nnForge's: fp32, [entry][feature_map][y][x] with x fastest
+ * (nnforge/layer_configuration_specific.cpp:62-73); a "plane" is one feature map of one entry,
+ * neuron_count_per_feature_map floats long. Device pointers handed to the kernels must be
+ * 16-byte aligned at their base (any hipMalloc / nnf_hip_malloc result is). The output may alias
+ * inputs[0] exactly (in-place), as every one of the reference testers on this path allows
+ * (e.g. nnforge/plain/batch_norm_layer_tester_plain.cpp:77-84); partial overlap is not supported.
+ *
+ * Arithmetic contract: every layer is evaluated in fp32 with the reference's own operation order
+ * and one rounding per operation (no contraction, no reassociation, no cross-layer algebra), so a
+ * fused chain produces the same bits as the same layers run one after another.
+ */
+#ifndef NNFORGE_HIP_H
+#define NNFORGE_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define NNF_HIP_API __attribute__((visibility("default")))
+
+/* ---- error codes (negative; positive values are hipError_t) -------------------------------- */
+#define NNF_HIP_OK 0
+#define NNF_HIP_EINVAL (-1)      /* null pointer, zero feature maps, malformed descriptor       */
+#define NNF_HIP_EUNSUPPORTED (-2) /* shape or option outside what the kernels implement          */
+#define NNF_HIP_EALIGN (-3)      /* a tensor base pointer is not 16-byte aligned                 */
+#define NNF_HIP_EOVERLAP (-4)    /* output overlaps an input other than "out == inputs[0]"      */
+#define NNF_HIP_ETOOBIG (-5)     /* element count does not fit the kernels' index range          */
+
+#define NNF_HIP_MAX_OPS 8
+#define NNF_HIP_MAX_INPUTS 4
+
+/* Layer kinds of the element-wise chain kernel. The names in comments are nnForge's layer type
+ * names (the keys of layer_tester_plain_factory, nnforge/plain/layer_tester_plain_factory.cpp:27-51). */
+typedef enum nnf_hip_op_kind
+{
+	NNF_HIP_OP_BATCH_NORM = 1, /* "BatchNorm": mult = gamma*inv_sigma; add = beta - mult*mean; y = x*mult + add
+	                              (nnforge/plain/batch_norm_layer_tester_plain.cpp:54-74)                       */
+	NNF_HIP_OP_RELU = 2,       /* "ReLU": y = x >= 0 ? x : x*negative_slope
+	                              (nnforge/plain/rectified_linear_layer_tester_plain.cpp:50-55)                 */
+	NNF_HIP_OP_PRELU = 3,      /* "PReLU": y = x * (x >= 0 ? 1 : a[feature_map])
+	                              (nnforge/plain/parametric_rectified_linear_layer_tester_plain.cpp:51-70)      */
+	NNF_HIP_OP_ELU = 4,        /* "ELU": y = x >= 0 ? x : expf(x) - 1
+	                              (nnforge/plain/exponential_linear_layer_tester_plain.cpp:47-52)               */
+	NNF_HIP_OP_SIGMOID = 5,    /* "Sigmoid": y = 1 / (expf(-x) + 1)
+	                              (nnforge/plain/sigmoid_layer_tester_plain.cpp:47-53)                          */
+	NNF_HIP_OP_TANH = 6        /* "TanH": e = expf(x * (steepness*2)); y = (e - 1)/(e + 1) * scale
+	                              (nnforge/plain/hyperbolic_tangent_layer_tester_plain.cpp:48-58)               */
+} nnf_hip_op_kind;
+
+/* One element-wise layer of a chain. */
+typedef struct nnf_hip_op
+{
+	int32_t kind;   /* nnf_hip_op_kind */
+	int32_t chunk;  /* BATCH_NORM: index into chunk_ptrs of gamma; beta, mean, inverse sigma follow at
+	                   chunk+1..chunk+3 (chunk order of nnforge/batch_norm_layer.cpp:96-106).
+	                   PRELU: index into chunk_ptrs of the per-feature-map slopes
+	                   (nnforge/parametric_rectified_linear_layer.cpp:87-94). Others: ignored.        */
+	float f0;       /* RELU: negative_slope. TANH: scale. Others: ignored.                           */
+	float f1;       /* TANH: steepness. Others: ignored.                                             */
+} nnf_hip_op;
+
+/*
+ * A fused group of layers evaluated in one pass over the tensor: up to NNF_HIP_MAX_INPUTS input
+ * tensors ("arms"), each optionally run through its own element-wise layers, joined by at most one
+ * "Add" layer (sum = 0; sum += arm_j in input order; v = sum*alpha -
+ * nnforge/plain/add_layer_tester_plain.cpp:54-61), followed by the layers after the join.
+ * Without an Add there is exactly one input and arm_op_count[0] + tail_op_count layers applied in order.
+ * All tensors share one shape: entry_count x feature_map_count x neuron_count_per_feature_map.
+ */
+typedef struct nnf_hip_chain_desc
+{
+	uint32_t entry_count;
+	uint32_t feature_map_count;
+	uint32_t neuron_count_per_feature_map;
+	uint32_t input_count;                       /* 1..NNF_HIP_MAX_INPUTS; > 1 requires has_add      */
+	uint32_t has_add;                           /* 0 or 1                                           */
+	float add_alpha;                            /* add_layer::alpha (nnforge/add_layer.h:27)        */
+	uint32_t arm_op_count[NNF_HIP_MAX_INPUTS];  /* layers applied to input j before the join        */
+	uint32_t tail_op_count;                     /* layers applied after the join                    */
+	nnf_hip_op ops[NNF_HIP_MAX_OPS];            /* arm 0's layers, arm 1's, ..., then the tail's    */
+} nnf_hip_chain_desc;
+
+/* ---- the hot path -------------------------------------------------------------------------- */
+
+/* Fused element-wise group. Replaces one run_forward_propagation call per layer of the group
+ * (nnforge/plain/forward_propagation_plain.cpp:137-186 calls them one by one). inputs[] holds
+ * input_count device pointers in the Add layer's input order; chunk_ptrs[] holds device pointers
+ * to the weight chunks the ops refer to (may be null when no op uses a chunk). */
+NNF_HIP_API int nnf_hip_chain_forward(void* stream, const nnf_hip_chain_desc* desc, float* output,
+	const float* const* inputs, const float* const* chunk_ptrs);
+
+/* Single-layer entry points, one per reference tester (same arithmetic as the chain kernel). */
+NNF_HIP_API int nnf_hip_batch_norm_forward(void* stream, float* output, const float* input,
+	const float* gamma, const float* beta, const float* mean, const float* inverse_sigma,
+	uint32_t entry_count, uint32_t feature_map_count, uint32_t neuron_count_per_feature_map);
+	/* nnforge/plain/batch_norm_layer_tester_plain.cpp:30-75 */
+NNF_HIP_API int nnf_hip_rectified_linear_forward(void* stream, float* output, const float* input,
+	float negative_slope, uint64_t elem_count);
+	/* nnforge/plain/rectified_linear_layer_tester_plain.cpp:30-56 */
+NNF_HIP_API int nnf_hip_parametric_rectified_linear_forward(void* stream, float* output, const float* input,
+	const float* slopes, uint32_t entry_count, uint32_t feature_map_count, uint32_t neuron_count_per_feature_map);
+	/* nnforge/plain/parametric_rectified_linear_layer_tester_plain.cpp:30-71 */
+NNF_HIP_API int nnf_hip_exponential_linear_forward(void* stream, float* output, const float* input, uint64_t elem_count);
+	/* nnforge/plain/exponential_linear_layer_tester_plain.cpp:30-53 */
+NNF_HIP_API int nnf_hip_sigmoid_forward(void* stream, float* output, const float* input, uint64_t elem_count);
+	/* nnforge/plain/sigmoid_layer_tester_plain.cpp:30-54 */
+NNF_HIP_API int nnf_hip_hyperbolic_tangent_forward(void* stream, float* output, const float* input,
+	float scale, float steepness, uint64_t elem_count);
+	/* nnforge/plain/hyperbolic_tangent_layer_tester_plain.cpp:30-59 */
+NNF_HIP_API int nnf_hip_add_forward(void* stream, float* output, const float* const* inputs, uint32_t input_count,
+	float alpha, uint64_t elem_count);
+	/* nnforge/plain/add_layer_tester_plain.cpp:32-62; any input_count >= 1 (launched in groups of
+	   NNF_HIP_MAX_INPUTS, which keeps the reference's left-to-right summation order) */
+
+/* Softmax across feature maps at every (entry, spatial position):
+ * nnforge/plain/softmax_layer_tester_plain.cpp:34-91 (max, expf(x - max), sum, multiply by 1/sum). */
+NNF_HIP_API int nnf_hip_softmax_forward(void* stream, float* output, const float* input,
+	uint32_t entry_count, uint32_t feature_map_count, uint32_t neuron_count_per_feature_map);
+
+/* 2-D average subsampling with non-overlapping window_width x window_height windows (output size =
+ * input size / window size rounded down; a leftover right/bottom margin is not read,
+ * nnforge/average_subsampling_layer.cpp:80-87), window values summed x-fastest then multiplied by mult:
+ * nnforge/plain/average_subsampling_layer_tester_plain.cpp:34-148 restricted to two spatial
+ * dimensions, no feature-map/entry subsampling. The caller passes the multiplier the tester would
+ * use (average_subsampling_layer::get_effective_alpha, nnforge/average_subsampling_layer.cpp:287-303). */
+NNF_HIP_API int nnf_hip_average_subsampling_forward(void* stream, float* output, const float* input,
+	uint32_t entry_count, uint32_t feature_map_count, uint32_t input_width, uint32_t input_height,
+	uint32_t window_width, uint32_t window_height, float mult);
+
+/* ---- runtime plumbing, so that host C++ above this ABI needs no HIP headers --------------------
+ * Counterparts in the reference: cuda_linear_buffer_device (nnforge/cuda/cuda_linear_buffer_device.cpp:28-45),
+ * cuda_stream / cuda_event (nnforge/cuda/cuda_stream.cpp, cuda_event.cpp), cuda_safe_call
+ * (nnforge/cuda/neural_network_cuda_exception.h:27-39). */
+NNF_HIP_API int nnf_hip_device_count(int* count);
+NNF_HIP_API int nnf_hip_set_device(int device_id);
+NNF_HIP_API int nnf_hip_device_info(int device_id, char* name, size_t name_capacity, uint64_t* global_memory_bytes,
+	uint32_t* compute_unit_count, uint32_t* wavefront_size, uint32_t* clock_khz);
+NNF_HIP_API int nnf_hip_malloc(void** device_ptr, size_t bytes); /* size rounded up to 16 bytes, like
+	the reference's device buffers (nnforge/cuda/util_cuda.cu:731-735) */
+NNF_HIP_API int nnf_hip_free(void* device_ptr);
+NNF_HIP_API int nnf_hip_memcpy_h2d(void* device_dst, const void* host_src, size_t bytes, void* stream); /* stream null: synchronous */
+NNF_HIP_API int nnf_hip_memcpy_d2h(void* host_dst, const void* device_src, size_t bytes, void* stream);
+NNF_HIP_API int nnf_hip_memcpy_d2d(void* device_dst, const void* device_src, size_t bytes, void* stream);
+NNF_HIP_API int nnf_hip_host_malloc(void** host_ptr, size_t bytes); /* pinned */
+NNF_HIP_API int nnf_hip_host_free(void* host_ptr);
+NNF_HIP_API int nnf_hip_stream_create(void** stream);
+NNF_HIP_API int nnf_hip_stream_destroy(void* stream);
+NNF_HIP_API int nnf_hip_stream_synchronize(void* stream);
+NNF_HIP_API int nnf_hip_device_synchronize(void);
+NNF_HIP_API int nnf_hip_event_create(void** event);
+NNF_HIP_API int nnf_hip_event_destroy(void* event);
+NNF_HIP_API int nnf_hip_event_record(void* event, void* stream);
+NNF_HIP_API int nnf_hip_event_synchronize(void* event);
+NNF_HIP_API int nnf_hip_event_elapsed_ms(float* milliseconds, void* start_event, void* stop_event);
+NNF_HIP_API int nnf_hip_stream_wait_event(void* stream, void* event);
+
+/* Plain device-to-device streaming copy kernel (float4 loads and stores, same launch shape as the
+ * chain kernel). Used as the yardstick for achievable HBM bandwidth and for scaling profiler
+ * counters; no counterpart in the reference. bytes must be a multiple of 16. */
+NNF_HIP_API int nnf_hip_copy_kernel(void* stream, void* device_dst, const void* device_src, size_t bytes);
+
+NNF_HIP_API const char* nnf_hip_error_string(int code);
+NNF_HIP_API const char* nnf_hip_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* NNFORGE_HIP_H */

@@ -1,0 +1,55 @@
+"""Build recipe: compiles the gfx950 library (hipcc) and the host-side C++ backend (g++) in-tree."""
+
+import os
+import shutil
+import subprocess
+
+PACKAGE_DIR = os.path.dirname(os.path.abspath(__file__))
+REPO_ROOT = os.path.dirname(PACKAGE_DIR)
+CSRC_DIR = os.path.join(PACKAGE_DIR, "csrc")
+
+HIP_LIBRARY = os.path.join(PACKAGE_DIR, "libnnforge_hip.so")
+HIP_SOURCES = ["nnf_chain.hip", "nnf_softmax.hip", "nnf_pool.hip", "nnf_capi.hip"]
+
+# -ffp-contract=off: every fp32 operation of the layer formulas rounds once, as the reference's
+#   source states them. -packed-fp32-ops is switched off as a target feature (hipcc only).
+HIP_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden",
+    "-ffp-contract=off", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall", "-Wno-unused-command-line-argument",
+]
+
+
+def _run(cmd, cwd=None):
+    proc = subprocess.run(cmd, cwd=cwd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("build step failed: %s\n%s" % (" ".join(cmd), proc.stdout))
+    return proc.stdout
+
+
+def hipcc_path():
+    for candidate in (shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if candidate and os.path.exists(candidate):
+            return candidate
+    raise RuntimeError("hipcc not found: the gfx950 library cannot be built")
+
+
+def build_hip_library(verbose=False):
+    """Compiles nnforge_amd/csrc/*.hip into nnforge_amd/libnnforge_hip.so (cross-compiles without a GPU)."""
+    tmp = HIP_LIBRARY + ".tmp"
+    cmd = [hipcc_path()] + HIP_FLAGS + ["-o", tmp] + [os.path.join(CSRC_DIR, s) for s in HIP_SOURCES]
+    out = _run(cmd)
+    os.replace(tmp, HIP_LIBRARY)
+    if verbose and out.strip():
+        print(out)
+    return HIP_LIBRARY
+
+
+def build_all(verbose=False):
+    built = [build_hip_library(verbose)]
+    return built
+
+
+if __name__ == "__main__":
+    for path in build_all(verbose=True):
+        print("built", path)

@@ -1,0 +1,378 @@
+// extern "C" surface of the library (declared in include/nnforge_hip.h): argument checks,
+// single-layer wrappers around the fused-group kernel, and the runtime plumbing (memory, streams,
+// events) that lets host C++ above this ABI stay free of HIP headers.
+#include "nnf_common.h"
+
+#include <cstring>
+
+namespace nnf
+{
+	namespace
+	{
+		constexpr int copy_block_size = 256;
+		constexpr int copy_unroll = 4;
+
+		// same tiling as the chain kernel: lane t moves float4s t, t + 256, ... of a 16 KiB tile
+		__global__ void __launch_bounds__(copy_block_size) copy_kernel_impl(floatx4* dst, const floatx4* src, uint32_t vectors)
+		{
+			const uint32_t tile_start = blockIdx.x * (copy_block_size * copy_unroll);
+			floatx4 v[copy_unroll];
+			#pragma unroll
+			for(int k = 0; k < copy_unroll; ++k)
+			{
+				const uint32_t i = tile_start + threadIdx.x + k * copy_block_size;
+				if (i < vectors)
+					v[k] = load_stream(src + i);
+			}
+			#pragma unroll
+			for(int k = 0; k < copy_unroll; ++k)
+			{
+				const uint32_t i = tile_start + threadIdx.x + k * copy_block_size;
+				if (i < vectors)
+					store_stream(dst + i, v[k]);
+			}
+		}
+
+		nnf_hip_chain_desc single_op_desc(uint32_t entry_count, uint32_t fm_count, uint32_t plane, int32_t kind, int32_t chunk, float f0, float f1)
+		{
+			nnf_hip_chain_desc d;
+			std::memset(&d, 0, sizeof(d));
+			d.entry_count = entry_count;
+			d.feature_map_count = fm_count;
+			d.neuron_count_per_feature_map = plane;
+			d.input_count = 1;
+			d.add_alpha = 1.0f;
+			d.arm_op_count[0] = 1;
+			d.ops[0].kind = kind;
+			d.ops[0].chunk = chunk;
+			d.ops[0].f0 = f0;
+			d.ops[0].f1 = f1;
+			return d;
+		}
+
+		// Layers without per-feature-map weights see the tensor as a flat array
+		// (e.g. nnforge/plain/rectified_linear_layer_tester_plain.cpp:47): split elem_count into a shape
+		// the fused-group kernel accepts.
+		bool flat_shape(uint64_t elem_count, uint32_t& entry_count, uint32_t& plane)
+		{
+			if (elem_count > 0xFFFF0000ull)
+				return false;
+			entry_count = 1;
+			plane = static_cast<uint32_t>(elem_count);
+			return true;
+		}
+
+		int flat_op(hipStream_t stream, float* output, const float* input, uint64_t elem_count, int32_t kind, float f0, float f1)
+		{
+			if (elem_count == 0)
+				return ((output == nullptr) || (input == nullptr)) ? NNF_HIP_EINVAL : NNF_HIP_OK;
+			uint32_t entry_count, plane;
+			if (!flat_shape(elem_count, entry_count, plane))
+				return NNF_HIP_ETOOBIG;
+			const nnf_hip_chain_desc d = single_op_desc(entry_count, 1, plane, kind, 0, f0, f1);
+			const float* inputs[1] = { input };
+			return chain_forward(stream, &d, output, inputs, nullptr);
+		}
+	}
+
+	int copy_kernel(hipStream_t stream, void* dst, const void* src, size_t bytes)
+	{
+		if ((dst == nullptr) || (src == nullptr) || ((bytes % 16) != 0))
+			return NNF_HIP_EINVAL;
+		if (!is_aligned16(dst) || !is_aligned16(src))
+			return NNF_HIP_EALIGN;
+		if (bytes == 0)
+			return NNF_HIP_OK;
+		if (bytes / 16 > 0xFFFF0000ull)
+			return NNF_HIP_ETOOBIG;
+		const uint32_t vectors = static_cast<uint32_t>(bytes / 16);
+		const uint32_t per_block = copy_block_size * copy_unroll;
+		hipLaunchKernelGGL(copy_kernel_impl, dim3((vectors + per_block - 1) / per_block), dim3(copy_block_size), 0, stream,
+			static_cast<floatx4*>(dst), static_cast<const floatx4*>(src), vectors);
+		return launch_status();
+	}
+}
+
+using namespace nnf;
+
+extern "C"
+{
+	int nnf_hip_chain_forward(void* stream, const nnf_hip_chain_desc* desc, float* output,
+		const float* const* inputs, const float* const* chunk_ptrs)
+	{
+		return chain_forward(static_cast<hipStream_t>(stream), desc, output, inputs, chunk_ptrs);
+	}
+
+	int nnf_hip_batch_norm_forward(void* stream, float* output, const float* input,
+		const float* gamma, const float* beta, const float* mean, const float* inverse_sigma,
+		uint32_t entry_count, uint32_t feature_map_count, uint32_t neuron_count_per_feature_map)
+	{
+		const nnf_hip_chain_desc d = single_op_desc(entry_count, feature_map_count, neuron_count_per_feature_map, NNF_HIP_OP_BATCH_NORM, 0, 0.0f, 0.0f);
+		const float* inputs[1] = { input };
+		const float* chunks[4] = { gamma, beta, mean, inverse_sigma };
+		return chain_forward(static_cast<hipStream_t>(stream), &d, output, inputs, chunks);
+	}
+
+	int nnf_hip_rectified_linear_forward(void* stream, float* output, const float* input, float negative_slope, uint64_t elem_count)
+	{
+		return flat_op(static_cast<hipStream_t>(stream), output, input, elem_count, NNF_HIP_OP_RELU, negative_slope, 0.0f);
+	}
+
+	int nnf_hip_parametric_rectified_linear_forward(void* stream, float* output, const float* input,
+		const float* slopes, uint32_t entry_count, uint32_t feature_map_count, uint32_t neuron_count_per_feature_map)
+	{
+		const nnf_hip_chain_desc d = single_op_desc(entry_count, feature_map_count, neuron_count_per_feature_map, NNF_HIP_OP_PRELU, 0, 0.0f, 0.0f);
+		const float* inputs[1] = { input };
+		const float* chunks[1] = { slopes };
+		return chain_forward(static_cast<hipStream_t>(stream), &d, output, inputs, chunks);
+	}
+
+	int nnf_hip_exponential_linear_forward(void* stream, float* output, const float* input, uint64_t elem_count)
+	{
+		return flat_op(static_cast<hipStream_t>(stream), output, input, elem_count, NNF_HIP_OP_ELU, 0.0f, 0.0f);
+	}
+
+	int nnf_hip_sigmoid_forward(void* stream, float* output, const float* input, uint64_t elem_count)
+	{
+		return flat_op(static_cast<hipStream_t>(stream), output, input, elem_count, NNF_HIP_OP_SIGMOID, 0.0f, 0.0f);
+	}
+
+	int nnf_hip_hyperbolic_tangent_forward(void* stream, float* output, const float* input, float scale, float steepness, uint64_t elem_count)
+	{
+		return flat_op(static_cast<hipStream_t>(stream), output, input, elem_count, NNF_HIP_OP_TANH, scale, steepness);
+	}
+
+	int nnf_hip_add_forward(void* stream, float* output, const float* const* inputs, uint32_t input_count, float alpha, uint64_t elem_count)
+	{
+		if ((inputs == nullptr) || (input_count == 0) || (output == nullptr))
+			return NNF_HIP_EINVAL;
+		if (elem_count == 0)
+			return NNF_HIP_OK;
+		uint32_t entry_count, plane;
+		if (!flat_shape(elem_count, entry_count, plane))
+			return NNF_HIP_ETOOBIG;
+		// The output may alias inputs[0] only; a later input that overlaps the output would be
+		// clobbered by the first partial launch, so it is rejected here for every input_count.
+		for(uint32_t j = 1; j < input_count; ++j)
+		{
+			if (inputs[j] == nullptr)
+				return NNF_HIP_EINVAL;
+			const uintptr_t a = reinterpret_cast<uintptr_t>(output), b = reinterpret_cast<uintptr_t>(inputs[j]);
+			const size_t bytes = static_cast<size_t>(elem_count) * sizeof(float);
+			if ((a < b + bytes) && (b < a + bytes))
+				return NNF_HIP_EOVERLAP;
+		}
+
+		// Left-to-right sum in groups of NNF_HIP_MAX_INPUTS: the partial sum (alpha = 1) becomes the
+		// first input of the next group. 0.0F + partial == partial bit for bit (a sum that started
+		// from +0.0F is never -0.0F), so the grouping does not change the result.
+		nnf_hip_chain_desc d;
+		std::memset(&d, 0, sizeof(d));
+		d.entry_count = entry_count;
+		d.feature_map_count = 1;
+		d.neuron_count_per_feature_map = plane;
+		d.has_add = 1;
+		uint32_t done = 0;
+		const float* group[NNF_HIP_MAX_INPUTS];
+		while (done < input_count)
+		{
+			uint32_t n = 0;
+			if (done > 0)
+				group[n++] = output;
+			while ((n < NNF_HIP_MAX_INPUTS) && (done < input_count))
+				group[n++] = inputs[done++];
+			d.input_count = n;
+			d.add_alpha = (done == input_count) ? alpha : 1.0f;
+			const int rc = chain_forward(static_cast<hipStream_t>(stream), &d, output, group, nullptr);
+			if (rc != NNF_HIP_OK)
+				return rc;
+		}
+		return NNF_HIP_OK;
+	}
+
+	int nnf_hip_softmax_forward(void* stream, float* output, const float* input,
+		uint32_t entry_count, uint32_t feature_map_count, uint32_t neuron_count_per_feature_map)
+	{
+		return softmax_forward(static_cast<hipStream_t>(stream), output, input, entry_count, feature_map_count, neuron_count_per_feature_map);
+	}
+
+	int nnf_hip_average_subsampling_forward(void* stream, float* output, const float* input,
+		uint32_t entry_count, uint32_t feature_map_count, uint32_t input_width, uint32_t input_height,
+		uint32_t window_width, uint32_t window_height, float mult)
+	{
+		return average_subsampling_forward(static_cast<hipStream_t>(stream), output, input, entry_count, feature_map_count,
+			input_width, input_height, window_width, window_height, mult);
+	}
+
+	int nnf_hip_copy_kernel(void* stream, void* device_dst, const void* device_src, size_t bytes)
+	{
+		return copy_kernel(static_cast<hipStream_t>(stream), device_dst, device_src, bytes);
+	}
+
+	// ---- runtime plumbing ------------------------------------------------------------------
+
+	int nnf_hip_device_count(int* count)
+	{
+		if (count == nullptr)
+			return NNF_HIP_EINVAL;
+		return hip_status(hipGetDeviceCount(count));
+	}
+
+	int nnf_hip_set_device(int device_id)
+	{
+		return hip_status(hipSetDevice(device_id));
+	}
+
+	int nnf_hip_device_info(int device_id, char* name, size_t name_capacity, uint64_t* global_memory_bytes,
+		uint32_t* compute_unit_count, uint32_t* wavefront_size, uint32_t* clock_khz)
+	{
+		hipDeviceProp_t prop;
+		const hipError_t e = hipGetDeviceProperties(&prop, device_id);
+		if (e != hipSuccess)
+			return hip_status(e);
+		if ((name != nullptr) && (name_capacity > 0))
+		{
+			std::strncpy(name, prop.name, name_capacity - 1);
+			name[name_capacity - 1] = '\0';
+		}
+		if (global_memory_bytes != nullptr)
+			*global_memory_bytes = prop.totalGlobalMem;
+		if (compute_unit_count != nullptr)
+			*compute_unit_count = static_cast<uint32_t>(prop.multiProcessorCount);
+		if (wavefront_size != nullptr)
+			*wavefront_size = static_cast<uint32_t>(prop.warpSize);
+		if (clock_khz != nullptr)
+			*clock_khz = static_cast<uint32_t>(prop.clockRate);
+		return NNF_HIP_OK;
+	}
+
+	int nnf_hip_malloc(void** device_ptr, size_t bytes)
+	{
+		if (device_ptr == nullptr)
+			return NNF_HIP_EINVAL;
+		const size_t padded = (bytes + 15) & ~static_cast<size_t>(15);
+		return hip_status(hipMalloc(device_ptr, padded == 0 ? 16 : padded));
+	}
+
+	int nnf_hip_free(void* device_ptr)
+	{
+		return hip_status(hipFree(device_ptr));
+	}
+
+	int nnf_hip_memcpy_h2d(void* device_dst, const void* host_src, size_t bytes, void* stream)
+	{
+		if (stream == nullptr)
+			return hip_status(hipMemcpy(device_dst, host_src, bytes, hipMemcpyHostToDevice));
+		return hip_status(hipMemcpyAsync(device_dst, host_src, bytes, hipMemcpyHostToDevice, static_cast<hipStream_t>(stream)));
+	}
+
+	int nnf_hip_memcpy_d2h(void* host_dst, const void* device_src, size_t bytes, void* stream)
+	{
+		if (stream == nullptr)
+			return hip_status(hipMemcpy(host_dst, device_src, bytes, hipMemcpyDeviceToHost));
+		return hip_status(hipMemcpyAsync(host_dst, device_src, bytes, hipMemcpyDeviceToHost, static_cast<hipStream_t>(stream)));
+	}
+
+	int nnf_hip_memcpy_d2d(void* device_dst, const void* device_src, size_t bytes, void* stream)
+	{
+		if (stream == nullptr)
+			return hip_status(hipMemcpy(device_dst, device_src, bytes, hipMemcpyDeviceToDevice));
+		return hip_status(hipMemcpyAsync(device_dst, device_src, bytes, hipMemcpyDeviceToDevice, static_cast<hipStream_t>(stream)));
+	}
+
+	int nnf_hip_host_malloc(void** host_ptr, size_t bytes)
+	{
+		if (host_ptr == nullptr)
+			return NNF_HIP_EINVAL;
+		return hip_status(hipHostMalloc(host_ptr, bytes == 0 ? 16 : bytes, hipHostMallocDefault));
+	}
+
+	int nnf_hip_host_free(void* host_ptr)
+	{
+		return hip_status(hipHostFree(host_ptr));
+	}
+
+	int nnf_hip_stream_create(void** stream)
+	{
+		if (stream == nullptr)
+			return NNF_HIP_EINVAL;
+		hipStream_t s = nullptr;
+		const hipError_t e = hipStreamCreateWithFlags(&s, hipStreamNonBlocking); // default priority
+		*stream = s;
+		return hip_status(e);
+	}
+
+	int nnf_hip_stream_destroy(void* stream)
+	{
+		return hip_status(hipStreamDestroy(static_cast<hipStream_t>(stream)));
+	}
+
+	int nnf_hip_stream_synchronize(void* stream)
+	{
+		return hip_status(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+	}
+
+	int nnf_hip_device_synchronize(void)
+	{
+		return hip_status(hipDeviceSynchronize());
+	}
+
+	int nnf_hip_event_create(void** event)
+	{
+		if (event == nullptr)
+			return NNF_HIP_EINVAL;
+		hipEvent_t ev = nullptr;
+		const hipError_t e = hipEventCreate(&ev);
+		*event = ev;
+		return hip_status(e);
+	}
+
+	int nnf_hip_event_destroy(void* event)
+	{
+		return hip_status(hipEventDestroy(static_cast<hipEvent_t>(event)));
+	}
+
+	int nnf_hip_event_record(void* event, void* stream)
+	{
+		return hip_status(hipEventRecord(static_cast<hipEvent_t>(event), static_cast<hipStream_t>(stream)));
+	}
+
+	int nnf_hip_event_synchronize(void* event)
+	{
+		return hip_status(hipEventSynchronize(static_cast<hipEvent_t>(event)));
+	}
+
+	int nnf_hip_event_elapsed_ms(float* milliseconds, void* start_event, void* stop_event)
+	{
+		if (milliseconds == nullptr)
+			return NNF_HIP_EINVAL;
+		return hip_status(hipEventElapsedTime(milliseconds, static_cast<hipEvent_t>(start_event), static_cast<hipEvent_t>(stop_event)));
+	}
+
+	int nnf_hip_stream_wait_event(void* stream, void* event)
+	{
+		return hip_status(hipStreamWaitEvent(static_cast<hipStream_t>(stream), static_cast<hipEvent_t>(event), 0));
+	}
+
+	const char* nnf_hip_error_string(int code)
+	{
+		switch (code)
+		{
+		case NNF_HIP_OK: return "success";
+		case NNF_HIP_EINVAL: return "nnforge_hip: invalid argument (null pointer, zero-sized dimension or malformed descriptor)";
+		case NNF_HIP_EUNSUPPORTED: return "nnforge_hip: shape or option not supported by the kernels";
+		case NNF_HIP_EALIGN: return "nnforge_hip: tensor base pointer is not 16-byte aligned";
+		case NNF_HIP_EOVERLAP: return "nnforge_hip: output overlaps an input (only output == inputs[0] is allowed)";
+		case NNF_HIP_ETOOBIG: return "nnforge_hip: element count exceeds the 32-bit index range of the kernels";
+		default:
+			if (code > 0)
+				return hipGetErrorString(static_cast<hipError_t>(code));
+			return "nnforge_hip: unknown error code";
+		}
+	}
+
+	const char* nnf_hip_version(void)
+	{
+		return "nnforge_hip 0.1 (gfx950)";
+	}
+}

@@ -1,0 +1,64 @@
+// Shared declarations of the gfx950 kernel translation units.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/nnforge_hip.h"
+#include "nnf_math.h"
+
+namespace nnf
+{
+	typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+	constexpr int wave_size = 64;
+
+	// 2^(i/32) table of nnf_expf in device memory (one copy per translation unit); kernels copy it
+	// to LDS before use.
+	static __device__ const uint64_t exp2_table_device[exp2_table_size] = { NNF_EXP2_TABLE_VALUES };
+
+	__device__ __forceinline__ void stage_exp2_table(uint64_t* lds_table)
+	{
+		if (threadIdx.x < exp2_table_size)
+			lds_table[threadIdx.x] = exp2_table_device[threadIdx.x];
+	}
+
+	// Streaming accesses: each byte of an activation tensor is touched once per launch, so loads
+	// and stores carry the non-temporal hint and do not displace what the caches hold.
+	__device__ __forceinline__ floatx4 load_stream(const floatx4* p)
+	{
+		return __builtin_nontemporal_load(p);
+	}
+
+	__device__ __forceinline__ void store_stream(floatx4* p, floatx4 v)
+	{
+		__builtin_nontemporal_store(v, p);
+	}
+
+	inline bool is_aligned16(const void* p)
+	{
+		return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
+	}
+
+	inline int hip_status(hipError_t e)
+	{
+		return static_cast<int>(e);
+	}
+
+	// Launch errors are reported by hipGetLastError right after the launch; asynchronous faults
+	// surface at the caller's next synchronising call, as with any HIP work.
+	inline int launch_status()
+	{
+		return hip_status(hipGetLastError());
+	}
+
+	// entry points implemented in the individual translation units
+	int chain_forward(hipStream_t stream, const nnf_hip_chain_desc* desc, float* output,
+		const float* const* inputs, const float* const* chunk_ptrs);
+	int softmax_forward(hipStream_t stream, float* output, const float* input,
+		uint32_t entry_count, uint32_t feature_map_count, uint32_t neuron_count_per_feature_map);
+	int average_subsampling_forward(hipStream_t stream, float* output, const float* input,
+		uint32_t entry_count, uint32_t feature_map_count, uint32_t input_width, uint32_t input_height,
+		uint32_t window_width, uint32_t window_height, float mult);
+	int copy_kernel(hipStream_t stream, void* dst, const void* src, size_t bytes);
+}

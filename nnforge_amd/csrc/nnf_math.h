@@ -1,0 +1,123 @@
+// Scalar fp32 arithmetic of the element-wise layers, written once and used by the gfx950 kernels
+// (compiled by hipcc) and by host-side unit tests of the same formulas (compiled by g++).
+//
+// Rounding policy: every fp32 operation below rounds once, in the order the reference's plain
+// testers write it; translation units that include this header are compiled with
+// -ffp-contract=off so that no multiply-add pair is fused. The only fused operations are the
+// explicit __builtin_fma calls inside nnf_expf, which work in double precision.
+#pragma once
+
+#include <stdint.h>
+
+#if defined(__HIPCC__)
+#define NNF_HD __host__ __device__ __forceinline__
+#else
+#define NNF_HD inline
+#endif
+
+namespace nnf
+{
+	// 2^(i/32) as IEEE-754 double bit patterns with i << 47 subtracted, i = 0..31: adding k << 47
+	// (k = 32*e + i) to entry i yields 2^(k/32) directly.
+	#define NNF_EXP2_TABLE_VALUES \
+		0x3ff0000000000000ull, 0x3fefd9b0d3158574ull, 0x3fefb5586cf9890full, 0x3fef9301d0125b51ull, \
+		0x3fef72b83c7d517bull, 0x3fef54873168b9aaull, 0x3fef387a6e756238ull, 0x3fef1e9df51fdee1ull, \
+		0x3fef06fe0a31b715ull, 0x3feef1a7373aa9cbull, 0x3feedea64c123422ull, 0x3feece086061892dull, \
+		0x3feebfdad5362a27ull, 0x3feeb42b569d4f82ull, 0x3feeab07dd485429ull, 0x3feea47eb03a5585ull, \
+		0x3feea09e667f3bcdull, 0x3fee9f75e8ec5f74ull, 0x3feea11473eb0187ull, 0x3feea589994cce13ull, \
+		0x3feeace5422aa0dbull, 0x3feeb737b0cdc5e5ull, 0x3feec49182a3f090ull, 0x3feed503b23e255dull, \
+		0x3feee89f995ad3adull, 0x3feeff76f2fb5e47ull, 0x3fef199bdd85529cull, 0x3fef3720dcef9069ull, \
+		0x3fef5818dcfba487ull, 0x3fef7c97337b9b5full, 0x3fefa4afa2a490daull, 0x3fefd0765b6e4540ull
+
+	constexpr int exp2_table_size = 32;
+
+	NNF_HD double bits_to_double(uint64_t u) { return __builtin_bit_cast(double, u); }
+	NNF_HD uint64_t double_to_bits(double d) { return __builtin_bit_cast(uint64_t, d); }
+
+	// expf with the result of a double-precision evaluation rounded once to fp32.
+	//
+	// The reference's plain testers call the C library's expf (e.g.
+	// nnforge/plain/exponential_linear_layer_tester_plain.cpp:51). glibc >= 2.27 evaluates expf as
+	// 2^(k/32) * p(r) in double precision (x*32/ln2 = k + r, |r| <= 1/2, 32-entry table, cubic p) and
+	// rounds the double to float, which makes it correctly rounded for all but a handful of inputs.
+	// This is the same published scheme with every multiply-add fused, the form an FMA-capable x86-64
+	// host evaluates; it returns the same bits as that expf for every one of the 2^32 fp32 inputs
+	// (checked exhaustively on the host by the unit tests; NaN payloads aside).
+	//   table: the 32 values of NNF_EXP2_TABLE_VALUES (LDS copy on the device).
+	NNF_HD float nnf_expf(float x, const uint64_t* table)
+	{
+		const double inv_ln2_times_32 = 0x1.71547652b82fep+5;
+		const double shift = 0x1.8p+52; // adding it rounds to an integer kept in the low mantissa bits
+		const double c0 = 0x1.c6af84b912394p-20; // (ln2/32)^3 / 6, minimax-adjusted
+		const double c1 = 0x1.ebfce50fac4f3p-13; // (ln2/32)^2 / 2
+		const double c2 = 0x1.62e42ff0c52d6p-6;  // ln2/32
+
+		const double xd = static_cast<double>(x);
+		double kd = __builtin_fma(inv_ln2_times_32, xd, shift);
+		const uint64_t ki = double_to_bits(kd);
+		kd -= shift;
+		const double r = __builtin_fma(inv_ln2_times_32, xd, -kd);
+		const uint64_t t = table[ki & (exp2_table_size - 1)] + (ki << 47);
+		const double s = bits_to_double(t);
+		const double z = __builtin_fma(c0, r, c1);
+		const double r2 = r * r;
+		double y = __builtin_fma(c2, r, 1.0);
+		y = __builtin_fma(z, r2, y);
+		y = y * s;
+		float res = static_cast<float>(y);
+		// Outside (log(2^-150), log(2^128)) the double path is meaningless (k does not fit): the
+		// results there are 0 and +inf. NaN fails both comparisons and comes out of the arithmetic as NaN.
+		res = x > 0x1.62e42ep6f ? __builtin_inff() : res;
+		res = x < -0x1.9fe368p6f ? 0.0f : res;
+		return res;
+	}
+
+	// nnforge/plain/batch_norm_layer_tester_plain.cpp:60-61
+	NNF_HD void nnf_batch_norm_coefficients(float gamma, float beta, float mean, float inverse_sigma, float& mult, float& add)
+	{
+		mult = gamma * inverse_sigma;
+		const float mult_mean = mult * mean;
+		add = beta - mult_mean;
+	}
+
+	// nnforge/plain/batch_norm_layer_tester_plain.cpp:70-71
+	NNF_HD float nnf_batch_norm(float x, float mult, float add)
+	{
+		const float scaled = x * mult;
+		return scaled + add;
+	}
+
+	// nnforge/plain/rectified_linear_layer_tester_plain.cpp:53-54
+	NNF_HD float nnf_rectified_linear(float x, float negative_slope)
+	{
+		return x >= 0.0f ? x : x * negative_slope;
+	}
+
+	// nnforge/plain/parametric_rectified_linear_layer_tester_plain.cpp:66-67
+	NNF_HD float nnf_parametric_rectified_linear(float x, float a)
+	{
+		return x * (x >= 0.0f ? 1.0f : a);
+	}
+
+	// nnforge/plain/exponential_linear_layer_tester_plain.cpp:50-51
+	NNF_HD float nnf_exponential_linear(float x, const uint64_t* table)
+	{
+		const float e = nnf_expf(x, table);
+		return x >= 0.0f ? x : (e - 1.0f);
+	}
+
+	// nnforge/plain/sigmoid_layer_tester_plain.cpp:50-51
+	NNF_HD float nnf_sigmoid(float x, const uint64_t* table)
+	{
+		const float e = nnf_expf(-x, table);
+		return 1.0f / (e + 1.0f);
+	}
+
+	// nnforge/plain/hyperbolic_tangent_layer_tester_plain.cpp:54-56; steepness2 = steepness * 2.0f
+	NNF_HD float nnf_hyperbolic_tangent(float x, float steepness2, float scale, const uint64_t* table)
+	{
+		const float e = nnf_expf(x * steepness2, table);
+		const float q = (e - 1.0f) / (e + 1.0f);
+		return q * scale;
+	}
+}

@@ -1,0 +1,125 @@
+// 2-D average subsampling with non-overlapping windows
+// (nnforge/plain/average_subsampling_layer_tester_plain.cpp:125-145): every output is the
+// left-to-right fp32 sum of its window (x fastest, then y) multiplied by mult. Both kernels keep
+// that summation order, so results equal the reference's bit for bit.
+#include "nnf_common.h"
+
+namespace nnf
+{
+	namespace
+	{
+		constexpr int pool_block_size = 256;
+		constexpr uint32_t global_pool_max_plane = 60; // 256 planes * 61 floats of padded LDS = 62.5 KB
+
+		// Window == whole plane (global pooling, e.g. 7x7 -> 1x1). A workgroup reduces 256 consecutive
+		// planes: it copies them to LDS with coalesced float4 loads, then lane t sums plane t front to
+		// back. Planes are stored with an odd stride so that the 64 lanes of a wavefront hit distinct banks.
+		__global__ void __launch_bounds__(pool_block_size) global_pool_kernel(float* out, const float* in, uint32_t plane_count, uint32_t plane, float mult)
+		{
+			extern __shared__ __align__(16) float lds_planes[];
+			const uint32_t stride = plane | 1u;
+			const uint32_t first_plane = blockIdx.x * pool_block_size;
+			const uint32_t planes_here = min(static_cast<uint32_t>(pool_block_size), plane_count - first_plane);
+			const uint32_t floats_here = planes_here * plane; // multiple of 4 except possibly in the last workgroup
+			const float* src = in + static_cast<size_t>(first_plane) * plane; // 16-byte aligned: first_plane is a multiple of 256
+
+			const uint32_t vectors = floats_here / 4;
+			for(uint32_t i = threadIdx.x; i < vectors; i += pool_block_size)
+			{
+				const floatx4 t = load_stream(reinterpret_cast<const floatx4*>(src) + i);
+				const float vals[4] = {t.x, t.y, t.z, t.w};
+				#pragma unroll
+				for(int e = 0; e < 4; ++e)
+				{
+					const uint32_t f = i * 4 + e;
+					const uint32_t p = f / plane;
+					lds_planes[p * stride + (f - p * plane)] = vals[e];
+				}
+			}
+			for(uint32_t f = vectors * 4 + threadIdx.x; f < floats_here; f += pool_block_size)
+			{
+				const uint32_t p = f / plane;
+				lds_planes[p * stride + (f - p * plane)] = src[f];
+			}
+			__syncthreads();
+
+			if (threadIdx.x < planes_here)
+			{
+				const float* my_plane = lds_planes + threadIdx.x * stride;
+				float sum = 0.0f;
+				for(uint32_t i = 0; i < plane; ++i)
+					sum += my_plane[i];
+				out[first_plane + threadIdx.x] = sum * mult;
+			}
+		}
+
+		// General case: one lane per output neuron, window read straight from memory.
+		__global__ void __launch_bounds__(pool_block_size) window_pool_kernel(
+			float* out, const float* in, uint32_t output_count,
+			uint32_t input_width, uint32_t input_height, uint32_t output_width, uint32_t output_height,
+			uint32_t window_width, uint32_t window_height, float mult)
+		{
+			const uint32_t o = blockIdx.x * pool_block_size + threadIdx.x;
+			if (o >= output_count)
+				return;
+			const uint32_t ox = o % output_width;
+			const uint32_t oy = (o / output_width) % output_height;
+			const uint32_t plane_id = o / (output_width * output_height);
+			const float* src = in + static_cast<size_t>(plane_id) * input_width * input_height
+				+ static_cast<size_t>(oy) * window_height * input_width + static_cast<size_t>(ox) * window_width;
+			float sum = 0.0f;
+			for(uint32_t wy = 0; wy < window_height; ++wy)
+			{
+				for(uint32_t wx = 0; wx < window_width; ++wx)
+					sum += src[wy * input_width + wx];
+			}
+			out[o] = sum * mult;
+		}
+	}
+
+	int average_subsampling_forward(hipStream_t stream, float* output, const float* input,
+		uint32_t entry_count, uint32_t feature_map_count, uint32_t input_width, uint32_t input_height,
+		uint32_t window_width, uint32_t window_height, float mult)
+	{
+		if ((output == nullptr) || (input == nullptr))
+			return NNF_HIP_EINVAL;
+		if ((feature_map_count == 0) || (input_width == 0) || (input_height == 0) || (window_width == 0) || (window_height == 0))
+			return NNF_HIP_EINVAL;
+		// nnforge/average_subsampling_layer.cpp:82-87: the input may not be smaller than the window; the
+		// output size is the quotient rounded down and a leftover right/bottom margin is not read
+		if ((input_width < window_width) || (input_height < window_height))
+			return NNF_HIP_EINVAL;
+		if (!is_aligned16(output) || !is_aligned16(input))
+			return NNF_HIP_EALIGN;
+
+		const uint32_t output_width = input_width / window_width;
+		const uint32_t output_height = input_height / window_height;
+		const uint64_t input_total = static_cast<uint64_t>(entry_count) * feature_map_count * input_width * input_height;
+		if (input_total == 0)
+			return NNF_HIP_OK;
+		if (input_total > 0xFFFF0000ull)
+			return NNF_HIP_ETOOBIG;
+		const uint32_t plane_count = entry_count * feature_map_count;
+		const uint32_t output_count = plane_count * output_width * output_height;
+		{
+			const uintptr_t a = reinterpret_cast<uintptr_t>(output), b = reinterpret_cast<uintptr_t>(input);
+			if ((a < b + input_total * sizeof(float)) && (b < a + static_cast<uint64_t>(output_count) * sizeof(float)))
+				return NNF_HIP_EOVERLAP; // the tester cannot run in place: get_input_index_layer_can_write is -1 for it
+		}
+
+		const uint32_t plane = input_width * input_height;
+		if ((window_width == input_width) && (window_height == input_height) && (plane <= global_pool_max_plane))
+		{
+			const size_t lds_bytes = static_cast<size_t>(pool_block_size) * (plane | 1u) * sizeof(float);
+			const dim3 grid((plane_count + pool_block_size - 1) / pool_block_size);
+			hipLaunchKernelGGL(global_pool_kernel, grid, dim3(pool_block_size), lds_bytes, stream, output, input, plane_count, plane, mult);
+		}
+		else
+		{
+			const dim3 grid((output_count + pool_block_size - 1) / pool_block_size);
+			hipLaunchKernelGGL(window_pool_kernel, grid, dim3(pool_block_size), 0, stream, output, input, output_count,
+				input_width, input_height, output_width, output_height, window_width, window_height, mult);
+		}
+		return launch_status();
+	}
+}

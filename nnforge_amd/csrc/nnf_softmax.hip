@@ -1,0 +1,355 @@
+// Softmax across feature maps at every (entry, spatial position), fp32
+// (nnforge/plain/softmax_layer_tester_plain.cpp:61-89): max over feature maps starting from
+// -1.0e37F, val = expf(x - max), sum of val, mult = 1/sum, out = val * mult.
+//
+// Two data shapes:
+//  - neuron_count_per_feature_map == 1: the feature maps of an entry are contiguous ("rows").
+//    A row lives in the registers of one wavefront (or one workgroup for long rows); max and sum
+//    are 64-lane reductions; the row is read once and written once. The sum is a fixed tree, so it
+//    can differ from the reference's left-to-right sum in the last bits.
+//  - neuron_count_per_feature_map > 1: feature maps are strided by the plane size ("columns").
+//    Lanes run along the spatial positions (coalesced), each lane walks its column in feature-map
+//    order with the reference's own sequential sum.
+#include "nnf_common.h"
+
+namespace nnf
+{
+	namespace
+	{
+		constexpr float softmax_max_init = -1.0e+37F; // nnforge/plain/softmax_layer_tester_plain.cpp:71
+
+		// std::max(a, b) as the reference evaluates it: (a < b) ? b : a, so a NaN in b is never picked
+		__device__ __forceinline__ float ref_max(float a, float b)
+		{
+			return (a < b) ? b : a;
+		}
+
+		template<int CTRL>
+		__device__ __forceinline__ float dpp_move(float v)
+		{
+			return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, false));
+		}
+
+		__device__ __forceinline__ float read_lane(float v, int lane)
+		{
+			return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+		}
+
+		// 64-lane all-reduce: four DPP steps combine each row of 16 lanes (quad swaps 0xB1 and 0x4E,
+		// row_half_mirror 0x141, row_mirror 0x140), then the four row results are read as scalars.
+		struct max_op { __device__ __forceinline__ float operator()(float a, float b) const { return ref_max(a, b); } };
+		struct sum_op { __device__ __forceinline__ float operator()(float a, float b) const { return a + b; } };
+
+		template<class OP>
+		__device__ __forceinline__ float wave_all_reduce(float v, OP op)
+		{
+			v = op(v, dpp_move<0xB1>(v));
+			v = op(v, dpp_move<0x4E>(v));
+			v = op(v, dpp_move<0x141>(v));
+			v = op(v, dpp_move<0x140>(v));
+			const float r0 = read_lane(v, 0);
+			const float r1 = read_lane(v, 16);
+			const float r2 = read_lane(v, 32);
+			const float r3 = read_lane(v, 48);
+			return op(op(r0, r1), op(r2, r3));
+		}
+
+		template<int W> struct vec_io;
+		template<> struct vec_io<4>
+		{
+			static __device__ __forceinline__ void load(const float* p, float (&d)[4])
+			{
+				const floatx4 t = *reinterpret_cast<const floatx4*>(p);
+				d[0] = t.x; d[1] = t.y; d[2] = t.z; d[3] = t.w;
+			}
+			static __device__ __forceinline__ void store(float* p, const float (&d)[4])
+			{
+				floatx4 t;
+				t.x = d[0]; t.y = d[1]; t.z = d[2]; t.w = d[3];
+				*reinterpret_cast<floatx4*>(p) = t;
+			}
+		};
+		template<> struct vec_io<1>
+		{
+			static __device__ __forceinline__ void load(const float* p, float (&d)[1]) { d[0] = *p; }
+			static __device__ __forceinline__ void store(float* p, const float (&d)[1]) { *p = d[0]; }
+		};
+
+		// One row per group of THREADS lanes (THREADS = 64: a wavefront; larger: a whole workgroup).
+		// Lane t holds vectors t, t + THREADS, ... of its row: VPT vectors of W floats.
+		// Rows per workgroup = blockDim.x / THREADS. Requires fm_count <= THREADS * VPT * W and,
+		// for W == 4, fm_count % 4 == 0 (then every row start is 16-byte aligned).
+		template<int THREADS, int VPT, int W>
+		__global__ void __launch_bounds__(1024) softmax_rows_kernel(float* out, const float* in, uint32_t rows, uint32_t fm_count)
+		{
+			__shared__ uint64_t lds_exp[exp2_table_size];
+			__shared__ float lds_partial[2][1024 / wave_size];
+			stage_exp2_table(lds_exp);
+			__syncthreads();
+
+			const uint32_t rows_per_block = blockDim.x / THREADS;
+			const uint32_t lane = threadIdx.x % THREADS;
+			const uint32_t row = blockIdx.x * rows_per_block + threadIdx.x / THREADS;
+			const bool row_valid = row < rows;
+			const float* src = in + static_cast<size_t>(row_valid ? row : 0) * fm_count;
+			float* dst = out + static_cast<size_t>(row_valid ? row : 0) * fm_count;
+
+			float v[VPT][W];
+			float m = softmax_max_init;
+			#pragma unroll
+			for(int k = 0; k < VPT; ++k)
+			{
+				const uint32_t c = (lane + k * THREADS) * W;
+				if (row_valid && (c < fm_count))
+				{
+					vec_io<W>::load(src + c, v[k]);
+					#pragma unroll
+					for(int e = 0; e < W; ++e)
+						m = ref_max(m, v[k][e]);
+				}
+			}
+			m = wave_all_reduce(m, max_op());
+			if (THREADS > wave_size)
+			{
+				const uint32_t wave = threadIdx.x / wave_size;
+				if ((threadIdx.x % wave_size) == 0)
+					lds_partial[0][wave] = m;
+				__syncthreads();
+				m = softmax_max_init;
+				for(uint32_t w = 0; w < THREADS / wave_size; ++w)
+					m = ref_max(m, lds_partial[0][w]);
+			}
+
+			float sum = 0.0f;
+			#pragma unroll
+			for(int k = 0; k < VPT; ++k)
+			{
+				const uint32_t c = (lane + k * THREADS) * W;
+				if (row_valid && (c < fm_count))
+				{
+					#pragma unroll
+					for(int e = 0; e < W; ++e)
+					{
+						v[k][e] = nnf_expf(v[k][e] - m, lds_exp);
+						sum += v[k][e];
+					}
+				}
+			}
+			sum = wave_all_reduce(sum, sum_op());
+			if (THREADS > wave_size)
+			{
+				const uint32_t wave = threadIdx.x / wave_size;
+				if ((threadIdx.x % wave_size) == 0)
+					lds_partial[1][wave] = sum;
+				__syncthreads();
+				sum = 0.0f;
+				for(uint32_t w = 0; w < THREADS / wave_size; ++w)
+					sum += lds_partial[1][w];
+			}
+
+			const float mult = 1.0f / sum;
+			#pragma unroll
+			for(int k = 0; k < VPT; ++k)
+			{
+				const uint32_t c = (lane + k * THREADS) * W;
+				if (row_valid && (c < fm_count))
+				{
+					#pragma unroll
+					for(int e = 0; e < W; ++e)
+						v[k][e] = v[k][e] * mult;
+					vec_io<W>::store(dst + c, v[k]);
+				}
+			}
+		}
+
+		// Rows longer than a workgroup's registers hold: one workgroup per row, three passes over the
+		// row (the second and third mostly served by the L2 cache), expf values parked in the output
+		// like the reference does.
+		__global__ void __launch_bounds__(1024) softmax_long_rows_kernel(float* out, const float* in, uint32_t fm_count)
+		{
+			__shared__ uint64_t lds_exp[exp2_table_size];
+			__shared__ float lds_partial[2][1024 / wave_size];
+			stage_exp2_table(lds_exp);
+
+			const float* src = in + static_cast<size_t>(blockIdx.x) * fm_count;
+			float* dst = out + static_cast<size_t>(blockIdx.x) * fm_count;
+			const uint32_t wave = threadIdx.x / wave_size;
+			const uint32_t wave_count = blockDim.x / wave_size;
+
+			float m = softmax_max_init;
+			for(uint32_t c = threadIdx.x; c < fm_count; c += blockDim.x)
+				m = ref_max(m, src[c]);
+			m = wave_all_reduce(m, max_op());
+			if ((threadIdx.x % wave_size) == 0)
+				lds_partial[0][wave] = m;
+			__syncthreads();
+			m = softmax_max_init;
+			for(uint32_t w = 0; w < wave_count; ++w)
+				m = ref_max(m, lds_partial[0][w]);
+
+			float sum = 0.0f;
+			for(uint32_t c = threadIdx.x; c < fm_count; c += blockDim.x)
+			{
+				const float val = nnf_expf(src[c] - m, lds_exp);
+				sum += val;
+				dst[c] = val;
+			}
+			sum = wave_all_reduce(sum, sum_op());
+			if ((threadIdx.x % wave_size) == 0)
+				lds_partial[1][wave] = sum;
+			__syncthreads();
+			sum = 0.0f;
+			for(uint32_t w = 0; w < wave_count; ++w)
+				sum += lds_partial[1][w];
+
+			const float mult = 1.0f / sum;
+			for(uint32_t c = threadIdx.x; c < fm_count; c += blockDim.x)
+				dst[c] = dst[c] * mult; // each lane re-reads only what it wrote itself
+		}
+
+		// neuron_count_per_feature_map > 1. One lane per (entry, position); consecutive lanes take
+		// consecutive positions. Same operation order as the reference, including the sequential sum.
+		// CACHED > 0: the column (fm_count <= CACHED) stays in registers: one read, one write.
+		template<int CACHED>
+		__global__ void __launch_bounds__(256) softmax_columns_kernel(float* out, const float* in, uint32_t columns, uint32_t fm_count, uint32_t plane)
+		{
+			__shared__ uint64_t lds_exp[exp2_table_size];
+			stage_exp2_table(lds_exp);
+			__syncthreads();
+
+			const uint32_t column = blockIdx.x * blockDim.x + threadIdx.x;
+			if (column >= columns)
+				return;
+			const uint32_t entry = column / plane;
+			const uint32_t pos = column - entry * plane;
+			const size_t base = static_cast<size_t>(entry) * fm_count * plane + pos;
+			const float* src = in + base;
+			float* dst = out + base;
+
+			if (CACHED > 0)
+			{
+				float v[CACHED > 0 ? CACHED : 1];
+				float m = softmax_max_init;
+				#pragma unroll
+				for(int c = 0; c < CACHED; ++c)
+				{
+					if (static_cast<uint32_t>(c) < fm_count)
+					{
+						v[c] = src[static_cast<size_t>(c) * plane];
+						m = ref_max(m, v[c]);
+					}
+				}
+				float sum = 0.0f;
+				#pragma unroll
+				for(int c = 0; c < CACHED; ++c)
+				{
+					if (static_cast<uint32_t>(c) < fm_count)
+					{
+						v[c] = nnf_expf(v[c] - m, lds_exp);
+						sum += v[c];
+					}
+				}
+				const float mult = 1.0f / sum;
+				#pragma unroll
+				for(int c = 0; c < CACHED; ++c)
+				{
+					if (static_cast<uint32_t>(c) < fm_count)
+						dst[static_cast<size_t>(c) * plane] = v[c] * mult;
+				}
+			}
+			else
+			{
+				float m = softmax_max_init;
+				for(uint32_t c = 0; c < fm_count; ++c)
+					m = ref_max(m, src[static_cast<size_t>(c) * plane]);
+				float sum = 0.0f;
+				for(uint32_t c = 0; c < fm_count; ++c)
+				{
+					const float val = nnf_expf(src[static_cast<size_t>(c) * plane] - m, lds_exp);
+					sum += val;
+					dst[static_cast<size_t>(c) * plane] = val;
+				}
+				const float mult = 1.0f / sum;
+				for(uint32_t c = 0; c < fm_count; ++c)
+					dst[static_cast<size_t>(c) * plane] *= mult;
+			}
+		}
+
+		template<int THREADS, int W>
+		void launch_rows(hipStream_t stream, float* out, const float* in, uint32_t rows, uint32_t fm_count, uint32_t vectors_per_lane)
+		{
+			// one wavefront per workgroup while there are few rows (spreads them over the compute units)
+			const uint32_t block = (THREADS > wave_size) ? THREADS : ((rows >= 4096) ? 256 : wave_size);
+			const uint32_t rows_per_block = block / THREADS;
+			const dim3 grid((rows + rows_per_block - 1) / rows_per_block);
+			if (vectors_per_lane <= 1)
+				hipLaunchKernelGGL((softmax_rows_kernel<THREADS, 1, W>), grid, dim3(block), 0, stream, out, in, rows, fm_count);
+			else if (vectors_per_lane <= 2)
+				hipLaunchKernelGGL((softmax_rows_kernel<THREADS, 2, W>), grid, dim3(block), 0, stream, out, in, rows, fm_count);
+			else if (vectors_per_lane <= 4)
+				hipLaunchKernelGGL((softmax_rows_kernel<THREADS, 4, W>), grid, dim3(block), 0, stream, out, in, rows, fm_count);
+			else
+				hipLaunchKernelGGL((softmax_rows_kernel<THREADS, 8, W>), grid, dim3(block), 0, stream, out, in, rows, fm_count);
+		}
+
+		template<int W>
+		bool try_launch_rows(hipStream_t stream, float* out, const float* in, uint32_t rows, uint32_t fm_count)
+		{
+			const uint32_t vectors = (fm_count + W - 1) / W;
+			if (vectors <= wave_size * 8)
+			{
+				launch_rows<wave_size, W>(stream, out, in, rows, fm_count, (vectors + wave_size - 1) / wave_size);
+				return true;
+			}
+			if (vectors <= 1024 * 8)
+			{
+				launch_rows<1024, W>(stream, out, in, rows, fm_count, (vectors + 1023) / 1024);
+				return true;
+			}
+			return false;
+		}
+	}
+
+	int softmax_forward(hipStream_t stream, float* output, const float* input,
+		uint32_t entry_count, uint32_t feature_map_count, uint32_t neuron_count_per_feature_map)
+	{
+		if ((output == nullptr) || (input == nullptr) || (feature_map_count == 0) || (neuron_count_per_feature_map == 0))
+			return NNF_HIP_EINVAL;
+		const uint64_t total64 = static_cast<uint64_t>(entry_count) * feature_map_count * neuron_count_per_feature_map;
+		if (total64 == 0)
+			return NNF_HIP_OK;
+		if (total64 > 0xFFFF0000ull)
+			return NNF_HIP_ETOOBIG;
+		if (!is_aligned16(output) || !is_aligned16(input))
+			return NNF_HIP_EALIGN;
+		if (output != input)
+		{
+			const uintptr_t a = reinterpret_cast<uintptr_t>(output), b = reinterpret_cast<uintptr_t>(input);
+			const size_t bytes = static_cast<size_t>(total64) * sizeof(float);
+			if ((a < b + bytes) && (b < a + bytes))
+				return NNF_HIP_EOVERLAP;
+		}
+
+		if (neuron_count_per_feature_map == 1)
+		{
+			bool launched;
+			if ((feature_map_count % 4) == 0)
+				launched = try_launch_rows<4>(stream, output, input, entry_count, feature_map_count);
+			else
+				launched = try_launch_rows<1>(stream, output, input, entry_count, feature_map_count);
+			if (!launched)
+				hipLaunchKernelGGL(softmax_long_rows_kernel, dim3(entry_count), dim3(1024), 0, stream, output, input, feature_map_count);
+		}
+		else
+		{
+			const uint32_t columns = entry_count * neuron_count_per_feature_map;
+			const dim3 block(256);
+			const dim3 grid((columns + 255) / 256);
+			if (feature_map_count <= 16)
+				hipLaunchKernelGGL(softmax_columns_kernel<16>, grid, block, 0, stream, output, input, columns, feature_map_count, neuron_count_per_feature_map);
+			else
+				hipLaunchKernelGGL(softmax_columns_kernel<0>, grid, block, 0, stream, output, input, columns, feature_map_count, neuron_count_per_feature_map);
+		}
+		return launch_status();
+	}
+}

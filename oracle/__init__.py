@@ -1,0 +1,173 @@
+"""ctypes binding of the CPU oracle (oracle/nnf_oracle.c).
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, by __graft_entry__.smoke() and by bench.py's
+cpu_baseline leg as the checker / the timed baseline. Nothing under nnforge_amd/ imports it.
+All functions take and return numpy float32 arrays in nnForge's [entry][feature_map][y][x] layout.
+"""
+
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+ORACLE_DIR = os.path.dirname(os.path.abspath(__file__))
+LIBRARY = os.path.join(ORACLE_DIR, "libnnf_oracle.so")
+
+_lib = None
+_FP = ctypes.POINTER(ctypes.c_float)
+_UP = ctypes.POINTER(ctypes.c_uint)
+
+
+def build():
+    """Compiles oracle/nnf_oracle.c with the Makefile beside it."""
+    proc = subprocess.run(["make", "-C", ORACLE_DIR, "-B", "libnnf_oracle.so"], stdout=subprocess.PIPE,
+                          stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("oracle build failed:\n" + proc.stdout)
+    return LIBRARY
+
+
+def load():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIBRARY):
+            build()
+        lib = ctypes.CDLL(LIBRARY)
+        lib.nnf_oracle_max_threads.restype = ctypes.c_int
+        lib.nnf_oracle_average_subsampling_plain_mult.restype = ctypes.c_float
+        lib.nnf_oracle_average_subsampling_plain_mult.argtypes = [ctypes.c_uint, ctypes.c_uint, ctypes.c_int, ctypes.c_float]
+        lib.nnf_oracle_average_subsampling_full_mult.restype = ctypes.c_float
+        lib.nnf_oracle_average_subsampling_full_mult.argtypes = [ctypes.c_int, _UP, ctypes.c_uint, ctypes.c_uint, ctypes.c_int, ctypes.c_float]
+        lib.nnf_oracle_batch_norm.argtypes = [_FP, _FP, _FP, _FP, _FP, _FP, ctypes.c_uint, ctypes.c_uint, ctypes.c_uint, ctypes.c_int]
+        lib.nnf_oracle_rectified_linear.argtypes = [_FP, _FP, ctypes.c_float, ctypes.c_longlong, ctypes.c_int]
+        lib.nnf_oracle_parametric_rectified_linear.argtypes = [_FP, _FP, _FP, ctypes.c_uint, ctypes.c_uint, ctypes.c_uint, ctypes.c_int]
+        lib.nnf_oracle_exponential_linear.argtypes = [_FP, _FP, ctypes.c_longlong, ctypes.c_int]
+        lib.nnf_oracle_sigmoid.argtypes = [_FP, _FP, ctypes.c_longlong, ctypes.c_int]
+        lib.nnf_oracle_hyperbolic_tangent.argtypes = [_FP, _FP, ctypes.c_float, ctypes.c_float, ctypes.c_longlong, ctypes.c_int]
+        lib.nnf_oracle_add.argtypes = [_FP, ctypes.POINTER(_FP), ctypes.c_int, ctypes.c_float, ctypes.c_longlong, ctypes.c_int]
+        lib.nnf_oracle_softmax.argtypes = [_FP, _FP, ctypes.c_uint, ctypes.c_uint, ctypes.c_uint, ctypes.c_int]
+        lib.nnf_oracle_average_subsampling.argtypes = [_FP, _FP, ctypes.c_uint, ctypes.c_uint, ctypes.c_uint, ctypes.c_int,
+                                                       _UP, _UP, _UP, ctypes.c_uint, ctypes.c_uint, ctypes.c_float, ctypes.c_int]
+        _lib = lib
+    return _lib
+
+
+def max_threads():
+    return load().nnf_oracle_max_threads()
+
+
+def _f32(a):
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    return a
+
+
+def _ptr(a):
+    return a.ctypes.data_as(_FP)
+
+
+def _out_for(x, out):
+    if out is None:
+        return np.empty_like(x)
+    assert out.dtype == np.float32 and out.flags.c_contiguous and out.size == x.size
+    return out
+
+
+def _shape3(x):
+    """(entry_count, feature_map_count, neuron_count_per_feature_map) of an [N][C][...] array."""
+    n, c = x.shape[0], x.shape[1]
+    plane = int(np.prod(x.shape[2:], dtype=np.int64)) if x.ndim > 2 else 1
+    return n, c, plane
+
+
+def batch_norm(x, gamma, beta, mean, inverse_sigma, out=None, threads=0):
+    x = _f32(x)
+    n, c, plane = _shape3(x)
+    g, b, m, s = (_f32(v) for v in (gamma, beta, mean, inverse_sigma))
+    assert g.size == b.size == m.size == s.size == c
+    out = _out_for(x, out)
+    load().nnf_oracle_batch_norm(_ptr(out), _ptr(x), _ptr(g), _ptr(b), _ptr(m), _ptr(s), n, c, plane, threads)
+    return out
+
+
+def rectified_linear(x, negative_slope=0.0, out=None, threads=0):
+    x = _f32(x)
+    out = _out_for(x, out)
+    load().nnf_oracle_rectified_linear(_ptr(out), _ptr(x), negative_slope, x.size, threads)
+    return out
+
+
+def parametric_rectified_linear(x, slopes, out=None, threads=0):
+    x = _f32(x)
+    n, c, plane = _shape3(x)
+    a = _f32(slopes)
+    assert a.size == c
+    out = _out_for(x, out)
+    load().nnf_oracle_parametric_rectified_linear(_ptr(out), _ptr(x), _ptr(a), n, c, plane, threads)
+    return out
+
+
+def exponential_linear(x, out=None, threads=0):
+    x = _f32(x)
+    out = _out_for(x, out)
+    load().nnf_oracle_exponential_linear(_ptr(out), _ptr(x), x.size, threads)
+    return out
+
+
+def sigmoid(x, out=None, threads=0):
+    x = _f32(x)
+    out = _out_for(x, out)
+    load().nnf_oracle_sigmoid(_ptr(out), _ptr(x), x.size, threads)
+    return out
+
+
+def hyperbolic_tangent(x, scale=1.0, steepness=1.0, out=None, threads=0):
+    x = _f32(x)
+    out = _out_for(x, out)
+    load().nnf_oracle_hyperbolic_tangent(_ptr(out), _ptr(x), scale, steepness, x.size, threads)
+    return out
+
+
+def add(inputs, alpha=1.0, out=None, threads=0):
+    arrays = [_f32(a) for a in inputs]
+    assert all(a.size == arrays[0].size for a in arrays)
+    out = _out_for(arrays[0], out)
+    ptrs = (_FP * len(arrays))(*[_ptr(a) for a in arrays])
+    load().nnf_oracle_add(_ptr(out), ptrs, len(arrays), alpha, arrays[0].size, threads)
+    return out
+
+
+def softmax(x, out=None, threads=0):
+    x = _f32(x)
+    n, c, plane = _shape3(x)
+    out = _out_for(x, out)
+    load().nnf_oracle_softmax(_ptr(out), _ptr(x), n, c, plane, threads)
+    return out
+
+
+def average_subsampling(x, window_sizes, feature_map_window=1, entry_window=1, mult=None, alpha=None, threads=0):
+    """x: [N][C][d_last]...[d_0] (numpy order, x last). window_sizes: per spatial dimension in
+    nnForge order (x first). mult None: the plain tester's own multiplier (see the C file)."""
+    x = _f32(x)
+    dims = list(x.shape[2:])[::-1]  # nnForge order: x first
+    if not dims:
+        dims = [1]
+    window_sizes = list(window_sizes)
+    assert len(window_sizes) == len(dims)
+    out_dims = [d // w for d, w in zip(dims, window_sizes)]
+    n_out = x.shape[0] // entry_window
+    c_out = x.shape[1] // feature_map_window
+    if mult is None:
+        mult = load().nnf_oracle_average_subsampling_plain_mult(feature_map_window, entry_window, int(alpha is not None),
+                                                                 float(alpha or 0.0))
+    out = np.empty([n_out, c_out] + out_dims[::-1], dtype=np.float32)
+    arr = lambda v: (ctypes.c_uint * len(v))(*v)
+    load().nnf_oracle_average_subsampling(_ptr(out), _ptr(x), n_out, x.shape[1], c_out, len(dims), arr(dims), arr(out_dims),
+                                          arr(window_sizes), feature_map_window, entry_window, mult, threads)
+    return out
+
+
+def average_subsampling_full_mult(window_sizes, feature_map_window=1, entry_window=1, alpha=None):
+    w = list(window_sizes)
+    return load().nnf_oracle_average_subsampling_full_mult(len(w), (ctypes.c_uint * len(w))(*w), feature_map_window,
+                                                           entry_window, int(alpha is not None), float(alpha or 0.0))

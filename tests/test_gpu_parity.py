@@ -1,0 +1,421 @@
+"""GPU parity: the HIP kernels, called through the C ABI, against the CPU oracle on identical seeded inputs.
+
+Bars (BASELINE north_star): batch norm and element-wise layers within max(2 ULP, 1e-6 relative) of
+the plain CPU tester; softmax within 1e-5 relative. On top of that the tests demand what the
+design promises: bit-for-bit equality wherever the operation order is the reference's own (every
+kernel except the row softmax, whose sum is a tree instead of a left-to-right loop).
+"""
+
+import ctypes
+
+import numpy as np
+import pytest
+
+import nnf_testing as T
+import oracle
+from nnforge_amd import capi
+
+pytestmark = pytest.mark.gpu
+
+BN, RELU, PRELU, ELU, SIGMOID, TANH = (capi.OP_BATCH_NORM, capi.OP_RELU, capi.OP_PRELU, capi.OP_ELU,
+                                       capi.OP_SIGMOID, capi.OP_TANH)
+
+
+def oracle_chain(x, steps):
+    """Runs the oracle layer by layer the way forward_propagation_plain drives the testers."""
+    v = x
+    for step in steps:
+        v = step(v)
+    return v
+
+
+def check_exact(got, want, what):
+    got = np.asarray(got, dtype=np.float32).reshape(-1)
+    want = np.asarray(want, dtype=np.float32).reshape(-1)
+    T.assert_close_elementwise(got, want, ulps=2, rel=1e-6, what=what)
+    mism = T.bit_mismatches(got, want)
+    assert mism == 0, "%s: %d of %d elements differ in bits (max %d ulp)" % (
+        what, mism, got.size, int(T.ulp_distance(got, want).max()))
+
+
+# ---------------------------------------------------------------------------------------------
+# benchmark configurations at their real sizes
+# ---------------------------------------------------------------------------------------------
+
+def test_config0_bn_relu_full_size(gpu):
+    n, c, h, w = 32, 64, 56, 56
+    x = T.normal(T.rng(0, 0), (n, c, h, w))
+    g, b, m, s = T.bn_params(T.rng(0, 1), c)
+    want = oracle.rectified_linear(oracle.batch_norm(x, g, b, m, s), 0.0)
+    got = gpu.chain((n, c, h * w), [[(BN, 0)]], [(RELU, 0, 0.0)], [x], [g, b, m, s])
+    check_exact(got, want, "config 0")
+    # -0.0 for negative pre-activations, as x * 0.0F gives in the reference
+    assert np.signbit(got[(want.reshape(-1) == 0)]).any()
+
+
+def test_config2_bn_add_prelu_full_size(gpu):
+    n, c, h, w = 128, 256, 56, 56
+    main = T.normal(T.rng(2, 0), (n, c, h, w))
+    residual = T.normal(T.rng(2, 1), (n, c, h, w))
+    g, b, m, s = T.bn_params(T.rng(2, 2), c)
+    slopes = T.uniform(T.rng(2, 3), c, 0.0, 0.25)
+    bn = oracle.batch_norm(main, g, b, m, s)
+    want = oracle.parametric_rectified_linear(oracle.add([residual, bn]), slopes)
+    del bn
+    # Add's inputs in schema order: [residual, batch-normed main path]
+    got = gpu.chain((n, c, h * w), [[], [(BN, 0)]], [(PRELU, 4)], [residual, main], [g, b, m, s, slopes])
+    check_exact(got, want, "config 2")
+
+
+def config3_input(shape):
+    gen = T.rng(3, 0)
+    x = T.normal(gen, shape, 2.0)
+    spikes = gen.random(shape) < 0.001
+    signs = np.where(gen.random(shape) < 0.5, np.float32(-50.0), np.float32(50.0))
+    return np.where(spikes, signs, x).astype(np.float32)
+
+
+def test_config3_activation_chain_full_size(gpu):
+    n, c, h, w = 64, 512, 28, 28
+    x = config3_input((n, c, h, w))
+    g, b, m, s = T.bn_params(T.rng(3, 1), c)
+    want = oracle_chain(x, [
+        lambda v: oracle.batch_norm(v, g, b, m, s),
+        oracle.exponential_linear,
+        oracle.sigmoid,
+        lambda v: oracle.hyperbolic_tangent(v, T.TANH_SCALE, T.TANH_STEEPNESS)])
+    got = gpu.chain((n, c, h * w), [[(BN, 0), (ELU,), (SIGMOID,), (TANH, 0, T.TANH_SCALE, T.TANH_STEEPNESS)]], [], [x], [g, b, m, s])
+    T.assert_close_elementwise(got, want.reshape(-1), 2, 1e-6, "config 3")
+    mism = T.bit_mismatches(got, want.reshape(-1))
+    print("config 3: %d of %d elements differ in bits from the oracle" % (mism, got.size))
+    assert mism == 0
+
+
+def config1_input(n, c):
+    gen = T.rng(1, 0)
+    x = T.normal(gen, (n, c), 4.0)
+    return np.where(gen.random((n, c)) < 0.01, np.float32(30.0), x).astype(np.float32)
+
+
+def run_softmax(gpu, x3, in_place=False, expect=0):
+    n, c, plane = x3.shape
+    d_in = gpu.to_device(x3)
+    d_out = d_in if in_place else gpu.torch.full((x3.size,), float("nan"), dtype=gpu.torch.float32, device=gpu.device)
+    rc = gpu.lib.nnf_hip_softmax_forward(gpu.stream, d_out.data_ptr(), d_in.data_ptr(), n, c, plane)
+    assert rc == expect, capi.error_string(rc)
+    return gpu.to_host(d_out, x3.shape)
+
+
+def assert_softmax_close(got, want, what):
+    """1e-5 relative (north_star); an absolute floor of one denormal step covers flushed tails."""
+    err = np.abs(got.astype(np.float64) - want.astype(np.float64))
+    tol = 1e-5 * np.abs(want.astype(np.float64)) + 1e-45
+    bad = ~(err <= tol) & ~(np.isnan(got) & np.isnan(want))
+    assert not bad.any(), "%s: %d elements outside 1e-5 relative, worst %g" % (
+        what, int(bad.sum()), float((err / np.maximum(np.abs(want), 1e-300)).max()))
+
+
+def test_config1_softmax_full_size(gpu):
+    n, c = 256, 1000
+    x = config1_input(n, c).reshape(n, c, 1)
+    want = oracle.softmax(x)
+    got = run_softmax(gpu, x)
+    assert_softmax_close(got, want, "config 1")
+    # rows sum to one within C * 2^-24 and the exponentials themselves are the oracle's bit for bit:
+    # value / row-multiplier reproduces them up to the last place
+    assert np.abs(got.astype(np.float64).sum(axis=1) - 1.0).max() < c * 2.0 ** -24
+    worst = float((np.abs(got.astype(np.float64) - want) / want.astype(np.float64)).max())
+    print("config 1: worst relative difference from the oracle %.3g" % worst)
+    assert worst < 2e-6
+
+
+# ---------------------------------------------------------------------------------------------
+# every fused group shape of the ResNet-50 stack (config 4), reduced entry count
+# ---------------------------------------------------------------------------------------------
+
+RESNET_SHAPES = [(64, 112), (64, 56), (128, 56), (128, 28), (256, 28), (256, 14), (512, 14), (512, 7),
+                 (256, 56), (512, 28), (1024, 14), (2048, 7)]
+
+
+@pytest.mark.parametrize("c,hw", RESNET_SHAPES)
+def test_resnet_group_shapes(gpu, c, hw):
+    n = 3
+    gen = T.rng(4, c * 1000 + hw)
+    x = T.normal(gen, (n, c, hw, hw))
+    r = T.normal(gen, (n, c, hw, hw))
+    g, b, m, s = T.bn_params(gen, c)
+    g2, b2, m2, s2 = T.bn_params(gen, c)
+    bn = oracle.batch_norm(x, g, b, m, s)
+    # BN + ReLU
+    got = gpu.chain((n, c, hw * hw), [[(BN, 0)]], [(RELU, 0, 0.0)], [x], [g, b, m, s])
+    check_exact(got, oracle.rectified_linear(bn), "BN+ReLU %dx%d^2" % (c, hw))
+    # BN + Add(residual) + ReLU, Add inputs = [residual, BN(main)]
+    got = gpu.chain((n, c, hw * hw), [[], [(BN, 0)]], [(RELU, 0, 0.0)], [r, x], [g, b, m, s])
+    check_exact(got, oracle.rectified_linear(oracle.add([r, bn])), "BN+Add+ReLU %dx%d^2" % (c, hw))
+    # BN(shortcut) + BN(main) + Add + ReLU
+    bn2 = oracle.batch_norm(r, g2, b2, m2, s2)
+    got = gpu.chain((n, c, hw * hw), [[(BN, 4)], [(BN, 0)]], [(RELU, 0, 0.0)], [r, x], [g, b, m, s, g2, b2, m2, s2])
+    check_exact(got, oracle.rectified_linear(oracle.add([bn2, bn])), "BN+BN+Add+ReLU %dx%d^2" % (c, hw))
+
+
+# ---------------------------------------------------------------------------------------------
+# single-layer entry points, awkward shapes, special values
+# ---------------------------------------------------------------------------------------------
+
+SPECIALS = np.array([0.0, -0.0, 1.0, -1.0, np.inf, -np.inf, np.nan, 1e-45, -1e-45, 1e-38, -1e-38, 1.1754944e-38,
+                     3.4028235e38, -3.4028235e38, 50.0, -50.0, 88.0, 88.7, 88.72, 88.73, 89.0, -87.0, -88.0, -103.0,
+                     -103.9, -103.97, -103.98, -104.0, -150.0, 1e-6, -1e-6, 0.5, -0.5, 17.0, -17.0, 30.0, -30.0],
+                    dtype=np.float32)
+
+
+def awkward_input(shape, seed):
+    gen = T.rng(9, seed)
+    x = T.normal(gen, shape, 4.0)
+    flat = x.reshape(-1)
+    k = min(flat.size, SPECIALS.size)
+    pos = gen.permutation(flat.size)[:k]
+    flat[pos] = SPECIALS[:k]
+    return x
+
+
+AWKWARD_SHAPES = [(1, 1, 1), (1, 1, 3), (2, 3, 1), (1, 5, 2), (3, 7, 3), (2, 3, 49), (5, 13, 49), (1, 3, 5 * 5), (2, 2, 4),
+                  (1, 64, 4097), (3, 5, 1023), (2, 4100, 1), (7, 3, 3136), (1, 2, 20000), (4, 1, 12544)]
+
+
+@pytest.mark.parametrize("shape", AWKWARD_SHAPES)
+def test_batch_norm_entry_point_awkward_shapes(gpu, shape):
+    n, c, plane = shape
+    x = awkward_input(shape, 1)
+    g, b, m, s = T.bn_params(T.rng(9, 2), c)
+    d_x = gpu.to_device(x)
+    d_p = [gpu.to_device(v) for v in (g, b, m, s)]
+    d_out = gpu.torch.full((x.size,), float("nan"), dtype=gpu.torch.float32, device=gpu.device)
+    rc = gpu.lib.nnf_hip_batch_norm_forward(gpu.stream, d_out.data_ptr(), d_x.data_ptr(), *[t.data_ptr() for t in d_p], n, c, plane)
+    assert rc == 0, capi.error_string(rc)
+    check_exact(gpu.to_host(d_out), oracle.batch_norm(x, g, b, m, s), "batch_norm %s" % (shape,))
+
+
+@pytest.mark.parametrize("shape", AWKWARD_SHAPES)
+def test_prelu_entry_point_awkward_shapes(gpu, shape):
+    n, c, plane = shape
+    x = awkward_input(shape, 3)
+    a = T.uniform(T.rng(9, 4), c, -0.5, 0.5)
+    d_x, d_a = gpu.to_device(x), gpu.to_device(a)
+    d_out = gpu.torch.full((x.size,), float("nan"), dtype=gpu.torch.float32, device=gpu.device)
+    rc = gpu.lib.nnf_hip_parametric_rectified_linear_forward(gpu.stream, d_out.data_ptr(), d_x.data_ptr(), d_a.data_ptr(), n, c, plane)
+    assert rc == 0, capi.error_string(rc)
+    check_exact(gpu.to_host(d_out), oracle.parametric_rectified_linear(x, a), "prelu %s" % (shape,))
+
+
+FLAT_SIZES = [1, 2, 3, 4, 5, 63, 64, 65, 1023, 1024, 1025, 4095, 4096, 4097, 100003, 1 << 20]
+
+
+def run_flat(gpu, fn, x, *args, in_place=False):
+    d_x = gpu.to_device(x)
+    d_out = d_x if in_place else gpu.torch.full((x.size,), float("nan"), dtype=gpu.torch.float32, device=gpu.device)
+    rc = fn(gpu.stream, d_out.data_ptr(), d_x.data_ptr(), *args, x.size)
+    assert rc == 0, capi.error_string(rc)
+    return gpu.to_host(d_out)
+
+
+@pytest.mark.parametrize("size", FLAT_SIZES)
+def test_flat_activation_entry_points(gpu, size):
+    x = awkward_input((size,), size)
+    lib = gpu.lib
+    for slope in (0.0, 0.1, -2.0):
+        check_exact(run_flat(gpu, lib.nnf_hip_rectified_linear_forward, x, slope), oracle.rectified_linear(x, slope), "relu slope %g" % slope)
+    check_exact(run_flat(gpu, lib.nnf_hip_exponential_linear_forward, x), oracle.exponential_linear(x), "elu")
+    check_exact(run_flat(gpu, lib.nnf_hip_sigmoid_forward, x), oracle.sigmoid(x), "sigmoid")
+    for scale, steep in ((1.0, 1.0), (T.TANH_SCALE, T.TANH_STEEPNESS), (1.7159, 0.666666)):
+        check_exact(run_flat(gpu, lib.nnf_hip_hyperbolic_tangent_forward, x, scale, steep),
+                    oracle.hyperbolic_tangent(x, scale, steep), "tanh %g %g" % (scale, steep))
+    # in place, as every tester on the path allows
+    check_exact(run_flat(gpu, lib.nnf_hip_sigmoid_forward, x, in_place=True), oracle.sigmoid(x), "sigmoid in place")
+
+
+def test_expf_dense_sweep_through_elu_and_sigmoid(gpu):
+    """Every fp32 in a few dense bit-pattern windows plus a coarse sweep of all negative floats:
+    expf on the device is the oracle's expf bit for bit."""
+    windows = []
+    for start in (np.float32(-1e-3), np.float32(-0.7), np.float32(-12.0), np.float32(-87.3), np.float32(-103.5)):
+        first = int(np.array(start, dtype=np.float32).view(np.uint32))
+        windows.append(np.arange(first, first + (1 << 18), dtype=np.uint32))
+    windows.append(np.arange(0x80000000, 0xFF800000, 4099, dtype=np.uint32))  # all negative floats, strided
+    x = np.concatenate(windows).view(np.float32)
+    check_exact(run_flat(gpu, gpu.lib.nnf_hip_exponential_linear_forward, x), oracle.exponential_linear(x), "elu sweep")
+    check_exact(run_flat(gpu, gpu.lib.nnf_hip_sigmoid_forward, x), oracle.sigmoid(x), "sigmoid sweep (negative)")
+    check_exact(run_flat(gpu, gpu.lib.nnf_hip_sigmoid_forward, -x), oracle.sigmoid(-x), "sigmoid sweep (positive)")
+
+
+@pytest.mark.parametrize("input_count", [1, 2, 3, 4, 5, 8, 9])
+@pytest.mark.parametrize("size,alpha", [(5, 1.0), (4099, 0.5), (1 << 18, -1.25)])
+def test_add_entry_point(gpu, input_count, size, alpha):
+    gen = T.rng(10, input_count * 31 + size)
+    xs = [T.normal(gen, (size,), 3.0) for _ in range(input_count)]
+    for x in xs:  # signed zeros meet in the sum
+        x[:: max(1, size // 7)] = -0.0
+    d_in = [gpu.to_device(x) for x in xs]
+    d_out = gpu.torch.full((size,), float("nan"), dtype=gpu.torch.float32, device=gpu.device)
+    ptrs = capi.pointer_array([t.data_ptr() for t in d_in])
+    rc = gpu.lib.nnf_hip_add_forward(gpu.stream, d_out.data_ptr(), ptrs, input_count, alpha, size)
+    assert rc == 0, capi.error_string(rc)
+    check_exact(gpu.to_host(d_out), oracle.add(xs, alpha), "add k=%d" % input_count)
+
+
+def test_fused_equals_unfused_bitwise(gpu):
+    """A fused group is the same arithmetic as its layers launched one by one."""
+    n, c, plane = 4, 24, 196
+    gen = T.rng(11, 0)
+    x = T.normal(gen, (n, c, plane), 2.0)
+    r = T.normal(gen, (n, c, plane))
+    g, b, m, s = T.bn_params(gen, c)
+    a = T.uniform(gen, c, 0.0, 0.25)
+    fused = gpu.chain((n, c, plane), [[], [(BN, 0), (ELU,)]], [(PRELU, 4), (SIGMOID,), (TANH, 0, 1.7159, 0.6666)], [r, x], [g, b, m, s, a], alpha=0.5)
+    v = gpu.chain((n, c, plane), [[(BN, 0)]], [], [x], [g, b, m, s])
+    v = gpu.chain((n, c, plane), [[(ELU,)]], [], [v])
+    v = gpu.chain((n, c, plane), [[], []], [], [r, v.reshape(n, c, plane)], alpha=0.5)
+    v = gpu.chain((n, c, plane), [[(PRELU, 0)]], [], [v], [a])
+    v = gpu.chain((n, c, plane), [[(SIGMOID,)]], [], [v])
+    v = gpu.chain((n, c, plane), [[(TANH, 0, 1.7159, 0.6666)]], [], [v])
+    assert T.bit_mismatches(fused, v) == 0
+    want = oracle.hyperbolic_tangent(oracle.sigmoid(oracle.parametric_rectified_linear(
+        oracle.add([r, oracle.exponential_linear(oracle.batch_norm(x, g, b, m, s))], 0.5), a)), 1.7159, 0.6666)
+    check_exact(fused, want, "fused group")
+
+
+def test_in_place_group(gpu):
+    n, c, plane = 2, 8, 49
+    gen = T.rng(12, 0)
+    x = T.normal(gen, (n, c, plane))
+    r = T.normal(gen, (n, c, plane))
+    g, b, m, s = T.bn_params(gen, c)
+    want = oracle.rectified_linear(oracle.add([oracle.batch_norm(x, g, b, m, s), r]))
+    got = gpu.chain((n, c, plane), [[(BN, 0)], []], [(RELU, 0, 0.0)], [x, r], [g, b, m, s], in_place=True)
+    check_exact(got, want, "in-place group")
+
+
+def test_identity_batch_norm_and_zero_entries(gpu):
+    x = awkward_input((2, 5, 33), 5)
+    one, zero = np.ones(5, np.float32), np.zeros(5, np.float32)
+    got = gpu.chain((2, 5, 33), [[(BN, 0)]], [], [x], [one, zero, zero, one])
+    # identity parameters: x * 1 + 0 (signed zero aside, -0 + 0 = +0, as in the reference)
+    check_exact(got, oracle.batch_norm(x, one, zero, zero, one), "identity BN")
+    # zero entries: nothing is launched, nothing is touched
+    d = gpu.to_device(np.full(8, 7.0, np.float32))
+    desc = capi.make_desc(0, 5, 33, [[(RELU, 0, 0.0)]])
+    ins = capi.pointer_array([d.data_ptr()])
+    assert gpu.lib.nnf_hip_chain_forward(gpu.stream, ctypes.byref(desc), d.data_ptr(), ins, None) == 0
+    assert (gpu.to_host(d) == 7.0).all()
+
+
+def test_argument_errors(gpu):
+    lib = gpu.lib
+    d = gpu.to_device(np.zeros(64, np.float32))
+    e = gpu.to_device(np.zeros(64, np.float32))
+    base = d.data_ptr()
+    s = gpu.stream
+    assert lib.nnf_hip_rectified_linear_forward(s, base + 4, base + 64, 0.0, 8) == capi.E_ALIGN
+    assert lib.nnf_hip_rectified_linear_forward(s, base + 16, base, 0.0, 8) == capi.E_OVERLAP
+    assert lib.nnf_hip_rectified_linear_forward(s, None, base, 0.0, 8) == capi.E_INVAL
+    assert lib.nnf_hip_rectified_linear_forward(s, base, base, 0.0, 1 << 33) == capi.E_TOOBIG
+    desc = capi.make_desc(1, 4, 4, [[], []], has_add=False)
+    ins = capi.pointer_array([d.data_ptr(), e.data_ptr()])
+    assert lib.nnf_hip_chain_forward(s, ctypes.byref(desc), d.data_ptr(), ins, None) == capi.E_INVAL
+    desc = capi.make_desc(1, 4, 4, [[(BN, 0)]])
+    assert lib.nnf_hip_chain_forward(s, ctypes.byref(desc), d.data_ptr(), ins, None) == capi.E_INVAL  # BN without chunks
+    desc = capi.make_desc(1, 4, 4, [[(99,)]])
+    assert lib.nnf_hip_chain_forward(s, ctypes.byref(desc), d.data_ptr(), ins, None) == capi.E_INVAL
+    # second input overlapping the output
+    desc = capi.make_desc(1, 4, 4, [[], []])
+    ins = capi.pointer_array([e.data_ptr(), d.data_ptr()])
+    assert lib.nnf_hip_chain_forward(s, ctypes.byref(desc), d.data_ptr(), ins, None) == capi.E_OVERLAP
+    assert lib.nnf_hip_softmax_forward(s, base, base + 16, 1, 8, 1) == capi.E_OVERLAP
+    assert lib.nnf_hip_average_subsampling_forward(s, e.data_ptr(), d.data_ptr(), 1, 1, 4, 4, 5, 2, 1.0) == capi.E_INVAL
+    assert b"aligned" in lib.nnf_hip_error_string(capi.E_ALIGN)
+    gpu.torch.cuda.synchronize()
+
+
+# ---------------------------------------------------------------------------------------------
+# softmax
+# ---------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("n,c", [(1, 1), (3, 2), (5, 3), (2, 4), (7, 10), (4, 64), (9, 255), (3, 256), (2, 257), (5, 1000), (64, 1000),
+                                 (3, 1001), (2, 2048), (2, 2049), (3, 4096), (2, 8200), (2, 32768), (1, 40000), (2, 33001), (5000, 12)])
+def test_softmax_rows(gpu, n, c):
+    gen = T.rng(13, n * 100000 + c)
+    x = T.normal(gen, (n, c, 1), 4.0)
+    x[gen.random((n, c, 1)) < 0.01] = 30.0
+    want = oracle.softmax(x)
+    got = run_softmax(gpu, x)
+    assert_softmax_close(got, want, "softmax rows %dx%d" % (n, c))
+    got2 = run_softmax(gpu, x, in_place=True)
+    assert T.bit_mismatches(got, got2) == 0
+
+
+@pytest.mark.parametrize("n,c,plane", [(2, 3, 2), (1, 10, 49), (3, 16, 5), (2, 17, 64), (2, 21, 1000), (1, 150, 333), (4, 5, 4096)])
+def test_softmax_columns_bit_exact(gpu, n, c, plane):
+    gen = T.rng(14, n * 100000 + c * 100 + plane)
+    x = T.normal(gen, (n, c, plane), 4.0)
+    x[gen.random((n, c, plane)) < 0.01] = 30.0
+    want = oracle.softmax(x)
+    got = run_softmax(gpu, x)
+    assert_softmax_close(got, want, "softmax columns")
+    assert T.bit_mismatches(got, want) == 0  # same left-to-right sum as the reference
+    assert T.bit_mismatches(run_softmax(gpu, x, in_place=True), want) == 0
+
+
+def test_softmax_special_rows(gpu):
+    c = 100
+    rows = np.zeros((7, c, 1), np.float32)
+    rows[0] = 5.0                      # uniform -> exactly 1/C up to rounding
+    rows[1, 3] = np.nan                # NaN poisons the row (max skips it, expf does not)
+    rows[2] = -3.0e38                  # below the -1e37 start value of the max: sum 0 -> 0 * inf = NaN
+    rows[3, 7] = 30.0                  # one-hot limit
+    rows[4] = np.linspace(-80, 80, c, dtype=np.float32).reshape(c, 1)
+    rows[5] = rows[4] + 1000.0         # shift invariance
+    rows[6, 0] = np.inf                # inf - inf = NaN at the maximum
+    want = oracle.softmax(rows)
+    got = run_softmax(gpu, rows)
+    assert_softmax_close(got, want, "softmax special rows")
+    assert np.isnan(got[1]).all() and np.isnan(got[2]).all()
+    assert abs(float(got[0, 0, 0]) - 1.0 / c) < 1e-9
+    assert got[3, 7, 0] > 0.999999
+    assert T.ulp_distance(got[4], got[5]).max() <= 2  # the shift moves every exponent argument by the same amount
+    cols = np.repeat(rows.transpose(2, 1, 0), 3, axis=0).copy()  # the same data laid out as columns
+    assert T.bit_mismatches(run_softmax(gpu, cols), oracle.softmax(cols)) == 0
+
+
+# ---------------------------------------------------------------------------------------------
+# average subsampling
+# ---------------------------------------------------------------------------------------------
+
+def run_pool(gpu, x, ww, wh, mult, expect=0):
+    n, c, h, w = x.shape
+    d_in = gpu.to_device(x)
+    out_shape = (n, c, h // wh, w // ww)
+    d_out = gpu.torch.full((int(np.prod(out_shape)),), float("nan"), dtype=gpu.torch.float32, device=gpu.device)
+    rc = gpu.lib.nnf_hip_average_subsampling_forward(gpu.stream, d_out.data_ptr(), d_in.data_ptr(), n, c, w, h, ww, wh, mult)
+    assert rc == expect, capi.error_string(rc)
+    return gpu.to_host(d_out, out_shape)
+
+
+@pytest.mark.parametrize("n,c", [(64, 2048), (3, 5), (1, 1), (2, 300)])
+def test_global_average_7x7(gpu, n, c):
+    x = T.normal(T.rng(15, n + c), (n, c, 7, 7))
+    plain_mult = 1.0  # what the plain tester uses when the schema sets no alpha: the window SUM
+    full_mult = oracle.average_subsampling_full_mult([7, 7])  # 1/49, the CUDA tester's / explicit alpha
+    for mult in (plain_mult, full_mult):
+        want = oracle.average_subsampling(x, [7, 7], mult=mult)
+        got = run_pool(gpu, x, 7, 7, mult)
+        assert T.bit_mismatches(got, want) == 0
+
+
+@pytest.mark.parametrize("shape,ww,wh", [((2, 3, 8, 8), 2, 2), ((1, 4, 9, 7), 3, 2), ((2, 2, 6, 10), 5, 3), ((1, 2, 4, 4), 4, 4),
+                                         ((3, 3, 5, 12), 12, 5), ((1, 1, 30, 30), 30, 30), ((2, 5, 16, 16), 1, 1), ((1, 3, 7, 9), 2, 3)])
+def test_average_subsampling_windows(gpu, shape, ww, wh):
+    x = T.normal(T.rng(16, sum(shape) + ww), shape)
+    mult = oracle.average_subsampling_full_mult([ww, wh])
+    want = oracle.average_subsampling(x, [ww, wh], mult=mult)
+    got = run_pool(gpu, x, ww, wh, mult)
+    assert got.shape == want.shape
+    assert T.bit_mismatches(got, want) == 0
