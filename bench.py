@@ -1,0 +1,383 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused element-wise inference path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload config0|...|config4] [--only]
+
+A step is one pass of the hot path over one batch of synthetic input that is already resident in
+HBM. The headline workload is the configuration the metric is quoted on: batch_norm ->
+rectified_linear, fp32, N=32 C=64 56x56 (config 0). Its tensors (51 MB per step) would fit the
+256 MB last-level cache, so the steps rotate through buffer sets totalling > 800 MB: every step
+reads from and writes to HBM. The other configurations are timed with fewer steps and reported
+under "per_config" on the same JSON line.
+
+Prints ONE JSON line. `value` = algorithmic bytes per step / wall time per step (GB/s), where the
+wall time brackets exactly K steps with a device synchronisation on both sides. `roofline` is
+measured with HIP events on the launch stream around the same K steps. `cpu_baseline` is the CPU
+restatement of nnForge's plain backend (oracle/, layer by layer, unfused, OpenMP on all host
+cores) timed in this process on the same workload.
+"""
+
+import argparse
+import ctypes
+import json
+import statistics
+import sys
+import time
+
+import numpy as np
+
+HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
+METRIC = "achieved HBM GB/s (% of MI355X peak) + elements/s, fused BN+ReLU fp32 fwd"
+SEED = 0x6E6E4600
+
+# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
+# (see profiles/); None until measured for a workload.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def fail(msg, code=2):
+    sys.stderr.write(msg + "\n")
+    sys.exit(code)
+
+
+class Runner:
+    """Device buffers (allocated through torch) and prepared C-ABI argument blocks."""
+
+    def __init__(self):
+        import torch
+        from nnforge_amd import capi
+
+        self.torch = torch
+        self.capi = capi
+        self.lib = capi.load()  # raises if the HIP library has not been built: no fallback
+        if not torch.cuda.is_available():
+            fail("bench.py needs a GPU: torch.cuda.is_available() is False")
+        torch.cuda.set_device(0)
+        self.device = torch.device("cuda:0")
+        self.stream = torch.cuda.current_stream().cuda_stream
+        self.gen = torch.Generator(device=self.device)
+        self.gen.manual_seed(SEED)
+        self.events = []
+
+    def randn(self, count, std=1.0):
+        t = self.torch.randn(count, generator=self.gen, device=self.device, dtype=self.torch.float32)
+        if std != 1.0:
+            t.mul_(std)
+        return t
+
+    def empty(self, count):
+        return self.torch.empty(count, device=self.device, dtype=self.torch.float32)
+
+    def bn_chunks(self, c):
+        t = self.torch
+        gamma = t.rand(c, generator=self.gen, device=self.device) + 0.5
+        beta = self.randn(c, 0.1 ** 0.5)
+        mean = self.randn(c, 0.1 ** 0.5)
+        var = t.rand(c, generator=self.gen, device=self.device) * 1.5 + 0.5
+        inv_sigma = 1.0 / t.sqrt(var + 1e-5)
+        return [gamma, beta, mean, inv_sigma]
+
+    def event(self):
+        p = ctypes.c_void_p()
+        self.capi.check(self.lib.nnf_hip_event_create(ctypes.byref(p)))
+        self.events.append(p)
+        return p
+
+    def sync(self):
+        self.torch.cuda.synchronize()
+
+    def prepare_group(self, group, sets):
+        """Allocates `sets` rotating buffer sets for a fused group; returns a launch closure."""
+        from nnforge_amd import workloads as w
+
+        capi = self.capi
+        total = w.group_elements(group)
+        chunks = []
+        for kind, c in group.chunks:
+            if kind == "bn":
+                chunks += self.bn_chunks(c)
+            else:
+                chunks.append(self.torch.rand(c, generator=self.gen, device=self.device) * 0.25)
+        desc = capi.make_desc(group.entry_count, group.feature_map_count, group.plane, group.arms, group.tail)
+        chunk_ptrs = capi.pointer_array([t.data_ptr() for t in chunks])
+        keep = [chunks]
+        calls = []
+        for _ in range(sets):
+            ins = [self.randn(total) for _ in group.arms]
+            out = self.empty(total)
+            keep.append((ins, out))
+            calls.append((out.data_ptr(), capi.pointer_array([t.data_ptr() for t in ins])))
+        fn = self.lib.nnf_hip_chain_forward
+        stream = self.stream
+        desc_ref = ctypes.byref(desc)
+
+        def launch(i):
+            out_ptr, in_ptrs = calls[i % sets]
+            rc = fn(stream, desc_ref, out_ptr, in_ptrs, chunk_ptrs)
+            if rc != 0:
+                raise RuntimeError(capi.error_string(rc))
+
+        launch.keep = (keep, desc, chunk_ptrs, calls)
+        return launch
+
+    def time_steps(self, step, steps, warmup):
+        """Returns (wall seconds per step, event seconds per step) for exactly `steps` steps."""
+        lib = self.lib
+        for i in range(warmup):
+            step(i)
+        e0, e1 = self.event(), self.event()
+        self.sync()
+        t0 = time.perf_counter()
+        lib.nnf_hip_event_record(e0, self.stream)
+        for i in range(steps):
+            step(warmup + i)
+        lib.nnf_hip_event_record(e1, self.stream)
+        self.sync()
+        t1 = time.perf_counter()
+        ms = ctypes.c_float()
+        self.capi.check(lib.nnf_hip_event_elapsed_ms(ctypes.byref(ms), e0, e1))
+        return (t1 - t0) / steps, ms.value * 1e-3 / steps
+
+
+def result_entry(name, alg_bytes, elements, wall_s, event_s, launches, extra=None):
+    entry = {
+        "workload": name,
+        "algorithmic_bytes_per_step": alg_bytes,
+        "elements_per_step": elements,
+        "launches_per_step": launches,
+        "ms_per_step": wall_s * 1e3,
+        "gbps": alg_bytes / wall_s / 1e9,
+        "pct_of_hbm_peak": 100.0 * alg_bytes / wall_s / 1e9 / HBM_PEAK_GBPS,
+        "elements_per_s": elements / wall_s,
+        "event_ms_per_step": event_s * 1e3,
+        "event_gbps": alg_bytes / event_s / 1e9,
+    }
+    if extra:
+        entry.update(extra)
+    return entry
+
+
+def rotation_sets(bytes_per_set, minimum_total=768 << 20, cap=32):
+    return int(max(2, min(cap, -(-minimum_total // bytes_per_set))))
+
+
+def bench_group(runner, label, group, steps, warmup):
+    from nnforge_amd import workloads as w
+
+    alg = w.group_algorithmic_bytes(group)
+    sets = rotation_sets(alg)
+    launch = runner.prepare_group(group, sets)
+    wall, ev = runner.time_steps(launch, steps, warmup)
+    entry = result_entry(label, alg, w.group_elements(group), wall, ev, 1,
+                         {"buffer_sets": sets, "shape": [group.entry_count, group.feature_map_count, group.plane]})
+    del launch
+    runner.torch.cuda.empty_cache()
+    return entry
+
+
+def bench_softmax(runner, steps, warmup):
+    from nnforge_amd import workloads as w
+
+    n, c, plane = w.CONFIG1_SHAPE
+    total = n * c * plane
+    sets = 64
+    ins = [runner.randn(total, 2.0) for _ in range(sets)]
+    for t in ins:
+        spikes = runner.torch.rand(total, generator=runner.gen, device=runner.device) < 0.01
+        t[spikes] = 30.0
+    outs = [runner.empty(total) for _ in range(sets)]
+    ptrs = [(o.data_ptr(), i.data_ptr()) for o, i in zip(outs, ins)]
+    fn, stream = runner.lib.nnf_hip_softmax_forward, runner.stream
+
+    def launch(i):
+        o, x = ptrs[i % sets]
+        rc = fn(stream, o, x, n, c, plane)
+        if rc != 0:
+            raise RuntimeError(runner.capi.error_string(rc))
+
+    wall, ev = runner.time_steps(launch, steps, warmup)
+    return result_entry("config1: softmax over feature maps N=256 C=1000 1x1", 2 * 4 * total, total, wall, ev, 1,
+                        {"buffer_sets": sets, "note": "2 MB per step: launch latency, not bandwidth, bounds this shape"})
+
+
+def bench_resnet50(runner, steps, warmup, n=64):
+    from nnforge_amd import workloads as w
+
+    groups = w.resnet50_groups(n)
+    launches = [runner.prepare_group(g, 1) for g in groups]
+    pool_shape, sm_shape = w.resnet50_tail(n)
+    pool_in = runner.randn(int(np.prod(pool_shape)))
+    pool_out = runner.empty(pool_shape[0] * pool_shape[1])
+    sm_in = runner.randn(sm_shape[0] * sm_shape[1], 2.0)
+    sm_out = runner.empty(sm_shape[0] * sm_shape[1])
+    lib, stream = runner.lib, runner.stream
+    pool_mult = 1.0 / 49.0
+
+    def step(i):
+        for launch in launches:
+            launch(0)
+        rc = lib.nnf_hip_average_subsampling_forward(stream, pool_out.data_ptr(), pool_in.data_ptr(), pool_shape[0], pool_shape[1], 7, 7, 7, 7, pool_mult)
+        rc |= lib.nnf_hip_softmax_forward(stream, sm_out.data_ptr(), sm_in.data_ptr(), sm_shape[0], sm_shape[1], 1)
+        if rc != 0:
+            raise RuntimeError("tail launch failed: %d" % rc)
+
+    wall, ev = runner.time_steps(step, steps, warmup)
+    g_bytes, p_bytes, s_bytes = w.resnet50_algorithmic_bytes(n)
+    elements = sum(w.group_elements(g) for g in groups) + pool_shape[0] * pool_shape[1] + sm_shape[0] * sm_shape[1]
+    entry = result_entry("config4: ResNet-50 post-convolution stack N=%d (49 fused groups + 7x7 average + softmax)" % n,
+                         g_bytes + p_bytes + s_bytes, elements, wall, ev, len(groups) + 2)
+    del launches
+    runner.torch.cuda.empty_cache()
+    return entry
+
+
+def bench_copy(runner, steps, warmup):
+    """Plain float4 copy kernel of the same launch shape: the yardstick for what HBM delivers."""
+    count = (256 << 20) // 4
+    sets = 4
+    src = [runner.randn(count) for _ in range(sets)]
+    dst = [runner.empty(count) for _ in range(sets)]
+    fn, stream = runner.lib.nnf_hip_copy_kernel, runner.stream
+
+    def launch(i):
+        rc = fn(stream, dst[i % sets].data_ptr(), src[i % sets].data_ptr(), count * 4)
+        if rc != 0:
+            raise RuntimeError(runner.capi.error_string(rc))
+
+    wall, ev = runner.time_steps(launch, steps, warmup)
+    return result_entry("copy kernel 256 MiB -> 256 MiB", 2 * 4 * count, count, wall, ev, 1, {"buffer_sets": sets})
+
+
+def cpu_baseline_config0(runner, group, seconds=8.0):
+    """nnForge's plain backend on config 0, restated in oracle/: batch_norm then rectified_linear,
+    one OpenMP pass per layer, the second in place. Also checks the GPU result bit for bit."""
+    import oracle
+    from nnforge_amd import workloads as w
+
+    n, c, plane = group.entry_count, group.feature_map_count, group.plane
+    gen = np.random.Generator(np.random.MT19937(SEED))
+    x = gen.standard_normal((n, c, plane), dtype=np.float32)
+    gamma = (gen.random(c, dtype=np.float32) + np.float32(0.5)).astype(np.float32)
+    beta = (gen.standard_normal(c, dtype=np.float32) * np.float32(0.1 ** 0.5)).astype(np.float32)
+    mean = (gen.standard_normal(c, dtype=np.float32) * np.float32(0.1 ** 0.5)).astype(np.float32)
+    var = (gen.random(c, dtype=np.float32) * np.float32(1.5) + np.float32(0.5)).astype(np.float32)
+    inv_sigma = (np.float32(1.0) / np.sqrt(var + np.float32(w.BN_EPSILON))).astype(np.float32)
+    threads = oracle.max_threads()
+    buf = np.empty_like(x)
+
+    def one_pass():
+        oracle.batch_norm(x, gamma, beta, mean, inv_sigma, out=buf)
+        oracle.rectified_linear(buf, 0.0, out=buf)
+
+    for _ in range(2):
+        one_pass()
+    times = []
+    t_end = time.perf_counter() + seconds
+    while (time.perf_counter() < t_end and len(times) < 2000) or len(times) < 5:
+        t0 = time.perf_counter()
+        one_pass()
+        times.append(time.perf_counter() - t0)
+    best = statistics.median(times)
+
+    # the same tensors through the GPU path, compared bit for bit
+    torch = runner.torch
+    d_x = torch.from_numpy(x.reshape(-1)).to(runner.device)
+    d_chunks = [torch.from_numpy(v).to(runner.device) for v in (gamma, beta, mean, inv_sigma)]
+    d_out = torch.empty_like(d_x)
+    desc = runner.capi.make_desc(n, c, plane, group.arms, group.tail)
+    runner.capi.chain_forward(desc, d_out.data_ptr(), [d_x.data_ptr()], [t.data_ptr() for t in d_chunks], runner.stream)
+    runner.sync()
+    got = d_out.cpu().numpy()
+    mismatches = int((got.view(np.uint32) != buf.reshape(-1).view(np.uint32)).sum())
+
+    alg = w.group_algorithmic_bytes(group)
+    return {
+        "value": alg / best / 1e9,
+        "unit": "GB/s",
+        "cores": threads,
+        "kind": "port",
+        "sample": "config 0 whole (N=32 C=64 56x56), %d passes of batch_norm then rectified_linear, unfused, median pass time" % len(times),
+        "ms_per_step": best * 1e3,
+        "elements_per_s": w.group_elements(group) / best,
+        "gpu_bit_mismatches_vs_cpu": mismatches,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=400)
+    ap.add_argument("--warmup", type=int, default=40)
+    ap.add_argument("--workload", default="config0", choices=["config0", "config1", "config2", "config3", "config4"])
+    ap.add_argument("--only", action="store_true", help="time only the chosen workload (no per_config survey, no CPU baseline)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        fail("bench.py: this path runs on one GPU (every kernel is independent per entry; there is no "
+             "multi-GPU leg to time). Run with --gpus 1.")
+
+    from nnforge_amd import workloads as w
+
+    runner = Runner()
+    per_config = {}
+
+    def run(name, steps, warmup):
+        if name == "config0":
+            return bench_group(runner, "config0: batch_norm -> rectified_linear N=32 C=64 56x56", w.config0(), steps, warmup)
+        if name == "config1":
+            return bench_softmax(runner, steps, warmup)
+        if name == "config2":
+            return bench_group(runner, "config2: batch_norm -> add(residual) -> parametric_rectified_linear N=128 C=256 56x56", w.config2(), steps, warmup)
+        if name == "config3":
+            return bench_group(runner, "config3: batch_norm -> exponential_linear -> sigmoid -> hyperbolic_tangent N=64 C=512 28x28", w.config3(), steps, warmup)
+        return bench_resnet50(runner, steps, warmup)
+
+    main_entry = run(args.workload, args.steps, args.warmup)
+    per_config[args.workload] = main_entry
+    cpu = None
+    if not args.only:
+        side_steps = {"config0": (200, 20), "config1": (400, 40), "config2": (20, 3), "config3": (60, 6), "config4": (5, 2)}
+        for name in ("config0", "config1", "config2", "config3", "config4"):
+            if name not in per_config:
+                per_config[name] = run(name, *side_steps[name])
+        per_config["copy_kernel"] = bench_copy(runner, 40, 5)
+        if args.workload == "config0":
+            cpu = cpu_baseline_config0(runner, w.config0())
+
+    launches = main_entry["launches_per_step"]
+    achieved = main_entry["algorithmic_bytes_per_step"] / launches / (main_entry["event_ms_per_step"] * 1e-3 / launches) / 1e9
+    line = {
+        "metric": METRIC,
+        "value": main_entry["gbps"],
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": main_entry["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": main_entry["workload"], "buffer_sets": main_entry.get("buffer_sets", 1),
+                   "layout": "[entry][feature_map][y][x] fp32"},
+        "pct_of_hbm_peak": main_entry["pct_of_hbm_peak"],
+        "elements_per_s": main_entry["elements_per_s"],
+        "roofline": {
+            "bound": "hbm",
+            "achieved": achieved,
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBPS,
+            "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+            "kernel": "nnf::chain_kernel" if args.workload != "config1" else "nnf::softmax_rows_kernel",
+            "algorithmic_bytes_per_launch": main_entry["algorithmic_bytes_per_step"] / launches,
+            "avg_launch_us": main_entry["event_ms_per_step"] * 1e3 / launches,
+        },
+        "cpu_baseline": cpu,
+        "per_config": per_config,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
