@@ -308,7 +308,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=400)
     ap.add_argument("--warmup", type=int, default=40)
-    ap.add_argument("--workload", default="config0", choices=["config0", "config1", "config2", "config3", "config4"])
+    ap.add_argument("--workload", default="config0", choices=["config0", "config1", "config2", "config3", "config4", "copy"],
+                    help="'copy' times the plain copy kernel (profiler-counter calibration and bandwidth yardstick)")
     ap.add_argument("--only", action="store_true", help="time only the chosen workload (no per_config survey, no CPU baseline)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -329,6 +330,8 @@ def main():
             return bench_group(runner, "config2: batch_norm -> add(residual) -> parametric_rectified_linear N=128 C=256 56x56", w.config2(), steps, warmup)
         if name == "config3":
             return bench_group(runner, "config3: batch_norm -> exponential_linear -> sigmoid -> hyperbolic_tangent N=64 C=512 28x28", w.config3(), steps, warmup)
+        if name == "copy":
+            return bench_copy(runner, steps, warmup)
         return bench_resnet50(runner, steps, warmup)
 
     main_entry = run(args.workload, args.steps, args.warmup)
@@ -369,7 +372,7 @@ def main():
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBPS,
             "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
-            "kernel": "nnf::chain_kernel" if args.workload != "config1" else "nnf::softmax_rows_kernel",
+            "kernel": {"config1": "nnf::softmax_rows_kernel", "copy": "nnf::copy_kernel_impl"}.get(args.workload, "nnf::chain_kernel"),
             "algorithmic_bytes_per_launch": main_entry["algorithmic_bytes_per_step"] / launches,
             "avg_launch_us": main_entry["event_ms_per_step"] * 1e3 / launches,
         },

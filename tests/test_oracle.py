@@ -1,0 +1,259 @@
+"""Pins the CPU oracle (oracle/nnf_oracle.c) without the reference running.
+
+The reference has no tests, golden vectors or fixtures, and its sources do not compile in this
+image (Boost and protobuf-generated headers are absent). Each oracle function is therefore pinned
+against an independent evaluation chosen so that a plausible slip (dropped term, wrong sign or
+index, transposed layout, fused multiply-add, wrong summation order) fails:
+  * numpy fp32 arithmetic, one rounding per operation, for batch norm / ReLU / PReLU / Add /
+    average subsampling: bit-for-bit equality;
+  * fp64 closed forms (expm1, logistic, tanh, softmax) with explicit error budgets for the layers
+    that call expf;
+  * identities and brute-force index checks with a distinct value in every element.
+"""
+
+import numpy as np
+import pytest
+
+import nnf_testing as T
+import oracle
+
+F = np.float32
+
+
+def bits_equal(a, b):
+    return T.bit_mismatches(a, b) == 0
+
+
+def test_batch_norm_matches_per_operation_fp32_and_layout():
+    gen = T.rng(20, 0)
+    n, c, plane = 3, 5, 7
+    x = T.normal(gen, (n, c, plane), 3.0)
+    g, b, m, s = T.bn_params(gen, c)
+    got = oracle.batch_norm(x, g, b, m, s)
+    mult = (g * s).astype(F)                      # one rounding
+    add = (b - (mult * m).astype(F)).astype(F)    # product rounded, then the difference
+    want = ((x * mult[None, :, None]).astype(F) + add[None, :, None]).astype(F)
+    assert bits_equal(got, want)
+    # a fused multiply-add would differ somewhere on this much data
+    big = T.normal(gen, (4, c, 4096), 3.0)
+    fused = (big.astype(np.float64) * mult[None, :, None].astype(np.float64) + add[None, :, None].astype(np.float64)).astype(F)
+    assert T.bit_mismatches(oracle.batch_norm(big, g, b, m, s), fused) > 0
+    # the fourth chunk is used as an inverse standard deviation as is: doubling it doubles mult
+    got2 = oracle.batch_norm(x, g, b, np.zeros(c, F), (2 * s).astype(F))
+    assert bits_equal(got2, ((x * (g * (2 * s).astype(F)).astype(F)[None, :, None]).astype(F) + b[None, :, None]).astype(F))
+
+
+def test_batch_norm_identity_and_gamma_zero():
+    x = T.normal(T.rng(20, 1), (2, 4, 9), 5.0)
+    one, zero = np.ones(4, F), np.zeros(4, F)
+    assert np.array_equal(oracle.batch_norm(x, one, zero, zero, one), x)
+    beta = np.array([1.5, -2.0, 0.25, 7.0], F)
+    got = oracle.batch_norm(x, zero, beta, T.normal(T.rng(20, 2), 4), one)
+    assert np.array_equal(got, np.broadcast_to(beta[None, :, None], x.shape))
+
+
+def test_batch_norm_feature_map_indexing_brute_force():
+    n, c, plane = 2, 3, 4
+    x = np.arange(n * c * plane, dtype=F).reshape(n, c, plane)
+    g = np.array([1, 10, 100], F)
+    b = np.array([0.5, 0.25, 0.125], F)
+    m = np.array([1, 2, 3], F)
+    s = np.array([1, 0.5, 0.25], F)
+    got = oracle.batch_norm(x, g, b, m, s)
+    for e in range(n):
+        for f in range(c):
+            for p in range(plane):
+                mult = F(g[f] * s[f])
+                assert got[e, f, p] == F(F(x[e, f, p] * mult) + F(b[f] - F(mult * m[f])))
+
+
+def test_rectified_linear():
+    x = np.array([-2.0, -0.0, 0.0, 3.0, np.nan, -np.inf, np.inf, -1e-45], F)
+    got = oracle.rectified_linear(x, 0.0)
+    assert np.array_equal(got[[2, 3, 6]], x[[2, 3, 6]])
+    assert got[0] == 0 and np.signbit(got[0])            # x * 0.0F keeps the sign: -0.0
+    assert got[1] == 0 and np.signbit(got[1])            # -0.0 >= 0 is true: passes through
+    assert np.isnan(got[4]) and np.isnan(got[5])         # -inf * 0 = NaN, as in the reference
+    y = T.normal(T.rng(21, 0), 1000, 2.0)
+    assert bits_equal(oracle.rectified_linear(y, 0.1), np.where(y >= 0, y, (y * F(0.1)).astype(F)))
+    once = oracle.rectified_linear(y, 0.0)
+    assert bits_equal(oracle.rectified_linear(once, 0.0), once)  # idempotent
+
+
+def test_parametric_rectified_linear():
+    gen = T.rng(22, 0)
+    n, c, plane = 3, 4, 5
+    x = T.normal(gen, (n, c, plane), 2.0)
+    a = np.array([0.25, 0.0, 1.0, -0.5], F)
+    got = oracle.parametric_rectified_linear(x, a)
+    want = (x * np.where(x >= 0, F(1.0), a[None, :, None])).astype(F)
+    assert bits_equal(got, want)
+    assert np.array_equal(got[:, 2], x[:, 2])                                  # a = 1: identity
+    relu = oracle.rectified_linear(x, 0.0)
+    assert np.array_equal(got[:, 1], relu[:, 1])                                # a = 0: ReLU (signed zeros compare equal)
+
+
+def test_exponential_linear_against_fp64():
+    x = np.concatenate([T.normal(T.rng(23, 0), 20000, 9.0), np.array([0.0, -0.0, 50.0, -50.0, -1e-8, -104.0, -200.0], F)]).astype(F)
+    got = oracle.exponential_linear(x).astype(np.float64)
+    x64 = x.astype(np.float64)
+    truth = np.where(x64 >= 0, x64, np.expm1(x64))
+    # expf is within 1 ULP of exp; expf(x) - 1 then rounds once more: error <= ulp(1)/2 + ulp(result)
+    assert np.all(np.abs(got - truth) <= 2.0 ** -24 * 1.5 + 2.0 ** -23 * np.abs(truth))
+    assert oracle.exponential_linear(np.array([-50.0], F))[0] == -1.0
+    assert oracle.exponential_linear(np.array([0.0], F))[0] == 0.0
+    pos = x[x >= 0]
+    assert np.array_equal(oracle.exponential_linear(pos), pos)
+    # expf(x) - 1, not expm1f: for tiny negative x the result is exactly 0 or -2^-24, never x itself
+    assert oracle.exponential_linear(np.array([-1e-8], F))[0] in (0.0, F(-2.0 ** -24))
+
+
+def test_sigmoid_against_fp64():
+    x = np.concatenate([T.normal(T.rng(24, 0), 20000, 16.0), np.array([0.0, 50.0, -50.0, 88.0, -88.0, 104.0, -104.0], F)]).astype(F)
+    got = oracle.sigmoid(x)
+    truth = 1.0 / (1.0 + np.exp(-x.astype(np.float64)))
+    assert np.all(np.abs(got.astype(np.float64) - truth) <= 3 * 2.0 ** -24 * np.maximum(truth, 2.0 ** -126))
+    assert oracle.sigmoid(np.array([0.0], F))[0] == 0.5
+    assert oracle.sigmoid(np.array([50.0], F))[0] == 1.0
+    assert oracle.sigmoid(np.array([-104.0], F))[0] == 0.0       # expf overflows to inf: 1/inf
+    # sigma(-x) = 1 - sigma(x) up to rounding
+    s_pos, s_neg = oracle.sigmoid(x).astype(np.float64), oracle.sigmoid(-x).astype(np.float64)
+    assert np.all(np.abs(s_pos + s_neg - 1.0) <= 2.0 ** -22)
+
+
+def test_hyperbolic_tangent_against_fp64():
+    x = np.concatenate([T.normal(T.rng(25, 0), 20000, 4.0), np.array([0.0, 1.0, -1.0, 20.0, -20.0], F)]).astype(F)
+    for scale, steep in ((1.0, 1.0), (1.7159, 0.6666), (1.7159, 0.666666)):
+        got = oracle.hyperbolic_tangent(x, scale, steep).astype(np.float64)
+        steep2 = F(F(steep) * F(2.0))
+        arg = (x * steep2).astype(F).astype(np.float64)
+        truth = np.tanh(arg / 2.0) * float(F(scale))
+        # (e - 1) loses relative accuracy near 0: absolute floor of a few ulp(1) times the scale
+        assert np.all(np.abs(got - truth) <= 4 * 2.0 ** -24 * scale + 4 * 2.0 ** -24 * np.abs(truth))
+        assert oracle.hyperbolic_tangent(np.array([0.0], F), scale, steep)[0] == 0.0
+    # odd function up to rounding; saturates at +-scale; overflow of expf gives NaN (inf/inf) as in the reference
+    y = oracle.hyperbolic_tangent(np.array([30.0, -30.0, 100.0], F), 1.7159, 0.6666)
+    assert y[0] == F(1.7159) and y[1] == -F(1.7159) and np.isnan(y[2])
+
+
+def test_add_order_alpha_and_signed_zero():
+    gen = T.rng(26, 0)
+    xs = [T.normal(gen, 5000, 100.0) for _ in range(4)]
+    got = oracle.add(xs, 0.5)
+    acc = np.zeros(5000, F)
+    for x in xs:
+        acc = (acc + x).astype(F)
+    assert bits_equal(got, (acc * F(0.5)).astype(F))
+    # summation is left to right: a different order changes bits somewhere
+    assert T.bit_mismatches(oracle.add(xs[::-1], 0.5), got) > 0
+    # two inputs commute; adding zeros is the identity times alpha
+    assert bits_equal(oracle.add(xs[:2]), oracle.add(xs[1::-1]))
+    assert bits_equal(oracle.add([xs[0], np.zeros(5000, F)], 3.0), (xs[0] * F(3.0)).astype(F))
+    # the sum starts from +0.0F: -0 + -0 comes out as +0
+    z = oracle.add([np.array([-0.0], F), np.array([-0.0], F)])
+    assert z[0] == 0 and not np.signbit(z[0])
+
+
+def softmax_truth(x):
+    # x - max is an fp32 subtraction in the reference (its rounding is part of the definition);
+    # everything after it in fp64
+    d = (x - x.max(axis=1, keepdims=True)).astype(F).astype(np.float64)
+    e = np.exp(d)
+    return e / e.sum(axis=1, keepdims=True)
+
+
+@pytest.mark.parametrize("shape", [(4, 1000, 1), (3, 7, 5), (2, 10, 4, 3), (1, 1, 6)])
+def test_softmax_against_fp64(shape):
+    gen = T.rng(27, sum(shape))
+    x = T.normal(gen, shape, 4.0)
+    x[gen.random(shape) < 0.01] = 30.0
+    got = oracle.softmax(x)
+    truth = softmax_truth(x)
+    c = shape[1]
+    assert np.all(np.abs(got - truth) <= (c + 8) * 2.0 ** -24 * truth + 1e-45)
+    assert np.all(np.abs(got.astype(np.float64).sum(axis=1) - 1.0) <= c * 2.0 ** -24)
+
+
+def test_softmax_layout_shift_and_special_cases():
+    # feature maps are strided by the plane size: softmax of [n][c][p] equals row softmax of the transposed data
+    x = T.normal(T.rng(27, 100), (3, 6, 5), 3.0)
+    rows = np.ascontiguousarray(x.transpose(0, 2, 1)).reshape(15, 6, 1)
+    assert bits_equal(oracle.softmax(x).transpose(0, 2, 1).reshape(15, 6, 1), oracle.softmax(rows))
+    # shift invariance with an exactly representable shift
+    r = ((np.arange(100, dtype=F) - 50) * F(0.5)).reshape(1, 100, 1)
+    assert bits_equal(oracle.softmax(r), oracle.softmax(r + F(64.0)))
+    # uniform input: every exponential is exactly 1, sum = C, result = fl(1/C)
+    u = oracle.softmax(np.full((2, 100, 1), 5.0, F))
+    assert np.all(u == F(1.0) / F(100.0))
+    # the maximum starts from -1.0e37F: rows entirely below it give sum 0 -> 0 * inf = NaN
+    assert np.isnan(oracle.softmax(np.full((1, 4, 1), -3.0e38, F))).all()
+    # a NaN is skipped by the max but poisons the sum
+    n = np.zeros((1, 5, 1), F)
+    n[0, 2] = np.nan
+    assert np.isnan(oracle.softmax(n)).all()
+    # multiply by the reciprocal of a left-to-right fp32 sum: with exponentials that are exact powers
+    # of two the whole computation can be redone by hand in fp32
+    ln2 = F(0.6931472)
+    k = np.array([0, -1, -2, -3, -1, -5, -2, 0, -7, -1], F)
+    with np.errstate(all="ignore"):
+        y = (k * ln2).astype(F).reshape(1, -1, 1)
+    got = oracle.softmax(y).reshape(-1)
+    e = oracle.exponential_linear(np.minimum(y.reshape(-1), F(-1e-30))) + F(1.0)  # expf(y) for y < 0 via the ELU oracle
+    e = np.where(y.reshape(-1) < 0, e, F(1.0)).astype(F)
+    acc = F(0.0)
+    for v in e:
+        acc = F(acc + v)
+    want = (e * F(F(1.0) / acc)).astype(F)
+    assert T.ulp_distance(got, want).max() <= 1
+
+
+def test_average_subsampling_brute_force_and_multipliers():
+    # distinct value per element, windows 3 (x) by 2 (y): every output is the ordered sum of its own window
+    n, c, h, w = 2, 3, 4, 9
+    x = T.normal(T.rng(28, 0), (n, c, h, w), 10.0)
+    mult = F(0.7)
+    got = oracle.average_subsampling(x, [3, 2], mult=float(mult))
+    assert got.shape == (n, c, 2, 3)
+    for e in range(n):
+        for f in range(c):
+            for oy in range(2):
+                for ox in range(3):
+                    s = F(0.0)
+                    for wy in range(2):          # y outer, x inner: x is the fastest dimension of the window walk
+                        for wx in range(3):
+                            s = F(s + x[e, f, oy * 2 + wy, ox * 3 + wx])
+                    assert got[e, f, oy, ox] == F(s * mult)
+    # a leftover margin is ignored (output size = input size / window, rounded down)
+    y = T.normal(T.rng(28, 1), (1, 1, 5, 7))
+    g2 = oracle.average_subsampling(y, [3, 2], mult=1.0)
+    assert g2.shape == (1, 1, 2, 2)
+    assert g2[0, 0, 1, 1] == F(F(F(F(F(F(y[0, 0, 2, 3] + y[0, 0, 2, 4]) + y[0, 0, 2, 5]) + y[0, 0, 3, 3]) + y[0, 0, 3, 4]) + y[0, 0, 3, 5]))
+    # constant input, 7x7 global window: 49 * v * mult
+    const = np.full((2, 8, 7, 7), 0.5, F)
+    assert np.all(oracle.average_subsampling(const, [7, 7], mult=1.0) == F(24.5))
+    # the plain tester's own multiplier without an alpha is 1 (it returns the window SUM);
+    # the full-configuration rule gives 1/49; an explicit alpha wins in both
+    assert np.all(oracle.average_subsampling(const, [7, 7]) == F(24.5))
+    assert oracle.average_subsampling_full_mult([7, 7]) == F(1.0) / F(49.0)
+    assert oracle.average_subsampling_full_mult([7, 7], alpha=0.25) == F(0.25)
+    assert np.all(oracle.average_subsampling(const, [7, 7], alpha=0.25) == F(24.5 * 0.25))
+
+
+def test_average_subsampling_feature_map_and_entry_windows():
+    n, c, h, w = 4, 6, 2, 2
+    x = T.normal(T.rng(28, 2), (n, c, h, w), 3.0)
+    got = oracle.average_subsampling(x, [2, 1], feature_map_window=3, entry_window=2, mult=1.0)
+    assert got.shape == (2, 2, 2, 1)
+    for oe in range(2):
+        for of in range(2):
+            for oy in range(2):
+                s = F(0.0)
+                for we in range(2):              # entries slowest, then feature maps, then x
+                    for wf in range(3):
+                        for wx in range(2):
+                            s = F(s + x[oe * 2 + we, of * 3 + wf, oy, wx])
+                assert got[oe, of, oy, 0] == s
+    # plain multiplier without alpha: 1 / (feature-map window * entry window)
+    got = oracle.average_subsampling(x, [2, 1], feature_map_window=3, entry_window=2)
+    ref = oracle.average_subsampling(x, [2, 1], feature_map_window=3, entry_window=2, mult=float(F(1.0) / F(6.0)))
+    assert bits_equal(got, ref)
