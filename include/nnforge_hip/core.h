@@ -1,0 +1,175 @@
+// Backend-neutral containers of the inference path, restated by name and meaning from nnForge so
+// that code written against nnForge's plug-in surface compiles against this backend without
+// Boost or protobuf: exceptions, tensor shape, weight containers, the layer base class and its
+// type-name registry.
+#pragma once
+
+#include <cstddef>
+#include <istream>
+#include <map>
+#include <memory>
+#include <ostream>
+#include <set>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+namespace nnforge
+{
+	// nnforge/neural_network_exception.h:23-34. Unlike the reference it does not assert(0) in debug
+	// builds: error paths are exercised by the tests.
+	class neural_network_exception : public std::runtime_error
+	{
+	public:
+		explicit neural_network_exception(const char * message) : std::runtime_error(message) {}
+		explicit neural_network_exception(const std::string& message) : std::runtime_error(message) {}
+		neural_network_exception(const std::string& message, const char * filename, int line_number);
+	};
+
+	// Shape of one entry of a layer's output: feature_map_count planes of
+	// dimension_sizes[0] x dimension_sizes[1] x ... neurons, dimension 0 (x) fastest in memory
+	// (nnforge/layer_configuration_specific.h:27-64, .cpp:62-117).
+	class layer_configuration_specific
+	{
+	public:
+		layer_configuration_specific() : feature_map_count(0) {}
+		layer_configuration_specific(unsigned int feature_map_count) : feature_map_count(feature_map_count) {}
+		layer_configuration_specific(unsigned int feature_map_count, const std::vector<unsigned int>& dimension_sizes)
+			: feature_map_count(feature_map_count), dimension_sizes(dimension_sizes) {}
+
+		// binary form: u32 feature_map_count, u32 dimension_count, u32 sizes[dimension_count]
+		void write(std::ostream& output_stream) const;
+		void read(std::istream& input_stream);
+
+		unsigned int get_neuron_count() const;
+		unsigned int get_neuron_count_per_feature_map() const;
+		unsigned int get_dimension_count() const { return static_cast<unsigned int>(dimension_sizes.size()); }
+
+		// offsets: one coordinate per dimension, x first
+		unsigned int get_pos(const std::vector<unsigned int>& offsets) const;
+		std::vector<unsigned int> get_offsets(unsigned int pos) const;
+
+		// throw neural_network_exception when the two objects differ
+		void check_equality(const layer_configuration_specific& other) const;
+		void check_equality(unsigned int neuron_count) const;
+
+		bool operator==(const layer_configuration_specific& other) const;
+		bool operator!=(const layer_configuration_specific& other) const { return !(*this == other); }
+
+	public:
+		unsigned int feature_map_count;
+		std::vector<unsigned int> dimension_sizes;
+	};
+
+	std::ostream& operator<<(std::ostream& out, const layer_configuration_specific& config);
+
+	// Weights of one layer: a list of chunks of floats (nnforge/layer_data.h:28-48).
+	// Binary form (layer_data.cpp:23-52): u32 chunk_count, then per chunk u32 length + floats.
+	class layer_data : public std::vector<std::vector<float> >
+	{
+	public:
+		typedef std::shared_ptr<layer_data> ptr;
+		typedef std::shared_ptr<const layer_data> const_ptr;
+
+		void write(std::ostream& binary_stream_to_write_to) const;
+		void read(std::istream& binary_stream_to_read_from);
+		void fill(float val);
+	};
+
+	// Integer side data of a layer (nnforge/layer_data_custom.h); none of the layers here has any.
+	class layer_data_custom : public std::vector<std::vector<int> >
+	{
+	public:
+		typedef std::shared_ptr<layer_data_custom> ptr;
+		typedef std::shared_ptr<const layer_data_custom> const_ptr;
+	};
+
+	typedef std::vector<unsigned int> data_config;
+	typedef std::vector<unsigned int> data_custom_config;
+
+	// Key/value view of a layer's "<type>_param { ... }" block of the text-format schema; nested
+	// blocks keep their order (e.g. one dimension_param per spatial dimension).
+	struct schema_param_block
+	{
+		std::map<std::string, std::string> scalars;
+		std::vector<std::pair<std::string, schema_param_block> > blocks;
+
+		bool has(const std::string& key) const { return scalars.find(key) != scalars.end(); }
+		float get_float(const std::string& key, float default_value) const;
+		unsigned int get_uint(const std::string& key, unsigned int default_value) const;
+		unsigned int require_uint(const std::string& key, const std::string& context) const;
+		std::vector<const schema_param_block *> children(const std::string& name) const;
+	};
+
+	// Base of the schema layers (nnforge/layer.h:37-121), forward/inference side only.
+	class layer
+	{
+	public:
+		typedef std::shared_ptr<layer> ptr;
+		typedef std::shared_ptr<const layer> const_ptr;
+
+		virtual ~layer() = default;
+
+		virtual layer::ptr clone() const = 0;
+
+		// default: same configuration as the first input
+		virtual layer_configuration_specific get_output_layer_configuration_specific(
+			const std::vector<layer_configuration_specific>& input_configuration_specific_list) const;
+
+		virtual std::string get_type_name() const = 0;
+
+		// floating point operations per entry of a forward pass (the reference's flops model)
+		virtual float get_forward_flops_per_entry(const std::vector<layer_configuration_specific>& input_configuration_specific_list) const = 0;
+
+		// name of the "<...>_param" block of this layer type in a schema file, empty if it has none
+		virtual std::string get_param_block_name() const { return std::string(); }
+		// reads the layer's parameters; block is null when the schema has no such block
+		virtual void read_params(const schema_param_block * block);
+		virtual void write_params(std::ostream& out, const std::string& indent) const;
+
+		virtual std::vector<std::string> get_parameter_strings() const { return std::vector<std::string>(); }
+
+		// all values 0.0F
+		layer_data::ptr create_layer_data() const;
+		layer_data_custom::ptr create_layer_data_custom() const;
+
+		// throw neural_network_exception when the data does not fit the layer
+		void check_layer_data_consistency(const layer_data& data) const;
+		void check_layer_data_custom_consistency(const layer_data_custom& data_custom) const;
+
+		// the deterministic part of the reference's randomize_data (identity batch norm, 0.25 PReLU slopes)
+		virtual void initialize_data(layer_data& data) const;
+
+		bool is_empty_data() const { return get_data_config().empty(); }
+		bool is_empty_data_custom() const { return get_data_custom_config().empty(); }
+
+		virtual data_config get_data_config() const { return data_config(); }
+		virtual data_custom_config get_data_custom_config() const { return data_custom_config(); }
+
+	public:
+		std::string instance_name;
+		std::vector<std::string> input_layer_instance_names;
+
+	protected:
+		layer() = default;
+	};
+
+	// Registry of layer prototypes by type name (nnforge/layer_factory.h).
+	class layer_factory
+	{
+	public:
+		bool register_layer(layer::const_ptr sample_layer);
+		bool unregister_layer(const std::string& layer_type_name);
+		// throws neural_network_exception for an unknown type
+		layer::ptr create_layer(const std::string& layer_type_name) const;
+		bool is_registered(const std::string& layer_type_name) const;
+		static layer_factory& get_singleton();
+
+	private:
+		layer_factory() = default;
+		std::map<std::string, layer::const_ptr> sample_name_layer_map;
+	};
+
+	// registers the layer types of this backend in layer_factory (nnforge/nnforge.cpp:25-62)
+	void init();
+}

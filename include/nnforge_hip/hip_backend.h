@@ -1,0 +1,281 @@
+// The "hip" backend: a sibling of nnForge's plain and cuda backends for MI355X. It provides
+// layer_tester objects per layer type, chosen by type name, and a forward_propagation
+// implementation that fuses runs of element-wise layers into single kernel launches.
+// Everything device-side goes through the C ABI of include/nnforge_hip.h; this header needs no
+// HIP headers.
+#pragma once
+
+#include "core.h"
+#include "layers.h"
+#include "propagation.h"
+#include "schema.h"
+#include "../nnforge_hip.h"
+
+#include <iosfwd>
+#include <map>
+#include <string>
+#include <vector>
+
+namespace nnforge
+{
+	namespace hip
+	{
+		// Failure of a C-ABI / HIP runtime call (nnforge/cuda/neural_network_cuda_exception.h:27-39)
+		class neural_network_hip_exception : public neural_network_exception
+		{
+		public:
+			neural_network_hip_exception(int error_code, const char * filename, int line_number);
+			int error_code;
+		};
+
+		void hip_check(int code, const char * filename, int line_number);
+		#define hip_safe_call(callstr) ::nnforge::hip::hip_check((callstr), __FILE__, __LINE__)
+
+		// Device allocation owned by the object (nnforge/cuda/cuda_linear_buffer_device.h); sizes are
+		// rounded up to 16 bytes by the allocator.
+		class hip_linear_buffer_device
+		{
+		public:
+			typedef std::shared_ptr<hip_linear_buffer_device> ptr;
+			typedef std::shared_ptr<const hip_linear_buffer_device> const_ptr;
+
+			explicit hip_linear_buffer_device(size_t size);
+			~hip_linear_buffer_device();
+			operator void *() { return buf; }
+			operator const void *() const { return buf; }
+			operator float *() { return static_cast<float *>(buf); }
+			operator const float *() const { return static_cast<const float *>(buf); }
+			size_t get_size() const { return size; }
+
+		private:
+			hip_linear_buffer_device(const hip_linear_buffer_device&) = delete;
+			hip_linear_buffer_device& operator =(const hip_linear_buffer_device&) = delete;
+			void * buf;
+			size_t size;
+		};
+
+		// Device selection and memory budget (nnforge/cuda/cuda_running_configuration.h)
+		class hip_running_configuration
+		{
+		public:
+			typedef std::shared_ptr<const hip_running_configuration> const_ptr;
+
+			// queries the device (throws when there is none)
+			hip_running_configuration(int device_id, float max_global_memory_usage_ratio, bool fuse_layers, bool dont_share_buffers, int max_entry_count);
+			// A configuration that never touches a device: for planning launches and buffers (and testing
+			// that logic) on a machine without a GPU. Running a network with it throws.
+			static std::shared_ptr<const hip_running_configuration> create_offline(
+				unsigned long long global_memory_size, float max_global_memory_usage_ratio, bool fuse_layers, bool dont_share_buffers, int max_entry_count);
+			bool is_offline() const { return offline; }
+			void set_device() const;
+			size_t get_max_bytes() const;
+
+			int device_id;
+			float max_global_memory_usage_ratio;
+			bool fuse_layers;
+			bool dont_share_buffers;
+			int max_entry_count;
+			std::string device_name;
+			unsigned long long global_memory_size;
+			unsigned int compute_unit_count;
+			unsigned int wavefront_size;
+			unsigned int clock_khz;
+
+		private:
+			hip_running_configuration() = default;
+			bool offline = false;
+		};
+
+		std::ostream& operator<<(std::ostream& out, const hip_running_configuration& config);
+
+		// Per layer instance object that enqueues the layer's forward pass on a stream
+		// (the contract of nnforge/cuda/layer_tester_cuda.h:34-96).
+		class layer_tester_hip
+		{
+		public:
+			typedef std::shared_ptr<layer_tester_hip> ptr;
+
+			virtual ~layer_tester_hip() = default;
+
+			void configure(
+				const std::vector<layer_configuration_specific>& input_configuration_specific_list,
+				const layer_configuration_specific& output_configuration_specific,
+				layer::const_ptr layer_schema,
+				hip_running_configuration::const_ptr hip_config);
+
+			// stream_id: a HIP stream handle. Buffers hold entry_count entries each. The output buffer
+			// may be the buffer of input get_input_index_layer_can_write().
+			virtual void enqueue_forward_propagation(
+				void * stream_id,
+				hip_linear_buffer_device::ptr output_buffer,
+				const std::vector<hip_linear_buffer_device::const_ptr>& schema_data,
+				const std::vector<hip_linear_buffer_device::const_ptr>& data,
+				const std::vector<hip_linear_buffer_device::const_ptr>& data_custom,
+				const std::vector<hip_linear_buffer_device::const_ptr>& input_buffers,
+				const std::vector<hip_linear_buffer_device::const_ptr>& persistent_working_data,
+				hip_linear_buffer_device::ptr temporary_working_fixed_buffer,
+				hip_linear_buffer_device::ptr temporary_working_per_entry_buffer,
+				unsigned int entry_count) = 0;
+
+			// uploads the weights: one device buffer per chunk, in chunk order
+			virtual std::vector<hip_linear_buffer_device::const_ptr> get_data(layer_data::const_ptr host_data) const;
+
+			virtual int get_input_index_layer_can_write() const { return -1; }
+			virtual std::pair<size_t, bool> get_temporary_working_fixed_buffer_size() const { return std::make_pair(static_cast<size_t>(0), false); }
+			virtual size_t get_temporary_working_per_entry_buffer_size() const { return 0; }
+
+			// Element-wise testers describe themselves as one op of a fused group: fills op (its chunk
+			// index is set by the caller) and returns how many weight chunks the op consumes, or -1
+			// when the layer cannot be part of a fused group.
+			virtual int get_chain_op(nnf_hip_op& op) const { return -1; }
+
+		protected:
+			layer_tester_hip() = default;
+			virtual void tester_configured() {}
+
+			layer::const_ptr layer_schema;
+			hip_running_configuration::const_ptr hip_config;
+			std::vector<layer_configuration_specific> input_configuration_specific_list;
+			std::vector<unsigned int> input_elem_count_per_entry_list;
+			std::vector<unsigned int> input_elem_count_per_feature_map_list;
+			layer_configuration_specific output_configuration_specific;
+			unsigned int output_elem_count_per_entry;
+			unsigned int output_elem_count_per_feature_map;
+
+		private:
+			layer_tester_hip(const layer_tester_hip&) = delete;
+			layer_tester_hip& operator =(const layer_tester_hip&) = delete;
+		};
+
+		// Prototype that makes testers of one layer type (nnforge/cuda/layer_testing_schema.h:36-71)
+		class layer_testing_schema
+		{
+		public:
+			typedef std::shared_ptr<layer_testing_schema> ptr;
+			typedef std::shared_ptr<const layer_testing_schema> const_ptr;
+			virtual ~layer_testing_schema() = default;
+
+			layer_testing_schema::ptr create(layer::const_ptr layer_schema) const;
+			layer_tester_hip::ptr create_tester(
+				const std::vector<layer_configuration_specific>& input_configuration_specific_list,
+				const layer_configuration_specific& output_configuration_specific,
+				hip_running_configuration::const_ptr hip_config) const;
+			virtual std::string get_type_name() const = 0;
+
+		protected:
+			layer_testing_schema() = default;
+			virtual layer_testing_schema::ptr create_specific() const = 0;
+			virtual layer_tester_hip::ptr create_tester_specific(
+				const std::vector<layer_configuration_specific>& input_configuration_specific_list,
+				const layer_configuration_specific& output_configuration_specific,
+				const hip_running_configuration& hip_config) const = 0;
+			layer::const_ptr layer_schema;
+		};
+
+		// String-keyed registry of the prototypes (nnforge/cuda/layer_testing_schema_factory.cpp:26-50;
+		// same role as layer_tester_plain_factory, nnforge/plain/layer_tester_plain_factory.cpp:27-51)
+		class layer_testing_schema_factory
+		{
+		public:
+			bool register_layer_testing_schema(layer_testing_schema::const_ptr sample_layer_testing_schema);
+			bool unregister_layer_testing_schema(const std::string& layer_type_name);
+			// throws "No layer tester is registered with type ..." for an unknown type
+			layer_testing_schema::ptr create_testing_schema_layer(layer::const_ptr layer) const;
+			static layer_testing_schema_factory& get_singleton();
+
+		private:
+			layer_testing_schema_factory() = default;
+			std::map<std::string, layer_testing_schema::const_ptr> sample_map;
+		};
+
+		// One launch of the forward pass: a single layer or a fused group of element-wise layers.
+		struct forward_step
+		{
+			std::vector<std::string> layer_names;  // members in execution order; back() produces the output
+			std::vector<std::string> input_names;  // layers whose buffers are read, in kernel input order
+			bool fused;                            // executed by the fused-group kernel
+			std::string description() const;       // e.g. "bn1+add1+relu1 <- conv_a, conv_b"
+		};
+
+		// nnforge/cuda/forward_propagation_cuda.h restated for one MI355X.
+		class forward_propagation_hip : public forward_propagation
+		{
+		public:
+			forward_propagation_hip(
+				const network_schema& schema,
+				const std::vector<std::string>& output_layer_names,
+				debug_state::ptr debug,
+				profile_state::ptr profile,
+				hip_running_configuration::const_ptr hip_config);
+			~forward_propagation_hip() override;
+
+			// the launch plan of the current configuration (valid after set_input_configuration_specific / run)
+			const std::vector<forward_step>& get_steps() const { return steps; }
+			// device bytes per entry of the current buffer plan, and the packet size derived from it
+			size_t get_per_entry_buffer_bytes() const { return per_entry_bytes; }
+			unsigned int get_max_entry_count() const { return max_entry_count; }
+
+		protected:
+			void actual_set_data(network_data::const_ptr data) override;
+			void actual_clear_data() override;
+			void actual_run(
+				structured_data_bunch_reader& reader,
+				structured_data_bunch_writer& writer,
+				unsigned int& entries_processed,
+				std::map<std::string, float>& action_seconds,
+				float& idle_seconds) override;
+			void layer_config_map_modified() override;
+
+		private:
+			struct impl;
+			std::unique_ptr<impl> p;
+			hip_running_configuration::const_ptr hip_config;
+			std::vector<forward_step> steps;
+			size_t per_entry_bytes;
+			unsigned int max_entry_count;
+		};
+
+		// nnforge/cuda/forward_propagation_cuda_factory.h
+		class forward_propagation_hip_factory : public forward_propagation_factory
+		{
+		public:
+			explicit forward_propagation_hip_factory(hip_running_configuration::const_ptr hip_config) : hip_config(hip_config) {}
+			forward_propagation::ptr create(
+				const network_schema& schema,
+				const std::vector<std::string>& output_layer_names,
+				debug_state::ptr debug,
+				profile_state::ptr profile) const override;
+
+		private:
+			hip_running_configuration::const_ptr hip_config;
+		};
+
+		// nnforge/cuda/factory_generator_cuda.h: options hip_device_id, hip_max_global_memory_usage_ratio,
+		// hip_fuse, hip_dont_share_buffers, hip_max_entry_count
+		class factory_generator_hip : public factory_generator
+		{
+		public:
+			factory_generator_hip();
+			void initialize() override;
+			forward_propagation_factory::ptr create_forward_propagation_factory() const override;
+			backward_propagation_factory::ptr create_backward_propagation_factory() const override; // throws: inference only
+			void info() const override;
+			std::vector<bool_option> get_bool_options() override;
+			std::vector<float_option> get_float_options() override;
+			std::vector<int_option> get_int_options() override;
+
+			int hip_device_id;
+			float hip_max_global_memory_usage_ratio;
+			bool hip_fuse;
+			bool hip_dont_share_buffers;
+			int hip_max_entry_count;
+
+		private:
+			hip_running_configuration::const_ptr hip_config;
+		};
+
+		// registers the layer types and the testers of this backend (nnforge/cuda/cuda.cpp:92-160,
+		// nnforge/plain/plain.cpp:92-126)
+		void init();
+	}
+}

@@ -1,0 +1,194 @@
+// Schema classes of the layers on the inference path: type names, parameters and weight-chunk
+// layouts as nnForge defines them.
+#pragma once
+
+#include "core.h"
+
+#include <limits>
+
+namespace nnforge
+{
+	// Placeholder for externally supplied data (nnforge/data_layer.h); type name "Data".
+	class data_layer : public layer
+	{
+	public:
+		data_layer() = default;
+		layer::ptr clone() const override;
+		std::string get_type_name() const override;
+		float get_forward_flops_per_entry(const std::vector<layer_configuration_specific>&) const override { return 0.0F; }
+		static const std::string layer_type_name;
+	};
+
+	// Four weight chunks of feature_map_count floats: gamma, beta, mean, inverse standard
+	// deviation (nnforge/batch_norm_layer.h:26, batch_norm_layer.cpp:96-106). epsilon is carried
+	// for schema round trips only; inference never reads it.
+	class batch_norm_layer : public layer
+	{
+	public:
+		explicit batch_norm_layer(unsigned int feature_map_count = 1, float epsilon = default_batch_normalization_epsilon);
+		layer::ptr clone() const override;
+		std::string get_type_name() const override;
+		float get_forward_flops_per_entry(const std::vector<layer_configuration_specific>& input_configuration_specific_list) const override;
+		std::string get_param_block_name() const override { return "batch_norm_param"; }
+		void read_params(const schema_param_block * block) override;
+		void write_params(std::ostream& out, const std::string& indent) const override;
+		data_config get_data_config() const override;
+		void initialize_data(layer_data& data) const override; // gamma 1, beta 0, mean 0, inverse sigma 1
+		std::vector<std::string> get_parameter_strings() const override;
+
+		static const std::string layer_type_name;
+		static const float default_batch_normalization_epsilon;
+
+		unsigned int feature_map_count;
+		float epsilon;
+
+	private:
+		void check();
+	};
+
+	// nnforge/rectified_linear_layer.h:24-47; type name "ReLU"
+	class rectified_linear_layer : public layer
+	{
+	public:
+		explicit rectified_linear_layer(float negative_slope = 0.0F);
+		layer::ptr clone() const override;
+		std::string get_type_name() const override;
+		float get_forward_flops_per_entry(const std::vector<layer_configuration_specific>& input_configuration_specific_list) const override;
+		std::string get_param_block_name() const override { return "relu_param"; }
+		void read_params(const schema_param_block * block) override;
+		void write_params(std::ostream& out, const std::string& indent) const override;
+		std::vector<std::string> get_parameter_strings() const override;
+
+		static const std::string layer_type_name;
+		float negative_slope;
+	};
+
+	// One slope per feature map in chunk 0 (nnforge/parametric_rectified_linear_layer.h:26-63); "PReLU"
+	class parametric_rectified_linear_layer : public layer
+	{
+	public:
+		explicit parametric_rectified_linear_layer(unsigned int feature_map_count = 1);
+		layer::ptr clone() const override;
+		std::string get_type_name() const override;
+		float get_forward_flops_per_entry(const std::vector<layer_configuration_specific>& input_configuration_specific_list) const override;
+		std::string get_param_block_name() const override { return "prelu_param"; }
+		void read_params(const schema_param_block * block) override;
+		void write_params(std::ostream& out, const std::string& indent) const override;
+		data_config get_data_config() const override;
+		void initialize_data(layer_data& data) const override; // 0.25
+		std::vector<std::string> get_parameter_strings() const override;
+
+		static const std::string layer_type_name;
+		unsigned int feature_map_count;
+
+	private:
+		void check();
+	};
+
+	// nnforge/exponential_linear_layer.h:26-40; "ELU" (no alpha parameter exists)
+	class exponential_linear_layer : public layer
+	{
+	public:
+		exponential_linear_layer() = default;
+		layer::ptr clone() const override;
+		std::string get_type_name() const override;
+		float get_forward_flops_per_entry(const std::vector<layer_configuration_specific>& input_configuration_specific_list) const override;
+		static const std::string layer_type_name;
+	};
+
+	// nnforge/sigmoid_layer.h:26-40; "Sigmoid"
+	class sigmoid_layer : public layer
+	{
+	public:
+		sigmoid_layer() = default;
+		layer::ptr clone() const override;
+		std::string get_type_name() const override;
+		float get_forward_flops_per_entry(const std::vector<layer_configuration_specific>& input_configuration_specific_list) const override;
+		static const std::string layer_type_name;
+	};
+
+	// f(x) = scale * tanh(steepness * x) (nnforge/hyperbolic_tangent_layer.h:30-56); "TanH"
+	class hyperbolic_tangent_layer : public layer
+	{
+	public:
+		explicit hyperbolic_tangent_layer(float scale = 1.0F, float steepness = 1.0F);
+		layer::ptr clone() const override;
+		std::string get_type_name() const override;
+		float get_forward_flops_per_entry(const std::vector<layer_configuration_specific>& input_configuration_specific_list) const override;
+		std::string get_param_block_name() const override { return "tanh_param"; }
+		void read_params(const schema_param_block * block) override;
+		void write_params(std::ostream& out, const std::string& indent) const override;
+		std::vector<std::string> get_parameter_strings() const override;
+
+		static const std::string layer_type_name;
+		float scale;
+		float steepness;
+	};
+
+	// Sum of all inputs times alpha (nnforge/add_layer.h:24-51); "Add"
+	class add_layer : public layer
+	{
+	public:
+		explicit add_layer(float alpha = 1.0F);
+		layer::ptr clone() const override;
+		// all inputs must have the same neuron count (nnforge/add_layer.cpp:44-55)
+		layer_configuration_specific get_output_layer_configuration_specific(
+			const std::vector<layer_configuration_specific>& input_configuration_specific_list) const override;
+		std::string get_type_name() const override;
+		float get_forward_flops_per_entry(const std::vector<layer_configuration_specific>& input_configuration_specific_list) const override;
+		std::string get_param_block_name() const override { return "add_param"; }
+		void read_params(const schema_param_block * block) override;
+		void write_params(std::ostream& out, const std::string& indent) const override;
+		std::vector<std::string> get_parameter_strings() const override;
+
+		static const std::string layer_type_name;
+		float alpha;
+	};
+
+	// nnforge/softmax_layer.h:23-37; "Softmax"
+	class softmax_layer : public layer
+	{
+	public:
+		softmax_layer() = default;
+		layer::ptr clone() const override;
+		std::string get_type_name() const override;
+		float get_forward_flops_per_entry(const std::vector<layer_configuration_specific>& input_configuration_specific_list) const override;
+		static const std::string layer_type_name;
+	};
+
+	// Spatial average subsampling with relative factors (the window sizes), the subset of
+	// nnforge/average_subsampling_layer.h this backend runs: two spatial dimensions, no
+	// feature-map or entry subsampling. "AverageSubsampling"
+	class average_subsampling_layer : public layer
+	{
+	public:
+		explicit average_subsampling_layer(
+			const std::vector<unsigned int>& subsampling_sizes = std::vector<unsigned int>(),
+			float alpha = -std::numeric_limits<float>::max());
+		layer::ptr clone() const override;
+		layer_configuration_specific get_output_layer_configuration_specific(
+			const std::vector<layer_configuration_specific>& input_configuration_specific_list) const override;
+		std::string get_type_name() const override;
+		float get_forward_flops_per_entry(const std::vector<layer_configuration_specific>& input_configuration_specific_list) const override;
+		std::string get_param_block_name() const override { return "average_subsampling_param"; }
+		void read_params(const schema_param_block * block) override;
+		void write_params(std::ostream& out, const std::string& indent) const override;
+		std::vector<std::string> get_parameter_strings() const override;
+
+		bool has_alpha() const { return alpha != -std::numeric_limits<float>::max(); }
+
+		// 1 / (number of window elements) unless alpha is set
+		// (average_subsampling_layer::get_effective_alpha given the full configurations,
+		// nnforge/average_subsampling_layer.cpp:287-303)
+		float get_effective_alpha() const;
+
+		// What the reference's PLAIN tester multiplies by: it passes bare feature-map counts where
+		// configurations are expected (nnforge/plain/average_subsampling_layer_tester_plain.cpp:82),
+		// so without an explicit alpha the spatial window does not divide and the factor is 1.
+		float get_plain_tester_alpha() const;
+
+		static const std::string layer_type_name;
+		std::vector<unsigned int> subsampling_sizes; // x first
+		float alpha;
+	};
+}

@@ -1,0 +1,221 @@
+// The plug-in boundary a backend implements: data readers/writers, forward_propagation and its
+// factory, factory_generator with its command-line options.
+#pragma once
+
+#include "core.h"
+#include "schema.h"
+
+#include <map>
+#include <set>
+#include <string>
+#include <vector>
+
+namespace nnforge
+{
+	// Source of input entries (nnforge/structured_data_bunch_reader.h:27-58).
+	class structured_data_bunch_reader
+	{
+	public:
+		typedef std::shared_ptr<structured_data_bunch_reader> ptr;
+		virtual ~structured_data_bunch_reader() = default;
+		virtual std::map<std::string, layer_configuration_specific> get_config_map() const = 0;
+		// fills one entry of every layer in data_map; false when the entry cannot be read
+		virtual bool read(unsigned int entry_id, const std::map<std::string, float *>& data_map) = 0;
+		virtual void set_epoch(unsigned int epoch_id) {}
+		virtual int get_entry_count() const { return -1; } // -1: unknown
+
+	protected:
+		structured_data_bunch_reader() = default;
+	};
+
+	// Sink of output entries (nnforge/structured_data_bunch_writer.h:27-50).
+	class structured_data_bunch_writer
+	{
+	public:
+		typedef std::shared_ptr<structured_data_bunch_writer> ptr;
+		virtual ~structured_data_bunch_writer() = default;
+		virtual void set_config_map(const std::map<std::string, layer_configuration_specific> config_map) = 0;
+		virtual void write(unsigned int entry_id, const std::map<std::string, const float *>& data_map) = 0;
+
+	protected:
+		structured_data_bunch_writer() = default;
+	};
+
+	// Reader over caller-owned arrays: layer name -> entry_count consecutive entries.
+	class memory_data_bunch_reader : public structured_data_bunch_reader
+	{
+	public:
+		memory_data_bunch_reader(unsigned int entry_count) : entry_count(entry_count) {}
+		void add(const std::string& layer_name, const layer_configuration_specific& config, const float * data);
+		std::map<std::string, layer_configuration_specific> get_config_map() const override { return config_map; }
+		bool read(unsigned int entry_id, const std::map<std::string, float *>& data_map) override;
+		int get_entry_count() const override { return static_cast<int>(entry_count); }
+
+	private:
+		unsigned int entry_count;
+		std::map<std::string, layer_configuration_specific> config_map;
+		std::map<std::string, const float *> data;
+	};
+
+	// Writer that keeps every entry in memory (the role of neuron_value_set_data_bunch_writer,
+	// nnforge/neuron_value_set_data_bunch_writer.cpp:21-39).
+	class memory_data_bunch_writer : public structured_data_bunch_writer
+	{
+	public:
+		void set_config_map(const std::map<std::string, layer_configuration_specific> config_map) override;
+		void write(unsigned int entry_id, const std::map<std::string, const float *>& data_map) override;
+
+		std::map<std::string, layer_configuration_specific> config_map;
+		std::map<std::string, std::vector<float> > values; // layer name -> entries back to back
+		unsigned int entry_count = 0;
+	};
+
+	// nnforge/debug_state.h, profile_state.h reduced to their switches
+	struct debug_state
+	{
+		typedef std::shared_ptr<debug_state> ptr;
+		explicit debug_state(bool debug_mode = false) : debug_mode(debug_mode) {}
+		bool is_debug() const { return debug_mode; }
+		bool debug_mode;
+	};
+
+	struct profile_state
+	{
+		typedef std::shared_ptr<profile_state> ptr;
+		explicit profile_state(bool profile_mode = false) : profile_mode(profile_mode) {}
+		bool is_profile() const { return profile_mode; }
+		bool profile_mode;
+	};
+
+	// nnforge/forward_propagation.h:39-115
+	class forward_propagation
+	{
+	public:
+		class stat
+		{
+		public:
+			unsigned int entry_processed_count;
+			float flops_per_entry;
+			float total_seconds;
+			float idle_seconds;
+		};
+
+		typedef std::shared_ptr<forward_propagation> ptr;
+
+		virtual ~forward_propagation() = default;
+
+		// narrows the data to the layers of the schema and checks it against them
+		void set_data(const network_data& data);
+		void clear_data();
+
+		// not needed before run(): run() takes the configurations from the reader
+		void set_input_configuration_specific(const std::map<std::string, layer_configuration_specific>& input_configuration_specific_map);
+
+		stat run(structured_data_bunch_reader& reader, structured_data_bunch_writer& writer);
+
+		bool is_schema_with_weights() const;
+
+		// seconds per action of the last run (filled when profiling is on); key = layer instance name,
+		// or the names of a fused group joined with '+'
+		const std::map<std::string, float>& get_last_action_seconds() const { return last_action_seconds; }
+
+	protected:
+		forward_propagation(
+			const network_schema& schema,
+			const std::vector<std::string>& output_layer_names,
+			debug_state::ptr debug,
+			profile_state::ptr profile);
+
+		virtual void actual_set_data(network_data::const_ptr data) = 0;
+		virtual void actual_clear_data() = 0;
+		virtual void actual_run(
+			structured_data_bunch_reader& reader,
+			structured_data_bunch_writer& writer,
+			unsigned int& entries_processed,
+			std::map<std::string, float>& action_seconds,
+			float& idle_seconds) = 0;
+		// called when set_input_configuration_specific changed layer_config_map
+		virtual void layer_config_map_modified() = 0;
+
+	protected:
+		network_schema::const_ptr schema; // reduced to what the outputs need
+		std::vector<std::string> output_layer_names;
+		debug_state::ptr debug;
+		profile_state::ptr profile;
+		std::map<std::string, layer_configuration_specific> layer_config_map;
+		float flops;
+		std::set<std::string> data_layer_names;
+		std::map<std::string, float> last_action_seconds;
+
+	private:
+		forward_propagation() = delete;
+		forward_propagation(const forward_propagation&) = delete;
+		forward_propagation& operator =(const forward_propagation&) = delete;
+	};
+
+	std::ostream& operator<< (std::ostream& out, const forward_propagation::stat& val);
+
+	// nnforge/forward_propagation_factory.h:30-46
+	class forward_propagation_factory
+	{
+	public:
+		typedef std::shared_ptr<forward_propagation_factory> ptr;
+		typedef std::shared_ptr<const forward_propagation_factory> const_ptr;
+		virtual ~forward_propagation_factory() = default;
+		virtual forward_propagation::ptr create(
+			const network_schema& schema,
+			const std::vector<std::string>& output_layer_names,
+			debug_state::ptr debug,
+			profile_state::ptr profile) const = 0;
+
+	protected:
+		forward_propagation_factory() = default;
+	};
+
+	// nnforge/backward_propagation_factory.h: the training side is outside this backend; the type
+	// exists so that factory_generator keeps its shape.
+	class backward_propagation_factory
+	{
+	public:
+		typedef std::shared_ptr<backward_propagation_factory> ptr;
+		virtual ~backward_propagation_factory() = default;
+	};
+
+	// option descriptors (nnforge/config_options.h): a name (optionally "long,S" with a short form),
+	// the variable to fill, its default and a description
+	template<class T> struct config_option
+	{
+		config_option(const char * name, T * var, const T& default_value, const char * description)
+			: name(name), var(var), default_value(default_value), description(description) {}
+		std::string name;
+		T * var;
+		T default_value;
+		std::string description;
+	};
+	typedef config_option<std::string> string_option;
+	typedef config_option<bool> bool_option;
+	typedef config_option<float> float_option;
+	typedef config_option<int> int_option;
+
+	// nnforge/factory_generator.h:27-56
+	class factory_generator
+	{
+	public:
+		typedef std::shared_ptr<factory_generator> ptr;
+		virtual ~factory_generator() = default;
+		virtual void initialize() = 0;
+		virtual forward_propagation_factory::ptr create_forward_propagation_factory() const = 0;
+		virtual backward_propagation_factory::ptr create_backward_propagation_factory() const = 0;
+		virtual void info() const = 0;
+		virtual std::vector<string_option> get_string_options() { return std::vector<string_option>(); }
+		virtual std::vector<bool_option> get_bool_options() { return std::vector<bool_option>(); }
+		virtual std::vector<float_option> get_float_options() { return std::vector<float_option>(); }
+		virtual std::vector<int_option> get_int_options() { return std::vector<int_option>(); }
+
+		// sets every option variable to its default (what the toolset does before parsing the command line)
+		void apply_default_options();
+
+	protected:
+		factory_generator() = default;
+	};
+}

@@ -1,0 +1,90 @@
+/*
+ * nnforge_hip_backend.h - C bridge over the C++ hip backend (include/nnforge_hip/hip_backend.h) for
+ * callers without a C++ toolchain: run a text-format nnForge schema on host arrays through
+ * factory_generator_hip -> forward_propagation_hip, or only plan it. The tests and tools drive the
+ * backend through this bridge; a C++ application uses the classes directly, as it would use
+ * nnForge's plain or cuda backend (examples/gtsrb/gtsrb.cpp:29-63 shows the reference's pattern).
+ *
+ * Return value: 0 = success; non-zero = failure, with the exception text in `report`.
+ */
+#ifndef NNFORGE_HIP_BACKEND_H
+#define NNFORGE_HIP_BACKEND_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define NNF_BACKEND_API __attribute__((visibility("default")))
+
+typedef struct nnf_backend_weights
+{
+	const char* layer_name;
+	uint32_t chunk_count;
+	const uint32_t* chunk_sizes;   /* floats per chunk */
+	const float* const* chunks;
+} nnf_backend_weights;
+
+typedef struct nnf_backend_input
+{
+	const char* layer_name;        /* a data layer of the schema */
+	uint32_t feature_map_count;
+	uint32_t dimension_count;
+	const uint32_t* dimension_sizes; /* x first */
+	const float* data;             /* entry_count entries back to back; may be null when only planning */
+} nnf_backend_input;
+
+typedef struct nnf_backend_output
+{
+	const char* layer_name;
+	float* data;                   /* receives entry_count entries */
+	size_t capacity_floats;
+	size_t written_floats;         /* set by the call */
+} nnf_backend_output;
+
+typedef struct nnf_backend_options
+{
+	int32_t fuse;                  /* hip_fuse */
+	int32_t dont_share_buffers;    /* hip_dont_share_buffers */
+	int32_t max_entry_count;       /* hip_max_entry_count; <= 0: default */
+	int32_t profile;               /* per-launch times in the report */
+	int32_t weights_from_folder;   /* 1: `weights_folder` holds <layer>.data files */
+	const char* weights_folder;
+} nnf_backend_options;
+
+/* Runs the schema on device 0. The report lists one line per launch ("step: ..."), the buffer plan
+ * and, with profile, per-launch seconds. */
+NNF_BACKEND_API int nnf_backend_run_schema(
+	const char* schema_text,
+	const nnf_backend_weights* weights, uint32_t weights_count,
+	const nnf_backend_input* inputs, uint32_t input_count,
+	uint32_t entry_count,
+	nnf_backend_output* outputs, uint32_t output_count,
+	const nnf_backend_options* options,
+	char* report, size_t report_capacity);
+
+/* Plans launches and buffers without touching a device (works on a machine without a GPU).
+ * memory_bytes: the device memory to plan for. */
+NNF_BACKEND_API int nnf_backend_plan_schema(
+	const char* schema_text,
+	const nnf_backend_input* inputs, uint32_t input_count,
+	const char* const* output_layer_names, uint32_t output_count,
+	const nnf_backend_options* options,
+	uint64_t memory_bytes,
+	char* report, size_t report_capacity);
+
+/* Parses a schema and writes it back in text format (round trip of the reader/writer). */
+NNF_BACKEND_API int nnf_backend_rewrite_schema(const char* schema_text, char* out_text, size_t out_capacity);
+
+/* Writes / reads <layer>.data files in nnForge's format (weights in, weights out through `weights`
+ * arrays owned by the caller; reading fills caller-provided chunks and checks their sizes). */
+NNF_BACKEND_API int nnf_backend_write_weights(const char* folder, const nnf_backend_weights* weights, uint32_t weights_count, char* report, size_t report_capacity);
+NNF_BACKEND_API int nnf_backend_read_weights(const char* folder, const char* layer_name, uint32_t chunk_count, const uint32_t* chunk_sizes, float* const* chunks, char* report, size_t report_capacity);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* NNFORGE_HIP_BACKEND_H */

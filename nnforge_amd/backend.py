@@ -1,0 +1,206 @@
+"""ctypes binding of the C bridge over the C++ hip backend (include/nnforge_hip_backend.h):
+run or plan a text-format nnForge schema. Used by the tests; contains no arithmetic."""
+
+import ctypes
+import os
+
+import numpy as np
+
+from . import build as _build
+
+_FP = ctypes.POINTER(ctypes.c_float)
+_UP = ctypes.POINTER(ctypes.c_uint32)
+
+
+class Weights(ctypes.Structure):
+    _fields_ = [("layer_name", ctypes.c_char_p), ("chunk_count", ctypes.c_uint32), ("chunk_sizes", _UP),
+                ("chunks", ctypes.POINTER(_FP))]
+
+
+class Input(ctypes.Structure):
+    _fields_ = [("layer_name", ctypes.c_char_p), ("feature_map_count", ctypes.c_uint32), ("dimension_count", ctypes.c_uint32),
+                ("dimension_sizes", _UP), ("data", _FP)]
+
+
+class Output(ctypes.Structure):
+    _fields_ = [("layer_name", ctypes.c_char_p), ("data", _FP), ("capacity_floats", ctypes.c_size_t),
+                ("written_floats", ctypes.c_size_t)]
+
+
+class Options(ctypes.Structure):
+    _fields_ = [("fuse", ctypes.c_int32), ("dont_share_buffers", ctypes.c_int32), ("max_entry_count", ctypes.c_int32),
+                ("profile", ctypes.c_int32), ("weights_from_folder", ctypes.c_int32), ("weights_folder", ctypes.c_char_p)]
+
+
+class BackendError(RuntimeError):
+    def __init__(self, code, message):
+        RuntimeError.__init__(self, message)
+        self.code = code
+
+
+_lib = None
+REPORT_CAPACITY = 1 << 16
+
+
+def load():
+    global _lib
+    if _lib is None:
+        path = _build.BACKEND_LIBRARY
+        if not os.path.exists(path):
+            raise RuntimeError("%s is missing: build it first (python -c 'import __graft_entry__ as g; g.build()')" % path)
+        lib = ctypes.CDLL(path)
+        lib.nnf_backend_run_schema.argtypes = [ctypes.c_char_p, ctypes.POINTER(Weights), ctypes.c_uint32, ctypes.POINTER(Input),
+                                               ctypes.c_uint32, ctypes.c_uint32, ctypes.POINTER(Output), ctypes.c_uint32,
+                                               ctypes.POINTER(Options), ctypes.c_char_p, ctypes.c_size_t]
+        lib.nnf_backend_plan_schema.argtypes = [ctypes.c_char_p, ctypes.POINTER(Input), ctypes.c_uint32,
+                                                ctypes.POINTER(ctypes.c_char_p), ctypes.c_uint32, ctypes.POINTER(Options),
+                                                ctypes.c_uint64, ctypes.c_char_p, ctypes.c_size_t]
+        lib.nnf_backend_rewrite_schema.argtypes = [ctypes.c_char_p, ctypes.c_char_p, ctypes.c_size_t]
+        lib.nnf_backend_write_weights.argtypes = [ctypes.c_char_p, ctypes.POINTER(Weights), ctypes.c_uint32, ctypes.c_char_p, ctypes.c_size_t]
+        lib.nnf_backend_read_weights.argtypes = [ctypes.c_char_p, ctypes.c_char_p, ctypes.c_uint32, _UP, ctypes.POINTER(_FP),
+                                                 ctypes.c_char_p, ctypes.c_size_t]
+        _lib = lib
+    return _lib
+
+
+def _options(fuse=True, dont_share_buffers=False, max_entry_count=0, profile=False, weights_folder=None):
+    o = Options()
+    o.fuse = int(fuse)
+    o.dont_share_buffers = int(dont_share_buffers)
+    o.max_entry_count = int(max_entry_count)
+    o.profile = int(profile)
+    o.weights_from_folder = int(weights_folder is not None)
+    o.weights_folder = weights_folder.encode() if weights_folder is not None else None
+    return o
+
+
+def _weights_array(weights, keep):
+    """weights: {layer name: [numpy chunk, ...]}"""
+    arr = (Weights * max(1, len(weights)))()
+    for i, (name, chunks) in enumerate(sorted(weights.items())):
+        chunks = [np.ascontiguousarray(c, dtype=np.float32) for c in chunks]
+        sizes = (ctypes.c_uint32 * len(chunks))(*[c.size for c in chunks])
+        ptrs = (_FP * len(chunks))(*[c.ctypes.data_as(_FP) for c in chunks])
+        keep.extend([chunks, sizes, ptrs])
+        arr[i].layer_name = name.encode()
+        arr[i].chunk_count = len(chunks)
+        arr[i].chunk_sizes = sizes
+        arr[i].chunks = ptrs
+    return arr
+
+
+def _inputs_array(inputs, keep, with_data=True):
+    """inputs: {data layer name: numpy array [entries][feature maps][...spatial, x last]} or, when
+    only planning, {name: (feature_map_count, [dimension sizes, x first])}"""
+    arr = (Input * max(1, len(inputs)))()
+    entry_count = None
+    for i, (name, value) in enumerate(sorted(inputs.items())):
+        if with_data:
+            a = np.ascontiguousarray(value, dtype=np.float32)
+            fm = a.shape[1]
+            dims = list(a.shape[2:])[::-1]
+            entry_count = a.shape[0] if entry_count is None else entry_count
+            assert a.shape[0] == entry_count
+            keep.append(a)
+            arr[i].data = a.ctypes.data_as(_FP)
+        else:
+            fm, dims = value
+        dim_arr = (ctypes.c_uint32 * max(1, len(dims)))(*dims)
+        keep.append(dim_arr)
+        arr[i].layer_name = name.encode()
+        arr[i].feature_map_count = fm
+        arr[i].dimension_count = len(dims)
+        arr[i].dimension_sizes = dim_arr
+    return arr, entry_count
+
+
+def parse_report(text):
+    res = {"steps": [], "seconds": {}, "outputs": {}, "raw": text}
+    for line in text.splitlines():
+        key, _, rest = line.partition(": ")
+        if key == "step":
+            kind, _, desc = rest.partition(" ")
+            layers, _, sources = desc.partition(" <- ")
+            res["steps"].append({"fused": kind == "fused", "layers": layers.split("+"), "inputs": sources.split(", ")})
+        elif key in ("per_entry_bytes", "max_entry_count", "entries"):
+            res[key] = int(rest)
+        elif key == "seconds":
+            name, _, sec = rest.rpartition(" ")
+            res["seconds"][name] = float(sec)
+        elif key == "output":
+            name, _, cfg = rest.partition(" ")
+            res["outputs"][name] = cfg
+        elif key == "stat":
+            res["stat"] = rest
+    return res
+
+
+def run_schema(schema_text, weights, inputs, output_shapes, **options):
+    """output_shapes: {output layer name: numpy shape of the whole result [entries][...]}.
+    Returns ({name: array}, parsed report)."""
+    lib = load()
+    keep = []
+    w = _weights_array(weights, keep)
+    ins, entry_count = _inputs_array(inputs, keep)
+    outs = (Output * len(output_shapes))()
+    arrays = {}
+    for i, (name, shape) in enumerate(sorted(output_shapes.items())):
+        a = np.full(shape, np.nan, dtype=np.float32)
+        arrays[name] = a
+        outs[i].layer_name = name.encode()
+        outs[i].data = a.ctypes.data_as(_FP)
+        outs[i].capacity_floats = a.size
+    report = ctypes.create_string_buffer(REPORT_CAPACITY)
+    opt = _options(**options)
+    rc = lib.nnf_backend_run_schema(schema_text.encode(), w, len(weights), ins, len(inputs), entry_count or 0, outs,
+                                    len(output_shapes), ctypes.byref(opt), report, REPORT_CAPACITY)
+    if rc != 0:
+        raise BackendError(rc, report.value.decode(errors="replace"))
+    for i, name in enumerate(sorted(output_shapes)):
+        assert outs[i].written_floats == arrays[name].size, (name, outs[i].written_floats, arrays[name].size)
+    return arrays, parse_report(report.value.decode())
+
+
+def plan_schema(schema_text, input_configs, output_names, memory_bytes=288 << 30, **options):
+    lib = load()
+    keep = []
+    ins, _ = _inputs_array(input_configs, keep, with_data=False)
+    names = (ctypes.c_char_p * len(output_names))(*[n.encode() for n in output_names])
+    report = ctypes.create_string_buffer(REPORT_CAPACITY)
+    opt = _options(**options)
+    rc = lib.nnf_backend_plan_schema(schema_text.encode(), ins, len(input_configs), names, len(output_names), ctypes.byref(opt),
+                                     memory_bytes, report, REPORT_CAPACITY)
+    if rc != 0:
+        raise BackendError(rc, report.value.decode(errors="replace"))
+    return parse_report(report.value.decode())
+
+
+def rewrite_schema(schema_text):
+    lib = load()
+    out = ctypes.create_string_buffer(REPORT_CAPACITY)
+    rc = lib.nnf_backend_rewrite_schema(schema_text.encode(), out, REPORT_CAPACITY)
+    if rc != 0:
+        raise BackendError(rc, out.value.decode(errors="replace"))
+    return out.value.decode()
+
+
+def write_weights(folder, weights):
+    lib = load()
+    keep = []
+    w = _weights_array(weights, keep)
+    report = ctypes.create_string_buffer(4096)
+    rc = lib.nnf_backend_write_weights(folder.encode(), w, len(weights), report, 4096)
+    if rc != 0:
+        raise BackendError(rc, report.value.decode(errors="replace"))
+
+
+def read_weights(folder, layer_name, chunk_sizes):
+    lib = load()
+    chunks = [np.empty(s, dtype=np.float32) for s in chunk_sizes]
+    sizes = (ctypes.c_uint32 * len(chunks))(*chunk_sizes)
+    ptrs = (_FP * len(chunks))(*[c.ctypes.data_as(_FP) for c in chunks])
+    report = ctypes.create_string_buffer(4096)
+    rc = lib.nnf_backend_read_weights(folder.encode(), layer_name.encode(), len(chunks), sizes, ptrs, report, 4096)
+    if rc != 0:
+        raise BackendError(rc, report.value.decode(errors="replace"))
+    return chunks

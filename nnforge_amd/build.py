@@ -45,8 +45,32 @@ def build_hip_library(verbose=False):
     return HIP_LIBRARY
 
 
+HOST_DIR = os.path.join(PACKAGE_DIR, "host")
+BACKEND_LIBRARY = os.path.join(PACKAGE_DIR, "libnnforge_hip_backend.so")
+BACKEND_SOURCES = ["core.cpp", "layers.cpp", "schema.cpp", "propagation.cpp", "hip_testers.cpp",
+                   "forward_propagation_hip.cpp", "backend_capi.cpp"]
+BACKEND_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden", "-Wall", "-Wextra",
+                 "-Wno-unused-parameter"]
+
+
+def build_backend_library(verbose=False):
+    """Compiles the host-side C++ backend (g++, no HIP headers) into libnnforge_hip_backend.so,
+    linked against libnnforge_hip.so in the same directory."""
+    if not os.path.exists(HIP_LIBRARY):
+        raise RuntimeError("build the HIP library first: %s is missing" % HIP_LIBRARY)
+    tmp = BACKEND_LIBRARY + ".tmp"
+    cmd = (["g++"] + BACKEND_FLAGS + ["-I", os.path.join(REPO_ROOT, "include"), "-o", tmp]
+           + [os.path.join(HOST_DIR, s) for s in BACKEND_SOURCES]
+           + ["-L", PACKAGE_DIR, "-lnnforge_hip", "-Wl,-rpath,$ORIGIN"])
+    out = _run(cmd)
+    os.replace(tmp, BACKEND_LIBRARY)
+    if verbose and out.strip():
+        print(out)
+    return BACKEND_LIBRARY
+
+
 def build_all(verbose=False):
-    built = [build_hip_library(verbose)]
+    built = [build_hip_library(verbose), build_backend_library(verbose)]
     return built
 
 

@@ -1,0 +1,216 @@
+// C bridge over the C++ hip backend (declared in include/nnforge_hip_backend.h).
+#include "nnforge_hip_backend.h"
+#include "nnforge_hip/hip_backend.h"
+
+#include <cstdio>
+#include <cstring>
+#include <exception>
+#include <sstream>
+
+using namespace nnforge;
+
+namespace
+{
+	void copy_text(const std::string& text, char * dst, size_t capacity)
+	{
+		if ((dst == nullptr) || (capacity == 0))
+			return;
+		const size_t n = std::min(text.size(), capacity - 1);
+		std::memcpy(dst, text.data(), n);
+		dst[n] = '\0';
+	}
+
+	network_schema parse_schema(const char * schema_text)
+	{
+		hip::init(); // idempotent: registration ignores duplicates
+		if (schema_text == nullptr)
+			throw neural_network_exception("schema text is null");
+		std::istringstream in(schema_text);
+		network_schema schema;
+		schema.read_proto(in);
+		return schema;
+	}
+
+	std::map<std::string, layer_configuration_specific> input_configs(const nnf_backend_input * inputs, uint32_t input_count)
+	{
+		std::map<std::string, layer_configuration_specific> res;
+		for(uint32_t i = 0; i < input_count; ++i)
+		{
+			std::vector<unsigned int> dims(inputs[i].dimension_sizes, inputs[i].dimension_sizes + inputs[i].dimension_count);
+			res[inputs[i].layer_name] = layer_configuration_specific(inputs[i].feature_map_count, dims);
+		}
+		return res;
+	}
+
+	void describe_plan(const hip::forward_propagation_hip& fp, std::ostream& out)
+	{
+		for(const hip::forward_step& s : fp.get_steps())
+			out << "step: " << (s.fused ? "fused " : "single ") << s.description() << "\n";
+		out << "per_entry_bytes: " << fp.get_per_entry_buffer_bytes() << "\n";
+		out << "max_entry_count: " << fp.get_max_entry_count() << "\n";
+	}
+
+	template<class F> int guarded(F f, char * report, size_t report_capacity)
+	{
+		try
+		{
+			std::ostringstream out;
+			f(out);
+			copy_text(out.str(), report, report_capacity);
+			return 0;
+		}
+		catch (const hip::neural_network_hip_exception& e)
+		{
+			copy_text(e.what(), report, report_capacity);
+			return (e.error_code != 0) ? e.error_code : 1;
+		}
+		catch (const std::exception& e)
+		{
+			copy_text(e.what(), report, report_capacity);
+			return 1;
+		}
+	}
+}
+
+extern "C"
+{
+	int nnf_backend_run_schema(
+		const char* schema_text,
+		const nnf_backend_weights* weights, uint32_t weights_count,
+		const nnf_backend_input* inputs, uint32_t input_count,
+		uint32_t entry_count,
+		nnf_backend_output* outputs, uint32_t output_count,
+		const nnf_backend_options* options,
+		char* report, size_t report_capacity)
+	{
+		return guarded([&](std::ostream& out)
+		{
+			const network_schema schema = parse_schema(schema_text);
+			if ((outputs == nullptr) || (output_count == 0))
+				throw neural_network_exception("No output layers specified for forward_propagation");
+
+			hip::factory_generator_hip generator;
+			generator.apply_default_options();
+			if (options != nullptr)
+			{
+				generator.hip_fuse = options->fuse != 0;
+				generator.hip_dont_share_buffers = options->dont_share_buffers != 0;
+				if (options->max_entry_count > 0)
+					generator.hip_max_entry_count = options->max_entry_count;
+			}
+			generator.initialize();
+			forward_propagation_factory::ptr factory = generator.create_forward_propagation_factory();
+
+			std::vector<std::string> output_names;
+			for(uint32_t i = 0; i < output_count; ++i)
+				output_names.push_back(outputs[i].layer_name);
+			const bool profile = (options != nullptr) && (options->profile != 0);
+			forward_propagation::ptr fp = factory->create(schema, output_names, debug_state::ptr(new debug_state(false)), profile_state::ptr(new profile_state(profile)));
+
+			network_data data;
+			if ((options != nullptr) && options->weights_from_folder)
+				data.read(options->weights_folder);
+			for(uint32_t i = 0; i < weights_count; ++i)
+			{
+				layer_data::ptr d(new layer_data());
+				for(uint32_t c = 0; c < weights[i].chunk_count; ++c)
+					d->push_back(std::vector<float>(weights[i].chunks[c], weights[i].chunks[c] + weights[i].chunk_sizes[c]));
+				data.add(weights[i].layer_name, d);
+			}
+			fp->set_data(data);
+
+			memory_data_bunch_reader reader(entry_count);
+			const std::map<std::string, layer_configuration_specific> configs = input_configs(inputs, input_count);
+			for(uint32_t i = 0; i < input_count; ++i)
+				reader.add(inputs[i].layer_name, configs.find(inputs[i].layer_name)->second, inputs[i].data);
+			memory_data_bunch_writer writer;
+			const forward_propagation::stat st = fp->run(reader, writer);
+
+			for(uint32_t i = 0; i < output_count; ++i)
+			{
+				const std::vector<float>& v = writer.values[outputs[i].layer_name];
+				if (v.size() > outputs[i].capacity_floats)
+					throw neural_network_exception("Output buffer for layer " + std::string(outputs[i].layer_name) + " is too small: " + std::to_string(outputs[i].capacity_floats) + " floats, " + std::to_string(v.size()) + " needed");
+				if (!v.empty())
+					std::memcpy(outputs[i].data, v.data(), v.size() * sizeof(float));
+				outputs[i].written_floats = v.size();
+				out << "output: " << outputs[i].layer_name << " " << writer.config_map[outputs[i].layer_name] << "\n";
+			}
+
+			const hip::forward_propagation_hip * hfp = dynamic_cast<const hip::forward_propagation_hip *>(fp.get());
+			if (hfp != nullptr)
+				describe_plan(*hfp, out);
+			out << "entries: " << st.entry_processed_count << "\n";
+			out << "stat: " << st << "\n";
+			for(const std::pair<const std::string, float>& a : fp->get_last_action_seconds())
+				out << "seconds: " << a.first << " " << a.second << "\n";
+		}, report, report_capacity);
+	}
+
+	int nnf_backend_plan_schema(
+		const char* schema_text,
+		const nnf_backend_input* inputs, uint32_t input_count,
+		const char* const* output_layer_names, uint32_t output_count,
+		const nnf_backend_options* options,
+		uint64_t memory_bytes,
+		char* report, size_t report_capacity)
+	{
+		return guarded([&](std::ostream& out)
+		{
+			const network_schema schema = parse_schema(schema_text);
+			std::vector<std::string> output_names;
+			for(uint32_t i = 0; i < output_count; ++i)
+				output_names.push_back(output_layer_names[i]);
+			const bool fuse = (options == nullptr) || (options->fuse != 0);
+			const bool dont_share = (options != nullptr) && (options->dont_share_buffers != 0);
+			const int max_entries = ((options != nullptr) && (options->max_entry_count > 0)) ? options->max_entry_count : 4096;
+			hip::hip_running_configuration::const_ptr config = hip::hip_running_configuration::create_offline(memory_bytes, 0.9F, fuse, dont_share, max_entries);
+			hip::forward_propagation_hip fp(schema, output_names, debug_state::ptr(new debug_state(false)), profile_state::ptr(new profile_state(false)), config);
+			fp.set_input_configuration_specific(input_configs(inputs, input_count));
+			describe_plan(fp, out);
+		}, report, report_capacity);
+	}
+
+	int nnf_backend_rewrite_schema(const char* schema_text, char* out_text, size_t out_capacity)
+	{
+		return guarded([&](std::ostream& out)
+		{
+			const network_schema schema = parse_schema(schema_text);
+			schema.write_proto(out);
+		}, out_text, out_capacity);
+	}
+
+	int nnf_backend_write_weights(const char* folder, const nnf_backend_weights* weights, uint32_t weights_count, char* report, size_t report_capacity)
+	{
+		return guarded([&](std::ostream&)
+		{
+			network_data data;
+			for(uint32_t i = 0; i < weights_count; ++i)
+			{
+				layer_data::ptr d(new layer_data());
+				for(uint32_t c = 0; c < weights[i].chunk_count; ++c)
+					d->push_back(std::vector<float>(weights[i].chunks[c], weights[i].chunks[c] + weights[i].chunk_sizes[c]));
+				data.add(weights[i].layer_name, d);
+			}
+			data.write(folder);
+		}, report, report_capacity);
+	}
+
+	int nnf_backend_read_weights(const char* folder, const char* layer_name, uint32_t chunk_count, const uint32_t* chunk_sizes, float* const* chunks, char* report, size_t report_capacity)
+	{
+		return guarded([&](std::ostream&)
+		{
+			network_data data;
+			data.read(folder);
+			layer_data::ptr d = data.get(layer_name);
+			if (d->size() != chunk_count)
+				throw neural_network_exception("data weight vector count " + std::to_string(d->size()) + " doesn't satisfy layer configuration " + std::to_string(chunk_count));
+			for(uint32_t c = 0; c < chunk_count; ++c)
+			{
+				if ((*d)[c].size() != chunk_sizes[c])
+					throw neural_network_exception("data weight count " + std::to_string((*d)[c].size()) + " for vector " + std::to_string(c) + " doesn't satisfy layer configuration " + std::to_string(chunk_sizes[c]));
+				std::memcpy(chunks[c], (*d)[c].data(), chunk_sizes[c] * sizeof(float));
+			}
+		}, report, report_capacity);
+	}
+}

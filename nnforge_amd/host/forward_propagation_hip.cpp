@@ -1,0 +1,669 @@
+// forward_propagation for one MI355X: plans the launches (fusing runs of element-wise layers),
+// plans the device buffers (liveness-based sharing, in-place where a tester allows it), then
+// streams packets of entries through the plan.
+#include "nnforge_hip/hip_backend.h"
+
+#include <algorithm>
+#include <chrono>
+#include <cstring>
+#include <iostream>
+#include <sstream>
+
+namespace nnforge
+{
+	namespace hip
+	{
+		bool get_add_alpha(const layer_tester_hip& tester, float& alpha); // hip_testers.cpp
+
+		std::string forward_step::description() const
+		{
+			std::string s;
+			for(size_t i = 0; i < layer_names.size(); ++i)
+				s += (i == 0 ? "" : "+") + layer_names[i];
+			s += " <- ";
+			for(size_t i = 0; i < input_names.size(); ++i)
+				s += (i == 0 ? "" : ", ") + input_names[i];
+			return s;
+		}
+
+		namespace
+		{
+			// one input tensor of a group under construction and the layers applied to it before the join
+			struct pending_arm
+			{
+				std::string source;
+				std::vector<std::string> ops;
+			};
+
+			// a group of element-wise layers whose result has not been written to memory yet
+			struct pending_group
+			{
+				std::vector<pending_arm> arms;
+				std::string add_layer_name; // empty: no join
+				std::vector<std::string> tail;
+
+				size_t op_count() const
+				{
+					size_t n = tail.size();
+					for(const pending_arm& a : arms)
+						n += a.ops.size();
+					return n;
+				}
+			};
+
+			struct step_plan
+			{
+				forward_step info;
+				layer_tester_hip::ptr tester;        // single-layer steps
+				nnf_hip_chain_desc desc;             // fused steps (entry_count filled per packet)
+				std::vector<std::string> chunk_layers; // fused steps: layers whose weight chunks are concatenated into chunk_ptrs
+				int output_buffer;
+				std::vector<int> input_buffers;
+			};
+
+			bool is_unary_elementwise(const std::string& type)
+			{
+				return (type == batch_norm_layer::layer_type_name) || (type == rectified_linear_layer::layer_type_name)
+					|| (type == parametric_rectified_linear_layer::layer_type_name) || (type == exponential_linear_layer::layer_type_name)
+					|| (type == sigmoid_layer::layer_type_name) || (type == hyperbolic_tangent_layer::layer_type_name);
+			}
+
+			struct pinned_buffer
+			{
+				explicit pinned_buffer(size_t bytes) : ptr(nullptr), bytes(bytes)
+				{
+					hip_safe_call(nnf_hip_host_malloc(&ptr, bytes));
+				}
+				~pinned_buffer()
+				{
+					if (ptr != nullptr)
+						nnf_hip_host_free(ptr);
+				}
+				pinned_buffer(const pinned_buffer&) = delete;
+				pinned_buffer& operator=(const pinned_buffer&) = delete;
+				void * ptr;
+				size_t bytes;
+			};
+
+			struct hip_event
+			{
+				hip_event() : ev(nullptr) { hip_safe_call(nnf_hip_event_create(&ev)); }
+				~hip_event() { if (ev != nullptr) nnf_hip_event_destroy(ev); }
+				hip_event(const hip_event&) = delete;
+				hip_event& operator=(const hip_event&) = delete;
+				void * ev;
+			};
+		}
+
+		struct forward_propagation_hip::impl
+		{
+			std::vector<layer::const_ptr> exec_layers; // layers with inputs, execution order
+			std::map<std::string, layer_tester_hip::ptr> testers;
+			std::map<std::string, std::vector<hip_linear_buffer_device::const_ptr> > weights;
+			network_data::const_ptr host_data;
+
+			std::vector<step_plan> plans;
+			std::vector<size_t> buffer_floats_per_entry;   // planned device buffers
+			std::map<std::string, int> value_to_buffer;    // data layers, step outputs
+			void * stream = nullptr;
+
+			~impl()
+			{
+				if (stream != nullptr)
+					nnf_hip_stream_destroy(stream);
+			}
+		};
+
+		forward_propagation_hip::forward_propagation_hip(
+			const network_schema& schema,
+			const std::vector<std::string>& output_layer_names,
+			debug_state::ptr debug,
+			profile_state::ptr profile,
+			hip_running_configuration::const_ptr hip_config)
+			: forward_propagation(schema, output_layer_names, debug, profile)
+			, p(new impl())
+			, hip_config(hip_config)
+			, per_entry_bytes(0)
+			, max_entry_count(0)
+		{
+			for(const layer::const_ptr& l : this->schema->get_layers_in_forward_propagation_order())
+			{
+				if (l->input_layer_instance_names.empty())
+				{
+					if (l->get_type_name() != data_layer::layer_type_name)
+						throw neural_network_exception("Layer " + l->instance_name + " of type " + l->get_type_name() + " has no inputs");
+					continue;
+				}
+				// fails here, at construction, for a layer type without a registered tester
+				layer_testing_schema_factory::get_singleton().create_testing_schema_layer(l);
+				p->exec_layers.push_back(l);
+			}
+		}
+
+		forward_propagation_hip::~forward_propagation_hip()
+		{
+		}
+
+		void forward_propagation_hip::actual_set_data(network_data::const_ptr data)
+		{
+			p->host_data = data;
+			p->weights.clear();
+			if (hip_config->is_offline())
+				return;
+			hip_config->set_device();
+			for(const layer::const_ptr& l : p->exec_layers)
+			{
+				layer_data::ptr d = data->find(l->instance_name);
+				if (!d)
+					continue;
+				std::map<std::string, layer_tester_hip::ptr>::const_iterator t = p->testers.find(l->instance_name);
+				if (t != p->testers.end())
+					p->weights[l->instance_name] = t->second->get_data(d);
+			}
+		}
+
+		void forward_propagation_hip::actual_clear_data()
+		{
+			p->host_data.reset();
+			p->weights.clear();
+		}
+
+		void forward_propagation_hip::layer_config_map_modified()
+		{
+			hip_config->set_device();
+
+			// testers for the new shapes
+			p->testers.clear();
+			for(const layer::const_ptr& l : p->exec_layers)
+			{
+				std::vector<layer_configuration_specific> inputs;
+				for(const std::string& input : l->input_layer_instance_names)
+					inputs.push_back(layer_config_map[input]);
+				layer_testing_schema::ptr ts = layer_testing_schema_factory::get_singleton().create_testing_schema_layer(l);
+				p->testers[l->instance_name] = ts->create_tester(inputs, layer_config_map[l->instance_name], hip_config);
+			}
+			if (p->host_data)
+				actual_set_data(p->host_data);
+
+			// ---- launch plan: fuse runs of element-wise layers ----------------------------------
+			const std::set<std::string> outputs(output_layer_names.begin(), output_layer_names.end());
+			std::map<std::string, pending_group> pending;
+			std::vector<std::pair<std::string, pending_group> > groups; // materialized, in execution order
+			std::vector<std::pair<std::string, bool> > step_order;      // (layer name, is_group)
+
+			auto materialize = [&](const std::string& name)
+			{
+				std::map<std::string, pending_group>::iterator it = pending.find(name);
+				if (it == pending.end())
+					return;
+				groups.push_back(std::make_pair(name, it->second));
+				step_order.push_back(std::make_pair(name, true));
+				pending.erase(it);
+			};
+			auto absorbable = [&](const std::string& producer, const layer_configuration_specific& consumer_config) -> bool
+			{
+				return hip_config->fuse_layers
+					&& (pending.find(producer) != pending.end())
+					&& (this->schema->get_consumer_count(producer) == 1)
+					&& (outputs.find(producer) == outputs.end())
+					&& (layer_config_map[producer] == consumer_config);
+			};
+
+			for(const layer::const_ptr& l : p->exec_layers)
+			{
+				const std::string& name = l->instance_name;
+				const std::string type = l->get_type_name();
+				const layer_configuration_specific& config = layer_config_map[name];
+				bool grouped = false;
+
+				if (is_unary_elementwise(type))
+				{
+					const std::string& producer = l->input_layer_instance_names.at(0);
+					pending_group g;
+					if (absorbable(producer, config) && (pending[producer].op_count() + 1 <= NNF_HIP_MAX_OPS))
+					{
+						g = pending[producer];
+						pending.erase(producer);
+						if (g.add_layer_name.empty())
+							g.arms[0].ops.push_back(name);
+						else
+							g.tail.push_back(name);
+					}
+					else
+					{
+						materialize(producer);
+						pending_arm a;
+						a.source = producer;
+						a.ops.push_back(name);
+						g.arms.push_back(a);
+					}
+					pending[name] = g;
+					grouped = true;
+				}
+				else if ((type == add_layer::layer_type_name) && (l->input_layer_instance_names.size() <= NNF_HIP_MAX_INPUTS) && hip_config->fuse_layers)
+				{
+					bool same_configs = true;
+					for(const std::string& producer : l->input_layer_instance_names)
+						same_configs = same_configs && (layer_config_map[producer] == config);
+					pending_group g;
+					g.add_layer_name = name;
+					size_t ops = 0;
+					for(const std::string& producer : l->input_layer_instance_names)
+					{
+						pending_arm a;
+						a.source = producer;
+						if (same_configs && absorbable(producer, config) && pending[producer].add_layer_name.empty()
+							&& (ops + pending[producer].op_count() <= NNF_HIP_MAX_OPS))
+						{
+							a = pending[producer].arms[0];
+							ops += a.ops.size();
+							pending.erase(producer);
+						}
+						else
+							materialize(producer);
+						g.arms.push_back(a);
+					}
+					pending[name] = g;
+					grouped = true;
+				}
+
+				if (!grouped)
+				{
+					for(const std::string& producer : l->input_layer_instance_names)
+						materialize(producer);
+					step_order.push_back(std::make_pair(name, false));
+				}
+				else if ((outputs.find(name) != outputs.end()) || (this->schema->get_consumer_count(name) != 1))
+					materialize(name);
+			}
+			// anything still pending feeds nothing (cannot happen for a reduced schema) - write it out anyway
+			while (!pending.empty())
+				materialize(pending.begin()->first);
+
+			// ---- steps ---------------------------------------------------------------------------
+			p->plans.clear();
+			steps.clear();
+			std::map<std::string, const pending_group *> group_by_name;
+			for(const std::pair<std::string, pending_group>& g : groups)
+				group_by_name[g.first] = &g.second;
+
+			for(const std::pair<std::string, bool>& so : step_order)
+			{
+				step_plan plan;
+				std::memset(&plan.desc, 0, sizeof(plan.desc));
+				plan.output_buffer = -1;
+				const std::string& name = so.first;
+				const layer_configuration_specific& config = layer_config_map[name];
+				if (!so.second)
+				{
+					layer::const_ptr l = this->schema->get_layer(name);
+					plan.info.layer_names.push_back(name);
+					plan.info.input_names = l->input_layer_instance_names;
+					plan.info.fused = false;
+					plan.tester = p->testers[name];
+				}
+				else
+				{
+					const pending_group& g = *group_by_name[name];
+					const bool single_layer = (g.op_count() + (g.add_layer_name.empty() ? 0 : 1)) == 1;
+					for(const pending_arm& a : g.arms)
+					{
+						plan.info.input_names.push_back(a.source);
+						for(const std::string& op : a.ops)
+							plan.info.layer_names.push_back(op);
+					}
+					if (!g.add_layer_name.empty())
+						plan.info.layer_names.push_back(g.add_layer_name);
+					for(const std::string& op : g.tail)
+						plan.info.layer_names.push_back(op);
+					if (single_layer)
+					{
+						// a group of one layer is that layer's own tester
+						plan.info.fused = false;
+						plan.tester = p->testers[plan.info.layer_names[0]];
+					}
+					else
+					{
+						plan.info.fused = true;
+						nnf_hip_chain_desc& d = plan.desc;
+						d.feature_map_count = config.feature_map_count;
+						d.neuron_count_per_feature_map = config.get_neuron_count_per_feature_map();
+						d.input_count = static_cast<uint32_t>(g.arms.size());
+						d.has_add = g.add_layer_name.empty() ? 0u : 1u;
+						d.add_alpha = 1.0F;
+						if (d.has_add)
+							get_add_alpha(*p->testers[g.add_layer_name], d.add_alpha);
+						uint32_t op_index = 0;
+						int chunk_index = 0;
+						auto push_op = [&](const std::string& layer_name)
+						{
+							nnf_hip_op& op = d.ops[op_index++];
+							const int chunks = p->testers[layer_name]->get_chain_op(op);
+							if (chunks < 0)
+								throw neural_network_exception("Layer " + layer_name + " cannot be part of a fused group");
+							op.chunk = chunk_index;
+							if (chunks > 0)
+							{
+								plan.chunk_layers.push_back(layer_name);
+								chunk_index += chunks;
+							}
+						};
+						for(size_t j = 0; j < g.arms.size(); ++j)
+						{
+							d.arm_op_count[j] = static_cast<uint32_t>(g.arms[j].ops.size());
+							for(const std::string& op : g.arms[j].ops)
+								push_op(op);
+						}
+						d.tail_op_count = static_cast<uint32_t>(g.tail.size());
+						for(const std::string& op : g.tail)
+							push_op(op);
+					}
+				}
+				p->plans.push_back(plan);
+				steps.push_back(plan.info);
+			}
+
+			// ---- buffers: dedicated for data and output layers, shared by liveness for the rest --
+			p->buffer_floats_per_entry.clear();
+			p->value_to_buffer.clear();
+			auto new_buffer = [&](size_t floats_per_entry) -> int
+			{
+				p->buffer_floats_per_entry.push_back(floats_per_entry);
+				return static_cast<int>(p->buffer_floats_per_entry.size()) - 1;
+			};
+			for(const std::string& n : data_layer_names)
+				p->value_to_buffer[n] = new_buffer(layer_config_map[n].get_neuron_count());
+
+			std::map<std::string, size_t> last_use;
+			for(size_t i = 0; i < p->plans.size(); ++i)
+				for(const std::string& in : p->plans[i].info.input_names)
+					last_use[in] = i;
+
+			std::vector<int> free_buffers;
+			std::set<int> shareable; // buffers that hold intermediate values
+			for(size_t i = 0; i < p->plans.size(); ++i)
+			{
+				step_plan& plan = p->plans[i];
+				const std::string& out_name = plan.info.layer_names.back();
+				const size_t out_floats = layer_config_map[out_name].get_neuron_count();
+				for(const std::string& in : plan.info.input_names)
+					plan.input_buffers.push_back(p->value_to_buffer.at(in));
+
+				const bool dedicated = (outputs.find(out_name) != outputs.end()) || hip_config->dont_share_buffers;
+				int chosen = -1;
+				if (!dedicated)
+				{
+					// in place: the first input dies here, nothing else reads its buffer in this step, same size
+					const int can_write = plan.info.fused ? 0 : plan.tester->get_input_index_layer_can_write();
+					if (can_write == 0)
+					{
+						const int b0 = plan.input_buffers[0];
+						const bool dies_here = last_use[plan.info.input_names[0]] == i;
+						const bool unique = std::count(plan.input_buffers.begin(), plan.input_buffers.end(), b0) == 1;
+						if (dies_here && unique && (shareable.find(b0) != shareable.end()) && (p->buffer_floats_per_entry[b0] == out_floats))
+							chosen = b0;
+					}
+					if (chosen < 0)
+					{
+						// smallest free buffer that is large enough
+						std::vector<int>::iterator best = free_buffers.end();
+						for(std::vector<int>::iterator it = free_buffers.begin(); it != free_buffers.end(); ++it)
+						{
+							if (p->buffer_floats_per_entry[*it] < out_floats)
+								continue;
+							if ((best == free_buffers.end()) || (p->buffer_floats_per_entry[*it] < p->buffer_floats_per_entry[*best]))
+								best = it;
+						}
+						if (best != free_buffers.end())
+						{
+							chosen = *best;
+							free_buffers.erase(best);
+						}
+					}
+				}
+				if (chosen < 0)
+				{
+					chosen = new_buffer(out_floats);
+					if (!dedicated)
+						shareable.insert(chosen);
+				}
+				plan.output_buffer = chosen;
+				p->value_to_buffer[out_name] = chosen;
+
+				// inputs that die here return to the pool (unless just reused in place)
+				for(size_t j = 0; j < plan.info.input_names.size(); ++j)
+				{
+					const int b = plan.input_buffers[j];
+					if ((last_use[plan.info.input_names[j]] == i) && (b != chosen) && (shareable.find(b) != shareable.end())
+						&& (std::find(free_buffers.begin(), free_buffers.end(), b) == free_buffers.end()))
+						free_buffers.push_back(b);
+				}
+			}
+
+			per_entry_bytes = 0;
+			for(size_t floats : p->buffer_floats_per_entry)
+				per_entry_bytes += floats * sizeof(float);
+
+			// packet size from the memory budget (nnforge/plain/forward_propagation_plain.cpp:403-444)
+			size_t weight_bytes = 0;
+			for(const std::pair<const std::string, std::vector<hip_linear_buffer_device::const_ptr> >& w : p->weights)
+				for(const hip_linear_buffer_device::const_ptr& b : w.second)
+					weight_bytes += b->get_size();
+			const size_t budget = hip_config->get_max_bytes();
+			if ((per_entry_bytes == 0) || (budget <= weight_bytes) || ((budget - weight_bytes) / per_entry_bytes == 0))
+				throw neural_network_exception("Insufficient memory to do forward prop for even one sample");
+			const size_t fit = (budget - weight_bytes) / per_entry_bytes;
+			max_entry_count = static_cast<unsigned int>(std::min<size_t>(fit, static_cast<size_t>(std::max(1, hip_config->max_entry_count))));
+
+			if (debug->is_debug())
+			{
+				std::cout << "forward prop hip: " << p->plans.size() << " launches, " << p->buffer_floats_per_entry.size() << " buffers, "
+					<< per_entry_bytes << " bytes per entry, max " << max_entry_count << " entries per packet" << std::endl;
+				for(const forward_step& s : steps)
+					std::cout << "  " << (s.fused ? "[fused] " : "        ") << s.description() << std::endl;
+			}
+		}
+
+		void forward_propagation_hip::actual_run(
+			structured_data_bunch_reader& reader,
+			structured_data_bunch_writer& writer,
+			unsigned int& entries_processed,
+			std::map<std::string, float>& action_seconds,
+			float& idle_seconds)
+		{
+			if (hip_config->is_offline())
+				throw neural_network_exception("This forward_propagation_hip was created for planning only (offline configuration): it cannot run");
+			hip_config->set_device();
+			if (p->stream == nullptr)
+				hip_safe_call(nnf_hip_stream_create(&p->stream));
+			for(const layer::const_ptr& l : p->exec_layers)
+				if (!l->is_empty_data() && (p->weights.find(l->instance_name) == p->weights.end()))
+					throw neural_network_exception("No data found with layer name " + l->instance_name);
+
+			unsigned int packet = max_entry_count;
+			const int reader_entry_count = reader.get_entry_count();
+			if (reader_entry_count > 0)
+				packet = std::min(packet, static_cast<unsigned int>(reader_entry_count));
+
+			// device buffers for one packet, pinned staging for inputs and outputs
+			std::vector<hip_linear_buffer_device::ptr> buffers;
+			for(size_t floats : p->buffer_floats_per_entry)
+				buffers.push_back(hip_linear_buffer_device::ptr(new hip_linear_buffer_device(floats * sizeof(float) * packet)));
+			std::map<std::string, std::unique_ptr<pinned_buffer> > staging;
+			for(const std::string& n : data_layer_names)
+				staging[n].reset(new pinned_buffer(static_cast<size_t>(layer_config_map[n].get_neuron_count()) * sizeof(float) * packet));
+			for(const std::string& n : output_layer_names)
+				if (staging.find(n) == staging.end())
+					staging[n].reset(new pinned_buffer(static_cast<size_t>(layer_config_map[n].get_neuron_count()) * sizeof(float) * packet));
+
+			// weight pointers of the fused steps
+			std::vector<std::vector<const float *> > chunk_ptrs(p->plans.size());
+			for(size_t i = 0; i < p->plans.size(); ++i)
+				for(const std::string& layer_name : p->plans[i].chunk_layers)
+					for(const hip_linear_buffer_device::const_ptr& b : p->weights.at(layer_name))
+						chunk_ptrs[i].push_back(static_cast<const float *>(*b));
+
+			const bool profiling = profile->is_profile();
+			std::vector<std::unique_ptr<hip_event> > events;
+			if (profiling)
+				for(size_t i = 0; i <= p->plans.size(); ++i)
+					events.emplace_back(new hip_event());
+
+			const std::vector<hip_linear_buffer_device::const_ptr> none;
+			unsigned int processed = 0;
+			double idle = 0.0;
+			action_seconds.clear();
+			for(;;)
+			{
+				// read a packet
+				const std::chrono::high_resolution_clock::time_point read_start = std::chrono::high_resolution_clock::now();
+				unsigned int entries_read = 0;
+				for(; entries_read < packet; ++entries_read)
+				{
+					std::map<std::string, float *> data_map;
+					for(const std::string& n : data_layer_names)
+						data_map[n] = static_cast<float *>(staging[n]->ptr) + static_cast<size_t>(entries_read) * layer_config_map[n].get_neuron_count();
+					if (!reader.read(processed + entries_read, data_map))
+						break;
+				}
+				idle += std::chrono::duration<double>(std::chrono::high_resolution_clock::now() - read_start).count();
+				if (entries_read == 0)
+					break;
+
+				for(const std::string& n : data_layer_names)
+					hip_safe_call(nnf_hip_memcpy_h2d(*buffers[p->value_to_buffer[n]], staging[n]->ptr,
+						static_cast<size_t>(layer_config_map[n].get_neuron_count()) * sizeof(float) * entries_read, p->stream));
+
+				for(size_t i = 0; i < p->plans.size(); ++i)
+				{
+					step_plan& plan = p->plans[i];
+					if (profiling)
+						hip_safe_call(nnf_hip_event_record(events[i]->ev, p->stream));
+					std::vector<hip_linear_buffer_device::const_ptr> inputs;
+					for(int b : plan.input_buffers)
+						inputs.push_back(buffers[b]);
+					if (plan.info.fused)
+					{
+						plan.desc.entry_count = entries_read;
+						std::vector<const float *> in_ptrs;
+						for(const hip_linear_buffer_device::const_ptr& b : inputs)
+							in_ptrs.push_back(static_cast<const float *>(*b));
+						hip_safe_call(nnf_hip_chain_forward(p->stream, &plan.desc, *buffers[plan.output_buffer], in_ptrs.data(),
+							chunk_ptrs[i].empty() ? nullptr : chunk_ptrs[i].data()));
+					}
+					else
+					{
+						const std::string& layer_name = plan.info.layer_names[0];
+						std::map<std::string, std::vector<hip_linear_buffer_device::const_ptr> >::const_iterator w = p->weights.find(layer_name);
+						plan.tester->enqueue_forward_propagation(p->stream, buffers[plan.output_buffer], none,
+							(w == p->weights.end()) ? none : w->second, none, inputs, none,
+							hip_linear_buffer_device::ptr(), hip_linear_buffer_device::ptr(), entries_read);
+					}
+				}
+				if (profiling)
+					hip_safe_call(nnf_hip_event_record(events[p->plans.size()]->ev, p->stream));
+
+				for(const std::string& n : output_layer_names)
+					hip_safe_call(nnf_hip_memcpy_d2h(staging[n]->ptr, *buffers[p->value_to_buffer.at(n)],
+						static_cast<size_t>(layer_config_map[n].get_neuron_count()) * sizeof(float) * entries_read, p->stream));
+				hip_safe_call(nnf_hip_stream_synchronize(p->stream));
+
+				if (profiling)
+				{
+					for(size_t i = 0; i < p->plans.size(); ++i)
+					{
+						float ms = 0.0F;
+						hip_safe_call(nnf_hip_event_elapsed_ms(&ms, events[i]->ev, events[i + 1]->ev));
+						std::string key;
+						for(const std::string& n : p->plans[i].info.layer_names)
+							key += (key.empty() ? "" : "+") + n;
+						action_seconds[key] += ms * 1.0e-3F;
+					}
+				}
+
+				for(unsigned int e = 0; e < entries_read; ++e)
+				{
+					std::map<std::string, const float *> data_map;
+					for(const std::string& n : output_layer_names)
+						data_map[n] = static_cast<const float *>(staging[n]->ptr) + static_cast<size_t>(e) * layer_config_map[n].get_neuron_count();
+					writer.write(processed + e, data_map);
+				}
+
+				processed += entries_read;
+				if (entries_read < packet)
+					break;
+			}
+
+			entries_processed = processed;
+			idle_seconds = static_cast<float>(idle);
+		}
+
+		// ---- factories -------------------------------------------------------------------------
+
+		forward_propagation::ptr forward_propagation_hip_factory::create(
+			const network_schema& schema,
+			const std::vector<std::string>& output_layer_names,
+			debug_state::ptr debug,
+			profile_state::ptr profile) const
+		{
+			return forward_propagation::ptr(new forward_propagation_hip(schema, output_layer_names, debug, profile, hip_config));
+		}
+
+		factory_generator_hip::factory_generator_hip()
+			: hip_device_id(0)
+			, hip_max_global_memory_usage_ratio(0.9F)
+			, hip_fuse(true)
+			, hip_dont_share_buffers(false)
+			, hip_max_entry_count(4096)
+		{
+		}
+
+		void factory_generator_hip::initialize()
+		{
+			hip::init();
+			hip_config = hip_running_configuration::const_ptr(new hip_running_configuration(
+				hip_device_id, hip_max_global_memory_usage_ratio, hip_fuse, hip_dont_share_buffers, hip_max_entry_count));
+		}
+
+		forward_propagation_factory::ptr factory_generator_hip::create_forward_propagation_factory() const
+		{
+			if (!hip_config)
+				throw neural_network_exception("factory_generator_hip::initialize() has not been called");
+			return forward_propagation_factory::ptr(new forward_propagation_hip_factory(hip_config));
+		}
+
+		backward_propagation_factory::ptr factory_generator_hip::create_backward_propagation_factory() const
+		{
+			throw neural_network_exception("The hip backend implements inference only: backward propagation is not supported");
+		}
+
+		void factory_generator_hip::info() const
+		{
+			if (hip_config)
+				std::cout << *hip_config;
+		}
+
+		std::vector<bool_option> factory_generator_hip::get_bool_options()
+		{
+			std::vector<bool_option> res;
+			res.push_back(bool_option("hip_fuse", &hip_fuse, true, "Fuse runs of element-wise layers (BatchNorm, activations, Add) into single kernel launches"));
+			res.push_back(bool_option("hip_dont_share_buffers", &hip_dont_share_buffers, false, "Don't share buffers between layers. Switch it on if you suspect a bug in there"));
+			return res;
+		}
+
+		std::vector<float_option> factory_generator_hip::get_float_options()
+		{
+			std::vector<float_option> res;
+			res.push_back(float_option("hip_max_global_memory_usage_ratio,G", &hip_max_global_memory_usage_ratio, 0.9F, "Part of the global memory to be used by the backend"));
+			return res;
+		}
+
+		std::vector<int_option> factory_generator_hip::get_int_options()
+		{
+			std::vector<int_option> res;
+			res.push_back(int_option("hip_device_id,D", &hip_device_id, 0, "HIP device ID"));
+			res.push_back(int_option("hip_max_entry_count", &hip_max_entry_count, 4096, "Upper bound of entries processed per packet"));
+			return res;
+		}
+	}
+}

@@ -1,0 +1,394 @@
+#include "nnforge_hip/layers.h"
+
+#include <cstdio>
+#include <sstream>
+
+namespace nnforge
+{
+	namespace
+	{
+		float neuron_count_of(const std::vector<layer_configuration_specific>& configs)
+		{
+			if (configs.empty())
+				throw neural_network_exception("flops requested for a layer without input configuration");
+			return static_cast<float>(configs[0].get_neuron_count());
+		}
+
+		std::string fixed3(float v)
+		{
+			char buf[64];
+			std::snprintf(buf, sizeof(buf), "%.3f", static_cast<double>(v));
+			return buf;
+		}
+
+		std::string float_text(float v)
+		{
+			char buf[64];
+			std::snprintf(buf, sizeof(buf), "%.9g", static_cast<double>(v));
+			return buf;
+		}
+	}
+
+	// ---- data ------------------------------------------------------------------------------
+
+	const std::string data_layer::layer_type_name = "Data";
+	layer::ptr data_layer::clone() const { return layer::ptr(new data_layer(*this)); }
+	std::string data_layer::get_type_name() const { return layer_type_name; }
+
+	// ---- batch norm ------------------------------------------------------------------------
+
+	const std::string batch_norm_layer::layer_type_name = "BatchNorm";
+	const float batch_norm_layer::default_batch_normalization_epsilon = 2.0e-5F;
+
+	batch_norm_layer::batch_norm_layer(unsigned int feature_map_count, float epsilon)
+		: feature_map_count(feature_map_count), epsilon(epsilon)
+	{
+		check();
+	}
+
+	void batch_norm_layer::check()
+	{
+		if (feature_map_count == 0)
+			throw neural_network_exception("Feature map count should be > 0 for batch norm layer");
+	}
+
+	layer::ptr batch_norm_layer::clone() const { return layer::ptr(new batch_norm_layer(*this)); }
+	std::string batch_norm_layer::get_type_name() const { return layer_type_name; }
+
+	float batch_norm_layer::get_forward_flops_per_entry(const std::vector<layer_configuration_specific>& configs) const
+	{
+		return neuron_count_of(configs) * 5.0F; // the reference's count (nnforge/batch_norm_layer.cpp:66)
+	}
+
+	void batch_norm_layer::read_params(const schema_param_block * block)
+	{
+		if (block == nullptr)
+			throw neural_network_exception("No batch_norm_param specified for layer " + instance_name + " of type " + layer_type_name);
+		feature_map_count = block->require_uint("feature_map_count", "batch_norm_param of layer " + instance_name);
+		epsilon = block->get_float("epsilon", default_batch_normalization_epsilon);
+		check();
+	}
+
+	void batch_norm_layer::write_params(std::ostream& out, const std::string& indent) const
+	{
+		out << indent << "feature_map_count: " << feature_map_count << "\n";
+		if (epsilon != default_batch_normalization_epsilon)
+			out << indent << "epsilon: " << float_text(epsilon) << "\n";
+	}
+
+	data_config batch_norm_layer::get_data_config() const
+	{
+		return data_config(4, feature_map_count);
+	}
+
+	void batch_norm_layer::initialize_data(layer_data& data) const
+	{
+		check_layer_data_consistency(data);
+		std::fill(data[0].begin(), data[0].end(), 1.0F);
+		std::fill(data[1].begin(), data[1].end(), 0.0F);
+		std::fill(data[2].begin(), data[2].end(), 0.0F);
+		std::fill(data[3].begin(), data[3].end(), 1.0F);
+	}
+
+	std::vector<std::string> batch_norm_layer::get_parameter_strings() const
+	{
+		std::stringstream ss;
+		ss << "fm " << feature_map_count;
+		if (epsilon != default_batch_normalization_epsilon)
+			ss << ", epsilon = " << epsilon;
+		return std::vector<std::string>(1, ss.str());
+	}
+
+	// ---- ReLU ------------------------------------------------------------------------------
+
+	const std::string rectified_linear_layer::layer_type_name = "ReLU";
+
+	rectified_linear_layer::rectified_linear_layer(float negative_slope) : negative_slope(negative_slope) {}
+	layer::ptr rectified_linear_layer::clone() const { return layer::ptr(new rectified_linear_layer(*this)); }
+	std::string rectified_linear_layer::get_type_name() const { return layer_type_name; }
+
+	float rectified_linear_layer::get_forward_flops_per_entry(const std::vector<layer_configuration_specific>& configs) const
+	{
+		return neuron_count_of(configs);
+	}
+
+	void rectified_linear_layer::read_params(const schema_param_block * block)
+	{
+		negative_slope = (block != nullptr) ? block->get_float("negative_slope", 0.0F) : 0.0F;
+	}
+
+	void rectified_linear_layer::write_params(std::ostream& out, const std::string& indent) const
+	{
+		if (negative_slope != 0.0F)
+			out << indent << "negative_slope: " << float_text(negative_slope) << "\n";
+	}
+
+	std::vector<std::string> rectified_linear_layer::get_parameter_strings() const
+	{
+		std::vector<std::string> res;
+		if (negative_slope != 0.0F)
+			res.push_back("negative slope " + float_text(negative_slope));
+		return res;
+	}
+
+	// ---- PReLU -----------------------------------------------------------------------------
+
+	const std::string parametric_rectified_linear_layer::layer_type_name = "PReLU";
+
+	parametric_rectified_linear_layer::parametric_rectified_linear_layer(unsigned int feature_map_count)
+		: feature_map_count(feature_map_count)
+	{
+		check();
+	}
+
+	void parametric_rectified_linear_layer::check()
+	{
+		if (feature_map_count == 0)
+			throw neural_network_exception("Feature map count should be > 0 for parametric rectified linear layer");
+	}
+
+	layer::ptr parametric_rectified_linear_layer::clone() const { return layer::ptr(new parametric_rectified_linear_layer(*this)); }
+	std::string parametric_rectified_linear_layer::get_type_name() const { return layer_type_name; }
+
+	float parametric_rectified_linear_layer::get_forward_flops_per_entry(const std::vector<layer_configuration_specific>& configs) const
+	{
+		return neuron_count_of(configs) * 2.0F;
+	}
+
+	void parametric_rectified_linear_layer::read_params(const schema_param_block * block)
+	{
+		if (block == nullptr)
+			throw neural_network_exception("No prelu_param specified for layer " + instance_name + " of type " + layer_type_name);
+		feature_map_count = block->require_uint("feature_map_count", "prelu_param of layer " + instance_name);
+		check();
+	}
+
+	void parametric_rectified_linear_layer::write_params(std::ostream& out, const std::string& indent) const
+	{
+		out << indent << "feature_map_count: " << feature_map_count << "\n";
+	}
+
+	data_config parametric_rectified_linear_layer::get_data_config() const
+	{
+		return data_config(1, feature_map_count);
+	}
+
+	void parametric_rectified_linear_layer::initialize_data(layer_data& data) const
+	{
+		check_layer_data_consistency(data);
+		std::fill(data[0].begin(), data[0].end(), 0.25F);
+	}
+
+	std::vector<std::string> parametric_rectified_linear_layer::get_parameter_strings() const
+	{
+		return std::vector<std::string>(1, "fm " + std::to_string(feature_map_count));
+	}
+
+	// ---- ELU, Sigmoid ----------------------------------------------------------------------
+
+	const std::string exponential_linear_layer::layer_type_name = "ELU";
+	layer::ptr exponential_linear_layer::clone() const { return layer::ptr(new exponential_linear_layer(*this)); }
+	std::string exponential_linear_layer::get_type_name() const { return layer_type_name; }
+	float exponential_linear_layer::get_forward_flops_per_entry(const std::vector<layer_configuration_specific>& configs) const
+	{
+		return neuron_count_of(configs) * 2.0F;
+	}
+
+	const std::string sigmoid_layer::layer_type_name = "Sigmoid";
+	layer::ptr sigmoid_layer::clone() const { return layer::ptr(new sigmoid_layer(*this)); }
+	std::string sigmoid_layer::get_type_name() const { return layer_type_name; }
+	float sigmoid_layer::get_forward_flops_per_entry(const std::vector<layer_configuration_specific>& configs) const
+	{
+		return neuron_count_of(configs) * 4.0F;
+	}
+
+	// ---- TanH ------------------------------------------------------------------------------
+
+	const std::string hyperbolic_tangent_layer::layer_type_name = "TanH";
+
+	hyperbolic_tangent_layer::hyperbolic_tangent_layer(float scale, float steepness) : scale(scale), steepness(steepness) {}
+	layer::ptr hyperbolic_tangent_layer::clone() const { return layer::ptr(new hyperbolic_tangent_layer(*this)); }
+	std::string hyperbolic_tangent_layer::get_type_name() const { return layer_type_name; }
+
+	float hyperbolic_tangent_layer::get_forward_flops_per_entry(const std::vector<layer_configuration_specific>& configs) const
+	{
+		return neuron_count_of(configs) * 6.0F;
+	}
+
+	void hyperbolic_tangent_layer::read_params(const schema_param_block * block)
+	{
+		scale = (block != nullptr) ? block->get_float("scale", 1.0F) : 1.0F;
+		steepness = (block != nullptr) ? block->get_float("steepness", 1.0F) : 1.0F;
+	}
+
+	void hyperbolic_tangent_layer::write_params(std::ostream& out, const std::string& indent) const
+	{
+		if (scale != 1.0F)
+			out << indent << "scale: " << float_text(scale) << "\n";
+		if (steepness != 1.0F)
+			out << indent << "steepness: " << float_text(steepness) << "\n";
+	}
+
+	std::vector<std::string> hyperbolic_tangent_layer::get_parameter_strings() const
+	{
+		std::string s;
+		if (scale != 1.0F)
+			s += "scale " + fixed3(scale);
+		if (steepness != 1.0F)
+			s += std::string(s.empty() ? "" : ", ") + "steepness " + fixed3(steepness);
+		return s.empty() ? std::vector<std::string>() : std::vector<std::string>(1, s);
+	}
+
+	// ---- Add -------------------------------------------------------------------------------
+
+	const std::string add_layer::layer_type_name = "Add";
+
+	add_layer::add_layer(float alpha) : alpha(alpha) {}
+	layer::ptr add_layer::clone() const { return layer::ptr(new add_layer(*this)); }
+	std::string add_layer::get_type_name() const { return layer_type_name; }
+
+	layer_configuration_specific add_layer::get_output_layer_configuration_specific(
+		const std::vector<layer_configuration_specific>& configs) const
+	{
+		if (configs.empty())
+			throw neural_network_exception("Layer " + instance_name + " has no input configuration");
+		const unsigned int neuron_count_per_entry = configs[0].get_neuron_count();
+		for(size_t i = 1; i < configs.size(); ++i)
+		{
+			if (configs[i].get_neuron_count() != neuron_count_per_entry)
+				throw neural_network_exception("Neuron count per entry mismatch in 2 input layers for add_layer");
+		}
+		return configs[0];
+	}
+
+	float add_layer::get_forward_flops_per_entry(const std::vector<layer_configuration_specific>& configs) const
+	{
+		return neuron_count_of(configs) * static_cast<float>(configs.size());
+	}
+
+	void add_layer::read_params(const schema_param_block * block)
+	{
+		alpha = (block != nullptr) ? block->get_float("alpha", 1.0F) : 1.0F;
+	}
+
+	void add_layer::write_params(std::ostream& out, const std::string& indent) const
+	{
+		if (alpha != 1.0F)
+			out << indent << "alpha: " << float_text(alpha) << "\n";
+	}
+
+	std::vector<std::string> add_layer::get_parameter_strings() const
+	{
+		std::vector<std::string> res;
+		if (alpha != 1.0F)
+			res.push_back("alpha " + float_text(alpha));
+		return res;
+	}
+
+	// ---- Softmax ---------------------------------------------------------------------------
+
+	const std::string softmax_layer::layer_type_name = "Softmax";
+	layer::ptr softmax_layer::clone() const { return layer::ptr(new softmax_layer(*this)); }
+	std::string softmax_layer::get_type_name() const { return layer_type_name; }
+
+	float softmax_layer::get_forward_flops_per_entry(const std::vector<layer_configuration_specific>& configs) const
+	{
+		if (configs.empty())
+			throw neural_network_exception("flops requested for a layer without input configuration");
+		return static_cast<float>(configs[0].get_neuron_count_per_feature_map() * (configs[0].feature_map_count * 3 - 1));
+	}
+
+	// ---- AverageSubsampling ----------------------------------------------------------------
+
+	const std::string average_subsampling_layer::layer_type_name = "AverageSubsampling";
+
+	average_subsampling_layer::average_subsampling_layer(const std::vector<unsigned int>& subsampling_sizes, float alpha)
+		: subsampling_sizes(subsampling_sizes), alpha(alpha)
+	{
+		for(unsigned int s : subsampling_sizes)
+			if (s == 0)
+				throw neural_network_exception("window dimension for average subsampling layer may not be zero");
+	}
+
+	layer::ptr average_subsampling_layer::clone() const { return layer::ptr(new average_subsampling_layer(*this)); }
+	std::string average_subsampling_layer::get_type_name() const { return layer_type_name; }
+
+	layer_configuration_specific average_subsampling_layer::get_output_layer_configuration_specific(
+		const std::vector<layer_configuration_specific>& configs) const
+	{
+		if (configs.empty())
+			throw neural_network_exception("Layer " + instance_name + " has no input configuration");
+		const layer_configuration_specific& in = configs[0];
+		if (in.get_dimension_count() != subsampling_sizes.size())
+			throw neural_network_exception("Dimension count in layer (" + std::to_string(subsampling_sizes.size()) + ") and input configuration (" + std::to_string(in.get_dimension_count()) + ") don't match");
+		layer_configuration_specific res(in.feature_map_count);
+		for(size_t i = 0; i < subsampling_sizes.size(); ++i)
+		{
+			if (in.dimension_sizes[i] < subsampling_sizes[i])
+				throw neural_network_exception("Input configuration size (" + std::to_string(in.dimension_sizes[i]) + ") of dimension (" + std::to_string(i) + ") is smaller than subsampling size (" + std::to_string(subsampling_sizes[i]) + ")");
+			res.dimension_sizes.push_back(in.dimension_sizes[i] / subsampling_sizes[i]);
+		}
+		return res;
+	}
+
+	float average_subsampling_layer::get_forward_flops_per_entry(const std::vector<layer_configuration_specific>& configs) const
+	{
+		const layer_configuration_specific out = get_output_layer_configuration_specific(configs);
+		float per_item = 1.0F;
+		for(unsigned int s : subsampling_sizes)
+			per_item *= static_cast<float>(s);
+		return static_cast<float>(out.get_neuron_count()) * per_item;
+	}
+
+	void average_subsampling_layer::read_params(const schema_param_block * block)
+	{
+		if (block == nullptr)
+			throw neural_network_exception("No average_subsampling_param specified for layer " + instance_name + " of type " + layer_type_name);
+		subsampling_sizes.clear();
+		for(const schema_param_block * dim : block->children("dimension_param"))
+		{
+			if (!dim->has("subsampling_size"))
+				throw neural_network_exception("Only relative subsampling_size is supported by the hip backend for average subsampling layer " + instance_name);
+			subsampling_sizes.push_back(dim->get_uint("subsampling_size", 1));
+		}
+		if (!block->children("feature_map_param").empty() || !block->children("entry_param").empty())
+			throw neural_network_exception("Feature map and entry subsampling are not supported by the hip backend (layer " + instance_name + ")");
+		alpha = block->has("alpha") ? block->get_float("alpha", 0.0F) : -std::numeric_limits<float>::max();
+		for(unsigned int s : subsampling_sizes)
+			if (s == 0)
+				throw neural_network_exception("window dimension for average subsampling layer may not be zero");
+	}
+
+	void average_subsampling_layer::write_params(std::ostream& out, const std::string& indent) const
+	{
+		for(unsigned int s : subsampling_sizes)
+			out << indent << "dimension_param { subsampling_size: " << s << " }\n";
+		if (has_alpha())
+			out << indent << "alpha: " << float_text(alpha) << "\n";
+	}
+
+	std::vector<std::string> average_subsampling_layer::get_parameter_strings() const
+	{
+		std::stringstream ss;
+		for(size_t i = 0; i < subsampling_sizes.size(); ++i)
+			ss << (i == 0 ? "" : "x") << subsampling_sizes[i];
+		if (has_alpha())
+			ss << ", alpha " << alpha;
+		return std::vector<std::string>(1, ss.str());
+	}
+
+	float average_subsampling_layer::get_effective_alpha() const
+	{
+		if (has_alpha())
+			return alpha;
+		unsigned int elems = 1;
+		for(unsigned int s : subsampling_sizes)
+			elems *= s;
+		return 1.0F / static_cast<float>(elems);
+	}
+
+	float average_subsampling_layer::get_plain_tester_alpha() const
+	{
+		return has_alpha() ? alpha : 1.0F;
+	}
+}

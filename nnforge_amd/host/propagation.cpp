@@ -1,0 +1,166 @@
+#include "nnforge_hip/propagation.h"
+
+#include <chrono>
+#include <cstdio>
+#include <cstring>
+
+namespace nnforge
+{
+	// ---- in-memory reader / writer ---------------------------------------------------------
+
+	void memory_data_bunch_reader::add(const std::string& layer_name, const layer_configuration_specific& config, const float * data_ptr)
+	{
+		config_map[layer_name] = config;
+		data[layer_name] = data_ptr;
+	}
+
+	bool memory_data_bunch_reader::read(unsigned int entry_id, const std::map<std::string, float *>& data_map)
+	{
+		if (entry_id >= entry_count)
+			return false;
+		for(const std::pair<const std::string, float *>& dst : data_map)
+		{
+			std::map<std::string, const float *>::const_iterator src = data.find(dst.first);
+			if (src == data.end())
+				throw neural_network_exception("No data supplied for layer " + dst.first);
+			const size_t neuron_count = config_map.find(dst.first)->second.get_neuron_count();
+			std::memcpy(dst.second, src->second + static_cast<size_t>(entry_id) * neuron_count, neuron_count * sizeof(float));
+		}
+		return true;
+	}
+
+	void memory_data_bunch_writer::set_config_map(const std::map<std::string, layer_configuration_specific> new_config_map)
+	{
+		config_map = new_config_map;
+		values.clear();
+		entry_count = 0;
+	}
+
+	void memory_data_bunch_writer::write(unsigned int entry_id, const std::map<std::string, const float *>& data_map)
+	{
+		for(const std::pair<const std::string, const float *>& src : data_map)
+		{
+			const size_t neuron_count = config_map[src.first].get_neuron_count();
+			std::vector<float>& dst = values[src.first];
+			if (dst.size() < (static_cast<size_t>(entry_id) + 1) * neuron_count)
+				dst.resize((static_cast<size_t>(entry_id) + 1) * neuron_count);
+			std::memcpy(dst.data() + static_cast<size_t>(entry_id) * neuron_count, src.second, neuron_count * sizeof(float));
+		}
+		if (entry_id + 1 > entry_count)
+			entry_count = entry_id + 1;
+	}
+
+	// ---- forward_propagation ---------------------------------------------------------------
+
+	forward_propagation::forward_propagation(
+		const network_schema& full_schema,
+		const std::vector<std::string>& output_layer_names,
+		debug_state::ptr debug,
+		profile_state::ptr profile)
+		: output_layer_names(output_layer_names)
+		, debug(debug ? debug : debug_state::ptr(new debug_state()))
+		, profile(profile ? profile : profile_state::ptr(new profile_state()))
+		, flops(0.0F)
+	{
+		if (output_layer_names.empty())
+			throw neural_network_exception("No output layers specified for forward_propagation");
+		network_schema::ptr reduced(new network_schema(full_schema.get_required_layers(output_layer_names)));
+		reduced->name = full_schema.name;
+		schema = reduced;
+		for(const layer::const_ptr& l : schema->get_data_layers())
+			data_layer_names.insert(l->instance_name);
+	}
+
+	bool forward_propagation::is_schema_with_weights() const
+	{
+		for(const layer::const_ptr& l : schema->get_layers())
+			if (!l->is_empty_data() || !l->is_empty_data_custom())
+				return true;
+		return false;
+	}
+
+	void forward_propagation::clear_data()
+	{
+		actual_clear_data();
+	}
+
+	void forward_propagation::set_data(const network_data& data)
+	{
+		const std::vector<layer::const_ptr> layer_list = schema->get_layers();
+		network_data::const_ptr new_data(new network_data(layer_list, data));
+		new_data->check_network_data_consistency(layer_list);
+		actual_set_data(new_data);
+	}
+
+	void forward_propagation::set_input_configuration_specific(const std::map<std::string, layer_configuration_specific>& input_configuration_specific_map)
+	{
+		bool same_input_config = true;
+		std::map<std::string, layer_configuration_specific> filtered;
+		for(const std::pair<const std::string, layer_configuration_specific>& item : input_configuration_specific_map)
+		{
+			if (data_layer_names.find(item.first) == data_layer_names.end())
+				continue;
+			filtered.insert(item);
+			std::map<std::string, layer_configuration_specific>::const_iterator known = layer_config_map.find(item.first);
+			if ((known == layer_config_map.end()) || (known->second != item.second))
+				same_input_config = false;
+		}
+		if (same_input_config && !layer_config_map.empty())
+			return;
+
+		layer_config_map = schema->get_layer_configuration_specific_map(filtered);
+
+		flops = 0.0F;
+		for(const layer::const_ptr& l : schema->get_layers())
+		{
+			if (l->input_layer_instance_names.empty())
+				continue;
+			std::vector<layer_configuration_specific> inputs;
+			for(const std::string& input : l->input_layer_instance_names)
+				inputs.push_back(layer_config_map[input]);
+			flops += l->get_forward_flops_per_entry(inputs);
+		}
+
+		layer_config_map_modified();
+	}
+
+	forward_propagation::stat forward_propagation::run(structured_data_bunch_reader& reader, structured_data_bunch_writer& writer)
+	{
+		stat res;
+		const std::chrono::high_resolution_clock::time_point start = std::chrono::high_resolution_clock::now();
+		set_input_configuration_specific(reader.get_config_map());
+		res.flops_per_entry = flops;
+		std::map<std::string, layer_configuration_specific> output_config_map;
+		for(const std::string& n : output_layer_names)
+			output_config_map[n] = layer_config_map[n];
+		writer.set_config_map(output_config_map);
+		last_action_seconds.clear();
+		float idle_seconds = 0.0F;
+		res.entry_processed_count = 0;
+		actual_run(reader, writer, res.entry_processed_count, last_action_seconds, idle_seconds);
+		const std::chrono::duration<float> sec = std::chrono::high_resolution_clock::now() - start;
+		res.total_seconds = sec.count();
+		res.idle_seconds = idle_seconds;
+		return res;
+	}
+
+	std::ostream& operator<< (std::ostream& out, const forward_propagation::stat& val)
+	{
+		const float idle_overhead = (val.total_seconds > 0.0F) ? val.idle_seconds / val.total_seconds : 0.0F;
+		const float gflops = (val.total_seconds > 0.0F) ? val.flops_per_entry * static_cast<float>(val.entry_processed_count) / val.total_seconds * 1.0e-9F : 0.0F;
+		char buf[256];
+		std::snprintf(buf, sizeof(buf), "%.2f seconds, idle %.1f%%, %u entries, %.2e flops per entry, %.1f GFLOPS",
+			static_cast<double>(val.total_seconds), static_cast<double>(idle_overhead * 100.0F), val.entry_processed_count,
+			static_cast<double>(val.flops_per_entry), static_cast<double>(gflops));
+		out << buf;
+		return out;
+	}
+
+	void factory_generator::apply_default_options()
+	{
+		for(string_option& o : get_string_options()) *o.var = o.default_value;
+		for(bool_option& o : get_bool_options()) *o.var = o.default_value;
+		for(float_option& o : get_float_options()) *o.var = o.default_value;
+		for(int_option& o : get_int_options()) *o.var = o.default_value;
+	}
+}

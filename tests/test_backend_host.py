@@ -1,0 +1,184 @@
+"""Host-side logic of the hip backend, no GPU: schema text format, weight files, the launch plan
+(fusion of element-wise runs), the buffer plan, and the error behaviour the reference's classes have."""
+
+import os
+
+import numpy as np
+import pytest
+
+import nnf_schemas as S
+import nnf_testing as T
+from nnforge_amd import backend
+
+
+def plan(layers, configs, outputs, **kw):
+    return backend.plan_schema(S.schema_text(layers), configs, outputs, **kw)
+
+
+def step_names(report):
+    return ["+".join(s["layers"]) for s in report["steps"]]
+
+
+def test_schema_round_trip_keeps_layers_inputs_and_parameters():
+    layers = S.classifier_tail(8) + [S.L("PReLU", "p", ["res_relu"], feature_map_count=8), S.L("TanH", "t", ["p"], scale=1.7159, steepness=0.666666),
+                                     S.L("ReLU", "leaky", ["t"], negative_slope=0.1), S.L("Add", "a3", ["t", "leaky", "p"], alpha=0.5)]
+    text = S.schema_text(layers, "round trip")
+    once = backend.rewrite_schema(text)
+    twice = backend.rewrite_schema(once)
+    assert once == twice
+    assert 'name: "round trip"' in once
+    for needle in ('type: "BatchNorm"', "feature_map_count: 8", 'input_layer_name: "shortcut_bn"', "scale: 1.71589994", "steepness: 0.666665971",
+                   "negative_slope: 0.100000001", "alpha: 0.5", "dimension_param { subsampling_size: 7 }", "alpha: 0.0204081628"):
+        assert needle in once, needle
+    # Add keeps the order of its inputs
+    a3 = once[once.index('name: "a3"'):]
+    assert a3.index('"t"') < a3.index('"leaky"') < a3.index('"p"')
+
+
+def test_schema_reader_accepts_the_reference_file_syntax():
+    # the formatting of examples/gtsrb/working_data/schema.txt: tabs, nested blocks on one line, comments tolerated
+    text = '''name: "GTSRB-like"
+layer {
+	type: "Data"
+	name: "images"
+}
+layer {
+	type: "TanH"   # comment
+	name: "tanh_0_layer"
+	input_layer_name: "images"
+	tanh_param {
+		scale: 1.7159
+		steepness: 0.666666
+	}
+}
+layer { type: "AverageSubsampling" name: "avg_0_layer" input_layer_name: "tanh_0_layer"
+	average_subsampling_param { dimension_param { subsampling_size: 2 } dimension_param { subsampling_size: 2 } } }
+'''
+    rep = backend.plan_schema(text, {"images": (3, [8, 6])}, ["avg_0_layer"])
+    assert step_names(rep) == ["tanh_0_layer", "avg_0_layer"]
+    assert rep["per_entry_bytes"] == 4 * (3 * 48 + 3 * 48 + 3 * 12)
+
+
+def test_schema_errors():
+    with pytest.raises(backend.BackendError, match="No layer is registered with type Convolution"):
+        backend.rewrite_schema('layer { type: "Convolution" name: "c" }')
+    with pytest.raises(backend.BackendError, match="Duplicate layer name"):
+        backend.rewrite_schema('layer { type: "Data" name: "x" } layer { type: "ReLU" name: "x" input_layer_name: "x" }')
+    with pytest.raises(backend.BackendError, match="unknown input layer"):
+        backend.rewrite_schema('layer { type: "ReLU" name: "r" input_layer_name: "nope" }')
+    with pytest.raises(backend.BackendError, match="cycle"):
+        backend.rewrite_schema('layer { type: "ReLU" name: "a" input_layer_name: "b" } layer { type: "ReLU" name: "b" input_layer_name: "a" }')
+    with pytest.raises(backend.BackendError, match="No batch_norm_param specified"):
+        backend.rewrite_schema('layer { type: "Data" name: "x" } layer { type: "BatchNorm" name: "bn" input_layer_name: "x" }')
+    with pytest.raises(backend.BackendError, match="Feature map count should be > 0"):
+        backend.rewrite_schema('layer { type: "Data" name: "x" } layer { type: "BatchNorm" name: "bn" input_layer_name: "x" batch_norm_param { feature_map_count: 0 } }')
+    with pytest.raises(backend.BackendError, match="missing '}'"):
+        backend.rewrite_schema('layer { type: "Data" name: "x" ')
+
+
+def test_plan_fuses_the_resnet_block_into_one_launch():
+    rep = plan(S.resnet_block(8), {"conv_main": (8, [7, 7]), "conv_shortcut": (8, [7, 7])}, ["res_relu"])
+    assert len(rep["steps"]) == 1
+    s = rep["steps"][0]
+    assert s["fused"] and s["layers"] == ["shortcut_bn", "main_bn", "res", "res_relu"]
+    assert s["inputs"] == ["conv_shortcut", "conv_main"]   # the Add's input order
+    assert rep["per_entry_bytes"] == 3 * 8 * 49 * 4        # two inputs and the output, nothing in between
+    # without fusion: one launch per layer, in place where the tester allows it
+    rep = plan(S.resnet_block(8), {"conv_main": (8, [7, 7]), "conv_shortcut": (8, [7, 7])}, ["res_relu"], fuse=False)
+    assert step_names(rep) == ["shortcut_bn", "main_bn", "res", "res_relu"]
+    assert not any(s["fused"] for s in rep["steps"])
+    # inputs (2) + main_bn + shortcut_bn + res (in place of shortcut_bn) + dedicated output
+    assert rep["per_entry_bytes"] == 5 * 8 * 49 * 4
+    rep = plan(S.resnet_block(8), {"conv_main": (8, [7, 7]), "conv_shortcut": (8, [7, 7])}, ["res_relu"], fuse=False, dont_share_buffers=True)
+    assert rep["per_entry_bytes"] == 6 * 8 * 49 * 4
+
+
+def test_plan_whole_tail_and_activation_chain():
+    rep = plan(S.classifier_tail(8), {"conv_main": (8, [7, 7]), "conv_shortcut": (8, [7, 7])}, ["prob"])
+    assert step_names(rep) == ["shortcut_bn+main_bn+res+res_relu", "pool", "prob"]
+    assert [s["fused"] for s in rep["steps"]] == [True, False, False]
+    rep = plan(S.activation_chain(6), {"x": (6, [5, 4])}, ["tanh"])
+    assert step_names(rep) == ["bn+elu+sig+tanh"]
+
+
+def test_plan_respects_multiple_consumers_outputs_and_shape_changes():
+    layers = [S.L("Data", "x"), S.L("BatchNorm", "bn", ["x"], feature_map_count=4), S.L("ReLU", "r1", ["bn"]), S.L("Sigmoid", "s", ["bn"]),
+              S.L("Add", "a", ["r1", "s"]), S.L("TanH", "t", ["a"])]
+    rep = plan(layers, {"x": (4, [3, 3])}, ["t"])
+    # bn feeds two layers: it is written to memory once, the rest fuses around the Add
+    assert step_names(rep) == ["bn", "r1+s+a+t"]
+    assert rep["steps"][1]["inputs"] == ["bn", "bn"]
+    # an output layer in the middle of a chain is written out, the chain continues from it
+    rep = plan(S.activation_chain(6), {"x": (6, [5, 4])}, ["tanh", "elu"])
+    assert step_names(rep) == ["bn+elu", "sig+tanh"]
+    # Add of differently shaped inputs with the same neuron count: allowed, but not fused with per-feature-map layers
+    layers = [S.L("Data", "x"), S.L("Data", "y"), S.L("BatchNorm", "bn", ["x"], feature_map_count=4), S.L("Add", "a", ["bn", "y"])]
+    rep = plan(layers, {"x": (4, [6]), "y": (6, [4])}, ["a"])
+    assert step_names(rep) == ["bn", "a"]
+    # more inputs than the fused kernel takes: the Add runs on its own
+    many = [S.L("Data", "x")] + [S.L("ReLU", "r%d" % i, ["x"], negative_slope=0.1 * i) for i in range(5)] + [S.L("Add", "a", ["r%d" % i for i in range(5)])]
+    rep = plan(many, {"x": (2, [4])}, ["a"])
+    assert step_names(rep) == ["r0", "r1", "r2", "r3", "r4", "a"]
+
+
+def test_plan_splits_chains_longer_than_the_kernel_takes():
+    layers = [S.L("Data", "x")]
+    prev = "x"
+    for i in range(11):
+        layers.append(S.L("ReLU", "r%d" % i, [prev], negative_slope=0.5))
+        prev = "r%d" % i
+    rep = plan(layers, {"x": (2, [4])}, [prev])
+    assert [len(s["layers"]) for s in rep["steps"]] == [8, 3]
+
+
+def test_plan_memory_budget():
+    cfg = {"conv_main": (8, [7, 7]), "conv_shortcut": (8, [7, 7])}
+    per_entry = 3 * 8 * 49 * 4
+    rep = plan(S.resnet_block(8), cfg, ["res_relu"], memory_bytes=100 * per_entry)
+    assert rep["max_entry_count"] in (89, 90)   # 0.9 of the memory (the ratio is an fp32 number)
+    rep = plan(S.resnet_block(8), cfg, ["res_relu"], memory_bytes=1 << 40, max_entry_count=77)
+    assert rep["max_entry_count"] == 77
+    with pytest.raises(backend.BackendError, match="Insufficient memory to do forward prop for even one sample"):
+        plan(S.resnet_block(8), cfg, ["res_relu"], memory_bytes=per_entry)
+
+
+def test_plan_errors():
+    cfg = {"conv_main": (8, [7, 7]), "conv_shortcut": (8, [7, 7])}
+    with pytest.raises(backend.BackendError, match="Layer not found"):
+        plan(S.resnet_block(8), cfg, ["nope"])
+    with pytest.raises(backend.BackendError, match="No input configuration supplied for data layer"):
+        plan(S.resnet_block(8), {"conv_main": (8, [7, 7])}, ["res_relu"])
+    with pytest.raises(backend.BackendError, match="Feature map count in layer"):
+        plan(S.resnet_block(8), {"conv_main": (4, [7, 7]), "conv_shortcut": (4, [7, 7])}, ["res_relu"])
+    with pytest.raises(backend.BackendError, match="Neuron count per entry mismatch"):
+        plan(S.resnet_block(8, False), {"conv_main": (8, [7, 7]), "conv_shortcut": (8, [7, 6])}, ["res_relu"])
+    with pytest.raises(backend.BackendError, match="smaller than subsampling size"):
+        plan(S.classifier_tail(8), {"conv_main": (8, [5, 5]), "conv_shortcut": (8, [5, 5])}, ["prob"])
+    # a plan made without a device cannot run
+    with pytest.raises(backend.BackendError, match="No output layers specified"):
+        plan(S.resnet_block(8), cfg, [])
+
+
+def test_weight_files_round_trip(tmp_path):
+    gen = T.rng(40, 0)
+    weights = {"main_bn": list(T.bn_params(gen, 8)), "p": [T.uniform(gen, 5, 0, 0.25)]}
+    folder = str(tmp_path / "ann_trained_000")
+    backend.write_weights(folder, weights)
+    assert sorted(os.listdir(folder)) == ["main_bn.data", "p.data"]
+    raw = open(os.path.join(folder, "p.data"), "rb").read()
+    # 16-byte GUID, u32 chunk count, u32 length, floats
+    assert raw[:16] == bytes([0xd1, 0x19, 0x35, 0xb5, 0x30, 0x59, 0x49, 0xe2, 0x9c, 0x33, 0x1c, 0x43, 0x22, 0xf8, 0x13, 0x0d])
+    assert np.frombuffer(raw[16:24], np.uint32).tolist() == [1, 5]
+    assert np.array_equal(np.frombuffer(raw[24:], np.float32), weights["p"][0])
+    got = backend.read_weights(folder, "main_bn", [8, 8, 8, 8])
+    for a, b in zip(got, weights["main_bn"]):
+        assert np.array_equal(a, b)
+    with pytest.raises(backend.BackendError, match="doesn't satisfy layer configuration"):
+        backend.read_weights(folder, "main_bn", [8, 8, 8])
+    with pytest.raises(backend.BackendError, match="No data found with layer name"):
+        backend.read_weights(folder, "absent", [1])
+    with pytest.raises(backend.BackendError, match="doesn't exist"):
+        backend.read_weights(folder + "_nope", "p", [5])
+    open(os.path.join(folder, "bad.data"), "wb").write(b"\0" * 40)
+    with pytest.raises(backend.BackendError, match="Unknown data GUID"):
+        backend.read_weights(folder, "p", [5])

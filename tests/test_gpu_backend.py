@@ -1,0 +1,101 @@
+"""The C++ hip backend end to end on the GPU: a text-format schema, nnForge-format weights and
+host tensors go in through factory_generator_hip -> forward_propagation_hip; the outputs must equal
+the CPU oracle run layer by layer the way the plain backend drives its testers."""
+
+import numpy as np
+import pytest
+
+import nnf_schemas as S
+import nnf_testing as T
+from nnforge_amd import backend
+
+pytestmark = pytest.mark.gpu
+
+
+def run(layers, weights, inputs, outputs, values, **kw):
+    shapes = {n: values[n].shape for n in outputs}
+    return backend.run_schema(S.schema_text(layers), weights, inputs, shapes, **kw)
+
+
+def assert_bits(got, want, what):
+    assert got.shape == want.shape
+    assert T.bit_mismatches(got, want) == 0, "%s: %d of %d elements differ" % (what, T.bit_mismatches(got, want), got.size)
+
+
+@pytest.mark.parametrize("fuse", [True, False])
+@pytest.mark.parametrize("shortcut_bn", [True, False])
+def test_resnet_block(fuse, shortcut_bn):
+    gen = T.rng(50, int(fuse) * 2 + int(shortcut_bn))
+    c, n = 16, 5
+    layers = S.resnet_block(c, shortcut_bn)
+    weights = S.make_weights(layers, gen)
+    inputs = {"conv_main": T.normal(gen, (n, c, 14, 14)), "conv_shortcut": T.normal(gen, (n, c, 14, 14))}
+    values = S.evaluate(layers, weights, inputs)
+    got, rep = run(layers, weights, inputs, ["res_relu"], values, fuse=fuse)
+    assert_bits(got["res_relu"], values["res_relu"], "resnet block")
+    assert rep["entries"] == n
+    assert len(rep["steps"]) == (1 if fuse else (4 if shortcut_bn else 3))
+
+
+def test_classifier_tail_with_several_outputs_and_packets():
+    gen = T.rng(51, 0)
+    c, n = 12, 11
+    layers = S.classifier_tail(c)
+    weights = S.make_weights(layers, gen)
+    inputs = {"conv_main": T.normal(gen, (n, c, 7, 7), 4.0), "conv_shortcut": T.normal(gen, (n, c, 7, 7), 4.0)}
+    values = S.evaluate(layers, weights, inputs)
+    # 11 entries in packets of 4: 4 + 4 + 3
+    got, rep = run(layers, weights, inputs, ["prob", "pool", "res_relu"], values, max_entry_count=4, profile=True)
+    assert rep["entries"] == n and rep["max_entry_count"] == 4
+    assert_bits(got["res_relu"], values["res_relu"], "block output")
+    assert_bits(got["pool"], values["pool"], "pool")
+    rel = np.abs(got["prob"] - values["prob"]) / values["prob"]
+    assert rel.max() < 1e-5
+    assert set(rep["seconds"]) == {"shortcut_bn+main_bn+res+res_relu", "pool", "prob"}
+    assert all(v > 0 for v in rep["seconds"].values())
+
+
+@pytest.mark.parametrize("fuse,share", [(True, True), (False, True), (False, False)])
+def test_activation_chain_and_branches(fuse, share):
+    gen = T.rng(52, 0)
+    c, n = 6, 7
+    layers = S.activation_chain(c) + [S.L("PReLU", "p", ["bn"], feature_map_count=c), S.L("Add", "mix", ["tanh", "p", "x"], alpha=0.5),
+                                      S.L("ReLU", "leaky", ["mix"], negative_slope=0.2)]
+    weights = S.make_weights(layers, gen)
+    x = T.normal(gen, (n, c, 9, 5), 2.0)
+    x.reshape(-1)[::97] = 50.0
+    x.reshape(-1)[5::89] = -50.0
+    inputs = {"x": x}
+    values = S.evaluate(layers, weights, inputs)
+    got, rep = run(layers, weights, inputs, ["leaky", "tanh"], values, fuse=fuse, dont_share_buffers=not share)
+    assert_bits(got["tanh"], values["tanh"], "tanh")
+    assert_bits(got["leaky"], values["leaky"], "leaky")
+
+
+def test_weights_from_nnforge_data_files(tmp_path):
+    gen = T.rng(53, 0)
+    layers = S.resnet_block(8)
+    weights = S.make_weights(layers, gen)
+    folder = str(tmp_path / "ann_trained_000")
+    backend.write_weights(folder, weights)
+    inputs = {"conv_main": T.normal(gen, (3, 8, 7, 7)), "conv_shortcut": T.normal(gen, (3, 8, 7, 7))}
+    values = S.evaluate(layers, weights, inputs)
+    got, _ = run(layers, {}, inputs, ["res_relu"], values, weights_folder=folder)
+    assert_bits(got["res_relu"], values["res_relu"], "weights from .data files")
+
+
+def test_run_errors():
+    gen = T.rng(54, 0)
+    layers = S.resnet_block(8)
+    weights = S.make_weights(layers, gen)
+    inputs = {"conv_main": T.normal(gen, (3, 8, 7, 7)), "conv_shortcut": T.normal(gen, (3, 8, 7, 7))}
+    values = S.evaluate(layers, weights, inputs)
+    with pytest.raises(backend.BackendError, match="No data found with layer name"):
+        run(layers, {"main_bn": weights["main_bn"]}, inputs, ["res_relu"], values)
+    bad = dict(weights)
+    bad["main_bn"] = weights["main_bn"][:3]
+    with pytest.raises(backend.BackendError, match="data weight vector count 3 doesn't satisfy layer configuration 4"):
+        run(layers, bad, inputs, ["res_relu"], values)
+    bad["main_bn"] = [w[:5] for w in weights["main_bn"]]
+    with pytest.raises(backend.BackendError, match="data weight count 5 for vector 0 doesn't satisfy layer configuration 8"):
+        run(layers, bad, inputs, ["res_relu"], values)
