@@ -8,11 +8,13 @@
 // PReLU slope) are computed once per workgroup into LDS and looked up by plane index.
 #include "nnf_common.h"
 
+#include <cstdlib>
+
 namespace nnf
 {
 	namespace
 	{
-		constexpr int chain_block_size = 256;
+
 		constexpr int max_slots = NNF_HIP_MAX_OPS;
 		constexpr uint32_t exp_table_bytes = exp2_table_size * sizeof(uint64_t);
 
@@ -64,27 +66,45 @@ namespace nnf
 		}
 
 		// Applies one layer to the U float4s a lane holds. The switch is uniform across the workgroup.
-		template<int U, int PL>
+		// DIRECT: where[k][0] is the feature map of float4 k and per-feature-map weights are read from
+		// memory (all lanes of a wavefront read the same one or two addresses: one cache line).
+		// Otherwise where[k][e] indexes the coefficient arrays the workgroup staged in LDS.
+		template<int U, bool DIRECT>
 		__device__ __forceinline__ void apply_op(
 			const chain_op& op,
+			const chain_args& a,
 			float (&v)[U][4],
-			const uint32_t (&pl)[U][PL],
+			const uint32_t (&where)[U][DIRECT ? 1 : 4],
 			const float2* lds_coeff,
-			uint32_t span,
 			const uint64_t* lds_exp)
 		{
 			switch (op.kind)
 			{
 			case NNF_HIP_OP_BATCH_NORM:
+				if (DIRECT)
 				{
-					const float2* coeff = lds_coeff + op.slot * span;
+					const chain_slot& slot = a.slots[op.slot];
+					#pragma unroll
+					for(int k = 0; k < U; ++k)
+					{
+						const uint32_t fm = where[k][0];
+						float mult, add;
+						nnf_batch_norm_coefficients(slot.p[0][fm], slot.p[1][fm], slot.p[2][fm], slot.p[3][fm], mult, add);
+						#pragma unroll
+						for(int e = 0; e < 4; ++e)
+							v[k][e] = nnf_batch_norm(v[k][e], mult, add);
+					}
+				}
+				else
+				{
+					const float2* coeff = lds_coeff + op.slot * a.span;
 					#pragma unroll
 					for(int k = 0; k < U; ++k)
 					{
 						#pragma unroll
 						for(int e = 0; e < 4; ++e)
 						{
-							const float2 ma = coeff[pl[k][PL == 1 ? 0 : e]];
+							const float2 ma = coeff[where[k][DIRECT ? 0 : e]];
 							v[k][e] = nnf_batch_norm(v[k][e], ma.x, ma.y);
 						}
 					}
@@ -100,14 +120,27 @@ namespace nnf
 				}
 				break;
 			case NNF_HIP_OP_PRELU:
+				if (DIRECT)
 				{
-					const float2* coeff = lds_coeff + op.slot * span;
+					const float* slopes = a.slots[op.slot].p[0];
+					#pragma unroll
+					for(int k = 0; k < U; ++k)
+					{
+						const float slope = slopes[where[k][0]];
+						#pragma unroll
+						for(int e = 0; e < 4; ++e)
+							v[k][e] = nnf_parametric_rectified_linear(v[k][e], slope);
+					}
+				}
+				else
+				{
+					const float2* coeff = lds_coeff + op.slot * a.span;
 					#pragma unroll
 					for(int k = 0; k < U; ++k)
 					{
 						#pragma unroll
 						for(int e = 0; e < 4; ++e)
-							v[k][e] = nnf_parametric_rectified_linear(v[k][e], coeff[pl[k][PL == 1 ? 0 : e]].x);
+							v[k][e] = nnf_parametric_rectified_linear(v[k][e], coeff[where[k][DIRECT ? 0 : e]].x);
 					}
 				}
 				break;
@@ -143,12 +176,16 @@ namespace nnf
 			}
 		}
 
-		// NIN: number of input tensors. U: float4s per lane. ALIGNED4: plane % 4 == 0, i.e. a float4 never straddles planes.
-		template<int NIN, int U, bool ALIGNED4>
-		__global__ void __launch_bounds__(chain_block_size) chain_kernel(const chain_args a)
+		// NIN: number of input tensors. BLOCK: lanes per workgroup. U: float4s per lane.
+		// DIRECT: plane % 4 == 0 (a float4 never straddles planes) and a tile touches no feature map
+		// twice; per-feature-map weights are then read straight from memory and the workgroup needs
+		// neither LDS coefficients nor a barrier. Otherwise coefficients of the planes the tile touches
+		// are staged in LDS and looked up per element.
+		template<int NIN, int BLOCK, int U, bool DIRECT>
+		__global__ void __launch_bounds__(BLOCK) chain_kernel(const chain_args a)
 		{
-			constexpr int TILE = chain_block_size * U * 4;
-			constexpr int PL = ALIGNED4 ? 1 : 4;
+			constexpr int TILE = BLOCK * U * 4;
+			constexpr int PL = DIRECT ? 1 : 4;
 			extern __shared__ __align__(16) unsigned char lds_raw[];
 			uint64_t* lds_exp = reinterpret_cast<uint64_t*>(lds_raw);
 			float2* lds_coeff = reinterpret_cast<float2*>(lds_raw + exp_table_bytes);
@@ -158,7 +195,7 @@ namespace nnf
 			const uint32_t start_in_plane = tile_start - first_plane * a.plane;
 			const uint32_t first_fm = first_plane % a.fm_count;
 
-			// issue all loads first: they are what the kernel waits for
+			// all tensor loads are issued before anything else: they are what the kernel waits for
 			float x[NIN][U][4];
 			#pragma unroll
 			for(int j = 0; j < NIN; ++j)
@@ -166,7 +203,7 @@ namespace nnf
 				#pragma unroll
 				for(int k = 0; k < U; ++k)
 				{
-					const uint32_t idx = tile_start + (threadIdx.x + k * chain_block_size) * 4;
+					const uint32_t idx = tile_start + (threadIdx.x + k * BLOCK) * 4;
 					if (idx + 3 < a.total)
 					{
 						const floatx4 t = load_stream(reinterpret_cast<const floatx4*>(a.in[j] + idx));
@@ -181,36 +218,47 @@ namespace nnf
 				}
 			}
 
-			// per-feature-map coefficients of the planes this tile touches
 			if (a.need_exp)
 				stage_exp2_table(lds_exp);
-			for(uint32_t s = 0; s < a.slot_count; ++s)
+			if (!DIRECT)
 			{
-				const chain_slot& slot = a.slots[s];
-				for(uint32_t i = threadIdx.x; i < a.span; i += chain_block_size)
+				for(uint32_t s = 0; s < a.slot_count; ++s)
 				{
-					const uint32_t fm = (first_fm + i) % a.fm_count;
-					float2 c;
-					if (slot.kind == NNF_HIP_OP_BATCH_NORM)
-						nnf_batch_norm_coefficients(slot.p[0][fm], slot.p[1][fm], slot.p[2][fm], slot.p[3][fm], c.x, c.y);
-					else
+					const chain_slot& slot = a.slots[s];
+					for(uint32_t i = threadIdx.x; i < a.span; i += BLOCK)
 					{
-						c.x = slot.p[0][fm];
-						c.y = 0.0f;
+						const uint32_t fm = (first_fm + i) % a.fm_count;
+						float2 c;
+						if (slot.kind == NNF_HIP_OP_BATCH_NORM)
+							nnf_batch_norm_coefficients(slot.p[0][fm], slot.p[1][fm], slot.p[2][fm], slot.p[3][fm], c.x, c.y);
+						else
+						{
+							c.x = slot.p[0][fm];
+							c.y = 0.0f;
+						}
+						lds_coeff[s * a.span + i] = c;
 					}
-					lds_coeff[s * a.span + i] = c;
 				}
 			}
-			__syncthreads();
+			if (!DIRECT || a.need_exp)
+				__syncthreads();
 
-			uint32_t pl[U][PL];
+			uint32_t where[U][PL];
 			#pragma unroll
 			for(int k = 0; k < U; ++k)
 			{
-				const uint32_t e0 = start_in_plane + (threadIdx.x + k * chain_block_size) * 4;
+				const uint32_t e0 = start_in_plane + (threadIdx.x + k * BLOCK) * 4;
 				#pragma unroll
 				for(int e = 0; e < PL; ++e)
-					pl[k][e] = plane_of<TILE>(e0 + e, a.plane, a.plane_magic);
+				{
+					uint32_t w = plane_of<TILE>(e0 + e, a.plane, a.plane_magic);
+					if (DIRECT)
+					{
+						w += first_fm; // < 2 * fm_count: the host picks this path only when span <= fm_count
+						w = (w >= a.fm_count) ? w - a.fm_count : w;
+					}
+					where[k][e] = w;
+				}
 			}
 
 			uint32_t op_index = 0;
@@ -219,7 +267,7 @@ namespace nnf
 			{
 				const uint32_t arm_end = op_index + a.arm_ops[j];
 				for(; op_index < arm_end; ++op_index)
-					apply_op<U, PL>(a.ops[op_index], x[j], pl, lds_coeff, a.span, lds_exp);
+					apply_op<U, DIRECT>(a.ops[op_index], a, x[j], where, lds_coeff, lds_exp);
 			}
 
 			if (a.has_add)
@@ -242,12 +290,12 @@ namespace nnf
 
 			const uint32_t tail_end = op_index + a.tail_ops;
 			for(; op_index < tail_end; ++op_index)
-				apply_op<U, PL>(a.ops[op_index], x[0], pl, lds_coeff, a.span, lds_exp);
+				apply_op<U, DIRECT>(a.ops[op_index], a, x[0], where, lds_coeff, lds_exp);
 
 			#pragma unroll
 			for(int k = 0; k < U; ++k)
 			{
-				const uint32_t idx = tile_start + (threadIdx.x + k * chain_block_size) * 4;
+				const uint32_t idx = tile_start + (threadIdx.x + k * BLOCK) * 4;
 				if (idx + 3 < a.total)
 				{
 					floatx4 t;
@@ -266,32 +314,56 @@ namespace nnf
 
 		typedef void (*chain_kernel_fn)(const chain_args);
 
-		template<int NIN, int U>
-		chain_kernel_fn pick_aligned(bool aligned4)
+		// Launch shapes (lanes per workgroup, float4s per lane), largest tile first.
+		struct launch_shape
 		{
-			return aligned4 ? chain_kernel<NIN, U, true> : chain_kernel<NIN, U, false>;
+			int block;
+			int unroll;
+		};
+		constexpr launch_shape launch_shapes[] = { {256, 4}, {256, 2}, {256, 1}, {64, 1} };
+		constexpr int launch_shape_count = sizeof(launch_shapes) / sizeof(launch_shapes[0]);
+
+		template<int NIN, int BLOCK, int U>
+		chain_kernel_fn pick_aligned(bool direct)
+		{
+			return direct ? chain_kernel<NIN, BLOCK, U, true> : chain_kernel<NIN, BLOCK, U, false>;
 		}
 
 		template<int NIN>
-		chain_kernel_fn pick_unroll(int unroll, bool aligned4)
+		chain_kernel_fn pick_shape(int shape, bool aligned4)
 		{
-			switch (unroll)
+			switch (shape)
 			{
-			case 4: return pick_aligned<NIN, 4>(aligned4);
-			case 2: return pick_aligned<NIN, 2>(aligned4);
-			default: return pick_aligned<NIN, 1>(aligned4);
+			case 0: return pick_aligned<NIN, 256, 4>(aligned4);
+			case 1: return pick_aligned<NIN, 256, 2>(aligned4);
+			case 2: return pick_aligned<NIN, 256, 1>(aligned4);
+			default: return pick_aligned<NIN, 64, 1>(aligned4);
 			}
 		}
 
-		chain_kernel_fn pick_kernel(uint32_t input_count, int unroll, bool aligned4)
+		chain_kernel_fn pick_kernel(uint32_t input_count, int shape, bool aligned4)
 		{
 			switch (input_count)
 			{
-			case 1: return pick_unroll<1>(unroll, aligned4);
-			case 2: return pick_unroll<2>(unroll, aligned4);
-			case 3: return pick_unroll<3>(unroll, aligned4);
-			default: return pick_unroll<4>(unroll, aligned4);
+			case 1: return pick_shape<1>(shape, aligned4);
+			case 2: return pick_shape<2>(shape, aligned4);
+			case 3: return pick_shape<3>(shape, aligned4);
+			default: return pick_shape<4>(shape, aligned4);
 			}
+		}
+
+		// Tuning override for experiments: NNF_HIP_CHAIN_SHAPE=<index into launch_shapes>; -1 = automatic.
+		int forced_shape()
+		{
+			static const int value = []
+			{
+				const char* s = getenv("NNF_HIP_CHAIN_SHAPE");
+				if ((s == nullptr) || (*s == '\0'))
+					return -1;
+				const int v = atoi(s);
+				return ((v >= 0) && (v < launch_shape_count)) ? v : -1;
+			}();
+			return value;
 		}
 
 		bool ranges_overlap(const void* a, const void* b, size_t bytes)
@@ -304,6 +376,8 @@ namespace nnf
 		constexpr size_t max_dynamic_lds = 64 * 1024;
 		// Below this many tiles a smaller tile is used so that more compute units get work.
 		constexpr uint32_t min_tiles_wanted = 1024;
+		// From this size on (64 MB per tensor) the smaller tile is used.
+		constexpr uint32_t large_tensor_elements = 1u << 24;
 	}
 
 	int chain_forward(hipStream_t stream, const nnf_hip_chain_desc* desc, float* output,
@@ -404,31 +478,61 @@ namespace nnf
 		}
 
 		// tile size: as large as keeps the coefficient arrays inside LDS and the grid wide enough
-		int unroll = 4;
-		size_t lds_bytes = 0;
-		for(;; unroll /= 2)
+		auto span_of = [&](int shape) -> uint32_t
 		{
-			const uint32_t tile = chain_block_size * unroll * 4;
-			a.span = (tile + a.plane - 2) / a.plane + 1;
-			lds_bytes = exp_table_bytes + static_cast<size_t>(a.slot_count) * a.span * sizeof(float2);
-			const uint32_t tiles = (a.total + tile - 1) / tile;
-			const bool fits = lds_bytes <= max_dynamic_lds;
-			if (unroll == 1)
-			{
-				if (!fits)
-					return NNF_HIP_EUNSUPPORTED;
-				break;
-			}
-			if (fits && (tiles >= min_tiles_wanted))
-				break;
-		}
-		const uint32_t tile = chain_block_size * unroll * 4;
-		a.plane_magic = (a.plane >= 2) ? static_cast<uint32_t>(((1ull << 32) + a.plane - 1) / a.plane) : 0u;
-		const uint32_t tiles = (a.total + tile - 1) / tile;
-		const bool aligned4 = (a.plane % 4) == 0;
+			const uint32_t tile = launch_shapes[shape].block * launch_shapes[shape].unroll * 4;
+			return (tile + a.plane - 2) / a.plane + 1;
+		};
+		// weights are read straight from memory when a float4 never straddles planes and a tile
+		// touches no feature map twice; otherwise the workgroup stages coefficients in LDS
+		auto direct_of = [&](int shape) -> bool
+		{
+			return ((a.plane % 4) == 0) && (span_of(shape) <= a.fm_count);
+		};
+		auto lds_bytes_of = [&](int shape) -> size_t
+		{
+			if (direct_of(shape))
+				return exp_table_bytes;
+			return exp_table_bytes + static_cast<size_t>(a.slot_count) * span_of(shape) * sizeof(float2);
+		};
+		auto tiles_of = [&](int shape) -> uint32_t
+		{
+			const uint32_t tile = launch_shapes[shape].block * launch_shapes[shape].unroll * 4;
+			return (a.total + tile - 1) / tile;
+		};
 
-		chain_kernel_fn kernel = pick_kernel(desc->input_count, unroll, aligned4);
-		hipLaunchKernelGGL(kernel, dim3(tiles), dim3(chain_block_size), lds_bytes, stream, a);
+		int shape = forced_shape();
+		if ((shape < 0) || (lds_bytes_of(shape) > max_dynamic_lds))
+		{
+			// Measured on MI355X: tensors of 64 MB and more stream best with two float4s per lane,
+			// smaller ones with four, as long as enough workgroups exist to cover the machine.
+			static const int large_order[] = { 1, 2, 3 };
+			static const int small_order[] = { 0, 1, 2, 3 };
+			const bool large = a.total >= large_tensor_elements;
+			const int* order = large ? large_order : small_order;
+			const int order_count = large ? 3 : 4;
+			shape = -1;
+			for(int i = 0; i < order_count; ++i)
+			{
+				const int s = order[i];
+				if (lds_bytes_of(s) > max_dynamic_lds)
+					continue;
+				if (large || (tiles_of(s) >= min_tiles_wanted) || (i == order_count - 1))
+				{
+					shape = s;
+					break;
+				}
+			}
+			if (shape < 0)
+				return NNF_HIP_EUNSUPPORTED;
+		}
+		const uint32_t tile = launch_shapes[shape].block * launch_shapes[shape].unroll * 4;
+		(void)tile;
+		a.span = span_of(shape);
+		a.plane_magic = (a.plane >= 2) ? static_cast<uint32_t>(((1ull << 32) + a.plane - 1) / a.plane) : 0u;
+
+		chain_kernel_fn kernel = pick_kernel(desc->input_count, shape, direct_of(shape));
+		hipLaunchKernelGGL(kernel, dim3(tiles_of(shape)), dim3(launch_shapes[shape].block), lds_bytes_of(shape), stream, a);
 		return launch_status();
 	}
 }
