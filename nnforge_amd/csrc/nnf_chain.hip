@@ -16,7 +16,7 @@ namespace nnf
 	{
 
 		constexpr int max_slots = NNF_HIP_MAX_OPS;
-		constexpr uint32_t exp_table_bytes = exp2_table_size * sizeof(uint64_t);
+		constexpr uint32_t exp_table_bytes = exp_lds_entries * sizeof(uint64_t);
 
 		struct chain_op
 		{
@@ -71,14 +71,15 @@ namespace nnf
 		// Otherwise where[k][e] indexes the coefficient arrays the workgroup staged in LDS.
 		template<int U, bool DIRECT>
 		__device__ __forceinline__ void apply_op(
+			int kind,
 			const chain_op& op,
 			const chain_args& a,
 			float (&v)[U][4],
 			const uint32_t (&where)[U][DIRECT ? 1 : 4],
 			const float2* lds_coeff,
-			const uint64_t* lds_exp)
+			const exp_context& exp_ctx)
 		{
-			switch (op.kind)
+			switch (kind)
 			{
 			case NNF_HIP_OP_BATCH_NORM:
 				if (DIRECT)
@@ -145,31 +146,13 @@ namespace nnf
 				}
 				break;
 			case NNF_HIP_OP_ELU:
-				#pragma unroll
-				for(int k = 0; k < U; ++k)
-				{
-					#pragma unroll
-					for(int e = 0; e < 4; ++e)
-						v[k][e] = nnf_exponential_linear(v[k][e], lds_exp);
-				}
+				nnf_exponential_linear<U * 4>(reinterpret_cast<float (&)[U * 4]>(v), exp_ctx);
 				break;
 			case NNF_HIP_OP_SIGMOID:
-				#pragma unroll
-				for(int k = 0; k < U; ++k)
-				{
-					#pragma unroll
-					for(int e = 0; e < 4; ++e)
-						v[k][e] = nnf_sigmoid(v[k][e], lds_exp);
-				}
+				nnf_sigmoid<U * 4>(reinterpret_cast<float (&)[U * 4]>(v), exp_ctx);
 				break;
 			case NNF_HIP_OP_TANH:
-				#pragma unroll
-				for(int k = 0; k < U; ++k)
-				{
-					#pragma unroll
-					for(int e = 0; e < 4; ++e)
-						v[k][e] = nnf_hyperbolic_tangent(v[k][e], op.f1, op.f0, lds_exp); // f1 holds steepness * 2
-				}
+				nnf_hyperbolic_tangent<U * 4>(reinterpret_cast<float (&)[U * 4]>(v), op.f1, op.f0, exp_ctx); // f1 holds steepness * 2
 				break;
 			default:
 				break;
@@ -181,7 +164,28 @@ namespace nnf
 		// twice; per-feature-map weights are then read straight from memory and the workgroup needs
 		// neither LDS coefficients nor a barrier. Otherwise coefficients of the planes the tile touches
 		// are staged in LDS and looked up per element.
-		template<int NIN, int BLOCK, int U, bool DIRECT>
+		// PROGRAM: 0 = the layer kinds are read from the arguments (any group); > 0 = index into
+		// known_programs: a single-input group whose layer kinds are compile-time constants, so that
+		// the whole chain becomes straight-line code (used for the groups that are bound by the
+		// vector ALU, i.e. the ones that call expf).
+		struct known_program
+		{
+			int op_count;
+			int kinds[NNF_HIP_MAX_OPS];
+		};
+		constexpr known_program known_programs[] = {
+			{ 0, {} },
+			{ 4, { NNF_HIP_OP_BATCH_NORM, NNF_HIP_OP_ELU, NNF_HIP_OP_SIGMOID, NNF_HIP_OP_TANH } },
+			{ 1, { NNF_HIP_OP_ELU } },
+			{ 1, { NNF_HIP_OP_SIGMOID } },
+			{ 1, { NNF_HIP_OP_TANH } },
+			{ 2, { NNF_HIP_OP_BATCH_NORM, NNF_HIP_OP_ELU } },
+			{ 2, { NNF_HIP_OP_BATCH_NORM, NNF_HIP_OP_SIGMOID } },
+			{ 2, { NNF_HIP_OP_BATCH_NORM, NNF_HIP_OP_TANH } },
+		};
+		constexpr int known_program_count = sizeof(known_programs) / sizeof(known_programs[0]);
+
+		template<int NIN, int BLOCK, int U, bool DIRECT, int PROGRAM>
 		__global__ void __launch_bounds__(BLOCK) chain_kernel(const chain_args a)
 		{
 			constexpr int TILE = BLOCK * U * 4;
@@ -242,6 +246,9 @@ namespace nnf
 			}
 			if (!DIRECT || a.need_exp)
 				__syncthreads();
+			exp_context exp_ctx = make_exp_context(lds_exp);
+			if (a.need_exp)
+				exp_ctx = exp_context_from_lds(lds_exp);
 
 			uint32_t where[U][PL];
 			#pragma unroll
@@ -262,15 +269,25 @@ namespace nnf
 			}
 
 			uint32_t op_index = 0;
-			#pragma unroll
-			for(int j = 0; j < NIN; ++j)
+			if (PROGRAM > 0)
 			{
-				const uint32_t arm_end = op_index + a.arm_ops[j];
-				for(; op_index < arm_end; ++op_index)
-					apply_op<U, DIRECT>(a.ops[op_index], a, x[j], where, lds_coeff, lds_exp);
+				#pragma unroll
+				for(int i = 0; i < known_programs[PROGRAM].op_count; ++i)
+					apply_op<U, DIRECT>(known_programs[PROGRAM].kinds[i], a.ops[i], a, x[0], where, lds_coeff, exp_ctx);
+				op_index = known_programs[PROGRAM].op_count;
+			}
+			else
+			{
+				#pragma unroll
+				for(int j = 0; j < NIN; ++j)
+				{
+					const uint32_t arm_end = op_index + a.arm_ops[j];
+					for(; op_index < arm_end; ++op_index)
+						apply_op<U, DIRECT>(a.ops[op_index].kind, a.ops[op_index], a, x[j], where, lds_coeff, exp_ctx);
+				}
 			}
 
-			if (a.has_add)
+			if ((PROGRAM == 0) && a.has_add)
 			{
 				// nnforge/plain/add_layer_tester_plain.cpp:56-59: sum starts at 0.0F
 				#pragma unroll
@@ -288,9 +305,12 @@ namespace nnf
 				}
 			}
 
-			const uint32_t tail_end = op_index + a.tail_ops;
-			for(; op_index < tail_end; ++op_index)
-				apply_op<U, DIRECT>(a.ops[op_index], a, x[0], where, lds_coeff, lds_exp);
+			if (PROGRAM == 0)
+			{
+				const uint32_t tail_end = op_index + a.tail_ops;
+				for(; op_index < tail_end; ++op_index)
+					apply_op<U, DIRECT>(a.ops[op_index].kind, a.ops[op_index], a, x[0], where, lds_coeff, exp_ctx);
+			}
 
 			#pragma unroll
 			for(int k = 0; k < U; ++k)
@@ -323,33 +343,62 @@ namespace nnf
 		constexpr launch_shape launch_shapes[] = { {256, 4}, {256, 2}, {256, 1}, {64, 1} };
 		constexpr int launch_shape_count = sizeof(launch_shapes) / sizeof(launch_shapes[0]);
 
-		template<int NIN, int BLOCK, int U>
-		chain_kernel_fn pick_aligned(bool direct)
+		template<int NIN, int BLOCK, int U, int PROGRAM>
+		chain_kernel_fn pick_direct(bool direct)
 		{
-			return direct ? chain_kernel<NIN, BLOCK, U, true> : chain_kernel<NIN, BLOCK, U, false>;
+			return direct ? chain_kernel<NIN, BLOCK, U, true, PROGRAM> : chain_kernel<NIN, BLOCK, U, false, PROGRAM>;
 		}
 
-		template<int NIN>
-		chain_kernel_fn pick_shape(int shape, bool aligned4)
+		template<int NIN, int PROGRAM>
+		chain_kernel_fn pick_shape(int shape, bool direct)
 		{
 			switch (shape)
 			{
-			case 0: return pick_aligned<NIN, 256, 4>(aligned4);
-			case 1: return pick_aligned<NIN, 256, 2>(aligned4);
-			case 2: return pick_aligned<NIN, 256, 1>(aligned4);
-			default: return pick_aligned<NIN, 64, 1>(aligned4);
+			case 0: return pick_direct<NIN, 256, 4, PROGRAM>(direct);
+			case 1: return pick_direct<NIN, 256, 2, PROGRAM>(direct);
+			case 2: return pick_direct<NIN, 256, 1, PROGRAM>(direct);
+			default: return pick_direct<NIN, 64, 1, PROGRAM>(direct);
 			}
 		}
 
-		chain_kernel_fn pick_kernel(uint32_t input_count, int shape, bool aligned4)
+		chain_kernel_fn pick_kernel(uint32_t input_count, int shape, bool direct, int program)
 		{
+			switch (program)
+			{
+			case 1: return pick_shape<1, 1>(shape, direct);
+			case 2: return pick_shape<1, 2>(shape, direct);
+			case 3: return pick_shape<1, 3>(shape, direct);
+			case 4: return pick_shape<1, 4>(shape, direct);
+			case 5: return pick_shape<1, 5>(shape, direct);
+			case 6: return pick_shape<1, 6>(shape, direct);
+			case 7: return pick_shape<1, 7>(shape, direct);
+			default: break;
+			}
 			switch (input_count)
 			{
-			case 1: return pick_shape<1>(shape, aligned4);
-			case 2: return pick_shape<2>(shape, aligned4);
-			case 3: return pick_shape<3>(shape, aligned4);
-			default: return pick_shape<4>(shape, aligned4);
+			case 1: return pick_shape<1, 0>(shape, direct);
+			case 2: return pick_shape<2, 0>(shape, direct);
+			case 3: return pick_shape<3, 0>(shape, direct);
+			default: return pick_shape<4, 0>(shape, direct);
 			}
+		}
+
+		// index into known_programs of a single-input group without Add, 0 when it is not one of them
+		int match_known_program(const nnf_hip_chain_desc& desc, uint32_t op_count)
+		{
+			if ((desc.input_count != 1) || desc.has_add)
+				return 0;
+			for(int p = 1; p < known_program_count; ++p)
+			{
+				if (known_programs[p].op_count != static_cast<int>(op_count))
+					continue;
+				bool same = true;
+				for(uint32_t i = 0; i < op_count; ++i)
+					same = same && (known_programs[p].kinds[i] == desc.ops[i].kind);
+				if (same)
+					return p;
+			}
+			return 0;
 		}
 
 		// Tuning override for experiments: NNF_HIP_CHAIN_SHAPE=<index into launch_shapes>; -1 = automatic.
@@ -531,7 +580,7 @@ namespace nnf
 		a.span = span_of(shape);
 		a.plane_magic = (a.plane >= 2) ? static_cast<uint32_t>(((1ull << 32) + a.plane - 1) / a.plane) : 0u;
 
-		chain_kernel_fn kernel = pick_kernel(desc->input_count, shape, direct_of(shape));
+		chain_kernel_fn kernel = pick_kernel(desc->input_count, shape, direct_of(shape), match_known_program(*desc, op_count));
 		hipLaunchKernelGGL(kernel, dim3(tiles_of(shape)), dim3(launch_shapes[shape].block), lds_bytes_of(shape), stream, a);
 		return launch_status();
 	}

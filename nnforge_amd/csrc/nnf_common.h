@@ -13,14 +13,26 @@ namespace nnf
 
 	constexpr int wave_size = 64;
 
-	// 2^(i/32) table of nnf_expf in device memory (one copy per translation unit); kernels copy it
-	// to LDS before use.
-	static __device__ const uint64_t exp2_table_device[exp2_table_size] = { NNF_EXP2_TABLE_VALUES };
+	// 2^(i/32) table of nnf_expf followed by the two constants of exp_context, in device memory
+	// (one copy per translation unit); kernels copy all of it to LDS before use.
+	constexpr int exp_lds_entries = exp2_table_size + 2;
+	static __device__ const uint64_t exp2_table_device[exp_lds_entries] = { NNF_EXP2_TABLE_VALUES, NNF_EXP_SHIFT_BITS, NNF_EXP_C1_BITS };
 
 	__device__ __forceinline__ void stage_exp2_table(uint64_t* lds_table)
 	{
-		if (threadIdx.x < exp2_table_size)
+		if (threadIdx.x < exp_lds_entries)
 			lds_table[threadIdx.x] = exp2_table_device[threadIdx.x];
+	}
+
+	// after the barrier that follows stage_exp2_table; the constants come from LDS so that they
+	// live in registers
+	__device__ __forceinline__ exp_context exp_context_from_lds(const uint64_t* lds_table)
+	{
+		exp_context ctx;
+		ctx.table = lds_table;
+		ctx.shift = bits_to_double(lds_table[exp2_table_size]);
+		ctx.c1 = bits_to_double(lds_table[exp2_table_size + 1]);
+		return ctx;
 	}
 
 	// Streaming accesses: each byte of an activation tensor is touched once per launch, so loads

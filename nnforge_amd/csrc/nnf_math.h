@@ -4,7 +4,7 @@
 // Rounding policy: every fp32 operation below rounds once, in the order the reference's plain
 // testers write it; translation units that include this header are compiled with
 // -ffp-contract=off so that no multiply-add pair is fused. The only fused operations are the
-// explicit __builtin_fma calls inside nnf_expf, which work in double precision.
+// explicit __builtin_fma calls, all of which are part of a documented evaluation scheme.
 #pragma once
 
 #include <stdint.h>
@@ -31,8 +31,37 @@ namespace nnf
 
 	constexpr int exp2_table_size = 32;
 
+	// Two constants of nnf_expf that the kernels keep in registers (read once per lane from LDS, so
+	// that the compiler holds them in VGPRs instead of re-materialising them before every use).
+	#define NNF_EXP_SHIFT_BITS 0x4338000000000000ull /* 0x1.8p+52 */
+	#define NNF_EXP_C1_BITS 0x3f2ebfce50fac4f3ull    /* 0x1.ebfce50fac4f3p-13 = (ln2/32)^2 / 2, minimax-adjusted */
+
 	NNF_HD double bits_to_double(uint64_t u) { return __builtin_bit_cast(double, u); }
 	NNF_HD uint64_t double_to_bits(double d) { return __builtin_bit_cast(uint64_t, d); }
+
+	// the two 32-bit halves of a little-endian IEEE-754 double
+	struct double_words
+	{
+		uint32_t lo;
+		uint32_t hi;
+	};
+
+	// What nnf_expf needs besides its argument.
+	struct exp_context
+	{
+		const uint64_t* table; // the 32 values of NNF_EXP2_TABLE_VALUES (LDS copy on the device)
+		double shift;          // NNF_EXP_SHIFT_BITS: adding it rounds to an integer kept in the low mantissa bits
+		double c1;             // NNF_EXP_C1_BITS
+	};
+
+	NNF_HD exp_context make_exp_context(const uint64_t* table)
+	{
+		exp_context ctx;
+		ctx.table = table;
+		ctx.shift = bits_to_double(NNF_EXP_SHIFT_BITS);
+		ctx.c1 = bits_to_double(NNF_EXP_C1_BITS);
+		return ctx;
+	}
 
 	// expf with the result of a double-precision evaluation rounded once to fp32.
 	//
@@ -43,23 +72,30 @@ namespace nnf
 	// This is the same published scheme with every multiply-add fused, the form an FMA-capable x86-64
 	// host evaluates; it returns the same bits as that expf for every one of the 2^32 fp32 inputs
 	// (checked exhaustively on the host by the unit tests; NaN payloads aside).
-	//   table: the 32 values of NNF_EXP2_TABLE_VALUES (LDS copy on the device).
-	NNF_HD float nnf_expf(float x, const uint64_t* table)
+	//
+	// The rounded integer k sits in the low word of the shifted sum; only the high word of the table
+	// entry takes part in applying the exponent (k << 47 = (k << 15) in the high word).
+	NNF_HD float nnf_expf(float x, const exp_context& ctx)
 	{
 		const double inv_ln2_times_32 = 0x1.71547652b82fep+5;
-		const double shift = 0x1.8p+52; // adding it rounds to an integer kept in the low mantissa bits
 		const double c0 = 0x1.c6af84b912394p-20; // (ln2/32)^3 / 6, minimax-adjusted
-		const double c1 = 0x1.ebfce50fac4f3p-13; // (ln2/32)^2 / 2
 		const double c2 = 0x1.62e42ff0c52d6p-6;  // ln2/32
 
 		const double xd = static_cast<double>(x);
-		double kd = __builtin_fma(inv_ln2_times_32, xd, shift);
-		const uint64_t ki = double_to_bits(kd);
-		kd -= shift;
+		double kd = __builtin_fma(inv_ln2_times_32, xd, ctx.shift);
+		const uint32_t k = static_cast<uint32_t>(double_to_bits(kd));
+		kd -= ctx.shift;
 		const double r = __builtin_fma(inv_ln2_times_32, xd, -kd);
-		const uint64_t t = table[ki & (exp2_table_size - 1)] + (ki << 47);
-		const double s = bits_to_double(t);
-		const double z = __builtin_fma(c0, r, c1);
+		double_words entry = reinterpret_cast<const double_words*>(ctx.table)[k & (exp2_table_size - 1)];
+		uint32_t scale_hi = entry.hi + (k << 15);
+#if defined(__HIP_DEVICE_COMPILE__)
+		// keeps the addition a 32-bit one (the compiler otherwise widens it to a 64-bit add with
+		// extra register moves)
+		asm volatile("" : "+v"(scale_hi));
+#endif
+		entry.hi = scale_hi;
+		const double s = __builtin_bit_cast(double, entry);
+		const double z = __builtin_fma(c0, r, ctx.c1);
 		const double r2 = r * r;
 		double y = __builtin_fma(c2, r, 1.0);
 		y = __builtin_fma(z, r2, y);
@@ -70,6 +106,42 @@ namespace nnf
 		res = x > 0x1.62e42ep6f ? __builtin_inff() : res;
 		res = x < -0x1.9fe368p6f ? 0.0f : res;
 		return res;
+	}
+
+	// numerator[i] / denominator[i] for denominators that are >= 1, +inf or NaN - the only divisions
+	// the layers below make (e + 1 with e = expf(...) >= 0). On the device: reciprocal estimate, one
+	// Newton step, then quotient, exact remainder and correction (each an FMA), which yields the
+	// correctly rounded quotient as long as the reciprocal is a normal number; a wavefront that holds
+	// a denominator above 2^126 (or inf / NaN) anywhere in the batch redoes the batch with the general
+	// IEEE division (one uniform branch per batch, so the fast sequences of a batch interleave freely).
+	// Compared with IEEE division over every possible e (all non-negative floats, +inf, NaN):
+	// identical bits.
+	template<int N>
+	NNF_HD void nnf_divide_by_ge1(const float (&numerator)[N], const float (&denominator)[N], float (&quotient)[N])
+	{
+#if defined(__HIP_DEVICE_COMPILE__)
+		bool out_of_range = false;
+		#pragma unroll
+		for(int i = 0; i < N; ++i)
+		{
+			float r = __builtin_amdgcn_rcpf(denominator[i]);
+			const float e = __builtin_fmaf(-denominator[i], r, 1.0f);
+			r = __builtin_fmaf(e, r, r);
+			float q = numerator[i] * r;
+			const float rem = __builtin_fmaf(-denominator[i], q, numerator[i]);
+			quotient[i] = __builtin_fmaf(rem, r, q);
+			out_of_range = out_of_range || !(denominator[i] <= 0x1p126f);
+		}
+		if (__builtin_expect(__any(out_of_range), 0))
+		{
+			#pragma unroll
+			for(int i = 0; i < N; ++i)
+				quotient[i] = numerator[i] / denominator[i];
+		}
+#else
+		for(int i = 0; i < N; ++i)
+			quotient[i] = numerator[i] / denominator[i];
+#endif
 	}
 
 	// nnforge/plain/batch_norm_layer_tester_plain.cpp:60-61
@@ -99,25 +171,51 @@ namespace nnf
 		return x * (x >= 0.0f ? 1.0f : a);
 	}
 
+	// The layers that call expf work on small batches of values (the registers a lane holds), in place.
+
 	// nnforge/plain/exponential_linear_layer_tester_plain.cpp:50-51
-	NNF_HD float nnf_exponential_linear(float x, const uint64_t* table)
+	template<int N>
+	NNF_HD void nnf_exponential_linear(float (&v)[N], const exp_context& ctx)
 	{
-		const float e = nnf_expf(x, table);
-		return x >= 0.0f ? x : (e - 1.0f);
+		#pragma unroll
+		for(int i = 0; i < N; ++i)
+		{
+			const float x = v[i];
+			const float e = nnf_expf(x, ctx);
+			v[i] = x >= 0.0f ? x : (e - 1.0f);
+		}
 	}
 
 	// nnforge/plain/sigmoid_layer_tester_plain.cpp:50-51
-	NNF_HD float nnf_sigmoid(float x, const uint64_t* table)
+	template<int N>
+	NNF_HD void nnf_sigmoid(float (&v)[N], const exp_context& ctx)
 	{
-		const float e = nnf_expf(-x, table);
-		return 1.0f / (e + 1.0f);
+		float one[N], denominator[N];
+		#pragma unroll
+		for(int i = 0; i < N; ++i)
+		{
+			const float e = nnf_expf(-v[i], ctx);
+			one[i] = 1.0f;
+			denominator[i] = e + 1.0f;
+		}
+		nnf_divide_by_ge1<N>(one, denominator, v);
 	}
 
 	// nnforge/plain/hyperbolic_tangent_layer_tester_plain.cpp:54-56; steepness2 = steepness * 2.0f
-	NNF_HD float nnf_hyperbolic_tangent(float x, float steepness2, float scale, const uint64_t* table)
+	template<int N>
+	NNF_HD void nnf_hyperbolic_tangent(float (&v)[N], float steepness2, float scale, const exp_context& ctx)
 	{
-		const float e = nnf_expf(x * steepness2, table);
-		const float q = (e - 1.0f) / (e + 1.0f);
-		return q * scale;
+		float numerator[N], denominator[N];
+		#pragma unroll
+		for(int i = 0; i < N; ++i)
+		{
+			const float e = nnf_expf(v[i] * steepness2, ctx);
+			numerator[i] = e - 1.0f;
+			denominator[i] = e + 1.0f;
+		}
+		nnf_divide_by_ge1<N>(numerator, denominator, v);
+		#pragma unroll
+		for(int i = 0; i < N; ++i)
+			v[i] = v[i] * scale;
 	}
 }

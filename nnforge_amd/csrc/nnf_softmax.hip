@@ -82,10 +82,11 @@ namespace nnf
 		template<int THREADS, int VPT, int W>
 		__global__ void __launch_bounds__(1024) softmax_rows_kernel(float* out, const float* in, uint32_t rows, uint32_t fm_count)
 		{
-			__shared__ uint64_t lds_exp[exp2_table_size];
+			__shared__ uint64_t lds_exp[exp_lds_entries];
 			__shared__ float lds_partial[2][1024 / wave_size];
 			stage_exp2_table(lds_exp);
 			__syncthreads();
+			const exp_context exp_ctx = exp_context_from_lds(lds_exp);
 
 			const uint32_t rows_per_block = blockDim.x / THREADS;
 			const uint32_t lane = threadIdx.x % THREADS;
@@ -130,7 +131,7 @@ namespace nnf
 					#pragma unroll
 					for(int e = 0; e < W; ++e)
 					{
-						v[k][e] = nnf_expf(v[k][e] - m, lds_exp);
+						v[k][e] = nnf_expf(v[k][e] - m, exp_ctx);
 						sum += v[k][e];
 					}
 				}
@@ -167,7 +168,7 @@ namespace nnf
 		// like the reference does.
 		__global__ void __launch_bounds__(1024) softmax_long_rows_kernel(float* out, const float* in, uint32_t fm_count)
 		{
-			__shared__ uint64_t lds_exp[exp2_table_size];
+			__shared__ uint64_t lds_exp[exp_lds_entries];
 			__shared__ float lds_partial[2][1024 / wave_size];
 			stage_exp2_table(lds_exp);
 
@@ -183,6 +184,7 @@ namespace nnf
 			if ((threadIdx.x % wave_size) == 0)
 				lds_partial[0][wave] = m;
 			__syncthreads();
+			const exp_context exp_ctx = exp_context_from_lds(lds_exp);
 			m = softmax_max_init;
 			for(uint32_t w = 0; w < wave_count; ++w)
 				m = ref_max(m, lds_partial[0][w]);
@@ -190,7 +192,7 @@ namespace nnf
 			float sum = 0.0f;
 			for(uint32_t c = threadIdx.x; c < fm_count; c += blockDim.x)
 			{
-				const float val = nnf_expf(src[c] - m, lds_exp);
+				const float val = nnf_expf(src[c] - m, exp_ctx);
 				sum += val;
 				dst[c] = val;
 			}
@@ -213,9 +215,10 @@ namespace nnf
 		template<int CACHED>
 		__global__ void __launch_bounds__(256) softmax_columns_kernel(float* out, const float* in, uint32_t columns, uint32_t fm_count, uint32_t plane)
 		{
-			__shared__ uint64_t lds_exp[exp2_table_size];
+			__shared__ uint64_t lds_exp[exp_lds_entries];
 			stage_exp2_table(lds_exp);
 			__syncthreads();
+			const exp_context exp_ctx = exp_context_from_lds(lds_exp);
 
 			const uint32_t column = blockIdx.x * blockDim.x + threadIdx.x;
 			if (column >= columns)
@@ -245,7 +248,7 @@ namespace nnf
 				{
 					if (static_cast<uint32_t>(c) < fm_count)
 					{
-						v[c] = nnf_expf(v[c] - m, lds_exp);
+						v[c] = nnf_expf(v[c] - m, exp_ctx);
 						sum += v[c];
 					}
 				}
@@ -265,7 +268,7 @@ namespace nnf
 				float sum = 0.0f;
 				for(uint32_t c = 0; c < fm_count; ++c)
 				{
-					const float val = nnf_expf(src[static_cast<size_t>(c) * plane] - m, lds_exp);
+					const float val = nnf_expf(src[static_cast<size_t>(c) * plane] - m, exp_ctx);
 					sum += val;
 					dst[static_cast<size_t>(c) * plane] = val;
 				}

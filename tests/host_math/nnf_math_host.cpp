@@ -11,6 +11,8 @@ namespace
 {
 	const uint64_t exp2_table[nnf::exp2_table_size] = { NNF_EXP2_TABLE_VALUES };
 
+	const nnf::exp_context exp_ctx = nnf::make_exp_context(exp2_table);
+
 	inline uint32_t bits_of(float f) { uint32_t u; std::memcpy(&u, &f, 4); return u; }
 	inline float float_of(uint32_t u) { float f; std::memcpy(&f, &u, 4); return f; }
 }
@@ -30,7 +32,7 @@ extern "C"
 		{
 			const uint32_t u = static_cast<uint32_t>(first + static_cast<unsigned long long>(i) * stride);
 			const float x = float_of(u);
-			const float a = nnf::nnf_expf(x, exp2_table);
+			const float a = nnf::nnf_expf(x, exp_ctx);
 			const float b = expf(x);
 			if ((bits_of(a) != bits_of(b)) && !((a != a) && (b != b)))
 			{
@@ -51,7 +53,7 @@ extern "C"
 	void nnf_host_expf(float* out, const float* in, long long count)
 	{
 		for(long long i = 0; i < count; ++i)
-			out[i] = nnf::nnf_expf(in[i], exp2_table);
+			out[i] = nnf::nnf_expf(in[i], exp_ctx);
 	}
 
 	// kind: nnf_hip_op_kind values (1 batch norm .. 6 tanh); p0..p3: per-kind scalars
@@ -72,9 +74,9 @@ extern "C"
 			case 1: y = nnf::nnf_batch_norm(x, mult, add); break;
 			case 2: y = nnf::nnf_rectified_linear(x, p0); break;
 			case 3: y = nnf::nnf_parametric_rectified_linear(x, p0); break;
-			case 4: y = nnf::nnf_exponential_linear(x, exp2_table); break;
-			case 5: y = nnf::nnf_sigmoid(x, exp2_table); break;
-			case 6: y = nnf::nnf_hyperbolic_tangent(x, steepness2, p0, exp2_table); break;
+			case 4: { float one[1] = { x }; nnf::nnf_exponential_linear<1>(one, exp_ctx); y = one[0]; } break;
+			case 5: { float one[1] = { x }; nnf::nnf_sigmoid<1>(one, exp_ctx); y = one[0]; } break;
+			case 6: { float one[1] = { x }; nnf::nnf_hyperbolic_tangent<1>(one, steepness2, p0, exp_ctx); y = one[0]; } break;
 			default: break;
 			}
 			out[i] = y;

@@ -419,3 +419,37 @@ def test_average_subsampling_windows(gpu, shape, ww, wh):
     got = run_pool(gpu, x, ww, wh, mult)
     assert got.shape == want.shape
     assert T.bit_mismatches(got, want) == 0
+
+
+# ---------------------------------------------------------------------------------------------
+# every fp32 input through the layers that call expf and divide
+# ---------------------------------------------------------------------------------------------
+
+def test_exp_layers_over_the_whole_fp32_range(gpu):
+    """ELU, Sigmoid and TanH against the oracle on a regular sweep of ALL fp32 bit patterns (every
+    61st by default, every single one with NNF_EXHAUSTIVE=1): the device expf and the device's
+    short division sequence must reproduce libm's expf and IEEE division bit for bit, including
+    the inputs where expf under- or overflows and where the quotient is subnormal."""
+    import os
+
+    stride = 1 if os.environ.get("NNF_EXHAUSTIVE") == "1" else 61
+    chunk = 1 << 26
+    lib = gpu.lib
+    total_bad = 0
+    checked = 0
+    for start in range(0, 1 << 32, chunk * stride):
+        bits = np.arange(start, min(start + chunk * stride, 1 << 32), stride, dtype=np.uint64).astype(np.uint32)
+        x = bits.view(np.float32)
+        with np.errstate(all="ignore"):
+            cases = [
+                (run_flat(gpu, lib.nnf_hip_exponential_linear_forward, x), oracle.exponential_linear(x), "elu"),
+                (run_flat(gpu, lib.nnf_hip_sigmoid_forward, x), oracle.sigmoid(x), "sigmoid"),
+                # steepness 0.5: the exponent argument is x itself, so e runs over the whole image of expf
+                (run_flat(gpu, lib.nnf_hip_hyperbolic_tangent_forward, x, 1.0, 0.5), oracle.hyperbolic_tangent(x, 1.0, 0.5), "tanh"),
+            ]
+        for got, want, what in cases:
+            bad = T.bit_mismatches(got, want)
+            assert bad == 0, "%s: %d mismatches in the chunk starting at bit pattern 0x%08x" % (what, bad, start)
+            total_bad += bad
+        checked += x.size
+    print("exp layers: %d inputs per layer checked, %d mismatches" % (checked, total_bad))
