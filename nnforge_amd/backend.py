@@ -7,6 +7,7 @@ import os
 import numpy as np
 
 from . import build as _build
+from .capi import _share_hip_runtime_with_torch
 
 _FP = ctypes.POINTER(ctypes.c_float)
 _UP = ctypes.POINTER(ctypes.c_uint32)
@@ -48,6 +49,7 @@ def load():
         path = _build.BACKEND_LIBRARY
         if not os.path.exists(path):
             raise RuntimeError("%s is missing: build it first (python -c 'import __graft_entry__ as g; g.build()')" % path)
+        _share_hip_runtime_with_torch()
         lib = ctypes.CDLL(path)
         lib.nnf_backend_run_schema.argtypes = [ctypes.c_char_p, ctypes.POINTER(Weights), ctypes.c_uint32, ctypes.POINTER(Input),
                                                ctypes.c_uint32, ctypes.c_uint32, ctypes.POINTER(Output), ctypes.c_uint32,

@@ -97,6 +97,17 @@ class NnfHipError(RuntimeError):
         self.code = code
 
 
+def _share_hip_runtime_with_torch():
+    """PyTorch wheels bundle their own HIP runtime. A process must not end up with two of them
+    (the one loaded second does not see the GPU), so when torch is installed it is imported before
+    this library is loaded: the library's libamdhip64 dependency then resolves to the runtime torch
+    already mapped. Without torch the system's ROCm runtime is used."""
+    try:
+        import torch  # noqa: F401
+    except ImportError:
+        pass
+
+
 def library_path():
     return _build.HIP_LIBRARY
 
@@ -110,6 +121,7 @@ def load():
     if not os.path.exists(path):
         raise RuntimeError(
             "%s is missing: build it first (python -c 'import __graft_entry__ as g; g.build()')" % path)
+    _share_hip_runtime_with_torch()
     lib = ctypes.CDLL(path)
     for name, argtypes in SIGNATURES.items():
         fn = getattr(lib, name)

@@ -69,7 +69,7 @@ namespace nnf
 		// DIRECT: where[k][0] is the feature map of float4 k and per-feature-map weights are read from
 		// memory (all lanes of a wavefront read the same one or two addresses: one cache line).
 		// Otherwise where[k][e] indexes the coefficient arrays the workgroup staged in LDS.
-		template<int U, bool DIRECT>
+		template<int U, bool DIRECT, int EXP_BATCH>
 		__device__ __forceinline__ void apply_op(
 			int kind,
 			const chain_op& op,
@@ -145,14 +145,25 @@ namespace nnf
 					}
 				}
 				break;
+			// The layers that call expf work on batches of EXP_BATCH values (a divisor of 4, or U * 4:
+			// the registers of a lane are contiguous). Wider batches
+			// let independent evaluations interleave but cost registers, and with them occupancy, in every
+			// group a kernel instance runs: the general instance, which also runs the bandwidth-bound
+			// groups, uses 1.
 			case NNF_HIP_OP_ELU:
-				nnf_exponential_linear<U * 4>(reinterpret_cast<float (&)[U * 4]>(v), exp_ctx);
+				#pragma unroll
+				for(int i = 0; i < U * 4; i += EXP_BATCH)
+					nnf_exponential_linear<EXP_BATCH>(reinterpret_cast<float (&)[EXP_BATCH]>(v[i / 4][i % 4]), exp_ctx);
 				break;
 			case NNF_HIP_OP_SIGMOID:
-				nnf_sigmoid<U * 4>(reinterpret_cast<float (&)[U * 4]>(v), exp_ctx);
+				#pragma unroll
+				for(int i = 0; i < U * 4; i += EXP_BATCH)
+					nnf_sigmoid<EXP_BATCH>(reinterpret_cast<float (&)[EXP_BATCH]>(v[i / 4][i % 4]), exp_ctx);
 				break;
 			case NNF_HIP_OP_TANH:
-				nnf_hyperbolic_tangent<U * 4>(reinterpret_cast<float (&)[U * 4]>(v), op.f1, op.f0, exp_ctx); // f1 holds steepness * 2
+				#pragma unroll
+				for(int i = 0; i < U * 4; i += EXP_BATCH)
+					nnf_hyperbolic_tangent<EXP_BATCH>(reinterpret_cast<float (&)[EXP_BATCH]>(v[i / 4][i % 4]), op.f1, op.f0, exp_ctx); // f1 holds steepness * 2
 				break;
 			default:
 				break;
@@ -273,7 +284,7 @@ namespace nnf
 			{
 				#pragma unroll
 				for(int i = 0; i < known_programs[PROGRAM].op_count; ++i)
-					apply_op<U, DIRECT>(known_programs[PROGRAM].kinds[i], a.ops[i], a, x[0], where, lds_coeff, exp_ctx);
+					apply_op<U, DIRECT, U * 4>(known_programs[PROGRAM].kinds[i], a.ops[i], a, x[0], where, lds_coeff, exp_ctx);
 				op_index = known_programs[PROGRAM].op_count;
 			}
 			else
@@ -283,7 +294,7 @@ namespace nnf
 				{
 					const uint32_t arm_end = op_index + a.arm_ops[j];
 					for(; op_index < arm_end; ++op_index)
-						apply_op<U, DIRECT>(a.ops[op_index].kind, a.ops[op_index], a, x[j], where, lds_coeff, exp_ctx);
+						apply_op<U, DIRECT, 1>(a.ops[op_index].kind, a.ops[op_index], a, x[j], where, lds_coeff, exp_ctx);
 				}
 			}
 
@@ -309,7 +320,7 @@ namespace nnf
 			{
 				const uint32_t tail_end = op_index + a.tail_ops;
 				for(; op_index < tail_end; ++op_index)
-					apply_op<U, DIRECT>(a.ops[op_index].kind, a.ops[op_index], a, x[0], where, lds_coeff, exp_ctx);
+					apply_op<U, DIRECT, 1>(a.ops[op_index].kind, a.ops[op_index], a, x[0], where, lds_coeff, exp_ctx);
 			}
 
 			#pragma unroll
@@ -354,7 +365,9 @@ namespace nnf
 		{
 			switch (shape)
 			{
-			case 0: return pick_direct<NIN, 256, 4, PROGRAM>(direct);
+			// the compile-time programs are bound by the vector ALU: four float4s per lane would only
+			// cost them occupancy
+			case 0: return pick_direct<NIN, 256, (PROGRAM > 0) ? 2 : 4, PROGRAM>(direct);
 			case 1: return pick_direct<NIN, 256, 2, PROGRAM>(direct);
 			case 2: return pick_direct<NIN, 256, 1, PROGRAM>(direct);
 			default: return pick_direct<NIN, 64, 1, PROGRAM>(direct);
@@ -575,12 +588,13 @@ namespace nnf
 			if (shape < 0)
 				return NNF_HIP_EUNSUPPORTED;
 		}
-		const uint32_t tile = launch_shapes[shape].block * launch_shapes[shape].unroll * 4;
-		(void)tile;
+		const int program = match_known_program(*desc, op_count);
+		if ((program > 0) && (shape == 0))
+			shape = 1; // the compile-time programs have no four-float4 instance (smaller tile: LDS still fits)
 		a.span = span_of(shape);
 		a.plane_magic = (a.plane >= 2) ? static_cast<uint32_t>(((1ull << 32) + a.plane - 1) / a.plane) : 0u;
 
-		chain_kernel_fn kernel = pick_kernel(desc->input_count, shape, direct_of(shape), match_known_program(*desc, op_count));
+		chain_kernel_fn kernel = pick_kernel(desc->input_count, shape, direct_of(shape), program);
 		hipLaunchKernelGGL(kernel, dim3(tiles_of(shape)), dim3(launch_shapes[shape].block), lds_bytes_of(shape), stream, a);
 		return launch_status();
 	}
