@@ -49,8 +49,10 @@ HOST_DIR = os.path.join(PACKAGE_DIR, "host")
 BACKEND_LIBRARY = os.path.join(PACKAGE_DIR, "libnnforge_hip_backend.so")
 BACKEND_SOURCES = ["core.cpp", "layers.cpp", "schema.cpp", "propagation.cpp", "hip_testers.cpp",
                    "forward_propagation_hip.cpp", "backend_capi.cpp"]
-BACKEND_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden", "-Wall", "-Wextra",
-                 "-Wno-unused-parameter"]
+# default symbol visibility: the C++ classes are the library's interface
+BACKEND_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wextra", "-Wno-unused-parameter"]
+
+USAGE_PROGRAM = os.path.join(REPO_ROOT, "tests", "cpp", "backend_usage")
 
 
 def build_backend_library(verbose=False):
@@ -69,8 +71,22 @@ def build_backend_library(verbose=False):
     return BACKEND_LIBRARY
 
 
+def build_usage_program(verbose=False):
+    """Compiles tests/cpp/backend_usage.cpp: a C++ program that uses the backend the way an nnForge
+    application uses one (run by the GPU tests)."""
+    tmp = USAGE_PROGRAM + ".tmp"
+    cmd = ["g++", "-O2", "-std=c++17", "-ffp-contract=off", "-Wall", "-I", os.path.join(REPO_ROOT, "include"), "-o", tmp,
+           USAGE_PROGRAM + ".cpp", "-L", PACKAGE_DIR, "-lnnforge_hip_backend", "-lnnforge_hip",
+           "-Wl,-rpath,$ORIGIN/../../nnforge_amd"]
+    out = _run(cmd)
+    os.replace(tmp, USAGE_PROGRAM)
+    if verbose and out.strip():
+        print(out)
+    return USAGE_PROGRAM
+
+
 def build_all(verbose=False):
-    built = [build_hip_library(verbose), build_backend_library(verbose)]
+    built = [build_hip_library(verbose), build_backend_library(verbose), build_usage_program(verbose)]
     return built
 
 

@@ -1,0 +1,179 @@
+// The hip backend used from C++ the way an nnForge application uses a backend
+// (examples/gtsrb/gtsrb.cpp:29-63 + toolset::run_inference, nnforge/toolset.cpp:551-575):
+// factory_generator -> forward_propagation_factory -> forward_propagation, a schema in text
+// format, weights as network_data, a reader and a writer. Prints "ok" when the network's output
+// equals a straightforward host evaluation of the same layers bit for bit.
+#include <nnforge_hip/hip_backend.h>
+
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <iostream>
+#include <random>
+#include <sstream>
+
+using namespace nnforge;
+
+namespace
+{
+	const char * schema_text = R"(
+name: "usage"
+layer { type: "Data" name: "conv_main" }
+layer { type: "Data" name: "conv_shortcut" }
+layer { type: "BatchNorm" name: "main_bn" input_layer_name: "conv_main" batch_norm_param { feature_map_count: 6 } }
+layer { type: "Add" name: "res" input_layer_name: "conv_shortcut" input_layer_name: "main_bn" }
+layer { type: "PReLU" name: "res_prelu" input_layer_name: "res" prelu_param { feature_map_count: 6 } }
+layer { type: "AverageSubsampling" name: "pool" input_layer_name: "res_prelu"
+	average_subsampling_param { dimension_param { subsampling_size: 7 } dimension_param { subsampling_size: 7 } alpha: 0.0204081628 } }
+layer { type: "Softmax" name: "prob" input_layer_name: "pool" }
+)";
+
+	// a reader that produces entries on the fly and ends after entry_count entries
+	class generated_reader : public structured_data_bunch_reader
+	{
+	public:
+		generated_reader(unsigned int entry_count, const layer_configuration_specific& config) : entry_count(entry_count), config(config) {}
+		std::map<std::string, layer_configuration_specific> get_config_map() const override
+		{
+			std::map<std::string, layer_configuration_specific> res;
+			res["conv_main"] = config;
+			res["conv_shortcut"] = config;
+			return res;
+		}
+		static float value(unsigned int entry_id, unsigned int layer, unsigned int i)
+		{
+			return std::sin(0.37f * static_cast<float>(i + 31 * entry_id) + 1.3f * static_cast<float>(layer)) * 2.0f;
+		}
+		bool read(unsigned int entry_id, const std::map<std::string, float *>& data_map) override
+		{
+			if (entry_id >= entry_count)
+				return false;
+			for(const std::pair<const std::string, float *>& item : data_map)
+				for(unsigned int i = 0; i < config.get_neuron_count(); ++i)
+					item.second[i] = value(entry_id, item.first == "conv_main" ? 0 : 1, i);
+			return true;
+		}
+		int get_entry_count() const override { return -1; } // unknown: the driver has to find the end
+
+	private:
+		unsigned int entry_count;
+		layer_configuration_specific config;
+	};
+}
+
+int main()
+{
+	try
+	{
+		hip::factory_generator_hip generator;
+		generator.apply_default_options();
+		generator.hip_max_entry_count = 5; // several packets
+		generator.initialize();
+		generator.info();
+
+		network_schema schema;
+		std::istringstream in(schema_text);
+		schema.read_proto(in);
+
+		const unsigned int c = 6, entries = 13;
+		network_data data(schema.get_layers());
+		data.initialize(schema.get_layers());
+		std::mt19937 gen(7);
+		std::uniform_real_distribution<float> dist(0.5F, 1.5F);
+		for(std::vector<float>& chunk : *data.get("main_bn"))
+			for(float& v : chunk)
+				v = dist(gen);
+		for(float& v : (*data.get("res_prelu"))[0])
+			v = dist(gen) * 0.2F;
+
+		std::vector<std::string> outputs;
+		outputs.push_back("prob");
+		outputs.push_back("res_prelu");
+		forward_propagation::ptr fp = generator.create_forward_propagation_factory()->create(
+			schema, outputs, debug_state::ptr(new debug_state(true)), profile_state::ptr(new profile_state(true)));
+		fp->set_data(data);
+
+		const layer_configuration_specific config(c, std::vector<unsigned int>(2, 7));
+		generated_reader reader(entries, config);
+		memory_data_bunch_writer writer;
+		const forward_propagation::stat st = fp->run(reader, writer);
+		std::cout << st << std::endl;
+		if (st.entry_processed_count != entries)
+		{
+			std::cout << "processed " << st.entry_processed_count << " entries, expected " << entries << std::endl;
+			return 1;
+		}
+
+		// host evaluation, same operation order (compiled without contraction)
+		const layer_data& bn = *data.get("main_bn");
+		const std::vector<float>& slopes = (*data.get("res_prelu"))[0];
+		unsigned int mismatches = 0;
+		for(unsigned int e = 0; e < entries; ++e)
+		{
+			float pooled[6];
+			for(unsigned int f = 0; f < c; ++f)
+			{
+				const float mult = bn[0][f] * bn[3][f];
+				const float add = bn[1][f] - mult * bn[2][f];
+				float sum = 0.0F;
+				for(unsigned int p = 0; p < 49; ++p)
+				{
+					const unsigned int i = f * 49 + p;
+					const float main_v = generated_reader::value(e, 0, i) * mult + add;
+					float r = 0.0F;
+					r += generated_reader::value(e, 1, i);
+					r += main_v;
+					r = r * 1.0F;
+					const float y = r * (r >= 0.0F ? 1.0F : slopes[f]);
+					const float got = writer.values["res_prelu"][static_cast<size_t>(e) * c * 49 + i];
+					if (std::memcmp(&got, &y, 4) != 0)
+						++mismatches;
+					sum += y;
+				}
+				pooled[f] = sum * 0.0204081628F;
+			}
+			float max_val = -1.0e+37F;
+			for(unsigned int f = 0; f < c; ++f)
+				max_val = std::max(max_val, pooled[f]);
+			float ex[6], sum = 0.0F;
+			for(unsigned int f = 0; f < c; ++f)
+			{
+				ex[f] = expf(pooled[f] - max_val);
+				sum += ex[f];
+			}
+			const float mult = 1.0F / sum;
+			for(unsigned int f = 0; f < c; ++f)
+			{
+				const float want = ex[f] * mult;
+				const float got = writer.values["prob"][static_cast<size_t>(e) * c + f];
+				if (std::fabs(got - want) > 1.0e-5F * want)
+					++mismatches;
+			}
+		}
+		for(const std::pair<const std::string, float>& a : fp->get_last_action_seconds())
+			std::cout << "action " << a.first << ": " << a.second << " s" << std::endl;
+		if (mismatches != 0)
+		{
+			std::cout << mismatches << " mismatches" << std::endl;
+			return 1;
+		}
+
+		// what the reference's classes throw, the backend throws too
+		try
+		{
+			generator.create_backward_propagation_factory();
+			std::cout << "backward propagation did not throw" << std::endl;
+			return 1;
+		}
+		catch (const neural_network_exception&)
+		{
+		}
+		std::cout << "ok" << std::endl;
+		return 0;
+	}
+	catch (const std::exception& e)
+	{
+		std::cout << "exception: " << e.what() << std::endl;
+		return 1;
+	}
+}

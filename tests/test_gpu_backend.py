@@ -99,3 +99,21 @@ def test_run_errors():
     bad["main_bn"] = [w[:5] for w in weights["main_bn"]]
     with pytest.raises(backend.BackendError, match="data weight count 5 for vector 0 doesn't satisfy layer configuration 8"):
         run(layers, bad, inputs, ["res_relu"], values)
+
+
+def test_cpp_application_uses_the_backend_like_a_reference_backend():
+    """tests/cpp/backend_usage.cpp: factory_generator_hip -> forward_propagation_hip from C++ with
+    a reader of unknown length, several packets, debug and profile switched on."""
+    import os
+    import subprocess
+
+    from nnforge_amd import build
+
+    assert os.path.exists(build.USAGE_PROGRAM), "build it first: python -c 'import __graft_entry__ as g; g.build()'"
+    proc = subprocess.run([build.USAGE_PROGRAM], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120)
+    assert proc.returncode == 0, proc.stdout
+    lines = proc.stdout.strip().splitlines()
+    assert lines[-1] == "ok", proc.stdout
+    assert any("[fused] main_bn+res+res_prelu <- conv_shortcut, conv_main" in l for l in lines), proc.stdout
+    assert any(l.startswith("action main_bn+res+res_prelu:") for l in lines), proc.stdout
+    assert any("13 entries" in l for l in lines), proc.stdout
