@@ -30,9 +30,14 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 METRIC = "achieved HBM GB/s (% of MI355X peak) + elements/s, fused BN+ReLU fp32 fwd"
 SEED = 0x6E6E4600
 
-# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
-# (see profiles/); None until measured for a workload.
-MEASURED_TRAFFIC_BYTES = {}
+# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs,
+# each counter scaled by what it reads for the 256 MiB copy kernel (profiles/chain_kernel_*.md);
+# None for workloads that have not been measured.
+MEASURED_TRAFFIC_BYTES = {
+    "config0": 51572531,    # algorithmic 51,381,248
+    "config2": 1233157734,  # algorithmic 1,233,130,496
+    "config3": 205645312,   # algorithmic 205,529,088
+}
 
 
 def fail(msg, code=2):
