@@ -4,8 +4,10 @@
 // Work split: the tensor is a flat array of floats cut into tiles of block_size * U float4s; one
 // workgroup per tile. Lane t of the workgroup owns float4s t, t + block_size, ... of the tile, so every
 // load and store instruction of a wavefront covers 1 KiB of consecutive memory. A tile spans only a
-// few feature-map planes; the per-feature-map coefficients of those planes (batch-norm mult/add,
-// PReLU slope) are computed once per workgroup into LDS and looked up by plane index.
+// few feature-map planes. When planes are float4-aligned, a lane reads the per-feature-map weights of
+// its float4 straight from memory (the lanes of a wavefront hit one or two addresses); otherwise the
+// coefficients of the planes a tile touches (batch-norm mult/add, PReLU slope) are computed once per
+// workgroup into LDS and looked up per element.
 #include "nnf_common.h"
 
 #include <cstdlib>

@@ -4,9 +4,10 @@
 //
 // Two data shapes:
 //  - neuron_count_per_feature_map == 1: the feature maps of an entry are contiguous ("rows").
-//    A row lives in the registers of one wavefront (or one workgroup for long rows); max and sum
-//    are 64-lane reductions; the row is read once and written once. The sum is a fixed tree, so it
-//    can differ from the reference's left-to-right sum in the last bits.
+//    A row lives in the registers of one wavefront, or of several when the row is long or the rows
+//    are few; max and sum are 64-lane reductions (combined through LDS across wavefronts); the row is
+//    read once and written once. The sum is a fixed tree, so it can differ from the reference's
+//    left-to-right sum in the last bits.
 //  - neuron_count_per_feature_map > 1: feature maps are strided by the plane size ("columns").
 //    Lanes run along the spatial positions (coalesced), each lane walks its column in feature-map
 //    order with the reference's own sequential sum.
