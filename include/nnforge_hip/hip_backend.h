@@ -225,6 +225,7 @@ namespace nnforge
 				std::map<std::string, float>& action_seconds,
 				float& idle_seconds) override;
 			void layer_config_map_modified() override;
+			float get_max_bytes_per_second() const override; // HBM peak of the MI355X
 
 		private:
 			struct impl;

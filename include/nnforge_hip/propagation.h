@@ -79,12 +79,19 @@ namespace nnforge
 		bool debug_mode;
 	};
 
+	// nnforge/profile_state.h: the switch and the folder the per-action reports go to (empty folder:
+	// times are collected but no file is written)
 	struct profile_state
 	{
 		typedef std::shared_ptr<profile_state> ptr;
-		explicit profile_state(bool profile_mode = false) : profile_mode(profile_mode) {}
+		explicit profile_state(bool profile_mode = false, const std::string& profile_folder = std::string())
+			: profile_mode(profile_mode), profile_folder(profile_folder), index(0) {}
 		bool is_profile() const { return profile_mode; }
+		// <folder>/<prefix>_NNN.<extension>, NNN counting up per call
+		std::string get_path_to_unique_file(const char * file_prefix, const char * file_extension);
 		bool profile_mode;
+		std::string profile_folder;
+		unsigned int index;
 	};
 
 	// nnforge/forward_propagation.h:39-115
@@ -137,6 +144,12 @@ namespace nnforge
 		// called when set_input_configuration_specific changed layer_config_map
 		virtual void layer_config_map_modified() = 0;
 
+		// what the backend can do at best, for the "relative to peak" columns of the profile report
+		// (nnforge/forward_propagation.h:94 get_max_flops; bytes per second is the figure that matters
+		// for the bandwidth-bound layers of this backend)
+		virtual float get_max_flops() const;
+		virtual float get_max_bytes_per_second() const { return 0.0F; }
+
 	protected:
 		network_schema::const_ptr schema; // reduced to what the outputs need
 		std::vector<std::string> output_layer_names;
@@ -146,6 +159,11 @@ namespace nnforge
 		float flops;
 		std::set<std::string> data_layer_names;
 		std::map<std::string, float> last_action_seconds;
+		// per action (same keys as the action seconds): the reference's flops model, the memory
+		// traffic the action needs per entry, and the layer types it covers
+		std::map<std::string, float> action_flops_per_entry;
+		std::map<std::string, float> action_bytes_per_entry;
+		std::map<std::string, std::string> action_layer_types;
 
 	private:
 		forward_propagation() = delete;

@@ -52,6 +52,7 @@ typedef struct nnf_backend_options
 	int32_t profile;               /* per-launch times in the report */
 	int32_t weights_from_folder;   /* 1: `weights_folder` holds <layer>.data files */
 	const char* weights_folder;
+	const char* profile_folder;    /* with profile: folder for forward_prop_perf_per_layer_action_NNN.csv; null: no file */
 } nnf_backend_options;
 
 /* Runs the schema on device 0. The report lists one line per launch ("step: ..."), the buffer plan

@@ -30,7 +30,8 @@ class Output(ctypes.Structure):
 
 class Options(ctypes.Structure):
     _fields_ = [("fuse", ctypes.c_int32), ("dont_share_buffers", ctypes.c_int32), ("max_entry_count", ctypes.c_int32),
-                ("profile", ctypes.c_int32), ("weights_from_folder", ctypes.c_int32), ("weights_folder", ctypes.c_char_p)]
+                ("profile", ctypes.c_int32), ("weights_from_folder", ctypes.c_int32), ("weights_folder", ctypes.c_char_p),
+                ("profile_folder", ctypes.c_char_p)]
 
 
 class BackendError(RuntimeError):
@@ -65,7 +66,8 @@ def load():
     return _lib
 
 
-def _options(fuse=True, dont_share_buffers=False, max_entry_count=0, profile=False, weights_folder=None):
+def _options(fuse=True, dont_share_buffers=False, max_entry_count=0, profile=False, weights_folder=None,
+             profile_folder=None):
     o = Options()
     o.fuse = int(fuse)
     o.dont_share_buffers = int(dont_share_buffers)
@@ -73,6 +75,7 @@ def _options(fuse=True, dont_share_buffers=False, max_entry_count=0, profile=Fal
     o.profile = int(profile)
     o.weights_from_folder = int(weights_folder is not None)
     o.weights_folder = weights_folder.encode() if weights_folder is not None else None
+    o.profile_folder = profile_folder.encode() if profile_folder is not None else None
     return o
 
 

@@ -105,7 +105,7 @@ extern "C"
 			for(uint32_t i = 0; i < output_count; ++i)
 				output_names.push_back(outputs[i].layer_name);
 			const bool profile = (options != nullptr) && (options->profile != 0);
-			forward_propagation::ptr fp = factory->create(schema, output_names, debug_state::ptr(new debug_state(false)), profile_state::ptr(new profile_state(profile)));
+			forward_propagation::ptr fp = factory->create(schema, output_names, debug_state::ptr(new debug_state(false)), profile_state::ptr(new profile_state(profile, (profile && (options->profile_folder != nullptr)) ? options->profile_folder : "")));
 
 			network_data data;
 			if ((options != nullptr) && options->weights_from_folder)

@@ -54,6 +54,7 @@ namespace nnforge
 			struct step_plan
 			{
 				forward_step info;
+				std::string key;                     // layer names joined with '+': the action name in reports
 				layer_tester_hip::ptr tester;        // single-layer steps
 				nnf_hip_chain_desc desc;             // fused steps (entry_count filled per packet)
 				std::vector<std::string> chunk_layers; // fused steps: layers whose weight chunks are concatenated into chunk_ptrs
@@ -105,12 +106,18 @@ namespace nnforge
 			std::vector<step_plan> plans;
 			std::vector<size_t> buffer_floats_per_entry;   // planned device buffers
 			std::map<std::string, int> value_to_buffer;    // data layers, step outputs
-			void * stream = nullptr;
+			void * stream = nullptr;          // kernels
+			void * upload_stream = nullptr;   // host -> device copies
+			void * download_stream = nullptr; // device -> host copies
 
 			~impl()
 			{
 				if (stream != nullptr)
 					nnf_hip_stream_destroy(stream);
+				if (upload_stream != nullptr)
+					nnf_hip_stream_destroy(upload_stream);
+				if (download_stream != nullptr)
+					nnf_hip_stream_destroy(download_stream);
 			}
 		};
 
@@ -283,6 +290,9 @@ namespace nnforge
 			// ---- steps ---------------------------------------------------------------------------
 			p->plans.clear();
 			steps.clear();
+			action_flops_per_entry.clear();
+			action_bytes_per_entry.clear();
+			action_layer_types.clear();
 			std::map<std::string, const pending_group *> group_by_name;
 			for(const std::pair<std::string, pending_group>& g : groups)
 				group_by_name[g.first] = &g.second;
@@ -359,6 +369,26 @@ namespace nnforge
 							push_op(op);
 					}
 				}
+				// report bookkeeping: name, layer types, flops (the reference's model) and memory traffic per entry
+				std::string types;
+				float step_flops = 0.0F;
+				for(const std::string& n : plan.info.layer_names)
+				{
+					plan.key += (plan.key.empty() ? "" : "+") + n;
+					layer::const_ptr l = this->schema->get_layer(n);
+					types += (types.empty() ? "" : "+") + l->get_type_name();
+					std::vector<layer_configuration_specific> inputs;
+					for(const std::string& input : l->input_layer_instance_names)
+						inputs.push_back(layer_config_map[input]);
+					step_flops += l->get_forward_flops_per_entry(inputs);
+				}
+				float step_bytes = static_cast<float>(config.get_neuron_count()) * sizeof(float);
+				for(const std::string& input : plan.info.input_names)
+					step_bytes += static_cast<float>(layer_config_map[input].get_neuron_count()) * sizeof(float);
+				action_flops_per_entry[plan.key] = step_flops;
+				action_bytes_per_entry[plan.key] = step_bytes;
+				action_layer_types[plan.key] = types;
+
 				p->plans.push_back(plan);
 				steps.push_back(plan.info);
 			}
@@ -464,6 +494,15 @@ namespace nnforge
 			}
 		}
 
+		// Packets of entries flow through three in-order queues with two I/O slots (the double buffering
+		// of nnforge/cuda/forward_propagation_cuda.cpp:84-112, 147-316):
+		//   host reads packet i into the pinned staging of slot i % 2   (needs: upload of packet i-2 done)
+		//   upload stream copies it to the slot's device input buffers   (needs: kernels of packet i-2 done)
+		//   kernel stream runs the launch plan                           (needs: upload i, download i-2 done)
+		//   download stream copies the slot's output buffers to staging  (needs: kernels i done)
+		//   host hands packet i-1 to the writer while packet i is in flight.
+		// Data and output layers have a device buffer per slot; everything in between is shared, which is
+		// safe because the kernel stream runs one packet after the other.
 		void forward_propagation_hip::actual_run(
 			structured_data_bunch_reader& reader,
 			structured_data_bunch_writer& writer,
@@ -475,7 +514,11 @@ namespace nnforge
 				throw neural_network_exception("This forward_propagation_hip was created for planning only (offline configuration): it cannot run");
 			hip_config->set_device();
 			if (p->stream == nullptr)
+			{
 				hip_safe_call(nnf_hip_stream_create(&p->stream));
+				hip_safe_call(nnf_hip_stream_create(&p->upload_stream));
+				hip_safe_call(nnf_hip_stream_create(&p->download_stream));
+			}
 			for(const layer::const_ptr& l : p->exec_layers)
 				if (!l->is_empty_data() && (p->weights.find(l->instance_name) == p->weights.end()))
 					throw neural_network_exception("No data found with layer name " + l->instance_name);
@@ -485,16 +528,35 @@ namespace nnforge
 			if (reader_entry_count > 0)
 				packet = std::min(packet, static_cast<unsigned int>(reader_entry_count));
 
-			// device buffers for one packet, pinned staging for inputs and outputs
-			std::vector<hip_linear_buffer_device::ptr> buffers;
-			for(size_t floats : p->buffer_floats_per_entry)
-				buffers.push_back(hip_linear_buffer_device::ptr(new hip_linear_buffer_device(floats * sizeof(float) * packet)));
-			std::map<std::string, std::unique_ptr<pinned_buffer> > staging;
+			constexpr int slot_count = 2;
+			const std::set<std::string> outputs(output_layer_names.begin(), output_layer_names.end());
+			// buffers[slot][b]: data and output layer buffers are per slot, the rest is shared
+			std::set<int> io_buffers;
 			for(const std::string& n : data_layer_names)
-				staging[n].reset(new pinned_buffer(static_cast<size_t>(layer_config_map[n].get_neuron_count()) * sizeof(float) * packet));
+				io_buffers.insert(p->value_to_buffer.at(n));
 			for(const std::string& n : output_layer_names)
-				if (staging.find(n) == staging.end())
-					staging[n].reset(new pinned_buffer(static_cast<size_t>(layer_config_map[n].get_neuron_count()) * sizeof(float) * packet));
+				io_buffers.insert(p->value_to_buffer.at(n));
+			std::vector<hip_linear_buffer_device::ptr> buffers[slot_count];
+			for(size_t b = 0; b < p->buffer_floats_per_entry.size(); ++b)
+			{
+				const size_t bytes = p->buffer_floats_per_entry[b] * sizeof(float) * packet;
+				buffers[0].push_back(hip_linear_buffer_device::ptr(new hip_linear_buffer_device(bytes)));
+				if (io_buffers.find(static_cast<int>(b)) != io_buffers.end())
+					buffers[1].push_back(hip_linear_buffer_device::ptr(new hip_linear_buffer_device(bytes)));
+				else
+					buffers[1].push_back(buffers[0].back());
+			}
+			std::map<std::string, std::unique_ptr<pinned_buffer> > staging[slot_count];
+			for(int s = 0; s < slot_count; ++s)
+			{
+				for(const std::string& n : data_layer_names)
+					staging[s][n].reset(new pinned_buffer(static_cast<size_t>(layer_config_map[n].get_neuron_count()) * sizeof(float) * packet));
+				for(const std::string& n : output_layer_names)
+					if (staging[s].find(n) == staging[s].end())
+						staging[s][n].reset(new pinned_buffer(static_cast<size_t>(layer_config_map[n].get_neuron_count()) * sizeof(float) * packet));
+			}
+			hip_event upload_done[slot_count], kernels_done[slot_count], download_done[slot_count];
+			bool slot_used[slot_count] = { false, false };
 
 			// weight pointers of the fused steps
 			std::vector<std::vector<const float *> > chunk_ptrs(p->plans.size());
@@ -504,98 +566,146 @@ namespace nnforge
 						chunk_ptrs[i].push_back(static_cast<const float *>(*b));
 
 			const bool profiling = profile->is_profile();
-			std::vector<std::unique_ptr<hip_event> > events;
+			std::vector<std::unique_ptr<hip_event> > step_events[slot_count];
 			if (profiling)
-				for(size_t i = 0; i <= p->plans.size(); ++i)
-					events.emplace_back(new hip_event());
+				for(int s = 0; s < slot_count; ++s)
+					for(size_t i = 0; i <= p->plans.size(); ++i)
+						step_events[s].emplace_back(new hip_event());
 
 			const std::vector<hip_linear_buffer_device::const_ptr> none;
-			unsigned int processed = 0;
+			unsigned int read_total = 0;
 			double idle = 0.0;
 			action_seconds.clear();
-			for(;;)
+
+			// what is in flight: at most the packet before the current one
+			struct in_flight
 			{
-				// read a packet
+				bool valid;
+				int slot;
+				unsigned int first_entry;
+				unsigned int entries;
+			} previous = { false, 0, 0, 0 };
+
+			auto finish = [&](const in_flight& f)
+			{
+				hip_safe_call(nnf_hip_event_synchronize(download_done[f.slot].ev));
+				if (profiling)
+				{
+					for(size_t i = 0; i < p->plans.size(); ++i)
+					{
+						float ms = 0.0F;
+						hip_safe_call(nnf_hip_event_elapsed_ms(&ms, step_events[f.slot][i]->ev, step_events[f.slot][i + 1]->ev));
+						action_seconds[p->plans[i].key] += ms * 1.0e-3F;
+					}
+				}
+				for(unsigned int e = 0; e < f.entries; ++e)
+				{
+					std::map<std::string, const float *> data_map;
+					for(const std::string& n : output_layer_names)
+						data_map[n] = static_cast<const float *>(staging[f.slot][n]->ptr) + static_cast<size_t>(e) * layer_config_map[n].get_neuron_count();
+					writer.write(f.first_entry + e, data_map);
+				}
+			};
+
+			for(unsigned int packet_id = 0; ; ++packet_id)
+			{
+				const int slot = static_cast<int>(packet_id % slot_count);
+				// the staging of this slot is free once its previous upload has finished; its output
+				// staging was consumed when that packet was handed to the writer
+				if (slot_used[slot])
+					hip_safe_call(nnf_hip_event_synchronize(upload_done[slot].ev));
+
 				const std::chrono::high_resolution_clock::time_point read_start = std::chrono::high_resolution_clock::now();
 				unsigned int entries_read = 0;
 				for(; entries_read < packet; ++entries_read)
 				{
 					std::map<std::string, float *> data_map;
 					for(const std::string& n : data_layer_names)
-						data_map[n] = static_cast<float *>(staging[n]->ptr) + static_cast<size_t>(entries_read) * layer_config_map[n].get_neuron_count();
-					if (!reader.read(processed + entries_read, data_map))
+						data_map[n] = static_cast<float *>(staging[slot][n]->ptr) + static_cast<size_t>(entries_read) * layer_config_map[n].get_neuron_count();
+					if (!reader.read(read_total + entries_read, data_map))
 						break;
 				}
 				idle += std::chrono::duration<double>(std::chrono::high_resolution_clock::now() - read_start).count();
-				if (entries_read == 0)
-					break;
 
-				for(const std::string& n : data_layer_names)
-					hip_safe_call(nnf_hip_memcpy_h2d(*buffers[p->value_to_buffer[n]], staging[n]->ptr,
-						static_cast<size_t>(layer_config_map[n].get_neuron_count()) * sizeof(float) * entries_read, p->stream));
-
-				for(size_t i = 0; i < p->plans.size(); ++i)
+				if (entries_read > 0)
 				{
-					step_plan& plan = p->plans[i];
-					if (profiling)
-						hip_safe_call(nnf_hip_event_record(events[i]->ev, p->stream));
-					std::vector<hip_linear_buffer_device::const_ptr> inputs;
-					for(int b : plan.input_buffers)
-						inputs.push_back(buffers[b]);
-					if (plan.info.fused)
+					// upload: the slot's input buffers may still be read by the kernels of packet i-2, or by
+					// its download when a layer worked in place on a data layer's buffer
+					if (slot_used[slot])
 					{
-						plan.desc.entry_count = entries_read;
-						std::vector<const float *> in_ptrs;
-						for(const hip_linear_buffer_device::const_ptr& b : inputs)
-							in_ptrs.push_back(static_cast<const float *>(*b));
-						hip_safe_call(nnf_hip_chain_forward(p->stream, &plan.desc, *buffers[plan.output_buffer], in_ptrs.data(),
-							chunk_ptrs[i].empty() ? nullptr : chunk_ptrs[i].data()));
+						hip_safe_call(nnf_hip_stream_wait_event(p->upload_stream, kernels_done[slot].ev));
+						hip_safe_call(nnf_hip_stream_wait_event(p->upload_stream, download_done[slot].ev));
 					}
-					else
-					{
-						const std::string& layer_name = plan.info.layer_names[0];
-						std::map<std::string, std::vector<hip_linear_buffer_device::const_ptr> >::const_iterator w = p->weights.find(layer_name);
-						plan.tester->enqueue_forward_propagation(p->stream, buffers[plan.output_buffer], none,
-							(w == p->weights.end()) ? none : w->second, none, inputs, none,
-							hip_linear_buffer_device::ptr(), hip_linear_buffer_device::ptr(), entries_read);
-					}
-				}
-				if (profiling)
-					hip_safe_call(nnf_hip_event_record(events[p->plans.size()]->ev, p->stream));
+					for(const std::string& n : data_layer_names)
+						hip_safe_call(nnf_hip_memcpy_h2d(*buffers[slot][p->value_to_buffer[n]], staging[slot][n]->ptr,
+							static_cast<size_t>(layer_config_map[n].get_neuron_count()) * sizeof(float) * entries_read, p->upload_stream));
+					hip_safe_call(nnf_hip_event_record(upload_done[slot].ev, p->upload_stream));
 
-				for(const std::string& n : output_layer_names)
-					hip_safe_call(nnf_hip_memcpy_d2h(staging[n]->ptr, *buffers[p->value_to_buffer.at(n)],
-						static_cast<size_t>(layer_config_map[n].get_neuron_count()) * sizeof(float) * entries_read, p->stream));
-				hip_safe_call(nnf_hip_stream_synchronize(p->stream));
-
-				if (profiling)
-				{
+					// kernels: need this packet's inputs and the slot's output buffers drained
+					hip_safe_call(nnf_hip_stream_wait_event(p->stream, upload_done[slot].ev));
+					if (slot_used[slot])
+						hip_safe_call(nnf_hip_stream_wait_event(p->stream, download_done[slot].ev));
 					for(size_t i = 0; i < p->plans.size(); ++i)
 					{
-						float ms = 0.0F;
-						hip_safe_call(nnf_hip_event_elapsed_ms(&ms, events[i]->ev, events[i + 1]->ev));
-						std::string key;
-						for(const std::string& n : p->plans[i].info.layer_names)
-							key += (key.empty() ? "" : "+") + n;
-						action_seconds[key] += ms * 1.0e-3F;
+						step_plan& plan = p->plans[i];
+						if (profiling)
+							hip_safe_call(nnf_hip_event_record(step_events[slot][i]->ev, p->stream));
+						std::vector<hip_linear_buffer_device::const_ptr> inputs;
+						for(int b : plan.input_buffers)
+							inputs.push_back(buffers[slot][b]);
+						if (plan.info.fused)
+						{
+							plan.desc.entry_count = entries_read;
+							std::vector<const float *> in_ptrs;
+							for(const hip_linear_buffer_device::const_ptr& b : inputs)
+								in_ptrs.push_back(static_cast<const float *>(*b));
+							hip_safe_call(nnf_hip_chain_forward(p->stream, &plan.desc, *buffers[slot][plan.output_buffer], in_ptrs.data(),
+								chunk_ptrs[i].empty() ? nullptr : chunk_ptrs[i].data()));
+						}
+						else
+						{
+							const std::string& layer_name = plan.info.layer_names[0];
+							std::map<std::string, std::vector<hip_linear_buffer_device::const_ptr> >::const_iterator w = p->weights.find(layer_name);
+							plan.tester->enqueue_forward_propagation(p->stream, buffers[slot][plan.output_buffer], none,
+								(w == p->weights.end()) ? none : w->second, none, inputs, none,
+								hip_linear_buffer_device::ptr(), hip_linear_buffer_device::ptr(), entries_read);
+						}
 					}
-				}
+					if (profiling)
+						hip_safe_call(nnf_hip_event_record(step_events[slot][p->plans.size()]->ev, p->stream));
+					hip_safe_call(nnf_hip_event_record(kernels_done[slot].ev, p->stream));
 
-				for(unsigned int e = 0; e < entries_read; ++e)
-				{
-					std::map<std::string, const float *> data_map;
+					// download
+					hip_safe_call(nnf_hip_stream_wait_event(p->download_stream, kernels_done[slot].ev));
 					for(const std::string& n : output_layer_names)
-						data_map[n] = static_cast<const float *>(staging[n]->ptr) + static_cast<size_t>(e) * layer_config_map[n].get_neuron_count();
-					writer.write(processed + e, data_map);
+						hip_safe_call(nnf_hip_memcpy_d2h(staging[slot][n]->ptr, *buffers[slot][p->value_to_buffer.at(n)],
+							static_cast<size_t>(layer_config_map[n].get_neuron_count()) * sizeof(float) * entries_read, p->download_stream));
+					hip_safe_call(nnf_hip_event_record(download_done[slot].ev, p->download_stream));
+					slot_used[slot] = true;
 				}
 
-				processed += entries_read;
+				// while this packet is in flight, hand the previous one to the writer
+				if (previous.valid)
+					finish(previous);
+				previous.valid = entries_read > 0;
+				previous.slot = slot;
+				previous.first_entry = read_total;
+				previous.entries = entries_read;
+				read_total += entries_read;
 				if (entries_read < packet)
 					break;
 			}
+			if (previous.valid)
+				finish(previous);
+			hip_safe_call(nnf_hip_stream_synchronize(p->stream));
 
-			entries_processed = processed;
+			entries_processed = read_total;
 			idle_seconds = static_cast<float>(idle);
+		}
+
+		float forward_propagation_hip::get_max_bytes_per_second() const
+		{
+			return 8.0e12F; // MI355X HBM3E peak
 		}
 
 		// ---- factories -------------------------------------------------------------------------

@@ -1,8 +1,10 @@
 #include "nnforge_hip/propagation.h"
 
+#include <algorithm>
 #include <chrono>
 #include <cstdio>
 #include <cstring>
+#include <fstream>
 
 namespace nnforge
 {
@@ -48,6 +50,58 @@ namespace nnforge
 		}
 		if (entry_id + 1 > entry_count)
 			entry_count = entry_id + 1;
+	}
+
+	std::string profile_state::get_path_to_unique_file(const char * file_prefix, const char * file_extension)
+	{
+		char buf[32];
+		std::snprintf(buf, sizeof(buf), "_%03u.", index++);
+		return profile_folder + "/" + file_prefix + buf + file_extension;
+	}
+
+	namespace
+	{
+		std::string percent(float v)
+		{
+			char buf[32];
+			std::snprintf(buf, sizeof(buf), "%.2f%%", static_cast<double>(v * 100.0F));
+			return buf;
+		}
+
+		// The per-action report of nnforge/profile_util.cpp:25-105 (tab separated, slowest first),
+		// with the bandwidth columns a memory-bound backend needs next to the GFLOPS ones.
+		void dump_action_performance(
+			const std::string& path,
+			unsigned int entry_count,
+			float total_seconds,
+			float max_flops,
+			float max_bytes_per_second,
+			const std::map<std::string, float>& seconds,
+			const std::map<std::string, float>& flops_per_entry,
+			const std::map<std::string, float>& bytes_per_entry,
+			const std::map<std::string, std::string>& types)
+		{
+			std::vector<std::pair<std::string, float> > entries(seconds.begin(), seconds.end());
+			std::sort(entries.begin(), entries.end(),
+				[] (const std::pair<std::string, float>& a, const std::pair<std::string, float>& b) { return a.second > b.second; });
+			std::ofstream out(path.c_str(), std::ios_base::out | std::ios_base::trunc);
+			if (!out)
+				throw neural_network_exception("Cannot open " + path + " for writing");
+			out << "Layer\tLayer type\tAction\tTime of total\tRelative to peak perf\tAbsolute time, seconds\tAbsolute perf, GFLOPS\tGB/s\tRelative to peak bandwidth" << std::endl;
+			for(const std::pair<std::string, float>& e : entries)
+			{
+				const auto lookup = [&e] (const std::map<std::string, float>& m) { std::map<std::string, float>::const_iterator it = m.find(e.first); return (it == m.end()) ? 0.0F : it->second; };
+				const float gflops = lookup(flops_per_entry) * static_cast<float>(entry_count) / e.second * 1.0e-9F;
+				const float gbps = lookup(bytes_per_entry) * static_cast<float>(entry_count) / e.second * 1.0e-9F;
+				std::map<std::string, std::string>::const_iterator type = types.find(e.first);
+				out << e.first << "\t" << ((type == types.end()) ? std::string() : type->second) << "\tforward";
+				out << "\t" << percent(e.second / total_seconds);
+				out << "\t" << ((max_flops > 0.0F) ? percent(gflops / (max_flops * 1.0e-9F)) : std::string("NA"));
+				out << "\t" << e.second << "\t" << gflops << "\t" << gbps;
+				out << "\t" << ((max_bytes_per_second > 0.0F) ? percent(gbps / (max_bytes_per_second * 1.0e-9F)) : std::string("NA"));
+				out << std::endl;
+			}
+		}
 	}
 
 	// ---- forward_propagation ---------------------------------------------------------------
@@ -141,7 +195,18 @@ namespace nnforge
 		const std::chrono::duration<float> sec = std::chrono::high_resolution_clock::now() - start;
 		res.total_seconds = sec.count();
 		res.idle_seconds = idle_seconds;
+
+		if (profile->is_profile() && !last_action_seconds.empty() && !profile->profile_folder.empty())
+			dump_action_performance(
+				profile->get_path_to_unique_file("forward_prop_perf_per_layer_action", "csv"),
+				res.entry_processed_count, res.total_seconds, get_max_flops(), get_max_bytes_per_second(),
+				last_action_seconds, action_flops_per_entry, action_bytes_per_entry, action_layer_types);
 		return res;
+	}
+
+	float forward_propagation::get_max_flops() const
+	{
+		return 0.0F; // unknown: the report then says NA (the reference throws "get_max_flops not implemented")
 	}
 
 	std::ostream& operator<< (std::ostream& out, const forward_propagation::stat& val)

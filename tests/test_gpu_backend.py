@@ -117,3 +117,46 @@ def test_cpp_application_uses_the_backend_like_a_reference_backend():
     assert any("[fused] main_bn+res+res_prelu <- conv_shortcut, conv_main" in l for l in lines), proc.stdout
     assert any(l.startswith("action main_bn+res+res_prelu:") for l in lines), proc.stdout
     assert any("13 entries" in l for l in lines), proc.stdout
+
+
+def test_many_packets_overlap_io_and_write_the_profile_report(tmp_path):
+    """37 entries in packets of 3 (13 packets, the last one short): uploads, kernels and downloads of
+    neighbouring packets overlap on two I/O slots, and every entry must still come out right. With a
+    profile folder the run leaves the per-action report of nnforge/profile_util.cpp:25-105."""
+    gen = T.rng(55, 0)
+    c, n = 8, 37
+    layers = S.classifier_tail(c)
+    weights = S.make_weights(layers, gen)
+    inputs = {"conv_main": T.normal(gen, (n, c, 7, 7), 4.0), "conv_shortcut": T.normal(gen, (n, c, 7, 7), 4.0)}
+    values = S.evaluate(layers, weights, inputs)
+    got, rep = run(layers, weights, inputs, ["prob", "pool", "res_relu"], values, max_entry_count=3, profile=True,
+                   profile_folder=str(tmp_path))
+    assert rep["entries"] == n
+    assert_bits(got["res_relu"], values["res_relu"], "block output")
+    assert_bits(got["pool"], values["pool"], "pool")
+    assert (np.abs(got["prob"] - values["prob"]) / values["prob"]).max() < 1e-5
+
+    lines = (tmp_path / "forward_prop_perf_per_layer_action_000.csv").read_text().splitlines()
+    header = lines[0].split("\t")
+    assert header[:3] == ["Layer", "Layer type", "Action"] and header[-2:] == ["GB/s", "Relative to peak bandwidth"]
+    rows = {r.split("\t")[0]: r.split("\t") for r in lines[1:]}
+    assert set(rows) == {"shortcut_bn+main_bn+res+res_relu", "pool", "prob"}
+    assert rows["shortcut_bn+main_bn+res+res_relu"][1] == "BatchNorm+BatchNorm+Add+ReLU"
+    assert all(r[2] == "forward" and len(r) == len(header) for r in rows.values())
+    times = [float(r.split("\t")[5]) for r in lines[1:]]
+    assert times == sorted(times, reverse=True) and times[-1] > 0
+    # the fused step moves 2 inputs + 1 output of c*49 floats per entry
+    fused = rows["shortcut_bn+main_bn+res+res_relu"]
+    assert abs(float(fused[7]) - 3 * c * 49 * 4 * n / float(fused[5]) * 1e-9) < 1e-3 * float(fused[7])
+
+
+def test_layer_in_place_on_a_data_layer_with_packets():
+    """The only layer writes where the data layer was uploaded: the next upload into that slot has to
+    wait for the download of the result."""
+    gen = T.rng(56, 0)
+    layers = [S.L("Data", "in"), S.L("TanH", "act", ["in"])]
+    n = 50
+    inputs = {"in": T.normal(gen, (n, 4, 10, 10))}
+    values = S.evaluate(layers, {}, inputs)
+    got, rep = run(layers, {}, inputs, ["act"], values, max_entry_count=7)
+    assert_bits(got["act"], values["act"], "tanh in place over 8 packets")
