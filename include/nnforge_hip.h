@@ -53,8 +53,11 @@ typedef enum nnf_hip_op_kind
 	                              (nnforge/plain/exponential_linear_layer_tester_plain.cpp:47-52)               */
 	NNF_HIP_OP_SIGMOID = 5,    /* "Sigmoid": y = 1 / (expf(-x) + 1)
 	                              (nnforge/plain/sigmoid_layer_tester_plain.cpp:47-53)                          */
-	NNF_HIP_OP_TANH = 6        /* "TanH": e = expf(x * (steepness*2)); y = (e - 1)/(e + 1) * scale
+	NNF_HIP_OP_TANH = 6,       /* "TanH": e = expf(x * (steepness*2)); y = (e - 1)/(e + 1) * scale
 	                              (nnforge/plain/hyperbolic_tangent_layer_tester_plain.cpp:48-58)               */
+	NNF_HIP_OP_ABSOLUTE = 7,   /* "Absolute": y = fabs(x) (nnforge/plain/absolute_layer_tester_plain.cpp:43-49)  */
+	NNF_HIP_OP_DROPOUT = 8     /* "Dropout" at inference: y = x (nnforge/plain/dropout_layer_tester_plain.cpp:45-48);
+	                              costs nothing inside a group                                                  */
 } nnf_hip_op_kind;
 
 /* One element-wise layer of a chain. */
@@ -122,6 +125,12 @@ NNF_HIP_API int nnf_hip_add_forward(void* stream, float* output, const float* co
 	/* nnforge/plain/add_layer_tester_plain.cpp:32-62; any input_count >= 1 (launched in groups of
 	   NNF_HIP_MAX_INPUTS, which keeps the reference's left-to-right summation order) */
 
+NNF_HIP_API int nnf_hip_absolute_forward(void* stream, float* output, const float* input, uint64_t elem_count);
+	/* nnforge/plain/absolute_layer_tester_plain.cpp:30-50 */
+NNF_HIP_API int nnf_hip_dropout_forward(void* stream, float* output, const float* input, uint64_t elem_count);
+	/* nnforge/plain/dropout_layer_tester_plain.cpp:33-49: the inference pass copies the input; with
+	   output == input nothing is launched */
+
 /* Softmax across feature maps at every (entry, spatial position):
  * nnforge/plain/softmax_layer_tester_plain.cpp:34-91 (max, expf(x - max), sum, multiply by 1/sum). */
 NNF_HIP_API int nnf_hip_softmax_forward(void* stream, float* output, const float* input,
@@ -136,6 +145,36 @@ NNF_HIP_API int nnf_hip_softmax_forward(void* stream, float* output, const float
 NNF_HIP_API int nnf_hip_average_subsampling_forward(void* stream, float* output, const float* input,
 	uint32_t entry_count, uint32_t feature_map_count, uint32_t input_width, uint32_t input_height,
 	uint32_t window_width, uint32_t window_height, float mult);
+
+/* Concatenation along feature maps: per entry the neurons of input 0, then of input 1, ...
+ * (nnforge/plain/concat_layer_tester_plain.cpp:33-59). input_neuron_counts[i] = feature maps * neurons
+ * per feature map of input i. */
+NNF_HIP_API int nnf_hip_concat_forward(void* stream, float* output, const float* const* inputs,
+	const uint32_t* input_neuron_counts, uint32_t input_count, uint32_t entry_count);
+
+/* Maxout: output feature map o = maximum over the input feature maps o, o + output_feature_map_count,
+ * o + 2*output_feature_map_count, ... (feature_map_subsampling_size of them), folded with
+ * std::max(new, current) from the first value on (nnforge/plain/maxout_layer_tester_plain.cpp:33-81). */
+NNF_HIP_API int nnf_hip_maxout_forward(void* stream, float* output, const float* input,
+	uint32_t entry_count, uint32_t output_feature_map_count, uint32_t neuron_count_per_feature_map,
+	uint32_t feature_map_subsampling_size);
+
+/* Max (or min) subsampling without tiling: windows of subsampling_sizes[d] every strides[d] elements
+ * (strides null: the window sizes) in up to NNF_HIP_MAX_SUBSAMPLING_DIMENSIONS spatial dimensions
+ * (x first), then over feature_map_subsampling_size neighbouring feature maps and
+ * entry_subsampling_size neighbouring entries; the fold starts at -1.0e37F (1.0e37F for min) and scans
+ * the window x fastest with std::max<float>(current, new)
+ * (nnforge/plain/max_subsampling_layer_tester_plain.cpp:175-290). Output size per dimension:
+ * (input + stride - window + (round_up ? window - 1 : 0)) / stride
+ * (nnforge/max_subsampling_layer.cpp:131-141); with round_ups[d] != 0 the part of a window beyond the
+ * input is skipped (nnforge/cuda/max_subsampling_layer_tester_cuda.cuh:97-116; the plain tester
+ * refuses round up). The input holds output_entry_count * entry_subsampling_size entries. The tiling
+ * variant of the layer (nnforge/plain/max_subsampling_layer_tester_plain.cpp:78-170) is not provided. */
+#define NNF_HIP_MAX_SUBSAMPLING_DIMENSIONS 4
+NNF_HIP_API int nnf_hip_max_subsampling_forward(void* stream, float* output, const float* input,
+	uint32_t output_entry_count, uint32_t input_feature_map_count, uint32_t dimension_count,
+	const uint32_t* input_sizes, const uint32_t* subsampling_sizes, const uint32_t* strides, const uint32_t* round_ups,
+	uint32_t feature_map_subsampling_size, uint32_t entry_subsampling_size, int32_t is_min);
 
 /* ---- runtime plumbing, so that host C++ above this ABI needs no HIP headers --------------------
  * Counterparts in the reference: cuda_linear_buffer_device (nnforge/cuda/cuda_linear_buffer_device.cpp:28-45),

@@ -19,6 +19,8 @@ OP_PRELU = 3
 OP_ELU = 4
 OP_SIGMOID = 5
 OP_TANH = 6
+OP_ABSOLUTE = 7
+OP_DROPOUT = 8
 
 E_INVAL = -1
 E_UNSUPPORTED = -2
@@ -61,6 +63,12 @@ SIGNATURES = {
     "nnf_hip_sigmoid_forward": [_VP, _VP, _VP, _U64],
     "nnf_hip_hyperbolic_tangent_forward": [_VP, _VP, _VP, _F, _F, _U64],
     "nnf_hip_add_forward": [_VP, _VP, _PP, _U32, _F, _U64],
+    "nnf_hip_absolute_forward": [_VP, _VP, _VP, _U64],
+    "nnf_hip_dropout_forward": [_VP, _VP, _VP, _U64],
+    "nnf_hip_concat_forward": [_VP, _VP, _PP, ctypes.POINTER(_U32), _U32, _U32],
+    "nnf_hip_maxout_forward": [_VP, _VP, _VP, _U32, _U32, _U32, _U32],
+    "nnf_hip_max_subsampling_forward": [_VP, _VP, _VP, _U32, _U32, _U32, ctypes.POINTER(_U32), ctypes.POINTER(_U32),
+                                        ctypes.POINTER(_U32), ctypes.POINTER(_U32), _U32, _U32, ctypes.c_int32],
     "nnf_hip_softmax_forward": [_VP, _VP, _VP, _U32, _U32, _U32],
     "nnf_hip_average_subsampling_forward": [_VP, _VP, _VP, _U32, _U32, _U32, _U32, _U32, _U32, _F],
     "nnf_hip_device_count": [ctypes.POINTER(ctypes.c_int)],

@@ -142,6 +142,41 @@ extern "C"
 		return flat_op(static_cast<hipStream_t>(stream), output, input, elem_count, NNF_HIP_OP_TANH, scale, steepness);
 	}
 
+	int nnf_hip_absolute_forward(void* stream, float* output, const float* input, uint64_t elem_count)
+	{
+		return flat_op(static_cast<hipStream_t>(stream), output, input, elem_count, NNF_HIP_OP_ABSOLUTE, 0.0f, 0.0f);
+	}
+
+	int nnf_hip_dropout_forward(void* stream, float* output, const float* input, uint64_t elem_count)
+	{
+		if ((output != nullptr) && (output == input))
+			return NNF_HIP_OK; // in place: nothing to move
+		return flat_op(static_cast<hipStream_t>(stream), output, input, elem_count, NNF_HIP_OP_DROPOUT, 0.0f, 0.0f);
+	}
+
+	int nnf_hip_concat_forward(void* stream, float* output, const float* const* inputs,
+		const uint32_t* input_neuron_counts, uint32_t input_count, uint32_t entry_count)
+	{
+		return concat_forward(static_cast<hipStream_t>(stream), output, inputs, input_neuron_counts, input_count, entry_count);
+	}
+
+	int nnf_hip_maxout_forward(void* stream, float* output, const float* input,
+		uint32_t entry_count, uint32_t output_feature_map_count, uint32_t neuron_count_per_feature_map,
+		uint32_t feature_map_subsampling_size)
+	{
+		return maxout_forward(static_cast<hipStream_t>(stream), output, input, entry_count, output_feature_map_count,
+			neuron_count_per_feature_map, feature_map_subsampling_size);
+	}
+
+	int nnf_hip_max_subsampling_forward(void* stream, float* output, const float* input,
+		uint32_t output_entry_count, uint32_t input_feature_map_count, uint32_t dimension_count,
+		const uint32_t* input_sizes, const uint32_t* subsampling_sizes, const uint32_t* strides, const uint32_t* round_ups,
+		uint32_t feature_map_subsampling_size, uint32_t entry_subsampling_size, int32_t is_min)
+	{
+		return max_subsampling_forward(static_cast<hipStream_t>(stream), output, input, output_entry_count, input_feature_map_count,
+			dimension_count, input_sizes, subsampling_sizes, strides, round_ups, feature_map_subsampling_size, entry_subsampling_size, is_min);
+	}
+
 	int nnf_hip_add_forward(void* stream, float* output, const float* const* inputs, uint32_t input_count, float alpha, uint64_t elem_count)
 	{
 		if ((inputs == nullptr) || (input_count == 0) || (output == nullptr))

@@ -167,7 +167,16 @@ namespace nnf
 				for(int i = 0; i < U * 4; i += EXP_BATCH)
 					nnf_hyperbolic_tangent<EXP_BATCH>(reinterpret_cast<float (&)[EXP_BATCH]>(v[i / 4][i % 4]), op.f1, op.f0, exp_ctx); // f1 holds steepness * 2
 				break;
-			default:
+			case NNF_HIP_OP_ABSOLUTE:
+				#pragma unroll
+				for(int k = 0; k < U; ++k)
+				{
+					#pragma unroll
+					for(int e = 0; e < 4; ++e)
+						v[k][e] = nnf_absolute(v[k][e]);
+				}
+				break;
+			default: // NNF_HIP_OP_DROPOUT: the value passes through
 				break;
 			}
 		}
@@ -526,6 +535,8 @@ namespace nnf
 				}
 				break;
 			case NNF_HIP_OP_RELU:
+			case NNF_HIP_OP_ABSOLUTE:
+			case NNF_HIP_OP_DROPOUT:
 				break;
 			case NNF_HIP_OP_TANH:
 				// nnforge/plain/hyperbolic_tangent_layer_tester_plain.cpp:49: steepness * 2.0F, rounded once on the host

@@ -72,5 +72,14 @@ namespace nnf
 	int average_subsampling_forward(hipStream_t stream, float* output, const float* input,
 		uint32_t entry_count, uint32_t feature_map_count, uint32_t input_width, uint32_t input_height,
 		uint32_t window_width, uint32_t window_height, float mult);
+	int concat_forward(hipStream_t stream, float* output, const float* const* inputs, const uint32_t* input_neuron_counts,
+		uint32_t input_count, uint32_t entry_count);
+	int maxout_forward(hipStream_t stream, float* output, const float* input,
+		uint32_t entry_count, uint32_t output_feature_map_count, uint32_t neuron_count_per_feature_map,
+		uint32_t feature_map_subsampling_size);
+	int max_subsampling_forward(hipStream_t stream, float* output, const float* input,
+		uint32_t output_entry_count, uint32_t input_feature_map_count, uint32_t dimension_count,
+		const uint32_t* input_sizes, const uint32_t* subsampling_sizes, const uint32_t* strides, const uint32_t* round_ups,
+		uint32_t feature_map_subsampling_size, uint32_t entry_subsampling_size, int32_t is_min);
 	int copy_kernel(hipStream_t stream, void* dst, const void* src, size_t bytes);
 }

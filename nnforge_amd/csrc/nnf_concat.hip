@@ -1,0 +1,150 @@
+// Concatenation along feature maps (nnforge/plain/concat_layer_tester_plain.cpp:45-58): per entry
+// the neurons of input 0, then of input 1, ... A pure copy, so the only concern is moving every
+// byte once with wide, coalesced accesses.
+#include "nnf_common.h"
+
+#include <algorithm>
+
+namespace nnf
+{
+	namespace
+	{
+		constexpr int concat_block_size = 256;
+		constexpr int concat_unroll = 4;            // accesses per lane
+		constexpr uint32_t concat_max_inputs = 8;   // per launch
+
+		struct concat_args
+		{
+			float* out;
+			const float* in[concat_max_inputs];
+			uint32_t length[concat_max_inputs];      // neurons per entry of each input
+			uint32_t offset[concat_max_inputs];      // where the input starts inside an output entry
+			uint32_t first_block[concat_max_inputs + 1]; // blockIdx.x range of each input
+			uint32_t input_count;
+			uint32_t output_length;                  // neurons per output entry
+			uint32_t entry_count;
+		};
+
+		// VEC: floats per access; 4 when every length is a multiple of 4 (then every offset is as well)
+		template<int VEC>
+		__global__ void __launch_bounds__(concat_block_size) concat_kernel(const concat_args a)
+		{
+			typedef float vec_t __attribute__((ext_vector_type(VEC)));
+			uint32_t i = 0;
+			while ((i + 1 < a.input_count) && (blockIdx.x >= a.first_block[i + 1]))
+				++i;
+			const uint32_t tile = (blockIdx.x - a.first_block[i]) * (concat_block_size * concat_unroll * VEC);
+			const uint32_t length = a.length[i];
+			for(uint32_t entry = blockIdx.y; entry < a.entry_count; entry += gridDim.y)
+			{
+				const float* src = a.in[i] + static_cast<size_t>(entry) * length;
+				float* dst = a.out + static_cast<size_t>(entry) * a.output_length + a.offset[i];
+				vec_t v[concat_unroll];
+				#pragma unroll
+				for(int k = 0; k < concat_unroll; ++k)
+				{
+					const uint32_t r = tile + (k * concat_block_size + threadIdx.x) * VEC;
+					if (r < length)
+						v[k] = __builtin_nontemporal_load(reinterpret_cast<const vec_t*>(src + r));
+				}
+				#pragma unroll
+				for(int k = 0; k < concat_unroll; ++k)
+				{
+					const uint32_t r = tile + (k * concat_block_size + threadIdx.x) * VEC;
+					if (r < length)
+						__builtin_nontemporal_store(v[k], reinterpret_cast<vec_t*>(dst + r));
+				}
+			}
+		}
+
+		template<>
+		__global__ void __launch_bounds__(concat_block_size) concat_kernel<1>(const concat_args a)
+		{
+			uint32_t i = 0;
+			while ((i + 1 < a.input_count) && (blockIdx.x >= a.first_block[i + 1]))
+				++i;
+			const uint32_t tile = (blockIdx.x - a.first_block[i]) * (concat_block_size * concat_unroll);
+			const uint32_t length = a.length[i];
+			for(uint32_t entry = blockIdx.y; entry < a.entry_count; entry += gridDim.y)
+			{
+				const float* src = a.in[i] + static_cast<size_t>(entry) * length;
+				float* dst = a.out + static_cast<size_t>(entry) * a.output_length + a.offset[i];
+				#pragma unroll
+				for(int k = 0; k < concat_unroll; ++k)
+				{
+					const uint32_t r = tile + k * concat_block_size + threadIdx.x;
+					if (r < length)
+						dst[r] = src[r];
+				}
+			}
+		}
+	}
+
+	int concat_forward(hipStream_t stream, float* output, const float* const* inputs, const uint32_t* input_neuron_counts,
+		uint32_t input_count, uint32_t entry_count)
+	{
+		if ((output == nullptr) || (inputs == nullptr) || (input_neuron_counts == nullptr) || (input_count == 0))
+			return NNF_HIP_EINVAL;
+		if (!is_aligned16(output))
+			return NNF_HIP_EALIGN;
+		uint64_t output_length = 0;
+		bool vector = true;
+		for(uint32_t i = 0; i < input_count; ++i)
+		{
+			if (input_neuron_counts[i] != 0) // an input without neurons is never read
+			{
+				if (inputs[i] == nullptr)
+					return NNF_HIP_EINVAL;
+				if (!is_aligned16(inputs[i]))
+					return NNF_HIP_EALIGN;
+			}
+			output_length += input_neuron_counts[i];
+			vector = vector && ((input_neuron_counts[i] % 4) == 0);
+		}
+		const uint64_t output_total = output_length * entry_count;
+		if (output_total == 0)
+			return NNF_HIP_OK;
+		if (output_total > 0xFFFF0000ull)
+			return NNF_HIP_ETOOBIG;
+		for(uint32_t i = 0; i < input_count; ++i)
+		{
+			const uintptr_t a = reinterpret_cast<uintptr_t>(output), b = reinterpret_cast<uintptr_t>(inputs[i]);
+			const uint64_t b_bytes = static_cast<uint64_t>(input_neuron_counts[i]) * entry_count * sizeof(float);
+			if ((b_bytes != 0) && (a < b + b_bytes) && (b < a + output_total * sizeof(float)))
+				return NNF_HIP_EOVERLAP;
+		}
+
+		const uint32_t per_block = concat_block_size * concat_unroll * (vector ? 4 : 1);
+		uint32_t offset = 0;
+		for(uint32_t first = 0; first < input_count; first += concat_max_inputs)
+		{
+			concat_args a = {};
+			a.out = output;
+			a.input_count = std::min(concat_max_inputs, input_count - first);
+			a.output_length = static_cast<uint32_t>(output_length);
+			a.entry_count = entry_count;
+			uint32_t blocks = 0;
+			for(uint32_t i = 0; i < a.input_count; ++i)
+			{
+				a.in[i] = inputs[first + i];
+				a.length[i] = input_neuron_counts[first + i];
+				a.offset[i] = offset;
+				a.first_block[i] = blocks;
+				offset += a.length[i];
+				blocks += (a.length[i] + per_block - 1) / per_block;
+			}
+			a.first_block[a.input_count] = blocks;
+			if (blocks == 0)
+				continue;
+			const dim3 grid(blocks, std::min(entry_count, 65535u));
+			if (vector)
+				hipLaunchKernelGGL(concat_kernel<4>, grid, dim3(concat_block_size), 0, stream, a);
+			else
+				hipLaunchKernelGGL(concat_kernel<1>, grid, dim3(concat_block_size), 0, stream, a);
+			const int status = launch_status();
+			if (status != NNF_HIP_OK)
+				return status;
+		}
+		return NNF_HIP_OK;
+	}
+}

@@ -165,6 +165,12 @@ namespace nnf
 		return x >= 0.0f ? x : x * negative_slope;
 	}
 
+	// nnforge/plain/absolute_layer_tester_plain.cpp:49 (fabs: clears the sign bit, of NaN as well)
+	NNF_HD float nnf_absolute(float x)
+	{
+		return __builtin_fabsf(x);
+	}
+
 	// nnforge/plain/parametric_rectified_linear_layer_tester_plain.cpp:66-67
 	NNF_HD float nnf_parametric_rectified_linear(float x, float a)
 	{

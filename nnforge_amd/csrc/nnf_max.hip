@@ -1,0 +1,422 @@
+// Maximum / minimum over windows (max subsampling) and over groups of feature maps (maxout).
+//
+// Both reference testers fold the values of a window in a fixed order with std::max / std::min,
+// whose result for equal values (+0.0 and -0.0) and for NaN depends on the argument order, and
+// max subsampling starts the fold at -1.0e37F / 1.0e37F. The kernels keep the order, the argument
+// order and the start value, so results equal the reference's bit for bit:
+//   nnforge/plain/max_subsampling_layer_tester_plain.cpp:175-290  std::max<float>(current, new), x fastest
+//   nnforge/plain/maxout_layer_tester_plain.cpp:56-80             std::max(new, current), starts at the first value
+#include "nnf_common.h"
+
+#include <algorithm>
+
+namespace nnf
+{
+	namespace
+	{
+		constexpr int max_block_size = 256;
+		constexpr uint32_t max_dims = NNF_HIP_MAX_SUBSAMPLING_DIMENSIONS;
+
+		// std::max<float>(current, new_val) / std::min<float>(current, new_val)
+		template<bool IS_MIN>
+		__device__ __forceinline__ float fold(float current, float new_val)
+		{
+			if (IS_MIN)
+				return (new_val < current) ? new_val : current;
+			return (current < new_val) ? new_val : current;
+		}
+
+		// n / divisor with magic = ceil(2^32 / divisor), exact while n * divisor < 2^32
+		__device__ __forceinline__ uint32_t fast_divide(uint32_t n, uint32_t divisor, uint32_t magic)
+		{
+			return (divisor == 1) ? n : __umulhi(n, magic);
+		}
+
+		template<bool IS_MIN>
+		__device__ __forceinline__ float fold_start()
+		{
+			return IS_MIN ? 1.0e37f : -1.0e37f;
+		}
+
+		// ---- 2-D windows, staged through LDS ------------------------------------------------------
+		//
+		// A workgroup produces a contiguous run of outputs: either `rows` output rows of one plane
+		// (large planes) or all rows of `planes` consecutive planes (small planes). The input it needs
+		// is one contiguous range of memory in both cases; it is copied to LDS with aligned float4
+		// loads (each input byte is fetched once per workgroup; only the window_height - stride_y rows
+		// shared by neighbouring row bands are fetched twice), then every lane scans its windows in LDS.
+		struct window2d_args
+		{
+			float* out;
+			const float* in;
+			uint32_t total_in;        // floats in the input tensor
+			uint32_t plane_count;     // entries * feature maps
+			uint32_t in_w, in_h, out_w, out_h;
+			uint32_t win_w, win_h, stride_x, stride_y;
+			uint32_t planes;          // planes per workgroup (1 when a plane is split into bands)
+			uint32_t rows;            // output rows per workgroup (out_h when planes > 1 or the plane is not split)
+			uint32_t bands;           // ceil(out_h / rows)
+			uint32_t out_w_magic;     // ceil(2^32 / out_w)
+			uint32_t band_magic;      // ceil(2^32 / (rows * out_w)): outputs per plane inside a workgroup
+		};
+
+		template<bool IS_MIN, int WIN_W, int WIN_H> // 0: read the size from the arguments
+		__global__ void __launch_bounds__(max_block_size) max_window2d_kernel(const window2d_args a)
+		{
+			extern __shared__ __align__(16) float lds_in[];
+
+			const uint32_t group = blockIdx.x / a.bands;
+			const uint32_t band = blockIdx.x - group * a.bands;
+			const uint32_t first_plane = group * a.planes;
+			const uint32_t planes_here = min(a.planes, a.plane_count - first_plane);
+			const uint32_t first_row = band * a.rows;
+			const uint32_t rows_here = min(a.rows, a.out_h - first_row);
+			const uint32_t in_plane = a.in_w * a.in_h;
+
+			// input rows [in_row0, in_row1) of planes [first_plane, first_plane + planes_here)
+			const uint32_t in_row0 = first_row * a.stride_y;
+			uint32_t in_row1 = a.in_h;
+			if (planes_here == 1)
+				in_row1 = min(a.in_h, (first_row + rows_here - 1) * a.stride_y + ((WIN_H > 0) ? WIN_H : a.win_h));
+			const uint32_t g0 = first_plane * in_plane + in_row0 * a.in_w;
+			const uint32_t g1 = (first_plane + planes_here - 1) * in_plane + in_row1 * a.in_w;
+			const uint32_t g0_aligned = g0 & ~3u;
+			const uint32_t shift = g0 - g0_aligned;
+			const uint32_t vectors = (g1 - g0_aligned + 3) / 4;
+			for(uint32_t i = threadIdx.x; i < vectors; i += max_block_size)
+			{
+				const uint32_t g = g0_aligned + i * 4;
+				if (g + 4 <= a.total_in)
+				{
+					const floatx4 t = load_stream(reinterpret_cast<const floatx4*>(a.in + g));
+					*reinterpret_cast<floatx4*>(lds_in + i * 4) = t;
+				}
+				else
+				{
+					for(uint32_t e = 0; (e < 4) && (g + e < a.total_in); ++e)
+						lds_in[i * 4 + e] = a.in[g + e];
+				}
+			}
+			__syncthreads();
+
+			const uint32_t win_w = (WIN_W > 0) ? WIN_W : a.win_w;
+			const uint32_t win_h = (WIN_H > 0) ? WIN_H : a.win_h;
+			const uint32_t outputs_per_plane = rows_here * a.out_w;
+			const uint32_t outputs_here = planes_here * outputs_per_plane;
+			float* dst = a.out + (first_plane * a.out_h + first_row) * a.out_w;
+			for(uint32_t o = threadIdx.x; o < outputs_here; o += max_block_size)
+			{
+				// rows_here differs from a.rows only in the last band, where planes_here == 1 and p is 0 anyway
+				const uint32_t p = (planes_here > 1) ? fast_divide(o, outputs_per_plane, a.band_magic) : 0u;
+				const uint32_t r = o - p * outputs_per_plane;
+				const uint32_t oy = fast_divide(r, a.out_w, a.out_w_magic);
+				const uint32_t ox = r - oy * a.out_w;
+				const uint32_t x0 = ox * a.stride_x;
+				const uint32_t y0 = (first_row + oy) * a.stride_y;
+				// windows that reach beyond the input (round up) are cut off there
+				const uint32_t fit_w = min(win_w, a.in_w - x0);
+				const uint32_t fit_h = min(win_h, a.in_h - y0);
+				const float* src = lds_in + shift + p * in_plane + (y0 - in_row0) * a.in_w + x0;
+				float current = fold_start<IS_MIN>();
+				if ((WIN_W > 0) && (WIN_H > 0))
+				{
+					#pragma unroll
+					for(int y = 0; y < WIN_H; ++y)
+					{
+						#pragma unroll
+						for(int x = 0; x < WIN_W; ++x)
+						{
+							if ((static_cast<uint32_t>(y) < fit_h) && (static_cast<uint32_t>(x) < fit_w))
+								current = fold<IS_MIN>(current, src[y * a.in_w + x]);
+						}
+					}
+				}
+				else
+				{
+					for(uint32_t y = 0; y < fit_h; ++y)
+						for(uint32_t x = 0; x < fit_w; ++x)
+							current = fold<IS_MIN>(current, src[y * a.in_w + x]);
+				}
+				dst[o] = current;
+			}
+		}
+
+		// ---- any window the layer allows: one lane per output, values read from memory ------------
+		struct window_nd_args
+		{
+			float* out;
+			const float* in;
+			uint32_t output_count;
+			uint32_t in_size[max_dims], out_size[max_dims], window[max_dims], stride[max_dims]; // unused dimensions are 1
+			uint32_t in_fm, out_fm, fm_window, entry_window, in_plane;
+		};
+
+		template<bool IS_MIN>
+		__global__ void __launch_bounds__(max_block_size) max_window_nd_kernel(const window_nd_args a)
+		{
+			const uint32_t o = blockIdx.x * max_block_size + threadIdx.x;
+			if (o >= a.output_count)
+				return;
+			uint32_t rem = o;
+			uint32_t start[max_dims], fit[max_dims];
+			#pragma unroll
+			for(uint32_t d = 0; d < max_dims; ++d)
+			{
+				const uint32_t q = rem / a.out_size[d];
+				start[d] = (rem - q * a.out_size[d]) * a.stride[d];
+				fit[d] = min(a.window[d], a.in_size[d] - start[d]);
+				rem = q;
+			}
+			const uint32_t out_entry = rem / a.out_fm;
+			const uint32_t out_fm_id = rem - out_entry * a.out_fm;
+			const size_t base = (static_cast<size_t>(out_entry) * a.entry_window * a.in_fm + static_cast<size_t>(out_fm_id) * a.fm_window) * a.in_plane;
+
+			float current = fold_start<IS_MIN>();
+			// scan order of the reference: x fastest, then y, z, w, feature map, entry
+			for(uint32_t en = 0; en < a.entry_window; ++en)
+			{
+				for(uint32_t fm = 0; fm < a.fm_window; ++fm)
+				{
+					const float* plane = a.in + base + (static_cast<size_t>(en) * a.in_fm + fm) * a.in_plane;
+					for(uint32_t w = 0; w < fit[3]; ++w)
+					{
+						for(uint32_t z = 0; z < fit[2]; ++z)
+						{
+							for(uint32_t y = 0; y < fit[1]; ++y)
+							{
+								const float* row = plane + ((static_cast<size_t>(start[3] + w) * a.in_size[2] + start[2] + z) * a.in_size[1] + start[1] + y) * a.in_size[0] + start[0];
+								for(uint32_t x = 0; x < fit[0]; ++x)
+									current = fold<IS_MIN>(current, row[x]);
+							}
+						}
+					}
+				}
+			}
+			a.out[o] = current;
+		}
+
+		// ---- maxout ------------------------------------------------------------------------------
+		// Per entry the output is `group` floats and output j folds the inputs j, j + group, j + 2*group, ...
+		// std::max(new_val, current) = (new_val < current) ? current : new_val
+		__device__ __forceinline__ float maxout_fold(float current, float new_val)
+		{
+			return (new_val < current) ? current : new_val;
+		}
+
+		// group is a multiple of 4: a lane folds four neighbouring outputs
+		__global__ void __launch_bounds__(max_block_size) maxout_vec4_kernel(float* out, const float* in, uint32_t entry_count, uint32_t group, uint32_t fold_count)
+		{
+			const uint32_t j = (blockIdx.x * max_block_size + threadIdx.x) * 4;
+			if (j >= group)
+				return;
+			for(uint32_t entry = blockIdx.y; entry < entry_count; entry += gridDim.y)
+			{
+				const float* src = in + static_cast<size_t>(entry) * group * fold_count + j;
+				floatx4 current = load_stream(reinterpret_cast<const floatx4*>(src));
+				for(uint32_t i = 1; i < fold_count; ++i)
+				{
+					const floatx4 new_val = load_stream(reinterpret_cast<const floatx4*>(src + static_cast<size_t>(i) * group));
+					current.x = maxout_fold(current.x, new_val.x);
+					current.y = maxout_fold(current.y, new_val.y);
+					current.z = maxout_fold(current.z, new_val.z);
+					current.w = maxout_fold(current.w, new_val.w);
+				}
+				store_stream(reinterpret_cast<floatx4*>(out + static_cast<size_t>(entry) * group + j), current);
+			}
+		}
+
+		__global__ void __launch_bounds__(max_block_size) maxout_scalar_kernel(float* out, const float* in, uint32_t entry_count, uint32_t group, uint32_t fold_count)
+		{
+			const uint32_t j = blockIdx.x * max_block_size + threadIdx.x;
+			if (j >= group)
+				return;
+			for(uint32_t entry = blockIdx.y; entry < entry_count; entry += gridDim.y)
+			{
+				const float* src = in + static_cast<size_t>(entry) * group * fold_count + j;
+				float current = src[0];
+				for(uint32_t i = 1; i < fold_count; ++i)
+					current = maxout_fold(current, src[static_cast<size_t>(i) * group]);
+				out[static_cast<size_t>(entry) * group + j] = current;
+			}
+		}
+
+		bool overlap(const void* a, uint64_t a_bytes, const void* b, uint64_t b_bytes)
+		{
+			const uintptr_t pa = reinterpret_cast<uintptr_t>(a), pb = reinterpret_cast<uintptr_t>(b);
+			return (pa < pb + b_bytes) && (pb < pa + a_bytes);
+		}
+
+		uint32_t magic_of(uint32_t divisor)
+		{
+			return (divisor >= 2) ? static_cast<uint32_t>(((1ull << 32) + divisor - 1) / divisor) : 0u; // fast_divide does not use it for 1
+		}
+
+		template<bool IS_MIN>
+		void launch_window2d(hipStream_t stream, const window2d_args& a, uint32_t grid, size_t lds_bytes)
+		{
+			if ((a.win_w == 3) && (a.win_h == 3))
+				hipLaunchKernelGGL((max_window2d_kernel<IS_MIN, 3, 3>), dim3(grid), dim3(max_block_size), lds_bytes, stream, a);
+			else if ((a.win_w == 2) && (a.win_h == 2))
+				hipLaunchKernelGGL((max_window2d_kernel<IS_MIN, 2, 2>), dim3(grid), dim3(max_block_size), lds_bytes, stream, a);
+			else
+				hipLaunchKernelGGL((max_window2d_kernel<IS_MIN, 0, 0>), dim3(grid), dim3(max_block_size), lds_bytes, stream, a);
+		}
+	}
+
+	int max_subsampling_forward(hipStream_t stream, float* output, const float* input,
+		uint32_t output_entry_count, uint32_t input_feature_map_count, uint32_t dimension_count,
+		const uint32_t* input_sizes, const uint32_t* subsampling_sizes, const uint32_t* strides, const uint32_t* round_ups,
+		uint32_t feature_map_subsampling_size, uint32_t entry_subsampling_size, int32_t is_min)
+	{
+		if ((output == nullptr) || (input == nullptr) || (input_sizes == nullptr) || (subsampling_sizes == nullptr))
+			return NNF_HIP_EINVAL;
+		if ((dimension_count < 1) || (dimension_count > max_dims))
+			return NNF_HIP_EUNSUPPORTED; // the reference's testers stop at 4 dimensions as well
+		if ((input_feature_map_count == 0) || (feature_map_subsampling_size == 0) || (entry_subsampling_size == 0))
+			return NNF_HIP_EINVAL;
+		if (!is_aligned16(output) || !is_aligned16(input))
+			return NNF_HIP_EALIGN;
+
+		window_nd_args nd = {};
+		uint64_t in_plane = 1, out_plane = 1;
+		bool round_up_anywhere = false;
+		for(uint32_t d = 0; d < max_dims; ++d)
+		{
+			nd.in_size[d] = nd.out_size[d] = nd.window[d] = nd.stride[d] = 1;
+			if (d >= dimension_count)
+				continue;
+			const uint32_t size = input_sizes[d], window = subsampling_sizes[d];
+			const uint32_t stride = (strides != nullptr) ? strides[d] : window;
+			const bool round_up = (round_ups != nullptr) && (round_ups[d] != 0);
+			if ((size == 0) || (window == 0) || (stride == 0))
+				return NNF_HIP_EINVAL;
+			// nnforge/max_subsampling_layer.cpp:135-139
+			const int64_t out_size = (static_cast<int64_t>(size) + stride - window + (round_up ? window - 1 : 0)) / stride;
+			if (out_size <= 0)
+				return NNF_HIP_EINVAL; // "produces 0 output size"
+			nd.in_size[d] = size;
+			nd.out_size[d] = static_cast<uint32_t>(out_size);
+			nd.window[d] = window;
+			nd.stride[d] = stride;
+			in_plane *= size;
+			out_plane *= static_cast<uint64_t>(out_size);
+			round_up_anywhere = round_up_anywhere || round_up;
+		}
+		const uint32_t out_fm = input_feature_map_count / feature_map_subsampling_size;
+		if (out_fm == 0)
+			return NNF_HIP_EINVAL;
+		const uint64_t input_total = static_cast<uint64_t>(output_entry_count) * entry_subsampling_size * input_feature_map_count * in_plane;
+		const uint64_t output_total = static_cast<uint64_t>(output_entry_count) * out_fm * out_plane;
+		if (output_total == 0)
+			return NNF_HIP_OK;
+		if ((input_total > 0xFFFF0000ull) || (output_total > 0xFFFF0000ull))
+			return NNF_HIP_ETOOBIG;
+		if (overlap(output, output_total * sizeof(float), input, input_total * sizeof(float)))
+			return NNF_HIP_EOVERLAP;
+
+		// 2-D (or 1-D) windows within a feature map: stage through LDS
+		constexpr uint32_t lds_floats_wanted = 8 * 1024; // 32 KB: four workgroups per compute unit
+		constexpr uint32_t lds_floats_max = 15 * 1024;
+		const bool within_plane = (feature_map_subsampling_size == 1) && (entry_subsampling_size == 1) && (dimension_count <= 2);
+		if (within_plane && (nd.out_size[0] * nd.out_size[1] < (1u << 16)))
+		{
+			window2d_args a = {};
+			a.out = output;
+			a.in = input;
+			a.total_in = static_cast<uint32_t>(input_total);
+			a.plane_count = output_entry_count * input_feature_map_count;
+			a.in_w = nd.in_size[0]; a.in_h = nd.in_size[1];
+			a.out_w = nd.out_size[0]; a.out_h = nd.out_size[1];
+			a.win_w = nd.window[0]; a.win_h = nd.window[1];
+			a.stride_x = nd.stride[0]; a.stride_y = nd.stride[1];
+			const uint32_t plane = a.in_w * a.in_h;
+			bool fits = true;
+			if (plane <= lds_floats_wanted)
+			{
+				// whole planes; enough of them for a few outputs per lane, few enough to keep the grid wide
+				a.planes = std::max(1u, std::min(lds_floats_wanted / plane, (4u * max_block_size + a.out_w * a.out_h - 1) / (a.out_w * a.out_h)));
+				a.rows = a.out_h;
+			}
+			else
+			{
+				a.planes = 1;
+				// rows per band: input rows needed = (rows - 1) * stride_y + win_h
+				const uint32_t rows_in = lds_floats_wanted / a.in_w;
+				a.rows = (rows_in >= a.win_h) ? (rows_in - a.win_h) / a.stride_y + 1 : 0;
+				if (a.rows == 0)
+				{
+					a.rows = 1;
+					fits = static_cast<uint64_t>(a.win_h) * a.in_w + 4 <= lds_floats_max;
+				}
+				a.rows = std::min(a.rows, a.out_h);
+				// bands of equal height
+				const uint32_t bands = (a.out_h + a.rows - 1) / a.rows;
+				a.rows = (a.out_h + bands - 1) / bands;
+			}
+			if (fits)
+			{
+				a.bands = (a.out_h + a.rows - 1) / a.rows;
+				a.out_w_magic = magic_of(a.out_w);
+				a.band_magic = magic_of(a.rows * a.out_w);
+				const uint32_t rows_in = (a.planes > 1 || a.bands == 1) ? a.in_h : std::min(a.in_h, (a.rows - 1) * a.stride_y + a.win_h);
+				const size_t lds_bytes = (static_cast<size_t>(a.planes - 1) * plane + static_cast<size_t>(rows_in) * a.in_w + 8) * sizeof(float);
+				const uint32_t grid = ((a.plane_count + a.planes - 1) / a.planes) * a.bands;
+				if (is_min)
+					launch_window2d<true>(stream, a, grid, lds_bytes);
+				else
+					launch_window2d<false>(stream, a, grid, lds_bytes);
+				return launch_status();
+			}
+		}
+
+		nd.out = output;
+		nd.in = input;
+		nd.output_count = static_cast<uint32_t>(output_total);
+		nd.in_fm = input_feature_map_count;
+		nd.out_fm = out_fm;
+		nd.fm_window = feature_map_subsampling_size;
+		nd.entry_window = entry_subsampling_size;
+		nd.in_plane = static_cast<uint32_t>(in_plane);
+		const dim3 grid((nd.output_count + max_block_size - 1) / max_block_size);
+		if (is_min)
+			hipLaunchKernelGGL(max_window_nd_kernel<true>, grid, dim3(max_block_size), 0, stream, nd);
+		else
+			hipLaunchKernelGGL(max_window_nd_kernel<false>, grid, dim3(max_block_size), 0, stream, nd);
+		return launch_status();
+	}
+
+	int maxout_forward(hipStream_t stream, float* output, const float* input,
+		uint32_t entry_count, uint32_t output_feature_map_count, uint32_t neuron_count_per_feature_map,
+		uint32_t feature_map_subsampling_size)
+	{
+		if ((output == nullptr) || (input == nullptr))
+			return NNF_HIP_EINVAL;
+		// nnforge/maxout_layer.cpp:36-40
+		if ((feature_map_subsampling_size < 2) || (output_feature_map_count == 0) || (neuron_count_per_feature_map == 0))
+			return NNF_HIP_EINVAL;
+		if (!is_aligned16(output) || !is_aligned16(input))
+			return NNF_HIP_EALIGN;
+		const uint64_t group64 = static_cast<uint64_t>(output_feature_map_count) * neuron_count_per_feature_map;
+		const uint64_t output_total = group64 * entry_count;
+		const uint64_t input_total = output_total * feature_map_subsampling_size;
+		if (output_total == 0)
+			return NNF_HIP_OK;
+		if (input_total > 0xFFFF0000ull)
+			return NNF_HIP_ETOOBIG;
+		if (overlap(output, output_total * sizeof(float), input, input_total * sizeof(float)))
+			return NNF_HIP_EOVERLAP;
+		const uint32_t group = static_cast<uint32_t>(group64);
+		const uint32_t rows = std::min(entry_count, 65535u);
+		if ((group % 4) == 0)
+		{
+			const dim3 grid((group / 4 + max_block_size - 1) / max_block_size, rows);
+			hipLaunchKernelGGL(maxout_vec4_kernel, grid, dim3(max_block_size), 0, stream, output, input, entry_count, group, feature_map_subsampling_size);
+		}
+		else
+		{
+			const dim3 grid((group + max_block_size - 1) / max_block_size, rows);
+			hipLaunchKernelGGL(maxout_scalar_kernel, grid, dim3(max_block_size), 0, stream, output, input, entry_count, group, feature_map_subsampling_size);
+		}
+		return launch_status();
+	}
+}

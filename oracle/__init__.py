@@ -49,6 +49,15 @@ def load():
         lib.nnf_oracle_softmax.argtypes = [_FP, _FP, ctypes.c_uint, ctypes.c_uint, ctypes.c_uint, ctypes.c_int]
         lib.nnf_oracle_average_subsampling.argtypes = [_FP, _FP, ctypes.c_uint, ctypes.c_uint, ctypes.c_uint, ctypes.c_int,
                                                        _UP, _UP, _UP, ctypes.c_uint, ctypes.c_uint, ctypes.c_float, ctypes.c_int]
+        lib.nnf_oracle_absolute.argtypes = [_FP, _FP, ctypes.c_size_t, ctypes.c_int]
+        lib.nnf_oracle_dropout.argtypes = [_FP, _FP, ctypes.c_size_t]
+        lib.nnf_oracle_concat.argtypes = [_FP, ctypes.POINTER(_FP), _UP, ctypes.c_int, ctypes.c_uint]
+        lib.nnf_oracle_maxout.argtypes = [_FP, _FP, ctypes.c_uint, ctypes.c_uint, ctypes.c_uint, ctypes.c_uint, ctypes.c_int]
+        lib.nnf_oracle_max_subsampling.argtypes = [_FP, _FP, ctypes.c_uint, ctypes.c_uint, ctypes.c_uint, ctypes.c_int,
+                                                   _UP, _UP, _UP, _UP, ctypes.c_uint, ctypes.c_uint, ctypes.c_int, ctypes.c_int,
+                                                   ctypes.c_int]
+        lib.nnf_oracle_max_subsampling_tiling.argtypes = [_FP, _FP, ctypes.c_uint, ctypes.c_uint, ctypes.c_int, _UP, _UP, _UP,
+                                                          ctypes.c_int, ctypes.c_int]
         _lib = lib
     return _lib
 
@@ -171,3 +180,78 @@ def average_subsampling_full_mult(window_sizes, feature_map_window=1, entry_wind
     w = list(window_sizes)
     return load().nnf_oracle_average_subsampling_full_mult(len(w), (ctypes.c_uint * len(w))(*w), feature_map_window,
                                                            entry_window, int(alpha is not None), float(alpha or 0.0))
+
+
+def absolute(x, out=None, threads=0):
+    x = _f32(x)
+    out = _out_for(x, out)
+    load().nnf_oracle_absolute(_ptr(out), _ptr(x), x.size, threads)
+    return out
+
+
+def dropout(x, out=None):
+    x = _f32(x)
+    out = _out_for(x, out)
+    load().nnf_oracle_dropout(_ptr(out), _ptr(x), x.size)
+    return out
+
+
+def concat(inputs):
+    """inputs: arrays [N][C_i][spatial...] with equal N and spatial sizes; joined along feature maps."""
+    arrays = [_f32(a) for a in inputs]
+    n = arrays[0].shape[0]
+    assert all(a.shape[0] == n and a.shape[2:] == arrays[0].shape[2:] for a in arrays)
+    counts = [a.size // n if n else 0 for a in arrays]
+    out = np.empty((n, sum(a.shape[1] for a in arrays)) + arrays[0].shape[2:], dtype=np.float32)
+    ptrs = (_FP * len(arrays))(*[_ptr(a) for a in arrays])
+    load().nnf_oracle_concat(_ptr(out), ptrs, (ctypes.c_uint * len(counts))(*counts), len(arrays), n)
+    return out
+
+
+def maxout(x, feature_map_subsampling_size, threads=0):
+    x = _f32(x)
+    n, c, plane = _shape3(x)
+    assert c % feature_map_subsampling_size == 0
+    c_out = c // feature_map_subsampling_size
+    out = np.empty((n, c_out) + x.shape[2:], dtype=np.float32)
+    load().nnf_oracle_maxout(_ptr(out), _ptr(x), n, c_out, plane, feature_map_subsampling_size, threads)
+    return out
+
+
+def max_subsampling_output_sizes(dims, window_sizes, strides=None, round_ups=None, tiling=False):
+    """nnForge order (x first); nnforge/max_subsampling_layer.cpp:119-141."""
+    strides = list(strides) if strides else list(window_sizes)
+    round_ups = list(round_ups) if round_ups else [False] * len(dims)
+    if tiling:
+        return [(d - (w - 1)) // w for d, w in zip(dims, window_sizes)]
+    return [(d + s - w + (w - 1 if r else 0)) // s for d, w, s, r in zip(dims, window_sizes, strides, round_ups)]
+
+
+def max_subsampling(x, window_sizes, strides=None, round_ups=None, feature_map_window=1, entry_window=1, is_min=False,
+                    tiling=False, threads=0):
+    """x: [N][C][d_last]...[d_0]; window_sizes, strides, round_ups per spatial dimension, x first."""
+    x = _f32(x)
+    dims = list(x.shape[2:])[::-1]
+    if not dims:
+        dims = [1]
+    window_sizes = list(window_sizes)
+    assert len(window_sizes) == len(dims)
+    strides = list(strides) if strides else list(window_sizes)
+    out_dims = max_subsampling_output_sizes(dims, window_sizes, strides, round_ups, tiling)
+    assert all(o > 0 for o in out_dims)
+    arr = lambda v: (ctypes.c_uint * len(v))(*v)
+    if tiling:
+        assert feature_map_window == 1 and entry_window == 1 and not (round_ups and any(round_ups))
+        tiles = int(np.prod(window_sizes))
+        out = np.empty([x.shape[0] * tiles, x.shape[1]] + out_dims[::-1], dtype=np.float32)
+        load().nnf_oracle_max_subsampling_tiling(_ptr(out), _ptr(x), x.shape[0], x.shape[1], len(dims), arr(dims), arr(out_dims),
+                                                 arr(window_sizes), int(is_min), threads)
+        return out
+    n_out = x.shape[0] // entry_window
+    c_out = x.shape[1] // feature_map_window
+    out = np.empty([n_out, c_out] + out_dims[::-1], dtype=np.float32)
+    truncate = int(bool(round_ups) and any(round_ups))
+    load().nnf_oracle_max_subsampling(_ptr(out), _ptr(x), n_out, x.shape[1], c_out, len(dims), arr(dims), arr(out_dims),
+                                      arr(window_sizes), arr(strides), feature_map_window, entry_window, int(is_min), truncate,
+                                      threads)
+    return out

@@ -340,3 +340,279 @@ NNF_ORACLE_API float nnf_oracle_average_subsampling_full_mult(int dimension_coun
 		elems *= window_sizes[d];
 	return 1.0F / (float)elems;
 }
+
+/* ---- neighbouring inference testers of the same chains ----------------------------------- */
+
+/* nnforge/plain/absolute_layer_tester_plain.cpp:43-49: out = fabs(in) */
+NNF_ORACLE_API void nnf_oracle_absolute(float* out, const float* in, size_t elem_count, int threads)
+{
+	const long long count = (long long)elem_count;
+	long long i;
+	#pragma omp parallel for schedule(guided) num_threads(thread_count(threads))
+	for (i = 0; i < count; ++i)
+		out[i] = fabsf(in[i]);
+}
+
+/* nnforge/plain/dropout_layer_tester_plain.cpp:45-48: at inference the layer passes its input on
+ * unchanged (a copy unless it runs in place) */
+NNF_ORACLE_API void nnf_oracle_dropout(float* out, const float* in, size_t elem_count)
+{
+	if (out != in)
+		memcpy(out, in, elem_count * sizeof(float));
+}
+
+/* nnforge/plain/concat_layer_tester_plain.cpp:45-58: per entry, the inputs' neurons one after the
+ * other (feature maps of input 0, then of input 1, ...) */
+NNF_ORACLE_API void nnf_oracle_concat(float* out, const float* const* inputs, const unsigned int* input_neuron_counts,
+	int input_count, unsigned int entry_count)
+{
+	size_t output_neuron_count = 0;
+	unsigned int entry_id;
+	int i;
+	for (i = 0; i < input_count; ++i)
+		output_neuron_count += input_neuron_counts[i];
+	for (entry_id = 0; entry_id < entry_count; ++entry_id)
+	{
+		float* dst = out + (size_t)entry_id * output_neuron_count;
+		for (i = 0; i < input_count; ++i)
+		{
+			memcpy(dst, inputs[i] + (size_t)entry_id * input_neuron_counts[i], (size_t)input_neuron_counts[i] * sizeof(float));
+			dst += input_neuron_counts[i];
+		}
+	}
+}
+
+/* std::max(a, b) and std::min(a, b) as the C++ library defines them: the first argument wins ties
+ * and unordered comparisons */
+static inline float std_max(float a, float b) { return (a < b) ? b : a; }
+static inline float std_min(float a, float b) { return (b < a) ? b : a; }
+
+/* nnforge/plain/maxout_layer_tester_plain.cpp:56-80: output feature map o is the maximum over the
+ * input feature maps o, o + out_fm, o + 2*out_fm, ...; starts from the first value and folds with
+ * std::max(new_val, current_max) */
+NNF_ORACLE_API void nnf_oracle_maxout(float* out, const float* in, unsigned int entry_count, unsigned int output_feature_map_count,
+	unsigned int plane, unsigned int feature_map_subsampling_size, int threads)
+{
+	const size_t output_neuron_count = (size_t)output_feature_map_count * plane;
+	const size_t input_neuron_count = output_neuron_count * feature_map_subsampling_size;
+	const int total_workload = (int)(entry_count * output_feature_map_count);
+	int workload_id;
+	#pragma omp parallel for schedule(guided) num_threads(thread_count(threads))
+	for (workload_id = 0; workload_id < total_workload; ++workload_id)
+	{
+		const int entry_id = workload_id / (int)output_feature_map_count;
+		const int fm = workload_id - entry_id * (int)output_feature_map_count;
+		const float* src = in + (size_t)entry_id * input_neuron_count + (size_t)fm * plane;
+		float* dst = out + (size_t)entry_id * output_neuron_count + (size_t)fm * plane;
+		unsigned int p, i;
+		for (p = 0; p < plane; ++p)
+		{
+			float current_max = src[p];
+			for (i = 1; i < feature_map_subsampling_size; ++i)
+				current_max = std_max(src[p + (size_t)i * output_neuron_count], current_max);
+			dst[p] = current_max;
+		}
+	}
+}
+
+/*
+ * nnforge/plain/max_subsampling_layer_tester_plain.cpp:175-290 (test_non_tiling): windows of
+ * window_sizes[d] elements every strides[d] elements over the spatial dimensions, then over
+ * feature_map_window neighbouring feature maps and entry_window neighbouring entries; the window is
+ * scanned x fastest, ..., feature map, entry, starting from -1.0e37F (maximum) or 1.0e37F (minimum)
+ * and folding with std::max<float>(current, new) / std::min<float>(current, new).
+ * The plain tester refuses round_up; `truncate` restates what the CUDA tester does for it
+ * (nnforge/cuda/max_subsampling_layer_tester_cuda.cuh:97-116, TRUNCATION): window elements that
+ * lie beyond the input in a spatial dimension are skipped. output_sizes come from
+ * nnforge/max_subsampling_layer.cpp:131-141.
+ */
+NNF_ORACLE_API void nnf_oracle_max_subsampling(float* out, const float* in, unsigned int output_entry_count,
+	unsigned int input_feature_map_count, unsigned int output_feature_map_count,
+	int dimension_count, const unsigned int* input_sizes, const unsigned int* output_sizes,
+	const unsigned int* window_sizes, const unsigned int* strides,
+	unsigned int feature_map_window, unsigned int entry_window, int is_min, int truncate, int threads)
+{
+	enum { max_dims = 6 };
+	unsigned int sub_sizes[max_dims + 2];
+	size_t slices[max_dims + 2];
+	size_t in_plane = 1, out_plane = 1;
+	unsigned int window_elems = 1;
+	int sub_count, d;
+	size_t* offsets;
+	unsigned int* positions; /* window element -> its position in every spatial dimension */
+	const int total_workload = (int)(output_entry_count * output_feature_map_count);
+	int workload_id;
+
+	if (dimension_count < 1 || dimension_count > max_dims)
+		return;
+	for (d = 0; d < dimension_count; ++d)
+	{
+		sub_sizes[d] = window_sizes[d];
+		in_plane *= input_sizes[d];
+		out_plane *= output_sizes[d];
+	}
+	sub_sizes[dimension_count] = feature_map_window;
+	sub_sizes[dimension_count + 1] = entry_window;
+	sub_count = dimension_count + 2;
+	slices[0] = 1;
+	for (d = 0; d < sub_count - 1; ++d)
+		slices[d + 1] = slices[d] * (d < dimension_count ? input_sizes[d] : input_feature_map_count);
+	for (d = 0; d < sub_count; ++d)
+		window_elems *= sub_sizes[d];
+
+	offsets = (size_t*)calloc(window_elems, sizeof(size_t));
+	positions = (unsigned int*)calloc((size_t)window_elems * max_dims, sizeof(unsigned int));
+	{
+		unsigned int pos[max_dims + 2];
+		unsigned int i;
+		memset(pos, 0, sizeof(pos));
+		for (i = 1; i < window_elems; ++i)
+		{
+			for (d = 0; d < sub_count; ++d)
+			{
+				if (++pos[d] < sub_sizes[d])
+					break;
+				pos[d] = 0;
+			}
+			for (d = 0; d < sub_count; ++d)
+				offsets[i] += pos[d] * slices[d];
+			for (d = 0; d < dimension_count; ++d)
+				positions[(size_t)i * max_dims + d] = pos[d];
+		}
+	}
+
+	#pragma omp parallel for schedule(guided) num_threads(thread_count(threads))
+	for (workload_id = 0; workload_id < total_workload; ++workload_id)
+	{
+		const int out_entry = workload_id / (int)output_feature_map_count;
+		const int out_fm = workload_id - out_entry * (int)output_feature_map_count;
+		const float* src_base = in
+			+ (size_t)out_entry * entry_window * in_plane * input_feature_map_count
+			+ (size_t)out_fm * feature_map_window * in_plane;
+		float* dst = out + ((size_t)out_entry * output_feature_map_count + out_fm) * out_plane;
+		unsigned int out_pos[max_dims];
+		size_t o;
+		memset(out_pos, 0, sizeof(out_pos));
+		for (o = 0; o < out_plane; ++o)
+		{
+			size_t first = 0;
+			float current = is_min ? 1.0e37F : -1.0e37F;
+			unsigned int i;
+			int dd;
+			for (dd = 0; dd < dimension_count; ++dd)
+				first += (size_t)out_pos[dd] * strides[dd] * slices[dd];
+			for (i = 0; i < window_elems; ++i)
+			{
+				float new_val;
+				if (truncate)
+				{
+					int inside = 1;
+					for (dd = 0; dd < dimension_count; ++dd)
+						if (out_pos[dd] * strides[dd] + positions[(size_t)i * max_dims + dd] >= input_sizes[dd])
+							inside = 0;
+					if (!inside)
+						continue;
+				}
+				new_val = src_base[first + offsets[i]];
+				current = is_min ? std_min(current, new_val) : std_max(current, new_val);
+			}
+			dst[o] = current;
+			for (dd = 0; dd < dimension_count; ++dd)
+			{
+				if (++out_pos[dd] < output_sizes[dd])
+					break;
+				out_pos[dd] = 0;
+			}
+		}
+	}
+	free(offsets);
+	free(positions);
+}
+
+/*
+ * nnforge/plain/max_subsampling_layer_tester_plain.cpp:78-170 (test_tiling): every input entry gives
+ * prod(window_sizes) output entries, one per shift of the window grid (shifts in the same x-fastest
+ * order as the window scan); output entry e*T + j at position o is the fold over the window that
+ * starts at o*window + shift_j. Output sizes are (input - (window - 1)) / window
+ * (nnforge/max_subsampling_layer.cpp:119-128).
+ */
+NNF_ORACLE_API void nnf_oracle_max_subsampling_tiling(float* out, const float* in, unsigned int input_entry_count,
+	unsigned int feature_map_count, int dimension_count, const unsigned int* input_sizes, const unsigned int* output_sizes,
+	const unsigned int* window_sizes, int is_min, int threads)
+{
+	enum { max_dims = 6 };
+	size_t slices[max_dims];
+	size_t in_plane = 1, out_plane = 1;
+	unsigned int window_elems = 1;
+	size_t* offsets;
+	const int total_workload = (int)(input_entry_count * feature_map_count);
+	int workload_id, d;
+
+	if (dimension_count < 1 || dimension_count > max_dims)
+		return;
+	slices[0] = 1;
+	for (d = 0; d < dimension_count; ++d)
+	{
+		if (d + 1 < dimension_count)
+			slices[d + 1] = slices[d] * input_sizes[d];
+		in_plane *= input_sizes[d];
+		out_plane *= output_sizes[d];
+		window_elems *= window_sizes[d];
+	}
+	offsets = (size_t*)calloc(window_elems, sizeof(size_t));
+	{
+		unsigned int pos[max_dims];
+		unsigned int i;
+		memset(pos, 0, sizeof(pos));
+		for (i = 1; i < window_elems; ++i)
+		{
+			for (d = 0; d < dimension_count; ++d)
+			{
+				if (++pos[d] < window_sizes[d])
+					break;
+				pos[d] = 0;
+			}
+			for (d = 0; d < dimension_count; ++d)
+				offsets[i] += pos[d] * slices[d];
+		}
+	}
+	{
+		const size_t output_neuron_count = out_plane * feature_map_count;
+		#pragma omp parallel for schedule(guided) num_threads(thread_count(threads))
+		for (workload_id = 0; workload_id < total_workload; ++workload_id)
+		{
+			const int entry_id = workload_id / (int)feature_map_count;
+			const int fm = workload_id - entry_id * (int)feature_map_count;
+			const float* src_base = in + ((size_t)entry_id * feature_map_count + fm) * in_plane;
+			float* dst_base = out + (size_t)entry_id * window_elems * output_neuron_count + (size_t)fm * out_plane;
+			unsigned int out_pos[max_dims];
+			size_t o;
+			memset(out_pos, 0, sizeof(out_pos));
+			for (o = 0; o < out_plane; ++o)
+			{
+				size_t first = 0;
+				unsigned int i, j;
+				int dd;
+				for (dd = 0; dd < dimension_count; ++dd)
+					first += (size_t)out_pos[dd] * window_sizes[dd] * slices[dd];
+				for (j = 0; j < window_elems; ++j)
+				{
+					float current = is_min ? 1.0e37F : -1.0e37F;
+					for (i = 0; i < window_elems; ++i)
+					{
+						const float new_val = src_base[first + offsets[j] + offsets[i]];
+						current = is_min ? std_min(current, new_val) : std_max(current, new_val);
+					}
+					dst_base[(size_t)j * output_neuron_count + o] = current;
+				}
+				for (dd = 0; dd < dimension_count; ++dd)
+				{
+					if (++out_pos[dd] < output_sizes[dd])
+						break;
+					out_pos[dd] = 0;
+				}
+			}
+		}
+	}
+	free(offsets);
+}

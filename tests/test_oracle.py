@@ -257,3 +257,163 @@ def test_average_subsampling_feature_map_and_entry_windows():
     got = oracle.average_subsampling(x, [2, 1], feature_map_window=3, entry_window=2)
     ref = oracle.average_subsampling(x, [2, 1], feature_map_window=3, entry_window=2, mult=float(F(1.0) / F(6.0)))
     assert bits_equal(got, ref)
+
+
+# ---- neighbouring testers: absolute, dropout, concat, maxout, max subsampling ------------------
+
+def fold_max(values, start=None, new_first=False):
+    """std::max folded over values the way the testers write it. new_first: std::max(new, current)
+    (maxout); otherwise std::max<float>(current, new) (max subsampling). std::max(a, b) = (a < b) ? b : a."""
+    cur = start
+    for v in values:
+        if cur is None:
+            cur = v
+            continue
+        a, b = (v, cur) if new_first else (cur, v)
+        cur = b if a < b else a
+    return cur
+
+
+def test_absolute_dropout():
+    x = T.normal(T.rng(40, 0), (3, 4, 5, 6), 5.0)
+    x.reshape(-1)[:4] = [-0.0, 0.0, -np.inf, np.nan]
+    got = oracle.absolute(x)
+    assert bits_equal(got, np.abs(x))
+    assert np.signbit(got).sum() == 0
+    d = oracle.dropout(x)
+    assert bits_equal(d, x) and d is not x
+    y = x.copy()
+    assert oracle.dropout(y, out=y) is y and bits_equal(y, x)   # in place: nothing moves
+
+
+def test_concat_joins_feature_maps_per_entry():
+    gen = T.rng(41, 0)
+    parts = [T.normal(gen, (4, c, 3, 5)) for c in (2, 7, 1)]
+    got = oracle.concat(parts)
+    assert got.shape == (4, 10, 3, 5)
+    assert bits_equal(got, np.concatenate(parts, axis=1))
+    # no spatial dimensions, one input
+    flat = [T.normal(gen, (6, 9))]
+    assert bits_equal(oracle.concat(flat), flat[0])
+
+
+def test_maxout_groups_strided_feature_maps():
+    gen = T.rng(42, 0)
+    n, c_out, k, h, w = 3, 4, 3, 2, 5
+    x = T.normal(gen, (n, c_out * k, h, w), 2.0)
+    got = oracle.maxout(x, k)
+    assert got.shape == (n, c_out, h, w)
+    # output map o covers input maps o, o + c_out, o + 2 c_out (not o*k .. o*k + k - 1)
+    want = x.reshape(n, k, c_out, h, w).max(axis=1)
+    assert bits_equal(got, want)
+    assert not bits_equal(got, x.reshape(n, c_out, k, h, w).max(axis=2))
+    # ties and unordered values: std::max(new, current) keeps the NEW value unless new < current
+    special = np.zeros((1, 3, 1, 4), F)
+    special[0, :, 0, 0] = [0.0, -0.0, 0.0]          # -> last +0.0
+    special[0, :, 0, 1] = [0.0, 0.0, -0.0]          # -> -0.0
+    special[0, :, 0, 2] = [np.nan, 1.0, 0.5]        # nan replaced by 1.0, 0.5 < 1.0 keeps 1.0
+    special[0, :, 0, 3] = [1.0, np.nan, 0.5]        # nan wins over 1.0, then 0.5 replaces nan
+    g = oracle.maxout(special, 3)[0, 0, 0]
+    for col in range(4):
+        want_v = fold_max([F(v) for v in special[0, :, 0, col]], new_first=True)
+        assert g[col].tobytes() == F(want_v).tobytes(), col
+    assert np.signbit(g[1]) and not np.signbit(g[0]) and g[2] == 1.0 and g[3] == 0.5
+
+
+def window_view_max(x, windows, strides, is_min=False):
+    """Independent evaluation with numpy's sliding windows; windows/strides in numpy axis order
+    (spatial axes of x after [N][C])."""
+    from numpy.lib.stride_tricks import sliding_window_view
+    axes = tuple(range(2, x.ndim))
+    v = sliding_window_view(x, tuple(windows), axis=axes)
+    index = (slice(None), slice(None)) + tuple(slice(None, None, s) for s in strides)
+    v = v[index]
+    red = tuple(range(x.ndim, x.ndim + len(windows)))
+    return v.min(axis=red) if is_min else v.max(axis=red)
+
+
+@pytest.mark.parametrize("shape,windows,strides", [
+    ((2, 3, 9, 11), (3, 3), (2, 2)),      # the ResNet pool1 pattern: 3x3 every 2
+    ((2, 3, 8, 12), (2, 2), (2, 2)),
+    ((1, 2, 7, 10), (3, 2), (1, 3)),      # y window 3 stride 1, x window 2 stride 3
+    ((2, 2, 13), (4,), (3,)),             # 1-D
+    ((1, 2, 5, 6, 7), (2, 3, 2), (2, 2, 1)),   # 3-D
+])
+@pytest.mark.parametrize("is_min", [False, True])
+def test_max_subsampling_against_sliding_windows(shape, windows, strides, is_min):
+    x = T.normal(T.rng(43, len(shape)), shape, 3.0)
+    # oracle takes nnForge order (x first): reverse
+    got = oracle.max_subsampling(x, list(windows)[::-1], strides=list(strides)[::-1], is_min=is_min)
+    want = window_view_max(x, windows, strides, is_min)
+    assert got.shape == want.shape
+    assert bits_equal(got, want)
+
+
+def test_max_subsampling_default_stride_is_the_window_and_margin_is_dropped():
+    x = T.normal(T.rng(43, 100), (2, 2, 7, 9))
+    got = oracle.max_subsampling(x, [2, 3])         # x window 2, y window 3
+    assert got.shape == (2, 2, 2, 4)
+    assert bits_equal(got, window_view_max(x, (3, 2), (3, 2)))
+
+
+def test_max_subsampling_round_up_skips_what_lies_outside():
+    x = T.normal(T.rng(43, 101), (2, 3, 8, 8))
+    got = oracle.max_subsampling(x, [3, 3], strides=[2, 2], round_ups=[True, True])
+    assert got.shape == (2, 3, 4, 4)                # (8 + 2 - 3 + 2) / 2 = 4; without round up 3
+    padded = np.full((2, 3, 9, 9), -np.inf, F)
+    padded[:, :, :8, :8] = x
+    assert bits_equal(got, window_view_max(padded, (3, 3), (2, 2)))
+    assert oracle.max_subsampling(x, [3, 3], strides=[2, 2]).shape == (2, 3, 3, 3)
+    # round up in x only
+    got = oracle.max_subsampling(x, [3, 3], strides=[2, 2], round_ups=[True, False])
+    assert got.shape == (2, 3, 3, 4)
+    assert bits_equal(got, window_view_max(padded[:, :, :8, :], (3, 3), (2, 2)))
+
+
+def test_max_subsampling_feature_map_and_entry_windows():
+    x = T.normal(T.rng(43, 102), (4, 6, 4, 6))
+    got = oracle.max_subsampling(x, [2, 2], feature_map_window=3, entry_window=2)
+    assert got.shape == (2, 2, 2, 3)
+    # neighbouring feature maps f*3 .. f*3+2 and entries e*2, e*2+1 join the window
+    want = x.reshape(2, 2, 2, 3, 2, 2, 3, 2).max(axis=(1, 3, 5, 7))
+    assert bits_equal(got, want)
+
+
+def test_max_subsampling_start_value_ties_and_nan():
+    # the fold starts at -1e37 / +1e37: smaller / larger inputs never show
+    x = np.full((1, 1, 2, 2), -3.0e38, F)
+    assert np.all(oracle.max_subsampling(x, [2, 2]) == F(-1.0e37))
+    assert np.all(oracle.max_subsampling(-x, [2, 2], is_min=True) == F(1.0e37))
+    # std::max<float>(current, new): the first of equal values stays, NaN never enters
+    x = np.array([[[[0.0, -0.0], [-0.0, 0.0]]]], F)
+    assert not np.signbit(oracle.max_subsampling(x, [2, 2])[0, 0, 0, 0])
+    assert np.signbit(oracle.max_subsampling(-x, [2, 2])[0, 0, 0, 0])
+    x = np.array([[[[np.nan, 2.0], [np.nan, -5.0]]]], F)
+    assert oracle.max_subsampling(x, [2, 2])[0, 0, 0, 0] == 2.0
+    assert oracle.max_subsampling(x, [2, 2], is_min=True)[0, 0, 0, 0] == -5.0
+    x = np.full((1, 1, 2, 2), np.nan, F)
+    assert oracle.max_subsampling(x, [2, 2])[0, 0, 0, 0] == F(-1.0e37)
+    # scan order x fastest: with windows 2 (x) by 2 (y) over +-0 the first zero met decides the sign
+    x = np.array([[[[-1.0, -0.0], [0.0, -2.0]]]], F)
+    want = fold_max([F(-1.0), F(-0.0), F(0.0), F(-2.0)], start=F(-1.0e37))
+    assert oracle.max_subsampling(x, [2, 2])[0, 0, 0, 0].tobytes() == F(want).tobytes()
+    assert np.signbit(want)
+
+
+def test_max_subsampling_tiling_brute_force():
+    # every input entry gives 2*3 output entries, one per shift of the window grid (x shift fastest)
+    n, c, h, w = 2, 2, 11, 7
+    x = T.normal(T.rng(43, 103), (n, c, h, w))
+    wx, wy = 2, 3
+    got = oracle.max_subsampling(x, [wx, wy], tiling=True)
+    oh, ow = (h - (wy - 1)) // wy, (w - (wx - 1)) // wx
+    assert got.shape == (n * wx * wy, c, oh, ow)
+    for e in range(n):
+        for sy in range(wy):
+            for sx in range(wx):
+                j = sy * wx + sx
+                for f in range(c):
+                    for oy in range(oh):
+                        for ox in range(ow):
+                            win = x[e, f, oy * wy + sy: oy * wy + sy + wy, ox * wx + sx: ox * wx + sx + wx]
+                            assert got[e * wx * wy + j, f, oy, ox] == win.max()
