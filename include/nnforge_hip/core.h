@@ -98,6 +98,8 @@ namespace nnforge
 		float get_float(const std::string& key, float default_value) const;
 		unsigned int get_uint(const std::string& key, unsigned int default_value) const;
 		unsigned int require_uint(const std::string& key, const std::string& context) const;
+		bool get_bool(const std::string& key, bool default_value) const; // text format: true / false
+		std::string get_string(const std::string& key, const std::string& default_value) const; // enum values, unquoted
 		std::vector<const schema_param_block *> children(const std::string& name) const;
 	};
 

@@ -191,4 +191,114 @@ namespace nnforge
 		std::vector<unsigned int> subsampling_sizes; // x first
 		float alpha;
 	};
+
+	// nnforge/absolute_layer.h; "Absolute"
+	class absolute_layer : public layer
+	{
+	public:
+		absolute_layer() = default;
+		layer::ptr clone() const override;
+		std::string get_type_name() const override;
+		float get_forward_flops_per_entry(const std::vector<layer_configuration_specific>& input_configuration_specific_list) const override;
+		static const std::string layer_type_name;
+	};
+
+	// nnforge/dropout_layer.h:26-52; "Dropout". At inference the layer passes its input on; the
+	// parameters are kept for schema round trips.
+	class dropout_layer : public layer
+	{
+	public:
+		explicit dropout_layer(float dropout_rate = 0.5F, bool per_feature_map = false);
+		layer::ptr clone() const override;
+		std::string get_type_name() const override;
+		float get_forward_flops_per_entry(const std::vector<layer_configuration_specific>&) const override { return 0.0F; }
+		std::string get_param_block_name() const override { return "dropout_param"; }
+		void read_params(const schema_param_block * block) override;
+		void write_params(std::ostream& out, const std::string& indent) const override;
+		std::vector<std::string> get_parameter_strings() const override;
+
+		static const std::string layer_type_name;
+		float dropout_rate;
+		bool per_feature_map;
+
+	private:
+		void check();
+	};
+
+	// Joins its inputs along feature maps (nnforge/concat_layer.h:23-45); "Concat"
+	class concat_layer : public layer
+	{
+	public:
+		concat_layer() = default;
+		layer::ptr clone() const override;
+		// feature maps add up; neurons per feature map must agree (nnforge/concat_layer.cpp:44-58)
+		layer_configuration_specific get_output_layer_configuration_specific(
+			const std::vector<layer_configuration_specific>& input_configuration_specific_list) const override;
+		std::string get_type_name() const override;
+		float get_forward_flops_per_entry(const std::vector<layer_configuration_specific>&) const override { return 0.0F; }
+		static const std::string layer_type_name;
+	};
+
+	// Maximum over feature_map_subsampling_size feature maps that lie output-feature-map-count apart
+	// (nnforge/maxout_layer.h:25-57); "Maxout"
+	class maxout_layer : public layer
+	{
+	public:
+		explicit maxout_layer(unsigned int feature_map_subsampling_size = 2);
+		layer::ptr clone() const override;
+		layer_configuration_specific get_output_layer_configuration_specific(
+			const std::vector<layer_configuration_specific>& input_configuration_specific_list) const override;
+		std::string get_type_name() const override;
+		float get_forward_flops_per_entry(const std::vector<layer_configuration_specific>& input_configuration_specific_list) const override;
+		std::string get_param_block_name() const override { return "maxout_param"; }
+		void read_params(const schema_param_block * block) override;
+		void write_params(std::ostream& out, const std::string& indent) const override;
+		std::vector<std::string> get_parameter_strings() const override;
+
+		static const std::string layer_type_name;
+		unsigned int feature_map_subsampling_size;
+
+	private:
+		void check();
+	};
+
+	// Maximum (or minimum) over windows (nnforge/max_subsampling_layer.h:27-82); "MaxSubsampling".
+	// This backend runs spatial windows with strides and round up, and feature-map subsampling;
+	// tiling and entry subsampling change the number of entries between layers, which its driver
+	// does not do, so the layer refuses them when it is configured.
+	class max_subsampling_layer : public layer
+	{
+	public:
+		explicit max_subsampling_layer(
+			const std::vector<unsigned int>& subsampling_sizes = std::vector<unsigned int>(),
+			unsigned int feature_map_subsampling_size = 1,
+			unsigned int entry_subsampling_size = 1,
+			bool is_min = false,
+			bool tiling = false,
+			const std::vector<bool>& round_ups = std::vector<bool>(),
+			const std::vector<unsigned int>& strides = std::vector<unsigned int>());
+		layer::ptr clone() const override;
+		// (input + stride - window + (round_up ? window - 1 : 0)) / stride per dimension
+		// (nnforge/max_subsampling_layer.cpp:106-144)
+		layer_configuration_specific get_output_layer_configuration_specific(
+			const std::vector<layer_configuration_specific>& input_configuration_specific_list) const override;
+		std::string get_type_name() const override;
+		float get_forward_flops_per_entry(const std::vector<layer_configuration_specific>& input_configuration_specific_list) const override;
+		std::string get_param_block_name() const override { return "max_subsampling_param"; }
+		void read_params(const schema_param_block * block) override;
+		void write_params(std::ostream& out, const std::string& indent) const override;
+		std::vector<std::string> get_parameter_strings() const override;
+
+		static const std::string layer_type_name;
+		std::vector<unsigned int> subsampling_sizes; // x first
+		unsigned int feature_map_subsampling_size;
+		unsigned int entry_subsampling_size;
+		bool is_min;
+		bool tiling;
+		std::vector<bool> round_ups;
+		std::vector<unsigned int> strides;
+
+	private:
+		void check();
+	};
 }

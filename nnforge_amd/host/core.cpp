@@ -189,6 +189,24 @@ namespace nnforge
 		return get_uint(key, 0);
 	}
 
+	bool schema_param_block::get_bool(const std::string& key, bool default_value) const
+	{
+		std::map<std::string, std::string>::const_iterator it = scalars.find(key);
+		if (it == scalars.end())
+			return default_value;
+		if ((it->second == "true") || (it->second == "True") || (it->second == "t") || (it->second == "1"))
+			return true;
+		if ((it->second == "false") || (it->second == "False") || (it->second == "f") || (it->second == "0"))
+			return false;
+		throw neural_network_exception("Cannot parse \"" + it->second + "\" as a boolean for " + key);
+	}
+
+	std::string schema_param_block::get_string(const std::string& key, const std::string& default_value) const
+	{
+		std::map<std::string, std::string>::const_iterator it = scalars.find(key);
+		return (it == scalars.end()) ? default_value : it->second;
+	}
+
 	std::vector<const schema_param_block *> schema_param_block::children(const std::string& name) const
 	{
 		std::vector<const schema_param_block *> res;
@@ -308,5 +326,10 @@ namespace nnforge
 		f.register_layer(layer::ptr(new add_layer()));
 		f.register_layer(layer::ptr(new softmax_layer()));
 		f.register_layer(layer::ptr(new average_subsampling_layer(std::vector<unsigned int>(1, 1))));
+		f.register_layer(layer::ptr(new absolute_layer()));
+		f.register_layer(layer::ptr(new dropout_layer()));
+		f.register_layer(layer::ptr(new concat_layer()));
+		f.register_layer(layer::ptr(new maxout_layer(2)));
+		f.register_layer(layer::ptr(new max_subsampling_layer(std::vector<unsigned int>(1, 1))));
 	}
 }

@@ -60,13 +60,15 @@ namespace nnforge
 				std::vector<std::string> chunk_layers; // fused steps: layers whose weight chunks are concatenated into chunk_ptrs
 				int output_buffer;
 				std::vector<int> input_buffers;
+				bool passes_input_on = false;        // every layer of the step is a Dropout
 			};
 
 			bool is_unary_elementwise(const std::string& type)
 			{
 				return (type == batch_norm_layer::layer_type_name) || (type == rectified_linear_layer::layer_type_name)
 					|| (type == parametric_rectified_linear_layer::layer_type_name) || (type == exponential_linear_layer::layer_type_name)
-					|| (type == sigmoid_layer::layer_type_name) || (type == hyperbolic_tangent_layer::layer_type_name);
+					|| (type == sigmoid_layer::layer_type_name) || (type == hyperbolic_tangent_layer::layer_type_name)
+					|| (type == absolute_layer::layer_type_name) || (type == dropout_layer::layer_type_name);
 			}
 
 			struct pinned_buffer
@@ -372,10 +374,12 @@ namespace nnforge
 				// report bookkeeping: name, layer types, flops (the reference's model) and memory traffic per entry
 				std::string types;
 				float step_flops = 0.0F;
+				plan.passes_input_on = true;
 				for(const std::string& n : plan.info.layer_names)
 				{
 					plan.key += (plan.key.empty() ? "" : "+") + n;
 					layer::const_ptr l = this->schema->get_layer(n);
+					plan.passes_input_on = plan.passes_input_on && (l->get_type_name() == dropout_layer::layer_type_name);
 					types += (types.empty() ? "" : "+") + l->get_type_name();
 					std::vector<layer_configuration_specific> inputs;
 					for(const std::string& input : l->input_layer_instance_names)
@@ -653,6 +657,8 @@ namespace nnforge
 						std::vector<hip_linear_buffer_device::const_ptr> inputs;
 						for(int b : plan.input_buffers)
 							inputs.push_back(buffers[slot][b]);
+						if (plan.passes_input_on && (plan.output_buffer == plan.input_buffers.at(0)))
+							continue; // Dropout layers only, in place: nothing to do at inference
 						if (plan.info.fused)
 						{
 							plan.desc.entry_count = entries_read;

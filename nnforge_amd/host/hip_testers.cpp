@@ -477,6 +477,142 @@ namespace nnforge
 				float mult = 1.0F;
 			};
 
+			class absolute_layer_tester_hip : public elementwise_tester
+			{
+			public:
+				void enqueue_forward_propagation(void * stream_id, hip_linear_buffer_device::ptr output_buffer,
+					const std::vector<hip_linear_buffer_device::const_ptr>&, const std::vector<hip_linear_buffer_device::const_ptr>&,
+					const std::vector<hip_linear_buffer_device::const_ptr>&, const std::vector<hip_linear_buffer_device::const_ptr>& input_buffers,
+					const std::vector<hip_linear_buffer_device::const_ptr>&, hip_linear_buffer_device::ptr, hip_linear_buffer_device::ptr,
+					unsigned int entry_count) override
+				{
+					require_inputs(input_buffers, 1, "Absolute");
+					hip_safe_call(nnf_hip_absolute_forward(stream_id, *output_buffer, float_ptr(input_buffers[0]),
+						static_cast<uint64_t>(entry_count) * output_elem_count_per_entry));
+				}
+
+				int get_chain_op(nnf_hip_op& op) const override
+				{
+					op.kind = NNF_HIP_OP_ABSOLUTE;
+					op.f0 = op.f1 = 0.0F;
+					return 0;
+				}
+			};
+
+			// Inference: the input passes through (nnforge/cuda/dropout_layer_tester_cuda.cpp:27-51); in
+			// place nothing is launched, inside a fused group the layer costs nothing.
+			class dropout_layer_tester_hip : public elementwise_tester
+			{
+			public:
+				void enqueue_forward_propagation(void * stream_id, hip_linear_buffer_device::ptr output_buffer,
+					const std::vector<hip_linear_buffer_device::const_ptr>&, const std::vector<hip_linear_buffer_device::const_ptr>&,
+					const std::vector<hip_linear_buffer_device::const_ptr>&, const std::vector<hip_linear_buffer_device::const_ptr>& input_buffers,
+					const std::vector<hip_linear_buffer_device::const_ptr>&, hip_linear_buffer_device::ptr, hip_linear_buffer_device::ptr,
+					unsigned int entry_count) override
+				{
+					require_inputs(input_buffers, 1, "Dropout");
+					hip_safe_call(nnf_hip_dropout_forward(stream_id, *output_buffer, float_ptr(input_buffers[0]),
+						static_cast<uint64_t>(entry_count) * output_elem_count_per_entry));
+				}
+
+				int get_chain_op(nnf_hip_op& op) const override
+				{
+					op.kind = NNF_HIP_OP_DROPOUT;
+					op.f0 = op.f1 = 0.0F;
+					return 0;
+				}
+			};
+
+			class concat_layer_tester_hip : public layer_tester_hip
+			{
+			public:
+				void enqueue_forward_propagation(void * stream_id, hip_linear_buffer_device::ptr output_buffer,
+					const std::vector<hip_linear_buffer_device::const_ptr>&, const std::vector<hip_linear_buffer_device::const_ptr>&,
+					const std::vector<hip_linear_buffer_device::const_ptr>&, const std::vector<hip_linear_buffer_device::const_ptr>& input_buffers,
+					const std::vector<hip_linear_buffer_device::const_ptr>&, hip_linear_buffer_device::ptr, hip_linear_buffer_device::ptr,
+					unsigned int entry_count) override
+				{
+					require_inputs(input_buffers, input_elem_count_per_entry_list.size(), "Concat");
+					std::vector<const float *> inputs;
+					std::vector<uint32_t> counts;
+					for(size_t i = 0; i < input_elem_count_per_entry_list.size(); ++i)
+					{
+						inputs.push_back(float_ptr(input_buffers[i]));
+						counts.push_back(input_elem_count_per_entry_list[i]);
+					}
+					hip_safe_call(nnf_hip_concat_forward(stream_id, *output_buffer, inputs.data(), counts.data(), static_cast<uint32_t>(inputs.size()), entry_count));
+				}
+			};
+
+			class maxout_layer_tester_hip : public layer_tester_hip
+			{
+			public:
+				void enqueue_forward_propagation(void * stream_id, hip_linear_buffer_device::ptr output_buffer,
+					const std::vector<hip_linear_buffer_device::const_ptr>&, const std::vector<hip_linear_buffer_device::const_ptr>&,
+					const std::vector<hip_linear_buffer_device::const_ptr>&, const std::vector<hip_linear_buffer_device::const_ptr>& input_buffers,
+					const std::vector<hip_linear_buffer_device::const_ptr>&, hip_linear_buffer_device::ptr, hip_linear_buffer_device::ptr,
+					unsigned int entry_count) override
+				{
+					require_inputs(input_buffers, 1, "Maxout");
+					hip_safe_call(nnf_hip_maxout_forward(stream_id, *output_buffer, float_ptr(input_buffers[0]), entry_count,
+						output_configuration_specific.feature_map_count, output_elem_count_per_feature_map, feature_map_subsampling_size));
+				}
+
+			protected:
+				void tester_configured() override
+				{
+					std::shared_ptr<const maxout_layer> l = std::dynamic_pointer_cast<const maxout_layer>(layer_schema);
+					if (!l)
+						throw neural_network_exception("Maxout tester configured with a layer of type " + layer_schema->get_type_name());
+					feature_map_subsampling_size = l->feature_map_subsampling_size;
+				}
+
+			private:
+				unsigned int feature_map_subsampling_size = 2;
+			};
+
+			class max_subsampling_layer_tester_hip : public layer_tester_hip
+			{
+			public:
+				void enqueue_forward_propagation(void * stream_id, hip_linear_buffer_device::ptr output_buffer,
+					const std::vector<hip_linear_buffer_device::const_ptr>&, const std::vector<hip_linear_buffer_device::const_ptr>&,
+					const std::vector<hip_linear_buffer_device::const_ptr>&, const std::vector<hip_linear_buffer_device::const_ptr>& input_buffers,
+					const std::vector<hip_linear_buffer_device::const_ptr>&, hip_linear_buffer_device::ptr, hip_linear_buffer_device::ptr,
+					unsigned int entry_count) override
+				{
+					require_inputs(input_buffers, 1, "MaxSubsampling");
+					hip_safe_call(nnf_hip_max_subsampling_forward(stream_id, *output_buffer, float_ptr(input_buffers[0]), entry_count,
+						input_configuration_specific_list[0].feature_map_count, static_cast<uint32_t>(input_sizes.size()),
+						input_sizes.data(), windows.data(), strides.data(), round_ups.data(), feature_map_subsampling_size, 1, is_min ? 1 : 0));
+				}
+
+			protected:
+				void tester_configured() override
+				{
+					std::shared_ptr<const max_subsampling_layer> l = std::dynamic_pointer_cast<const max_subsampling_layer>(layer_schema);
+					if (!l)
+						throw neural_network_exception("MaxSubsampling tester configured with a layer of type " + layer_schema->get_type_name());
+					if (l->tiling || (l->entry_subsampling_size != 1))
+						throw neural_network_exception("The hip max subsampling tester does not run tiling or entry subsampling (layer " + layer_schema->instance_name + ")");
+					const layer_configuration_specific& in = input_configuration_specific_list.at(0);
+					if ((in.get_dimension_count() < 1) || (in.get_dimension_count() > NNF_HIP_MAX_SUBSAMPLING_DIMENSIONS))
+						throw neural_network_exception("The hip max subsampling tester handles 1 to 4 spatial dimensions, layer " + layer_schema->instance_name + " has " + std::to_string(in.get_dimension_count()));
+					input_sizes.assign(in.dimension_sizes.begin(), in.dimension_sizes.end());
+					windows.assign(l->subsampling_sizes.begin(), l->subsampling_sizes.end());
+					strides.assign(l->strides.begin(), l->strides.end());
+					round_ups.clear();
+					for(bool r : l->round_ups)
+						round_ups.push_back(r ? 1u : 0u);
+					feature_map_subsampling_size = l->feature_map_subsampling_size;
+					is_min = l->is_min;
+				}
+
+			private:
+				std::vector<uint32_t> input_sizes, windows, strides, round_ups;
+				unsigned int feature_map_subsampling_size = 1;
+				bool is_min = false;
+			};
+
 			template<class LAYER, class TESTER>
 			class simple_testing_schema : public layer_testing_schema
 			{
@@ -525,6 +661,11 @@ namespace nnforge
 			register_tester<add_layer, add_layer_tester_hip>();
 			register_tester<softmax_layer, softmax_layer_tester_hip>();
 			register_tester<average_subsampling_layer, average_subsampling_layer_tester_hip>();
+			register_tester<absolute_layer, absolute_layer_tester_hip>();
+			register_tester<dropout_layer, dropout_layer_tester_hip>();
+			register_tester<concat_layer, concat_layer_tester_hip>();
+			register_tester<maxout_layer, maxout_layer_tester_hip>();
+			register_tester<max_subsampling_layer, max_subsampling_layer_tester_hip>();
 		}
 	}
 }

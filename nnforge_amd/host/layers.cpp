@@ -391,4 +391,293 @@ namespace nnforge
 	{
 		return has_alpha() ? alpha : 1.0F;
 	}
+
+	// ---- Absolute ----------------------------------------------------------------------------
+
+	const std::string absolute_layer::layer_type_name = "Absolute";
+	layer::ptr absolute_layer::clone() const { return layer::ptr(new absolute_layer(*this)); }
+	std::string absolute_layer::get_type_name() const { return layer_type_name; }
+	float absolute_layer::get_forward_flops_per_entry(const std::vector<layer_configuration_specific>& configs) const
+	{
+		return neuron_count_of(configs);
+	}
+
+	// ---- Dropout -----------------------------------------------------------------------------
+
+	const std::string dropout_layer::layer_type_name = "Dropout";
+
+	dropout_layer::dropout_layer(float dropout_rate, bool per_feature_map)
+		: dropout_rate(dropout_rate), per_feature_map(per_feature_map)
+	{
+		check();
+	}
+
+	void dropout_layer::check()
+	{
+		if ((dropout_rate < 0.0F) || (dropout_rate >= 1.0F))
+			throw neural_network_exception("Error constructing dropout_layer: dropout_rate equals " + float_text(dropout_rate) + ", it should be in [0.0F,1.0F)");
+	}
+
+	layer::ptr dropout_layer::clone() const { return layer::ptr(new dropout_layer(*this)); }
+	std::string dropout_layer::get_type_name() const { return layer_type_name; }
+
+	void dropout_layer::read_params(const schema_param_block * block)
+	{
+		// nnforge/dropout_layer.cpp:82-88: a missing block gives the defaults of the message
+		dropout_rate = (block != nullptr) ? block->get_float("dropout_rate", 0.5F) : 0.5F;
+		per_feature_map = (block != nullptr) ? block->get_bool("per_feature_map", false) : false;
+		check();
+	}
+
+	void dropout_layer::write_params(std::ostream& out, const std::string& indent) const
+	{
+		// nnforge/dropout_layer.cpp:70-80 writes the block only for a rate other than 0.5
+		if (dropout_rate != 0.5F)
+		{
+			out << indent << "dropout_rate: " << float_text(dropout_rate) << "\n";
+			if (per_feature_map)
+				out << indent << "per_feature_map: true\n";
+		}
+	}
+
+	std::vector<std::string> dropout_layer::get_parameter_strings() const
+	{
+		char buf[64];
+		std::snprintf(buf, sizeof(buf), "dropout rate %.3f", static_cast<double>(dropout_rate));
+		std::string res(buf);
+		if (per_feature_map)
+			res += ", per fm";
+		return std::vector<std::string>(1, res);
+	}
+
+	// ---- Concat ------------------------------------------------------------------------------
+
+	const std::string concat_layer::layer_type_name = "Concat";
+	layer::ptr concat_layer::clone() const { return layer::ptr(new concat_layer(*this)); }
+	std::string concat_layer::get_type_name() const { return layer_type_name; }
+
+	layer_configuration_specific concat_layer::get_output_layer_configuration_specific(
+		const std::vector<layer_configuration_specific>& configs) const
+	{
+		if (configs.empty())
+			throw neural_network_exception("Layer " + instance_name + " has no input configuration");
+		unsigned int feature_map_count = configs[0].feature_map_count;
+		const unsigned int neuron_count_per_feature_map = configs[0].get_neuron_count_per_feature_map();
+		for(size_t i = 1; i < configs.size(); ++i)
+		{
+			feature_map_count += configs[i].feature_map_count;
+			if (configs[i].get_neuron_count_per_feature_map() != neuron_count_per_feature_map)
+				throw neural_network_exception("Neuron count per feature maps mismatch in 2 input layers for concat_layer");
+		}
+		return layer_configuration_specific(feature_map_count, configs[0].dimension_sizes);
+	}
+
+	// ---- Maxout ------------------------------------------------------------------------------
+
+	const std::string maxout_layer::layer_type_name = "Maxout";
+
+	maxout_layer::maxout_layer(unsigned int feature_map_subsampling_size)
+		: feature_map_subsampling_size(feature_map_subsampling_size)
+	{
+		check();
+	}
+
+	void maxout_layer::check()
+	{
+		if (feature_map_subsampling_size < 2)
+			throw neural_network_exception("Feature map subsampling size should be >= 2 for maxout layer");
+	}
+
+	layer::ptr maxout_layer::clone() const { return layer::ptr(new maxout_layer(*this)); }
+	std::string maxout_layer::get_type_name() const { return layer_type_name; }
+
+	layer_configuration_specific maxout_layer::get_output_layer_configuration_specific(
+		const std::vector<layer_configuration_specific>& configs) const
+	{
+		if (configs.empty())
+			throw neural_network_exception("Layer " + instance_name + " has no input configuration");
+		if ((configs[0].feature_map_count % feature_map_subsampling_size) != 0)
+			throw neural_network_exception("Feature map count in layer (" + std::to_string(configs[0].feature_map_count) + ") is not evenly divisible by feature map subsampling count (" + std::to_string(feature_map_subsampling_size) + ")");
+		return layer_configuration_specific(configs[0].feature_map_count / feature_map_subsampling_size, configs[0].dimension_sizes);
+	}
+
+	float maxout_layer::get_forward_flops_per_entry(const std::vector<layer_configuration_specific>& configs) const
+	{
+		return static_cast<float>(get_output_layer_configuration_specific(configs).get_neuron_count()) * static_cast<float>(feature_map_subsampling_size - 1);
+	}
+
+	void maxout_layer::read_params(const schema_param_block * block)
+	{
+		if (block == nullptr)
+			throw neural_network_exception("No maxout_param specified for layer " + instance_name + " of type " + layer_type_name);
+		feature_map_subsampling_size = block->require_uint("feature_map_subsampling_size", "maxout_param of layer " + instance_name);
+		check();
+	}
+
+	void maxout_layer::write_params(std::ostream& out, const std::string& indent) const
+	{
+		out << indent << "feature_map_subsampling_size: " << feature_map_subsampling_size << "\n";
+	}
+
+	std::vector<std::string> maxout_layer::get_parameter_strings() const
+	{
+		return std::vector<std::string>(1, "fm subsampling " + std::to_string(feature_map_subsampling_size));
+	}
+
+	// ---- MaxSubsampling ----------------------------------------------------------------------
+
+	const std::string max_subsampling_layer::layer_type_name = "MaxSubsampling";
+
+	max_subsampling_layer::max_subsampling_layer(
+		const std::vector<unsigned int>& subsampling_sizes,
+		unsigned int feature_map_subsampling_size,
+		unsigned int entry_subsampling_size,
+		bool is_min,
+		bool tiling,
+		const std::vector<bool>& round_ups,
+		const std::vector<unsigned int>& strides)
+		: subsampling_sizes(subsampling_sizes)
+		, feature_map_subsampling_size(feature_map_subsampling_size)
+		, entry_subsampling_size(entry_subsampling_size)
+		, is_min(is_min)
+		, tiling(tiling)
+	{
+		if (!round_ups.empty() && (round_ups.size() != subsampling_sizes.size()))
+			throw neural_network_exception("Invalid dimension count " + std::to_string(round_ups.size()) + " for round ups");
+		if (!strides.empty() && (strides.size() != subsampling_sizes.size()))
+			throw neural_network_exception("Invalid dimension count " + std::to_string(strides.size()) + " for strides");
+		this->round_ups = round_ups.empty() ? std::vector<bool>(subsampling_sizes.size(), false) : round_ups;
+		this->strides = strides.empty() ? subsampling_sizes : strides;
+		check();
+	}
+
+	void max_subsampling_layer::check()
+	{
+		for(unsigned int s : subsampling_sizes)
+			if (s == 0)
+				throw neural_network_exception("window dimension for max subsampling layer may not be zero");
+		if (feature_map_subsampling_size == 0)
+			throw neural_network_exception("feature map subsampling size for max subsampling layer may not be zero");
+		if (entry_subsampling_size == 0)
+			throw neural_network_exception("feature map subsampling size for max subsampling layer may not be zero"); // the reference's wording
+		if (tiling && (entry_subsampling_size > 1))
+			throw neural_network_exception("entry_subsampling_size cannot be set with tiling at the same time for max subsampling layer");
+		if (tiling && (feature_map_subsampling_size > 1))
+			throw neural_network_exception("feature_map_subsampling_size cannot be set with tiling at the same time for max subsampling layer");
+		for(size_t i = 0; i < strides.size(); ++i)
+			if (strides[i] == 0)
+				throw neural_network_exception("stride dimension (" + std::to_string(i) + ") is 0");
+		if (tiling)
+			for(bool r : round_ups)
+				if (r)
+					throw neural_network_exception("round up cannot be set with tiling at the same time for max subsampling layer");
+	}
+
+	layer::ptr max_subsampling_layer::clone() const { return layer::ptr(new max_subsampling_layer(*this)); }
+	std::string max_subsampling_layer::get_type_name() const { return layer_type_name; }
+
+	layer_configuration_specific max_subsampling_layer::get_output_layer_configuration_specific(
+		const std::vector<layer_configuration_specific>& configs) const
+	{
+		if (configs.empty())
+			throw neural_network_exception("Layer " + instance_name + " has no input configuration");
+		const layer_configuration_specific& in = configs[0];
+		if (in.get_dimension_count() != subsampling_sizes.size())
+			throw neural_network_exception("Dimension count in layer (" + std::to_string(subsampling_sizes.size()) + ") and input configuration (" + std::to_string(in.get_dimension_count()) + ") don't match");
+		if (tiling || (entry_subsampling_size != 1))
+			throw neural_network_exception("Tiling and entry subsampling of max subsampling layer " + instance_name + " change the number of entries between layers, which the hip backend does not support");
+		layer_configuration_specific res(in.feature_map_count / feature_map_subsampling_size);
+		for(size_t i = 0; i < subsampling_sizes.size(); ++i)
+		{
+			const int new_size = (static_cast<int>(in.dimension_sizes[i]) + static_cast<int>(strides[i]) - static_cast<int>(subsampling_sizes[i])
+				+ (round_ups[i] ? static_cast<int>(subsampling_sizes[i]) - 1 : 0)) / static_cast<int>(strides[i]);
+			if (new_size <= 0)
+				throw neural_network_exception("Input configuration size (" + std::to_string(in.dimension_sizes[i]) + ") of dimension (" + std::to_string(i) + ") produces 0 output size");
+			res.dimension_sizes.push_back(static_cast<unsigned int>(new_size));
+		}
+		return res;
+	}
+
+	float max_subsampling_layer::get_forward_flops_per_entry(const std::vector<layer_configuration_specific>& configs) const
+	{
+		const unsigned int neuron_count = get_output_layer_configuration_specific(configs).get_neuron_count();
+		unsigned int per_item = feature_map_subsampling_size * entry_subsampling_size;
+		for(unsigned int s : subsampling_sizes)
+			per_item *= s;
+		return static_cast<float>(neuron_count) * static_cast<float>(per_item - 1);
+	}
+
+	void max_subsampling_layer::read_params(const schema_param_block * block)
+	{
+		if (block == nullptr)
+			throw neural_network_exception("No max_subsampling_param specified for layer " + instance_name + " of type " + layer_type_name);
+		subsampling_sizes.clear();
+		round_ups.clear();
+		strides.clear();
+		for(const schema_param_block * dim : block->children("dimension_param"))
+		{
+			const unsigned int size = dim->require_uint("subsampling_size", "max_subsampling_param of layer " + instance_name);
+			subsampling_sizes.push_back(size);
+			round_ups.push_back(dim->get_bool("round_up", false));
+			strides.push_back(dim->has("stride") ? dim->get_uint("stride", size) : size);
+		}
+		const std::vector<const schema_param_block *> fm = block->children("feature_map_param");
+		feature_map_subsampling_size = fm.empty() ? 1 : fm[0]->require_uint("subsampling_size", "feature_map_param of layer " + instance_name);
+		const std::vector<const schema_param_block *> en = block->children("entry_param");
+		entry_subsampling_size = en.empty() ? 1 : en[0]->require_uint("subsampling_size", "entry_param of layer " + instance_name);
+		tiling = block->get_bool("tiling", false);
+		const std::string function = block->get_string("function", "MAX");
+		if ((function != "MAX") && (function != "MIN"))
+			throw neural_network_exception("Unknown function " + function + " in max_subsampling_param of layer " + instance_name);
+		is_min = (function == "MIN");
+		check();
+	}
+
+	void max_subsampling_layer::write_params(std::ostream& out, const std::string& indent) const
+	{
+		for(size_t i = 0; i < subsampling_sizes.size(); ++i)
+		{
+			out << indent << "dimension_param { subsampling_size: " << subsampling_sizes[i];
+			if (round_ups[i])
+				out << " round_up: true";
+			if (strides[i] != subsampling_sizes[i])
+				out << " stride: " << strides[i];
+			out << " }\n";
+		}
+		if (tiling)
+			out << indent << "tiling: true\n";
+		if (feature_map_subsampling_size != 1)
+			out << indent << "feature_map_param { subsampling_size: " << feature_map_subsampling_size << " }\n";
+		if (entry_subsampling_size != 1)
+			out << indent << "entry_param { subsampling_size: " << entry_subsampling_size << " }\n";
+		if (is_min)
+			out << indent << "function: MIN\n";
+	}
+
+	std::vector<std::string> max_subsampling_layer::get_parameter_strings() const
+	{
+		std::stringstream ss;
+		if (is_min)
+			ss << "MIN";
+		if (!subsampling_sizes.empty())
+		{
+			if (!ss.str().empty())
+				ss << ", ";
+			for(size_t i = 0; i < subsampling_sizes.size(); ++i)
+				ss << (i == 0 ? "" : "x") << subsampling_sizes[i] << (round_ups[i] ? "_roundup_" : "");
+		}
+		if (strides != subsampling_sizes)
+		{
+			ss << ", stride ";
+			for(size_t i = 0; i < strides.size(); ++i)
+				ss << (i == 0 ? "" : "x") << strides[i];
+		}
+		if (feature_map_subsampling_size != 1)
+			ss << (ss.str().empty() ? "" : ", ") << "fm " << feature_map_subsampling_size;
+		if (entry_subsampling_size != 1)
+			ss << (ss.str().empty() ? "" : ", ") << "samples " << entry_subsampling_size;
+		if (tiling)
+			ss << (ss.str().empty() ? "" : ", ") << "tiling";
+		return std::vector<std::string>(1, ss.str());
+	}
 }

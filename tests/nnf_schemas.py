@@ -13,7 +13,8 @@ def L(type_name, name, inputs=(), **params):
 
 
 PARAM_BLOCK = {"BatchNorm": "batch_norm_param", "ReLU": "relu_param", "PReLU": "prelu_param", "TanH": "tanh_param",
-               "Add": "add_param", "AverageSubsampling": "average_subsampling_param"}
+               "Add": "add_param", "AverageSubsampling": "average_subsampling_param", "Dropout": "dropout_param",
+               "Maxout": "maxout_param", "MaxSubsampling": "max_subsampling_param"}
 
 
 def schema_text(layers, name="test_net"):
@@ -29,8 +30,21 @@ def schema_text(layers, name="test_net"):
             out.append("\t%s {" % PARAM_BLOCK[l["type"]])
             for k, v in p.items():
                 if k == "windows":
-                    for w in v:
-                        out.append("\t\tdimension_param { subsampling_size: %d }" % w)
+                    for d, w in enumerate(v):
+                        extra = ""
+                        if p.get("round_ups") and p["round_ups"][d]:
+                            extra += " round_up: true"
+                        if p.get("strides"):
+                            extra += " stride: %d" % p["strides"][d]
+                        out.append("\t\tdimension_param { subsampling_size: %d%s }" % (w, extra))
+                elif k in ("strides", "round_ups"):
+                    continue
+                elif k == "fm_window":
+                    out.append("\t\tfeature_map_param { subsampling_size: %d }" % v)
+                elif k == "function":
+                    out.append("\t\tfunction: %s" % v)
+                elif isinstance(v, bool):
+                    out.append("\t\t%s: %s" % (k, "true" if v else "false"))
                 else:
                     out.append("\t\t%s: %r" % (k, v))
             out.append("\t}")
@@ -75,6 +89,17 @@ def evaluate(layers, weights, inputs):
         elif t == "AverageSubsampling":
             # the plain tester's multiplier: window sum unless alpha is given
             v = oracle.average_subsampling(ins[0], p["windows"], alpha=p.get("alpha"))
+        elif t == "Absolute":
+            v = oracle.absolute(ins[0])
+        elif t == "Dropout":
+            v = oracle.dropout(ins[0])
+        elif t == "Concat":
+            v = oracle.concat(ins)
+        elif t == "Maxout":
+            v = oracle.maxout(ins[0], p["feature_map_subsampling_size"])
+        elif t == "MaxSubsampling":
+            v = oracle.max_subsampling(ins[0], p["windows"], strides=p.get("strides"), round_ups=p.get("round_ups"),
+                                       feature_map_window=p.get("fm_window", 1), is_min=p.get("function") == "MIN")
         else:
             raise ValueError(t)
         values[name] = v
@@ -101,3 +126,23 @@ def classifier_tail(c=8):
 def activation_chain(c=6):
     return [L("Data", "x"), L("BatchNorm", "bn", ["x"], feature_map_count=c), L("ELU", "elu", ["bn"]), L("Sigmoid", "sig", ["elu"]),
             L("TanH", "tanh", ["sig"], scale=1.7159, steepness=0.6666)]
+
+
+def inception_like(c=8):
+    """A stem pooled 3x3 every 2 (rounded up), three branches (BatchNorm+ReLU, Absolute behind a
+    Dropout, a min pooling with stride 1 cut back by a second branch input), joined by Concat, halved by
+    Maxout, then Dropout in front of the output activation."""
+    return [
+        L("Data", "stem"),
+        L("MaxSubsampling", "pool1", ["stem"], windows=[3, 3], strides=[2, 2], round_ups=[True, True]),
+        L("BatchNorm", "b1_bn", ["pool1"], feature_map_count=c),
+        L("ReLU", "b1_relu", ["b1_bn"]),
+        L("Dropout", "b2_drop", ["pool1"], dropout_rate=0.25),
+        L("Absolute", "b2_abs", ["b2_drop"]),
+        L("PReLU", "b3_prelu", ["pool1"], feature_map_count=c),
+        L("Concat", "join", ["b1_relu", "b2_abs", "b3_prelu", "pool1"]),
+        L("Maxout", "mo", ["join"], feature_map_subsampling_size=2),
+        L("Dropout", "drop", ["mo"]),
+        L("MaxSubsampling", "pool2", ["drop"], windows=[2, 2], function="MIN"),
+        L("TanH", "out", ["pool2"]),
+    ]

@@ -182,3 +182,55 @@ def test_weight_files_round_trip(tmp_path):
     open(os.path.join(folder, "bad.data"), "wb").write(b"\0" * 40)
     with pytest.raises(backend.BackendError, match="Unknown data GUID"):
         backend.read_weights(folder, "p", [5])
+
+
+# ---- the neighbouring layers: Absolute, Dropout, Concat, Maxout, MaxSubsampling -------------------
+
+def test_neighbour_layers_schema_round_trip():
+    layers = S.inception_like(8) + [
+        S.L("MaxSubsampling", "fmpool", ["pool1"], windows=[1, 1], fm_window=4),
+        S.L("Dropout", "half", ["pool1"], dropout_rate=0.5, per_feature_map=True)]
+    once = backend.rewrite_schema(S.schema_text(layers))
+    assert once == backend.rewrite_schema(once)
+    for needle in ("dimension_param { subsampling_size: 3 round_up: true stride: 2 }", "dimension_param { subsampling_size: 2 }",
+                   "function: MIN", "feature_map_param { subsampling_size: 4 }", "dropout_rate: 0.25",
+                   "feature_map_subsampling_size: 2", 'type: "Concat"', 'type: "Absolute"'):
+        assert needle in once, needle
+    # the reference writes no dropout_param at all for the default rate, even when per_feature_map is set
+    # (nnforge/dropout_layer.cpp:70-80)
+    half = once[once.index('name: "half"'):]
+    assert "dropout_param" not in half.split("layer {")[0]
+
+
+def test_plan_of_the_inception_like_block():
+    rep = plan(S.inception_like(8), {"stem": (8, [29, 29])}, ["out"])
+    # pool1 feeds four layers: written once. Dropout and Absolute fuse; the Concat, Maxout and the pooling run on
+    # their own; the Dropout behind Maxout fuses into... nothing element-wise follows it before pool2, so it stands
+    # alone (and costs no launch when it runs in place); TanH follows pool2.
+    assert step_names(rep) == ["pool1", "b1_bn+b1_relu", "b2_drop+b2_abs", "b3_prelu", "join", "mo", "drop", "pool2", "out"]
+    assert rep["steps"][4]["inputs"] == ["b1_relu", "b2_abs", "b3_prelu", "pool1"]
+
+
+def test_neighbour_layer_configuration_rules():
+    # output sizes of max subsampling: (in + stride - window + (round_up ? window - 1 : 0)) / stride
+    for size, window, stride, up, want in [(112, 3, 2, False, 55), (112, 3, 2, True, 56), (7, 2, 2, False, 3), (7, 2, 2, True, 4), (5, 5, 1, False, 1)]:
+        layers = [S.L("Data", "x"), S.L("MaxSubsampling", "p", ["x"], windows=[window], strides=[stride], round_ups=[up])]
+        rep = plan(layers, {"x": (2, [size])}, ["p"])
+        # two feature maps in, two out, one buffer each
+        assert rep["per_entry_bytes"] == 2 * 4 * (size + want)
+    with pytest.raises(backend.BackendError, match="produces 0 output size"):
+        plan([S.L("Data", "x"), S.L("MaxSubsampling", "p", ["x"], windows=[5])], {"x": (2, [4])}, ["p"])
+    with pytest.raises(backend.BackendError, match="don't match"):
+        plan([S.L("Data", "x"), S.L("MaxSubsampling", "p", ["x"], windows=[2])], {"x": (2, [4, 4])}, ["p"])
+    with pytest.raises(backend.BackendError, match="hip backend does not support"):
+        plan([S.L("Data", "x"), S.L("MaxSubsampling", "p", ["x"], windows=[2], tiling=True)], {"x": (2, [8])}, ["p"])
+    with pytest.raises(backend.BackendError, match="stride dimension"):
+        plan([S.L("Data", "x"), S.L("MaxSubsampling", "p", ["x"], windows=[2], strides=[0])], {"x": (2, [8])}, ["p"])
+    with pytest.raises(backend.BackendError, match="not evenly divisible"):
+        plan([S.L("Data", "x"), S.L("Maxout", "m", ["x"], feature_map_subsampling_size=3)], {"x": (4, [8])}, ["m"])
+    with pytest.raises(backend.BackendError, match="should be >= 2"):
+        plan([S.L("Data", "x"), S.L("Maxout", "m", ["x"], feature_map_subsampling_size=1)], {"x": (4, [8])}, ["m"])
+    with pytest.raises(backend.BackendError, match="Neuron count per feature maps mismatch"):
+        plan([S.L("Data", "x"), S.L("Data", "y"), S.L("Concat", "c", ["x", "y"])], {"x": (4, [8]), "y": (4, [9])}, ["c"])
+    with pytest.raises(backend.BackendError, match="dropout_rate"):
+        plan([S.L("Data", "x"), S.L("Dropout", "d", ["x"], dropout_rate=1.0)], {"x": (4, [8])}, ["d"])

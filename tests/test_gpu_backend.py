@@ -160,3 +160,32 @@ def test_layer_in_place_on_a_data_layer_with_packets():
     values = S.evaluate(layers, {}, inputs)
     got, rep = run(layers, {}, inputs, ["act"], values, max_entry_count=7)
     assert_bits(got["act"], values["act"], "tanh in place over 8 packets")
+
+
+@pytest.mark.parametrize("fuse", [True, False])
+def test_inception_like_block_with_the_neighbouring_layers(fuse):
+    """MaxSubsampling (rounded up, overlapping), Dropout, Absolute, PReLU, Concat of four inputs, Maxout,
+    min pooling and TanH through the driver, in packets, against the oracle layer by layer."""
+    gen = T.rng(57, int(fuse))
+    c, n = 8, 21
+    layers = S.inception_like(c)
+    weights = S.make_weights(layers, gen)
+    inputs = {"stem": T.normal(gen, (n, c, 29, 29), 2.0)}
+    values = S.evaluate(layers, weights, inputs)
+    assert values["pool1"].shape == (n, c, 15, 15) and values["join"].shape == (n, 4 * c, 15, 15)
+    assert values["mo"].shape == (n, 2 * c, 15, 15) and values["out"].shape == (n, 2 * c, 7, 7)
+    got, rep = run(layers, weights, inputs, ["out", "join", "drop"], values, fuse=fuse, max_entry_count=8)
+    assert rep["entries"] == n
+    assert_bits(got["join"], values["join"], "concat")
+    assert_bits(got["drop"], values["drop"], "dropout behind maxout")
+    assert_bits(got["out"], values["out"], "output")
+
+
+def test_dropout_only_network():
+    """Dropout straight from the data layer to the output: in place there is nothing to launch."""
+    gen = T.rng(58, 0)
+    layers = [S.L("Data", "in"), S.L("Dropout", "d1", ["in"]), S.L("Dropout", "d2", ["d1"], dropout_rate=0.1)]
+    inputs = {"in": T.normal(gen, (9, 3, 5, 5))}
+    values = S.evaluate(layers, {}, inputs)
+    got, rep = run(layers, {}, inputs, ["d2"], values, max_entry_count=4)
+    assert_bits(got["d2"], inputs["in"], "dropout chain")
