@@ -236,6 +236,67 @@ def bench_resnet50(runner, steps, warmup, n=64):
     return entry
 
 
+def _u32(values):
+    return (ctypes.c_uint32 * len(values))(*values)
+
+
+def bench_max_subsampling(runner, steps, warmup, n=64, c=64, size=112):
+    """ResNet pool1: 3x3 windows every 2, rounded up (112x112 -> 56x56)."""
+    out_size = (size + 2 - 3 + 2) // 2
+    in_count, out_count = n * c * size * size, n * c * out_size * out_size
+    sets = rotation_sets(4 * (in_count + out_count))
+    ins = [runner.randn(in_count) for _ in range(sets)]
+    outs = [runner.empty(out_count) for _ in range(sets)]
+    dims, win, stride, up = _u32([size, size]), _u32([3, 3]), _u32([2, 2]), _u32([1, 1])
+    fn, stream = runner.lib.nnf_hip_max_subsampling_forward, runner.stream
+
+    def launch(i):
+        rc = fn(stream, outs[i % sets].data_ptr(), ins[i % sets].data_ptr(), n, c, 2, dims, win, stride, up, 1, 1, 0)
+        if rc != 0:
+            raise RuntimeError(runner.capi.error_string(rc))
+
+    wall, ev = runner.time_steps(launch, steps, warmup)
+    return result_entry("max_subsampling 3x3 stride 2 round up, N=%d C=%d %dx%d -> %dx%d" % (n, c, size, size, out_size, out_size),
+                        4 * (in_count + out_count), out_count, wall, ev, 1, {"buffer_sets": sets})
+
+
+def bench_concat(runner, steps, warmup, n=32, fms=(64, 128, 32, 32), plane=28 * 28):
+    counts = [c * plane for c in fms]
+    total = n * sum(counts)
+    sets = rotation_sets(8 * total)
+    ins = [[runner.randn(n * k) for k in counts] for _ in range(sets)]
+    outs = [runner.empty(total) for _ in range(sets)]
+    ptrs = [runner.capi.pointer_array([t.data_ptr() for t in group]) for group in ins]
+    lengths = _u32(counts)
+    fn, stream = runner.lib.nnf_hip_concat_forward, runner.stream
+
+    def launch(i):
+        rc = fn(stream, outs[i % sets].data_ptr(), ptrs[i % sets], lengths, len(counts), n)
+        if rc != 0:
+            raise RuntimeError(runner.capi.error_string(rc))
+
+    wall, ev = runner.time_steps(launch, steps, warmup)
+    return result_entry("concat of %s feature maps, N=%d 28x28" % ("+".join(str(c) for c in fms), n), 8 * total, total, wall, ev, 1,
+                        {"buffer_sets": sets})
+
+
+def bench_maxout(runner, steps, warmup, n=64, c_out=256, plane=14 * 14, k=2):
+    out_count = n * c_out * plane
+    sets = rotation_sets(4 * out_count * (k + 1))
+    ins = [runner.randn(out_count * k) for _ in range(sets)]
+    outs = [runner.empty(out_count) for _ in range(sets)]
+    fn, stream = runner.lib.nnf_hip_maxout_forward, runner.stream
+
+    def launch(i):
+        rc = fn(stream, outs[i % sets].data_ptr(), ins[i % sets].data_ptr(), n, c_out, plane, k)
+        if rc != 0:
+            raise RuntimeError(runner.capi.error_string(rc))
+
+    wall, ev = runner.time_steps(launch, steps, warmup)
+    return result_entry("maxout %d -> %d feature maps, N=%d 14x14" % (c_out * k, c_out, n), 4 * out_count * (k + 1), out_count, wall, ev, 1,
+                        {"buffer_sets": sets})
+
+
 def bench_copy(runner, steps, warmup):
     """Plain float4 copy kernel of the same launch shape: the yardstick for what HBM delivers."""
     count = (256 << 20) // 4
@@ -313,7 +374,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=400)
     ap.add_argument("--warmup", type=int, default=40)
-    ap.add_argument("--workload", default="config0", choices=["config0", "config1", "config2", "config3", "config4", "copy"],
+    ap.add_argument("--workload", default="config0", choices=["config0", "config1", "config2", "config3", "config4", "copy", "max_subsampling", "concat", "maxout"],
                     help="'copy' times the plain copy kernel (profiler-counter calibration and bandwidth yardstick)")
     ap.add_argument("--only", action="store_true", help="time only the chosen workload (no per_config survey, no CPU baseline)")
     args = ap.parse_args()
@@ -337,6 +398,12 @@ def main():
             return bench_group(runner, "config3: batch_norm -> exponential_linear -> sigmoid -> hyperbolic_tangent N=64 C=512 28x28", w.config3(), steps, warmup)
         if name == "copy":
             return bench_copy(runner, steps, warmup)
+        if name == "max_subsampling":
+            return bench_max_subsampling(runner, steps, warmup)
+        if name == "concat":
+            return bench_concat(runner, steps, warmup)
+        if name == "maxout":
+            return bench_maxout(runner, steps, warmup)
         return bench_resnet50(runner, steps, warmup)
 
     main_entry = run(args.workload, args.steps, args.warmup)
@@ -348,6 +415,10 @@ def main():
             if name not in per_config:
                 per_config[name] = run(name, *side_steps[name])
         per_config["copy_kernel"] = bench_copy(runner, 40, 5)
+        # the neighbouring layers of the same chains
+        for name, (k, wu) in (("max_subsampling", (40, 5)), ("concat", (100, 10)), ("maxout", (100, 10))):
+            if name not in per_config:
+                per_config[name] = run(name, k, wu)
         if args.workload == "config0":
             cpu = cpu_baseline_config0(runner, w.config0())
 
@@ -377,7 +448,8 @@ def main():
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBPS,
             "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
-            "kernel": {"config1": "nnf::softmax_rows_kernel", "copy": "nnf::copy_kernel_impl"}.get(args.workload, "nnf::chain_kernel"),
+            "kernel": {"config1": "nnf::softmax_rows_kernel", "copy": "nnf::copy_kernel_impl", "max_subsampling": "nnf::max_window2d_kernel",
+                       "concat": "nnf::concat_kernel", "maxout": "nnf::maxout_vec4_kernel"}.get(args.workload, "nnf::chain_kernel"),
             "algorithmic_bytes_per_launch": main_entry["algorithmic_bytes_per_step"] / launches,
             "avg_launch_us": main_entry["event_ms_per_step"] * 1e3 / launches,
         },

@@ -9,6 +9,7 @@
 #include "nnf_common.h"
 
 #include <algorithm>
+#include <cstdlib>
 
 namespace nnf
 {
@@ -60,7 +61,11 @@ namespace nnf
 			uint32_t band_magic;      // ceil(2^32 / (rows * out_w)): outputs per plane inside a workgroup
 		};
 
-		template<bool IS_MIN, int WIN_W, int WIN_H> // 0: read the size from the arguments
+		constexpr int stage_vectors_per_lane = 8; // float4 loads a lane has in flight while staging
+
+		// WIN_W, WIN_H: window size known at compile time, 0: read it from the arguments.
+		// TRUNC: windows may reach beyond the input (round up) and are cut off there.
+		template<bool IS_MIN, int WIN_W, int WIN_H, bool TRUNC>
 		__global__ void __launch_bounds__(max_block_size) max_window2d_kernel(const window2d_args a)
 		{
 			extern __shared__ __align__(16) float lds_in[];
@@ -72,35 +77,52 @@ namespace nnf
 			const uint32_t first_row = band * a.rows;
 			const uint32_t rows_here = min(a.rows, a.out_h - first_row);
 			const uint32_t in_plane = a.in_w * a.in_h;
+			const uint32_t win_w = (WIN_W > 0) ? WIN_W : a.win_w;
+			const uint32_t win_h = (WIN_H > 0) ? WIN_H : a.win_h;
 
 			// input rows [in_row0, in_row1) of planes [first_plane, first_plane + planes_here)
 			const uint32_t in_row0 = first_row * a.stride_y;
 			uint32_t in_row1 = a.in_h;
 			if (planes_here == 1)
-				in_row1 = min(a.in_h, (first_row + rows_here - 1) * a.stride_y + ((WIN_H > 0) ? WIN_H : a.win_h));
+				in_row1 = min(a.in_h, (first_row + rows_here - 1) * a.stride_y + win_h);
 			const uint32_t g0 = first_plane * in_plane + in_row0 * a.in_w;
 			const uint32_t g1 = (first_plane + planes_here - 1) * in_plane + in_row1 * a.in_w;
 			const uint32_t g0_aligned = g0 & ~3u;
 			const uint32_t shift = g0 - g0_aligned;
 			const uint32_t vectors = (g1 - g0_aligned + 3) / 4;
-			for(uint32_t i = threadIdx.x; i < vectors; i += max_block_size)
+			// all loads of a round are issued before the first one is stored to LDS
+			for(uint32_t base = 0; base < vectors; base += stage_vectors_per_lane * max_block_size)
 			{
-				const uint32_t g = g0_aligned + i * 4;
-				if (g + 4 <= a.total_in)
+				floatx4 t[stage_vectors_per_lane];
+				#pragma unroll
+				for(int k = 0; k < stage_vectors_per_lane; ++k)
 				{
-					const floatx4 t = load_stream(reinterpret_cast<const floatx4*>(a.in + g));
-					*reinterpret_cast<floatx4*>(lds_in + i * 4) = t;
+					const uint32_t i = base + k * max_block_size + threadIdx.x;
+					const uint32_t g = g0_aligned + i * 4;
+					if (i < vectors)
+					{
+						if (g + 4 <= a.total_in)
+							t[k] = load_stream(reinterpret_cast<const floatx4*>(a.in + g));
+						else
+						{
+							// the last, partial vector of the tensor
+							t[k].x = a.in[g];
+							t[k].y = (g + 1 < a.total_in) ? a.in[g + 1] : 0.0f;
+							t[k].z = (g + 2 < a.total_in) ? a.in[g + 2] : 0.0f;
+							t[k].w = 0.0f;
+						}
+					}
 				}
-				else
+				#pragma unroll
+				for(int k = 0; k < stage_vectors_per_lane; ++k)
 				{
-					for(uint32_t e = 0; (e < 4) && (g + e < a.total_in); ++e)
-						lds_in[i * 4 + e] = a.in[g + e];
+					const uint32_t i = base + k * max_block_size + threadIdx.x;
+					if (i < vectors)
+						*reinterpret_cast<floatx4*>(lds_in + i * 4) = t[k];
 				}
 			}
 			__syncthreads();
 
-			const uint32_t win_w = (WIN_W > 0) ? WIN_W : a.win_w;
-			const uint32_t win_h = (WIN_H > 0) ? WIN_H : a.win_h;
 			const uint32_t outputs_per_plane = rows_here * a.out_w;
 			const uint32_t outputs_here = planes_here * outputs_per_plane;
 			float* dst = a.out + (first_plane * a.out_h + first_row) * a.out_w;
@@ -113,26 +135,28 @@ namespace nnf
 				const uint32_t ox = r - oy * a.out_w;
 				const uint32_t x0 = ox * a.stride_x;
 				const uint32_t y0 = (first_row + oy) * a.stride_y;
-				// windows that reach beyond the input (round up) are cut off there
-				const uint32_t fit_w = min(win_w, a.in_w - x0);
-				const uint32_t fit_h = min(win_h, a.in_h - y0);
 				const float* src = lds_in + shift + p * in_plane + (y0 - in_row0) * a.in_w + x0;
+				// A window position beyond the input reads the last position inside instead. That value
+				// has been folded before (it precedes in scan order) and folding a value twice changes
+				// nothing, so this equals skipping the position.
+				const uint32_t last_x = TRUNC ? min(win_w, a.in_w - x0) - 1 : 0u;
+				const uint32_t last_y = TRUNC ? min(win_h, a.in_h - y0) - 1 : 0u;
 				float current = fold_start<IS_MIN>();
 				if ((WIN_W > 0) && (WIN_H > 0))
 				{
 					#pragma unroll
 					for(int y = 0; y < WIN_H; ++y)
 					{
+						const float* row = src + (TRUNC ? min(static_cast<uint32_t>(y), last_y) : static_cast<uint32_t>(y)) * a.in_w;
 						#pragma unroll
 						for(int x = 0; x < WIN_W; ++x)
-						{
-							if ((static_cast<uint32_t>(y) < fit_h) && (static_cast<uint32_t>(x) < fit_w))
-								current = fold<IS_MIN>(current, src[y * a.in_w + x]);
-						}
+							current = fold<IS_MIN>(current, row[TRUNC ? min(static_cast<uint32_t>(x), last_x) : static_cast<uint32_t>(x)]);
 					}
 				}
 				else
 				{
+					const uint32_t fit_w = TRUNC ? last_x + 1 : win_w;
+					const uint32_t fit_h = TRUNC ? last_y + 1 : win_h;
 					for(uint32_t y = 0; y < fit_h; ++y)
 						for(uint32_t x = 0; x < fit_w; ++x)
 							current = fold<IS_MIN>(current, src[y * a.in_w + x]);
@@ -251,15 +275,27 @@ namespace nnf
 			return (divisor >= 2) ? static_cast<uint32_t>(((1ull << 32) + divisor - 1) / divisor) : 0u; // fast_divide does not use it for 1
 		}
 
-		template<bool IS_MIN>
+		template<bool IS_MIN, bool TRUNC>
 		void launch_window2d(hipStream_t stream, const window2d_args& a, uint32_t grid, size_t lds_bytes)
 		{
 			if ((a.win_w == 3) && (a.win_h == 3))
-				hipLaunchKernelGGL((max_window2d_kernel<IS_MIN, 3, 3>), dim3(grid), dim3(max_block_size), lds_bytes, stream, a);
+				hipLaunchKernelGGL((max_window2d_kernel<IS_MIN, 3, 3, TRUNC>), dim3(grid), dim3(max_block_size), lds_bytes, stream, a);
 			else if ((a.win_w == 2) && (a.win_h == 2))
-				hipLaunchKernelGGL((max_window2d_kernel<IS_MIN, 2, 2>), dim3(grid), dim3(max_block_size), lds_bytes, stream, a);
+				hipLaunchKernelGGL((max_window2d_kernel<IS_MIN, 2, 2, TRUNC>), dim3(grid), dim3(max_block_size), lds_bytes, stream, a);
 			else
-				hipLaunchKernelGGL((max_window2d_kernel<IS_MIN, 0, 0>), dim3(grid), dim3(max_block_size), lds_bytes, stream, a);
+				hipLaunchKernelGGL((max_window2d_kernel<IS_MIN, 0, 0, TRUNC>), dim3(grid), dim3(max_block_size), lds_bytes, stream, a);
+		}
+
+		// LDS floats a workgroup of the 2-D kernel stages; NNF_HIP_POOL_LDS_FLOATS overrides it (tuning)
+		uint32_t staging_floats()
+		{
+			static const uint32_t value = []() -> uint32_t
+			{
+				const char* text = std::getenv("NNF_HIP_POOL_LDS_FLOATS");
+				const long v = (text != nullptr) ? std::atol(text) : 0;
+				return ((v >= 256) && (v <= 15 * 1024)) ? static_cast<uint32_t>(v) : 8u * 1024u;
+			}();
+			return value;
 		}
 	}
 
@@ -315,7 +351,7 @@ namespace nnf
 			return NNF_HIP_EOVERLAP;
 
 		// 2-D (or 1-D) windows within a feature map: stage through LDS
-		constexpr uint32_t lds_floats_wanted = 8 * 1024; // 32 KB: four workgroups per compute unit
+		const uint32_t lds_floats_wanted = staging_floats();
 		constexpr uint32_t lds_floats_max = 15 * 1024;
 		const bool within_plane = (feature_map_subsampling_size == 1) && (entry_subsampling_size == 1) && (dimension_count <= 2);
 		if (within_plane && (nd.out_size[0] * nd.out_size[1] < (1u << 16)))
@@ -362,9 +398,15 @@ namespace nnf
 				const size_t lds_bytes = (static_cast<size_t>(a.planes - 1) * plane + static_cast<size_t>(rows_in) * a.in_w + 8) * sizeof(float);
 				const uint32_t grid = ((a.plane_count + a.planes - 1) / a.planes) * a.bands;
 				if (is_min)
-					launch_window2d<true>(stream, a, grid, lds_bytes);
+				{
+					if (round_up_anywhere) launch_window2d<true, true>(stream, a, grid, lds_bytes);
+					else launch_window2d<true, false>(stream, a, grid, lds_bytes);
+				}
 				else
-					launch_window2d<false>(stream, a, grid, lds_bytes);
+				{
+					if (round_up_anywhere) launch_window2d<false, true>(stream, a, grid, lds_bytes);
+					else launch_window2d<false, false>(stream, a, grid, lds_bytes);
+				}
 				return launch_status();
 			}
 		}
