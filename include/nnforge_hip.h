@@ -176,6 +176,33 @@ NNF_HIP_API int nnf_hip_max_subsampling_forward(void* stream, float* output, con
 	const uint32_t* input_sizes, const uint32_t* subsampling_sizes, const uint32_t* strides, const uint32_t* round_ups,
 	uint32_t feature_map_subsampling_size, uint32_t entry_subsampling_size, int32_t is_min);
 
+/* Per-feature-map running statistics on the device: the state stat_data_bunch_writer keeps per
+ * feature map (nnforge/stat_data_bunch_writer.h:45-63) and fills on the host from outputs copied
+ * back (nnforge/stat_data_bunch_writer.cpp:45-79). average = (float)mean and
+ * std_dev = sqrtf((float)(m2 / n)) as in nnforge/stat_data_bunch_writer.cpp:97-98. The reference
+ * updates the state one value at a time; the device reduces runs of entries and merges them in a
+ * fixed order, all in double precision: mean and m2 agree with the sequential update to double
+ * rounding (at most one fp32 unit in the last place after the conversion), min and max compare
+ * equal. Used to refresh batch norm weights (nnforge/toolset.cpp:1562-1630). */
+typedef struct nnf_hip_running_stat
+{
+	double n;
+	double mean;
+	double m2;       /* sum of squared deviations from the mean */
+	float min_val;
+	float max_val;
+} nnf_hip_running_stat;
+
+/* n = 0, mean = 0, m2 = 0, min = FLT_MAX, max = -FLT_MAX for feature_map_count states (device memory) */
+NNF_HIP_API int nnf_hip_feature_map_stat_init(void* stream, nnf_hip_running_stat* device_stats, uint32_t feature_map_count);
+/* device workspace one accumulate call of up to entry_count entries needs */
+NNF_HIP_API int nnf_hip_feature_map_stat_workspace_bytes(uint32_t entry_count, uint32_t feature_map_count,
+	uint32_t neuron_count_per_feature_map, size_t* bytes);
+/* folds entry_count entries of input ([entry][feature_map][neurons]) into device_stats */
+NNF_HIP_API int nnf_hip_feature_map_stat_accumulate(void* stream, nnf_hip_running_stat* device_stats,
+	void* device_workspace, size_t workspace_bytes, const float* input,
+	uint32_t entry_count, uint32_t feature_map_count, uint32_t neuron_count_per_feature_map);
+
 /* ---- runtime plumbing, so that host C++ above this ABI needs no HIP headers --------------------
  * Counterparts in the reference: cuda_linear_buffer_device (nnforge/cuda/cuda_linear_buffer_device.cpp:28-45),
  * cuda_stream / cuda_event (nnforge/cuda/cuda_stream.cpp, cuda_event.cpp), cuda_safe_call

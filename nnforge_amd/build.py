@@ -9,7 +9,7 @@ REPO_ROOT = os.path.dirname(PACKAGE_DIR)
 CSRC_DIR = os.path.join(PACKAGE_DIR, "csrc")
 
 HIP_LIBRARY = os.path.join(PACKAGE_DIR, "libnnforge_hip.so")
-HIP_SOURCES = ["nnf_chain.hip", "nnf_softmax.hip", "nnf_pool.hip", "nnf_max.hip", "nnf_concat.hip", "nnf_capi.hip"]
+HIP_SOURCES = ["nnf_chain.hip", "nnf_softmax.hip", "nnf_pool.hip", "nnf_max.hip", "nnf_concat.hip", "nnf_stat.hip", "nnf_capi.hip"]
 
 # -ffp-contract=off: every fp32 operation of the layer formulas rounds once, as the reference's
 #   source states them. -packed-fp32-ops is switched off as a target feature (hipcc only).

@@ -177,6 +177,23 @@ extern "C"
 			dimension_count, input_sizes, subsampling_sizes, strides, round_ups, feature_map_subsampling_size, entry_subsampling_size, is_min);
 	}
 
+	int nnf_hip_feature_map_stat_init(void* stream, nnf_hip_running_stat* device_stats, uint32_t feature_map_count)
+	{
+		return feature_map_stat_init(static_cast<hipStream_t>(stream), device_stats, feature_map_count);
+	}
+
+	int nnf_hip_feature_map_stat_workspace_bytes(uint32_t entry_count, uint32_t feature_map_count, uint32_t neuron_count_per_feature_map, size_t* bytes)
+	{
+		return feature_map_stat_workspace_bytes(entry_count, feature_map_count, neuron_count_per_feature_map, bytes);
+	}
+
+	int nnf_hip_feature_map_stat_accumulate(void* stream, nnf_hip_running_stat* device_stats, void* device_workspace, size_t workspace_bytes,
+		const float* input, uint32_t entry_count, uint32_t feature_map_count, uint32_t neuron_count_per_feature_map)
+	{
+		return feature_map_stat_accumulate(static_cast<hipStream_t>(stream), device_stats, device_workspace, workspace_bytes, input,
+			entry_count, feature_map_count, neuron_count_per_feature_map);
+	}
+
 	int nnf_hip_add_forward(void* stream, float* output, const float* const* inputs, uint32_t input_count, float alpha, uint64_t elem_count)
 	{
 		if ((inputs == nullptr) || (input_count == 0) || (output == nullptr))

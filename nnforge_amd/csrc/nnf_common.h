@@ -81,5 +81,9 @@ namespace nnf
 		uint32_t output_entry_count, uint32_t input_feature_map_count, uint32_t dimension_count,
 		const uint32_t* input_sizes, const uint32_t* subsampling_sizes, const uint32_t* strides, const uint32_t* round_ups,
 		uint32_t feature_map_subsampling_size, uint32_t entry_subsampling_size, int32_t is_min);
+	int feature_map_stat_init(hipStream_t stream, nnf_hip_running_stat* device_stats, uint32_t feature_map_count);
+	int feature_map_stat_workspace_bytes(uint32_t entry_count, uint32_t feature_map_count, uint32_t neuron_count_per_feature_map, size_t* bytes);
+	int feature_map_stat_accumulate(hipStream_t stream, nnf_hip_running_stat* device_stats, void* workspace, size_t workspace_bytes,
+		const float* input, uint32_t entry_count, uint32_t feature_map_count, uint32_t neuron_count_per_feature_map);
 	int copy_kernel(hipStream_t stream, void* dst, const void* src, size_t bytes);
 }

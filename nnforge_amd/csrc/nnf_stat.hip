@@ -1,0 +1,246 @@
+// Per-feature-map statistics of a tensor on the device: count, mean, sum of squared deviations
+// (double precision), minimum and maximum - the running state of nnForge's stat_data_bunch_writer
+// (nnforge/stat_data_bunch_writer.cpp:45-79), which the reference fills on the host, one value at
+// a time, from outputs copied back entry by entry.
+//
+// The reference's update is sequential (Welford). Here every workgroup reduces a run of entries of
+// one feature map to (n, mean, m2) and the runs are merged in a fixed order with the pairwise
+// update of Chan et al., also in double precision; the result does not depend on scheduling.
+// Inside a workgroup the sums are taken of (x - pivot), the pivot being the run's first value, so
+// that a mean far from zero does not cancel the deviation. mean and m2 agree with the sequential
+// update to a few units of double rounding; after the reference's conversion to fp32 that is
+// at most one unit in the last place. Minimum and maximum use the reference's comparisons
+// (NaN never enters); which of +0.0 / -0.0 is reported when both occur is not defined here.
+#include "nnf_common.h"
+
+#include <algorithm>
+
+namespace nnf
+{
+	namespace
+	{
+		constexpr int stat_block_size = 256;
+		constexpr int stat_unroll = 4;                    // loads a lane has in flight
+		constexpr uint32_t stat_floats_per_block = 32768; // a run is about this long ...
+		constexpr uint32_t stat_blocks_wanted = 2048;     // ... unless that leaves the grid this narrow
+
+		struct stat_plan
+		{
+			uint32_t entries_per_run;
+			uint32_t runs;
+		};
+
+		stat_plan plan_runs(uint32_t entry_count, uint32_t feature_map_count, uint32_t plane)
+		{
+			stat_plan p;
+			const uint32_t by_size = std::max(1u, stat_floats_per_block / plane);
+			const uint32_t runs_wanted = std::max(1u, std::min(entry_count, (stat_blocks_wanted + feature_map_count - 1) / feature_map_count));
+			const uint32_t by_grid = (entry_count + runs_wanted - 1) / runs_wanted;
+			p.entries_per_run = std::max(1u, std::min(by_size, by_grid));
+			// the kernel divides flat indices by the plane size with a multiplication, exact while
+			// index * divisor < 2^32; a run of one entry needs no division
+			const uint64_t units = ((plane % 4) == 0) ? plane / 4 : plane;
+			if (static_cast<uint64_t>(p.entries_per_run) * units * units >= (1ull << 32))
+				p.entries_per_run = 1;
+			p.runs = (entry_count + p.entries_per_run - 1) / p.entries_per_run;
+			return p;
+		}
+
+		__device__ __forceinline__ void accumulate(float v, double pivot, double& s1, double& s2, float& mn, float& mx)
+		{
+			const double d = static_cast<double>(v) - pivot;
+			s1 += d;
+			s2 = fma(d, d, s2);
+			mn = (v < mn) ? v : mn; // std::min(current, val)
+			mx = (mx < v) ? v : mx; // std::max(current, val)
+		}
+
+		// grid: (runs, feature maps). VEC: floats per load (4 when plane is a multiple of 4).
+		template<int VEC>
+		__global__ void __launch_bounds__(stat_block_size) stat_runs_kernel(
+			nnf_hip_running_stat* partial, const float* in, uint32_t entry_count, uint32_t feature_map_count, uint32_t plane,
+			uint32_t entries_per_run, uint32_t unit_magic)
+		{
+			typedef float vec_t __attribute__((ext_vector_type(VEC)));
+			__shared__ double lds_s1[stat_block_size / wave_size], lds_s2[stat_block_size / wave_size];
+			__shared__ float lds_mn[stat_block_size / wave_size], lds_mx[stat_block_size / wave_size];
+
+			const uint32_t run = blockIdx.x, fm = blockIdx.y;
+			const uint32_t e0 = run * entries_per_run;
+			const uint32_t entries_here = min(entries_per_run, entry_count - e0);
+			const uint32_t units_per_plane = plane / VEC;
+			const uint32_t units = entries_here * units_per_plane;
+			const size_t entry_stride = static_cast<size_t>(feature_map_count) * plane;
+			const float* base = in + (static_cast<size_t>(e0) * feature_map_count + fm) * plane;
+			const double pivot = static_cast<double>(base[0]);
+
+			double s1 = 0.0, s2 = 0.0;
+			float mn = 3.402823466e+38f, mx = -3.402823466e+38f;
+			for(uint32_t first = 0; first < units; first += stat_block_size * stat_unroll)
+			{
+				vec_t v[stat_unroll];
+				#pragma unroll
+				for(int k = 0; k < stat_unroll; ++k)
+				{
+					const uint32_t t = first + k * stat_block_size + threadIdx.x;
+					if (t < units)
+					{
+						const uint32_t e = (entries_here == 1) ? 0u : ((units_per_plane == 1) ? t : __umulhi(t, unit_magic));
+						const uint32_t i = t - e * units_per_plane;
+						v[k] = __builtin_nontemporal_load(reinterpret_cast<const vec_t*>(base + e * entry_stride + static_cast<size_t>(i) * VEC));
+					}
+				}
+				#pragma unroll
+				for(int k = 0; k < stat_unroll; ++k)
+				{
+					const uint32_t t = first + k * stat_block_size + threadIdx.x;
+					if (t < units)
+					{
+						#pragma unroll
+						for(int c = 0; c < VEC; ++c)
+							accumulate(v[k][c], pivot, s1, s2, mn, mx);
+					}
+				}
+			}
+
+			// wavefront, then workgroup
+			#pragma unroll
+			for(int offset = wave_size / 2; offset > 0; offset /= 2)
+			{
+				s1 += __shfl_xor(s1, offset);
+				s2 += __shfl_xor(s2, offset);
+				const float other_mn = __shfl_xor(mn, offset), other_mx = __shfl_xor(mx, offset);
+				mn = (other_mn < mn) ? other_mn : mn;
+				mx = (mx < other_mx) ? other_mx : mx;
+			}
+			const uint32_t wave = threadIdx.x / wave_size;
+			if ((threadIdx.x % wave_size) == 0)
+			{
+				lds_s1[wave] = s1; lds_s2[wave] = s2; lds_mn[wave] = mn; lds_mx[wave] = mx;
+			}
+			__syncthreads();
+			if (threadIdx.x == 0)
+			{
+				for(uint32_t w = 1; w < stat_block_size / wave_size; ++w)
+				{
+					s1 += lds_s1[w];
+					s2 += lds_s2[w];
+					mn = (lds_mn[w] < mn) ? lds_mn[w] : mn;
+					mx = (mx < lds_mx[w]) ? lds_mx[w] : mx;
+				}
+				const double n = static_cast<double>(entries_here) * static_cast<double>(plane);
+				nnf_hip_running_stat r;
+				r.n = n;
+				r.mean = pivot + s1 / n;
+				const double m2 = s2 - s1 * s1 / n;
+				r.m2 = (m2 < 0.0) ? 0.0 : m2; // rounding may leave a tiny negative value where the deviation is zero
+				r.min_val = mn;
+				r.max_val = mx;
+				partial[static_cast<size_t>(run) * feature_map_count + fm] = r;
+			}
+		}
+
+		// One lane per feature map folds the runs into the running state, run 0 first.
+		__global__ void __launch_bounds__(stat_block_size) stat_merge_kernel(
+			nnf_hip_running_stat* state, const nnf_hip_running_stat* partial, uint32_t feature_map_count, uint32_t runs)
+		{
+			const uint32_t fm = blockIdx.x * stat_block_size + threadIdx.x;
+			if (fm >= feature_map_count)
+				return;
+			nnf_hip_running_stat s = state[fm];
+			for(uint32_t run = 0; run < runs; ++run)
+			{
+				const nnf_hip_running_stat b = partial[static_cast<size_t>(run) * feature_map_count + fm];
+				const double n = s.n + b.n;
+				const double delta = b.mean - s.mean;
+				if (s.n == 0.0)
+					s.mean = b.mean;
+				else
+					s.mean = s.mean + delta * (b.n / n);
+				s.m2 = s.m2 + b.m2 + delta * delta * (s.n * b.n / n);
+				s.n = n;
+				s.min_val = (b.min_val < s.min_val) ? b.min_val : s.min_val;
+				s.max_val = (s.max_val < b.max_val) ? b.max_val : s.max_val;
+			}
+			state[fm] = s;
+		}
+
+		__global__ void __launch_bounds__(stat_block_size) stat_init_kernel(nnf_hip_running_stat* state, uint32_t feature_map_count)
+		{
+			const uint32_t fm = blockIdx.x * stat_block_size + threadIdx.x;
+			if (fm >= feature_map_count)
+				return;
+			// nnforge/stat_data_bunch_writer.h:48-55
+			nnf_hip_running_stat s;
+			s.n = 0.0;
+			s.mean = 0.0;
+			s.m2 = 0.0;
+			s.min_val = 3.402823466e+38f;
+			s.max_val = -3.402823466e+38f;
+			state[fm] = s;
+		}
+	}
+
+	int feature_map_stat_init(hipStream_t stream, nnf_hip_running_stat* device_stats, uint32_t feature_map_count)
+	{
+		if ((device_stats == nullptr) || (feature_map_count == 0))
+			return NNF_HIP_EINVAL;
+		if (!is_aligned16(device_stats))
+			return NNF_HIP_EALIGN;
+		hipLaunchKernelGGL(stat_init_kernel, dim3((feature_map_count + stat_block_size - 1) / stat_block_size), dim3(stat_block_size), 0, stream,
+			device_stats, feature_map_count);
+		return launch_status();
+	}
+
+	int feature_map_stat_workspace_bytes(uint32_t entry_count, uint32_t feature_map_count, uint32_t neuron_count_per_feature_map, size_t* bytes)
+	{
+		if ((bytes == nullptr) || (feature_map_count == 0) || (neuron_count_per_feature_map == 0))
+			return NNF_HIP_EINVAL;
+		const stat_plan p = plan_runs(std::max(1u, entry_count), feature_map_count, neuron_count_per_feature_map);
+		*bytes = static_cast<size_t>(p.runs) * feature_map_count * sizeof(nnf_hip_running_stat);
+		return NNF_HIP_OK;
+	}
+
+	int feature_map_stat_accumulate(hipStream_t stream, nnf_hip_running_stat* device_stats, void* workspace, size_t workspace_bytes,
+		const float* input, uint32_t entry_count, uint32_t feature_map_count, uint32_t neuron_count_per_feature_map)
+	{
+		if ((device_stats == nullptr) || (feature_map_count == 0) || (neuron_count_per_feature_map == 0))
+			return NNF_HIP_EINVAL;
+		if (entry_count == 0)
+			return NNF_HIP_OK; // nothing to fold in
+		if (input == nullptr)
+			return NNF_HIP_EINVAL;
+		if (!is_aligned16(device_stats) || !is_aligned16(input) || !is_aligned16(workspace))
+			return NNF_HIP_EALIGN;
+		const uint64_t total = static_cast<uint64_t>(entry_count) * feature_map_count * neuron_count_per_feature_map;
+		if ((total > 0xFFFF0000ull) || (feature_map_count > 65535u))
+			return NNF_HIP_ETOOBIG;
+		const stat_plan p = plan_runs(entry_count, feature_map_count, neuron_count_per_feature_map);
+		const size_t needed = static_cast<size_t>(p.runs) * feature_map_count * sizeof(nnf_hip_running_stat);
+		if ((workspace == nullptr) || (workspace_bytes < needed))
+			return NNF_HIP_EINVAL;
+
+		nnf_hip_running_stat* partial = static_cast<nnf_hip_running_stat*>(workspace);
+		const dim3 grid(p.runs, feature_map_count);
+		if ((neuron_count_per_feature_map % 4) == 0)
+		{
+			const uint32_t units = neuron_count_per_feature_map / 4;
+			const uint32_t magic = (units >= 2) ? static_cast<uint32_t>(((1ull << 32) + units - 1) / units) : 0u;
+			hipLaunchKernelGGL(stat_runs_kernel<4>, grid, dim3(stat_block_size), 0, stream, partial, input, entry_count, feature_map_count,
+				neuron_count_per_feature_map, p.entries_per_run, magic);
+		}
+		else
+		{
+			const uint32_t units = neuron_count_per_feature_map;
+			const uint32_t magic = (units >= 2) ? static_cast<uint32_t>(((1ull << 32) + units - 1) / units) : 0u;
+			hipLaunchKernelGGL(stat_runs_kernel<1>, grid, dim3(stat_block_size), 0, stream, partial, input, entry_count, feature_map_count,
+				neuron_count_per_feature_map, p.entries_per_run, magic);
+		}
+		int status = launch_status();
+		if (status != NNF_HIP_OK)
+			return status;
+		hipLaunchKernelGGL(stat_merge_kernel, dim3((feature_map_count + stat_block_size - 1) / stat_block_size), dim3(stat_block_size), 0, stream,
+			device_stats, partial, feature_map_count, p.runs);
+		return launch_status();
+	}
+}

@@ -58,6 +58,10 @@ def load():
                                                    ctypes.c_int]
         lib.nnf_oracle_max_subsampling_tiling.argtypes = [_FP, _FP, ctypes.c_uint, ctypes.c_uint, ctypes.c_int, _UP, _UP, _UP,
                                                           ctypes.c_int, ctypes.c_int]
+        lib.nnf_oracle_feature_map_stat_init.argtypes = [ctypes.c_void_p, ctypes.c_uint]
+        lib.nnf_oracle_feature_map_stat_write.argtypes = [ctypes.c_void_p, _FP, ctypes.c_uint, ctypes.c_uint, ctypes.c_uint, ctypes.c_int]
+        lib.nnf_oracle_feature_map_stat_get.argtypes = [ctypes.c_void_p, ctypes.c_uint, _FP, _FP, _FP, _FP]
+        lib.nnf_oracle_update_bn_weights.argtypes = [_FP, _FP, _FP, _FP, ctypes.c_uint]
         _lib = lib
     return _lib
 
@@ -255,3 +259,42 @@ def max_subsampling(x, window_sizes, strides=None, round_ups=None, feature_map_w
                                       arr(window_sizes), arr(strides), feature_map_window, entry_window, int(is_min), truncate,
                                       threads)
     return out
+
+
+class RunningStat(ctypes.Structure):
+    """nnforge/stat_data_bunch_writer.h:45-63"""
+    _fields_ = [("n", ctypes.c_double), ("mean", ctypes.c_double), ("m2", ctypes.c_double),
+                ("min_val", ctypes.c_float), ("max_val", ctypes.c_float)]
+
+
+STAT_DTYPE = np.dtype([("n", "<f8"), ("mean", "<f8"), ("m2", "<f8"), ("min_val", "<f4"), ("max_val", "<f4")])
+
+
+class FeatureMapStat:
+    """stat_data_bunch_writer for one layer: write() batches of entries, then get()."""
+
+    def __init__(self, feature_map_count):
+        self.state = np.zeros(feature_map_count, dtype=STAT_DTYPE)
+        load().nnf_oracle_feature_map_stat_init(self.state.ctypes.data_as(ctypes.c_void_p), feature_map_count)
+
+    def write(self, x, threads=0):
+        x = _f32(x)
+        n, c, plane = _shape3(x)
+        assert c == self.state.size
+        load().nnf_oracle_feature_map_stat_write(self.state.ctypes.data_as(ctypes.c_void_p), _ptr(x), n, c, plane, threads)
+        return self
+
+    def get(self):
+        """{'min', 'max', 'average', 'std_dev'}: float32 arrays per feature map"""
+        c = self.state.size
+        res = {k: np.empty(c, dtype=np.float32) for k in ("min", "max", "average", "std_dev")}
+        load().nnf_oracle_feature_map_stat_get(self.state.ctypes.data_as(ctypes.c_void_p), c, _ptr(res["min"]), _ptr(res["max"]),
+                                               _ptr(res["average"]), _ptr(res["std_dev"]))
+        return res
+
+
+def update_bn_weights(mean, inverse_sigma, average, std_dev):
+    """Returns the refreshed (mean, inverse_sigma)."""
+    m, s = _f32(mean).copy(), _f32(inverse_sigma).copy()
+    load().nnf_oracle_update_bn_weights(_ptr(m), _ptr(s), _ptr(_f32(average)), _ptr(_f32(std_dev)), m.size)
+    return m, s

@@ -616,3 +616,98 @@ NNF_ORACLE_API void nnf_oracle_max_subsampling_tiling(float* out, const float* i
 	}
 	free(offsets);
 }
+
+/* ---- per-feature-map statistics and the batch norm refresh built on them ------------------- */
+
+/* nnforge/stat_data_bunch_writer.h:45-63: the running state of one feature map */
+typedef struct nnf_oracle_running_stat
+{
+	double n;
+	double mean;
+	double m2;
+	float min_val;
+	float max_val;
+} nnf_oracle_running_stat;
+
+NNF_ORACLE_API void nnf_oracle_feature_map_stat_init(nnf_oracle_running_stat* stats, unsigned int feature_map_count)
+{
+	unsigned int f;
+	for (f = 0; f < feature_map_count; ++f)
+	{
+		stats[f].n = 0.0;
+		stats[f].mean = 0.0;
+		stats[f].m2 = 0.0;
+		stats[f].min_val = 3.402823466e+38F;  /* std::numeric_limits<float>::max() */
+		stats[f].max_val = -3.402823466e+38F;
+	}
+}
+
+/*
+ * nnforge/stat_data_bunch_writer.cpp:45-79, for entry_count entries one after the other: every value
+ * of a feature map, in memory order, updates min (std::min(current, val)), max (std::max(current, val))
+ * and the single-pass mean / sum of squared deviations in double precision. Feature maps do not
+ * interact, so they run in parallel here; each one sees its values in the reference's order.
+ */
+NNF_ORACLE_API void nnf_oracle_feature_map_stat_write(nnf_oracle_running_stat* stats, const float* data,
+	unsigned int entry_count, unsigned int feature_map_count, unsigned int plane, int threads)
+{
+	int f;
+	#pragma omp parallel for schedule(guided) num_threads(thread_count(threads))
+	for (f = 0; f < (int)feature_map_count; ++f)
+	{
+		nnf_oracle_running_stat s = stats[f];
+		unsigned int e, i;
+		for (e = 0; e < entry_count; ++e)
+		{
+			const float* src = data + ((size_t)e * feature_map_count + (size_t)f) * plane;
+			for (i = 0; i < plane; ++i)
+			{
+				const float val = src[i];
+				double val_d, delta, delta2;
+				s.min_val = std_min(s.min_val, val);
+				s.max_val = std_max(s.max_val, val);
+				s.n += 1.0;
+				val_d = (double)val;
+				delta = val_d - s.mean;
+				s.mean += delta / s.n;
+				delta2 = val_d - s.mean;
+				s.m2 += delta * delta2;
+			}
+		}
+		stats[f] = s;
+	}
+}
+
+/* nnforge/stat_data_bunch_writer.cpp:92-106: average = (float)mean, std_dev = sqrtf((float)(m2 / n)) */
+NNF_ORACLE_API void nnf_oracle_feature_map_stat_get(const nnf_oracle_running_stat* stats, unsigned int feature_map_count,
+	float* min_val, float* max_val, float* average, float* std_dev)
+{
+	unsigned int f;
+	for (f = 0; f < feature_map_count; ++f)
+	{
+		average[f] = (float)stats[f].mean;
+		std_dev[f] = sqrtf((float)(stats[f].m2 / stats[f].n));
+		min_val[f] = stats[f].min_val;
+		max_val[f] = stats[f].max_val;
+	}
+}
+
+/*
+ * nnforge/toolset.cpp:1608-1617: the statistics were taken on the layer's output with gamma 1 and
+ * beta 0, i.e. on (x - mean) * inv_sigma; the new weights make that output have mean 0 and
+ * deviation 1:  inv_sigma' = inv_sigma / std_dev,  mean' = mean + average / inv_sigma  (fp32).
+ */
+NNF_ORACLE_API void nnf_oracle_update_bn_weights(float* mean, float* inverse_sigma, const float* average, const float* std_dev,
+	unsigned int feature_map_count)
+{
+	unsigned int f;
+	for (f = 0; f < feature_map_count; ++f)
+	{
+		const float old_mean = mean[f];
+		const float old_invsigma = inverse_sigma[f];
+		const float new_invsigma = old_invsigma / std_dev[f];
+		const float new_mean = old_mean + average[f] / old_invsigma;
+		mean[f] = new_mean;
+		inverse_sigma[f] = new_invsigma;
+	}
+}

@@ -417,3 +417,72 @@ def test_max_subsampling_tiling_brute_force():
                         for ox in range(ow):
                             win = x[e, f, oy * wy + sy: oy * wy + sy + wy, ox * wx + sx: ox * wx + sx + wx]
                             assert got[e * wx * wy + j, f, oy, ox] == win.max()
+
+
+# ---- per-feature-map statistics and the batch norm refresh ---------------------------------------
+
+def test_feature_map_stat_against_two_pass_fp64():
+    gen = T.rng(44, 0)
+    n, c, h, w = 7, 5, 6, 9
+    x = (T.normal(gen, (n, c, h, w), 2.0) + np.arange(c, dtype=F)[None, :, None, None] * F(10.0)).astype(F)
+    stat = oracle.FeatureMapStat(c).write(x)
+    per_fm = x.transpose(1, 0, 2, 3).reshape(c, -1).astype(np.float64)
+    st = stat.state
+    assert np.all(st["n"] == n * h * w)
+    assert np.allclose(st["mean"], per_fm.mean(axis=1), rtol=1e-13, atol=0)
+    assert np.allclose(st["m2"], ((per_fm - per_fm.mean(axis=1, keepdims=True)) ** 2).sum(axis=1), rtol=1e-12, atol=0)
+    got = stat.get()
+    assert np.array_equal(got["min"], per_fm.min(axis=1).astype(F)) and np.array_equal(got["max"], per_fm.max(axis=1).astype(F))
+    assert T.ulp_distance(got["average"], per_fm.mean(axis=1).astype(F)).max() <= 1
+    # population deviation (divides by n, not n - 1), rounded to fp32 BEFORE the square root
+    want_std = np.sqrt(per_fm.var(axis=1).astype(F))
+    assert T.ulp_distance(got["std_dev"], want_std).max() <= 1
+    assert not np.allclose(got["std_dev"], per_fm.std(axis=1, ddof=1), rtol=1e-4, atol=0)
+    # feature map f of entry e is x[e, f]: a transposed layout would mix the shifted means
+    assert np.all(np.abs(got["average"] - np.arange(c) * 10.0) < 1.0)
+
+
+def test_feature_map_stat_is_sequential_and_stable():
+    gen = T.rng(44, 1)
+    x = T.normal(gen, (12, 3, 50))
+    whole = oracle.FeatureMapStat(3).write(x)
+    parts = oracle.FeatureMapStat(3).write(x[:5]).write(x[5:6]).write(x[6:])
+    assert whole.state.tobytes() == parts.state.tobytes()     # packets do not change the result
+    # a large offset with a small spread: the single-pass update keeps the deviation
+    y = (F(1000.0) + T.normal(gen, (64, 2, 100), 0.01)).astype(F)
+    st = oracle.FeatureMapStat(2).write(y).get()
+    per_fm = y.transpose(1, 0, 2).reshape(2, -1).astype(np.float64)
+    assert np.allclose(st["std_dev"], per_fm.std(axis=1), rtol=1e-6, atol=0)
+    # one value: deviation 0; no value: 0/0
+    one = oracle.FeatureMapStat(1).write(np.full((1, 1, 1), 3.5, F)).get()
+    assert one["average"][0] == F(3.5) and one["std_dev"][0] == 0.0 and one["min"][0] == F(3.5) and one["max"][0] == F(3.5)
+    with np.errstate(all="ignore"):
+        empty = oracle.FeatureMapStat(1).get()
+    assert np.isnan(empty["std_dev"][0]) and empty["min"][0] == np.finfo(F).max and empty["max"][0] == -np.finfo(F).max
+
+
+def test_feature_map_stat_min_max_follow_std_min_max():
+    x = np.array([[[np.nan, 2.0, -0.0, 0.0, -7.0, np.nan]]], F)
+    st = oracle.FeatureMapStat(1).write(x)
+    got = st.get()
+    assert got["min"][0] == F(-7.0) and got["max"][0] == F(2.0)     # NaN never enters min / max ...
+    assert np.isnan(got["average"][0])                               # ... but poisons the mean
+    zeros = oracle.FeatureMapStat(1).write(np.array([[[-0.0, 0.0]]], F)).get()
+    assert np.signbit(zeros["min"][0]) and np.signbit(zeros["max"][0])   # the first of equal values stays
+
+
+def test_update_bn_weights_formula_and_effect():
+    gen = T.rng(44, 2)
+    c = 6
+    _, _, mean, inv_sigma = T.bn_params(gen, c)
+    average, std_dev = T.normal(gen, (c,), 0.3), T.uniform(gen, c, 0.5, 2.0)
+    new_mean, new_inv = oracle.update_bn_weights(mean, inv_sigma, average, std_dev)
+    assert bits_equal(new_inv, (inv_sigma / std_dev).astype(F))
+    assert bits_equal(new_mean, (mean + (average / inv_sigma).astype(F)).astype(F))
+    # closed loop: statistics of the output with gamma 1, beta 0 -> refreshed weights -> mean 0, deviation 1
+    x = (T.normal(gen, (40, c, 64), 3.0) + F(5.0)).astype(F)
+    ones, zeros = np.ones(c, F), np.zeros(c, F)
+    st = oracle.FeatureMapStat(c).write(oracle.batch_norm(x, ones, zeros, mean, inv_sigma)).get()
+    m2, s2 = oracle.update_bn_weights(mean, inv_sigma, st["average"], st["std_dev"])
+    after = oracle.FeatureMapStat(c).write(oracle.batch_norm(x, ones, zeros, m2, s2)).get()
+    assert np.abs(after["average"]).max() < 1e-5 and np.abs(after["std_dev"] - 1.0).max() < 1e-5
