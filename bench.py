@@ -297,6 +297,28 @@ def bench_maxout(runner, steps, warmup, n=64, c_out=256, plane=14 * 14, k=2):
                         {"buffer_sets": sets})
 
 
+def bench_feature_map_stat(runner, steps, warmup, n=128, c=256, plane=56 * 56):
+    """Per-feature-map statistics of a batch norm input of config 2's shape: read once, 32 bytes per feature map written."""
+    total = n * c * plane
+    sets = rotation_sets(4 * total, cap=4)
+    ins = [runner.randn(total) for _ in range(sets)]
+    state = runner.torch.zeros(c * 32, dtype=runner.torch.uint8, device=runner.device)
+    need = ctypes.c_size_t()
+    runner.capi.check(runner.lib.nnf_hip_feature_map_stat_workspace_bytes(n, c, plane, ctypes.byref(need)))
+    work = runner.torch.empty(max(16, need.value), dtype=runner.torch.uint8, device=runner.device)
+    runner.capi.check(runner.lib.nnf_hip_feature_map_stat_init(runner.stream, state.data_ptr(), c))
+    fn, stream = runner.lib.nnf_hip_feature_map_stat_accumulate, runner.stream
+
+    def launch(i):
+        rc = fn(stream, state.data_ptr(), work.data_ptr(), need.value, ins[i % sets].data_ptr(), n, c, plane)
+        if rc != 0:
+            raise RuntimeError(runner.capi.error_string(rc))
+
+    wall, ev = runner.time_steps(launch, steps, warmup)
+    return result_entry("feature map statistics N=%d C=%d 56x56 (mean, deviation, min, max per feature map)" % (n, c), 4 * total, total, wall, ev, 2,
+                        {"buffer_sets": sets, "note": "two launches per step: runs of entries, then their ordered merge"})
+
+
 def bench_copy(runner, steps, warmup):
     """Plain float4 copy kernel of the same launch shape: the yardstick for what HBM delivers."""
     count = (256 << 20) // 4
@@ -374,7 +396,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=400)
     ap.add_argument("--warmup", type=int, default=40)
-    ap.add_argument("--workload", default="config0", choices=["config0", "config1", "config2", "config3", "config4", "copy", "max_subsampling", "concat", "maxout"],
+    ap.add_argument("--workload", default="config0", choices=["config0", "config1", "config2", "config3", "config4", "copy", "max_subsampling", "concat", "maxout", "feature_map_stat"],
                     help="'copy' times the plain copy kernel (profiler-counter calibration and bandwidth yardstick)")
     ap.add_argument("--only", action="store_true", help="time only the chosen workload (no per_config survey, no CPU baseline)")
     args = ap.parse_args()
@@ -404,6 +426,8 @@ def main():
             return bench_concat(runner, steps, warmup)
         if name == "maxout":
             return bench_maxout(runner, steps, warmup)
+        if name == "feature_map_stat":
+            return bench_feature_map_stat(runner, steps, warmup)
         return bench_resnet50(runner, steps, warmup)
 
     main_entry = run(args.workload, args.steps, args.warmup)
@@ -416,7 +440,7 @@ def main():
                 per_config[name] = run(name, *side_steps[name])
         per_config["copy_kernel"] = bench_copy(runner, 40, 5)
         # the neighbouring layers of the same chains
-        for name, (k, wu) in (("max_subsampling", (40, 5)), ("concat", (100, 10)), ("maxout", (100, 10))):
+        for name, (k, wu) in (("max_subsampling", (40, 5)), ("concat", (100, 10)), ("maxout", (100, 10)), ("feature_map_stat", (20, 3))):
             if name not in per_config:
                 per_config[name] = run(name, k, wu)
         if args.workload == "config0":
@@ -449,7 +473,8 @@ def main():
             "frac": achieved / HBM_PEAK_GBPS,
             "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
             "kernel": {"config1": "nnf::softmax_rows_kernel", "copy": "nnf::copy_kernel_impl", "max_subsampling": "nnf::max_window2d_kernel",
-                       "concat": "nnf::concat_kernel", "maxout": "nnf::maxout_vec4_kernel"}.get(args.workload, "nnf::chain_kernel"),
+                       "concat": "nnf::concat_kernel", "maxout": "nnf::maxout_vec4_kernel",
+                       "feature_map_stat": "nnf::stat_runs_kernel"}.get(args.workload, "nnf::chain_kernel"),
             "algorithmic_bytes_per_launch": main_entry["algorithmic_bytes_per_step"] / launches,
             "avg_launch_us": main_entry["event_ms_per_step"] * 1e3 / launches,
         },

@@ -70,6 +70,55 @@ namespace nnforge
 		unsigned int entry_count = 0;
 	};
 
+	// nnforge/feature_map_data_stat.h:23-35
+	class feature_map_data_stat
+	{
+	public:
+		float min;
+		float max;
+		float average;
+		float std_dev;
+	};
+	std::ostream& operator<< (std::ostream& out, const feature_map_data_stat& val);
+
+	// Writer that keeps per-feature-map statistics of everything written to it instead of the
+	// values (nnforge/stat_data_bunch_writer.h:27-69): minimum, maximum and the single-pass mean /
+	// sum of squared deviations in double precision. A backend that reduces its outputs on the
+	// device hands the partial states over with merge() instead of calling write() per entry.
+	class stat_data_bunch_writer : public structured_data_bunch_writer
+	{
+	public:
+		typedef std::shared_ptr<stat_data_bunch_writer> ptr;
+
+		// same layout as nnf_hip_running_stat of the C ABI
+		struct running_stat
+		{
+			running_stat();
+			double n;
+			double mean;
+			double m2;
+			float min_val;
+			float max_val;
+		};
+
+		stat_data_bunch_writer();
+		void set_config_map(const std::map<std::string, layer_configuration_specific> config_map) override;
+		void write(unsigned int entry_id, const std::map<std::string, const float *>& data_map) override;
+		std::map<std::string, std::vector<feature_map_data_stat> > get_stat() const;
+
+		// folds states accumulated elsewhere over `entries` further entries into this writer
+		// (pairwise update of mean and sum of squared deviations)
+		void merge(const std::string& layer_name, const std::vector<running_stat>& partial);
+		void add_entries(unsigned int entries) { entry_count += entries; }
+		unsigned int get_entry_count() const { return entry_count; }
+		const std::map<std::string, layer_configuration_specific>& get_config_map() const { return config_map; }
+
+	private:
+		std::map<std::string, layer_configuration_specific> config_map;
+		std::map<std::string, std::vector<running_stat> > layer_name_to_running_stat_list_map;
+		unsigned int entry_count;
+	};
+
 	// nnforge/debug_state.h, profile_state.h reduced to their switches
 	struct debug_state
 	{
@@ -189,6 +238,21 @@ namespace nnforge
 	protected:
 		forward_propagation_factory() = default;
 	};
+
+	// Refreshes mean and inverse sigma of every BatchNorm layer from the statistics of the data the
+	// reader supplies (toolset::update_bn_weights, nnforge/toolset.cpp:1562-1630): per layer, a forward
+	// pass up to that layer with gamma 1 and beta 0 into a stat_data_bunch_writer, then
+	// inv_sigma' = inv_sigma / std_dev, mean' = mean + average / inv_sigma. Layers are handled in
+	// forward order, each one seeing the refreshed weights of those before it. data is modified in place.
+	// log (optional) receives the lines the reference prints.
+	void update_bn_weights(
+		const network_schema& schema,
+		network_data& data,
+		structured_data_bunch_reader& reader,
+		const forward_propagation_factory& factory,
+		debug_state::ptr debug = debug_state::ptr(),
+		profile_state::ptr profile = profile_state::ptr(),
+		std::ostream * log = nullptr);
 
 	// nnforge/backward_propagation_factory.h: the training side is outside this backend; the type
 	// exists so that factory_generator keeps its shape.

@@ -53,6 +53,8 @@ typedef struct nnf_backend_options
 	int32_t weights_from_folder;   /* 1: `weights_folder` holds <layer>.data files */
 	const char* weights_folder;
 	const char* profile_folder;    /* with profile: folder for forward_prop_perf_per_layer_action_NNN.csv; null: no file */
+	int32_t stat_on_host;          /* nnf_backend_layer_statistics: copy the outputs back and update the statistics
+	                                  value by value on the host, as the reference does, instead of reducing on the device */
 } nnf_backend_options;
 
 /* Runs the schema on device 0. The report lists one line per launch ("step: ..."), the buffer plan
@@ -64,6 +66,31 @@ NNF_BACKEND_API int nnf_backend_run_schema(
 	uint32_t entry_count,
 	nnf_backend_output* outputs, uint32_t output_count,
 	const nnf_backend_options* options,
+	char* report, size_t report_capacity);
+
+/* Statistics of one layer's output over entry_count entries (forward_propagation::run into a
+ * stat_data_bunch_writer): minimum, maximum, average and standard deviation per feature map, each
+ * array feature_map_count floats long. */
+NNF_BACKEND_API int nnf_backend_layer_statistics(
+	const char* schema_text,
+	const nnf_backend_weights* weights, uint32_t weights_count,
+	const nnf_backend_input* inputs, uint32_t input_count,
+	uint32_t entry_count,
+	const char* layer_name, uint32_t feature_map_count,
+	float* min_values, float* max_values, float* averages, float* std_devs,
+	const nnf_backend_options* options,
+	char* report, size_t report_capacity);
+
+/* toolset::update_bn_weights (nnforge/toolset.cpp:1562-1630) on in-memory data: refreshes mean and
+ * inverse sigma of every BatchNorm layer from the inputs' statistics and writes all weights to
+ * out_folder as <layer>.data files. The report holds the lines the reference prints. */
+NNF_BACKEND_API int nnf_backend_update_bn_weights(
+	const char* schema_text,
+	const nnf_backend_weights* weights, uint32_t weights_count,
+	const nnf_backend_input* inputs, uint32_t input_count,
+	uint32_t entry_count,
+	const nnf_backend_options* options,
+	const char* out_folder,
 	char* report, size_t report_capacity);
 
 /* Plans launches and buffers without touching a device (works on a machine without a GPU).

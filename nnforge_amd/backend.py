@@ -31,7 +31,7 @@ class Output(ctypes.Structure):
 class Options(ctypes.Structure):
     _fields_ = [("fuse", ctypes.c_int32), ("dont_share_buffers", ctypes.c_int32), ("max_entry_count", ctypes.c_int32),
                 ("profile", ctypes.c_int32), ("weights_from_folder", ctypes.c_int32), ("weights_folder", ctypes.c_char_p),
-                ("profile_folder", ctypes.c_char_p)]
+                ("profile_folder", ctypes.c_char_p), ("stat_on_host", ctypes.c_int32)]
 
 
 class BackendError(RuntimeError):
@@ -62,12 +62,18 @@ def load():
         lib.nnf_backend_write_weights.argtypes = [ctypes.c_char_p, ctypes.POINTER(Weights), ctypes.c_uint32, ctypes.c_char_p, ctypes.c_size_t]
         lib.nnf_backend_read_weights.argtypes = [ctypes.c_char_p, ctypes.c_char_p, ctypes.c_uint32, _UP, ctypes.POINTER(_FP),
                                                  ctypes.c_char_p, ctypes.c_size_t]
+        lib.nnf_backend_layer_statistics.argtypes = [ctypes.c_char_p, ctypes.POINTER(Weights), ctypes.c_uint32, ctypes.POINTER(Input),
+                                                     ctypes.c_uint32, ctypes.c_uint32, ctypes.c_char_p, ctypes.c_uint32, _FP, _FP, _FP, _FP,
+                                                     ctypes.POINTER(Options), ctypes.c_char_p, ctypes.c_size_t]
+        lib.nnf_backend_update_bn_weights.argtypes = [ctypes.c_char_p, ctypes.POINTER(Weights), ctypes.c_uint32, ctypes.POINTER(Input),
+                                                      ctypes.c_uint32, ctypes.c_uint32, ctypes.POINTER(Options), ctypes.c_char_p,
+                                                      ctypes.c_char_p, ctypes.c_size_t]
         _lib = lib
     return _lib
 
 
 def _options(fuse=True, dont_share_buffers=False, max_entry_count=0, profile=False, weights_folder=None,
-             profile_folder=None):
+             profile_folder=None, stat_on_host=False):
     o = Options()
     o.fuse = int(fuse)
     o.dont_share_buffers = int(dont_share_buffers)
@@ -76,6 +82,7 @@ def _options(fuse=True, dont_share_buffers=False, max_entry_count=0, profile=Fal
     o.weights_from_folder = int(weights_folder is not None)
     o.weights_folder = weights_folder.encode() if weights_folder is not None else None
     o.profile_folder = profile_folder.encode() if profile_folder is not None else None
+    o.stat_on_host = int(stat_on_host)
     return o
 
 
@@ -127,7 +134,7 @@ def parse_report(text):
             kind, _, desc = rest.partition(" ")
             layers, _, sources = desc.partition(" <- ")
             res["steps"].append({"fused": kind == "fused", "layers": layers.split("+"), "inputs": sources.split(", ")})
-        elif key in ("per_entry_bytes", "max_entry_count", "entries"):
+        elif key in ("per_entry_bytes", "max_entry_count", "entries", "writer_entries"):
             res[key] = int(rest)
         elif key == "seconds":
             name, _, sec = rest.rpartition(" ")
@@ -164,6 +171,39 @@ def run_schema(schema_text, weights, inputs, output_shapes, **options):
     for i, name in enumerate(sorted(output_shapes)):
         assert outs[i].written_floats == arrays[name].size, (name, outs[i].written_floats, arrays[name].size)
     return arrays, parse_report(report.value.decode())
+
+
+def layer_statistics(schema_text, weights, inputs, layer_name, feature_map_count, **options):
+    """Per-feature-map statistics of one layer's output: {'min', 'max', 'average', 'std_dev'} and the parsed report."""
+    lib = load()
+    keep = []
+    w = _weights_array(weights, keep)
+    ins, entry_count = _inputs_array(inputs, keep)
+    res = {k: np.full(feature_map_count, np.nan, dtype=np.float32) for k in ("min", "max", "average", "std_dev")}
+    report = ctypes.create_string_buffer(REPORT_CAPACITY)
+    opt = _options(**options)
+    rc = lib.nnf_backend_layer_statistics(schema_text.encode(), w, len(weights), ins, len(inputs), entry_count or 0, layer_name.encode(),
+                                          feature_map_count, *[res[k].ctypes.data_as(_FP) for k in ("min", "max", "average", "std_dev")],
+                                          ctypes.byref(opt), report, REPORT_CAPACITY)
+    if rc != 0:
+        raise BackendError(rc, report.value.decode(errors="replace"))
+    return res, parse_report(report.value.decode())
+
+
+def update_bn_weights(schema_text, weights, inputs, out_folder, **options):
+    """Refreshes the BatchNorm weights from the inputs' statistics and writes all weights to out_folder;
+    returns the lines the reference prints while doing so."""
+    lib = load()
+    keep = []
+    w = _weights_array(weights, keep)
+    ins, entry_count = _inputs_array(inputs, keep)
+    report = ctypes.create_string_buffer(1 << 20)
+    opt = _options(**options)
+    rc = lib.nnf_backend_update_bn_weights(schema_text.encode(), w, len(weights), ins, len(inputs), entry_count or 0, ctypes.byref(opt),
+                                           out_folder.encode(), report, 1 << 20)
+    if rc != 0:
+        raise BackendError(rc, report.value.decode(errors="replace"))
+    return report.value.decode()
 
 
 def plan_schema(schema_text, input_configs, output_names, memory_bytes=288 << 30, **options):

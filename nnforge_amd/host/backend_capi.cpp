@@ -50,6 +50,44 @@ namespace
 		out << "max_entry_count: " << fp.get_max_entry_count() << "\n";
 	}
 
+	void apply_options(hip::factory_generator_hip& generator, const nnf_backend_options * options)
+	{
+		generator.apply_default_options();
+		if (options != nullptr)
+		{
+			generator.hip_fuse = options->fuse != 0;
+			generator.hip_dont_share_buffers = options->dont_share_buffers != 0;
+			if (options->max_entry_count > 0)
+				generator.hip_max_entry_count = options->max_entry_count;
+		}
+		generator.initialize();
+	}
+
+	void fill_data(network_data& data, const nnf_backend_weights * weights, uint32_t weights_count, const nnf_backend_options * options)
+	{
+		if ((options != nullptr) && options->weights_from_folder)
+			data.read(options->weights_folder);
+		for(uint32_t i = 0; i < weights_count; ++i)
+		{
+			layer_data::ptr d(new layer_data());
+			for(uint32_t c = 0; c < weights[i].chunk_count; ++c)
+				d->push_back(std::vector<float>(weights[i].chunks[c], weights[i].chunks[c] + weights[i].chunk_sizes[c]));
+			data.add(weights[i].layer_name, d);
+		}
+	}
+
+	// hands everything on to a stat_data_bunch_writer without being one: the backend then takes the
+	// general path (outputs copied back, write() per entry)
+	class forwarding_writer : public structured_data_bunch_writer
+	{
+	public:
+		explicit forwarding_writer(structured_data_bunch_writer& target) : target(target) {}
+		void set_config_map(const std::map<std::string, layer_configuration_specific> config_map) override { target.set_config_map(config_map); }
+		void write(unsigned int entry_id, const std::map<std::string, const float *>& data_map) override { target.write(entry_id, data_map); }
+	private:
+		structured_data_bunch_writer& target;
+	};
+
 	template<class F> int guarded(F f, char * report, size_t report_capacity)
 	{
 		try
@@ -144,6 +182,89 @@ extern "C"
 			out << "stat: " << st << "\n";
 			for(const std::pair<const std::string, float>& a : fp->get_last_action_seconds())
 				out << "seconds: " << a.first << " " << a.second << "\n";
+		}, report, report_capacity);
+	}
+
+	int nnf_backend_layer_statistics(
+		const char* schema_text,
+		const nnf_backend_weights* weights, uint32_t weights_count,
+		const nnf_backend_input* inputs, uint32_t input_count,
+		uint32_t entry_count,
+		const char* layer_name, uint32_t feature_map_count,
+		float* min_values, float* max_values, float* averages, float* std_devs,
+		const nnf_backend_options* options,
+		char* report, size_t report_capacity)
+	{
+		return guarded([&](std::ostream& out)
+		{
+			const network_schema schema = parse_schema(schema_text);
+			if (layer_name == nullptr)
+				throw neural_network_exception("No output layers specified for forward_propagation");
+			hip::factory_generator_hip generator;
+			apply_options(generator, options);
+			forward_propagation::ptr fp = generator.create_forward_propagation_factory()->create(schema, std::vector<std::string>(1, layer_name),
+				debug_state::ptr(new debug_state(false)), profile_state::ptr(new profile_state(false)));
+			network_data data;
+			fill_data(data, weights, weights_count, options);
+			fp->set_data(data);
+
+			memory_data_bunch_reader reader(entry_count);
+			const std::map<std::string, layer_configuration_specific> configs = input_configs(inputs, input_count);
+			for(uint32_t i = 0; i < input_count; ++i)
+				reader.add(inputs[i].layer_name, configs.find(inputs[i].layer_name)->second, inputs[i].data);
+
+			stat_data_bunch_writer writer;
+			forward_propagation::stat st;
+			if ((options != nullptr) && (options->stat_on_host != 0))
+			{
+				forwarding_writer through(writer);
+				st = fp->run(reader, through);
+			}
+			else
+				st = fp->run(reader, writer);
+
+			const std::vector<feature_map_data_stat> stat = writer.get_stat().at(layer_name);
+			if (stat.size() != feature_map_count)
+				throw neural_network_exception("Layer " + std::string(layer_name) + " has " + std::to_string(stat.size()) + " feature maps, room for " + std::to_string(feature_map_count) + " supplied");
+			for(size_t f = 0; f < stat.size(); ++f)
+			{
+				min_values[f] = stat[f].min;
+				max_values[f] = stat[f].max;
+				averages[f] = stat[f].average;
+				std_devs[f] = stat[f].std_dev;
+			}
+			out << "entries: " << st.entry_processed_count << "\n";
+			out << "writer_entries: " << writer.get_entry_count() << "\n";
+		}, report, report_capacity);
+	}
+
+	int nnf_backend_update_bn_weights(
+		const char* schema_text,
+		const nnf_backend_weights* weights, uint32_t weights_count,
+		const nnf_backend_input* inputs, uint32_t input_count,
+		uint32_t entry_count,
+		const nnf_backend_options* options,
+		const char* out_folder,
+		char* report, size_t report_capacity)
+	{
+		return guarded([&](std::ostream& out)
+		{
+			const network_schema schema = parse_schema(schema_text);
+			if (out_folder == nullptr)
+				throw neural_network_exception("No folder given for the refreshed weights");
+			hip::factory_generator_hip generator;
+			apply_options(generator, options);
+			forward_propagation_factory::ptr factory = generator.create_forward_propagation_factory();
+			network_data data;
+			fill_data(data, weights, weights_count, options);
+
+			memory_data_bunch_reader reader(entry_count);
+			const std::map<std::string, layer_configuration_specific> configs = input_configs(inputs, input_count);
+			for(uint32_t i = 0; i < input_count; ++i)
+				reader.add(inputs[i].layer_name, configs.find(inputs[i].layer_name)->second, inputs[i].data);
+
+			update_bn_weights(schema, data, reader, *factory, debug_state::ptr(), profile_state::ptr(), &out);
+			data.write(out_folder);
 		}, report, report_capacity);
 	}
 

@@ -550,14 +550,36 @@ namespace nnforge
 				else
 					buffers[1].push_back(buffers[0].back());
 			}
+			// A statistics writer (nnforge/stat_data_bunch_writer.h) only wants per-feature-map figures of the
+			// outputs: they are reduced where they lie, in device memory, and nothing but the running
+			// states (32 bytes per feature map) travels to the host at the end of the run.
+			stat_data_bunch_writer * stat_writer = dynamic_cast<stat_data_bunch_writer *>(&writer);
+			const bool stats_on_device = (stat_writer != nullptr);
+			std::map<std::string, hip_linear_buffer_device::ptr> stat_states, stat_workspaces;
+			std::map<std::string, size_t> stat_workspace_bytes;
+			if (stats_on_device)
+			{
+				for(const std::string& n : output_layer_names)
+				{
+					const layer_configuration_specific& c = layer_config_map[n];
+					stat_states[n].reset(new hip_linear_buffer_device(static_cast<size_t>(c.feature_map_count) * sizeof(nnf_hip_running_stat)));
+					size_t bytes = 0;
+					hip_safe_call(nnf_hip_feature_map_stat_workspace_bytes(packet, c.feature_map_count, c.get_neuron_count_per_feature_map(), &bytes));
+					stat_workspaces[n].reset(new hip_linear_buffer_device(bytes));
+					stat_workspace_bytes[n] = bytes;
+					hip_safe_call(nnf_hip_feature_map_stat_init(p->stream, static_cast<nnf_hip_running_stat *>(static_cast<void *>(*stat_states[n])), c.feature_map_count));
+				}
+			}
+
 			std::map<std::string, std::unique_ptr<pinned_buffer> > staging[slot_count];
 			for(int s = 0; s < slot_count; ++s)
 			{
 				for(const std::string& n : data_layer_names)
 					staging[s][n].reset(new pinned_buffer(static_cast<size_t>(layer_config_map[n].get_neuron_count()) * sizeof(float) * packet));
-				for(const std::string& n : output_layer_names)
-					if (staging[s].find(n) == staging[s].end())
-						staging[s][n].reset(new pinned_buffer(static_cast<size_t>(layer_config_map[n].get_neuron_count()) * sizeof(float) * packet));
+				if (!stats_on_device)
+					for(const std::string& n : output_layer_names)
+						if (staging[s].find(n) == staging[s].end())
+							staging[s][n].reset(new pinned_buffer(static_cast<size_t>(layer_config_map[n].get_neuron_count()) * sizeof(float) * packet));
 			}
 			hip_event upload_done[slot_count], kernels_done[slot_count], download_done[slot_count];
 			bool slot_used[slot_count] = { false, false };
@@ -602,7 +624,7 @@ namespace nnforge
 						action_seconds[p->plans[i].key] += ms * 1.0e-3F;
 					}
 				}
-				for(unsigned int e = 0; e < f.entries; ++e)
+				for(unsigned int e = 0; (e < f.entries) && !stats_on_device; ++e)
 				{
 					std::map<std::string, const float *> data_map;
 					for(const std::string& n : output_layer_names)
@@ -679,11 +701,23 @@ namespace nnforge
 					}
 					if (profiling)
 						hip_safe_call(nnf_hip_event_record(step_events[slot][p->plans.size()]->ev, p->stream));
+					if (stats_on_device)
+					{
+						for(const std::string& n : output_layer_names)
+						{
+							const layer_configuration_specific& c = layer_config_map[n];
+							hip_safe_call(nnf_hip_feature_map_stat_accumulate(p->stream,
+								static_cast<nnf_hip_running_stat *>(static_cast<void *>(*stat_states[n])), *stat_workspaces[n], stat_workspace_bytes[n],
+								static_cast<const float *>(static_cast<const void *>(*buffers[slot][p->value_to_buffer.at(n)])),
+								entries_read, c.feature_map_count, c.get_neuron_count_per_feature_map()));
+						}
+					}
 					hip_safe_call(nnf_hip_event_record(kernels_done[slot].ev, p->stream));
 
 					// download
 					hip_safe_call(nnf_hip_stream_wait_event(p->download_stream, kernels_done[slot].ev));
 					for(const std::string& n : output_layer_names)
+						if (!stats_on_device)
 						hip_safe_call(nnf_hip_memcpy_d2h(staging[slot][n]->ptr, *buffers[slot][p->value_to_buffer.at(n)],
 							static_cast<size_t>(layer_config_map[n].get_neuron_count()) * sizeof(float) * entries_read, p->download_stream));
 					hip_safe_call(nnf_hip_event_record(download_done[slot].ev, p->download_stream));
@@ -704,6 +738,18 @@ namespace nnforge
 			if (previous.valid)
 				finish(previous);
 			hip_safe_call(nnf_hip_stream_synchronize(p->stream));
+
+			if (stats_on_device)
+			{
+				static_assert(sizeof(stat_data_bunch_writer::running_stat) == sizeof(nnf_hip_running_stat), "running state layouts differ");
+				for(const std::string& n : output_layer_names)
+				{
+					std::vector<stat_data_bunch_writer::running_stat> states(layer_config_map[n].feature_map_count);
+					hip_safe_call(nnf_hip_memcpy_d2h(states.data(), *stat_states[n], states.size() * sizeof(nnf_hip_running_stat), nullptr));
+					stat_writer->merge(n, states);
+				}
+				stat_writer->add_entries(read_total);
+			}
 
 			entries_processed = read_total;
 			idle_seconds = static_cast<float>(idle);

@@ -1,6 +1,8 @@
 #include "nnforge_hip/propagation.h"
 
 #include <algorithm>
+#include <cmath>
+#include <limits>
 #include <chrono>
 #include <cstdio>
 #include <cstring>
@@ -50,6 +52,158 @@ namespace nnforge
 		}
 		if (entry_id + 1 > entry_count)
 			entry_count = entry_id + 1;
+	}
+
+	// ---- statistics writer ------------------------------------------------------------------
+
+	std::ostream& operator<< (std::ostream& out, const feature_map_data_stat& val)
+	{
+		out << "Average " << val.average << ", StdDev " << val.std_dev << ", Min " << val.min << ", Max " << val.max;
+		return out;
+	}
+
+	stat_data_bunch_writer::running_stat::running_stat()
+		: n(0.0), mean(0.0), m2(0.0)
+		, min_val(std::numeric_limits<float>::max())
+		, max_val(-std::numeric_limits<float>::max())
+	{
+	}
+
+	stat_data_bunch_writer::stat_data_bunch_writer() : entry_count(0)
+	{
+	}
+
+	void stat_data_bunch_writer::set_config_map(const std::map<std::string, layer_configuration_specific> new_config_map)
+	{
+		config_map = new_config_map;
+		layer_name_to_running_stat_list_map.clear();
+		for(const std::pair<const std::string, layer_configuration_specific>& item : config_map)
+			layer_name_to_running_stat_list_map[item.first] = std::vector<running_stat>(item.second.feature_map_count);
+	}
+
+	void stat_data_bunch_writer::write(unsigned int, const std::map<std::string, const float *>& data_map)
+	{
+		for(const std::pair<const std::string, const float *>& item : data_map)
+		{
+			std::vector<running_stat>& stats = layer_name_to_running_stat_list_map.at(item.first);
+			const unsigned int neuron_count_per_feature_map = config_map.at(item.first).get_neuron_count_per_feature_map();
+			const float * data = item.second;
+			for(running_stat& s : stats)
+			{
+				for(unsigned int i = 0; i < neuron_count_per_feature_map; ++i, ++data)
+				{
+					const float val = *data;
+					s.min_val = std::min(s.min_val, val);
+					s.max_val = std::max(s.max_val, val);
+					s.n += 1.0;
+					const double val_d = static_cast<double>(val);
+					const double delta = val_d - s.mean;
+					s.mean += delta / s.n;
+					const double delta2 = val_d - s.mean;
+					s.m2 += delta * delta2;
+				}
+			}
+		}
+		++entry_count;
+	}
+
+	void stat_data_bunch_writer::merge(const std::string& layer_name, const std::vector<running_stat>& partial)
+	{
+		std::vector<running_stat>& stats = layer_name_to_running_stat_list_map.at(layer_name);
+		if (partial.size() != stats.size())
+			throw neural_network_exception("Statistics of " + std::to_string(partial.size()) + " feature maps supplied for layer " + layer_name + " with " + std::to_string(stats.size()));
+		for(size_t f = 0; f < stats.size(); ++f)
+		{
+			running_stat& s = stats[f];
+			const running_stat& b = partial[f];
+			if (b.n == 0.0)
+				continue;
+			const double n = s.n + b.n;
+			const double delta = b.mean - s.mean;
+			s.mean = (s.n == 0.0) ? b.mean : s.mean + delta * (b.n / n);
+			s.m2 = s.m2 + b.m2 + delta * delta * (s.n * b.n / n);
+			s.n = n;
+			s.min_val = std::min(s.min_val, b.min_val);
+			s.max_val = std::max(s.max_val, b.max_val);
+		}
+	}
+
+	std::map<std::string, std::vector<feature_map_data_stat> > stat_data_bunch_writer::get_stat() const
+	{
+		std::map<std::string, std::vector<feature_map_data_stat> > res;
+		for(const std::pair<const std::string, std::vector<running_stat> >& item : layer_name_to_running_stat_list_map)
+		{
+			std::vector<feature_map_data_stat> list;
+			for(const running_stat& s : item.second)
+			{
+				feature_map_data_stat st;
+				st.average = static_cast<float>(s.mean);
+				st.std_dev = sqrtf(static_cast<float>(s.m2 / s.n));
+				st.min = s.min_val;
+				st.max = s.max_val;
+				list.push_back(st);
+			}
+			res[item.first] = list;
+		}
+		return res;
+	}
+
+	void update_bn_weights(
+		const network_schema& schema,
+		network_data& data,
+		structured_data_bunch_reader& reader,
+		const forward_propagation_factory& factory,
+		debug_state::ptr debug,
+		profile_state::ptr profile,
+		std::ostream * log)
+	{
+		std::vector<std::string> bn_layers;
+		for(const layer::const_ptr& l : schema.get_layers_in_forward_propagation_order())
+			if (l->get_type_name() == "BatchNorm")
+				bn_layers.push_back(l->instance_name);
+		if (log != nullptr)
+		{
+			*log << "Updating Batch Normalization weights for these layers: ";
+			for(size_t i = 0; i < bn_layers.size(); ++i)
+				*log << (i == 0 ? "" : ", ") << bn_layers[i];
+			*log << std::endl;
+		}
+
+		for(const std::string& layer_name : bn_layers)
+		{
+			if (log != nullptr)
+				*log << layer_name << std::endl;
+			forward_propagation::ptr forward_prop = factory.create(schema, std::vector<std::string>(1, layer_name), debug, profile);
+
+			layer_data::ptr dt = data.get(layer_name);
+			if (dt->size() != 4)
+				throw neural_network_exception("data weight vector count " + std::to_string(dt->size()) + " doesn't satisfy layer configuration 4 for layer " + layer_name);
+			const std::vector<float> gamma_saved = dt->at(0);
+			const std::vector<float> beta_saved = dt->at(1);
+			std::fill(dt->at(0).begin(), dt->at(0).end(), 1.0F);
+			std::fill(dt->at(1).begin(), dt->at(1).end(), 0.0F);
+
+			forward_prop->set_data(data);
+
+			stat_data_bunch_writer writer;
+			forward_prop->run(reader, writer);
+
+			const std::vector<feature_map_data_stat> stat = writer.get_stat().at(layer_name);
+			for(size_t feature_map_id = 0; feature_map_id < stat.size(); ++feature_map_id)
+			{
+				if (log != nullptr)
+					*log << feature_map_id << ": " << stat[feature_map_id] << std::endl;
+				const float old_mean = dt->at(2)[feature_map_id];
+				const float old_invsigma = dt->at(3)[feature_map_id];
+				const float new_invsigma = old_invsigma / stat[feature_map_id].std_dev;
+				const float new_mean = old_mean + stat[feature_map_id].average / old_invsigma;
+				dt->at(2)[feature_map_id] = new_mean;
+				dt->at(3)[feature_map_id] = new_invsigma;
+			}
+
+			dt->at(0) = gamma_saved;
+			dt->at(1) = beta_saved;
+		}
 	}
 
 	std::string profile_state::get_path_to_unique_file(const char * file_prefix, const char * file_extension)

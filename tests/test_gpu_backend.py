@@ -7,7 +7,10 @@ import pytest
 
 import nnf_schemas as S
 import nnf_testing as T
+import oracle
 from nnforge_amd import backend
+
+F32 = np.float32
 
 pytestmark = pytest.mark.gpu
 
@@ -189,3 +192,75 @@ def test_dropout_only_network():
     values = S.evaluate(layers, {}, inputs)
     got, rep = run(layers, {}, inputs, ["d2"], values, max_entry_count=4)
     assert_bits(got["d2"], inputs["in"], "dropout chain")
+
+
+# ---- statistics of a layer's output and the batch norm refresh built on them -----------------------
+
+def two_bn_net(c=6):
+    """stem -> BatchNorm -> ReLU -> max pooling -> BatchNorm -> TanH: the second BatchNorm sees data shaped by the first."""
+    return [S.L("Data", "stem"), S.L("BatchNorm", "bn1", ["stem"], feature_map_count=c), S.L("ReLU", "relu1", ["bn1"]),
+            S.L("MaxSubsampling", "pool", ["relu1"], windows=[2, 2]), S.L("BatchNorm", "bn2", ["pool"], feature_map_count=c),
+            S.L("TanH", "out", ["bn2"])]
+
+
+@pytest.mark.parametrize("on_host", [False, True])
+def test_layer_statistics_on_device_and_on_host(on_host):
+    """forward_propagation::run into a stat_data_bunch_writer. On the host (outputs copied back, one value
+    at a time) the figures equal the oracle's bit for bit; reduced on the device they agree to one fp32 ulp."""
+    gen = T.rng(59, int(on_host))
+    c, n = 6, 23
+    layers = two_bn_net(c)
+    weights = S.make_weights(layers, gen)
+    inputs = {"stem": (T.normal(gen, (n, c, 12, 12), 2.0) + F32(1.5)).astype(F32)}
+    values = S.evaluate(layers, weights, inputs)
+    want = oracle.FeatureMapStat(c).write(values["bn2"]).get()
+    got, rep = backend.layer_statistics(S.schema_text(layers), weights, inputs, "bn2", c, max_entry_count=5, stat_on_host=on_host)
+    assert rep["entries"] == n and rep["writer_entries"] == n
+    assert np.array_equal(got["min"], want["min"]) and np.array_equal(got["max"], want["max"])
+    if on_host:
+        assert T.bit_mismatches(got["average"], want["average"]) == 0 and T.bit_mismatches(got["std_dev"], want["std_dev"]) == 0
+    else:
+        assert T.ulp_distance(got["average"], want["average"]).max() <= 1
+        assert T.ulp_distance(got["std_dev"], want["std_dev"]).max() <= 1
+
+
+def test_update_bn_weights_refreshes_every_batch_norm_in_forward_order(tmp_path):
+    """toolset::update_bn_weights: the oracle replays it layer by layer (statistics with gamma 1 / beta 0,
+    then the two formulas); the backend must arrive at the same mean / inverse sigma to one ulp of what
+    the statistics allow, leave gamma and beta alone, and the refreshed layers must then produce mean 0,
+    deviation 1 on that data."""
+    gen = T.rng(60, 0)
+    c, n = 6, 40
+    layers = two_bn_net(c)
+    weights = S.make_weights(layers, gen)
+    inputs = {"stem": (T.normal(gen, (n, c, 12, 12), 3.0) - F32(2.0)).astype(F32)}
+
+    # the reference's procedure on the CPU
+    ref = {k: [a.copy() for a in v] for k, v in weights.items()}
+    ones, zeros = np.ones(c, F32), np.zeros(c, F32)
+    for name in ("bn1", "bn2"):
+        trial = {k: list(v) for k, v in ref.items()}
+        trial[name] = [ones, zeros, ref[name][2], ref[name][3]]
+        out = S.evaluate(layers, trial, inputs)[name]
+        st = oracle.FeatureMapStat(c).write(out).get()
+        new_mean, new_inv = oracle.update_bn_weights(ref[name][2], ref[name][3], st["average"], st["std_dev"])
+        ref[name] = [ref[name][0], ref[name][1], new_mean, new_inv]
+
+    log = backend.update_bn_weights(S.schema_text(layers), weights, inputs, str(tmp_path), max_entry_count=16)
+    assert "Updating Batch Normalization weights for these layers: bn1, bn2" in log
+    assert log.count("Average ") == 2 * c
+    for name in ("bn1", "bn2"):
+        gamma, beta, mean, inv = backend.read_weights(str(tmp_path), name, [c] * 4)
+        assert T.bit_mismatches(gamma, weights[name][0]) == 0 and T.bit_mismatches(beta, weights[name][1]) == 0
+        # one ulp in average / std_dev moves the results by about that much relative to their size
+        assert np.allclose(inv, ref[name][3], rtol=3e-7, atol=0), name
+        assert np.allclose(mean, ref[name][2], rtol=3e-7, atol=3e-7), name
+        assert not np.allclose(inv, weights[name][3], rtol=1e-3)
+
+    # closed loop with the refreshed weights: normalised outputs
+    new_weights = {name: backend.read_weights(str(tmp_path), name, [c] * 4) for name in ("bn1", "bn2")}
+    plain = {name: [ones, zeros, w[2], w[3]] for name, w in new_weights.items()}
+    probe = dict(new_weights)
+    probe["bn2"] = plain["bn2"]
+    st2, _ = backend.layer_statistics(S.schema_text(layers), probe, inputs, "bn2", c)
+    assert np.abs(st2["average"]).max() < 1e-5 and np.abs(st2["std_dev"] - 1.0).max() < 1e-5
