@@ -633,6 +633,19 @@ namespace nnforge
 				}
 			};
 
+			// Whatever ends this function - the normal return or an exception from the reader, the writer or a
+			// launch - nothing declared above (device buffers, pinned staging, events) may be released while
+			// copies or kernels that use it are still in flight: this guard is destroyed first and waits.
+			struct drain_streams
+			{
+				void * streams[3];
+				~drain_streams()
+				{
+					for(void * s : streams)
+						nnf_hip_stream_synchronize(s);
+				}
+			} drain_on_exit = { { p->upload_stream, p->stream, p->download_stream } };
+
 			for(unsigned int packet_id = 0; ; ++packet_id)
 			{
 				const int slot = static_cast<int>(packet_id % slot_count);

@@ -18,7 +18,15 @@
  * closed forms expm1 / logistic / tanh / softmax with error budgets for the ones that call expf),
  * plus identities (identity batch norm, PReLU(a=1) = x, PReLU(a=0) = ReLU(0), Add(x, 0) = alpha*x,
  * softmax rows sum to 1 and are shift invariant, pooling of a constant) and brute-force index
- * checks on tiny shapes with distinct values per element. Not pinned by anything: the bit pattern
+ * checks on tiny shapes with distinct values per element. The layers next to that path are pinned
+ * the same way: absolute / dropout / concat against numpy's abs, identity and concatenate; maxout
+ * against a reshape-and-max that fails for the wrong feature-map grouping, plus a Python fold of
+ * std::max for the order-dependent cases (+0.0 / -0.0, NaN); max subsampling against numpy sliding
+ * windows in 1, 2 and 3 dimensions with strides, padded windows for round up, a reshape-and-max for
+ * feature-map / entry windows, the start value, tie and NaN cases, and a brute-force loop for tiling;
+ * the statistics against two-pass fp64 numpy (mean, population variance, fp32 rounding before the
+ * square root), packet invariance, a large-offset case, and the batch norm refresh against its two
+ * fp32 formulas and the closed loop (refreshed weights give mean 0, deviation 1). Not pinned by anything: the bit pattern
  * of the reference *as shipped* (built with -ffast-math -O3 -march=native, Settings.mk:26-28),
  * which depends on the compiler's contraction and vector-libm choices - "parity unpinned" for that;
  * this file states the source-level semantics.

@@ -5,6 +5,7 @@
 // equals a straightforward host evaluation of the same layers bit for bit.
 #include <nnforge_hip/hip_backend.h>
 
+#include <algorithm>
 #include <cmath>
 #include <cstdio>
 #include <cstring>
@@ -167,6 +168,76 @@ int main()
 		}
 		catch (const neural_network_exception&)
 		{
+		}
+
+		// a reader that fails in the middle of a run: the exception reaches the caller, nothing is freed
+		// under a copy or kernel still in flight, and the same object runs again afterwards
+		class failing_reader : public generated_reader
+		{
+		public:
+			using generated_reader::generated_reader;
+			bool read(unsigned int entry_id, const std::map<std::string, float *>& data_map) override
+			{
+				if (entry_id == 8)
+					throw neural_network_exception("reader failed at entry 8");
+				return generated_reader::read(entry_id, data_map);
+			}
+		};
+		try
+		{
+			failing_reader bad(entries, config);
+			memory_data_bunch_writer sink;
+			fp->run(bad, sink);
+			std::cout << "failing reader did not throw" << std::endl;
+			return 1;
+		}
+		catch (const neural_network_exception& e)
+		{
+			if (std::string(e.what()).find("entry 8") == std::string::npos)
+			{
+				std::cout << "unexpected exception: " << e.what() << std::endl;
+				return 1;
+			}
+		}
+		{
+			memory_data_bunch_writer again;
+			fp->run(reader, again);
+			if (again.values["res_prelu"] != writer.values["res_prelu"])
+			{
+				std::cout << "run after a failed run differs" << std::endl;
+				return 1;
+			}
+		}
+
+		// toolset::update_bn_weights as a library call: afterwards the batch norm output, taken with
+		// gamma 1 and beta 0, has mean 0 and deviation 1 over the reader's data
+		update_bn_weights(schema, data, reader, *generator.create_forward_propagation_factory(), debug_state::ptr(), profile_state::ptr(), nullptr);
+		{
+			network_data probe_data(schema.get_layers(), data); // shares the layers' weights with data ...
+			layer_data::ptr plain_bn(new layer_data(*data.get("main_bn"))); // ... so the modified layer gets its own copy
+			std::fill((*plain_bn)[0].begin(), (*plain_bn)[0].end(), 1.0F);
+			std::fill((*plain_bn)[1].begin(), (*plain_bn)[1].end(), 0.0F);
+			probe_data.add("main_bn", plain_bn);
+			forward_propagation::ptr probe = generator.create_forward_propagation_factory()->create(
+				schema, std::vector<std::string>(1, "main_bn"), debug_state::ptr(), profile_state::ptr());
+			probe->set_data(probe_data);
+			stat_data_bunch_writer stat_writer;
+			probe->run(reader, stat_writer);
+			const std::vector<feature_map_data_stat> after = stat_writer.get_stat().at("main_bn");
+			for(const feature_map_data_stat& st2 : after)
+			{
+				std::cout << st2 << std::endl;
+				if ((std::fabs(st2.average) > 1.0e-5F) || (std::fabs(st2.std_dev - 1.0F) > 1.0e-5F))
+				{
+					std::cout << "batch norm output is not normalised after update_bn_weights" << std::endl;
+					return 1;
+				}
+			}
+			if (stat_writer.get_entry_count() != entries)
+			{
+				std::cout << "statistics over " << stat_writer.get_entry_count() << " entries, expected " << entries << std::endl;
+				return 1;
+			}
 		}
 		std::cout << "ok" << std::endl;
 		return 0;
