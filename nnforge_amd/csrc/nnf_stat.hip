@@ -51,8 +51,10 @@ namespace nnf
 			const double d = static_cast<double>(v) - pivot;
 			s1 += d;
 			s2 = fma(d, d, s2);
-			mn = (v < mn) ? v : mn; // std::min(current, val)
-			mx = (mx < v) ? v : mx; // std::max(current, val)
+			// std::min(current, val) / std::max(current, val) never take a NaN val, and current is never NaN:
+			// that is fminf / fmaxf (one instruction each)
+			mn = __builtin_fminf(mn, v);
+			mx = __builtin_fmaxf(mx, v);
 		}
 
 		// grid: (runs, feature maps). VEC: floats per load (4 when plane is a multiple of 4).
@@ -70,7 +72,7 @@ namespace nnf
 			const uint32_t entries_here = min(entries_per_run, entry_count - e0);
 			const uint32_t units_per_plane = plane / VEC;
 			const uint32_t units = entries_here * units_per_plane;
-			const size_t entry_stride = static_cast<size_t>(feature_map_count) * plane;
+			const uint32_t entry_gap = (feature_map_count - 1) * plane;
 			const float* base = in + (static_cast<size_t>(e0) * feature_map_count + fm) * plane;
 			const double pivot = static_cast<double>(base[0]);
 
@@ -85,9 +87,10 @@ namespace nnf
 					const uint32_t t = first + k * stat_block_size + threadIdx.x;
 					if (t < units)
 					{
+						// element t of the run lies t * VEC floats into it plus the other feature maps of the
+						// entries before it: e * (entry_stride - plane); the tensor has fewer than 2^32 floats
 						const uint32_t e = (entries_here == 1) ? 0u : ((units_per_plane == 1) ? t : __umulhi(t, unit_magic));
-						const uint32_t i = t - e * units_per_plane;
-						v[k] = __builtin_nontemporal_load(reinterpret_cast<const vec_t*>(base + e * entry_stride + static_cast<size_t>(i) * VEC));
+						v[k] = __builtin_nontemporal_load(reinterpret_cast<const vec_t*>(base + (t * VEC + e * entry_gap)));
 					}
 				}
 				#pragma unroll
@@ -148,19 +151,30 @@ namespace nnf
 			if (fm >= feature_map_count)
 				return;
 			nnf_hip_running_stat s = state[fm];
-			for(uint32_t run = 0; run < runs; ++run)
+			constexpr uint32_t batch = 8; // partial states fetched together: the merge itself is a dependent chain
+			for(uint32_t first = 0; first < runs; first += batch)
 			{
-				const nnf_hip_running_stat b = partial[static_cast<size_t>(run) * feature_map_count + fm];
-				const double n = s.n + b.n;
-				const double delta = b.mean - s.mean;
-				if (s.n == 0.0)
-					s.mean = b.mean;
-				else
-					s.mean = s.mean + delta * (b.n / n);
-				s.m2 = s.m2 + b.m2 + delta * delta * (s.n * b.n / n);
-				s.n = n;
-				s.min_val = (b.min_val < s.min_val) ? b.min_val : s.min_val;
-				s.max_val = (s.max_val < b.max_val) ? b.max_val : s.max_val;
+				nnf_hip_running_stat b[batch];
+				#pragma unroll
+				for(uint32_t k = 0; k < batch; ++k)
+					if (first + k < runs)
+						b[k] = partial[static_cast<size_t>(first + k) * feature_map_count + fm];
+				#pragma unroll
+				for(uint32_t k = 0; k < batch; ++k)
+				{
+					if (first + k >= runs)
+						break;
+					const double n = s.n + b[k].n;
+					const double delta = b[k].mean - s.mean;
+					if (s.n == 0.0)
+						s.mean = b[k].mean;
+					else
+						s.mean = s.mean + delta * (b[k].n / n);
+					s.m2 = s.m2 + b[k].m2 + delta * delta * (s.n * b[k].n / n);
+					s.n = n;
+					s.min_val = (b[k].min_val < s.min_val) ? b[k].min_val : s.min_val;
+					s.max_val = (s.max_val < b[k].max_val) ? b[k].max_val : s.max_val;
+				}
 			}
 			state[fm] = s;
 		}

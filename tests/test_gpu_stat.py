@@ -133,3 +133,14 @@ def test_statistics_reject_bad_arguments(gpu):
     assert lib.nnf_hip_feature_map_stat_accumulate(s, state.data_ptr(), work.data_ptr(), 1 << 16, x.data_ptr() + 4, 4, 4, 255) == capi.E_ALIGN
     assert lib.nnf_hip_feature_map_stat_accumulate(s, state.data_ptr(), work.data_ptr(), 1 << 16, x.data_ptr(), 4, 0, 256) == capi.E_INVAL
     gpu.torch.cuda.synchronize()
+
+
+def test_statistics_keep_subnormal_minimum_and_maximum(gpu):
+    """min / max go through the hardware's fp32 minimum / maximum: subnormal values must come back as they are."""
+    tiny = np.array([1, 5, 77, 0x7FFFFF, 0x80000003, 0x80000009], dtype=np.uint32).view(F)   # +-subnormals
+    x = np.tile(tiny, 40).reshape(2, 1, 120).astype(F)
+    got = DeviceStat(gpu, 1).write(x).host()
+    want = oracle.FeatureMapStat(1).write(x).state
+    assert got["min_val"].tobytes() == want["min_val"].tobytes() and got["max_val"].tobytes() == want["max_val"].tobytes()
+    assert got["min_val"][0] == np.array([0x80000009], dtype=np.uint32).view(F)[0]
+    assert got["max_val"][0] == np.array([0x7FFFFF], dtype=np.uint32).view(F)[0]
