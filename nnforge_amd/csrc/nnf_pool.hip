@@ -9,31 +9,57 @@ namespace nnf
 	namespace
 	{
 		constexpr int pool_block_size = 256;
-		constexpr uint32_t global_pool_max_plane = 60; // 256 planes * 61 floats of padded LDS = 62.5 KB
+		constexpr uint32_t global_pool_planes = 64;    // planes per workgroup of the global pooling kernel
+		constexpr uint32_t global_pool_max_plane = 240; // 64 planes * 241 floats of padded LDS = 60 KB
 
-		// Window == whole plane (global pooling, e.g. 7x7 -> 1x1). A workgroup reduces 256 consecutive
-		// planes: it copies them to LDS with coalesced float4 loads, then lane t sums plane t front to
-		// back. Planes are stored with an odd stride so that the 64 lanes of a wavefront hit distinct banks.
-		__global__ void __launch_bounds__(pool_block_size) global_pool_kernel(float* out, const float* in, uint32_t plane_count, uint32_t plane, float mult)
+		// Window == whole plane (global pooling, e.g. 7x7 -> 1x1). A workgroup reduces 64 consecutive
+		// planes: its 256 lanes copy them to LDS with coalesced float4 loads, then lane t of the first
+		// wavefront sums plane t front to back. Planes are stored with an odd stride so that the 64 lanes
+		// hit distinct banks. Many small workgroups: the load, barrier and summation phases of
+		// different workgroups on a compute unit overlap.
+		__global__ void __launch_bounds__(pool_block_size) global_pool_kernel(float* out, const float* in, uint32_t plane_count, uint32_t plane, uint32_t plane_magic, float mult)
 		{
 			extern __shared__ __align__(16) float lds_planes[];
 			const uint32_t stride = plane | 1u;
-			const uint32_t first_plane = blockIdx.x * pool_block_size;
-			const uint32_t planes_here = min(static_cast<uint32_t>(pool_block_size), plane_count - first_plane);
+			const uint32_t first_plane = blockIdx.x * global_pool_planes;
+			const uint32_t planes_here = min(global_pool_planes, plane_count - first_plane);
 			const uint32_t floats_here = planes_here * plane; // multiple of 4 except possibly in the last workgroup
-			const float* src = in + static_cast<size_t>(first_plane) * plane; // 16-byte aligned: first_plane is a multiple of 256
+			const float* src = in + static_cast<size_t>(first_plane) * plane; // 16-byte aligned: first_plane is a multiple of 64
 
 			const uint32_t vectors = floats_here / 4;
-			for(uint32_t i = threadIdx.x; i < vectors; i += pool_block_size)
+			// eight loads in flight per lane before the first value goes to LDS
+			constexpr int stage = 8;
+			for(uint32_t base = 0; base < vectors; base += stage * pool_block_size)
 			{
-				const floatx4 t = load_stream(reinterpret_cast<const floatx4*>(src) + i);
-				const float vals[4] = {t.x, t.y, t.z, t.w};
+				floatx4 t[stage];
 				#pragma unroll
-				for(int e = 0; e < 4; ++e)
+				for(int k = 0; k < stage; ++k)
 				{
-					const uint32_t f = i * 4 + e;
-					const uint32_t p = f / plane;
-					lds_planes[p * stride + (f - p * plane)] = vals[e];
+					const uint32_t i = base + k * pool_block_size + threadIdx.x;
+					if (i < vectors)
+						t[k] = load_stream(reinterpret_cast<const floatx4*>(src) + i);
+				}
+				#pragma unroll
+				for(int k = 0; k < stage; ++k)
+				{
+					const uint32_t i = base + k * pool_block_size + threadIdx.x;
+					if (i < vectors)
+					{
+						const float vals[4] = {t[k].x, t[k].y, t[k].z, t[k].w};
+						// floats_here * plane < 2^32: the multiplication by ceil(2^32 / plane) divides exactly
+						uint32_t p = __umulhi(i * 4, plane_magic);
+						uint32_t r = i * 4 - p * plane;
+						#pragma unroll
+						for(int e = 0; e < 4; ++e)
+						{
+							lds_planes[p * stride + r] = vals[e];
+							if (++r == plane)
+							{
+								r = 0;
+								++p;
+							}
+						}
+					}
 				}
 			}
 			for(uint32_t f = vectors * 4 + threadIdx.x; f < floats_here; f += pool_block_size)
@@ -47,6 +73,7 @@ namespace nnf
 			{
 				const float* my_plane = lds_planes + threadIdx.x * stride;
 				float sum = 0.0f;
+				#pragma unroll 8
 				for(uint32_t i = 0; i < plane; ++i)
 					sum += my_plane[i];
 				out[first_plane + threadIdx.x] = sum * mult;
@@ -108,11 +135,13 @@ namespace nnf
 		}
 
 		const uint32_t plane = input_width * input_height;
-		if ((window_width == input_width) && (window_height == input_height) && (plane <= global_pool_max_plane))
+		if ((window_width == input_width) && (window_height == input_height) && (plane >= 2) && (plane <= global_pool_max_plane))
 		{
-			const size_t lds_bytes = static_cast<size_t>(pool_block_size) * (plane | 1u) * sizeof(float);
-			const dim3 grid((plane_count + pool_block_size - 1) / pool_block_size);
-			hipLaunchKernelGGL(global_pool_kernel, grid, dim3(pool_block_size), lds_bytes, stream, output, input, plane_count, plane, mult);
+			const size_t lds_bytes = static_cast<size_t>(global_pool_planes) * (plane | 1u) * sizeof(float);
+			const dim3 grid((plane_count + global_pool_planes - 1) / global_pool_planes);
+			// plane >= 2 here: a 1x1 window over a 1x1 plane takes the general kernel
+			const uint32_t plane_magic = static_cast<uint32_t>(((1ull << 32) + plane - 1) / plane);
+			hipLaunchKernelGGL(global_pool_kernel, grid, dim3(pool_block_size), lds_bytes, stream, output, input, plane_count, plane, plane_magic, mult);
 		}
 		else
 		{
