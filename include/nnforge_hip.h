@@ -235,6 +235,15 @@ NNF_HIP_API int nnf_hip_stream_wait_event(void* stream, void* event);
  * counters; no counterpart in the reference. bytes must be a multiple of 16. */
 NNF_HIP_API int nnf_hip_copy_kernel(void* stream, void* device_dst, const void* device_src, size_t bytes);
 
+/* Self-check of the two short division sequences the Sigmoid and TanH kernels use in place of the
+ * general IEEE division (reciprocal estimate + one Newton step for 1/(e + 1); quotient, exact
+ * remainder, one correction for (e - 1)/(e + 1)): enqueues a sweep over every non-negative float e with
+ * e + 1 <= 2^126 and adds the number of results that differ in bits from IEEE division to
+ * device_mismatch_counts[0] (reciprocal) and [1] (quotient), two counters in device memory that the
+ * caller has zeroed. Both must stay 0: the bit parity of nnforge/plain/sigmoid_layer_tester_plain.cpp:51
+ * and nnforge/plain/hyperbolic_tangent_layer_tester_plain.cpp:55-56 rests on it. */
+NNF_HIP_API int nnf_hip_check_division_sequences(void* stream, uint64_t* device_mismatch_counts);
+
 NNF_HIP_API const char* nnf_hip_error_string(int code);
 NNF_HIP_API const char* nnf_hip_version(void);
 

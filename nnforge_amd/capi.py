@@ -96,6 +96,7 @@ SIGNATURES = {
     "nnf_hip_event_elapsed_ms": [ctypes.POINTER(_F), _VP, _VP],
     "nnf_hip_stream_wait_event": [_VP, _VP],
     "nnf_hip_copy_kernel": [_VP, _VP, _VP, ctypes.c_size_t],
+    "nnf_hip_check_division_sequences": [_VP, _VP],
 }
 STRING_FUNCTIONS = {"nnf_hip_error_string": [ctypes.c_int], "nnf_hip_version": []}
 

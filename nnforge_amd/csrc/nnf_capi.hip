@@ -33,6 +33,29 @@ namespace nnf
 			}
 		}
 
+		// Sweep behind nnf_hip_check_division_sequences: lane-strided over the bit patterns of every
+		// non-negative float e with e + 1 <= 2^126.
+		__global__ void __launch_bounds__(256) division_check_kernel(unsigned long long* mismatches)
+		{
+			constexpr uint32_t last_bits = 0x7E800000u; // 2^126
+			unsigned long long bad_reciprocal = 0, bad_quotient = 0;
+			const uint64_t stride = static_cast<uint64_t>(gridDim.x) * blockDim.x;
+			for(uint64_t u = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x; u <= last_bits; u += stride)
+			{
+				const float e = __uint_as_float(static_cast<uint32_t>(u));
+				const float d = e + 1.0f;
+				if (!(d <= 0x1p126f))
+					continue;
+				const float n = e - 1.0f;
+				bad_reciprocal += __float_as_uint(nnf_fast_reciprocal_of_ge1(d)) != __float_as_uint(1.0f / d);
+				bad_quotient += __float_as_uint(nnf_fast_tanh_quotient(n, d)) != __float_as_uint(n / d);
+			}
+			if (bad_reciprocal != 0)
+				atomicAdd(&mismatches[0], bad_reciprocal);
+			if (bad_quotient != 0)
+				atomicAdd(&mismatches[1], bad_quotient);
+		}
+
 		nnf_hip_chain_desc single_op_desc(uint32_t entry_count, uint32_t fm_count, uint32_t plane, int32_t kind, int32_t chunk, float f0, float f1)
 		{
 			nnf_hip_chain_desc d;
@@ -254,6 +277,16 @@ extern "C"
 	{
 		return average_subsampling_forward(static_cast<hipStream_t>(stream), output, input, entry_count, feature_map_count,
 			input_width, input_height, window_width, window_height, mult);
+	}
+
+	int nnf_hip_check_division_sequences(void* stream, uint64_t* device_mismatch_counts)
+	{
+		if (device_mismatch_counts == nullptr)
+			return NNF_HIP_EINVAL;
+		static_assert(sizeof(unsigned long long) == sizeof(uint64_t), "counter width");
+		hipLaunchKernelGGL(division_check_kernel, dim3(4096), dim3(256), 0, static_cast<hipStream_t>(stream),
+			reinterpret_cast<unsigned long long*>(device_mismatch_counts));
+		return launch_status();
 	}
 
 	int nnf_hip_copy_kernel(void* stream, void* device_dst, const void* device_src, size_t bytes)

@@ -69,13 +69,16 @@ namespace nnf
 	// nnforge/plain/exponential_linear_layer_tester_plain.cpp:51). glibc >= 2.27 evaluates expf as
 	// 2^(k/32) * p(r) in double precision (x*32/ln2 = k + r, |r| <= 1/2, 32-entry table, cubic p) and
 	// rounds the double to float, which makes it correctly rounded for all but a handful of inputs.
-	// This is the same published scheme with every multiply-add fused, the form an FMA-capable x86-64
-	// host evaluates; it returns the same bits as that expf for every one of the 2^32 fp32 inputs
-	// (checked exhaustively on the host by the unit tests; NaN payloads aside).
+	// This is the same published scheme with the argument reduction fused and the cubic in Horner
+	// form (7 double-precision operations); it returns the same bits as that expf for every one of
+	// the 2^32 fp32 inputs (checked exhaustively on the host by the unit tests; NaN payloads aside).
 	//
 	// The rounded integer k sits in the low word of the shifted sum; only the high word of the table
 	// entry takes part in applying the exponent (k << 47 = (k << 15) in the high word).
-	NNF_HD float nnf_expf(float x, const exp_context& ctx)
+	//
+	// nnf_expf_core is the arithmetic alone: valid for log(2^-150) < x < log(2^128), NaN in, NaN out;
+	// outside that range k does not fit and the value is meaningless (nnf_expf_out_of_range repairs it).
+	NNF_HD float nnf_expf_core(float x, const exp_context& ctx)
 	{
 		const double inv_ln2_times_32 = 0x1.71547652b82fep+5;
 		const double c0 = 0x1.c6af84b912394p-20; // (ln2/32)^3 / 6, minimax-adjusted
@@ -88,60 +91,145 @@ namespace nnf
 		const double r = __builtin_fma(inv_ln2_times_32, xd, -kd);
 		double_words entry = reinterpret_cast<const double_words*>(ctx.table)[k & (exp2_table_size - 1)];
 		uint32_t scale_hi = entry.hi + (k << 15);
-#if defined(__HIP_DEVICE_COMPILE__)
+	#if defined(__HIP_DEVICE_COMPILE__)
 		// keeps the addition a 32-bit one (the compiler otherwise widens it to a 64-bit add with
 		// extra register moves)
 		asm volatile("" : "+v"(scale_hi));
-#endif
+	#endif
 		entry.hi = scale_hi;
 		const double s = __builtin_bit_cast(double, entry);
-		const double z = __builtin_fma(c0, r, ctx.c1);
-		const double r2 = r * r;
-		double y = __builtin_fma(c2, r, 1.0);
-		y = __builtin_fma(z, r2, y);
+		double y = __builtin_fma(c0, r, ctx.c1);
+		y = __builtin_fma(y, r, c2);
+		y = __builtin_fma(y, r, 1.0);
 		y = y * s;
-		float res = static_cast<float>(y);
-		// Outside (log(2^-150), log(2^128)) the double path is meaningless (k does not fit): the
-		// results there are 0 and +inf. NaN fails both comparisons and comes out of the arithmetic as NaN.
+		return static_cast<float>(y);
+	}
+
+	// Results outside the range of nnf_expf_core: +inf above log(2^128), 0 below log(2^-150).
+	// NaN fails both comparisons and keeps the NaN the arithmetic produced.
+	NNF_HD float nnf_expf_out_of_range(float x, float res)
+	{
 		res = x > 0x1.62e42ep6f ? __builtin_inff() : res;
 		res = x < -0x1.9fe368p6f ? 0.0f : res;
 		return res;
 	}
 
-	// numerator[i] / denominator[i] for denominators that are >= 1, +inf or NaN - the only divisions
-	// the layers below make (e + 1 with e = expf(...) >= 0). On the device: reciprocal estimate, one
-	// Newton step, then quotient, exact remainder and correction (each an FMA), which yields the
-	// correctly rounded quotient as long as the reciprocal is a normal number; a wavefront that holds
-	// a denominator above 2^126 (or inf / NaN) anywhere in the batch redoes the batch with the general
-	// IEEE division (one uniform branch per batch, so the fast sequences of a batch interleave freely).
-	// Compared with IEEE division over every possible e (all non-negative floats, +inf, NaN):
-	// identical bits.
-	template<int N>
-	NNF_HD void nnf_divide_by_ge1(const float (&numerator)[N], const float (&denominator)[N], float (&quotient)[N])
+	NNF_HD float nnf_expf(float x, const exp_context& ctx)
 	{
-#if defined(__HIP_DEVICE_COMPILE__)
+		return nnf_expf_out_of_range(x, nnf_expf_core(x, ctx));
+	}
+
+	// res[i] = expf(x[i]) for the small batch of values a lane holds. On the device the range repair
+	// is one comparison per value and one wavefront-uniform branch per batch: only a wavefront that
+	// holds an |x| above 87 (or a NaN) anywhere in the batch runs the two selects per value; every
+	// other wavefront runs the arithmetic alone (|x| <= 87 is inside the range of nnf_expf_core and
+	// its results are normal numbers).
+	template<int N>
+	NNF_HD void nnf_expf_batch(const float (&x)[N], float (&res)[N], const exp_context& ctx)
+	{
+	#if defined(__HIP_DEVICE_COMPILE__)
+		bool repair = false;
+		#pragma unroll
+		for(int i = 0; i < N; ++i)
+		{
+			res[i] = nnf_expf_core(x[i], ctx);
+			repair = repair || !(__builtin_fabsf(x[i]) <= 87.0f);
+		}
+		if (__builtin_expect(__any(repair), 0))
+		{
+			#pragma unroll
+			for(int i = 0; i < N; ++i)
+				res[i] = nnf_expf_out_of_range(x[i], res[i]);
+		}
+	#else
+		for(int i = 0; i < N; ++i)
+			res[i] = nnf_expf(x[i], ctx);
+	#endif
+	}
+
+	// The only divisions the layers below make have the denominator d = e + 1 with e = expf(...) >= 0,
+	// i.e. d >= 1, +inf or NaN. On the device they start from the hardware reciprocal estimate r0
+	// (within 1 ulp of 1/d):
+	//   1 / d             = fma(fma(-d, r0, 1), r0, r0)            (one Newton step)
+	//   (e - 1) / (e + 1) = fma(fma(-d, q0, n), r0, q0), q0 = n*r0  (quotient, exact remainder, correction)
+	// Both were compared with IEEE division for every non-negative float e with e + 1 <= 2^126 (all
+	// 2^31 of them, and the device library's self-check repeats that sweep): identical bits. The
+	// second sequence is only claimed for the pair n = e - 1, d = e + 1, not for arbitrary numerators.
+	// A wavefront that holds a denominator above 2^126 (or inf / NaN) anywhere in the batch, where the
+	// reciprocal leaves the normal range, redoes the batch with the general IEEE division (one
+	// uniform branch per batch, so the fast sequences of a batch interleave freely).
+	NNF_HD float nnf_fast_reciprocal_of_ge1(float d)
+	{
+	#if defined(__HIP_DEVICE_COMPILE__)
+		const float r = __builtin_amdgcn_rcpf(d);
+		const float e = __builtin_fmaf(-d, r, 1.0f);
+		return __builtin_fmaf(e, r, r);
+	#else
+		return 1.0f / d;
+	#endif
+	}
+
+	NNF_HD float nnf_fast_tanh_quotient(float n, float d)
+	{
+	#if defined(__HIP_DEVICE_COMPILE__)
+		const float r = __builtin_amdgcn_rcpf(d);
+		const float q = n * r;
+		const float rem = __builtin_fmaf(-d, q, n);
+		return __builtin_fmaf(rem, r, q);
+	#else
+		return n / d;
+	#endif
+	}
+
+	// 1 / (e[i] + 1), e[i] = expf(...)
+	template<int N>
+	NNF_HD void nnf_reciprocal_of_exp_plus_one(const float (&e)[N], float (&quotient)[N])
+	{
+	#if defined(__HIP_DEVICE_COMPILE__)
 		bool out_of_range = false;
 		#pragma unroll
 		for(int i = 0; i < N; ++i)
 		{
-			float r = __builtin_amdgcn_rcpf(denominator[i]);
-			const float e = __builtin_fmaf(-denominator[i], r, 1.0f);
-			r = __builtin_fmaf(e, r, r);
-			float q = numerator[i] * r;
-			const float rem = __builtin_fmaf(-denominator[i], q, numerator[i]);
-			quotient[i] = __builtin_fmaf(rem, r, q);
-			out_of_range = out_of_range || !(denominator[i] <= 0x1p126f);
+			const float d = e[i] + 1.0f;
+			quotient[i] = nnf_fast_reciprocal_of_ge1(d);
+			out_of_range = out_of_range || !(d <= 0x1p126f);
 		}
 		if (__builtin_expect(__any(out_of_range), 0))
 		{
 			#pragma unroll
 			for(int i = 0; i < N; ++i)
-				quotient[i] = numerator[i] / denominator[i];
+				quotient[i] = 1.0f / (e[i] + 1.0f);
 		}
-#else
+	#else
 		for(int i = 0; i < N; ++i)
-			quotient[i] = numerator[i] / denominator[i];
-#endif
+			quotient[i] = 1.0f / (e[i] + 1.0f);
+	#endif
+	}
+
+	// (e[i] - 1) / (e[i] + 1), e[i] = expf(...)
+	template<int N>
+	NNF_HD void nnf_exp_minus_one_over_exp_plus_one(const float (&e)[N], float (&quotient)[N])
+	{
+	#if defined(__HIP_DEVICE_COMPILE__)
+		bool out_of_range = false;
+		#pragma unroll
+		for(int i = 0; i < N; ++i)
+		{
+			const float n = e[i] - 1.0f;
+			const float d = e[i] + 1.0f;
+			quotient[i] = nnf_fast_tanh_quotient(n, d);
+			out_of_range = out_of_range || !(d <= 0x1p126f);
+		}
+		if (__builtin_expect(__any(out_of_range), 0))
+		{
+			#pragma unroll
+			for(int i = 0; i < N; ++i)
+				quotient[i] = (e[i] - 1.0f) / (e[i] + 1.0f);
+		}
+	#else
+		for(int i = 0; i < N; ++i)
+			quotient[i] = (e[i] - 1.0f) / (e[i] + 1.0f);
+	#endif
 	}
 
 	// nnforge/plain/batch_norm_layer_tester_plain.cpp:60-61
@@ -183,43 +271,35 @@ namespace nnf
 	template<int N>
 	NNF_HD void nnf_exponential_linear(float (&v)[N], const exp_context& ctx)
 	{
+		float e[N];
+		nnf_expf_batch<N>(v, e, ctx);
 		#pragma unroll
 		for(int i = 0; i < N; ++i)
-		{
-			const float x = v[i];
-			const float e = nnf_expf(x, ctx);
-			v[i] = x >= 0.0f ? x : (e - 1.0f);
-		}
+			v[i] = v[i] >= 0.0f ? v[i] : (e[i] - 1.0f);
 	}
 
 	// nnforge/plain/sigmoid_layer_tester_plain.cpp:50-51
 	template<int N>
 	NNF_HD void nnf_sigmoid(float (&v)[N], const exp_context& ctx)
 	{
-		float one[N], denominator[N];
+		float e[N];
 		#pragma unroll
 		for(int i = 0; i < N; ++i)
-		{
-			const float e = nnf_expf(-v[i], ctx);
-			one[i] = 1.0f;
-			denominator[i] = e + 1.0f;
-		}
-		nnf_divide_by_ge1<N>(one, denominator, v);
+			v[i] = -v[i];
+		nnf_expf_batch<N>(v, e, ctx);
+		nnf_reciprocal_of_exp_plus_one<N>(e, v);
 	}
 
 	// nnforge/plain/hyperbolic_tangent_layer_tester_plain.cpp:54-56; steepness2 = steepness * 2.0f
 	template<int N>
 	NNF_HD void nnf_hyperbolic_tangent(float (&v)[N], float steepness2, float scale, const exp_context& ctx)
 	{
-		float numerator[N], denominator[N];
+		float e[N];
 		#pragma unroll
 		for(int i = 0; i < N; ++i)
-		{
-			const float e = nnf_expf(v[i] * steepness2, ctx);
-			numerator[i] = e - 1.0f;
-			denominator[i] = e + 1.0f;
-		}
-		nnf_divide_by_ge1<N>(numerator, denominator, v);
+			v[i] = v[i] * steepness2;
+		nnf_expf_batch<N>(v, e, ctx);
+		nnf_exp_minus_one_over_exp_plus_one<N>(e, v);
 		#pragma unroll
 		for(int i = 0; i < N; ++i)
 			v[i] = v[i] * scale;

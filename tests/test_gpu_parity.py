@@ -453,3 +453,13 @@ def test_exp_layers_over_the_whole_fp32_range(gpu):
             total_bad += bad
         checked += x.size
     print("exp layers: %d inputs per layer checked, %d mismatches" % (checked, total_bad))
+
+
+def test_short_division_sequences_equal_ieee_division_for_every_denominator(gpu):
+    """The device's own sweep over every non-negative float e with e + 1 <= 2^126 (2^31 values): the
+    reciprocal sequence of Sigmoid and the quotient sequence of TanH return the bits of IEEE division."""
+    counts = gpu.torch.zeros(2, dtype=gpu.torch.int64, device=gpu.device)
+    rc = gpu.lib.nnf_hip_check_division_sequences(gpu.stream, counts.data_ptr())
+    assert rc == 0, capi.error_string(rc)
+    gpu.torch.cuda.synchronize()
+    assert counts.tolist() == [0, 0]
