@@ -91,7 +91,16 @@ class Runner:
     def sync(self):
         self.torch.cuda.synchronize()
 
-    def prepare_group(self, group, sets):
+    def config3_input(self, count):
+        """x ~ N(0, 2) (variance) with 0.1 % of the entries at +-50, as BASELINE.json states config 3."""
+        t = self.randn(count, 2.0 ** 0.5)
+        spikes = self.torch.rand(count, generator=self.gen, device=self.device) < 0.001
+        signs = self.torch.rand(count, generator=self.gen, device=self.device) < 0.5
+        t[spikes & signs] = 50.0
+        t[spikes & ~signs] = -50.0
+        return t
+
+    def prepare_group(self, group, sets, make_input=None):
         """Allocates `sets` rotating buffer sets for a fused group; returns a launch closure."""
         from nnforge_amd import workloads as w
 
@@ -108,7 +117,7 @@ class Runner:
         keep = [chunks]
         calls = []
         for _ in range(sets):
-            ins = [self.randn(total) for _ in group.arms]
+            ins = [(make_input or self.randn)(total) for _ in group.arms]
             out = self.empty(total)
             keep.append((ins, out))
             calls.append((out.data_ptr(), capi.pointer_array([t.data_ptr() for t in ins])))
@@ -166,12 +175,12 @@ def rotation_sets(bytes_per_set, minimum_total=768 << 20, cap=32):
     return int(max(2, min(cap, -(-minimum_total // bytes_per_set))))
 
 
-def bench_group(runner, label, group, steps, warmup):
+def bench_group(runner, label, group, steps, warmup, make_input=None):
     from nnforge_amd import workloads as w
 
     alg = w.group_algorithmic_bytes(group)
     sets = rotation_sets(alg)
-    launch = runner.prepare_group(group, sets)
+    launch = runner.prepare_group(group, sets, make_input)
     wall, ev = runner.time_steps(launch, steps, warmup)
     entry = result_entry(label, alg, w.group_elements(group), wall, ev, 1,
                          {"buffer_sets": sets, "shape": [group.entry_count, group.feature_map_count, group.plane]})
@@ -417,7 +426,7 @@ def main():
         if name == "config2":
             return bench_group(runner, "config2: batch_norm -> add(residual) -> parametric_rectified_linear N=128 C=256 56x56", w.config2(), steps, warmup)
         if name == "config3":
-            return bench_group(runner, "config3: batch_norm -> exponential_linear -> sigmoid -> hyperbolic_tangent N=64 C=512 28x28", w.config3(), steps, warmup)
+            return bench_group(runner, "config3: batch_norm -> exponential_linear -> sigmoid -> hyperbolic_tangent N=64 C=512 28x28", w.config3(), steps, warmup, runner.config3_input)
         if name == "copy":
             return bench_copy(runner, steps, warmup)
         if name == "max_subsampling":

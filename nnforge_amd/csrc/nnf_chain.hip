@@ -18,7 +18,8 @@ namespace nnf
 	{
 
 		constexpr int max_slots = NNF_HIP_MAX_OPS;
-		constexpr uint32_t exp_table_bytes = exp_lds_entries * sizeof(uint64_t);
+		// one copy of the expf table per wavefront of the largest workgroup (256 lanes)
+		constexpr uint32_t exp_table_bytes = exp_lds_entries * sizeof(uint64_t) * (256 / wave_size);
 
 		struct chain_op
 		{
@@ -207,8 +208,10 @@ namespace nnf
 		};
 		constexpr int known_program_count = sizeof(known_programs) / sizeof(known_programs[0]);
 
-		template<int NIN, int BLOCK, int U, bool DIRECT, int PROGRAM>
-		__global__ void __launch_bounds__(BLOCK) chain_kernel(const chain_args a)
+		// One tile of the tensor. FULL: every float4 of the tile lies inside the tensor, so loads and
+		// stores are unconditional (the ragged last tile takes the other instance).
+		template<int NIN, int BLOCK, int U, bool DIRECT, int PROGRAM, bool FULL>
+		__device__ __forceinline__ void chain_tile(const chain_args& a)
 		{
 			constexpr int TILE = BLOCK * U * 4;
 			constexpr int PL = DIRECT ? 1 : 4;
@@ -221,7 +224,12 @@ namespace nnf
 			const uint32_t start_in_plane = tile_start - first_plane * a.plane;
 			const uint32_t first_fm = first_plane % a.fm_count;
 
-			// all tensor loads are issued before anything else: they are what the kernel waits for
+			// All loads are issued before anything else, oldest first: the lane's expf table entry, the
+			// tensors, then (compile-time programs) the weights of a leading batch norm.
+			constexpr bool program_has_exp = PROGRAM > 0; // every compile-time program calls expf
+			uint64_t exp_entry = 0;
+			if (program_has_exp || a.need_exp)
+				exp_entry = load_exp2_table_entry();
 			float x[NIN][U][4];
 			#pragma unroll
 			for(int j = 0; j < NIN; ++j)
@@ -230,7 +238,7 @@ namespace nnf
 				for(int k = 0; k < U; ++k)
 				{
 					const uint32_t idx = tile_start + (threadIdx.x + k * BLOCK) * 4;
-					if (idx + 3 < a.total)
+					if (FULL || (idx + 3 < a.total))
 					{
 						const floatx4 t = load_stream(reinterpret_cast<const floatx4*>(a.in[j] + idx));
 						x[j][k][0] = t.x; x[j][k][1] = t.y; x[j][k][2] = t.z; x[j][k][3] = t.w;
@@ -243,34 +251,6 @@ namespace nnf
 					}
 				}
 			}
-
-			if (a.need_exp)
-				stage_exp2_table(lds_exp);
-			if (!DIRECT)
-			{
-				for(uint32_t s = 0; s < a.slot_count; ++s)
-				{
-					const chain_slot& slot = a.slots[s];
-					for(uint32_t i = threadIdx.x; i < a.span; i += BLOCK)
-					{
-						const uint32_t fm = (first_fm + i) % a.fm_count;
-						float2 c;
-						if (slot.kind == NNF_HIP_OP_BATCH_NORM)
-							nnf_batch_norm_coefficients(slot.p[0][fm], slot.p[1][fm], slot.p[2][fm], slot.p[3][fm], c.x, c.y);
-						else
-						{
-							c.x = slot.p[0][fm];
-							c.y = 0.0f;
-						}
-						lds_coeff[s * a.span + i] = c;
-					}
-				}
-			}
-			if (!DIRECT || a.need_exp)
-				__syncthreads();
-			exp_context exp_ctx = make_exp_context(lds_exp);
-			if (a.need_exp)
-				exp_ctx = exp_context_from_lds(lds_exp);
 
 			uint32_t where[U][PL];
 			#pragma unroll
@@ -290,11 +270,64 @@ namespace nnf
 				}
 			}
 
+			// compile-time program that starts with a batch norm, weights read straight from memory
+			constexpr bool leading_batch_norm = DIRECT && (PROGRAM > 0) && (known_programs[PROGRAM].kinds[0] == NNF_HIP_OP_BATCH_NORM);
+			float lead_weights[U][4] = {};
+			if (leading_batch_norm)
+			{
+				const chain_slot& slot = a.slots[a.ops[0].slot];
+				#pragma unroll
+				for(int k = 0; k < U; ++k)
+				{
+					#pragma unroll
+					for(int c = 0; c < 4; ++c)
+						lead_weights[k][c] = slot.p[c][where[k][0]];
+				}
+			}
+
+			// expf table: one private copy per wavefront, so the direct path has no workgroup barrier
+			exp_context exp_ctx = make_exp_context(lds_exp);
+			if (program_has_exp || a.need_exp)
+				exp_ctx = stage_exp2_table_per_wavefront(lds_exp, exp_entry);
+			if (!DIRECT)
+			{
+				for(uint32_t s = 0; s < a.slot_count; ++s)
+				{
+					const chain_slot& slot = a.slots[s];
+					for(uint32_t i = threadIdx.x; i < a.span; i += BLOCK)
+					{
+						const uint32_t fm = (first_fm + i) % a.fm_count;
+						float2 c;
+						if (slot.kind == NNF_HIP_OP_BATCH_NORM)
+							nnf_batch_norm_coefficients(slot.p[0][fm], slot.p[1][fm], slot.p[2][fm], slot.p[3][fm], c.x, c.y);
+						else
+						{
+							c.x = slot.p[0][fm];
+							c.y = 0.0f;
+						}
+						lds_coeff[s * a.span + i] = c;
+					}
+				}
+				__syncthreads();
+			}
+
 			uint32_t op_index = 0;
 			if (PROGRAM > 0)
 			{
+				if (leading_batch_norm)
+				{
+					#pragma unroll
+					for(int k = 0; k < U; ++k)
+					{
+						float mult, add;
+						nnf_batch_norm_coefficients(lead_weights[k][0], lead_weights[k][1], lead_weights[k][2], lead_weights[k][3], mult, add);
+						#pragma unroll
+						for(int e = 0; e < 4; ++e)
+							x[0][k][e] = nnf_batch_norm(x[0][k][e], mult, add);
+					}
+				}
 				#pragma unroll
-				for(int i = 0; i < known_programs[PROGRAM].op_count; ++i)
+				for(int i = leading_batch_norm ? 1 : 0; i < known_programs[PROGRAM].op_count; ++i)
 					apply_op<U, DIRECT, U * 4>(known_programs[PROGRAM].kinds[i], a.ops[i], a, x[0], where, lds_coeff, exp_ctx);
 				op_index = known_programs[PROGRAM].op_count;
 			}
@@ -338,7 +371,7 @@ namespace nnf
 			for(int k = 0; k < U; ++k)
 			{
 				const uint32_t idx = tile_start + (threadIdx.x + k * BLOCK) * 4;
-				if (idx + 3 < a.total)
+				if (FULL || (idx + 3 < a.total))
 				{
 					floatx4 t;
 					t.x = x[0][k][0]; t.y = x[0][k][1]; t.z = x[0][k][2]; t.w = x[0][k][3];
@@ -352,6 +385,16 @@ namespace nnf
 							a.out[idx + e] = x[0][k][e];
 				}
 			}
+		}
+
+		template<int NIN, int BLOCK, int U, bool DIRECT, int PROGRAM>
+		__global__ void __launch_bounds__(BLOCK) chain_kernel(const chain_args a)
+		{
+			constexpr uint32_t tile = BLOCK * U * 4;
+			if (blockIdx.x * tile + tile <= a.total) // total <= 0xFFFF0000: the sum does not wrap
+				chain_tile<NIN, BLOCK, U, DIRECT, PROGRAM, true>(a);
+			else
+				chain_tile<NIN, BLOCK, U, DIRECT, PROGRAM, false>(a);
 		}
 
 		typedef void (*chain_kernel_fn)(const chain_args);

@@ -35,6 +35,29 @@ namespace nnf
 		return ctx;
 	}
 
+	// Wavefront-private variant in two steps: every wavefront of the workgroup copies the table into
+	// its own exp_lds_entries slots of lds_tables and reads only those, so no workgroup barrier is
+	// needed (the LDS operations of one wavefront execute in program order). The global load of the
+	// lane's table entry is issued first, unconditionally, so that a kernel can put its tensor and
+	// weight loads behind it and wait for all of them once; the LDS copy follows those loads.
+	__device__ __forceinline__ uint64_t load_exp2_table_entry()
+	{
+		const uint32_t lane = threadIdx.x % wave_size;
+		return exp2_table_device[lane < exp_lds_entries ? lane : exp_lds_entries - 1];
+	}
+
+	__device__ __forceinline__ exp_context stage_exp2_table_per_wavefront(uint64_t* lds_tables, uint64_t entry)
+	{
+		const uint32_t lane = threadIdx.x % wave_size;
+		uint64_t* own = lds_tables + (threadIdx.x / wave_size) * exp_lds_entries;
+		if (lane < exp_lds_entries)
+			own[lane] = entry;
+		__builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+		__builtin_amdgcn_wave_barrier();
+		__builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+		return exp_context_from_lds(own);
+	}
+
 	// Streaming accesses: each byte of an activation tensor is touched once per launch, so loads
 	// and stores carry the non-temporal hint and do not displace what the caches hold.
 	__device__ __forceinline__ floatx4 load_stream(const floatx4* p)

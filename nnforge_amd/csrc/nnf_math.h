@@ -94,7 +94,7 @@ namespace nnf
 	#if defined(__HIP_DEVICE_COMPILE__)
 		// keeps the addition a 32-bit one (the compiler otherwise widens it to a 64-bit add with
 		// extra register moves)
-		asm volatile("" : "+v"(scale_hi));
+		asm("" : "+v"(scale_hi));
 	#endif
 		entry.hi = scale_hi;
 		const double s = __builtin_bit_cast(double, entry);
@@ -123,9 +123,10 @@ namespace nnf
 	// is one comparison per value and one wavefront-uniform branch per batch: only a wavefront that
 	// holds an |x| above 87 (or a NaN) anywhere in the batch runs the two selects per value; every
 	// other wavefront runs the arithmetic alone (|x| <= 87 is inside the range of nnf_expf_core and
-	// its results are normal numbers).
+	// its results are normal numbers). Returns whether this wavefront took the repair branch; when
+	// it did not, every res[i] lies in [exp(-87), exp(87)] (about 1.6e-38 .. 6.1e37).
 	template<int N>
-	NNF_HD void nnf_expf_batch(const float (&x)[N], float (&res)[N], const exp_context& ctx)
+	NNF_HD bool nnf_expf_batch(const float (&x)[N], float (&res)[N], const exp_context& ctx)
 	{
 	#if defined(__HIP_DEVICE_COMPILE__)
 		bool repair = false;
@@ -133,17 +134,20 @@ namespace nnf
 		for(int i = 0; i < N; ++i)
 		{
 			res[i] = nnf_expf_core(x[i], ctx);
-			repair = repair || !(__builtin_fabsf(x[i]) <= 87.0f);
+			repair |= !(__builtin_fabsf(x[i]) <= 87.0f);
 		}
-		if (__builtin_expect(__any(repair), 0))
+		const bool any_repair = __any(repair);
+		if (__builtin_expect(any_repair, 0))
 		{
 			#pragma unroll
 			for(int i = 0; i < N; ++i)
 				res[i] = nnf_expf_out_of_range(x[i], res[i]);
 		}
+		return any_repair;
 	#else
 		for(int i = 0; i < N; ++i)
 			res[i] = nnf_expf(x[i], ctx);
+		return true;
 	#endif
 	}
 
@@ -155,9 +159,9 @@ namespace nnf
 	// Both were compared with IEEE division for every non-negative float e with e + 1 <= 2^126 (all
 	// 2^31 of them, and the device library's self-check repeats that sweep): identical bits. The
 	// second sequence is only claimed for the pair n = e - 1, d = e + 1, not for arbitrary numerators.
-	// A wavefront that holds a denominator above 2^126 (or inf / NaN) anywhere in the batch, where the
-	// reciprocal leaves the normal range, redoes the batch with the general IEEE division (one
-	// uniform branch per batch, so the fast sequences of a batch interleave freely).
+	// Above 2^126 (and for inf / NaN) the reciprocal leaves the normal range: a wavefront whose expf
+	// batch took the repair branch (general_division: some |x| > 87 or NaN, the only way to an
+	// e above exp(87) < 2^126) uses the general IEEE division for the whole batch instead.
 	NNF_HD float nnf_fast_reciprocal_of_ge1(float d)
 	{
 	#if defined(__HIP_DEVICE_COMPILE__)
@@ -181,55 +185,40 @@ namespace nnf
 	#endif
 	}
 
-	// 1 / (e[i] + 1), e[i] = expf(...)
+	// 1 / (e[i] + 1), e[i] = expf(...); general_division is uniform across the wavefront
 	template<int N>
-	NNF_HD void nnf_reciprocal_of_exp_plus_one(const float (&e)[N], float (&quotient)[N])
+	NNF_HD void nnf_reciprocal_of_exp_plus_one(const float (&e)[N], float (&quotient)[N], bool general_division)
 	{
-	#if defined(__HIP_DEVICE_COMPILE__)
-		bool out_of_range = false;
-		#pragma unroll
-		for(int i = 0; i < N; ++i)
-		{
-			const float d = e[i] + 1.0f;
-			quotient[i] = nnf_fast_reciprocal_of_ge1(d);
-			out_of_range = out_of_range || !(d <= 0x1p126f);
-		}
-		if (__builtin_expect(__any(out_of_range), 0))
+		if (__builtin_expect(general_division, 0))
 		{
 			#pragma unroll
 			for(int i = 0; i < N; ++i)
 				quotient[i] = 1.0f / (e[i] + 1.0f);
 		}
-	#else
-		for(int i = 0; i < N; ++i)
-			quotient[i] = 1.0f / (e[i] + 1.0f);
-	#endif
+		else
+		{
+			#pragma unroll
+			for(int i = 0; i < N; ++i)
+				quotient[i] = nnf_fast_reciprocal_of_ge1(e[i] + 1.0f);
+		}
 	}
 
-	// (e[i] - 1) / (e[i] + 1), e[i] = expf(...)
+	// (e[i] - 1) / (e[i] + 1), e[i] = expf(...); general_division is uniform across the wavefront
 	template<int N>
-	NNF_HD void nnf_exp_minus_one_over_exp_plus_one(const float (&e)[N], float (&quotient)[N])
+	NNF_HD void nnf_exp_minus_one_over_exp_plus_one(const float (&e)[N], float (&quotient)[N], bool general_division)
 	{
-	#if defined(__HIP_DEVICE_COMPILE__)
-		bool out_of_range = false;
-		#pragma unroll
-		for(int i = 0; i < N; ++i)
-		{
-			const float n = e[i] - 1.0f;
-			const float d = e[i] + 1.0f;
-			quotient[i] = nnf_fast_tanh_quotient(n, d);
-			out_of_range = out_of_range || !(d <= 0x1p126f);
-		}
-		if (__builtin_expect(__any(out_of_range), 0))
+		if (__builtin_expect(general_division, 0))
 		{
 			#pragma unroll
 			for(int i = 0; i < N; ++i)
 				quotient[i] = (e[i] - 1.0f) / (e[i] + 1.0f);
 		}
-	#else
-		for(int i = 0; i < N; ++i)
-			quotient[i] = (e[i] - 1.0f) / (e[i] + 1.0f);
-	#endif
+		else
+		{
+			#pragma unroll
+			for(int i = 0; i < N; ++i)
+				quotient[i] = nnf_fast_tanh_quotient(e[i] - 1.0f, e[i] + 1.0f);
+		}
 	}
 
 	// nnforge/plain/batch_norm_layer_tester_plain.cpp:60-61
@@ -286,8 +275,8 @@ namespace nnf
 		#pragma unroll
 		for(int i = 0; i < N; ++i)
 			v[i] = -v[i];
-		nnf_expf_batch<N>(v, e, ctx);
-		nnf_reciprocal_of_exp_plus_one<N>(e, v);
+		const bool general_division = nnf_expf_batch<N>(v, e, ctx);
+		nnf_reciprocal_of_exp_plus_one<N>(e, v, general_division);
 	}
 
 	// nnforge/plain/hyperbolic_tangent_layer_tester_plain.cpp:54-56; steepness2 = steepness * 2.0f
@@ -298,8 +287,8 @@ namespace nnf
 		#pragma unroll
 		for(int i = 0; i < N; ++i)
 			v[i] = v[i] * steepness2;
-		nnf_expf_batch<N>(v, e, ctx);
-		nnf_exp_minus_one_over_exp_plus_one<N>(e, v);
+		const bool general_division = nnf_expf_batch<N>(v, e, ctx);
+		nnf_exp_minus_one_over_exp_plus_one<N>(e, v, general_division);
 		#pragma unroll
 		for(int i = 0; i < N; ++i)
 			v[i] = v[i] * scale;
