@@ -129,12 +129,14 @@ namespace nnf
 				const uint32_t c = (lane + k * THREADS) * W;
 				if (row_valid && (c < fm_count))
 				{
+					float x[W];
 					#pragma unroll
 					for(int e = 0; e < W; ++e)
-					{
-						v[k][e] = nnf_expf(v[k][e] - m, exp_ctx);
+						x[e] = v[k][e] - m;
+					nnf_expf_batch<W>(x, v[k], exp_ctx);
+					#pragma unroll
+					for(int e = 0; e < W; ++e)
 						sum += v[k][e];
-					}
 				}
 			}
 			sum = wave_all_reduce(sum, sum_op());
@@ -211,8 +213,16 @@ namespace nnf
 		}
 
 		// neuron_count_per_feature_map > 1. One lane per (entry, position); consecutive lanes take
-		// consecutive positions. Same operation order as the reference, including the sequential sum.
-		// CACHED > 0: the column (fm_count <= CACHED) stays in registers: one read, one write.
+		// consecutive positions, so every load and store of a wavefront covers 256 consecutive bytes.
+		// Same operation order as the reference, including the sequential sum over feature maps.
+		//
+		// CACHED > 0: the column (fm_count <= CACHED) stays in registers: one read, one write. All
+		// CACHED loads are issued at once; the ones beyond fm_count re-read the last feature map
+		// (folding a value into the maximum twice changes nothing) and take no part in the sum.
+		// CACHED == 0: three passes in batches of eight feature maps (eight loads in flight per lane),
+		// expf values parked in the output like the reference does; a lane re-reads only what it wrote.
+		constexpr int softmax_column_batch = 8;
+
 		template<int CACHED>
 		__global__ void __launch_bounds__(256) softmax_columns_kernel(float* out, const float* in, uint32_t columns, uint32_t fm_count, uint32_t plane)
 		{
@@ -229,53 +239,191 @@ namespace nnf
 			const size_t base = static_cast<size_t>(entry) * fm_count * plane + pos;
 			const float* src = in + base;
 			float* dst = out + base;
+			const uint32_t last = fm_count - 1;
 
 			if (CACHED > 0)
 			{
-				float v[CACHED > 0 ? CACHED : 1];
+				constexpr int COUNT = CACHED > 0 ? CACHED : softmax_column_batch;
+				constexpr int B = COUNT < softmax_column_batch ? COUNT : softmax_column_batch;
+				static_assert(COUNT % B == 0, "whole batches");
+				float v[COUNT];
+				#pragma unroll
+				for(int c = 0; c < COUNT; ++c)
+					v[c] = src[static_cast<size_t>(min(static_cast<uint32_t>(c), last)) * plane];
 				float m = softmax_max_init;
 				#pragma unroll
-				for(int c = 0; c < CACHED; ++c)
-				{
-					if (static_cast<uint32_t>(c) < fm_count)
-					{
-						v[c] = src[static_cast<size_t>(c) * plane];
-						m = ref_max(m, v[c]);
-					}
-				}
+				for(int c = 0; c < COUNT; ++c)
+					m = ref_max(m, v[c]);
 				float sum = 0.0f;
 				#pragma unroll
-				for(int c = 0; c < CACHED; ++c)
+				for(int c0 = 0; c0 < COUNT; c0 += B)
 				{
-					if (static_cast<uint32_t>(c) < fm_count)
+					if (static_cast<uint32_t>(c0) < fm_count) // uniform
 					{
-						v[c] = nnf_expf(v[c] - m, exp_ctx);
-						sum += v[c];
+						float x[B], e[B];
+						#pragma unroll
+						for(int i = 0; i < B; ++i)
+							x[i] = v[c0 + i] - m;
+						nnf_expf_batch<B>(x, e, exp_ctx);
+						#pragma unroll
+						for(int i = 0; i < B; ++i)
+						{
+							v[c0 + i] = e[i];
+							if (static_cast<uint32_t>(c0 + i) < fm_count) // uniform
+								sum += e[i];
+						}
 					}
 				}
 				const float mult = 1.0f / sum;
 				#pragma unroll
-				for(int c = 0; c < CACHED; ++c)
+				for(int c = 0; c < COUNT; ++c)
 				{
-					if (static_cast<uint32_t>(c) < fm_count)
+					if (static_cast<uint32_t>(c) < fm_count) // uniform
 						dst[static_cast<size_t>(c) * plane] = v[c] * mult;
 				}
 			}
 			else
 			{
+				constexpr int B = softmax_column_batch;
 				float m = softmax_max_init;
-				for(uint32_t c = 0; c < fm_count; ++c)
-					m = ref_max(m, src[static_cast<size_t>(c) * plane]);
-				float sum = 0.0f;
-				for(uint32_t c = 0; c < fm_count; ++c)
+				for(uint32_t c0 = 0; c0 < fm_count; c0 += B)
 				{
-					const float val = nnf_expf(src[static_cast<size_t>(c) * plane] - m, exp_ctx);
-					sum += val;
-					dst[static_cast<size_t>(c) * plane] = val;
+					float x[B];
+					#pragma unroll
+					for(int i = 0; i < B; ++i)
+						x[i] = src[static_cast<size_t>(min(c0 + i, last)) * plane];
+					#pragma unroll
+					for(int i = 0; i < B; ++i)
+						m = ref_max(m, x[i]);
+				}
+				float sum = 0.0f;
+				for(uint32_t c0 = 0; c0 < fm_count; c0 += B)
+				{
+					float x[B], e[B];
+					#pragma unroll
+					for(int i = 0; i < B; ++i)
+						x[i] = src[static_cast<size_t>(min(c0 + i, last)) * plane] - m;
+					nnf_expf_batch<B>(x, e, exp_ctx);
+					#pragma unroll
+					for(int i = 0; i < B; ++i)
+					{
+						if (c0 + i < fm_count) // uniform
+						{
+							sum += e[i];
+							dst[static_cast<size_t>(c0 + i) * plane] = e[i];
+						}
+					}
 				}
 				const float mult = 1.0f / sum;
-				for(uint32_t c = 0; c < fm_count; ++c)
-					dst[static_cast<size_t>(c) * plane] *= mult;
+				for(uint32_t c0 = 0; c0 < fm_count; c0 += B)
+				{
+					float x[B];
+					#pragma unroll
+					for(int i = 0; i < B; ++i)
+						x[i] = dst[static_cast<size_t>(min(c0 + i, last)) * plane];
+					#pragma unroll
+					for(int i = 0; i < B; ++i)
+					{
+						if (c0 + i < fm_count) // uniform
+							dst[static_cast<size_t>(c0 + i) * plane] = x[i] * mult;
+					}
+				}
+			}
+		}
+
+		// neuron_count_per_feature_map > 1 with few columns and many feature maps: one lane per column
+		// would leave most of the machine idle and make every lane walk a long column alone. A
+		// workgroup of 256 lanes takes P consecutive columns; the feature maps are cut into S = 256 / P
+		// contiguous slices, lane (slice, position) walks its slice in batches of eight, and the slices
+		// are combined through LDS in slice order. The maximum is the reference's; the sum is S
+		// sequential partial sums added in order instead of one sequential sum, so results can differ
+		// from the reference in the last bits (bar: 1e-5 relative, as for rows).
+		template<int P>
+		__global__ void __launch_bounds__(256) softmax_columns_sliced_kernel(float* out, const float* in, uint32_t columns, uint32_t fm_count, uint32_t plane)
+		{
+			constexpr int S = 256 / P;
+			constexpr int B = softmax_column_batch;
+			__shared__ uint64_t lds_exp[exp_lds_entries];
+			__shared__ float lds_partial[2][S][P];
+			stage_exp2_table(lds_exp);
+			__syncthreads();
+			const exp_context exp_ctx = exp_context_from_lds(lds_exp);
+
+			const uint32_t p = threadIdx.x % P;
+			const uint32_t slice = threadIdx.x / P;
+			const uint32_t column = blockIdx.x * P + p;
+			const bool valid = column < columns;
+			const uint32_t col = valid ? column : columns - 1; // lanes past the end shadow the last column and store nothing
+			const uint32_t entry = col / plane;
+			const uint32_t pos = col - entry * plane;
+			const size_t base = static_cast<size_t>(entry) * fm_count * plane + pos;
+			const float* src = in + base;
+			float* dst = out + base;
+
+			const uint32_t per_slice = (fm_count + S - 1) / S;
+			const uint32_t c_begin = min(slice * per_slice, fm_count);
+			const uint32_t c_end = min(c_begin + per_slice, fm_count);
+			const uint32_t c_last = (c_end > c_begin) ? c_end - 1 : 0; // an empty slice runs no batch
+
+			float m = softmax_max_init;
+			for(uint32_t c0 = c_begin; c0 < c_end; c0 += B)
+			{
+				float x[B];
+				#pragma unroll
+				for(int i = 0; i < B; ++i)
+					x[i] = src[static_cast<size_t>(min(c0 + i, c_last)) * plane];
+				#pragma unroll
+				for(int i = 0; i < B; ++i)
+					m = ref_max(m, x[i]);
+			}
+			lds_partial[0][slice][p] = m;
+			__syncthreads();
+			m = softmax_max_init;
+			#pragma unroll
+			for(int s = 0; s < S; ++s)
+				m = ref_max(m, lds_partial[0][s][p]);
+
+			float sum = 0.0f;
+			for(uint32_t c0 = c_begin; c0 < c_end; c0 += B)
+			{
+				float x[B], e[B];
+				#pragma unroll
+				for(int i = 0; i < B; ++i)
+					x[i] = src[static_cast<size_t>(min(c0 + i, c_last)) * plane] - m;
+				nnf_expf_batch<B>(x, e, exp_ctx);
+				#pragma unroll
+				for(int i = 0; i < B; ++i)
+				{
+					if (c0 + i < c_end)
+					{
+						sum += e[i];
+						if (valid)
+							dst[static_cast<size_t>(c0 + i) * plane] = e[i];
+					}
+				}
+			}
+			lds_partial[1][slice][p] = sum;
+			__syncthreads();
+			sum = 0.0f;
+			#pragma unroll
+			for(int s = 0; s < S; ++s)
+				sum += lds_partial[1][s][p];
+
+			const float mult = 1.0f / sum;
+			if (!valid)
+				return;
+			for(uint32_t c0 = c_begin; c0 < c_end; c0 += B)
+			{
+				float x[B];
+				#pragma unroll
+				for(int i = 0; i < B; ++i)
+					x[i] = dst[static_cast<size_t>(min(c0 + i, c_last)) * plane];
+				#pragma unroll
+				for(int i = 0; i < B; ++i)
+				{
+					if (c0 + i < c_end)
+						dst[static_cast<size_t>(c0 + i) * plane] = x[i] * mult;
+				}
 			}
 		}
 
@@ -307,6 +455,10 @@ namespace nnf
 		// spread over as many lanes as it has vectors. Measured on 256 rows of 1000 floats: 3.1 us
 		// with 256 lanes per row against 4.3 us with one wavefront per row.
 		constexpr uint32_t few_rows = 2048;
+
+		// Columns (neuron_count_per_feature_map > 1) of more than 64 feature maps: up to this many
+		// columns the feature maps of a column are shared out over 16 lanes.
+		constexpr uint32_t sliced_columns_limit = 65536;
 
 		template<int W>
 		bool try_launch_rows(hipStream_t stream, float* out, const float* in, uint32_t rows, uint32_t fm_count)
@@ -371,10 +523,34 @@ namespace nnf
 		else
 		{
 			const uint32_t columns = entry_count * neuron_count_per_feature_map;
-			const dim3 block(256);
-			const dim3 grid((columns + 255) / 256);
-			if (feature_map_count <= 16)
+			if ((feature_map_count > 64) && (columns <= sliced_columns_limit))
+			{
+				// a whole wavefront along the positions (256-byte accesses) once that still gives every
+				// compute unit a few workgroups
+				if (columns >= 64u * 512u)
+					hipLaunchKernelGGL(softmax_columns_sliced_kernel<64>, dim3((columns + 63) / 64), dim3(256), 0, stream,
+						output, input, columns, feature_map_count, neuron_count_per_feature_map);
+				else
+					hipLaunchKernelGGL(softmax_columns_sliced_kernel<16>, dim3((columns + 15) / 16), dim3(256), 0, stream,
+						output, input, columns, feature_map_count, neuron_count_per_feature_map);
+				return launch_status();
+			}
+			// few columns: one wavefront per workgroup spreads them over more compute units
+			const uint32_t block_size = (columns >= 256u * 1024u) ? 256u : 64u;
+			const dim3 block(block_size);
+			const dim3 grid((columns + block_size - 1) / block_size);
+			if (feature_map_count <= 2)
+				hipLaunchKernelGGL(softmax_columns_kernel<2>, grid, block, 0, stream, output, input, columns, feature_map_count, neuron_count_per_feature_map);
+			else if (feature_map_count <= 4)
+				hipLaunchKernelGGL(softmax_columns_kernel<4>, grid, block, 0, stream, output, input, columns, feature_map_count, neuron_count_per_feature_map);
+			else if (feature_map_count <= 8)
+				hipLaunchKernelGGL(softmax_columns_kernel<8>, grid, block, 0, stream, output, input, columns, feature_map_count, neuron_count_per_feature_map);
+			else if (feature_map_count <= 16)
 				hipLaunchKernelGGL(softmax_columns_kernel<16>, grid, block, 0, stream, output, input, columns, feature_map_count, neuron_count_per_feature_map);
+			else if (feature_map_count <= 32)
+				hipLaunchKernelGGL(softmax_columns_kernel<32>, grid, block, 0, stream, output, input, columns, feature_map_count, neuron_count_per_feature_map);
+			else if (feature_map_count <= 64)
+				hipLaunchKernelGGL(softmax_columns_kernel<64>, grid, block, 0, stream, output, input, columns, feature_map_count, neuron_count_per_feature_map);
 			else
 				hipLaunchKernelGGL(softmax_columns_kernel<0>, grid, block, 0, stream, output, input, columns, feature_map_count, neuron_count_per_feature_map);
 		}

@@ -352,8 +352,11 @@ def test_softmax_rows(gpu, n, c):
     assert T.bit_mismatches(got, got2) == 0
 
 
-@pytest.mark.parametrize("n,c,plane", [(2, 3, 2), (1, 10, 49), (3, 16, 5), (2, 17, 64), (2, 21, 1000), (1, 150, 333), (4, 5, 4096)])
+@pytest.mark.parametrize("n,c,plane", [(2, 1, 5), (2, 2, 777), (2, 3, 2), (3, 4, 130), (1, 10, 49), (3, 16, 5), (2, 17, 64), (2, 21, 1000),
+                                       (3, 33, 300), (2, 64, 129), (1, 70, 70001), (4, 5, 4096)])
 def test_softmax_columns_bit_exact(gpu, n, c, plane):
+    """One lane per column (up to 64 feature maps, or more than 65536 columns): the reference's own
+    left-to-right sum, so the bits are the oracle's."""
     gen = T.rng(14, n * 100000 + c * 100 + plane)
     x = T.normal(gen, (n, c, plane), 4.0)
     x[gen.random((n, c, plane)) < 0.01] = 30.0
@@ -362,6 +365,20 @@ def test_softmax_columns_bit_exact(gpu, n, c, plane):
     assert_softmax_close(got, want, "softmax columns")
     assert T.bit_mismatches(got, want) == 0  # same left-to-right sum as the reference
     assert T.bit_mismatches(run_softmax(gpu, x, in_place=True), want) == 0
+
+
+@pytest.mark.parametrize("n,c,plane", [(1, 150, 333), (4, 1000, 49), (2, 65, 7), (3, 257, 100), (1, 4100, 3), (1, 66, 65536)])
+def test_softmax_columns_sliced(gpu, n, c, plane):
+    """Few columns of many feature maps: a column is shared out over 16 lanes whose partial sums are
+    added in slice order, so the bar is the one stated for softmax, 1e-5 relative."""
+    gen = T.rng(15, n * 100000 + c * 100 + plane)
+    x = T.normal(gen, (n, c, plane), 4.0)
+    x[gen.random((n, c, plane)) < 0.01] = 30.0
+    want = oracle.softmax(x)
+    got = run_softmax(gpu, x)
+    assert_softmax_close(got, want, "softmax sliced columns")
+    assert np.abs(got.astype(np.float64).sum(axis=1) - 1.0).max() < c * 2.0 ** -24
+    assert T.bit_mismatches(run_softmax(gpu, x, in_place=True), got) == 0
 
 
 def test_softmax_special_rows(gpu):
@@ -381,8 +398,12 @@ def test_softmax_special_rows(gpu):
     assert abs(float(got[0, 0, 0]) - 1.0 / c) < 1e-9
     assert got[3, 7, 0] > 0.999999
     assert T.bit_mismatches(got[4], got[5]) == 0  # x - max is the same number in both rows
-    cols = np.repeat(rows.transpose(2, 1, 0), 3, axis=0).copy()  # the same data laid out as columns
-    assert T.bit_mismatches(run_softmax(gpu, cols), oracle.softmax(cols)) == 0
+    cols = np.repeat(rows.transpose(2, 1, 0), 3, axis=0).copy()  # the same data laid out as columns (sliced kernel)
+    got_cols = run_softmax(gpu, cols)
+    assert_softmax_close(got_cols, oracle.softmax(cols), "softmax special columns")
+    assert T.bit_mismatches(np.isnan(got_cols), np.isnan(oracle.softmax(cols))) == 0
+    narrow = np.ascontiguousarray(cols[:, :60, :])                # 60 feature maps: one lane per column, bit-exact
+    assert T.bit_mismatches(run_softmax(gpu, narrow), oracle.softmax(narrow)) == 0
 
 
 # ---------------------------------------------------------------------------------------------
