@@ -104,6 +104,8 @@ namespace nnf
 		uint32_t output_entry_count, uint32_t input_feature_map_count, uint32_t dimension_count,
 		const uint32_t* input_sizes, const uint32_t* subsampling_sizes, const uint32_t* strides, const uint32_t* round_ups,
 		uint32_t feature_map_subsampling_size, uint32_t entry_subsampling_size, int32_t is_min);
+	bool window2d_launch(hipStream_t stream, int op, float mult, float* output, const float* input, uint32_t input_total, uint32_t plane_count,
+		uint32_t in_w, uint32_t in_h, uint32_t out_w, uint32_t out_h, uint32_t win_w, uint32_t win_h, uint32_t stride_x, uint32_t stride_y);
 	int feature_map_stat_init(hipStream_t stream, nnf_hip_running_stat* device_stats, uint32_t feature_map_count);
 	int feature_map_stat_workspace_bytes(uint32_t entry_count, uint32_t feature_map_count, uint32_t neuron_count_per_feature_map, size_t* bytes);
 	int feature_map_stat_accumulate(hipStream_t stream, nnf_hip_running_stat* device_stats, void* workspace, size_t workspace_bytes,

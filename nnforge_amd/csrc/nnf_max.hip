@@ -27,6 +27,29 @@ namespace nnf
 			return (current < new_val) ? new_val : current;
 		}
 
+		// What the LDS-staged 2-D window kernel does with the values of a window, scanned x fastest:
+		// maximum, minimum (both from the -/+1.0e37F start value), or their left-to-right sum times a
+		// multiplier (average subsampling, nnforge/plain/average_subsampling_layer_tester_plain.cpp:125-145).
+		constexpr int window_op_max = 0;
+		constexpr int window_op_min = 1;
+		constexpr int window_op_sum = 2;
+
+		template<int OP>
+		__device__ __forceinline__ float window_fold(float current, float new_val)
+		{
+			if (OP == window_op_sum)
+				return current + new_val;
+			return fold<OP == window_op_min>(current, new_val);
+		}
+
+		template<int OP>
+		__device__ __forceinline__ float window_fold_start()
+		{
+			if (OP == window_op_sum)
+				return 0.0f;
+			return (OP == window_op_min) ? 1.0e37f : -1.0e37f;
+		}
+
 		// n / divisor with magic = ceil(2^32 / divisor), exact while n * divisor < 2^32
 		__device__ __forceinline__ uint32_t fast_divide(uint32_t n, uint32_t divisor, uint32_t magic)
 		{
@@ -59,13 +82,15 @@ namespace nnf
 			uint32_t bands;           // ceil(out_h / rows)
 			uint32_t out_w_magic;     // ceil(2^32 / out_w)
 			uint32_t band_magic;      // ceil(2^32 / (rows * out_w)): outputs per plane inside a workgroup
+			float mult;               // window_op_sum: the sum is multiplied by it
 		};
 
 		constexpr int stage_vectors_per_lane = 8; // float4 loads a lane has in flight while staging
 
 		// WIN_W, WIN_H: window size known at compile time, 0: read it from the arguments.
-		// TRUNC: windows may reach beyond the input (round up) and are cut off there.
-		template<bool IS_MIN, int WIN_W, int WIN_H, bool TRUNC>
+		// TRUNC: windows may reach beyond the input (round up) and are cut off there (maximum and
+		// minimum only: repeating a value would change a sum).
+		template<int OP, int WIN_W, int WIN_H, bool TRUNC>
 		__global__ void __launch_bounds__(max_block_size) max_window2d_kernel(const window2d_args a)
 		{
 			extern __shared__ __align__(16) float lds_in[];
@@ -141,7 +166,8 @@ namespace nnf
 				// nothing, so this equals skipping the position.
 				const uint32_t last_x = TRUNC ? min(win_w, a.in_w - x0) - 1 : 0u;
 				const uint32_t last_y = TRUNC ? min(win_h, a.in_h - y0) - 1 : 0u;
-				float current = fold_start<IS_MIN>();
+				static_assert(!(TRUNC && (OP == window_op_sum)), "a truncated window re-reads values");
+				float current = window_fold_start<OP>();
 				if ((WIN_W > 0) && (WIN_H > 0))
 				{
 					#pragma unroll
@@ -150,7 +176,7 @@ namespace nnf
 						const float* row = src + (TRUNC ? min(static_cast<uint32_t>(y), last_y) : static_cast<uint32_t>(y)) * a.in_w;
 						#pragma unroll
 						for(int x = 0; x < WIN_W; ++x)
-							current = fold<IS_MIN>(current, row[TRUNC ? min(static_cast<uint32_t>(x), last_x) : static_cast<uint32_t>(x)]);
+							current = window_fold<OP>(current, row[TRUNC ? min(static_cast<uint32_t>(x), last_x) : static_cast<uint32_t>(x)]);
 					}
 				}
 				else
@@ -159,9 +185,9 @@ namespace nnf
 					const uint32_t fit_h = TRUNC ? last_y + 1 : win_h;
 					for(uint32_t y = 0; y < fit_h; ++y)
 						for(uint32_t x = 0; x < fit_w; ++x)
-							current = fold<IS_MIN>(current, src[y * a.in_w + x]);
+							current = window_fold<OP>(current, src[y * a.in_w + x]);
 				}
-				dst[o] = current;
+				dst[o] = (OP == window_op_sum) ? current * a.mult : current;
 			}
 		}
 
@@ -275,15 +301,15 @@ namespace nnf
 			return (divisor >= 2) ? static_cast<uint32_t>(((1ull << 32) + divisor - 1) / divisor) : 0u; // fast_divide does not use it for 1
 		}
 
-		template<bool IS_MIN, bool TRUNC>
+		template<int OP, bool TRUNC>
 		void launch_window2d(hipStream_t stream, const window2d_args& a, uint32_t grid, size_t lds_bytes)
 		{
 			if ((a.win_w == 3) && (a.win_h == 3))
-				hipLaunchKernelGGL((max_window2d_kernel<IS_MIN, 3, 3, TRUNC>), dim3(grid), dim3(max_block_size), lds_bytes, stream, a);
+				hipLaunchKernelGGL((max_window2d_kernel<OP, 3, 3, TRUNC>), dim3(grid), dim3(max_block_size), lds_bytes, stream, a);
 			else if ((a.win_w == 2) && (a.win_h == 2))
-				hipLaunchKernelGGL((max_window2d_kernel<IS_MIN, 2, 2, TRUNC>), dim3(grid), dim3(max_block_size), lds_bytes, stream, a);
+				hipLaunchKernelGGL((max_window2d_kernel<OP, 2, 2, TRUNC>), dim3(grid), dim3(max_block_size), lds_bytes, stream, a);
 			else
-				hipLaunchKernelGGL((max_window2d_kernel<IS_MIN, 0, 0, TRUNC>), dim3(grid), dim3(max_block_size), lds_bytes, stream, a);
+				hipLaunchKernelGGL((max_window2d_kernel<OP, 0, 0, TRUNC>), dim3(grid), dim3(max_block_size), lds_bytes, stream, a);
 		}
 
 		// LDS floats a workgroup of the 2-D kernel stages; NNF_HIP_POOL_LDS_FLOATS overrides it (tuning)
@@ -297,6 +323,70 @@ namespace nnf
 			}();
 			return value;
 		}
+	}
+
+	// Plans and launches the LDS-staged 2-D window kernel. op: 0 maximum, 1 minimum, 2 maximum with
+	// windows cut off at the input edge (round up), 3 minimum likewise, 4 sum times mult. Returns
+	// false (nothing launched) when the shape does not suit the kernel: more than 65535 outputs per
+	// plane, or a single band of window_height input rows that does not fit LDS.
+	bool window2d_launch(hipStream_t stream, int op, float mult, float* output, const float* input, uint32_t input_total, uint32_t plane_count,
+		uint32_t in_w, uint32_t in_h, uint32_t out_w, uint32_t out_h, uint32_t win_w, uint32_t win_h, uint32_t stride_x, uint32_t stride_y)
+	{
+		const uint32_t lds_floats_wanted = staging_floats();
+		constexpr uint32_t lds_floats_max = 15 * 1024;
+		if (static_cast<uint64_t>(out_w) * out_h >= (1u << 16))
+			return false;
+		window2d_args a = {};
+		a.out = output;
+		a.in = input;
+		a.total_in = input_total;
+		a.plane_count = plane_count;
+		a.in_w = in_w; a.in_h = in_h;
+		a.out_w = out_w; a.out_h = out_h;
+		a.win_w = win_w; a.win_h = win_h;
+		a.stride_x = stride_x; a.stride_y = stride_y;
+		a.mult = mult;
+		const uint32_t plane = a.in_w * a.in_h;
+		bool fits = true;
+		if (plane <= lds_floats_wanted)
+		{
+			// whole planes; enough of them for a few outputs per lane, few enough to keep the grid wide
+			a.planes = std::max(1u, std::min(lds_floats_wanted / plane, (4u * max_block_size + a.out_w * a.out_h - 1) / (a.out_w * a.out_h)));
+			a.rows = a.out_h;
+		}
+		else
+		{
+			a.planes = 1;
+			// rows per band: input rows needed = (rows - 1) * stride_y + win_h
+			const uint32_t rows_in = lds_floats_wanted / a.in_w;
+			a.rows = (rows_in >= a.win_h) ? (rows_in - a.win_h) / a.stride_y + 1 : 0;
+			if (a.rows == 0)
+			{
+				a.rows = 1;
+				fits = static_cast<uint64_t>(a.win_h) * a.in_w + 4 <= lds_floats_max;
+			}
+			a.rows = std::min(a.rows, a.out_h);
+			// bands of equal height
+			const uint32_t bands = (a.out_h + a.rows - 1) / a.rows;
+			a.rows = (a.out_h + bands - 1) / bands;
+		}
+		if (!fits)
+			return false;
+		a.bands = (a.out_h + a.rows - 1) / a.rows;
+		a.out_w_magic = magic_of(a.out_w);
+		a.band_magic = magic_of(a.rows * a.out_w);
+		const uint32_t rows_in = (a.planes > 1 || a.bands == 1) ? a.in_h : std::min(a.in_h, (a.rows - 1) * a.stride_y + a.win_h);
+		const size_t lds_bytes = (static_cast<size_t>(a.planes - 1) * plane + static_cast<size_t>(rows_in) * a.in_w + 8) * sizeof(float);
+		const uint32_t grid = ((a.plane_count + a.planes - 1) / a.planes) * a.bands;
+		switch (op)
+		{
+		case 0: launch_window2d<window_op_max, false>(stream, a, grid, lds_bytes); break;
+		case 1: launch_window2d<window_op_min, false>(stream, a, grid, lds_bytes); break;
+		case 2: launch_window2d<window_op_max, true>(stream, a, grid, lds_bytes); break;
+		case 3: launch_window2d<window_op_min, true>(stream, a, grid, lds_bytes); break;
+		default: launch_window2d<window_op_sum, false>(stream, a, grid, lds_bytes); break;
+		}
+		return true;
 	}
 
 	int max_subsampling_forward(hipStream_t stream, float* output, const float* input,
@@ -351,64 +441,13 @@ namespace nnf
 			return NNF_HIP_EOVERLAP;
 
 		// 2-D (or 1-D) windows within a feature map: stage through LDS
-		const uint32_t lds_floats_wanted = staging_floats();
-		constexpr uint32_t lds_floats_max = 15 * 1024;
 		const bool within_plane = (feature_map_subsampling_size == 1) && (entry_subsampling_size == 1) && (dimension_count <= 2);
-		if (within_plane && (nd.out_size[0] * nd.out_size[1] < (1u << 16)))
+		if (within_plane)
 		{
-			window2d_args a = {};
-			a.out = output;
-			a.in = input;
-			a.total_in = static_cast<uint32_t>(input_total);
-			a.plane_count = output_entry_count * input_feature_map_count;
-			a.in_w = nd.in_size[0]; a.in_h = nd.in_size[1];
-			a.out_w = nd.out_size[0]; a.out_h = nd.out_size[1];
-			a.win_w = nd.window[0]; a.win_h = nd.window[1];
-			a.stride_x = nd.stride[0]; a.stride_y = nd.stride[1];
-			const uint32_t plane = a.in_w * a.in_h;
-			bool fits = true;
-			if (plane <= lds_floats_wanted)
-			{
-				// whole planes; enough of them for a few outputs per lane, few enough to keep the grid wide
-				a.planes = std::max(1u, std::min(lds_floats_wanted / plane, (4u * max_block_size + a.out_w * a.out_h - 1) / (a.out_w * a.out_h)));
-				a.rows = a.out_h;
-			}
-			else
-			{
-				a.planes = 1;
-				// rows per band: input rows needed = (rows - 1) * stride_y + win_h
-				const uint32_t rows_in = lds_floats_wanted / a.in_w;
-				a.rows = (rows_in >= a.win_h) ? (rows_in - a.win_h) / a.stride_y + 1 : 0;
-				if (a.rows == 0)
-				{
-					a.rows = 1;
-					fits = static_cast<uint64_t>(a.win_h) * a.in_w + 4 <= lds_floats_max;
-				}
-				a.rows = std::min(a.rows, a.out_h);
-				// bands of equal height
-				const uint32_t bands = (a.out_h + a.rows - 1) / a.rows;
-				a.rows = (a.out_h + bands - 1) / bands;
-			}
-			if (fits)
-			{
-				a.bands = (a.out_h + a.rows - 1) / a.rows;
-				a.out_w_magic = magic_of(a.out_w);
-				a.band_magic = magic_of(a.rows * a.out_w);
-				const uint32_t rows_in = (a.planes > 1 || a.bands == 1) ? a.in_h : std::min(a.in_h, (a.rows - 1) * a.stride_y + a.win_h);
-				const size_t lds_bytes = (static_cast<size_t>(a.planes - 1) * plane + static_cast<size_t>(rows_in) * a.in_w + 8) * sizeof(float);
-				const uint32_t grid = ((a.plane_count + a.planes - 1) / a.planes) * a.bands;
-				if (is_min)
-				{
-					if (round_up_anywhere) launch_window2d<true, true>(stream, a, grid, lds_bytes);
-					else launch_window2d<true, false>(stream, a, grid, lds_bytes);
-				}
-				else
-				{
-					if (round_up_anywhere) launch_window2d<false, true>(stream, a, grid, lds_bytes);
-					else launch_window2d<false, false>(stream, a, grid, lds_bytes);
-				}
+			const int op = is_min ? (round_up_anywhere ? 3 : 1) : (round_up_anywhere ? 2 : 0);
+			if (window2d_launch(stream, op, 0.0f, output, input, static_cast<uint32_t>(input_total), output_entry_count * input_feature_map_count,
+				nd.in_size[0], nd.in_size[1], nd.out_size[0], nd.out_size[1], nd.window[0], nd.window[1], nd.stride[0], nd.stride[1]))
 				return launch_status();
-			}
 		}
 
 		nd.out = output;

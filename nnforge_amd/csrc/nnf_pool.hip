@@ -1,7 +1,9 @@
 // 2-D average subsampling with non-overlapping windows
 // (nnforge/plain/average_subsampling_layer_tester_plain.cpp:125-145): every output is the
-// left-to-right fp32 sum of its window (x fastest, then y) multiplied by mult. Both kernels keep
-// that summation order, so results equal the reference's bit for bit.
+// left-to-right fp32 sum of its window (x fastest, then y) multiplied by mult. All kernels keep
+// that summation order, so results equal the reference's bit for bit. Windows smaller than the
+// plane go through the LDS-staged 2-D window kernel shared with max subsampling (nnf_max.hip);
+// the one-lane-per-output kernel below remains for the shapes that kernel declines.
 #include "nnf_common.h"
 
 namespace nnf
@@ -142,6 +144,11 @@ namespace nnf
 			// plane >= 2 here: a 1x1 window over a 1x1 plane takes the general kernel
 			const uint32_t plane_magic = static_cast<uint32_t>(((1ull << 32) + plane - 1) / plane);
 			hipLaunchKernelGGL(global_pool_kernel, grid, dim3(pool_block_size), lds_bytes, stream, output, input, plane_count, plane, plane_magic, mult);
+		}
+		else if (window2d_launch(stream, 4, mult, output, input, static_cast<uint32_t>(input_total), plane_count,
+			input_width, input_height, output_width, output_height, window_width, window_height, window_width, window_height))
+		{
+			// staged through LDS by the 2-D window kernel: contiguous float4 reads, windows summed x fastest
 		}
 		else
 		{

@@ -432,7 +432,12 @@ def test_global_average_7x7(gpu, n, c):
 
 
 @pytest.mark.parametrize("shape,ww,wh", [((2, 3, 8, 8), 2, 2), ((1, 4, 9, 7), 3, 2), ((2, 2, 6, 10), 5, 3), ((1, 2, 4, 4), 4, 4),
-                                         ((3, 3, 5, 12), 12, 5), ((1, 1, 30, 30), 30, 30), ((2, 5, 16, 16), 1, 1), ((1, 3, 7, 9), 2, 3)])
+                                         ((3, 3, 5, 12), 12, 5), ((1, 1, 30, 30), 30, 30), ((2, 5, 16, 16), 1, 1), ((1, 3, 7, 9), 2, 3),
+                                         # planes larger than a workgroup's staging buffer (bands of rows), leftover margins
+                                         ((1, 2, 120, 100), 2, 2), ((2, 3, 113, 115), 3, 3), ((1, 1, 300, 70), 7, 5), ((2, 2, 56, 56), 2, 2),
+                                         ((1, 2, 97, 4100), 4, 3),
+                                         # more than 65535 outputs per plane: the one-lane-per-output kernel
+                                         ((1, 1, 300, 300), 1, 1), ((1, 1, 520, 260), 2, 1)])
 def test_average_subsampling_windows(gpu, shape, ww, wh):
     x = T.normal(T.rng(16, sum(shape) + ww), shape)
     mult = oracle.average_subsampling_full_mult([ww, wh])
