@@ -208,10 +208,8 @@ namespace nnf
 		};
 		constexpr int known_program_count = sizeof(known_programs) / sizeof(known_programs[0]);
 
-		// One tile of the tensor. FULL: every float4 of the tile lies inside the tensor, so loads and
-		// stores are unconditional (the ragged last tile takes the other instance).
-		template<int NIN, int BLOCK, int U, bool DIRECT, int PROGRAM, bool FULL>
-		__device__ __forceinline__ void chain_tile(const chain_args& a)
+		template<int NIN, int BLOCK, int U, bool DIRECT, int PROGRAM>
+		__global__ void __launch_bounds__(BLOCK) chain_kernel(const chain_args a)
 		{
 			constexpr int TILE = BLOCK * U * 4;
 			constexpr int PL = DIRECT ? 1 : 4;
@@ -220,16 +218,14 @@ namespace nnf
 			float2* lds_coeff = reinterpret_cast<float2*>(lds_raw + exp_table_bytes);
 
 			const uint32_t tile_start = blockIdx.x * static_cast<uint32_t>(TILE);
-			const uint32_t first_plane = tile_start / a.plane;
-			const uint32_t start_in_plane = tile_start - first_plane * a.plane;
-			const uint32_t first_fm = first_plane % a.fm_count;
 
-			// All loads are issued before anything else, oldest first: the lane's expf table entry, the
-			// tensors, then (compile-time programs) the weights of a leading batch norm.
-			constexpr bool program_has_exp = PROGRAM > 0; // every compile-time program calls expf
-			uint64_t exp_entry = 0;
-			if (program_has_exp || a.need_exp)
-				exp_entry = load_exp2_table_entry();
+			// All loads are issued before anything else: the tensors first (nothing but the tile index
+			// goes into their addresses), then the lane's expf table entry and (compile-time programs) the
+			// weights of a leading batch norm; the index arithmetic runs while they are in flight.
+			// Only one float4 of the whole tensor can be partial: the one that starts at tail_start when the
+			// element count is not a multiple of four. Its up to three values travel through scalar loads
+			// and stores of their own, so that every other access is a float4 guarded by one comparison.
+			const uint32_t tail_start = a.total & ~3u;
 			float x[NIN][U][4];
 			#pragma unroll
 			for(int j = 0; j < NIN; ++j)
@@ -238,19 +234,45 @@ namespace nnf
 				for(int k = 0; k < U; ++k)
 				{
 					const uint32_t idx = tile_start + (threadIdx.x + k * BLOCK) * 4;
-					if (FULL || (idx + 3 < a.total))
+					floatx4 t = {0.0f, 0.0f, 0.0f, 0.0f};
+					if (idx < tail_start)
+						t = load_stream(reinterpret_cast<const floatx4*>(a.in[j] + idx));
+					x[j][k][0] = t.x; x[j][k][1] = t.y; x[j][k][2] = t.z; x[j][k][3] = t.w;
+				}
+			}
+			// float4 index of the partial vector inside this tile, if it is here
+			const uint32_t tail_vector = (tail_start - tile_start) / 4;
+			const bool owns_tail = (tail_start != a.total) && (tail_start >= tile_start) && (tail_vector < static_cast<uint32_t>(BLOCK * U))
+				&& ((tail_vector % BLOCK) == threadIdx.x);
+			if (owns_tail)
+			{
+				const uint32_t k_tail = tail_vector / BLOCK;
+				#pragma unroll
+				for(int j = 0; j < NIN; ++j)
+				{
+					float tail[3];
+					#pragma unroll
+					for(int e = 0; e < 3; ++e)
+						tail[e] = (tail_start + e < a.total) ? a.in[j][tail_start + e] : 0.0f;
+					#pragma unroll
+					for(int k = 0; k < U; ++k)
 					{
-						const floatx4 t = load_stream(reinterpret_cast<const floatx4*>(a.in[j] + idx));
-						x[j][k][0] = t.x; x[j][k][1] = t.y; x[j][k][2] = t.z; x[j][k][3] = t.w;
-					}
-					else
-					{
-						#pragma unroll
-						for(int e = 0; e < 4; ++e)
-							x[j][k][e] = (idx + e < a.total) ? a.in[j][idx + e] : 0.0f;
+						if (static_cast<uint32_t>(k) == k_tail)
+						{
+							x[j][k][0] = tail[0]; x[j][k][1] = tail[1]; x[j][k][2] = tail[2];
+						}
 					}
 				}
 			}
+
+			constexpr bool program_has_exp = PROGRAM > 0; // every compile-time program calls expf
+			uint64_t exp_entry = 0;
+			if (program_has_exp || a.need_exp)
+				exp_entry = load_exp2_table_entry();
+
+			const uint32_t first_plane = tile_start / a.plane;
+			const uint32_t start_in_plane = tile_start - first_plane * a.plane;
+			const uint32_t first_fm = first_plane % a.fm_count;
 
 			uint32_t where[U][PL];
 			#pragma unroll
@@ -371,30 +393,28 @@ namespace nnf
 			for(int k = 0; k < U; ++k)
 			{
 				const uint32_t idx = tile_start + (threadIdx.x + k * BLOCK) * 4;
-				if (FULL || (idx + 3 < a.total))
+				if (idx < tail_start)
 				{
 					floatx4 t;
 					t.x = x[0][k][0]; t.y = x[0][k][1]; t.z = x[0][k][2]; t.w = x[0][k][3];
 					store_stream(reinterpret_cast<floatx4*>(a.out + idx), t);
 				}
-				else
+			}
+			if (owns_tail)
+			{
+				const uint32_t k_tail = tail_vector / BLOCK;
+				#pragma unroll
+				for(int k = 0; k < U; ++k)
 				{
-					#pragma unroll
-					for(int e = 0; e < 4; ++e)
-						if (idx + e < a.total)
-							a.out[idx + e] = x[0][k][e];
+					if (static_cast<uint32_t>(k) == k_tail)
+					{
+						#pragma unroll
+						for(int e = 0; e < 3; ++e)
+							if (tail_start + e < a.total)
+								a.out[tail_start + e] = x[0][k][e];
+					}
 				}
 			}
-		}
-
-		template<int NIN, int BLOCK, int U, bool DIRECT, int PROGRAM>
-		__global__ void __launch_bounds__(BLOCK) chain_kernel(const chain_args a)
-		{
-			constexpr uint32_t tile = BLOCK * U * 4;
-			if (blockIdx.x * tile + tile <= a.total) // total <= 0xFFFF0000: the sum does not wrap
-				chain_tile<NIN, BLOCK, U, DIRECT, PROGRAM, true>(a);
-			else
-				chain_tile<NIN, BLOCK, U, DIRECT, PROGRAM, false>(a);
 		}
 
 		typedef void (*chain_kernel_fn)(const chain_args);
