@@ -68,6 +68,34 @@ namespace nnf
 			return __umulhi(e, plane_magic);
 		}
 
+		// DIRECT path: the COUNT weights of the feature map of each float4 a lane holds. When all lanes
+		// of the wavefront agree on the feature map of float4 k (a plane is many wavefront rows long, so
+		// they do except where a row crosses a plane boundary), the weights are fetched once per
+		// wavefront through the scalar cache and stay out of the vector memory pipeline that streams
+		// the tensors; otherwise every lane reads its own.
+		template<int U, int COUNT>
+		__device__ __forceinline__ void load_direct_weights(const chain_slot& slot, const uint32_t (&where)[U][1], float (&w)[U][COUNT])
+		{
+			#pragma unroll
+			for(int k = 0; k < U; ++k)
+			{
+				const uint32_t fm = where[k][0];
+				const uint32_t wave_fm = __builtin_amdgcn_readfirstlane(fm);
+				if (__all(fm == wave_fm))
+				{
+					#pragma unroll
+					for(int c = 0; c < COUNT; ++c)
+						w[k][c] = slot.p[c][wave_fm];
+				}
+				else
+				{
+					#pragma unroll
+					for(int c = 0; c < COUNT; ++c)
+						w[k][c] = slot.p[c][fm];
+				}
+			}
+		}
+
 		// Applies one layer to the U float4s a lane holds. The switch is uniform across the workgroup.
 		// DIRECT: where[k][0] is the feature map of float4 k and per-feature-map weights are read from
 		// memory (all lanes of a wavefront read the same one or two addresses: one cache line).
@@ -87,13 +115,13 @@ namespace nnf
 			case NNF_HIP_OP_BATCH_NORM:
 				if (DIRECT)
 				{
-					const chain_slot& slot = a.slots[op.slot];
+					float w[U][4];
+					load_direct_weights<U, 4>(a.slots[op.slot], reinterpret_cast<const uint32_t (&)[U][1]>(where), w);
 					#pragma unroll
 					for(int k = 0; k < U; ++k)
 					{
-						const uint32_t fm = where[k][0];
 						float mult, add;
-						nnf_batch_norm_coefficients(slot.p[0][fm], slot.p[1][fm], slot.p[2][fm], slot.p[3][fm], mult, add);
+						nnf_batch_norm_coefficients(w[k][0], w[k][1], w[k][2], w[k][3], mult, add);
 						#pragma unroll
 						for(int e = 0; e < 4; ++e)
 							v[k][e] = nnf_batch_norm(v[k][e], mult, add);
@@ -126,14 +154,14 @@ namespace nnf
 			case NNF_HIP_OP_PRELU:
 				if (DIRECT)
 				{
-					const float* slopes = a.slots[op.slot].p[0];
+					float w[U][1];
+					load_direct_weights<U, 1>(a.slots[op.slot], reinterpret_cast<const uint32_t (&)[U][1]>(where), w);
 					#pragma unroll
 					for(int k = 0; k < U; ++k)
 					{
-						const float slope = slopes[where[k][0]];
 						#pragma unroll
 						for(int e = 0; e < 4; ++e)
-							v[k][e] = nnf_parametric_rectified_linear(v[k][e], slope);
+							v[k][e] = nnf_parametric_rectified_linear(v[k][e], w[k][0]);
 					}
 				}
 				else
@@ -297,14 +325,7 @@ namespace nnf
 			float lead_weights[U][4] = {};
 			if (leading_batch_norm)
 			{
-				const chain_slot& slot = a.slots[a.ops[0].slot];
-				#pragma unroll
-				for(int k = 0; k < U; ++k)
-				{
-					#pragma unroll
-					for(int c = 0; c < 4; ++c)
-						lead_weights[k][c] = slot.p[c][where[k][0]];
-				}
+				load_direct_weights<U, 4>(a.slots[a.ops[0].slot], reinterpret_cast<const uint32_t (&)[U][1]>(where), lead_weights);
 			}
 
 			// expf table: one private copy per wavefront, so the direct path has no workgroup barrier
