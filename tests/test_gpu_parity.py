@@ -247,6 +247,33 @@ def test_expf_dense_sweep_through_elu_and_sigmoid(gpu):
     check_exact(run_flat(gpu, gpu.lib.nnf_hip_sigmoid_forward, -x), oracle.sigmoid(-x), "sigmoid sweep (positive)")
 
 
+def test_exp_range_edges_dense(gpu):
+    """Every fp32 in windows around the arguments where the device code changes path: |x| = 87 (range
+    repair branch), expf(x) + 1 = 2^126 (x = 87.34: the short division sequences end), log(2^128)
+    (expf overflows, TanH turns NaN), log(2^-126) and log(2^-150) (expf results go subnormal, then 0) -
+    with ordinary values in the same wavefronts, so that both sides of every wavefront-uniform
+    branch hold live lanes."""
+    windows = []
+    for centre in (87.0, 87.336, 88.7228, -87.0, -87.3365, -103.972):
+        first = int(np.array(centre, dtype=np.float32).view(np.uint32)) - (1 << 15)
+        windows.append(np.arange(first, first + (1 << 16), dtype=np.uint32))
+    edge = np.concatenate(windows).view(np.float32)
+    x = np.empty(edge.size * 2, np.float32)
+    x[0::2] = edge
+    x[1::2] = T.normal(T.rng(17, 0), edge.size, 2.0)  # every other lane holds an ordinary value
+    with np.errstate(all="ignore"):
+        for sign in (1.0, -1.0):
+            v = (x * np.float32(sign)).astype(np.float32)
+            check_exact(run_flat(gpu, gpu.lib.nnf_hip_exponential_linear_forward, v), oracle.exponential_linear(v), "elu edges")
+            check_exact(run_flat(gpu, gpu.lib.nnf_hip_sigmoid_forward, v), oracle.sigmoid(v), "sigmoid edges")
+            check_exact(run_flat(gpu, gpu.lib.nnf_hip_hyperbolic_tangent_forward, v, 1.0, 0.5), oracle.hyperbolic_tangent(v, 1.0, 0.5), "tanh edges")
+            check_exact(run_flat(gpu, gpu.lib.nnf_hip_hyperbolic_tangent_forward, v, T.TANH_SCALE, T.TANH_STEEPNESS),
+                        oracle.hyperbolic_tangent(v, T.TANH_SCALE, T.TANH_STEEPNESS), "tanh edges, scaled")
+        rows = edge[: (edge.size // 1000) * 1000].reshape(-1, 1000, 1)  # row softmax: x - max crosses the same edges
+        got = run_softmax(gpu, np.ascontiguousarray(-np.abs(rows)))
+        assert_softmax_close(got, oracle.softmax(np.ascontiguousarray(-np.abs(rows))), "softmax edges")
+
+
 @pytest.mark.parametrize("input_count", [1, 2, 3, 4, 5, 8, 9])
 @pytest.mark.parametrize("size,alpha", [(5, 1.0), (4099, 0.5), (1 << 18, -1.25)])
 def test_add_entry_point(gpu, input_count, size, alpha):
