@@ -331,6 +331,75 @@ namespace nnf
 			}
 		}
 
+		// Columns of up to 16 feature maps when the plane is a multiple of four (more would cost occupancy): a lane takes four neighbouring
+		// positions, so every access is a float4 (1 KiB per wavefront) and four independent columns
+		// keep the expf pipeline busy. Same operation order per column as above: bit-exact.
+		template<int CACHED>
+		__global__ void __launch_bounds__(256) softmax_columns_vec4_kernel(float* out, const float* in, uint32_t column_quads, uint32_t fm_count, uint32_t plane)
+		{
+			__shared__ uint64_t lds_exp[exp_lds_entries];
+			stage_exp2_table(lds_exp);
+			__syncthreads();
+			const exp_context exp_ctx = exp_context_from_lds(lds_exp);
+
+			const uint32_t quad = blockIdx.x * blockDim.x + threadIdx.x;
+			if (quad >= column_quads)
+				return;
+			const uint32_t quads_per_plane = plane / 4;
+			const uint32_t entry = quad / quads_per_plane;
+			const uint32_t pos = (quad - entry * quads_per_plane) * 4;
+			const size_t base = static_cast<size_t>(entry) * fm_count * plane + pos;
+			const float* src = in + base;
+			float* dst = out + base;
+			const uint32_t last = fm_count - 1;
+
+			float v[CACHED][4];
+			#pragma unroll
+			for(int c = 0; c < CACHED; ++c)
+			{
+				const floatx4 t = load_stream(reinterpret_cast<const floatx4*>(src + static_cast<size_t>(min(static_cast<uint32_t>(c), last)) * plane));
+				v[c][0] = t.x; v[c][1] = t.y; v[c][2] = t.z; v[c][3] = t.w;
+			}
+			float m[4] = { softmax_max_init, softmax_max_init, softmax_max_init, softmax_max_init };
+			#pragma unroll
+			for(int c = 0; c < CACHED; ++c)
+			{
+				#pragma unroll
+				for(int e = 0; e < 4; ++e)
+					m[e] = ref_max(m[e], v[c][e]);
+			}
+			float sum[4] = { 0.0f, 0.0f, 0.0f, 0.0f };
+			#pragma unroll
+			for(int c = 0; c < CACHED; ++c)
+			{
+				if (static_cast<uint32_t>(c) < fm_count) // uniform
+				{
+					float x[4];
+					#pragma unroll
+					for(int e = 0; e < 4; ++e)
+						x[e] = v[c][e] - m[e];
+					nnf_expf_batch<4>(x, v[c], exp_ctx);
+					#pragma unroll
+					for(int e = 0; e < 4; ++e)
+						sum[e] += v[c][e];
+				}
+			}
+			float mult[4];
+			#pragma unroll
+			for(int e = 0; e < 4; ++e)
+				mult[e] = 1.0f / sum[e];
+			#pragma unroll
+			for(int c = 0; c < CACHED; ++c)
+			{
+				if (static_cast<uint32_t>(c) < fm_count) // uniform
+				{
+					floatx4 t;
+					t.x = v[c][0] * mult[0]; t.y = v[c][1] * mult[1]; t.z = v[c][2] * mult[2]; t.w = v[c][3] * mult[3];
+					store_stream(reinterpret_cast<floatx4*>(dst + static_cast<size_t>(c) * plane), t);
+				}
+			}
+		}
+
 		// neuron_count_per_feature_map > 1 with few columns and many feature maps: one lane per column
 		// would leave most of the machine idle and make every lane walk a long column alone. A
 		// workgroup of 256 lanes takes P consecutive columns; the feature maps are cut into S = 256 / P
@@ -539,6 +608,21 @@ namespace nnf
 			const uint32_t block_size = (columns >= 256u * 1024u) ? 256u : 64u;
 			const dim3 block(block_size);
 			const dim3 grid((columns + block_size - 1) / block_size);
+			if (((neuron_count_per_feature_map % 4) == 0) && (feature_map_count <= 16) && (columns >= 4u * 64u * 1024u))
+			{
+				// four positions per lane while that still leaves every compute unit several wavefronts
+				const uint32_t quads = columns / 4;
+				const dim3 quad_grid((quads + 255) / 256);
+				if (feature_map_count <= 2)
+					hipLaunchKernelGGL(softmax_columns_vec4_kernel<2>, quad_grid, dim3(256), 0, stream, output, input, quads, feature_map_count, neuron_count_per_feature_map);
+				else if (feature_map_count <= 4)
+					hipLaunchKernelGGL(softmax_columns_vec4_kernel<4>, quad_grid, dim3(256), 0, stream, output, input, quads, feature_map_count, neuron_count_per_feature_map);
+				else if (feature_map_count <= 8)
+					hipLaunchKernelGGL(softmax_columns_vec4_kernel<8>, quad_grid, dim3(256), 0, stream, output, input, quads, feature_map_count, neuron_count_per_feature_map);
+				else
+					hipLaunchKernelGGL(softmax_columns_vec4_kernel<16>, quad_grid, dim3(256), 0, stream, output, input, quads, feature_map_count, neuron_count_per_feature_map);
+				return launch_status();
+			}
 			if (feature_map_count <= 2)
 				hipLaunchKernelGGL(softmax_columns_kernel<2>, grid, block, 0, stream, output, input, columns, feature_map_count, neuron_count_per_feature_map);
 			else if (feature_map_count <= 4)

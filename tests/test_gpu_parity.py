@@ -380,7 +380,9 @@ def test_softmax_rows(gpu, n, c):
 
 
 @pytest.mark.parametrize("n,c,plane", [(2, 1, 5), (2, 2, 777), (2, 3, 2), (3, 4, 130), (1, 10, 49), (3, 16, 5), (2, 17, 64), (2, 21, 1000),
-                                       (3, 33, 300), (2, 64, 129), (1, 70, 70001), (4, 5, 4096)])
+                                       (3, 33, 300), (2, 64, 129), (1, 70, 70001), (4, 5, 4096),
+                                       # four positions per lane (plane a multiple of 4, at least 262144 columns, up to 16 feature maps)
+                                       (1, 2, 262144), (1, 3, 262148), (2, 8, 131072), (1, 16, 262144), (1, 17, 262144)])
 def test_softmax_columns_bit_exact(gpu, n, c, plane):
     """One lane per column (up to 64 feature maps, or more than 65536 columns): the reference's own
     left-to-right sum, so the bits are the oracle's."""
