@@ -400,18 +400,22 @@ namespace nnf
 			}
 		}
 
-		// neuron_count_per_feature_map > 1 with few columns and many feature maps: one lane per column
-		// would leave most of the machine idle and make every lane walk a long column alone. A
-		// workgroup of 256 lanes takes P consecutive columns; the feature maps are cut into S = 256 / P
-		// contiguous slices, lane (slice, position) walks its slice in batches of eight, and the slices
-		// are combined through LDS in slice order. The maximum is the reference's; the sum is S
-		// sequential partial sums added in order instead of one sequential sum, so results can differ
-		// from the reference in the last bits (bar: 1e-5 relative, as for rows).
-		template<int P>
+		// neuron_count_per_feature_map > 1 and more than 64 feature maps: one lane per column would make
+		// every lane walk a long column alone, with three passes over memory. A workgroup of 256 lanes
+		// takes P consecutive columns; the feature maps are cut into S = 256 / P contiguous slices, lane
+		// (slice, position) walks its slice in batches of eight, and the slices are combined through LDS
+		// in slice order. The maximum is the reference's; the sum is S sequential partial sums added in
+		// order instead of one sequential sum, so results can differ from the reference in the last bits
+		// (bar: 1e-5 relative, as for rows).
+		// STAGED: the workgroup's fm_count x P values stay in LDS between the passes (dynamic LDS of
+		// that size): one read and one write of memory. Otherwise the second and third pass re-read
+		// memory (small tensors: from the caches), expf values parked in the output.
+		template<int P, bool STAGED>
 		__global__ void __launch_bounds__(256) softmax_columns_sliced_kernel(float* out, const float* in, uint32_t columns, uint32_t fm_count, uint32_t plane)
 		{
 			constexpr int S = 256 / P;
 			constexpr int B = softmax_column_batch;
+			extern __shared__ __align__(16) float lds_values[]; // STAGED: [feature map][position]
 			__shared__ uint64_t lds_exp[exp_lds_entries];
 			__shared__ float lds_partial[2][S][P];
 			stage_exp2_table(lds_exp);
@@ -443,7 +447,11 @@ namespace nnf
 					x[i] = src[static_cast<size_t>(min(c0 + i, c_last)) * plane];
 				#pragma unroll
 				for(int i = 0; i < B; ++i)
+				{
 					m = ref_max(m, x[i]);
+					if (STAGED && (c0 + i < c_end))
+						lds_values[(c0 + i) * P + p] = x[i];
+				}
 			}
 			lds_partial[0][slice][p] = m;
 			__syncthreads();
@@ -458,7 +466,10 @@ namespace nnf
 				float x[B], e[B];
 				#pragma unroll
 				for(int i = 0; i < B; ++i)
-					x[i] = src[static_cast<size_t>(min(c0 + i, c_last)) * plane] - m;
+				{
+					const uint32_t c = min(c0 + i, c_last);
+					x[i] = (STAGED ? lds_values[c * P + p] : src[static_cast<size_t>(c) * plane]) - m;
+				}
 				nnf_expf_batch<B>(x, e, exp_ctx);
 				#pragma unroll
 				for(int i = 0; i < B; ++i)
@@ -466,7 +477,9 @@ namespace nnf
 					if (c0 + i < c_end)
 					{
 						sum += e[i];
-						if (valid)
+						if (STAGED)
+							lds_values[(c0 + i) * P + p] = e[i]; // a lane rewrites only what it wrote itself
+						else if (valid)
 							dst[static_cast<size_t>(c0 + i) * plane] = e[i];
 					}
 				}
@@ -486,7 +499,10 @@ namespace nnf
 				float x[B];
 				#pragma unroll
 				for(int i = 0; i < B; ++i)
-					x[i] = dst[static_cast<size_t>(min(c0 + i, c_last)) * plane];
+				{
+					const uint32_t c = min(c0 + i, c_last);
+					x[i] = STAGED ? lds_values[c * P + p] : dst[static_cast<size_t>(c) * plane];
+				}
 				#pragma unroll
 				for(int i = 0; i < B; ++i)
 				{
@@ -525,8 +541,11 @@ namespace nnf
 		// with 256 lanes per row against 4.3 us with one wavefront per row.
 		constexpr uint32_t few_rows = 2048;
 
-		// Columns (neuron_count_per_feature_map > 1) of more than 64 feature maps: up to this many
-		// columns the feature maps of a column are shared out over 16 lanes.
+		// Columns (neuron_count_per_feature_map > 1) of more than 64 feature maps are shared out over
+		// the lanes of a workgroup: always when the workgroup's values fit this much LDS (they are
+		// then read from memory once), otherwise up to this many columns (small tensors, re-read from
+		// the caches); beyond both, one lane walks a column in three passes.
+		constexpr size_t staged_bytes_limit = 60 * 1024;
 		constexpr uint32_t sliced_columns_limit = 65536;
 
 		template<int W>
@@ -592,17 +611,38 @@ namespace nnf
 		else
 		{
 			const uint32_t columns = entry_count * neuron_count_per_feature_map;
-			if ((feature_map_count > 64) && (columns <= sliced_columns_limit))
+			if (feature_map_count > 64)
 			{
 				// a whole wavefront along the positions (256-byte accesses) once that still gives every
-				// compute unit a few workgroups
-				if (columns >= 64u * 512u)
-					hipLaunchKernelGGL(softmax_columns_sliced_kernel<64>, dim3((columns + 63) / 64), dim3(256), 0, stream,
-						output, input, columns, feature_map_count, neuron_count_per_feature_map);
-				else
-					hipLaunchKernelGGL(softmax_columns_sliced_kernel<16>, dim3((columns + 15) / 16), dim3(256), 0, stream,
-						output, input, columns, feature_map_count, neuron_count_per_feature_map);
-				return launch_status();
+				// compute unit a few workgroups; fewer positions when that is what lets the values fit LDS
+				uint32_t positions = (columns >= 64u * 512u) ? 64u : 16u;
+				while ((positions > 16u) && (static_cast<size_t>(feature_map_count) * positions * sizeof(float) > staged_bytes_limit))
+					positions /= 2;
+				const size_t staged_bytes = static_cast<size_t>(feature_map_count) * positions * sizeof(float);
+				const dim3 sliced_grid((columns + positions - 1) / positions);
+				if (staged_bytes <= staged_bytes_limit)
+				{
+					if (positions == 64)
+						hipLaunchKernelGGL((softmax_columns_sliced_kernel<64, true>), sliced_grid, dim3(256), staged_bytes, stream,
+							output, input, columns, feature_map_count, neuron_count_per_feature_map);
+					else if (positions == 32)
+						hipLaunchKernelGGL((softmax_columns_sliced_kernel<32, true>), sliced_grid, dim3(256), staged_bytes, stream,
+							output, input, columns, feature_map_count, neuron_count_per_feature_map);
+					else
+						hipLaunchKernelGGL((softmax_columns_sliced_kernel<16, true>), sliced_grid, dim3(256), staged_bytes, stream,
+							output, input, columns, feature_map_count, neuron_count_per_feature_map);
+					return launch_status();
+				}
+				if (columns <= sliced_columns_limit)
+				{
+					if (columns >= 64u * 512u)
+						hipLaunchKernelGGL((softmax_columns_sliced_kernel<64, false>), dim3((columns + 63) / 64), dim3(256), 0, stream,
+							output, input, columns, feature_map_count, neuron_count_per_feature_map);
+					else
+						hipLaunchKernelGGL((softmax_columns_sliced_kernel<16, false>), dim3((columns + 15) / 16), dim3(256), 0, stream,
+							output, input, columns, feature_map_count, neuron_count_per_feature_map);
+					return launch_status();
+				}
 			}
 			// few columns: one wavefront per workgroup spreads them over more compute units
 			const uint32_t block_size = (columns >= 256u * 1024u) ? 256u : 64u;

@@ -380,12 +380,12 @@ def test_softmax_rows(gpu, n, c):
 
 
 @pytest.mark.parametrize("n,c,plane", [(2, 1, 5), (2, 2, 777), (2, 3, 2), (3, 4, 130), (1, 10, 49), (3, 16, 5), (2, 17, 64), (2, 21, 1000),
-                                       (3, 33, 300), (2, 64, 129), (1, 70, 70001), (4, 5, 4096),
+                                       (3, 33, 300), (2, 64, 129), (1, 1100, 70001), (4, 5, 4096),
                                        # four positions per lane (plane a multiple of 4, at least 262144 columns, up to 16 feature maps)
                                        (1, 2, 262144), (1, 3, 262148), (2, 8, 131072), (1, 16, 262144), (1, 17, 262144)])
 def test_softmax_columns_bit_exact(gpu, n, c, plane):
-    """One lane per column (up to 64 feature maps, or more than 65536 columns): the reference's own
-    left-to-right sum, so the bits are the oracle's."""
+    """One lane per column (up to 64 feature maps, or columns too many and too long for the shared-out
+    kernel): the reference's own left-to-right sum, so the bits are the oracle's."""
     gen = T.rng(14, n * 100000 + c * 100 + plane)
     x = T.normal(gen, (n, c, plane), 4.0)
     x[gen.random((n, c, plane)) < 0.01] = 30.0
@@ -396,9 +396,12 @@ def test_softmax_columns_bit_exact(gpu, n, c, plane):
     assert T.bit_mismatches(run_softmax(gpu, x, in_place=True), want) == 0
 
 
-@pytest.mark.parametrize("n,c,plane", [(1, 150, 333), (4, 1000, 49), (2, 65, 7), (3, 257, 100), (1, 4100, 3), (1, 66, 65536)])
+@pytest.mark.parametrize("n,c,plane", [(1, 150, 333), (4, 1000, 49), (2, 65, 7), (3, 257, 100), (1, 4100, 3), (1, 66, 65536),
+                                       # values staged in LDS: 64 positions x up to 240 feature maps, 32 x up to 480, 16 x up to 960
+                                       (1, 70, 70001), (2, 150, 40000), (1, 240, 33000), (1, 241, 33000), (3, 960, 50), (3, 961, 50),
+                                       (1, 300, 65536), (1, 300, 65537), (1, 480, 33000), (1, 481, 33000)])
 def test_softmax_columns_sliced(gpu, n, c, plane):
-    """Few columns of many feature maps: a column is shared out over 16 lanes whose partial sums are
+    """More than 64 feature maps: a column is shared out over 4 or 16 lanes whose partial sums are
     added in slice order, so the bar is the one stated for softmax, 1e-5 relative."""
     gen = T.rng(15, n * 100000 + c * 100 + plane)
     x = T.normal(gen, (n, c, plane), 4.0)
