@@ -6,27 +6,31 @@
 // the one-lane-per-output kernel below remains for the shapes that kernel declines.
 #include "nnf_common.h"
 
+#include <algorithm>
+#include <cstdlib>
+
 namespace nnf
 {
 	namespace
 	{
 		constexpr int pool_block_size = 256;
-		constexpr uint32_t global_pool_planes = 64;    // planes per workgroup of the global pooling kernel
+		constexpr uint32_t global_pool_planes = 64;    // most planes a workgroup of the global pooling kernel takes
 		constexpr uint32_t global_pool_max_plane = 240; // 64 planes * 241 floats of padded LDS = 60 KB
+		constexpr uint32_t global_pool_lds_floats = 4096; // a workgroup stages about this much: more, smaller workgroups per compute unit
 
-		// Window == whole plane (global pooling, e.g. 7x7 -> 1x1). A workgroup reduces 64 consecutive
-		// planes: its 256 lanes copy them to LDS with coalesced float4 loads, then lane t of the first
-		// wavefront sums plane t front to back. Planes are stored with an odd stride so that the 64 lanes
+		// Window == whole plane (global pooling, e.g. 7x7 -> 1x1). A workgroup reduces planes_per_group
+		// (a multiple of 4, at most 64) consecutive planes: its 256 lanes copy them to LDS with coalesced
+		// float4 loads, then lane t of the first wavefront sums plane t front to back. Planes are stored with an odd stride so that the 64 lanes
 		// hit distinct banks. Many small workgroups: the load, barrier and summation phases of
 		// different workgroups on a compute unit overlap.
-		__global__ void __launch_bounds__(pool_block_size) global_pool_kernel(float* out, const float* in, uint32_t plane_count, uint32_t plane, uint32_t plane_magic, float mult)
+		__global__ void __launch_bounds__(pool_block_size) global_pool_kernel(float* out, const float* in, uint32_t plane_count, uint32_t plane, uint32_t plane_magic, float mult, uint32_t planes_per_group)
 		{
 			extern __shared__ __align__(16) float lds_planes[];
 			const uint32_t stride = plane | 1u;
-			const uint32_t first_plane = blockIdx.x * global_pool_planes;
-			const uint32_t planes_here = min(global_pool_planes, plane_count - first_plane);
+			const uint32_t first_plane = blockIdx.x * planes_per_group;
+			const uint32_t planes_here = min(planes_per_group, plane_count - first_plane);
 			const uint32_t floats_here = planes_here * plane; // multiple of 4 except possibly in the last workgroup
-			const float* src = in + static_cast<size_t>(first_plane) * plane; // 16-byte aligned: first_plane is a multiple of 64
+			const float* src = in + static_cast<size_t>(first_plane) * plane; // 16-byte aligned: first_plane is a multiple of 4
 
 			const uint32_t vectors = floats_here / 4;
 			// eight loads in flight per lane before the first value goes to LDS
@@ -139,11 +143,15 @@ namespace nnf
 		const uint32_t plane = input_width * input_height;
 		if ((window_width == input_width) && (window_height == input_height) && (plane >= 2) && (plane <= global_pool_max_plane))
 		{
-			const size_t lds_bytes = static_cast<size_t>(global_pool_planes) * (plane | 1u) * sizeof(float);
-			const dim3 grid((plane_count + global_pool_planes - 1) / global_pool_planes);
+			// 64 planes of 7x7; fewer of larger planes, so that a compute unit holds several workgroups
+			uint32_t planes_per_group = std::min(global_pool_planes, std::max(8u, (global_pool_lds_floats / plane) & ~3u));
+			if (const char* text = std::getenv("NNF_HIP_GLOBAL_POOL_PLANES"))
+				planes_per_group = std::min(global_pool_planes, std::max(4u, static_cast<uint32_t>(std::atoi(text)) & ~3u));
+			const size_t lds_bytes = static_cast<size_t>(planes_per_group) * (plane | 1u) * sizeof(float);
+			const dim3 grid((plane_count + planes_per_group - 1) / planes_per_group);
 			// plane >= 2 here: a 1x1 window over a 1x1 plane takes the general kernel
 			const uint32_t plane_magic = static_cast<uint32_t>(((1ull << 32) + plane - 1) / plane);
-			hipLaunchKernelGGL(global_pool_kernel, grid, dim3(pool_block_size), lds_bytes, stream, output, input, plane_count, plane, plane_magic, mult);
+			hipLaunchKernelGGL(global_pool_kernel, grid, dim3(pool_block_size), lds_bytes, stream, output, input, plane_count, plane, plane_magic, mult, planes_per_group);
 		}
 		else if (window2d_launch(stream, 4, mult, output, input, static_cast<uint32_t>(input_total), plane_count,
 			input_width, input_height, output_width, output_height, window_width, window_height, window_width, window_height))
