@@ -468,6 +468,9 @@ def test_global_average_7x7(gpu, n, c):
                                          # planes larger than a workgroup's staging buffer (bands of rows), leftover margins
                                          ((1, 2, 120, 100), 2, 2), ((2, 3, 113, 115), 3, 3), ((1, 1, 300, 70), 7, 5), ((2, 2, 56, 56), 2, 2),
                                          ((1, 2, 97, 4100), 4, 3),
+                                         # whole-plane windows of several sizes (global pooling kernel up to 240 floats per plane)
+                                         ((5, 70, 14, 14), 14, 14), ((3, 9, 15, 15), 15, 15), ((2, 5, 15, 16), 16, 15), ((2, 3, 16, 16), 16, 16),
+                                         ((70, 3, 8, 8), 8, 8),
                                          # more than 65535 outputs per plane: the one-lane-per-output kernel
                                          ((1, 1, 300, 300), 1, 1), ((1, 1, 520, 260), 2, 1)])
 def test_average_subsampling_windows(gpu, shape, ww, wh):
