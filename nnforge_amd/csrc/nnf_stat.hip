@@ -14,6 +14,7 @@
 #include "nnf_common.h"
 
 #include <algorithm>
+#include <cstdlib>
 
 namespace nnf
 {
@@ -21,29 +22,61 @@ namespace nnf
 	{
 		constexpr int stat_block_size = 256;
 		constexpr int stat_unroll = 4;                    // loads a lane has in flight
-		constexpr uint32_t stat_floats_per_block = 32768; // a run is about this long ...
-		constexpr uint32_t stat_blocks_wanted = 2048;     // ... unless that leaves the grid this narrow
+		// Workgroups of this kernel an MI355X holds at once: 256 compute units x 7 workgroups of 256
+		// lanes (the kernel needs 70 vector registers, which leaves room for 7 wavefronts per SIMD).
+		// The grid is cut so that it fills whole rounds of that many.
+		constexpr uint32_t stat_resident_blocks = 1792;
+		// what starting and finishing a workgroup costs, in floats of streaming (wavefront and LDS
+		// reductions, the partial state)
+		constexpr uint64_t stat_block_overhead_floats = 8192;
 
 		struct stat_plan
 		{
 			uint32_t entries_per_run;
 			uint32_t runs;
+			uint32_t segments;          // pieces a plane is cut into (> 1 only with one entry per run)
+			uint32_t units_per_segment; // in loads (float4s when the plane is a multiple of 4, else floats)
 		};
 
+		// The grid is (runs of entries) x (feature maps), every workgroup streaming entries_per_run
+		// planes. All workgroups take equally long, so the launch lasts
+		// ceil(workgroups / resident) rounds of one workgroup's time: the run length that minimises
+		// rounds x (run length + overhead) is chosen. Measured on 128 entries of 256 feature maps of
+		// 56x56: 6 runs of 22 entries (1536 workgroups, one round) 67.5 us, 13 runs of 10 (3328, two
+		// nearly full rounds) 69-71 us, 8 runs of 16 (2048, one round and a seventh of another) 83 us.
 		stat_plan plan_runs(uint32_t entry_count, uint32_t feature_map_count, uint32_t plane)
 		{
-			stat_plan p;
-			const uint32_t by_size = std::max(1u, stat_floats_per_block / plane);
-			const uint32_t runs_wanted = std::max(1u, std::min(entry_count, (stat_blocks_wanted + feature_map_count - 1) / feature_map_count));
-			const uint32_t by_grid = (entry_count + runs_wanted - 1) / runs_wanted;
-			p.entries_per_run = std::max(1u, std::min(by_size, by_grid));
 			// the kernel divides flat indices by the plane size with a multiplication, exact while
 			// index * divisor < 2^32; a run of one entry needs no division
 			const uint64_t units = ((plane % 4) == 0) ? plane / 4 : plane;
-			if (static_cast<uint64_t>(p.entries_per_run) * units * units >= (1ull << 32))
-				p.entries_per_run = 1;
-			p.runs = (entry_count + p.entries_per_run - 1) / p.entries_per_run;
-			return p;
+			stat_plan best = { 1, entry_count, 1, static_cast<uint32_t>(units) };
+			uint64_t best_cost = ~0ull;
+			for(uint32_t entries_per_run = 1; entries_per_run <= entry_count; ++entries_per_run)
+			{
+				if ((entries_per_run > 1) && (static_cast<uint64_t>(entries_per_run) * units * units >= (1ull << 32)))
+					break;
+				const uint32_t runs = (entry_count + entries_per_run - 1) / entries_per_run;
+				const uint64_t blocks = static_cast<uint64_t>(runs) * feature_map_count;
+				const uint64_t rounds = (blocks + stat_resident_blocks - 1) / stat_resident_blocks;
+				const uint64_t cost = rounds * (static_cast<uint64_t>(entries_per_run) * plane + stat_block_overhead_floats);
+				if (cost < best_cost)
+				{
+					best_cost = cost;
+					best.entries_per_run = entries_per_run;
+					best.runs = runs;
+				}
+			}
+			// Few planes, each long (statistics of input images, say): a plane is cut into segments so that
+			// the grid still covers the machine; a segment keeps at least two rounds of loads per lane.
+			const uint64_t blocks = static_cast<uint64_t>(best.runs) * feature_map_count;
+			const uint64_t min_segment_units = static_cast<uint64_t>(stat_block_size) * stat_unroll * 2;
+			if ((best.entries_per_run == 1) && (blocks * 2 <= stat_resident_blocks) && (units >= 2 * min_segment_units))
+			{
+				const uint64_t wanted = std::min<uint64_t>(stat_resident_blocks / blocks, units / min_segment_units);
+				best.units_per_segment = static_cast<uint32_t>((units + wanted - 1) / wanted);
+				best.segments = static_cast<uint32_t>((units + best.units_per_segment - 1) / best.units_per_segment);
+			}
+			return best;
 		}
 
 		__device__ __forceinline__ void accumulate(float v, double pivot, double& s1, double& s2, float& mn, float& mx)
@@ -57,23 +90,25 @@ namespace nnf
 			mx = __builtin_fmaxf(mx, v);
 		}
 
-		// grid: (runs, feature maps). VEC: floats per load (4 when plane is a multiple of 4).
+		// grid: (runs x segments, feature maps). VEC: floats per load (4 when plane is a multiple of 4).
 		template<int VEC>
 		__global__ void __launch_bounds__(stat_block_size) stat_runs_kernel(
 			nnf_hip_running_stat* partial, const float* in, uint32_t entry_count, uint32_t feature_map_count, uint32_t plane,
-			uint32_t entries_per_run, uint32_t unit_magic)
+			uint32_t entries_per_run, uint32_t unit_magic, uint32_t segments, uint32_t units_per_segment)
 		{
 			typedef float vec_t __attribute__((ext_vector_type(VEC)));
 			__shared__ double lds_s1[stat_block_size / wave_size], lds_s2[stat_block_size / wave_size];
 			__shared__ float lds_mn[stat_block_size / wave_size], lds_mx[stat_block_size / wave_size];
 
-			const uint32_t run = blockIdx.x, fm = blockIdx.y;
+			const uint32_t run = blockIdx.x / segments, segment = blockIdx.x - run * segments, fm = blockIdx.y;
 			const uint32_t e0 = run * entries_per_run;
 			const uint32_t entries_here = min(entries_per_run, entry_count - e0);
 			const uint32_t units_per_plane = plane / VEC;
-			const uint32_t units = entries_here * units_per_plane;
+			// segments > 1: one entry per run, this workgroup takes a piece of its plane
+			const uint32_t unit_begin = segment * units_per_segment;
+			const uint32_t units = (segments > 1) ? min(units_per_segment, units_per_plane - unit_begin) : entries_here * units_per_plane;
 			const uint32_t entry_gap = (feature_map_count - 1) * plane;
-			const float* base = in + (static_cast<size_t>(e0) * feature_map_count + fm) * plane;
+			const float* base = in + (static_cast<size_t>(e0) * feature_map_count + fm) * plane + static_cast<size_t>(unit_begin) * VEC;
 			const double pivot = static_cast<double>(base[0]);
 
 			double s1 = 0.0, s2 = 0.0;
@@ -131,7 +166,7 @@ namespace nnf
 					mn = (lds_mn[w] < mn) ? lds_mn[w] : mn;
 					mx = (mx < lds_mx[w]) ? lds_mx[w] : mx;
 				}
-				const double n = static_cast<double>(entries_here) * static_cast<double>(plane);
+				const double n = static_cast<double>(units) * static_cast<double>(VEC);
 				nnf_hip_running_stat r;
 				r.n = n;
 				r.mean = pivot + s1 / n;
@@ -139,7 +174,7 @@ namespace nnf
 				r.m2 = (m2 < 0.0) ? 0.0 : m2; // rounding may leave a tiny negative value where the deviation is zero
 				r.min_val = mn;
 				r.max_val = mx;
-				partial[static_cast<size_t>(run) * feature_map_count + fm] = r;
+				partial[static_cast<size_t>(blockIdx.x) * feature_map_count + fm] = r;
 			}
 		}
 
@@ -211,7 +246,7 @@ namespace nnf
 		if ((bytes == nullptr) || (feature_map_count == 0) || (neuron_count_per_feature_map == 0))
 			return NNF_HIP_EINVAL;
 		const stat_plan p = plan_runs(std::max(1u, entry_count), feature_map_count, neuron_count_per_feature_map);
-		*bytes = static_cast<size_t>(p.runs) * feature_map_count * sizeof(nnf_hip_running_stat);
+		*bytes = static_cast<size_t>(p.runs) * p.segments * feature_map_count * sizeof(nnf_hip_running_stat);
 		return NNF_HIP_OK;
 	}
 
@@ -230,31 +265,31 @@ namespace nnf
 		if ((total > 0xFFFF0000ull) || (feature_map_count > 65535u))
 			return NNF_HIP_ETOOBIG;
 		const stat_plan p = plan_runs(entry_count, feature_map_count, neuron_count_per_feature_map);
-		const size_t needed = static_cast<size_t>(p.runs) * feature_map_count * sizeof(nnf_hip_running_stat);
+		const size_t needed = static_cast<size_t>(p.runs) * p.segments * feature_map_count * sizeof(nnf_hip_running_stat);
 		if ((workspace == nullptr) || (workspace_bytes < needed))
 			return NNF_HIP_EINVAL;
 
 		nnf_hip_running_stat* partial = static_cast<nnf_hip_running_stat*>(workspace);
-		const dim3 grid(p.runs, feature_map_count);
+		const dim3 grid(p.runs * p.segments, feature_map_count);
 		if ((neuron_count_per_feature_map % 4) == 0)
 		{
 			const uint32_t units = neuron_count_per_feature_map / 4;
 			const uint32_t magic = (units >= 2) ? static_cast<uint32_t>(((1ull << 32) + units - 1) / units) : 0u;
 			hipLaunchKernelGGL(stat_runs_kernel<4>, grid, dim3(stat_block_size), 0, stream, partial, input, entry_count, feature_map_count,
-				neuron_count_per_feature_map, p.entries_per_run, magic);
+				neuron_count_per_feature_map, p.entries_per_run, magic, p.segments, p.units_per_segment);
 		}
 		else
 		{
 			const uint32_t units = neuron_count_per_feature_map;
 			const uint32_t magic = (units >= 2) ? static_cast<uint32_t>(((1ull << 32) + units - 1) / units) : 0u;
 			hipLaunchKernelGGL(stat_runs_kernel<1>, grid, dim3(stat_block_size), 0, stream, partial, input, entry_count, feature_map_count,
-				neuron_count_per_feature_map, p.entries_per_run, magic);
+				neuron_count_per_feature_map, p.entries_per_run, magic, p.segments, p.units_per_segment);
 		}
 		int status = launch_status();
 		if (status != NNF_HIP_OK)
 			return status;
 		hipLaunchKernelGGL(stat_merge_kernel, dim3((feature_map_count + stat_block_size - 1) / stat_block_size), dim3(stat_block_size), 0, stream,
-			device_stats, partial, feature_map_count, p.runs);
+			device_stats, partial, feature_map_count, p.runs * p.segments);
 		return launch_status();
 	}
 }

@@ -68,7 +68,10 @@ def check(got, want, scale):
     (256, 1000),           # no spatial dimensions
     (3, 5, 13, 3),
     (1, 1, 1),
-    (2, 3, 300, 300),      # long planes: one entry per run
+    (2, 3, 300, 300),      # long planes: one entry per run, planes cut into segments
+    (8, 3, 224, 224),      # statistics of input images: few planes, each cut into segments
+    (1, 1, 100003),        # one long plane, not a multiple of 4: segments of single floats
+    (3, 2, 16388),         # segments of unequal length
     (1000, 2, 4),          # many entries per run
 ])
 def test_statistics_match_the_sequential_update(gpu, shape):
