@@ -153,6 +153,25 @@ class Runner:
         return (t1 - t0) / steps, ms.value * 1e-3 / steps
 
 
+def time_steps_queued(runner, step, steps, hold_ms=12.0):
+    """Device time per step with the host out of the way: the stream is first held busy by a spin
+    kernel, the `steps` launches queue up behind it, and HIP events bracket them on the stream. For
+    launches of a few microseconds, where issuing them one by one from Python (about 3.5 us each)
+    is slower than the device runs them."""
+    lib = runner.lib
+    e0, e1 = runner.event(), runner.event()
+    runner.sync()
+    runner.torch.cuda._sleep(int(hold_ms * 2.4e6))  # cycles of the spin kernel, on the current stream
+    lib.nnf_hip_event_record(e0, runner.stream)
+    for i in range(steps):
+        step(i)
+    lib.nnf_hip_event_record(e1, runner.stream)
+    runner.sync()
+    ms = ctypes.c_float()
+    runner.capi.check(lib.nnf_hip_event_elapsed_ms(ctypes.byref(ms), e0, e1))
+    return ms.value * 1e-3 / steps
+
+
 def result_entry(name, alg_bytes, elements, wall_s, event_s, launches, extra=None):
     entry = {
         "workload": name,
@@ -210,8 +229,12 @@ def bench_softmax(runner, steps, warmup):
             raise RuntimeError(runner.capi.error_string(rc))
 
     wall, ev = runner.time_steps(launch, steps, warmup)
+    queued = time_steps_queued(runner, launch, min(steps, 2000))
     return result_entry("config1: softmax over feature maps N=256 C=1000 1x1", 2 * 4 * total, total, wall, ev, 1,
-                        {"buffer_sets": sets, "note": "2 MB per step: launch latency, not bandwidth, bounds this shape"})
+                        {"buffer_sets": sets, "queued_event_ms_per_step": queued * 1e3, "queued_event_gbps": 2 * 4 * total / queued / 1e9,
+                         "note": "2 MB per step: launch latency, not bandwidth, bounds this shape; ms_per_step includes the host's "
+                                 "launch calls from Python, queued_event_ms_per_step is the device time per launch with the launches "
+                                 "queued behind a spin kernel"})
 
 
 def bench_resnet50(runner, steps, warmup, n=64):

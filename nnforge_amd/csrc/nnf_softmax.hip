@@ -85,9 +85,6 @@ namespace nnf
 		{
 			__shared__ uint64_t lds_exp[exp_lds_entries];
 			__shared__ float lds_partial[2][1024 / wave_size];
-			stage_exp2_table(lds_exp);
-			__syncthreads();
-			const exp_context exp_ctx = exp_context_from_lds(lds_exp);
 
 			const uint32_t rows_per_block = blockDim.x / THREADS;
 			const uint32_t lane = threadIdx.x % THREADS;
@@ -96,7 +93,19 @@ namespace nnf
 			const float* src = in + static_cast<size_t>(row_valid ? row : 0) * fm_count;
 			float* dst = out + static_cast<size_t>(row_valid ? row : 0) * fm_count;
 
+			// the row is requested first; the expf table is copied to LDS while it is on its way
 			float v[VPT][W];
+			#pragma unroll
+			for(int k = 0; k < VPT; ++k)
+			{
+				const uint32_t c = (lane + k * THREADS) * W;
+				if (row_valid && (c < fm_count))
+					vec_io<W>::load(src + c, v[k]);
+			}
+			stage_exp2_table(lds_exp);
+			__syncthreads();
+			const exp_context exp_ctx = exp_context_from_lds(lds_exp);
+
 			float m = softmax_max_init;
 			#pragma unroll
 			for(int k = 0; k < VPT; ++k)
@@ -104,7 +113,6 @@ namespace nnf
 				const uint32_t c = (lane + k * THREADS) * W;
 				if (row_valid && (c < fm_count))
 				{
-					vec_io<W>::load(src + c, v[k]);
 					#pragma unroll
 					for(int e = 0; e < W; ++e)
 						m = ref_max(m, v[k][e]);
