@@ -235,19 +235,23 @@ namespace nnf
 		__global__ void __launch_bounds__(256) softmax_columns_kernel(float* out, const float* in, uint32_t columns, uint32_t fm_count, uint32_t plane)
 		{
 			__shared__ uint64_t lds_exp[exp_lds_entries];
-			stage_exp2_table(lds_exp);
-			__syncthreads();
-			const exp_context exp_ctx = exp_context_from_lds(lds_exp);
-
 			const uint32_t column = blockIdx.x * blockDim.x + threadIdx.x;
-			if (column >= columns)
-				return;
-			const uint32_t entry = column / plane;
-			const uint32_t pos = column - entry * plane;
+			const bool valid = column < columns;
+			const uint32_t col = valid ? column : columns - 1; // lanes past the end shadow the last column and store nothing
+			const uint32_t entry = col / plane;
+			const uint32_t pos = col - entry * plane;
 			const size_t base = static_cast<size_t>(entry) * fm_count * plane + pos;
 			const float* src = in + base;
 			float* dst = out + base;
 			const uint32_t last = fm_count - 1;
+
+			// The table first: in a streaming kernel the wavefronts of a workgroup should not wait at the
+			// barrier for the first wavefront's column loads to come back ahead of its table entry.
+			stage_exp2_table(lds_exp);
+			__syncthreads();
+			const exp_context exp_ctx = exp_context_from_lds(lds_exp);
+			if (!valid)
+				return;
 
 			if (CACHED > 0)
 			{
@@ -346,13 +350,9 @@ namespace nnf
 		__global__ void __launch_bounds__(256) softmax_columns_vec4_kernel(float* out, const float* in, uint32_t column_quads, uint32_t fm_count, uint32_t plane)
 		{
 			__shared__ uint64_t lds_exp[exp_lds_entries];
-			stage_exp2_table(lds_exp);
-			__syncthreads();
-			const exp_context exp_ctx = exp_context_from_lds(lds_exp);
-
-			const uint32_t quad = blockIdx.x * blockDim.x + threadIdx.x;
-			if (quad >= column_quads)
-				return;
+			const uint32_t quad_id = blockIdx.x * blockDim.x + threadIdx.x;
+			const bool valid = quad_id < column_quads;
+			const uint32_t quad = valid ? quad_id : column_quads - 1; // lanes past the end shadow the last quad and store nothing
 			const uint32_t quads_per_plane = plane / 4;
 			const uint32_t entry = quad / quads_per_plane;
 			const uint32_t pos = (quad - entry * quads_per_plane) * 4;
@@ -360,6 +360,12 @@ namespace nnf
 			const float* src = in + base;
 			float* dst = out + base;
 			const uint32_t last = fm_count - 1;
+
+			stage_exp2_table(lds_exp);
+			__syncthreads();
+			const exp_context exp_ctx = exp_context_from_lds(lds_exp);
+			if (!valid)
+				return;
 
 			float v[CACHED][4];
 			#pragma unroll
