@@ -524,3 +524,44 @@ def test_short_division_sequences_equal_ieee_division_for_every_denominator(gpu)
     assert rc == 0, capi.error_string(rc)
     gpu.torch.cuda.synchronize()
     assert counts.tolist() == [0, 0]
+
+
+def test_largest_tensor_the_kernels_index(gpu):
+    """0xFFFF0000 elements (65535 x 256 x 256, 17 GB): the largest count the 32-bit tile arithmetic
+    accepts. The CPU oracle would need minutes and tens of GB for it, so the check is a size-independent
+    one: batch norm -> ReLU is two fp32 roundings per element, which plain device tensor arithmetic
+    reproduces exactly (multiply, add and maximum as separate operations), compared on the device
+    over the whole tensor, in place, plus the oracle on the first and the last entries."""
+    torch = gpu.torch
+    free, _ = torch.cuda.mem_get_info()
+    n, c, plane = 65535, 256, 256
+    total = n * c * plane
+    assert total == 0xFFFF0000
+    if free < 3.2 * 4 * total:
+        pytest.skip("needs about 55 GB of free device memory")
+    gen = torch.Generator(device=gpu.device)
+    gen.manual_seed(20)
+    x = torch.randn(total, generator=gen, device=gpu.device, dtype=torch.float32)
+    g, b, m, s = T.bn_params(T.rng(20, 1), c)
+    head = x[: 2 * c * plane].cpu().numpy().reshape(2, c, plane)
+    tail = x[-2 * c * plane:].cpu().numpy().reshape(2, c, plane)
+    d_w = [gpu.to_device(v) for v in (g, b, m, s)]
+    mult = d_w[0] * d_w[3]
+    add = d_w[1] - mult * d_w[2]
+    want = x.view(n, c, plane) * mult.view(1, c, 1)
+    want += add.view(1, c, 1)
+    want = torch.where(want >= 0, want, want * 0.0)  # -0.0 for negative values, as the reference's x * 0.0F
+    desc = capi.make_desc(n, c, plane, [[(BN, 0), (RELU, 0, 0.0)]], [])
+    rc = gpu.lib.nnf_hip_chain_forward(gpu.stream, ctypes.byref(desc), x.data_ptr(), capi.pointer_array([x.data_ptr()]),
+                                       capi.pointer_array([t.data_ptr() for t in d_w]))
+    assert rc == 0, capi.error_string(rc)
+    torch.cuda.synchronize()
+    differing = int((x.view(torch.int32) != want.view(-1).view(torch.int32)).sum().item())
+    assert differing == 0, "%d of %d elements differ from the device-side evaluation" % (differing, total)
+    del want
+    for got, src in ((x[: 2 * c * plane], head), (x[-2 * c * plane:], tail)):
+        ref = oracle.rectified_linear(oracle.batch_norm(src, g, b, m, s), 0.0)
+        assert T.bit_mismatches(got.cpu().numpy(), ref.reshape(-1)) == 0
+    # one element more is refused before anything is launched
+    desc = capi.make_desc(n, c, plane + 1, [[(RELU, 0, 0.0)]], [])
+    assert gpu.lib.nnf_hip_chain_forward(gpu.stream, ctypes.byref(desc), x.data_ptr(), capi.pointer_array([x.data_ptr()]), None) == capi.E_TOOBIG
