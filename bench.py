@@ -292,6 +292,30 @@ def bench_max_subsampling(runner, steps, warmup, n=64, c=64, size=112):
                         4 * (in_count + out_count), out_count, wall, ev, 1, {"buffer_sets": sets})
 
 
+def bench_bn_relu_max_subsampling(runner, steps, warmup, n=64, c=64, size=112):
+    """The ResNet stem behind conv1: batch_norm -> rectified_linear -> 3x3 max pooling every 2 (rounded up), one
+    launch: the pooling kernel applies the two layers to the values it reads."""
+    out_size = (size + 2 - 3 + 2) // 2
+    in_count, out_count = n * c * size * size, n * c * out_size * out_size
+    sets = rotation_sets(4 * (in_count + out_count))
+    ins = [runner.randn(in_count) for _ in range(sets)]
+    outs = [runner.empty(out_count) for _ in range(sets)]
+    chunks = runner.bn_chunks(c)
+    chunk_ptrs = runner.capi.pointer_array([t.data_ptr() for t in chunks])
+    desc = runner.capi.make_desc(n, c, size * size, [[(runner.capi.OP_BATCH_NORM, 0), (runner.capi.OP_RELU, 0, 0.0)]], [])
+    dims, win, stride, up = _u32([size, size]), _u32([3, 3]), _u32([2, 2]), _u32([1, 1])
+    fn, stream = runner.lib.nnf_hip_max_subsampling_fused_forward, runner.stream
+
+    def launch(i):
+        rc = fn(stream, outs[i % sets].data_ptr(), ins[i % sets].data_ptr(), ctypes.byref(desc), chunk_ptrs, n, c, 2, dims, win, stride, up, 1, 1, 0)
+        if rc != 0:
+            raise RuntimeError(runner.capi.error_string(rc))
+
+    wall, ev = runner.time_steps(launch, steps, warmup)
+    return result_entry("batch_norm -> rectified_linear -> max_subsampling 3x3 stride 2 round up, N=%d C=%d %dx%d -> %dx%d" % (n, c, size, size, out_size, out_size),
+                        4 * (in_count + out_count + 4 * c), out_count, wall, ev, 1, {"buffer_sets": sets})
+
+
 def bench_concat(runner, steps, warmup, n=32, fms=(64, 128, 32, 32), plane=28 * 28):
     counts = [c * plane for c in fms]
     total = n * sum(counts)
@@ -428,7 +452,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=400)
     ap.add_argument("--warmup", type=int, default=40)
-    ap.add_argument("--workload", default="config0", choices=["config0", "config1", "config2", "config3", "config4", "copy", "max_subsampling", "concat", "maxout", "feature_map_stat"],
+    ap.add_argument("--workload", default="config0", choices=["config0", "config1", "config2", "config3", "config4", "copy", "max_subsampling", "bn_relu_max_subsampling", "concat", "maxout", "feature_map_stat"],
                     help="'copy' times the plain copy kernel (profiler-counter calibration and bandwidth yardstick)")
     ap.add_argument("--only", action="store_true", help="time only the chosen workload (no per_config survey, no CPU baseline)")
     args = ap.parse_args()
@@ -454,6 +478,8 @@ def main():
             return bench_copy(runner, steps, warmup)
         if name == "max_subsampling":
             return bench_max_subsampling(runner, steps, warmup)
+        if name == "bn_relu_max_subsampling":
+            return bench_bn_relu_max_subsampling(runner, steps, warmup)
         if name == "concat":
             return bench_concat(runner, steps, warmup)
         if name == "maxout":
@@ -504,7 +530,7 @@ def main():
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBPS,
             "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
-            "kernel": {"config1": "nnf::softmax_rows_kernel", "copy": "nnf::copy_kernel_impl", "max_subsampling": "nnf::max_window2d_kernel",
+            "kernel": {"config1": "nnf::softmax_rows_kernel", "copy": "nnf::copy_kernel_impl", "max_subsampling": "nnf::max_window2d_kernel", "bn_relu_max_subsampling": "nnf::max_window2d_prologue_kernel",
                        "concat": "nnf::concat_kernel", "maxout": "nnf::maxout_vec4_kernel",
                        "feature_map_stat": "nnf::stat_runs_kernel"}.get(args.workload, "nnf::chain_kernel"),
             "algorithmic_bytes_per_launch": main_entry["algorithmic_bytes_per_step"] / launches,

@@ -176,6 +176,34 @@ NNF_HIP_API int nnf_hip_max_subsampling_forward(void* stream, float* output, con
 	const uint32_t* input_sizes, const uint32_t* subsampling_sizes, const uint32_t* strides, const uint32_t* round_ups,
 	uint32_t feature_map_subsampling_size, uint32_t entry_subsampling_size, int32_t is_min);
 
+/* Subsampling with the element-wise layers in front of it folded in: `prologue` describes a
+ * single-input group without Add (input_count 1, has_add 0; its arm 0 and tail layers are applied in
+ * order; its feature_map_count and neuron_count_per_feature_map must be the subsampling input's) whose
+ * result feeds the subsampling layer and nothing else. The layers are applied to the input values on
+ * their way into the workgroup's staging buffer, so the group's result - what
+ * nnforge/plain/forward_propagation_plain.cpp:137-186 would store between the two testers - is never
+ * written to memory; the output carries the same bits as the layers run one after another. Other
+ * arguments as for nnf_hip_max_subsampling_forward / nnf_hip_average_subsampling_forward. Only the
+ * LDS-staged window kernel applies a prologue: NNF_HIP_EUNSUPPORTED (nothing launched) for windows
+ * over feature maps or entries, more than two spatial dimensions, whole-plane average windows, planes
+ * of fewer than four floats, more than 65535 outputs per plane, and groups with more than two layers
+ * that carry weights (batch norm, PReLU). The *_fusable
+ * functions answer that from the shapes alone (NNF_HIP_OK / NNF_HIP_EUNSUPPORTED; no device needed). */
+NNF_HIP_API int nnf_hip_max_subsampling_fused_forward(void* stream, float* output, const float* input,
+	const nnf_hip_chain_desc* prologue, const float* const* chunk_ptrs,
+	uint32_t output_entry_count, uint32_t input_feature_map_count, uint32_t dimension_count,
+	const uint32_t* input_sizes, const uint32_t* subsampling_sizes, const uint32_t* strides, const uint32_t* round_ups,
+	uint32_t feature_map_subsampling_size, uint32_t entry_subsampling_size, int32_t is_min);
+NNF_HIP_API int nnf_hip_average_subsampling_fused_forward(void* stream, float* output, const float* input,
+	const nnf_hip_chain_desc* prologue, const float* const* chunk_ptrs,
+	uint32_t entry_count, uint32_t feature_map_count, uint32_t input_width, uint32_t input_height,
+	uint32_t window_width, uint32_t window_height, float mult);
+NNF_HIP_API int nnf_hip_max_subsampling_fusable(uint32_t output_entry_count, uint32_t input_feature_map_count, uint32_t dimension_count,
+	const uint32_t* input_sizes, const uint32_t* subsampling_sizes, const uint32_t* strides, const uint32_t* round_ups,
+	uint32_t feature_map_subsampling_size, uint32_t entry_subsampling_size);
+NNF_HIP_API int nnf_hip_average_subsampling_fusable(uint32_t entry_count, uint32_t feature_map_count, uint32_t input_width, uint32_t input_height,
+	uint32_t window_width, uint32_t window_height);
+
 /* Per-feature-map running statistics on the device: the state stat_data_bunch_writer keeps per
  * feature map (nnforge/stat_data_bunch_writer.h:45-63) and fills on the host from outputs copied
  * back (nnforge/stat_data_bunch_writer.cpp:45-79). average = (float)mean and

@@ -129,6 +129,20 @@ namespace nnforge
 			// when the layer cannot be part of a fused group.
 			virtual int get_chain_op(nnf_hip_op& op) const { return -1; }
 
+			// Subsampling testers can apply the element-wise layers in front of them to the values they
+			// read, so that the result of those layers is never stored. can_apply_prologue: whether this
+			// tester's shapes allow it. enqueue_forward_propagation_with_prologue: the forward pass over
+			// input_buffer with the layers of prologue (a single-input group without Add whose shape is
+			// this tester's input; its weights in chunk_ptrs) applied first.
+			virtual bool can_apply_prologue() const { return false; }
+			virtual void enqueue_forward_propagation_with_prologue(
+				void * stream_id,
+				hip_linear_buffer_device::ptr output_buffer,
+				hip_linear_buffer_device::const_ptr input_buffer,
+				const nnf_hip_chain_desc& prologue,
+				const float * const * chunk_ptrs,
+				unsigned int entry_count);
+
 		protected:
 			layer_tester_hip() = default;
 			virtual void tester_configured() {}
@@ -193,7 +207,8 @@ namespace nnforge
 		{
 			std::vector<std::string> layer_names;  // members in execution order; back() produces the output
 			std::vector<std::string> input_names;  // layers whose buffers are read, in kernel input order
-			bool fused;                            // executed by the fused-group kernel
+			bool fused;                            // several layers in one launch: the fused-group kernel, or a subsampling
+			                                       // layer (the last name) that applies the element-wise layers in front of it
 			std::string description() const;       // e.g. "bn1+add1+relu1 <- conv_a, conv_b"
 		};
 

@@ -52,6 +52,7 @@ _U32 = ctypes.c_uint32
 _U64 = ctypes.c_uint64
 _F = ctypes.c_float
 _PP = ctypes.POINTER(ctypes.c_void_p)
+_UP = ctypes.POINTER(ctypes.c_uint32)
 
 # name -> argtypes, exactly the declarations of include/nnforge_hip.h (all return int unless noted)
 SIGNATURES = {
@@ -97,6 +98,10 @@ SIGNATURES = {
     "nnf_hip_stream_wait_event": [_VP, _VP],
     "nnf_hip_copy_kernel": [_VP, _VP, _VP, ctypes.c_size_t],
     "nnf_hip_check_division_sequences": [_VP, _VP],
+    "nnf_hip_max_subsampling_fused_forward": [_VP, _VP, _VP, ctypes.POINTER(ChainDesc), _PP, _U32, _U32, _U32, _UP, _UP, _UP, _UP, _U32, _U32, ctypes.c_int32],
+    "nnf_hip_average_subsampling_fused_forward": [_VP, _VP, _VP, ctypes.POINTER(ChainDesc), _PP, _U32, _U32, _U32, _U32, _U32, _U32, _F],
+    "nnf_hip_max_subsampling_fusable": [_U32, _U32, _U32, _UP, _UP, _UP, _UP, _U32, _U32],
+    "nnf_hip_average_subsampling_fusable": [_U32, _U32, _U32, _U32, _U32, _U32],
 }
 STRING_FUNCTIONS = {"nnf_hip_error_string": [ctypes.c_int], "nnf_hip_version": []}
 

@@ -3,6 +3,7 @@
 // events) that lets host C++ above this ABI stay free of HIP headers.
 #include "nnf_common.h"
 
+#include <algorithm>
 #include <cstring>
 
 namespace nnf
@@ -287,6 +288,75 @@ extern "C"
 		hipLaunchKernelGGL(division_check_kernel, dim3(4096), dim3(256), 0, static_cast<hipStream_t>(stream),
 			reinterpret_cast<unsigned long long*>(device_mismatch_counts));
 		return launch_status();
+	}
+
+	int nnf_hip_max_subsampling_fused_forward(void* stream, float* output, const float* input,
+		const nnf_hip_chain_desc* prologue, const float* const* chunk_ptrs,
+		uint32_t output_entry_count, uint32_t input_feature_map_count, uint32_t dimension_count,
+		const uint32_t* input_sizes, const uint32_t* subsampling_sizes, const uint32_t* strides, const uint32_t* round_ups,
+		uint32_t feature_map_subsampling_size, uint32_t entry_subsampling_size, int32_t is_min)
+	{
+		if ((prologue == nullptr) || (prologue->feature_map_count != input_feature_map_count))
+			return NNF_HIP_EINVAL;
+		if ((input_sizes != nullptr) && (dimension_count >= 1) && (dimension_count <= 4))
+		{
+			uint64_t plane = 1;
+			for(uint32_t i = 0; i < dimension_count; ++i)
+				plane *= input_sizes[i];
+			if (plane != prologue->neuron_count_per_feature_map)
+				return NNF_HIP_EINVAL;
+		}
+		if (const int rc = prologue_status(*prologue, chunk_ptrs))
+			return rc;
+		return max_subsampling_forward_with_prologue(static_cast<hipStream_t>(stream), output, input, output_entry_count, input_feature_map_count,
+			dimension_count, input_sizes, subsampling_sizes, strides, round_ups, feature_map_subsampling_size, entry_subsampling_size, is_min,
+			prologue, chunk_ptrs, false);
+	}
+
+	int nnf_hip_average_subsampling_fused_forward(void* stream, float* output, const float* input,
+		const nnf_hip_chain_desc* prologue, const float* const* chunk_ptrs,
+		uint32_t entry_count, uint32_t feature_map_count, uint32_t input_width, uint32_t input_height,
+		uint32_t window_width, uint32_t window_height, float mult)
+	{
+		if ((prologue == nullptr) || (prologue->feature_map_count != feature_map_count)
+			|| (static_cast<uint64_t>(input_width) * input_height != prologue->neuron_count_per_feature_map))
+			return NNF_HIP_EINVAL;
+		if (const int rc = prologue_status(*prologue, chunk_ptrs))
+			return rc;
+		return average_subsampling_forward_with_prologue(static_cast<hipStream_t>(stream), output, input, entry_count, feature_map_count,
+			input_width, input_height, window_width, window_height, mult, prologue, chunk_ptrs, false);
+	}
+
+	namespace
+	{
+		// any single-layer group: the shape checks do not depend on which layers the prologue holds
+		nnf_hip_chain_desc planning_prologue(uint32_t feature_map_count)
+		{
+			nnf_hip_chain_desc d;
+			std::memset(&d, 0, sizeof(d));
+			d.feature_map_count = feature_map_count;
+			d.input_count = 1;
+			d.arm_op_count[0] = 1;
+			d.ops[0].kind = NNF_HIP_OP_ABSOLUTE;
+			return d;
+		}
+	}
+
+	int nnf_hip_max_subsampling_fusable(uint32_t output_entry_count, uint32_t input_feature_map_count, uint32_t dimension_count,
+		const uint32_t* input_sizes, const uint32_t* subsampling_sizes, const uint32_t* strides, const uint32_t* round_ups,
+		uint32_t feature_map_subsampling_size, uint32_t entry_subsampling_size)
+	{
+		const nnf_hip_chain_desc d = planning_prologue(input_feature_map_count);
+		return max_subsampling_forward_with_prologue(nullptr, nullptr, nullptr, std::max(1u, output_entry_count), input_feature_map_count, dimension_count,
+			input_sizes, subsampling_sizes, strides, round_ups, feature_map_subsampling_size, entry_subsampling_size, 0, &d, nullptr, true);
+	}
+
+	int nnf_hip_average_subsampling_fusable(uint32_t entry_count, uint32_t feature_map_count, uint32_t input_width, uint32_t input_height,
+		uint32_t window_width, uint32_t window_height)
+	{
+		const nnf_hip_chain_desc d = planning_prologue(feature_map_count);
+		return average_subsampling_forward_with_prologue(nullptr, nullptr, nullptr, std::max(1u, entry_count), feature_map_count, input_width, input_height,
+			window_width, window_height, 1.0f, &d, nullptr, true);
 	}
 
 	int nnf_hip_copy_kernel(void* stream, void* device_dst, const void* device_src, size_t bytes)

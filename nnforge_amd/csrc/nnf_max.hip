@@ -69,6 +69,184 @@ namespace nnf
 		// is one contiguous range of memory in both cases; it is copied to LDS with aligned float4
 		// loads (each input byte is fetched once per workgroup; only the window_height - stride_y rows
 		// shared by neighbouring row bands are fetched twice), then every lane scans its windows in LDS.
+		// Element-wise layers applied to every input value on its way into LDS ("prologue"): the layers
+		// of a single-input group that feeds the subsampling layer and nothing else, so that the
+		// group's result is never written to memory. Same formulas, same order, one rounding per
+		// operation as the chain kernel: the staged values carry the bits the unfused layers would
+		// have stored.
+		constexpr uint32_t prologue_weighted_max = 2;  // layers with weights (batch norm, PReLU) a prologue may hold
+		constexpr uint32_t prologue_coef_floats = 768; // LDS a workgroup sets aside for its planes' coefficients
+		constexpr uint32_t prologue_planes_max = 256;  // one lane per plane fetches the weights
+
+		struct window_prologue
+		{
+			uint32_t op_count;
+			uint32_t fm_count;
+			uint32_t need_exp;
+			uint32_t in_plane_magic;         // ceil(2^32 / input plane size)
+			uint32_t weighted_count;         // layers with weights; every plane has 2 coefficients per such layer
+			uint32_t slot[NNF_HIP_MAX_OPS];  // where a layer's coefficients start among a plane's
+			int32_t kind[NNF_HIP_MAX_OPS];
+			float f0[NNF_HIP_MAX_OPS];
+			float f1[NNF_HIP_MAX_OPS];       // TanH: steepness * 2
+			int32_t weighted_kind[prologue_weighted_max];
+			const float* weights[prologue_weighted_max][4]; // batch norm: gamma, beta, mean, inverse sigma; PReLU: slopes
+		};
+
+		// Batch norm's multiplier and addend and PReLU's slope of the planes a workgroup stages are worked
+		// out once per plane, by lane plane_in_workgroup, and kept in LDS:
+		// coef[plane_in_workgroup * 2 * pro.weighted_count + pro.slot[layer]]. In two steps, so that a kernel
+		// can issue these loads in front of its tensor loads and wait for them behind.
+		struct prologue_weights
+		{
+			float w[prologue_weighted_max][4];
+		};
+
+		__device__ __forceinline__ prologue_weights load_prologue_weights(uint32_t first_fm, uint32_t planes_here, const window_prologue& pro)
+		{
+			prologue_weights r;
+			uint32_t fm = first_fm + threadIdx.x;
+			if (fm >= pro.fm_count)
+				fm %= pro.fm_count;
+			#pragma unroll
+			for(uint32_t j = 0; j < prologue_weighted_max; ++j)
+			{
+				#pragma unroll
+				for(int c = 0; c < 4; ++c)
+					r.w[j][c] = 0.0f;
+				if ((j < pro.weighted_count) && (threadIdx.x < planes_here))
+				{
+					r.w[j][0] = pro.weights[j][0][fm];
+					if (pro.weighted_kind[j] == NNF_HIP_OP_BATCH_NORM)
+					{
+						#pragma unroll
+						for(int c = 1; c < 4; ++c)
+							r.w[j][c] = pro.weights[j][c][fm];
+					}
+				}
+			}
+			return r;
+		}
+
+		__device__ __forceinline__ void stage_prologue_coefficients(float* coef, prologue_weights r, uint32_t planes_here, const window_prologue& pro)
+		{
+			// The weights are not looked at before this point: without it the compiler works the
+			// coefficients out, and waits for the weights, in front of the tensor loads.
+			#pragma unroll
+			for(uint32_t j = 0; j < prologue_weighted_max; ++j)
+			{
+				#pragma unroll
+				for(int c = 0; c < 4; ++c)
+					asm volatile("" : "+v"(r.w[j][c]));
+			}
+			#pragma unroll
+			for(uint32_t j = 0; j < prologue_weighted_max; ++j)
+			{
+				if ((j < pro.weighted_count) && (threadIdx.x < planes_here))
+				{
+					float* dst = coef + (threadIdx.x * pro.weighted_count + j) * 2;
+					if (pro.weighted_kind[j] == NNF_HIP_OP_BATCH_NORM)
+						nnf_batch_norm_coefficients(r.w[j][0], r.w[j][1], r.w[j][2], r.w[j][3], dst[0], dst[1]);
+					else
+						dst[0] = r.w[j][0];
+				}
+			}
+		}
+
+		// One layer after another over all the float4s a lane has loaded in a round, so that a layer's
+		// kind is looked up once and the coefficient reads of the round are in flight together.
+		// off[k]: where the coefficients of vector k's plane start in coef.
+		// EXP false: compiled without the layers that call expf (the host picks it when the group has none),
+		// which leaves the kernel with far fewer registers per lane.
+		constexpr int coef_batch = 4; // vectors whose batch norm coefficients are read from LDS together
+
+		template<int VECTORS, bool EXP>
+		__device__ __forceinline__ void apply_prologue(float (&v)[VECTORS][4], const uint32_t (&off)[VECTORS],
+			const float* coef, const window_prologue& pro, const exp_context& exp_ctx)
+		{
+			for(uint32_t i = 0; i < pro.op_count; ++i)
+			{
+				const int32_t kind = pro.kind[i];
+				const uint32_t slot = pro.slot[i];
+				const float f0 = pro.f0[i], f1 = pro.f1[i];
+				switch (kind)
+				{
+				case NNF_HIP_OP_BATCH_NORM:
+					#pragma unroll
+					for(int k0 = 0; k0 < VECTORS; k0 += coef_batch)
+					{
+						float mult[coef_batch], add[coef_batch];
+						#pragma unroll
+						for(int k = 0; (k < coef_batch) && (k0 + k < VECTORS); ++k)
+						{
+							mult[k] = coef[off[k0 + k] + slot];
+							add[k] = coef[off[k0 + k] + slot + 1];
+						}
+						#pragma unroll
+						for(int k = 0; (k < coef_batch) && (k0 + k < VECTORS); ++k)
+						{
+							#pragma unroll
+							for(int e = 0; e < 4; ++e)
+								v[k0 + k][e] = nnf_batch_norm(v[k0 + k][e], mult[k], add[k]);
+						}
+					}
+					break;
+				case NNF_HIP_OP_PRELU:
+					{
+						float slope[VECTORS];
+						#pragma unroll
+						for(int k = 0; k < VECTORS; ++k)
+							slope[k] = coef[off[k] + slot];
+						#pragma unroll
+						for(int k = 0; k < VECTORS; ++k)
+						{
+							#pragma unroll
+							for(int e = 0; e < 4; ++e)
+								v[k][e] = nnf_parametric_rectified_linear(v[k][e], slope[k]);
+						}
+					}
+					break;
+				case NNF_HIP_OP_RELU:
+					#pragma unroll
+					for(int k = 0; k < VECTORS; ++k)
+					{
+						#pragma unroll
+						for(int e = 0; e < 4; ++e)
+							v[k][e] = nnf_rectified_linear(v[k][e], f0);
+					}
+					break;
+				case NNF_HIP_OP_ABSOLUTE:
+					#pragma unroll
+					for(int k = 0; k < VECTORS; ++k)
+					{
+						#pragma unroll
+						for(int e = 0; e < 4; ++e)
+							v[k][e] = nnf_absolute(v[k][e]);
+					}
+					break;
+				case NNF_HIP_OP_ELU:
+				case NNF_HIP_OP_SIGMOID:
+				case NNF_HIP_OP_TANH:
+					if (EXP)
+					{
+						#pragma unroll
+						for(int k = 0; k < VECTORS; ++k)
+						{
+							if (kind == NNF_HIP_OP_ELU)
+								nnf_exponential_linear<4>(v[k], exp_ctx);
+							else if (kind == NNF_HIP_OP_SIGMOID)
+								nnf_sigmoid<4>(v[k], exp_ctx);
+							else
+								nnf_hyperbolic_tangent<4>(v[k], f1, f0, exp_ctx);
+						}
+					}
+					break;
+				default: // NNF_HIP_OP_DROPOUT: the value passes through
+					break;
+				}
+			}
+		}
+
 		struct window2d_args
 		{
 			float* out;
@@ -90,10 +268,16 @@ namespace nnf
 		// WIN_W, WIN_H: window size known at compile time, 0: read it from the arguments.
 		// TRUNC: windows may reach beyond the input (round up) and are cut off there (maximum and
 		// minimum only: repeating a value would change a sum).
-		template<int OP, int WIN_W, int WIN_H, bool TRUNC>
-		__global__ void __launch_bounds__(max_block_size) max_window2d_kernel(const window2d_args a)
+		// PROLOGUE: the staged values go through the layers of pro first, with the weights of the feature
+		// map each value belongs to (a float4 may straddle two planes when several planes that are not
+		// a multiple of four floats long share a workgroup; the host declines planes of under 4 floats).
+		template<int OP, int WIN_W, int WIN_H, bool TRUNC, bool PROLOGUE, bool EXP>
+		__device__ __forceinline__ void window2d_body(const window2d_args& a, const window_prologue& pro)
 		{
 			extern __shared__ __align__(16) float lds_in[];
+			__shared__ uint64_t lds_exp[EXP ? exp_lds_entries : 1];
+			__shared__ float lds_coef[PROLOGUE ? prologue_coef_floats : 1];
+			exp_context exp_ctx = make_exp_context(lds_exp);
 
 			const uint32_t group = blockIdx.x / a.bands;
 			const uint32_t band = blockIdx.x - group * a.bands;
@@ -116,11 +300,16 @@ namespace nnf
 			const uint32_t shift = g0 - g0_aligned;
 			const uint32_t vectors = (g1 - g0_aligned + 3) / 4;
 			// all loads of a round are issued before the first one is stored to LDS
-			for(uint32_t base = 0; base < vectors; base += stage_vectors_per_lane * max_block_size)
+			constexpr int STAGE = stage_vectors_per_lane;
+			// the weights are requested first and looked at once the first round's tensor loads are out
+			prologue_weights weights;
+			if (PROLOGUE)
+				weights = load_prologue_weights(first_plane % pro.fm_count, planes_here, pro);
+			for(uint32_t base = 0; base < vectors; base += STAGE * max_block_size)
 			{
-				floatx4 t[stage_vectors_per_lane];
+				floatx4 t[STAGE];
 				#pragma unroll
-				for(int k = 0; k < stage_vectors_per_lane; ++k)
+				for(int k = 0; k < STAGE; ++k)
 				{
 					const uint32_t i = base + k * max_block_size + threadIdx.x;
 					const uint32_t g = g0_aligned + i * 4;
@@ -138,8 +327,79 @@ namespace nnf
 						}
 					}
 				}
+				if (PROLOGUE && (base == 0))
+				{
+					stage_prologue_coefficients(lds_coef, weights, planes_here, pro);
+					if (EXP)
+						stage_exp2_table(lds_exp);
+					__syncthreads();
+					if (EXP)
+						exp_ctx = exp_context_from_lds(lds_exp);
+				}
+				if (PROLOGUE)
+				{
+					float v[STAGE][4];
+					uint32_t off[STAGE];
+					// Planes that are not a multiple of four floats long: a float4 may straddle two of them (never
+					// three: the host declines planes of under 4 floats). Bit k: vector k does.
+					const bool straddle = (planes_here > 1) && ((in_plane & 3u) != 0);
+					uint32_t straddling = 0;
+					#pragma unroll
+					for(int k = 0; k < STAGE; ++k)
+					{
+						const uint32_t i = base + k * max_block_size + threadIdx.x;
+						const bool valid = i < vectors;
+						v[k][0] = valid ? t[k].x : 0.0f; v[k][1] = valid ? t[k].y : 0.0f; v[k][2] = valid ? t[k].z : 0.0f; v[k][3] = valid ? t[k].w : 0.0f;
+						// plane, inside the workgroup's range, of the first float of this float4 (floats in front
+						// of the range count as plane 0: they are staged but not read)
+						const uint32_t first_pos = max(i * 4, shift) - shift;
+						const uint32_t p = ((planes_here > 1) && valid) ? fast_divide(first_pos, in_plane, pro.in_plane_magic) : 0u;
+						off[k] = p * (2 * pro.weighted_count);
+						// floats from staged position (p + 1) * in_plane + shift on belong to plane p + 1; beyond
+						// the last plane of the workgroup they are not read
+						if (straddle && valid && (p + 1 < planes_here) && (i * 4 + 3 >= (p + 1) * in_plane + shift))
+							straddling |= 1u << k;
+					}
+					apply_prologue<STAGE, EXP>(v, off, lds_coef, pro, exp_ctx);
+					// The floats of the second plane of a straddling float4 were given the first plane's
+					// coefficients: they are fetched again and go through the layers with their own.
+					while (__any(straddling != 0))
+					{
+						const int k_mine = (straddling != 0) ? __ffs(straddling) - 1 : 0;
+						const bool mine = straddling != 0;
+						const uint32_t i = base + k_mine * max_block_size + threadIdx.x;
+						const uint32_t first_pos = max(i * 4, shift) - shift;
+						const uint32_t p_next = mine ? fast_divide(first_pos, in_plane, pro.in_plane_magic) + 1 : 0u;
+						const uint32_t split = mine ? p_next * in_plane + shift - i * 4 : 4u; // 1..3: first float of plane p_next
+						float w[1][4];
+						#pragma unroll
+						for(uint32_t e = 0; e < 4; ++e)
+						{
+							const uint32_t g = g0_aligned + i * 4 + e;
+							w[0][e] = (mine && (e >= split) && (g < a.total_in)) ? a.in[g] : 0.0f;
+						}
+						const uint32_t off_next[1] = { p_next * (2 * pro.weighted_count) };
+						apply_prologue<1, EXP>(w, off_next, lds_coef, pro, exp_ctx);
+						#pragma unroll
+						for(int k = 0; k < STAGE; ++k)
+						{
+							#pragma unroll
+							for(uint32_t e = 1; e < 4; ++e)
+							{
+								if (mine && (k == k_mine) && (e >= split))
+									v[k][e] = w[0][e];
+							}
+						}
+						straddling &= straddling - 1;
+					}
+					#pragma unroll
+					for(int k = 0; k < STAGE; ++k)
+					{
+						t[k].x = v[k][0]; t[k].y = v[k][1]; t[k].z = v[k][2]; t[k].w = v[k][3];
+					}
+				}
 				#pragma unroll
-				for(int k = 0; k < stage_vectors_per_lane; ++k)
+				for(int k = 0; k < STAGE; ++k)
 				{
 					const uint32_t i = base + k * max_block_size + threadIdx.x;
 					if (i < vectors)
@@ -189,6 +449,27 @@ namespace nnf
 				}
 				dst[o] = (OP == window_op_sum) ? current * a.mult : current;
 			}
+		}
+
+		template<int OP, int WIN_W, int WIN_H, bool TRUNC>
+		__global__ void __launch_bounds__(max_block_size) max_window2d_kernel(const window2d_args a)
+		{
+			window_prologue none; // not read
+			window2d_body<OP, WIN_W, WIN_H, TRUNC, false, false>(a, none);
+		}
+
+		// Without expf the layers fit 96 registers per lane, which lets a compute unit hold five workgroups
+		// instead of four (measured: 10 % faster); with expf that would spill.
+		template<int OP, int WIN_W, int WIN_H, bool TRUNC>
+		__global__ void __launch_bounds__(max_block_size) __attribute__((amdgpu_waves_per_eu(5, 5))) max_window2d_prologue_kernel(const window2d_args a, const window_prologue pro)
+		{
+			window2d_body<OP, WIN_W, WIN_H, TRUNC, true, false>(a, pro);
+		}
+
+		template<int OP, int WIN_W, int WIN_H, bool TRUNC>
+		__global__ void __launch_bounds__(max_block_size) max_window2d_exp_prologue_kernel(const window2d_args a, const window_prologue pro)
+		{
+			window2d_body<OP, WIN_W, WIN_H, TRUNC, true, true>(a, pro);
 		}
 
 		// ---- any window the layer allows: one lane per output, values read from memory ------------
@@ -302,14 +583,92 @@ namespace nnf
 		}
 
 		template<int OP, bool TRUNC>
-		void launch_window2d(hipStream_t stream, const window2d_args& a, uint32_t grid, size_t lds_bytes)
+		void launch_window2d(hipStream_t stream, const window2d_args& a, uint32_t grid, size_t lds_bytes, const window_prologue* pro)
 		{
+			if (pro != nullptr)
+			{
+				const dim3 g(grid), b(max_block_size);
+				const bool w3 = (a.win_w == 3) && (a.win_h == 3), w2 = (a.win_w == 2) && (a.win_h == 2);
+				if (pro->need_exp)
+				{
+					if (w3) hipLaunchKernelGGL((max_window2d_exp_prologue_kernel<OP, 3, 3, TRUNC>), g, b, lds_bytes, stream, a, *pro);
+					else if (w2) hipLaunchKernelGGL((max_window2d_exp_prologue_kernel<OP, 2, 2, TRUNC>), g, b, lds_bytes, stream, a, *pro);
+					else hipLaunchKernelGGL((max_window2d_exp_prologue_kernel<OP, 0, 0, TRUNC>), g, b, lds_bytes, stream, a, *pro);
+				}
+				else
+				{
+					if (w3) hipLaunchKernelGGL((max_window2d_prologue_kernel<OP, 3, 3, TRUNC>), g, b, lds_bytes, stream, a, *pro);
+					else if (w2) hipLaunchKernelGGL((max_window2d_prologue_kernel<OP, 2, 2, TRUNC>), g, b, lds_bytes, stream, a, *pro);
+					else hipLaunchKernelGGL((max_window2d_prologue_kernel<OP, 0, 0, TRUNC>), g, b, lds_bytes, stream, a, *pro);
+				}
+				return;
+			}
 			if ((a.win_w == 3) && (a.win_h == 3))
 				hipLaunchKernelGGL((max_window2d_kernel<OP, 3, 3, TRUNC>), dim3(grid), dim3(max_block_size), lds_bytes, stream, a);
 			else if ((a.win_w == 2) && (a.win_h == 2))
 				hipLaunchKernelGGL((max_window2d_kernel<OP, 2, 2, TRUNC>), dim3(grid), dim3(max_block_size), lds_bytes, stream, a);
 			else
 				hipLaunchKernelGGL((max_window2d_kernel<OP, 0, 0, TRUNC>), dim3(grid), dim3(max_block_size), lds_bytes, stream, a);
+		}
+
+		// The layers of a single-input group without Add, in order, as the kernel wants them. False when
+		// the description is not such a group or a weight pointer is missing.
+		bool fill_prologue(window_prologue& pro, const nnf_hip_chain_desc& desc, const float* const* chunk_ptrs, uint32_t feature_map_count, uint32_t in_plane)
+		{
+			if ((desc.input_count != 1) || desc.has_add || (feature_map_count == 0))
+				return false;
+			const uint32_t op_count = desc.arm_op_count[0] + desc.tail_op_count;
+			if ((op_count == 0) || (op_count > NNF_HIP_MAX_OPS))
+				return false;
+			pro.op_count = op_count;
+			pro.fm_count = feature_map_count;
+			pro.weighted_count = 0;
+			pro.need_exp = 0;
+			pro.in_plane_magic = magic_of(in_plane);
+			for(uint32_t i = 0; i < op_count; ++i)
+			{
+				const nnf_hip_op& src = desc.ops[i];
+				pro.kind[i] = src.kind;
+				pro.f0[i] = src.f0;
+				pro.f1[i] = src.f1;
+				pro.slot[i] = 2 * pro.weighted_count;
+				switch (src.kind)
+				{
+				case NNF_HIP_OP_BATCH_NORM:
+				case NNF_HIP_OP_PRELU:
+					{
+						const uint32_t j = pro.weighted_count++;
+						if (j < prologue_weighted_max)
+							pro.weighted_kind[j] = src.kind;
+						if ((chunk_ptrs == nullptr) || (src.chunk < 0))
+							return false;
+						const int chunk_count = (src.kind == NNF_HIP_OP_BATCH_NORM) ? 4 : 1;
+						for(int c = 0; c < chunk_count; ++c)
+						{
+							if (chunk_ptrs[src.chunk + c] == nullptr)
+								return false;
+							if (j < prologue_weighted_max)
+								pro.weights[j][c] = chunk_ptrs[src.chunk + c];
+						}
+					}
+					break;
+				case NNF_HIP_OP_TANH:
+					pro.f1[i] = src.f1 * 2.0f; // nnforge/plain/hyperbolic_tangent_layer_tester_plain.cpp:49
+					pro.need_exp = 1;
+					break;
+				case NNF_HIP_OP_ELU:
+				case NNF_HIP_OP_SIGMOID:
+					pro.need_exp = 1;
+					break;
+				case NNF_HIP_OP_RELU:
+				case NNF_HIP_OP_ABSOLUTE:
+				case NNF_HIP_OP_DROPOUT:
+					break;
+				default:
+					return false;
+				}
+			}
+			return true;
 		}
 
 		// LDS floats a workgroup of the 2-D kernel stages; NNF_HIP_POOL_LDS_FLOATS overrides it (tuning)
@@ -331,6 +690,28 @@ namespace nnf
 	// plane, or a single band of window_height input rows that does not fit LDS.
 	bool window2d_launch(hipStream_t stream, int op, float mult, float* output, const float* input, uint32_t input_total, uint32_t plane_count,
 		uint32_t in_w, uint32_t in_h, uint32_t out_w, uint32_t out_h, uint32_t win_w, uint32_t win_h, uint32_t stride_x, uint32_t stride_y)
+	{
+		return window2d_launch_with_prologue(stream, op, mult, output, input, input_total, plane_count, in_w, in_h, out_w, out_h,
+			win_w, win_h, stride_x, stride_y, nullptr, nullptr, 0, false);
+	}
+
+	// NNF_HIP_OK when desc describes layers a subsampling kernel can apply to its input: one input, no
+	// Add, 1..NNF_HIP_MAX_OPS known layers, every weight pointer they name present (NNF_HIP_EINVAL
+	// otherwise), at most two of them with weights (NNF_HIP_EUNSUPPORTED).
+	int prologue_status(const nnf_hip_chain_desc& desc, const float* const* chunk_ptrs)
+	{
+		window_prologue pro = {};
+		if (!fill_prologue(pro, desc, chunk_ptrs, std::max(1u, desc.feature_map_count), std::max(1u, desc.neuron_count_per_feature_map)))
+			return NNF_HIP_EINVAL;
+		return (pro.weighted_count > prologue_weighted_max) ? NNF_HIP_EUNSUPPORTED : NNF_HIP_OK;
+	}
+
+	// As window2d_launch; with prologue != null the layers of that single-input group are applied to the
+	// input on its way into LDS (feature_map_count: feature maps of the input). plan_only: nothing is
+	// launched, the return value tells whether this shape would run (with the prologue, if one is given).
+	bool window2d_launch_with_prologue(hipStream_t stream, int op, float mult, float* output, const float* input, uint32_t input_total, uint32_t plane_count,
+		uint32_t in_w, uint32_t in_h, uint32_t out_w, uint32_t out_h, uint32_t win_w, uint32_t win_h, uint32_t stride_x, uint32_t stride_y,
+		const nnf_hip_chain_desc* prologue, const float* const* chunk_ptrs, uint32_t feature_map_count, bool plan_only)
 	{
 		const uint32_t lds_floats_wanted = staging_floats();
 		constexpr uint32_t lds_floats_max = 15 * 1024;
@@ -372,28 +753,52 @@ namespace nnf
 		}
 		if (!fits)
 			return false;
+		window_prologue pro = {};
+		if (prologue != nullptr)
+		{
+			// a float4 of a workgroup's range may straddle two planes, not three
+			if ((a.planes > 1) && (plane < 4))
+				return false;
+			if (!plan_only && (!fill_prologue(pro, *prologue, chunk_ptrs, feature_map_count, plane) || (pro.weighted_count > prologue_weighted_max)))
+				return false;
+			// the planes of a workgroup keep their coefficients in LDS
+			a.planes = std::min(a.planes, std::min(prologue_planes_max, prologue_coef_floats / (2 * prologue_weighted_max)));
+		}
+		if (plan_only)
+			return true;
 		a.bands = (a.out_h + a.rows - 1) / a.rows;
 		a.out_w_magic = magic_of(a.out_w);
 		a.band_magic = magic_of(a.rows * a.out_w);
 		const uint32_t rows_in = (a.planes > 1 || a.bands == 1) ? a.in_h : std::min(a.in_h, (a.rows - 1) * a.stride_y + a.win_h);
 		const size_t lds_bytes = (static_cast<size_t>(a.planes - 1) * plane + static_cast<size_t>(rows_in) * a.in_w + 8) * sizeof(float);
 		const uint32_t grid = ((a.plane_count + a.planes - 1) / a.planes) * a.bands;
+		const window_prologue* use = (prologue != nullptr) ? &pro : nullptr;
 		switch (op)
 		{
-		case 0: launch_window2d<window_op_max, false>(stream, a, grid, lds_bytes); break;
-		case 1: launch_window2d<window_op_min, false>(stream, a, grid, lds_bytes); break;
-		case 2: launch_window2d<window_op_max, true>(stream, a, grid, lds_bytes); break;
-		case 3: launch_window2d<window_op_min, true>(stream, a, grid, lds_bytes); break;
-		default: launch_window2d<window_op_sum, false>(stream, a, grid, lds_bytes); break;
+		case 0: launch_window2d<window_op_max, false>(stream, a, grid, lds_bytes, use); break;
+		case 1: launch_window2d<window_op_min, false>(stream, a, grid, lds_bytes, use); break;
+		case 2: launch_window2d<window_op_max, true>(stream, a, grid, lds_bytes, use); break;
+		case 3: launch_window2d<window_op_min, true>(stream, a, grid, lds_bytes, use); break;
+		default: launch_window2d<window_op_sum, false>(stream, a, grid, lds_bytes, use); break;
 		}
 		return true;
 	}
 
-	int max_subsampling_forward(hipStream_t stream, float* output, const float* input,
+	// prologue != null: the layers of that group are applied to the input first (LDS-staged kernel only:
+	// NNF_HIP_EUNSUPPORTED for shapes it does not take). plan_only: nothing is launched and no pointer is
+	// looked at; NNF_HIP_OK means the call would run.
+	int max_subsampling_forward_with_prologue(hipStream_t stream, float* output, const float* input,
 		uint32_t output_entry_count, uint32_t input_feature_map_count, uint32_t dimension_count,
 		const uint32_t* input_sizes, const uint32_t* subsampling_sizes, const uint32_t* strides, const uint32_t* round_ups,
-		uint32_t feature_map_subsampling_size, uint32_t entry_subsampling_size, int32_t is_min)
+		uint32_t feature_map_subsampling_size, uint32_t entry_subsampling_size, int32_t is_min,
+		const nnf_hip_chain_desc* prologue, const float* const* chunk_ptrs, bool plan_only)
 	{
+		if (plan_only)
+		{
+			// planning looks at shapes only: stand-ins that pass the pointer checks below, never dereferenced
+			output = reinterpret_cast<float*>(static_cast<uintptr_t>(16));
+			input = reinterpret_cast<const float*>(static_cast<uintptr_t>(1) << 46);
+		}
 		if ((output == nullptr) || (input == nullptr) || (input_sizes == nullptr) || (subsampling_sizes == nullptr))
 			return NNF_HIP_EINVAL;
 		if ((dimension_count < 1) || (dimension_count > max_dims))
@@ -445,10 +850,15 @@ namespace nnf
 		if (within_plane)
 		{
 			const int op = is_min ? (round_up_anywhere ? 3 : 1) : (round_up_anywhere ? 2 : 0);
-			if (window2d_launch(stream, op, 0.0f, output, input, static_cast<uint32_t>(input_total), output_entry_count * input_feature_map_count,
-				nd.in_size[0], nd.in_size[1], nd.out_size[0], nd.out_size[1], nd.window[0], nd.window[1], nd.stride[0], nd.stride[1]))
-				return launch_status();
+			if (window2d_launch_with_prologue(stream, op, 0.0f, output, input, static_cast<uint32_t>(input_total), output_entry_count * input_feature_map_count,
+				nd.in_size[0], nd.in_size[1], nd.out_size[0], nd.out_size[1], nd.window[0], nd.window[1], nd.stride[0], nd.stride[1],
+				prologue, chunk_ptrs, input_feature_map_count, plan_only))
+				return plan_only ? NNF_HIP_OK : launch_status();
 		}
+		if (prologue != nullptr)
+			return NNF_HIP_EUNSUPPORTED; // only the LDS-staged kernel applies a prologue
+		if (plan_only)
+			return NNF_HIP_OK;
 
 		nd.out = output;
 		nd.in = input;
@@ -464,6 +874,15 @@ namespace nnf
 		else
 			hipLaunchKernelGGL(max_window_nd_kernel<false>, grid, dim3(max_block_size), 0, stream, nd);
 		return launch_status();
+	}
+
+	int max_subsampling_forward(hipStream_t stream, float* output, const float* input,
+		uint32_t output_entry_count, uint32_t input_feature_map_count, uint32_t dimension_count,
+		const uint32_t* input_sizes, const uint32_t* subsampling_sizes, const uint32_t* strides, const uint32_t* round_ups,
+		uint32_t feature_map_subsampling_size, uint32_t entry_subsampling_size, int32_t is_min)
+	{
+		return max_subsampling_forward_with_prologue(stream, output, input, output_entry_count, input_feature_map_count, dimension_count,
+			input_sizes, subsampling_sizes, strides, round_ups, feature_map_subsampling_size, entry_subsampling_size, is_min, nullptr, nullptr, false);
 	}
 
 	int maxout_forward(hipStream_t stream, float* output, const float* input,

@@ -114,6 +114,24 @@ namespace nnf
 		uint32_t entry_count, uint32_t feature_map_count, uint32_t input_width, uint32_t input_height,
 		uint32_t window_width, uint32_t window_height, float mult)
 	{
+		return average_subsampling_forward_with_prologue(stream, output, input, entry_count, feature_map_count, input_width, input_height,
+			window_width, window_height, mult, nullptr, nullptr, false);
+	}
+
+	// prologue != null: the layers of that group are applied to the input first (LDS-staged window kernel
+	// only: NNF_HIP_EUNSUPPORTED for whole-plane windows and other shapes it does not take). plan_only:
+	// nothing is launched and no pointer is looked at; NNF_HIP_OK means the call would run.
+	int average_subsampling_forward_with_prologue(hipStream_t stream, float* output, const float* input,
+		uint32_t entry_count, uint32_t feature_map_count, uint32_t input_width, uint32_t input_height,
+		uint32_t window_width, uint32_t window_height, float mult,
+		const nnf_hip_chain_desc* prologue, const float* const* chunk_ptrs, bool plan_only)
+	{
+		if (plan_only)
+		{
+			// planning looks at shapes only: stand-ins that pass the pointer checks below, never dereferenced
+			output = reinterpret_cast<float*>(static_cast<uintptr_t>(16));
+			input = reinterpret_cast<const float*>(static_cast<uintptr_t>(1) << 46);
+		}
 		if ((output == nullptr) || (input == nullptr))
 			return NNF_HIP_EINVAL;
 		if ((feature_map_count == 0) || (input_width == 0) || (input_height == 0) || (window_width == 0) || (window_height == 0))
@@ -141,6 +159,17 @@ namespace nnf
 		}
 
 		const uint32_t plane = input_width * input_height;
+		if (prologue != nullptr)
+		{
+			const bool whole_plane = (window_width == input_width) && (window_height == input_height) && (plane >= 2) && (plane <= global_pool_max_plane);
+			if (whole_plane || !window2d_launch_with_prologue(stream, 4, mult, output, input, static_cast<uint32_t>(input_total), plane_count,
+				input_width, input_height, output_width, output_height, window_width, window_height, window_width, window_height,
+				prologue, chunk_ptrs, feature_map_count, plan_only))
+				return NNF_HIP_EUNSUPPORTED;
+			return plan_only ? NNF_HIP_OK : launch_status();
+		}
+		if (plan_only)
+			return NNF_HIP_OK;
 		if ((window_width == input_width) && (window_height == input_height) && (plane >= 2) && (plane <= global_pool_max_plane))
 		{
 			// 64 planes of 7x7; fewer of larger planes, so that a compute unit holds several workgroups

@@ -61,6 +61,7 @@ namespace nnforge
 				int output_buffer;
 				std::vector<int> input_buffers;
 				bool passes_input_on = false;        // every layer of the step is a Dropout
+				bool prologue = false;               // desc holds element-wise layers that the tester (a subsampling layer) applies to its input
 			};
 
 			bool is_unary_elementwise(const std::string& type)
@@ -199,6 +200,7 @@ namespace nnforge
 			std::map<std::string, pending_group> pending;
 			std::vector<std::pair<std::string, pending_group> > groups; // materialized, in execution order
 			std::vector<std::pair<std::string, bool> > step_order;      // (layer name, is_group)
+			std::map<std::string, pending_group> prologues;             // subsampling layer -> the group it applies to its input
 
 			auto materialize = [&](const std::string& name)
 			{
@@ -278,6 +280,30 @@ namespace nnforge
 
 				if (!grouped)
 				{
+					// A subsampling layer takes the pending group that feeds it along: the group's layers are
+					// applied to the values on their way into the subsampling kernel's staging buffer.
+					if (hip_config->fuse_layers && (l->input_layer_instance_names.size() == 1) && p->testers[name]->can_apply_prologue())
+					{
+						const std::string& producer = l->input_layer_instance_names[0];
+						std::map<std::string, pending_group>::iterator it = pending.find(producer);
+						if ((it != pending.end()) && it->second.add_layer_name.empty() && (it->second.arms.size() == 1)
+							&& (this->schema->get_consumer_count(producer) == 1) && (outputs.find(producer) == outputs.end()))
+						{
+							unsigned int weighted = 0;
+							bool only_dropout = true; // such a group costs no launch on its own
+							for(const std::string& op_layer : it->second.arms[0].ops)
+							{
+								nnf_hip_op op;
+								weighted += (p->testers[op_layer]->get_chain_op(op) > 0) ? 1u : 0u;
+								only_dropout = only_dropout && (this->schema->get_layer(op_layer)->get_type_name() == dropout_layer::layer_type_name);
+							}
+							if ((weighted <= 2) && !only_dropout)
+							{
+								prologues[name] = it->second;
+								pending.erase(it);
+							}
+						}
+					}
 					for(const std::string& producer : l->input_layer_instance_names)
 						materialize(producer);
 					step_order.push_back(std::make_pair(name, false));
@@ -306,7 +332,54 @@ namespace nnforge
 				plan.output_buffer = -1;
 				const std::string& name = so.first;
 				const layer_configuration_specific& config = layer_config_map[name];
-				if (!so.second)
+				// the group's layers as the kernels want them; shape: the tensors the group works on
+				auto fill_desc = [&](const pending_group& g, const layer_configuration_specific& shape)
+				{
+					nnf_hip_chain_desc& d = plan.desc;
+					d.feature_map_count = shape.feature_map_count;
+					d.neuron_count_per_feature_map = shape.get_neuron_count_per_feature_map();
+					d.input_count = static_cast<uint32_t>(g.arms.size());
+					d.has_add = g.add_layer_name.empty() ? 0u : 1u;
+					d.add_alpha = 1.0F;
+					if (d.has_add)
+						get_add_alpha(*p->testers[g.add_layer_name], d.add_alpha);
+					uint32_t op_index = 0;
+					int chunk_index = 0;
+					auto push_op = [&](const std::string& layer_name)
+					{
+						nnf_hip_op& op = d.ops[op_index++];
+						const int chunks = p->testers[layer_name]->get_chain_op(op);
+						if (chunks < 0)
+							throw neural_network_exception("Layer " + layer_name + " cannot be part of a fused group");
+						op.chunk = chunk_index;
+						if (chunks > 0)
+						{
+							plan.chunk_layers.push_back(layer_name);
+							chunk_index += chunks;
+						}
+					};
+					for(size_t j = 0; j < g.arms.size(); ++j)
+					{
+						d.arm_op_count[j] = static_cast<uint32_t>(g.arms[j].ops.size());
+						for(const std::string& op : g.arms[j].ops)
+							push_op(op);
+					}
+					d.tail_op_count = static_cast<uint32_t>(g.tail.size());
+					for(const std::string& op : g.tail)
+						push_op(op);
+				};
+				if (!so.second && (prologues.find(name) != prologues.end()))
+				{
+					const pending_group& g = prologues[name];
+					plan.info.layer_names = g.arms[0].ops;
+					plan.info.layer_names.push_back(name);
+					plan.info.input_names.push_back(g.arms[0].source);
+					plan.info.fused = true;
+					plan.prologue = true;
+					plan.tester = p->testers[name];
+					fill_desc(g, layer_config_map[g.arms[0].source]);
+				}
+				else if (!so.second)
 				{
 					layer::const_ptr l = this->schema->get_layer(name);
 					plan.info.layer_names.push_back(name);
@@ -337,38 +410,7 @@ namespace nnforge
 					else
 					{
 						plan.info.fused = true;
-						nnf_hip_chain_desc& d = plan.desc;
-						d.feature_map_count = config.feature_map_count;
-						d.neuron_count_per_feature_map = config.get_neuron_count_per_feature_map();
-						d.input_count = static_cast<uint32_t>(g.arms.size());
-						d.has_add = g.add_layer_name.empty() ? 0u : 1u;
-						d.add_alpha = 1.0F;
-						if (d.has_add)
-							get_add_alpha(*p->testers[g.add_layer_name], d.add_alpha);
-						uint32_t op_index = 0;
-						int chunk_index = 0;
-						auto push_op = [&](const std::string& layer_name)
-						{
-							nnf_hip_op& op = d.ops[op_index++];
-							const int chunks = p->testers[layer_name]->get_chain_op(op);
-							if (chunks < 0)
-								throw neural_network_exception("Layer " + layer_name + " cannot be part of a fused group");
-							op.chunk = chunk_index;
-							if (chunks > 0)
-							{
-								plan.chunk_layers.push_back(layer_name);
-								chunk_index += chunks;
-							}
-						};
-						for(size_t j = 0; j < g.arms.size(); ++j)
-						{
-							d.arm_op_count[j] = static_cast<uint32_t>(g.arms[j].ops.size());
-							for(const std::string& op : g.arms[j].ops)
-								push_op(op);
-						}
-						d.tail_op_count = static_cast<uint32_t>(g.tail.size());
-						for(const std::string& op : g.tail)
-							push_op(op);
+						fill_desc(g, config);
 					}
 				}
 				// report bookkeeping: name, layer types, flops (the reference's model) and memory traffic per entry
@@ -428,7 +470,7 @@ namespace nnforge
 				if (!dedicated)
 				{
 					// in place: the first input dies here, nothing else reads its buffer in this step, same size
-					const int can_write = plan.info.fused ? 0 : plan.tester->get_input_index_layer_can_write();
+					const int can_write = plan.prologue ? -1 : (plan.info.fused ? 0 : plan.tester->get_input_index_layer_can_write());
 					if (can_write == 0)
 					{
 						const int b0 = plan.input_buffers[0];
@@ -694,7 +736,13 @@ namespace nnforge
 							inputs.push_back(buffers[slot][b]);
 						if (plan.passes_input_on && (plan.output_buffer == plan.input_buffers.at(0)))
 							continue; // Dropout layers only, in place: nothing to do at inference
-						if (plan.info.fused)
+						if (plan.prologue)
+						{
+							plan.desc.entry_count = entries_read;
+							plan.tester->enqueue_forward_propagation_with_prologue(p->stream, buffers[slot][plan.output_buffer], inputs.at(0), plan.desc,
+								chunk_ptrs[i].empty() ? nullptr : chunk_ptrs[i].data(), entries_read);
+						}
+						else if (plan.info.fused)
 						{
 							plan.desc.entry_count = entries_read;
 							std::vector<const float *> in_ptrs;

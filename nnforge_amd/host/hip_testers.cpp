@@ -140,6 +140,12 @@ namespace nnforge
 			return res;
 		}
 
+		void layer_tester_hip::enqueue_forward_propagation_with_prologue(void *, hip_linear_buffer_device::ptr, hip_linear_buffer_device::const_ptr,
+			const nnf_hip_chain_desc&, const float * const *, unsigned int)
+		{
+			throw neural_network_exception("Layer " + layer_schema->instance_name + " of type " + layer_schema->get_type_name() + " cannot apply other layers to its input");
+		}
+
 		layer_testing_schema::ptr layer_testing_schema::create(layer::const_ptr layer_schema) const
 		{
 			layer_testing_schema::ptr res = create_specific();
@@ -455,6 +461,20 @@ namespace nnforge
 						entry_count, output_configuration_specific.feature_map_count, input_width, input_height, window_width, window_height, mult));
 				}
 
+				bool can_apply_prologue() const override
+				{
+					return nnf_hip_average_subsampling_fusable(1, output_configuration_specific.feature_map_count, input_width, input_height,
+						window_width, window_height) == NNF_HIP_OK;
+				}
+
+				void enqueue_forward_propagation_with_prologue(void * stream_id, hip_linear_buffer_device::ptr output_buffer,
+					hip_linear_buffer_device::const_ptr input_buffer, const nnf_hip_chain_desc& prologue, const float * const * chunk_ptrs,
+					unsigned int entry_count) override
+				{
+					hip_safe_call(nnf_hip_average_subsampling_fused_forward(stream_id, *output_buffer, float_ptr(input_buffer), &prologue, chunk_ptrs,
+						entry_count, output_configuration_specific.feature_map_count, input_width, input_height, window_width, window_height, mult));
+				}
+
 			protected:
 				void tester_configured() override
 				{
@@ -582,6 +602,21 @@ namespace nnforge
 				{
 					require_inputs(input_buffers, 1, "MaxSubsampling");
 					hip_safe_call(nnf_hip_max_subsampling_forward(stream_id, *output_buffer, float_ptr(input_buffers[0]), entry_count,
+						input_configuration_specific_list[0].feature_map_count, static_cast<uint32_t>(input_sizes.size()),
+						input_sizes.data(), windows.data(), strides.data(), round_ups.data(), feature_map_subsampling_size, 1, is_min ? 1 : 0));
+				}
+
+				bool can_apply_prologue() const override
+				{
+					return nnf_hip_max_subsampling_fusable(1, input_configuration_specific_list[0].feature_map_count, static_cast<uint32_t>(input_sizes.size()),
+						input_sizes.data(), windows.data(), strides.data(), round_ups.data(), feature_map_subsampling_size, 1) == NNF_HIP_OK;
+				}
+
+				void enqueue_forward_propagation_with_prologue(void * stream_id, hip_linear_buffer_device::ptr output_buffer,
+					hip_linear_buffer_device::const_ptr input_buffer, const nnf_hip_chain_desc& prologue, const float * const * chunk_ptrs,
+					unsigned int entry_count) override
+				{
+					hip_safe_call(nnf_hip_max_subsampling_fused_forward(stream_id, *output_buffer, float_ptr(input_buffer), &prologue, chunk_ptrs, entry_count,
 						input_configuration_specific_list[0].feature_map_count, static_cast<uint32_t>(input_sizes.size()),
 						input_sizes.data(), windows.data(), strides.data(), round_ups.data(), feature_map_subsampling_size, 1, is_min ? 1 : 0));
 				}

@@ -55,8 +55,9 @@ layer { type: "AverageSubsampling" name: "avg_0_layer" input_layer_name: "tanh_0
 	average_subsampling_param { dimension_param { subsampling_size: 2 } dimension_param { subsampling_size: 2 } } }
 '''
     rep = backend.plan_schema(text, {"images": (3, [8, 6])}, ["avg_0_layer"])
-    assert step_names(rep) == ["tanh_0_layer", "avg_0_layer"]
-    assert rep["per_entry_bytes"] == 4 * (3 * 48 + 3 * 48 + 3 * 12)
+    # the average pooling applies TanH to the values it reads: one launch, no buffer for TanH's result
+    assert step_names(rep) == ["tanh_0_layer+avg_0_layer"]
+    assert rep["per_entry_bytes"] == 4 * (3 * 48 + 3 * 12)
 
 
 def test_schema_errors():
@@ -209,6 +210,53 @@ def test_plan_of_the_inception_like_block():
     # alone (and costs no launch when it runs in place); TanH follows pool2.
     assert step_names(rep) == ["pool1", "b1_bn+b1_relu", "b2_drop+b2_abs", "b3_prelu", "join", "mo", "drop", "pool2", "out"]
     assert rep["steps"][4]["inputs"] == ["b1_relu", "b2_abs", "b3_prelu", "pool1"]
+
+
+def stem_net(c=8):
+    """BatchNorm -> ReLU -> overlapping max pooling, then TanH -> Absolute -> 2x2 average pooling (the stage of
+    nnForge's GTSRB example, examples/gtsrb/schema.txt), then a global average."""
+    return [S.L("Data", "conv1"), S.L("BatchNorm", "bn", ["conv1"], feature_map_count=c), S.L("ReLU", "relu", ["bn"]),
+            S.L("MaxSubsampling", "pool1", ["relu"], windows=[3, 3], strides=[2, 2], round_ups=[True, True]),
+            S.L("TanH", "tanh", ["pool1"], scale=1.7159, steepness=0.6666), S.L("Absolute", "abs", ["tanh"]),
+            S.L("AverageSubsampling", "pool2", ["abs"], windows=[2, 2]),
+            S.L("ELU", "elu", ["pool2"]), S.L("AverageSubsampling", "global", ["elu"], windows=[7, 7], alpha=1.0 / 49.0)]
+
+
+def test_plan_folds_a_group_into_the_subsampling_layer_behind_it():
+    rep = plan(stem_net(), {"conv1": (8, [28, 28])}, ["global"])
+    # the whole-plane average has a kernel of its own that applies no layers: ELU runs in front of it
+    assert step_names(rep) == ["bn+relu+pool1", "tanh+abs+pool2", "elu", "global"]
+    assert [s["fused"] for s in rep["steps"]] == [True, True, False, False]
+    assert rep["steps"][0]["inputs"] == ["conv1"] and rep["steps"][1]["inputs"] == ["pool1"]
+    # no intermediate tensor of the groups is planned: conv1, pool1 (14x14), pool2 (7x7, ELU in place), global
+    assert rep["per_entry_bytes"] == 8 * 4 * (28 * 28 + 14 * 14 + 7 * 7 + 1)
+    # a 7x7 window over 14x14 planes is an ordinary window: ELU goes along
+    assert step_names(plan(stem_net(), {"conv1": (8, [56, 56])}, ["global"]))[2:] == ["elu+global"]
+    rep = plan(stem_net(), {"conv1": (8, [28, 28])}, ["global"], fuse=False)
+    assert len(rep["steps"]) == 8 and not any(s["fused"] for s in rep["steps"])
+
+
+def test_plan_keeps_a_group_out_of_the_subsampling_layer_when_it_must_be_stored():
+    c = 4
+    base = [S.L("Data", "x"), S.L("BatchNorm", "bn", ["x"], feature_map_count=c), S.L("ReLU", "relu", ["bn"]),
+            S.L("MaxSubsampling", "pool", ["relu"], windows=[2, 2])]
+    # the group's result is an output, or has a second consumer
+    assert step_names(plan(base, {"x": (c, [8, 8])}, ["pool", "relu"])) == ["bn+relu", "pool"]
+    two = base + [S.L("MaxSubsampling", "pool_b", ["relu"], windows=[4, 4])]
+    assert step_names(plan(two, {"x": (c, [8, 8])}, ["pool", "pool_b"])) == ["bn+relu", "pool", "pool_b"]
+    # a group with an Add
+    block = S.resnet_block(c) + [S.L("MaxSubsampling", "pool", ["res_relu"], windows=[2, 2])]
+    assert step_names(plan(block, {"conv_main": (c, [8, 8]), "conv_shortcut": (c, [8, 8])}, ["pool"])) == ["shortcut_bn+main_bn+res+res_relu", "pool"]
+    # more than two layers with weights
+    heavy = [S.L("Data", "x"), S.L("BatchNorm", "bn1", ["x"], feature_map_count=c), S.L("PReLU", "pr", ["bn1"], feature_map_count=c),
+             S.L("BatchNorm", "bn2", ["pr"], feature_map_count=c), S.L("MaxSubsampling", "pool", ["bn2"], windows=[2, 2])]
+    assert step_names(plan(heavy, {"x": (c, [8, 8])}, ["pool"])) == ["bn1+pr+bn2", "pool"]
+    assert step_names(plan(heavy[:3] + [S.L("MaxSubsampling", "pool", ["pr"], windows=[2, 2])], {"x": (c, [8, 8])}, ["pool"])) == ["bn1+pr+pool"]
+    # windows over feature maps, three spatial dimensions
+    fm = base[:3] + [S.L("MaxSubsampling", "pool", ["relu"], windows=[2, 2], fm_window=2)]
+    assert step_names(plan(fm, {"x": (c, [8, 8])}, ["pool"])) == ["bn+relu", "pool"]
+    deep = base[:3] + [S.L("MaxSubsampling", "pool", ["relu"], windows=[2, 2, 2])]
+    assert step_names(plan(deep, {"x": (c, [8, 8, 8])}, ["pool"])) == ["bn+relu", "pool"]
 
 
 def test_neighbour_layer_configuration_rules():

@@ -184,6 +184,34 @@ def test_inception_like_block_with_the_neighbouring_layers(fuse):
     assert_bits(got["out"], values["out"], "output")
 
 
+@pytest.mark.parametrize("fuse", [True, False])
+@pytest.mark.parametrize("size", [28, 57])
+def test_groups_folded_into_the_subsampling_layers_behind_them(fuse, size):
+    """BatchNorm -> ReLU -> max pooling (3x3 every 2, rounded up), TanH -> Absolute -> 2x2 average pooling, ELU -> 7x7
+    average: with fusion on, each pooling layer applies the layers in front of it to the values it reads (one launch,
+    no intermediate tensor) - the whole-plane average excepted, which keeps its own kernel. Same bits either way."""
+    gen = T.rng(62, size + int(fuse))
+    c, n = 10, 13
+    layers = [S.L("Data", "conv1"), S.L("BatchNorm", "bn", ["conv1"], feature_map_count=c), S.L("ReLU", "relu", ["bn"]),
+              S.L("MaxSubsampling", "pool1", ["relu"], windows=[3, 3], strides=[2, 2], round_ups=[True, True]),
+              S.L("TanH", "tanh", ["pool1"], scale=1.7159, steepness=0.6666), S.L("Absolute", "abs", ["tanh"]),
+              S.L("AverageSubsampling", "pool2", ["abs"], windows=[2, 2]),
+              S.L("ELU", "elu", ["pool2"]), S.L("AverageSubsampling", "global", ["elu"], windows=[7, 7], alpha=1.0 / 49.0)]
+    weights = S.make_weights(layers, gen)
+    inputs = {"conv1": T.normal(gen, (n, c, size, size), 2.0)}
+    values = S.evaluate(layers, weights, inputs)
+    got, rep = run(layers, weights, inputs, ["global", "pool2"], values, fuse=fuse, max_entry_count=5)
+    assert rep["entries"] == n
+    assert_bits(got["pool2"], values["pool2"], "average pooling behind TanH and Absolute")
+    assert_bits(got["global"], values["global"], "global average behind ELU")
+    names = ["+".join(s["layers"]) for s in rep["steps"]]
+    if fuse:
+        # 28: pool2 is 7x7 and the last window covers the whole plane; 57: pool2 is 14x14 (29x29 halved), the 7x7 window is an ordinary one
+        assert names == ["bn+relu+pool1", "tanh+abs+pool2"] + (["elu", "global"] if size == 28 else ["elu+global"])
+    else:
+        assert len(names) == 8
+
+
 def test_dropout_only_network():
     """Dropout straight from the data layer to the output: in place there is nothing to launch."""
     gen = T.rng(58, 0)

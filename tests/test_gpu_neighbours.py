@@ -188,3 +188,174 @@ def test_neighbour_entry_points_reject_bad_arguments(gpu):
     assert lib.nnf_hip_concat_forward(s, e.data_ptr(), capi.pointer_array([d.data_ptr()]), u32([16]), 1, 0) == 0
     assert lib.nnf_hip_maxout_forward(s, e.data_ptr(), d.data_ptr(), 0, 4, 4, 2) == 0
     gpu.torch.cuda.synchronize()
+
+
+# ---------------------------------------------------------------------------------------------
+# subsampling with the element-wise layers in front of it folded in
+# ---------------------------------------------------------------------------------------------
+
+def prologue_case(kind, gen, c):
+    """-> (ops of the single arm, weight chunks, oracle steps) of a group in front of a subsampling layer"""
+    if kind == "bn_relu":
+        g, b, m, s = T.bn_params(gen, c)
+        return ([(capi.OP_BATCH_NORM, 0), (capi.OP_RELU, 0, 0.0)], [g, b, m, s],
+                [lambda v: oracle.batch_norm(v, g, b, m, s), lambda v: oracle.rectified_linear(v, 0.0)])
+    if kind == "tanh_abs":
+        return ([(capi.OP_TANH, 0, 1.7159, 0.6666), (capi.OP_ABSOLUTE,)], [],
+                [lambda v: oracle.hyperbolic_tangent(v, 1.7159, 0.6666), oracle.absolute])
+    if kind == "bn_prelu_elu_sigmoid":
+        g, b, m, s = T.bn_params(gen, c)
+        a = T.uniform(gen, c, -0.5, 0.5)
+        return ([(capi.OP_BATCH_NORM, 0), (capi.OP_PRELU, 4), (capi.OP_DROPOUT,), (capi.OP_ELU,), (capi.OP_SIGMOID,)], [g, b, m, s, a],
+                [lambda v: oracle.batch_norm(v, g, b, m, s), lambda v: oracle.parametric_rectified_linear(v, a),
+                 oracle.exponential_linear, oracle.sigmoid])
+    if kind == "prelu_bn":
+        g, b, m, s = T.bn_params(gen, c)
+        a = T.uniform(gen, c, -0.5, 0.5)
+        return ([(capi.OP_PRELU, 0), (capi.OP_ABSOLUTE,), (capi.OP_BATCH_NORM, 1)], [a, g, b, m, s],
+                [lambda v: oracle.parametric_rectified_linear(v, a), oracle.absolute, lambda v: oracle.batch_norm(v, g, b, m, s)])
+    if kind == "leaky":
+        return ([(capi.OP_RELU, 0, 0.1)], [], [lambda v: oracle.rectified_linear(v, 0.1)])
+    raise ValueError(kind)
+
+
+def prologue_input(gen, shape):
+    """Values across the activations' ranges, with the exp range edges, zeros and infinities in."""
+    x = T.normal(gen, shape, 3.0)
+    flat = x.reshape(-1)
+    idx = gen.integers(0, flat.size, size=max(4, flat.size // 50))
+    flat[idx] = gen.choice(np.array([0.0, -0.0, np.inf, -np.inf, 88.8, -88.8, -104.0, 3.0e38, -3.0e38, 1.0e-40], F), size=idx.size)
+    return x
+
+
+FUSED_MAX_CASES = [
+    # shape, windows (x first), strides, round_ups, group
+    ((4, 64, 112, 112), [3, 3], [2, 2], [True, True], "bn_relu"),       # ResNet stem: bands of a plane per workgroup
+    ((2, 6, 112, 112), [3, 3], [2, 2], None, "bn_prelu_elu_sigmoid"),
+    ((8, 96, 55, 55), [3, 3], [2, 2], None, "bn_relu"),                # planes of 3025 floats, several per workgroup
+    ((16, 32, 28, 28), [2, 2], None, None, "tanh_abs"),                # several planes per workgroup
+    ((9, 3, 12, 12), [2, 2], None, None, "bn_prelu_elu_sigmoid"),      # more planes per workgroup than feature maps
+    ((5, 7, 6, 10), [3, 2], [2, 2], [True, False], "bn_relu"),         # run-time window, odd plane counts
+    ((6, 10, 7, 7), [3, 3], [2, 2], None, "bn_prelu_elu_sigmoid"),     # planes of 49 floats: float4s straddle planes
+    ((4, 3, 13, 13), [3, 3], [2, 2], [True, True], "bn_relu"),         # ... with more planes per workgroup than feature maps
+    ((3, 5, 2, 3), [2, 1], [1, 1], None, "bn_relu"),                   # planes of 6 floats
+    ((40, 30, 3, 3), [2, 2], [1, 1], None, "prelu_bn"),                # more planes than a workgroup takes coefficients for
+    ((2, 3, 112, 112), [3, 3], [2, 2], None, "prelu_bn"),
+    ((2, 2, 300, 200), [4, 7], [4, 5], None, "leaky"),
+    ((1, 3, 4, 4000), [3, 2], [2, 2], None, "bn_relu"),                # one output row per band
+]
+
+
+def run_fused_max(gpu, x, ops, chunks, windows, strides, round_ups, is_min=False, fm=1, en=1, expect=0):
+    n, c = x.shape[0], x.shape[1]
+    dims = list(x.shape[2:])[::-1]
+    plane = int(np.prod(dims))
+    out_dims = oracle.max_subsampling_output_sizes(dims, windows, strides, round_ups)
+    want_shape = (n // en, c // fm) + tuple(out_dims[::-1])
+    desc = capi.make_desc(n, c, plane, [ops], [])
+    d_in = gpu.to_device(x)
+    d_chunks = [gpu.to_device(a) for a in chunks]
+    chk = capi.pointer_array([t.data_ptr() for t in d_chunks])
+    d_out = gpu.torch.full((max(1, int(np.prod(want_shape))),), float("nan"), dtype=gpu.torch.float32, device=gpu.device)
+    shape_args = (n // en, c, len(dims), u32(dims), u32(windows), u32(strides) if strides else None,
+                  u32([int(r) for r in round_ups]) if round_ups else None, fm, en)
+    assert gpu.lib.nnf_hip_max_subsampling_fusable(*shape_args) == expect
+    rc = gpu.lib.nnf_hip_max_subsampling_fused_forward(gpu.stream, d_out.data_ptr(), d_in.data_ptr(), ctypes.byref(desc),
+                                                       chk if d_chunks else None, *(shape_args + (int(is_min),)))
+    assert rc == expect, capi.error_string(rc)
+    if expect != 0:
+        gpu.torch.cuda.synchronize()
+        return None
+    return gpu.to_host(d_out, want_shape)
+
+
+@pytest.mark.parametrize("is_min", [False, True])
+@pytest.mark.parametrize("shape,windows,strides,round_ups,group", FUSED_MAX_CASES)
+def test_max_subsampling_with_group_folded_in(gpu, shape, windows, strides, round_ups, group, is_min):
+    gen = T.rng(66, sum(shape))
+    ops, chunks, steps = prologue_case(group, gen, shape[1])
+    x = prologue_input(gen, shape)
+    v = x
+    for step in steps:
+        v = step(v)
+    want = oracle.max_subsampling(v, windows, strides=strides, round_ups=round_ups, is_min=is_min)
+    got = run_fused_max(gpu, x, ops, chunks, windows, strides, round_ups, is_min=is_min)
+    assert got.shape == want.shape
+    assert T.bit_mismatches(got, want) == 0
+
+
+def run_fused_pool(gpu, x, ops, chunks, ww, wh, mult, expect=0):
+    n, c, h, w = x.shape
+    desc = capi.make_desc(n, c, h * w, [ops], [])
+    d_in = gpu.to_device(x)
+    d_chunks = [gpu.to_device(a) for a in chunks]
+    chk = capi.pointer_array([t.data_ptr() for t in d_chunks])
+    out_shape = (n, c, h // wh, w // ww)
+    d_out = gpu.torch.full((int(np.prod(out_shape)),), float("nan"), dtype=gpu.torch.float32, device=gpu.device)
+    assert gpu.lib.nnf_hip_average_subsampling_fusable(n, c, w, h, ww, wh) == expect
+    rc = gpu.lib.nnf_hip_average_subsampling_fused_forward(gpu.stream, d_out.data_ptr(), d_in.data_ptr(), ctypes.byref(desc),
+                                                           chk if d_chunks else None, n, c, w, h, ww, wh, mult)
+    assert rc == expect, capi.error_string(rc)
+    if expect != 0:
+        gpu.torch.cuda.synchronize()
+        return None
+    return gpu.to_host(d_out, out_shape)
+
+
+@pytest.mark.parametrize("shape,ww,wh,group", [
+    ((8, 38, 28, 28), 2, 2, "tanh_abs"),               # the GTSRB stages: TanH -> Absolute -> AverageSubsampling
+    ((3, 5, 12, 12), 2, 2, "tanh_abs"),
+    ((2, 64, 56, 56), 2, 2, "bn_relu"),
+    ((1, 2, 120, 100), 2, 2, "bn_prelu_elu_sigmoid"),  # bands of rows
+    ((2, 3, 113, 115), 3, 3, "bn_relu"),               # leftover margins, plane not a multiple of 4
+    ((1, 4, 9, 7), 3, 2, "leaky"),                     # small planes of 63 floats
+    ((7, 9, 5, 5), 2, 2, "bn_prelu_elu_sigmoid"),      # planes of 25 floats, margins
+])
+def test_average_subsampling_with_group_folded_in(gpu, shape, ww, wh, group):
+    gen = T.rng(67, sum(shape) + ww)
+    ops, chunks, steps = prologue_case(group, gen, shape[1])
+    x = T.normal(gen, shape, 2.0)
+    v = x
+    for step in steps:
+        v = step(v)
+    mult = oracle.average_subsampling_full_mult([ww, wh])
+    want = oracle.average_subsampling(v, [ww, wh], mult=mult)
+    got = run_fused_pool(gpu, x, ops, chunks, ww, wh, mult)
+    assert got.shape == want.shape
+    assert T.bit_mismatches(got, want) == 0
+
+
+def test_subsampling_that_cannot_fold_a_group_in_says_so(gpu):
+    gen = T.rng(68, 0)
+    ops, chunks, _ = prologue_case("bn_relu", gen, 6)
+    # several planes of 3 floats per workgroup (a float4 would straddle three planes), windows over feature
+    # maps, 3-D, rows too wide for the staging buffer
+    run_fused_max(gpu, T.normal(gen, (4, 6, 1, 3)), ops, chunks, [1, 1], None, None, expect=capi.E_UNSUPPORTED)
+    run_fused_max(gpu, T.normal(gen, (4, 6, 8, 8)), ops, chunks, [2, 2], None, None, fm=2, expect=capi.E_UNSUPPORTED)
+    run_fused_max(gpu, T.normal(gen, (2, 6, 4, 6, 8)), ops, chunks, [2, 2, 2], None, None, expect=capi.E_UNSUPPORTED)
+    run_fused_max(gpu, T.normal(gen, (1, 6, 3, 20000)), ops, chunks, [2, 3], [2, 1], None, expect=capi.E_UNSUPPORTED)
+    # whole-plane average windows have their own kernel
+    run_fused_pool(gpu, T.normal(gen, (4, 6, 7, 7)), ops, chunks, 7, 7, 1.0, expect=capi.E_UNSUPPORTED)
+    # a group with an Add, a group of another shape, a missing weight pointer
+    x = gpu.to_device(T.normal(gen, (2, 6, 8, 8)))
+    out = gpu.torch.empty(2 * 6 * 16, dtype=gpu.torch.float32, device=gpu.device)
+    d_chunks = [gpu.to_device(a) for a in chunks]
+    chk = capi.pointer_array([t.data_ptr() for t in d_chunks])
+    shape_args = (2, 6, 2, u32([8, 8]), u32([2, 2]), None, None, 1, 1, 0)
+    call = gpu.lib.nnf_hip_max_subsampling_fused_forward
+    with_add = capi.make_desc(2, 6, 64, [[], ops], [])
+    assert call(gpu.stream, out.data_ptr(), x.data_ptr(), ctypes.byref(with_add), chk, *shape_args) == capi.E_INVAL
+    other_fm = capi.make_desc(2, 5, 64, [ops], [])
+    assert call(gpu.stream, out.data_ptr(), x.data_ptr(), ctypes.byref(other_fm), chk, *shape_args) == capi.E_INVAL
+    other_plane = capi.make_desc(2, 6, 63, [ops], [])
+    assert call(gpu.stream, out.data_ptr(), x.data_ptr(), ctypes.byref(other_plane), chk, *shape_args) == capi.E_INVAL
+    good = capi.make_desc(2, 6, 64, [ops], [])
+    assert call(gpu.stream, out.data_ptr(), x.data_ptr(), None, chk, *shape_args) == capi.E_INVAL
+    assert call(gpu.stream, out.data_ptr(), x.data_ptr(), ctypes.byref(good), None, *shape_args) == capi.E_INVAL
+    assert call(gpu.stream, out.data_ptr(), x.data_ptr(), ctypes.byref(good), chk, *shape_args) == 0
+    # two layers with weights are applied, a third is one too many
+    two = capi.make_desc(2, 6, 64, [[(capi.OP_BATCH_NORM, 0)] * 2], [])
+    three = capi.make_desc(2, 6, 64, [[(capi.OP_BATCH_NORM, 0)] * 3], [])
+    assert call(gpu.stream, out.data_ptr(), x.data_ptr(), ctypes.byref(two), chk, *shape_args) == 0
+    assert call(gpu.stream, out.data_ptr(), x.data_ptr(), ctypes.byref(three), chk, *shape_args) == capi.E_UNSUPPORTED
+    gpu.torch.cuda.synchronize()
