@@ -128,6 +128,57 @@ namespace nnf
 			return r;
 		}
 
+		// One plane per workgroup: the plane's weights through the scalar data cache (the index is the same
+		// in every lane), its coefficients in registers - no LDS table, no barrier, and a wavefront looks
+		// at the weights only after its tensor loads are out.
+		struct uniform_weights
+		{
+			float w[prologue_weighted_max][4];
+		};
+
+		__device__ __forceinline__ uniform_weights load_uniform_weights(uint32_t fm, const window_prologue& pro)
+		{
+			uniform_weights r;
+			const uint32_t fm_s = __builtin_amdgcn_readfirstlane(fm);
+			#pragma unroll
+			for(uint32_t j = 0; j < prologue_weighted_max; ++j)
+			{
+				#pragma unroll
+				for(int c = 0; c < 4; ++c)
+					r.w[j][c] = 0.0f;
+				if (j < pro.weighted_count)
+				{
+					r.w[j][0] = pro.weights[j][0][fm_s];
+					if (pro.weighted_kind[j] == NNF_HIP_OP_BATCH_NORM)
+					{
+						#pragma unroll
+						for(int c = 1; c < 4; ++c)
+							r.w[j][c] = pro.weights[j][c][fm_s];
+					}
+				}
+			}
+			return r;
+		}
+
+		__device__ __forceinline__ void uniform_coefficients(float (&own)[prologue_weighted_max][2], uniform_weights r, const window_prologue& pro)
+		{
+			#pragma unroll
+			for(uint32_t j = 0; j < prologue_weighted_max; ++j)
+			{
+				#pragma unroll
+				for(int c = 0; c < 4; ++c)
+					asm volatile("" : "+s"(r.w[j][c]));
+			}
+			#pragma unroll
+			for(uint32_t j = 0; j < prologue_weighted_max; ++j)
+			{
+				own[j][0] = r.w[j][0];
+				own[j][1] = 0.0f;
+				if ((j < pro.weighted_count) && (pro.weighted_kind[j] == NNF_HIP_OP_BATCH_NORM))
+					nnf_batch_norm_coefficients(r.w[j][0], r.w[j][1], r.w[j][2], r.w[j][3], own[j][0], own[j][1]);
+			}
+		}
+
 		__device__ __forceinline__ void stage_prologue_coefficients(float* coef, prologue_weights r, uint32_t planes_here, const window_prologue& pro)
 		{
 			// The weights are not looked at before this point: without it the compiler works the
@@ -160,9 +211,11 @@ namespace nnf
 		// which leaves the kernel with far fewer registers per lane.
 		constexpr int coef_batch = 4; // vectors whose batch norm coefficients are read from LDS together
 
-		template<int VECTORS, bool EXP>
+		// UNIFORM: every value belongs to the same plane, whose coefficients are in own (registers)
+		// instead of coef (LDS).
+		template<int VECTORS, bool EXP, bool UNIFORM>
 		__device__ __forceinline__ void apply_prologue(float (&v)[VECTORS][4], const uint32_t (&off)[VECTORS],
-			const float* coef, const window_prologue& pro, const exp_context& exp_ctx)
+			const float* coef, const float (&own)[prologue_weighted_max][2], const window_prologue& pro, const exp_context& exp_ctx)
 		{
 			for(uint32_t i = 0; i < pro.op_count; ++i)
 			{
@@ -172,6 +225,20 @@ namespace nnf
 				switch (kind)
 				{
 				case NNF_HIP_OP_BATCH_NORM:
+					if (UNIFORM)
+					{
+						static_assert(prologue_weighted_max == 2, "the coefficients of a layer are picked from two sets");
+						const float mult = (slot == 0) ? own[0][0] : own[1][0];
+						const float add = (slot == 0) ? own[0][1] : own[1][1];
+						#pragma unroll
+						for(int k = 0; k < VECTORS; ++k)
+						{
+							#pragma unroll
+							for(int e = 0; e < 4; ++e)
+								v[k][e] = nnf_batch_norm(v[k][e], mult, add);
+						}
+						break;
+					}
 					#pragma unroll
 					for(int k0 = 0; k0 < VECTORS; k0 += coef_batch)
 					{
@@ -192,6 +259,18 @@ namespace nnf
 					}
 					break;
 				case NNF_HIP_OP_PRELU:
+					if (UNIFORM)
+					{
+						const float slope = (slot == 0) ? own[0][0] : own[1][0];
+						#pragma unroll
+						for(int k = 0; k < VECTORS; ++k)
+						{
+							#pragma unroll
+							for(int e = 0; e < 4; ++e)
+								v[k][e] = nnf_parametric_rectified_linear(v[k][e], slope);
+						}
+					}
+					else
 					{
 						float slope[VECTORS];
 						#pragma unroll
@@ -271,7 +350,7 @@ namespace nnf
 		// PROLOGUE: the staged values go through the layers of pro first, with the weights of the feature
 		// map each value belongs to (a float4 may straddle two planes when several planes that are not
 		// a multiple of four floats long share a workgroup; the host declines planes of under 4 floats).
-		template<int OP, int WIN_W, int WIN_H, bool TRUNC, bool PROLOGUE, bool EXP>
+		template<int OP, int WIN_W, int WIN_H, bool TRUNC, bool PROLOGUE, bool EXP, bool UNIFORM>
 		__device__ __forceinline__ void window2d_body(const window2d_args& a, const window_prologue& pro)
 		{
 			extern __shared__ __align__(16) float lds_in[];
@@ -303,8 +382,16 @@ namespace nnf
 			constexpr int STAGE = stage_vectors_per_lane;
 			// the weights are requested first and looked at once the first round's tensor loads are out
 			prologue_weights weights;
+			uniform_weights plane_weights;
+			float own_coef[prologue_weighted_max][2];
+			constexpr bool uniform = PROLOGUE && UNIFORM; // every workgroup of the launch stages (part of) one plane
 			if (PROLOGUE)
-				weights = load_prologue_weights(first_plane % pro.fm_count, planes_here, pro);
+			{
+				if (uniform)
+					plane_weights = load_uniform_weights(first_plane % pro.fm_count, pro);
+				else
+					weights = load_prologue_weights(first_plane % pro.fm_count, planes_here, pro);
+			}
 			for(uint32_t base = 0; base < vectors; base += STAGE * max_block_size)
 			{
 				floatx4 t[STAGE];
@@ -329,10 +416,14 @@ namespace nnf
 				}
 				if (PROLOGUE && (base == 0))
 				{
-					stage_prologue_coefficients(lds_coef, weights, planes_here, pro);
+					if (uniform)
+						uniform_coefficients(own_coef, plane_weights, pro);
+					else
+						stage_prologue_coefficients(lds_coef, weights, planes_here, pro);
 					if (EXP)
 						stage_exp2_table(lds_exp);
-					__syncthreads();
+					if (EXP || !uniform)
+						__syncthreads();
 					if (EXP)
 						exp_ctx = exp_context_from_lds(lds_exp);
 				}
@@ -360,7 +451,10 @@ namespace nnf
 						if (straddle && valid && (p + 1 < planes_here) && (i * 4 + 3 >= (p + 1) * in_plane + shift))
 							straddling |= 1u << k;
 					}
-					apply_prologue<STAGE, EXP>(v, off, lds_coef, pro, exp_ctx);
+					if (uniform)
+						apply_prologue<STAGE, EXP, true>(v, off, lds_coef, own_coef, pro, exp_ctx);
+					else
+						apply_prologue<STAGE, EXP, false>(v, off, lds_coef, own_coef, pro, exp_ctx);
 					// The floats of the second plane of a straddling float4 were given the first plane's
 					// coefficients: they are fetched again and go through the layers with their own.
 					while (__any(straddling != 0))
@@ -379,7 +473,7 @@ namespace nnf
 							w[0][e] = (mine && (e >= split) && (g < a.total_in)) ? a.in[g] : 0.0f;
 						}
 						const uint32_t off_next[1] = { p_next * (2 * pro.weighted_count) };
-						apply_prologue<1, EXP>(w, off_next, lds_coef, pro, exp_ctx);
+						apply_prologue<1, EXP, false>(w, off_next, lds_coef, own_coef, pro, exp_ctx);
 						#pragma unroll
 						for(int k = 0; k < STAGE; ++k)
 						{
@@ -455,21 +549,22 @@ namespace nnf
 		__global__ void __launch_bounds__(max_block_size) max_window2d_kernel(const window2d_args a)
 		{
 			window_prologue none; // not read
-			window2d_body<OP, WIN_W, WIN_H, TRUNC, false, false>(a, none);
+			window2d_body<OP, WIN_W, WIN_H, TRUNC, false, false, false>(a, none);
 		}
 
-		// Without expf the layers fit 96 registers per lane, which lets a compute unit hold five workgroups
-		// instead of four (measured: 10 % faster); with expf that would spill.
-		template<int OP, int WIN_W, int WIN_H, bool TRUNC>
+		// UNIFORM: one plane per workgroup (a.planes == 1). Without expf the layers fit 96 registers per lane,
+		// which lets a compute unit hold five workgroups instead of four (measured: 10 % faster); with expf
+		// that would spill.
+		template<int OP, int WIN_W, int WIN_H, bool TRUNC, bool UNIFORM>
 		__global__ void __launch_bounds__(max_block_size) __attribute__((amdgpu_waves_per_eu(5, 5))) max_window2d_prologue_kernel(const window2d_args a, const window_prologue pro)
 		{
-			window2d_body<OP, WIN_W, WIN_H, TRUNC, true, false>(a, pro);
+			window2d_body<OP, WIN_W, WIN_H, TRUNC, true, false, UNIFORM>(a, pro);
 		}
 
-		template<int OP, int WIN_W, int WIN_H, bool TRUNC>
+		template<int OP, int WIN_W, int WIN_H, bool TRUNC, bool UNIFORM>
 		__global__ void __launch_bounds__(max_block_size) max_window2d_exp_prologue_kernel(const window2d_args a, const window_prologue pro)
 		{
-			window2d_body<OP, WIN_W, WIN_H, TRUNC, true, true>(a, pro);
+			window2d_body<OP, WIN_W, WIN_H, TRUNC, true, true, UNIFORM>(a, pro);
 		}
 
 		// ---- any window the layer allows: one lane per output, values read from memory ------------
@@ -582,25 +677,34 @@ namespace nnf
 			return (divisor >= 2) ? static_cast<uint32_t>(((1ull << 32) + divisor - 1) / divisor) : 0u; // fast_divide does not use it for 1
 		}
 
+		template<int OP, bool TRUNC, bool UNIFORM>
+		void launch_window2d_prologue(hipStream_t stream, const window2d_args& a, uint32_t grid, size_t lds_bytes, const window_prologue& pro)
+		{
+			const dim3 g(grid), b(max_block_size);
+			const bool w3 = (a.win_w == 3) && (a.win_h == 3), w2 = (a.win_w == 2) && (a.win_h == 2);
+			if (pro.need_exp)
+			{
+				if (w3) hipLaunchKernelGGL((max_window2d_exp_prologue_kernel<OP, 3, 3, TRUNC, UNIFORM>), g, b, lds_bytes, stream, a, pro);
+				else if (w2) hipLaunchKernelGGL((max_window2d_exp_prologue_kernel<OP, 2, 2, TRUNC, UNIFORM>), g, b, lds_bytes, stream, a, pro);
+				else hipLaunchKernelGGL((max_window2d_exp_prologue_kernel<OP, 0, 0, TRUNC, UNIFORM>), g, b, lds_bytes, stream, a, pro);
+			}
+			else
+			{
+				if (w3) hipLaunchKernelGGL((max_window2d_prologue_kernel<OP, 3, 3, TRUNC, UNIFORM>), g, b, lds_bytes, stream, a, pro);
+				else if (w2) hipLaunchKernelGGL((max_window2d_prologue_kernel<OP, 2, 2, TRUNC, UNIFORM>), g, b, lds_bytes, stream, a, pro);
+				else hipLaunchKernelGGL((max_window2d_prologue_kernel<OP, 0, 0, TRUNC, UNIFORM>), g, b, lds_bytes, stream, a, pro);
+			}
+		}
+
 		template<int OP, bool TRUNC>
 		void launch_window2d(hipStream_t stream, const window2d_args& a, uint32_t grid, size_t lds_bytes, const window_prologue* pro)
 		{
 			if (pro != nullptr)
 			{
-				const dim3 g(grid), b(max_block_size);
-				const bool w3 = (a.win_w == 3) && (a.win_h == 3), w2 = (a.win_w == 2) && (a.win_h == 2);
-				if (pro->need_exp)
-				{
-					if (w3) hipLaunchKernelGGL((max_window2d_exp_prologue_kernel<OP, 3, 3, TRUNC>), g, b, lds_bytes, stream, a, *pro);
-					else if (w2) hipLaunchKernelGGL((max_window2d_exp_prologue_kernel<OP, 2, 2, TRUNC>), g, b, lds_bytes, stream, a, *pro);
-					else hipLaunchKernelGGL((max_window2d_exp_prologue_kernel<OP, 0, 0, TRUNC>), g, b, lds_bytes, stream, a, *pro);
-				}
+				if (a.planes == 1)
+					launch_window2d_prologue<OP, TRUNC, true>(stream, a, grid, lds_bytes, *pro);
 				else
-				{
-					if (w3) hipLaunchKernelGGL((max_window2d_prologue_kernel<OP, 3, 3, TRUNC>), g, b, lds_bytes, stream, a, *pro);
-					else if (w2) hipLaunchKernelGGL((max_window2d_prologue_kernel<OP, 2, 2, TRUNC>), g, b, lds_bytes, stream, a, *pro);
-					else hipLaunchKernelGGL((max_window2d_prologue_kernel<OP, 0, 0, TRUNC>), g, b, lds_bytes, stream, a, *pro);
-				}
+					launch_window2d_prologue<OP, TRUNC, false>(stream, a, grid, lds_bytes, *pro);
 				return;
 			}
 			if ((a.win_w == 3) && (a.win_h == 3))
