@@ -310,6 +310,82 @@ def test_fused_equals_unfused_bitwise(gpu):
     check_exact(fused, want, "fused group")
 
 
+def random_layer(gen, c, chunks, allow_exp=True):
+    """-> (op tuple, oracle step) of one random element-wise layer; weights are appended to chunks"""
+    kinds = [BN, RELU, PRELU, capi.OP_ABSOLUTE, capi.OP_DROPOUT] + ([ELU, SIGMOID, TANH] if allow_exp else [])
+    kind = kinds[int(gen.integers(0, len(kinds)))]
+    if kind == BN:
+        g, b, m, s = T.bn_params(gen, c)
+        first = len(chunks)
+        chunks.extend([g, b, m, s])
+        return (BN, first), lambda v: oracle.batch_norm(v, g, b, m, s)
+    if kind == RELU:
+        slope = float(gen.choice(np.array([0.0, 0.1, -0.5, 1.0], np.float32)))
+        return (RELU, 0, slope), lambda v: oracle.rectified_linear(v, slope)
+    if kind == PRELU:
+        a = T.uniform(gen, c, -0.5, 0.5)
+        first = len(chunks)
+        chunks.append(a)
+        return (PRELU, first), lambda v: oracle.parametric_rectified_linear(v, a)
+    if kind == capi.OP_ABSOLUTE:
+        return (capi.OP_ABSOLUTE,), oracle.absolute
+    if kind == capi.OP_DROPOUT:
+        return (capi.OP_DROPOUT,), oracle.dropout
+    if kind == ELU:
+        return (ELU,), oracle.exponential_linear
+    if kind == SIGMOID:
+        return (SIGMOID,), oracle.sigmoid
+    scale, steepness = float(gen.uniform(0.5, 2.0)), float(gen.uniform(0.2, 1.5))
+    return (TANH, 0, scale, steepness), lambda v: oracle.hyperbolic_tangent(v, scale, steepness)
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_groups_equal_the_layers_one_by_one(gpu, seed):
+    """Groups drawn at random - 1 to 4 inputs, any split of up to 8 layers over the arms and the tail, any layer
+    kinds, shapes with odd planes and element counts - against the oracle run layer by layer, bit for bit."""
+    gen = T.rng(13, seed)
+    n = int(gen.integers(1, 6))
+    c = int(gen.choice([1, 3, 8, 17, 64, 130]))
+    plane = int(gen.choice([1, 2, 7, 49, 196, 225, 784, 1000, 3136]))
+    input_count = int(gen.choice([1, 1, 2, 2, 3, 4]))
+    has_add = (input_count > 1) or bool(gen.integers(0, 2))
+    budget = capi.MAX_OPS
+    chunks, arms, arm_steps = [], [], []
+    for _ in range(input_count):
+        count = int(gen.integers(0, min(3, budget) + 1))
+        budget -= count
+        ops, steps = [], []
+        for _ in range(count):
+            op, step = random_layer(gen, c, chunks)
+            ops.append(op)
+            steps.append(step)
+        arms.append(ops)
+        arm_steps.append(steps)
+    tail, tail_steps = [], []
+    if has_add:
+        for _ in range(int(gen.integers(0, min(3, budget) + 1))):
+            op, step = random_layer(gen, c, chunks)
+            tail.append(op)
+            tail_steps.append(step)
+    elif not arms[0]:
+        op, step = random_layer(gen, c, chunks)
+        arms[0].append(op)
+        arm_steps[0].append(step)
+    alpha = float(gen.choice(np.array([1.0, 0.5, -1.25], np.float32)))
+    inputs = [awkward_input((n, c, plane), 100 * seed + j) if j == 0 else T.normal(gen, (n, c, plane), 2.0) for j in range(input_count)]
+    values = []
+    for x, steps in zip(inputs, arm_steps):
+        v = x
+        for step in steps:
+            v = step(v)
+        values.append(v)
+    want = oracle.add(values, alpha).reshape(inputs[0].shape) if has_add else values[0]
+    for step in tail_steps:
+        want = step(want)
+    got = gpu.chain((n, c, plane), arms, tail, inputs, chunks, has_add=has_add, alpha=alpha)
+    check_exact(got, want, "random group %d: %d inputs, arms %s, tail %s" % (seed, input_count, arms, tail))
+
+
 def test_in_place_group(gpu):
     n, c, plane = 2, 8, 49
     gen = T.rng(12, 0)
