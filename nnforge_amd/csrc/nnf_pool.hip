@@ -86,6 +86,19 @@ namespace nnf
 			}
 		}
 
+		// NNF_HIP_GLOBAL_POOL_PLANES overrides the planes per workgroup of the global pooling kernel (tuning); read once
+		uint32_t forced_planes_per_group()
+		{
+			static const uint32_t value = []() -> uint32_t
+			{
+				const char* text = std::getenv("NNF_HIP_GLOBAL_POOL_PLANES");
+				if ((text == nullptr) || (*text == '\0'))
+					return 0u;
+				return std::min(global_pool_planes, std::max(4u, static_cast<uint32_t>(std::atoi(text)) & ~3u));
+			}();
+			return value;
+		}
+
 		// General case: one lane per output neuron, window read straight from memory.
 		__global__ void __launch_bounds__(pool_block_size) window_pool_kernel(
 			float* out, const float* in, uint32_t output_count,
@@ -174,8 +187,8 @@ namespace nnf
 		{
 			// 64 planes of 7x7; fewer of larger planes, so that a compute unit holds several workgroups
 			uint32_t planes_per_group = std::min(global_pool_planes, std::max(8u, (global_pool_lds_floats / plane) & ~3u));
-			if (const char* text = std::getenv("NNF_HIP_GLOBAL_POOL_PLANES"))
-				planes_per_group = std::min(global_pool_planes, std::max(4u, static_cast<uint32_t>(std::atoi(text)) & ~3u));
+			if (forced_planes_per_group() != 0)
+				planes_per_group = forced_planes_per_group();
 			const size_t lds_bytes = static_cast<size_t>(planes_per_group) * (plane | 1u) * sizeof(float);
 			const dim3 grid((plane_count + planes_per_group - 1) / planes_per_group);
 			// plane >= 2 here: a 1x1 window over a 1x1 plane takes the general kernel
