@@ -498,7 +498,7 @@ def main():
                 per_config[name] = run(name, *side_steps[name])
         per_config["copy_kernel"] = bench_copy(runner, 40, 5)
         # the neighbouring layers of the same chains
-        for name, (k, wu) in (("max_subsampling", (40, 5)), ("concat", (100, 10)), ("maxout", (100, 10)), ("feature_map_stat", (20, 3))):
+        for name, (k, wu) in (("max_subsampling", (40, 5)), ("bn_relu_max_subsampling", (40, 5)), ("concat", (100, 10)), ("maxout", (100, 10)), ("feature_map_stat", (20, 3))):
             if name not in per_config:
                 per_config[name] = run(name, k, wu)
         if args.workload == "config0":
