@@ -162,6 +162,7 @@ namespace nnf
 
 		__device__ __forceinline__ void uniform_coefficients(float (&own)[prologue_weighted_max][2], uniform_weights r, const window_prologue& pro)
 		{
+			// the weights are not looked at (nor waited for) before this point
 			#pragma unroll
 			for(uint32_t j = 0; j < prologue_weighted_max; ++j)
 			{
