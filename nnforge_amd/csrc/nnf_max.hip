@@ -506,16 +506,42 @@ namespace nnf
 			const uint32_t outputs_per_plane = rows_here * a.out_w;
 			const uint32_t outputs_here = planes_here * outputs_per_plane;
 			float* dst = a.out + (first_plane * a.out_h + first_row) * a.out_w;
-			for(uint32_t o = threadIdx.x; o < outputs_here; o += max_block_size)
+
+			// A lane takes outputs tid, tid + 256, ... of the workgroup's run. Where its window starts - column
+			// x0 and row y0 of the plane, float index win of the staged copy - is worked out once with
+			// divisions and then carried from one output to the next with additions: 256 outputs further is
+			// step_p planes, step_y rows and step_x columns further, with a carry from columns into rows
+			// and from rows into planes (integer multiplications run at a quarter of the rate of additions
+			// here, and the scan, not the memory, was what bounded this kernel).
+			const uint32_t step_p = max_block_size / outputs_per_plane;
+			const uint32_t step_rest = max_block_size - step_p * outputs_per_plane;
+			const uint32_t step_y = step_rest / a.out_w;
+			const uint32_t step_x = step_rest - step_y * a.out_w;
+			const uint32_t row_floats = a.stride_y * a.in_w;        // one output row further
+			const uint32_t x_limit = a.out_w * a.stride_x;          // x0 of the column behind the last one
+			const uint32_t y_limit = (first_row + rows_here) * a.stride_y;
+			const uint32_t x_advance = step_x * a.stride_x;
+			const uint32_t y_advance = step_y * a.stride_y;
+			const uint32_t win_advance = step_p * in_plane + step_y * row_floats + x_advance;
+			const uint32_t x_carry_win = row_floats - x_limit;                 // back to column 0, one row down
+			const uint32_t y_carry_y = rows_here * a.stride_y;
+			const uint32_t y_carry_win = in_plane - rows_here * row_floats;    // back to row 0, one plane on
+
+			uint32_t x0, y0, win;
 			{
 				// rows_here differs from a.rows only in the last band, where planes_here == 1 and p is 0 anyway
+				const uint32_t o = threadIdx.x;
 				const uint32_t p = (planes_here > 1) ? fast_divide(o, outputs_per_plane, a.band_magic) : 0u;
 				const uint32_t r = o - p * outputs_per_plane;
 				const uint32_t oy = fast_divide(r, a.out_w, a.out_w_magic);
 				const uint32_t ox = r - oy * a.out_w;
-				const uint32_t x0 = ox * a.stride_x;
-				const uint32_t y0 = (first_row + oy) * a.stride_y;
-				const float* src = lds_in + shift + p * in_plane + (y0 - in_row0) * a.in_w + x0;
+				x0 = ox * a.stride_x;
+				y0 = (first_row + oy) * a.stride_y;
+				win = shift + p * in_plane + (y0 - in_row0) * a.in_w + x0;
+			}
+			for(uint32_t o = threadIdx.x; o < outputs_here; o += max_block_size)
+			{
+				const float* src = lds_in + win;
 				// A window position beyond the input reads the last position inside instead. That value
 				// has been folded before (it precedes in scan order) and folding a value twice changes
 				// nothing, so this equals skipping the position.
@@ -525,24 +551,50 @@ namespace nnf
 				float current = window_fold_start<OP>();
 				if ((WIN_W > 0) && (WIN_H > 0))
 				{
+					// min(y, last_y) * in_w and min(x, last_x) without multiplications
+					uint32_t row_offset[WIN_H > 0 ? WIN_H : 1], column_offset[WIN_W > 0 ? WIN_W : 1];
+					row_offset[0] = 0;
+					#pragma unroll
+					for(int y = 1; y < WIN_H; ++y)
+						row_offset[y] = TRUNC ? row_offset[y - 1] + ((static_cast<uint32_t>(y) <= last_y) ? a.in_w : 0u) : static_cast<uint32_t>(y) * a.in_w;
+					#pragma unroll
+					for(int x = 0; x < WIN_W; ++x)
+						column_offset[x] = TRUNC ? min(static_cast<uint32_t>(x), last_x) : static_cast<uint32_t>(x);
 					#pragma unroll
 					for(int y = 0; y < WIN_H; ++y)
 					{
-						const float* row = src + (TRUNC ? min(static_cast<uint32_t>(y), last_y) : static_cast<uint32_t>(y)) * a.in_w;
+						const float* row = src + row_offset[y];
 						#pragma unroll
 						for(int x = 0; x < WIN_W; ++x)
-							current = window_fold<OP>(current, row[TRUNC ? min(static_cast<uint32_t>(x), last_x) : static_cast<uint32_t>(x)]);
+							current = window_fold<OP>(current, row[column_offset[x]]);
 					}
 				}
 				else
 				{
 					const uint32_t fit_w = TRUNC ? last_x + 1 : win_w;
 					const uint32_t fit_h = TRUNC ? last_y + 1 : win_h;
-					for(uint32_t y = 0; y < fit_h; ++y)
+					const float* row = src;
+					for(uint32_t y = 0; y < fit_h; ++y, row += a.in_w)
 						for(uint32_t x = 0; x < fit_w; ++x)
-							current = window_fold<OP>(current, src[y * a.in_w + x]);
+							current = window_fold<OP>(current, row[x]);
 				}
 				dst[o] = (OP == window_op_sum) ? current * a.mult : current;
+
+				// 256 outputs further
+				x0 += x_advance;
+				y0 += y_advance;
+				win += win_advance;
+				if (x0 >= x_limit)
+				{
+					x0 -= x_limit;
+					y0 += a.stride_y;
+					win += x_carry_win;
+				}
+				if (y0 >= y_limit)
+				{
+					y0 -= y_carry_y;
+					win += y_carry_win;
+				}
 			}
 		}
 
