@@ -103,7 +103,8 @@ NNF_BACKEND_API int nnf_backend_plan_schema(
 	uint64_t memory_bytes,
 	char* report, size_t report_capacity);
 
-/* Parses a schema and writes it back in text format (round trip of the reader/writer). */
+/* Parses a schema and writes it back in text format (round trip of the reader/writer). A buffer too
+ * small for the whole text is an error (the message says how many bytes are needed). */
 NNF_BACKEND_API int nnf_backend_rewrite_schema(const char* schema_text, char* out_text, size_t out_capacity);
 
 /* Writes / reads <layer>.data files in nnForge's format (weights in, weights out through `weights`

@@ -85,6 +85,22 @@ def build_usage_program(verbose=False):
     return USAGE_PROGRAM
 
 
+SANITIZED_PROGRAM_SOURCE = os.path.join(REPO_ROOT, "tests", "cpp", "host_sanitized.cpp")
+
+
+def build_sanitized_host_program(output_path):
+    """Compiles the backend's host sources together with tests/cpp/host_sanitized.cpp under AddressSanitizer and
+    UndefinedBehaviorSanitizer (host code only: the program never touches a device). Used by the CPU tests."""
+    if not os.path.exists(HIP_LIBRARY):
+        raise RuntimeError("build the HIP library first: %s is missing" % HIP_LIBRARY)
+    cmd = ["g++", "-O1", "-g", "-std=c++17", "-fsanitize=address,undefined", "-fno-sanitize-recover=all", "-Wall",
+           "-I", os.path.join(REPO_ROOT, "include"), "-o", output_path, SANITIZED_PROGRAM_SOURCE]
+    cmd += [os.path.join(HOST_DIR, s) for s in BACKEND_SOURCES]
+    cmd += ["-L", PACKAGE_DIR, "-lnnforge_hip", "-Wl,-rpath," + PACKAGE_DIR]
+    _run(cmd)
+    return output_path
+
+
 def build_all(verbose=False):
     built = [build_hip_library(verbose), build_backend_library(verbose), build_usage_program(verbose)]
     return built

@@ -297,7 +297,12 @@ extern "C"
 		return guarded([&](std::ostream& out)
 		{
 			const network_schema schema = parse_schema(schema_text);
-			schema.write_proto(out);
+			std::ostringstream text;
+			schema.write_proto(text);
+			// the text is the result: cut short it would be a different schema
+			if (text.str().size() + 1 > out_capacity)
+				throw neural_network_exception("The schema text takes " + std::to_string(text.str().size() + 1) + " bytes, the buffer holds " + std::to_string(out_capacity));
+			out << text.str();
 		}, out_text, out_capacity);
 	}
 

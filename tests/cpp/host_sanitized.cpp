@@ -1,0 +1,133 @@
+// Host-side code of the backend (schema reader and writer, layer configuration rules, launch and
+// buffer planner, weight files) driven through the C bridge without a device. The tests build this
+// program together with the backend's sources under AddressSanitizer and UndefinedBehaviorSanitizer:
+// it feeds the reader well-formed and damaged text and must end with "ok" and no sanitizer report.
+#include <nnforge_hip_backend.h>
+
+#include <cstdio>
+#include <cstring>
+#include <string>
+#include <vector>
+
+namespace
+{
+	const char * good_schema = R"(
+name: "host_checks"
+layer { type: "Data" name: "conv1" }
+layer { type: "BatchNorm" name: "bn" input_layer_name: "conv1" batch_norm_param { feature_map_count: 8 } }
+layer { type: "ReLU" name: "relu" input_layer_name: "bn" relu_param { negative_slope: 0.1 } }
+layer { type: "MaxSubsampling" name: "pool1" input_layer_name: "relu"
+	max_subsampling_param { dimension_param { subsampling_size: 3 stride: 2 round_up: true } dimension_param { subsampling_size: 3 stride: 2 round_up: true } } }
+layer { type: "TanH" name: "tanh" input_layer_name: "pool1" tanh_param { scale: 1.7159 steepness: 0.6666 } }
+layer { type: "Absolute" name: "abs" input_layer_name: "tanh" }
+layer { type: "AverageSubsampling" name: "pool2" input_layer_name: "abs"
+	average_subsampling_param { dimension_param { subsampling_size: 2 } dimension_param { subsampling_size: 2 } } }
+layer { type: "PReLU" name: "prelu" input_layer_name: "pool2" prelu_param { feature_map_count: 8 } }
+layer { type: "Dropout" name: "drop" input_layer_name: "prelu" dropout_param { dropout_rate: 0.25 } }
+layer { type: "Add" name: "sum" input_layer_name: "drop" input_layer_name: "pool2" add_param { alpha: 0.5 } }
+layer { type: "Concat" name: "cat" input_layer_name: "sum" input_layer_name: "pool2" }
+layer { type: "Maxout" name: "mo" input_layer_name: "cat" maxout_param { feature_map_subsampling_size: 2 } }
+layer { type: "ELU" name: "elu" input_layer_name: "mo" }
+layer { type: "Sigmoid" name: "sig" input_layer_name: "elu" }
+layer { type: "Softmax" name: "prob" input_layer_name: "sig" }
+)";
+
+	int failures = 0;
+
+	void expect(bool condition, const std::string& what)
+	{
+		if (!condition)
+		{
+			std::printf("FAILED: %s\n", what.c_str());
+			++failures;
+		}
+	}
+
+	int plan(const std::string& text, uint32_t width, uint32_t height, std::string& report, int fuse = 1)
+	{
+		const uint32_t dims[2] = { width, height };
+		nnf_backend_input input = { "conv1", 8, 2, dims, nullptr };
+		const char * outputs[1] = { "prob" };
+		nnf_backend_options options;
+		std::memset(&options, 0, sizeof(options));
+		options.fuse = fuse;
+		std::vector<char> buffer(1 << 16);
+		const int rc = nnf_backend_plan_schema(text.c_str(), &input, 1, outputs, 1, &options, 1ull << 30, buffer.data(), buffer.size());
+		report = buffer.data();
+		return rc;
+	}
+}
+
+int main(int argc, char ** argv)
+{
+	const std::string folder = (argc > 1) ? argv[1] : ".";
+	const std::string good(good_schema);
+	std::string report;
+
+	// the whole schema plans, with and without fusion, at several input sizes
+	for(uint32_t size : { 28u, 57u, 112u })
+	{
+		expect(plan(good, size, size, report, 1) == 0, "plan with fusion: " + report);
+		expect(report.find("bn+relu+pool1") != std::string::npos, "the pooling layer takes the group in front of it along: " + report);
+		expect(plan(good, size, size, report, 0) == 0, "plan without fusion: " + report);
+	}
+	// sizes the layers reject
+	expect(plan(good, 2, 2, report) != 0, "an input smaller than the windows is refused");
+	expect(plan(good, 0, 5, report) != 0, "an empty dimension is refused");
+
+	// the text written back parses again to the same text
+	std::vector<char> once(1 << 16), twice(1 << 16);
+	expect(nnf_backend_rewrite_schema(good.c_str(), once.data(), once.size()) == 0, "rewrite");
+	expect(nnf_backend_rewrite_schema(once.data(), twice.data(), twice.size()) == 0, "rewrite of the rewritten text");
+	expect(std::strcmp(once.data(), twice.data()) == 0, "the writer's output is a fixed point of reader + writer");
+	// a buffer that is too small is reported, not overrun
+	std::vector<char> tiny(16);
+	expect(nnf_backend_rewrite_schema(good.c_str(), tiny.data(), tiny.size()) != 0, "a short output buffer is an error");
+
+	// damaged text: every prefix of the schema, single characters replaced, blocks doubled
+	int accepted = 0, refused = 0;
+	for(size_t cut = 0; cut < good.size(); cut += 7)
+		(plan(good.substr(0, cut), 28, 28, report) == 0) ? ++accepted : ++refused;
+	const char replacements[] = { '{', '}', '"', ':', '-', '9', 'x', '\0', '#', '\n' };
+	for(size_t at = 3; at < good.size(); at += 11)
+	{
+		for(char c : replacements)
+		{
+			std::string damaged = good;
+			damaged[at] = c;
+			(plan(damaged, 28, 28, report) == 0) ? ++accepted : ++refused;
+		}
+	}
+	for(size_t at = 0; at + 40 < good.size(); at += 97)
+	{
+		std::string doubled = good;
+		doubled.insert(at, good.substr(at, 40));
+		(plan(doubled, 28, 28, report) == 0) ? ++accepted : ++refused;
+	}
+	expect(refused > accepted, "most damaged texts are refused (" + std::to_string(refused) + " refused, " + std::to_string(accepted) + " still well-formed)");
+
+	// weight files: written, read back, read with wrong expectations
+	{
+		const std::vector<float> gamma = { 1.0f, 2.0f, 3.0f }, slopes = { 0.25f };
+		const uint32_t bn_sizes[4] = { 3, 3, 3, 3 };
+		const float * bn_chunks[4] = { gamma.data(), gamma.data(), gamma.data(), gamma.data() };
+		const uint32_t prelu_sizes[1] = { 1 };
+		const float * prelu_chunks[1] = { slopes.data() };
+		nnf_backend_weights weights[2] = { { "bn", 4, bn_sizes, bn_chunks }, { "prelu", 1, prelu_sizes, prelu_chunks } };
+		std::vector<char> buffer(4096);
+		expect(nnf_backend_write_weights(folder.c_str(), weights, 2, buffer.data(), buffer.size()) == 0, std::string("write weights: ") + buffer.data());
+		std::vector<float> back(12, -1.0f);
+		float * back_chunks[4] = { back.data(), back.data() + 3, back.data() + 6, back.data() + 9 };
+		expect(nnf_backend_read_weights(folder.c_str(), "bn", 4, bn_sizes, back_chunks, buffer.data(), buffer.size()) == 0, std::string("read weights: ") + buffer.data());
+		expect((back[0] == 1.0f) && (back[5] == 3.0f) && (back[11] == 3.0f), "the weights read are the weights written");
+		const uint32_t wrong_sizes[4] = { 3, 3, 2, 3 };
+		expect(nnf_backend_read_weights(folder.c_str(), "bn", 4, wrong_sizes, back_chunks, buffer.data(), buffer.size()) != 0, "a chunk of another size is refused");
+		expect(nnf_backend_read_weights(folder.c_str(), "bn", 3, bn_sizes, back_chunks, buffer.data(), buffer.size()) != 0, "another chunk count is refused");
+		expect(nnf_backend_read_weights(folder.c_str(), "missing", 1, prelu_sizes, back_chunks, buffer.data(), buffer.size()) != 0, "a layer without a file is refused");
+		expect(nnf_backend_read_weights((folder + "/nowhere").c_str(), "bn", 4, bn_sizes, back_chunks, buffer.data(), buffer.size()) != 0, "a missing folder is refused");
+	}
+
+	if (failures == 0)
+		std::printf("ok\n");
+	return failures == 0 ? 0 : 1;
+}

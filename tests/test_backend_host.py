@@ -282,3 +282,24 @@ def test_neighbour_layer_configuration_rules():
         plan([S.L("Data", "x"), S.L("Data", "y"), S.L("Concat", "c", ["x", "y"])], {"x": (4, [8]), "y": (4, [9])}, ["c"])
     with pytest.raises(backend.BackendError, match="dropout_rate"):
         plan([S.L("Data", "x"), S.L("Dropout", "d", ["x"], dropout_rate=1.0)], {"x": (4, [8])}, ["d"])
+
+
+def test_host_code_under_address_and_undefined_behaviour_sanitizers(tmp_path):
+    """Schema reader and writer, configuration rules, planner and weight files, built with -fsanitize=address,undefined
+    and fed the full schema, about a thousand damaged variants of it and wrong weight-file expectations
+    (tests/cpp/host_sanitized.cpp): no report from either sanitizer, every expectation of the program met."""
+    import subprocess
+
+    from nnforge_amd import build
+
+    program = build.build_sanitized_host_program(str(tmp_path / "host_sanitized"))
+    env = dict(os.environ)
+    # the HIP runtime the kernel library links keeps process-lifetime allocations: leaks are not what is looked for here
+    env["ASAN_OPTIONS"] = "detect_leaks=0"
+    weights_folder = tmp_path / "weights"
+    weights_folder.mkdir()
+    proc = subprocess.run([program, str(weights_folder)], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, env=env, timeout=300)
+    assert proc.returncode == 0, proc.stdout[-4000:]
+    assert proc.stdout.strip().endswith("ok"), proc.stdout[-4000:]
+    assert "runtime error" not in proc.stdout and "AddressSanitizer" not in proc.stdout
+
