@@ -146,3 +146,68 @@ def inception_like(c=8):
         L("MaxSubsampling", "pool2", ["drop"], windows=[2, 2], function="MIN"),
         L("TanH", "out", ["pool2"]),
     ]
+
+
+def random_network(gen, layer_count=14, c=6, size=12):
+    """A random DAG of the layer types the backend runs: chains of element-wise layers, Adds and Concats of values of
+    equal shape, Maxout, max / min / average pooling, with some values consumed more than once.
+    -> (layers, {value name: (feature maps, [w, h])}, output names)."""
+    layers = [L("Data", "in0"), L("Data", "in1")]
+    shapes = {"in0": (c, [size, size]), "in1": (c, [size, size])}
+    names = ["in0", "in1"]
+    unary = ["BatchNorm", "ReLU", "PReLU", "ELU", "Sigmoid", "TanH", "Absolute", "Dropout"]
+    for i in range(layer_count):
+        name = "l%d" % i
+        # mostly continue from the newest value (chains), sometimes branch off an older one
+        src = names[-1] if gen.random() < 0.65 else names[int(gen.integers(0, len(names)))]
+        fm, dims = shapes[src]
+        roll = gen.random()
+        same_shape = [n for n in names if shapes[n] == shapes[src] and n != src]
+        same_plane = [n for n in names if shapes[n][1] == dims and n != src]
+        if roll < 0.50:
+            t = unary[int(gen.integers(0, len(unary)))]
+            params = {}
+            if t in ("BatchNorm", "PReLU"):
+                params["feature_map_count"] = fm
+            elif t == "ReLU" and gen.random() < 0.5:
+                params["negative_slope"] = 0.125
+            elif t == "TanH":
+                params = {"scale": 1.7159, "steepness": 0.6666}
+            elif t == "Dropout":
+                params = {"dropout_rate": 0.25}
+            layers.append(L(t, name, [src], **params))
+            shapes[name] = (fm, dims)
+        elif roll < 0.65 and same_shape:
+            others = [same_shape[int(j)] for j in gen.permutation(len(same_shape))[:int(gen.integers(1, 3))]]
+            params = {"alpha": 0.5} if gen.random() < 0.3 else {}
+            layers.append(L("Add", name, [src] + others, **params))
+            shapes[name] = (fm, dims)
+        elif roll < 0.75 and same_plane:
+            others = [same_plane[int(j)] for j in gen.permutation(len(same_plane))[:int(gen.integers(1, 3))]]
+            layers.append(L("Concat", name, [src] + others))
+            shapes[name] = (fm + sum(shapes[o][0] for o in others), dims)
+        elif roll < 0.82 and fm % 2 == 0 and fm >= 4:
+            layers.append(L("Maxout", name, [src], feature_map_subsampling_size=2))
+            shapes[name] = (fm // 2, dims)
+        elif roll < 0.92 and min(dims) >= 6:
+            if gen.random() < 0.5:
+                layers.append(L("MaxSubsampling", name, [src], windows=[3, 3], strides=[2, 2], round_ups=[True, True],
+                                **({"function": "MIN"} if gen.random() < 0.3 else {})))
+                shapes[name] = (fm, [(d + 2 - 3 + 2) // 2 for d in dims])
+            else:
+                layers.append(L("MaxSubsampling", name, [src], windows=[2, 2]))
+                shapes[name] = (fm, [d // 2 for d in dims])
+        elif min(dims) >= 4:
+            layers.append(L("AverageSubsampling", name, [src], windows=[2, 2]))
+            shapes[name] = (fm, [d // 2 for d in dims])
+        else:
+            layers.append(L("Absolute", name, [src]))
+            shapes[name] = (fm, dims)
+        names.append(name)
+    consumed = {i for l in layers for i in l["inputs"]}
+    outputs = [n for n in names[2:] if n not in consumed]          # every value nobody reads
+    extra = [n for n in names[2:] if n in consumed]
+    if extra:
+        outputs.append(extra[int(gen.integers(0, len(extra)))])    # and one that is read as well
+    return layers, shapes, outputs
+

@@ -284,6 +284,37 @@ def test_neighbour_layer_configuration_rules():
         plan([S.L("Data", "x"), S.L("Dropout", "d", ["x"], dropout_rate=1.0)], {"x": (4, [8])}, ["d"])
 
 
+@pytest.mark.parametrize("seed", range(30))
+def test_plan_of_random_networks_keeps_every_layer_once_and_in_order(seed):
+    gen = T.rng(70, seed)
+    layers, shapes, outputs = S.random_network(gen)
+    configs = {"in0": shapes["in0"], "in1": shapes["in1"]}
+    executed = [l["name"] for l in layers if l["type"] != "Data"]
+    needed = set()      # layers the outputs depend on (the planner drops the rest)
+    by_name = {l["name"]: l for l in layers}
+    todo = list(outputs)
+    while todo:
+        n = todo.pop()
+        if n in needed:
+            continue
+        needed.add(n)
+        todo.extend(by_name[n]["inputs"])
+    for fuse in (True, False):
+        rep = plan(layers, configs, outputs, fuse=fuse)
+        seen = [n for s in rep["steps"] for n in s["layers"]]
+        assert sorted(seen) == sorted(n for n in executed if n in needed), "every needed layer exactly once"
+        produced = {"in0", "in1"}
+        for s in rep["steps"]:
+            assert all(i in produced for i in s["inputs"]), "a step reads only what earlier steps wrote: %s" % s
+            produced.add(s["layers"][-1])
+            # inside a step only the last layer's value exists afterwards: nobody outside may read the others
+            for inner in s["layers"][:-1]:
+                readers = [l["name"] for l in layers if inner in l["inputs"] and l["name"] in needed]
+                assert all(r in s["layers"] for r in readers) and inner not in outputs
+        if not fuse:
+            assert all(len(s["layers"]) == 1 for s in rep["steps"])
+
+
 def test_host_code_under_address_and_undefined_behaviour_sanitizers(tmp_path):
     """Schema reader and writer, configuration rules, planner and weight files, built with -fsanitize=address,undefined
     and fed the full schema, about a thousand damaged variants of it and wrong weight-file expectations

@@ -212,6 +212,26 @@ def test_groups_folded_into_the_subsampling_layers_behind_them(fuse, size):
         assert len(names) == 8
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_random_networks_equal_the_oracle_layer_by_layer(seed):
+    """Random DAGs of every layer type the backend runs (the generator of the planner tests), in packets, with
+    fusion and buffer sharing on: every output equals the oracle run layer by layer, bit for bit; the same
+    network without fusion and with dedicated buffers gives the same bits."""
+    gen = T.rng(70, seed)
+    layers, shapes, outputs = S.random_network(gen)
+    weights = S.make_weights(layers, gen)
+    n = 7
+    inputs = {k: T.normal(gen, (n, shapes[k][0]) + tuple(shapes[k][1][::-1]), 1.5) for k in ("in0", "in1")}
+    values = S.evaluate(layers, weights, inputs)
+    got, rep = run(layers, weights, inputs, outputs, values, fuse=True, max_entry_count=3)
+    assert rep["entries"] == n
+    for name in outputs:
+        assert_bits(got[name], values[name], "seed %d, output %s, steps %s" % (seed, name, ["+".join(s["layers"]) for s in rep["steps"]]))
+    plain, _ = run(layers, weights, inputs, outputs, values, fuse=False, dont_share_buffers=True)
+    for name in outputs:
+        assert_bits(plain[name], values[name], "seed %d unfused, output %s" % (seed, name))
+
+
 def test_dropout_only_network():
     """Dropout straight from the data layer to the output: in place there is nothing to launch."""
     gen = T.rng(58, 0)
