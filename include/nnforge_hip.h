@@ -184,11 +184,11 @@ NNF_HIP_API int nnf_hip_max_subsampling_forward(void* stream, float* output, con
  * nnforge/plain/forward_propagation_plain.cpp:137-186 would store between the two testers - is never
  * written to memory; the output carries the same bits as the layers run one after another. Other
  * arguments as for nnf_hip_max_subsampling_forward / nnf_hip_average_subsampling_forward. Only the
- * LDS-staged window kernel applies a prologue: NNF_HIP_EUNSUPPORTED (nothing launched) for windows
- * over feature maps or entries, more than two spatial dimensions, whole-plane average windows, planes
- * of fewer than four floats, more than 65535 outputs per plane, and groups with more than two layers
- * that carry weights (batch norm, PReLU). The *_fusable
- * functions answer that from the shapes alone (NNF_HIP_OK / NNF_HIP_EUNSUPPORTED; no device needed). */
+ * LDS-staged kernels (2-D windows, whole-plane averages) apply a prologue: NNF_HIP_EUNSUPPORTED
+ * (nothing launched) for windows over feature maps or entries, more than two spatial dimensions,
+ * planes of fewer than four floats, more than 65535 outputs per plane, and groups with more than two
+ * layers that carry weights (batch norm, PReLU). The *_fusable functions answer that from the shapes
+ * alone (NNF_HIP_OK / NNF_HIP_EUNSUPPORTED; no device needed). */
 NNF_HIP_API int nnf_hip_max_subsampling_fused_forward(void* stream, float* output, const float* input,
 	const nnf_hip_chain_desc* prologue, const float* const* chunk_ptrs,
 	uint32_t output_entry_count, uint32_t input_feature_map_count, uint32_t dimension_count,

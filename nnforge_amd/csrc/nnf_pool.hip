@@ -5,6 +5,7 @@
 // plane go through the LDS-staged 2-D window kernel shared with max subsampling (nnf_max.hip);
 // the one-lane-per-output kernel below remains for the shapes that kernel declines.
 #include "nnf_common.h"
+#include "nnf_prologue.h"
 
 #include <algorithm>
 #include <cstdlib>
@@ -86,6 +87,126 @@ namespace nnf
 			}
 		}
 
+		// The same with the element-wise layers in front of the subsampling layer applied to the values between
+		// the load and the LDS store. Lane p works out the coefficients of plane p of the workgroup (at most
+		// 64 planes) into an LDS table. A float4 may hold the end of one plane and the start of the next
+		// (planes of 49 floats): then it goes through the layers twice, once with each plane's
+		// coefficients, and every float keeps the result that is its own.
+		template<bool EXP>
+		__global__ void __launch_bounds__(pool_block_size) global_pool_prologue_kernel(float* out, const float* in, uint32_t plane_count, uint32_t plane,
+			uint32_t plane_magic, float mult, uint32_t planes_per_group, const window_prologue pro)
+		{
+			extern __shared__ __align__(16) float lds_planes[];
+			__shared__ uint64_t lds_exp[EXP ? exp_lds_entries : 1];
+			__shared__ float lds_coef[global_pool_planes * 2 * prologue_weighted_max];
+			exp_context exp_ctx = make_exp_context(lds_exp);
+			const float none[prologue_weighted_max][2] = {};
+
+			const uint32_t stride = plane | 1u;
+			const uint32_t first_plane = blockIdx.x * planes_per_group;
+			const uint32_t planes_here = min(planes_per_group, plane_count - first_plane);
+			const uint32_t floats_here = planes_here * plane;
+			const float* src = in + static_cast<size_t>(first_plane) * plane;
+			const uint32_t coef_stride = 2 * pro.weighted_count;
+
+			const prologue_weights weights = load_prologue_weights(first_plane % pro.fm_count, planes_here, pro);
+			const uint32_t vectors = floats_here / 4;
+			constexpr int stage = 4; // a workgroup stages about 4096 floats: one round
+			for(uint32_t base = 0; base < vectors; base += stage * pool_block_size)
+			{
+				floatx4 t[stage];
+				#pragma unroll
+				for(int k = 0; k < stage; ++k)
+				{
+					const uint32_t i = base + k * pool_block_size + threadIdx.x;
+					t[k] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+					if (i < vectors)
+						t[k] = load_stream(reinterpret_cast<const floatx4*>(src) + i);
+				}
+				if (base == 0)
+				{
+					stage_prologue_coefficients(lds_coef, weights, planes_here, pro);
+					if (EXP)
+						stage_exp2_table(lds_exp);
+					__syncthreads();
+					if (EXP)
+						exp_ctx = exp_context_from_lds(lds_exp);
+				}
+				float v[stage][4];
+				uint32_t first_plane_of[stage], off[stage];
+				bool straddles = false;
+				#pragma unroll
+				for(int k = 0; k < stage; ++k)
+				{
+					const uint32_t i = min(base + k * pool_block_size + threadIdx.x, vectors - 1);
+					v[k][0] = t[k].x; v[k][1] = t[k].y; v[k][2] = t[k].z; v[k][3] = t[k].w;
+					// floats_here * plane < 2^32: the multiplication by ceil(2^32 / plane) divides exactly
+					first_plane_of[k] = __umulhi(i * 4, plane_magic);
+					off[k] = first_plane_of[k] * coef_stride;
+					straddles = straddles || (i * 4 + 3 >= (first_plane_of[k] + 1) * plane);
+				}
+				apply_prologue<stage, EXP, false>(v, off, lds_coef, none, pro, exp_ctx);
+				if (__any(straddles))
+				{
+					// one float4 at a time: the copies that go through the layers a second time stay few
+					#pragma unroll
+					for(int k = 0; k < stage; ++k)
+					{
+						const uint32_t i = min(base + k * pool_block_size + threadIdx.x, vectors - 1);
+						float w[1][4] = { { t[k].x, t[k].y, t[k].z, t[k].w } };
+						const uint32_t next_off[1] = { min(first_plane_of[k] + 1, planes_here - 1) * coef_stride }; // beyond the last plane: not stored
+						apply_prologue<1, EXP, false>(w, next_off, lds_coef, none, pro, exp_ctx);
+						#pragma unroll
+						for(uint32_t e = 1; e < 4; ++e)
+						{
+							if (i * 4 + e >= (first_plane_of[k] + 1) * plane)
+								v[k][e] = w[0][e];
+						}
+					}
+				}
+				#pragma unroll
+				for(int k = 0; k < stage; ++k)
+				{
+					const uint32_t i = base + k * pool_block_size + threadIdx.x;
+					if (i < vectors)
+					{
+						uint32_t p = first_plane_of[k];
+						uint32_t r = i * 4 - p * plane;
+						#pragma unroll
+						for(int e = 0; e < 4; ++e)
+						{
+							lds_planes[p * stride + r] = v[k][e];
+							if (++r == plane)
+							{
+								r = 0;
+								++p;
+							}
+						}
+					}
+				}
+			}
+			// the up to three floats behind the last whole float4 (last workgroup of a plane count that is no multiple of 4)
+			for(uint32_t f = vectors * 4 + threadIdx.x; f < floats_here; f += pool_block_size)
+			{
+				const uint32_t p = f / plane;
+				float one[1][4] = { { src[f], 0.0f, 0.0f, 0.0f } };
+				const uint32_t one_off[1] = { p * coef_stride };
+				apply_prologue<1, EXP, false>(one, one_off, lds_coef, none, pro, exp_ctx);
+				lds_planes[p * stride + (f - p * plane)] = one[0][0];
+			}
+			__syncthreads();
+
+			if (threadIdx.x < planes_here)
+			{
+				const float* my_plane = lds_planes + threadIdx.x * stride;
+				float sum = 0.0f;
+				#pragma unroll 8
+				for(uint32_t i = 0; i < plane; ++i)
+					sum += my_plane[i];
+				out[first_plane + threadIdx.x] = sum * mult;
+			}
+		}
+
 		// NNF_HIP_GLOBAL_POOL_PLANES overrides the planes per workgroup of the global pooling kernel (tuning); read once
 		uint32_t forced_planes_per_group()
 		{
@@ -97,6 +218,14 @@ namespace nnf
 				return std::min(global_pool_planes, std::max(4u, static_cast<uint32_t>(std::atoi(text)) & ~3u));
 			}();
 			return value;
+		}
+
+		// 64 planes of 7x7; fewer of larger planes, so that a compute unit holds several workgroups
+		uint32_t global_pool_planes_per_group(uint32_t plane)
+		{
+			if (forced_planes_per_group() != 0)
+				return forced_planes_per_group();
+			return std::min(global_pool_planes, std::max(8u, (global_pool_lds_floats / plane) & ~3u));
 		}
 
 		// General case: one lane per output neuron, window read straight from memory.
@@ -175,7 +304,27 @@ namespace nnf
 		if (prologue != nullptr)
 		{
 			const bool whole_plane = (window_width == input_width) && (window_height == input_height) && (plane >= 2) && (plane <= global_pool_max_plane);
-			if (whole_plane || !window2d_launch_with_prologue(stream, 4, mult, output, input, static_cast<uint32_t>(input_total), plane_count,
+			if (whole_plane)
+			{
+				// a float4 may straddle two planes, not three
+				if (plane < 4)
+					return NNF_HIP_EUNSUPPORTED;
+				if (plan_only)
+					return NNF_HIP_OK;
+				window_prologue pro = {};
+				if (!fill_prologue(pro, *prologue, chunk_ptrs, feature_map_count, plane) || (pro.weighted_count > prologue_weighted_max))
+					return NNF_HIP_EUNSUPPORTED;
+				const uint32_t planes_per_group = global_pool_planes_per_group(plane);
+				const size_t lds_bytes = static_cast<size_t>(planes_per_group) * (plane | 1u) * sizeof(float);
+				const dim3 grid((plane_count + planes_per_group - 1) / planes_per_group);
+				const uint32_t plane_magic = static_cast<uint32_t>(((1ull << 32) + plane - 1) / plane);
+				if (pro.need_exp)
+					hipLaunchKernelGGL(global_pool_prologue_kernel<true>, grid, dim3(pool_block_size), lds_bytes, stream, output, input, plane_count, plane, plane_magic, mult, planes_per_group, pro);
+				else
+					hipLaunchKernelGGL(global_pool_prologue_kernel<false>, grid, dim3(pool_block_size), lds_bytes, stream, output, input, plane_count, plane, plane_magic, mult, planes_per_group, pro);
+				return launch_status();
+			}
+			if (!window2d_launch_with_prologue(stream, 4, mult, output, input, static_cast<uint32_t>(input_total), plane_count,
 				input_width, input_height, output_width, output_height, window_width, window_height, window_width, window_height,
 				prologue, chunk_ptrs, feature_map_count, plan_only))
 				return NNF_HIP_EUNSUPPORTED;
@@ -185,10 +334,7 @@ namespace nnf
 			return NNF_HIP_OK;
 		if ((window_width == input_width) && (window_height == input_height) && (plane >= 2) && (plane <= global_pool_max_plane))
 		{
-			// 64 planes of 7x7; fewer of larger planes, so that a compute unit holds several workgroups
-			uint32_t planes_per_group = std::min(global_pool_planes, std::max(8u, (global_pool_lds_floats / plane) & ~3u));
-			if (forced_planes_per_group() != 0)
-				planes_per_group = forced_planes_per_group();
+			const uint32_t planes_per_group = global_pool_planes_per_group(plane);
 			const size_t lds_bytes = static_cast<size_t>(planes_per_group) * (plane | 1u) * sizeof(float);
 			const dim3 grid((plane_count + planes_per_group - 1) / planes_per_group);
 			// plane >= 2 here: a 1x1 window over a 1x1 plane takes the general kernel

@@ -224,14 +224,17 @@ def stem_net(c=8):
 
 def test_plan_folds_a_group_into_the_subsampling_layer_behind_it():
     rep = plan(stem_net(), {"conv1": (8, [28, 28])}, ["global"])
-    # the whole-plane average has a kernel of its own that applies no layers: ELU runs in front of it
-    assert step_names(rep) == ["bn+relu+pool1", "tanh+abs+pool2", "elu", "global"]
-    assert [s["fused"] for s in rep["steps"]] == [True, True, False, False]
+    # the last average covers the whole 7x7 plane (the global pooling kernel): it takes ELU along as well
+    assert step_names(rep) == ["bn+relu+pool1", "tanh+abs+pool2", "elu+global"]
+    assert [s["fused"] for s in rep["steps"]] == [True, True, True]
     assert rep["steps"][0]["inputs"] == ["conv1"] and rep["steps"][1]["inputs"] == ["pool1"]
-    # no intermediate tensor of the groups is planned: conv1, pool1 (14x14), pool2 (7x7, ELU in place), global
+    # no intermediate tensor of the groups is planned: conv1, pool1 (14x14), pool2 (7x7), global
     assert rep["per_entry_bytes"] == 8 * 4 * (28 * 28 + 14 * 14 + 7 * 7 + 1)
-    # a 7x7 window over 14x14 planes is an ordinary window: ELU goes along
+    # a 7x7 window over 14x14 planes is an ordinary window
     assert step_names(plan(stem_net(), {"conv1": (8, [56, 56])}, ["global"]))[2:] == ["elu+global"]
+    # whole planes of fewer than four floats are left to the plain kernel
+    tiny = [S.L("Data", "x"), S.L("ReLU", "relu", ["x"]), S.L("AverageSubsampling", "avg", ["relu"], windows=[3, 1])]
+    assert step_names(plan(tiny, {"x": (8, [3, 1])}, ["avg"])) == ["relu", "avg"]
     rep = plan(stem_net(), {"conv1": (8, [28, 28])}, ["global"], fuse=False)
     assert len(rep["steps"]) == 8 and not any(s["fused"] for s in rep["steps"])
 

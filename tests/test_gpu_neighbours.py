@@ -310,6 +310,14 @@ def run_fused_pool(gpu, x, ops, chunks, ww, wh, mult, expect=0):
     ((2, 3, 113, 115), 3, 3, "bn_relu"),               # leftover margins, plane not a multiple of 4
     ((1, 4, 9, 7), 3, 2, "leaky"),                     # small planes of 63 floats
     ((7, 9, 5, 5), 2, 2, "bn_prelu_elu_sigmoid"),      # planes of 25 floats, margins
+    # whole-plane windows: the global pooling kernel
+    ((64, 128, 7, 7), 7, 7, "bn_relu"),                # a ResNet-like tail: 49 floats per plane, float4s straddle planes
+    ((3, 5, 7, 7), 7, 7, "bn_prelu_elu_sigmoid"),      # the last workgroup holds 15 planes: 735 floats, three behind the last float4
+    ((9, 70, 8, 8), 8, 8, "tanh_abs"),
+    ((5, 33, 14, 14), 14, 14, "prelu_bn"),
+    ((2, 7, 15, 15), 15, 15, "bn_relu"),               # 225 floats per plane
+    ((6, 11, 3, 5), 5, 3, "leaky"),
+    ((1, 1, 2, 2), 2, 2, "bn_relu"),
 ])
 def test_average_subsampling_with_group_folded_in(gpu, shape, ww, wh, group):
     gen = T.rng(67, sum(shape) + ww)
@@ -334,8 +342,8 @@ def test_subsampling_that_cannot_fold_a_group_in_says_so(gpu):
     run_fused_max(gpu, T.normal(gen, (4, 6, 8, 8)), ops, chunks, [2, 2], None, None, fm=2, expect=capi.E_UNSUPPORTED)
     run_fused_max(gpu, T.normal(gen, (2, 6, 4, 6, 8)), ops, chunks, [2, 2, 2], None, None, expect=capi.E_UNSUPPORTED)
     run_fused_max(gpu, T.normal(gen, (1, 6, 3, 20000)), ops, chunks, [2, 3], [2, 1], None, expect=capi.E_UNSUPPORTED)
-    # whole-plane average windows have their own kernel
-    run_fused_pool(gpu, T.normal(gen, (4, 6, 7, 7)), ops, chunks, 7, 7, 1.0, expect=capi.E_UNSUPPORTED)
+    # whole-plane average windows over planes of fewer than four floats
+    run_fused_pool(gpu, T.normal(gen, (4, 6, 1, 3)), ops, chunks, 3, 1, 1.0, expect=capi.E_UNSUPPORTED)
     # a group with an Add, a group of another shape, a missing weight pointer
     x = gpu.to_device(T.normal(gen, (2, 6, 8, 8)))
     out = gpu.torch.empty(2 * 6 * 16, dtype=gpu.torch.float32, device=gpu.device)
