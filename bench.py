@@ -14,7 +14,8 @@ Prints ONE JSON line. `value` = algorithmic bytes per step / wall time per step 
 wall time brackets exactly K steps with a device synchronisation on both sides. `roofline` is
 measured with HIP events on the launch stream around the same K steps. `cpu_baseline` is the CPU
 restatement of nnForge's plain backend (oracle/, layer by layer, unfused, OpenMP on all host
-cores) timed in this process on the same workload.
+cores) timed in this process on the same workload; `per_config[...].cpu` holds the same for every
+configuration, each on a bounded number of passes.
 """
 
 import argparse
@@ -447,6 +448,131 @@ def cpu_baseline_config0(runner, group, seconds=8.0):
     }
 
 
+class CpuPlainBackend:
+    """nnForge's plain backend restated in oracle/, driven the way forward_propagation_plain drives its testers: one
+    OpenMP pass per layer, in place where the tester allows it. Inputs are views of one pool of random floats (the
+    values do not matter for the time; expf-heavy layers get the spread BASELINE.json states through `scale`)."""
+
+    def __init__(self, max_elements):
+        import oracle
+
+        self.oracle = oracle
+        self.threads = oracle.max_threads()
+        gen = np.random.Generator(np.random.MT19937(SEED + 1))
+        self.pool = gen.standard_normal(max_elements, dtype=np.float32)
+        self.work = [np.empty(max_elements, dtype=np.float32) for _ in range(3)]
+        self.gen = gen
+
+    def weights(self, group):
+        chunks = []
+        for kind, c in group.chunks:
+            if kind == "bn":
+                chunks += [(self.gen.random(c, dtype=np.float32) + np.float32(0.5)), self.gen.standard_normal(c, dtype=np.float32) * np.float32(0.3),
+                           self.gen.standard_normal(c, dtype=np.float32) * np.float32(0.3), (self.gen.random(c, dtype=np.float32) + np.float32(0.6))]
+            else:
+                chunks.append(self.gen.random(c, dtype=np.float32) * np.float32(0.25))
+        return [np.ascontiguousarray(v, dtype=np.float32) for v in chunks]
+
+    def layer(self, op, chunks, src, dst):
+        from nnforge_amd import capi
+
+        o = self.oracle
+        kind = op[0]
+        if kind == capi.OP_BATCH_NORM:
+            o.batch_norm(src, *chunks[op[1]:op[1] + 4], out=dst)
+        elif kind == capi.OP_RELU:
+            o.rectified_linear(src, op[2] if len(op) > 2 else 0.0, out=dst)
+        elif kind == capi.OP_PRELU:
+            o.parametric_rectified_linear(src, chunks[op[1]], out=dst)
+        elif kind == capi.OP_ELU:
+            o.exponential_linear(src, out=dst)
+        elif kind == capi.OP_SIGMOID:
+            o.sigmoid(src, out=dst)
+        elif kind == capi.OP_TANH:
+            o.hyperbolic_tangent(src, op[2], op[3], out=dst)
+        else:
+            raise ValueError("layer kind %r" % (kind,))
+
+    def group_pass(self, group, chunks):
+        """One forward pass of the group's layers, unfused."""
+        n, c, plane = group.entry_count, group.feature_map_count, group.plane
+        total = n * c * plane
+        values = []
+        for j, arm in enumerate(group.arms):
+            v = self.pool[:total].reshape(n, c, plane)
+            buf = self.work[j % 2][:total].reshape(n, c, plane)
+            for op in arm:
+                self.layer(op, chunks, v, buf)
+                v = buf
+            values.append(v)
+        if len(group.arms) > 1:
+            out = self.work[2][:total].reshape(n, c, plane)
+            self.oracle.add(values, 1.0, out=out)
+            v = out
+        else:
+            v = values[0]
+            if not group.arms[0]:
+                raise ValueError("a group without layers")
+        for op in group.tail:
+            buf = v if v.base is not self.pool else self.work[2][:total].reshape(n, c, plane)
+            self.layer(op, chunks, v, buf)
+            v = buf
+        return v
+
+    def time_passes(self, one_pass, seconds, most=200):
+        one_pass()
+        times = []
+        t_end = time.perf_counter() + seconds
+        while (time.perf_counter() < t_end and len(times) < most) or len(times) < 2:
+            t0 = time.perf_counter()
+            one_pass()
+            times.append(time.perf_counter() - t0)
+        return statistics.median(times), len(times)
+
+
+def cpu_per_config(per_config, seconds_each=2.0):
+    """Adds {"cpu": ...} to the entries of configs 1-4: the same workload on the host through the oracle, layer by
+    layer and unfused, on a bounded number of passes. GB/s of the same algorithmic bytes, so the columns compare."""
+    from nnforge_amd import workloads as w
+
+    groups4 = w.resnet50_groups(64)
+    largest = max([w.group_elements(w.config2()), w.group_elements(w.config3())] + [w.group_elements(g) for g in groups4])
+    cpu = CpuPlainBackend(largest)
+
+    def attach(name, seconds, passes, what):
+        e = per_config[name]
+        e["cpu"] = {"ms_per_step": seconds * 1e3, "gbps": e["algorithmic_bytes_per_step"] / seconds / 1e9,
+                    "elements_per_s": e["elements_per_step"] / seconds, "cores": cpu.threads, "kind": "port",
+                    "sample": "%s, %d passes, median" % (what, passes)}
+
+    if "config1" in per_config:
+        n, c, plane = w.CONFIG1_SHAPE
+        x = (cpu.pool[:n * c * plane] * np.float32(2.0)).reshape(n, c, plane)
+        out = np.empty_like(x)
+        sec, k = cpu.time_passes(lambda: cpu.oracle.softmax(x, out=out), seconds_each)
+        attach("config1", sec, k, "softmax 256 x 1000 whole")
+    for name, group, scale in (("config2", w.config2(), 1.0), ("config3", w.config3(), 2.0 ** 0.5)):
+        if name in per_config:
+            chunks = cpu.weights(group)
+            sec, k = cpu.time_passes(lambda: cpu.group_pass(group, chunks), seconds_each)
+            attach(name, sec, k, "%s whole, one pass per layer" % name)
+    if "config4" in per_config:
+        prepared = [(g, cpu.weights(g)) for g in groups4]
+        pool_shape, sm_shape = w.resnet50_tail(64)
+        pool_in = cpu.pool[:int(np.prod(pool_shape))].reshape(pool_shape)
+        sm_in = (cpu.pool[:sm_shape[0] * sm_shape[1]] * np.float32(2.0)).reshape(sm_shape)
+        sm_out = np.empty_like(sm_in)
+
+        def stack():
+            for g, chunks in prepared:
+                cpu.group_pass(g, chunks)
+            cpu.oracle.average_subsampling(pool_in, [7, 7], mult=1.0 / 49.0)
+            cpu.oracle.softmax(sm_in, out=sm_out)
+
+        sec, k = cpu.time_passes(stack, seconds_each, most=3)
+        attach("config4", sec, k, "the whole stack (49 groups unfused + average + softmax)")
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -503,6 +629,9 @@ def main():
                 per_config[name] = run(name, k, wu)
         if args.workload == "config0":
             cpu = cpu_baseline_config0(runner, w.config0())
+            per_config["config0"]["cpu"] = {k: cpu[k] for k in ("ms_per_step", "elements_per_s", "cores", "kind", "sample")}
+            per_config["config0"]["cpu"]["gbps"] = cpu["value"]
+        cpu_per_config(per_config)
 
     launches = main_entry["launches_per_step"]
     achieved = main_entry["algorithmic_bytes_per_step"] / launches / (main_entry["event_ms_per_step"] * 1e-3 / launches) / 1e9
