@@ -160,7 +160,7 @@ namespace nnf
 						stage_prologue_coefficients(lds_coef, weights, planes_here, pro);
 					if (EXP)
 						stage_exp2_table(lds_exp);
-					if (EXP || !uniform)
+					if (EXP || (!uniform && (pro.weighted_count != 0)))
 						__syncthreads();
 					if (EXP)
 						exp_ctx = exp_context_from_lds(lds_exp);
@@ -171,18 +171,21 @@ namespace nnf
 					uint32_t off[STAGE];
 					// Planes that are not a multiple of four floats long: a float4 may straddle two of them (never
 					// three: the host declines planes of under 4 floats). Bit k: vector k does.
-					const bool straddle = (planes_here > 1) && ((in_plane & 3u) != 0);
+					// which plane a value belongs to matters only to layers with weights, and only with several planes here
+					const bool per_plane = !uniform && (planes_here > 1) && (pro.weighted_count != 0);
+					const bool straddle = per_plane && ((in_plane & 3u) != 0);
 					uint32_t straddling = 0;
 					#pragma unroll
 					for(int k = 0; k < STAGE; ++k)
 					{
 						const uint32_t i = base + k * max_block_size + threadIdx.x;
 						const bool valid = i < vectors;
+						// lanes past the end put zeros through the layers
 						v[k][0] = valid ? t[k].x : 0.0f; v[k][1] = valid ? t[k].y : 0.0f; v[k][2] = valid ? t[k].z : 0.0f; v[k][3] = valid ? t[k].w : 0.0f;
 						// plane, inside the workgroup's range, of the first float of this float4 (floats in front
 						// of the range count as plane 0: they are staged but not read)
 						const uint32_t first_pos = max(i * 4, shift) - shift;
-						const uint32_t p = ((planes_here > 1) && valid) ? fast_divide(first_pos, in_plane, pro.in_plane_magic) : 0u;
+						const uint32_t p = (per_plane && valid) ? fast_divide(first_pos, in_plane, pro.in_plane_magic) : 0u;
 						off[k] = p * (2 * pro.weighted_count);
 						// floats from staged position (p + 1) * in_plane + shift on belong to plane p + 1; beyond
 						// the last plane of the workgroup they are not read
