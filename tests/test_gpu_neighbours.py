@@ -333,6 +333,22 @@ def test_average_subsampling_with_group_folded_in(gpu, shape, ww, wh, group):
     assert T.bit_mismatches(got, want) == 0
 
 
+@pytest.mark.parametrize("shape", [(4, 16, 128, 128), (64, 256, 8, 8)])
+def test_exp_layers_folded_into_subsampling_over_a_sweep_of_all_exponents(gpu, shape):
+    """ELU, Sigmoid and TanH inside the subsampling kernels (their own expf batches and range repair) on a regular
+    sweep of fp32 bit patterns - every 4099th, so every exponent and both signs, NaNs and infinities included. A 1x1
+    average window passes each value through (0.0F + x, times 1), so the output is the layer's result element by
+    element: bit for bit the oracle's. One plane per workgroup (bands) and many small planes per workgroup."""
+    count = int(np.prod(shape))
+    bits = (np.arange(count, dtype=np.uint64) * 4099 % (1 << 32)).astype(np.uint32)
+    x = bits.view(F).reshape(shape)
+    for op, fn in (((capi.OP_ELU,), oracle.exponential_linear), ((capi.OP_SIGMOID,), oracle.sigmoid),
+                   ((capi.OP_TANH, 0, 1.7159, 0.6666), lambda v: oracle.hyperbolic_tangent(v, 1.7159, 0.6666))):
+        want = oracle.average_subsampling(fn(x), [1, 1], mult=1.0)
+        got = run_fused_pool(gpu, x, [op], [], 1, 1, 1.0)
+        assert T.bit_mismatches(got, want) == 0, "layer kind %d" % op[0]
+
+
 def test_subsampling_that_cannot_fold_a_group_in_says_so(gpu):
     gen = T.rng(68, 0)
     ops, chunks, _ = prologue_case("bn_relu", gen, 6)
