@@ -35,10 +35,23 @@ def hipcc_path():
 
 
 def build_hip_library(verbose=False):
-    """Compiles nnforge_amd/csrc/*.hip into nnforge_amd/libnnforge_hip.so (cross-compiles without a GPU)."""
-    tmp = HIP_LIBRARY + ".tmp"
-    cmd = [hipcc_path()] + HIP_FLAGS + ["-o", tmp] + [os.path.join(CSRC_DIR, s) for s in HIP_SOURCES]
-    out = _run(cmd)
+    """Compiles nnforge_amd/csrc/*.hip into nnforge_amd/libnnforge_hip.so (cross-compiles without a GPU): one
+    object per source, a few sources at a time, then one link."""
+    import concurrent.futures
+    import tempfile
+
+    hipcc = hipcc_path()
+    compile_flags = [f for f in HIP_FLAGS if f != "-shared"] + ["-c"]
+    with tempfile.TemporaryDirectory(prefix="nnforge_hip_build_") as tmp_dir:
+        def compile_one(source):
+            obj = os.path.join(tmp_dir, os.path.splitext(source)[0] + ".o")
+            return obj, _run([hipcc] + compile_flags + ["-o", obj, os.path.join(CSRC_DIR, source)])
+
+        with concurrent.futures.ThreadPoolExecutor(max_workers=4) as pool:
+            results = list(pool.map(compile_one, HIP_SOURCES))
+        tmp = HIP_LIBRARY + ".tmp"
+        out = "".join(text for _, text in results)
+        out += _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-fvisibility=hidden", "-o", tmp] + [obj for obj, _ in results])
     os.replace(tmp, HIP_LIBRARY)
     if verbose and out.strip():
         print(out)
