@@ -588,6 +588,9 @@ def main():
 
     from nnforge_amd import workloads as w
 
+    import __graft_entry__
+
+    __graft_entry__.ensure_built()
     runner = Runner()
     per_config = {}
 

@@ -15,6 +15,13 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
 
 
+def pytest_sessionstart(session):
+    # a fresh checkout holds no built libraries (they are not under version control): build them once
+    import __graft_entry__
+
+    __graft_entry__.ensure_built()
+
+
 @pytest.fixture(scope="session")
 def gpu():
     """Session-wide handle for GPU tests: fails loudly (no skip, no fallback) when the HIP
