@@ -121,3 +121,26 @@ class GpuHarness:
         rc = self.lib.nnf_hip_chain_forward(self.stream, ctypes.byref(desc), d_out.data_ptr(), ins, chk if d_chunks else None)
         assert rc == expect, capi.error_string(rc)
         return self.to_host(d_out)
+
+
+def golden_expf():
+    """(x, expf(x)) of tests/golden/expf_vectors.npy: 8192 inputs and glibc 2.35's expf of them (see make_expf_vectors.py)."""
+    import os
+
+    data = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "expf_vectors.npy"))
+    return data[0].view(np.float32).copy(), data[1].view(np.float32).copy()
+
+
+def layers_from_golden_expf(x, e):
+    """What ELU, Sigmoid(-x) and TanH(steepness 0.5, scale 1) must return for inputs x whose expf is e, by the reference's
+    formulas in IEEE fp32 operations (numpy float32 arithmetic rounds once per operation):
+    nnforge/plain/exponential_linear_layer_tester_plain.cpp:50, sigmoid_layer_tester_plain.cpp:51,
+    hyperbolic_tangent_layer_tester_plain.cpp:49-55."""
+    one = np.float32(1.0)
+    with np.errstate(all="ignore"):
+        elu = np.where(x >= 0, x, e - one).astype(np.float32)
+        elu = np.where(np.isnan(x), (e - one), elu).astype(np.float32)  # NaN >= 0 is false: the expf branch
+        sigmoid_of_minus_x = (one / (e + one)).astype(np.float32)
+        tanh = (((e - one) / (e + one)) * one).astype(np.float32)
+    return elu, sigmoid_of_minus_x, tanh
+

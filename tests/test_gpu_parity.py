@@ -592,6 +592,17 @@ def test_exp_layers_over_the_whole_fp32_range(gpu):
     print("exp layers: %d inputs per layer checked, %d mismatches" % (checked, total_bad))
 
 
+def test_device_expf_against_the_golden_vectors(gpu):
+    """The device's ELU, Sigmoid and TanH on the 8192 inputs of tests/golden/expf_vectors.npy against the reference's
+    formulas applied to the recorded glibc expf values: no host libm is involved when this runs."""
+    x, e = T.golden_expf()
+    elu, sig, tanh = T.layers_from_golden_expf(x, e)
+    shape = (1, 1, x.size)
+    assert T.bit_mismatches(gpu.chain(shape, [[(ELU,)]], [], [x.reshape(shape)]), elu) == 0
+    assert T.bit_mismatches(gpu.chain(shape, [[(SIGMOID,)]], [], [(-x).reshape(shape)]), sig) == 0
+    assert T.bit_mismatches(gpu.chain(shape, [[(TANH, 0, 1.0, 0.5)]], [], [x.reshape(shape)]), tanh) == 0
+
+
 def test_short_division_sequences_equal_ieee_division_for_every_denominator(gpu):
     """The device's own sweep over every non-negative float e with e + 1 <= 2^126 (2^31 values): the
     reciprocal sequence of Sigmoid and the quotient sequence of TanH return the bits of IEEE division."""

@@ -486,3 +486,16 @@ def test_update_bn_weights_formula_and_effect():
     m2, s2 = oracle.update_bn_weights(mean, inv_sigma, st["average"], st["std_dev"])
     after = oracle.FeatureMapStat(c).write(oracle.batch_norm(x, ones, zeros, m2, s2)).get()
     assert np.abs(after["average"]).max() < 1e-5 and np.abs(after["std_dev"] - 1.0).max() < 1e-5
+
+
+def test_host_expf_is_the_function_the_golden_vectors_were_taken_from():
+    """tests/golden/expf_vectors.npy holds glibc 2.35's expf on 8192 inputs (all exponents, the underflow and overflow
+    edges, zeros, infinities, NaN). The oracle's ELU, Sigmoid and TanH call the host's expf: on these inputs they must
+    return what the reference's formulas give for the recorded expf values, bit for bit - so a host with another expf
+    would show up here instead of as a mysterious GPU mismatch."""
+    x, e = T.golden_expf()
+    elu, sig, tanh = T.layers_from_golden_expf(x, e)
+    assert T.bit_mismatches(oracle.exponential_linear(x), elu) == 0
+    assert T.bit_mismatches(oracle.sigmoid(-x), sig) == 0
+    assert T.bit_mismatches(oracle.hyperbolic_tangent(x, 1.0, 0.5), tanh) == 0
+
