@@ -38,6 +38,8 @@ MEASURED_TRAFFIC_BYTES = {
     "config0": 51565056,    # algorithmic 51,381,248
     "config2": 1233228800,  # algorithmic 1,233,130,496
     "config3": 205650944,   # algorithmic 205,529,088
+    "config1": 2117540,     # algorithmic 2,048,000 (profiles/softmax_and_resnet50_stack.md)
+    "config4": 124914115,   # average over the 51 launches of a step: 6,370,619,861 per step, algorithmic 6,359,339,008
 }
 
 
