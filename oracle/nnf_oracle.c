@@ -26,7 +26,9 @@
  * feature-map / entry windows, the start value, tie and NaN cases, and a brute-force loop for tiling;
  * the statistics against two-pass fp64 numpy (mean, population variance, fp32 rounding before the
  * square root), packet invariance, a large-offset case, and the batch norm refresh against its two
- * fp32 formulas and the closed loop (refreshed weights give mean 0, deviation 1). Not pinned by anything: the bit pattern
+ * fp32 formulas and the closed loop (refreshed weights give mean 0, deviation 1). The libm expf this file calls
+ * is itself checked against recorded values (tests/golden/expf_vectors.npy: glibc 2.35 on 8192 inputs), so a host
+ * whose expf differs is noticed. Not pinned by anything: the bit pattern
  * of the reference *as shipped* (built with -ffast-math -O3 -march=native, Settings.mk:26-28),
  * which depends on the compiler's contraction and vector-libm choices - "parity unpinned" for that;
  * this file states the source-level semantics.
