@@ -176,6 +176,19 @@ NNF_HIP_API int nnf_hip_max_subsampling_forward(void* stream, float* output, con
 	const uint32_t* input_sizes, const uint32_t* subsampling_sizes, const uint32_t* strides, const uint32_t* round_ups,
 	uint32_t feature_map_subsampling_size, uint32_t entry_subsampling_size, int32_t is_min);
 
+/* Average subsampling in the reference's full form: 1 to NNF_HIP_MAX_SUBSAMPLING_DIMENSIONS spatial
+ * dimensions (input_sizes / subsampling_sizes: x first), windows over feature maps and over entries
+ * (output feature maps = input_feature_map_count / feature_map_subsampling_size; the input holds
+ * output_entry_count * entry_subsampling_size entries). Every output is the left-to-right fp32 sum of its
+ * window - x fastest, then the further dimensions, then feature maps, then entries - times mult:
+ * nnforge/plain/average_subsampling_layer_tester_plain.cpp:34-148. Output size per dimension = input size /
+ * window size rounded down (nnforge/average_subsampling_layer.cpp:80-87). 1-D and 2-D windows within a
+ * feature map take the kernels of nnf_hip_average_subsampling_forward. */
+NNF_HIP_API int nnf_hip_average_subsampling_nd_forward(void* stream, float* output, const float* input,
+	uint32_t output_entry_count, uint32_t input_feature_map_count, uint32_t dimension_count,
+	const uint32_t* input_sizes, const uint32_t* subsampling_sizes,
+	uint32_t feature_map_subsampling_size, uint32_t entry_subsampling_size, float mult);
+
 /* Subsampling with the element-wise layers in front of it folded in: `prologue` describes a
  * single-input group without Add (input_count 1, has_add 0; its arm 0 and tail layers are applied in
  * order; its feature_map_count and neuron_count_per_feature_map must be the subsampling input's) whose

@@ -177,19 +177,36 @@ namespace nnforge
 
 		bool has_alpha() const { return alpha != -std::numeric_limits<float>::max(); }
 
-		// 1 / (number of window elements) unless alpha is set
+		// 1 / (number of window elements) unless alpha is set, for relative spatial windows only
 		// (average_subsampling_layer::get_effective_alpha given the full configurations,
 		// nnforge/average_subsampling_layer.cpp:287-303)
 		float get_effective_alpha() const;
 
 		// What the reference's PLAIN tester multiplies by: it passes bare feature-map counts where
 		// configurations are expected (nnforge/plain/average_subsampling_layer_tester_plain.cpp:82),
-		// so without an explicit alpha the spatial window does not divide and the factor is 1.
-		float get_plain_tester_alpha() const;
+		// so without an explicit alpha the spatial window does not divide and only the feature-map and
+		// entry windows do: 1 / (feature_map_window * entry_subsampling_size).
+		float get_plain_tester_alpha(unsigned int feature_map_window = 1) const;
+
+		// the window of dimension i / over feature maps for these input and output sizes
+		// (nnforge/average_subsampling_layer.cpp:104-132: a relative size is the window itself, an absolute
+		// one is the wanted output size and the window is input / output, which must reproduce it)
+		unsigned int get_subsampling_size(unsigned int dimension_id, unsigned int input, unsigned int output) const;
+		unsigned int get_fm_subsampling_size(unsigned int input, unsigned int output) const;
+
+		// 1 / (number of window elements, feature maps and entries included) unless alpha is set, for these
+		// windows (average_subsampling_layer::get_effective_alpha given the full configurations)
+		float get_effective_alpha(const std::vector<unsigned int>& windows, unsigned int feature_map_window) const;
 
 		static const std::string layer_type_name;
-		std::vector<unsigned int> subsampling_sizes; // x first
+		std::vector<unsigned int> subsampling_sizes;    // x first: window size (relative) or output size (absolute)
+		std::vector<bool> subsampling_relative;         // per dimension; empty = all relative
+		unsigned int feature_map_subsampling_size = 1;  // window (relative) or output feature map count (absolute)
+		bool feature_map_relative = true;
+		unsigned int entry_subsampling_size = 1;
 		float alpha;
+
+		bool is_relative(size_t dimension_id) const { return (dimension_id >= subsampling_relative.size()) || subsampling_relative[dimension_id]; }
 	};
 
 	// nnforge/absolute_layer.h; "Absolute"

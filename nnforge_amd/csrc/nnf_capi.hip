@@ -290,6 +290,15 @@ extern "C"
 		return launch_status();
 	}
 
+	int nnf_hip_average_subsampling_nd_forward(void* stream, float* output, const float* input,
+		uint32_t output_entry_count, uint32_t input_feature_map_count, uint32_t dimension_count,
+		const uint32_t* input_sizes, const uint32_t* subsampling_sizes,
+		uint32_t feature_map_subsampling_size, uint32_t entry_subsampling_size, float mult)
+	{
+		return average_subsampling_nd_forward(static_cast<hipStream_t>(stream), output, input, output_entry_count, input_feature_map_count,
+			dimension_count, input_sizes, subsampling_sizes, feature_map_subsampling_size, entry_subsampling_size, mult);
+	}
+
 	int nnf_hip_max_subsampling_fused_forward(void* stream, float* output, const float* input,
 		const nnf_hip_chain_desc* prologue, const float* const* chunk_ptrs,
 		uint32_t output_entry_count, uint32_t input_feature_map_count, uint32_t dimension_count,

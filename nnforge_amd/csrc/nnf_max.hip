@@ -28,7 +28,7 @@ namespace nnf
 			return (current < new_val) ? new_val : current;
 		}
 
-		// What the LDS-staged 2-D window kernel does with the values of a window, scanned x fastest:
+		// What the window kernels do with the values of a window, scanned x fastest:
 		// maximum, minimum (both from the -/+1.0e37F start value), or their left-to-right sum times a
 		// multiplier (average subsampling, nnforge/plain/average_subsampling_layer_tester_plain.cpp:125-145).
 		constexpr int window_op_max = 0;
@@ -49,12 +49,6 @@ namespace nnf
 			if (OP == window_op_sum)
 				return 0.0f;
 			return (OP == window_op_min) ? 1.0e37f : -1.0e37f;
-		}
-
-		template<bool IS_MIN>
-		__device__ __forceinline__ float fold_start()
-		{
-			return IS_MIN ? 1.0e37f : -1.0e37f;
 		}
 
 		// ---- 2-D windows, staged through LDS ------------------------------------------------------
@@ -368,10 +362,11 @@ namespace nnf
 			uint32_t output_count;
 			uint32_t in_size[max_dims], out_size[max_dims], window[max_dims], stride[max_dims]; // unused dimensions are 1
 			uint32_t in_fm, out_fm, fm_window, entry_window, in_plane;
+			float mult; // window_op_sum: the sum is multiplied by it
 		};
 
-		template<bool IS_MIN>
-		__global__ void __launch_bounds__(max_block_size) max_window_nd_kernel(const window_nd_args a)
+		template<int OP>
+		__global__ void __launch_bounds__(max_block_size) window_nd_kernel(const window_nd_args a)
 		{
 			const uint32_t o = blockIdx.x * max_block_size + threadIdx.x;
 			if (o >= a.output_count)
@@ -390,7 +385,7 @@ namespace nnf
 			const uint32_t out_fm_id = rem - out_entry * a.out_fm;
 			const size_t base = (static_cast<size_t>(out_entry) * a.entry_window * a.in_fm + static_cast<size_t>(out_fm_id) * a.fm_window) * a.in_plane;
 
-			float current = fold_start<IS_MIN>();
+			float current = window_fold_start<OP>();
 			// scan order of the reference: x fastest, then y, z, w, feature map, entry
 			for(uint32_t en = 0; en < a.entry_window; ++en)
 			{
@@ -405,13 +400,13 @@ namespace nnf
 							{
 								const float* row = plane + ((static_cast<size_t>(start[3] + w) * a.in_size[2] + start[2] + z) * a.in_size[1] + start[1] + y) * a.in_size[0] + start[0];
 								for(uint32_t x = 0; x < fit[0]; ++x)
-									current = fold<IS_MIN>(current, row[x]);
+									current = window_fold<OP>(current, row[x]);
 							}
 						}
 					}
 				}
 			}
-			a.out[o] = current;
+			a.out[o] = (OP == window_op_sum) ? current * a.mult : current;
 		}
 
 		// ---- maxout ------------------------------------------------------------------------------
@@ -702,9 +697,70 @@ namespace nnf
 		nd.in_plane = static_cast<uint32_t>(in_plane);
 		const dim3 grid((nd.output_count + max_block_size - 1) / max_block_size);
 		if (is_min)
-			hipLaunchKernelGGL(max_window_nd_kernel<true>, grid, dim3(max_block_size), 0, stream, nd);
+			hipLaunchKernelGGL(window_nd_kernel<window_op_min>, grid, dim3(max_block_size), 0, stream, nd);
 		else
-			hipLaunchKernelGGL(max_window_nd_kernel<false>, grid, dim3(max_block_size), 0, stream, nd);
+			hipLaunchKernelGGL(window_nd_kernel<window_op_max>, grid, dim3(max_block_size), 0, stream, nd);
+		return launch_status();
+	}
+
+	// Average subsampling in the reference's full form (nnforge/plain/average_subsampling_layer_tester_plain.cpp:34-148):
+	// 1 to 4 spatial dimensions, windows over feature maps and over entries, every output the left-to-right fp32
+	// sum of its window - x fastest, then the further dimensions, feature maps, entries - times mult. Output size =
+	// input size / window size rounded down per dimension; a margin is not read. Plain 1-D / 2-D windows go to
+	// the staged kernels of average_subsampling_forward; everything else takes one lane per output.
+	int average_subsampling_nd_forward(hipStream_t stream, float* output, const float* input,
+		uint32_t output_entry_count, uint32_t input_feature_map_count, uint32_t dimension_count,
+		const uint32_t* input_sizes, const uint32_t* subsampling_sizes,
+		uint32_t feature_map_subsampling_size, uint32_t entry_subsampling_size, float mult)
+	{
+		if ((output == nullptr) || (input == nullptr) || (input_sizes == nullptr) || (subsampling_sizes == nullptr))
+			return NNF_HIP_EINVAL;
+		if ((dimension_count < 1) || (dimension_count > max_dims))
+			return NNF_HIP_EUNSUPPORTED;
+		if ((input_feature_map_count == 0) || (feature_map_subsampling_size == 0) || (entry_subsampling_size == 0))
+			return NNF_HIP_EINVAL;
+		if ((dimension_count <= 2) && (feature_map_subsampling_size == 1) && (entry_subsampling_size == 1))
+			return average_subsampling_forward(stream, output, input, output_entry_count, input_feature_map_count,
+				input_sizes[0], (dimension_count > 1) ? input_sizes[1] : 1u, subsampling_sizes[0], (dimension_count > 1) ? subsampling_sizes[1] : 1u, mult);
+		if (!is_aligned16(output) || !is_aligned16(input))
+			return NNF_HIP_EALIGN;
+		window_nd_args nd = {};
+		uint64_t in_plane = 1, out_plane = 1;
+		for(uint32_t d = 0; d < max_dims; ++d)
+		{
+			nd.in_size[d] = nd.out_size[d] = nd.window[d] = nd.stride[d] = 1;
+			if (d >= dimension_count)
+				continue;
+			if ((input_sizes[d] == 0) || (subsampling_sizes[d] == 0) || (input_sizes[d] < subsampling_sizes[d]))
+				return NNF_HIP_EINVAL; // nnforge/average_subsampling_layer.cpp:82-87
+			nd.in_size[d] = input_sizes[d];
+			nd.window[d] = nd.stride[d] = subsampling_sizes[d];
+			nd.out_size[d] = input_sizes[d] / subsampling_sizes[d];
+			in_plane *= nd.in_size[d];
+			out_plane *= nd.out_size[d];
+		}
+		const uint32_t out_fm = input_feature_map_count / feature_map_subsampling_size;
+		if (out_fm == 0)
+			return NNF_HIP_EINVAL;
+		const uint64_t input_total = static_cast<uint64_t>(output_entry_count) * entry_subsampling_size * input_feature_map_count * in_plane;
+		const uint64_t output_total = static_cast<uint64_t>(output_entry_count) * out_fm * out_plane;
+		if (output_total == 0)
+			return NNF_HIP_OK;
+		if ((input_total > 0xFFFF0000ull) || (output_total > 0xFFFF0000ull))
+			return NNF_HIP_ETOOBIG;
+		if (overlap(output, output_total * sizeof(float), input, input_total * sizeof(float)))
+			return NNF_HIP_EOVERLAP;
+		nd.out = output;
+		nd.in = input;
+		nd.output_count = static_cast<uint32_t>(output_total);
+		nd.in_fm = input_feature_map_count;
+		nd.out_fm = out_fm;
+		nd.fm_window = feature_map_subsampling_size;
+		nd.entry_window = entry_subsampling_size;
+		nd.in_plane = static_cast<uint32_t>(in_plane);
+		nd.mult = mult;
+		const dim3 grid((nd.output_count + max_block_size - 1) / max_block_size);
+		hipLaunchKernelGGL(window_nd_kernel<window_op_sum>, grid, dim3(max_block_size), 0, stream, nd);
 		return launch_status();
 	}
 

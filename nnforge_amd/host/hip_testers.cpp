@@ -457,14 +457,19 @@ namespace nnforge
 					unsigned int entry_count) override
 				{
 					require_inputs(input_buffers, 1, "AverageSubsampling");
-					hip_safe_call(nnf_hip_average_subsampling_forward(stream_id, *output_buffer, float_ptr(input_buffers[0]),
-						entry_count, output_configuration_specific.feature_map_count, input_width, input_height, window_width, window_height, mult));
+					if (plain_2d)
+						hip_safe_call(nnf_hip_average_subsampling_forward(stream_id, *output_buffer, float_ptr(input_buffers[0]),
+							entry_count, output_configuration_specific.feature_map_count, input_sizes[0], input_sizes[1], windows[0], windows[1], mult));
+					else
+						hip_safe_call(nnf_hip_average_subsampling_nd_forward(stream_id, *output_buffer, float_ptr(input_buffers[0]), entry_count,
+							input_configuration_specific_list[0].feature_map_count, dimension_count, input_sizes.data(), windows.data(),
+							feature_map_window, 1, mult));
 				}
 
 				bool can_apply_prologue() const override
 				{
-					return nnf_hip_average_subsampling_fusable(1, output_configuration_specific.feature_map_count, input_width, input_height,
-						window_width, window_height) == NNF_HIP_OK;
+					return plain_2d && (nnf_hip_average_subsampling_fusable(1, output_configuration_specific.feature_map_count, input_sizes[0], input_sizes[1],
+						windows[0], windows[1]) == NNF_HIP_OK);
 				}
 
 				void enqueue_forward_propagation_with_prologue(void * stream_id, hip_linear_buffer_device::ptr output_buffer,
@@ -472,7 +477,7 @@ namespace nnforge
 					unsigned int entry_count) override
 				{
 					hip_safe_call(nnf_hip_average_subsampling_fused_forward(stream_id, *output_buffer, float_ptr(input_buffer), &prologue, chunk_ptrs,
-						entry_count, output_configuration_specific.feature_map_count, input_width, input_height, window_width, window_height, mult));
+						entry_count, output_configuration_specific.feature_map_count, input_sizes[0], input_sizes[1], windows[0], windows[1], mult));
 				}
 
 			protected:
@@ -482,18 +487,31 @@ namespace nnforge
 					if (!l)
 						throw neural_network_exception("AverageSubsampling tester configured with a layer of type " + layer_schema->get_type_name());
 					const layer_configuration_specific& in = input_configuration_specific_list.at(0);
-					if ((in.get_dimension_count() < 1) || (in.get_dimension_count() > 2) || (l->subsampling_sizes.size() != in.get_dimension_count()))
-						throw neural_network_exception("The hip average subsampling tester handles 1 or 2 spatial dimensions, layer " + layer_schema->instance_name + " has " + std::to_string(in.get_dimension_count()));
-					input_width = in.dimension_sizes[0];
-					input_height = (in.get_dimension_count() > 1) ? in.dimension_sizes[1] : 1;
-					window_width = l->subsampling_sizes[0];
-					window_height = (l->subsampling_sizes.size() > 1) ? l->subsampling_sizes[1] : 1;
-					// The multiplier of the reference's plain tester: window sum unless the schema sets alpha.
-					mult = l->get_plain_tester_alpha();
+					if ((in.get_dimension_count() < 1) || (in.get_dimension_count() > NNF_HIP_MAX_SUBSAMPLING_DIMENSIONS) || (l->subsampling_sizes.size() != in.get_dimension_count()))
+						throw neural_network_exception("The hip average subsampling tester handles 1 to 4 spatial dimensions, layer " + layer_schema->instance_name + " has " + std::to_string(in.get_dimension_count()));
+					if (l->entry_subsampling_size != 1)
+						throw neural_network_exception("The hip average subsampling tester does not run entry subsampling (layer " + layer_schema->instance_name + "): it changes the number of entries between layers");
+					dimension_count = in.get_dimension_count();
+					input_sizes.assign(in.dimension_sizes.begin(), in.dimension_sizes.end());
+					windows.clear();
+					for(unsigned int i = 0; i < dimension_count; ++i)
+						windows.push_back(l->get_subsampling_size(i, in.dimension_sizes[i], output_configuration_specific.dimension_sizes[i]));
+					feature_map_window = l->get_fm_subsampling_size(in.feature_map_count, output_configuration_specific.feature_map_count);
+					plain_2d = (dimension_count <= 2) && (feature_map_window == 1);
+					// the 2-D entry point takes width and height: a 1-D layer is one row high
+					while (input_sizes.size() < 2)
+					{
+						input_sizes.push_back(1);
+						windows.push_back(1);
+					}
+					// The multiplier of the reference's plain tester: window sum (over feature maps: their mean) unless the schema sets alpha.
+					mult = l->get_plain_tester_alpha(feature_map_window);
 				}
 
 			private:
-				unsigned int input_width = 1, input_height = 1, window_width = 1, window_height = 1;
+				std::vector<uint32_t> input_sizes, windows;
+				uint32_t dimension_count = 1, feature_map_window = 1;
+				bool plain_2d = true;
 				float mult = 1.0F;
 			};
 

@@ -321,22 +321,63 @@ namespace nnforge
 		const layer_configuration_specific& in = configs[0];
 		if (in.get_dimension_count() != subsampling_sizes.size())
 			throw neural_network_exception("Dimension count in layer (" + std::to_string(subsampling_sizes.size()) + ") and input configuration (" + std::to_string(in.get_dimension_count()) + ") don't match");
-		layer_configuration_specific res(in.feature_map_count);
+		layer_configuration_specific res;
+		// nnforge/average_subsampling_layer.cpp:74-81
+		if (feature_map_relative)
+			res.feature_map_count = in.feature_map_count / feature_map_subsampling_size;
+		else
+		{
+			res.feature_map_count = feature_map_subsampling_size;
+			get_fm_subsampling_size(in.feature_map_count, res.feature_map_count);
+		}
+		if (res.feature_map_count == 0)
+			throw neural_network_exception("Input feature map count (" + std::to_string(in.feature_map_count) + ") is smaller than feature map subsampling size (" + std::to_string(feature_map_subsampling_size) + ")");
 		for(size_t i = 0; i < subsampling_sizes.size(); ++i)
 		{
-			if (in.dimension_sizes[i] < subsampling_sizes[i])
-				throw neural_network_exception("Input configuration size (" + std::to_string(in.dimension_sizes[i]) + ") of dimension (" + std::to_string(i) + ") is smaller than subsampling size (" + std::to_string(subsampling_sizes[i]) + ")");
-			res.dimension_sizes.push_back(in.dimension_sizes[i] / subsampling_sizes[i]);
+			if (is_relative(i))
+			{
+				if (in.dimension_sizes[i] < subsampling_sizes[i])
+					throw neural_network_exception("Input configuration size (" + std::to_string(in.dimension_sizes[i]) + ") of dimension (" + std::to_string(i) + ") is smaller than subsampling size (" + std::to_string(subsampling_sizes[i]) + ")");
+				res.dimension_sizes.push_back(in.dimension_sizes[i] / subsampling_sizes[i]);
+			}
+			else
+			{
+				if (in.dimension_sizes[i] < subsampling_sizes[i])
+					throw neural_network_exception("Input configuration size (" + std::to_string(in.dimension_sizes[i]) + ") of dimension (" + std::to_string(i) + ") is smaller than subsampled size (" + std::to_string(subsampling_sizes[i]) + ")");
+				get_subsampling_size(static_cast<unsigned int>(i), in.dimension_sizes[i], subsampling_sizes[i]);
+				res.dimension_sizes.push_back(subsampling_sizes[i]);
+			}
 		}
 		return res;
 	}
 
+	unsigned int average_subsampling_layer::get_subsampling_size(unsigned int dimension_id, unsigned int input, unsigned int output) const
+	{
+		if (is_relative(dimension_id))
+			return subsampling_sizes[dimension_id];
+		const unsigned int factor = (output == 0) ? 0 : input / output;
+		if ((factor == 0) || (input / factor != output))
+			throw neural_network_exception("Cannot calculate subsampling factor for input " + std::to_string(input) + " and output " + std::to_string(output));
+		return factor;
+	}
+
+	unsigned int average_subsampling_layer::get_fm_subsampling_size(unsigned int input, unsigned int output) const
+	{
+		if (feature_map_relative)
+			return feature_map_subsampling_size;
+		const unsigned int factor = (output == 0) ? 0 : input / output;
+		if ((factor == 0) || (input / factor != output))
+			throw neural_network_exception("Cannot calculate fm subsampling factor for input " + std::to_string(input) + " and output " + std::to_string(output));
+		return factor;
+	}
+
 	float average_subsampling_layer::get_forward_flops_per_entry(const std::vector<layer_configuration_specific>& configs) const
 	{
+		// nnforge/average_subsampling_layer.cpp:267-285: output neurons * window elements
 		const layer_configuration_specific out = get_output_layer_configuration_specific(configs);
-		float per_item = 1.0F;
-		for(unsigned int s : subsampling_sizes)
-			per_item *= static_cast<float>(s);
+		float per_item = static_cast<float>(get_fm_subsampling_size(configs[0].feature_map_count, out.feature_map_count));
+		for(size_t i = 0; i < subsampling_sizes.size(); ++i)
+			per_item *= static_cast<float>(get_subsampling_size(static_cast<unsigned int>(i), configs[0].dimension_sizes[i], out.dimension_sizes[i]));
 		return static_cast<float>(out.get_neuron_count()) * per_item;
 	}
 
@@ -345,24 +386,56 @@ namespace nnforge
 		if (block == nullptr)
 			throw neural_network_exception("No average_subsampling_param specified for layer " + instance_name + " of type " + layer_type_name);
 		subsampling_sizes.clear();
+		subsampling_relative.clear();
 		for(const schema_param_block * dim : block->children("dimension_param"))
 		{
-			if (!dim->has("subsampling_size"))
-				throw neural_network_exception("Only relative subsampling_size is supported by the hip backend for average subsampling layer " + instance_name);
-			subsampling_sizes.push_back(dim->get_uint("subsampling_size", 1));
+			// nnforge/average_subsampling_layer.cpp:186-194
+			if (dim->has("subsampling_size"))
+			{
+				subsampling_sizes.push_back(dim->get_uint("subsampling_size", 1));
+				subsampling_relative.push_back(true);
+			}
+			else if (dim->has("subsampled_size"))
+			{
+				subsampling_sizes.push_back(dim->get_uint("subsampled_size", 1));
+				subsampling_relative.push_back(false);
+			}
+			else
+				throw neural_network_exception("Neither subsampling_size nor subsampled_size specified for dimension_param of average_subsampling_layer");
 		}
-		if (!block->children("feature_map_param").empty() || !block->children("entry_param").empty())
-			throw neural_network_exception("Feature map and entry subsampling are not supported by the hip backend (layer " + instance_name + ")");
+		feature_map_subsampling_size = 1;
+		feature_map_relative = true;
+		const std::vector<const schema_param_block *> fm = block->children("feature_map_param");
+		if (!fm.empty())
+		{
+			if (fm[0]->has("subsampling_size"))
+				feature_map_subsampling_size = fm[0]->get_uint("subsampling_size", 1);
+			else if (fm[0]->has("subsampled_size"))
+			{
+				feature_map_subsampling_size = fm[0]->get_uint("subsampled_size", 1);
+				feature_map_relative = false;
+			}
+			else
+				throw neural_network_exception("Neither subsampling_size nor subsampled_size specified for feature_map_param of average_subsampling_layer");
+		}
+		const std::vector<const schema_param_block *> en = block->children("entry_param");
+		entry_subsampling_size = en.empty() ? 1 : en[0]->require_uint("subsampling_size", "entry_param of layer " + instance_name);
 		alpha = block->has("alpha") ? block->get_float("alpha", 0.0F) : -std::numeric_limits<float>::max();
 		for(unsigned int s : subsampling_sizes)
 			if (s == 0)
 				throw neural_network_exception("window dimension for average subsampling layer may not be zero");
+		if ((feature_map_subsampling_size == 0) || (entry_subsampling_size == 0))
+			throw neural_network_exception("feature map and entry subsampling sizes for average subsampling layer may not be zero");
 	}
 
 	void average_subsampling_layer::write_params(std::ostream& out, const std::string& indent) const
 	{
-		for(unsigned int s : subsampling_sizes)
-			out << indent << "dimension_param { subsampling_size: " << s << " }\n";
+		for(size_t i = 0; i < subsampling_sizes.size(); ++i)
+			out << indent << "dimension_param { " << (is_relative(i) ? "subsampling_size: " : "subsampled_size: ") << subsampling_sizes[i] << " }\n";
+		if (!feature_map_relative || (feature_map_subsampling_size != 1))
+			out << indent << "feature_map_param { " << (feature_map_relative ? "subsampling_size: " : "subsampled_size: ") << feature_map_subsampling_size << " }\n";
+		if (entry_subsampling_size != 1)
+			out << indent << "entry_param { subsampling_size: " << entry_subsampling_size << " }\n";
 		if (has_alpha())
 			out << indent << "alpha: " << float_text(alpha) << "\n";
 	}
@@ -371,7 +444,11 @@ namespace nnforge
 	{
 		std::stringstream ss;
 		for(size_t i = 0; i < subsampling_sizes.size(); ++i)
-			ss << (i == 0 ? "" : "x") << subsampling_sizes[i];
+			ss << (i == 0 ? "" : "x") << (is_relative(i) ? "" : "->") << subsampling_sizes[i];
+		if (!feature_map_relative || (feature_map_subsampling_size != 1))
+			ss << ", fm " << (feature_map_relative ? "" : "->") << feature_map_subsampling_size;
+		if (entry_subsampling_size != 1)
+			ss << ", samples " << entry_subsampling_size;
 		if (has_alpha())
 			ss << ", alpha " << alpha;
 		return std::vector<std::string>(1, ss.str());
@@ -379,17 +456,22 @@ namespace nnforge
 
 	float average_subsampling_layer::get_effective_alpha() const
 	{
+		return get_effective_alpha(subsampling_sizes, feature_map_relative ? feature_map_subsampling_size : 1);
+	}
+
+	float average_subsampling_layer::get_effective_alpha(const std::vector<unsigned int>& windows, unsigned int feature_map_window) const
+	{
 		if (has_alpha())
 			return alpha;
-		unsigned int elems = 1;
-		for(unsigned int s : subsampling_sizes)
+		unsigned int elems = feature_map_window * entry_subsampling_size;
+		for(unsigned int s : windows)
 			elems *= s;
 		return 1.0F / static_cast<float>(elems);
 	}
 
-	float average_subsampling_layer::get_plain_tester_alpha() const
+	float average_subsampling_layer::get_plain_tester_alpha(unsigned int feature_map_window) const
 	{
-		return has_alpha() ? alpha : 1.0F;
+		return has_alpha() ? alpha : 1.0F / static_cast<float>(feature_map_window * entry_subsampling_size);
 	}
 
 	// ---- Absolute ----------------------------------------------------------------------------

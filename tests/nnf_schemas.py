@@ -39,6 +39,13 @@ def schema_text(layers, name="test_net"):
                         out.append("\t\tdimension_param { subsampling_size: %d%s }" % (w, extra))
                 elif k in ("strides", "round_ups"):
                     continue
+                elif k == "subsampled":
+                    for size in v:
+                        out.append("\t\tdimension_param { subsampled_size: %d }" % size)
+                elif k == "fm_subsampled":
+                    out.append("\t\tfeature_map_param { subsampled_size: %d }" % v)
+                elif k == "entry_window":
+                    out.append("\t\tentry_param { subsampling_size: %d }" % v)
                 elif k == "fm_window":
                     out.append("\t\tfeature_map_param { subsampling_size: %d }" % v)
                 elif k == "function":
@@ -88,7 +95,11 @@ def evaluate(layers, weights, inputs):
             v = oracle.softmax(ins[0])
         elif t == "AverageSubsampling":
             # the plain tester's multiplier: window sum unless alpha is given
-            v = oracle.average_subsampling(ins[0], p["windows"], alpha=p.get("alpha"))
+            x = ins[0]
+            dims = list(x.shape[2:])[::-1]
+            windows = p["windows"] if "windows" in p else [d // o for d, o in zip(dims, p["subsampled"])]
+            fm_window = p.get("fm_window", 1) if "fm_subsampled" not in p else x.shape[1] // p["fm_subsampled"]
+            v = oracle.average_subsampling(x, windows, feature_map_window=fm_window, alpha=p.get("alpha"))
         elif t == "Absolute":
             v = oracle.absolute(ins[0])
         elif t == "Dropout":

@@ -262,6 +262,40 @@ def test_plan_keeps_a_group_out_of_the_subsampling_layer_when_it_must_be_stored(
     assert step_names(plan(deep, {"x": (c, [8, 8, 8])}, ["pool"])) == ["bn+relu", "pool"]
 
 
+def test_average_subsampling_layer_in_the_full_form():
+    """Up to four spatial dimensions, windows over feature maps, sizes given as windows or as wanted output sizes
+    (nnforge/average_subsampling_layer.cpp:62-132, 147-224): text round trip and output configurations."""
+    layers = [S.L("Data", "x"),
+              S.L("AverageSubsampling", "a3", ["x"], windows=[2, 3, 2], fm_window=2),
+              S.L("AverageSubsampling", "abs", ["a3"], subsampled=[3, 1, 2], fm_subsampled=2, alpha=0.25)]
+    text = S.schema_text(layers)
+    once = backend.rewrite_schema(text)
+    assert backend.rewrite_schema(once) == once
+    for needle in ("dimension_param { subsampling_size: 3 }", "feature_map_param { subsampling_size: 2 }",
+                   "dimension_param { subsampled_size: 3 }", "feature_map_param { subsampled_size: 2 }", "alpha: 0.25"):
+        assert needle in once, needle
+    # x: 8 maps of 6 x 7 x 9 -> a3: 4 maps of 3 x 2 x 4 -> abs: 2 maps of 3 x 1 x 2 (windows 1 x 2 x 2 over 2 maps)
+    rep = plan(layers, {"x": (8, [6, 7, 9])}, ["abs"])
+    assert step_names(rep) == ["a3", "abs"]
+    assert rep["per_entry_bytes"] == 4 * (8 * 6 * 7 * 9 + 4 * 3 * 2 * 4 + 2 * 3 * 1 * 2)
+    # an output size the input cannot be divided into: 7 -> 3 gives windows of 2 and 3 outputs, 7 -> 4 does not work out
+    with pytest.raises(backend.BackendError, match="Cannot calculate subsampling factor"):
+        plan([S.L("Data", "x"), S.L("AverageSubsampling", "a", ["x"], subsampled=[4])], {"x": (2, [7])}, ["a"])
+    with pytest.raises(backend.BackendError, match="Cannot calculate fm subsampling factor"):
+        plan([S.L("Data", "x"), S.L("AverageSubsampling", "a", ["x"], windows=[1], fm_subsampled=4)], {"x": (7, [4])}, ["a"])
+    with pytest.raises(backend.BackendError, match="smaller than subsampled size"):
+        plan([S.L("Data", "x"), S.L("AverageSubsampling", "a", ["x"], subsampled=[9])], {"x": (2, [7])}, ["a"])
+    with pytest.raises(backend.BackendError, match="Neither subsampling_size nor subsampled_size"):
+        backend.plan_schema('layer { type: "Data" name: "x" }\nlayer { type: "AverageSubsampling" name: "a" input_layer_name: "x" '
+                            'average_subsampling_param { dimension_param { } } }\n', {"x": (2, [7])}, ["a"])
+    # windows over entries change the number of entries between layers: the driver does not run them
+    with pytest.raises(backend.BackendError, match="entry subsampling"):
+        plan([S.L("Data", "x"), S.L("AverageSubsampling", "a", ["x"], windows=[2], entry_window=2)], {"x": (2, [8])}, ["a"])
+    # five spatial dimensions are beyond the kernels
+    with pytest.raises(backend.BackendError, match="1 to 4 spatial dimensions"):
+        plan([S.L("Data", "x"), S.L("AverageSubsampling", "a", ["x"], windows=[1, 1, 1, 1, 2])], {"x": (2, [2, 2, 2, 2, 2])}, ["a"])
+
+
 def test_neighbour_layer_configuration_rules():
     # output sizes of max subsampling: (in + stride - window + (round_up ? window - 1 : 0)) / stride
     for size, window, stride, up, want in [(112, 3, 2, False, 55), (112, 3, 2, True, 56), (7, 2, 2, False, 3), (7, 2, 2, True, 4), (5, 5, 1, False, 1)]:

@@ -233,6 +233,27 @@ def test_random_networks_equal_the_oracle_layer_by_layer(seed):
         assert_bits(plain[name], values[name], "seed %d unfused, output %s" % (seed, name))
 
 
+def test_average_subsampling_in_the_full_form_through_the_driver():
+    """3-D average subsampling with windows over feature maps, then one given by its output sizes, behind element-wise
+    layers, in packets: equals the oracle layer by layer (the plain tester's multiplier: no division by the spatial
+    window, only by the feature-map window, unless alpha is set)."""
+    gen = T.rng(63, 0)
+    c, n = 8, 9
+    layers = [S.L("Data", "x"), S.L("BatchNorm", "bn", ["x"], feature_map_count=c), S.L("ReLU", "relu", ["bn"]),
+              S.L("AverageSubsampling", "a3", ["relu"], windows=[2, 3, 2], fm_window=2),
+              S.L("TanH", "tanh", ["a3"]),
+              S.L("AverageSubsampling", "abs", ["tanh"], subsampled=[3, 1, 2], fm_subsampled=2, alpha=0.125)]
+    weights = S.make_weights(layers, gen)
+    inputs = {"x": T.normal(gen, (n, c, 9, 7, 6), 2.0)}
+    values = S.evaluate(layers, weights, inputs)
+    assert values["a3"].shape == (n, 4, 4, 2, 3) and values["abs"].shape == (n, 2, 2, 1, 3)
+    got, rep = run(layers, weights, inputs, ["abs", "a3"], values, max_entry_count=4)
+    assert_bits(got["a3"], values["a3"], "3-D average with feature-map windows")
+    assert_bits(got["abs"], values["abs"], "average given by its output sizes")
+    # these shapes have no staged kernel: the groups in front run on their own
+    assert ["+".join(s["layers"]) for s in rep["steps"]] == ["bn+relu", "a3", "tanh", "abs"]
+
+
 def test_dropout_only_network():
     """Dropout straight from the data layer to the output: in place there is nothing to launch."""
     gen = T.rng(58, 0)

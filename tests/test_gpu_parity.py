@@ -558,6 +558,53 @@ def test_average_subsampling_windows(gpu, shape, ww, wh):
     assert T.bit_mismatches(got, want) == 0
 
 
+def run_pool_nd(gpu, x, windows, fm_window=1, entry_window=1, mult=1.0, expect=0):
+    """windows: per spatial dimension, x first"""
+    dims = list(x.shape[2:])[::-1]
+    out_dims = [d // w for d, w in zip(dims, windows)]
+    out_shape = (x.shape[0] // entry_window, x.shape[1] // fm_window) + tuple(out_dims[::-1])
+    d_in = gpu.to_device(x)
+    d_out = gpu.torch.full((max(1, int(np.prod(out_shape))),), float("nan"), dtype=gpu.torch.float32, device=gpu.device)
+    u32 = lambda v: (ctypes.c_uint32 * len(v))(*v)
+    rc = gpu.lib.nnf_hip_average_subsampling_nd_forward(gpu.stream, d_out.data_ptr(), d_in.data_ptr(), x.shape[0] // entry_window, x.shape[1],
+                                                        len(dims), u32(dims), u32(windows), fm_window, entry_window, mult)
+    assert rc == expect, capi.error_string(rc)
+    return gpu.to_host(d_out, out_shape) if expect == 0 else None
+
+
+@pytest.mark.parametrize("shape,windows,fm_window,entry_window", [
+    ((3, 4, 37), [4], 1, 1),                        # 1-D: the staged 2-D kernel
+    ((2, 3, 12, 10), [2, 3], 1, 1),                 # 2-D: the staged 2-D kernel
+    ((2, 6, 12, 10), [2, 3], 3, 1),                 # windows over feature maps
+    ((6, 4, 8, 8), [2, 2], 1, 2),                   # windows over entries
+    ((6, 9, 5, 7), [2, 2], 3, 3),                   # both, with margins
+    ((2, 3, 6, 7, 8), [2, 3, 2], 1, 1),             # 3-D
+    ((4, 4, 3, 4, 5, 6), [2, 2, 2, 3], 2, 2),       # 4-D with feature-map and entry windows
+    ((2, 8, 9), [3], 4, 1),                         # 1-D with feature-map windows
+    ((3, 5, 1, 1), [1, 1], 5, 3),                   # pure feature-map / entry averaging
+])
+def test_average_subsampling_in_the_full_form(gpu, shape, windows, fm_window, entry_window):
+    x = T.normal(T.rng(17, sum(shape) + fm_window), shape)
+    mult = oracle.average_subsampling_full_mult(windows, fm_window, entry_window)
+    want = oracle.average_subsampling(x, windows, feature_map_window=fm_window, entry_window=entry_window, mult=mult)
+    got = run_pool_nd(gpu, x, windows, fm_window, entry_window, mult)
+    assert got.shape == want.shape
+    assert T.bit_mismatches(got, want) == 0
+
+
+def test_average_subsampling_full_form_rejects_bad_arguments(gpu):
+    x = T.normal(T.rng(17, 99), (2, 4, 6, 6, 6))
+    run_pool_nd(gpu, x, [7, 2, 2], expect=capi.E_INVAL)          # window larger than the input
+    run_pool_nd(gpu, x, [2, 2, 2], fm_window=5, expect=capi.E_INVAL)   # more feature maps per window than there are
+    d = gpu.to_device(x)
+    u32 = lambda v: (ctypes.c_uint32 * len(v))(*v)
+    call = gpu.lib.nnf_hip_average_subsampling_nd_forward
+    assert call(gpu.stream, d.data_ptr(), d.data_ptr(), 2, 4, 3, u32([6, 6, 6]), u32([2, 2, 2]), 1, 1, 1.0) == capi.E_OVERLAP
+    assert call(gpu.stream, d.data_ptr(), d.data_ptr(), 2, 4, 5, u32([6] * 5), u32([2] * 5), 1, 1, 1.0) == capi.E_UNSUPPORTED
+    assert call(gpu.stream, None, d.data_ptr(), 2, 4, 3, u32([6, 6, 6]), u32([2, 2, 2]), 1, 1, 1.0) == capi.E_INVAL
+    gpu.torch.cuda.synchronize()
+
+
 # ---------------------------------------------------------------------------------------------
 # every fp32 input through the layers that call expf and divide
 # ---------------------------------------------------------------------------------------------
