@@ -169,12 +169,23 @@ NNF_HIP_API int nnf_hip_maxout_forward(void* stream, float* output, const float*
  * (nnforge/max_subsampling_layer.cpp:131-141); with round_ups[d] != 0 the part of a window beyond the
  * input is skipped (nnforge/cuda/max_subsampling_layer_tester_cuda.cuh:97-116; the plain tester
  * refuses round up). The input holds output_entry_count * entry_subsampling_size entries. The tiling
- * variant of the layer (nnforge/plain/max_subsampling_layer_tester_plain.cpp:78-170) is not provided. */
+ * variant of the layer is nnf_hip_max_subsampling_tiling_forward. */
 #define NNF_HIP_MAX_SUBSAMPLING_DIMENSIONS 4
 NNF_HIP_API int nnf_hip_max_subsampling_forward(void* stream, float* output, const float* input,
 	uint32_t output_entry_count, uint32_t input_feature_map_count, uint32_t dimension_count,
 	const uint32_t* input_sizes, const uint32_t* subsampling_sizes, const uint32_t* strides, const uint32_t* round_ups,
 	uint32_t feature_map_subsampling_size, uint32_t entry_subsampling_size, int32_t is_min);
+
+/* Max (or min) subsampling with tiling (nnforge/plain/max_subsampling_layer_tester_plain.cpp:78-170):
+ * windows of subsampling_sizes[d] every subsampling_sizes[d] elements, computed once per shift of the
+ * window grid by 0 .. subsampling_sizes[d] - 1 elements in every dimension. Input entry e gives the output
+ * entries e * T + j, T = product of the window sizes, j = the shifts taken together x fastest; each holds
+ * feature_map_count feature maps of (input_sizes[d] - (subsampling_sizes[d] - 1)) / subsampling_sizes[d]
+ * elements per dimension (nnforge/max_subsampling_layer.cpp:113-121; input sizes below
+ * 2 * subsampling size - 1 are refused). The fold is that of nnf_hip_max_subsampling_forward. */
+NNF_HIP_API int nnf_hip_max_subsampling_tiling_forward(void* stream, float* output, const float* input,
+	uint32_t input_entry_count, uint32_t feature_map_count, uint32_t dimension_count,
+	const uint32_t* input_sizes, const uint32_t* subsampling_sizes, int32_t is_min);
 
 /* Average subsampling in the reference's full form: 1 to NNF_HIP_MAX_SUBSAMPLING_DIMENSIONS spatial
  * dimensions (input_sizes / subsampling_sizes: x first), windows over feature maps and over entries

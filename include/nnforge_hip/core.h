@@ -104,6 +104,31 @@ namespace nnforge
 	};
 
 	// Base of the schema layers (nnforge/layer.h:37-121), forward/inference side only.
+	// By how much a layer changes the number of entries that flow through it: max subsampling with tiling makes
+	// several entries of one (a factor), windows over entries make one of several (one over a factor)
+	// (nnforge/tiling_factor.h:24-56).
+	class tiling_factor
+	{
+	public:
+		tiling_factor(unsigned int f = 1, bool b_multiply = true);
+
+		// the factor as a count; throws for "one over ..."
+		operator unsigned int() const;
+		std::string str() const;
+		tiling_factor get_inverse() const;
+		tiling_factor& operator *=(const tiling_factor& other);
+
+	private:
+		unsigned int f;
+		bool b_multiply;
+
+		friend bool operator ==(const tiling_factor& t1, const tiling_factor& t2);
+	};
+
+	tiling_factor operator *(const tiling_factor& t1, const tiling_factor& t2);
+	bool operator ==(const tiling_factor& t1, const tiling_factor& t2);
+	bool operator !=(const tiling_factor& t1, const tiling_factor& t2);
+
 	class layer
 	{
 	public:
@@ -130,6 +155,9 @@ namespace nnforge
 		virtual void write_params(std::ostream& out, const std::string& indent) const;
 
 		virtual std::vector<std::string> get_parameter_strings() const { return std::vector<std::string>(); }
+
+		// how the layer changes the number of entries (nnforge/layer.cpp:150-153: it does not)
+		virtual tiling_factor get_tiling_factor() const { return tiling_factor(1); }
 
 		// all values 0.0F
 		layer_data::ptr create_layer_data() const;

@@ -103,7 +103,8 @@ namespace nnforge
 				layer::const_ptr layer_schema,
 				hip_running_configuration::const_ptr hip_config);
 
-			// stream_id: a HIP stream handle. Buffers hold entry_count entries each. The output buffer
+			// stream_id: a HIP stream handle. entry_count counts the entries of the output; the inputs hold as many,
+			// except where the layer itself changes the count (windows over entries, tiling). The output buffer
 			// may be the buffer of input get_input_index_layer_can_write().
 			virtual void enqueue_forward_propagation(
 				void * stream_id,

@@ -194,6 +194,9 @@ namespace nnforge
 		unsigned int get_subsampling_size(unsigned int dimension_id, unsigned int input, unsigned int output) const;
 		unsigned int get_fm_subsampling_size(unsigned int input, unsigned int output) const;
 
+		// one output entry per entry_subsampling_size input entries (nnforge/average_subsampling_layer.cpp:240-243)
+		tiling_factor get_tiling_factor() const override { return tiling_factor(entry_subsampling_size).get_inverse(); }
+
 		// 1 / (number of window elements, feature maps and entries included) unless alpha is set, for these
 		// windows (average_subsampling_layer::get_effective_alpha given the full configurations)
 		float get_effective_alpha(const std::vector<unsigned int>& windows, unsigned int feature_map_window) const;
@@ -280,9 +283,8 @@ namespace nnforge
 	};
 
 	// Maximum (or minimum) over windows (nnforge/max_subsampling_layer.h:27-82); "MaxSubsampling".
-	// This backend runs spatial windows with strides and round up, and feature-map subsampling;
-	// tiling and entry subsampling change the number of entries between layers, which its driver
-	// does not do, so the layer refuses them when it is configured.
+	// Spatial windows with strides and round up, windows over feature maps and over entries, and tiling:
+	// with tiling every input entry gives one output entry per shift of the window grid.
 	class max_subsampling_layer : public layer
 	{
 	public:
@@ -295,8 +297,8 @@ namespace nnforge
 			const std::vector<bool>& round_ups = std::vector<bool>(),
 			const std::vector<unsigned int>& strides = std::vector<unsigned int>());
 		layer::ptr clone() const override;
-		// (input + stride - window + (round_up ? window - 1 : 0)) / stride per dimension
-		// (nnforge/max_subsampling_layer.cpp:106-144)
+		// (input + stride - window + (round_up ? window - 1 : 0)) / stride per dimension; with tiling
+		// (input - (window - 1)) / window (nnforge/max_subsampling_layer.cpp:106-144)
 		layer_configuration_specific get_output_layer_configuration_specific(
 			const std::vector<layer_configuration_specific>& input_configuration_specific_list) const override;
 		std::string get_type_name() const override;
@@ -305,6 +307,10 @@ namespace nnforge
 		void read_params(const schema_param_block * block) override;
 		void write_params(std::ostream& out, const std::string& indent) const override;
 		std::vector<std::string> get_parameter_strings() const override;
+		// tiling: the product of the window sizes; otherwise one over entry_subsampling_size
+		// (nnforge/max_subsampling_layer.cpp:239-268)
+		tiling_factor get_tiling_factor() const override;
+		std::vector<tiling_factor> get_tiling_factor_list() const;
 
 		static const std::string layer_type_name;
 		std::vector<unsigned int> subsampling_sizes; // x first

@@ -205,6 +205,10 @@ namespace nnforge
 		debug_state::ptr debug;
 		profile_state::ptr profile;
 		std::map<std::string, layer_configuration_specific> layer_config_map;
+		// entries a layer holds per entry read, and that figure for the output layers, which must agree on it
+		// (nnforge/forward_propagation.h:103-104, forward_propagation.cpp:54-61)
+		std::map<std::string, unsigned int> cumulative_tiling_factor_map;
+		unsigned int output_layers_tiling_factor;
 		float flops;
 		std::set<std::string> data_layer_names;
 		std::map<std::string, float> last_action_seconds;

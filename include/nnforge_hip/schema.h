@@ -39,6 +39,11 @@ namespace nnforge
 		std::map<std::string, layer_configuration_specific> get_layer_configuration_specific_map(
 			const std::map<std::string, layer_configuration_specific>& input_configuration_specific_map) const;
 
+		// per layer: how many entries it holds for each entry the data layers supply. Data layers hold 1; a layer
+		// multiplies the factor of its inputs, which must agree, by its own (nnforge/network_schema.cpp:651-680).
+		// Throws when the inputs of a layer disagree or the product is not a whole number.
+		std::map<std::string, unsigned int> get_cumulative_tiling_factor_map() const;
+
 		// number of layers that read the output of the given layer
 		unsigned int get_consumer_count(const std::string& instance_name) const;
 

@@ -99,6 +99,7 @@ SIGNATURES = {
     "nnf_hip_copy_kernel": [_VP, _VP, _VP, ctypes.c_size_t],
     "nnf_hip_check_division_sequences": [_VP, _VP],
     "nnf_hip_average_subsampling_nd_forward": [_VP, _VP, _VP, _U32, _U32, _U32, _UP, _UP, _U32, _U32, _F],
+    "nnf_hip_max_subsampling_tiling_forward": [_VP, _VP, _VP, _U32, _U32, _U32, _UP, _UP, ctypes.c_int32],
     "nnf_hip_max_subsampling_fused_forward": [_VP, _VP, _VP, ctypes.POINTER(ChainDesc), _PP, _U32, _U32, _U32, _UP, _UP, _UP, _UP, _U32, _U32, ctypes.c_int32],
     "nnf_hip_average_subsampling_fused_forward": [_VP, _VP, _VP, ctypes.POINTER(ChainDesc), _PP, _U32, _U32, _U32, _U32, _U32, _U32, _F],
     "nnf_hip_max_subsampling_fusable": [_U32, _U32, _U32, _UP, _UP, _UP, _UP, _U32, _U32],

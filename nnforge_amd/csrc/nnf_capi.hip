@@ -299,6 +299,14 @@ extern "C"
 			dimension_count, input_sizes, subsampling_sizes, feature_map_subsampling_size, entry_subsampling_size, mult);
 	}
 
+	int nnf_hip_max_subsampling_tiling_forward(void* stream, float* output, const float* input,
+		uint32_t input_entry_count, uint32_t feature_map_count, uint32_t dimension_count,
+		const uint32_t* input_sizes, const uint32_t* subsampling_sizes, int32_t is_min)
+	{
+		return max_subsampling_tiling_forward(static_cast<hipStream_t>(stream), output, input, input_entry_count, feature_map_count,
+			dimension_count, input_sizes, subsampling_sizes, is_min);
+	}
+
 	int nnf_hip_max_subsampling_fused_forward(void* stream, float* output, const float* input,
 		const nnf_hip_chain_desc* prologue, const float* const* chunk_ptrs,
 		uint32_t output_entry_count, uint32_t input_feature_map_count, uint32_t dimension_count,

@@ -113,6 +113,9 @@ namespace nnf
 		const uint32_t* input_sizes, const uint32_t* subsampling_sizes, const uint32_t* strides, const uint32_t* round_ups,
 		uint32_t feature_map_subsampling_size, uint32_t entry_subsampling_size, int32_t is_min,
 		const nnf_hip_chain_desc* prologue, const float* const* chunk_ptrs, bool plan_only);
+	int max_subsampling_tiling_forward(hipStream_t stream, float* output, const float* input,
+		uint32_t input_entry_count, uint32_t feature_map_count, uint32_t dimension_count,
+		const uint32_t* input_sizes, const uint32_t* subsampling_sizes, int32_t is_min);
 	int average_subsampling_nd_forward(hipStream_t stream, float* output, const float* input,
 		uint32_t output_entry_count, uint32_t input_feature_map_count, uint32_t dimension_count,
 		const uint32_t* input_sizes, const uint32_t* subsampling_sizes,

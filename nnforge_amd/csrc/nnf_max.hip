@@ -363,9 +363,12 @@ namespace nnf
 			uint32_t in_size[max_dims], out_size[max_dims], window[max_dims], stride[max_dims]; // unused dimensions are 1
 			uint32_t in_fm, out_fm, fm_window, entry_window, in_plane;
 			float mult; // window_op_sum: the sum is multiplied by it
+			uint32_t tile_count; // TILING: output entries per input entry, the product of the window sizes
 		};
 
-		template<int OP>
+		// TILING: output entry e * tile_count + j holds the windows of input entry e whose grid is shifted by j,
+		// taken apart x fastest like the window scan (nnforge/plain/max_subsampling_layer_tester_plain.cpp:78-170)
+		template<int OP, bool TILING = false>
 		__global__ void __launch_bounds__(max_block_size) window_nd_kernel(const window_nd_args a)
 		{
 			const uint32_t o = blockIdx.x * max_block_size + threadIdx.x;
@@ -383,7 +386,23 @@ namespace nnf
 			}
 			const uint32_t out_entry = rem / a.out_fm;
 			const uint32_t out_fm_id = rem - out_entry * a.out_fm;
-			const size_t base = (static_cast<size_t>(out_entry) * a.entry_window * a.in_fm + static_cast<size_t>(out_fm_id) * a.fm_window) * a.in_plane;
+			size_t base;
+			if (TILING)
+			{
+				const uint32_t in_entry = out_entry / a.tile_count;
+				uint32_t shift = out_entry - in_entry * a.tile_count;
+				#pragma unroll
+				for(uint32_t d = 0; d < max_dims; ++d)
+				{
+					const uint32_t q = shift / a.window[d];
+					start[d] += shift - q * a.window[d];
+					fit[d] = a.window[d]; // the output sizes leave room for every shift
+					shift = q;
+				}
+				base = (static_cast<size_t>(in_entry) * a.in_fm + out_fm_id) * a.in_plane;
+			}
+			else
+				base = (static_cast<size_t>(out_entry) * a.entry_window * a.in_fm + static_cast<size_t>(out_fm_id) * a.fm_window) * a.in_plane;
 
 			float current = window_fold_start<OP>();
 			// scan order of the reference: x fastest, then y, z, w, feature map, entry
@@ -700,6 +719,65 @@ namespace nnf
 			hipLaunchKernelGGL(window_nd_kernel<window_op_min>, grid, dim3(max_block_size), 0, stream, nd);
 		else
 			hipLaunchKernelGGL(window_nd_kernel<window_op_max>, grid, dim3(max_block_size), 0, stream, nd);
+		return launch_status();
+	}
+
+	// Max subsampling with tiling (nnforge/plain/max_subsampling_layer_tester_plain.cpp:78-170): windows every
+	// window-size elements, once per shift of the window grid; input entry e gives the output entries
+	// e * T .. e * T + T - 1, T = product of the window sizes. Output size = (input - (window - 1)) / window
+	// (nnforge/max_subsampling_layer.cpp:113-121). One lane per output; the shifted grids read the same input
+	// T times over, out of the caches.
+	int max_subsampling_tiling_forward(hipStream_t stream, float* output, const float* input,
+		uint32_t input_entry_count, uint32_t feature_map_count, uint32_t dimension_count,
+		const uint32_t* input_sizes, const uint32_t* subsampling_sizes, int32_t is_min)
+	{
+		if ((output == nullptr) || (input == nullptr) || (input_sizes == nullptr) || (subsampling_sizes == nullptr))
+			return NNF_HIP_EINVAL;
+		if ((dimension_count < 1) || (dimension_count > max_dims))
+			return NNF_HIP_EUNSUPPORTED;
+		if (feature_map_count == 0)
+			return NNF_HIP_EINVAL;
+		if (!is_aligned16(output) || !is_aligned16(input))
+			return NNF_HIP_EALIGN;
+		window_nd_args nd = {};
+		uint64_t in_plane = 1, out_plane = 1, tile_count = 1;
+		for(uint32_t d = 0; d < max_dims; ++d)
+		{
+			nd.in_size[d] = nd.out_size[d] = nd.window[d] = nd.stride[d] = 1;
+			if (d >= dimension_count)
+				continue;
+			const uint32_t size = input_sizes[d], window = subsampling_sizes[d];
+			if ((window == 0) || (static_cast<uint64_t>(size) + 1 < static_cast<uint64_t>(window) * 2))
+				return NNF_HIP_EINVAL; // "smaller than subsampling size * 2 - 1"
+			nd.in_size[d] = size;
+			nd.window[d] = nd.stride[d] = window;
+			nd.out_size[d] = (size - (window - 1)) / window;
+			in_plane *= size;
+			out_plane *= nd.out_size[d];
+			tile_count *= window;
+			if (tile_count > 0xFFFFull)
+				return NNF_HIP_ETOOBIG;
+		}
+		const uint64_t input_total = static_cast<uint64_t>(input_entry_count) * feature_map_count * in_plane;
+		const uint64_t output_total = static_cast<uint64_t>(input_entry_count) * tile_count * feature_map_count * out_plane;
+		if (output_total == 0)
+			return NNF_HIP_OK;
+		if ((input_total > 0xFFFF0000ull) || (output_total > 0xFFFF0000ull))
+			return NNF_HIP_ETOOBIG;
+		if (overlap(output, output_total * sizeof(float), input, input_total * sizeof(float)))
+			return NNF_HIP_EOVERLAP;
+		nd.out = output;
+		nd.in = input;
+		nd.output_count = static_cast<uint32_t>(output_total);
+		nd.in_fm = nd.out_fm = feature_map_count;
+		nd.fm_window = nd.entry_window = 1;
+		nd.in_plane = static_cast<uint32_t>(in_plane);
+		nd.tile_count = static_cast<uint32_t>(tile_count);
+		const dim3 grid((nd.output_count + max_block_size - 1) / max_block_size);
+		if (is_min)
+			hipLaunchKernelGGL((window_nd_kernel<window_op_min, true>), grid, dim3(max_block_size), 0, stream, nd);
+		else
+			hipLaunchKernelGGL((window_nd_kernel<window_op_max, true>), grid, dim3(max_block_size), 0, stream, nd);
 		return launch_status();
 	}
 

@@ -218,6 +218,65 @@ namespace nnforge
 
 	// ---- layer -----------------------------------------------------------------------------
 
+	// ---- tiling_factor (nnforge/tiling_factor.cpp:24-140) --------------------------------------
+
+	tiling_factor::tiling_factor(unsigned int f, bool b_multiply)
+		: f(f), b_multiply(b_multiply || (f == 1))
+	{
+	}
+
+	tiling_factor::operator unsigned int() const
+	{
+		if (!b_multiply)
+			throw neural_network_exception("Cannot convert tiling_factor " + str() + " to unsigned int");
+		return f;
+	}
+
+	std::string tiling_factor::str() const
+	{
+		return b_multiply ? std::to_string(f) : ("1/" + std::to_string(f));
+	}
+
+	tiling_factor tiling_factor::get_inverse() const
+	{
+		return tiling_factor(f, !b_multiply);
+	}
+
+	tiling_factor& tiling_factor::operator *=(const tiling_factor& other)
+	{
+		if (b_multiply == other.b_multiply)
+			f *= other.f;
+		else if ((f >= other.f) && (f % other.f == 0))
+			f /= other.f;
+		else if ((f < other.f) && (other.f % f == 0))
+		{
+			f = other.f / f;
+			b_multiply = !b_multiply;
+		}
+		else
+			throw neural_network_exception("Cannot multiply tiling factor " + str() + " and " + other.str() + " ");
+		if (f == 1)
+			b_multiply = true;
+		return *this;
+	}
+
+	tiling_factor operator *(const tiling_factor& t1, const tiling_factor& t2)
+	{
+		tiling_factor res = t1;
+		res *= t2;
+		return res;
+	}
+
+	bool operator ==(const tiling_factor& t1, const tiling_factor& t2)
+	{
+		return (t1.f == t2.f) && (t1.b_multiply == t2.b_multiply);
+	}
+
+	bool operator !=(const tiling_factor& t1, const tiling_factor& t2)
+	{
+		return !(t1 == t2);
+	}
+
 	layer_configuration_specific layer::get_output_layer_configuration_specific(
 		const std::vector<layer_configuration_specific>& input_configuration_specific_list) const
 	{

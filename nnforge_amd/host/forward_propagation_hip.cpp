@@ -62,6 +62,7 @@ namespace nnforge
 				std::vector<int> input_buffers;
 				bool passes_input_on = false;        // every layer of the step is a Dropout
 				bool prologue = false;               // desc holds element-wise layers that the tester (a subsampling layer) applies to its input
+				unsigned int entry_factor = 1;       // entries of the step's output per entry read (the cumulative tiling factor of its last layer)
 			};
 
 			bool is_unary_elementwise(const std::string& type)
@@ -417,6 +418,7 @@ namespace nnforge
 				std::string types;
 				float step_flops = 0.0F;
 				plan.passes_input_on = true;
+				plan.entry_factor = cumulative_tiling_factor_map.at(plan.info.layer_names.back());
 				for(const std::string& n : plan.info.layer_names)
 				{
 					plan.key += (plan.key.empty() ? "" : "+") + n;
@@ -426,11 +428,11 @@ namespace nnforge
 					std::vector<layer_configuration_specific> inputs;
 					for(const std::string& input : l->input_layer_instance_names)
 						inputs.push_back(layer_config_map[input]);
-					step_flops += l->get_forward_flops_per_entry(inputs);
+					step_flops += l->get_forward_flops_per_entry(inputs) * static_cast<float>(cumulative_tiling_factor_map.at(n));
 				}
-				float step_bytes = static_cast<float>(config.get_neuron_count()) * sizeof(float);
+				float step_bytes = static_cast<float>(config.get_neuron_count()) * sizeof(float) * static_cast<float>(plan.entry_factor);
 				for(const std::string& input : plan.info.input_names)
-					step_bytes += static_cast<float>(layer_config_map[input].get_neuron_count()) * sizeof(float);
+					step_bytes += static_cast<float>(layer_config_map[input].get_neuron_count()) * sizeof(float) * static_cast<float>(cumulative_tiling_factor_map.at(input));
 				action_flops_per_entry[plan.key] = step_flops;
 				action_bytes_per_entry[plan.key] = step_bytes;
 				action_layer_types[plan.key] = types;
@@ -461,7 +463,8 @@ namespace nnforge
 			{
 				step_plan& plan = p->plans[i];
 				const std::string& out_name = plan.info.layer_names.back();
-				const size_t out_floats = layer_config_map[out_name].get_neuron_count();
+				// per entry read: a layer behind a tiling layer holds several entries for each (nnforge/plain/forward_propagation_plain.cpp:281)
+				const size_t out_floats = static_cast<size_t>(layer_config_map[out_name].get_neuron_count()) * plan.entry_factor;
 				for(const std::string& in : plan.info.input_names)
 					plan.input_buffers.push_back(p->value_to_buffer.at(in));
 
@@ -606,7 +609,7 @@ namespace nnforge
 					const layer_configuration_specific& c = layer_config_map[n];
 					stat_states[n].reset(new hip_linear_buffer_device(static_cast<size_t>(c.feature_map_count) * sizeof(nnf_hip_running_stat)));
 					size_t bytes = 0;
-					hip_safe_call(nnf_hip_feature_map_stat_workspace_bytes(packet, c.feature_map_count, c.get_neuron_count_per_feature_map(), &bytes));
+					hip_safe_call(nnf_hip_feature_map_stat_workspace_bytes(packet * output_layers_tiling_factor, c.feature_map_count, c.get_neuron_count_per_feature_map(), &bytes));
 					stat_workspaces[n].reset(new hip_linear_buffer_device(bytes));
 					stat_workspace_bytes[n] = bytes;
 					hip_safe_call(nnf_hip_feature_map_stat_init(p->stream, static_cast<nnf_hip_running_stat *>(static_cast<void *>(*stat_states[n])), c.feature_map_count));
@@ -621,7 +624,7 @@ namespace nnforge
 				if (!stats_on_device)
 					for(const std::string& n : output_layer_names)
 						if (staging[s].find(n) == staging[s].end())
-							staging[s][n].reset(new pinned_buffer(static_cast<size_t>(layer_config_map[n].get_neuron_count()) * sizeof(float) * packet));
+							staging[s][n].reset(new pinned_buffer(static_cast<size_t>(layer_config_map[n].get_neuron_count()) * sizeof(float) * packet * output_layers_tiling_factor));
 			}
 			hip_event upload_done[slot_count], kernels_done[slot_count], download_done[slot_count];
 			bool slot_used[slot_count] = { false, false };
@@ -666,12 +669,14 @@ namespace nnforge
 						action_seconds[p->plans[i].key] += ms * 1.0e-3F;
 					}
 				}
-				for(unsigned int e = 0; (e < f.entries) && !stats_on_device; ++e)
+				// every entry the output layers hold goes to the writer, numbered in sequence
+				// (nnforge/cuda/forward_propagation_cuda.cpp:271-278)
+				for(unsigned int e = 0; (e < f.entries * output_layers_tiling_factor) && !stats_on_device; ++e)
 				{
 					std::map<std::string, const float *> data_map;
 					for(const std::string& n : output_layer_names)
 						data_map[n] = static_cast<const float *>(staging[f.slot][n]->ptr) + static_cast<size_t>(e) * layer_config_map[n].get_neuron_count();
-					writer.write(f.first_entry + e, data_map);
+					writer.write(f.first_entry * output_layers_tiling_factor + e, data_map);
 				}
 			};
 
@@ -729,6 +734,7 @@ namespace nnforge
 					for(size_t i = 0; i < p->plans.size(); ++i)
 					{
 						step_plan& plan = p->plans[i];
+						const unsigned int step_entries = entries_read * plan.entry_factor; // nnforge/plain/forward_propagation_plain.cpp:185
 						if (profiling)
 							hip_safe_call(nnf_hip_event_record(step_events[slot][i]->ev, p->stream));
 						std::vector<hip_linear_buffer_device::const_ptr> inputs;
@@ -738,13 +744,13 @@ namespace nnforge
 							continue; // Dropout layers only, in place: nothing to do at inference
 						if (plan.prologue)
 						{
-							plan.desc.entry_count = entries_read;
+							plan.desc.entry_count = step_entries;
 							plan.tester->enqueue_forward_propagation_with_prologue(p->stream, buffers[slot][plan.output_buffer], inputs.at(0), plan.desc,
-								chunk_ptrs[i].empty() ? nullptr : chunk_ptrs[i].data(), entries_read);
+								chunk_ptrs[i].empty() ? nullptr : chunk_ptrs[i].data(), step_entries);
 						}
 						else if (plan.info.fused)
 						{
-							plan.desc.entry_count = entries_read;
+							plan.desc.entry_count = step_entries;
 							std::vector<const float *> in_ptrs;
 							for(const hip_linear_buffer_device::const_ptr& b : inputs)
 								in_ptrs.push_back(static_cast<const float *>(*b));
@@ -757,7 +763,7 @@ namespace nnforge
 							std::map<std::string, std::vector<hip_linear_buffer_device::const_ptr> >::const_iterator w = p->weights.find(layer_name);
 							plan.tester->enqueue_forward_propagation(p->stream, buffers[slot][plan.output_buffer], none,
 								(w == p->weights.end()) ? none : w->second, none, inputs, none,
-								hip_linear_buffer_device::ptr(), hip_linear_buffer_device::ptr(), entries_read);
+								hip_linear_buffer_device::ptr(), hip_linear_buffer_device::ptr(), step_entries);
 						}
 					}
 					if (profiling)
@@ -770,7 +776,7 @@ namespace nnforge
 							hip_safe_call(nnf_hip_feature_map_stat_accumulate(p->stream,
 								static_cast<nnf_hip_running_stat *>(static_cast<void *>(*stat_states[n])), *stat_workspaces[n], stat_workspace_bytes[n],
 								static_cast<const float *>(static_cast<const void *>(*buffers[slot][p->value_to_buffer.at(n)])),
-								entries_read, c.feature_map_count, c.get_neuron_count_per_feature_map()));
+								entries_read * output_layers_tiling_factor, c.feature_map_count, c.get_neuron_count_per_feature_map()));
 						}
 					}
 					hip_safe_call(nnf_hip_event_record(kernels_done[slot].ev, p->stream));
@@ -780,7 +786,7 @@ namespace nnforge
 					for(const std::string& n : output_layer_names)
 						if (!stats_on_device)
 						hip_safe_call(nnf_hip_memcpy_d2h(staging[slot][n]->ptr, *buffers[slot][p->value_to_buffer.at(n)],
-							static_cast<size_t>(layer_config_map[n].get_neuron_count()) * sizeof(float) * entries_read, p->download_stream));
+							static_cast<size_t>(layer_config_map[n].get_neuron_count()) * sizeof(float) * entries_read * output_layers_tiling_factor, p->download_stream));
 					hip_safe_call(nnf_hip_event_record(download_done[slot].ev, p->download_stream));
 					slot_used[slot] = true;
 				}
@@ -809,7 +815,7 @@ namespace nnforge
 					hip_safe_call(nnf_hip_memcpy_d2h(states.data(), *stat_states[n], states.size() * sizeof(nnf_hip_running_stat), nullptr));
 					stat_writer->merge(n, states);
 				}
-				stat_writer->add_entries(read_total);
+				stat_writer->add_entries(read_total * output_layers_tiling_factor);
 			}
 
 			entries_processed = read_total;

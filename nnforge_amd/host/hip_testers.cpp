@@ -457,13 +457,14 @@ namespace nnforge
 					unsigned int entry_count) override
 				{
 					require_inputs(input_buffers, 1, "AverageSubsampling");
+					// entry_count counts the entries of the output; the input holds entry_window times as many
 					if (plain_2d)
 						hip_safe_call(nnf_hip_average_subsampling_forward(stream_id, *output_buffer, float_ptr(input_buffers[0]),
 							entry_count, output_configuration_specific.feature_map_count, input_sizes[0], input_sizes[1], windows[0], windows[1], mult));
 					else
 						hip_safe_call(nnf_hip_average_subsampling_nd_forward(stream_id, *output_buffer, float_ptr(input_buffers[0]), entry_count,
 							input_configuration_specific_list[0].feature_map_count, dimension_count, input_sizes.data(), windows.data(),
-							feature_map_window, 1, mult));
+							feature_map_window, entry_window, mult));
 				}
 
 				bool can_apply_prologue() const override
@@ -489,15 +490,14 @@ namespace nnforge
 					const layer_configuration_specific& in = input_configuration_specific_list.at(0);
 					if ((in.get_dimension_count() < 1) || (in.get_dimension_count() > NNF_HIP_MAX_SUBSAMPLING_DIMENSIONS) || (l->subsampling_sizes.size() != in.get_dimension_count()))
 						throw neural_network_exception("The hip average subsampling tester handles 1 to 4 spatial dimensions, layer " + layer_schema->instance_name + " has " + std::to_string(in.get_dimension_count()));
-					if (l->entry_subsampling_size != 1)
-						throw neural_network_exception("The hip average subsampling tester does not run entry subsampling (layer " + layer_schema->instance_name + "): it changes the number of entries between layers");
+					entry_window = l->entry_subsampling_size;
 					dimension_count = in.get_dimension_count();
 					input_sizes.assign(in.dimension_sizes.begin(), in.dimension_sizes.end());
 					windows.clear();
 					for(unsigned int i = 0; i < dimension_count; ++i)
 						windows.push_back(l->get_subsampling_size(i, in.dimension_sizes[i], output_configuration_specific.dimension_sizes[i]));
 					feature_map_window = l->get_fm_subsampling_size(in.feature_map_count, output_configuration_specific.feature_map_count);
-					plain_2d = (dimension_count <= 2) && (feature_map_window == 1);
+					plain_2d = (dimension_count <= 2) && (feature_map_window == 1) && (entry_window == 1);
 					// the 2-D entry point takes width and height: a 1-D layer is one row high
 					while (input_sizes.size() < 2)
 					{
@@ -510,7 +510,7 @@ namespace nnforge
 
 			private:
 				std::vector<uint32_t> input_sizes, windows;
-				uint32_t dimension_count = 1, feature_map_window = 1;
+				uint32_t dimension_count = 1, feature_map_window = 1, entry_window = 1;
 				bool plain_2d = true;
 				float mult = 1.0F;
 			};
@@ -619,14 +619,25 @@ namespace nnforge
 					unsigned int entry_count) override
 				{
 					require_inputs(input_buffers, 1, "MaxSubsampling");
+					// entry_count counts the entries of the output
+					if (tile_count != 0)
+					{
+						if (entry_count % tile_count != 0)
+							throw neural_network_exception("Max subsampling with tiling (layer " + layer_schema->instance_name + "): " + std::to_string(entry_count)
+								+ " output entries are not a multiple of " + std::to_string(tile_count));
+						hip_safe_call(nnf_hip_max_subsampling_tiling_forward(stream_id, *output_buffer, float_ptr(input_buffers[0]), entry_count / tile_count,
+							input_configuration_specific_list[0].feature_map_count, static_cast<uint32_t>(input_sizes.size()),
+							input_sizes.data(), windows.data(), is_min ? 1 : 0));
+						return;
+					}
 					hip_safe_call(nnf_hip_max_subsampling_forward(stream_id, *output_buffer, float_ptr(input_buffers[0]), entry_count,
 						input_configuration_specific_list[0].feature_map_count, static_cast<uint32_t>(input_sizes.size()),
-						input_sizes.data(), windows.data(), strides.data(), round_ups.data(), feature_map_subsampling_size, 1, is_min ? 1 : 0));
+						input_sizes.data(), windows.data(), strides.data(), round_ups.data(), feature_map_subsampling_size, entry_window, is_min ? 1 : 0));
 				}
 
 				bool can_apply_prologue() const override
 				{
-					return nnf_hip_max_subsampling_fusable(1, input_configuration_specific_list[0].feature_map_count, static_cast<uint32_t>(input_sizes.size()),
+					return (tile_count == 0) && (entry_window == 1) && nnf_hip_max_subsampling_fusable(1, input_configuration_specific_list[0].feature_map_count, static_cast<uint32_t>(input_sizes.size()),
 						input_sizes.data(), windows.data(), strides.data(), round_ups.data(), feature_map_subsampling_size, 1) == NNF_HIP_OK;
 				}
 
@@ -645,8 +656,6 @@ namespace nnforge
 					std::shared_ptr<const max_subsampling_layer> l = std::dynamic_pointer_cast<const max_subsampling_layer>(layer_schema);
 					if (!l)
 						throw neural_network_exception("MaxSubsampling tester configured with a layer of type " + layer_schema->get_type_name());
-					if (l->tiling || (l->entry_subsampling_size != 1))
-						throw neural_network_exception("The hip max subsampling tester does not run tiling or entry subsampling (layer " + layer_schema->instance_name + ")");
 					const layer_configuration_specific& in = input_configuration_specific_list.at(0);
 					if ((in.get_dimension_count() < 1) || (in.get_dimension_count() > NNF_HIP_MAX_SUBSAMPLING_DIMENSIONS))
 						throw neural_network_exception("The hip max subsampling tester handles 1 to 4 spatial dimensions, layer " + layer_schema->instance_name + " has " + std::to_string(in.get_dimension_count()));
@@ -657,12 +666,15 @@ namespace nnforge
 					for(bool r : l->round_ups)
 						round_ups.push_back(r ? 1u : 0u);
 					feature_map_subsampling_size = l->feature_map_subsampling_size;
+					entry_window = l->entry_subsampling_size;
+					tile_count = l->tiling ? static_cast<unsigned int>(l->get_tiling_factor()) : 0;
 					is_min = l->is_min;
 				}
 
 			private:
 				std::vector<uint32_t> input_sizes, windows, strides, round_ups;
-				unsigned int feature_map_subsampling_size = 1;
+				unsigned int feature_map_subsampling_size = 1, entry_window = 1;
+				unsigned int tile_count = 0; // 0: no tiling
 				bool is_min = false;
 			};
 

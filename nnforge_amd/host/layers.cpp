@@ -666,17 +666,42 @@ namespace nnforge
 		const layer_configuration_specific& in = configs[0];
 		if (in.get_dimension_count() != subsampling_sizes.size())
 			throw neural_network_exception("Dimension count in layer (" + std::to_string(subsampling_sizes.size()) + ") and input configuration (" + std::to_string(in.get_dimension_count()) + ") don't match");
-		if (tiling || (entry_subsampling_size != 1))
-			throw neural_network_exception("Tiling and entry subsampling of max subsampling layer " + instance_name + " change the number of entries between layers, which the hip backend does not support");
 		layer_configuration_specific res(in.feature_map_count / feature_map_subsampling_size);
 		for(size_t i = 0; i < subsampling_sizes.size(); ++i)
 		{
+			if (tiling)
+			{
+				if (in.dimension_sizes[i] < (subsampling_sizes[i] * 2 - 1))
+					throw neural_network_exception("Input configuration size (" + std::to_string(in.dimension_sizes[i]) + ") of dimension (" + std::to_string(i)
+						+ ") is smaller than subsampling size (" + std::to_string(subsampling_sizes[i]) + ") * 2 - 1");
+				res.dimension_sizes.push_back((in.dimension_sizes[i] - (subsampling_sizes[i] - 1)) / subsampling_sizes[i]);
+				continue;
+			}
 			const int new_size = (static_cast<int>(in.dimension_sizes[i]) + static_cast<int>(strides[i]) - static_cast<int>(subsampling_sizes[i])
 				+ (round_ups[i] ? static_cast<int>(subsampling_sizes[i]) - 1 : 0)) / static_cast<int>(strides[i]);
 			if (new_size <= 0)
 				throw neural_network_exception("Input configuration size (" + std::to_string(in.dimension_sizes[i]) + ") of dimension (" + std::to_string(i) + ") produces 0 output size");
 			res.dimension_sizes.push_back(static_cast<unsigned int>(new_size));
 		}
+		return res;
+	}
+
+	tiling_factor max_subsampling_layer::get_tiling_factor() const
+	{
+		if (!tiling)
+			return tiling_factor(entry_subsampling_size).get_inverse();
+		tiling_factor res(1);
+		for(const tiling_factor& t : get_tiling_factor_list())
+			res *= t;
+		return res;
+	}
+
+	std::vector<tiling_factor> max_subsampling_layer::get_tiling_factor_list() const
+	{
+		std::vector<tiling_factor> res;
+		if (tiling)
+			for(unsigned int s : subsampling_sizes)
+				res.push_back(tiling_factor(s));
 		return res;
 	}
 

@@ -268,6 +268,7 @@ namespace nnforge
 		: output_layer_names(output_layer_names)
 		, debug(debug ? debug : debug_state::ptr(new debug_state()))
 		, profile(profile ? profile : profile_state::ptr(new profile_state()))
+		, output_layers_tiling_factor(1)
 		, flops(0.0F)
 	{
 		if (output_layer_names.empty())
@@ -277,6 +278,13 @@ namespace nnforge
 		schema = reduced;
 		for(const layer::const_ptr& l : schema->get_data_layers())
 			data_layer_names.insert(l->instance_name);
+
+		cumulative_tiling_factor_map = schema->get_cumulative_tiling_factor_map();
+		output_layers_tiling_factor = cumulative_tiling_factor_map.at(output_layer_names[0]);
+		for(const std::string& n : output_layer_names)
+			if (cumulative_tiling_factor_map.at(n) != output_layers_tiling_factor)
+				throw neural_network_exception("Inconsistent tiling factors across output layers: "
+					+ std::to_string(output_layers_tiling_factor) + " and " + std::to_string(cumulative_tiling_factor_map.at(n)));
 	}
 
 	bool forward_propagation::is_schema_with_weights() const
@@ -326,7 +334,8 @@ namespace nnforge
 			std::vector<layer_configuration_specific> inputs;
 			for(const std::string& input : l->input_layer_instance_names)
 				inputs.push_back(layer_config_map[input]);
-			flops += l->get_forward_flops_per_entry(inputs);
+			// nnforge/network_action_schema.cpp:166-170
+			flops += l->get_forward_flops_per_entry(inputs) * static_cast<float>(cumulative_tiling_factor_map.at(l->instance_name));
 		}
 
 		layer_config_map_modified();

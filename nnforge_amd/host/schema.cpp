@@ -333,6 +333,27 @@ namespace nnforge
 		return res;
 	}
 
+	std::map<std::string, unsigned int> network_schema::get_cumulative_tiling_factor_map() const
+	{
+		std::map<std::string, unsigned int> res;
+		for(const layer::const_ptr& l : layers)
+		{
+			if (l->input_layer_instance_names.empty())
+			{
+				res[l->instance_name] = 1;
+				continue;
+			}
+			const unsigned int input_factor = res.at(l->input_layer_instance_names[0]);
+			for(const std::string& input : l->input_layer_instance_names)
+				if (res.at(input) != input_factor)
+					throw neural_network_exception("Tiling factors mismatch for inputs of layer " + l->instance_name + ": "
+						+ std::to_string(input_factor) + " and " + std::to_string(res.at(input)));
+			// the conversion throws when the layer would leave a fraction of an entry
+			res[l->instance_name] = static_cast<unsigned int>(tiling_factor(input_factor) * l->get_tiling_factor());
+		}
+		return res;
+	}
+
 	unsigned int network_schema::get_consumer_count(const std::string& instance_name) const
 	{
 		unsigned int count = 0;

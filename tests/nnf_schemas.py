@@ -99,7 +99,8 @@ def evaluate(layers, weights, inputs):
             dims = list(x.shape[2:])[::-1]
             windows = p["windows"] if "windows" in p else [d // o for d, o in zip(dims, p["subsampled"])]
             fm_window = p.get("fm_window", 1) if "fm_subsampled" not in p else x.shape[1] // p["fm_subsampled"]
-            v = oracle.average_subsampling(x, windows, feature_map_window=fm_window, alpha=p.get("alpha"))
+            v = oracle.average_subsampling(x, windows, feature_map_window=fm_window, entry_window=p.get("entry_window", 1),
+                                           alpha=p.get("alpha"))
         elif t == "Absolute":
             v = oracle.absolute(ins[0])
         elif t == "Dropout":
@@ -110,7 +111,8 @@ def evaluate(layers, weights, inputs):
             v = oracle.maxout(ins[0], p["feature_map_subsampling_size"])
         elif t == "MaxSubsampling":
             v = oracle.max_subsampling(ins[0], p["windows"], strides=p.get("strides"), round_ups=p.get("round_ups"),
-                                       feature_map_window=p.get("fm_window", 1), is_min=p.get("function") == "MIN")
+                                       feature_map_window=p.get("fm_window", 1), entry_window=p.get("entry_window", 1),
+                                       is_min=p.get("function") == "MIN", tiling=p.get("tiling", False))
         else:
             raise ValueError(t)
         values[name] = v

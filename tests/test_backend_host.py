@@ -288,8 +288,8 @@ def test_average_subsampling_layer_in_the_full_form():
     with pytest.raises(backend.BackendError, match="Neither subsampling_size nor subsampled_size"):
         backend.plan_schema('layer { type: "Data" name: "x" }\nlayer { type: "AverageSubsampling" name: "a" input_layer_name: "x" '
                             'average_subsampling_param { dimension_param { } } }\n', {"x": (2, [7])}, ["a"])
-    # windows over entries change the number of entries between layers: the driver does not run them
-    with pytest.raises(backend.BackendError, match="entry subsampling"):
+    # a window over entries needs a whole number of them: on its own it leaves half an entry per entry read
+    with pytest.raises(backend.BackendError, match="Cannot convert tiling_factor 1/2"):
         plan([S.L("Data", "x"), S.L("AverageSubsampling", "a", ["x"], windows=[2], entry_window=2)], {"x": (2, [8])}, ["a"])
     # five spatial dimensions are beyond the kernels
     with pytest.raises(backend.BackendError, match="1 to 4 spatial dimensions"):
@@ -307,8 +307,8 @@ def test_neighbour_layer_configuration_rules():
         plan([S.L("Data", "x"), S.L("MaxSubsampling", "p", ["x"], windows=[5])], {"x": (2, [4])}, ["p"])
     with pytest.raises(backend.BackendError, match="don't match"):
         plan([S.L("Data", "x"), S.L("MaxSubsampling", "p", ["x"], windows=[2])], {"x": (2, [4, 4])}, ["p"])
-    with pytest.raises(backend.BackendError, match="hip backend does not support"):
-        plan([S.L("Data", "x"), S.L("MaxSubsampling", "p", ["x"], windows=[2], tiling=True)], {"x": (2, [8])}, ["p"])
+    with pytest.raises(backend.BackendError, match=r"smaller than subsampling size \(3\) \* 2 - 1"):
+        plan([S.L("Data", "x"), S.L("MaxSubsampling", "p", ["x"], windows=[3], tiling=True)], {"x": (2, [4])}, ["p"])
     with pytest.raises(backend.BackendError, match="stride dimension"):
         plan([S.L("Data", "x"), S.L("MaxSubsampling", "p", ["x"], windows=[2], strides=[0])], {"x": (2, [8])}, ["p"])
     with pytest.raises(backend.BackendError, match="not evenly divisible"):
@@ -319,6 +319,38 @@ def test_neighbour_layer_configuration_rules():
         plan([S.L("Data", "x"), S.L("Data", "y"), S.L("Concat", "c", ["x", "y"])], {"x": (4, [8]), "y": (4, [9])}, ["c"])
     with pytest.raises(backend.BackendError, match="dropout_rate"):
         plan([S.L("Data", "x"), S.L("Dropout", "d", ["x"], dropout_rate=1.0)], {"x": (4, [8])}, ["d"])
+
+
+def test_tiling_factors_scale_buffers_and_must_agree():
+    """nnforge/network_schema.cpp:651-680, nnforge/forward_propagation.cpp:54-61: a layer holds (entries read) x (the
+    product of the tiling factors on the way to it) entries; inputs of a layer and the output layers must agree."""
+    # x: 2 maps of 9 x 7 -> tiling windows 2 x 3: 6 entries of 2 maps of (9-1)/2 x (7-2)/3 = 4 x 1
+    tiled = [S.L("Data", "x"), S.L("MaxSubsampling", "p", ["x"], windows=[2, 3], tiling=True), S.L("ReLU", "r", ["p"]),
+             S.L("AverageSubsampling", "tiles_mean", ["r"], windows=[1, 1], entry_window=3),
+             S.L("MaxSubsampling", "tiles_max", ["tiles_mean"], windows=[1, 1], entry_window=2)]
+    rep = plan(tiled, {"x": (2, [9, 7])}, ["tiles_max"], fuse=False)
+    assert step_names(rep) == ["p", "r", "tiles_mean", "tiles_max"]
+    # buffers per entry read: x, p (6 entries; r works in place), tiles_mean (2 entries), tiles_max (1 entry)
+    assert rep["per_entry_bytes"] == 4 * (2 * 9 * 7 + 6 * 2 * 4 + 2 * 2 * 4 + 2 * 4)
+    # the element-wise layer in front of a layer with a window over entries is not folded into it
+    rep = plan(tiled, {"x": (2, [9, 7])}, ["tiles_max"])
+    assert step_names(rep) == ["p", "r", "tiles_mean", "tiles_max"]
+    # an output in the middle: 6 entries per entry read
+    rep = plan(tiled, {"x": (2, [9, 7])}, ["r"])
+    assert rep["per_entry_bytes"] == 4 * (2 * 9 * 7 + 6 * 2 * 4 + 6 * 2 * 4)
+    # a window over 4 of the 6 entries leaves one and a half
+    with pytest.raises(backend.BackendError, match="Cannot multiply tiling factor 6 and 1/4"):
+        plan(tiled[:3] + [S.L("AverageSubsampling", "bad", ["r"], windows=[1, 1], entry_window=4)], {"x": (2, [9, 7])}, ["bad"])
+    # the two inputs of an Add hold different numbers of entries
+    with pytest.raises(backend.BackendError, match="Tiling factors mismatch for inputs of layer a: 6 and 2"):
+        plan(tiled[:4] + [S.L("MaxSubsampling", "q", ["x"], windows=[2, 3], strides=[2, 6]), S.L("Add", "a", ["p", "tiles_mean"])],
+             {"x": (2, [9, 7])}, ["a"])
+    with pytest.raises(backend.BackendError, match="Inconsistent tiling factors across output layers: 6 and 2"):
+        plan(tiled, {"x": (2, [9, 7])}, ["r", "tiles_mean"])
+    # written out and read back
+    once = backend.rewrite_schema(S.schema_text(tiled))
+    assert "tiling: true" in once and once.count("entry_param { subsampling_size:") == 2
+    assert backend.rewrite_schema(once) == once
 
 
 @pytest.mark.parametrize("seed", range(30))

@@ -254,6 +254,41 @@ def test_average_subsampling_in_the_full_form_through_the_driver():
     assert ["+".join(s["layers"]) for s in rep["steps"]] == ["bn+relu", "a3", "tanh", "abs"]
 
 
+@pytest.mark.parametrize("fuse", [True, False])
+def test_tiling_and_windows_over_entries_through_the_driver(fuse):
+    """Max subsampling with tiling makes 4 entries of each entry read, the layers behind it run on all of them, and
+    windows over entries fold them again (nnforge/plain/forward_propagation_plain.cpp:185-192: every tester gets
+    entries read x the cumulative tiling factor of its layer, the writer every entry of the output layers). In packets of
+    4 entries read; the outputs equal the oracle run layer by layer on the whole input."""
+    gen = T.rng(62, int(fuse))
+    c, n = 6, 9
+    layers = [S.L("Data", "x"), S.L("BatchNorm", "bn", ["x"], feature_map_count=c), S.L("ReLU", "relu", ["bn"]),
+              S.L("MaxSubsampling", "tiles", ["relu"], windows=[2, 2], tiling=True),
+              S.L("BatchNorm", "bn2", ["tiles"], feature_map_count=c), S.L("TanH", "tanh", ["bn2"]),
+              S.L("AverageSubsampling", "gap", ["tanh"], windows=[6, 5]),
+              S.L("MaxSubsampling", "pairs_min", ["gap"], windows=[1, 1], entry_window=2, function="MIN"),
+              S.L("AverageSubsampling", "mean", ["pairs_min"], windows=[1, 1], entry_window=2)]
+    weights = S.make_weights(layers, gen)
+    inputs = {"x": T.normal(gen, (n, c, 11, 13), 2.0)}
+    values = S.evaluate(layers, weights, inputs)
+    assert values["tiles"].shape == (4 * n, c, 5, 6) and values["pairs_min"].shape == (2 * n, c, 1, 1) and values["mean"].shape == (n, c, 1, 1)
+    got, rep = run(layers, weights, inputs, ["mean"], values, max_entry_count=4, fuse=fuse)
+    assert rep["entries"] == n
+    assert_bits(got["mean"], values["mean"], "mean over the tiles")
+    # outputs that hold 4 entries per entry read, in the order the tiles were made
+    got, rep = run(layers, weights, inputs, ["tanh", "gap"], values, max_entry_count=4, fuse=fuse)
+    assert_bits(got["tanh"], values["tanh"], "layers behind the tiling layer")
+    assert_bits(got["gap"], values["gap"], "average over whole planes of the tiles")
+    if fuse:
+        assert ["+".join(s["layers"]) for s in rep["steps"]] == ["bn+relu", "tiles", "bn2+tanh", "gap"]
+    # statistics over the tiled entries, reduced on the device
+    stat, rep = backend.layer_statistics(S.schema_text(layers), weights, inputs, "tanh", c, max_entry_count=4, fuse=fuse)
+    want = oracle.FeatureMapStat(c).write(values["tanh"]).get()
+    assert rep["entries"] == n and rep["writer_entries"] == 4 * n
+    assert np.array_equal(stat["min"], want["min"]) and np.array_equal(stat["max"], want["max"])
+    assert T.ulp_distance(stat["average"], want["average"]).max() <= 1 and T.ulp_distance(stat["std_dev"], want["std_dev"]).max() <= 1
+
+
 def test_dropout_only_network():
     """Dropout straight from the data layer to the output: in place there is nothing to launch."""
     gen = T.rng(58, 0)

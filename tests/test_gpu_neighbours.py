@@ -168,10 +168,49 @@ def test_max_subsampling_over_feature_maps_and_entries(gpu, fm, en):
     assert T.bit_mismatches(got, want) == 0
 
 
+TILING_CASES = [
+    # shape, windows (x first)
+    ((3, 4, 9, 11), [2, 3]),              # 6 output entries per input entry
+    ((2, 3, 7, 5), [2, 2]),               # the smallest sizes some windows allow: 5 >= 2 * 2 - 1... and margins left over
+    ((5, 2, 23), [4]),                    # 1-D
+    ((2, 2, 5, 6, 9), [3, 2, 2]),         # 3-D
+    ((1, 2, 3, 5, 4, 7), [2, 2, 2, 1]),   # 4-D, a window of 1 in one dimension
+    ((4, 8, 28, 28), [2, 2]),
+    ((2, 1, 3, 3), [1, 1]),               # one tile: plain copy
+]
+
+
+@pytest.mark.parametrize("is_min", [False, True])
+@pytest.mark.parametrize("shape,windows", TILING_CASES)
+def test_max_subsampling_with_tiling(gpu, shape, windows, is_min):
+    """nnforge/plain/max_subsampling_layer_tester_plain.cpp:78-170: every shift of the window grid is an output entry."""
+    x = spiced(T.rng(66, sum(shape) + len(windows)), shape)
+    want = oracle.max_subsampling(x, windows, tiling=True, is_min=is_min)
+    assert want.shape[0] == shape[0] * int(np.prod(windows))
+    dims = list(shape[2:])[::-1]
+    d_in = gpu.to_device(x)
+    d_out = gpu.torch.full((want.size,), float("nan"), dtype=gpu.torch.float32, device=gpu.device)
+    rc = gpu.lib.nnf_hip_max_subsampling_tiling_forward(gpu.stream, d_out.data_ptr(), d_in.data_ptr(), shape[0], shape[1], len(dims),
+                                                        u32(dims), u32(windows), int(is_min))
+    assert rc == 0, capi.error_string(rc)
+    got = gpu.to_host(d_out, want.shape)
+    assert T.bit_mismatches(got, want) == 0
+    # tile 0 is the plain layer with the window as its stride, cut to the tiling's output sizes
+    plain = oracle.max_subsampling(x, windows, is_min=is_min)
+    tile0 = got.reshape((shape[0], -1) + got.shape[1:])[:, 0]
+    cut = (slice(None), slice(None)) + tuple(slice(0, n) for n in got.shape[2:])
+    assert T.bit_mismatches(tile0, plain[cut]) == 0
+
+
 def test_neighbour_entry_points_reject_bad_arguments(gpu):
     lib, s = gpu.lib, gpu.stream
     d = gpu.to_device(np.zeros(256, F))
     e = gpu.to_device(np.zeros(256, F))
+    # tiling: an input below 2 * window - 1, 5 dimensions, in place
+    assert lib.nnf_hip_max_subsampling_tiling_forward(s, e.data_ptr(), d.data_ptr(), 1, 1, 2, u32([8, 4]), u32([2, 3]), 0) == capi.E_INVAL
+    assert lib.nnf_hip_max_subsampling_tiling_forward(s, e.data_ptr(), d.data_ptr(), 1, 1, 5, u32([2] * 5), u32([1] * 5), 0) == capi.E_UNSUPPORTED
+    assert lib.nnf_hip_max_subsampling_tiling_forward(s, d.data_ptr(), d.data_ptr(), 1, 1, 2, u32([8, 8]), u32([2, 2]), 0) == capi.E_OVERLAP
+    assert lib.nnf_hip_max_subsampling_tiling_forward(s, e.data_ptr(), d.data_ptr(), 0, 1, 2, u32([8, 8]), u32([2, 2]), 0) == 0
     # max subsampling: 5 dimensions, zero stride, window larger than the input, in place
     assert lib.nnf_hip_max_subsampling_forward(s, e.data_ptr(), d.data_ptr(), 1, 1, 5, u32([2] * 5), u32([1] * 5), None, None, 1, 1, 0) == capi.E_UNSUPPORTED
     assert lib.nnf_hip_max_subsampling_forward(s, e.data_ptr(), d.data_ptr(), 1, 1, 2, u32([8, 8]), u32([2, 2]), u32([0, 2]), None, 1, 1, 0) == capi.E_INVAL
