@@ -20,7 +20,11 @@ layer { type: "MaxSubsampling" name: "pool1" input_layer_name: "relu"
 	max_subsampling_param { dimension_param { subsampling_size: 3 stride: 2 round_up: true } dimension_param { subsampling_size: 3 stride: 2 round_up: true } } }
 layer { type: "TanH" name: "tanh" input_layer_name: "pool1" tanh_param { scale: 1.7159 steepness: 0.6666 } }
 layer { type: "Absolute" name: "abs" input_layer_name: "tanh" }
-layer { type: "AverageSubsampling" name: "pool2" input_layer_name: "abs"
+layer { type: "MaxSubsampling" name: "tiles" input_layer_name: "abs"
+	max_subsampling_param { tiling: true dimension_param { subsampling_size: 2 } dimension_param { subsampling_size: 2 } } }
+layer { type: "AverageSubsampling" name: "untile" input_layer_name: "tiles"
+	average_subsampling_param { dimension_param { subsampling_size: 1 } dimension_param { subsampling_size: 1 } entry_param { subsampling_size: 4 } } }
+layer { type: "AverageSubsampling" name: "pool2" input_layer_name: "untile"
 	average_subsampling_param { dimension_param { subsampling_size: 2 } dimension_param { subsampling_size: 2 } } }
 layer { type: "PReLU" name: "prelu" input_layer_name: "pool2" prelu_param { feature_map_count: 8 } }
 layer { type: "Dropout" name: "drop" input_layer_name: "prelu" dropout_param { dropout_rate: 0.25 } }
