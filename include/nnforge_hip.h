@@ -36,6 +36,10 @@ extern "C" {
 #define NNF_HIP_EOVERLAP (-4)    /* output overlaps an input other than "out == inputs[0]"      */
 #define NNF_HIP_ETOOBIG (-5)     /* element count does not fit the kernels' index range          */
 
+/* The kernels index tensors with 32 bits: a tensor (an input, an output) of more elements than this makes
+ * an entry point return NNF_HIP_ETOOBIG. Callers that split their work into batches size them to it. */
+#define NNF_HIP_MAX_ELEMENT_COUNT 0xFFFF0000ull
+
 #define NNF_HIP_MAX_OPS 8
 #define NNF_HIP_MAX_INPUTS 4
 

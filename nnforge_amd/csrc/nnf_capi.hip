@@ -79,7 +79,7 @@ namespace nnf
 		// the fused-group kernel accepts.
 		bool flat_shape(uint64_t elem_count, uint32_t& entry_count, uint32_t& plane)
 		{
-			if (elem_count > 0xFFFF0000ull)
+			if (elem_count > NNF_HIP_MAX_ELEMENT_COUNT)
 				return false;
 			entry_count = 1;
 			plane = static_cast<uint32_t>(elem_count);
@@ -107,7 +107,7 @@ namespace nnf
 			return NNF_HIP_EALIGN;
 		if (bytes == 0)
 			return NNF_HIP_OK;
-		if (bytes / 16 > 0xFFFF0000ull)
+		if (bytes / 16 > NNF_HIP_MAX_ELEMENT_COUNT)
 			return NNF_HIP_ETOOBIG;
 		const uint32_t vectors = static_cast<uint32_t>(bytes / 16);
 		const uint32_t per_block = copy_block_size * copy_unroll;

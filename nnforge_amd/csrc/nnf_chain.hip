@@ -562,7 +562,7 @@ namespace nnf
 		const uint64_t total64 = static_cast<uint64_t>(desc->entry_count) * desc->feature_map_count * desc->neuron_count_per_feature_map;
 		if (total64 == 0)
 			return NNF_HIP_OK; // nothing to do, as the reference's loops over zero elements
-		if (total64 > 0xFFFF0000ull)
+		if (total64 > NNF_HIP_MAX_ELEMENT_COUNT)
 			return NNF_HIP_ETOOBIG;
 		const size_t bytes = static_cast<size_t>(total64) * sizeof(float);
 

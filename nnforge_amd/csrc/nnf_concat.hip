@@ -104,7 +104,7 @@ namespace nnf
 		const uint64_t output_total = output_length * entry_count;
 		if (output_total == 0)
 			return NNF_HIP_OK;
-		if (output_total > 0xFFFF0000ull)
+		if (output_total > NNF_HIP_MAX_ELEMENT_COUNT)
 			return NNF_HIP_ETOOBIG;
 		for(uint32_t i = 0; i < input_count; ++i)
 		{

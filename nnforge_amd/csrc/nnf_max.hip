@@ -686,7 +686,7 @@ namespace nnf
 		const uint64_t output_total = static_cast<uint64_t>(output_entry_count) * out_fm * out_plane;
 		if (output_total == 0)
 			return NNF_HIP_OK;
-		if ((input_total > 0xFFFF0000ull) || (output_total > 0xFFFF0000ull))
+		if ((input_total > NNF_HIP_MAX_ELEMENT_COUNT) || (output_total > NNF_HIP_MAX_ELEMENT_COUNT))
 			return NNF_HIP_ETOOBIG;
 		if (overlap(output, output_total * sizeof(float), input, input_total * sizeof(float)))
 			return NNF_HIP_EOVERLAP;
@@ -762,7 +762,7 @@ namespace nnf
 		const uint64_t output_total = static_cast<uint64_t>(input_entry_count) * tile_count * feature_map_count * out_plane;
 		if (output_total == 0)
 			return NNF_HIP_OK;
-		if ((input_total > 0xFFFF0000ull) || (output_total > 0xFFFF0000ull))
+		if ((input_total > NNF_HIP_MAX_ELEMENT_COUNT) || (output_total > NNF_HIP_MAX_ELEMENT_COUNT))
 			return NNF_HIP_ETOOBIG;
 		if (overlap(output, output_total * sizeof(float), input, input_total * sizeof(float)))
 			return NNF_HIP_EOVERLAP;
@@ -824,7 +824,7 @@ namespace nnf
 		const uint64_t output_total = static_cast<uint64_t>(output_entry_count) * out_fm * out_plane;
 		if (output_total == 0)
 			return NNF_HIP_OK;
-		if ((input_total > 0xFFFF0000ull) || (output_total > 0xFFFF0000ull))
+		if ((input_total > NNF_HIP_MAX_ELEMENT_COUNT) || (output_total > NNF_HIP_MAX_ELEMENT_COUNT))
 			return NNF_HIP_ETOOBIG;
 		if (overlap(output, output_total * sizeof(float), input, input_total * sizeof(float)))
 			return NNF_HIP_EOVERLAP;
@@ -867,7 +867,7 @@ namespace nnf
 		const uint64_t input_total = output_total * feature_map_subsampling_size;
 		if (output_total == 0)
 			return NNF_HIP_OK;
-		if (input_total > 0xFFFF0000ull)
+		if (input_total > NNF_HIP_MAX_ELEMENT_COUNT)
 			return NNF_HIP_ETOOBIG;
 		if (overlap(output, output_total * sizeof(float), input, input_total * sizeof(float)))
 			return NNF_HIP_EOVERLAP;

@@ -290,7 +290,7 @@ namespace nnf
 		const uint64_t input_total = static_cast<uint64_t>(entry_count) * feature_map_count * input_width * input_height;
 		if (input_total == 0)
 			return NNF_HIP_OK;
-		if (input_total > 0xFFFF0000ull)
+		if (input_total > NNF_HIP_MAX_ELEMENT_COUNT)
 			return NNF_HIP_ETOOBIG;
 		const uint32_t plane_count = entry_count * feature_map_count;
 		const uint32_t output_count = plane_count * output_width * output_height;

@@ -600,7 +600,7 @@ namespace nnf
 		const uint64_t total64 = static_cast<uint64_t>(entry_count) * feature_map_count * neuron_count_per_feature_map;
 		if (total64 == 0)
 			return NNF_HIP_OK;
-		if (total64 > 0xFFFF0000ull)
+		if (total64 > NNF_HIP_MAX_ELEMENT_COUNT)
 			return NNF_HIP_ETOOBIG;
 		if (!is_aligned16(output) || !is_aligned16(input))
 			return NNF_HIP_EALIGN;

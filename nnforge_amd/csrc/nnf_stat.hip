@@ -262,7 +262,7 @@ namespace nnf
 		if (!is_aligned16(device_stats) || !is_aligned16(input) || !is_aligned16(workspace))
 			return NNF_HIP_EALIGN;
 		const uint64_t total = static_cast<uint64_t>(entry_count) * feature_map_count * neuron_count_per_feature_map;
-		if ((total > 0xFFFF0000ull) || (feature_map_count > 65535u))
+		if ((total > NNF_HIP_MAX_ELEMENT_COUNT) || (feature_map_count > 65535u))
 			return NNF_HIP_ETOOBIG;
 		const stat_plan p = plan_runs(entry_count, feature_map_count, neuron_count_per_feature_map);
 		const size_t needed = static_cast<size_t>(p.runs) * p.segments * feature_map_count * sizeof(nnf_hip_running_stat);

@@ -533,6 +533,14 @@ namespace nnforge
 				throw neural_network_exception("Insufficient memory to do forward prop for even one sample");
 			const size_t fit = (budget - weight_bytes) / per_entry_bytes;
 			max_entry_count = static_cast<unsigned int>(std::min<size_t>(fit, static_cast<size_t>(std::max(1, hip_config->max_entry_count))));
+			// and no tensor of a packet may outgrow the kernels' 32-bit indices
+			size_t largest_floats_per_entry = 1;
+			for(size_t floats : p->buffer_floats_per_entry)
+				largest_floats_per_entry = std::max(largest_floats_per_entry, floats);
+			const size_t index_fit = static_cast<size_t>(NNF_HIP_MAX_ELEMENT_COUNT / largest_floats_per_entry);
+			if (index_fit == 0)
+				throw neural_network_exception("A single entry of " + std::to_string(largest_floats_per_entry) + " values in one layer is beyond the hip kernels' index range");
+			max_entry_count = static_cast<unsigned int>(std::min<size_t>(max_entry_count, index_fit));
 
 			if (debug->is_debug())
 			{

@@ -321,6 +321,20 @@ def test_neighbour_layer_configuration_rules():
         plan([S.L("Data", "x"), S.L("Dropout", "d", ["x"], dropout_rate=1.0)], {"x": (4, [8])}, ["d"])
 
 
+def test_packets_stay_within_the_kernels_index_range():
+    """Memory would allow 4096 entries of 64 x 256 x 256 values per packet; the kernels index a tensor with 32 bits
+    (NNF_HIP_MAX_ELEMENT_COUNT = 0xFFFF0000 elements), so the packet is cut to what still fits."""
+    layers = [S.L("Data", "x"), S.L("ReLU", "r", ["x"]), S.L("MaxSubsampling", "p", ["r"], windows=[2, 2])]
+    rep = plan(layers, {"x": (64, [256, 256])}, ["p"])
+    assert rep["max_entry_count"] == 0xFFFF0000 // (64 * 256 * 256) == 1023
+    rep = plan(layers, {"x": (64, [16, 16])}, ["p"])
+    assert rep["max_entry_count"] == 4096
+    # the largest tensor decides: here the concatenation of both inputs
+    joined = [S.L("Data", "x"), S.L("Data", "y"), S.L("Concat", "c", ["x", "y"])]
+    rep = plan(joined, {"x": (64, [256, 256]), "y": (32, [256, 256])}, ["c"])
+    assert rep["max_entry_count"] == 0xFFFF0000 // (96 * 256 * 256)
+
+
 def test_tiling_factors_scale_buffers_and_must_agree():
     """nnforge/network_schema.cpp:651-680, nnforge/forward_propagation.cpp:54-61: a layer holds (entries read) x (the
     product of the tiling factors on the way to it) entries; inputs of a layer and the output layers must agree."""
