@@ -529,9 +529,18 @@ namespace nnforge
 				for(const hip_linear_buffer_device::const_ptr& b : w.second)
 					weight_bytes += b->get_size();
 			const size_t budget = hip_config->get_max_bytes();
-			if ((per_entry_bytes == 0) || (budget <= weight_bytes) || ((budget - weight_bytes) / per_entry_bytes == 0))
+			// data and output layers have a second device buffer, for the packet whose I/O overlaps the kernels
+			std::set<int> io_buffers;
+			for(const std::string& n : data_layer_names)
+				io_buffers.insert(p->value_to_buffer.at(n));
+			for(const std::string& n : output_layer_names)
+				io_buffers.insert(p->value_to_buffer.at(n));
+			size_t device_bytes_per_entry = per_entry_bytes;
+			for(int b : io_buffers)
+				device_bytes_per_entry += p->buffer_floats_per_entry[b] * sizeof(float);
+			if ((per_entry_bytes == 0) || (budget <= weight_bytes) || ((budget - weight_bytes) / device_bytes_per_entry == 0))
 				throw neural_network_exception("Insufficient memory to do forward prop for even one sample");
-			const size_t fit = (budget - weight_bytes) / per_entry_bytes;
+			const size_t fit = (budget - weight_bytes) / device_bytes_per_entry;
 			max_entry_count = static_cast<unsigned int>(std::min<size_t>(fit, static_cast<size_t>(std::max(1, hip_config->max_entry_count))));
 			// and no tensor of a packet may outgrow the kernels' 32-bit indices
 			size_t largest_floats_per_entry = 1;

@@ -135,12 +135,13 @@ def test_plan_splits_chains_longer_than_the_kernel_takes():
 def test_plan_memory_budget():
     cfg = {"conv_main": (8, [7, 7]), "conv_shortcut": (8, [7, 7])}
     per_entry = 3 * 8 * 49 * 4
-    rep = plan(S.resnet_block(8), cfg, ["res_relu"], memory_bytes=100 * per_entry)
+    # all three buffers belong to data or output layers: each exists twice, once per packet in flight
+    rep = plan(S.resnet_block(8), cfg, ["res_relu"], memory_bytes=200 * per_entry)
     assert rep["max_entry_count"] in (89, 90)   # 0.9 of the memory (the ratio is an fp32 number)
     rep = plan(S.resnet_block(8), cfg, ["res_relu"], memory_bytes=1 << 40, max_entry_count=77)
     assert rep["max_entry_count"] == 77
     with pytest.raises(backend.BackendError, match="Insufficient memory to do forward prop for even one sample"):
-        plan(S.resnet_block(8), cfg, ["res_relu"], memory_bytes=per_entry)
+        plan(S.resnet_block(8), cfg, ["res_relu"], memory_bytes=2 * per_entry)
 
 
 def test_plan_errors():
@@ -329,6 +330,13 @@ def test_packets_stay_within_the_kernels_index_range():
     assert rep["max_entry_count"] == 0xFFFF0000 // (64 * 256 * 256) == 1023
     rep = plan(layers, {"x": (64, [16, 16])}, ["p"])
     assert rep["max_entry_count"] == 4096
+    # memory: every buffer once, those of data and output layers twice (two packets overlap their I/O with the kernels)
+    rep = plan(layers, {"x": (64, [256, 256])}, ["p"], memory_bytes=1 << 30)
+    x_bytes, p_bytes = 4 * 64 * 256 * 256, 4 * 64 * 128 * 128
+    assert rep["per_entry_bytes"] == x_bytes + p_bytes          # r works in place on x's buffer
+    assert rep["max_entry_count"] == int(0.9 * (1 << 30)) // (2 * x_bytes + 2 * p_bytes) == 23
+    with pytest.raises(backend.BackendError, match="Insufficient memory"):
+        plan(layers, {"x": (64, [256, 256])}, ["p"], memory_bytes=32 << 20)
     # the largest tensor decides: here the concatenation of both inputs
     joined = [S.L("Data", "x"), S.L("Data", "y"), S.L("Concat", "c", ["x", "y"])]
     rep = plan(joined, {"x": (64, [256, 256]), "y": (32, [256, 256])}, ["c"])
