@@ -428,6 +428,231 @@ namespace nnf
 			a.out[o] = (OP == window_op_sum) ? current * a.mult : current;
 		}
 
+		// ---- tiling in 1 or 2 dimensions, staged through LDS ---------------------------------------
+		// A workgroup stages whole planes (small ones, several) or the input rows of a band of output rows, once, and
+		// every lane then takes output positions of that range: at a position it folds the window of each of the
+		// win_w * win_h shifted grids out of LDS and stores it to that grid's output entry. The input is read from
+		// memory once (twice where bands overlap) instead of once per grid.
+		struct tiling2d_args
+		{
+			float* out;
+			const float* in;
+			uint32_t in_w, in_h, out_w, out_h, win_w, win_h;
+			uint32_t fm_count, plane_count; // planes = entries * feature maps
+			uint32_t planes;                // whole planes per workgroup; 1: bands of `rows` output rows, `bands` per plane
+			uint32_t rows, bands;
+		};
+
+		template<int OP, int WIN_W, int WIN_H>
+		__global__ void __launch_bounds__(max_block_size) tiling2d_kernel(const tiling2d_args a)
+		{
+			extern __shared__ float staged[];
+			const uint32_t win_w = (WIN_W > 0) ? WIN_W : a.win_w, win_h = (WIN_H > 0) ? WIN_H : a.win_h;
+			const uint32_t in_plane = a.in_w * a.in_h, out_plane = a.out_w * a.out_h;
+			uint32_t first_plane, planes_here, oy0, oy1;
+			if (a.planes > 1)
+			{
+				first_plane = blockIdx.x * a.planes;
+				planes_here = min(a.planes, a.plane_count - first_plane);
+				oy0 = 0;
+				oy1 = a.out_h;
+			}
+			else
+			{
+				first_plane = blockIdx.x / a.bands;
+				planes_here = 1;
+				oy0 = (blockIdx.x - first_plane * a.bands) * a.rows;
+				oy1 = min(oy0 + a.rows, a.out_h);
+			}
+			// input rows oy0 * win_h .. oy1 * win_h + win_h - 2 of every plane: the last grid's last window ends there
+			// (out_h * win_h + win_h - 1 <= in_h by the layer's output size); several planes are staged whole
+			const uint32_t first_row = oy0 * win_h;
+			const uint32_t staged_floats = (a.planes > 1) ? planes_here * in_plane : (oy1 * win_h + win_h - 1 - first_row) * a.in_w;
+			const float* src = a.in + static_cast<size_t>(first_plane) * in_plane + first_row * a.in_w;
+			#pragma unroll 8
+			for(uint32_t i = threadIdx.x; i < staged_floats; i += max_block_size)
+				staged[i] = src[i];
+			__syncthreads();
+
+			const uint32_t positions_per_plane = (oy1 - oy0) * a.out_w;
+			const uint32_t positions = planes_here * positions_per_plane;
+			const size_t grid_stride = static_cast<size_t>(a.fm_count) * out_plane; // from one output entry to the next
+			for(uint32_t pos = threadIdx.x; pos < positions; pos += max_block_size)
+			{
+				const uint32_t p = pos / positions_per_plane;
+				const uint32_t rem = pos - p * positions_per_plane;
+				const uint32_t oy = rem / a.out_w;
+				const uint32_t ox = rem - oy * a.out_w;
+				const uint32_t plane_id = first_plane + p;
+				const uint32_t entry = plane_id / a.fm_count;
+				const uint32_t fm = plane_id - entry * a.fm_count;
+				const float* corner = staged + p * in_plane + oy * win_h * a.in_w + ox * win_w;
+				float* dst = a.out + (static_cast<size_t>(entry) * (win_w * win_h) * a.fm_count + fm) * out_plane + (oy0 + oy) * a.out_w + ox;
+				// grids in the order of the window scan: x shift fastest
+				#pragma unroll
+				for(uint32_t sy = 0; sy < win_h; ++sy)
+				{
+					#pragma unroll
+					for(uint32_t sx = 0; sx < win_w; ++sx)
+					{
+						float current = window_fold_start<OP>();
+						#pragma unroll
+						for(uint32_t y = 0; y < win_h; ++y)
+						{
+							#pragma unroll
+							for(uint32_t x = 0; x < win_w; ++x)
+								current = window_fold<OP>(current, corner[(sy + y) * a.in_w + sx + x]);
+						}
+						*dst = current;
+						dst += grid_stride;
+					}
+				}
+			}
+		}
+
+		// -> true when the staged kernel took the work
+		bool launch_tiling2d(hipStream_t stream, bool is_min, float* output, const float* input, uint32_t plane_count, uint32_t fm_count,
+			uint32_t in_w, uint32_t in_h, uint32_t out_w, uint32_t out_h, uint32_t win_w, uint32_t win_h)
+		{
+			constexpr uint32_t lds_floats_max = 15 * 1024;
+			tiling2d_args a = {};
+			a.out = output;
+			a.in = input;
+			a.in_w = in_w; a.in_h = in_h; a.out_w = out_w; a.out_h = out_h; a.win_w = win_w; a.win_h = win_h;
+			a.fm_count = fm_count;
+			a.plane_count = plane_count;
+			const uint64_t in_plane = static_cast<uint64_t>(in_w) * in_h;
+			const uint64_t band_floats_min = static_cast<uint64_t>(2 * win_h - 1) * in_w; // one output row
+			if (band_floats_min > lds_floats_max)
+				return false;
+			uint32_t grid, staged_floats;
+			if (in_plane * 2 <= lds_floats_max)
+			{
+				// small planes: enough of them for four positions per lane, as far as LDS holds them
+				const uint32_t wanted = (4 * max_block_size + out_w * out_h - 1) / (out_w * out_h);
+				a.planes = max(1u, min(min(wanted, static_cast<uint32_t>(lds_floats_max / in_plane)), plane_count));
+			}
+			else
+				a.planes = 1;
+			if (a.planes > 1)
+			{
+				a.rows = out_h;
+				a.bands = 1;
+				grid = (plane_count + a.planes - 1) / a.planes;
+				staged_floats = a.planes * static_cast<uint32_t>(in_plane);
+			}
+			else
+			{
+				// (rows * win_h + win_h - 1) * in_w <= lds_floats_max
+				a.rows = min(out_h, static_cast<uint32_t>((lds_floats_max / in_w - (win_h - 1)) / win_h));
+				a.bands = (out_h + a.rows - 1) / a.rows;
+				// few planes: more, lower bands (not below 4 output rows) until about 1024 workgroups share the work
+				const uint32_t bands_wanted = (1024 + plane_count - 1) / plane_count;
+				a.bands = max(a.bands, min(bands_wanted, max(1u, out_h / 4)));
+				a.rows = (out_h + a.bands - 1) / a.bands; // bands of equal height
+				a.bands = (out_h + a.rows - 1) / a.rows;
+				grid = plane_count * a.bands;
+				staged_floats = (a.rows * win_h + win_h - 1) * in_w;
+			}
+			const size_t lds_bytes = static_cast<size_t>(staged_floats) * sizeof(float);
+			const dim3 g(grid), b(max_block_size);
+			const bool w2 = (win_w == 2) && (win_h == 2), w3 = (win_w == 3) && (win_h == 3);
+			if (is_min)
+			{
+				if (w2) hipLaunchKernelGGL((tiling2d_kernel<window_op_min, 2, 2>), g, b, lds_bytes, stream, a);
+				else if (w3) hipLaunchKernelGGL((tiling2d_kernel<window_op_min, 3, 3>), g, b, lds_bytes, stream, a);
+				else hipLaunchKernelGGL((tiling2d_kernel<window_op_min, 0, 0>), g, b, lds_bytes, stream, a);
+			}
+			else
+			{
+				if (w2) hipLaunchKernelGGL((tiling2d_kernel<window_op_max, 2, 2>), g, b, lds_bytes, stream, a);
+				else if (w3) hipLaunchKernelGGL((tiling2d_kernel<window_op_max, 3, 3>), g, b, lds_bytes, stream, a);
+				else hipLaunchKernelGGL((tiling2d_kernel<window_op_max, 0, 0>), g, b, lds_bytes, stream, a);
+			}
+			return true;
+		}
+
+		// ---- windows over feature maps and entries only: whole rows folded with float4 ------------
+		// Spatial windows of 1: output row r (a plane, or a whole entry when there is no window over feature maps)
+		// is the fold of the input rows (entry e * entry_window + en, row fo * fm_window + fm), feature maps inside
+		// entries as in the reference's scan. Rows are multiples of 4 floats; a lane folds one float4 of a row.
+		struct window_rows_args
+		{
+			float* out;
+			const float* in;
+			uint32_t row_vectors;      // float4s per row
+			uint32_t out_rows;         // output entries * rows_per_out_entry
+			uint32_t rows_per_out_entry, rows_per_in_entry;
+			uint32_t fm_window, entry_window;
+			float mult;
+		};
+
+		template<int OP>
+		__global__ void __launch_bounds__(max_block_size) window_rows_kernel(const window_rows_args a)
+		{
+			const uint32_t j = blockIdx.x * max_block_size + threadIdx.x;
+			if (j >= a.row_vectors)
+				return;
+			for(uint32_t r = blockIdx.y; r < a.out_rows; r += gridDim.y)
+			{
+				const uint32_t entry = r / a.rows_per_out_entry;
+				const uint32_t row = r - entry * a.rows_per_out_entry;
+				const floatx4* src = reinterpret_cast<const floatx4*>(a.in)
+					+ (static_cast<size_t>(entry) * a.entry_window * a.rows_per_in_entry + static_cast<size_t>(row) * a.fm_window) * a.row_vectors + j;
+				const float start = window_fold_start<OP>();
+				floatx4 current = { start, start, start, start };
+				for(uint32_t en = 0; en < a.entry_window; ++en)
+				{
+					for(uint32_t fm = 0; fm < a.fm_window; ++fm)
+					{
+						const floatx4 v = load_stream(src + (static_cast<size_t>(en) * a.rows_per_in_entry + fm) * a.row_vectors);
+						current.x = window_fold<OP>(current.x, v.x);
+						current.y = window_fold<OP>(current.y, v.y);
+						current.z = window_fold<OP>(current.z, v.z);
+						current.w = window_fold<OP>(current.w, v.w);
+					}
+				}
+				if (OP == window_op_sum)
+				{
+					current.x *= a.mult;
+					current.y *= a.mult;
+					current.z *= a.mult;
+					current.w *= a.mult;
+				}
+				store_stream(reinterpret_cast<floatx4*>(a.out) + static_cast<size_t>(r) * a.row_vectors + j, current);
+			}
+		}
+
+		// rows shorter than this leave most lanes of a workgroup idle: the one-lane-per-output kernel does better
+		constexpr uint32_t window_rows_min_vectors = 64;
+
+		// -> true when the rows kernel took the work
+		bool launch_window_rows(hipStream_t stream, int op, float mult, float* output, const float* input, uint32_t output_entry_count,
+			uint32_t in_fm, uint32_t out_fm, uint64_t plane, uint32_t fm_window, uint32_t entry_window)
+		{
+			window_rows_args a = {};
+			const uint64_t row_floats = (fm_window == 1) ? static_cast<uint64_t>(in_fm) * plane : plane;
+			if ((row_floats % 4 != 0) || (row_floats / 4 < window_rows_min_vectors))
+				return false;
+			a.out = output;
+			a.in = input;
+			a.row_vectors = static_cast<uint32_t>(row_floats / 4);
+			a.rows_per_out_entry = (fm_window == 1) ? 1 : out_fm;
+			a.rows_per_in_entry = (fm_window == 1) ? 1 : in_fm;
+			a.out_rows = output_entry_count * a.rows_per_out_entry;
+			a.fm_window = fm_window;
+			a.entry_window = entry_window;
+			a.mult = mult;
+			const dim3 grid((a.row_vectors + max_block_size - 1) / max_block_size, min(a.out_rows, 65535u));
+			if (op == window_op_sum)
+				hipLaunchKernelGGL(window_rows_kernel<window_op_sum>, grid, dim3(max_block_size), 0, stream, a);
+			else if (op == window_op_min)
+				hipLaunchKernelGGL(window_rows_kernel<window_op_min>, grid, dim3(max_block_size), 0, stream, a);
+			else
+				hipLaunchKernelGGL(window_rows_kernel<window_op_max>, grid, dim3(max_block_size), 0, stream, a);
+			return true;
+		}
+
 		// ---- maxout ------------------------------------------------------------------------------
 		// Per entry the output is `group` floats and output j folds the inputs j, j + group, j + 2*group, ...
 		// std::max(new_val, current) = (new_val < current) ? current : new_val
@@ -657,6 +882,7 @@ namespace nnf
 		window_nd_args nd = {};
 		uint64_t in_plane = 1, out_plane = 1;
 		bool round_up_anywhere = false;
+		bool identity_in_plane = true; // windows of one element at every position
 		for(uint32_t d = 0; d < max_dims; ++d)
 		{
 			nd.in_size[d] = nd.out_size[d] = nd.window[d] = nd.stride[d] = 1;
@@ -664,6 +890,7 @@ namespace nnf
 				continue;
 			const uint32_t size = input_sizes[d], window = subsampling_sizes[d];
 			const uint32_t stride = (strides != nullptr) ? strides[d] : window;
+			identity_in_plane = identity_in_plane && (window == 1) && (stride == 1);
 			const bool round_up = (round_ups != nullptr) && (round_ups[d] != 0);
 			if ((size == 0) || (window == 0) || (stride == 0))
 				return NNF_HIP_EINVAL;
@@ -705,6 +932,11 @@ namespace nnf
 			return NNF_HIP_EUNSUPPORTED; // only the LDS-staged kernel applies a prologue
 		if (plan_only)
 			return NNF_HIP_OK;
+
+		// windows over feature maps and entries only
+		if (identity_in_plane && launch_window_rows(stream, is_min ? window_op_min : window_op_max, 0.0f, output, input, output_entry_count,
+			input_feature_map_count, out_fm, in_plane, feature_map_subsampling_size, entry_subsampling_size))
+			return launch_status();
 
 		nd.out = output;
 		nd.in = input;
@@ -766,6 +998,9 @@ namespace nnf
 			return NNF_HIP_ETOOBIG;
 		if (overlap(output, output_total * sizeof(float), input, input_total * sizeof(float)))
 			return NNF_HIP_EOVERLAP;
+		if ((dimension_count <= 2) && launch_tiling2d(stream, is_min != 0, output, input, input_entry_count * feature_map_count, feature_map_count,
+			nd.in_size[0], nd.in_size[1], nd.out_size[0], nd.out_size[1], nd.window[0], nd.window[1]))
+			return launch_status();
 		nd.out = output;
 		nd.in = input;
 		nd.output_count = static_cast<uint32_t>(output_total);
@@ -837,6 +1072,13 @@ namespace nnf
 		nd.entry_window = entry_subsampling_size;
 		nd.in_plane = static_cast<uint32_t>(in_plane);
 		nd.mult = mult;
+		// windows over feature maps and entries only
+		bool identity_in_plane = true;
+		for(uint32_t d = 0; d < max_dims; ++d)
+			identity_in_plane = identity_in_plane && (nd.window[d] == 1);
+		if (identity_in_plane && launch_window_rows(stream, window_op_sum, mult, output, input, output_entry_count,
+			input_feature_map_count, out_fm, in_plane, feature_map_subsampling_size, entry_subsampling_size))
+			return launch_status();
 		const dim3 grid((nd.output_count + max_block_size - 1) / max_block_size);
 		hipLaunchKernelGGL(window_nd_kernel<window_op_sum>, grid, dim3(max_block_size), 0, stream, nd);
 		return launch_status();

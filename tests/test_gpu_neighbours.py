@@ -177,6 +177,11 @@ TILING_CASES = [
     ((1, 2, 3, 5, 4, 7), [2, 2, 2, 1]),   # 4-D, a window of 1 in one dimension
     ((4, 8, 28, 28), [2, 2]),
     ((2, 1, 3, 3), [1, 1]),               # one tile: plain copy
+    ((7, 37, 6, 5), [2, 2]),              # 259 small planes: 256 in the first workgroup, 3 in the second
+    ((1, 2, 200, 300), [3, 2]),           # bands of a large plane
+    ((2, 3, 112, 112), [3, 3]),           # a whole plane per workgroup
+    ((2, 1, 5, 20000), [2, 2]),           # rows too wide to stage: one lane per output
+    ((3, 2, 40000), [3]),                 # 1-D, wide
 ]
 
 
@@ -200,6 +205,31 @@ def test_max_subsampling_with_tiling(gpu, shape, windows, is_min):
     tile0 = got.reshape((shape[0], -1) + got.shape[1:])[:, 0]
     cut = (slice(None), slice(None)) + tuple(slice(0, n) for n in got.shape[2:])
     assert T.bit_mismatches(tile0, plain[cut]) == 0
+
+
+@pytest.mark.parametrize("is_min", [False, True])
+@pytest.mark.parametrize("shape,fm,en", [
+    ((8, 6, 16, 16, 2), 1, 4),       # 3-D so that the staged 2-D kernel stays out: entries folded as rows of float4
+    ((4, 13, 16, 20, 1), 3, 2),      # planes as rows, a feature map left over
+    ((6, 12, 9, 10, 1), 1, 3),       # planes of 90 values, entries of 1080
+    ((6, 12, 9, 10, 1), 4, 1),       # planes of 90 values with a window over feature maps: one lane per output
+    ((6, 12, 16, 16), 2, 3),         # 2-D
+])
+def test_max_subsampling_over_feature_maps_and_entries_only(gpu, shape, fm, en, is_min):
+    x = spiced(T.rng(67, sum(shape) + fm), shape)
+    ones = [1] * (len(shape) - 2)
+    got = run_max_subsampling(gpu, x, ones, None, None, fm=fm, en=en, is_min=is_min)
+    want = oracle.max_subsampling(x, ones, feature_map_window=fm, entry_window=en, is_min=is_min)
+    assert got.shape == want.shape
+    assert T.bit_mismatches(got, want) == 0
+    # the same thing said with numpy: fold over the entry and feature-map axes
+    c_out = shape[1] // fm
+    folded = x[:, :c_out * fm].reshape((shape[0] // en, en, c_out, fm) + shape[2:])
+    with np.errstate(invalid="ignore"):
+        # the fold starts at -+1.0e37F, which bounds the result
+        ref = np.minimum(folded.min(axis=(1, 3)), F(1.0e37)) if is_min else np.maximum(folded.max(axis=(1, 3)), F(-1.0e37))
+    plain = ~np.isnan(ref)    # windows without NaN (the reference's fold skips NaN, numpy's does not)
+    assert np.array_equal(got[plain], ref[plain])
 
 
 def test_neighbour_entry_points_reject_bad_arguments(gpu):

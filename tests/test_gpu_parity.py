@@ -582,6 +582,11 @@ def run_pool_nd(gpu, x, windows, fm_window=1, entry_window=1, mult=1.0, expect=0
     ((4, 4, 3, 4, 5, 6), [2, 2, 2, 3], 2, 2),       # 4-D with feature-map and entry windows
     ((2, 8, 9), [3], 4, 1),                         # 1-D with feature-map windows
     ((3, 5, 1, 1), [1, 1], 5, 3),                   # pure feature-map / entry averaging
+    ((8, 6, 16, 16), [1, 1], 1, 4),                 # windows over entries only: whole entries folded as rows of float4
+    ((4, 13, 16, 20), [1, 1], 3, 2),                # planes as rows, a feature map left over
+    ((6, 12, 9, 10), [1, 1], 1, 3),                 # planes of 90 values, entries of 1080: rows of float4 all the same
+    ((6, 12, 9, 10), [1, 1], 4, 1),                 # ... but not with a window over feature maps: one lane per output
+    ((2, 4, 4, 4, 4, 4), [1, 1, 1, 1], 2, 2),       # 4-D, windows of 1
 ])
 def test_average_subsampling_in_the_full_form(gpu, shape, windows, fm_window, entry_window):
     x = T.normal(T.rng(17, sum(shape) + fm_window), shape)
