@@ -39,6 +39,8 @@ MEASURED_TRAFFIC_BYTES = {
     "config2": 1233228800,  # algorithmic 1,233,130,496
     "config3": 205650944,   # algorithmic 205,529,088
     "config1": 2117540,     # algorithmic 2,048,000 (profiles/softmax_and_resnet50_stack.md)
+    "max_subsampling_tiling": 402617602,  # algorithmic 403,767,296 (profiles/tiling_and_entry_window_kernels.md)
+    "entry_window": 256931085,            # algorithmic 256,901,120
     "config4": 124914115,   # average over the 51 launches of a step: 6,370,619,861 per step, algorithmic 6,359,339,008
 }
 
@@ -356,6 +358,45 @@ def bench_maxout(runner, steps, warmup, n=64, c_out=256, plane=14 * 14, k=2):
                         {"buffer_sets": sets})
 
 
+def bench_max_subsampling_tiling(runner, steps, warmup, n=64, c=64, size=112):
+    """Max subsampling with tiling, 2x2 windows: four output entries of 55x55 per input entry of 112x112."""
+    out_size = (size - 1) // 2
+    in_count, out_count = n * c * size * size, 4 * n * c * out_size * out_size
+    sets = rotation_sets(4 * (in_count + out_count))
+    ins = [runner.randn(in_count) for _ in range(sets)]
+    outs = [runner.empty(out_count) for _ in range(sets)]
+    dims, win = _u32([size, size]), _u32([2, 2])
+    fn, stream = runner.lib.nnf_hip_max_subsampling_tiling_forward, runner.stream
+
+    def launch(i):
+        rc = fn(stream, outs[i % sets].data_ptr(), ins[i % sets].data_ptr(), n, c, 2, dims, win, 0)
+        if rc != 0:
+            raise RuntimeError(runner.capi.error_string(rc))
+
+    wall, ev = runner.time_steps(launch, steps, warmup)
+    return result_entry("max_subsampling with tiling 2x2, N=%d C=%d %dx%d -> %d entries of %dx%d" % (n, c, size, size, 4 * n, out_size, out_size),
+                        4 * (in_count + out_count), out_count, wall, ev, 1, {"buffer_sets": sets})
+
+
+def bench_entry_window(runner, steps, warmup, n=64, c=256, plane=56 * 56, window=4):
+    """Average over windows of 4 entries (what folds the entries of a tiling layer again), spatial windows of 1."""
+    in_count, out_count = n * c * plane, n // window * c * plane
+    sets = rotation_sets(4 * (in_count + out_count))
+    ins = [runner.randn(in_count) for _ in range(sets)]
+    outs = [runner.empty(out_count) for _ in range(sets)]
+    dims, win = _u32([plane]), _u32([1])
+    fn, stream = runner.lib.nnf_hip_average_subsampling_nd_forward, runner.stream
+
+    def launch(i):
+        rc = fn(stream, outs[i % sets].data_ptr(), ins[i % sets].data_ptr(), n // window, c, 1, dims, win, 1, window, 1.0 / window)
+        if rc != 0:
+            raise RuntimeError(runner.capi.error_string(rc))
+
+    wall, ev = runner.time_steps(launch, steps, warmup)
+    return result_entry("average_subsampling over %d entries, N=%d C=%d 56x56" % (window, n, c), 4 * (in_count + out_count), out_count, wall, ev, 1,
+                        {"buffer_sets": sets})
+
+
 def bench_feature_map_stat(runner, steps, warmup, n=128, c=256, plane=56 * 56):
     """Per-feature-map statistics of a batch norm input of config 2's shape: read once, 32 bytes per feature map written."""
     total = n * c * plane
@@ -580,7 +621,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=400)
     ap.add_argument("--warmup", type=int, default=40)
-    ap.add_argument("--workload", default="config0", choices=["config0", "config1", "config2", "config3", "config4", "copy", "max_subsampling", "bn_relu_max_subsampling", "concat", "maxout", "feature_map_stat"],
+    ap.add_argument("--workload", default="config0", choices=["config0", "config1", "config2", "config3", "config4", "copy", "max_subsampling", "bn_relu_max_subsampling", "max_subsampling_tiling",
+                             "entry_window", "concat", "maxout", "feature_map_stat"],
                     help="'copy' times the plain copy kernel (profiler-counter calibration and bandwidth yardstick)")
     ap.add_argument("--only", action="store_true", help="time only the chosen workload (no per_config survey, no CPU baseline)")
     args = ap.parse_args()
@@ -611,6 +653,10 @@ def main():
             return bench_max_subsampling(runner, steps, warmup)
         if name == "bn_relu_max_subsampling":
             return bench_bn_relu_max_subsampling(runner, steps, warmup)
+        if name == "max_subsampling_tiling":
+            return bench_max_subsampling_tiling(runner, steps, warmup)
+        if name == "entry_window":
+            return bench_entry_window(runner, steps, warmup)
         if name == "concat":
             return bench_concat(runner, steps, warmup)
         if name == "maxout":
@@ -629,7 +675,7 @@ def main():
                 per_config[name] = run(name, *side_steps[name])
         per_config["copy_kernel"] = bench_copy(runner, 40, 5)
         # the neighbouring layers of the same chains
-        for name, (k, wu) in (("max_subsampling", (40, 5)), ("bn_relu_max_subsampling", (40, 5)), ("concat", (100, 10)), ("maxout", (100, 10)), ("feature_map_stat", (20, 3))):
+        for name, (k, wu) in (("max_subsampling", (40, 5)), ("bn_relu_max_subsampling", (40, 5)), ("max_subsampling_tiling", (40, 5)), ("entry_window", (40, 5)), ("concat", (100, 10)), ("maxout", (100, 10)), ("feature_map_stat", (20, 3))):
             if name not in per_config:
                 per_config[name] = run(name, k, wu)
         if args.workload == "config0":
@@ -665,6 +711,7 @@ def main():
             "frac": achieved / HBM_PEAK_GBPS,
             "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
             "kernel": {"config1": "nnf::softmax_rows_kernel", "copy": "nnf::copy_kernel_impl", "max_subsampling": "nnf::max_window2d_kernel", "bn_relu_max_subsampling": "nnf::max_window2d_prologue_kernel",
+                       "max_subsampling_tiling": "nnf::tiling2d_kernel", "entry_window": "nnf::window_rows_kernel",
                        "concat": "nnf::concat_kernel", "maxout": "nnf::maxout_vec4_kernel",
                        "feature_map_stat": "nnf::stat_runs_kernel"}.get(args.workload, "nnf::chain_kernel"),
             "algorithmic_bytes_per_launch": main_entry["algorithmic_bytes_per_step"] / launches,
