@@ -111,3 +111,27 @@ def test_softmax_and_global_average_stay_fast(gpu):
     us = time_launches(gpu, lambda i: gpu.lib.nnf_hip_average_subsampling_forward(gpu.stream, sums.data_ptr(), planes.data_ptr(), 64, 2048, 7, 7, 7, 7, 1.0 / 49.0),
                        reps=100, warmup=10)
     assert us < 17.0, "the 7x7 global average takes %.1f us per launch (about 8.3 us expected)" % us
+
+
+def test_tiling_and_entry_windows_stay_on_their_own_kernels(gpu):
+    """Both have a general one-lane-per-output kernel to fall back on that is 2.5 to 3.5 times slower."""
+    n, c, size = 64, 64, 112
+    sets = 2
+    ins = buffers(gpu, n * c * size * size, sets)
+    outs = [gpu.torch.empty(4 * n * c * 55 * 55, dtype=gpu.torch.float32, device=gpu.device) for _ in range(sets)]
+
+    def tiling(i):
+        rc = gpu.lib.nnf_hip_max_subsampling_tiling_forward(gpu.stream, outs[i % sets].data_ptr(), ins[i % sets].data_ptr(), n, c, 2,
+                                                            u32([size, size]), u32([2, 2]), 0)
+        assert rc == 0, capi.error_string(rc)
+
+    us = time_launches(gpu, tiling, reps=30, warmup=3)
+    assert us < 180.0, "max subsampling with tiling takes %.1f us per launch (about 89 us expected)" % us
+
+    def entry_window(i):
+        rc = gpu.lib.nnf_hip_average_subsampling_nd_forward(gpu.stream, outs[i % sets].data_ptr(), ins[i % sets].data_ptr(), n // 4, c, 1,
+                                                            u32([size * size]), u32([1]), 1, 4, 0.25)
+        assert rc == 0, capi.error_string(rc)
+
+    us = time_launches(gpu, entry_window, reps=30, warmup=3)
+    assert us < 86.0, "the average over 4 entries takes %.1f us per launch (about 43 us expected)" % us
