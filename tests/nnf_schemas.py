@@ -161,12 +161,15 @@ def inception_like(c=8):
     ]
 
 
-def random_network(gen, layer_count=14, c=6, size=12):
+def random_network(gen, layer_count=14, c=6, size=12, with_entry_factors=False):
     """A random DAG of the layer types the backend runs: chains of element-wise layers, Adds and Concats of values of
-    equal shape, Maxout, max / min / average pooling, with some values consumed more than once.
+    equal shape, Maxout, max / min / average pooling, with some values consumed more than once. with_entry_factors:
+    also max subsampling with tiling and windows over entries, so that values hold different numbers of entries per
+    entry read (layers with several inputs then only join values that agree on it, and so do the outputs).
     -> (layers, {value name: (feature maps, [w, h])}, output names)."""
     layers = [L("Data", "in0"), L("Data", "in1")]
     shapes = {"in0": (c, [size, size]), "in1": (c, [size, size])}
+    factors = {"in0": 1, "in1": 1}   # entries per entry read
     names = ["in0", "in1"]
     unary = ["BatchNorm", "ReLU", "PReLU", "ELU", "Sigmoid", "TanH", "Absolute", "Dropout"]
     for i in range(layer_count):
@@ -175,9 +178,20 @@ def random_network(gen, layer_count=14, c=6, size=12):
         src = names[-1] if gen.random() < 0.65 else names[int(gen.integers(0, len(names)))]
         fm, dims = shapes[src]
         roll = gen.random()
-        same_shape = [n for n in names if shapes[n] == shapes[src] and n != src]
-        same_plane = [n for n in names if shapes[n][1] == dims and n != src]
-        if roll < 0.50:
+        same_shape = [n for n in names if shapes[n] == shapes[src] and factors[n] == factors[src] and n != src]
+        same_plane = [n for n in names if shapes[n][1] == dims and factors[n] == factors[src] and n != src]
+        factors[name] = factors[src]
+        if with_entry_factors and roll < 0.22 and min(dims) >= 5 and factors[src] == 1:
+            layers.append(L("MaxSubsampling", name, [src], windows=[2, 2], tiling=True, **({"function": "MIN"} if gen.random() < 0.3 else {})))
+            shapes[name] = (fm, [(d - 1) // 2 for d in dims])
+            factors[name] = 4
+        elif with_entry_factors and roll < 0.30 and factors[src] > 1:
+            window = 2 if (factors[src] == 4 and gen.random() < 0.5) else factors[src]
+            kind = "AverageSubsampling" if gen.random() < 0.5 else "MaxSubsampling"
+            layers.append(L(kind, name, [src], windows=[1, 1], entry_window=window))
+            shapes[name] = (fm, dims)
+            factors[name] = factors[src] // window
+        elif roll < 0.50:
             t = unary[int(gen.integers(0, len(unary)))]
             params = {}
             if t in ("BatchNorm", "PReLU"):
@@ -222,5 +236,8 @@ def random_network(gen, layer_count=14, c=6, size=12):
     extra = [n for n in names[2:] if n in consumed]
     if extra:
         outputs.append(extra[int(gen.integers(0, len(extra)))])    # and one that is read as well
+    if with_entry_factors:
+        # the outputs must agree on the number of entries: those of the last one's kind
+        outputs = [n for n in outputs if factors[n] == factors[outputs[-1]]]
     return layers, shapes, outputs
 

@@ -375,10 +375,11 @@ def test_tiling_factors_scale_buffers_and_must_agree():
     assert backend.rewrite_schema(once) == once
 
 
-@pytest.mark.parametrize("seed", range(30))
+@pytest.mark.parametrize("seed", list(range(30)) + [-s for s in range(1, 13)])
 def test_plan_of_random_networks_keeps_every_layer_once_and_in_order(seed):
-    gen = T.rng(70, seed)
-    layers, shapes, outputs = S.random_network(gen)
+    # negative seeds: networks with tiling layers and windows over entries
+    gen = T.rng(70 if seed >= 0 else 71, abs(seed))
+    layers, shapes, outputs = S.random_network(gen, with_entry_factors=seed < 0)
     configs = {"in0": shapes["in0"], "in1": shapes["in1"]}
     executed = [l["name"] for l in layers if l["type"] != "Data"]
     needed = set()      # layers the outputs depend on (the planner drops the rest)

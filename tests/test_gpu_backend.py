@@ -213,13 +213,14 @@ def test_groups_folded_into_the_subsampling_layers_behind_them(fuse, size):
         assert len(names) == 8
 
 
-@pytest.mark.parametrize("seed", range(12))
+@pytest.mark.parametrize("seed", list(range(12)) + [-s for s in range(1, 13)])
 def test_random_networks_equal_the_oracle_layer_by_layer(seed):
     """Random DAGs of every layer type the backend runs (the generator of the planner tests), in packets, with
     fusion and buffer sharing on: every output equals the oracle run layer by layer, bit for bit; the same
-    network without fusion and with dedicated buffers gives the same bits."""
-    gen = T.rng(70, seed)
-    layers, shapes, outputs = S.random_network(gen)
+    network without fusion and with dedicated buffers gives the same bits. Negative seeds: networks with tiling
+    layers and windows over entries, whose values hold different numbers of entries."""
+    gen = T.rng(70 if seed >= 0 else 71, abs(seed))
+    layers, shapes, outputs = S.random_network(gen, with_entry_factors=seed < 0)
     weights = S.make_weights(layers, gen)
     n = 7
     inputs = {k: T.normal(gen, (n, shapes[k][0]) + tuple(shapes[k][1][::-1]), 1.5) for k in ("in0", "in1")}
