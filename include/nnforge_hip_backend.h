@@ -71,6 +71,34 @@ NNF_BACKEND_API int nnf_backend_run_schema(
 /* Statistics of one layer's output over entry_count entries (forward_propagation::run into a
  * stat_data_bunch_writer): minimum, maximum, average and standard deviation per feature map, each
  * array feature_map_count floats long. */
+/* A data set file of nnForge (".dt": nnforge/structured_data_stream_reader.cpp:28-61) and the layer it belongs to. */
+typedef struct nnf_backend_dataset_file
+{
+	const char* layer_name;
+	const char* path;
+} nnf_backend_dataset_file;
+
+/* Inference from data set files to data set files, one network, the way toolset::run_inference does it in its
+ * dump mode (nnforge/toolset.cpp:551-655): a file per data layer goes in through structured_data_bunch_stream_reader
+ * (a data layer named dataset_value reads the constant 1), the outputs are collected by
+ * neuron_value_set_data_bunch_writer, every compact_samples consecutive entries of an output are replaced by their
+ * mean (0 or 1: none; the entries a tiling layer made of one input entry), and each output layer is written to its
+ * file. The report lists the outputs, the launch plan and the run's statistics. */
+NNF_BACKEND_API int nnf_backend_run_dataset(
+	const char* schema_text,
+	const nnf_backend_weights* weights, uint32_t weights_count,
+	const nnf_backend_dataset_file* inputs, uint32_t input_count,
+	const nnf_backend_dataset_file* outputs, uint32_t output_count,
+	uint32_t compact_samples,
+	const nnf_backend_options* options,
+	char* report, size_t report_capacity);
+
+/* Host only: reads part `part` of `part_count` equal parts of a data set file through the same readers (part_count 0 or
+ * 1: the whole file), folds every compact_samples consecutive entries into their mean and writes the result as a data
+ * set file. The report holds the configuration, the entry counts and the per-neuron average of what was read. */
+NNF_BACKEND_API int nnf_backend_rewrite_dataset(const char* in_path, const char* out_path, uint32_t compact_samples,
+	uint32_t part_count, uint32_t part, char* report, size_t report_capacity);
+
 NNF_BACKEND_API int nnf_backend_layer_statistics(
 	const char* schema_text,
 	const nnf_backend_weights* weights, uint32_t weights_count,

@@ -34,6 +34,10 @@ class Options(ctypes.Structure):
                 ("profile_folder", ctypes.c_char_p), ("stat_on_host", ctypes.c_int32)]
 
 
+class DatasetFile(ctypes.Structure):
+    _fields_ = [("layer_name", ctypes.c_char_p), ("path", ctypes.c_char_p)]
+
+
 class BackendError(RuntimeError):
     def __init__(self, code, message):
         RuntimeError.__init__(self, message)
@@ -68,6 +72,11 @@ def load():
         lib.nnf_backend_update_bn_weights.argtypes = [ctypes.c_char_p, ctypes.POINTER(Weights), ctypes.c_uint32, ctypes.POINTER(Input),
                                                       ctypes.c_uint32, ctypes.c_uint32, ctypes.POINTER(Options), ctypes.c_char_p,
                                                       ctypes.c_char_p, ctypes.c_size_t]
+        lib.nnf_backend_run_dataset.argtypes = [ctypes.c_char_p, ctypes.POINTER(Weights), ctypes.c_uint32, ctypes.POINTER(DatasetFile),
+                                                ctypes.c_uint32, ctypes.POINTER(DatasetFile), ctypes.c_uint32, ctypes.c_uint32,
+                                                ctypes.POINTER(Options), ctypes.c_char_p, ctypes.c_size_t]
+        lib.nnf_backend_rewrite_dataset.argtypes = [ctypes.c_char_p, ctypes.c_char_p, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32,
+                                                    ctypes.c_char_p, ctypes.c_size_t]
         _lib = lib
     return _lib
 
@@ -249,3 +258,67 @@ def read_weights(folder, layer_name, chunk_sizes):
     if rc != 0:
         raise BackendError(rc, report.value.decode(errors="replace"))
     return chunks
+
+
+# ---- data set files (".dt") -------------------------------------------------------------------------
+
+DATASET_GUID = bytes([0x2c, 0x62, 0xe0, 0x5a, 0xc6, 0x21, 0x43, 0xb2, 0xa8, 0x2c, 0x85, 0xcd, 0x58, 0x58, 0x15, 0xd9])
+
+
+def write_dataset(path, array):
+    """array [entries][feature maps][...spatial, x last] -> nnForge's data set file: GUID, u32 feature maps, u32 dimension
+    count, u32 sizes (x first), u32 entry count, fp32 entries (nnforge/structured_data_stream_writer.cpp:26-66)."""
+    a = np.ascontiguousarray(array, dtype="<f4")
+    dims = list(a.shape[2:])[::-1]
+    with open(path, "wb") as f:
+        f.write(DATASET_GUID)
+        f.write(np.array([a.shape[1], len(dims)] + dims + [a.shape[0]], dtype="<u4").tobytes())
+        f.write(a.tobytes())
+
+
+def read_dataset(path):
+    """-> array [entries][feature maps][...spatial, x last] of a data set file."""
+    with open(path, "rb") as f:
+        raw = f.read()
+    if raw[:16] != DATASET_GUID:
+        raise ValueError("%s is not a structured data file" % path)
+    fm, dim_count = np.frombuffer(raw, dtype="<u4", count=2, offset=16)
+    dims = [int(d) for d in np.frombuffer(raw, dtype="<u4", count=int(dim_count), offset=24)]
+    offset = 24 + 4 * int(dim_count)
+    entries = int(np.frombuffer(raw, dtype="<u4", count=1, offset=offset)[0])
+    per_entry = int(fm) * int(np.prod(dims, dtype=np.int64))
+    data = np.frombuffer(raw, dtype="<f4", count=entries * per_entry, offset=offset + 4)
+    return data.reshape([entries, int(fm)] + dims[::-1]).copy()
+
+
+def _dataset_files(files, keep):
+    arr = (DatasetFile * max(1, len(files)))()
+    for i, (name, path) in enumerate(sorted(files.items())):
+        keep.extend([name.encode(), str(path).encode()])
+        arr[i].layer_name, arr[i].path = keep[-2], keep[-1]
+    return arr
+
+
+def run_dataset(schema_text, weights, input_files, output_files, compact_samples=1, **options):
+    """input_files / output_files: {layer name: path of a data set file}. Returns the parsed report."""
+    lib = load()
+    keep = []
+    w = _weights_array(weights, keep)
+    ins, outs = _dataset_files(input_files, keep), _dataset_files(output_files, keep)
+    report = ctypes.create_string_buffer(REPORT_CAPACITY)
+    opt = _options(**options)
+    rc = lib.nnf_backend_run_dataset(schema_text.encode(), w, len(weights), ins, len(input_files), outs, len(output_files), compact_samples,
+                                     ctypes.byref(opt), report, REPORT_CAPACITY)
+    if rc != 0:
+        raise BackendError(rc, report.value.decode(errors="replace"))
+    return parse_report(report.value.decode())
+
+
+def rewrite_dataset(in_path, out_path, compact_samples=1, part_count=1, part=0):
+    """Host only. Returns the report text (configuration, entry counts, per-neuron average of what was read)."""
+    lib = load()
+    report = ctypes.create_string_buffer(1 << 20)
+    rc = lib.nnf_backend_rewrite_dataset(str(in_path).encode(), str(out_path).encode(), compact_samples, part_count, part, report, 1 << 20)
+    if rc != 0:
+        raise BackendError(rc, report.value.decode(errors="replace"))
+    return report.value.decode()

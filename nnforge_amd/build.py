@@ -60,7 +60,7 @@ def build_hip_library(verbose=False):
 
 HOST_DIR = os.path.join(PACKAGE_DIR, "host")
 BACKEND_LIBRARY = os.path.join(PACKAGE_DIR, "libnnforge_hip_backend.so")
-BACKEND_SOURCES = ["core.cpp", "layers.cpp", "schema.cpp", "propagation.cpp", "hip_testers.cpp",
+BACKEND_SOURCES = ["core.cpp", "layers.cpp", "schema.cpp", "propagation.cpp", "data_streams.cpp", "hip_testers.cpp",
                    "forward_propagation_hip.cpp", "backend_capi.cpp"]
 # default symbol visibility: the C++ classes are the library's interface
 BACKEND_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wextra", "-Wno-unused-parameter"]

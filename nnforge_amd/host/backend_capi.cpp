@@ -1,6 +1,9 @@
 // C bridge over the C++ hip backend (declared in include/nnforge_hip_backend.h).
 #include "nnforge_hip_backend.h"
 #include "nnforge_hip/hip_backend.h"
+#include "nnforge_hip/data_streams.h"
+
+#include <fstream>
 
 #include <cstdio>
 #include <cstring>
@@ -182,6 +185,116 @@ extern "C"
 			out << "stat: " << st << "\n";
 			for(const std::pair<const std::string, float>& a : fp->get_last_action_seconds())
 				out << "seconds: " << a.first << " " << a.second << "\n";
+		}, report, report_capacity);
+	}
+
+	int nnf_backend_run_dataset(
+		const char* schema_text,
+		const nnf_backend_weights* weights, uint32_t weights_count,
+		const nnf_backend_dataset_file* inputs, uint32_t input_count,
+		const nnf_backend_dataset_file* outputs, uint32_t output_count,
+		uint32_t compact_samples,
+		const nnf_backend_options* options,
+		char* report, size_t report_capacity)
+	{
+		return guarded([&](std::ostream& out)
+		{
+			const network_schema schema = parse_schema(schema_text);
+			if ((outputs == nullptr) || (output_count == 0))
+				throw neural_network_exception("No output layers specified for forward_propagation");
+			std::vector<std::string> output_names;
+			for(uint32_t i = 0; i < output_count; ++i)
+				output_names.push_back(outputs[i].layer_name);
+
+			hip::factory_generator_hip generator;
+			apply_options(generator, options);
+			forward_propagation::ptr fp = generator.create_forward_propagation_factory()->create(schema, output_names,
+				debug_state::ptr(new debug_state(false)), profile_state::ptr(new profile_state(false)));
+			network_data data;
+			fill_data(data, weights, weights_count, options);
+			fp->set_data(data);
+
+			// the reader toolset::get_structured_data_bunch_reader builds (nnforge/toolset.cpp:659-678): a file per data
+			// layer, and the constant 1 for a data layer called dataset_value
+			std::map<std::string, structured_data_reader::ptr> readers;
+			for(uint32_t i = 0; i < input_count; ++i)
+			{
+				std::shared_ptr<std::istream> in(new std::ifstream(inputs[i].path, std::ios_base::in | std::ios_base::binary));
+				if (!*in)
+					throw neural_network_exception(std::string("Cannot open ") + inputs[i].path);
+				readers[inputs[i].layer_name] = structured_data_reader::ptr(new structured_data_stream_reader(in));
+			}
+			readers["dataset_value"] = structured_data_reader::ptr(new structured_data_constant_reader(1.0F, layer_configuration_specific(1)));
+			structured_data_bunch_stream_reader reader(readers);
+
+			neuron_value_set_data_bunch_writer writer;
+			const forward_propagation::stat st = fp->run(reader, writer);
+
+			// what run_inference does in its dump mode (nnforge/toolset.cpp:592-650): fold the samples of an entry, write a file per layer
+			for(uint32_t i = 0; i < output_count; ++i)
+			{
+				std::pair<layer_configuration_specific, neuron_value_set::ptr>& res = writer.layer_name_to_config_and_value_set_map.at(outputs[i].layer_name);
+				res.second->compact((compact_samples == 0) ? 1 : compact_samples);
+				std::shared_ptr<std::ostream> file(new std::ofstream(outputs[i].path, std::ios_base::out | std::ios_base::trunc | std::ios_base::binary));
+				if (!*file)
+					throw neural_network_exception(std::string("Cannot open ") + outputs[i].path + " for writing");
+				{
+					structured_data_stream_writer dw(file, res.first);
+					unsigned int entry_id = 0;
+					for(const std::shared_ptr<std::vector<float> >& entry : res.second->neuron_value_list)
+						dw.write(entry_id++, entry->data());
+				}
+				out << "output: " << outputs[i].layer_name << " " << res.first << " entries " << res.second->neuron_value_list.size() << "\n";
+			}
+			const hip::forward_propagation_hip * hfp = dynamic_cast<const hip::forward_propagation_hip *>(fp.get());
+			if (hfp != nullptr)
+				describe_plan(*hfp, out);
+			out << "entries: " << st.entry_processed_count << "\n";
+			out << "stat: " << st << "\n";
+		}, report, report_capacity);
+	}
+
+	int nnf_backend_rewrite_dataset(const char* in_path, const char* out_path, uint32_t compact_samples, uint32_t part_count, uint32_t part,
+		char* report, size_t report_capacity)
+	{
+		return guarded([&](std::ostream& out)
+		{
+			if ((in_path == nullptr) || (out_path == nullptr))
+				throw neural_network_exception("dataset path is null");
+			std::shared_ptr<std::istream> in(new std::ifstream(in_path, std::ios_base::in | std::ios_base::binary));
+			if (!*in)
+				throw neural_network_exception(std::string("Cannot open ") + in_path);
+			std::map<std::string, structured_data_reader::ptr> readers;
+			readers["data"] = structured_data_reader::ptr(new structured_data_stream_reader(in));
+			structured_data_bunch_stream_reader reader(readers, (part_count == 0) ? 1 : part_count);
+			reader.set_epoch(part);
+			const layer_configuration_specific config = reader.get_config_map().at("data");
+
+			neuron_value_set values(config.get_neuron_count());
+			std::vector<float> entry(config.get_neuron_count());
+			std::map<std::string, float *> data_map;
+			data_map["data"] = entry.data();
+			for(unsigned int entry_id = 0; reader.read(entry_id, data_map); ++entry_id)
+				values.add_entry(entry.data());
+			out << "config: " << config << "\n";
+			out << "entries_read: " << values.neuron_value_list.size() << " of " << reader.get_entry_count() << "\n";
+			if (!values.neuron_value_list.empty())
+			{
+				out << "average:";
+				out.precision(17);
+				const std::shared_ptr<std::vector<double> > average = values.get_average();
+				for(double v : *average)
+					out << " " << v;
+				out << "\n";
+			}
+			values.compact((compact_samples == 0) ? 1 : compact_samples);
+			std::shared_ptr<std::ostream> file(new std::ofstream(out_path, std::ios_base::out | std::ios_base::trunc | std::ios_base::binary));
+			if (!*file)
+				throw neural_network_exception(std::string("Cannot open ") + out_path + " for writing");
+			structured_data_stream_writer dw(file, config);
+			for(const std::shared_ptr<std::vector<float> >& e : values.neuron_value_list)
+				dw.write(e->data());
+			out << "entries_written: " << values.neuron_value_list.size() << "\n";
 		}, report, report_capacity);
 	}
 

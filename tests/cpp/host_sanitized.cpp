@@ -131,6 +131,46 @@ int main(int argc, char ** argv)
 		expect(nnf_backend_read_weights((folder + "/nowhere").c_str(), "bn", 4, bn_sizes, back_chunks, buffer.data(), buffer.size()) != 0, "a missing folder is refused");
 	}
 
+	// data set files: a good one, every prefix of it, and headers that announce more than the file holds
+	{
+		const uint32_t header[5] = { 2, 2, 3, 2, 6 }; // 2 feature maps of 3 x 2, 6 entries
+		const unsigned char guid[16] = { 0x2c, 0x62, 0xe0, 0x5a, 0xc6, 0x21, 0x43, 0xb2, 0xa8, 0x2c, 0x85, 0xcd, 0x58, 0x58, 0x15, 0xd9 };
+		std::string bytes(reinterpret_cast<const char *>(guid), sizeof(guid));
+		bytes.append(reinterpret_cast<const char *>(header), sizeof(header));
+		for(int i = 0; i < 6 * 12; ++i)
+		{
+			const float v = 0.5f * static_cast<float>(i);
+			bytes.append(reinterpret_cast<const char *>(&v), sizeof(v));
+		}
+		const std::string in_path = folder + "/in.dt", out_path = folder + "/out.dt";
+		const auto store = [&in_path] (const std::string& content)
+		{
+			std::FILE * f = std::fopen(in_path.c_str(), "wb");
+			std::fwrite(content.data(), 1, content.size(), f);
+			std::fclose(f);
+		};
+		std::vector<char> buffer(1 << 16);
+		store(bytes);
+		expect(nnf_backend_rewrite_dataset(in_path.c_str(), out_path.c_str(), 1, 1, 0, buffer.data(), buffer.size()) == 0, std::string("rewrite dataset: ") + buffer.data());
+		expect(std::string(buffer.data()).find("entries_read: 6 of 6") != std::string::npos, std::string("all entries read: ") + buffer.data());
+		expect(nnf_backend_rewrite_dataset(in_path.c_str(), out_path.c_str(), 3, 2, 1, buffer.data(), buffer.size()) == 0, std::string("second half, groups of 3: ") + buffer.data());
+		expect(std::string(buffer.data()).find("entries_written: 1") != std::string::npos, std::string("one group written: ") + buffer.data());
+		expect(nnf_backend_rewrite_dataset(in_path.c_str(), out_path.c_str(), 4, 1, 0, buffer.data(), buffer.size()) != 0, "6 entries do not fold into groups of 4");
+		int cut_refused = 0;
+		for(size_t cut = 0; cut < bytes.size(); cut += 3)
+		{
+			store(bytes.substr(0, cut));
+			if (nnf_backend_rewrite_dataset(in_path.c_str(), out_path.c_str(), 1, 1, 0, buffer.data(), buffer.size()) != 0)
+				++cut_refused;
+		}
+		expect(cut_refused == static_cast<int>((bytes.size() + 2) / 3), "every cut data set file is refused");
+		std::string huge = bytes;
+		const uint32_t many = 0xFFFFFFFFu;
+		huge.replace(16 + 4, 4, reinterpret_cast<const char *>(&many), 4); // dimension count
+		store(huge);
+		expect(nnf_backend_rewrite_dataset(in_path.c_str(), out_path.c_str(), 1, 1, 0, buffer.data(), buffer.size()) != 0, "an implausible dimension count is refused");
+	}
+
 	if (failures == 0)
 		std::printf("ok\n");
 	return failures == 0 ? 0 : 1;

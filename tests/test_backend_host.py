@@ -10,6 +10,8 @@ import nnf_schemas as S
 import nnf_testing as T
 from nnforge_amd import backend
 
+F = np.float32
+
 
 def plan(layers, configs, outputs, **kw):
     return backend.plan_schema(S.schema_text(layers), configs, outputs, **kw)
@@ -320,6 +322,61 @@ def test_neighbour_layer_configuration_rules():
         plan([S.L("Data", "x"), S.L("Data", "y"), S.L("Concat", "c", ["x", "y"])], {"x": (4, [8]), "y": (4, [9])}, ["c"])
     with pytest.raises(backend.BackendError, match="dropout_rate"):
         plan([S.L("Data", "x"), S.L("Dropout", "d", ["x"], dropout_rate=1.0)], {"x": (4, [8])}, ["d"])
+
+
+def test_data_set_files_round_trip_parts_and_compaction(tmp_path):
+    """nnForge's .dt files (nnforge/structured_data_stream_reader.cpp:28-61, structured_data_stream_writer.cpp:26-66), read
+    through structured_data_bunch_stream_reader into a neuron_value_set and written again."""
+    gen = T.rng(72, 0)
+    x = T.normal(gen, (10, 3, 4, 5), 2.0)
+    src, dst = tmp_path / "x.dt", tmp_path / "y.dt"
+    backend.write_dataset(src, x)
+    # the layout, byte for byte: GUID, feature maps, dimension count, sizes x first, entry count, entries
+    raw = src.read_bytes()
+    assert raw[:16] == bytes.fromhex("2c62e05ac62143b2a82c85cd585815d9")
+    assert list(np.frombuffer(raw, "<u4", 5, 16)) == [3, 2, 5, 4, 10] and len(raw) == 36 + x.nbytes
+    report = backend.rewrite_dataset(src, dst)
+    assert dst.read_bytes() == raw
+    lines = dict(l.split(": ", 1) for l in report.splitlines())
+    assert lines["entries_read"] == "10 of 10" and lines["entries_written"] == "10"
+    # neuron_value_set::get_average: per neuron over the entries, in double
+    average = np.array([float(v) for v in lines["average"].split()])
+    assert np.allclose(average, x.reshape(10, -1).astype(np.float64).mean(axis=0), rtol=1e-13, atol=1e-15)
+    # three parts of 10 entries: 4, 3 and 3 entries (the first 10 % 3 parts are one longer), chosen by the epoch
+    for part, (first, count) in enumerate([(0, 4), (4, 3), (7, 3)]):
+        report = backend.rewrite_dataset(src, dst, part_count=3, part=part)
+        assert "entries_read: %d of %d" % (count, count) in report
+        assert T.bit_mismatches(backend.read_dataset(dst), x[first:first + count]) == 0
+    assert T.bit_mismatches(backend.read_dataset(dst), backend.read_dataset(dst)) == 0
+    report = backend.rewrite_dataset(src, dst, part_count=3, part=4)   # epoch 4 is part 1 again
+    assert T.bit_mismatches(backend.read_dataset(dst), x[4:7]) == 0
+    # neuron_value_set::compact: every 5 consecutive entries become their mean, summed left to right in fp32, times 1/5
+    backend.rewrite_dataset(src, dst, compact_samples=5)
+    got = backend.read_dataset(dst)
+    want = np.zeros((2, 3, 4, 5), F)
+    for e in range(10):
+        want[e // 5] = (want[e // 5] + x[e]).astype(F)
+    want = (want * (F(1.0) / F(5.0))).astype(F)
+    assert got.shape == want.shape and T.bit_mismatches(got, want) == 0
+    with pytest.raises(backend.BackendError, match="no evenly divisible by sample count 4"):
+        backend.rewrite_dataset(src, dst, compact_samples=4)
+    # damaged files
+    bad = tmp_path / "bad.dt"
+    bad.write_bytes(b"\x00" + raw[1:])
+    with pytest.raises(backend.BackendError, match="Unknown structured data GUID encountered in input stream: 0062e05a-c621-43b2-a82c-85cd585815d9"):
+        backend.rewrite_dataset(bad, dst)
+    bad.write_bytes(raw[:30])
+    with pytest.raises(backend.BackendError, match="ends inside its header"):
+        backend.rewrite_dataset(bad, dst)
+    bad.write_bytes(raw[:36 + 7 * 240 + 100])
+    with pytest.raises(backend.BackendError, match="fewer than the 10 entries its header announces: entry 7"):
+        backend.rewrite_dataset(bad, dst)
+    with pytest.raises(backend.BackendError, match="Cannot open"):
+        backend.rewrite_dataset(tmp_path / "missing.dt", dst)
+    # an empty data set
+    backend.write_dataset(src, x[:0])
+    report = backend.rewrite_dataset(src, dst)
+    assert "entries_read: 0 of 0" in report and backend.read_dataset(dst).shape == (0, 3, 4, 5)
 
 
 def test_packets_stay_within_the_kernels_index_range():

@@ -290,6 +290,43 @@ def test_tiling_and_windows_over_entries_through_the_driver(fuse):
     assert T.ulp_distance(stat["average"], want["average"]).max() <= 1 and T.ulp_distance(stat["std_dev"], want["std_dev"]).max() <= 1
 
 
+def test_inference_from_data_set_files_to_data_set_files(tmp_path):
+    """The toolset's inference in its dump mode (nnforge/toolset.cpp:551-655) for one network: .dt files in through
+    structured_data_bunch_stream_reader, outputs collected by neuron_value_set_data_bunch_writer, the four entries a
+    tiling layer made of every input entry folded into their mean (neuron_value_set::compact), .dt files out."""
+    gen = T.rng(61, 0)
+    c, n = 5, 11
+    layers = [S.L("Data", "images"), S.L("Data", "dataset_value"),
+              S.L("BatchNorm", "bn", ["images"], feature_map_count=c), S.L("ReLU", "relu", ["bn"]),
+              S.L("MaxSubsampling", "tiles", ["relu"], windows=[2, 2], tiling=True),
+              S.L("Sigmoid", "sig", ["tiles"]),
+              S.L("AverageSubsampling", "gap", ["sig"], windows=[4, 3]),
+              S.L("Softmax", "prob", ["gap"]),
+              S.L("ReLU", "flag", ["dataset_value"])]
+    weights = S.make_weights(layers, gen)
+    images = T.normal(gen, (n, c, 7, 9), 2.0)
+    values = S.evaluate(layers, weights, {"images": images, "dataset_value": np.ones((n, 1), F32)})
+    assert values["prob"].shape == (4 * n, c, 1, 1)
+    backend.write_dataset(tmp_path / "images.dt", images)
+    outputs = {"prob": tmp_path / "out_prob.dt", "sig": tmp_path / "out_sig.dt"}
+    rep = backend.run_dataset(S.schema_text(layers), weights, {"images": tmp_path / "images.dt"}, outputs, compact_samples=4, max_entry_count=4)
+    assert rep["entries"] == n
+    for name in outputs:
+        got = backend.read_dataset(outputs[name])
+        # compact: left-to-right fp32 sum of the 4 tiles of an entry, times 0.25
+        tiles = values[name].reshape((n, 4) + values[name].shape[1:])
+        want = (((tiles[:, 0] + tiles[:, 1]) + tiles[:, 2]) + tiles[:, 3]) * F32(0.25)
+        assert_bits(got, want.astype(F32), "compacted output " + name)
+    # without compaction every tile is an entry of the file; the constant data layer reads 1
+    outputs = {"prob": tmp_path / "all_prob.dt"}
+    backend.run_dataset(S.schema_text(layers), weights, {"images": tmp_path / "images.dt"}, outputs, max_entry_count=3)
+    assert_bits(backend.read_dataset(outputs["prob"]), values["prob"], "every tile")
+    backend.run_dataset(S.schema_text(layers), weights, {"images": tmp_path / "images.dt"}, {"flag": tmp_path / "flag.dt"})
+    assert_bits(backend.read_dataset(tmp_path / "flag.dt"), np.ones((n, 1), F32), "the dataset_value layer")
+    with pytest.raises(backend.BackendError, match="Cannot open"):
+        backend.run_dataset(S.schema_text(layers), weights, {"images": tmp_path / "nowhere.dt"}, outputs)
+
+
 def test_dropout_only_network():
     """Dropout straight from the data layer to the output: in place there is nothing to launch."""
     gen = T.rng(58, 0)
