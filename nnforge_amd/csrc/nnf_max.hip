@@ -446,7 +446,7 @@ namespace nnf
 		template<int OP, int WIN_W, int WIN_H>
 		__global__ void __launch_bounds__(max_block_size) tiling2d_kernel(const tiling2d_args a)
 		{
-			extern __shared__ float staged[];
+			extern __shared__ __attribute__((aligned(16))) float staged[];
 			const uint32_t win_w = (WIN_W > 0) ? WIN_W : a.win_w, win_h = (WIN_H > 0) ? WIN_H : a.win_h;
 			const uint32_t in_plane = a.in_w * a.in_h, out_plane = a.out_w * a.out_h;
 			uint32_t first_plane, planes_here, oy0, oy1;
@@ -469,9 +469,32 @@ namespace nnf
 			const uint32_t first_row = oy0 * win_h;
 			const uint32_t staged_floats = (a.planes > 1) ? planes_here * in_plane : (oy1 * win_h + win_h - 1 - first_row) * a.in_w;
 			const float* src = a.in + static_cast<size_t>(first_plane) * in_plane + first_row * a.in_w;
-			#pragma unroll 8
-			for(uint32_t i = threadIdx.x; i < staged_floats; i += max_block_size)
-				staged[i] = src[i];
+			if (((reinterpret_cast<uintptr_t>(src) & 15) == 0) && (staged_floats % 4 == 0))
+			{
+				// the usual case (even sizes): float4, four loads in flight per lane before the first LDS store
+				constexpr uint32_t in_flight = 4;
+				const floatx4* src4 = reinterpret_cast<const floatx4*>(src);
+				floatx4* staged4 = reinterpret_cast<floatx4*>(staged);
+				const uint32_t vectors = staged_floats / 4;
+				for(uint32_t base = threadIdx.x; base < vectors; base += max_block_size * in_flight)
+				{
+					floatx4 t[in_flight];
+					#pragma unroll
+					for(uint32_t k = 0; k < in_flight; ++k)
+						if (base + k * max_block_size < vectors)
+							t[k] = load_stream(src4 + base + k * max_block_size);
+					#pragma unroll
+					for(uint32_t k = 0; k < in_flight; ++k)
+						if (base + k * max_block_size < vectors)
+							staged4[base + k * max_block_size] = t[k];
+				}
+			}
+			else
+			{
+				#pragma unroll 8
+				for(uint32_t i = threadIdx.x; i < staged_floats; i += max_block_size)
+					staged[i] = src[i];
+			}
 			__syncthreads();
 
 			const uint32_t positions_per_plane = (oy1 - oy0) * a.out_w;

@@ -126,7 +126,7 @@ def test_tiling_and_entry_windows_stay_on_their_own_kernels(gpu):
         assert rc == 0, capi.error_string(rc)
 
     us = time_launches(gpu, tiling, reps=30, warmup=3)
-    assert us < 180.0, "max subsampling with tiling takes %.1f us per launch (about 89 us expected)" % us
+    assert us < 165.0, "max subsampling with tiling takes %.1f us per launch (about 82 us expected)" % us
 
     def entry_window(i):
         rc = gpu.lib.nnf_hip_average_subsampling_nd_forward(gpu.stream, outs[i % sets].data_ptr(), ins[i % sets].data_ptr(), n // 4, c, 1,
