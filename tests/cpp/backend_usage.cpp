@@ -4,6 +4,9 @@
 // format, weights as network_data, a reader and a writer. Prints "ok" when the network's output
 // equals a straightforward host evaluation of the same layers bit for bit.
 #include <nnforge_hip/hip_backend.h>
+#include <nnforge_hip/data_streams.h>
+
+#include <fstream>
 
 #include <algorithm>
 #include <cmath>
@@ -62,7 +65,7 @@ layer { type: "Softmax" name: "prob" input_layer_name: "pool" }
 	};
 }
 
-int main()
+int main(int argc, char ** argv)
 {
 	try
 	{
@@ -206,6 +209,48 @@ int main()
 			{
 				std::cout << "run after a failed run differs" << std::endl;
 				return 1;
+			}
+		}
+
+		// the same data from data set files, the way toolset::run_inference reads and collects it: bits as before
+		{
+			const std::string folder = (argc > 1) ? argv[1] : ".";
+			std::map<std::string, structured_data_reader::ptr> file_readers;
+			for(const char * layer_name : { "conv_main", "conv_shortcut" })
+			{
+				const std::string path = folder + "/" + layer_name + ".dt";
+				{
+					std::shared_ptr<std::ostream> file(new std::ofstream(path, std::ios_base::out | std::ios_base::trunc | std::ios_base::binary));
+					structured_data_stream_writer dw(file, config);
+					std::vector<float> entry(config.get_neuron_count());
+					std::map<std::string, float *> one;
+					one[layer_name] = entry.data();
+					for(unsigned int entry_id = 0; reader.read(entry_id, one); ++entry_id)
+						dw.write(entry_id, entry.data());
+				}
+				file_readers[layer_name] = structured_data_reader::ptr(new structured_data_stream_reader(
+					std::shared_ptr<std::istream>(new std::ifstream(path, std::ios_base::in | std::ios_base::binary))));
+			}
+			structured_data_bunch_stream_reader from_files(file_readers);
+			if (from_files.get_entry_count() != static_cast<int>(entries))
+			{
+				std::cout << "data set files hold " << from_files.get_entry_count() << " entries, expected " << entries << std::endl;
+				return 1;
+			}
+			neuron_value_set_data_bunch_writer collected;
+			fp->run(from_files, collected);
+			for(const char * layer_name : { "prob", "res_prelu" })
+			{
+				const neuron_value_set& got = *collected.layer_name_to_config_and_value_set_map.at(layer_name).second;
+				const std::vector<float>& want = writer.values[layer_name];
+				bool same = got.neuron_value_list.size() == entries;
+				for(unsigned int e = 0; same && (e < entries); ++e)
+					same = std::memcmp(got.neuron_value_list[e]->data(), want.data() + static_cast<size_t>(e) * got.neuron_count, got.neuron_count * sizeof(float)) == 0;
+				if (!same)
+				{
+					std::cout << "run from data set files differs for " << layer_name << std::endl;
+					return 1;
+				}
 			}
 		}
 

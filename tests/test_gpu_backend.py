@@ -104,16 +104,17 @@ def test_run_errors():
         run(layers, bad, inputs, ["res_relu"], values)
 
 
-def test_cpp_application_uses_the_backend_like_a_reference_backend():
+def test_cpp_application_uses_the_backend_like_a_reference_backend(tmp_path):
     """tests/cpp/backend_usage.cpp: factory_generator_hip -> forward_propagation_hip from C++ with
-    a reader of unknown length, several packets, debug and profile switched on."""
+    a reader of unknown length, several packets, debug and profile switched on; then the same data through
+    data set files written into the folder given."""
     import os
     import subprocess
 
     from nnforge_amd import build
 
     assert os.path.exists(build.USAGE_PROGRAM), "build it first: python -c 'import __graft_entry__ as g; g.build()'"
-    proc = subprocess.run([build.USAGE_PROGRAM], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120)
+    proc = subprocess.run([build.USAGE_PROGRAM, str(tmp_path)], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120)
     assert proc.returncode == 0, proc.stdout
     lines = proc.stdout.strip().splitlines()
     assert lines[-1] == "ok", proc.stdout
