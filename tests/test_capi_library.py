@@ -27,6 +27,19 @@ def test_library_exports_every_declared_symbol():
     assert bound == set(names)
 
 
+def test_backend_library_exports_every_declared_symbol():
+    from nnforge_amd import backend
+
+    text = open(os.path.join(build.REPO_ROOT, "include", "nnforge_hip_backend.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    names = sorted(set(re.findall(r"NNF_BACKEND_API\s+[\w\s\*]+?\b(nnf_backend_\w+)\s*\(", text)))
+    assert len(names) >= 9, names
+    lib = backend.load()
+    for name in names:
+        assert hasattr(lib, name), name
+        assert getattr(lib, name).argtypes is not None, "no ctypes signature for " + name
+
+
 def test_struct_layout_matches_the_header():
     # nnf_hip_op: 4 x 4 bytes; nnf_hip_chain_desc: 6 + 4 + 1 words, then 8 ops
     assert ctypes.sizeof(capi.Op) == 16
