@@ -251,10 +251,18 @@ typedef struct nnf_hip_running_stat
 
 /* n = 0, mean = 0, m2 = 0, min = FLT_MAX, max = -FLT_MAX for feature_map_count states (device memory) */
 NNF_HIP_API int nnf_hip_feature_map_stat_init(void* stream, nnf_hip_running_stat* device_stats, uint32_t feature_map_count);
-/* device workspace one accumulate call of up to entry_count entries needs */
+/* device workspace (partial states of the runs of entries the reduction is cut into) that lets an accumulate
+ * call of entry_count entries use the launch shape it prefers. A workspace of this size also serves every call
+ * with fewer entries: accumulate plans its runs inside the workspace it is given. */
 NNF_HIP_API int nnf_hip_feature_map_stat_workspace_bytes(uint32_t entry_count, uint32_t feature_map_count,
 	uint32_t neuron_count_per_feature_map, size_t* bytes);
-/* folds entry_count entries of input ([entry][feature_map][neurons]) into device_stats */
+/* number of partial states (32 bytes each) an accumulate call of entry_count entries would write into a
+ * workspace of workspace_bytes; NNF_HIP_EINVAL when no launch shape fits that workspace. No device needed. */
+NNF_HIP_API int nnf_hip_feature_map_stat_partial_count(uint32_t entry_count, uint32_t feature_map_count,
+	uint32_t neuron_count_per_feature_map, size_t workspace_bytes, uint32_t* partial_states);
+/* folds entry_count entries of input ([entry][feature_map][neurons]) into device_stats; NNF_HIP_EINVAL when the
+ * workspace is too small for any launch shape (it never is when sized by nnf_hip_feature_map_stat_workspace_bytes
+ * for this or a larger entry count) */
 NNF_HIP_API int nnf_hip_feature_map_stat_accumulate(void* stream, nnf_hip_running_stat* device_stats,
 	void* device_workspace, size_t workspace_bytes, const float* input,
 	uint32_t entry_count, uint32_t feature_map_count, uint32_t neuron_count_per_feature_map);

@@ -72,6 +72,7 @@ SIGNATURES = {
                                         ctypes.POINTER(_U32), ctypes.POINTER(_U32), _U32, _U32, ctypes.c_int32],
     "nnf_hip_feature_map_stat_init": [_VP, _VP, _U32],
     "nnf_hip_feature_map_stat_workspace_bytes": [_U32, _U32, _U32, ctypes.POINTER(ctypes.c_size_t)],
+    "nnf_hip_feature_map_stat_partial_count": [_U32, _U32, _U32, ctypes.c_size_t, ctypes.POINTER(_U32)],
     "nnf_hip_feature_map_stat_accumulate": [_VP, _VP, _VP, ctypes.c_size_t, _VP, _U32, _U32, _U32],
     "nnf_hip_softmax_forward": [_VP, _VP, _VP, _U32, _U32, _U32],
     "nnf_hip_average_subsampling_forward": [_VP, _VP, _VP, _U32, _U32, _U32, _U32, _U32, _U32, _F],

@@ -211,6 +211,12 @@ extern "C"
 		return feature_map_stat_workspace_bytes(entry_count, feature_map_count, neuron_count_per_feature_map, bytes);
 	}
 
+	int nnf_hip_feature_map_stat_partial_count(uint32_t entry_count, uint32_t feature_map_count, uint32_t neuron_count_per_feature_map,
+		size_t workspace_bytes, uint32_t* partial_states)
+	{
+		return feature_map_stat_partial_count(entry_count, feature_map_count, neuron_count_per_feature_map, workspace_bytes, partial_states);
+	}
+
 	int nnf_hip_feature_map_stat_accumulate(void* stream, nnf_hip_running_stat* device_stats, void* device_workspace, size_t workspace_bytes,
 		const float* input, uint32_t entry_count, uint32_t feature_map_count, uint32_t neuron_count_per_feature_map)
 	{

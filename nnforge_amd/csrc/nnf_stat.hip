@@ -44,12 +44,18 @@ namespace nnf
 		// rounds x (run length + overhead) is chosen. Measured on 128 entries of 256 feature maps of
 		// 56x56: 6 runs of 22 entries (1536 workgroups, one round) 67.5 us, 13 runs of 10 (3328, two
 		// nearly full rounds) 69-71 us, 8 runs of 16 (2048, one round and a seventh of another) 83 us.
-		stat_plan plan_runs(uint32_t entry_count, uint32_t feature_map_count, uint32_t plane)
+		//
+		// capacity: partial states the workspace holds; plans that need more are passed over. The longest
+		// run the index arithmetic allows gives the fewest partial states, and that number never grows when
+		// entries are taken away, so a workspace sized for some entry count holds a plan for every smaller
+		// count as well (not necessarily with the same number of runs: 16 entries may be cut into 16 runs
+		// where 29 entries were cut into 15). runs == 0 in the result: no plan fits the capacity.
+		stat_plan plan_runs(uint32_t entry_count, uint32_t feature_map_count, uint32_t plane, uint64_t capacity)
 		{
 			// the kernel divides flat indices by the plane size with a multiplication, exact while
 			// index * divisor < 2^32; a run of one entry needs no division
 			const uint64_t units = ((plane % 4) == 0) ? plane / 4 : plane;
-			stat_plan best = { 1, entry_count, 1, static_cast<uint32_t>(units) };
+			stat_plan best = { 1, 0, 1, static_cast<uint32_t>(units) };
 			uint64_t best_cost = ~0ull;
 			for(uint32_t entries_per_run = 1; entries_per_run <= entry_count; ++entries_per_run)
 			{
@@ -57,6 +63,8 @@ namespace nnf
 					break;
 				const uint32_t runs = (entry_count + entries_per_run - 1) / entries_per_run;
 				const uint64_t blocks = static_cast<uint64_t>(runs) * feature_map_count;
+				if (blocks > capacity)
+					continue;
 				const uint64_t rounds = (blocks + stat_resident_blocks - 1) / stat_resident_blocks;
 				const uint64_t cost = rounds * (static_cast<uint64_t>(entries_per_run) * plane + stat_block_overhead_floats);
 				if (cost < best_cost)
@@ -68,11 +76,13 @@ namespace nnf
 			}
 			// Few planes, each long (statistics of input images, say): a plane is cut into segments so that
 			// the grid still covers the machine; a segment keeps at least two rounds of loads per lane.
+			if (best.runs == 0)
+				return best;
 			const uint64_t blocks = static_cast<uint64_t>(best.runs) * feature_map_count;
 			const uint64_t min_segment_units = static_cast<uint64_t>(stat_block_size) * stat_unroll * 2;
 			if ((best.entries_per_run == 1) && (blocks * 2 <= stat_resident_blocks) && (units >= 2 * min_segment_units))
 			{
-				const uint64_t wanted = std::min<uint64_t>(stat_resident_blocks / blocks, units / min_segment_units);
+				const uint64_t wanted = std::min<uint64_t>(std::min<uint64_t>(stat_resident_blocks, capacity) / blocks, units / min_segment_units);
 				best.units_per_segment = static_cast<uint32_t>((units + wanted - 1) / wanted);
 				best.segments = static_cast<uint32_t>((units + best.units_per_segment - 1) / best.units_per_segment);
 			}
@@ -245,8 +255,23 @@ namespace nnf
 	{
 		if ((bytes == nullptr) || (feature_map_count == 0) || (neuron_count_per_feature_map == 0))
 			return NNF_HIP_EINVAL;
-		const stat_plan p = plan_runs(std::max(1u, entry_count), feature_map_count, neuron_count_per_feature_map);
+		const stat_plan p = plan_runs(std::max(1u, entry_count), feature_map_count, neuron_count_per_feature_map, ~0ull);
 		*bytes = static_cast<size_t>(p.runs) * p.segments * feature_map_count * sizeof(nnf_hip_running_stat);
+		return NNF_HIP_OK;
+	}
+
+	int feature_map_stat_partial_count(uint32_t entry_count, uint32_t feature_map_count, uint32_t neuron_count_per_feature_map,
+		size_t workspace_bytes, uint32_t* partial_states)
+	{
+		if ((partial_states == nullptr) || (feature_map_count == 0) || (neuron_count_per_feature_map == 0))
+			return NNF_HIP_EINVAL;
+		*partial_states = 0;
+		if (entry_count == 0)
+			return NNF_HIP_OK;
+		const stat_plan p = plan_runs(entry_count, feature_map_count, neuron_count_per_feature_map, workspace_bytes / sizeof(nnf_hip_running_stat));
+		if (p.runs == 0)
+			return NNF_HIP_EINVAL;
+		*partial_states = p.runs * p.segments * feature_map_count;
 		return NNF_HIP_OK;
 	}
 
@@ -264,9 +289,12 @@ namespace nnf
 		const uint64_t total = static_cast<uint64_t>(entry_count) * feature_map_count * neuron_count_per_feature_map;
 		if ((total > NNF_HIP_MAX_ELEMENT_COUNT) || (feature_map_count > 65535u))
 			return NNF_HIP_ETOOBIG;
-		const stat_plan p = plan_runs(entry_count, feature_map_count, neuron_count_per_feature_map);
-		const size_t needed = static_cast<size_t>(p.runs) * p.segments * feature_map_count * sizeof(nnf_hip_running_stat);
-		if ((workspace == nullptr) || (workspace_bytes < needed))
+		if (workspace == nullptr)
+			return NNF_HIP_EINVAL;
+		// the plan is made inside what the workspace holds: a workspace sized for a packet of entries also
+		// serves every shorter packet
+		const stat_plan p = plan_runs(entry_count, feature_map_count, neuron_count_per_feature_map, workspace_bytes / sizeof(nnf_hip_running_stat));
+		if (p.runs == 0)
 			return NNF_HIP_EINVAL;
 
 		nnf_hip_running_stat* partial = static_cast<nnf_hip_running_stat*>(workspace);

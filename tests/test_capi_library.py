@@ -70,3 +70,27 @@ def test_argument_checks_need_no_gpu():
     for code in (0, capi.E_INVAL, capi.E_UNSUPPORTED, capi.E_ALIGN, capi.E_OVERLAP, capi.E_TOOBIG, 1, 98):
         assert lib.nnf_hip_error_string(code)
     assert b"gfx950" in lib.nnf_hip_version()
+
+
+def test_statistics_workspace_of_a_packet_serves_every_shorter_packet():
+    """The driver sizes the statistics workspace once, for a full packet, and the last packet of a run is
+    shorter. The reduction is cut into runs of entries so that the grid fills whole rounds of resident
+    workgroups, and fewer entries can mean MORE runs (256 feature maps of 7x7: 29 entries -> 15 runs, 16
+    entries -> 16 runs): the plan therefore has to be made inside the workspace that is there."""
+    lib = capi.load()
+    need, count = ctypes.c_size_t(), ctypes.c_uint32()
+    grew = 0
+    for fm, plane, packet in ((64, 49, 29), (256, 49, 12), (256, 49, 64), (2048, 49, 64), (64, 3136, 40), (3, 224 * 224, 8),
+                              (1000, 1, 300), (7, 100003, 5), (512, 196, 33)):
+        assert lib.nnf_hip_feature_map_stat_workspace_bytes(packet, fm, plane, ctypes.byref(need)) == 0
+        assert need.value % 32 == 0 and need.value >= 32 * fm
+        for entries in range(1, packet + 1):
+            assert lib.nnf_hip_feature_map_stat_partial_count(entries, fm, plane, need.value, ctypes.byref(count)) == 0, (fm, plane, packet, entries)
+            assert fm <= count.value <= need.value // 32 and count.value % fm == 0
+            own = ctypes.c_size_t()
+            assert lib.nnf_hip_feature_map_stat_workspace_bytes(entries, fm, plane, ctypes.byref(own)) == 0
+            grew += own.value > need.value
+    assert grew > 0, "no case where a shorter packet prefers more partial states: the test lost its point"
+    # a workspace below one state per feature map holds no plan; zero entries need none
+    assert lib.nnf_hip_feature_map_stat_partial_count(4, 64, 49, 32 * 63, ctypes.byref(count)) == capi.E_INVAL
+    assert lib.nnf_hip_feature_map_stat_partial_count(0, 64, 49, 0, ctypes.byref(count)) == 0 and count.value == 0

@@ -368,6 +368,23 @@ def test_layer_statistics_on_device_and_on_host(on_host):
         assert T.ulp_distance(got["std_dev"], want["std_dev"]).max() <= 1
 
 
+def test_layer_statistics_with_a_short_last_packet_and_more_workgroups_than_the_device_holds():
+    """256 feature maps of 7x7 in packets of 12 entries, 19 entries in all: the last packet of 7 prefers another cut
+    into runs than the full one, and feature maps x entries is beyond one round of resident workgroups."""
+    gen = T.rng(61, 0)
+    c, n = 256, 19
+    layers = two_bn_net(c)
+    weights = S.make_weights(layers, gen)
+    inputs = {"stem": (T.normal(gen, (n, c, 14, 14), 2.0) + F32(0.5)).astype(F32)}
+    values = S.evaluate(layers, weights, inputs)
+    want = oracle.FeatureMapStat(c).write(values["bn2"]).get()
+    got, rep = backend.layer_statistics(S.schema_text(layers), weights, inputs, "bn2", c, max_entry_count=12)
+    assert rep["entries"] == n and rep["writer_entries"] == n
+    assert np.array_equal(got["min"], want["min"]) and np.array_equal(got["max"], want["max"])
+    assert T.ulp_distance(got["average"], want["average"]).max() <= 1
+    assert T.ulp_distance(got["std_dev"], want["std_dev"]).max() <= 1
+
+
 def test_update_bn_weights_refreshes_every_batch_norm_in_forward_order(tmp_path):
     """toolset::update_bn_weights: the oracle replays it layer by layer (statistics with gamma 1 / beta 0,
     then the two formulas); the backend must arrive at the same mean / inverse sigma to one ulp of what

@@ -98,6 +98,25 @@ def test_statistics_accumulate_over_packets(gpu):
     assert dev.host().tobytes() == before
 
 
+@pytest.mark.parametrize("c,plane,packet,n", [(256, 49, 12, 19), (64, 49, 29, 45), (512, 16, 20, 33)])
+def test_short_last_packet_fits_the_workspace_of_a_full_one(gpu, c, plane, packet, n):
+    """More workgroups than the device holds at once (feature maps x entries > 1792) and a last packet that would
+    rather be cut into more runs than the full packet was: the workspace sized for the full packet must do."""
+    gen = T.rng(74, c + n)
+    x = T.normal(gen, (n, c, plane), 1.5)
+    need = ctypes.c_size_t()
+    assert gpu.lib.nnf_hip_feature_map_stat_workspace_bytes(packet, c, plane, ctypes.byref(need)) == 0
+    work = gpu.torch.empty(need.value, dtype=gpu.torch.uint8, device=gpu.device)
+    dev = DeviceStat(gpu, c)
+    for first in range(0, n, packet):
+        part = gpu.to_device(x[first:first + packet])
+        rc = gpu.lib.nnf_hip_feature_map_stat_accumulate(gpu.stream, dev.state.data_ptr(), work.data_ptr(), need.value, part.data_ptr(),
+                                                         min(packet, n - first), c, plane)
+        assert rc == 0, capi.error_string(rc)
+    want = oracle.FeatureMapStat(c).write(x).state
+    check(dev.host(), want, scale=10.0)
+
+
 def test_statistics_of_a_large_offset_and_of_constants(gpu):
     gen = T.rng(72, 0)
     x = (F(1000.0) + T.normal(gen, (64, 4, 28, 28), 0.01)).astype(F)
