@@ -35,6 +35,7 @@ extern "C" {
 #define NNF_HIP_EALIGN (-3)      /* a tensor base pointer is not 16-byte aligned                 */
 #define NNF_HIP_EOVERLAP (-4)    /* output overlaps an input other than "out == inputs[0]"      */
 #define NNF_HIP_ETOOBIG (-5)     /* element count does not fit the kernels' index range          */
+#define NNF_HIP_ESCRATCH (-6)    /* shape beyond what the library's static scratch array holds   */
 
 /* The kernels index tensors with 32 bits: a tensor (an input, an output) of more elements than this makes
  * an entry point return NNF_HIP_ETOOBIG. Callers that split their work into batches size them to it. */
@@ -266,6 +267,24 @@ NNF_HIP_API int nnf_hip_feature_map_stat_partial_count(uint32_t entry_count, uin
 NNF_HIP_API int nnf_hip_feature_map_stat_accumulate(void* stream, nnf_hip_running_stat* device_stats,
 	void* device_workspace, size_t workspace_bytes, const float* input,
 	uint32_t entry_count, uint32_t feature_map_count, uint32_t neuron_count_per_feature_map);
+
+/* nnf_hip_feature_map_stat_accumulate for callers that cannot allocate device memory and so have no workspace to
+ * pass: code that records a HIP graph, tight serving loops, harnesses that forbid hipMalloc. No counterpart in the
+ * reference. Same kernels and same results as nnf_hip_feature_map_stat_accumulate; the partial states go into a
+ * fixed array of NNF_HIP_STAT_STATIC_SCRATCH_BYTES inside the library's device image (each GPU the library runs on
+ * holds its own copy until the process ends), whose address is looked up once per device: by
+ * nnf_hip_feature_map_stat_init, else by the first call here, in both cases for the device that is current, which
+ * must be the stream's. The call itself allocates nothing and frees nothing. Limit:
+ * NNF_HIP_STAT_STATIC_SCRATCH_BYTES / 32 = 8192 partial states, one per feature map and run of entries. The runs
+ * are planned inside that limit; a shape is refused (NNF_HIP_ESCRATCH, nothing launched) only when even the longest
+ * runs the kernels' index arithmetic allows leave more states than that: more than 8192 feature maps, or planes of
+ * u loads (u = neuron_count_per_feature_map / 4, or neuron_count_per_feature_map when that is no multiple of 4) with
+ * feature_map_count * ceil(entry_count / max(1, floor((2^32 - 1) / u^2))) > 8192. All calls on one GPU share the
+ * array: calls that can overlap (different streams, different threads) race on it and must be ordered by the
+ * caller; nothing in it has to be cleared between calls (the first launch writes every state the second reads). */
+#define NNF_HIP_STAT_STATIC_SCRATCH_BYTES 262144
+NNF_HIP_API int nnf_hip_feature_map_stat_accumulate_static(void* stream, nnf_hip_running_stat* device_stats,
+	const float* input, uint32_t entry_count, uint32_t feature_map_count, uint32_t neuron_count_per_feature_map);
 
 /* ---- runtime plumbing, so that host C++ above this ABI needs no HIP headers --------------------
  * Counterparts in the reference: cuda_linear_buffer_device (nnforge/cuda/cuda_linear_buffer_device.cpp:28-45),

@@ -27,6 +27,7 @@ E_UNSUPPORTED = -2
 E_ALIGN = -3
 E_OVERLAP = -4
 E_TOOBIG = -5
+E_SCRATCH = -6
 
 
 class Op(ctypes.Structure):
@@ -73,6 +74,7 @@ SIGNATURES = {
     "nnf_hip_feature_map_stat_init": [_VP, _VP, _U32],
     "nnf_hip_feature_map_stat_workspace_bytes": [_U32, _U32, _U32, ctypes.POINTER(ctypes.c_size_t)],
     "nnf_hip_feature_map_stat_partial_count": [_U32, _U32, _U32, ctypes.c_size_t, ctypes.POINTER(_U32)],
+    "nnf_hip_feature_map_stat_accumulate_static": [_VP, _VP, _VP, _U32, _U32, _U32],
     "nnf_hip_feature_map_stat_accumulate": [_VP, _VP, _VP, ctypes.c_size_t, _VP, _U32, _U32, _U32],
     "nnf_hip_softmax_forward": [_VP, _VP, _VP, _U32, _U32, _U32],
     "nnf_hip_average_subsampling_forward": [_VP, _VP, _VP, _U32, _U32, _U32, _U32, _U32, _U32, _F],

@@ -224,6 +224,13 @@ extern "C"
 			entry_count, feature_map_count, neuron_count_per_feature_map);
 	}
 
+	int nnf_hip_feature_map_stat_accumulate_static(void* stream, nnf_hip_running_stat* device_stats,
+		const float* input, uint32_t entry_count, uint32_t feature_map_count, uint32_t neuron_count_per_feature_map)
+	{
+		return feature_map_stat_accumulate_static(static_cast<hipStream_t>(stream), device_stats, input,
+			entry_count, feature_map_count, neuron_count_per_feature_map);
+	}
+
 	int nnf_hip_add_forward(void* stream, float* output, const float* const* inputs, uint32_t input_count, float alpha, uint64_t elem_count)
 	{
 		if ((inputs == nullptr) || (input_count == 0) || (output == nullptr))
@@ -542,6 +549,7 @@ extern "C"
 		case NNF_HIP_EALIGN: return "nnforge_hip: tensor base pointer is not 16-byte aligned";
 		case NNF_HIP_EOVERLAP: return "nnforge_hip: output overlaps an input (only output == inputs[0] is allowed)";
 		case NNF_HIP_ETOOBIG: return "nnforge_hip: element count exceeds the 32-bit index range of the kernels";
+		case NNF_HIP_ESCRATCH: return "nnforge_hip: shape needs more partial states than the library's static scratch array holds (NNF_HIP_STAT_STATIC_SCRATCH_BYTES); use the entry point that takes a workspace";
 		default:
 			if (code > 0)
 				return hipGetErrorString(static_cast<hipError_t>(code));

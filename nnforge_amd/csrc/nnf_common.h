@@ -132,5 +132,7 @@ namespace nnf
 		size_t workspace_bytes, uint32_t* partial_states);
 	int feature_map_stat_accumulate(hipStream_t stream, nnf_hip_running_stat* device_stats, void* workspace, size_t workspace_bytes,
 		const float* input, uint32_t entry_count, uint32_t feature_map_count, uint32_t neuron_count_per_feature_map);
+	int feature_map_stat_accumulate_static(hipStream_t stream, nnf_hip_running_stat* device_stats,
+		const float* input, uint32_t entry_count, uint32_t feature_map_count, uint32_t neuron_count_per_feature_map);
 	int copy_kernel(hipStream_t stream, void* dst, const void* src, size_t bytes);
 }

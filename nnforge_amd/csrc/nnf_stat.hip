@@ -15,6 +15,7 @@
 
 #include <algorithm>
 #include <cstdlib>
+#include <mutex>
 
 namespace nnf
 {
@@ -29,6 +30,41 @@ namespace nnf
 		// what starting and finishing a workgroup costs, in floats of streaming (wavefront and LDS
 		// reductions, the partial state)
 		constexpr uint64_t stat_block_overhead_floats = 8192;
+
+		// Partial states of nnf_hip_feature_map_stat_accumulate_static: a fixed array in the library's device
+		// image instead of a caller's workspace. Every device the library runs on holds its own copy at its own
+		// address for the life of the process. In host code the name `scratch` is only a handle for
+		// hipGetSymbolAddress, never an address a kernel may be given.
+		constexpr size_t stat_static_states = NNF_HIP_STAT_STATIC_SCRATCH_BYTES / sizeof(nnf_hip_running_stat);
+		static __device__ __align__(256) unsigned char scratch[NNF_HIP_STAT_STATIC_SCRATCH_BYTES];
+
+		constexpr int stat_max_devices = 64;
+		std::mutex scratch_mutex;
+		void* scratch_address[stat_max_devices] = {}; // per device, looked up once with that device current
+
+		// address of the current device's copy of `scratch`
+		int static_scratch_of_current_device(void** address)
+		{
+			int device = -1;
+			hipError_t e = hipGetDevice(&device);
+			if (e != hipSuccess)
+				return hip_status(e);
+			if ((device < 0) || (device >= stat_max_devices))
+				return NNF_HIP_EUNSUPPORTED;
+			std::lock_guard<std::mutex> lock(scratch_mutex);
+			if (scratch_address[device] == nullptr)
+			{
+				void* found = nullptr;
+				e = hipGetSymbolAddress(&found, HIP_SYMBOL(scratch));
+				if (e != hipSuccess)
+					return hip_status(e);
+				if (found == nullptr)
+					return NNF_HIP_EINVAL;
+				scratch_address[device] = found;
+			}
+			*address = scratch_address[device];
+			return NNF_HIP_OK;
+		}
 
 		struct stat_plan
 		{
@@ -248,7 +284,12 @@ namespace nnf
 			return NNF_HIP_EALIGN;
 		hipLaunchKernelGGL(stat_init_kernel, dim3((feature_map_count + stat_block_size - 1) / stat_block_size), dim3(stat_block_size), 0, stream,
 			device_stats, feature_map_count);
-		return launch_status();
+		const int status = launch_status();
+		// Set-up of the statistics path on this device: the address of its static scratch array is looked up here,
+		// so that nnf_hip_feature_map_stat_accumulate_static finds it ready (a failure is reported there).
+		void* unused = nullptr;
+		static_scratch_of_current_device(&unused);
+		return status;
 	}
 
 	int feature_map_stat_workspace_bytes(uint32_t entry_count, uint32_t feature_map_count, uint32_t neuron_count_per_feature_map, size_t* bytes)
@@ -275,20 +316,68 @@ namespace nnf
 		return NNF_HIP_OK;
 	}
 
+	namespace
+	{
+		// argument checks shared by the two accumulate entry points; NNF_HIP_OK with *nothing_to_do set for zero entries
+		int check_accumulate_arguments(const nnf_hip_running_stat* device_stats, const float* input,
+			uint32_t entry_count, uint32_t feature_map_count, uint32_t neuron_count_per_feature_map, bool* nothing_to_do)
+		{
+			*nothing_to_do = false;
+			if ((device_stats == nullptr) || (feature_map_count == 0) || (neuron_count_per_feature_map == 0))
+				return NNF_HIP_EINVAL;
+			if (entry_count == 0)
+			{
+				*nothing_to_do = true; // nothing to fold in
+				return NNF_HIP_OK;
+			}
+			if (input == nullptr)
+				return NNF_HIP_EINVAL;
+			if (!is_aligned16(device_stats) || !is_aligned16(input))
+				return NNF_HIP_EALIGN;
+			const uint64_t total = static_cast<uint64_t>(entry_count) * feature_map_count * neuron_count_per_feature_map;
+			if ((total > NNF_HIP_MAX_ELEMENT_COUNT) || (feature_map_count > 65535u))
+				return NNF_HIP_ETOOBIG;
+			return NNF_HIP_OK;
+		}
+
+		// the two launches: runs of entries into `partial` (every state of the plan is written, none is read
+		// before), then their merge into device_stats in run order
+		int launch_accumulate(hipStream_t stream, nnf_hip_running_stat* device_stats, nnf_hip_running_stat* partial, const stat_plan& p,
+			const float* input, uint32_t entry_count, uint32_t feature_map_count, uint32_t neuron_count_per_feature_map)
+		{
+			const dim3 grid(p.runs * p.segments, feature_map_count);
+			if ((neuron_count_per_feature_map % 4) == 0)
+			{
+				const uint32_t units = neuron_count_per_feature_map / 4;
+				const uint32_t magic = (units >= 2) ? static_cast<uint32_t>(((1ull << 32) + units - 1) / units) : 0u;
+				hipLaunchKernelGGL(stat_runs_kernel<4>, grid, dim3(stat_block_size), 0, stream, partial, input, entry_count, feature_map_count,
+					neuron_count_per_feature_map, p.entries_per_run, magic, p.segments, p.units_per_segment);
+			}
+			else
+			{
+				const uint32_t units = neuron_count_per_feature_map;
+				const uint32_t magic = (units >= 2) ? static_cast<uint32_t>(((1ull << 32) + units - 1) / units) : 0u;
+				hipLaunchKernelGGL(stat_runs_kernel<1>, grid, dim3(stat_block_size), 0, stream, partial, input, entry_count, feature_map_count,
+					neuron_count_per_feature_map, p.entries_per_run, magic, p.segments, p.units_per_segment);
+			}
+			int status = launch_status();
+			if (status != NNF_HIP_OK)
+				return status;
+			hipLaunchKernelGGL(stat_merge_kernel, dim3((feature_map_count + stat_block_size - 1) / stat_block_size), dim3(stat_block_size), 0, stream,
+				device_stats, partial, feature_map_count, p.runs * p.segments);
+			return launch_status();
+		}
+	}
+
 	int feature_map_stat_accumulate(hipStream_t stream, nnf_hip_running_stat* device_stats, void* workspace, size_t workspace_bytes,
 		const float* input, uint32_t entry_count, uint32_t feature_map_count, uint32_t neuron_count_per_feature_map)
 	{
-		if ((device_stats == nullptr) || (feature_map_count == 0) || (neuron_count_per_feature_map == 0))
-			return NNF_HIP_EINVAL;
-		if (entry_count == 0)
-			return NNF_HIP_OK; // nothing to fold in
-		if (input == nullptr)
-			return NNF_HIP_EINVAL;
-		if (!is_aligned16(device_stats) || !is_aligned16(input) || !is_aligned16(workspace))
+		bool nothing_to_do = false;
+		const int rc = check_accumulate_arguments(device_stats, input, entry_count, feature_map_count, neuron_count_per_feature_map, &nothing_to_do);
+		if ((rc != NNF_HIP_OK) || nothing_to_do)
+			return rc;
+		if (!is_aligned16(workspace))
 			return NNF_HIP_EALIGN;
-		const uint64_t total = static_cast<uint64_t>(entry_count) * feature_map_count * neuron_count_per_feature_map;
-		if ((total > NNF_HIP_MAX_ELEMENT_COUNT) || (feature_map_count > 65535u))
-			return NNF_HIP_ETOOBIG;
 		if (workspace == nullptr)
 			return NNF_HIP_EINVAL;
 		// the plan is made inside what the workspace holds: a workspace sized for a packet of entries also
@@ -296,28 +385,29 @@ namespace nnf
 		const stat_plan p = plan_runs(entry_count, feature_map_count, neuron_count_per_feature_map, workspace_bytes / sizeof(nnf_hip_running_stat));
 		if (p.runs == 0)
 			return NNF_HIP_EINVAL;
+		return launch_accumulate(stream, device_stats, static_cast<nnf_hip_running_stat*>(workspace), p, input, entry_count, feature_map_count,
+			neuron_count_per_feature_map);
+	}
 
-		nnf_hip_running_stat* partial = static_cast<nnf_hip_running_stat*>(workspace);
-		const dim3 grid(p.runs * p.segments, feature_map_count);
-		if ((neuron_count_per_feature_map % 4) == 0)
-		{
-			const uint32_t units = neuron_count_per_feature_map / 4;
-			const uint32_t magic = (units >= 2) ? static_cast<uint32_t>(((1ull << 32) + units - 1) / units) : 0u;
-			hipLaunchKernelGGL(stat_runs_kernel<4>, grid, dim3(stat_block_size), 0, stream, partial, input, entry_count, feature_map_count,
-				neuron_count_per_feature_map, p.entries_per_run, magic, p.segments, p.units_per_segment);
-		}
-		else
-		{
-			const uint32_t units = neuron_count_per_feature_map;
-			const uint32_t magic = (units >= 2) ? static_cast<uint32_t>(((1ull << 32) + units - 1) / units) : 0u;
-			hipLaunchKernelGGL(stat_runs_kernel<1>, grid, dim3(stat_block_size), 0, stream, partial, input, entry_count, feature_map_count,
-				neuron_count_per_feature_map, p.entries_per_run, magic, p.segments, p.units_per_segment);
-		}
-		int status = launch_status();
-		if (status != NNF_HIP_OK)
-			return status;
-		hipLaunchKernelGGL(stat_merge_kernel, dim3((feature_map_count + stat_block_size - 1) / stat_block_size), dim3(stat_block_size), 0, stream,
-			device_stats, partial, feature_map_count, p.runs * p.segments);
-		return launch_status();
+	int feature_map_stat_accumulate_static(hipStream_t stream, nnf_hip_running_stat* device_stats,
+		const float* input, uint32_t entry_count, uint32_t feature_map_count, uint32_t neuron_count_per_feature_map)
+	{
+		bool nothing_to_do = false;
+		const int rc = check_accumulate_arguments(device_stats, input, entry_count, feature_map_count, neuron_count_per_feature_map, &nothing_to_do);
+		if ((rc != NNF_HIP_OK) || nothing_to_do)
+			return rc;
+		// one partial state per feature map is the least any launch shape needs
+		if (feature_map_count > stat_static_states)
+			return NNF_HIP_ESCRATCH;
+		const stat_plan p = plan_runs(entry_count, feature_map_count, neuron_count_per_feature_map, stat_static_states);
+		if (p.runs == 0)
+			return NNF_HIP_ESCRATCH; // planes so long that the entries cannot share runs, and too many of them
+		void* partial = nullptr;
+		const int found = static_scratch_of_current_device(&partial);
+		if (found != NNF_HIP_OK)
+			return found;
+		// nothing in the array has to start at zero: the first launch writes every state the second one reads
+		return launch_accumulate(stream, device_stats, static_cast<nnf_hip_running_stat*>(partial), p, input, entry_count, feature_map_count,
+			neuron_count_per_feature_map);
 	}
 }
