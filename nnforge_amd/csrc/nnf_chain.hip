@@ -10,6 +10,8 @@
 // workgroup into LDS and looked up per element.
 #include "nnf_common.h"
 
+#include <algorithm>
+#include <atomic>
 #include <cstdlib>
 
 namespace nnf
@@ -210,6 +212,182 @@ namespace nnf
 			}
 		}
 
+		// ---- pieces of a tile's life, shared by the kernel that takes one tile per workgroup and the one that
+		// walks over several -------------------------------------------------------------------------------------
+
+		// The U float4s a lane owns in the tile that starts at element tile_start, for every input tensor.
+		// Only one float4 of a whole tensor can be partial: the one that starts at tail_start when the
+		// element count is not a multiple of four. It is left out here (zeros) and travels through scalar
+		// loads and stores of its own, so that every other access is a float4 guarded by one comparison.
+		template<int NIN, int BLOCK, int U>
+		__device__ __forceinline__ void load_tile(const chain_args& a, uint32_t tile_start, uint32_t tail_start, float (&x)[NIN][U][4])
+		{
+			#pragma unroll
+			for(int j = 0; j < NIN; ++j)
+			{
+				#pragma unroll
+				for(int k = 0; k < U; ++k)
+				{
+					const uint32_t idx = tile_start + (threadIdx.x + k * BLOCK) * 4;
+					floatx4 t = {0.0f, 0.0f, 0.0f, 0.0f};
+					if (idx < tail_start)
+						t = load_stream(reinterpret_cast<const floatx4*>(a.in[j] + idx));
+					x[j][k][0] = t.x; x[j][k][1] = t.y; x[j][k][2] = t.z; x[j][k][3] = t.w;
+				}
+			}
+		}
+
+		// Whether this lane owns the tensor's partial float4 in the tile at tile_start, and as which of its U.
+		template<int BLOCK, int U>
+		__device__ __forceinline__ bool owns_tail_vector(const chain_args& a, uint32_t tile_start, uint32_t tail_start, uint32_t& k_tail)
+		{
+			const uint32_t tail_vector = (tail_start - tile_start) / 4; // float4 index inside this tile, if it is here
+			k_tail = tail_vector / BLOCK;
+			return (tail_start != a.total) && (tail_start >= tile_start) && (tail_vector < static_cast<uint32_t>(BLOCK * U))
+				&& ((tail_vector % BLOCK) == threadIdx.x);
+		}
+
+		template<int NIN, int U>
+		__device__ __forceinline__ void load_tail_vector(const chain_args& a, uint32_t tail_start, uint32_t k_tail, float (&x)[NIN][U][4])
+		{
+			#pragma unroll
+			for(int j = 0; j < NIN; ++j)
+			{
+				float tail[3];
+				#pragma unroll
+				for(int e = 0; e < 3; ++e)
+					tail[e] = (tail_start + e < a.total) ? a.in[j][tail_start + e] : 0.0f;
+				#pragma unroll
+				for(int k = 0; k < U; ++k)
+				{
+					if (static_cast<uint32_t>(k) == k_tail)
+					{
+						x[j][k][0] = tail[0]; x[j][k][1] = tail[1]; x[j][k][2] = tail[2];
+					}
+				}
+			}
+		}
+
+		template<int BLOCK, int U>
+		__device__ __forceinline__ void store_tile(const chain_args& a, uint32_t tile_start, uint32_t tail_start, const float (&v)[U][4])
+		{
+			#pragma unroll
+			for(int k = 0; k < U; ++k)
+			{
+				const uint32_t idx = tile_start + (threadIdx.x + k * BLOCK) * 4;
+				if (idx < tail_start)
+				{
+					floatx4 t;
+					t.x = v[k][0]; t.y = v[k][1]; t.z = v[k][2]; t.w = v[k][3];
+					store_stream(reinterpret_cast<floatx4*>(a.out + idx), t);
+				}
+			}
+		}
+
+		template<int U>
+		__device__ __forceinline__ void store_tail_vector(const chain_args& a, uint32_t tail_start, uint32_t k_tail, const float (&v)[U][4])
+		{
+			#pragma unroll
+			for(int k = 0; k < U; ++k)
+			{
+				if (static_cast<uint32_t>(k) == k_tail)
+				{
+					#pragma unroll
+					for(int e = 0; e < 3; ++e)
+						if (tail_start + e < a.total)
+							a.out[tail_start + e] = v[k][e];
+				}
+			}
+		}
+
+		// Where the lane's values lie: DIRECT - the feature map of each float4; otherwise the index of each
+		// element's plane among the planes the tile touches (= its slot in the LDS coefficient arrays).
+		// first_fm: feature map of the tile's first plane.
+		template<int BLOCK, int U, bool DIRECT>
+		__device__ __forceinline__ void locate_tile(const chain_args& a, uint32_t tile_start, uint32_t (&where)[U][DIRECT ? 1 : 4], uint32_t& first_fm)
+		{
+			constexpr int TILE = BLOCK * U * 4;
+			const uint32_t first_plane = tile_start / a.plane;
+			const uint32_t start_in_plane = tile_start - first_plane * a.plane;
+			first_fm = first_plane % a.fm_count;
+			#pragma unroll
+			for(int k = 0; k < U; ++k)
+			{
+				const uint32_t e0 = start_in_plane + (threadIdx.x + k * BLOCK) * 4;
+				#pragma unroll
+				for(int e = 0; e < (DIRECT ? 1 : 4); ++e)
+				{
+					uint32_t w = plane_of<TILE>(e0 + e, a.plane, a.plane_magic);
+					if (DIRECT)
+					{
+						w += first_fm; // < 2 * fm_count: the host picks this path only when span <= fm_count
+						w = (w >= a.fm_count) ? w - a.fm_count : w;
+					}
+					where[k][e] = w;
+				}
+			}
+		}
+
+		// Coefficients of the planes a tile touches, once per workgroup into LDS (the caller adds the barrier):
+		// batch norm's multiplier and addend, PReLU's slope.
+		template<int BLOCK>
+		__device__ __forceinline__ void stage_coefficients(const chain_args& a, uint32_t first_fm, float2* lds_coeff)
+		{
+			for(uint32_t s = 0; s < a.slot_count; ++s)
+			{
+				const chain_slot& slot = a.slots[s];
+				for(uint32_t i = threadIdx.x; i < a.span; i += BLOCK)
+				{
+					const uint32_t fm = (first_fm + i) % a.fm_count;
+					float2 c;
+					if (slot.kind == NNF_HIP_OP_BATCH_NORM)
+						nnf_batch_norm_coefficients(slot.p[0][fm], slot.p[1][fm], slot.p[2][fm], slot.p[3][fm], c.x, c.y);
+					else
+					{
+						c.x = slot.p[0][fm];
+						c.y = 0.0f;
+					}
+					lds_coeff[s * a.span + i] = c;
+				}
+			}
+		}
+
+		// The group's layers in the order the arguments list them: every input's own layers, the Add that
+		// joins the inputs (if any), the layers behind it. The result is left in x[0].
+		template<int NIN, int U, bool DIRECT>
+		__device__ __forceinline__ void run_listed_layers(const chain_args& a, float (&x)[NIN][U][4], const uint32_t (&where)[U][DIRECT ? 1 : 4],
+			const float2* lds_coeff, const exp_context& exp_ctx)
+		{
+			uint32_t op_index = 0;
+			#pragma unroll
+			for(int j = 0; j < NIN; ++j)
+			{
+				const uint32_t arm_end = op_index + a.arm_ops[j];
+				for(; op_index < arm_end; ++op_index)
+					apply_op<U, DIRECT, 1>(a.ops[op_index].kind, a.ops[op_index], a, x[j], where, lds_coeff, exp_ctx);
+			}
+			if (a.has_add)
+			{
+				// nnforge/plain/add_layer_tester_plain.cpp:56-59: sum starts at 0.0F
+				#pragma unroll
+				for(int k = 0; k < U; ++k)
+				{
+					#pragma unroll
+					for(int e = 0; e < 4; ++e)
+					{
+						float sum = 0.0f + x[0][k][e];
+						#pragma unroll
+						for(int j = 1; j < NIN; ++j)
+							sum = sum + x[j][k][e];
+						x[0][k][e] = sum * a.alpha;
+					}
+				}
+			}
+			const uint32_t tail_end = op_index + a.tail_ops;
+			for(; op_index < tail_end; ++op_index)
+				apply_op<U, DIRECT, 1>(a.ops[op_index].kind, a.ops[op_index], a, x[0], where, lds_coeff, exp_ctx);
+		}
+
 		// NIN: number of input tensors. BLOCK: lanes per workgroup. U: float4s per lane.
 		// DIRECT: plane % 4 == 0 (a float4 never straddles planes) and a tile touches no feature map
 		// twice; per-feature-map weights are then read straight from memory and the workgroup needs
@@ -250,75 +428,22 @@ namespace nnf
 			// All loads are issued before anything else: the tensors first (nothing but the tile index
 			// goes into their addresses), then the lane's expf table entry and (compile-time programs) the
 			// weights of a leading batch norm; the index arithmetic runs while they are in flight.
-			// Only one float4 of the whole tensor can be partial: the one that starts at tail_start when the
-			// element count is not a multiple of four. Its up to three values travel through scalar loads
-			// and stores of their own, so that every other access is a float4 guarded by one comparison.
 			const uint32_t tail_start = a.total & ~3u;
 			float x[NIN][U][4];
-			#pragma unroll
-			for(int j = 0; j < NIN; ++j)
-			{
-				#pragma unroll
-				for(int k = 0; k < U; ++k)
-				{
-					const uint32_t idx = tile_start + (threadIdx.x + k * BLOCK) * 4;
-					floatx4 t = {0.0f, 0.0f, 0.0f, 0.0f};
-					if (idx < tail_start)
-						t = load_stream(reinterpret_cast<const floatx4*>(a.in[j] + idx));
-					x[j][k][0] = t.x; x[j][k][1] = t.y; x[j][k][2] = t.z; x[j][k][3] = t.w;
-				}
-			}
-			// float4 index of the partial vector inside this tile, if it is here
-			const uint32_t tail_vector = (tail_start - tile_start) / 4;
-			const bool owns_tail = (tail_start != a.total) && (tail_start >= tile_start) && (tail_vector < static_cast<uint32_t>(BLOCK * U))
-				&& ((tail_vector % BLOCK) == threadIdx.x);
+			load_tile<NIN, BLOCK, U>(a, tile_start, tail_start, x);
+			uint32_t k_tail;
+			const bool owns_tail = owns_tail_vector<BLOCK, U>(a, tile_start, tail_start, k_tail);
 			if (owns_tail)
-			{
-				const uint32_t k_tail = tail_vector / BLOCK;
-				#pragma unroll
-				for(int j = 0; j < NIN; ++j)
-				{
-					float tail[3];
-					#pragma unroll
-					for(int e = 0; e < 3; ++e)
-						tail[e] = (tail_start + e < a.total) ? a.in[j][tail_start + e] : 0.0f;
-					#pragma unroll
-					for(int k = 0; k < U; ++k)
-					{
-						if (static_cast<uint32_t>(k) == k_tail)
-						{
-							x[j][k][0] = tail[0]; x[j][k][1] = tail[1]; x[j][k][2] = tail[2];
-						}
-					}
-				}
-			}
+				load_tail_vector<NIN, U>(a, tail_start, k_tail, x);
 
 			constexpr bool program_has_exp = PROGRAM > 0; // every compile-time program calls expf
 			uint64_t exp_entry = 0;
 			if (program_has_exp || a.need_exp)
 				exp_entry = load_exp2_table_entry();
 
-			const uint32_t first_plane = tile_start / a.plane;
-			const uint32_t start_in_plane = tile_start - first_plane * a.plane;
-			const uint32_t first_fm = first_plane % a.fm_count;
-
 			uint32_t where[U][PL];
-			#pragma unroll
-			for(int k = 0; k < U; ++k)
-			{
-				const uint32_t e0 = start_in_plane + (threadIdx.x + k * BLOCK) * 4;
-				#pragma unroll
-				for(int e = 0; e < PL; ++e)
-				{
-					uint32_t w = plane_of<TILE>(e0 + e, a.plane, a.plane_magic);
-					if (DIRECT)
-					{
-						w += first_fm; // < 2 * fm_count: the host picks this path only when span <= fm_count
-						w = (w >= a.fm_count) ? w - a.fm_count : w;
-					}
-					where[k][e] = w;
-				}
-			}
+			uint32_t first_fm;
+			locate_tile<BLOCK, U, DIRECT>(a, tile_start, where, first_fm);
 
 			// compile-time program that starts with a batch norm, weights read straight from memory
 			constexpr bool leading_batch_norm = DIRECT && (PROGRAM > 0) && (known_programs[PROGRAM].kinds[0] == NNF_HIP_OP_BATCH_NORM);
@@ -334,27 +459,10 @@ namespace nnf
 				exp_ctx = stage_exp2_table_per_wavefront(lds_exp, exp_entry);
 			if (!DIRECT)
 			{
-				for(uint32_t s = 0; s < a.slot_count; ++s)
-				{
-					const chain_slot& slot = a.slots[s];
-					for(uint32_t i = threadIdx.x; i < a.span; i += BLOCK)
-					{
-						const uint32_t fm = (first_fm + i) % a.fm_count;
-						float2 c;
-						if (slot.kind == NNF_HIP_OP_BATCH_NORM)
-							nnf_batch_norm_coefficients(slot.p[0][fm], slot.p[1][fm], slot.p[2][fm], slot.p[3][fm], c.x, c.y);
-						else
-						{
-							c.x = slot.p[0][fm];
-							c.y = 0.0f;
-						}
-						lds_coeff[s * a.span + i] = c;
-					}
-				}
+				stage_coefficients<BLOCK>(a, first_fm, lds_coeff);
 				__syncthreads();
 			}
 
-			uint32_t op_index = 0;
 			if (PROGRAM > 0)
 			{
 				if (leading_batch_norm)
@@ -372,82 +480,91 @@ namespace nnf
 				#pragma unroll
 				for(int i = leading_batch_norm ? 1 : 0; i < known_programs[PROGRAM].op_count; ++i)
 					apply_op<U, DIRECT, U * 4>(known_programs[PROGRAM].kinds[i], a.ops[i], a, x[0], where, lds_coeff, exp_ctx);
-				op_index = known_programs[PROGRAM].op_count;
 			}
 			else
+				run_listed_layers<NIN, U, DIRECT>(a, x, where, lds_coeff, exp_ctx);
+
+			store_tile<BLOCK, U>(a, tile_start, tail_start, x[0]);
+			if (owns_tail)
+				store_tail_vector<U>(a, tail_start, k_tail, x[0]);
+		}
+
+		// The same group on a grid that stays put: as many workgroups as the device holds at once (or fewer), each
+		// walking over tiles blockIdx.x, blockIdx.x + gridDim.x, ... with the next tile's loads issued before the
+		// current tile is computed and stored, so a lane always has loads in flight. Tiles that run at the same
+		// moment are neighbours in memory, as with one tile per workgroup. Planes are float4-aligned and no tile
+		// touches a feature map twice (the DIRECT case above): weights come straight from memory, no LDS
+		// coefficients, no barrier.
+		template<int NIN, int BLOCK, int U>
+		__global__ void __launch_bounds__(BLOCK) chain_kernel_persistent(const chain_args a, const uint32_t tile_count)
+		{
+			constexpr int TILE = BLOCK * U * 4;
+			extern __shared__ __align__(16) unsigned char lds_raw[];
+			uint64_t* lds_exp = reinterpret_cast<uint64_t*>(lds_raw);
+
+			const uint32_t tail_start = a.total & ~3u;
+			uint32_t tile = blockIdx.x;
+			if (tile >= tile_count)
+				return;
+			float x[NIN][U][4];
+			load_tile<NIN, BLOCK, U>(a, tile * static_cast<uint32_t>(TILE), tail_start, x);
+
+			exp_context exp_ctx = make_exp_context(lds_exp);
+			if (a.need_exp)
+				exp_ctx = stage_exp2_table_per_wavefront(lds_exp, load_exp2_table_entry());
+
+			for(;;)
 			{
+				const uint32_t tile_start = tile * static_cast<uint32_t>(TILE);
+				const uint32_t next_tile = tile + gridDim.x;
+				const bool more = next_tile < tile_count;
+				float next_x[NIN][U][4];
+				if (more)
+					load_tile<NIN, BLOCK, U>(a, next_tile * static_cast<uint32_t>(TILE), tail_start, next_x);
+
+				uint32_t k_tail;
+				const bool owns_tail = owns_tail_vector<BLOCK, U>(a, tile_start, tail_start, k_tail);
+				if (owns_tail)
+					load_tail_vector<NIN, U>(a, tail_start, k_tail, x);
+				uint32_t where[U][1];
+				uint32_t first_fm;
+				locate_tile<BLOCK, U, true>(a, tile_start, where, first_fm);
+				run_listed_layers<NIN, U, true>(a, x, where, nullptr, exp_ctx);
+				store_tile<BLOCK, U>(a, tile_start, tail_start, x[0]);
+				if (owns_tail)
+					store_tail_vector<U>(a, tail_start, k_tail, x[0]);
+
+				if (!more)
+					break;
 				#pragma unroll
 				for(int j = 0; j < NIN; ++j)
 				{
-					const uint32_t arm_end = op_index + a.arm_ops[j];
-					for(; op_index < arm_end; ++op_index)
-						apply_op<U, DIRECT, 1>(a.ops[op_index].kind, a.ops[op_index], a, x[j], where, lds_coeff, exp_ctx);
-				}
-			}
-
-			if ((PROGRAM == 0) && a.has_add)
-			{
-				// nnforge/plain/add_layer_tester_plain.cpp:56-59: sum starts at 0.0F
-				#pragma unroll
-				for(int k = 0; k < U; ++k)
-				{
 					#pragma unroll
-					for(int e = 0; e < 4; ++e)
-					{
-						float sum = 0.0f + x[0][k][e];
-						#pragma unroll
-						for(int j = 1; j < NIN; ++j)
-							sum = sum + x[j][k][e];
-						x[0][k][e] = sum * a.alpha;
-					}
-				}
-			}
-
-			if (PROGRAM == 0)
-			{
-				const uint32_t tail_end = op_index + a.tail_ops;
-				for(; op_index < tail_end; ++op_index)
-					apply_op<U, DIRECT, 1>(a.ops[op_index].kind, a.ops[op_index], a, x[0], where, lds_coeff, exp_ctx);
-			}
-
-			#pragma unroll
-			for(int k = 0; k < U; ++k)
-			{
-				const uint32_t idx = tile_start + (threadIdx.x + k * BLOCK) * 4;
-				if (idx < tail_start)
-				{
-					floatx4 t;
-					t.x = x[0][k][0]; t.y = x[0][k][1]; t.z = x[0][k][2]; t.w = x[0][k][3];
-					store_stream(reinterpret_cast<floatx4*>(a.out + idx), t);
-				}
-			}
-			if (owns_tail)
-			{
-				const uint32_t k_tail = tail_vector / BLOCK;
-				#pragma unroll
-				for(int k = 0; k < U; ++k)
-				{
-					if (static_cast<uint32_t>(k) == k_tail)
+					for(int k = 0; k < U; ++k)
 					{
 						#pragma unroll
-						for(int e = 0; e < 3; ++e)
-							if (tail_start + e < a.total)
-								a.out[tail_start + e] = x[0][k][e];
+						for(int e = 0; e < 4; ++e)
+							x[j][k][e] = next_x[j][k][e];
 					}
 				}
+				tile = next_tile;
 			}
 		}
 
 		typedef void (*chain_kernel_fn)(const chain_args);
+		typedef void (*chain_persistent_kernel_fn)(const chain_args, const uint32_t);
 
-		// Launch shapes (lanes per workgroup, float4s per lane), largest tile first.
+		// Launch shapes (lanes per workgroup, float4s per lane), largest tile first; the last one is the
+		// grid that stays put (chain_kernel_persistent).
 		struct launch_shape
 		{
 			int block;
 			int unroll;
+			bool persistent;
 		};
-		constexpr launch_shape launch_shapes[] = { {256, 4}, {256, 2}, {256, 1}, {64, 1} };
+		constexpr launch_shape launch_shapes[] = { {256, 4, false}, {256, 2, false}, {256, 1, false}, {64, 1, false}, {256, 4, true} };
 		constexpr int launch_shape_count = sizeof(launch_shapes) / sizeof(launch_shapes[0]);
+		constexpr int persistent_shape = 4;
 
 		template<int NIN, int BLOCK, int U, int PROGRAM>
 		chain_kernel_fn pick_direct(bool direct)
@@ -489,6 +606,31 @@ namespace nnf
 			case 3: return pick_shape<3, 0>(shape, direct);
 			default: return pick_shape<4, 0>(shape, direct);
 			}
+		}
+
+		chain_persistent_kernel_fn pick_persistent_kernel(uint32_t input_count)
+		{
+			return chain_kernel_persistent<1, 256, 4>; // one input only: see persistent_max_inputs
+		}
+
+		// compute units of the current device (asked once per device)
+		uint32_t compute_unit_count()
+		{
+			constexpr int max_devices = 64;
+			static std::atomic<uint32_t> known[max_devices];
+			int device = 0;
+			if ((hipGetDevice(&device) != hipSuccess) || (device < 0) || (device >= max_devices))
+				return 256;
+			uint32_t count = known[device].load(std::memory_order_relaxed);
+			if (count == 0)
+			{
+				int value = 0;
+				if ((hipDeviceGetAttribute(&value, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess) || (value <= 0))
+					value = 256;
+				count = static_cast<uint32_t>(value);
+				known[device].store(count, std::memory_order_relaxed);
+			}
+			return count;
 		}
 
 		// index into known_programs of a single-input group without Add, 0 when it is not one of them
@@ -535,6 +677,12 @@ namespace nnf
 		constexpr uint32_t min_tiles_wanted = 1024;
 		// From this size on (64 MB per tensor) the smaller tile is used.
 		constexpr uint32_t large_tensor_elements = 1u << 24;
+		// The grid that stays put is built for groups with one input: it holds two tiles per lane and input (74
+		// vector registers with one input, five workgroups per compute unit; 106 with two, where it measured no
+		// faster than one tile per workgroup at any size).
+		constexpr uint32_t resident_workgroups_per_compute_unit = 8; // of 256 lanes at up to 64 vector registers
+		constexpr uint32_t persistent_max_inputs = 1;
+		constexpr uint32_t persistent_workgroups_per_compute_unit = 5;
 	}
 
 	int chain_forward(hipStream_t stream, const nnf_hip_chain_desc* desc, float* output,
@@ -646,6 +794,8 @@ namespace nnf
 		// touches no feature map twice; otherwise the workgroup stages coefficients in LDS
 		auto direct_of = [&](int shape) -> bool
 		{
+			if (a.slot_count == 0)
+				return true; // no layer reads per-feature-map weights: nothing to look up, nothing to stage
 			return ((a.plane % 4) == 0) && (span_of(shape) <= a.fm_count);
 		};
 		auto lds_bytes_of = [&](int shape) -> size_t
@@ -660,16 +810,27 @@ namespace nnf
 			return (a.total + tile - 1) / tile;
 		};
 
-		int shape = forced_shape();
-		if ((shape < 0) || (lds_bytes_of(shape) > max_dynamic_lds))
+		const int program = match_known_program(*desc, op_count);
+		// the grid that stays put exists for the interpreted layer list with weights read straight from memory
+		auto persistent_possible = [&]() -> bool
 		{
-			// Measured on MI355X: tensors of 64 MB and more stream best with two float4s per lane,
-			// smaller ones with four, as long as enough workgroups exist to cover the machine.
-			static const int large_order[] = { 1, 2, 3 };
-			static const int small_order[] = { 0, 1, 2, 3 };
+			return (program == 0) && (desc->input_count <= persistent_max_inputs) && direct_of(persistent_shape);
+		};
+		int shape = forced_shape();
+		if ((shape == persistent_shape) && !persistent_possible())
+			shape = -1;
+		const bool automatic = (shape < 0) || (lds_bytes_of(shape) > max_dynamic_lds);
+		if (automatic)
+		{
+			// Measured on MI355X. One input: tensors of 64 MB and more stream best with two float4s per lane,
+			// smaller ones with four, as long as enough workgroups exist to cover the machine. Several inputs:
+			// two float4s per lane at every size (4 % faster than four from 10 to 130 MB per tensor).
+			static const int small_tile_order[] = { 1, 2, 3 };
+			static const int any_tile_order[] = { 0, 1, 2, 3 };
 			const bool large = a.total >= large_tensor_elements;
-			const int* order = large ? large_order : small_order;
-			const int order_count = large ? 3 : 4;
+			const bool small_tiles = large || (desc->input_count > 1);
+			const int* order = small_tiles ? small_tile_order : any_tile_order;
+			const int order_count = small_tiles ? 3 : 4;
 			shape = -1;
 			for(int i = 0; i < order_count; ++i)
 			{
@@ -685,12 +846,26 @@ namespace nnf
 			if (shape < 0)
 				return NNF_HIP_EUNSUPPORTED;
 		}
-		const int program = match_known_program(*desc, op_count);
 		if ((program > 0) && (shape == 0))
 			shape = 1; // the compile-time programs have no four-float4 instance (smaller tile: LDS still fits)
+		// One input, four float4s per lane, and more tiles than the device holds workgroups at once (8 per compute
+		// unit: above 33 MB per tensor): a second, partial round of workgroups would follow the first and the time per
+		// byte jumps (32 MB: 11.0 us, 38.5 MB: 15.5 us). There the grid that stays put takes over, five workgroups
+		// per compute unit walking over the tiles with the next tile's loads in flight while the current one is
+		// stored (38.5 MB: 13.3 us, 51.4 MB: 18.8 -> 17.3 us). With fewer tiles every workgroup has one tile anyway and
+		// the plain grid is as fast or faster (25.7 MB: 9.1 against 9.4 us); from 64 MB on the two are equal.
+		if (automatic && (shape == 0) && (tiles_of(0) > compute_unit_count() * resident_workgroups_per_compute_unit) && persistent_possible())
+			shape = persistent_shape;
 		a.span = span_of(shape);
 		a.plane_magic = (a.plane >= 2) ? static_cast<uint32_t>(((1ull << 32) + a.plane - 1) / a.plane) : 0u;
 
+		if (launch_shapes[shape].persistent)
+		{
+			const uint32_t tiles = tiles_of(shape);
+			const uint32_t grid = std::min(tiles, compute_unit_count() * persistent_workgroups_per_compute_unit);
+			hipLaunchKernelGGL(pick_persistent_kernel(desc->input_count), dim3(grid), dim3(launch_shapes[shape].block), exp_table_bytes, stream, a, tiles);
+			return launch_status();
+		}
 		chain_kernel_fn kernel = pick_kernel(desc->input_count, shape, direct_of(shape), program);
 		hipLaunchKernelGGL(kernel, dim3(tiles_of(shape)), dim3(launch_shapes[shape].block), lds_bytes_of(shape), stream, a);
 		return launch_status();

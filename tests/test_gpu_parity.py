@@ -130,6 +130,48 @@ def test_config1_softmax_full_size(gpu):
 
 
 # ---------------------------------------------------------------------------------------------
+# one-input groups with more tiles than the device holds workgroups at once (33 to 67 MB per tensor): these
+# take the grid that stays put, every workgroup walking over several tiles
+# ---------------------------------------------------------------------------------------------
+
+def test_groups_on_the_walking_grid_full_size(gpu):
+    # batch_norm -> rectified_linear on a ResNet-50 shape at N=64: 64 feature maps of 56x56 (51 MB)
+    n, c, hw = 64, 64, 56
+    gen = T.rng(13, 0)
+    x = T.normal(gen, (n, c, hw * hw))
+    g, b, m, s = T.bn_params(gen, c)
+    bn = oracle.batch_norm(x, g, b, m, s)
+    got = gpu.chain((n, c, hw * hw), [[(BN, 0)]], [(RELU, 0, 0.0)], [x], [g, b, m, s])
+    check_exact(got, oracle.rectified_linear(bn), "BN+ReLU 64x64x56^2")
+    # in place, with a per-feature-map slope behind the batch norm
+    slopes = T.uniform(gen, c, 0.0, 0.25)
+    got = gpu.chain((n, c, hw * hw), [[(BN, 0), (PRELU, 4)]], [], [x], [g, b, m, s, slopes], in_place=True)
+    check_exact(got, oracle.parametric_rectified_linear(bn, slopes), "BN+PReLU 64x64x56^2 in place")
+    # a group that calls expf and is not one of the compile-time programs: the layer list is interpreted
+    y = config3_input((9, 256, 4096))   # 37.7 MB
+    g, b, m, s = T.bn_params(gen, 256)
+    want = oracle.sigmoid(oracle.rectified_linear(oracle.batch_norm(y, g, b, m, s), 0.1))
+    got = gpu.chain((9, 256, 4096), [[(BN, 0), (RELU, 0, 0.1), (SIGMOID,)]], [], [y], [g, b, m, s])
+    check_exact(got, want, "BN+ReLU+Sigmoid 9x256x4096")
+
+
+@pytest.mark.parametrize("total", [9000001, 9000002, 9000003, 8650752 + 4096 * 3 + 5, 16777215])
+def test_walking_grid_with_a_partial_last_vector(gpu, total):
+    """No weights: any element count goes. The last float4 of the tensor is partial, in the last tile, which one of the
+    workgroups reaches on its last round (or its first: 8650752 + ... puts it a few tiles behind one round of 2048 + 64)."""
+    x = T.normal(T.rng(14, total % 97), total)
+    got = gpu.chain((1, 1, total), [[(RELU, 0, 0.25), (capi.OP_ABSOLUTE,)]], [], [x])
+    check_exact(got, np.abs(oracle.rectified_linear(x, 0.25)), "ReLU+Absolute on %d elements" % total)
+    assert gpu.lib.nnf_hip_rectified_linear_forward  # the single-layer entry point takes the same path:
+    d_in = gpu.to_device(x)
+    d_out = gpu.torch.full((total + 1,), float("nan"), dtype=gpu.torch.float32, device=gpu.device)
+    assert gpu.lib.nnf_hip_rectified_linear_forward(gpu.stream, d_out.data_ptr(), d_in.data_ptr(), 0.0, total) == 0
+    out = gpu.to_host(d_out)
+    check_exact(out[:total], oracle.rectified_linear(x, 0.0), "rectified_linear on %d elements" % total)
+    assert np.isnan(out[total]), "wrote past the end"
+
+
+# ---------------------------------------------------------------------------------------------
 # every fused group shape of the ResNet-50 stack (config 4), reduced entry count
 # ---------------------------------------------------------------------------------------------
 
