@@ -84,6 +84,66 @@ namespace nnforge
 		typedef std::shared_ptr<const layer_data_custom> const_ptr;
 	};
 
+	// What is done to a layer (nnforge/layer_action.h:26-88). This backend only ever runs "forward"; the other
+	// kinds exist so that keys built elsewhere compare and print as the reference's do.
+	class layer_action
+	{
+	public:
+		enum action_type
+		{
+			forward = 0,
+			backward_data = 1,
+			backward_weights = 2,
+			backward_data_and_weights = 3,
+			update_weights = 4
+		};
+
+		layer_action() = default;
+		layer_action(action_type at, int backprop_index = -1) : at(at), backprop_index(backprop_index) {}
+
+		action_type get_action_type() const { return at; }
+		int get_backprop_index() const { return backprop_index; }
+		std::string str() const;
+
+	private:
+		action_type at = forward;
+		int backprop_index = -1;
+
+		friend bool operator <(const layer_action& x, const layer_action& y);
+	};
+
+	inline bool operator <(const layer_action& x, const layer_action& y)
+	{
+		return ((static_cast<unsigned long long>(x.at) << 32) | static_cast<unsigned int>(x.backprop_index))
+			< ((static_cast<unsigned long long>(y.at) << 32) | static_cast<unsigned int>(y.backprop_index));
+	}
+
+	// Key of the per-action tables of a propagation (nnforge/layer_name_with_action.h:25-69).
+	class layer_name_with_action
+	{
+	public:
+		layer_name_with_action() = default;
+		layer_name_with_action(const std::string& name, layer_action action) : name(name), action(action) {}
+
+		const std::string& get_name() const { return name; }
+		const layer_action& get_action() const { return action; }
+
+	private:
+		std::string name;
+		layer_action action;
+
+		friend bool operator <(const layer_name_with_action& x, const layer_name_with_action& y);
+	};
+
+	inline bool operator <(const layer_name_with_action& x, const layer_name_with_action& y)
+	{
+		if (x.name < y.name)
+			return true;
+		if (y.name < x.name)
+			return false;
+		return x.action < y.action;
+	}
+
 	typedef std::vector<unsigned int> data_config;
 	typedef std::vector<unsigned int> data_custom_config;
 

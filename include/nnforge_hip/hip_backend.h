@@ -61,11 +61,13 @@ namespace nnforge
 			typedef std::shared_ptr<const hip_running_configuration> const_ptr;
 
 			// queries the device (throws when there is none)
-			hip_running_configuration(int device_id, float max_global_memory_usage_ratio, bool fuse_layers, bool dont_share_buffers, int max_entry_count);
+			hip_running_configuration(int device_id, float max_global_memory_usage_ratio, bool fuse_layers, bool dont_share_buffers, int max_entry_count,
+				int kernel_stream_count = default_kernel_stream_count);
 			// A configuration that never touches a device: for planning launches and buffers (and testing
 			// that logic) on a machine without a GPU. Running a network with it throws.
 			static std::shared_ptr<const hip_running_configuration> create_offline(
-				unsigned long long global_memory_size, float max_global_memory_usage_ratio, bool fuse_layers, bool dont_share_buffers, int max_entry_count);
+				unsigned long long global_memory_size, float max_global_memory_usage_ratio, bool fuse_layers, bool dont_share_buffers, int max_entry_count,
+				int kernel_stream_count = default_kernel_stream_count);
 			bool is_offline() const { return offline; }
 			void set_device() const;
 			size_t get_max_bytes() const;
@@ -75,6 +77,11 @@ namespace nnforge
 			bool fuse_layers;
 			bool dont_share_buffers;
 			int max_entry_count;
+			// Streams the kernels of a packet are spread over: steps that do not depend on each other overlap the
+			// start of one with the end of another. Measured on the ResNet-50 post-convolution stack (49 independent
+			// fused groups): 64 entries 1108 us on one stream, 1047 us on two or three; 8 entries 249, 193, 183 us.
+			static constexpr int default_kernel_stream_count = 3;
+			int kernel_stream_count;
 			std::string device_name;
 			unsigned long long global_memory_size;
 			unsigned int compute_unit_count;
@@ -121,9 +128,20 @@ namespace nnforge
 			// uploads the weights: one device buffer per chunk, in chunk order
 			virtual std::vector<hip_linear_buffer_device::const_ptr> get_data(layer_data::const_ptr host_data) const;
 
+			// integer side data of the layer: tells the tester (notify_data_custom), then uploads one device buffer per chunk
+			virtual std::vector<hip_linear_buffer_device::const_ptr> set_get_data_custom(layer_data_custom::const_ptr host_data_custom);
+
+			// device buffers the tester fills once and keeps across calls; handed back to it with every enqueue
+			virtual std::vector<hip_linear_buffer_device::const_ptr> get_persistent_working_data() const;
+
 			virtual int get_input_index_layer_can_write() const { return -1; }
+			// minimum size, and whether the tester would make use of a larger buffer
 			virtual std::pair<size_t, bool> get_temporary_working_fixed_buffer_size() const { return std::make_pair(static_cast<size_t>(0), false); }
 			virtual size_t get_temporary_working_per_entry_buffer_size() const { return 0; }
+
+			// nnforge/cuda/layer_tester_cuda.h:82 asks which inputs the tester wants to read through a texture; this
+			// backend has no texture path and no tester overrides it: always empty
+			virtual std::vector<unsigned int> get_linear_addressing_through_texture_per_entry() const { return std::vector<unsigned int>(); }
 
 			// Element-wise testers describe themselves as one op of a fused group: fills op (its chunk
 			// index is set by the caller) and returns how many weight chunks the op consumes, or -1
@@ -147,6 +165,7 @@ namespace nnforge
 		protected:
 			layer_tester_hip() = default;
 			virtual void tester_configured() {}
+			virtual void notify_data_custom(layer_data_custom::const_ptr host_data_custom) {}
 
 			layer::const_ptr layer_schema;
 			hip_running_configuration::const_ptr hip_config;
@@ -210,6 +229,13 @@ namespace nnforge
 			std::vector<std::string> input_names;  // layers whose buffers are read, in kernel input order
 			bool fused;                            // several layers in one launch: the fused-group kernel, or a subsampling
 			                                       // layer (the last name) that applies the element-wise layers in front of it
+			// Where the launch goes (nnforge/cuda/forward_propagation_cuda.cpp:414-423 runs independent actions on
+			// separate streams): the kernel stream, the earlier steps on OTHER streams it has to wait for (they
+			// wrote what it reads, or still read or wrote the buffer it writes; steps on its own stream come
+			// before it anyway), and whether a later step on another stream waits for this one.
+			unsigned int stream_index = 0;
+			std::vector<unsigned int> wait_for_steps;
+			bool signals_other_streams = false;
 			std::string description() const;       // e.g. "bn1+add1+relu1 <- conv_a, conv_b"
 		};
 
@@ -231,6 +257,20 @@ namespace nnforge
 			size_t get_per_entry_buffer_bytes() const { return per_entry_bytes; }
 			unsigned int get_max_entry_count() const { return max_entry_count; }
 
+			// Times the launch plan alone, on data that stays in device memory: reads one packet of up to entry_count
+			// entries from the reader and uploads it, runs the plan warmup times untimed, then `passes` times bracketed
+			// by a device synchronisation on both sides (wall clock) and by events on the kernel stream. Nothing is
+			// copied back and the writer's role is empty: this is the figure of merit of the kernels and of the way
+			// the driver enqueues them, without the host link. No counterpart in the reference.
+			struct kernel_timing
+			{
+				unsigned int entry_count;      // entries the packet held
+				unsigned int launch_count;     // launches per pass
+				float wall_seconds_per_pass;
+				float device_seconds_per_pass; // from events on the kernel stream
+			};
+			kernel_timing time_kernels(structured_data_bunch_reader& reader, unsigned int entry_count, unsigned int warmup, unsigned int passes);
+
 		protected:
 			void actual_set_data(network_data::const_ptr data) override;
 			void actual_clear_data() override;
@@ -238,13 +278,16 @@ namespace nnforge
 				structured_data_bunch_reader& reader,
 				structured_data_bunch_writer& writer,
 				unsigned int& entries_processed,
-				std::map<std::string, float>& action_seconds,
+				std::map<layer_name_with_action, float>& action_seconds,
 				float& idle_seconds) override;
 			void layer_config_map_modified() override;
 			float get_max_bytes_per_second() const override; // HBM peak of the MI355X
 
 		private:
 			struct impl;
+			struct run_buffers;
+			// streams, device buffers for packets of `packet` entries (data and output layers once per I/O slot), weight pointers
+			void prepare_run(run_buffers& r, unsigned int packet, int slot_count);
 			std::unique_ptr<impl> p;
 			hip_running_configuration::const_ptr hip_config;
 			std::vector<forward_step> steps;
@@ -268,7 +311,8 @@ namespace nnforge
 		};
 
 		// nnforge/cuda/factory_generator_cuda.h: options hip_device_id, hip_max_global_memory_usage_ratio,
-		// hip_fuse, hip_dont_share_buffers, hip_max_entry_count
+		// hip_fuse, hip_dont_share_buffers, hip_single_command_stream (as cuda_single_command_stream,
+		// nnforge/cuda/factory_generator_cuda.cpp:105-106), hip_kernel_stream_count, hip_max_entry_count
 		class factory_generator_hip : public factory_generator
 		{
 		public:
@@ -285,6 +329,8 @@ namespace nnforge
 			float hip_max_global_memory_usage_ratio;
 			bool hip_fuse;
 			bool hip_dont_share_buffers;
+			bool hip_single_command_stream;
+			int hip_kernel_stream_count;
 			int hip_max_entry_count;
 
 		private:

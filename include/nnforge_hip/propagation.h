@@ -171,9 +171,12 @@ namespace nnforge
 
 		bool is_schema_with_weights() const;
 
-		// seconds per action of the last run (filled when profiling is on); key = layer instance name,
-		// or the names of a fused group joined with '+'
-		const std::map<std::string, float>& get_last_action_seconds() const { return last_action_seconds; }
+		// seconds per action of the last run (filled when profiling is on). A backend that runs several layers
+		// in one launch reports the launch under its last layer (the one whose output is stored);
+		// get_action_layer_names tells which layers such an action covers.
+		const std::map<layer_name_with_action, float>& get_last_action_seconds() const { return last_action_seconds; }
+		// the layers an action covers in execution order, joined with '+' (the action's own name when it covers one)
+		std::string get_action_layer_names(const layer_name_with_action& action) const;
 
 	protected:
 		forward_propagation(
@@ -188,7 +191,7 @@ namespace nnforge
 			structured_data_bunch_reader& reader,
 			structured_data_bunch_writer& writer,
 			unsigned int& entries_processed,
-			std::map<std::string, float>& action_seconds,
+			std::map<layer_name_with_action, float>& action_seconds,
 			float& idle_seconds) = 0;
 		// called when set_input_configuration_specific changed layer_config_map
 		virtual void layer_config_map_modified() = 0;
@@ -211,12 +214,14 @@ namespace nnforge
 		unsigned int output_layers_tiling_factor;
 		float flops;
 		std::set<std::string> data_layer_names;
-		std::map<std::string, float> last_action_seconds;
-		// per action (same keys as the action seconds): the reference's flops model, the memory
-		// traffic the action needs per entry, and the layer types it covers
-		std::map<std::string, float> action_flops_per_entry;
-		std::map<std::string, float> action_bytes_per_entry;
-		std::map<std::string, std::string> action_layer_types;
+		std::map<layer_name_with_action, float> last_action_seconds;
+		// per action (same keys as the action seconds): the reference's flops model
+		// (nnforge/forward_propagation.h:103) and, beside it, the memory traffic the action needs per entry
+		std::map<layer_name_with_action, float> action_flops_per_entry;
+		std::map<layer_name_with_action, float> action_bytes_per_entry;
+		// for actions that cover several layers: the layers' names and their types, each joined with '+'
+		std::map<layer_name_with_action, std::string> action_layer_names;
+		std::map<layer_name_with_action, std::string> action_layer_types;
 
 	private:
 		forward_propagation() = delete;

@@ -84,6 +84,7 @@ namespace nnforge
 		void read(const std::string& folder_path);
 
 		layer_data::ptr find(const std::string& instance_name) const; // empty when absent
+		layer_data_custom::ptr find_custom(const std::string& instance_name) const; // empty when absent
 		layer_data::ptr get(const std::string& instance_name) const;  // throws when absent
 		void add(const std::string& instance_name, layer_data::ptr data);
 

@@ -55,6 +55,7 @@ typedef struct nnf_backend_options
 	const char* profile_folder;    /* with profile: folder for forward_prop_perf_per_layer_action_NNN.csv; null: no file */
 	int32_t stat_on_host;          /* nnf_backend_layer_statistics: copy the outputs back and update the statistics
 	                                  value by value on the host, as the reference does, instead of reducing on the device */
+	int32_t kernel_stream_count;   /* hip_kernel_stream_count; 1 = hip_single_command_stream; <= 0: default */
 } nnf_backend_options;
 
 /* Runs the schema on device 0. The report lists one line per launch ("step: ..."), the buffer plan
@@ -119,6 +120,22 @@ NNF_BACKEND_API int nnf_backend_update_bn_weights(
 	uint32_t entry_count,
 	const nnf_backend_options* options,
 	const char* out_folder,
+	char* report, size_t report_capacity);
+
+/* Times the launch plan of the schema alone, on one packet of entry_count entries that stays in device memory
+ * (forward_propagation_hip::time_kernels): uploaded once, then `warmup` untimed and `passes` timed runs of the plan,
+ * nothing copied back. The report lists the plan like nnf_backend_run_schema, then "launches: N", "timed_entries: N",
+ * "wall_seconds_per_pass: S" (device synchronisation on both sides of the timed passes) and
+ * "device_seconds_per_pass: S" (events on the kernel stream). Inputs whose data pointers are equal are fine: the
+ * values do not matter for the time. */
+NNF_BACKEND_API int nnf_backend_time_kernels(
+	const char* schema_text,
+	const nnf_backend_weights* weights, uint32_t weights_count,
+	const nnf_backend_input* inputs, uint32_t input_count,
+	uint32_t entry_count,
+	const char* const* output_layer_names, uint32_t output_count,
+	const nnf_backend_options* options,
+	uint32_t warmup, uint32_t passes,
 	char* report, size_t report_capacity);
 
 /* Plans launches and buffers without touching a device (works on a machine without a GPU).

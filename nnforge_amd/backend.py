@@ -31,7 +31,7 @@ class Output(ctypes.Structure):
 class Options(ctypes.Structure):
     _fields_ = [("fuse", ctypes.c_int32), ("dont_share_buffers", ctypes.c_int32), ("max_entry_count", ctypes.c_int32),
                 ("profile", ctypes.c_int32), ("weights_from_folder", ctypes.c_int32), ("weights_folder", ctypes.c_char_p),
-                ("profile_folder", ctypes.c_char_p), ("stat_on_host", ctypes.c_int32)]
+                ("profile_folder", ctypes.c_char_p), ("stat_on_host", ctypes.c_int32), ("kernel_stream_count", ctypes.c_int32)]
 
 
 class DatasetFile(ctypes.Structure):
@@ -62,6 +62,9 @@ def load():
         lib.nnf_backend_plan_schema.argtypes = [ctypes.c_char_p, ctypes.POINTER(Input), ctypes.c_uint32,
                                                 ctypes.POINTER(ctypes.c_char_p), ctypes.c_uint32, ctypes.POINTER(Options),
                                                 ctypes.c_uint64, ctypes.c_char_p, ctypes.c_size_t]
+        lib.nnf_backend_time_kernels.argtypes = [ctypes.c_char_p, ctypes.POINTER(Weights), ctypes.c_uint32, ctypes.POINTER(Input),
+                                                 ctypes.c_uint32, ctypes.c_uint32, ctypes.POINTER(ctypes.c_char_p), ctypes.c_uint32,
+                                                 ctypes.POINTER(Options), ctypes.c_uint32, ctypes.c_uint32, ctypes.c_char_p, ctypes.c_size_t]
         lib.nnf_backend_rewrite_schema.argtypes = [ctypes.c_char_p, ctypes.c_char_p, ctypes.c_size_t]
         lib.nnf_backend_write_weights.argtypes = [ctypes.c_char_p, ctypes.POINTER(Weights), ctypes.c_uint32, ctypes.c_char_p, ctypes.c_size_t]
         lib.nnf_backend_read_weights.argtypes = [ctypes.c_char_p, ctypes.c_char_p, ctypes.c_uint32, _UP, ctypes.POINTER(_FP),
@@ -82,7 +85,7 @@ def load():
 
 
 def _options(fuse=True, dont_share_buffers=False, max_entry_count=0, profile=False, weights_folder=None,
-             profile_folder=None, stat_on_host=False):
+             profile_folder=None, stat_on_host=False, kernel_stream_count=0):
     o = Options()
     o.fuse = int(fuse)
     o.dont_share_buffers = int(dont_share_buffers)
@@ -92,6 +95,7 @@ def _options(fuse=True, dont_share_buffers=False, max_entry_count=0, profile=Fal
     o.weights_folder = weights_folder.encode() if weights_folder is not None else None
     o.profile_folder = profile_folder.encode() if profile_folder is not None else None
     o.stat_on_host = int(stat_on_host)
+    o.kernel_stream_count = int(kernel_stream_count)
     return o
 
 
@@ -140,11 +144,17 @@ def parse_report(text):
     for line in text.splitlines():
         key, _, rest = line.partition(": ")
         if key == "step":
+            # "fused|single <layers> <- <inputs> @<kernel stream>[ after <step>,<step>...]"
             kind, _, desc = rest.partition(" ")
+            desc, _, placement = desc.rpartition(" @")
+            stream, _, waits = placement.partition(" after ")
             layers, _, sources = desc.partition(" <- ")
-            res["steps"].append({"fused": kind == "fused", "layers": layers.split("+"), "inputs": sources.split(", ")})
-        elif key in ("per_entry_bytes", "max_entry_count", "entries", "writer_entries"):
+            res["steps"].append({"fused": kind == "fused", "layers": layers.split("+"), "inputs": sources.split(", "),
+                                 "stream": int(stream), "after": [int(w) for w in waits.split(",")] if waits else []})
+        elif key in ("per_entry_bytes", "max_entry_count", "entries", "writer_entries", "launches", "timed_entries"):
             res[key] = int(rest)
+        elif key in ("wall_seconds_per_pass", "device_seconds_per_pass"):
+            res[key] = float(rest)
         elif key == "seconds":
             name, _, sec = rest.rpartition(" ")
             res["seconds"][name] = float(sec)
@@ -224,6 +234,33 @@ def plan_schema(schema_text, input_configs, output_names, memory_bytes=288 << 30
     opt = _options(**options)
     rc = lib.nnf_backend_plan_schema(schema_text.encode(), ins, len(input_configs), names, len(output_names), ctypes.byref(opt),
                                      memory_bytes, report, REPORT_CAPACITY)
+    if rc != 0:
+        raise BackendError(rc, report.value.decode(errors="replace"))
+    return parse_report(report.value.decode())
+
+
+def time_kernels(schema_text, weights, inputs, output_names, warmup=2, passes=5, shared_input_pool=None, entry_count=None, **options):
+    """Device time of the schema's launch plan on one resident packet (forward_propagation_hip::time_kernels).
+    inputs: {data layer: array [entries][feature maps][...]} or, with shared_input_pool (a flat float32 array at least as
+    long as the largest input), {data layer: (feature_map_count, [dimension sizes, x first])} - every data layer then reads
+    its entries from the start of the pool (the values do not matter for the time). Returns the parsed report."""
+    lib = load()
+    keep = []
+    w = _weights_array(weights, keep)
+    if shared_input_pool is None:
+        ins, entry_count = _inputs_array(inputs, keep)
+    else:
+        pool = np.ascontiguousarray(shared_input_pool, dtype=np.float32)
+        keep.append(pool)
+        ins, _ = _inputs_array(inputs, keep, with_data=False)
+        for i, (name, (fm, dims)) in enumerate(sorted(inputs.items())):
+            assert entry_count * fm * int(np.prod(dims, dtype=np.int64)) <= pool.size, name
+            ins[i].data = pool.ctypes.data_as(_FP)
+    names = (ctypes.c_char_p * len(output_names))(*[n.encode() for n in output_names])
+    report = ctypes.create_string_buffer(REPORT_CAPACITY)
+    opt = _options(**options)
+    rc = lib.nnf_backend_time_kernels(schema_text.encode(), w, len(weights), ins, len(inputs), entry_count or 0, names, len(output_names),
+                                      ctypes.byref(opt), warmup, passes, report, REPORT_CAPACITY)
     if rc != 0:
         raise BackendError(rc, report.value.decode(errors="replace"))
     return parse_report(report.value.decode())

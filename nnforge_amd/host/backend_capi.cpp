@@ -47,8 +47,14 @@ namespace
 
 	void describe_plan(const hip::forward_propagation_hip& fp, std::ostream& out)
 	{
+		// "step: fused|single <layers> <- <inputs> @<kernel stream>[ after <step index>,...]"
 		for(const hip::forward_step& s : fp.get_steps())
-			out << "step: " << (s.fused ? "fused " : "single ") << s.description() << "\n";
+		{
+			out << "step: " << (s.fused ? "fused " : "single ") << s.description() << " @" << s.stream_index;
+			for(size_t i = 0; i < s.wait_for_steps.size(); ++i)
+				out << ((i == 0) ? " after " : ",") << s.wait_for_steps[i];
+			out << "\n";
+		}
 		out << "per_entry_bytes: " << fp.get_per_entry_buffer_bytes() << "\n";
 		out << "max_entry_count: " << fp.get_max_entry_count() << "\n";
 	}
@@ -62,6 +68,8 @@ namespace
 			generator.hip_dont_share_buffers = options->dont_share_buffers != 0;
 			if (options->max_entry_count > 0)
 				generator.hip_max_entry_count = options->max_entry_count;
+			if (options->kernel_stream_count > 0)
+				generator.hip_kernel_stream_count = options->kernel_stream_count;
 		}
 		generator.initialize();
 	}
@@ -131,15 +139,7 @@ extern "C"
 				throw neural_network_exception("No output layers specified for forward_propagation");
 
 			hip::factory_generator_hip generator;
-			generator.apply_default_options();
-			if (options != nullptr)
-			{
-				generator.hip_fuse = options->fuse != 0;
-				generator.hip_dont_share_buffers = options->dont_share_buffers != 0;
-				if (options->max_entry_count > 0)
-					generator.hip_max_entry_count = options->max_entry_count;
-			}
-			generator.initialize();
+			apply_options(generator, options);
 			forward_propagation_factory::ptr factory = generator.create_forward_propagation_factory();
 
 			std::vector<std::string> output_names;
@@ -183,8 +183,8 @@ extern "C"
 				describe_plan(*hfp, out);
 			out << "entries: " << st.entry_processed_count << "\n";
 			out << "stat: " << st << "\n";
-			for(const std::pair<const std::string, float>& a : fp->get_last_action_seconds())
-				out << "seconds: " << a.first << " " << a.second << "\n";
+			for(const std::pair<const layer_name_with_action, float>& a : fp->get_last_action_seconds())
+				out << "seconds: " << fp->get_action_layer_names(a.first) << " " << a.second << "\n";
 		}, report, report_capacity);
 	}
 
@@ -398,10 +398,52 @@ extern "C"
 			const bool fuse = (options == nullptr) || (options->fuse != 0);
 			const bool dont_share = (options != nullptr) && (options->dont_share_buffers != 0);
 			const int max_entries = ((options != nullptr) && (options->max_entry_count > 0)) ? options->max_entry_count : 4096;
-			hip::hip_running_configuration::const_ptr config = hip::hip_running_configuration::create_offline(memory_bytes, 0.9F, fuse, dont_share, max_entries);
+			const int kernel_streams = ((options != nullptr) && (options->kernel_stream_count > 0)) ? options->kernel_stream_count : hip::hip_running_configuration::default_kernel_stream_count;
+			hip::hip_running_configuration::const_ptr config = hip::hip_running_configuration::create_offline(memory_bytes, 0.9F, fuse, dont_share, max_entries, kernel_streams);
 			hip::forward_propagation_hip fp(schema, output_names, debug_state::ptr(new debug_state(false)), profile_state::ptr(new profile_state(false)), config);
 			fp.set_input_configuration_specific(input_configs(inputs, input_count));
 			describe_plan(fp, out);
+		}, report, report_capacity);
+	}
+
+	int nnf_backend_time_kernels(
+		const char* schema_text,
+		const nnf_backend_weights* weights, uint32_t weights_count,
+		const nnf_backend_input* inputs, uint32_t input_count,
+		uint32_t entry_count,
+		const char* const* output_layer_names, uint32_t output_count,
+		const nnf_backend_options* options,
+		uint32_t warmup, uint32_t passes,
+		char* report, size_t report_capacity)
+	{
+		return guarded([&](std::ostream& out)
+		{
+			const network_schema schema = parse_schema(schema_text);
+			std::vector<std::string> output_names;
+			for(uint32_t i = 0; i < output_count; ++i)
+				output_names.push_back(output_layer_names[i]);
+			hip::factory_generator_hip generator;
+			apply_options(generator, options);
+			forward_propagation::ptr fp = generator.create_forward_propagation_factory()->create(schema, output_names,
+				debug_state::ptr(new debug_state(false)), profile_state::ptr(new profile_state(false)));
+			network_data data;
+			fill_data(data, weights, weights_count, options);
+			fp->set_data(data);
+
+			memory_data_bunch_reader reader(entry_count);
+			const std::map<std::string, layer_configuration_specific> configs = input_configs(inputs, input_count);
+			for(uint32_t i = 0; i < input_count; ++i)
+				reader.add(inputs[i].layer_name, configs.find(inputs[i].layer_name)->second, inputs[i].data);
+			hip::forward_propagation_hip * hfp = dynamic_cast<hip::forward_propagation_hip *>(fp.get());
+			if (hfp == nullptr)
+				throw neural_network_exception("The factory did not make a forward_propagation_hip");
+			const hip::forward_propagation_hip::kernel_timing t = hfp->time_kernels(reader, entry_count, warmup, passes);
+			describe_plan(*hfp, out);
+			out << "launches: " << t.launch_count << "\n";
+			out << "timed_entries: " << t.entry_count << "\n";
+			out.precision(9);
+			out << "wall_seconds_per_pass: " << t.wall_seconds_per_pass << "\n";
+			out << "device_seconds_per_pass: " << t.device_seconds_per_pass << "\n";
 		}, report, report_capacity);
 	}
 

@@ -7,6 +7,19 @@
 
 namespace nnforge
 {
+	// nnforge/layer_action.h:56-78
+	std::string layer_action::str() const
+	{
+		switch (at)
+		{
+		case forward: return "forward";
+		case backward_weights: return "backward_weights";
+		case backward_data_and_weights: return "backward_data_and_weights";
+		case update_weights: return "update_weights";
+		default: return "backward_data_" + std::to_string(backprop_index);
+		}
+	}
+
 	namespace
 	{
 		template<class T> void write_pod(std::ostream& s, const T& v)

@@ -54,7 +54,8 @@ namespace nnforge
 			struct step_plan
 			{
 				forward_step info;
-				std::string key;                     // layer names joined with '+': the action name in reports
+				std::string key;                     // layer names joined with '+': what reports show for the step
+				layer_name_with_action action;       // the step's key in the per-action tables: its last layer, forward
 				layer_tester_hip::ptr tester;        // single-layer steps
 				nnf_hip_chain_desc desc;             // fused steps (entry_count filled per packet)
 				std::vector<std::string> chunk_layers; // fused steps: layers whose weight chunks are concatenated into chunk_ptrs
@@ -63,6 +64,10 @@ namespace nnforge
 				bool passes_input_on = false;        // every layer of the step is a Dropout
 				bool prologue = false;               // desc holds element-wise layers that the tester (a subsampling layer) applies to its input
 				unsigned int entry_factor = 1;       // entries of the step's output per entry read (the cumulative tiling factor of its last layer)
+				bool launches_nothing() const        // Dropout layers only, in place: nothing to do at inference
+				{
+					return passes_input_on && (output_buffer == input_buffers.at(0));
+				}
 			};
 
 			bool is_unary_elementwise(const std::string& type)
@@ -105,25 +110,129 @@ namespace nnforge
 			std::vector<layer::const_ptr> exec_layers; // layers with inputs, execution order
 			std::map<std::string, layer_tester_hip::ptr> testers;
 			std::map<std::string, std::vector<hip_linear_buffer_device::const_ptr> > weights;
+			std::map<std::string, std::vector<hip_linear_buffer_device::const_ptr> > weights_custom;    // integer side data
+			std::map<std::string, std::vector<hip_linear_buffer_device::const_ptr> > persistent_working; // per tester, made at configuration
 			network_data::const_ptr host_data;
 
 			std::vector<step_plan> plans;
 			std::vector<size_t> buffer_floats_per_entry;   // planned device buffers
 			std::map<std::string, int> value_to_buffer;    // data layers, step outputs
-			void * stream = nullptr;          // kernels
+			void * stream = nullptr;          // kernels: the main kernel stream, kernel_streams[0]
+			std::vector<void *> kernel_streams; // as many as the plan uses (steps' stream_index); the ones behind [0] take steps that do not depend on what [0] is doing
 			void * upload_stream = nullptr;   // host -> device copies
 			void * download_stream = nullptr; // device -> host copies
+			std::vector<std::unique_ptr<hip_event> > step_done;   // per step: recorded behind it when a step on another stream waits for it
+			std::vector<std::unique_ptr<hip_event> > stream_done; // per kernel stream behind [0]: end of its part of a packet
+
+			void create_streams(size_t kernel_stream_count)
+			{
+				if (upload_stream == nullptr)
+				{
+					hip_safe_call(nnf_hip_stream_create(&upload_stream));
+					hip_safe_call(nnf_hip_stream_create(&download_stream));
+				}
+				while (kernel_streams.size() < std::max<size_t>(1, kernel_stream_count))
+				{
+					void * s = nullptr;
+					hip_safe_call(nnf_hip_stream_create(&s));
+					kernel_streams.push_back(s);
+					if (kernel_streams.size() > 1)
+						stream_done.emplace_back(new hip_event());
+				}
+				stream = kernel_streams[0];
+				while (step_done.size() < plans.size())
+					step_done.emplace_back(new hip_event());
+			}
+
+			// Enqueues the launch plan for one packet whose data layer buffers are filled: every step on its
+			// kernel stream, behind the steps it depends on. The caller has made every kernel stream wait for
+			// whatever the packet itself waits for; on return kernel_streams[0] has been made to wait for the
+			// others, so that whatever is enqueued on it next runs after the whole packet.
+			void enqueue_plan(
+				const std::vector<hip_linear_buffer_device::ptr>& buffers,
+				unsigned int entries_read,
+				const std::vector<std::vector<const float *> >& chunk_ptrs,
+				const std::vector<std::pair<hip_linear_buffer_device::ptr, hip_linear_buffer_device::ptr> >& temporary_buffers,
+				const std::vector<std::unique_ptr<hip_event> > * profile_events);
 
 			~impl()
 			{
-				if (stream != nullptr)
-					nnf_hip_stream_destroy(stream);
+				for(void * s : kernel_streams)
+					nnf_hip_stream_destroy(s);
 				if (upload_stream != nullptr)
 					nnf_hip_stream_destroy(upload_stream);
 				if (download_stream != nullptr)
 					nnf_hip_stream_destroy(download_stream);
 			}
 		};
+
+		void forward_propagation_hip::impl::enqueue_plan(
+			const std::vector<hip_linear_buffer_device::ptr>& buffers,
+			unsigned int entries_read,
+			const std::vector<std::vector<const float *> >& chunk_ptrs,
+			const std::vector<std::pair<hip_linear_buffer_device::ptr, hip_linear_buffer_device::ptr> >& temporary_buffers,
+			const std::vector<std::unique_ptr<hip_event> > * profile_events)
+		{
+			const std::vector<hip_linear_buffer_device::const_ptr> none;
+			std::vector<bool> stream_used(kernel_streams.size(), false);
+			for(size_t i = 0; i < plans.size(); ++i)
+			{
+				step_plan& plan = plans[i];
+				void * const step_stream = kernel_streams.at(plan.info.stream_index);
+				const unsigned int step_entries = entries_read * plan.entry_factor; // nnforge/plain/forward_propagation_plain.cpp:185
+				if (profile_events != nullptr)
+					hip_safe_call(nnf_hip_event_record((*profile_events)[i]->ev, step_stream));
+				if (plan.launches_nothing())
+					continue;
+				// cross-stream dependencies (nnforge/cuda/forward_propagation_cuda.cpp:414-423)
+				for(unsigned int earlier : plan.info.wait_for_steps)
+					hip_safe_call(nnf_hip_stream_wait_event(step_stream, step_done[earlier]->ev));
+				stream_used[plan.info.stream_index] = true;
+
+				std::vector<hip_linear_buffer_device::const_ptr> inputs;
+				for(int b : plan.input_buffers)
+					inputs.push_back(buffers[b]);
+				if (plan.prologue)
+				{
+					plan.desc.entry_count = step_entries;
+					plan.tester->enqueue_forward_propagation_with_prologue(step_stream, buffers[plan.output_buffer], inputs.at(0), plan.desc,
+						chunk_ptrs[i].empty() ? nullptr : chunk_ptrs[i].data(), step_entries);
+				}
+				else if (plan.info.fused)
+				{
+					plan.desc.entry_count = step_entries;
+					std::vector<const float *> in_ptrs;
+					for(const hip_linear_buffer_device::const_ptr& b : inputs)
+						in_ptrs.push_back(static_cast<const float *>(*b));
+					hip_safe_call(nnf_hip_chain_forward(step_stream, &plan.desc, *buffers[plan.output_buffer], in_ptrs.data(),
+						chunk_ptrs[i].empty() ? nullptr : chunk_ptrs[i].data()));
+				}
+				else
+				{
+					const std::string& layer_name = plan.info.layer_names[0];
+					const auto of_layer = [&layer_name, &none] (const std::map<std::string, std::vector<hip_linear_buffer_device::const_ptr> >& m)
+						-> const std::vector<hip_linear_buffer_device::const_ptr>&
+					{
+						std::map<std::string, std::vector<hip_linear_buffer_device::const_ptr> >::const_iterator it = m.find(layer_name);
+						return (it == m.end()) ? none : it->second;
+					};
+					plan.tester->enqueue_forward_propagation(step_stream, buffers[plan.output_buffer], none,
+						of_layer(weights), of_layer(weights_custom), inputs, of_layer(persistent_working),
+						temporary_buffers[i].first, temporary_buffers[i].second, step_entries);
+				}
+				if (plan.info.signals_other_streams)
+					hip_safe_call(nnf_hip_event_record(step_done[i]->ev, step_stream));
+			}
+			if (profile_events != nullptr)
+				hip_safe_call(nnf_hip_event_record((*profile_events)[plans.size()]->ev, kernel_streams[0]));
+			for(size_t s = 1; s < kernel_streams.size(); ++s)
+			{
+				if (!stream_used[s])
+					continue;
+				hip_safe_call(nnf_hip_event_record(stream_done[s - 1]->ev, kernel_streams[s]));
+				hip_safe_call(nnf_hip_stream_wait_event(kernel_streams[0], stream_done[s - 1]->ev));
+			}
+		}
 
 		forward_propagation_hip::forward_propagation_hip(
 			const network_schema& schema,
@@ -159,17 +268,22 @@ namespace nnforge
 		{
 			p->host_data = data;
 			p->weights.clear();
+			p->weights_custom.clear();
 			if (hip_config->is_offline())
 				return;
 			hip_config->set_device();
+			// nnforge/cuda/forward_propagation_cuda.cpp:1016-1050: every tester uploads its own layer's data
 			for(const layer::const_ptr& l : p->exec_layers)
 			{
-				layer_data::ptr d = data->find(l->instance_name);
-				if (!d)
-					continue;
 				std::map<std::string, layer_tester_hip::ptr>::const_iterator t = p->testers.find(l->instance_name);
-				if (t != p->testers.end())
+				if (t == p->testers.end())
+					continue;
+				layer_data::ptr d = data->find(l->instance_name);
+				if (d)
 					p->weights[l->instance_name] = t->second->get_data(d);
+				layer_data_custom::ptr dc = data->find_custom(l->instance_name);
+				if (dc)
+					p->weights_custom[l->instance_name] = t->second->set_get_data_custom(dc);
 			}
 		}
 
@@ -177,6 +291,7 @@ namespace nnforge
 		{
 			p->host_data.reset();
 			p->weights.clear();
+			p->weights_custom.clear();
 		}
 
 		void forward_propagation_hip::layer_config_map_modified()
@@ -193,6 +308,10 @@ namespace nnforge
 				layer_testing_schema::ptr ts = layer_testing_schema_factory::get_singleton().create_testing_schema_layer(l);
 				p->testers[l->instance_name] = ts->create_tester(inputs, layer_config_map[l->instance_name], hip_config);
 			}
+			p->persistent_working.clear();
+			if (!hip_config->is_offline())
+				for(const std::pair<const std::string, layer_tester_hip::ptr>& t : p->testers)
+					p->persistent_working[t.first] = t.second->get_persistent_working_data();
 			if (p->host_data)
 				actual_set_data(p->host_data);
 
@@ -321,6 +440,7 @@ namespace nnforge
 			steps.clear();
 			action_flops_per_entry.clear();
 			action_bytes_per_entry.clear();
+			action_layer_names.clear();
 			action_layer_types.clear();
 			std::map<std::string, const pending_group *> group_by_name;
 			for(const std::pair<std::string, pending_group>& g : groups)
@@ -433,9 +553,11 @@ namespace nnforge
 				float step_bytes = static_cast<float>(config.get_neuron_count()) * sizeof(float) * static_cast<float>(plan.entry_factor);
 				for(const std::string& input : plan.info.input_names)
 					step_bytes += static_cast<float>(layer_config_map[input].get_neuron_count()) * sizeof(float) * static_cast<float>(cumulative_tiling_factor_map.at(input));
-				action_flops_per_entry[plan.key] = step_flops;
-				action_bytes_per_entry[plan.key] = step_bytes;
-				action_layer_types[plan.key] = types;
+				plan.action = layer_name_with_action(plan.info.layer_names.back(), layer_action(layer_action::forward));
+				action_flops_per_entry[plan.action] = step_flops;
+				action_bytes_per_entry[plan.action] = step_bytes;
+				action_layer_names[plan.action] = plan.key;
+				action_layer_types[plan.action] = types;
 
 				p->plans.push_back(plan);
 				steps.push_back(plan.info);
@@ -519,6 +641,66 @@ namespace nnforge
 				}
 			}
 
+			// ---- kernel streams: which steps may overlap --------------------------------------------
+			// A step depends on the earlier steps that wrote the buffers it reads and, because buffers are
+			// shared, on the earlier steps that read or wrote the buffer it writes. A step goes to the
+			// stream whose last step it depends on (a chain stays on its stream and needs no event), else
+			// to the stream with the least work so far; it waits for the latest of its dependencies on
+			// each other stream (streams run in order, so that one covers the earlier ones). With per-action
+			// times wanted every step goes to one stream: overlapping actions have no time of their own.
+			{
+				const size_t stream_count = profile->is_profile() ? 1 : static_cast<size_t>(std::max(1, hip_config->kernel_stream_count));
+				const size_t buffer_count = p->buffer_floats_per_entry.size();
+				std::vector<int> last_writer(buffer_count, -1);
+				std::vector<std::vector<int> > readers(buffer_count);
+				std::vector<int> stream_last(stream_count, -1);
+				std::vector<double> stream_work(stream_count, 0.0);
+				for(size_t i = 0; i < p->plans.size(); ++i)
+				{
+					step_plan& plan = p->plans[i];
+					plan.info.stream_index = 0;
+					plan.info.wait_for_steps.clear();
+					plan.info.signals_other_streams = false;
+					if (plan.launches_nothing())
+						continue; // the value stays where it is: whoever reads it depends on its writer
+					std::set<int> deps;
+					for(int b : plan.input_buffers)
+						if (last_writer[b] >= 0)
+							deps.insert(last_writer[b]);
+					const int out = plan.output_buffer;
+					if (last_writer[out] >= 0)
+						deps.insert(last_writer[out]);
+					deps.insert(readers[out].begin(), readers[out].end());
+
+					size_t chosen = stream_count;
+					for(size_t s = 0; s < stream_count; ++s)
+						if ((stream_last[s] >= 0) && (deps.find(stream_last[s]) != deps.end()) && ((chosen == stream_count) || (stream_last[s] > stream_last[chosen])))
+							chosen = s;
+					if (chosen == stream_count)
+						chosen = static_cast<size_t>(std::min_element(stream_work.begin(), stream_work.end()) - stream_work.begin());
+					plan.info.stream_index = static_cast<unsigned int>(chosen);
+					std::vector<int> latest_on_stream(stream_count, -1);
+					for(int d : deps)
+						latest_on_stream[p->plans[d].info.stream_index] = std::max(latest_on_stream[p->plans[d].info.stream_index], d);
+					for(size_t s = 0; s < stream_count; ++s)
+					{
+						if ((s == chosen) || (latest_on_stream[s] < 0))
+							continue;
+						plan.info.wait_for_steps.push_back(static_cast<unsigned int>(latest_on_stream[s]));
+						p->plans[latest_on_stream[s]].info.signals_other_streams = true;
+					}
+					stream_last[chosen] = static_cast<int>(i);
+					stream_work[chosen] += static_cast<double>(action_bytes_per_entry[plan.action]);
+
+					for(int b : plan.input_buffers)
+						readers[b].push_back(static_cast<int>(i));
+					last_writer[out] = static_cast<int>(i);
+					readers[out].clear();
+				}
+				for(size_t i = 0; i < p->plans.size(); ++i)
+					steps[i] = p->plans[i].info;
+			}
+
 			per_entry_bytes = 0;
 			for(size_t floats : p->buffer_floats_per_entry)
 				per_entry_bytes += floats * sizeof(float);
@@ -560,34 +742,95 @@ namespace nnforge
 			}
 		}
 
-		// Packets of entries flow through three in-order queues with two I/O slots (the double buffering
+		namespace
+		{
+			// Whatever ends a run - the normal return or an exception from the reader, the writer or a launch -
+			// nothing the run owns (device buffers, pinned staging, events) may be released while copies or
+			// kernels that use it are still in flight: declared after them, this guard is destroyed first and waits.
+			struct drain_streams
+			{
+				std::vector<void *> streams;
+				~drain_streams()
+				{
+					for(void * s : streams)
+						nnf_hip_stream_synchronize(s);
+				}
+			};
+		}
+
+		// Device buffers of a run: data and output layer buffers once per I/O slot, the rest shared; the
+		// working buffers testers ask for, per step (steps on different streams may run at the same time).
+		struct forward_propagation_hip::run_buffers
+		{
+			std::vector<hip_linear_buffer_device::ptr> buffers[2];
+			std::vector<std::pair<hip_linear_buffer_device::ptr, hip_linear_buffer_device::ptr> > temporary;
+			std::vector<std::vector<const float *> > chunk_ptrs; // weight pointers of the fused steps
+		};
+
+		void forward_propagation_hip::prepare_run(run_buffers& r, unsigned int packet, int slot_count)
+		{
+			hip_config->set_device();
+			unsigned int stream_count = 1;
+			for(const forward_step& step : steps)
+				stream_count = std::max(stream_count, step.stream_index + 1);
+			p->create_streams(stream_count);
+			for(const layer::const_ptr& l : p->exec_layers)
+				if (!l->is_empty_data() && (p->weights.find(l->instance_name) == p->weights.end()))
+					throw neural_network_exception("No data found with layer name " + l->instance_name);
+
+			std::set<int> io_buffers;
+			for(const std::string& n : data_layer_names)
+				io_buffers.insert(p->value_to_buffer.at(n));
+			for(const std::string& n : output_layer_names)
+				io_buffers.insert(p->value_to_buffer.at(n));
+			for(size_t b = 0; b < p->buffer_floats_per_entry.size(); ++b)
+			{
+				const size_t bytes = p->buffer_floats_per_entry[b] * sizeof(float) * packet;
+				r.buffers[0].push_back(hip_linear_buffer_device::ptr(new hip_linear_buffer_device(bytes)));
+				if ((slot_count > 1) && (io_buffers.find(static_cast<int>(b)) != io_buffers.end()))
+					r.buffers[1].push_back(hip_linear_buffer_device::ptr(new hip_linear_buffer_device(bytes)));
+				else
+					r.buffers[1].push_back(r.buffers[0].back());
+			}
+			for(const step_plan& plan : p->plans)
+			{
+				std::pair<hip_linear_buffer_device::ptr, hip_linear_buffer_device::ptr> t;
+				if (!plan.info.fused && plan.tester)
+				{
+					const size_t fixed = plan.tester->get_temporary_working_fixed_buffer_size().first;
+					const size_t per_entry = plan.tester->get_temporary_working_per_entry_buffer_size();
+					if (fixed > 0)
+						t.first.reset(new hip_linear_buffer_device(fixed));
+					if (per_entry > 0)
+						t.second.reset(new hip_linear_buffer_device(per_entry * packet * plan.entry_factor));
+				}
+				r.temporary.push_back(t);
+			}
+			r.chunk_ptrs.assign(p->plans.size(), std::vector<const float *>());
+			for(size_t i = 0; i < p->plans.size(); ++i)
+				for(const std::string& layer_name : p->plans[i].chunk_layers)
+					for(const hip_linear_buffer_device::const_ptr& b : p->weights.at(layer_name))
+						r.chunk_ptrs[i].push_back(static_cast<const float *>(*b));
+		}
+
+		// Packets of entries flow through in-order queues with two I/O slots (the double buffering
 		// of nnforge/cuda/forward_propagation_cuda.cpp:84-112, 147-316):
 		//   host reads packet i into the pinned staging of slot i % 2   (needs: upload of packet i-2 done)
 		//   upload stream copies it to the slot's device input buffers   (needs: kernels of packet i-2 done)
-		//   kernel stream runs the launch plan                           (needs: upload i, download i-2 done)
+		//   kernel streams run the launch plan                           (needs: upload i, download i-2, kernels i-1 done)
 		//   download stream copies the slot's output buffers to staging  (needs: kernels i done)
 		//   host hands packet i-1 to the writer while packet i is in flight.
 		// Data and output layers have a device buffer per slot; everything in between is shared, which is
-		// safe because the kernel stream runs one packet after the other.
+		// safe because the kernels of one packet start after those of the packet before.
 		void forward_propagation_hip::actual_run(
 			structured_data_bunch_reader& reader,
 			structured_data_bunch_writer& writer,
 			unsigned int& entries_processed,
-			std::map<std::string, float>& action_seconds,
+			std::map<layer_name_with_action, float>& action_seconds,
 			float& idle_seconds)
 		{
 			if (hip_config->is_offline())
 				throw neural_network_exception("This forward_propagation_hip was created for planning only (offline configuration): it cannot run");
-			hip_config->set_device();
-			if (p->stream == nullptr)
-			{
-				hip_safe_call(nnf_hip_stream_create(&p->stream));
-				hip_safe_call(nnf_hip_stream_create(&p->upload_stream));
-				hip_safe_call(nnf_hip_stream_create(&p->download_stream));
-			}
-			for(const layer::const_ptr& l : p->exec_layers)
-				if (!l->is_empty_data() && (p->weights.find(l->instance_name) == p->weights.end()))
-					throw neural_network_exception("No data found with layer name " + l->instance_name);
 
 			unsigned int packet = max_entry_count;
 			const int reader_entry_count = reader.get_entry_count();
@@ -595,23 +838,9 @@ namespace nnforge
 				packet = std::min(packet, static_cast<unsigned int>(reader_entry_count));
 
 			constexpr int slot_count = 2;
-			const std::set<std::string> outputs(output_layer_names.begin(), output_layer_names.end());
-			// buffers[slot][b]: data and output layer buffers are per slot, the rest is shared
-			std::set<int> io_buffers;
-			for(const std::string& n : data_layer_names)
-				io_buffers.insert(p->value_to_buffer.at(n));
-			for(const std::string& n : output_layer_names)
-				io_buffers.insert(p->value_to_buffer.at(n));
-			std::vector<hip_linear_buffer_device::ptr> buffers[slot_count];
-			for(size_t b = 0; b < p->buffer_floats_per_entry.size(); ++b)
-			{
-				const size_t bytes = p->buffer_floats_per_entry[b] * sizeof(float) * packet;
-				buffers[0].push_back(hip_linear_buffer_device::ptr(new hip_linear_buffer_device(bytes)));
-				if (io_buffers.find(static_cast<int>(b)) != io_buffers.end())
-					buffers[1].push_back(hip_linear_buffer_device::ptr(new hip_linear_buffer_device(bytes)));
-				else
-					buffers[1].push_back(buffers[0].back());
-			}
+			run_buffers r;
+			prepare_run(r, packet, slot_count);
+
 			// A statistics writer (nnforge/stat_data_bunch_writer.h) only wants per-feature-map figures of the
 			// outputs: they are reduced where they lie, in device memory, and nothing but the running
 			// states (32 bytes per feature map) travels to the host at the end of the run.
@@ -646,13 +875,6 @@ namespace nnforge
 			hip_event upload_done[slot_count], kernels_done[slot_count], download_done[slot_count];
 			bool slot_used[slot_count] = { false, false };
 
-			// weight pointers of the fused steps
-			std::vector<std::vector<const float *> > chunk_ptrs(p->plans.size());
-			for(size_t i = 0; i < p->plans.size(); ++i)
-				for(const std::string& layer_name : p->plans[i].chunk_layers)
-					for(const hip_linear_buffer_device::const_ptr& b : p->weights.at(layer_name))
-						chunk_ptrs[i].push_back(static_cast<const float *>(*b));
-
 			const bool profiling = profile->is_profile();
 			std::vector<std::unique_ptr<hip_event> > step_events[slot_count];
 			if (profiling)
@@ -660,7 +882,6 @@ namespace nnforge
 					for(size_t i = 0; i <= p->plans.size(); ++i)
 						step_events[s].emplace_back(new hip_event());
 
-			const std::vector<hip_linear_buffer_device::const_ptr> none;
 			unsigned int read_total = 0;
 			double idle = 0.0;
 			action_seconds.clear();
@@ -683,7 +904,7 @@ namespace nnforge
 					{
 						float ms = 0.0F;
 						hip_safe_call(nnf_hip_event_elapsed_ms(&ms, step_events[f.slot][i]->ev, step_events[f.slot][i + 1]->ev));
-						action_seconds[p->plans[i].key] += ms * 1.0e-3F;
+						action_seconds[p->plans[i].action] += ms * 1.0e-3F;
 					}
 				}
 				// every entry the output layers hold goes to the writer, numbered in sequence
@@ -697,18 +918,10 @@ namespace nnforge
 				}
 			};
 
-			// Whatever ends this function - the normal return or an exception from the reader, the writer or a
-			// launch - nothing declared above (device buffers, pinned staging, events) may be released while
-			// copies or kernels that use it are still in flight: this guard is destroyed first and waits.
-			struct drain_streams
-			{
-				void * streams[3];
-				~drain_streams()
-				{
-					for(void * s : streams)
-						nnf_hip_stream_synchronize(s);
-				}
-			} drain_on_exit = { { p->upload_stream, p->stream, p->download_stream } };
+			drain_streams drain_on_exit;
+			drain_on_exit.streams = p->kernel_streams;
+			drain_on_exit.streams.push_back(p->upload_stream);
+			drain_on_exit.streams.push_back(p->download_stream);
 
 			for(unsigned int packet_id = 0; ; ++packet_id)
 			{
@@ -740,51 +953,21 @@ namespace nnforge
 						hip_safe_call(nnf_hip_stream_wait_event(p->upload_stream, download_done[slot].ev));
 					}
 					for(const std::string& n : data_layer_names)
-						hip_safe_call(nnf_hip_memcpy_h2d(*buffers[slot][p->value_to_buffer[n]], staging[slot][n]->ptr,
+						hip_safe_call(nnf_hip_memcpy_h2d(*r.buffers[slot][p->value_to_buffer[n]], staging[slot][n]->ptr,
 							static_cast<size_t>(layer_config_map[n].get_neuron_count()) * sizeof(float) * entries_read, p->upload_stream));
 					hip_safe_call(nnf_hip_event_record(upload_done[slot].ev, p->upload_stream));
 
-					// kernels: need this packet's inputs and the slot's output buffers drained
-					hip_safe_call(nnf_hip_stream_wait_event(p->stream, upload_done[slot].ev));
-					if (slot_used[slot])
-						hip_safe_call(nnf_hip_stream_wait_event(p->stream, download_done[slot].ev));
-					for(size_t i = 0; i < p->plans.size(); ++i)
+					// kernels: need this packet's inputs, the slot's output buffers drained and - on the streams
+					// beside the main one, which is in order anyway - the kernels of the packet before finished
+					for(size_t ks = 0; ks < p->kernel_streams.size(); ++ks)
 					{
-						step_plan& plan = p->plans[i];
-						const unsigned int step_entries = entries_read * plan.entry_factor; // nnforge/plain/forward_propagation_plain.cpp:185
-						if (profiling)
-							hip_safe_call(nnf_hip_event_record(step_events[slot][i]->ev, p->stream));
-						std::vector<hip_linear_buffer_device::const_ptr> inputs;
-						for(int b : plan.input_buffers)
-							inputs.push_back(buffers[slot][b]);
-						if (plan.passes_input_on && (plan.output_buffer == plan.input_buffers.at(0)))
-							continue; // Dropout layers only, in place: nothing to do at inference
-						if (plan.prologue)
-						{
-							plan.desc.entry_count = step_entries;
-							plan.tester->enqueue_forward_propagation_with_prologue(p->stream, buffers[slot][plan.output_buffer], inputs.at(0), plan.desc,
-								chunk_ptrs[i].empty() ? nullptr : chunk_ptrs[i].data(), step_entries);
-						}
-						else if (plan.info.fused)
-						{
-							plan.desc.entry_count = step_entries;
-							std::vector<const float *> in_ptrs;
-							for(const hip_linear_buffer_device::const_ptr& b : inputs)
-								in_ptrs.push_back(static_cast<const float *>(*b));
-							hip_safe_call(nnf_hip_chain_forward(p->stream, &plan.desc, *buffers[slot][plan.output_buffer], in_ptrs.data(),
-								chunk_ptrs[i].empty() ? nullptr : chunk_ptrs[i].data()));
-						}
-						else
-						{
-							const std::string& layer_name = plan.info.layer_names[0];
-							std::map<std::string, std::vector<hip_linear_buffer_device::const_ptr> >::const_iterator w = p->weights.find(layer_name);
-							plan.tester->enqueue_forward_propagation(p->stream, buffers[slot][plan.output_buffer], none,
-								(w == p->weights.end()) ? none : w->second, none, inputs, none,
-								hip_linear_buffer_device::ptr(), hip_linear_buffer_device::ptr(), step_entries);
-						}
+						hip_safe_call(nnf_hip_stream_wait_event(p->kernel_streams[ks], upload_done[slot].ev));
+						if (slot_used[slot])
+							hip_safe_call(nnf_hip_stream_wait_event(p->kernel_streams[ks], download_done[slot].ev));
+						if ((ks > 0) && previous.valid)
+							hip_safe_call(nnf_hip_stream_wait_event(p->kernel_streams[ks], kernels_done[previous.slot].ev));
 					}
-					if (profiling)
-						hip_safe_call(nnf_hip_event_record(step_events[slot][p->plans.size()]->ev, p->stream));
+					p->enqueue_plan(r.buffers[slot], entries_read, r.chunk_ptrs, r.temporary, profiling ? &step_events[slot] : nullptr);
 					if (stats_on_device)
 					{
 						for(const std::string& n : output_layer_names)
@@ -792,7 +975,7 @@ namespace nnforge
 							const layer_configuration_specific& c = layer_config_map[n];
 							hip_safe_call(nnf_hip_feature_map_stat_accumulate(p->stream,
 								static_cast<nnf_hip_running_stat *>(static_cast<void *>(*stat_states[n])), *stat_workspaces[n], stat_workspace_bytes[n],
-								static_cast<const float *>(static_cast<const void *>(*buffers[slot][p->value_to_buffer.at(n)])),
+								static_cast<const float *>(static_cast<const void *>(*r.buffers[slot][p->value_to_buffer.at(n)])),
 								entries_read * output_layers_tiling_factor, c.feature_map_count, c.get_neuron_count_per_feature_map()));
 						}
 					}
@@ -802,7 +985,7 @@ namespace nnforge
 					hip_safe_call(nnf_hip_stream_wait_event(p->download_stream, kernels_done[slot].ev));
 					for(const std::string& n : output_layer_names)
 						if (!stats_on_device)
-						hip_safe_call(nnf_hip_memcpy_d2h(staging[slot][n]->ptr, *buffers[slot][p->value_to_buffer.at(n)],
+						hip_safe_call(nnf_hip_memcpy_d2h(staging[slot][n]->ptr, *r.buffers[slot][p->value_to_buffer.at(n)],
 							static_cast<size_t>(layer_config_map[n].get_neuron_count()) * sizeof(float) * entries_read * output_layers_tiling_factor, p->download_stream));
 					hip_safe_call(nnf_hip_event_record(download_done[slot].ev, p->download_stream));
 					slot_used[slot] = true;
@@ -839,6 +1022,76 @@ namespace nnforge
 			idle_seconds = static_cast<float>(idle);
 		}
 
+		forward_propagation_hip::kernel_timing forward_propagation_hip::time_kernels(
+			structured_data_bunch_reader& reader, unsigned int entry_count, unsigned int warmup, unsigned int passes)
+		{
+			if (hip_config->is_offline())
+				throw neural_network_exception("This forward_propagation_hip was created for planning only (offline configuration): it cannot run");
+			set_input_configuration_specific(reader.get_config_map());
+			const unsigned int packet = std::min(std::max(1U, entry_count), max_entry_count);
+			run_buffers r;
+			prepare_run(r, packet, 1);
+			drain_streams drain_on_exit;
+			drain_on_exit.streams = p->kernel_streams;
+
+			// one packet, read and uploaded once
+			unsigned int entries_read = 0;
+			{
+				std::map<std::string, std::unique_ptr<pinned_buffer> > staging;
+				for(const std::string& n : data_layer_names)
+					staging[n].reset(new pinned_buffer(static_cast<size_t>(layer_config_map[n].get_neuron_count()) * sizeof(float) * packet));
+				for(; entries_read < packet; ++entries_read)
+				{
+					std::map<std::string, float *> data_map;
+					for(const std::string& n : data_layer_names)
+						data_map[n] = static_cast<float *>(staging[n]->ptr) + static_cast<size_t>(entries_read) * layer_config_map[n].get_neuron_count();
+					if (!reader.read(entries_read, data_map))
+						break;
+				}
+				if (entries_read == 0)
+					throw neural_network_exception("time_kernels: the reader holds no entries");
+				for(const std::string& n : data_layer_names)
+					hip_safe_call(nnf_hip_memcpy_h2d(*r.buffers[0][p->value_to_buffer[n]], staging[n]->ptr,
+						static_cast<size_t>(layer_config_map[n].get_neuron_count()) * sizeof(float) * entries_read, nullptr));
+			}
+
+			hip_event start, stop, pass_done;
+			// a pass: every kernel stream behind the end of the pass before (the main one is in order anyway)
+			auto one_pass = [&](bool first)
+			{
+				if (!first)
+					for(size_t ks = 1; ks < p->kernel_streams.size(); ++ks)
+						hip_safe_call(nnf_hip_stream_wait_event(p->kernel_streams[ks], pass_done.ev));
+				p->enqueue_plan(r.buffers[0], entries_read, r.chunk_ptrs, r.temporary, nullptr);
+				hip_safe_call(nnf_hip_event_record(pass_done.ev, p->stream));
+			};
+			hip_safe_call(nnf_hip_device_synchronize());
+			for(unsigned int i = 0; i < warmup; ++i)
+				one_pass(i == 0);
+			hip_safe_call(nnf_hip_device_synchronize());
+
+			kernel_timing res;
+			res.entry_count = entries_read;
+			res.launch_count = 0;
+			for(const step_plan& plan : p->plans)
+				res.launch_count += plan.launches_nothing() ? 0 : 1;
+			const std::chrono::high_resolution_clock::time_point t0 = std::chrono::high_resolution_clock::now();
+			hip_safe_call(nnf_hip_event_record(start.ev, p->stream));
+			for(size_t ks = 1; ks < p->kernel_streams.size(); ++ks)
+				hip_safe_call(nnf_hip_stream_wait_event(p->kernel_streams[ks], start.ev));
+			for(unsigned int i = 0; i < passes; ++i)
+				one_pass(i == 0);
+			hip_safe_call(nnf_hip_event_record(stop.ev, p->stream));
+			hip_safe_call(nnf_hip_device_synchronize());
+			const std::chrono::duration<float> wall = std::chrono::high_resolution_clock::now() - t0;
+			float ms = 0.0F;
+			hip_safe_call(nnf_hip_event_elapsed_ms(&ms, start.ev, stop.ev));
+			const float n = static_cast<float>(std::max(1U, passes));
+			res.wall_seconds_per_pass = wall.count() / n;
+			res.device_seconds_per_pass = ms * 1.0e-3F / n;
+			return res;
+		}
+
 		float forward_propagation_hip::get_max_bytes_per_second() const
 		{
 			return 8.0e12F; // MI355X HBM3E peak
@@ -860,6 +1113,8 @@ namespace nnforge
 			, hip_max_global_memory_usage_ratio(0.9F)
 			, hip_fuse(true)
 			, hip_dont_share_buffers(false)
+			, hip_single_command_stream(false)
+			, hip_kernel_stream_count(hip_running_configuration::default_kernel_stream_count)
 			, hip_max_entry_count(4096)
 		{
 		}
@@ -868,7 +1123,8 @@ namespace nnforge
 		{
 			hip::init();
 			hip_config = hip_running_configuration::const_ptr(new hip_running_configuration(
-				hip_device_id, hip_max_global_memory_usage_ratio, hip_fuse, hip_dont_share_buffers, hip_max_entry_count));
+				hip_device_id, hip_max_global_memory_usage_ratio, hip_fuse, hip_dont_share_buffers, hip_max_entry_count,
+				hip_single_command_stream ? 1 : std::max(1, hip_kernel_stream_count)));
 		}
 
 		forward_propagation_factory::ptr factory_generator_hip::create_forward_propagation_factory() const
@@ -894,6 +1150,7 @@ namespace nnforge
 			std::vector<bool_option> res;
 			res.push_back(bool_option("hip_fuse", &hip_fuse, true, "Fuse runs of element-wise layers (BatchNorm, activations, Add) into single kernel launches"));
 			res.push_back(bool_option("hip_dont_share_buffers", &hip_dont_share_buffers, false, "Don't share buffers between layers. Switch it on if you suspect a bug in there"));
+			res.push_back(bool_option("hip_single_command_stream", &hip_single_command_stream, false, "Use single stream for kernels. Switch it on if you suspect a bug in there"));
 			return res;
 		}
 
@@ -909,6 +1166,7 @@ namespace nnforge
 			std::vector<int_option> res;
 			res.push_back(int_option("hip_device_id,D", &hip_device_id, 0, "HIP device ID"));
 			res.push_back(int_option("hip_max_entry_count", &hip_max_entry_count, 4096, "Upper bound of entries processed per packet"));
+			res.push_back(int_option("hip_kernel_stream_count", &hip_kernel_stream_count, hip_running_configuration::default_kernel_stream_count, "Streams the kernels of independent layers are spread over"));
 			return res;
 		}
 	}

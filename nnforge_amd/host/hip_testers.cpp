@@ -36,12 +36,16 @@ namespace nnforge
 				nnf_hip_free(buf);
 		}
 
-		hip_running_configuration::hip_running_configuration(int device_id, float max_global_memory_usage_ratio, bool fuse_layers, bool dont_share_buffers, int max_entry_count)
+		constexpr int hip_running_configuration::default_kernel_stream_count;
+
+		hip_running_configuration::hip_running_configuration(int device_id, float max_global_memory_usage_ratio, bool fuse_layers, bool dont_share_buffers, int max_entry_count,
+			int kernel_stream_count)
 			: device_id(device_id)
 			, max_global_memory_usage_ratio(max_global_memory_usage_ratio)
 			, fuse_layers(fuse_layers)
 			, dont_share_buffers(dont_share_buffers)
 			, max_entry_count(max_entry_count)
+			, kernel_stream_count(kernel_stream_count)
 			, global_memory_size(0)
 			, compute_unit_count(0)
 			, wavefront_size(0)
@@ -61,9 +65,11 @@ namespace nnforge
 		}
 
 		hip_running_configuration::const_ptr hip_running_configuration::create_offline(
-			unsigned long long global_memory_size, float max_global_memory_usage_ratio, bool fuse_layers, bool dont_share_buffers, int max_entry_count)
+			unsigned long long global_memory_size, float max_global_memory_usage_ratio, bool fuse_layers, bool dont_share_buffers, int max_entry_count,
+			int kernel_stream_count)
 		{
 			std::shared_ptr<hip_running_configuration> res(new hip_running_configuration());
+			res->kernel_stream_count = kernel_stream_count;
 			res->device_id = -1;
 			res->max_global_memory_usage_ratio = max_global_memory_usage_ratio;
 			res->fuse_layers = fuse_layers;
@@ -96,7 +102,8 @@ namespace nnforge
 			out << "Device name = " << config.device_name << std::endl;
 			out << "Global memory = " << (config.global_memory_size >> 20) << " MB" << std::endl;
 			out << "Compute units = " << config.compute_unit_count << ", wavefront " << config.wavefront_size << ", clock " << (config.clock_khz / 1000) << " MHz" << std::endl;
-			out << "Memory usage ratio = " << config.max_global_memory_usage_ratio << ", fuse element-wise layers = " << (config.fuse_layers ? "yes" : "no") << std::endl;
+			out << "Memory usage ratio = " << config.max_global_memory_usage_ratio << ", fuse element-wise layers = " << (config.fuse_layers ? "yes" : "no")
+				<< ", kernel streams = " << config.kernel_stream_count << std::endl;
 			return out;
 		}
 
@@ -138,6 +145,28 @@ namespace nnforge
 				res.push_back(buf);
 			}
 			return res;
+		}
+
+		std::vector<hip_linear_buffer_device::const_ptr> layer_tester_hip::set_get_data_custom(layer_data_custom::const_ptr host_data_custom)
+		{
+			notify_data_custom(host_data_custom);
+			std::vector<hip_linear_buffer_device::const_ptr> res;
+			if (!host_data_custom)
+				return res;
+			for(const std::vector<int>& chunk : *host_data_custom)
+			{
+				const size_t bytes = chunk.size() * sizeof(int);
+				hip_linear_buffer_device::ptr buf(new hip_linear_buffer_device(bytes));
+				if (bytes > 0)
+					hip_safe_call(nnf_hip_memcpy_h2d(*buf, chunk.data(), bytes, nullptr));
+				res.push_back(buf);
+			}
+			return res;
+		}
+
+		std::vector<hip_linear_buffer_device::const_ptr> layer_tester_hip::get_persistent_working_data() const
+		{
+			return std::vector<hip_linear_buffer_device::const_ptr>();
 		}
 
 		void layer_tester_hip::enqueue_forward_propagation_with_prologue(void *, hip_linear_buffer_device::ptr, hip_linear_buffer_device::const_ptr,

@@ -230,25 +230,27 @@ namespace nnforge
 			float total_seconds,
 			float max_flops,
 			float max_bytes_per_second,
-			const std::map<std::string, float>& seconds,
-			const std::map<std::string, float>& flops_per_entry,
-			const std::map<std::string, float>& bytes_per_entry,
-			const std::map<std::string, std::string>& types)
+			const std::map<layer_name_with_action, float>& seconds,
+			const std::map<layer_name_with_action, float>& flops_per_entry,
+			const std::map<layer_name_with_action, float>& bytes_per_entry,
+			const std::map<layer_name_with_action, std::string>& names,
+			const std::map<layer_name_with_action, std::string>& types)
 		{
-			std::vector<std::pair<std::string, float> > entries(seconds.begin(), seconds.end());
-			std::sort(entries.begin(), entries.end(),
-				[] (const std::pair<std::string, float>& a, const std::pair<std::string, float>& b) { return a.second > b.second; });
+			typedef std::pair<layer_name_with_action, float> entry;
+			std::vector<entry> entries(seconds.begin(), seconds.end());
+			std::sort(entries.begin(), entries.end(), [] (const entry& a, const entry& b) { return a.second > b.second; });
 			std::ofstream out(path.c_str(), std::ios_base::out | std::ios_base::trunc);
 			if (!out)
 				throw neural_network_exception("Cannot open " + path + " for writing");
 			out << "Layer\tLayer type\tAction\tTime of total\tRelative to peak perf\tAbsolute time, seconds\tAbsolute perf, GFLOPS\tGB/s\tRelative to peak bandwidth" << std::endl;
-			for(const std::pair<std::string, float>& e : entries)
+			for(const entry& e : entries)
 			{
-				const auto lookup = [&e] (const std::map<std::string, float>& m) { std::map<std::string, float>::const_iterator it = m.find(e.first); return (it == m.end()) ? 0.0F : it->second; };
+				const auto lookup = [&e] (const std::map<layer_name_with_action, float>& m) { std::map<layer_name_with_action, float>::const_iterator it = m.find(e.first); return (it == m.end()) ? 0.0F : it->second; };
+				const auto text = [&e] (const std::map<layer_name_with_action, std::string>& m, const std::string& otherwise) { std::map<layer_name_with_action, std::string>::const_iterator it = m.find(e.first); return (it == m.end()) ? otherwise : it->second; };
 				const float gflops = lookup(flops_per_entry) * static_cast<float>(entry_count) / e.second * 1.0e-9F;
 				const float gbps = lookup(bytes_per_entry) * static_cast<float>(entry_count) / e.second * 1.0e-9F;
-				std::map<std::string, std::string>::const_iterator type = types.find(e.first);
-				out << e.first << "\t" << ((type == types.end()) ? std::string() : type->second) << "\tforward";
+				// an action that covers several layers lists all of them (and their types) in the first two columns
+				out << text(names, e.first.get_name()) << "\t" << text(types, std::string()) << "\t" << e.first.get_action().str();
 				out << "\t" << percent(e.second / total_seconds);
 				out << "\t" << ((max_flops > 0.0F) ? percent(gflops / (max_flops * 1.0e-9F)) : std::string("NA"));
 				out << "\t" << e.second << "\t" << gflops << "\t" << gbps;
@@ -363,8 +365,14 @@ namespace nnforge
 			dump_action_performance(
 				profile->get_path_to_unique_file("forward_prop_perf_per_layer_action", "csv"),
 				res.entry_processed_count, res.total_seconds, get_max_flops(), get_max_bytes_per_second(),
-				last_action_seconds, action_flops_per_entry, action_bytes_per_entry, action_layer_types);
+				last_action_seconds, action_flops_per_entry, action_bytes_per_entry, action_layer_names, action_layer_types);
 		return res;
+	}
+
+	std::string forward_propagation::get_action_layer_names(const layer_name_with_action& action) const
+	{
+		std::map<layer_name_with_action, std::string>::const_iterator it = action_layer_names.find(action);
+		return (it == action_layer_names.end()) ? action.get_name() : it->second;
 	}
 
 	float forward_propagation::get_max_flops() const

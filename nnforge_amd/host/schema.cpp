@@ -482,6 +482,12 @@ namespace nnforge
 		return (it == data_list.end()) ? layer_data::ptr() : it->second;
 	}
 
+	layer_data_custom::ptr network_data::find_custom(const std::string& instance_name) const
+	{
+		std::map<std::string, layer_data_custom::ptr>::const_iterator it = data_custom_list.find(instance_name);
+		return (it == data_custom_list.end()) ? layer_data_custom::ptr() : it->second;
+	}
+
 	layer_data::ptr network_data::get(const std::string& instance_name) const
 	{
 		layer_data::ptr res = find(instance_name);

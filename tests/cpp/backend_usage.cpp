@@ -154,8 +154,8 @@ int main(int argc, char ** argv)
 					++mismatches;
 			}
 		}
-		for(const std::pair<const std::string, float>& a : fp->get_last_action_seconds())
-			std::cout << "action " << a.first << ": " << a.second << " s" << std::endl;
+		for(const std::pair<const layer_name_with_action, float>& a : fp->get_last_action_seconds())
+			std::cout << "action " << a.first.get_name() << " " << a.first.get_action().str() << " (" << fp->get_action_layer_names(a.first) << "): " << a.second << " s" << std::endl;
 		if (mismatches != 0)
 		{
 			std::cout << mismatches << " mismatches" << std::endl;

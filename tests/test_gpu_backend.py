@@ -119,7 +119,8 @@ def test_cpp_application_uses_the_backend_like_a_reference_backend(tmp_path):
     lines = proc.stdout.strip().splitlines()
     assert lines[-1] == "ok", proc.stdout
     assert any("[fused] main_bn+res+res_prelu <- conv_shortcut, conv_main" in l for l in lines), proc.stdout
-    assert any(l.startswith("action main_bn+res+res_prelu:") for l in lines), proc.stdout
+    # actions are keyed the reference's way (layer_name_with_action): a fused launch reports under its last layer
+    assert any(l.startswith("action res_prelu forward (main_bn+res+res_prelu):") for l in lines), proc.stdout
     assert any("13 entries" in l for l in lines), proc.stdout
 
 
