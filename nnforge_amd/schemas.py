@@ -1,0 +1,117 @@
+"""Networks as Python data and as nnForge's text-format schema (nnforge/proto/nnforge.proto): the form the hip backend
+reads. Used by the benchmark (the ResNet-50 post-convolution graph) and by the tests (small networks)."""
+
+from nnforge_amd import workloads
+
+
+def L(type_name, name, inputs=(), **params):
+    return {"type": type_name, "name": name, "inputs": list(inputs), "params": params}
+
+
+PARAM_BLOCK = {"BatchNorm": "batch_norm_param", "ReLU": "relu_param", "PReLU": "prelu_param", "TanH": "tanh_param",
+               "Add": "add_param", "AverageSubsampling": "average_subsampling_param", "Dropout": "dropout_param",
+               "Maxout": "maxout_param", "MaxSubsampling": "max_subsampling_param"}
+
+
+def schema_text(layers, name="test_net"):
+    out = ['name: "%s"' % name]
+    for l in layers:
+        out.append("layer {")
+        out.append('\ttype: "%s"' % l["type"])
+        out.append('\tname: "%s"' % l["name"])
+        for i in l["inputs"]:
+            out.append('\tinput_layer_name: "%s"' % i)
+        p = l["params"]
+        if p and l["type"] in PARAM_BLOCK:
+            out.append("\t%s {" % PARAM_BLOCK[l["type"]])
+            for k, v in p.items():
+                if k == "windows":
+                    for d, w in enumerate(v):
+                        extra = ""
+                        if p.get("round_ups") and p["round_ups"][d]:
+                            extra += " round_up: true"
+                        if p.get("strides"):
+                            extra += " stride: %d" % p["strides"][d]
+                        out.append("\t\tdimension_param { subsampling_size: %d%s }" % (w, extra))
+                elif k in ("strides", "round_ups"):
+                    continue
+                elif k == "subsampled":
+                    for size in v:
+                        out.append("\t\tdimension_param { subsampled_size: %d }" % size)
+                elif k == "fm_subsampled":
+                    out.append("\t\tfeature_map_param { subsampled_size: %d }" % v)
+                elif k == "entry_window":
+                    out.append("\t\tentry_param { subsampling_size: %d }" % v)
+                elif k == "fm_window":
+                    out.append("\t\tfeature_map_param { subsampling_size: %d }" % v)
+                elif k == "function":
+                    out.append("\t\tfunction: %s" % v)
+                elif isinstance(v, bool):
+                    out.append("\t\t%s: %s" % (k, "true" if v else "false"))
+                else:
+                    out.append("\t\t%s: %r" % (k, v))
+            out.append("\t}")
+        out.append("}")
+    return "\n".join(out) + "\n"
+
+
+def resnet50_post_convolution(with_pool1=False):
+    """Everything behind the convolutions of ResNet-50 as examples/imagenet/imagenet_toolset.cpp:476-550 and 729-831 build it,
+    with the layer names used there; every convolution's output is a data layer of the same name (conv1, resNx_shortcut,
+    resNx_reduce_fm, resNx_bottleneck, resNx_restore_fm, logits). The residual of a block that keeps its shape is the output of
+    the block before, as in the network. with_pool1: the 3x3 max pooling every 2 (rounded up) behind relu1.
+    Returns (layers, {data layer: (feature maps, [width, height])}, output layer names): the outputs are the values only
+    convolutions (or nothing) consume - without them the graph would have no sinks."""
+    layers, inputs, outputs = [], {}, []
+
+    def data(name, fm, size):
+        layers.append(L("Data", name))
+        inputs[name] = (fm, [size, size])
+
+    def bn(name, source, fm):
+        layers.append(L("BatchNorm", name, [source], feature_map_count=fm))
+
+    data("conv1", 64, 112)
+    bn("conv1_bn", "conv1", 64)
+    layers.append(L("ReLU", "relu1", ["conv1_bn"]))
+    last = "relu1"
+    if with_pool1:
+        layers.append(L("MaxSubsampling", "pool1", ["relu1"], windows=[3, 3], strides=[2, 2], round_ups=[True, True]))
+        last = "pool1"
+    outputs.append(last)
+    last_fm, resolution, restored = 64, 56, 256
+    for stage, block_count in enumerate(workloads.RESNET50_BLOCKS):
+        for block in range(block_count):
+            reduction = (block == 0) and (stage != 0)
+            if reduction:
+                restored *= 2
+            bottleneck = restored // 4
+            name = "res%d%s" % (stage + 2, chr(ord("a") + block))
+            to_add = last
+            if reduction or (last_fm != restored):
+                data(name + "_shortcut", restored, resolution // 2 if reduction else resolution)
+                bn(name + "_shortcut_bn", name + "_shortcut", restored)
+                to_add = name + "_shortcut_bn"
+            # the stride of 2 sits on the 3x3 convolution: reduce_fm still runs at the resolution before
+            data(name + "_reduce_fm", bottleneck, resolution)
+            bn(name + "_reduce_fm_bn", name + "_reduce_fm", bottleneck)
+            layers.append(L("ReLU", name + "_reduce_fm_relu", [name + "_reduce_fm_bn"]))
+            outputs.append(name + "_reduce_fm_relu")
+            if reduction:
+                resolution //= 2
+            data(name + "_bottleneck", bottleneck, resolution)
+            bn(name + "_bottleneck_bn", name + "_bottleneck", bottleneck)
+            layers.append(L("ReLU", name + "_bottleneck_relu", [name + "_bottleneck_bn"]))
+            outputs.append(name + "_bottleneck_relu")
+            data(name + "_restore_fm", restored, resolution)
+            bn(name + "_restore_fm_bn", name + "_restore_fm", restored)
+            layers.append(L("Add", name, [to_add, name + "_restore_fm_bn"]))
+            layers.append(L("ReLU", name + "_relu", [name]))
+            outputs.append(name + "_relu")
+            last, last_fm = name + "_relu", restored
+    layers.append(L("AverageSubsampling", "pool5", [last], windows=[7, 7], alpha=1.0 / 49.0))
+    outputs.append("pool5")
+    data("logits", 1000, 1)
+    layers.append(L("Softmax", "prob", ["logits"]))
+    outputs.append("prob")
+    return layers, inputs, outputs

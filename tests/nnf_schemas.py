@@ -8,55 +8,7 @@ import nnf_testing as T
 import oracle
 
 
-def L(type_name, name, inputs=(), **params):
-    return {"type": type_name, "name": name, "inputs": list(inputs), "params": params}
-
-
-PARAM_BLOCK = {"BatchNorm": "batch_norm_param", "ReLU": "relu_param", "PReLU": "prelu_param", "TanH": "tanh_param",
-               "Add": "add_param", "AverageSubsampling": "average_subsampling_param", "Dropout": "dropout_param",
-               "Maxout": "maxout_param", "MaxSubsampling": "max_subsampling_param"}
-
-
-def schema_text(layers, name="test_net"):
-    out = ['name: "%s"' % name]
-    for l in layers:
-        out.append("layer {")
-        out.append('\ttype: "%s"' % l["type"])
-        out.append('\tname: "%s"' % l["name"])
-        for i in l["inputs"]:
-            out.append('\tinput_layer_name: "%s"' % i)
-        p = l["params"]
-        if p and l["type"] in PARAM_BLOCK:
-            out.append("\t%s {" % PARAM_BLOCK[l["type"]])
-            for k, v in p.items():
-                if k == "windows":
-                    for d, w in enumerate(v):
-                        extra = ""
-                        if p.get("round_ups") and p["round_ups"][d]:
-                            extra += " round_up: true"
-                        if p.get("strides"):
-                            extra += " stride: %d" % p["strides"][d]
-                        out.append("\t\tdimension_param { subsampling_size: %d%s }" % (w, extra))
-                elif k in ("strides", "round_ups"):
-                    continue
-                elif k == "subsampled":
-                    for size in v:
-                        out.append("\t\tdimension_param { subsampled_size: %d }" % size)
-                elif k == "fm_subsampled":
-                    out.append("\t\tfeature_map_param { subsampled_size: %d }" % v)
-                elif k == "entry_window":
-                    out.append("\t\tentry_param { subsampling_size: %d }" % v)
-                elif k == "fm_window":
-                    out.append("\t\tfeature_map_param { subsampling_size: %d }" % v)
-                elif k == "function":
-                    out.append("\t\tfunction: %s" % v)
-                elif isinstance(v, bool):
-                    out.append("\t\t%s: %s" % (k, "true" if v else "false"))
-                else:
-                    out.append("\t\t%s: %r" % (k, v))
-            out.append("\t}")
-        out.append("}")
-    return "\n".join(out) + "\n"
+from nnforge_amd.schemas import L, PARAM_BLOCK, schema_text  # noqa: F401 (re-exported: the tests build their networks with these)
 
 
 def make_weights(layers, gen):

@@ -215,6 +215,71 @@ def test_plan_of_the_inception_like_block():
     assert rep["steps"][4]["inputs"] == ["b1_relu", "b2_abs", "b3_prelu", "pool1"]
 
 
+def test_plan_of_the_resnet50_post_convolution_graph_equals_the_benchmark_group_list():
+    """Config 4 as a network: the graph examples/imagenet/imagenet_toolset.cpp:476-550, 729-831 builds, convolution outputs as
+    data layers. The driver's fusion pass must arrive at the 49 groups nnforge_amd.workloads lists by hand (kind, shape,
+    order), then the 7x7 average and the softmax; the residual of a block that keeps its shape is the block before."""
+    from nnforge_amd import schemas, workloads as w
+
+    layers, configs, outputs = schemas.resnet50_post_convolution()
+    assert len([l for l in layers if l["type"] == "BatchNorm"]) == 53   # 1 stem + 16 blocks x 3 + 4 shortcuts
+    rep = plan(layers, configs, outputs)
+    steps = rep["steps"]
+    groups = w.resnet50_groups(1)
+    assert len(steps) == len(groups) + 2 == 51
+    by_name = {l["name"]: l for l in layers}
+    shapes = dict(configs)
+    for l in layers:   # every layer here keeps the shape of its first input, but for the pooling
+        if l["type"] != "Data":
+            shapes[l["name"]] = shapes[l["inputs"][0]]
+    per_entry_bytes = 0
+    for step, g in zip(steps, groups):
+        assert step["fused"]
+        kinds = [by_name[n]["type"] for n in step["layers"]]
+        fm, dims = shapes[step["layers"][-1]]
+        assert (fm, dims[0] * dims[1]) == (g.feature_map_count, g.plane), (step, g.name)
+        assert len(step["inputs"]) == len(g.arms)
+        want = {1: ["BatchNorm", "ReLU"], 2: ["BatchNorm", "Add", "ReLU"]}[len(g.arms)]
+        if len(g.arms) == 2 and g.arms[0]:
+            want = ["BatchNorm"] + want   # the first block of a stage: batch norm on the shortcut as well
+        assert kinds == want, (step, g.name)
+        per_entry_bytes += w.group_algorithmic_bytes(g)
+    assert steps[49]["layers"] == ["pool5"] and steps[49]["inputs"] == ["res5c_relu"] and not steps[49]["fused"]
+    assert steps[50]["layers"] == ["prob"] and steps[50]["inputs"] == ["logits"]
+    # the bytes the launches move per entry are the benchmark's algorithmic bytes (weights aside: 4 bytes per weight)
+    def floats(name):
+        fm, dims = shapes[name]
+        return fm * dims[0] * dims[1]
+
+    weights_bytes = sum(4 * (4 if kind == "bn" else 1) * c for g in groups for kind, c in g.chunks)
+    g_bytes, p_bytes, s_bytes = w.resnet50_algorithmic_bytes(1)
+    assert per_entry_bytes == g_bytes
+    moved = sum(floats(name) for name in configs)                                                 # every data layer read once
+    moved += sum(floats(s["layers"][-1]) for s in steps[:49])                                     # every group's output written
+    moved += sum(floats(src) for s in steps[:49] for src in s["inputs"] if src not in configs)    # residuals read back
+    moved += 2048 * 49 + 2048 + 1000                                                              # pool5 input and output, prob output
+    assert 4 * moved == g_bytes - weights_bytes + p_bytes + s_bytes
+    # residual chains: a block that keeps its shape reads the block before - on its stream, or behind an event
+    producer = {s["layers"][-1]: i for i, s in enumerate(steps)}
+    chained = 0
+    for i, s in enumerate(steps):
+        for source in s["inputs"]:
+            if source in producer:
+                j = producer[source]
+                assert j < i and (steps[j]["stream"] == s["stream"] or any(w_ >= j and steps[w_]["stream"] == steps[j]["stream"] for w_ in s["after"])), (i, s)
+                chained += 1
+    assert chained == 12 + 1   # 16 blocks minus the 4 with a shortcut convolution, and pool5 behind res5c_relu
+    assert len({s["stream"] for s in steps}) == 3
+    # one kernel stream: the same steps, nothing to wait for
+    single = plan(layers, configs, outputs, kernel_stream_count=1)
+    assert [s["layers"] for s in single["steps"]] == [s["layers"] for s in steps]
+    assert all(s["stream"] == 0 and not s["after"] for s in single["steps"])
+    # with the stem's pooling in the graph, batch norm and ReLU are applied on the way into the pooling kernel
+    layers, configs, outputs = schemas.resnet50_post_convolution(with_pool1=True)
+    rep = plan(layers, configs, outputs)
+    assert len(rep["steps"]) == 51 and rep["steps"][0]["layers"] == ["conv1_bn", "relu1", "pool1"] and rep["steps"][0]["fused"]
+
+
 def stem_net(c=8):
     """BatchNorm -> ReLU -> overlapping max pooling, then TanH -> Absolute -> 2x2 average pooling (the stage of
     nnForge's GTSRB example, examples/gtsrb/schema.txt), then a global average."""

@@ -329,6 +329,29 @@ def test_inference_from_data_set_files_to_data_set_files(tmp_path):
         backend.run_dataset(S.schema_text(layers), weights, {"images": tmp_path / "nowhere.dt"}, outputs)
 
 
+@pytest.mark.parametrize("streams", [0, 1])
+def test_resnet50_post_convolution_graph_layer_by_layer(streams):
+    """Config 4 through the driver at a small entry count: every output of the 51 launches against the oracle run layer by
+    layer (bit for bit; softmax to 1e-5), with the kernels on three streams (the default) and on one."""
+    from nnforge_amd import schemas
+
+    gen = T.rng(62, 0)
+    n = 3
+    layers, configs, outputs = schemas.resnet50_post_convolution()
+    weights = S.make_weights(layers, gen)
+    inputs = {name: T.normal(gen, (n, fm, dims[1], dims[0])) for name, (fm, dims) in sorted(configs.items())}
+    inputs["logits"] = T.normal(gen, (n, 1000, 1, 1), 4.0)
+    values = S.evaluate(layers, weights, inputs)
+    got, rep = run(layers, weights, inputs, outputs, values, max_entry_count=2, kernel_stream_count=streams)
+    assert len(rep["steps"]) == 51 and rep["entries"] == n
+    assert len({s["stream"] for s in rep["steps"]}) == (1 if streams == 1 else 3)
+    for name in outputs:
+        if name == "prob":
+            assert np.all(np.abs(got[name] - values[name]) <= 1e-5 * np.abs(values[name])), name
+        else:
+            assert_bits(got[name], values[name], name)
+
+
 def test_dropout_only_network():
     """Dropout straight from the data layer to the output: in place there is nothing to launch."""
     gen = T.rng(58, 0)
