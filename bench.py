@@ -206,8 +206,10 @@ def bench_group(runner, label, group, steps, warmup, make_input=None):
     sets = rotation_sets(alg)
     launch = runner.prepare_group(group, sets, make_input)
     wall, ev = runner.time_steps(launch, steps, warmup)
+    queued = time_steps_queued(runner, launch, min(max(steps, 50), 400), hold_ms=8.0)
     entry = result_entry(label, alg, w.group_elements(group), wall, ev, 1,
-                         {"buffer_sets": sets, "shape": [group.entry_count, group.feature_map_count, group.plane]})
+                         {"buffer_sets": sets, "shape": [group.entry_count, group.feature_map_count, group.plane],
+                          "queued_event_ms_per_step": queued * 1e3, "queued_event_gbps": alg / queued / 1e9})
     del launch
     runner.torch.cuda.empty_cache()
     return entry
@@ -242,7 +244,50 @@ def bench_softmax(runner, steps, warmup):
                                  "queued behind a spin kernel"})
 
 
-def bench_resnet50(runner, steps, warmup, n=64):
+def resnet50_network(n, gen):
+    """Config 4 as a network for the hip backend: schema text, weights, data layer shapes, output names."""
+    from nnforge_amd import schemas
+
+    layers, configs, outputs = schemas.resnet50_post_convolution()
+    weights = {}
+    for l in layers:
+        if l["type"] == "BatchNorm":
+            c = l["params"]["feature_map_count"]
+            weights[l["name"]] = [gen.random(c, dtype=np.float32) + np.float32(0.5), gen.standard_normal(c, dtype=np.float32) * np.float32(0.3),
+                                  gen.standard_normal(c, dtype=np.float32) * np.float32(0.3), gen.random(c, dtype=np.float32) + np.float32(0.6)]
+    return schemas.schema_text(layers, "ResNet-50 post-convolution"), weights, configs, outputs
+
+
+def bench_resnet50(runner, steps, warmup, n=64, kernel_stream_count=0):
+    """Config 4 through the product driver: the ResNet-50 post-convolution graph (convolution outputs as data layers) handed to
+    forward_propagation_hip, whose fusion pass makes the 49 groups + average + softmax and enqueues them on its kernel streams;
+    one packet of n entries resident in device memory, `steps` passes of the launch plan timed by the driver itself
+    (device synchronisation on both sides; events on its kernel stream). The group list of nnforge_amd.workloads is only the
+    cross-check that the driver arrives at the same launches."""
+    from nnforge_amd import backend, workloads as w
+
+    gen = np.random.Generator(np.random.MT19937(SEED + 4))
+    text, weights, configs, outputs = resnet50_network(n, gen)
+    largest = max(fm * dims[0] * dims[1] for fm, dims in configs.values())
+    pool = gen.standard_normal(n * largest, dtype=np.float32)
+    rep = backend.time_kernels(text, weights, configs, outputs, warmup=warmup, passes=steps, shared_input_pool=pool, entry_count=n,
+                               max_entry_count=n, kernel_stream_count=kernel_stream_count)
+    groups = w.resnet50_groups(n)
+    assert rep["timed_entries"] == n and rep["launches"] == len(groups) + 2, rep["raw"]
+    for step, g in zip(rep["steps"], groups):
+        assert len(step["inputs"]) == len(g.arms) and len(step["layers"]) == sum(len(a) for a in g.arms) + len(g.tail) + (len(g.arms) > 1), (step, g.name)
+    g_bytes, p_bytes, s_bytes = w.resnet50_algorithmic_bytes(n)
+    pool_shape, sm_shape = w.resnet50_tail(n)
+    elements = sum(w.group_elements(g) for g in groups) + pool_shape[0] * pool_shape[1] + sm_shape[0] * sm_shape[1]
+    return result_entry("config4: ResNet-50 post-convolution stack N=%d (49 fused groups + 7x7 average + softmax) through forward_propagation_hip" % n,
+                        g_bytes + p_bytes + s_bytes, elements, rep["wall_seconds_per_pass"], rep["device_seconds_per_pass"], rep["launches"],
+                        {"kernel_streams": len({st["stream"] for st in rep["steps"]}),
+                         "note": "timed inside the C++ driver (forward_propagation_hip::time_kernels): one resident packet, the launch plan "
+                                 "enqueued on the driver's kernel streams, nothing copied to or from the host in the timed region"})
+
+
+def bench_resnet50_direct(runner, steps, warmup, n=64):
+    """The same 51 launches issued one by one at the C ABI from this script, one stream: the cross-check beside the driver's figure."""
     from nnforge_amd import workloads as w
 
     groups = w.resnet50_groups(n)
@@ -266,8 +311,7 @@ def bench_resnet50(runner, steps, warmup, n=64):
     wall, ev = runner.time_steps(step, steps, warmup)
     g_bytes, p_bytes, s_bytes = w.resnet50_algorithmic_bytes(n)
     elements = sum(w.group_elements(g) for g in groups) + pool_shape[0] * pool_shape[1] + sm_shape[0] * sm_shape[1]
-    entry = result_entry("config4: ResNet-50 post-convolution stack N=%d (49 fused groups + 7x7 average + softmax)" % n,
-                         g_bytes + p_bytes + s_bytes, elements, wall, ev, len(groups) + 2)
+    entry = result_entry("config4 launches issued at the C ABI from Python, one stream (cross-check)", g_bytes + p_bytes + s_bytes, elements, wall, ev, len(groups) + 2)
     del launches
     runner.torch.cuda.empty_cache()
     return entry
@@ -434,6 +478,55 @@ def bench_copy(runner, steps, warmup):
 
     wall, ev = runner.time_steps(launch, steps, warmup)
     return result_entry("copy kernel 256 MiB -> 256 MiB", 2 * 4 * count, count, wall, ev, 1, {"buffer_sets": sets})
+
+
+def bench_yardsticks(runner, steps, warmup):
+    """What independent copy routines reach on the same buffers, beside the library's own kernels: the runtime's device-to-device
+    copy (hipMemcpyAsync through nnf_hip_memcpy_d2d), torch's copy_ and add kernels, the library's copy kernel and its fused
+    batch_norm -> rectified_linear, at three tensor sizes. GB/s of bytes read + bytes written, device time with the launches
+    queued behind a spin kernel (so that the host's launch calls do not count)."""
+    from nnforge_amd import workloads as w
+
+    torch, lib, capi, stream = runner.torch, runner.lib, runner.capi, runner.stream
+    rows = []
+    for label, n, c, plane in (("25.7 MB per tensor (config 0)", 32, 64, 3136), ("268 MB per tensor", 107, 200, 3136), ("411 MB per tensor (config 2)", 128, 256, 3136)):
+        count = n * c * plane
+        sets = rotation_sets(8 * count, cap=16)
+        a = [runner.randn(count) for _ in range(sets)]
+        b = [runner.randn(count) for _ in range(sets)]
+        out = [runner.empty(count) for _ in range(sets)]
+        reps = max(10, min(steps, int(2e9 // (8 * count))))
+        group = w.bn_relu("bn_relu", n, c, plane)
+        chunks = runner.bn_chunks(c)
+        chunk_ptrs = capi.pointer_array([t.data_ptr() for t in chunks])
+        desc = capi.make_desc(n, c, plane, group.arms, group.tail)
+        in_ptrs = [capi.pointer_array([t.data_ptr()]) for t in a]
+        desc2 = capi.make_desc(n, c, plane, [[], []], [], has_add=True)
+        in2_ptrs = [capi.pointer_array([x.data_ptr(), y.data_ptr()]) for x, y in zip(a, b)]
+
+        def check(rc):
+            if rc != 0:
+                raise RuntimeError(capi.error_string(rc))
+
+        candidates = [
+            ("own copy kernel (1 read, 1 write)", 2, lambda i: check(lib.nnf_hip_copy_kernel(stream, out[i % sets].data_ptr(), a[i % sets].data_ptr(), 4 * count))),
+            ("own batch_norm -> rectified_linear (1 read, 1 write)", 2, lambda i: check(lib.nnf_hip_chain_forward(stream, ctypes.byref(desc), out[i % sets].data_ptr(), in_ptrs[i % sets], chunk_ptrs))),
+            ("hipMemcpyAsync device to device (1 read, 1 write)", 2, lambda i: check(lib.nnf_hip_memcpy_d2d(out[i % sets].data_ptr(), a[i % sets].data_ptr(), 4 * count, stream))),
+            ("torch copy_ (1 read, 1 write)", 2, lambda i: out[i % sets].copy_(a[i % sets])),
+            ("own add of two tensors (2 reads, 1 write)", 3, lambda i: check(lib.nnf_hip_chain_forward(stream, ctypes.byref(desc2), out[i % sets].data_ptr(), in2_ptrs[i % sets], None))),
+            ("torch add(a, b, out=c) (2 reads, 1 write)", 3, lambda i: torch.add(a[i % sets], b[i % sets], out=out[i % sets])),
+        ]
+        for name, tensors, fn in candidates:
+            for i in range(3):
+                fn(i)
+            sec = min(time_steps_queued(runner, fn, reps, hold_ms=6.0) for _ in range(2))
+            rows.append({"size": label, "routine": name, "us": sec * 1e6, "gbps": tensors * 4 * count / sec / 1e9,
+                         "pct_of_hbm_peak": 100.0 * tensors * 4 * count / sec / 1e9 / HBM_PEAK_GBPS})
+        del a, b, out
+        torch.cuda.empty_cache()
+    entry = bench_copy(runner, steps, warmup)
+    entry["yardsticks"] = rows
+    return entry
 
 
 def cpu_baseline_config0(runner, group, seconds=8.0):
@@ -622,8 +715,11 @@ def main():
     ap.add_argument("--steps", type=int, default=400)
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--workload", default="config0", choices=["config0", "config1", "config2", "config3", "config4", "copy", "max_subsampling", "bn_relu_max_subsampling", "max_subsampling_tiling",
-                             "entry_window", "concat", "maxout", "feature_map_stat"],
-                    help="'copy' times the plain copy kernel (profiler-counter calibration and bandwidth yardstick)")
+                             "entry_window", "concat", "maxout", "feature_map_stat", "config4_direct", "yardsticks"],
+                    help="'copy' times the plain copy kernel (profiler-counter calibration and bandwidth yardstick); 'yardsticks' the runtime's and "
+                         "torch's copy routines beside the library's kernels; 'config4_direct' the launches of config4 issued at the C ABI from this script")
+    ap.add_argument("--entries", type=int, default=64, help="config4: entries per packet (BASELINE.json's configuration has 64)")
+    ap.add_argument("--kernel-streams", type=int, default=0, help="config4: kernel streams of the driver (hip_kernel_stream_count); 0 = its default")
     ap.add_argument("--only", action="store_true", help="time only the chosen workload (no per_config survey, no CPU baseline)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -663,7 +759,11 @@ def main():
             return bench_maxout(runner, steps, warmup)
         if name == "feature_map_stat":
             return bench_feature_map_stat(runner, steps, warmup)
-        return bench_resnet50(runner, steps, warmup)
+        if name == "config4_direct":
+            return bench_resnet50_direct(runner, steps, warmup)
+        if name == "yardsticks":
+            return bench_yardsticks(runner, steps, warmup)
+        return bench_resnet50(runner, steps, warmup, n=args.entries, kernel_stream_count=args.kernel_streams)
 
     main_entry = run(args.workload, args.steps, args.warmup)
     per_config[args.workload] = main_entry

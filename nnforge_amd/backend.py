@@ -144,13 +144,11 @@ def parse_report(text):
     for line in text.splitlines():
         key, _, rest = line.partition(": ")
         if key == "step":
-            # "fused|single <layers> <- <inputs> @<kernel stream>[ after <step>,<step>...]"
+            # "fused|single <layers> <- <inputs> @<kernel stream>"
             kind, _, desc = rest.partition(" ")
-            desc, _, placement = desc.rpartition(" @")
-            stream, _, waits = placement.partition(" after ")
+            desc, _, stream = desc.rpartition(" @")
             layers, _, sources = desc.partition(" <- ")
-            res["steps"].append({"fused": kind == "fused", "layers": layers.split("+"), "inputs": sources.split(", "),
-                                 "stream": int(stream), "after": [int(w) for w in waits.split(",")] if waits else []})
+            res["steps"].append({"fused": kind == "fused", "layers": layers.split("+"), "inputs": sources.split(", "), "stream": int(stream)})
         elif key in ("per_entry_bytes", "max_entry_count", "entries", "writer_entries", "launches", "timed_entries"):
             res[key] = int(rest)
         elif key in ("wall_seconds_per_pass", "device_seconds_per_pass"):

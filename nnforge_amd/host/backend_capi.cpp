@@ -47,14 +47,9 @@ namespace
 
 	void describe_plan(const hip::forward_propagation_hip& fp, std::ostream& out)
 	{
-		// "step: fused|single <layers> <- <inputs> @<kernel stream>[ after <step index>,...]"
+		// "step: fused|single <layers> <- <inputs> @<kernel stream>"
 		for(const hip::forward_step& s : fp.get_steps())
-		{
-			out << "step: " << (s.fused ? "fused " : "single ") << s.description() << " @" << s.stream_index;
-			for(size_t i = 0; i < s.wait_for_steps.size(); ++i)
-				out << ((i == 0) ? " after " : ",") << s.wait_for_steps[i];
-			out << "\n";
-		}
+			out << "step: " << (s.fused ? "fused " : "single ") << s.description() << " @" << s.stream_index << "\n";
 		out << "per_entry_bytes: " << fp.get_per_entry_buffer_bytes() << "\n";
 		out << "max_entry_count: " << fp.get_max_entry_count() << "\n";
 	}

@@ -121,7 +121,6 @@ namespace nnforge
 			std::vector<void *> kernel_streams; // as many as the plan uses (steps' stream_index); the ones behind [0] take steps that do not depend on what [0] is doing
 			void * upload_stream = nullptr;   // host -> device copies
 			void * download_stream = nullptr; // device -> host copies
-			std::vector<std::unique_ptr<hip_event> > step_done;   // per step: recorded behind it when a step on another stream waits for it
 			std::vector<std::unique_ptr<hip_event> > stream_done; // per kernel stream behind [0]: end of its part of a packet
 
 			void create_streams(size_t kernel_stream_count)
@@ -140,12 +139,10 @@ namespace nnforge
 						stream_done.emplace_back(new hip_event());
 				}
 				stream = kernel_streams[0];
-				while (step_done.size() < plans.size())
-					step_done.emplace_back(new hip_event());
 			}
 
 			// Enqueues the launch plan for one packet whose data layer buffers are filled: every step on its
-			// kernel stream, behind the steps it depends on. The caller has made every kernel stream wait for
+			// kernel stream (steps that depend on each other share one). The caller has made every kernel stream wait for
 			// whatever the packet itself waits for; on return kernel_streams[0] has been made to wait for the
 			// others, so that whatever is enqueued on it next runs after the whole packet.
 			void enqueue_plan(
@@ -184,9 +181,6 @@ namespace nnforge
 					hip_safe_call(nnf_hip_event_record((*profile_events)[i]->ev, step_stream));
 				if (plan.launches_nothing())
 					continue;
-				// cross-stream dependencies (nnforge/cuda/forward_propagation_cuda.cpp:414-423)
-				for(unsigned int earlier : plan.info.wait_for_steps)
-					hip_safe_call(nnf_hip_stream_wait_event(step_stream, step_done[earlier]->ev));
 				stream_used[plan.info.stream_index] = true;
 
 				std::vector<hip_linear_buffer_device::const_ptr> inputs;
@@ -220,8 +214,6 @@ namespace nnforge
 						of_layer(weights), of_layer(weights_custom), inputs, of_layer(persistent_working),
 						temporary_buffers[i].first, temporary_buffers[i].second, step_entries);
 				}
-				if (plan.info.signals_other_streams)
-					hip_safe_call(nnf_hip_event_record(step_done[i]->ev, step_stream));
 			}
 			if (profile_events != nullptr)
 				hip_safe_call(nnf_hip_event_record((*profile_events)[plans.size()]->ev, kernel_streams[0]));
@@ -643,62 +635,67 @@ namespace nnforge
 
 			// ---- kernel streams: which steps may overlap --------------------------------------------
 			// A step depends on the earlier steps that wrote the buffers it reads and, because buffers are
-			// shared, on the earlier steps that read or wrote the buffer it writes. A step goes to the
-			// stream whose last step it depends on (a chain stays on its stream and needs no event), else
-			// to the stream with the least work so far; it waits for the latest of its dependencies on
-			// each other stream (streams run in order, so that one covers the earlier ones). With per-action
-			// times wanted every step goes to one stream: overlapping actions have no time of their own.
+			// shared, on the earlier steps that read or wrote the buffer it writes. Steps connected by such
+			// dependencies, directly or through other steps, go to one stream, in order; steps that have nothing to
+			// do with each other take the streams in turn, so that the start of one overlaps the end of another.
+			// No step ever waits for another stream: an event recorded behind a kernel and waited for on another
+			// stream costs more than a small kernel takes (measured on MI355X, 51 launches of 1 to 25 MB: 198 us on
+			// one stream, 146 us on two without events, 401 us on two with 17 such record / wait pairs), which is why
+			// nnforge/cuda/forward_propagation_cuda.cpp:414-423's event per dependency is not taken over.
+			// With per-action times wanted every step goes to one stream: overlapping actions have no time of their own.
 			{
 				const size_t stream_count = profile->is_profile() ? 1 : static_cast<size_t>(std::max(1, hip_config->kernel_stream_count));
 				const size_t buffer_count = p->buffer_floats_per_entry.size();
+				const size_t step_count = p->plans.size();
+				std::vector<size_t> component(step_count);
+				for(size_t i = 0; i < step_count; ++i)
+					component[i] = i;
+				const auto root_of = [&component] (size_t i)
+				{
+					while (component[i] != i)
+						i = component[i] = component[component[i]];
+					return i;
+				};
 				std::vector<int> last_writer(buffer_count, -1);
 				std::vector<std::vector<int> > readers(buffer_count);
-				std::vector<int> stream_last(stream_count, -1);
-				std::vector<double> stream_work(stream_count, 0.0);
-				for(size_t i = 0; i < p->plans.size(); ++i)
+				for(size_t i = 0; i < step_count; ++i)
 				{
-					step_plan& plan = p->plans[i];
-					plan.info.stream_index = 0;
-					plan.info.wait_for_steps.clear();
-					plan.info.signals_other_streams = false;
+					const step_plan& plan = p->plans[i];
 					if (plan.launches_nothing())
 						continue; // the value stays where it is: whoever reads it depends on its writer
-					std::set<int> deps;
+					const auto depends_on = [&] (int earlier)
+					{
+						// the smaller index becomes the root: a component is named after its first step
+						const size_t a = root_of(i), b = root_of(static_cast<size_t>(earlier));
+						component[std::max(a, b)] = std::min(a, b);
+					};
 					for(int b : plan.input_buffers)
 						if (last_writer[b] >= 0)
-							deps.insert(last_writer[b]);
+							depends_on(last_writer[b]);
 					const int out = plan.output_buffer;
 					if (last_writer[out] >= 0)
-						deps.insert(last_writer[out]);
-					deps.insert(readers[out].begin(), readers[out].end());
-
-					size_t chosen = stream_count;
-					for(size_t s = 0; s < stream_count; ++s)
-						if ((stream_last[s] >= 0) && (deps.find(stream_last[s]) != deps.end()) && ((chosen == stream_count) || (stream_last[s] > stream_last[chosen])))
-							chosen = s;
-					if (chosen == stream_count)
-						chosen = static_cast<size_t>(std::min_element(stream_work.begin(), stream_work.end()) - stream_work.begin());
-					plan.info.stream_index = static_cast<unsigned int>(chosen);
-					std::vector<int> latest_on_stream(stream_count, -1);
-					for(int d : deps)
-						latest_on_stream[p->plans[d].info.stream_index] = std::max(latest_on_stream[p->plans[d].info.stream_index], d);
-					for(size_t s = 0; s < stream_count; ++s)
-					{
-						if ((s == chosen) || (latest_on_stream[s] < 0))
-							continue;
-						plan.info.wait_for_steps.push_back(static_cast<unsigned int>(latest_on_stream[s]));
-						p->plans[latest_on_stream[s]].info.signals_other_streams = true;
-					}
-					stream_last[chosen] = static_cast<int>(i);
-					stream_work[chosen] += static_cast<double>(action_bytes_per_entry[plan.action]);
-
+						depends_on(last_writer[out]);
+					for(int r : readers[out])
+						depends_on(r);
 					for(int b : plan.input_buffers)
 						readers[b].push_back(static_cast<int>(i));
 					last_writer[out] = static_cast<int>(i);
 					readers[out].clear();
 				}
-				for(size_t i = 0; i < p->plans.size(); ++i)
+				std::map<size_t, unsigned int> stream_of_component;
+				unsigned int next_stream = 0;
+				for(size_t i = 0; i < step_count; ++i)
+				{
+					const size_t c = root_of(i);
+					std::map<size_t, unsigned int>::const_iterator known = stream_of_component.find(c);
+					if (known == stream_of_component.end())
+					{
+						known = stream_of_component.insert(std::make_pair(c, next_stream)).first;
+						next_stream = (next_stream + 1) % static_cast<unsigned int>(stream_count);
+					}
+					p->plans[i].info.stream_index = known->second;
 					steps[i] = p->plans[i].info;
+				}
 			}
 
 			per_entry_bytes = 0;
@@ -957,15 +954,14 @@ namespace nnforge
 							static_cast<size_t>(layer_config_map[n].get_neuron_count()) * sizeof(float) * entries_read, p->upload_stream));
 					hip_safe_call(nnf_hip_event_record(upload_done[slot].ev, p->upload_stream));
 
-					// kernels: need this packet's inputs, the slot's output buffers drained and - on the streams
-					// beside the main one, which is in order anyway - the kernels of the packet before finished
+					// kernels: need this packet's inputs and the slot's output buffers drained. The kernels of the
+					// packet before need no wait: all steps that touch a buffer share a kernel stream, which
+					// runs in order
 					for(size_t ks = 0; ks < p->kernel_streams.size(); ++ks)
 					{
 						hip_safe_call(nnf_hip_stream_wait_event(p->kernel_streams[ks], upload_done[slot].ev));
 						if (slot_used[slot])
 							hip_safe_call(nnf_hip_stream_wait_event(p->kernel_streams[ks], download_done[slot].ev));
-						if ((ks > 0) && previous.valid)
-							hip_safe_call(nnf_hip_stream_wait_event(p->kernel_streams[ks], kernels_done[previous.slot].ev));
 					}
 					p->enqueue_plan(r.buffers[slot], entries_read, r.chunk_ptrs, r.temporary, profiling ? &step_events[slot] : nullptr);
 					if (stats_on_device)
@@ -1055,19 +1051,16 @@ namespace nnforge
 						static_cast<size_t>(layer_config_map[n].get_neuron_count()) * sizeof(float) * entries_read, nullptr));
 			}
 
-			hip_event start, stop, pass_done;
-			// a pass: every kernel stream behind the end of the pass before (the main one is in order anyway)
-			auto one_pass = [&](bool first)
+			hip_event start, stop;
+			// A pass after a pass needs no wait between them: all steps that touch a buffer share a kernel stream,
+			// which runs in order. (Every pass still ends with the main stream waiting for the others, as a packet does.)
+			auto one_pass = [&]()
 			{
-				if (!first)
-					for(size_t ks = 1; ks < p->kernel_streams.size(); ++ks)
-						hip_safe_call(nnf_hip_stream_wait_event(p->kernel_streams[ks], pass_done.ev));
 				p->enqueue_plan(r.buffers[0], entries_read, r.chunk_ptrs, r.temporary, nullptr);
-				hip_safe_call(nnf_hip_event_record(pass_done.ev, p->stream));
 			};
 			hip_safe_call(nnf_hip_device_synchronize());
 			for(unsigned int i = 0; i < warmup; ++i)
-				one_pass(i == 0);
+				one_pass();
 			hip_safe_call(nnf_hip_device_synchronize());
 
 			kernel_timing res;
@@ -1080,7 +1073,7 @@ namespace nnforge
 			for(size_t ks = 1; ks < p->kernel_streams.size(); ++ks)
 				hip_safe_call(nnf_hip_stream_wait_event(p->kernel_streams[ks], start.ev));
 			for(unsigned int i = 0; i < passes; ++i)
-				one_pass(i == 0);
+				one_pass();
 			hip_safe_call(nnf_hip_event_record(stop.ev, p->stream));
 			hip_safe_call(nnf_hip_device_synchronize());
 			const std::chrono::duration<float> wall = std::chrono::high_resolution_clock::now() - t0;
