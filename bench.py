@@ -666,32 +666,72 @@ class CpuPlainBackend:
         return statistics.median(times), len(times)
 
 
-def cpu_per_config(per_config, seconds_each=2.0):
+def gpu_group_result(runner, group, chunks, pool_device):
+    """The group on the GPU with every input read from the start of pool_device and the weights of `chunks`: what
+    CpuPlainBackend.group_pass computes on the host from the same numbers."""
+    from nnforge_amd import workloads as w
+
+    torch, capi = runner.torch, runner.capi
+    total = w.group_elements(group)
+    d_chunks = [torch.from_numpy(c).to(runner.device) for c in chunks]
+    d_out = torch.empty(total, dtype=torch.float32, device=runner.device)
+    desc = capi.make_desc(group.entry_count, group.feature_map_count, group.plane, group.arms, group.tail)
+    capi.chain_forward(desc, d_out.data_ptr(), [pool_device.data_ptr()] * len(group.arms), [t.data_ptr() for t in d_chunks], runner.stream)
+    runner.sync()
+    return d_out.cpu().numpy()
+
+
+def bit_mismatches(got, want):
+    got, want = np.ascontiguousarray(got, dtype=np.float32).reshape(-1), np.ascontiguousarray(want, dtype=np.float32).reshape(-1)
+    differ = got.view(np.uint32) != want.view(np.uint32)
+    return int((differ & ~(np.isnan(got) & np.isnan(want))).sum())
+
+
+def cpu_per_config(runner, per_config, seconds_each=2.0):
     """Adds {"cpu": ...} to the entries of configs 1-4: the same workload on the host through the oracle, layer by
-    layer and unfused, on a bounded number of passes. GB/s of the same algorithmic bytes, so the columns compare."""
+    layer and unfused, on a bounded number of passes. GB/s of the same algorithmic bytes, so the columns compare.
+    The oracle's results of one pass are also what the GPU's are checked against, at full size:
+    gpu_bit_mismatches_vs_cpu (softmax: worst relative difference, its bar being 1e-5 relative, not bit equality)."""
     from nnforge_amd import workloads as w
 
     groups4 = w.resnet50_groups(64)
     largest = max([w.group_elements(w.config2()), w.group_elements(w.config3())] + [w.group_elements(g) for g in groups4])
     cpu = CpuPlainBackend(largest)
+    torch = runner.torch
+    pool_device = torch.from_numpy(cpu.pool).to(runner.device)
 
-    def attach(name, seconds, passes, what):
+    def attach(name, seconds, passes, what, check):
         e = per_config[name]
         e["cpu"] = {"ms_per_step": seconds * 1e3, "gbps": e["algorithmic_bytes_per_step"] / seconds / 1e9,
                     "elements_per_s": e["elements_per_step"] / seconds, "cores": cpu.threads, "kind": "port",
                     "sample": "%s, %d passes, median" % (what, passes)}
+        e.update(check)
+
+    def softmax_worst_relative(x, want):
+        n, c, plane = x.shape
+        d_in = torch.from_numpy(x.reshape(-1)).to(runner.device)
+        d_out = torch.empty_like(d_in)
+        runner.capi.check(runner.lib.nnf_hip_softmax_forward(runner.stream, d_out.data_ptr(), d_in.data_ptr(), n, c, plane))
+        runner.sync()
+        got = d_out.cpu().numpy().reshape(want.shape).astype(np.float64)
+        ref = want.astype(np.float64)
+        return float((np.abs(got - ref) / np.maximum(np.abs(ref), 1e-300)).max())
 
     if "config1" in per_config:
         n, c, plane = w.CONFIG1_SHAPE
-        x = (cpu.pool[:n * c * plane] * np.float32(2.0)).reshape(n, c, plane)
+        gen = np.random.Generator(np.random.MT19937(SEED + 2))
+        x = (cpu.pool[:n * c * plane] * np.float32(2.0)).reshape(n, c, plane).copy()
+        x[gen.random(x.shape) < 0.01] = np.float32(30.0)   # logits ~ N(0, 4) with 1 % at +30
         out = np.empty_like(x)
         sec, k = cpu.time_passes(lambda: cpu.oracle.softmax(x, out=out), seconds_each)
-        attach("config1", sec, k, "softmax 256 x 1000 whole")
-    for name, group, scale in (("config2", w.config2(), 1.0), ("config3", w.config3(), 2.0 ** 0.5)):
+        attach("config1", sec, k, "softmax 256 x 1000 whole", {"gpu_worst_relative_difference_vs_cpu": softmax_worst_relative(x, out)})
+    for name, group in (("config2", w.config2()), ("config3", w.config3())):
         if name in per_config:
             chunks = cpu.weights(group)
             sec, k = cpu.time_passes(lambda: cpu.group_pass(group, chunks), seconds_each)
-            attach(name, sec, k, "%s whole, one pass per layer" % name)
+            want = cpu.group_pass(group, chunks)
+            attach(name, sec, k, "%s whole, one pass per layer" % name,
+                   {"gpu_bit_mismatches_vs_cpu": bit_mismatches(gpu_group_result(runner, group, chunks, pool_device), want)})
     if "config4" in per_config:
         prepared = [(g, cpu.weights(g)) for g in groups4]
         pool_shape, sm_shape = w.resnet50_tail(64)
@@ -706,7 +746,17 @@ def cpu_per_config(per_config, seconds_each=2.0):
             cpu.oracle.softmax(sm_in, out=sm_out)
 
         sec, k = cpu.time_passes(stack, seconds_each, most=3)
-        attach("config4", sec, k, "the whole stack (49 groups unfused + average + softmax)")
+        mismatches = 0
+        for g, chunks in prepared:
+            mismatches += bit_mismatches(gpu_group_result(runner, g, chunks, pool_device), cpu.group_pass(g, chunks))
+        want_pool = cpu.oracle.average_subsampling(pool_in, [7, 7], mult=1.0 / 49.0)
+        d_pool = torch.empty(pool_shape[0] * pool_shape[1], dtype=torch.float32, device=runner.device)
+        runner.capi.check(runner.lib.nnf_hip_average_subsampling_forward(runner.stream, d_pool.data_ptr(), pool_device.data_ptr(), pool_shape[0], pool_shape[1], 7, 7, 7, 7, 1.0 / 49.0))
+        runner.sync()
+        mismatches += bit_mismatches(d_pool.cpu().numpy(), want_pool)
+        attach("config4", sec, k, "the whole stack (49 groups unfused + average + softmax)",
+               {"gpu_bit_mismatches_vs_cpu": mismatches, "gpu_worst_relative_difference_vs_cpu_softmax": softmax_worst_relative(sm_in, sm_out),
+                "checked": "the 49 groups and the 7x7 average bit for bit at N=64 through the C ABI, the softmax to its relative bar"})
 
 
 def main():
@@ -782,7 +832,7 @@ def main():
             cpu = cpu_baseline_config0(runner, w.config0())
             per_config["config0"]["cpu"] = {k: cpu[k] for k in ("ms_per_step", "elements_per_s", "cores", "kind", "sample")}
             per_config["config0"]["cpu"]["gbps"] = cpu["value"]
-        cpu_per_config(per_config)
+        cpu_per_config(runner, per_config)
 
     launches = main_entry["launches_per_step"]
     achieved = main_entry["algorithmic_bytes_per_step"] / launches / (main_entry["event_ms_per_step"] * 1e-3 / launches) / 1e9
@@ -809,6 +859,12 @@ def main():
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBPS,
+            # achieved and frac: HIP events on the launch stream around the timed steps, launched one by one by the host.
+            # queued_*: the same launches queued behind a spin kernel first (where measured), so that the host's launch
+            # calls are out of the picture
+            "timing": "events around the timed steps",
+            "queued_achieved": main_entry.get("queued_event_gbps"),
+            "queued_frac": (main_entry["queued_event_gbps"] / HBM_PEAK_GBPS) if main_entry.get("queued_event_gbps") else None,
             "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
             "kernel": {"config1": "nnf::softmax_rows_kernel", "copy": "nnf::copy_kernel_impl", "max_subsampling": "nnf::max_window2d_kernel", "bn_relu_max_subsampling": "nnf::max_window2d_prologue_kernel",
                        "max_subsampling_tiling": "nnf::tiling2d_kernel", "entry_window": "nnf::window_rows_kernel",
