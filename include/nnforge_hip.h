@@ -100,6 +100,13 @@ typedef struct nnf_hip_chain_desc
 
 /* ---- the hot path -------------------------------------------------------------------------- */
 
+/* One environment variable is read by the library, once per process, for profiling launch shapes against each other:
+ * NNF_HIP_CHAIN_SHAPE = 0 | 1 | 2 | 3 | 4 makes nnf_hip_chain_forward (and the single-layer entry points built on it) use
+ * 256 lanes x 4 float4s, 256 x 2, 256 x 1, 64 x 1 per workgroup, or (4) the grid that stays put, walking over tiles of
+ * 256 x 4, instead of choosing by tensor size. A shape that does not fit the call (coefficient tables beyond LDS; 4 with
+ * more than one input, with planes that are not float4-aligned or with one of the compile-time expf groups) is ignored.
+ * Results do not depend on it. Unset or empty: automatic. */
+
 /* Fused element-wise group. Replaces one run_forward_propagation call per layer of the group
  * (nnforge/plain/forward_propagation_plain.cpp:137-186 calls them one by one). inputs[] holds
  * input_count device pointers in the Add layer's input order; chunk_ptrs[] holds device pointers

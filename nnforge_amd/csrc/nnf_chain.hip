@@ -651,7 +651,8 @@ namespace nnf
 			return 0;
 		}
 
-		// Tuning override for experiments: NNF_HIP_CHAIN_SHAPE=<index into launch_shapes>; -1 = automatic.
+		// NNF_HIP_CHAIN_SHAPE=<index into launch_shapes> (declared in nnforge_hip.h) forces a launch shape where it is
+		// possible; read once per process. -1 = automatic.
 		int forced_shape()
 		{
 			static const int value = []

@@ -207,24 +207,9 @@ namespace nnf
 			}
 		}
 
-		// NNF_HIP_GLOBAL_POOL_PLANES overrides the planes per workgroup of the global pooling kernel (tuning); read once
-		uint32_t forced_planes_per_group()
-		{
-			static const uint32_t value = []() -> uint32_t
-			{
-				const char* text = std::getenv("NNF_HIP_GLOBAL_POOL_PLANES");
-				if ((text == nullptr) || (*text == '\0'))
-					return 0u;
-				return std::min(global_pool_planes, std::max(4u, static_cast<uint32_t>(std::atoi(text)) & ~3u));
-			}();
-			return value;
-		}
-
 		// 64 planes of 7x7; fewer of larger planes, so that a compute unit holds several workgroups
 		uint32_t global_pool_planes_per_group(uint32_t plane)
 		{
-			if (forced_planes_per_group() != 0)
-				return forced_planes_per_group();
 			return std::min(global_pool_planes, std::max(8u, (global_pool_lds_floats / plane) & ~3u));
 		}
 
