@@ -258,7 +258,7 @@ def resnet50_network(n, gen):
     return schemas.schema_text(layers, "ResNet-50 post-convolution"), weights, configs, outputs
 
 
-def bench_resnet50(runner, steps, warmup, n=64, kernel_stream_count=0):
+def bench_resnet50(runner, steps, warmup, n=64, kernel_stream_count=0, one_launch_per_group=False):
     """Config 4 through the product driver: the ResNet-50 post-convolution graph (convolution outputs as data layers) handed to
     forward_propagation_hip, whose fusion pass makes the 49 groups + average + softmax and enqueues them on its kernel streams;
     one packet of n entries resident in device memory, `steps` passes of the launch plan timed by the driver itself
@@ -271,17 +271,20 @@ def bench_resnet50(runner, steps, warmup, n=64, kernel_stream_count=0):
     largest = max(fm * dims[0] * dims[1] for fm, dims in configs.values())
     pool = gen.standard_normal(n * largest, dtype=np.float32)
     rep = backend.time_kernels(text, weights, configs, outputs, warmup=warmup, passes=steps, shared_input_pool=pool, entry_count=n,
-                               max_entry_count=n, kernel_stream_count=kernel_stream_count)
+                               max_entry_count=n, kernel_stream_count=kernel_stream_count, one_launch_per_group=one_launch_per_group)
     groups = w.resnet50_groups(n)
     assert rep["timed_entries"] == n and rep["launches"] == len(groups) + 2, rep["raw"]
-    for step, g in zip(rep["steps"], groups):
-        assert len(step["inputs"]) == len(g.arms) and len(step["layers"]) == sum(len(a) for a in g.arms) + len(g.tail) + (len(g.arms) > 1), (step, g.name)
+    # the driver orders the steps by depth in the graph: same launches as the hand-written list, not the same order
+    planned = sorted((len(step["inputs"]), len(step["layers"])) for step in rep["steps"] if step["fused"])
+    listed = sorted((len(g.arms), sum(len(a) for a in g.arms) + len(g.tail) + (len(g.arms) > 1)) for g in groups)
+    assert planned == listed, rep["raw"]
     g_bytes, p_bytes, s_bytes = w.resnet50_algorithmic_bytes(n)
     pool_shape, sm_shape = w.resnet50_tail(n)
     elements = sum(w.group_elements(g) for g in groups) + pool_shape[0] * pool_shape[1] + sm_shape[0] * sm_shape[1]
     return result_entry("config4: ResNet-50 post-convolution stack N=%d (49 fused groups + 7x7 average + softmax) through forward_propagation_hip" % n,
                         g_bytes + p_bytes + s_bytes, elements, rep["wall_seconds_per_pass"], rep["device_seconds_per_pass"], rep["launches"],
                         {"kernel_streams": len({st["stream"] for st in rep["steps"]}),
+                         "runs_of_groups_launched_together": len({st["run"] for st in rep["steps"] if st["run"] is not None}),
                          "note": "timed inside the C++ driver (forward_propagation_hip::time_kernels): one resident packet, the launch plan "
                                  "enqueued on the driver's kernel streams, nothing copied to or from the host in the timed region"})
 
@@ -515,6 +518,9 @@ def bench_yardsticks(runner, steps, warmup):
             ("torch copy_ (1 read, 1 write)", 2, lambda i: out[i % sets].copy_(a[i % sets])),
             ("own add of two tensors (2 reads, 1 write)", 3, lambda i: check(lib.nnf_hip_chain_forward(stream, ctypes.byref(desc2), out[i % sets].data_ptr(), in2_ptrs[i % sets], None))),
             ("torch add(a, b, out=c) (2 reads, 1 write)", 3, lambda i: torch.add(a[i % sets], b[i % sets], out=out[i % sets])),
+            ("torch fill_ (write only)", 1, lambda i: out[i % sets].fill_(1.0)),
+            ("hipMemsetAsync through torch zero_ (write only)", 1, lambda i: out[i % sets].zero_()),
+            ("torch sum (read only, reduced to one float)", 1, lambda i: torch.sum(a[i % sets])),
         ]
         for name, tensors, fn in candidates:
             for i in range(3):
@@ -769,6 +775,7 @@ def main():
                     help="'copy' times the plain copy kernel (profiler-counter calibration and bandwidth yardstick); 'yardsticks' the runtime's and "
                          "torch's copy routines beside the library's kernels; 'config4_direct' the launches of config4 issued at the C ABI from this script")
     ap.add_argument("--entries", type=int, default=64, help="config4: entries per packet (BASELINE.json's configuration has 64)")
+    ap.add_argument("--one-launch-per-group", action="store_true", help="config4: switch the driver's hip_batch_independent_groups off")
     ap.add_argument("--kernel-streams", type=int, default=0, help="config4: kernel streams of the driver (hip_kernel_stream_count); 0 = its default")
     ap.add_argument("--only", action="store_true", help="time only the chosen workload (no per_config survey, no CPU baseline)")
     args = ap.parse_args()
@@ -813,7 +820,7 @@ def main():
             return bench_resnet50_direct(runner, steps, warmup)
         if name == "yardsticks":
             return bench_yardsticks(runner, steps, warmup)
-        return bench_resnet50(runner, steps, warmup, n=args.entries, kernel_stream_count=args.kernel_streams)
+        return bench_resnet50(runner, steps, warmup, n=args.entries, kernel_stream_count=args.kernel_streams, one_launch_per_group=args.one_launch_per_group)
 
     main_entry = run(args.workload, args.steps, args.warmup)
     per_config[args.workload] = main_entry

@@ -114,6 +114,19 @@ typedef struct nnf_hip_chain_desc
 NNF_HIP_API int nnf_hip_chain_forward(void* stream, const nnf_hip_chain_desc* desc, float* output,
 	const float* const* inputs, const float* const* chunk_ptrs);
 
+/* group_count fused groups that have nothing to do with each other, in as few launches as possible: groups that share a
+ * kernel instance (same number of inputs, same tile size, weights fetched the same way) go six to a launch, whose grid
+ * is their tiles one after the other. Same results as group_count calls of nnf_hip_chain_forward with descs[i],
+ * outputs[i], inputs[i], chunk_ptrs[i] (chunk_ptrs, or an entry of it, may be null where no layer has weights); what a
+ * launch loses while the device fills and drains is paid once per launch instead of once per group. The groups run in
+ * no particular order and possibly at the same time: the output of a group may overlap no other group's output or
+ * inputs (NNF_HIP_EOVERLAP, nothing launched; within a group output == inputs[0] stays allowed). Every group is checked
+ * before the first launch. In the reference the driver loop calls one tester after the other
+ * (nnforge/plain/forward_propagation_plain.cpp:137-186); independent actions on separate streams are what
+ * nnforge/cuda/forward_propagation_cuda.cpp:414-423 does about it. */
+NNF_HIP_API int nnf_hip_chain_forward_batch(void* stream, uint32_t group_count, const nnf_hip_chain_desc* descs,
+	float* const* outputs, const float* const* const* inputs, const float* const* const* chunk_ptrs);
+
 /* Single-layer entry points, one per reference tester (same arithmetic as the chain kernel). */
 NNF_HIP_API int nnf_hip_batch_norm_forward(void* stream, float* output, const float* input,
 	const float* gamma, const float* beta, const float* mean, const float* inverse_sigma,

@@ -56,6 +56,7 @@ typedef struct nnf_backend_options
 	int32_t stat_on_host;          /* nnf_backend_layer_statistics: copy the outputs back and update the statistics
 	                                  value by value on the host, as the reference does, instead of reducing on the device */
 	int32_t kernel_stream_count;   /* hip_kernel_stream_count; 1 = hip_single_command_stream; <= 0: default */
+	int32_t one_launch_per_group;  /* 1: hip_batch_independent_groups off (every fused group gets a launch of its own) */
 } nnf_backend_options;
 
 /* Runs the schema on device 0. The report lists one line per launch ("step: ..."), the buffer plan

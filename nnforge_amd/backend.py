@@ -31,7 +31,8 @@ class Output(ctypes.Structure):
 class Options(ctypes.Structure):
     _fields_ = [("fuse", ctypes.c_int32), ("dont_share_buffers", ctypes.c_int32), ("max_entry_count", ctypes.c_int32),
                 ("profile", ctypes.c_int32), ("weights_from_folder", ctypes.c_int32), ("weights_folder", ctypes.c_char_p),
-                ("profile_folder", ctypes.c_char_p), ("stat_on_host", ctypes.c_int32), ("kernel_stream_count", ctypes.c_int32)]
+                ("profile_folder", ctypes.c_char_p), ("stat_on_host", ctypes.c_int32), ("kernel_stream_count", ctypes.c_int32),
+                ("one_launch_per_group", ctypes.c_int32)]
 
 
 class DatasetFile(ctypes.Structure):
@@ -85,7 +86,7 @@ def load():
 
 
 def _options(fuse=True, dont_share_buffers=False, max_entry_count=0, profile=False, weights_folder=None,
-             profile_folder=None, stat_on_host=False, kernel_stream_count=0):
+             profile_folder=None, stat_on_host=False, kernel_stream_count=0, one_launch_per_group=False):
     o = Options()
     o.fuse = int(fuse)
     o.dont_share_buffers = int(dont_share_buffers)
@@ -96,6 +97,7 @@ def _options(fuse=True, dont_share_buffers=False, max_entry_count=0, profile=Fal
     o.profile_folder = profile_folder.encode() if profile_folder is not None else None
     o.stat_on_host = int(stat_on_host)
     o.kernel_stream_count = int(kernel_stream_count)
+    o.one_launch_per_group = int(one_launch_per_group)
     return o
 
 
@@ -144,11 +146,13 @@ def parse_report(text):
     for line in text.splitlines():
         key, _, rest = line.partition(": ")
         if key == "step":
-            # "fused|single <layers> <- <inputs> @<kernel stream>"
+            # "fused|single <layers> <- <inputs> @<kernel stream>[ #<run of groups launched together>]"
             kind, _, desc = rest.partition(" ")
-            desc, _, stream = desc.rpartition(" @")
+            desc, _, placement = desc.rpartition(" @")
+            stream, _, run = placement.partition(" #")
             layers, _, sources = desc.partition(" <- ")
-            res["steps"].append({"fused": kind == "fused", "layers": layers.split("+"), "inputs": sources.split(", "), "stream": int(stream)})
+            res["steps"].append({"fused": kind == "fused", "layers": layers.split("+"), "inputs": sources.split(", "), "stream": int(stream),
+                                 "run": int(run) if run else None})
         elif key in ("per_entry_bytes", "max_entry_count", "entries", "writer_entries", "launches", "timed_entries"):
             res[key] = int(rest)
         elif key in ("wall_seconds_per_pass", "device_seconds_per_pass"):

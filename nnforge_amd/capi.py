@@ -58,6 +58,7 @@ _UP = ctypes.POINTER(ctypes.c_uint32)
 # name -> argtypes, exactly the declarations of include/nnforge_hip.h (all return int unless noted)
 SIGNATURES = {
     "nnf_hip_chain_forward": [_VP, ctypes.POINTER(ChainDesc), _VP, _PP, _PP],
+    "nnf_hip_chain_forward_batch": [_VP, _U32, ctypes.POINTER(ChainDesc), ctypes.POINTER(_VP), ctypes.POINTER(ctypes.POINTER(_VP)), ctypes.POINTER(ctypes.POINTER(_VP))],
     "nnf_hip_batch_norm_forward": [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _U32, _U32, _U32],
     "nnf_hip_rectified_linear_forward": [_VP, _VP, _VP, _F, _U64],
     "nnf_hip_parametric_rectified_linear_forward": [_VP, _VP, _VP, _VP, _U32, _U32, _U32],

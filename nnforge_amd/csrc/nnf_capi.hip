@@ -127,6 +127,12 @@ extern "C"
 		return chain_forward(static_cast<hipStream_t>(stream), desc, output, inputs, chunk_ptrs);
 	}
 
+	int nnf_hip_chain_forward_batch(void* stream, uint32_t group_count, const nnf_hip_chain_desc* descs, float* const* outputs,
+		const float* const* const* inputs, const float* const* const* chunk_ptrs)
+	{
+		return chain_forward_batch(static_cast<hipStream_t>(stream), group_count, descs, outputs, inputs, chunk_ptrs);
+	}
+
 	int nnf_hip_batch_norm_forward(void* stream, float* output, const float* input,
 		const float* gamma, const float* beta, const float* mean, const float* inverse_sigma,
 		uint32_t entry_count, uint32_t feature_map_count, uint32_t neuron_count_per_feature_map)

@@ -13,6 +13,7 @@
 #include <algorithm>
 #include <atomic>
 #include <cstdlib>
+#include <vector>
 
 namespace nnf
 {
@@ -414,16 +415,16 @@ namespace nnf
 		};
 		constexpr int known_program_count = sizeof(known_programs) / sizeof(known_programs[0]);
 
+		// One tile of one group, by one workgroup: the body of the two kernels below.
 		template<int NIN, int BLOCK, int U, bool DIRECT, int PROGRAM>
-		__global__ void __launch_bounds__(BLOCK) chain_kernel(const chain_args a)
+		__device__ __forceinline__ void chain_tile(const chain_args& a, const uint32_t tile_index, unsigned char* lds_raw)
 		{
 			constexpr int TILE = BLOCK * U * 4;
 			constexpr int PL = DIRECT ? 1 : 4;
-			extern __shared__ __align__(16) unsigned char lds_raw[];
 			uint64_t* lds_exp = reinterpret_cast<uint64_t*>(lds_raw);
 			float2* lds_coeff = reinterpret_cast<float2*>(lds_raw + exp_table_bytes);
 
-			const uint32_t tile_start = blockIdx.x * static_cast<uint32_t>(TILE);
+			const uint32_t tile_start = tile_index * static_cast<uint32_t>(TILE);
 
 			// All loads are issued before anything else: the tensors first (nothing but the tile index
 			// goes into their addresses), then the lane's expf table entry and (compile-time programs) the
@@ -487,6 +488,38 @@ namespace nnf
 			store_tile<BLOCK, U>(a, tile_start, tail_start, x[0]);
 			if (owns_tail)
 				store_tail_vector<U>(a, tail_start, k_tail, x[0]);
+		}
+
+		template<int NIN, int BLOCK, int U, bool DIRECT, int PROGRAM>
+		__global__ void __launch_bounds__(BLOCK) chain_kernel(const chain_args a)
+		{
+			extern __shared__ __align__(16) unsigned char lds_raw[];
+			chain_tile<NIN, BLOCK, U, DIRECT, PROGRAM>(a, blockIdx.x, lds_raw);
+		}
+
+		// Several groups that have nothing to do with each other in one launch: the grid is the groups' tiles one
+		// after the other, a workgroup finds its group by its index and then does what chain_kernel does. The time a
+		// launch loses while the device fills and drains is paid once for all of them (measured with 51 one-read-
+		// one-write tensors of the ResNet-50 stack's sizes: 915 us one by one, 831 us six per launch, at 64 entries;
+		// 214 against 121 us at 8 entries). All groups of a launch share NIN, the launch shape and DIRECT.
+		constexpr uint32_t max_batch = 6; // 6 x sizeof(chain_args) stays inside 4 KB of kernel arguments
+		struct chain_batch_args
+		{
+			uint32_t count;
+			uint32_t tile_end[max_batch]; // running total of the groups' tile counts
+			chain_args group[max_batch];
+		};
+		static_assert(sizeof(chain_batch_args) <= 4096, "kernel arguments of a batch beyond 4 KB");
+
+		template<int NIN, int BLOCK, int U, bool DIRECT>
+		__global__ void __launch_bounds__(BLOCK) chain_batch_kernel(const chain_batch_args b)
+		{
+			extern __shared__ __align__(16) unsigned char lds_raw[];
+			uint32_t g = 0;
+			while ((g + 1 < b.count) && (blockIdx.x >= b.tile_end[g]))
+				++g;
+			const uint32_t tile_index = blockIdx.x - ((g == 0) ? 0u : b.tile_end[g - 1]);
+			chain_tile<NIN, BLOCK, U, DIRECT, 0>(b.group[g], tile_index, lds_raw);
 		}
 
 		// The same group on a grid that stays put: as many workgroups as the device holds at once (or fewer), each
@@ -666,11 +699,16 @@ namespace nnf
 			return value;
 		}
 
-		bool ranges_overlap(const void* a, const void* b, size_t bytes)
+		bool ranges_overlap(const void* a, size_t a_bytes, const void* b, size_t b_bytes)
 		{
 			const uintptr_t pa = reinterpret_cast<uintptr_t>(a);
 			const uintptr_t pb = reinterpret_cast<uintptr_t>(b);
-			return (pa < pb + bytes) && (pb < pa + bytes);
+			return (pa < pb + b_bytes) && (pb < pa + a_bytes);
+		}
+
+		bool ranges_overlap(const void* a, const void* b, size_t bytes)
+		{
+			return ranges_overlap(a, bytes, b, bytes);
 		}
 
 		constexpr size_t max_dynamic_lds = 64 * 1024;
@@ -686,189 +724,347 @@ namespace nnf
 		constexpr uint32_t persistent_workgroups_per_compute_unit = 5;
 	}
 
+	namespace
+	{
+		// A group checked and ready to launch: the kernel's arguments and the launch shape chosen for it.
+		struct prepared_group
+		{
+			chain_args a;
+			bool nothing_to_do; // zero elements
+			int shape;          // index into launch_shapes
+			bool direct;
+			int program;        // index into known_programs, 0: the layer list is interpreted
+			uint32_t input_count;
+			uint32_t tiles;
+			size_t lds_bytes;
+			size_t bytes;       // of one tensor
+		};
+
+		// Checks the call's arguments and fills p. single_launch: the group gets a launch of its own, so the grid
+		// that stays put is a candidate; as one of several groups of a launch it is not.
+		int prepare_group(const nnf_hip_chain_desc* desc, float* output, const float* const* inputs, const float* const* chunk_ptrs,
+			bool single_launch, prepared_group& p)
+		{
+			if ((desc == nullptr) || (output == nullptr) || (inputs == nullptr))
+				return NNF_HIP_EINVAL;
+			if ((desc->feature_map_count == 0) || (desc->neuron_count_per_feature_map == 0))
+				return NNF_HIP_EINVAL;
+			if ((desc->input_count < 1) || (desc->input_count > NNF_HIP_MAX_INPUTS))
+				return NNF_HIP_EINVAL;
+			if ((desc->input_count > 1) && !desc->has_add)
+				return NNF_HIP_EINVAL;
+
+			uint32_t op_count = desc->tail_op_count;
+			for(uint32_t j = 0; j < NNF_HIP_MAX_INPUTS; ++j)
+			{
+				if ((j >= desc->input_count) && (desc->arm_op_count[j] != 0))
+					return NNF_HIP_EINVAL;
+				op_count += desc->arm_op_count[j];
+			}
+			if (op_count > NNF_HIP_MAX_OPS)
+				return NNF_HIP_EINVAL;
+
+			p = prepared_group();
+			p.input_count = desc->input_count;
+			const uint64_t total64 = static_cast<uint64_t>(desc->entry_count) * desc->feature_map_count * desc->neuron_count_per_feature_map;
+			if (total64 == 0)
+			{
+				p.nothing_to_do = true; // as the reference's loops over zero elements
+				return NNF_HIP_OK;
+			}
+			if (total64 > NNF_HIP_MAX_ELEMENT_COUNT)
+				return NNF_HIP_ETOOBIG;
+			p.bytes = static_cast<size_t>(total64) * sizeof(float);
+
+			chain_args& a = p.a;
+			if (!is_aligned16(output))
+				return NNF_HIP_EALIGN;
+			for(uint32_t j = 0; j < desc->input_count; ++j)
+			{
+				if (inputs[j] == nullptr)
+					return NNF_HIP_EINVAL;
+				if (!is_aligned16(inputs[j]))
+					return NNF_HIP_EALIGN;
+				const bool exact_alias_of_first = (j == 0) && (inputs[j] == output);
+				if (!exact_alias_of_first && ranges_overlap(inputs[j], output, p.bytes))
+					return NNF_HIP_EOVERLAP;
+				a.in[j] = inputs[j];
+			}
+			a.out = output;
+			a.total = static_cast<uint32_t>(total64);
+			a.fm_count = desc->feature_map_count;
+			a.plane = desc->neuron_count_per_feature_map;
+			a.has_add = desc->has_add ? 1u : 0u;
+			a.alpha = desc->add_alpha;
+			for(uint32_t j = 0; j < NNF_HIP_MAX_INPUTS; ++j)
+				a.arm_ops[j] = desc->arm_op_count[j];
+			a.tail_ops = desc->tail_op_count;
+
+			for(uint32_t i = 0; i < op_count; ++i)
+			{
+				const nnf_hip_op& src = desc->ops[i];
+				chain_op& dst = a.ops[i];
+				dst.kind = src.kind;
+				dst.slot = -1;
+				dst.f0 = src.f0;
+				dst.f1 = src.f1;
+				switch (src.kind)
+				{
+				case NNF_HIP_OP_BATCH_NORM:
+				case NNF_HIP_OP_PRELU:
+					{
+						if ((chunk_ptrs == nullptr) || (src.chunk < 0))
+							return NNF_HIP_EINVAL;
+						const int chunk_count = (src.kind == NNF_HIP_OP_BATCH_NORM) ? 4 : 1;
+						chain_slot& slot = a.slots[a.slot_count];
+						for(int c = 0; c < chunk_count; ++c)
+						{
+							if (chunk_ptrs[src.chunk + c] == nullptr)
+								return NNF_HIP_EINVAL;
+							slot.p[c] = chunk_ptrs[src.chunk + c];
+						}
+						slot.kind = src.kind;
+						dst.slot = static_cast<int32_t>(a.slot_count);
+						++a.slot_count;
+					}
+					break;
+				case NNF_HIP_OP_RELU:
+				case NNF_HIP_OP_ABSOLUTE:
+				case NNF_HIP_OP_DROPOUT:
+					break;
+				case NNF_HIP_OP_TANH:
+					// nnforge/plain/hyperbolic_tangent_layer_tester_plain.cpp:49: steepness * 2.0F, rounded once on the host
+					dst.f1 = src.f1 * 2.0f;
+					a.need_exp = 1;
+					break;
+				case NNF_HIP_OP_ELU:
+				case NNF_HIP_OP_SIGMOID:
+					a.need_exp = 1;
+					break;
+				default:
+					return NNF_HIP_EINVAL;
+				}
+			}
+
+			// tile size: as large as keeps the coefficient arrays inside LDS and the grid wide enough
+			auto span_of = [&](int shape) -> uint32_t
+			{
+				const uint32_t tile = launch_shapes[shape].block * launch_shapes[shape].unroll * 4;
+				return (tile + a.plane - 2) / a.plane + 1;
+			};
+			// weights are read straight from memory when a float4 never straddles planes and a tile
+			// touches no feature map twice; otherwise the workgroup stages coefficients in LDS
+			auto direct_of = [&](int shape) -> bool
+			{
+				if (a.slot_count == 0)
+					return true; // no layer reads per-feature-map weights: nothing to look up, nothing to stage
+				return ((a.plane % 4) == 0) && (span_of(shape) <= a.fm_count);
+			};
+			auto lds_bytes_of = [&](int shape) -> size_t
+			{
+				if (direct_of(shape))
+					return exp_table_bytes;
+				return exp_table_bytes + static_cast<size_t>(a.slot_count) * span_of(shape) * sizeof(float2);
+			};
+			auto tiles_of = [&](int shape) -> uint32_t
+			{
+				const uint32_t tile = launch_shapes[shape].block * launch_shapes[shape].unroll * 4;
+				return (a.total + tile - 1) / tile;
+			};
+
+			const int program = match_known_program(*desc, op_count);
+			// the grid that stays put exists for the interpreted layer list with weights read straight from memory
+			auto persistent_possible = [&]() -> bool
+			{
+				return single_launch && (program == 0) && (desc->input_count <= persistent_max_inputs) && direct_of(persistent_shape);
+			};
+			int shape = forced_shape();
+			if ((shape == persistent_shape) && !persistent_possible())
+				shape = -1;
+			const bool automatic = (shape < 0) || (lds_bytes_of(shape) > max_dynamic_lds);
+			if (automatic)
+			{
+				// Measured on MI355X. One input: tensors of 64 MB and more stream best with two float4s per lane,
+				// smaller ones with four, as long as enough workgroups exist to cover the machine. Several inputs:
+				// two float4s per lane at every size (4 % faster than four from 10 to 130 MB per tensor).
+				// As one of several groups of a launch: two float4s per lane whatever the size - the grid is all the
+				// groups' tiles, so a small group need not be cut finer to cover the machine, and groups of one tile
+				// size share launches (the 49 groups of the ResNet-50 stack at 64 entries, launched together where
+				// they can be: 1078 us with four float4s for all, 1067 with two, 1189 with one, 1085 chosen by size).
+				static const int small_tile_order[] = { 1, 2, 3 };
+				static const int any_tile_order[] = { 0, 1, 2, 3 };
+				const bool large = (a.total >= large_tensor_elements) || !single_launch;
+				const bool small_tiles = large || (desc->input_count > 1);
+				const int* order = small_tiles ? small_tile_order : any_tile_order;
+				const int order_count = small_tiles ? 3 : 4;
+				shape = -1;
+				for(int i = 0; i < order_count; ++i)
+				{
+					const int s = order[i];
+					if (lds_bytes_of(s) > max_dynamic_lds)
+						continue;
+					if (large || (tiles_of(s) >= min_tiles_wanted) || (i == order_count - 1))
+					{
+						shape = s;
+						break;
+					}
+				}
+				if (shape < 0)
+					return NNF_HIP_EUNSUPPORTED;
+			}
+			if ((program > 0) && (shape == 0))
+				shape = 1; // the compile-time programs have no four-float4 instance (smaller tile: LDS still fits)
+			// One input, four float4s per lane, and more tiles than the device holds workgroups at once (8 per compute
+			// unit: above 33 MB per tensor): a second, partial round of workgroups would follow the first and the time per
+			// byte jumps (32 MB: 11.0 us, 38.5 MB: 15.5 us). There the grid that stays put takes over, five workgroups
+			// per compute unit walking over the tiles with the next tile's loads in flight while the current one is
+			// stored (38.5 MB: 13.3 us, 51.4 MB: 18.8 -> 17.3 us). With fewer tiles every workgroup has one tile anyway and
+			// the plain grid is as fast or faster (25.7 MB: 9.1 against 9.4 us); from 64 MB on the two are equal.
+			if (automatic && (shape == 0) && (tiles_of(0) > compute_unit_count() * resident_workgroups_per_compute_unit) && persistent_possible())
+				shape = persistent_shape;
+			a.span = span_of(shape);
+			a.plane_magic = (a.plane >= 2) ? static_cast<uint32_t>(((1ull << 32) + a.plane - 1) / a.plane) : 0u;
+			p.shape = shape;
+			p.direct = direct_of(shape);
+			p.program = program;
+			p.tiles = tiles_of(shape);
+			p.lds_bytes = launch_shapes[shape].persistent ? exp_table_bytes : lds_bytes_of(shape);
+			return NNF_HIP_OK;
+		}
+
+		int launch_group(hipStream_t stream, const prepared_group& p)
+		{
+			if (p.nothing_to_do)
+				return NNF_HIP_OK;
+			const launch_shape& shape = launch_shapes[p.shape];
+			if (shape.persistent)
+			{
+				const uint32_t grid = std::min(p.tiles, compute_unit_count() * persistent_workgroups_per_compute_unit);
+				hipLaunchKernelGGL(pick_persistent_kernel(p.input_count), dim3(grid), dim3(shape.block), p.lds_bytes, stream, p.a, p.tiles);
+				return launch_status();
+			}
+			hipLaunchKernelGGL(pick_kernel(p.input_count, p.shape, p.direct, p.program), dim3(p.tiles), dim3(shape.block), p.lds_bytes, stream, p.a);
+			return launch_status();
+		}
+
+		typedef void (*chain_batch_kernel_fn)(const chain_batch_args);
+
+		template<int NIN>
+		chain_batch_kernel_fn pick_batch_kernel_of(int shape, bool direct)
+		{
+			switch (shape)
+			{
+			case 0: return direct ? chain_batch_kernel<NIN, 256, 4, true> : chain_batch_kernel<NIN, 256, 4, false>;
+			case 1: return direct ? chain_batch_kernel<NIN, 256, 2, true> : chain_batch_kernel<NIN, 256, 2, false>;
+			case 2: return direct ? chain_batch_kernel<NIN, 256, 1, true> : chain_batch_kernel<NIN, 256, 1, false>;
+			default: return direct ? chain_batch_kernel<NIN, 64, 1, true> : chain_batch_kernel<NIN, 64, 1, false>;
+			}
+		}
+
+		chain_batch_kernel_fn pick_batch_kernel(uint32_t input_count, int shape, bool direct)
+		{
+			switch (input_count)
+			{
+			case 1: return pick_batch_kernel_of<1>(shape, direct);
+			case 2: return pick_batch_kernel_of<2>(shape, direct);
+			case 3: return pick_batch_kernel_of<3>(shape, direct);
+			default: return pick_batch_kernel_of<4>(shape, direct);
+			}
+		}
+	}
+
 	int chain_forward(hipStream_t stream, const nnf_hip_chain_desc* desc, float* output,
 		const float* const* inputs, const float* const* chunk_ptrs)
 	{
-		if ((desc == nullptr) || (output == nullptr) || (inputs == nullptr))
-			return NNF_HIP_EINVAL;
-		if ((desc->feature_map_count == 0) || (desc->neuron_count_per_feature_map == 0))
-			return NNF_HIP_EINVAL;
-		if ((desc->input_count < 1) || (desc->input_count > NNF_HIP_MAX_INPUTS))
-			return NNF_HIP_EINVAL;
-		if ((desc->input_count > 1) && !desc->has_add)
-			return NNF_HIP_EINVAL;
+		prepared_group p;
+		const int rc = prepare_group(desc, output, inputs, chunk_ptrs, true, p);
+		return (rc != NNF_HIP_OK) ? rc : launch_group(stream, p);
+	}
 
-		uint32_t op_count = desc->tail_op_count;
-		for(uint32_t j = 0; j < NNF_HIP_MAX_INPUTS; ++j)
+	int chain_forward_batch(hipStream_t stream, uint32_t group_count, const nnf_hip_chain_desc* descs, float* const* outputs,
+		const float* const* const* inputs, const float* const* const* chunk_ptrs)
+	{
+		if (group_count == 0)
+			return NNF_HIP_OK;
+		if ((descs == nullptr) || (outputs == nullptr) || (inputs == nullptr))
+			return NNF_HIP_EINVAL;
+		if (group_count == 1)
+			return chain_forward(stream, &descs[0], outputs[0], inputs[0], (chunk_ptrs == nullptr) ? nullptr : chunk_ptrs[0]);
+
+		// everything is checked before anything is launched
+		std::vector<prepared_group> groups(group_count);
+		for(uint32_t i = 0; i < group_count; ++i)
 		{
-			if ((j >= desc->input_count) && (desc->arm_op_count[j] != 0))
-				return NNF_HIP_EINVAL;
-			op_count += desc->arm_op_count[j];
+			const int rc = prepare_group(&descs[i], outputs[i], inputs[i], (chunk_ptrs == nullptr) ? nullptr : chunk_ptrs[i], false, groups[i]);
+			if (rc != NNF_HIP_OK)
+				return rc;
 		}
-		if (op_count > NNF_HIP_MAX_OPS)
-			return NNF_HIP_EINVAL;
-
-		const uint64_t total64 = static_cast<uint64_t>(desc->entry_count) * desc->feature_map_count * desc->neuron_count_per_feature_map;
-		if (total64 == 0)
-			return NNF_HIP_OK; // nothing to do, as the reference's loops over zero elements
-		if (total64 > NNF_HIP_MAX_ELEMENT_COUNT)
-			return NNF_HIP_ETOOBIG;
-		const size_t bytes = static_cast<size_t>(total64) * sizeof(float);
-
-		chain_args a = {};
-		if (!is_aligned16(output))
-			return NNF_HIP_EALIGN;
-		for(uint32_t j = 0; j < desc->input_count; ++j)
+		// the groups run in no particular order, possibly at the same time: what one writes no other may touch
+		for(uint32_t i = 0; i < group_count; ++i)
 		{
-			if (inputs[j] == nullptr)
-				return NNF_HIP_EINVAL;
-			if (!is_aligned16(inputs[j]))
-				return NNF_HIP_EALIGN;
-			const bool exact_alias_of_first = (j == 0) && (inputs[j] == output);
-			if (!exact_alias_of_first && ranges_overlap(inputs[j], output, bytes))
-				return NNF_HIP_EOVERLAP;
-			a.in[j] = inputs[j];
-		}
-		a.out = output;
-		a.total = static_cast<uint32_t>(total64);
-		a.fm_count = desc->feature_map_count;
-		a.plane = desc->neuron_count_per_feature_map;
-		a.has_add = desc->has_add ? 1u : 0u;
-		a.alpha = desc->add_alpha;
-		for(uint32_t j = 0; j < NNF_HIP_MAX_INPUTS; ++j)
-			a.arm_ops[j] = desc->arm_op_count[j];
-		a.tail_ops = desc->tail_op_count;
-
-		for(uint32_t i = 0; i < op_count; ++i)
-		{
-			const nnf_hip_op& src = desc->ops[i];
-			chain_op& dst = a.ops[i];
-			dst.kind = src.kind;
-			dst.slot = -1;
-			dst.f0 = src.f0;
-			dst.f1 = src.f1;
-			switch (src.kind)
+			if (groups[i].nothing_to_do)
+				continue;
+			for(uint32_t j = 0; j < group_count; ++j)
 			{
-			case NNF_HIP_OP_BATCH_NORM:
-			case NNF_HIP_OP_PRELU:
-				{
-					if ((chunk_ptrs == nullptr) || (src.chunk < 0))
-						return NNF_HIP_EINVAL;
-					const int chunk_count = (src.kind == NNF_HIP_OP_BATCH_NORM) ? 4 : 1;
-					chain_slot& slot = a.slots[a.slot_count];
-					for(int c = 0; c < chunk_count; ++c)
-					{
-						if (chunk_ptrs[src.chunk + c] == nullptr)
-							return NNF_HIP_EINVAL;
-						slot.p[c] = chunk_ptrs[src.chunk + c];
-					}
-					slot.kind = src.kind;
-					dst.slot = static_cast<int32_t>(a.slot_count);
-					++a.slot_count;
-				}
-				break;
-			case NNF_HIP_OP_RELU:
-			case NNF_HIP_OP_ABSOLUTE:
-			case NNF_HIP_OP_DROPOUT:
-				break;
-			case NNF_HIP_OP_TANH:
-				// nnforge/plain/hyperbolic_tangent_layer_tester_plain.cpp:49: steepness * 2.0F, rounded once on the host
-				dst.f1 = src.f1 * 2.0f;
-				a.need_exp = 1;
-				break;
-			case NNF_HIP_OP_ELU:
-			case NNF_HIP_OP_SIGMOID:
-				a.need_exp = 1;
-				break;
-			default:
-				return NNF_HIP_EINVAL;
-			}
-		}
-
-		// tile size: as large as keeps the coefficient arrays inside LDS and the grid wide enough
-		auto span_of = [&](int shape) -> uint32_t
-		{
-			const uint32_t tile = launch_shapes[shape].block * launch_shapes[shape].unroll * 4;
-			return (tile + a.plane - 2) / a.plane + 1;
-		};
-		// weights are read straight from memory when a float4 never straddles planes and a tile
-		// touches no feature map twice; otherwise the workgroup stages coefficients in LDS
-		auto direct_of = [&](int shape) -> bool
-		{
-			if (a.slot_count == 0)
-				return true; // no layer reads per-feature-map weights: nothing to look up, nothing to stage
-			return ((a.plane % 4) == 0) && (span_of(shape) <= a.fm_count);
-		};
-		auto lds_bytes_of = [&](int shape) -> size_t
-		{
-			if (direct_of(shape))
-				return exp_table_bytes;
-			return exp_table_bytes + static_cast<size_t>(a.slot_count) * span_of(shape) * sizeof(float2);
-		};
-		auto tiles_of = [&](int shape) -> uint32_t
-		{
-			const uint32_t tile = launch_shapes[shape].block * launch_shapes[shape].unroll * 4;
-			return (a.total + tile - 1) / tile;
-		};
-
-		const int program = match_known_program(*desc, op_count);
-		// the grid that stays put exists for the interpreted layer list with weights read straight from memory
-		auto persistent_possible = [&]() -> bool
-		{
-			return (program == 0) && (desc->input_count <= persistent_max_inputs) && direct_of(persistent_shape);
-		};
-		int shape = forced_shape();
-		if ((shape == persistent_shape) && !persistent_possible())
-			shape = -1;
-		const bool automatic = (shape < 0) || (lds_bytes_of(shape) > max_dynamic_lds);
-		if (automatic)
-		{
-			// Measured on MI355X. One input: tensors of 64 MB and more stream best with two float4s per lane,
-			// smaller ones with four, as long as enough workgroups exist to cover the machine. Several inputs:
-			// two float4s per lane at every size (4 % faster than four from 10 to 130 MB per tensor).
-			static const int small_tile_order[] = { 1, 2, 3 };
-			static const int any_tile_order[] = { 0, 1, 2, 3 };
-			const bool large = a.total >= large_tensor_elements;
-			const bool small_tiles = large || (desc->input_count > 1);
-			const int* order = small_tiles ? small_tile_order : any_tile_order;
-			const int order_count = small_tiles ? 3 : 4;
-			shape = -1;
-			for(int i = 0; i < order_count; ++i)
-			{
-				const int s = order[i];
-				if (lds_bytes_of(s) > max_dynamic_lds)
+				if ((j == i) || groups[j].nothing_to_do)
 					continue;
-				if (large || (tiles_of(s) >= min_tiles_wanted) || (i == order_count - 1))
-				{
-					shape = s;
-					break;
-				}
+				if (ranges_overlap(groups[i].a.out, groups[i].bytes, groups[j].a.out, groups[j].bytes))
+					return NNF_HIP_EOVERLAP;
+				for(uint32_t k = 0; k < groups[j].input_count; ++k)
+					if (ranges_overlap(groups[i].a.out, groups[i].bytes, groups[j].a.in[k], groups[j].bytes))
+						return NNF_HIP_EOVERLAP;
 			}
-			if (shape < 0)
-				return NNF_HIP_EUNSUPPORTED;
 		}
-		if ((program > 0) && (shape == 0))
-			shape = 1; // the compile-time programs have no four-float4 instance (smaller tile: LDS still fits)
-		// One input, four float4s per lane, and more tiles than the device holds workgroups at once (8 per compute
-		// unit: above 33 MB per tensor): a second, partial round of workgroups would follow the first and the time per
-		// byte jumps (32 MB: 11.0 us, 38.5 MB: 15.5 us). There the grid that stays put takes over, five workgroups
-		// per compute unit walking over the tiles with the next tile's loads in flight while the current one is
-		// stored (38.5 MB: 13.3 us, 51.4 MB: 18.8 -> 17.3 us). With fewer tiles every workgroup has one tile anyway and
-		// the plain grid is as fast or faster (25.7 MB: 9.1 against 9.4 us); from 64 MB on the two are equal.
-		if (automatic && (shape == 0) && (tiles_of(0) > compute_unit_count() * resident_workgroups_per_compute_unit) && persistent_possible())
-			shape = persistent_shape;
-		a.span = span_of(shape);
-		a.plane_magic = (a.plane >= 2) ? static_cast<uint32_t>(((1ull << 32) + a.plane - 1) / a.plane) : 0u;
 
-		if (launch_shapes[shape].persistent)
+		std::vector<bool> launched(group_count, false);
+		for(uint32_t first = 0; first < group_count; ++first)
 		{
-			const uint32_t tiles = tiles_of(shape);
-			const uint32_t grid = std::min(tiles, compute_unit_count() * persistent_workgroups_per_compute_unit);
-			hipLaunchKernelGGL(pick_persistent_kernel(desc->input_count), dim3(grid), dim3(launch_shapes[shape].block), exp_table_bytes, stream, a, tiles);
-			return launch_status();
+			if (launched[first])
+				continue;
+			const prepared_group& lead = groups[first];
+			launched[first] = true;
+			if (lead.nothing_to_do)
+				continue;
+			// the groups behind it that can share its kernel instance, max_batch to a launch; the compile-time
+			// expf programs are bound by the vector ALU, not by launches: they keep their own kernels
+			std::vector<uint32_t> members(1, first);
+			if (lead.program == 0)
+				for(uint32_t j = first + 1; (j < group_count) && (members.size() < max_batch); ++j)
+				{
+					const prepared_group& g = groups[j];
+					if (!launched[j] && !g.nothing_to_do && (g.program == 0) && (g.input_count == lead.input_count) && (g.shape == lead.shape) && (g.direct == lead.direct))
+					{
+						members.push_back(j);
+						launched[j] = true;
+					}
+				}
+			if (members.size() == 1)
+			{
+				const int rc = launch_group(stream, lead);
+				if (rc != NNF_HIP_OK)
+					return rc;
+				continue;
+			}
+			chain_batch_args b = {};
+			b.count = static_cast<uint32_t>(members.size());
+			size_t lds_bytes = 0;
+			uint64_t tiles = 0;
+			for(size_t m = 0; m < members.size(); ++m)
+			{
+				const prepared_group& g = groups[members[m]];
+				b.group[m] = g.a;
+				tiles += g.tiles;
+				b.tile_end[m] = static_cast<uint32_t>(tiles);
+				lds_bytes = std::max(lds_bytes, g.lds_bytes);
+			}
+			if (tiles > 0x7FFFFFFFull)
+				return NNF_HIP_ETOOBIG;
+			hipLaunchKernelGGL(pick_batch_kernel(lead.input_count, lead.shape, lead.direct), dim3(static_cast<uint32_t>(tiles)), dim3(launch_shapes[lead.shape].block),
+				lds_bytes, stream, b);
+			const int rc = launch_status();
+			if (rc != NNF_HIP_OK)
+				return rc;
 		}
-		chain_kernel_fn kernel = pick_kernel(desc->input_count, shape, direct_of(shape), program);
-		hipLaunchKernelGGL(kernel, dim3(tiles_of(shape)), dim3(launch_shapes[shape].block), lds_bytes_of(shape), stream, a);
-		return launch_status();
+		return NNF_HIP_OK;
 	}
 }

@@ -90,6 +90,8 @@ namespace nnf
 	// entry points implemented in the individual translation units
 	int chain_forward(hipStream_t stream, const nnf_hip_chain_desc* desc, float* output,
 		const float* const* inputs, const float* const* chunk_ptrs);
+	int chain_forward_batch(hipStream_t stream, uint32_t group_count, const nnf_hip_chain_desc* descs, float* const* outputs,
+		const float* const* const* inputs, const float* const* const* chunk_ptrs);
 	int softmax_forward(hipStream_t stream, float* output, const float* input,
 		uint32_t entry_count, uint32_t feature_map_count, uint32_t neuron_count_per_feature_map);
 	int average_subsampling_forward(hipStream_t stream, float* output, const float* input,

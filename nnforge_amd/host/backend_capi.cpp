@@ -47,9 +47,14 @@ namespace
 
 	void describe_plan(const hip::forward_propagation_hip& fp, std::ostream& out)
 	{
-		// "step: fused|single <layers> <- <inputs> @<kernel stream>"
+		// "step: fused|single <layers> <- <inputs> @<kernel stream>[ #<run of groups launched together>]"
 		for(const hip::forward_step& s : fp.get_steps())
-			out << "step: " << (s.fused ? "fused " : "single ") << s.description() << " @" << s.stream_index << "\n";
+		{
+			out << "step: " << (s.fused ? "fused " : "single ") << s.description() << " @" << s.stream_index;
+			if (s.batch_index >= 0)
+				out << " #" << s.batch_index;
+			out << "\n";
+		}
 		out << "per_entry_bytes: " << fp.get_per_entry_buffer_bytes() << "\n";
 		out << "max_entry_count: " << fp.get_max_entry_count() << "\n";
 	}
@@ -65,6 +70,7 @@ namespace
 				generator.hip_max_entry_count = options->max_entry_count;
 			if (options->kernel_stream_count > 0)
 				generator.hip_kernel_stream_count = options->kernel_stream_count;
+			generator.hip_batch_independent_groups = options->one_launch_per_group == 0;
 		}
 		generator.initialize();
 	}
@@ -394,7 +400,8 @@ extern "C"
 			const bool dont_share = (options != nullptr) && (options->dont_share_buffers != 0);
 			const int max_entries = ((options != nullptr) && (options->max_entry_count > 0)) ? options->max_entry_count : 4096;
 			const int kernel_streams = ((options != nullptr) && (options->kernel_stream_count > 0)) ? options->kernel_stream_count : hip::hip_running_configuration::default_kernel_stream_count;
-			hip::hip_running_configuration::const_ptr config = hip::hip_running_configuration::create_offline(memory_bytes, 0.9F, fuse, dont_share, max_entries, kernel_streams);
+			const bool batch = (options == nullptr) || (options->one_launch_per_group == 0);
+			hip::hip_running_configuration::const_ptr config = hip::hip_running_configuration::create_offline(memory_bytes, 0.9F, fuse, dont_share, max_entries, kernel_streams, batch);
 			hip::forward_propagation_hip fp(schema, output_names, debug_state::ptr(new debug_state(false)), profile_state::ptr(new profile_state(false)), config);
 			fp.set_input_configuration_specific(input_configs(inputs, input_count));
 			describe_plan(fp, out);

@@ -186,7 +186,32 @@ namespace nnforge
 				std::vector<hip_linear_buffer_device::const_ptr> inputs;
 				for(int b : plan.input_buffers)
 					inputs.push_back(buffers[b]);
-				if (plan.prologue)
+				if (plan.info.batch_index >= 0)
+				{
+					// the first step of a run of independent fused groups launches all of them
+					if ((i > 0) && (plans[i - 1].info.batch_index == plan.info.batch_index))
+						continue;
+					std::vector<nnf_hip_chain_desc> descs;
+					std::vector<float *> outputs;
+					std::vector<std::vector<const float *> > in_ptrs;
+					std::vector<const float * const *> in_ptr_ptrs, chunk_ptr_ptrs;
+					for(size_t m = i; (m < plans.size()) && (plans[m].info.batch_index == plan.info.batch_index); ++m)
+					{
+						step_plan& member = plans[m];
+						member.desc.entry_count = entries_read * member.entry_factor;
+						descs.push_back(member.desc);
+						outputs.push_back(*buffers[member.output_buffer]);
+						in_ptrs.push_back(std::vector<const float *>());
+						for(int b : member.input_buffers)
+							in_ptrs.back().push_back(static_cast<const float *>(*static_cast<hip_linear_buffer_device::const_ptr>(buffers[b])));
+						chunk_ptr_ptrs.push_back(chunk_ptrs[m].empty() ? nullptr : chunk_ptrs[m].data());
+					}
+					for(const std::vector<const float *>& v : in_ptrs)
+						in_ptr_ptrs.push_back(v.data());
+					hip_safe_call(nnf_hip_chain_forward_batch(step_stream, static_cast<uint32_t>(descs.size()), descs.data(), outputs.data(),
+						in_ptr_ptrs.data(), chunk_ptr_ptrs.data()));
+				}
+				else if (plan.prologue)
 				{
 					plan.desc.entry_count = step_entries;
 					plan.tester->enqueue_forward_propagation_with_prologue(step_stream, buffers[plan.output_buffer], inputs.at(0), plan.desc,
@@ -427,6 +452,47 @@ namespace nnforge
 			while (!pending.empty())
 				materialize(pending.begin()->first);
 
+			// ---- order: steps that depend on nothing first ------------------------------------------------
+			// With independent groups launched together (see below) a run of such groups ends where a step depends on
+			// one of them. Sorting the steps by their depth in the graph (a step comes one level behind the deepest
+			// producer of its inputs; steps of a level keep their order) makes the runs as long as the graph allows: in
+			// a network of branches every level is one run, in a chain nothing moves.
+			if (hip_config->batch_independent_groups && !profile->is_profile())
+			{
+				std::map<std::string, const pending_group *> group_of;
+				for(const std::pair<std::string, pending_group>& g : groups)
+					group_of[g.first] = &g.second;
+				std::map<std::string, unsigned int> level_of_value; // by the name of the layer whose output a step stores
+				std::vector<std::pair<unsigned int, size_t> > keyed;
+				for(size_t i = 0; i < step_order.size(); ++i)
+				{
+					const std::string& name = step_order[i].first;
+					std::vector<std::string> sources;
+					if (step_order[i].second)
+						for(const pending_arm& a : group_of[name]->arms)
+							sources.push_back(a.source);
+					else if (prologues.find(name) != prologues.end())
+						sources.push_back(prologues[name].arms[0].source);
+					else
+						sources = this->schema->get_layer(name)->input_layer_instance_names;
+					unsigned int level = 0;
+					for(const std::string& source : sources)
+					{
+						std::map<std::string, unsigned int>::const_iterator it = level_of_value.find(source);
+						if (it != level_of_value.end()) // data layers are on no level
+							level = std::max(level, it->second + 1);
+					}
+					level_of_value[name] = level;
+					keyed.push_back(std::make_pair(level, i));
+				}
+				std::stable_sort(keyed.begin(), keyed.end(),
+					[] (const std::pair<unsigned int, size_t>& a, const std::pair<unsigned int, size_t>& b) { return a.first < b.first; });
+				std::vector<std::pair<std::string, bool> > sorted;
+				for(const std::pair<unsigned int, size_t>& k : keyed)
+					sorted.push_back(step_order[k.second]);
+				step_order.swap(sorted);
+			}
+
 			// ---- steps ---------------------------------------------------------------------------
 			p->plans.clear();
 			steps.clear();
@@ -643,8 +709,14 @@ namespace nnforge
 			// one stream, 146 us on two without events, 401 us on two with 17 such record / wait pairs), which is why
 			// nnforge/cuda/forward_propagation_cuda.cpp:414-423's event per dependency is not taken over.
 			// With per-action times wanted every step goes to one stream: overlapping actions have no time of their own.
+			//
+			// Better than overlapping the ends of launches is not to have them: runs of consecutive fused groups that do
+			// not depend on each other are handed to the kernels in one call (nnf_hip_chain_forward_batch), which puts
+			// groups of a kind into one launch. A step joins the run unless it depends on a step already in it (a
+			// dependency through steps in between would have ended the run at those). Such runs take one stream.
 			{
-				const size_t stream_count = profile->is_profile() ? 1 : static_cast<size_t>(std::max(1, hip_config->kernel_stream_count));
+				const bool batching = hip_config->batch_independent_groups && !profile->is_profile();
+				const size_t stream_count = (profile->is_profile() || batching) ? 1 : static_cast<size_t>(std::max(1, hip_config->kernel_stream_count));
 				const size_t buffer_count = p->buffer_floats_per_entry.size();
 				const size_t step_count = p->plans.size();
 				std::vector<size_t> component(step_count);
@@ -658,6 +730,7 @@ namespace nnforge
 				};
 				std::vector<int> last_writer(buffer_count, -1);
 				std::vector<std::vector<int> > readers(buffer_count);
+				std::vector<std::set<int> > depends_directly_on(step_count);
 				for(size_t i = 0; i < step_count; ++i)
 				{
 					const step_plan& plan = p->plans[i];
@@ -665,6 +738,7 @@ namespace nnforge
 						continue; // the value stays where it is: whoever reads it depends on its writer
 					const auto depends_on = [&] (int earlier)
 					{
+						depends_directly_on[i].insert(earlier);
 						// the smaller index becomes the root: a component is named after its first step
 						const size_t a = root_of(i), b = root_of(static_cast<size_t>(earlier));
 						component[std::max(a, b)] = std::min(a, b);
@@ -694,8 +768,33 @@ namespace nnforge
 						next_stream = (next_stream + 1) % static_cast<unsigned int>(stream_count);
 					}
 					p->plans[i].info.stream_index = known->second;
-					steps[i] = p->plans[i].info;
 				}
+
+				int batch_count = 0;
+				std::vector<int> run; // the steps of the batch being formed
+				for(size_t i = 0; i < step_count; ++i)
+				{
+					step_plan& plan = p->plans[i];
+					plan.info.batch_index = -1;
+					if (plan.launches_nothing())
+						continue; // no launch: neither joins a run nor ends one
+					const bool can_join = batching && plan.info.fused && !plan.prologue;
+					bool depends_on_run = false;
+					for(int member : run)
+						depends_on_run = depends_on_run || (depends_directly_on[i].find(member) != depends_directly_on[i].end());
+					if (!can_join || depends_on_run)
+					{
+						batch_count += run.empty() ? 0 : 1;
+						run.clear();
+					}
+					if (can_join)
+					{
+						plan.info.batch_index = batch_count;
+						run.push_back(static_cast<int>(i));
+					}
+				}
+				for(size_t i = 0; i < step_count; ++i)
+					steps[i] = p->plans[i].info;
 			}
 
 			per_entry_bytes = 0;
@@ -1107,6 +1206,7 @@ namespace nnforge
 			, hip_fuse(true)
 			, hip_dont_share_buffers(false)
 			, hip_single_command_stream(false)
+			, hip_batch_independent_groups(true)
 			, hip_kernel_stream_count(hip_running_configuration::default_kernel_stream_count)
 			, hip_max_entry_count(4096)
 		{
@@ -1117,7 +1217,7 @@ namespace nnforge
 			hip::init();
 			hip_config = hip_running_configuration::const_ptr(new hip_running_configuration(
 				hip_device_id, hip_max_global_memory_usage_ratio, hip_fuse, hip_dont_share_buffers, hip_max_entry_count,
-				hip_single_command_stream ? 1 : std::max(1, hip_kernel_stream_count)));
+				hip_single_command_stream ? 1 : std::max(1, hip_kernel_stream_count), hip_batch_independent_groups));
 		}
 
 		forward_propagation_factory::ptr factory_generator_hip::create_forward_propagation_factory() const
@@ -1144,6 +1244,7 @@ namespace nnforge
 			res.push_back(bool_option("hip_fuse", &hip_fuse, true, "Fuse runs of element-wise layers (BatchNorm, activations, Add) into single kernel launches"));
 			res.push_back(bool_option("hip_dont_share_buffers", &hip_dont_share_buffers, false, "Don't share buffers between layers. Switch it on if you suspect a bug in there"));
 			res.push_back(bool_option("hip_single_command_stream", &hip_single_command_stream, false, "Use single stream for kernels. Switch it on if you suspect a bug in there"));
+			res.push_back(bool_option("hip_batch_independent_groups", &hip_batch_independent_groups, true, "Launch consecutive fused groups that do not depend on each other together (takes one kernel stream)"));
 			return res;
 		}
 

@@ -39,13 +39,14 @@ namespace nnforge
 		constexpr int hip_running_configuration::default_kernel_stream_count;
 
 		hip_running_configuration::hip_running_configuration(int device_id, float max_global_memory_usage_ratio, bool fuse_layers, bool dont_share_buffers, int max_entry_count,
-			int kernel_stream_count)
+			int kernel_stream_count, bool batch_independent_groups)
 			: device_id(device_id)
 			, max_global_memory_usage_ratio(max_global_memory_usage_ratio)
 			, fuse_layers(fuse_layers)
 			, dont_share_buffers(dont_share_buffers)
 			, max_entry_count(max_entry_count)
 			, kernel_stream_count(kernel_stream_count)
+			, batch_independent_groups(batch_independent_groups)
 			, global_memory_size(0)
 			, compute_unit_count(0)
 			, wavefront_size(0)
@@ -66,10 +67,11 @@ namespace nnforge
 
 		hip_running_configuration::const_ptr hip_running_configuration::create_offline(
 			unsigned long long global_memory_size, float max_global_memory_usage_ratio, bool fuse_layers, bool dont_share_buffers, int max_entry_count,
-			int kernel_stream_count)
+			int kernel_stream_count, bool batch_independent_groups)
 		{
 			std::shared_ptr<hip_running_configuration> res(new hip_running_configuration());
 			res->kernel_stream_count = kernel_stream_count;
+			res->batch_independent_groups = batch_independent_groups;
 			res->device_id = -1;
 			res->max_global_memory_usage_ratio = max_global_memory_usage_ratio;
 			res->fuse_layers = fuse_layers;
@@ -103,6 +105,7 @@ namespace nnforge
 			out << "Global memory = " << (config.global_memory_size >> 20) << " MB" << std::endl;
 			out << "Compute units = " << config.compute_unit_count << ", wavefront " << config.wavefront_size << ", clock " << (config.clock_khz / 1000) << " MHz" << std::endl;
 			out << "Memory usage ratio = " << config.max_global_memory_usage_ratio << ", fuse element-wise layers = " << (config.fuse_layers ? "yes" : "no")
+				<< ", independent groups launched together = " << (config.batch_independent_groups ? "yes" : "no")
 				<< ", kernel streams = " << config.kernel_stream_count << std::endl;
 			return out;
 		}

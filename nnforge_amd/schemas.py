@@ -109,6 +109,7 @@ def resnet50_post_convolution(with_pool1=False):
             layers.append(L("ReLU", name + "_relu", [name]))
             outputs.append(name + "_relu")
             last, last_fm = name + "_relu", restored
+    outputs.pop()   # the last block feeds the pooling below and no convolution
     layers.append(L("AverageSubsampling", "pool5", [last], windows=[7, 7], alpha=1.0 / 49.0))
     outputs.append("pool5")
     data("logits", 1000, 1)

@@ -123,6 +123,38 @@ class GpuHarness:
         return self.to_host(d_out)
 
 
+def _chain_batch(self, groups, in_place=None):
+    """groups: [(shape3, arms, tail, inputs, chunks, has_add, alpha)]; one nnf_hip_chain_forward_batch call.
+    in_place[i]: group i writes over its first input. Returns the outputs as flat numpy arrays."""
+    count = len(groups)
+    descs = (capi.ChainDesc * count)()
+    keep, outs, in_arrays, chunk_arrays = [], [], [], []
+    for i, (shape3, arms, tail, inputs, chunks, has_add, alpha) in enumerate(groups):
+        n, c, plane = shape3
+        descs[i] = capi.make_desc(n, c, plane, arms, tail, has_add=has_add, add_alpha=alpha)
+        # a tensor without elements still needs an address to hand over
+        d_in = [self.to_device(a) if a.size else self.torch.empty(4, dtype=self.torch.float32, device=self.device) for a in inputs]
+        d_chunks = [self.to_device(a) for a in chunks]
+        if in_place is not None and in_place[i]:
+            d_out = d_in[0]
+        else:
+            d_out = self.torch.full((max(4, n * c * plane),), float("nan"), dtype=self.torch.float32, device=self.device)
+        keep.append((d_in, d_chunks, d_out))
+        outs.append(d_out)
+        in_arrays.append(capi.pointer_array([t.data_ptr() for t in d_in]))
+        chunk_arrays.append(capi.pointer_array([t.data_ptr() for t in d_chunks]) if d_chunks else None)
+    pp = ctypes.POINTER(ctypes.c_void_p)
+    in_ptrs = (pp * count)(*[ctypes.cast(a, pp) for a in in_arrays])
+    chunk_ptrs = (pp * count)(*[ctypes.cast(a, pp) if a is not None else pp() for a in chunk_arrays])
+    rc = self.lib.nnf_hip_chain_forward_batch(self.stream, count, descs, capi.pointer_array([t.data_ptr() for t in outs]), in_ptrs, chunk_ptrs)
+    assert rc == 0, capi.error_string(rc)
+    self.torch.cuda.synchronize()
+    return [t.cpu().numpy()[:g[0][0] * g[0][1] * g[0][2]] for t, g in zip(outs, groups)]
+
+
+GpuHarness.chain_batch = _chain_batch
+
+
 def golden_expf():
     """(x, expf(x)) of tests/golden/expf_vectors.npy: 8192 inputs and glibc 2.35's expf of them (see make_expf_vectors.py)."""
     import os

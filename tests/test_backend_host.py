@@ -217,13 +217,14 @@ def test_plan_of_the_inception_like_block():
 
 def test_plan_of_the_resnet50_post_convolution_graph_equals_the_benchmark_group_list():
     """Config 4 as a network: the graph examples/imagenet/imagenet_toolset.cpp:476-550, 729-831 builds, convolution outputs as
-    data layers. The driver's fusion pass must arrive at the 49 groups nnforge_amd.workloads lists by hand (kind, shape,
-    order), then the 7x7 average and the softmax; the residual of a block that keeps its shape is the block before."""
+    data layers. With one launch per group the driver's fusion pass must arrive at the 49 groups nnforge_amd.workloads lists by
+    hand (kind, shape, order), then the 7x7 average and the softmax; the residual of a block that keeps its shape is the block
+    before. By default the steps are ordered by depth in the graph and independent groups are launched together."""
     from nnforge_amd import schemas, workloads as w
 
     layers, configs, outputs = schemas.resnet50_post_convolution()
     assert len([l for l in layers if l["type"] == "BatchNorm"]) == 53   # 1 stem + 16 blocks x 3 + 4 shortcuts
-    rep = plan(layers, configs, outputs)
+    rep = plan(layers, configs, outputs, one_launch_per_group=True)
     steps = rep["steps"]
     groups = w.resnet50_groups(1)
     assert len(steps) == len(groups) + 2 == 51
@@ -232,25 +233,26 @@ def test_plan_of_the_resnet50_post_convolution_graph_equals_the_benchmark_group_
     for l in layers:   # every layer here keeps the shape of its first input, but for the pooling
         if l["type"] != "Data":
             shapes[l["name"]] = shapes[l["inputs"][0]]
-    per_entry_bytes = 0
-    for step, g in zip(steps, groups):
-        assert step["fused"]
-        kinds = [by_name[n]["type"] for n in step["layers"]]
-        fm, dims = shapes[step["layers"][-1]]
-        assert (fm, dims[0] * dims[1]) == (g.feature_map_count, g.plane), (step, g.name)
-        assert len(step["inputs"]) == len(g.arms)
-        want = {1: ["BatchNorm", "ReLU"], 2: ["BatchNorm", "Add", "ReLU"]}[len(g.arms)]
-        if len(g.arms) == 2 and g.arms[0]:
-            want = ["BatchNorm"] + want   # the first block of a stage: batch norm on the shortcut as well
-        assert kinds == want, (step, g.name)
-        per_entry_bytes += w.group_algorithmic_bytes(g)
-    assert steps[49]["layers"] == ["pool5"] and steps[49]["inputs"] == ["res5c_relu"] and not steps[49]["fused"]
-    assert steps[50]["layers"] == ["prob"] and steps[50]["inputs"] == ["logits"]
-    # the bytes the launches move per entry are the benchmark's algorithmic bytes (weights aside: 4 bytes per weight)
+
     def floats(name):
         fm, dims = shapes[name]
         return fm * dims[0] * dims[1]
 
+    def kinds_wanted(g):
+        want = {1: ["BatchNorm", "ReLU"], 2: ["BatchNorm", "Add", "ReLU"]}[len(g.arms)]
+        return (["BatchNorm"] + want) if (len(g.arms) == 2 and g.arms[0]) else want   # first block of a stage: batch norm on the shortcut as well
+
+    per_entry_bytes = 0
+    for step, g in zip(steps, groups):
+        assert step["fused"] and step["run"] is None
+        fm, dims = shapes[step["layers"][-1]]
+        assert (fm, dims[0] * dims[1]) == (g.feature_map_count, g.plane), (step, g.name)
+        assert len(step["inputs"]) == len(g.arms)
+        assert [by_name[n]["type"] for n in step["layers"]] == kinds_wanted(g), (step, g.name)
+        per_entry_bytes += w.group_algorithmic_bytes(g)
+    assert steps[49]["layers"] == ["pool5"] and steps[49]["inputs"] == ["res5c_relu"] and not steps[49]["fused"]
+    assert steps[50]["layers"] == ["prob"] and steps[50]["inputs"] == ["logits"]
+    # the bytes the launches move per entry are the benchmark's algorithmic bytes (weights aside: 4 bytes per weight)
     weights_bytes = sum(4 * (4 if kind == "bn" else 1) * c for g in groups for kind, c in g.chunks)
     g_bytes, p_bytes, s_bytes = w.resnet50_algorithmic_bytes(1)
     assert per_entry_bytes == g_bytes
@@ -270,14 +272,30 @@ def test_plan_of_the_resnet50_post_convolution_graph_equals_the_benchmark_group_
                 chained += 1
     assert chained == 12 + 1   # 16 blocks minus the 4 with a shortcut convolution, and pool5 behind res5c_relu
     assert [s["stream"] for s in steps[:6]] == [0, 1, 2, 0, 1, 2] and len({s["stream"] for s in steps}) == 3
-    # one kernel stream: the same steps, nothing to wait for
-    single = plan(layers, configs, outputs, kernel_stream_count=1)
+    # one kernel stream: the same steps
+    single = plan(layers, configs, outputs, one_launch_per_group=True, kernel_stream_count=1)
     assert [s["layers"] for s in single["steps"]] == [s["layers"] for s in steps]
     assert all(s["stream"] == 0 for s in single["steps"])
+
+    # the default: the same launches ordered by depth in the graph - everything that reads convolution outputs only comes
+    # first, the blocks that read the block before follow level by level - and every level's groups launched together
+    batched = plan(layers, configs, outputs)["steps"]
+    assert sorted(tuple(s["layers"]) for s in batched) == sorted(tuple(s["layers"]) for s in steps)
+    assert all(s["stream"] == 0 for s in batched)
+    position = {s["layers"][-1]: i for i, s in enumerate(batched)}
+    for i, s in enumerate(batched):
+        for source in s["inputs"]:
+            if source in position:
+                assert position[source] < i and batched[position[source]]["run"] != s["run"], (i, s)   # never in a run with its producer
+    runs = [s["run"] for s in batched]
+    assert runs[:37] == [0] * 37 and batched[37]["layers"] == ["prob"] and runs[37] is None   # 1 + 16 + 16 + 4 groups, then the softmax
+    assert [batched[i]["layers"][-1] for i in range(38, 42)] == ["res2b_relu", "res3b_relu", "res4b_relu", "res5b_relu"] and runs[38:42] == [1] * 4
+    assert runs[42:46] == [2] * 4 and runs[46:48] == [3] * 2 and batched[48]["layers"] == ["pool5"] and runs[48:] == [None, 4, 5]
     # with the stem's pooling in the graph, batch norm and ReLU are applied on the way into the pooling kernel
     layers, configs, outputs = schemas.resnet50_post_convolution(with_pool1=True)
     rep = plan(layers, configs, outputs)
     assert len(rep["steps"]) == 51 and rep["steps"][0]["layers"] == ["conv1_bn", "relu1", "pool1"] and rep["steps"][0]["fused"]
+    assert rep["steps"][0]["run"] is None and rep["steps"][1]["run"] == 0   # the pooling step is no fused group: it launches alone
 
 
 def stem_net(c=8):

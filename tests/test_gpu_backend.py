@@ -234,6 +234,11 @@ def test_random_networks_equal_the_oracle_layer_by_layer(seed):
     plain, _ = run(layers, weights, inputs, outputs, values, fuse=False, dont_share_buffers=True)
     for name in outputs:
         assert_bits(plain[name], values[name], "seed %d unfused, output %s" % (seed, name))
+    # fused, every group launched on its own, independent steps spread over the kernel streams, buffers shared
+    spread, rep = run(layers, weights, inputs, outputs, values, fuse=True, max_entry_count=3, one_launch_per_group=True, kernel_stream_count=3)
+    assert all(s["run"] is None for s in rep["steps"])
+    for name in outputs:
+        assert_bits(spread[name], values[name], "seed %d on kernel streams, output %s" % (seed, name))
 
 
 def test_average_subsampling_in_the_full_form_through_the_driver():
@@ -329,10 +334,11 @@ def test_inference_from_data_set_files_to_data_set_files(tmp_path):
         backend.run_dataset(S.schema_text(layers), weights, {"images": tmp_path / "nowhere.dt"}, outputs)
 
 
-@pytest.mark.parametrize("streams", [0, 1])
-def test_resnet50_post_convolution_graph_layer_by_layer(streams):
-    """Config 4 through the driver at a small entry count: every output of the 51 launches against the oracle run layer by
-    layer (bit for bit; softmax to 1e-5), with the kernels on three streams (the default) and on one."""
+@pytest.mark.parametrize("mode", ["together", "streams", "plain"])
+def test_resnet50_post_convolution_graph_layer_by_layer(mode):
+    """Config 4 through the driver at a small entry count: every output of the 51 steps against the oracle run layer by
+    layer (bit for bit; softmax to 1e-5) - with independent groups launched together (the default), with one launch per
+    group spread over three kernel streams, and with one launch per group on one stream."""
     from nnforge_amd import schemas
 
     gen = T.rng(62, 0)
@@ -342,9 +348,11 @@ def test_resnet50_post_convolution_graph_layer_by_layer(streams):
     inputs = {name: T.normal(gen, (n, fm, dims[1], dims[0])) for name, (fm, dims) in sorted(configs.items())}
     inputs["logits"] = T.normal(gen, (n, 1000, 1, 1), 4.0)
     values = S.evaluate(layers, weights, inputs)
-    got, rep = run(layers, weights, inputs, outputs, values, max_entry_count=2, kernel_stream_count=streams)
+    options = {"together": {}, "streams": {"one_launch_per_group": True}, "plain": {"one_launch_per_group": True, "kernel_stream_count": 1}}[mode]
+    got, rep = run(layers, weights, inputs, outputs, values, max_entry_count=2, **options)
     assert len(rep["steps"]) == 51 and rep["entries"] == n
-    assert len({s["stream"] for s in rep["steps"]}) == (1 if streams == 1 else 3)
+    assert len({s["stream"] for s in rep["steps"]}) == (3 if mode == "streams" else 1)
+    assert len({s["run"] for s in rep["steps"]} - {None}) == (6 if mode == "together" else 0)
     for name in outputs:
         if name == "prob":
             assert np.all(np.abs(got[name] - values[name]) <= 1e-5 * np.abs(values[name])), name

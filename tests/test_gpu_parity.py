@@ -381,10 +381,10 @@ def random_layer(gen, c, chunks, allow_exp=True):
     return (TANH, 0, scale, steepness), lambda v: oracle.hyperbolic_tangent(v, scale, steepness)
 
 
-@pytest.mark.parametrize("seed", range(40))
-def test_random_groups_equal_the_layers_one_by_one(gpu, seed):
-    """Groups drawn at random - 1 to 4 inputs, any split of up to 8 layers over the arms and the tail, any layer
-    kinds, shapes with odd planes and element counts - against the oracle run layer by layer, bit for bit."""
+def random_group(seed, allow_exp=True):
+    """A group drawn at random - 1 to 4 inputs, any split of up to 8 layers over the arms and the tail, any layer kinds,
+    shapes with odd planes and element counts - and what the oracle, run layer by layer, makes of it.
+    -> (shape3, arms, tail, inputs, chunks, has_add, alpha, want)"""
     gen = T.rng(13, seed)
     n = int(gen.integers(1, 6))
     c = int(gen.choice([1, 3, 8, 17, 64, 130]))
@@ -398,7 +398,7 @@ def test_random_groups_equal_the_layers_one_by_one(gpu, seed):
         budget -= count
         ops, steps = [], []
         for _ in range(count):
-            op, step = random_layer(gen, c, chunks)
+            op, step = random_layer(gen, c, chunks, allow_exp)
             ops.append(op)
             steps.append(step)
         arms.append(ops)
@@ -406,11 +406,11 @@ def test_random_groups_equal_the_layers_one_by_one(gpu, seed):
     tail, tail_steps = [], []
     if has_add:
         for _ in range(int(gen.integers(0, min(3, budget) + 1))):
-            op, step = random_layer(gen, c, chunks)
+            op, step = random_layer(gen, c, chunks, allow_exp)
             tail.append(op)
             tail_steps.append(step)
     elif not arms[0]:
-        op, step = random_layer(gen, c, chunks)
+        op, step = random_layer(gen, c, chunks, allow_exp)
         arms[0].append(op)
         arm_steps[0].append(step)
     alpha = float(gen.choice(np.array([1.0, 0.5, -1.25], np.float32)))
@@ -424,8 +424,53 @@ def test_random_groups_equal_the_layers_one_by_one(gpu, seed):
     want = oracle.add(values, alpha).reshape(inputs[0].shape) if has_add else values[0]
     for step in tail_steps:
         want = step(want)
-    got = gpu.chain((n, c, plane), arms, tail, inputs, chunks, has_add=has_add, alpha=alpha)
-    check_exact(got, want, "random group %d: %d inputs, arms %s, tail %s" % (seed, input_count, arms, tail))
+    return (n, c, plane), arms, tail, inputs, chunks, has_add, alpha, want
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_groups_equal_the_layers_one_by_one(gpu, seed):
+    """Random groups against the oracle run layer by layer, bit for bit."""
+    shape3, arms, tail, inputs, chunks, has_add, alpha, want = random_group(seed)
+    got = gpu.chain(shape3, arms, tail, inputs, chunks, has_add=has_add, alpha=alpha)
+    check_exact(got, want, "random group %d: %d inputs, arms %s, tail %s" % (seed, len(inputs), arms, tail))
+
+
+@pytest.mark.parametrize("first_seed,count", [(0, 40), (40, 17), (100, 2), (200, 7)])
+def test_independent_groups_in_one_call_equal_the_groups_one_by_one(gpu, first_seed, count):
+    """nnf_hip_chain_forward_batch: groups that share a kernel instance go several to a launch. Random groups of all
+    kinds in one call (among them groups without elements, groups that work in place and one of the compile-time expf
+    programs, which keeps a launch of its own) against the oracle, bit for bit."""
+    groups = [random_group(first_seed + i, allow_exp=(i % 3 == 0)) for i in range(count)]
+    n, c, plane = 3, 16, 196
+    x = config3_input((n, c, plane))
+    g, b, m, s = T.bn_params(T.rng(15, first_seed), c)
+    groups.append(((n, c, plane), [[(BN, 0), (ELU,), (SIGMOID,), (TANH, 0, T.TANH_SCALE, T.TANH_STEEPNESS)]], [], [x], [g, b, m, s], False, 1.0,
+                   oracle.hyperbolic_tangent(oracle.sigmoid(oracle.exponential_linear(oracle.batch_norm(x, g, b, m, s))), T.TANH_SCALE, T.TANH_STEEPNESS)))
+    groups.append(((0, 4, 49), [[(RELU, 0, 0.0)]], [], [np.zeros((0, 4, 49), np.float32)], [], False, 1.0, np.zeros((0, 4, 49), np.float32)))
+    in_place = [i % 4 == 1 for i in range(len(groups))]
+    got = gpu.chain_batch([(sh, arms, tail, ins, chunks, has_add, alpha) for sh, arms, tail, ins, chunks, has_add, alpha, _ in groups], in_place)
+    for i, (out, group) in enumerate(zip(got, groups)):
+        check_exact(out, group[7], "group %d of the call (seed %d)" % (i, first_seed + i))
+
+
+def test_groups_of_one_call_must_not_touch_each_other(gpu):
+    x = gpu.to_device(T.normal(T.rng(16, 0), 4096))
+    y = gpu.torch.empty(8192, dtype=gpu.torch.float32, device=gpu.device)
+    descs = (capi.ChainDesc * 2)(capi.make_desc(1, 1, 4096, [[(RELU, 0, 0.0)]]), capi.make_desc(1, 1, 4096, [[(capi.OP_ABSOLUTE,)]]))
+
+    def call(outs, ins):
+        in_arrays = [capi.pointer_array([a]) for a in ins]
+        in_ptrs = (ctypes.POINTER(ctypes.c_void_p) * 2)(*[ctypes.cast(a, ctypes.POINTER(ctypes.c_void_p)) for a in in_arrays])
+        return gpu.lib.nnf_hip_chain_forward_batch(gpu.stream, 2, descs, capi.pointer_array(outs), in_ptrs, None)
+
+    base = y.data_ptr()
+    assert call([base, base + 16384], [x.data_ptr(), x.data_ptr()]) == 0                       # a shared input is fine
+    assert call([base, base + 8192], [x.data_ptr(), x.data_ptr()]) == capi.E_OVERLAP           # two outputs overlap
+    assert call([base, base + 16384], [x.data_ptr(), base]) == capi.E_OVERLAP                  # one reads what the other writes
+    assert call([base, base + 16384], [base, x.data_ptr()]) == 0                               # in place within a group
+    assert gpu.lib.nnf_hip_chain_forward_batch(gpu.stream, 0, None, None, None, None) == 0
+    assert gpu.lib.nnf_hip_chain_forward_batch(gpu.stream, 2, None, None, None, None) == capi.E_INVAL
+    gpu.torch.cuda.synchronize()
 
 
 def test_in_place_group(gpu):
