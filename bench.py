@@ -35,13 +35,16 @@ SEED = 0x6E6E4600
 # each counter scaled by what it reads for the 256 MiB copy kernel (profiles/chain_kernel_*.md);
 # None for workloads that have not been measured.
 MEASURED_TRAFFIC_BYTES = {
-    "config0": 51565056,    # algorithmic 51,381,248
+    "config0": 51602922,    # algorithmic 51,381,248
     "config2": 1233228800,  # algorithmic 1,233,130,496
     "config3": 205650944,   # algorithmic 205,529,088
     "config1": 2117540,     # algorithmic 2,048,000 (profiles/softmax_and_resnet50_stack.md)
     "max_subsampling_tiling": 402617602,  # algorithmic 403,767,296 (profiles/tiling_and_entry_window_kernels.md)
     "entry_window": 256931085,            # algorithmic 256,901,120
-    "config4": 124914115,   # average over the 51 launches of a step: 6,370,619,861 per step, algorithmic 6,359,339,008
+    "config4": 124804803,   # per step, average over the 51 steps of a pass through the driver (17 kernel launches: independent groups
+                            # share launches): 6,365,044,940 per pass, algorithmic 6,359,339,008 (profiles/chain_batch_kernel_config4_through_driver.md)
+    "config4_direct": 124914115,  # average over the 51 launches of a step: 6,370,619,861 per step (profiles/softmax_and_resnet50_stack.md)
+    "walking_grid": 102999701,    # algorithmic 102,761,472 (profiles/chain_kernel_persistent_walking_grid.md)
 }
 
 
@@ -771,7 +774,7 @@ def main():
     ap.add_argument("--steps", type=int, default=400)
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--workload", default="config0", choices=["config0", "config1", "config2", "config3", "config4", "copy", "max_subsampling", "bn_relu_max_subsampling", "max_subsampling_tiling",
-                             "entry_window", "concat", "maxout", "feature_map_stat", "config4_direct", "yardsticks"],
+                             "entry_window", "concat", "maxout", "feature_map_stat", "config4_direct", "yardsticks", "walking_grid"],
                     help="'copy' times the plain copy kernel (profiler-counter calibration and bandwidth yardstick); 'yardsticks' the runtime's and "
                          "torch's copy routines beside the library's kernels; 'config4_direct' the launches of config4 issued at the C ABI from this script")
     ap.add_argument("--entries", type=int, default=64, help="config4: entries per packet (BASELINE.json's configuration has 64)")
@@ -816,6 +819,8 @@ def main():
             return bench_maxout(runner, steps, warmup)
         if name == "feature_map_stat":
             return bench_feature_map_stat(runner, steps, warmup)
+        if name == "walking_grid":
+            return bench_group(runner, "batch_norm -> rectified_linear N=64 C=64 56x56 (51 MB per tensor: the grid that stays put)", w.bn_relu("bn_relu", 64, 64, 56 * 56), steps, warmup)
         if name == "config4_direct":
             return bench_resnet50_direct(runner, steps, warmup)
         if name == "yardsticks":
@@ -876,7 +881,8 @@ def main():
             "kernel": {"config1": "nnf::softmax_rows_kernel", "copy": "nnf::copy_kernel_impl", "max_subsampling": "nnf::max_window2d_kernel", "bn_relu_max_subsampling": "nnf::max_window2d_prologue_kernel",
                        "max_subsampling_tiling": "nnf::tiling2d_kernel", "entry_window": "nnf::window_rows_kernel",
                        "concat": "nnf::concat_kernel", "maxout": "nnf::maxout_vec4_kernel",
-                       "feature_map_stat": "nnf::stat_runs_kernel"}.get(args.workload, "nnf::chain_kernel"),
+                       "feature_map_stat": "nnf::stat_runs_kernel", "walking_grid": "nnf::chain_kernel_persistent",
+                       "config4": "nnf::chain_batch_kernel"}.get(args.workload, "nnf::chain_kernel"),
             "algorithmic_bytes_per_launch": main_entry["algorithmic_bytes_per_step"] / launches,
             "avg_launch_us": main_entry["event_ms_per_step"] * 1e3 / launches,
         },
