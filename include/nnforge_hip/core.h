@@ -147,12 +147,21 @@ namespace nnforge
 	typedef std::vector<unsigned int> data_config;
 	typedef std::vector<unsigned int> data_custom_config;
 
-	// Key/value view of a layer's "<type>_param { ... }" block of the text-format schema; nested
-	// blocks keep their order (e.g. one dimension_param per spatial dimension).
+	// A message of the text-format schema ("layer { ... }", "<type>_param { ... }", "dimension_param { ... }"): its
+	// scalar fields as text and its nested messages, which keep their order (e.g. one dimension_param per spatial
+	// dimension). It stands where the reference has the classes protoc generates from nnforge/proto/nnforge.proto:
+	// layer::read_proto / write_proto receive the layer's message as one of these.
 	struct schema_param_block
 	{
 		std::map<std::string, std::string> scalars;
+		std::vector<std::string> scalar_order; // the keys in the order set() received them: the order a writer emits
 		std::vector<std::pair<std::string, schema_param_block> > blocks;
+
+		// the first nested message of that name, null when there is none
+		const schema_param_block * child(const std::string& name) const;
+		// for writers: a scalar field (value as it appears in the text format), a nested message
+		void set(const std::string& key, const std::string& value_text);
+		schema_param_block& add_block(const std::string& name);
 
 		bool has(const std::string& key) const { return scalars.find(key) != scalars.end(); }
 		float get_float(const std::string& key, float default_value) const;
@@ -208,11 +217,12 @@ namespace nnforge
 		// floating point operations per entry of a forward pass (the reference's flops model)
 		virtual float get_forward_flops_per_entry(const std::vector<layer_configuration_specific>& input_configuration_specific_list) const = 0;
 
-		// name of the "<...>_param" block of this layer type in a schema file, empty if it has none
-		virtual std::string get_param_block_name() const { return std::string(); }
-		// reads the layer's parameters; block is null when the schema has no such block
-		virtual void read_params(const schema_param_block * block);
-		virtual void write_params(std::ostream& out, const std::string& indent) const;
+		// nnforge/layer.h:64-66. layer_proto points at the layer's message of the schema - here a schema_param_block
+		// (the "layer { ... }" block) where the reference has a protobuf::Layer. read_proto takes the layer's parameters
+		// from its "<type>_param" message (defaults, or an exception, when that is missing, as in the reference);
+		// write_proto adds that message when the reference's writer would.
+		virtual void read_proto(const void * layer_proto);
+		virtual void write_proto(void * layer_proto) const;
 
 		virtual std::vector<std::string> get_parameter_strings() const { return std::vector<std::string>(); }
 

@@ -29,9 +29,8 @@ namespace nnforge
 		layer::ptr clone() const override;
 		std::string get_type_name() const override;
 		float get_forward_flops_per_entry(const std::vector<layer_configuration_specific>& input_configuration_specific_list) const override;
-		std::string get_param_block_name() const override { return "batch_norm_param"; }
-		void read_params(const schema_param_block * block) override;
-		void write_params(std::ostream& out, const std::string& indent) const override;
+		void read_proto(const void * layer_proto) override;
+		void write_proto(void * layer_proto) const override;
 		data_config get_data_config() const override;
 		void initialize_data(layer_data& data) const override; // gamma 1, beta 0, mean 0, inverse sigma 1
 		std::vector<std::string> get_parameter_strings() const override;
@@ -54,9 +53,8 @@ namespace nnforge
 		layer::ptr clone() const override;
 		std::string get_type_name() const override;
 		float get_forward_flops_per_entry(const std::vector<layer_configuration_specific>& input_configuration_specific_list) const override;
-		std::string get_param_block_name() const override { return "relu_param"; }
-		void read_params(const schema_param_block * block) override;
-		void write_params(std::ostream& out, const std::string& indent) const override;
+		void read_proto(const void * layer_proto) override;
+		void write_proto(void * layer_proto) const override;
 		std::vector<std::string> get_parameter_strings() const override;
 
 		static const std::string layer_type_name;
@@ -71,9 +69,8 @@ namespace nnforge
 		layer::ptr clone() const override;
 		std::string get_type_name() const override;
 		float get_forward_flops_per_entry(const std::vector<layer_configuration_specific>& input_configuration_specific_list) const override;
-		std::string get_param_block_name() const override { return "prelu_param"; }
-		void read_params(const schema_param_block * block) override;
-		void write_params(std::ostream& out, const std::string& indent) const override;
+		void read_proto(const void * layer_proto) override;
+		void write_proto(void * layer_proto) const override;
 		data_config get_data_config() const override;
 		void initialize_data(layer_data& data) const override; // 0.25
 		std::vector<std::string> get_parameter_strings() const override;
@@ -115,9 +112,8 @@ namespace nnforge
 		layer::ptr clone() const override;
 		std::string get_type_name() const override;
 		float get_forward_flops_per_entry(const std::vector<layer_configuration_specific>& input_configuration_specific_list) const override;
-		std::string get_param_block_name() const override { return "tanh_param"; }
-		void read_params(const schema_param_block * block) override;
-		void write_params(std::ostream& out, const std::string& indent) const override;
+		void read_proto(const void * layer_proto) override;
+		void write_proto(void * layer_proto) const override;
 		std::vector<std::string> get_parameter_strings() const override;
 
 		static const std::string layer_type_name;
@@ -136,9 +132,8 @@ namespace nnforge
 			const std::vector<layer_configuration_specific>& input_configuration_specific_list) const override;
 		std::string get_type_name() const override;
 		float get_forward_flops_per_entry(const std::vector<layer_configuration_specific>& input_configuration_specific_list) const override;
-		std::string get_param_block_name() const override { return "add_param"; }
-		void read_params(const schema_param_block * block) override;
-		void write_params(std::ostream& out, const std::string& indent) const override;
+		void read_proto(const void * layer_proto) override;
+		void write_proto(void * layer_proto) const override;
 		std::vector<std::string> get_parameter_strings() const override;
 
 		static const std::string layer_type_name;
@@ -170,9 +165,8 @@ namespace nnforge
 			const std::vector<layer_configuration_specific>& input_configuration_specific_list) const override;
 		std::string get_type_name() const override;
 		float get_forward_flops_per_entry(const std::vector<layer_configuration_specific>& input_configuration_specific_list) const override;
-		std::string get_param_block_name() const override { return "average_subsampling_param"; }
-		void read_params(const schema_param_block * block) override;
-		void write_params(std::ostream& out, const std::string& indent) const override;
+		void read_proto(const void * layer_proto) override;
+		void write_proto(void * layer_proto) const override;
 		std::vector<std::string> get_parameter_strings() const override;
 
 		bool has_alpha() const { return alpha != -std::numeric_limits<float>::max(); }
@@ -232,9 +226,8 @@ namespace nnforge
 		layer::ptr clone() const override;
 		std::string get_type_name() const override;
 		float get_forward_flops_per_entry(const std::vector<layer_configuration_specific>&) const override { return 0.0F; }
-		std::string get_param_block_name() const override { return "dropout_param"; }
-		void read_params(const schema_param_block * block) override;
-		void write_params(std::ostream& out, const std::string& indent) const override;
+		void read_proto(const void * layer_proto) override;
+		void write_proto(void * layer_proto) const override;
 		std::vector<std::string> get_parameter_strings() const override;
 
 		static const std::string layer_type_name;
@@ -270,9 +263,8 @@ namespace nnforge
 			const std::vector<layer_configuration_specific>& input_configuration_specific_list) const override;
 		std::string get_type_name() const override;
 		float get_forward_flops_per_entry(const std::vector<layer_configuration_specific>& input_configuration_specific_list) const override;
-		std::string get_param_block_name() const override { return "maxout_param"; }
-		void read_params(const schema_param_block * block) override;
-		void write_params(std::ostream& out, const std::string& indent) const override;
+		void read_proto(const void * layer_proto) override;
+		void write_proto(void * layer_proto) const override;
 		std::vector<std::string> get_parameter_strings() const override;
 
 		static const std::string layer_type_name;
@@ -303,9 +295,8 @@ namespace nnforge
 			const std::vector<layer_configuration_specific>& input_configuration_specific_list) const override;
 		std::string get_type_name() const override;
 		float get_forward_flops_per_entry(const std::vector<layer_configuration_specific>& input_configuration_specific_list) const override;
-		std::string get_param_block_name() const override { return "max_subsampling_param"; }
-		void read_params(const schema_param_block * block) override;
-		void write_params(std::ostream& out, const std::string& indent) const override;
+		void read_proto(const void * layer_proto) override;
+		void write_proto(void * layer_proto) const override;
 		std::vector<std::string> get_parameter_strings() const override;
 		// tiling: the product of the window sizes; otherwise one over entry_subsampling_size
 		// (nnforge/max_subsampling_layer.cpp:239-268)

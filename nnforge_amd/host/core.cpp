@@ -220,6 +220,27 @@ namespace nnforge
 		return (it == scalars.end()) ? default_value : it->second;
 	}
 
+	const schema_param_block * schema_param_block::child(const std::string& name) const
+	{
+		for(const std::pair<std::string, schema_param_block>& b : blocks)
+			if (b.first == name)
+				return &b.second;
+		return nullptr;
+	}
+
+	void schema_param_block::set(const std::string& key, const std::string& value_text)
+	{
+		if (scalars.find(key) == scalars.end())
+			scalar_order.push_back(key);
+		scalars[key] = value_text;
+	}
+
+	schema_param_block& schema_param_block::add_block(const std::string& name)
+	{
+		blocks.push_back(std::make_pair(name, schema_param_block()));
+		return blocks.back().second;
+	}
+
 	std::vector<const schema_param_block *> schema_param_block::children(const std::string& name) const
 	{
 		std::vector<const schema_param_block *> res;
@@ -298,11 +319,11 @@ namespace nnforge
 		return input_configuration_specific_list.front();
 	}
 
-	void layer::read_params(const schema_param_block *)
+	void layer::read_proto(const void *)
 	{
 	}
 
-	void layer::write_params(std::ostream&, const std::string&) const
+	void layer::write_proto(void *) const
 	{
 	}
 

@@ -60,8 +60,9 @@ namespace nnforge
 		return neuron_count_of(configs) * 5.0F; // the reference's count (nnforge/batch_norm_layer.cpp:66)
 	}
 
-	void batch_norm_layer::read_params(const schema_param_block * block)
+	void batch_norm_layer::read_proto(const void * layer_proto)
 	{
+		const schema_param_block * block = static_cast<const schema_param_block *>(layer_proto)->child("batch_norm_param");
 		if (block == nullptr)
 			throw neural_network_exception("No batch_norm_param specified for layer " + instance_name + " of type " + layer_type_name);
 		feature_map_count = block->require_uint("feature_map_count", "batch_norm_param of layer " + instance_name);
@@ -69,11 +70,12 @@ namespace nnforge
 		check();
 	}
 
-	void batch_norm_layer::write_params(std::ostream& out, const std::string& indent) const
+	void batch_norm_layer::write_proto(void * layer_proto) const
 	{
-		out << indent << "feature_map_count: " << feature_map_count << "\n";
+		schema_param_block& param = static_cast<schema_param_block *>(layer_proto)->add_block("batch_norm_param");
+		param.set("feature_map_count", std::to_string(feature_map_count));
 		if (epsilon != default_batch_normalization_epsilon)
-			out << indent << "epsilon: " << float_text(epsilon) << "\n";
+			param.set("epsilon", float_text(epsilon));
 	}
 
 	data_config batch_norm_layer::get_data_config() const
@@ -112,15 +114,16 @@ namespace nnforge
 		return neuron_count_of(configs);
 	}
 
-	void rectified_linear_layer::read_params(const schema_param_block * block)
+	void rectified_linear_layer::read_proto(const void * layer_proto)
 	{
+		const schema_param_block * block = static_cast<const schema_param_block *>(layer_proto)->child("relu_param");
 		negative_slope = (block != nullptr) ? block->get_float("negative_slope", 0.0F) : 0.0F;
 	}
 
-	void rectified_linear_layer::write_params(std::ostream& out, const std::string& indent) const
+	void rectified_linear_layer::write_proto(void * layer_proto) const
 	{
 		if (negative_slope != 0.0F)
-			out << indent << "negative_slope: " << float_text(negative_slope) << "\n";
+			static_cast<schema_param_block *>(layer_proto)->add_block("relu_param").set("negative_slope", float_text(negative_slope));
 	}
 
 	std::vector<std::string> rectified_linear_layer::get_parameter_strings() const
@@ -155,17 +158,18 @@ namespace nnforge
 		return neuron_count_of(configs) * 2.0F;
 	}
 
-	void parametric_rectified_linear_layer::read_params(const schema_param_block * block)
+	void parametric_rectified_linear_layer::read_proto(const void * layer_proto)
 	{
+		const schema_param_block * block = static_cast<const schema_param_block *>(layer_proto)->child("prelu_param");
 		if (block == nullptr)
 			throw neural_network_exception("No prelu_param specified for layer " + instance_name + " of type " + layer_type_name);
 		feature_map_count = block->require_uint("feature_map_count", "prelu_param of layer " + instance_name);
 		check();
 	}
 
-	void parametric_rectified_linear_layer::write_params(std::ostream& out, const std::string& indent) const
+	void parametric_rectified_linear_layer::write_proto(void * layer_proto) const
 	{
-		out << indent << "feature_map_count: " << feature_map_count << "\n";
+		static_cast<schema_param_block *>(layer_proto)->add_block("prelu_param").set("feature_map_count", std::to_string(feature_map_count));
 	}
 
 	data_config parametric_rectified_linear_layer::get_data_config() const
@@ -215,18 +219,22 @@ namespace nnforge
 		return neuron_count_of(configs) * 6.0F;
 	}
 
-	void hyperbolic_tangent_layer::read_params(const schema_param_block * block)
+	void hyperbolic_tangent_layer::read_proto(const void * layer_proto)
 	{
+		const schema_param_block * block = static_cast<const schema_param_block *>(layer_proto)->child("tanh_param");
 		scale = (block != nullptr) ? block->get_float("scale", 1.0F) : 1.0F;
 		steepness = (block != nullptr) ? block->get_float("steepness", 1.0F) : 1.0F;
 	}
 
-	void hyperbolic_tangent_layer::write_params(std::ostream& out, const std::string& indent) const
+	void hyperbolic_tangent_layer::write_proto(void * layer_proto) const
 	{
+		if ((scale == 1.0F) && (steepness == 1.0F))
+			return;
+		schema_param_block& param = static_cast<schema_param_block *>(layer_proto)->add_block("tanh_param");
 		if (scale != 1.0F)
-			out << indent << "scale: " << float_text(scale) << "\n";
+			param.set("scale", float_text(scale));
 		if (steepness != 1.0F)
-			out << indent << "steepness: " << float_text(steepness) << "\n";
+			param.set("steepness", float_text(steepness));
 	}
 
 	std::vector<std::string> hyperbolic_tangent_layer::get_parameter_strings() const
@@ -266,15 +274,16 @@ namespace nnforge
 		return neuron_count_of(configs) * static_cast<float>(configs.size());
 	}
 
-	void add_layer::read_params(const schema_param_block * block)
+	void add_layer::read_proto(const void * layer_proto)
 	{
+		const schema_param_block * block = static_cast<const schema_param_block *>(layer_proto)->child("add_param");
 		alpha = (block != nullptr) ? block->get_float("alpha", 1.0F) : 1.0F;
 	}
 
-	void add_layer::write_params(std::ostream& out, const std::string& indent) const
+	void add_layer::write_proto(void * layer_proto) const
 	{
 		if (alpha != 1.0F)
-			out << indent << "alpha: " << float_text(alpha) << "\n";
+			static_cast<schema_param_block *>(layer_proto)->add_block("add_param").set("alpha", float_text(alpha));
 	}
 
 	std::vector<std::string> add_layer::get_parameter_strings() const
@@ -381,8 +390,9 @@ namespace nnforge
 		return static_cast<float>(out.get_neuron_count()) * per_item;
 	}
 
-	void average_subsampling_layer::read_params(const schema_param_block * block)
+	void average_subsampling_layer::read_proto(const void * layer_proto)
 	{
+		const schema_param_block * block = static_cast<const schema_param_block *>(layer_proto)->child("average_subsampling_param");
 		if (block == nullptr)
 			throw neural_network_exception("No average_subsampling_param specified for layer " + instance_name + " of type " + layer_type_name);
 		subsampling_sizes.clear();
@@ -428,16 +438,17 @@ namespace nnforge
 			throw neural_network_exception("feature map and entry subsampling sizes for average subsampling layer may not be zero");
 	}
 
-	void average_subsampling_layer::write_params(std::ostream& out, const std::string& indent) const
+	void average_subsampling_layer::write_proto(void * layer_proto) const
 	{
+		schema_param_block& param = static_cast<schema_param_block *>(layer_proto)->add_block("average_subsampling_param");
 		for(size_t i = 0; i < subsampling_sizes.size(); ++i)
-			out << indent << "dimension_param { " << (is_relative(i) ? "subsampling_size: " : "subsampled_size: ") << subsampling_sizes[i] << " }\n";
+			param.add_block("dimension_param").set(is_relative(i) ? "subsampling_size" : "subsampled_size", std::to_string(subsampling_sizes[i]));
 		if (!feature_map_relative || (feature_map_subsampling_size != 1))
-			out << indent << "feature_map_param { " << (feature_map_relative ? "subsampling_size: " : "subsampled_size: ") << feature_map_subsampling_size << " }\n";
+			param.add_block("feature_map_param").set(feature_map_relative ? "subsampling_size" : "subsampled_size", std::to_string(feature_map_subsampling_size));
 		if (entry_subsampling_size != 1)
-			out << indent << "entry_param { subsampling_size: " << entry_subsampling_size << " }\n";
+			param.add_block("entry_param").set("subsampling_size", std::to_string(entry_subsampling_size));
 		if (has_alpha())
-			out << indent << "alpha: " << float_text(alpha) << "\n";
+			param.set("alpha", float_text(alpha));
 	}
 
 	std::vector<std::string> average_subsampling_layer::get_parameter_strings() const
@@ -503,22 +514,24 @@ namespace nnforge
 	layer::ptr dropout_layer::clone() const { return layer::ptr(new dropout_layer(*this)); }
 	std::string dropout_layer::get_type_name() const { return layer_type_name; }
 
-	void dropout_layer::read_params(const schema_param_block * block)
+	void dropout_layer::read_proto(const void * layer_proto)
 	{
+		const schema_param_block * block = static_cast<const schema_param_block *>(layer_proto)->child("dropout_param");
 		// nnforge/dropout_layer.cpp:82-88: a missing block gives the defaults of the message
 		dropout_rate = (block != nullptr) ? block->get_float("dropout_rate", 0.5F) : 0.5F;
 		per_feature_map = (block != nullptr) ? block->get_bool("per_feature_map", false) : false;
 		check();
 	}
 
-	void dropout_layer::write_params(std::ostream& out, const std::string& indent) const
+	void dropout_layer::write_proto(void * layer_proto) const
 	{
 		// nnforge/dropout_layer.cpp:70-80 writes the block only for a rate other than 0.5
 		if (dropout_rate != 0.5F)
 		{
-			out << indent << "dropout_rate: " << float_text(dropout_rate) << "\n";
+			schema_param_block& param = static_cast<schema_param_block *>(layer_proto)->add_block("dropout_param");
+			param.set("dropout_rate", float_text(dropout_rate));
 			if (per_feature_map)
-				out << indent << "per_feature_map: true\n";
+				param.set("per_feature_map", "true");
 		}
 	}
 
@@ -588,17 +601,18 @@ namespace nnforge
 		return static_cast<float>(get_output_layer_configuration_specific(configs).get_neuron_count()) * static_cast<float>(feature_map_subsampling_size - 1);
 	}
 
-	void maxout_layer::read_params(const schema_param_block * block)
+	void maxout_layer::read_proto(const void * layer_proto)
 	{
+		const schema_param_block * block = static_cast<const schema_param_block *>(layer_proto)->child("maxout_param");
 		if (block == nullptr)
 			throw neural_network_exception("No maxout_param specified for layer " + instance_name + " of type " + layer_type_name);
 		feature_map_subsampling_size = block->require_uint("feature_map_subsampling_size", "maxout_param of layer " + instance_name);
 		check();
 	}
 
-	void maxout_layer::write_params(std::ostream& out, const std::string& indent) const
+	void maxout_layer::write_proto(void * layer_proto) const
 	{
-		out << indent << "feature_map_subsampling_size: " << feature_map_subsampling_size << "\n";
+		static_cast<schema_param_block *>(layer_proto)->add_block("maxout_param").set("feature_map_subsampling_size", std::to_string(feature_map_subsampling_size));
 	}
 
 	std::vector<std::string> maxout_layer::get_parameter_strings() const
@@ -714,8 +728,9 @@ namespace nnforge
 		return static_cast<float>(neuron_count) * static_cast<float>(per_item - 1);
 	}
 
-	void max_subsampling_layer::read_params(const schema_param_block * block)
+	void max_subsampling_layer::read_proto(const void * layer_proto)
 	{
+		const schema_param_block * block = static_cast<const schema_param_block *>(layer_proto)->child("max_subsampling_param");
 		if (block == nullptr)
 			throw neural_network_exception("No max_subsampling_param specified for layer " + instance_name + " of type " + layer_type_name);
 		subsampling_sizes.clear();
@@ -740,25 +755,26 @@ namespace nnforge
 		check();
 	}
 
-	void max_subsampling_layer::write_params(std::ostream& out, const std::string& indent) const
+	void max_subsampling_layer::write_proto(void * layer_proto) const
 	{
+		schema_param_block& param = static_cast<schema_param_block *>(layer_proto)->add_block("max_subsampling_param");
 		for(size_t i = 0; i < subsampling_sizes.size(); ++i)
 		{
-			out << indent << "dimension_param { subsampling_size: " << subsampling_sizes[i];
+			schema_param_block& dim = param.add_block("dimension_param");
+			dim.set("subsampling_size", std::to_string(subsampling_sizes[i]));
 			if (round_ups[i])
-				out << " round_up: true";
+				dim.set("round_up", "true");
 			if (strides[i] != subsampling_sizes[i])
-				out << " stride: " << strides[i];
-			out << " }\n";
+				dim.set("stride", std::to_string(strides[i]));
 		}
 		if (tiling)
-			out << indent << "tiling: true\n";
+			param.set("tiling", "true");
 		if (feature_map_subsampling_size != 1)
-			out << indent << "feature_map_param { subsampling_size: " << feature_map_subsampling_size << " }\n";
+			param.add_block("feature_map_param").set("subsampling_size", std::to_string(feature_map_subsampling_size));
 		if (entry_subsampling_size != 1)
-			out << indent << "entry_param { subsampling_size: " << entry_subsampling_size << " }\n";
+			param.add_block("entry_param").set("subsampling_size", std::to_string(entry_subsampling_size));
 		if (is_min)
-			out << indent << "function: MIN\n";
+			param.set("function", "MIN");
 	}
 
 	std::vector<std::string> max_subsampling_layer::get_parameter_strings() const

@@ -236,18 +236,39 @@ namespace nnforge
 			l->instance_name = lb->scalars.find("name")->second;
 			for(const schema_param_block * in : lb->children("input_layer_name"))
 				l->input_layer_instance_names.push_back(in->scalars.find("value")->second);
-			const std::string param_name = l->get_param_block_name();
-			const schema_param_block * param = nullptr;
-			if (!param_name.empty())
-			{
-				std::vector<const schema_param_block *> found = lb->children(param_name);
-				if (!found.empty())
-					param = found.front();
-			}
-			l->read_params(param);
+			l->read_proto(lb);
 			layer_list.push_back(l);
 		}
 		rebuild(layer_list);
+	}
+
+	namespace
+	{
+		void write_inline(std::ostream& out, const schema_param_block& block)
+		{
+			for(const std::string& key : block.scalar_order)
+				out << key << ": " << block.scalars.find(key)->second << " ";
+			for(const std::pair<std::string, schema_param_block>& nested : block.blocks)
+			{
+				out << nested.first << " { ";
+				write_inline(out, nested.second);
+				out << "} ";
+			}
+		}
+
+		// the fields of a message a layer wrote: nested messages first (a line each), then the scalars, as the
+		// files this backend has always written
+		void write_fields(std::ostream& out, const schema_param_block& block, const std::string& indent)
+		{
+			for(const std::pair<std::string, schema_param_block>& nested : block.blocks)
+			{
+				out << indent << nested.first << " { ";
+				write_inline(out, nested.second);
+				out << "}\n";
+			}
+			for(const std::string& key : block.scalar_order)
+				out << indent << key << ": " << block.scalars.find(key)->second << "\n";
+		}
 	}
 
 	void network_schema::write_proto(std::ostream& out) const
@@ -261,10 +282,15 @@ namespace nnforge
 			out << "\tname: \"" << l->instance_name << "\"\n";
 			for(const std::string& input : l->input_layer_instance_names)
 				out << "\tinput_layer_name: \"" << input << "\"\n";
-			std::ostringstream params;
-			l->write_params(params, "\t\t");
-			if (!l->get_param_block_name().empty() && !params.str().empty())
-				out << "\t" << l->get_param_block_name() << " {\n" << params.str() << "\t}\n";
+			// the layer adds its "<type>_param" message (if it has anything to say); nested messages of that go on one line
+			schema_param_block message;
+			l->write_proto(&message);
+			for(const std::pair<std::string, schema_param_block>& param : message.blocks)
+			{
+				out << "\t" << param.first << " {\n";
+				write_fields(out, param.second, "\t\t");
+				out << "\t}\n";
+			}
 			out << "}\n";
 		}
 	}
