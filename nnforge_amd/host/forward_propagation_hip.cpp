@@ -828,6 +828,24 @@ namespace nnforge
 			if (index_fit == 0)
 				throw neural_network_exception("A single entry of " + std::to_string(largest_floats_per_entry) + " values in one layer is beyond the hip kernels' index range");
 			max_entry_count = static_cast<unsigned int>(std::min<size_t>(max_entry_count, index_fit));
+			// A run into a statistics writer also holds, per output layer, the running states and the workspace of the
+			// reduction (a few KB to MB): where the budget is that tight, the packet gives them room
+			{
+				size_t stat_bytes = 0;
+				for(const std::string& n : output_layer_names)
+				{
+					const layer_configuration_specific& c = layer_config_map[n];
+					size_t workspace = 0;
+					if (nnf_hip_feature_map_stat_workspace_bytes(max_entry_count * output_layers_tiling_factor, c.feature_map_count, c.get_neuron_count_per_feature_map(), &workspace) == NNF_HIP_OK)
+						stat_bytes += workspace + static_cast<size_t>(c.feature_map_count) * sizeof(nnf_hip_running_stat);
+				}
+				const size_t used = weight_bytes + device_bytes_per_entry * max_entry_count;
+				if ((used + stat_bytes > budget) && (max_entry_count > 1))
+				{
+					const size_t give_up = (used + stat_bytes - budget + device_bytes_per_entry - 1) / device_bytes_per_entry;
+					max_entry_count = static_cast<unsigned int>(std::max<size_t>(1, max_entry_count - std::min<size_t>(give_up, max_entry_count - 1)));
+				}
+			}
 
 			if (debug->is_debug())
 			{

@@ -139,7 +139,9 @@ def test_plan_memory_budget():
     per_entry = 3 * 8 * 49 * 4
     # all three buffers belong to data or output layers: each exists twice, once per packet in flight
     rep = plan(S.resnet_block(8), cfg, ["res_relu"], memory_bytes=200 * per_entry)
-    assert rep["max_entry_count"] in (89, 90)   # 0.9 of the memory (the ratio is an fp32 number)
+    # 0.9 of the memory (the ratio is an fp32 number) holds 89 or 90 entries; two or three of them make room for the
+    # running states and the workspace a run into a statistics writer would need for the output layer
+    assert 86 <= rep["max_entry_count"] <= 88
     rep = plan(S.resnet_block(8), cfg, ["res_relu"], memory_bytes=1 << 40, max_entry_count=77)
     assert rep["max_entry_count"] == 77
     with pytest.raises(backend.BackendError, match="Insufficient memory to do forward prop for even one sample"):
