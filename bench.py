@@ -523,7 +523,6 @@ def bench_yardsticks(runner, steps, warmup):
             ("torch add(a, b, out=c) (2 reads, 1 write)", 3, lambda i: torch.add(a[i % sets], b[i % sets], out=out[i % sets])),
             ("torch fill_ (write only)", 1, lambda i: out[i % sets].fill_(1.0)),
             ("hipMemsetAsync through torch zero_ (write only)", 1, lambda i: out[i % sets].zero_()),
-            ("torch sum (read only, reduced to one float)", 1, lambda i: torch.sum(a[i % sets])),
         ]
         for name, tensors, fn in candidates:
             for i in range(3):
