@@ -887,14 +887,15 @@ namespace nnf
 				// Measured on MI355X. One input: tensors of 64 MB and more stream best with two float4s per lane,
 				// smaller ones with four, as long as enough workgroups exist to cover the machine. Several inputs:
 				// two float4s per lane at every size (4 % faster than four from 10 to 130 MB per tensor).
-				// As one of several groups of a launch: two float4s per lane whatever the size - the grid is all the
-				// groups' tiles, so a small group need not be cut finer to cover the machine, and groups of one tile
-				// size share launches (the 49 groups of the ResNet-50 stack at 64 entries, launched together where
-				// they can be: 1078 us with four float4s for all, 1067 with two, 1189 with one, 1085 chosen by size).
+				// As one of several groups of a launch: the tile size follows the number of inputs alone (four float4s per lane
+				// with one input, two with several) - the grid is all the groups' tiles, so a small group need not be cut
+				// finer to cover the machine, and groups of one tile size share launches (the 49 groups of the ResNet-50
+				// stack at 64 entries, launched together where they can be: 1067-1071 us this way, 1078 with four float4s
+				// for all, 1067 with two for all, 1189 with one, 1085 with the sizes chosen as for single launches).
 				static const int small_tile_order[] = { 1, 2, 3 };
 				static const int any_tile_order[] = { 0, 1, 2, 3 };
 				const bool large = (a.total >= large_tensor_elements) || !single_launch;
-				const bool small_tiles = large || (desc->input_count > 1);
+				const bool small_tiles = (single_launch && large) || (desc->input_count > 1);
 				const int* order = small_tiles ? small_tile_order : any_tile_order;
 				const int order_count = small_tiles ? 3 : 4;
 				shape = -1;
