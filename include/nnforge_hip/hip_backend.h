@@ -292,9 +292,11 @@ namespace nnforge
 		private:
 			struct impl;
 			struct run_buffers;
-			// streams, device buffers for packets of `packet` entries (data and output layers once per I/O slot), weight pointers
-			void prepare_run(run_buffers& r, unsigned int packet, int slot_count);
+			// streams, device buffers for packets of `packet` entries (data and output layers once per I/O slot), pinned
+			// staging, weight pointers; what the run before left is used again when it was made for the same sizes
+			run_buffers& prepare_run(unsigned int packet, int slot_count, bool with_output_staging, bool stats_on_device);
 			std::unique_ptr<impl> p;
+			std::unique_ptr<run_buffers> kept_run; // released when the weights, the shapes or the packet size change
 			hip_running_configuration::const_ptr hip_config;
 			std::vector<forward_step> steps;
 			size_t per_entry_bytes;

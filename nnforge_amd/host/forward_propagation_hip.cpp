@@ -105,6 +105,25 @@ namespace nnforge
 			};
 		}
 
+		// What a run holds on the device and in pinned host memory: data and output layer buffers once per I/O
+		// slot, the rest shared; the working buffers testers ask for, per step (steps on different streams may
+		// run at the same time); pinned staging per slot; the states and the workspace of the statistics. Kept
+		// in the object from one run to the next while the packet size, the kind of writer, the weights and the
+		// plan stay the same, so that a caller who runs data set after data set allocates once.
+		struct forward_propagation_hip::run_buffers
+		{
+			unsigned int packet = 0;
+			int slot_count = 0;
+			bool with_output_staging = false;
+			bool stats_on_device = false;
+			std::vector<hip_linear_buffer_device::ptr> buffers[2];
+			std::vector<std::pair<hip_linear_buffer_device::ptr, hip_linear_buffer_device::ptr> > temporary;
+			std::vector<std::vector<const float *> > chunk_ptrs; // weight pointers of the fused steps
+			std::map<std::string, std::unique_ptr<pinned_buffer> > staging[2];
+			std::map<std::string, hip_linear_buffer_device::ptr> stat_states, stat_workspaces;
+			std::map<std::string, size_t> stat_workspace_bytes;
+		};
+
 		struct forward_propagation_hip::impl
 		{
 			std::vector<layer::const_ptr> exec_layers; // layers with inputs, execution order
@@ -283,6 +302,7 @@ namespace nnforge
 
 		void forward_propagation_hip::actual_set_data(network_data::const_ptr data)
 		{
+			kept_run.reset(); // it holds pointers to the weights
 			p->host_data = data;
 			p->weights.clear();
 			p->weights_custom.clear();
@@ -306,6 +326,7 @@ namespace nnforge
 
 		void forward_propagation_hip::actual_clear_data()
 		{
+			kept_run.reset();
 			p->host_data.reset();
 			p->weights.clear();
 			p->weights_custom.clear();
@@ -314,6 +335,7 @@ namespace nnforge
 		void forward_propagation_hip::layer_config_map_modified()
 		{
 			hip_config->set_device();
+			kept_run.reset(); // sized for the plan that is about to be replaced
 
 			// testers for the new shapes
 			p->testers.clear();
@@ -872,18 +894,19 @@ namespace nnforge
 			};
 		}
 
-		// Device buffers of a run: data and output layer buffers once per I/O slot, the rest shared; the
-		// working buffers testers ask for, per step (steps on different streams may run at the same time).
-		struct forward_propagation_hip::run_buffers
-		{
-			std::vector<hip_linear_buffer_device::ptr> buffers[2];
-			std::vector<std::pair<hip_linear_buffer_device::ptr, hip_linear_buffer_device::ptr> > temporary;
-			std::vector<std::vector<const float *> > chunk_ptrs; // weight pointers of the fused steps
-		};
-
-		void forward_propagation_hip::prepare_run(run_buffers& r, unsigned int packet, int slot_count)
+		forward_propagation_hip::run_buffers& forward_propagation_hip::prepare_run(unsigned int packet, int slot_count, bool with_output_staging, bool stats_on_device)
 		{
 			hip_config->set_device();
+			if (kept_run && (kept_run->packet == packet) && (kept_run->slot_count == slot_count)
+				&& (kept_run->with_output_staging == with_output_staging) && (kept_run->stats_on_device == stats_on_device))
+				return *kept_run;
+			kept_run.reset(); // what the run before held goes first: both sets need not fit side by side
+			std::unique_ptr<run_buffers> fresh(new run_buffers());
+			run_buffers& r = *fresh;
+			r.packet = packet;
+			r.slot_count = slot_count;
+			r.with_output_staging = with_output_staging;
+			r.stats_on_device = stats_on_device;
 			unsigned int stream_count = 1;
 			for(const forward_step& step : steps)
 				stream_count = std::max(stream_count, step.stream_index + 1);
@@ -925,6 +948,31 @@ namespace nnforge
 				for(const std::string& layer_name : p->plans[i].chunk_layers)
 					for(const hip_linear_buffer_device::const_ptr& b : p->weights.at(layer_name))
 						r.chunk_ptrs[i].push_back(static_cast<const float *>(*b));
+
+			// pinned staging per I/O slot: the data layers, and the output layers unless only their statistics are wanted
+			for(int s = 0; s < slot_count; ++s)
+			{
+				for(const std::string& n : data_layer_names)
+					r.staging[s][n].reset(new pinned_buffer(static_cast<size_t>(layer_config_map[n].get_neuron_count()) * sizeof(float) * packet));
+				if (with_output_staging)
+					for(const std::string& n : output_layer_names)
+						if (r.staging[s].find(n) == r.staging[s].end())
+							r.staging[s][n].reset(new pinned_buffer(static_cast<size_t>(layer_config_map[n].get_neuron_count()) * sizeof(float) * packet * output_layers_tiling_factor));
+			}
+			if (stats_on_device)
+			{
+				for(const std::string& n : output_layer_names)
+				{
+					const layer_configuration_specific& c = layer_config_map[n];
+					r.stat_states[n].reset(new hip_linear_buffer_device(static_cast<size_t>(c.feature_map_count) * sizeof(nnf_hip_running_stat)));
+					size_t bytes = 0;
+					hip_safe_call(nnf_hip_feature_map_stat_workspace_bytes(packet * output_layers_tiling_factor, c.feature_map_count, c.get_neuron_count_per_feature_map(), &bytes));
+					r.stat_workspaces[n].reset(new hip_linear_buffer_device(bytes));
+					r.stat_workspace_bytes[n] = bytes;
+				}
+			}
+			kept_run = std::move(fresh);
+			return *kept_run;
 		}
 
 		// Packets of entries flow through in-order queues with two I/O slots (the double buffering
@@ -951,41 +999,21 @@ namespace nnforge
 			if (reader_entry_count > 0)
 				packet = std::min(packet, static_cast<unsigned int>(reader_entry_count));
 
-			constexpr int slot_count = 2;
-			run_buffers r;
-			prepare_run(r, packet, slot_count);
-
 			// A statistics writer (nnforge/stat_data_bunch_writer.h) only wants per-feature-map figures of the
 			// outputs: they are reduced where they lie, in device memory, and nothing but the running
 			// states (32 bytes per feature map) travels to the host at the end of the run.
 			stat_data_bunch_writer * stat_writer = dynamic_cast<stat_data_bunch_writer *>(&writer);
 			const bool stats_on_device = (stat_writer != nullptr);
-			std::map<std::string, hip_linear_buffer_device::ptr> stat_states, stat_workspaces;
-			std::map<std::string, size_t> stat_workspace_bytes;
-			if (stats_on_device)
-			{
-				for(const std::string& n : output_layer_names)
-				{
-					const layer_configuration_specific& c = layer_config_map[n];
-					stat_states[n].reset(new hip_linear_buffer_device(static_cast<size_t>(c.feature_map_count) * sizeof(nnf_hip_running_stat)));
-					size_t bytes = 0;
-					hip_safe_call(nnf_hip_feature_map_stat_workspace_bytes(packet * output_layers_tiling_factor, c.feature_map_count, c.get_neuron_count_per_feature_map(), &bytes));
-					stat_workspaces[n].reset(new hip_linear_buffer_device(bytes));
-					stat_workspace_bytes[n] = bytes;
-					hip_safe_call(nnf_hip_feature_map_stat_init(p->stream, static_cast<nnf_hip_running_stat *>(static_cast<void *>(*stat_states[n])), c.feature_map_count));
-				}
-			}
 
-			std::map<std::string, std::unique_ptr<pinned_buffer> > staging[slot_count];
-			for(int s = 0; s < slot_count; ++s)
-			{
-				for(const std::string& n : data_layer_names)
-					staging[s][n].reset(new pinned_buffer(static_cast<size_t>(layer_config_map[n].get_neuron_count()) * sizeof(float) * packet));
-				if (!stats_on_device)
-					for(const std::string& n : output_layer_names)
-						if (staging[s].find(n) == staging[s].end())
-							staging[s][n].reset(new pinned_buffer(static_cast<size_t>(layer_config_map[n].get_neuron_count()) * sizeof(float) * packet * output_layers_tiling_factor));
-			}
+			constexpr int slot_count = 2;
+			run_buffers& r = prepare_run(packet, slot_count, !stats_on_device, stats_on_device);
+			std::map<std::string, std::unique_ptr<pinned_buffer> > (&staging)[2] = r.staging;
+			std::map<std::string, hip_linear_buffer_device::ptr>& stat_states = r.stat_states;
+			std::map<std::string, hip_linear_buffer_device::ptr>& stat_workspaces = r.stat_workspaces;
+			std::map<std::string, size_t>& stat_workspace_bytes = r.stat_workspace_bytes;
+			if (stats_on_device)
+				for(const std::string& n : output_layer_names)
+					hip_safe_call(nnf_hip_feature_map_stat_init(p->stream, static_cast<nnf_hip_running_stat *>(static_cast<void *>(*stat_states[n])), layer_config_map[n].feature_map_count));
 			hip_event upload_done[slot_count], kernels_done[slot_count], download_done[slot_count];
 			bool slot_used[slot_count] = { false, false };
 
@@ -1142,17 +1170,14 @@ namespace nnforge
 				throw neural_network_exception("This forward_propagation_hip was created for planning only (offline configuration): it cannot run");
 			set_input_configuration_specific(reader.get_config_map());
 			const unsigned int packet = std::min(std::max(1U, entry_count), max_entry_count);
-			run_buffers r;
-			prepare_run(r, packet, 1);
+			run_buffers& r = prepare_run(packet, 1, false, false);
 			drain_streams drain_on_exit;
 			drain_on_exit.streams = p->kernel_streams;
 
 			// one packet, read and uploaded once
 			unsigned int entries_read = 0;
 			{
-				std::map<std::string, std::unique_ptr<pinned_buffer> > staging;
-				for(const std::string& n : data_layer_names)
-					staging[n].reset(new pinned_buffer(static_cast<size_t>(layer_config_map[n].get_neuron_count()) * sizeof(float) * packet));
+				std::map<std::string, std::unique_ptr<pinned_buffer> >& staging = r.staging[0];
 				for(; entries_read < packet; ++entries_read)
 				{
 					std::map<std::string, float *> data_map;

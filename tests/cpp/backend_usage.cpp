@@ -254,6 +254,39 @@ int main(int argc, char ** argv)
 			}
 		}
 
+		// One object, run after run: what a run allocated is used again by the next one and must follow new
+		// weights and another kind of writer. Reference: a fresh object with the new weights.
+		{
+			network_data other(schema.get_layers(), data);
+			layer_data::ptr steeper(new layer_data(*data.get("res_prelu")));
+			for(float& v : (*steeper)[0])
+				v *= 3.0F;
+			other.add("res_prelu", steeper);
+			forward_propagation::ptr fresh = generator.create_forward_propagation_factory()->create(
+				schema, outputs, debug_state::ptr(), profile_state::ptr());
+			fresh->set_data(other);
+			memory_data_bunch_writer want;
+			fresh->run(reader, want);
+			if (want.values["res_prelu"] == writer.values["res_prelu"])
+			{
+				std::cout << "other slopes, same output: the check checks nothing" << std::endl;
+				return 1;
+			}
+			fp->set_data(other);
+			memory_data_bunch_writer got;
+			fp->run(reader, got);
+			stat_data_bunch_writer statistics_between;
+			fp->run(reader, statistics_between);
+			memory_data_bunch_writer got_again;
+			fp->run(reader, got_again);
+			if ((got.values != want.values) || (got_again.values != want.values) || (statistics_between.get_entry_count() != entries))
+			{
+				std::cout << "runs of one object after new weights / another writer differ from a fresh object" << std::endl;
+				return 1;
+			}
+			fp->set_data(data);
+		}
+
 		// toolset::update_bn_weights as a library call: afterwards the batch norm output, taken with
 		// gamma 1 and beta 0, has mean 0 and deviation 1 over the reader's data
 		update_bn_weights(schema, data, reader, *generator.create_forward_propagation_factory(), debug_state::ptr(), profile_state::ptr(), nullptr);
