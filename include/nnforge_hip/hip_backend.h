@@ -62,7 +62,7 @@ namespace nnforge
 
 			// queries the device (throws when there is none)
 			hip_running_configuration(int device_id, float max_global_memory_usage_ratio, bool fuse_layers, bool dont_share_buffers, int max_entry_count,
-				int kernel_stream_count = default_kernel_stream_count, bool batch_independent_groups = true);
+				int kernel_stream_count = default_kernel_stream_count, bool batch_independent_groups = true, unsigned int reserved_thread_count = 1);
 			// A configuration that never touches a device: for planning launches and buffers (and testing
 			// that logic) on a machine without a GPU. Running a network with it throws.
 			static std::shared_ptr<const hip_running_configuration> create_offline(
@@ -71,6 +71,12 @@ namespace nnforge
 			bool is_offline() const { return offline; }
 			void set_device() const;
 			size_t get_max_bytes() const;
+			// The threads that read input entries, one job per entry, while the thread that called run() hands the packet
+			// before to the writer (nnforge/cuda/cuda_multi_running_configuration.h:55, .cpp:96-97): as many as the
+			// process has processors, less reserved_thread_count, at least 1 and at most max_job_thread_count (reading
+			// entries is copying: beyond that the host's memory is the limit, not its cores). None when offline.
+			threadpool_job_runner::ptr get_job_runner() const { return job_runner; }
+			static constexpr unsigned int max_job_thread_count = 16;
 
 			int device_id;
 			float max_global_memory_usage_ratio;
@@ -88,6 +94,7 @@ namespace nnforge
 			// on the 49 groups of the ResNet-50 post-convolution stack, all in one call: 64 entries 1091 -> 1042 us,
 			// 8 entries 243 -> 172 us.
 			bool batch_independent_groups;
+			unsigned int reserved_thread_count;
 			std::string device_name;
 			unsigned long long global_memory_size;
 			unsigned int compute_unit_count;
@@ -97,6 +104,7 @@ namespace nnforge
 		private:
 			hip_running_configuration() = default;
 			bool offline = false;
+			threadpool_job_runner::ptr job_runner;
 		};
 
 		std::ostream& operator<<(std::ostream& out, const hip_running_configuration& config);
@@ -262,6 +270,8 @@ namespace nnforge
 			// device bytes per entry of the current buffer plan, and the packet size derived from it
 			size_t get_per_entry_buffer_bytes() const { return per_entry_bytes; }
 			unsigned int get_max_entry_count() const { return max_entry_count; }
+			// run() makes its packets no larger than this much pinned staging (input + output entries) per I/O slot
+			static constexpr size_t max_io_staging_bytes_per_slot = static_cast<size_t>(64) << 20;
 
 			// Times the launch plan alone, on data that stays in device memory: reads one packet of up to entry_count
 			// entries from the reader and uploads it, runs the plan warmup times untimed, then `passes` times bracketed
@@ -320,7 +330,8 @@ namespace nnforge
 
 		// nnforge/cuda/factory_generator_cuda.h: options hip_device_id, hip_max_global_memory_usage_ratio,
 		// hip_fuse, hip_dont_share_buffers, hip_single_command_stream (as cuda_single_command_stream,
-		// nnforge/cuda/factory_generator_cuda.cpp:105-106), hip_batch_independent_groups, hip_kernel_stream_count, hip_max_entry_count
+		// nnforge/cuda/factory_generator_cuda.cpp:105-106), hip_batch_independent_groups, hip_kernel_stream_count, hip_max_entry_count,
+		// hip_reserved_thread_count (as cuda_reserved_thread_count, nnforge/cuda/factory_generator_cuda.cpp:95)
 		class factory_generator_hip : public factory_generator
 		{
 		public:
@@ -341,6 +352,7 @@ namespace nnforge
 			bool hip_batch_independent_groups;
 			int hip_kernel_stream_count;
 			int hip_max_entry_count;
+			int hip_reserved_thread_count;
 
 		private:
 			hip_running_configuration::const_ptr hip_config;

@@ -5,6 +5,7 @@
 #include "core.h"
 #include "schema.h"
 
+#include <functional>
 #include <map>
 #include <set>
 #include <string>
@@ -12,6 +13,34 @@
 
 namespace nnforge
 {
+	// A fixed set of threads that run the jobs posted to them, first posted first started
+	// (nnforge/threadpool_job_runner.h:28-52; where the reference says service.post(job), say post(job)).
+	// Backends hand the reading of input entries to it, one job per entry.
+	class threadpool_job_runner
+	{
+	public:
+		typedef std::shared_ptr<threadpool_job_runner> ptr;
+
+		explicit threadpool_job_runner(unsigned int thread_count);
+		// finishes the jobs already posted, then joins the threads
+		~threadpool_job_runner();
+
+		// a job must not let an exception escape
+		void post(std::function<void()> job);
+
+		unsigned int thread_count;
+
+	private:
+		struct impl;
+		std::unique_ptr<impl> p;
+		threadpool_job_runner() = delete;
+		threadpool_job_runner(const threadpool_job_runner&) = delete;
+		threadpool_job_runner& operator =(const threadpool_job_runner&) = delete;
+	};
+
+	// processors this process may run on (its affinity mask; never less than 1)
+	unsigned int get_available_processor_count();
+
 	// Source of input entries (nnforge/structured_data_bunch_reader.h:27-58).
 	class structured_data_bunch_reader
 	{

@@ -57,6 +57,8 @@ typedef struct nnf_backend_options
 	                                  value by value on the host, as the reference does, instead of reducing on the device */
 	int32_t kernel_stream_count;   /* hip_kernel_stream_count; 1 = hip_single_command_stream; <= 0: default */
 	int32_t one_launch_per_group;  /* 1: hip_batch_independent_groups off (every fused group gets a launch of its own) */
+	int32_t host_thread_count;     /* threads that read input entries (sets hip_reserved_thread_count to the processors beyond
+	                                  them; at most 16 are used); <= 0: default, all processors but one */
 } nnf_backend_options;
 
 /* Runs the schema on device 0. The report lists one line per launch ("step: ..."), the buffer plan

@@ -32,7 +32,7 @@ class Options(ctypes.Structure):
     _fields_ = [("fuse", ctypes.c_int32), ("dont_share_buffers", ctypes.c_int32), ("max_entry_count", ctypes.c_int32),
                 ("profile", ctypes.c_int32), ("weights_from_folder", ctypes.c_int32), ("weights_folder", ctypes.c_char_p),
                 ("profile_folder", ctypes.c_char_p), ("stat_on_host", ctypes.c_int32), ("kernel_stream_count", ctypes.c_int32),
-                ("one_launch_per_group", ctypes.c_int32)]
+                ("one_launch_per_group", ctypes.c_int32), ("host_thread_count", ctypes.c_int32)]
 
 
 class DatasetFile(ctypes.Structure):
@@ -86,7 +86,7 @@ def load():
 
 
 def _options(fuse=True, dont_share_buffers=False, max_entry_count=0, profile=False, weights_folder=None,
-             profile_folder=None, stat_on_host=False, kernel_stream_count=0, one_launch_per_group=False):
+             profile_folder=None, stat_on_host=False, kernel_stream_count=0, one_launch_per_group=False, host_thread_count=0):
     o = Options()
     o.fuse = int(fuse)
     o.dont_share_buffers = int(dont_share_buffers)
@@ -98,6 +98,7 @@ def _options(fuse=True, dont_share_buffers=False, max_entry_count=0, profile=Fal
     o.stat_on_host = int(stat_on_host)
     o.kernel_stream_count = int(kernel_stream_count)
     o.one_launch_per_group = int(one_launch_per_group)
+    o.host_thread_count = int(host_thread_count)
     return o
 
 

@@ -71,6 +71,8 @@ namespace
 			if (options->kernel_stream_count > 0)
 				generator.hip_kernel_stream_count = options->kernel_stream_count;
 			generator.hip_batch_independent_groups = options->one_launch_per_group == 0;
+			if (options->host_thread_count > 0)
+				generator.hip_reserved_thread_count = std::max(0, static_cast<int>(get_available_processor_count()) - options->host_thread_count);
 		}
 		generator.initialize();
 	}
@@ -98,6 +100,43 @@ namespace
 		void write(unsigned int entry_id, const std::map<std::string, const float *>& data_map) override { target.write(entry_id, data_map); }
 	private:
 		structured_data_bunch_writer& target;
+	};
+
+	// every entry goes straight to its place in the caller's arrays
+	class caller_arrays_writer : public structured_data_bunch_writer
+	{
+	public:
+		caller_arrays_writer(nnf_backend_output * outputs, uint32_t output_count) : entries_written(output_count, 0)
+		{
+			for(uint32_t i = 0; i < output_count; ++i)
+				by_name[outputs[i].layer_name] = std::make_pair(i, &outputs[i]);
+		}
+		void set_config_map(const std::map<std::string, layer_configuration_specific> config_map) override { this->config_map = config_map; }
+		void write(unsigned int entry_id, const std::map<std::string, const float *>& data_map) override
+		{
+			for(const std::pair<const std::string, const float *>& src : data_map)
+			{
+				const std::pair<uint32_t, nnf_backend_output *>& dst = by_name.at(src.first);
+				const size_t neuron_count = config_map.at(src.first).get_neuron_count();
+				if ((static_cast<size_t>(entry_id) + 1) * neuron_count > dst.second->capacity_floats)
+					throw neural_network_exception("Output buffer for layer " + src.first + " is too small: " + std::to_string(dst.second->capacity_floats) + " floats, "
+						+ std::to_string((static_cast<size_t>(entry_id) + 1) * neuron_count) + " needed");
+				std::memcpy(dst.second->data + static_cast<size_t>(entry_id) * neuron_count, src.second, neuron_count * sizeof(float));
+				entries_written[dst.first] = std::max(entries_written[dst.first], entry_id + 1);
+			}
+		}
+		size_t written_floats(uint32_t output_index) const
+		{
+			for(const std::pair<const std::string, std::pair<uint32_t, nnf_backend_output *> >& o : by_name)
+				if (o.second.first == output_index)
+					return static_cast<size_t>(entries_written[output_index]) * (config_map.count(o.first) ? config_map.at(o.first).get_neuron_count() : 0);
+			return 0;
+		}
+		std::map<std::string, layer_configuration_specific> config_map;
+
+	private:
+		std::map<std::string, std::pair<uint32_t, nnf_backend_output *> > by_name;
+		std::vector<unsigned int> entries_written;
 	};
 
 	template<class F> int guarded(F f, char * report, size_t report_capacity)
@@ -165,17 +204,12 @@ extern "C"
 			const std::map<std::string, layer_configuration_specific> configs = input_configs(inputs, input_count);
 			for(uint32_t i = 0; i < input_count; ++i)
 				reader.add(inputs[i].layer_name, configs.find(inputs[i].layer_name)->second, inputs[i].data);
-			memory_data_bunch_writer writer;
+			caller_arrays_writer writer(outputs, output_count);
 			const forward_propagation::stat st = fp->run(reader, writer);
 
 			for(uint32_t i = 0; i < output_count; ++i)
 			{
-				const std::vector<float>& v = writer.values[outputs[i].layer_name];
-				if (v.size() > outputs[i].capacity_floats)
-					throw neural_network_exception("Output buffer for layer " + std::string(outputs[i].layer_name) + " is too small: " + std::to_string(outputs[i].capacity_floats) + " floats, " + std::to_string(v.size()) + " needed");
-				if (!v.empty())
-					std::memcpy(outputs[i].data, v.data(), v.size() * sizeof(float));
-				outputs[i].written_floats = v.size();
+				outputs[i].written_floats = writer.written_floats(i);
 				out << "output: " << outputs[i].layer_name << " " << writer.config_map[outputs[i].layer_name] << "\n";
 			}
 

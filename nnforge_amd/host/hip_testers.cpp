@@ -39,7 +39,7 @@ namespace nnforge
 		constexpr int hip_running_configuration::default_kernel_stream_count;
 
 		hip_running_configuration::hip_running_configuration(int device_id, float max_global_memory_usage_ratio, bool fuse_layers, bool dont_share_buffers, int max_entry_count,
-			int kernel_stream_count, bool batch_independent_groups)
+			int kernel_stream_count, bool batch_independent_groups, unsigned int reserved_thread_count)
 			: device_id(device_id)
 			, max_global_memory_usage_ratio(max_global_memory_usage_ratio)
 			, fuse_layers(fuse_layers)
@@ -47,6 +47,7 @@ namespace nnforge
 			, max_entry_count(max_entry_count)
 			, kernel_stream_count(kernel_stream_count)
 			, batch_independent_groups(batch_independent_groups)
+			, reserved_thread_count(reserved_thread_count)
 			, global_memory_size(0)
 			, compute_unit_count(0)
 			, wavefront_size(0)
@@ -63,6 +64,8 @@ namespace nnforge
 			hip_safe_call(nnf_hip_device_info(device_id, name, sizeof(name), &mem, &compute_unit_count, &wavefront_size, &clock_khz));
 			device_name = name;
 			global_memory_size = mem;
+			const unsigned int processors = get_available_processor_count();
+			job_runner.reset(new threadpool_job_runner(std::min(max_job_thread_count, (processors > reserved_thread_count) ? processors - reserved_thread_count : 1U)));
 		}
 
 		hip_running_configuration::const_ptr hip_running_configuration::create_offline(
@@ -72,6 +75,7 @@ namespace nnforge
 			std::shared_ptr<hip_running_configuration> res(new hip_running_configuration());
 			res->kernel_stream_count = kernel_stream_count;
 			res->batch_independent_groups = batch_independent_groups;
+			res->reserved_thread_count = 1;
 			res->device_id = -1;
 			res->max_global_memory_usage_ratio = max_global_memory_usage_ratio;
 			res->fuse_layers = fuse_layers;
@@ -107,6 +111,8 @@ namespace nnforge
 			out << "Memory usage ratio = " << config.max_global_memory_usage_ratio << ", fuse element-wise layers = " << (config.fuse_layers ? "yes" : "no")
 				<< ", independent groups launched together = " << (config.batch_independent_groups ? "yes" : "no")
 				<< ", kernel streams = " << config.kernel_stream_count << std::endl;
+			if (config.get_job_runner())
+				out << "Job runner thread count = " << config.get_job_runner()->thread_count << std::endl;
 			return out;
 		}
 

@@ -6,10 +6,83 @@
 #include <chrono>
 #include <cstdio>
 #include <cstring>
+#include <condition_variable>
+#include <deque>
 #include <fstream>
+#include <mutex>
+#include <thread>
+
+#include <sched.h>
 
 namespace nnforge
 {
+	struct threadpool_job_runner::impl
+	{
+		std::mutex m;
+		std::condition_variable wake;
+		std::deque<std::function<void()> > jobs;
+		bool stopping = false;
+		std::vector<std::thread> threads;
+
+		void work()
+		{
+			for(;;)
+			{
+				std::function<void()> job;
+				{
+					std::unique_lock<std::mutex> lock(m);
+					wake.wait(lock, [this]() { return stopping || !jobs.empty(); });
+					if (jobs.empty())
+						return; // stopping and nothing left
+					job = std::move(jobs.front());
+					jobs.pop_front();
+				}
+				job();
+			}
+		}
+	};
+
+	threadpool_job_runner::threadpool_job_runner(unsigned int thread_count)
+		: thread_count(std::max(1U, thread_count))
+		, p(new impl())
+	{
+		for(unsigned int i = 0; i < this->thread_count; ++i)
+			p->threads.emplace_back(&impl::work, p.get());
+	}
+
+	threadpool_job_runner::~threadpool_job_runner()
+	{
+		{
+			std::lock_guard<std::mutex> lock(p->m);
+			p->stopping = true;
+		}
+		p->wake.notify_all();
+		for(std::thread& t : p->threads)
+			t.join();
+	}
+
+	void threadpool_job_runner::post(std::function<void()> job)
+	{
+		{
+			std::lock_guard<std::mutex> lock(p->m);
+			p->jobs.push_back(std::move(job));
+		}
+		p->wake.notify_one();
+	}
+
+	unsigned int get_available_processor_count()
+	{
+		cpu_set_t set;
+		CPU_ZERO(&set);
+		if (sched_getaffinity(0, sizeof(set), &set) == 0)
+		{
+			const int allowed = CPU_COUNT(&set);
+			if (allowed > 0)
+				return static_cast<unsigned int>(allowed);
+		}
+		return std::max(1U, std::thread::hardware_concurrency());
+	}
+
 	// ---- in-memory reader / writer ---------------------------------------------------------
 
 	void memory_data_bunch_reader::add(const std::string& layer_name, const layer_configuration_specific& config, const float * data_ptr)

@@ -3,7 +3,9 @@
 // program together with the backend's sources under AddressSanitizer and UndefinedBehaviorSanitizer:
 // it feeds the reader well-formed and damaged text and must end with "ok" and no sanitizer report.
 #include <nnforge_hip_backend.h>
+#include <nnforge_hip/propagation.h>
 
+#include <atomic>
 #include <cstdio>
 #include <cstring>
 #include <string>
@@ -109,6 +111,26 @@ int main(int argc, char ** argv)
 		(plan(doubled, 28, 28, report) == 0) ? ++accepted : ++refused;
 	}
 	expect(refused > accepted, "most damaged texts are refused (" + std::to_string(refused) + " refused, " + std::to_string(accepted) + " still well-formed)");
+
+	// the job runner: every job posted runs exactly once, on one of its threads, also those still queued when it goes
+	{
+		constexpr int job_count = 5000;
+		std::vector<int> ran(job_count, 0);
+		std::atomic<int> total(0);
+		{
+			nnforge::threadpool_job_runner runner(4);
+			expect(runner.thread_count == 4, "thread count as asked");
+			for(int i = 0; i < job_count; ++i)
+				runner.post([&ran, &total, i]() { ++ran[i]; total.fetch_add(1); });
+		}
+		bool once_each = true;
+		for(int r : ran)
+			once_each = once_each && (r == 1);
+		expect(once_each && (total.load() == job_count), "every posted job ran exactly once before the runner was gone");
+		nnforge::threadpool_job_runner at_least_one(0);
+		expect(at_least_one.thread_count == 1, "a runner has at least one thread");
+		expect(nnforge::get_available_processor_count() >= 1, "at least one processor");
+	}
 
 	// weight files: written, read back, read with wrong expectations
 	{

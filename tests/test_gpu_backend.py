@@ -155,6 +155,23 @@ def test_many_packets_overlap_io_and_write_the_profile_report(tmp_path):
     assert abs(float(fused[7]) - 3 * c * 49 * 4 * n / float(fused[5]) * 1e-9) < 1e-3 * float(fused[7])
 
 
+@pytest.mark.parametrize("threads", [1, 3, 16])
+def test_entries_read_by_the_job_runner_threads(threads):
+    """The entries of a packet are read by the job runner's threads, one job per entry, while the packet before
+    goes to the writer: whatever the number of threads, every entry lands in its own place (41 entries in
+    packets of 6: full packets, a short last one, and reads asked beyond the last entry)."""
+    gen = T.rng(57, 0)
+    c, n = 5, 41
+    layers = S.classifier_tail(c)
+    weights = S.make_weights(layers, gen)
+    inputs = {"conv_main": T.normal(gen, (n, c, 7, 7), 4.0), "conv_shortcut": T.normal(gen, (n, c, 7, 7), 4.0)}
+    values = S.evaluate(layers, weights, inputs)
+    got, rep = run(layers, weights, inputs, ["pool", "res_relu"], values, max_entry_count=6, host_thread_count=threads)
+    assert rep["entries"] == n
+    assert_bits(got["res_relu"], values["res_relu"], "block output with %d reading threads" % threads)
+    assert_bits(got["pool"], values["pool"], "pool with %d reading threads" % threads)
+
+
 def test_layer_in_place_on_a_data_layer_with_packets():
     """The only layer writes where the data layer was uploaded: the next upload into that slot has to
     wait for the download of the result."""
