@@ -253,6 +253,21 @@ NNF_HIP_API int nnf_hip_max_subsampling_fusable(uint32_t output_entry_count, uin
 NNF_HIP_API int nnf_hip_average_subsampling_fusable(uint32_t entry_count, uint32_t feature_map_count, uint32_t input_width, uint32_t input_height,
 	uint32_t window_width, uint32_t window_height);
 
+/* The same for a group of two inputs joined by an Add (input_count 2, has_add 1: each input's own layers,
+ * the sum times add_alpha as in nnforge/plain/add_layer_tester_plain.cpp:56-59, the tail layers) in front of
+ * an average over whole planes - the last block of a residual network in front of its global average
+ * (examples/imagenet/imagenet_toolset.cpp:518-522, 815-826): inputs[0] and inputs[1] have the shape of the
+ * subsampling input, neither the sum nor the group's result is ever stored, and the output carries the bits
+ * of the layers run one after another. NNF_HIP_EUNSUPPORTED for windows smaller than the plane, planes of
+ * fewer than 4 or more than 240 floats and groups with more than two layers that carry weights;
+ * nnf_hip_average_subsampling_joinable answers that from the shapes alone. */
+NNF_HIP_API int nnf_hip_average_subsampling_joined_forward(void* stream, float* output, const float* const* inputs,
+	const nnf_hip_chain_desc* prologue, const float* const* chunk_ptrs,
+	uint32_t entry_count, uint32_t feature_map_count, uint32_t input_width, uint32_t input_height,
+	uint32_t window_width, uint32_t window_height, float mult);
+NNF_HIP_API int nnf_hip_average_subsampling_joinable(uint32_t entry_count, uint32_t feature_map_count, uint32_t input_width, uint32_t input_height,
+	uint32_t window_width, uint32_t window_height);
+
 /* Per-feature-map running statistics on the device: the state stat_data_bunch_writer keeps per
  * feature map (nnforge/stat_data_bunch_writer.h:45-63) and fills on the host from outputs copied
  * back (nnforge/stat_data_bunch_writer.cpp:45-79). average = (float)mean and

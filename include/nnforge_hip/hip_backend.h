@@ -164,14 +164,15 @@ namespace nnforge
 
 			// Subsampling testers can apply the element-wise layers in front of them to the values they
 			// read, so that the result of those layers is never stored. can_apply_prologue: whether this
-			// tester's shapes allow it. enqueue_forward_propagation_with_prologue: the forward pass over
-			// input_buffer with the layers of prologue (a single-input group without Add whose shape is
-			// this tester's input; its weights in chunk_ptrs) applied first.
-			virtual bool can_apply_prologue() const { return false; }
+			// tester's shapes allow it for a group of prologue_input_count inputs (1: a chain of layers; 2: two
+			// chains joined by an Add, with layers behind it). enqueue_forward_propagation_with_prologue: the
+			// forward pass with the layers of prologue (whose shape is this tester's input; its inputs in
+			// input_buffers, its weights in chunk_ptrs) applied first.
+			virtual bool can_apply_prologue(unsigned int prologue_input_count) const { return false; }
 			virtual void enqueue_forward_propagation_with_prologue(
 				void * stream_id,
 				hip_linear_buffer_device::ptr output_buffer,
-				hip_linear_buffer_device::const_ptr input_buffer,
+				const std::vector<hip_linear_buffer_device::const_ptr>& input_buffers,
 				const nnf_hip_chain_desc& prologue,
 				const float * const * chunk_ptrs,
 				unsigned int entry_count);

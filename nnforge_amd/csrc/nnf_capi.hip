@@ -359,7 +359,22 @@ extern "C"
 			return NNF_HIP_EINVAL;
 		if (const int rc = prologue_status(*prologue, chunk_ptrs))
 			return rc;
-		return average_subsampling_forward_with_prologue(static_cast<hipStream_t>(stream), output, input, entry_count, feature_map_count,
+		return average_subsampling_forward_with_prologue(static_cast<hipStream_t>(stream), output, input, nullptr, entry_count, feature_map_count,
+			input_width, input_height, window_width, window_height, mult, prologue, chunk_ptrs, false);
+	}
+
+	int nnf_hip_average_subsampling_joined_forward(void* stream, float* output, const float* const* inputs,
+		const nnf_hip_chain_desc* prologue, const float* const* chunk_ptrs,
+		uint32_t entry_count, uint32_t feature_map_count, uint32_t input_width, uint32_t input_height,
+		uint32_t window_width, uint32_t window_height, float mult)
+	{
+		if ((prologue == nullptr) || (inputs == nullptr) || (prologue->input_count != 2) || (prologue->has_add == 0)
+			|| (prologue->feature_map_count != feature_map_count)
+			|| (static_cast<uint64_t>(input_width) * input_height != prologue->neuron_count_per_feature_map))
+			return NNF_HIP_EINVAL;
+		if (const int rc = prologue_status(*prologue, chunk_ptrs, true))
+			return rc;
+		return average_subsampling_forward_with_prologue(static_cast<hipStream_t>(stream), output, inputs[0], inputs[1], entry_count, feature_map_count,
 			input_width, input_height, window_width, window_height, mult, prologue, chunk_ptrs, false);
 	}
 
@@ -391,7 +406,18 @@ extern "C"
 		uint32_t window_width, uint32_t window_height)
 	{
 		const nnf_hip_chain_desc d = planning_prologue(feature_map_count);
-		return average_subsampling_forward_with_prologue(nullptr, nullptr, nullptr, std::max(1u, entry_count), feature_map_count, input_width, input_height,
+		return average_subsampling_forward_with_prologue(nullptr, nullptr, nullptr, nullptr, std::max(1u, entry_count), feature_map_count, input_width, input_height,
+			window_width, window_height, 1.0f, &d, nullptr, true);
+	}
+
+	int nnf_hip_average_subsampling_joinable(uint32_t entry_count, uint32_t feature_map_count, uint32_t input_width, uint32_t input_height,
+		uint32_t window_width, uint32_t window_height)
+	{
+		nnf_hip_chain_desc d = planning_prologue(feature_map_count);
+		d.input_count = 2;
+		d.has_add = 1;
+		d.add_alpha = 1.0f;
+		return average_subsampling_forward_with_prologue(nullptr, nullptr, nullptr, nullptr, std::max(1u, entry_count), feature_map_count, input_width, input_height,
 			window_width, window_height, 1.0f, &d, nullptr, true);
 	}
 

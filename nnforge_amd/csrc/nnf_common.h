@@ -106,7 +106,7 @@ namespace nnf
 		uint32_t output_entry_count, uint32_t input_feature_map_count, uint32_t dimension_count,
 		const uint32_t* input_sizes, const uint32_t* subsampling_sizes, const uint32_t* strides, const uint32_t* round_ups,
 		uint32_t feature_map_subsampling_size, uint32_t entry_subsampling_size, int32_t is_min);
-	int prologue_status(const nnf_hip_chain_desc& desc, const float* const* chunk_ptrs);
+	int prologue_status(const nnf_hip_chain_desc& desc, const float* const* chunk_ptrs, bool allow_join = false);
 	bool window2d_launch_with_prologue(hipStream_t stream, int op, float mult, float* output, const float* input, uint32_t input_total, uint32_t plane_count,
 		uint32_t in_w, uint32_t in_h, uint32_t out_w, uint32_t out_h, uint32_t win_w, uint32_t win_h, uint32_t stride_x, uint32_t stride_y,
 		const nnf_hip_chain_desc* prologue, const float* const* chunk_ptrs, uint32_t feature_map_count, bool plan_only);
@@ -122,7 +122,7 @@ namespace nnf
 		uint32_t output_entry_count, uint32_t input_feature_map_count, uint32_t dimension_count,
 		const uint32_t* input_sizes, const uint32_t* subsampling_sizes,
 		uint32_t feature_map_subsampling_size, uint32_t entry_subsampling_size, float mult);
-	int average_subsampling_forward_with_prologue(hipStream_t stream, float* output, const float* input,
+	int average_subsampling_forward_with_prologue(hipStream_t stream, float* output, const float* input, const float* input2,
 		uint32_t entry_count, uint32_t feature_map_count, uint32_t input_width, uint32_t input_height,
 		uint32_t window_width, uint32_t window_height, float mult,
 		const nnf_hip_chain_desc* prologue, const float* const* chunk_ptrs, bool plan_only);

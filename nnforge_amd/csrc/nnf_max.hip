@@ -187,9 +187,9 @@ namespace nnf
 							straddling |= 1u << k;
 					}
 					if (uniform)
-						apply_prologue<STAGE, EXP, true>(v, off, lds_coef, own_coef, pro, exp_ctx);
+						apply_prologue<STAGE, EXP, true>(v, off, lds_coef, own_coef, pro, exp_ctx, 0, pro.op_count);
 					else
-						apply_prologue<STAGE, EXP, false>(v, off, lds_coef, own_coef, pro, exp_ctx);
+						apply_prologue<STAGE, EXP, false>(v, off, lds_coef, own_coef, pro, exp_ctx, 0, pro.op_count);
 					// The floats of the second plane of a straddling float4 were given the first plane's
 					// coefficients: they are fetched again and go through the layers with their own.
 					while (__any(straddling != 0))
@@ -208,7 +208,7 @@ namespace nnf
 							w[0][e] = (mine && (e >= split) && (g < a.total_in)) ? a.in[g] : 0.0f;
 						}
 						const uint32_t off_next[1] = { p_next * (2 * pro.weighted_count) };
-						apply_prologue<1, EXP, false>(w, off_next, lds_coef, own_coef, pro, exp_ctx);
+						apply_prologue<1, EXP, false>(w, off_next, lds_coef, own_coef, pro, exp_ctx, 0, pro.op_count);
 						#pragma unroll
 						for(int k = 0; k < STAGE; ++k)
 						{
@@ -781,12 +781,12 @@ namespace nnf
 	}
 
 	// NNF_HIP_OK when desc describes layers a subsampling kernel can apply to its input: one input, no
-	// Add, 1..NNF_HIP_MAX_OPS known layers, every weight pointer they name present (NNF_HIP_EINVAL
-	// otherwise), at most two of them with weights (NNF_HIP_EUNSUPPORTED).
-	int prologue_status(const nnf_hip_chain_desc& desc, const float* const* chunk_ptrs)
+	// Add (with allow_join also: two inputs joined by an Add), 1..NNF_HIP_MAX_OPS known layers, every weight
+	// pointer they name present (NNF_HIP_EINVAL otherwise), at most two of them with weights (NNF_HIP_EUNSUPPORTED).
+	int prologue_status(const nnf_hip_chain_desc& desc, const float* const* chunk_ptrs, bool allow_join)
 	{
 		window_prologue pro = {};
-		if (!fill_prologue(pro, desc, chunk_ptrs, std::max(1u, desc.feature_map_count), std::max(1u, desc.neuron_count_per_feature_map)))
+		if (!fill_prologue(pro, desc, chunk_ptrs, std::max(1u, desc.feature_map_count), std::max(1u, desc.neuron_count_per_feature_map), allow_join))
 			return NNF_HIP_EINVAL;
 		return (pro.weighted_count > prologue_weighted_max) ? NNF_HIP_EUNSUPPORTED : NNF_HIP_OK;
 	}

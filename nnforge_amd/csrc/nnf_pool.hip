@@ -92,8 +92,9 @@ namespace nnf
 		// 64 planes) into an LDS table. A float4 may hold the end of one plane and the start of the next
 		// (planes of 49 floats): then it goes through the layers twice, once with each plane's
 		// coefficients, and every float keeps the result that is its own.
-		template<bool EXP>
-		__global__ void __launch_bounds__(pool_block_size) global_pool_prologue_kernel(float* out, const float* in, uint32_t plane_count, uint32_t plane,
+		// JOIN: the group has two inputs (in, in2: same shape) that an Add sums after each one's own layers.
+		template<bool EXP, bool JOIN>
+		__global__ void __launch_bounds__(pool_block_size) global_pool_prologue_kernel(float* out, const float* in, const float* in2, uint32_t plane_count, uint32_t plane,
 			uint32_t plane_magic, float mult, uint32_t planes_per_group, const window_prologue pro)
 		{
 			extern __shared__ __align__(16) float lds_planes[];
@@ -107,6 +108,7 @@ namespace nnf
 			const uint32_t planes_here = min(planes_per_group, plane_count - first_plane);
 			const uint32_t floats_here = planes_here * plane;
 			const float* src = in + static_cast<size_t>(first_plane) * plane;
+			const float* src2 = JOIN ? in2 + static_cast<size_t>(first_plane) * plane : nullptr;
 			const uint32_t coef_stride = 2 * pro.weighted_count;
 
 			const prologue_weights weights = load_prologue_weights(first_plane % pro.fm_count, planes_here, pro);
@@ -114,14 +116,20 @@ namespace nnf
 			constexpr int stage = 4; // a workgroup stages about 4096 floats: one round
 			for(uint32_t base = 0; base < vectors; base += stage * pool_block_size)
 			{
-				floatx4 t[stage];
+				floatx4 t[stage], t2[stage]; // t2, u: unused without JOIN
 				#pragma unroll
 				for(int k = 0; k < stage; ++k)
 				{
 					const uint32_t i = base + k * pool_block_size + threadIdx.x;
 					t[k] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+					if (JOIN)
+						t2[k] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
 					if (i < vectors)
+					{
 						t[k] = load_stream(reinterpret_cast<const floatx4*>(src) + i);
+						if (JOIN)
+							t2[k] = load_stream(reinterpret_cast<const floatx4*>(src2) + i);
+					}
 				}
 				if (base == 0)
 				{
@@ -132,7 +140,7 @@ namespace nnf
 					if (EXP)
 						exp_ctx = exp_context_from_lds(lds_exp);
 				}
-				float v[stage][4];
+				float v[stage][4], u[stage][4];
 				uint32_t first_plane_of[stage], off[stage];
 				bool straddles = false;
 				#pragma unroll
@@ -140,12 +148,16 @@ namespace nnf
 				{
 					const uint32_t i = min(base + k * pool_block_size + threadIdx.x, vectors - 1);
 					v[k][0] = t[k].x; v[k][1] = t[k].y; v[k][2] = t[k].z; v[k][3] = t[k].w;
+					if (JOIN)
+					{
+						u[k][0] = t2[k].x; u[k][1] = t2[k].y; u[k][2] = t2[k].z; u[k][3] = t2[k].w;
+					}
 					// floats_here * plane < 2^32: the multiplication by ceil(2^32 / plane) divides exactly
 					first_plane_of[k] = __umulhi(i * 4, plane_magic);
 					off[k] = first_plane_of[k] * coef_stride;
 					straddles = straddles || (i * 4 + 3 >= (first_plane_of[k] + 1) * plane);
 				}
-				apply_prologue<stage, EXP, false>(v, off, lds_coef, none, pro, exp_ctx);
+				apply_prologue_group<stage, EXP, JOIN>(v, u, off, lds_coef, none, pro, exp_ctx);
 				if (__any(straddles))
 				{
 					// one float4 at a time: the copies that go through the layers a second time stay few
@@ -154,8 +166,13 @@ namespace nnf
 					{
 						const uint32_t i = min(base + k * pool_block_size + threadIdx.x, vectors - 1);
 						float w[1][4] = { { t[k].x, t[k].y, t[k].z, t[k].w } };
+						float w2[1][4] = { { 0.0f, 0.0f, 0.0f, 0.0f } };
+						if (JOIN)
+						{
+							w2[0][0] = t2[k].x; w2[0][1] = t2[k].y; w2[0][2] = t2[k].z; w2[0][3] = t2[k].w;
+						}
 						const uint32_t next_off[1] = { min(first_plane_of[k] + 1, planes_here - 1) * coef_stride }; // beyond the last plane: not stored
-						apply_prologue<1, EXP, false>(w, next_off, lds_coef, none, pro, exp_ctx);
+						apply_prologue_group<1, EXP, JOIN>(w, w2, next_off, lds_coef, none, pro, exp_ctx);
 						#pragma unroll
 						for(uint32_t e = 1; e < 4; ++e)
 						{
@@ -190,8 +207,9 @@ namespace nnf
 			{
 				const uint32_t p = f / plane;
 				float one[1][4] = { { src[f], 0.0f, 0.0f, 0.0f } };
+				float one2[1][4] = { { JOIN ? src2[f] : 0.0f, 0.0f, 0.0f, 0.0f } };
 				const uint32_t one_off[1] = { p * coef_stride };
-				apply_prologue<1, EXP, false>(one, one_off, lds_coef, none, pro, exp_ctx);
+				apply_prologue_group<1, EXP, JOIN>(one, one2, one_off, lds_coef, none, pro, exp_ctx);
 				lds_planes[p * stride + (f - p * plane)] = one[0][0];
 			}
 			__syncthreads();
@@ -241,25 +259,28 @@ namespace nnf
 		uint32_t entry_count, uint32_t feature_map_count, uint32_t input_width, uint32_t input_height,
 		uint32_t window_width, uint32_t window_height, float mult)
 	{
-		return average_subsampling_forward_with_prologue(stream, output, input, entry_count, feature_map_count, input_width, input_height,
+		return average_subsampling_forward_with_prologue(stream, output, input, nullptr, entry_count, feature_map_count, input_width, input_height,
 			window_width, window_height, mult, nullptr, nullptr, false);
 	}
 
-	// prologue != null: the layers of that group are applied to the input first (LDS-staged window kernel
-	// only: NNF_HIP_EUNSUPPORTED for whole-plane windows and other shapes it does not take). plan_only:
-	// nothing is launched and no pointer is looked at; NNF_HIP_OK means the call would run.
-	int average_subsampling_forward_with_prologue(hipStream_t stream, float* output, const float* input,
+	// prologue != null: the layers of that group are applied to the input first (the LDS-staged kernels only:
+	// whole-plane averages and 2-D windows; NNF_HIP_EUNSUPPORTED for shapes they do not take). A group of two
+	// inputs joined by an Add (input2: its second input, same shape as input) goes with whole-plane averages
+	// only. plan_only: nothing is launched and no pointer is looked at; NNF_HIP_OK means the call would run.
+	int average_subsampling_forward_with_prologue(hipStream_t stream, float* output, const float* input, const float* input2,
 		uint32_t entry_count, uint32_t feature_map_count, uint32_t input_width, uint32_t input_height,
 		uint32_t window_width, uint32_t window_height, float mult,
 		const nnf_hip_chain_desc* prologue, const float* const* chunk_ptrs, bool plan_only)
 	{
+		const bool join = (prologue != nullptr) && (prologue->input_count == 2);
 		if (plan_only)
 		{
 			// planning looks at shapes only: stand-ins that pass the pointer checks below, never dereferenced
 			output = reinterpret_cast<float*>(static_cast<uintptr_t>(16));
 			input = reinterpret_cast<const float*>(static_cast<uintptr_t>(1) << 46);
+			input2 = join ? reinterpret_cast<const float*>(static_cast<uintptr_t>(1) << 47) : nullptr;
 		}
-		if ((output == nullptr) || (input == nullptr))
+		if ((output == nullptr) || (input == nullptr) || (join != (input2 != nullptr)))
 			return NNF_HIP_EINVAL;
 		if ((feature_map_count == 0) || (input_width == 0) || (input_height == 0) || (window_width == 0) || (window_height == 0))
 			return NNF_HIP_EINVAL;
@@ -267,7 +288,7 @@ namespace nnf
 		// output size is the quotient rounded down and a leftover right/bottom margin is not read
 		if ((input_width < window_width) || (input_height < window_height))
 			return NNF_HIP_EINVAL;
-		if (!is_aligned16(output) || !is_aligned16(input))
+		if (!is_aligned16(output) || !is_aligned16(input) || !is_aligned16(input2))
 			return NNF_HIP_EALIGN;
 
 		const uint32_t output_width = input_width / window_width;
@@ -283,6 +304,9 @@ namespace nnf
 			const uintptr_t a = reinterpret_cast<uintptr_t>(output), b = reinterpret_cast<uintptr_t>(input);
 			if ((a < b + input_total * sizeof(float)) && (b < a + static_cast<uint64_t>(output_count) * sizeof(float)))
 				return NNF_HIP_EOVERLAP; // the tester cannot run in place: get_input_index_layer_can_write is -1 for it
+			const uintptr_t c = reinterpret_cast<uintptr_t>(input2);
+			if (join && (a < c + input_total * sizeof(float)) && (c < a + static_cast<uint64_t>(output_count) * sizeof(float)))
+				return NNF_HIP_EOVERLAP;
 		}
 
 		const uint32_t plane = input_width * input_height;
@@ -297,18 +321,22 @@ namespace nnf
 				if (plan_only)
 					return NNF_HIP_OK;
 				window_prologue pro = {};
-				if (!fill_prologue(pro, *prologue, chunk_ptrs, feature_map_count, plane) || (pro.weighted_count > prologue_weighted_max))
+				if (!fill_prologue(pro, *prologue, chunk_ptrs, feature_map_count, plane, true) || (pro.weighted_count > prologue_weighted_max))
 					return NNF_HIP_EUNSUPPORTED;
 				const uint32_t planes_per_group = global_pool_planes_per_group(plane);
 				const size_t lds_bytes = static_cast<size_t>(planes_per_group) * (plane | 1u) * sizeof(float);
 				const dim3 grid((plane_count + planes_per_group - 1) / planes_per_group);
 				const uint32_t plane_magic = static_cast<uint32_t>(((1ull << 32) + plane - 1) / plane);
+				auto kernel = global_pool_prologue_kernel<false, false>;
 				if (pro.need_exp)
-					hipLaunchKernelGGL(global_pool_prologue_kernel<true>, grid, dim3(pool_block_size), lds_bytes, stream, output, input, plane_count, plane, plane_magic, mult, planes_per_group, pro);
-				else
-					hipLaunchKernelGGL(global_pool_prologue_kernel<false>, grid, dim3(pool_block_size), lds_bytes, stream, output, input, plane_count, plane, plane_magic, mult, planes_per_group, pro);
+					kernel = join ? global_pool_prologue_kernel<true, true> : global_pool_prologue_kernel<true, false>;
+				else if (join)
+					kernel = global_pool_prologue_kernel<false, true>;
+				hipLaunchKernelGGL(kernel, grid, dim3(pool_block_size), lds_bytes, stream, output, input, input2, plane_count, plane, plane_magic, mult, planes_per_group, pro);
 				return launch_status();
 			}
+			if (join)
+				return NNF_HIP_EUNSUPPORTED; // the window kernels take single-input groups
 			if (!window2d_launch_with_prologue(stream, 4, mult, output, input, static_cast<uint32_t>(input_total), plane_count,
 				input_width, input_height, output_width, output_height, window_width, window_height, window_width, window_height,
 				prologue, chunk_ptrs, feature_map_count, plan_only))

@@ -1,6 +1,8 @@
 // Element-wise layers that a subsampling kernel applies to its input values on their way into LDS
 // ("prologue"): the layers of a single-input group that feeds the subsampling layer and nothing
-// else, so that the group's result is never written to memory. Same formulas, same order, one
+// else, so that the group's result is never written to memory. The whole-plane average also takes a
+// group of two inputs joined by an Add (the last block of a residual network in front of its global
+// average). Same formulas, same order, one
 // rounding per operation as the chain kernel: the staged values carry the bits the unfused layers
 // would have stored. Shared by the 2-D window kernels (nnf_max.hip) and the whole-plane average
 // kernel (nnf_pool.hip).
@@ -27,6 +29,9 @@ namespace nnf
 		struct window_prologue
 		{
 			uint32_t op_count;
+			uint32_t arm_ops[2];             // layers applied to input 0 / input 1 before the join (one input: all of them, 0)
+			uint32_t join;                   // 1: two inputs, summed by an Add after their own layers, the rest applied to the sum
+			float alpha;                     // the Add's multiplier
 			uint32_t fm_count;
 			uint32_t need_exp;
 			uint32_t in_plane_magic;         // ceil(2^32 / input plane size)
@@ -159,12 +164,13 @@ namespace nnf
 		constexpr int coef_batch = 4; // vectors whose batch norm coefficients are read from LDS together
 
 		// UNIFORM: every value belongs to the same plane, whose coefficients are in own (registers)
-		// instead of coef (LDS).
+		// instead of coef (LDS). Applies the layers first_op .. end_op - 1.
 		template<int VECTORS, bool EXP, bool UNIFORM>
 		__device__ __forceinline__ void apply_prologue(float (&v)[VECTORS][4], const uint32_t (&off)[VECTORS],
-			const float* coef, const float (&own)[prologue_weighted_max][2], const window_prologue& pro, const exp_context& exp_ctx)
+			const float* coef, const float (&own)[prologue_weighted_max][2], const window_prologue& pro, const exp_context& exp_ctx,
+			uint32_t first_op, uint32_t end_op)
 		{
-			for(uint32_t i = 0; i < pro.op_count; ++i)
+			for(uint32_t i = first_op; i < end_op; ++i)
 			{
 				const int32_t kind = pro.kind[i];
 				const uint32_t slot = pro.slot[i];
@@ -274,21 +280,58 @@ namespace nnf
 		}
 
 
+		// The whole group over the values of input 0 (v) and, with JOIN, input 1 (u): each input's own layers, the
+		// Add (nnforge/plain/add_layer_tester_plain.cpp:56-59: the sum starts at 0.0F, inputs in order, times
+		// alpha), the layers behind it. The result is left in v.
+		template<int VECTORS, bool EXP, bool JOIN>
+		__device__ __forceinline__ void apply_prologue_group(float (&v)[VECTORS][4], float (&u)[VECTORS][4], const uint32_t (&off)[VECTORS],
+			const float* coef, const float (&own)[prologue_weighted_max][2], const window_prologue& pro, const exp_context& exp_ctx)
+		{
+			if (!JOIN)
+			{
+				apply_prologue<VECTORS, EXP, false>(v, off, coef, own, pro, exp_ctx, 0, pro.op_count);
+				return;
+			}
+			const uint32_t arm0_end = pro.arm_ops[0];
+			const uint32_t arm1_end = arm0_end + pro.arm_ops[1];
+			apply_prologue<VECTORS, EXP, false>(v, off, coef, own, pro, exp_ctx, 0, arm0_end);
+			apply_prologue<VECTORS, EXP, false>(u, off, coef, own, pro, exp_ctx, arm0_end, arm1_end);
+			#pragma unroll
+			for(int k = 0; k < VECTORS; ++k)
+			{
+				#pragma unroll
+				for(int e = 0; e < 4; ++e)
+				{
+					float sum = 0.0f + v[k][e];
+					sum = sum + u[k][e];
+					v[k][e] = sum * pro.alpha;
+				}
+			}
+			apply_prologue<VECTORS, EXP, false>(v, off, coef, own, pro, exp_ctx, arm1_end, pro.op_count);
+		}
+
 		uint32_t magic_of(uint32_t divisor)
 		{
 			return (divisor >= 2) ? static_cast<uint32_t>(((1ull << 32) + divisor - 1) / divisor) : 0u; // fast_divide does not use it for 1
 		}
 
-		// The layers of a single-input group without Add, in order, as the kernel wants them. False when
-		// the description is not such a group or a weight pointer is missing.
-		bool fill_prologue(window_prologue& pro, const nnf_hip_chain_desc& desc, const float* const* chunk_ptrs, uint32_t feature_map_count, uint32_t in_plane)
+		// The layers of a single-input group without Add - or, with allow_join, of two inputs joined by an Add -
+		// in order, as the kernel wants them. False when the description is not such a group or a weight
+		// pointer is missing.
+		bool fill_prologue(window_prologue& pro, const nnf_hip_chain_desc& desc, const float* const* chunk_ptrs, uint32_t feature_map_count, uint32_t in_plane,
+			bool allow_join = false)
 		{
-			if ((desc.input_count != 1) || desc.has_add || (feature_map_count == 0))
+			const bool join = allow_join && (desc.input_count == 2) && (desc.has_add != 0);
+			if ((!join && ((desc.input_count != 1) || desc.has_add)) || (feature_map_count == 0))
 				return false;
-			const uint32_t op_count = desc.arm_op_count[0] + desc.tail_op_count;
-			if ((op_count == 0) || (op_count > NNF_HIP_MAX_OPS))
+			const uint32_t op_count = desc.arm_op_count[0] + (join ? desc.arm_op_count[1] : 0u) + desc.tail_op_count;
+			if (((op_count == 0) && !join) || (op_count > NNF_HIP_MAX_OPS))
 				return false;
 			pro.op_count = op_count;
+			pro.join = join ? 1u : 0u;
+			pro.alpha = desc.add_alpha;
+			pro.arm_ops[0] = join ? desc.arm_op_count[0] : op_count;
+			pro.arm_ops[1] = join ? desc.arm_op_count[1] : 0u;
 			pro.fm_count = feature_map_count;
 			pro.weighted_count = 0;
 			pro.need_exp = 0;

@@ -236,7 +236,7 @@ namespace nnforge
 				else if (plan.prologue)
 				{
 					plan.desc.entry_count = step_entries;
-					plan.tester->enqueue_forward_propagation_with_prologue(step_stream, buffers[plan.output_buffer], inputs.at(0), plan.desc,
+					plan.tester->enqueue_forward_propagation_with_prologue(step_stream, buffers[plan.output_buffer], inputs, plan.desc,
 						chunk_ptrs[i].empty() ? nullptr : chunk_ptrs[i].data(), step_entries);
 				}
 				else if (plan.info.fused)
@@ -443,17 +443,24 @@ namespace nnforge
 				if (!grouped)
 				{
 					// A subsampling layer takes the pending group that feeds it along: the group's layers are
-					// applied to the values on their way into the subsampling kernel's staging buffer.
-					if (hip_config->fuse_layers && (l->input_layer_instance_names.size() == 1) && p->testers[name]->can_apply_prologue())
+					// applied to the values on their way into the subsampling kernel's staging buffer. A chain of
+					// layers over one input goes with every subsampling kernel that stages its input; two chains
+					// joined by an Add (the last block of a residual network) with the average over whole planes.
+					if (hip_config->fuse_layers && (l->input_layer_instance_names.size() == 1))
 					{
 						const std::string& producer = l->input_layer_instance_names[0];
 						std::map<std::string, pending_group>::iterator it = pending.find(producer);
-						if ((it != pending.end()) && it->second.add_layer_name.empty() && (it->second.arms.size() == 1)
+						const bool chain = (it != pending.end()) && it->second.add_layer_name.empty() && (it->second.arms.size() == 1);
+						const bool joined = (it != pending.end()) && !it->second.add_layer_name.empty() && (it->second.arms.size() == 2);
+						if ((chain || joined) && p->testers[name]->can_apply_prologue(static_cast<unsigned int>(it->second.arms.size()))
 							&& (this->schema->get_consumer_count(producer) == 1) && (outputs.find(producer) == outputs.end()))
 						{
 							unsigned int weighted = 0;
-							bool only_dropout = true; // such a group costs no launch on its own
-							for(const std::string& op_layer : it->second.arms[0].ops)
+							bool only_dropout = chain; // such a group costs no launch on its own
+							std::vector<std::string> op_layers = it->second.tail;
+							for(const pending_arm& arm : it->second.arms)
+								op_layers.insert(op_layers.end(), arm.ops.begin(), arm.ops.end());
+							for(const std::string& op_layer : op_layers)
 							{
 								nnf_hip_op op;
 								weighted += (p->testers[op_layer]->get_chain_op(op) > 0) ? 1u : 0u;
@@ -497,7 +504,8 @@ namespace nnforge
 						for(const pending_arm& a : group_of[name]->arms)
 							sources.push_back(a.source);
 					else if (prologues.find(name) != prologues.end())
-						sources.push_back(prologues[name].arms[0].source);
+						for(const pending_arm& arm : prologues[name].arms)
+							sources.push_back(arm.source);
 					else
 						sources = this->schema->get_layer(name)->input_layer_instance_names;
 					unsigned int level = 0;
@@ -575,9 +583,15 @@ namespace nnforge
 				if (!so.second && (prologues.find(name) != prologues.end()))
 				{
 					const pending_group& g = prologues[name];
-					plan.info.layer_names = g.arms[0].ops;
+					for(const pending_arm& arm : g.arms)
+					{
+						plan.info.input_names.push_back(arm.source);
+						plan.info.layer_names.insert(plan.info.layer_names.end(), arm.ops.begin(), arm.ops.end());
+					}
+					if (!g.add_layer_name.empty())
+						plan.info.layer_names.push_back(g.add_layer_name);
+					plan.info.layer_names.insert(plan.info.layer_names.end(), g.tail.begin(), g.tail.end());
 					plan.info.layer_names.push_back(name);
-					plan.info.input_names.push_back(g.arms[0].source);
 					plan.info.fused = true;
 					plan.prologue = true;
 					plan.tester = p->testers[name];

@@ -178,7 +178,7 @@ namespace nnforge
 			return std::vector<hip_linear_buffer_device::const_ptr>();
 		}
 
-		void layer_tester_hip::enqueue_forward_propagation_with_prologue(void *, hip_linear_buffer_device::ptr, hip_linear_buffer_device::const_ptr,
+		void layer_tester_hip::enqueue_forward_propagation_with_prologue(void *, hip_linear_buffer_device::ptr, const std::vector<hip_linear_buffer_device::const_ptr>&,
 			const nnf_hip_chain_desc&, const float * const *, unsigned int)
 		{
 			throw neural_network_exception("Layer " + layer_schema->instance_name + " of type " + layer_schema->get_type_name() + " cannot apply other layers to its input");
@@ -505,17 +505,31 @@ namespace nnforge
 							feature_map_window, entry_window, mult));
 				}
 
-				bool can_apply_prologue() const override
+				bool can_apply_prologue(unsigned int prologue_input_count) const override
 				{
-					return plain_2d && (nnf_hip_average_subsampling_fusable(1, output_configuration_specific.feature_map_count, input_sizes[0], input_sizes[1],
+					if (!plain_2d)
+						return false;
+					if (prologue_input_count == 1)
+						return nnf_hip_average_subsampling_fusable(1, output_configuration_specific.feature_map_count, input_sizes[0], input_sizes[1],
+							windows[0], windows[1]) == NNF_HIP_OK;
+					// two inputs joined by an Add: the average over whole planes takes them
+					return (prologue_input_count == 2) && (nnf_hip_average_subsampling_joinable(1, output_configuration_specific.feature_map_count, input_sizes[0], input_sizes[1],
 						windows[0], windows[1]) == NNF_HIP_OK);
 				}
 
 				void enqueue_forward_propagation_with_prologue(void * stream_id, hip_linear_buffer_device::ptr output_buffer,
-					hip_linear_buffer_device::const_ptr input_buffer, const nnf_hip_chain_desc& prologue, const float * const * chunk_ptrs,
+					const std::vector<hip_linear_buffer_device::const_ptr>& input_buffers, const nnf_hip_chain_desc& prologue, const float * const * chunk_ptrs,
 					unsigned int entry_count) override
 				{
-					hip_safe_call(nnf_hip_average_subsampling_fused_forward(stream_id, *output_buffer, float_ptr(input_buffer), &prologue, chunk_ptrs,
+					require_inputs(input_buffers, prologue.input_count, "AverageSubsampling with layers folded in");
+					if (prologue.input_count == 1)
+					{
+						hip_safe_call(nnf_hip_average_subsampling_fused_forward(stream_id, *output_buffer, float_ptr(input_buffers[0]), &prologue, chunk_ptrs,
+							entry_count, output_configuration_specific.feature_map_count, input_sizes[0], input_sizes[1], windows[0], windows[1], mult));
+						return;
+					}
+					const float * const inputs[2] = { float_ptr(input_buffers[0]), float_ptr(input_buffers[1]) };
+					hip_safe_call(nnf_hip_average_subsampling_joined_forward(stream_id, *output_buffer, inputs, &prologue, chunk_ptrs,
 						entry_count, output_configuration_specific.feature_map_count, input_sizes[0], input_sizes[1], windows[0], windows[1], mult));
 				}
 
@@ -673,17 +687,18 @@ namespace nnforge
 						input_sizes.data(), windows.data(), strides.data(), round_ups.data(), feature_map_subsampling_size, entry_window, is_min ? 1 : 0));
 				}
 
-				bool can_apply_prologue() const override
+				bool can_apply_prologue(unsigned int prologue_input_count) const override
 				{
-					return (tile_count == 0) && (entry_window == 1) && nnf_hip_max_subsampling_fusable(1, input_configuration_specific_list[0].feature_map_count, static_cast<uint32_t>(input_sizes.size()),
+					return (prologue_input_count == 1) && (tile_count == 0) && (entry_window == 1) && nnf_hip_max_subsampling_fusable(1, input_configuration_specific_list[0].feature_map_count, static_cast<uint32_t>(input_sizes.size()),
 						input_sizes.data(), windows.data(), strides.data(), round_ups.data(), feature_map_subsampling_size, 1) == NNF_HIP_OK;
 				}
 
 				void enqueue_forward_propagation_with_prologue(void * stream_id, hip_linear_buffer_device::ptr output_buffer,
-					hip_linear_buffer_device::const_ptr input_buffer, const nnf_hip_chain_desc& prologue, const float * const * chunk_ptrs,
+					const std::vector<hip_linear_buffer_device::const_ptr>& input_buffers, const nnf_hip_chain_desc& prologue, const float * const * chunk_ptrs,
 					unsigned int entry_count) override
 				{
-					hip_safe_call(nnf_hip_max_subsampling_fused_forward(stream_id, *output_buffer, float_ptr(input_buffer), &prologue, chunk_ptrs, entry_count,
+					require_inputs(input_buffers, 1, "MaxSubsampling with layers folded in");
+					hip_safe_call(nnf_hip_max_subsampling_fused_forward(stream_id, *output_buffer, float_ptr(input_buffers[0]), &prologue, chunk_ptrs, entry_count,
 						input_configuration_specific_list[0].feature_map_count, static_cast<uint32_t>(input_sizes.size()),
 						input_sizes.data(), windows.data(), strides.data(), round_ups.data(), feature_map_subsampling_size, 1, is_min ? 1 : 0));
 				}

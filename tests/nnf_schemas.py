@@ -82,9 +82,9 @@ def resnet_block(c=8, with_shortcut_bn=True):
     return layers
 
 
-def classifier_tail(c=8):
+def classifier_tail(c=8, with_shortcut_bn=True):
     """ResNet-like tail: block -> 7x7 global pooling -> softmax."""
-    return resnet_block(c) + [L("AverageSubsampling", "pool", ["res_relu"], windows=[7, 7], alpha=1.0 / 49.0),
+    return resnet_block(c, with_shortcut_bn) + [L("AverageSubsampling", "pool", ["res_relu"], windows=[7, 7], alpha=1.0 / 49.0),
                               L("Softmax", "prob", ["pool"])]
 
 

@@ -98,8 +98,16 @@ def test_plan_fuses_the_resnet_block_into_one_launch():
 
 def test_plan_whole_tail_and_activation_chain():
     rep = plan(S.classifier_tail(8), {"conv_main": (8, [7, 7]), "conv_shortcut": (8, [7, 7])}, ["prob"])
+    # the average over whole planes takes the joined group in front of it along
+    assert step_names(rep) == ["shortcut_bn+main_bn+res+res_relu+pool", "prob"]
+    assert [s["fused"] for s in rep["steps"]] == [True, False]
+    assert rep["steps"][0]["inputs"] == ["conv_shortcut", "conv_main"]
+    # ... unless the group's result is wanted as well, or layers may not be fused
+    rep = plan(S.classifier_tail(8), {"conv_main": (8, [7, 7]), "conv_shortcut": (8, [7, 7])}, ["prob", "res_relu"])
     assert step_names(rep) == ["shortcut_bn+main_bn+res+res_relu", "pool", "prob"]
     assert [s["fused"] for s in rep["steps"]] == [True, False, False]
+    rep = plan(S.classifier_tail(8), {"conv_main": (8, [7, 7]), "conv_shortcut": (8, [7, 7])}, ["prob"], fuse=False)
+    assert step_names(rep) == ["shortcut_bn", "main_bn", "res", "res_relu", "pool", "prob"]
     rep = plan(S.activation_chain(6), {"x": (6, [5, 4])}, ["tanh"])
     assert step_names(rep) == ["bn+elu+sig+tanh"]
 
@@ -220,8 +228,9 @@ def test_plan_of_the_inception_like_block():
 def test_plan_of_the_resnet50_post_convolution_graph_equals_the_benchmark_group_list():
     """Config 4 as a network: the graph examples/imagenet/imagenet_toolset.cpp:476-550, 729-831 builds, convolution outputs as
     data layers. With one launch per group the driver's fusion pass must arrive at the 49 groups nnforge_amd.workloads lists by
-    hand (kind, shape, order), then the 7x7 average and the softmax; the residual of a block that keeps its shape is the block
-    before. By default the steps are ordered by depth in the graph and independent groups are launched together."""
+    hand (kind, shape, order), the last of them folded into the 7x7 average behind it, then the softmax; the residual of a block
+    that keeps its shape is the block before. By default the steps are ordered by depth in the graph and independent groups are
+    launched together."""
     from nnforge_amd import schemas, workloads as w
 
     layers, configs, outputs = schemas.resnet50_post_convolution()
@@ -229,7 +238,7 @@ def test_plan_of_the_resnet50_post_convolution_graph_equals_the_benchmark_group_
     rep = plan(layers, configs, outputs, one_launch_per_group=True)
     steps = rep["steps"]
     groups = w.resnet50_groups(1)
-    assert len(steps) == len(groups) + 2 == 51
+    assert len(steps) == len(groups) + 1 == 50
     by_name = {l["name"]: l for l in layers}
     shapes = dict(configs)
     for l in layers:   # every layer here keeps the shape of its first input, but for the pooling
@@ -245,24 +254,26 @@ def test_plan_of_the_resnet50_post_convolution_graph_equals_the_benchmark_group_
         return (["BatchNorm"] + want) if (len(g.arms) == 2 and g.arms[0]) else want   # first block of a stage: batch norm on the shortcut as well
 
     per_entry_bytes = 0
-    for step, g in zip(steps, groups):
+    for i, (step, g) in enumerate(zip(steps, groups)):
         assert step["fused"] and step["run"] is None
-        fm, dims = shapes[step["layers"][-1]]
+        group_layers = step["layers"] if i < 48 else step["layers"][:-1]   # the last group has the average behind it in its step
+        fm, dims = shapes[group_layers[-1]]
         assert (fm, dims[0] * dims[1]) == (g.feature_map_count, g.plane), (step, g.name)
         assert len(step["inputs"]) == len(g.arms)
-        assert [by_name[n]["type"] for n in step["layers"]] == kinds_wanted(g), (step, g.name)
+        assert [by_name[n]["type"] for n in group_layers] == kinds_wanted(g), (step, g.name)
         per_entry_bytes += w.group_algorithmic_bytes(g)
-    assert steps[49]["layers"] == ["pool5"] and steps[49]["inputs"] == ["res5c_relu"] and not steps[49]["fused"]
-    assert steps[50]["layers"] == ["prob"] and steps[50]["inputs"] == ["logits"]
+    assert steps[48]["layers"][-2:] == ["res5c_relu", "pool5"] and steps[48]["inputs"] == ["res5b_relu", "res5c_restore_fm"]
+    assert steps[49]["layers"] == ["prob"] and steps[49]["inputs"] == ["logits"] and not steps[49]["fused"]
     # the bytes the launches move per entry are the benchmark's algorithmic bytes (weights aside: 4 bytes per weight)
     weights_bytes = sum(4 * (4 if kind == "bn" else 1) * c for g in groups for kind, c in g.chunks)
     g_bytes, p_bytes, s_bytes = w.resnet50_algorithmic_bytes(1)
     assert per_entry_bytes == g_bytes
     moved = sum(floats(name) for name in configs)                                                 # every data layer read once
-    moved += sum(floats(s["layers"][-1]) for s in steps[:49])                                     # every group's output written
+    moved += sum(floats(s["layers"][-1]) for s in steps[:48])                                     # every group's output written ...
     moved += sum(floats(src) for s in steps[:49] for src in s["inputs"] if src not in configs)    # residuals read back
-    moved += 2048 * 49 + 2048 + 1000                                                              # pool5 input and output, prob output
-    assert 4 * moved == g_bytes - weights_bytes + p_bytes + s_bytes
+    moved += 2048 + 1000                                                                          # pool5 output, prob output
+    # ... but the last group's: neither written nor read back by the average, which the benchmark's algorithmic bytes count
+    assert 4 * (moved + 2 * 2048 * 49) == g_bytes - weights_bytes + p_bytes + s_bytes
     # residual chains: a block that keeps its shape reads the block before, so it shares that block's stream (no step
     # ever waits for another stream); steps that have nothing to do with each other take the three streams in turn
     producer = {s["layers"][-1]: i for i, s in enumerate(steps)}
@@ -272,7 +283,7 @@ def test_plan_of_the_resnet50_post_convolution_graph_equals_the_benchmark_group_
             if source in producer:
                 assert producer[source] < i and steps[producer[source]]["stream"] == s["stream"], (i, s)
                 chained += 1
-    assert chained == 12 + 1   # 16 blocks minus the 4 with a shortcut convolution, and pool5 behind res5c_relu
+    assert chained == 12   # 16 blocks minus the 4 with a shortcut convolution
     assert [s["stream"] for s in steps[:6]] == [0, 1, 2, 0, 1, 2] and len({s["stream"] for s in steps}) == 3
     # one kernel stream: the same steps
     single = plan(layers, configs, outputs, one_launch_per_group=True, kernel_stream_count=1)
@@ -292,11 +303,12 @@ def test_plan_of_the_resnet50_post_convolution_graph_equals_the_benchmark_group_
     runs = [s["run"] for s in batched]
     assert runs[:37] == [0] * 37 and batched[37]["layers"] == ["prob"] and runs[37] is None   # 1 + 16 + 16 + 4 groups, then the softmax
     assert [batched[i]["layers"][-1] for i in range(38, 42)] == ["res2b_relu", "res3b_relu", "res4b_relu", "res5b_relu"] and runs[38:42] == [1] * 4
-    assert runs[42:46] == [2] * 4 and runs[46:48] == [3] * 2 and batched[48]["layers"] == ["pool5"] and runs[48:] == [None, 4, 5]
+    # the last block's group goes with the average: a launch of its own among the groups of its level
+    assert runs[42:45] == [2] * 3 and batched[45]["layers"][-1] == "pool5" and runs[45] is None and runs[46:] == [3, 3, 4, 5]
     # with the stem's pooling in the graph, batch norm and ReLU are applied on the way into the pooling kernel
     layers, configs, outputs = schemas.resnet50_post_convolution(with_pool1=True)
     rep = plan(layers, configs, outputs)
-    assert len(rep["steps"]) == 51 and rep["steps"][0]["layers"] == ["conv1_bn", "relu1", "pool1"] and rep["steps"][0]["fused"]
+    assert len(rep["steps"]) == 50 and rep["steps"][0]["layers"] == ["conv1_bn", "relu1", "pool1"] and rep["steps"][0]["fused"]
     assert rep["steps"][0]["run"] is None and rep["steps"][1]["run"] == 0   # the pooling step is no fused group: it launches alone
 
 

@@ -155,6 +155,29 @@ def test_many_packets_overlap_io_and_write_the_profile_report(tmp_path):
     assert abs(float(fused[7]) - 3 * c * 49 * 4 * n / float(fused[5]) * 1e-9) < 1e-3 * float(fused[7])
 
 
+@pytest.mark.parametrize("shortcut_bn", [True, False])
+def test_last_block_of_a_residual_network_folded_into_its_global_average(shortcut_bn):
+    """BatchNorm(main) [+ BatchNorm(shortcut)] -> Add -> ReLU -> 7x7 average with only the average (and what follows it)
+    wanted: the average's kernel applies the joined group to the two tensors on their way in - one launch, the group's
+    result never stored - and the outputs carry the bits of the layers run one by one."""
+    gen = T.rng(58, int(shortcut_bn))
+    c, n = 40, 11
+    layers = S.classifier_tail(c, with_shortcut_bn=shortcut_bn)
+    weights = S.make_weights(layers, gen)
+    inputs = {"conv_main": T.normal(gen, (n, c, 7, 7), 4.0), "conv_shortcut": T.normal(gen, (n, c, 7, 7), 4.0)}
+    values = S.evaluate(layers, weights, inputs)
+    got, rep = run(layers, weights, inputs, ["prob", "pool"], values, max_entry_count=4)
+    names = ["+".join(s["layers"]) for s in rep["steps"]]
+    assert len(names) == 2 and names[0].endswith("+res+res_relu+pool") and names[1] == "prob", names
+    assert len(rep["steps"][0]["inputs"]) == 2 and rep["steps"][0]["fused"]
+    assert_bits(got["pool"], values["pool"], "average over the folded block")
+    assert (np.abs(got["prob"] - values["prob"]) / values["prob"]).max() < 1e-5
+    # without fusion: the same bits from six launches
+    plain, rep = run(layers, weights, inputs, ["prob", "pool"], values, max_entry_count=4, fuse=False)
+    assert len(rep["steps"]) == (6 if shortcut_bn else 5)
+    assert_bits(plain["pool"], got["pool"], "fused against unfused")
+
+
 @pytest.mark.parametrize("threads", [1, 3, 16])
 def test_entries_read_by_the_job_runner_threads(threads):
     """The entries of a packet are read by the job runner's threads, one job per entry, while the packet before
@@ -353,9 +376,10 @@ def test_inference_from_data_set_files_to_data_set_files(tmp_path):
 
 @pytest.mark.parametrize("mode", ["together", "streams", "plain"])
 def test_resnet50_post_convolution_graph_layer_by_layer(mode):
-    """Config 4 through the driver at a small entry count: every output of the 51 steps against the oracle run layer by
-    layer (bit for bit; softmax to 1e-5) - with independent groups launched together (the default), with one launch per
-    group spread over three kernel streams, and with one launch per group on one stream."""
+    """Config 4 through the driver at a small entry count: every output of the 50 steps (48 groups, the last block's group
+    with the 7x7 average behind it, the softmax) against the oracle run layer by layer (bit for bit; softmax to 1e-5) - with
+    independent groups launched together (the default), with one launch per group spread over three kernel streams, and
+    with one launch per group on one stream."""
     from nnforge_amd import schemas
 
     gen = T.rng(62, 0)
@@ -367,7 +391,8 @@ def test_resnet50_post_convolution_graph_layer_by_layer(mode):
     values = S.evaluate(layers, weights, inputs)
     options = {"together": {}, "streams": {"one_launch_per_group": True}, "plain": {"one_launch_per_group": True, "kernel_stream_count": 1}}[mode]
     got, rep = run(layers, weights, inputs, outputs, values, max_entry_count=2, **options)
-    assert len(rep["steps"]) == 51 and rep["entries"] == n
+    assert len(rep["steps"]) == 50 and rep["entries"] == n
+    assert [s["layers"][-2:] for s in rep["steps"] if s["layers"][-1] == "pool5"] == [["res5c_relu", "pool5"]]
     assert len({s["stream"] for s in rep["steps"]}) == (3 if mode == "streams" else 1)
     assert len({s["run"] for s in rep["steps"]} - {None}) == (6 if mode == "together" else 0)
     for name in outputs:

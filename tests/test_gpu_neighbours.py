@@ -402,6 +402,90 @@ def test_average_subsampling_with_group_folded_in(gpu, shape, ww, wh, group):
     assert T.bit_mismatches(got, want) == 0
 
 
+JOINED_POOL_CASES = [
+    # shape, arms ("bn": BatchNorm, "-": nothing, "leaky": ReLU 0.1, "elu"), alpha, tail
+    ((64, 128, 7, 7), ("-", "bn"), 1.0, "relu"),        # residual + BatchNorm(main) -> Add -> ReLU: the last block of a ResNet
+    ((5, 24, 7, 7), ("bn", "bn"), 1.0, "relu"),         # BatchNorm on both arms (a block with a projection shortcut)
+    ((3, 5, 7, 7), ("bn", "elu"), 0.5, "sigmoid"),      # 15 planes in the last workgroup, three floats behind the last float4
+    ((9, 70, 8, 8), ("leaky", "-"), 2.0, "none"),       # planes that are multiples of 4 floats, nothing behind the Add
+    ((2, 7, 15, 15), ("bn", "-"), 1.0, "prelu"),        # 225 floats per plane, weights on an arm and behind the join
+    ((1, 1, 2, 2), ("-", "-"), 1.0, "relu"),
+]
+
+
+def joined_arm(kind, gen, c, chunks):
+    """-> (ops, oracle function) of one arm; weight chunks are appended to chunks"""
+    if kind == "bn":
+        g, b, m, s = T.bn_params(gen, c)
+        first = len(chunks)
+        chunks += [g, b, m, s]
+        return [(capi.OP_BATCH_NORM, first)], lambda v: oracle.batch_norm(v, g, b, m, s)
+    if kind == "leaky":
+        return [(capi.OP_RELU, 0, 0.1)], lambda v: oracle.rectified_linear(v, 0.1)
+    if kind == "elu":
+        return [(capi.OP_ELU,)], oracle.exponential_linear
+    return [], lambda v: v
+
+
+@pytest.mark.parametrize("shape,arms,alpha,tail", JOINED_POOL_CASES)
+def test_whole_plane_average_with_a_joined_group_folded_in(gpu, shape, arms, alpha, tail):
+    """Two inputs, each with its own layers, an Add, the layers behind it and the average over whole planes in one
+    launch: the bits of the layers run one after another by the oracle."""
+    gen = T.rng(69, sum(shape) + len(tail))
+    n, c, h, w = shape
+    chunks = []
+    arm_ops, arm_fns = zip(*[joined_arm(kind, gen, c, chunks) for kind in arms])
+    if tail == "relu":
+        tail_ops, tail_fn = [(capi.OP_RELU, 0, 0.0)], lambda v: oracle.rectified_linear(v, 0.0)
+    elif tail == "sigmoid":
+        tail_ops, tail_fn = [(capi.OP_SIGMOID,)], oracle.sigmoid
+    elif tail == "prelu":
+        a = T.uniform(gen, c, -0.5, 0.5)
+        tail_ops, tail_fn = [(capi.OP_PRELU, len(chunks))], lambda v: oracle.parametric_rectified_linear(v, a)
+        chunks.append(a)
+    else:
+        tail_ops, tail_fn = [], lambda v: v
+    xs = [prologue_input(gen, shape) if i == 0 else T.normal(gen, shape, 2.0) for i in range(2)]
+    joined = tail_fn(oracle.add([fn(x) for fn, x in zip(arm_fns, xs)], alpha))
+    mult = oracle.average_subsampling_full_mult([w, h])
+    want = oracle.average_subsampling(joined, [w, h], mult=mult)
+
+    desc = capi.make_desc(n, c, h * w, [list(ops) for ops in arm_ops], tail_ops, add_alpha=alpha)
+    d_ins = [gpu.to_device(x) for x in xs]
+    d_chunks = [gpu.to_device(a) for a in chunks]
+    chk = capi.pointer_array([t.data_ptr() for t in d_chunks])
+    ins = capi.pointer_array([t.data_ptr() for t in d_ins])
+    d_out = gpu.torch.full((n * c,), float("nan"), dtype=gpu.torch.float32, device=gpu.device)
+    assert gpu.lib.nnf_hip_average_subsampling_joinable(n, c, w, h, w, h) == 0
+    rc = gpu.lib.nnf_hip_average_subsampling_joined_forward(gpu.stream, d_out.data_ptr(), ins, ctypes.byref(desc), chk if d_chunks else None,
+                                                            n, c, w, h, w, h, mult)
+    assert rc == 0, capi.error_string(rc)
+    got = gpu.to_host(d_out, want.shape)
+    assert T.bit_mismatches(got, want) == 0
+
+
+def test_joined_groups_the_average_cannot_take_are_refused(gpu):
+    gen = T.rng(70, 0)
+    n, c, h, w = 2, 6, 8, 8
+    d_ins = [gpu.to_device(T.normal(gen, (n, c, h, w))) for _ in range(2)]
+    ins = capi.pointer_array([t.data_ptr() for t in d_ins])
+    d_out = gpu.torch.zeros(n * c * 16, dtype=gpu.torch.float32, device=gpu.device)
+    desc = capi.make_desc(n, c, h * w, [[], []], [(capi.OP_RELU, 0, 0.0)])
+    call = gpu.lib.nnf_hip_average_subsampling_joined_forward
+    # windows smaller than the plane
+    assert gpu.lib.nnf_hip_average_subsampling_joinable(n, c, w, h, 2, 2) == capi.E_UNSUPPORTED
+    assert call(gpu.stream, d_out.data_ptr(), ins, ctypes.byref(desc), None, n, c, w, h, 2, 2, 0.25) == capi.E_UNSUPPORTED
+    # a single-input description, a missing second input, a shape that is not the description's
+    single = capi.make_desc(n, c, h * w, [[(capi.OP_RELU, 0, 0.0)]], [])
+    assert call(gpu.stream, d_out.data_ptr(), ins, ctypes.byref(single), None, n, c, w, h, w, h, 1.0) == capi.E_INVAL
+    one = capi.pointer_array([d_ins[0].data_ptr(), 0])
+    assert call(gpu.stream, d_out.data_ptr(), one, ctypes.byref(desc), None, n, c, w, h, w, h, 1.0) == capi.E_INVAL
+    assert call(gpu.stream, d_out.data_ptr(), ins, ctypes.byref(desc), None, n, c + 1, w, h, w, h, 1.0) == capi.E_INVAL
+    # the output may not lie inside an input
+    assert call(gpu.stream, d_ins[1].data_ptr(), ins, ctypes.byref(desc), None, n, c, w, h, w, h, 1.0) == capi.E_OVERLAP
+    gpu.torch.cuda.synchronize()
+
+
 @pytest.mark.parametrize("shape", [(4, 16, 128, 128), (64, 256, 8, 8)])
 def test_exp_layers_folded_into_subsampling_over_a_sweep_of_all_exponents(gpu, shape):
     """ELU, Sigmoid and TanH inside the subsampling kernels (their own expf batches and range repair) on a regular
