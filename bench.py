@@ -43,8 +43,9 @@ MEASURED_TRAFFIC_BYTES = {
     "config1": 2117540,     # algorithmic 2,048,000 (profiles/softmax_and_resnet50_stack.md)
     "max_subsampling_tiling": 402617602,  # algorithmic 403,767,296 (profiles/tiling_and_entry_window_kernels.md)
     "entry_window": 256931085,            # algorithmic 256,901,120
-    "config4": 6365044940,  # per pass of the launch plan through the driver (51 plan steps in 17 kernel launches: independent groups
-                            # share launches), algorithmic 6,359,339,008 (profiles/chain_batch_kernel_config4_through_driver.md)
+    "config4": 6313909451,  # per pass of the launch plan through the driver (50 plan steps in 16 kernel launches: independent groups
+                            # share launches, the last group is applied by the average's kernel and neither written nor read
+                            # back), algorithmic 6,359,339,008 (profiles/chain_batch_kernel_config4_through_driver.md)
     "config4_direct": 6370619861,  # per step = the 51 launches of a pass (profiles/softmax_and_resnet50_stack.md)
     "walking_grid": 102999701,    # algorithmic 102,761,472 (profiles/chain_kernel_persistent_walking_grid.md)
 }
@@ -789,9 +790,21 @@ def cpu_per_config(runner, per_config, seconds_each=2.0):
         runner.capi.check(runner.lib.nnf_hip_average_subsampling_forward(runner.stream, d_pool.data_ptr(), pool_device.data_ptr(), pool_shape[0], pool_shape[1], 7, 7, 7, 7, 1.0 / 49.0))
         runner.sync()
         mismatches += bit_mismatches(d_pool.cpu().numpy(), want_pool)
+        # the form the driver runs the tail in: the last group applied by the average's kernel on the way in
+        last, last_chunks = prepared[-1]
+        assert len(last.arms) == 2 and (last.feature_map_count, last.plane) == (pool_shape[1], 49)
+        want_folded = cpu.oracle.average_subsampling(np.array(cpu.group_pass(last, last_chunks)).reshape(pool_shape), [7, 7], mult=1.0 / 49.0)
+        d_chunks = [torch.from_numpy(a).to(runner.device) for a in last_chunks]
+        desc = runner.capi.make_desc(last.entry_count, last.feature_map_count, last.plane, last.arms, last.tail)
+        runner.capi.check(runner.lib.nnf_hip_average_subsampling_joined_forward(
+            runner.stream, d_pool.data_ptr(), runner.capi.pointer_array([pool_device.data_ptr()] * 2), ctypes.byref(desc),
+            runner.capi.pointer_array([t.data_ptr() for t in d_chunks]), pool_shape[0], pool_shape[1], 7, 7, 7, 7, 1.0 / 49.0))
+        runner.sync()
+        mismatches += bit_mismatches(d_pool.cpu().numpy(), want_folded)
         attach("config4", sec, k, "the whole stack (49 groups unfused + average + softmax)",
                {"gpu_bit_mismatches_vs_cpu": mismatches, "gpu_worst_relative_difference_vs_cpu_softmax": softmax_worst_relative(sm_in, sm_out),
-                "checked": "the 49 groups and the 7x7 average bit for bit at N=64 through the C ABI, the softmax to its relative bar"})
+                "checked": "the 49 groups, the 7x7 average and the last group folded into the average bit for bit at N=64 through the C ABI, "
+                           "the softmax to its relative bar"})
 
 
 def main():
