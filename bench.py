@@ -870,7 +870,7 @@ def main():
     per_config[args.workload] = main_entry
     cpu = None
     if not args.only:
-        side_steps = {"config0": (200, 20), "config1": (400, 40), "config2": (20, 3), "config3": (60, 6), "config4": (5, 2)}
+        side_steps = {"config0": (200, 20), "config1": (400, 40), "config2": (20, 3), "config3": (60, 6), "config4": (10, 3)}
         for name in ("config0", "config1", "config2", "config3", "config4"):
             if name not in per_config:
                 per_config[name] = run(name, *side_steps[name])
