@@ -163,12 +163,22 @@ namespace nnf
 		// which leaves the kernel with far fewer registers per lane.
 		constexpr int coef_batch = 4; // vectors whose batch norm coefficients are read from LDS together
 
+		// Where the coefficients of a vector's values lie when the four values may belong to two planes: values
+		// [0, split) take the coefficients at off (the argument beside this one), the others those at off2.
+		template<int VECTORS>
+		struct two_plane_offsets
+		{
+			uint32_t off2[VECTORS];
+			uint32_t split[VECTORS];
+		};
+
 		// UNIFORM: every value belongs to the same plane, whose coefficients are in own (registers)
-		// instead of coef (LDS). Applies the layers first_op .. end_op - 1.
-		template<int VECTORS, bool EXP, bool UNIFORM>
+		// instead of coef (LDS). SPLIT: a vector's values may belong to two planes (two says which).
+		// Applies the layers first_op .. end_op - 1.
+		template<int VECTORS, bool EXP, bool UNIFORM, bool SPLIT = false>
 		__device__ __forceinline__ void apply_prologue(float (&v)[VECTORS][4], const uint32_t (&off)[VECTORS],
 			const float* coef, const float (&own)[prologue_weighted_max][2], const window_prologue& pro, const exp_context& exp_ctx,
-			uint32_t first_op, uint32_t end_op)
+			uint32_t first_op, uint32_t end_op, const two_plane_offsets<VECTORS>* two = nullptr)
 		{
 			for(uint32_t i = first_op; i < end_op; ++i)
 			{
@@ -189,6 +199,29 @@ namespace nnf
 							#pragma unroll
 							for(int e = 0; e < 4; ++e)
 								v[k][e] = nnf_batch_norm(v[k][e], mult, add);
+						}
+						break;
+					}
+					if (SPLIT)
+					{
+						float mult[VECTORS][2], add[VECTORS][2];
+						#pragma unroll
+						for(int k = 0; k < VECTORS; ++k)
+						{
+							mult[k][0] = coef[off[k] + slot];
+							add[k][0] = coef[off[k] + slot + 1];
+							mult[k][1] = coef[two->off2[k] + slot];
+							add[k][1] = coef[two->off2[k] + slot + 1];
+						}
+						#pragma unroll
+						for(int k = 0; k < VECTORS; ++k)
+						{
+							#pragma unroll
+							for(int e = 0; e < 4; ++e)
+							{
+								const bool first_plane = static_cast<uint32_t>(e) < two->split[k];
+								v[k][e] = nnf_batch_norm(v[k][e], first_plane ? mult[k][0] : mult[k][1], first_plane ? add[k][0] : add[k][1]);
+							}
 						}
 						break;
 					}
@@ -221,6 +254,23 @@ namespace nnf
 							#pragma unroll
 							for(int e = 0; e < 4; ++e)
 								v[k][e] = nnf_parametric_rectified_linear(v[k][e], slope);
+						}
+					}
+					else if (SPLIT)
+					{
+						float slope[VECTORS][2];
+						#pragma unroll
+						for(int k = 0; k < VECTORS; ++k)
+						{
+							slope[k][0] = coef[off[k] + slot];
+							slope[k][1] = coef[two->off2[k] + slot];
+						}
+						#pragma unroll
+						for(int k = 0; k < VECTORS; ++k)
+						{
+							#pragma unroll
+							for(int e = 0; e < 4; ++e)
+								v[k][e] = nnf_parametric_rectified_linear(v[k][e], (static_cast<uint32_t>(e) < two->split[k]) ? slope[k][0] : slope[k][1]);
 						}
 					}
 					else
@@ -283,19 +333,20 @@ namespace nnf
 		// The whole group over the values of input 0 (v) and, with JOIN, input 1 (u): each input's own layers, the
 		// Add (nnforge/plain/add_layer_tester_plain.cpp:56-59: the sum starts at 0.0F, inputs in order, times
 		// alpha), the layers behind it. The result is left in v.
-		template<int VECTORS, bool EXP, bool JOIN>
+		template<int VECTORS, bool EXP, bool JOIN, bool UNIFORM = false, bool SPLIT = false>
 		__device__ __forceinline__ void apply_prologue_group(float (&v)[VECTORS][4], float (&u)[VECTORS][4], const uint32_t (&off)[VECTORS],
-			const float* coef, const float (&own)[prologue_weighted_max][2], const window_prologue& pro, const exp_context& exp_ctx)
+			const float* coef, const float (&own)[prologue_weighted_max][2], const window_prologue& pro, const exp_context& exp_ctx,
+			const two_plane_offsets<VECTORS>* two = nullptr)
 		{
 			if (!JOIN)
 			{
-				apply_prologue<VECTORS, EXP, false>(v, off, coef, own, pro, exp_ctx, 0, pro.op_count);
+				apply_prologue<VECTORS, EXP, UNIFORM, SPLIT>(v, off, coef, own, pro, exp_ctx, 0, pro.op_count, two);
 				return;
 			}
 			const uint32_t arm0_end = pro.arm_ops[0];
 			const uint32_t arm1_end = arm0_end + pro.arm_ops[1];
-			apply_prologue<VECTORS, EXP, false>(v, off, coef, own, pro, exp_ctx, 0, arm0_end);
-			apply_prologue<VECTORS, EXP, false>(u, off, coef, own, pro, exp_ctx, arm0_end, arm1_end);
+			apply_prologue<VECTORS, EXP, UNIFORM, SPLIT>(v, off, coef, own, pro, exp_ctx, 0, arm0_end, two);
+			apply_prologue<VECTORS, EXP, UNIFORM, SPLIT>(u, off, coef, own, pro, exp_ctx, arm0_end, arm1_end, two);
 			#pragma unroll
 			for(int k = 0; k < VECTORS; ++k)
 			{
@@ -307,7 +358,7 @@ namespace nnf
 					v[k][e] = sum * pro.alpha;
 				}
 			}
-			apply_prologue<VECTORS, EXP, false>(v, off, coef, own, pro, exp_ctx, arm1_end, pro.op_count);
+			apply_prologue<VECTORS, EXP, UNIFORM, SPLIT>(v, off, coef, own, pro, exp_ctx, arm1_end, pro.op_count, two);
 		}
 
 		uint32_t magic_of(uint32_t divisor)

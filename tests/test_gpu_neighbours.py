@@ -387,6 +387,13 @@ def run_fused_pool(gpu, x, ops, chunks, ww, wh, mult, expect=0):
     ((2, 7, 15, 15), 15, 15, "bn_relu"),               # 225 floats per plane
     ((6, 11, 3, 5), 5, 3, "leaky"),
     ((1, 1, 2, 2), 2, 2, "bn_relu"),
+    # odd planes: every wavefront on its own 32 planes, the layers applied per plane on the way out of LDS
+    ((1, 37, 7, 7), 7, 7, "bn_prelu_elu_sigmoid"),     # 37 planes: a full wavefront and one with 5 planes (245 floats: one behind the last float4)
+    ((70, 3, 3, 3), 3, 3, "bn_relu"),                  # 210 planes of 9 floats: the last wavefront holds 18 of them
+    ((5, 33, 5, 5), 5, 5, "prelu_bn"),
+    ((3, 7, 9, 9), 9, 9, "tanh_abs"),
+    ((2, 3, 11, 11), 11, 11, "bn_prelu_elu_sigmoid"),  # 121 floats per plane: 62 KB of LDS per workgroup
+    ((2, 5, 13, 13), 13, 13, "bn_relu"),               # 169 floats per plane: beyond that kernel, odd all the same
 ])
 def test_average_subsampling_with_group_folded_in(gpu, shape, ww, wh, group):
     gen = T.rng(67, sum(shape) + ww)
@@ -410,6 +417,10 @@ JOINED_POOL_CASES = [
     ((9, 70, 8, 8), ("leaky", "-"), 2.0, "none"),       # planes that are multiples of 4 floats, nothing behind the Add
     ((2, 7, 15, 15), ("bn", "-"), 1.0, "prelu"),        # 225 floats per plane, weights on an arm and behind the join
     ((1, 1, 2, 2), ("-", "-"), 1.0, "relu"),
+    ((1, 37, 7, 7), ("bn", "elu"), 1.0, "sigmoid"),     # a wavefront with 5 planes: 245 floats, one behind the last float4
+    ((70, 3, 3, 3), ("bn", "leaky"), 1.0, "relu"),      # 210 planes of 9 floats
+    ((4, 9, 5, 5), ("-", "bn"), 0.25, "prelu"),
+    ((2, 3, 11, 11), ("bn", "-"), 1.0, "relu"),         # 121 floats per plane: two staged tensors do not fit the odd-plane kernel
 ]
 
 

@@ -634,6 +634,10 @@ def test_global_average_7x7(gpu, n, c):
                                          # whole-plane windows of several sizes (global pooling kernel up to 240 floats per plane)
                                          ((5, 70, 14, 14), 14, 14), ((3, 9, 15, 15), 15, 15), ((2, 5, 15, 16), 16, 15), ((2, 3, 16, 16), 16, 16),
                                          ((70, 3, 8, 8), 8, 8),
+                                         # odd planes: every wavefront on its own 32 planes (37 planes: a wavefront with 5; 210 planes of 9 floats;
+                                         # 121 floats per plane; 169 and 225 are beyond that kernel)
+                                         ((1, 37, 7, 7), 7, 7), ((70, 3, 3, 3), 3, 3), ((5, 33, 5, 5), 5, 5), ((3, 7, 9, 9), 9, 9), ((2, 3, 11, 11), 11, 11),
+                                         ((2, 5, 13, 13), 13, 13), ((9, 1, 3, 1), 1, 3),
                                          # more than 65535 outputs per plane: the one-lane-per-output kernel
                                          ((1, 1, 300, 300), 1, 1), ((1, 1, 520, 260), 2, 1)])
 def test_average_subsampling_windows(gpu, shape, ww, wh):
