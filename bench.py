@@ -48,6 +48,8 @@ MEASURED_TRAFFIC_BYTES = {
                             # back), algorithmic 6,359,339,008 (profiles/chain_batch_kernel_config4_through_driver.md)
     "config4_direct": 6370619861,  # per step = the 51 launches of a pass (profiles/softmax_and_resnet50_stack.md)
     "walking_grid": 102999701,    # algorithmic 102,761,472 (profiles/chain_kernel_persistent_walking_grid.md)
+    "global_average": 26245200,         # algorithmic 26,214,400 (profiles/global_pool_linear_kernel_7x7_average.md)
+    "joined_global_average": 52080216,  # algorithmic 51,937,280
 }
 
 
@@ -397,6 +399,42 @@ def bench_bn_relu_max_subsampling(runner, steps, warmup, n=64, c=64, size=112):
     wall, ev = runner.time_steps(launch, steps, warmup)
     return result_entry("batch_norm -> rectified_linear -> max_subsampling 3x3 stride 2 round up, N=%d C=%d %dx%d -> %dx%d" % (n, c, size, size, out_size, out_size),
                         4 * (in_count + out_count + 4 * c), out_count, wall, ev, 1, {"buffer_sets": sets})
+
+
+def bench_global_average(runner, steps, warmup, n=64, c=2048, size=7, joined=False):
+    """The end of a ResNet: the 7x7 average over 2048 feature maps - alone, or (joined) with the last block's
+    BatchNorm(main) + residual -> Add -> ReLU applied to the two tensors on their way in, one launch."""
+    plane = size * size
+    in_count, out_count = n * c * plane, n * c
+    tensors = 2 if joined else 1
+    alg = 4 * (tensors * in_count + out_count) + (16 * c if joined else 0)
+    sets = max(rotation_sets(alg), 24)
+    ins = [[runner.randn(in_count) for _ in range(tensors)] for _ in range(sets)]
+    outs = [runner.empty(out_count) for _ in range(sets)]
+    lib, capi, stream = runner.lib, runner.capi, runner.stream
+    mult = 1.0 / plane
+    if joined:
+        chunks = runner.bn_chunks(c)
+        chunk_ptrs = capi.pointer_array([t.data_ptr() for t in chunks])
+        desc = capi.make_desc(n, c, plane, [[], [(capi.OP_BATCH_NORM, 0)]], [(capi.OP_RELU, 0, 0.0)])
+        in_ptrs = [capi.pointer_array([t.data_ptr() for t in pair]) for pair in ins]
+
+        def launch(i):
+            rc = lib.nnf_hip_average_subsampling_joined_forward(stream, outs[i % sets].data_ptr(), in_ptrs[i % sets], ctypes.byref(desc), chunk_ptrs,
+                                                                n, c, size, size, size, size, mult)
+            if rc != 0:
+                raise RuntimeError(capi.error_string(rc))
+    else:
+        def launch(i):
+            rc = lib.nnf_hip_average_subsampling_forward(stream, outs[i % sets].data_ptr(), ins[i % sets][0].data_ptr(), n, c, size, size, size, size, mult)
+            if rc != 0:
+                raise RuntimeError(capi.error_string(rc))
+
+    wall, ev = runner.time_steps(launch, steps, warmup)
+    queued = time_steps_queued(runner, launch, min(max(steps, 50), 400), hold_ms=8.0)
+    what = "batch_norm + residual -> add -> rectified_linear -> average over %dx%d, one launch" if joined else "average over %dx%d (whole planes)"
+    return result_entry((what % (size, size)) + ", N=%d C=%d" % (n, c), alg, out_count, wall, ev, 1,
+                        {"buffer_sets": sets, "queued_event_ms_per_step": queued * 1e3, "queued_event_gbps": alg / queued / 1e9})
 
 
 def bench_concat(runner, steps, warmup, n=32, fms=(64, 128, 32, 32), plane=28 * 28):
@@ -813,7 +851,8 @@ def main():
     ap.add_argument("--steps", type=int, default=400)
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--workload", default="config0", choices=["config0", "config1", "config2", "config3", "config4", "copy", "max_subsampling", "bn_relu_max_subsampling", "max_subsampling_tiling",
-                             "entry_window", "concat", "maxout", "feature_map_stat", "config4_direct", "yardsticks", "walking_grid"],
+                             "entry_window", "concat", "maxout", "feature_map_stat", "config4_direct", "yardsticks", "walking_grid",
+                             "global_average", "joined_global_average"],
                     help="'copy' times the plain copy kernel (profiler-counter calibration and bandwidth yardstick); 'yardsticks' the runtime's and "
                          "torch's copy routines beside the library's kernels; 'config4_direct' the launches of config4 issued at the C ABI from this script")
     ap.add_argument("--entries", type=int, default=64, help="config4: entries per packet (BASELINE.json's configuration has 64)")
@@ -858,6 +897,10 @@ def main():
             return bench_maxout(runner, steps, warmup)
         if name == "feature_map_stat":
             return bench_feature_map_stat(runner, steps, warmup)
+        if name == "global_average":
+            return bench_global_average(runner, steps, warmup)
+        if name == "joined_global_average":
+            return bench_global_average(runner, steps, warmup, joined=True)
         if name == "walking_grid":
             return bench_group(runner, "batch_norm -> rectified_linear N=64 C=64 56x56 (51 MB per tensor: the grid that stays put)", w.bn_relu("bn_relu", 64, 64, 56 * 56), steps, warmup)
         if name == "config4_direct":
@@ -876,7 +919,8 @@ def main():
                 per_config[name] = run(name, *side_steps[name])
         per_config["copy_kernel"] = bench_copy(runner, 40, 5)
         # the neighbouring layers of the same chains
-        for name, (k, wu) in (("max_subsampling", (40, 5)), ("bn_relu_max_subsampling", (40, 5)), ("max_subsampling_tiling", (40, 5)), ("entry_window", (40, 5)), ("concat", (100, 10)), ("maxout", (100, 10)), ("feature_map_stat", (20, 3))):
+        for name, (k, wu) in (("global_average", (100, 10)), ("joined_global_average", (100, 10)), ("max_subsampling", (40, 5)), ("bn_relu_max_subsampling", (40, 5)),
+                              ("max_subsampling_tiling", (40, 5)), ("entry_window", (40, 5)), ("concat", (100, 10)), ("maxout", (100, 10)), ("feature_map_stat", (20, 3))):
             if name not in per_config:
                 per_config[name] = run(name, k, wu)
         if args.workload == "config0":
@@ -921,6 +965,7 @@ def main():
                        "max_subsampling_tiling": "nnf::tiling2d_kernel", "entry_window": "nnf::window_rows_kernel",
                        "concat": "nnf::concat_kernel", "maxout": "nnf::maxout_vec4_kernel",
                        "feature_map_stat": "nnf::stat_runs_kernel", "walking_grid": "nnf::chain_kernel_persistent",
+                       "global_average": "nnf::global_pool_linear_kernel", "joined_global_average": "nnf::global_pool_linear_kernel",
                        "config4": "all kernels of one pass of the launch plan (nnf::chain_batch_kernel, nnf::chain_kernel, nnf::global_pool_kernel, nnf::softmax_rows_kernel)",
                        "config4_direct": "all kernels of one pass (nnf::chain_kernel x 49, nnf::global_pool_kernel, nnf::softmax_rows_kernel)"}.get(args.workload, "nnf::chain_kernel"),
             "algorithmic_bytes_per_launch": main_entry["algorithmic_bytes_per_step"] / launches,
