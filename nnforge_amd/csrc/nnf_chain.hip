@@ -501,17 +501,20 @@ namespace nnf
 		// after the other, a workgroup finds its group by its index and then does what chain_kernel does. The time a
 		// launch loses while the device fills and drains is paid once for all of them (measured with 51 one-read-
 		// one-write tensors of the ResNet-50 stack's sizes: 915 us one by one, 831 us six per launch, at 64 entries;
-		// 214 against 121 us at 8 entries). All groups of a launch share NIN, the launch shape and DIRECT.
+		// 214 against 121 us at 8 entries). All groups of a launch share NIN and the launch shape. DIRECT_MODE: how
+		// they read their weights - all through LDS coefficients (0), all straight from memory (1), or each its own way
+		// (2: direct_mask says which; the workgroup takes one path or the other as a whole).
 		constexpr uint32_t max_batch = 6; // 6 x sizeof(chain_args) stays inside 4 KB of kernel arguments
 		struct chain_batch_args
 		{
 			uint32_t count;
+			uint32_t direct_mask;         // bit g: group g reads its weights straight from memory
 			uint32_t tile_end[max_batch]; // running total of the groups' tile counts
 			chain_args group[max_batch];
 		};
 		static_assert(sizeof(chain_batch_args) <= 4096, "kernel arguments of a batch beyond 4 KB");
 
-		template<int NIN, int BLOCK, int U, bool DIRECT>
+		template<int NIN, int BLOCK, int U, int DIRECT_MODE>
 		__global__ void __launch_bounds__(BLOCK) chain_batch_kernel(const chain_batch_args b)
 		{
 			extern __shared__ __align__(16) unsigned char lds_raw[];
@@ -519,7 +522,10 @@ namespace nnf
 			while ((g + 1 < b.count) && (blockIdx.x >= b.tile_end[g]))
 				++g;
 			const uint32_t tile_index = blockIdx.x - ((g == 0) ? 0u : b.tile_end[g - 1]);
-			chain_tile<NIN, BLOCK, U, DIRECT, 0>(b.group[g], tile_index, lds_raw);
+			if ((DIRECT_MODE == 1) || ((DIRECT_MODE == 2) && (((b.direct_mask >> g) & 1u) != 0)))
+				chain_tile<NIN, BLOCK, U, true, 0>(b.group[g], tile_index, lds_raw);
+			else
+				chain_tile<NIN, BLOCK, U, false, 0>(b.group[g], tile_index, lds_raw);
 		}
 
 		// The same group on a grid that stays put: as many workgroups as the device holds at once (or fewer), each
@@ -950,26 +956,37 @@ namespace nnf
 
 		typedef void (*chain_batch_kernel_fn)(const chain_batch_args);
 
-		template<int NIN>
-		chain_batch_kernel_fn pick_batch_kernel_of(int shape, bool direct)
+		template<int NIN, int BLOCK, int U>
+		chain_batch_kernel_fn pick_batch_kernel_mode(int direct_mode)
 		{
-			switch (shape)
+			switch (direct_mode)
 			{
-			case 0: return direct ? chain_batch_kernel<NIN, 256, 4, true> : chain_batch_kernel<NIN, 256, 4, false>;
-			case 1: return direct ? chain_batch_kernel<NIN, 256, 2, true> : chain_batch_kernel<NIN, 256, 2, false>;
-			case 2: return direct ? chain_batch_kernel<NIN, 256, 1, true> : chain_batch_kernel<NIN, 256, 1, false>;
-			default: return direct ? chain_batch_kernel<NIN, 64, 1, true> : chain_batch_kernel<NIN, 64, 1, false>;
+			case 0: return chain_batch_kernel<NIN, BLOCK, U, 0>;
+			case 1: return chain_batch_kernel<NIN, BLOCK, U, 1>;
+			default: return chain_batch_kernel<NIN, BLOCK, U, 2>;
 			}
 		}
 
-		chain_batch_kernel_fn pick_batch_kernel(uint32_t input_count, int shape, bool direct)
+		template<int NIN>
+		chain_batch_kernel_fn pick_batch_kernel_of(int shape, int direct_mode)
+		{
+			switch (shape)
+			{
+			case 0: return pick_batch_kernel_mode<NIN, 256, 4>(direct_mode);
+			case 1: return pick_batch_kernel_mode<NIN, 256, 2>(direct_mode);
+			case 2: return pick_batch_kernel_mode<NIN, 256, 1>(direct_mode);
+			default: return pick_batch_kernel_mode<NIN, 64, 1>(direct_mode);
+			}
+		}
+
+		chain_batch_kernel_fn pick_batch_kernel(uint32_t input_count, int shape, int direct_mode)
 		{
 			switch (input_count)
 			{
-			case 1: return pick_batch_kernel_of<1>(shape, direct);
-			case 2: return pick_batch_kernel_of<2>(shape, direct);
-			case 3: return pick_batch_kernel_of<3>(shape, direct);
-			default: return pick_batch_kernel_of<4>(shape, direct);
+			case 1: return pick_batch_kernel_of<1>(shape, direct_mode);
+			case 2: return pick_batch_kernel_of<2>(shape, direct_mode);
+			case 3: return pick_batch_kernel_of<3>(shape, direct_mode);
+			default: return pick_batch_kernel_of<4>(shape, direct_mode);
 			}
 		}
 	}
@@ -1033,7 +1050,7 @@ namespace nnf
 				for(uint32_t j = first + 1; (j < group_count) && (members.size() < max_batch); ++j)
 				{
 					const prepared_group& g = groups[j];
-					if (!launched[j] && !g.nothing_to_do && (g.program == 0) && (g.input_count == lead.input_count) && (g.shape == lead.shape) && (g.direct == lead.direct))
+					if (!launched[j] && !g.nothing_to_do && (g.program == 0) && (g.input_count == lead.input_count) && (g.shape == lead.shape))
 					{
 						members.push_back(j);
 						launched[j] = true;
@@ -1054,13 +1071,16 @@ namespace nnf
 			{
 				const prepared_group& g = groups[members[m]];
 				b.group[m] = g.a;
+				b.direct_mask |= g.direct ? (1u << m) : 0u;
 				tiles += g.tiles;
 				b.tile_end[m] = static_cast<uint32_t>(tiles);
 				lds_bytes = std::max(lds_bytes, g.lds_bytes);
 			}
 			if (tiles > 0x7FFFFFFFull)
 				return NNF_HIP_ETOOBIG;
-			hipLaunchKernelGGL(pick_batch_kernel(lead.input_count, lead.shape, lead.direct), dim3(static_cast<uint32_t>(tiles)), dim3(launch_shapes[lead.shape].block),
+			const uint32_t all_direct = (1u << b.count) - 1u;
+			const int direct_mode = (b.direct_mask == all_direct) ? 1 : ((b.direct_mask == 0) ? 0 : 2);
+			hipLaunchKernelGGL(pick_batch_kernel(lead.input_count, lead.shape, direct_mode), dim3(static_cast<uint32_t>(tiles)), dim3(launch_shapes[lead.shape].block),
 				lds_bytes, stream, b);
 			const int rc = launch_status();
 			if (rc != NNF_HIP_OK)
