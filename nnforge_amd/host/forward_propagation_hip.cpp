@@ -994,11 +994,12 @@ namespace nnforge
 
 		// Packets of entries flow through in-order queues with two I/O slots (the double buffering
 		// of nnforge/cuda/forward_propagation_cuda.cpp:84-112, 147-316):
-		//   host reads packet i into the pinned staging of slot i % 2   (needs: upload of packet i-2 done)
-		//   upload stream copies it to the slot's device input buffers   (needs: kernels of packet i-2 done)
+		//   the job runner's threads read packet i into the pinned staging of slot i % 2, one job per entry
+		//                                                                (needs: upload of packet i-2 done)
+		//   meanwhile the calling thread hands packet i-1 to the writer  (needs: download i-1 done)
+		//   upload stream copies packet i to the slot's device input buffers (needs: kernels of packet i-2 done)
 		//   kernel streams run the launch plan                           (needs: upload i, download i-2, kernels i-1 done)
 		//   download stream copies the slot's output buffers to staging  (needs: kernels i done)
-		//   host hands packet i-1 to the writer while packet i is in flight.
 		// Data and output layers have a device buffer per slot; everything in between is shared, which is
 		// safe because the kernels of one packet start after those of the packet before.
 		void forward_propagation_hip::actual_run(
