@@ -176,9 +176,13 @@ def random_network(gen, layer_count=14, c=6, size=12, with_entry_factors=False):
             else:
                 layers.append(L("MaxSubsampling", name, [src], windows=[2, 2]))
                 shapes[name] = (fm, [d // 2 for d in dims])
-        elif min(dims) >= 4:
+        elif min(dims) >= 4 and gen.random() < 0.6:
             layers.append(L("AverageSubsampling", name, [src], windows=[2, 2]))
             shapes[name] = (fm, [d // 2 for d in dims])
+        elif min(dims) >= 2:
+            # the average over whole planes (behind an Add and its layers: one launch with them)
+            layers.append(L("AverageSubsampling", name, [src], windows=list(dims)))
+            shapes[name] = (fm, [1, 1])
         else:
             layers.append(L("Absolute", name, [src]))
             shapes[name] = (fm, dims)
