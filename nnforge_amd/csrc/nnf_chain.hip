@@ -39,7 +39,10 @@ namespace nnf
 			int32_t reserved;
 		};
 
-		struct chain_args
+		// SLOTS: layers with per-feature-map weights the group may hold (a single launch takes up to max_slots; the
+		// groups of a shared launch travel side by side in the kernel arguments and take batch_slots at most)
+		template<int SLOTS>
+		struct chain_args_t
 		{
 			const float* in[NNF_HIP_MAX_INPUTS];
 			float* out;
@@ -55,8 +58,11 @@ namespace nnf
 			uint32_t slot_count;
 			uint32_t need_exp;
 			chain_op ops[NNF_HIP_MAX_OPS];
-			chain_slot slots[max_slots];
+			chain_slot slots[SLOTS];
 		};
+		typedef chain_args_t<max_slots> chain_args;
+		constexpr int batch_slots = 3;
+		typedef chain_args_t<batch_slots> chain_batch_group_args;
 
 		// Plane index (relative to the first plane of the tile) of tile-local element offset e,
 		// where e already includes the offset of the tile start inside its first plane.
@@ -103,11 +109,11 @@ namespace nnf
 		// DIRECT: where[k][0] is the feature map of float4 k and per-feature-map weights are read from
 		// memory (all lanes of a wavefront read the same one or two addresses: one cache line).
 		// Otherwise where[k][e] indexes the coefficient arrays the workgroup staged in LDS.
-		template<int U, bool DIRECT, int EXP_BATCH>
+		template<int U, bool DIRECT, int EXP_BATCH, class A>
 		__device__ __forceinline__ void apply_op(
 			int kind,
 			const chain_op& op,
-			const chain_args& a,
+			const A& a,
 			float (&v)[U][4],
 			const uint32_t (&where)[U][DIRECT ? 1 : 4],
 			const float2* lds_coeff,
@@ -220,8 +226,8 @@ namespace nnf
 		// Only one float4 of a whole tensor can be partial: the one that starts at tail_start when the
 		// element count is not a multiple of four. It is left out here (zeros) and travels through scalar
 		// loads and stores of its own, so that every other access is a float4 guarded by one comparison.
-		template<int NIN, int BLOCK, int U>
-		__device__ __forceinline__ void load_tile(const chain_args& a, uint32_t tile_start, uint32_t tail_start, float (&x)[NIN][U][4])
+		template<int NIN, int BLOCK, int U, class A>
+		__device__ __forceinline__ void load_tile(const A& a, uint32_t tile_start, uint32_t tail_start, float (&x)[NIN][U][4])
 		{
 			#pragma unroll
 			for(int j = 0; j < NIN; ++j)
@@ -239,8 +245,8 @@ namespace nnf
 		}
 
 		// Whether this lane owns the tensor's partial float4 in the tile at tile_start, and as which of its U.
-		template<int BLOCK, int U>
-		__device__ __forceinline__ bool owns_tail_vector(const chain_args& a, uint32_t tile_start, uint32_t tail_start, uint32_t& k_tail)
+		template<int BLOCK, int U, class A>
+		__device__ __forceinline__ bool owns_tail_vector(const A& a, uint32_t tile_start, uint32_t tail_start, uint32_t& k_tail)
 		{
 			const uint32_t tail_vector = (tail_start - tile_start) / 4; // float4 index inside this tile, if it is here
 			k_tail = tail_vector / BLOCK;
@@ -248,8 +254,8 @@ namespace nnf
 				&& ((tail_vector % BLOCK) == threadIdx.x);
 		}
 
-		template<int NIN, int U>
-		__device__ __forceinline__ void load_tail_vector(const chain_args& a, uint32_t tail_start, uint32_t k_tail, float (&x)[NIN][U][4])
+		template<int NIN, int U, class A>
+		__device__ __forceinline__ void load_tail_vector(const A& a, uint32_t tail_start, uint32_t k_tail, float (&x)[NIN][U][4])
 		{
 			#pragma unroll
 			for(int j = 0; j < NIN; ++j)
@@ -269,8 +275,8 @@ namespace nnf
 			}
 		}
 
-		template<int BLOCK, int U>
-		__device__ __forceinline__ void store_tile(const chain_args& a, uint32_t tile_start, uint32_t tail_start, const float (&v)[U][4])
+		template<int BLOCK, int U, class A>
+		__device__ __forceinline__ void store_tile(const A& a, uint32_t tile_start, uint32_t tail_start, const float (&v)[U][4])
 		{
 			#pragma unroll
 			for(int k = 0; k < U; ++k)
@@ -285,8 +291,8 @@ namespace nnf
 			}
 		}
 
-		template<int U>
-		__device__ __forceinline__ void store_tail_vector(const chain_args& a, uint32_t tail_start, uint32_t k_tail, const float (&v)[U][4])
+		template<int U, class A>
+		__device__ __forceinline__ void store_tail_vector(const A& a, uint32_t tail_start, uint32_t k_tail, const float (&v)[U][4])
 		{
 			#pragma unroll
 			for(int k = 0; k < U; ++k)
@@ -304,8 +310,8 @@ namespace nnf
 		// Where the lane's values lie: DIRECT - the feature map of each float4; otherwise the index of each
 		// element's plane among the planes the tile touches (= its slot in the LDS coefficient arrays).
 		// first_fm: feature map of the tile's first plane.
-		template<int BLOCK, int U, bool DIRECT>
-		__device__ __forceinline__ void locate_tile(const chain_args& a, uint32_t tile_start, uint32_t (&where)[U][DIRECT ? 1 : 4], uint32_t& first_fm)
+		template<int BLOCK, int U, bool DIRECT, class A>
+		__device__ __forceinline__ void locate_tile(const A& a, uint32_t tile_start, uint32_t (&where)[U][DIRECT ? 1 : 4], uint32_t& first_fm)
 		{
 			constexpr int TILE = BLOCK * U * 4;
 			const uint32_t first_plane = tile_start / a.plane;
@@ -331,8 +337,8 @@ namespace nnf
 
 		// Coefficients of the planes a tile touches, once per workgroup into LDS (the caller adds the barrier):
 		// batch norm's multiplier and addend, PReLU's slope.
-		template<int BLOCK>
-		__device__ __forceinline__ void stage_coefficients(const chain_args& a, uint32_t first_fm, float2* lds_coeff)
+		template<int BLOCK, class A>
+		__device__ __forceinline__ void stage_coefficients(const A& a, uint32_t first_fm, float2* lds_coeff)
 		{
 			for(uint32_t s = 0; s < a.slot_count; ++s)
 			{
@@ -355,8 +361,8 @@ namespace nnf
 
 		// The group's layers in the order the arguments list them: every input's own layers, the Add that
 		// joins the inputs (if any), the layers behind it. The result is left in x[0].
-		template<int NIN, int U, bool DIRECT>
-		__device__ __forceinline__ void run_listed_layers(const chain_args& a, float (&x)[NIN][U][4], const uint32_t (&where)[U][DIRECT ? 1 : 4],
+		template<int NIN, int U, bool DIRECT, class A>
+		__device__ __forceinline__ void run_listed_layers(const A& a, float (&x)[NIN][U][4], const uint32_t (&where)[U][DIRECT ? 1 : 4],
 			const float2* lds_coeff, const exp_context& exp_ctx)
 		{
 			uint32_t op_index = 0;
@@ -416,8 +422,8 @@ namespace nnf
 		constexpr int known_program_count = sizeof(known_programs) / sizeof(known_programs[0]);
 
 		// One tile of one group, by one workgroup: the body of the two kernels below.
-		template<int NIN, int BLOCK, int U, bool DIRECT, int PROGRAM>
-		__device__ __forceinline__ void chain_tile(const chain_args& a, const uint32_t tile_index, unsigned char* lds_raw)
+		template<int NIN, int BLOCK, int U, bool DIRECT, int PROGRAM, class A>
+		__device__ __forceinline__ void chain_tile(const A& a, const uint32_t tile_index, unsigned char* lds_raw)
 		{
 			constexpr int TILE = BLOCK * U * 4;
 			constexpr int PL = DIRECT ? 1 : 4;
@@ -504,13 +510,13 @@ namespace nnf
 		// 214 against 121 us at 8 entries). All groups of a launch share NIN and the launch shape. DIRECT_MODE: how
 		// they read their weights - all through LDS coefficients (0), all straight from memory (1), or each its own way
 		// (2: direct_mask says which; the workgroup takes one path or the other as a whole).
-		constexpr uint32_t max_batch = 6; // 6 x sizeof(chain_args) stays inside 4 KB of kernel arguments
+		constexpr uint32_t max_batch = 11; // what 4 KB of kernel arguments hold
 		struct chain_batch_args
 		{
 			uint32_t count;
 			uint32_t direct_mask;         // bit g: group g reads its weights straight from memory
 			uint32_t tile_end[max_batch]; // running total of the groups' tile counts
-			chain_args group[max_batch];
+			chain_batch_group_args group[max_batch];
 		};
 		static_assert(sizeof(chain_batch_args) <= 4096, "kernel arguments of a batch beyond 4 KB");
 
@@ -956,6 +962,33 @@ namespace nnf
 
 		typedef void (*chain_batch_kernel_fn)(const chain_batch_args);
 
+		// a group's arguments in the form they take among the arguments of a shared launch (slot_count <= batch_slots)
+		chain_batch_group_args batch_group_args_of(const chain_args& a)
+		{
+			chain_batch_group_args c = {};
+			for(int j = 0; j < NNF_HIP_MAX_INPUTS; ++j)
+			{
+				c.in[j] = a.in[j];
+				c.arm_ops[j] = a.arm_ops[j];
+			}
+			c.out = a.out;
+			c.total = a.total;
+			c.fm_count = a.fm_count;
+			c.plane = a.plane;
+			c.plane_magic = a.plane_magic;
+			c.span = a.span;
+			c.has_add = a.has_add;
+			c.alpha = a.alpha;
+			c.tail_ops = a.tail_ops;
+			c.slot_count = a.slot_count;
+			c.need_exp = a.need_exp;
+			for(int i = 0; i < NNF_HIP_MAX_OPS; ++i)
+				c.ops[i] = a.ops[i];
+			for(int i = 0; i < batch_slots; ++i)
+				c.slots[i] = a.slots[i];
+			return c;
+		}
+
 		template<int NIN, int BLOCK, int U>
 		chain_batch_kernel_fn pick_batch_kernel_mode(int direct_mode)
 		{
@@ -1046,11 +1079,12 @@ namespace nnf
 			// the groups behind it that can share its kernel instance, max_batch to a launch; the compile-time
 			// expf programs are bound by the vector ALU, not by launches: they keep their own kernels
 			std::vector<uint32_t> members(1, first);
-			if (lead.program == 0)
+			if ((lead.program == 0) && (lead.a.slot_count <= static_cast<uint32_t>(batch_slots)))
 				for(uint32_t j = first + 1; (j < group_count) && (members.size() < max_batch); ++j)
 				{
 					const prepared_group& g = groups[j];
-					if (!launched[j] && !g.nothing_to_do && (g.program == 0) && (g.input_count == lead.input_count) && (g.shape == lead.shape))
+					if (!launched[j] && !g.nothing_to_do && (g.program == 0) && (g.input_count == lead.input_count) && (g.shape == lead.shape)
+						&& (g.a.slot_count <= static_cast<uint32_t>(batch_slots)))
 					{
 						members.push_back(j);
 						launched[j] = true;
@@ -1070,7 +1104,7 @@ namespace nnf
 			for(size_t m = 0; m < members.size(); ++m)
 			{
 				const prepared_group& g = groups[members[m]];
-				b.group[m] = g.a;
+				b.group[m] = batch_group_args_of(g.a);
 				b.direct_mask |= g.direct ? (1u << m) : 0u;
 				tiles += g.tiles;
 				b.tile_end[m] = static_cast<uint32_t>(tiles);
