@@ -115,7 +115,7 @@ NNF_HIP_API int nnf_hip_chain_forward(void* stream, const nnf_hip_chain_desc* de
 	const float* const* inputs, const float* const* chunk_ptrs);
 
 /* group_count fused groups that have nothing to do with each other, in as few launches as possible: groups that share a
- * kernel instance (same number of inputs, same tile size) go six to a launch, whose grid
+ * kernel instance (same number of inputs, same tile size, at most three layers with weights) go eleven to a launch, whose grid
  * is their tiles one after the other. Same results as group_count calls of nnf_hip_chain_forward with descs[i],
  * outputs[i], inputs[i], chunk_ptrs[i] (chunk_ptrs, or an entry of it, may be null where no layer has weights); what a
  * launch loses while the device fills and drains is paid once per launch instead of once per group. The groups run in

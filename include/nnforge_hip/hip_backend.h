@@ -90,7 +90,7 @@ namespace nnforge
 			static constexpr int default_kernel_stream_count = 3;
 			int kernel_stream_count;
 			// Runs of consecutive fused groups that do not depend on each other go to the kernels in one call, groups of
-			// a kind six to a launch; such runs take one kernel stream (kernel_stream_count then plays no part). Measured
+			// a kind eleven to a launch; such runs take one kernel stream (kernel_stream_count then plays no part). Measured
 			// on the 49 groups of the ResNet-50 post-convolution stack, all in one call: 64 entries 1091 -> 1042 us,
 			// 8 entries 243 -> 172 us.
 			bool batch_independent_groups;
