@@ -43,7 +43,7 @@ MEASURED_TRAFFIC_BYTES = {
     "config1": 2117540,     # algorithmic 2,048,000 (profiles/softmax_and_resnet50_stack.md)
     "max_subsampling_tiling": 402617602,  # algorithmic 403,767,296 (profiles/tiling_and_entry_window_kernels.md)
     "entry_window": 256931085,            # algorithmic 256,901,120
-    "config4": 6312949326,  # per pass of the launch plan through the driver (50 plan steps in 11 kernel launches: independent groups
+    "config4": 6313457776,  # per pass of the launch plan through the driver (50 plan steps in 8 kernel launches: independent groups
                             # share launches, the last group is applied by the average's kernel and neither written nor read
                             # back), algorithmic 6,359,339,008 (profiles/chain_batch_kernel_config4_through_driver.md)
     "config4_direct": 6370619861,  # per step = the 51 launches of a pass (profiles/softmax_and_resnet50_stack.md)
@@ -966,7 +966,7 @@ def main():
                        "concat": "nnf::concat_kernel", "maxout": "nnf::maxout_vec4_kernel",
                        "feature_map_stat": "nnf::stat_runs_kernel", "walking_grid": "nnf::chain_kernel_persistent",
                        "global_average": "nnf::global_pool_linear_kernel", "joined_global_average": "nnf::global_pool_linear_kernel",
-                       "config4": "all kernels of one pass of the launch plan (nnf::chain_batch_kernel, nnf::chain_kernel, nnf::global_pool_kernel, nnf::softmax_rows_kernel)",
+                       "config4": "all kernels of one pass of the launch plan (nnf::chain_batch_mixed_kernel, nnf::chain_batch_kernel, nnf::chain_kernel, nnf::global_pool_linear_kernel, nnf::softmax_rows_kernel)",
                        "config4_direct": "all kernels of one pass (nnf::chain_kernel x 49, nnf::global_pool_kernel, nnf::softmax_rows_kernel)"}.get(args.workload, "nnf::chain_kernel"),
             "algorithmic_bytes_per_launch": main_entry["algorithmic_bytes_per_step"] / launches,
             "avg_launch_us": main_entry["event_ms_per_step"] * 1e3 / launches,

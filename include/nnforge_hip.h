@@ -43,6 +43,8 @@ extern "C" {
 
 #define NNF_HIP_MAX_OPS 8
 #define NNF_HIP_MAX_INPUTS 4
+/* nnf_hip_chain_forward_batch: most groups one kernel launch takes (what fits into 4 KB of kernel arguments) */
+#define NNF_HIP_MAX_GROUPS_PER_LAUNCH 11
 
 /* Layer kinds of the element-wise chain kernel. The names in comments are nnForge's layer type
  * names (the keys of layer_tester_plain_factory, nnforge/plain/layer_tester_plain_factory.cpp:27-51). */
@@ -115,8 +117,8 @@ NNF_HIP_API int nnf_hip_chain_forward(void* stream, const nnf_hip_chain_desc* de
 	const float* const* inputs, const float* const* chunk_ptrs);
 
 /* group_count fused groups that have nothing to do with each other, in as few launches as possible: groups that share a
- * kernel instance (same number of inputs, same tile size, at most three layers with weights) go eleven to a launch, whose grid
- * is their tiles one after the other. Same results as group_count calls of nnf_hip_chain_forward with descs[i],
+ * kernel instance (same number of inputs and same tile size, or any mix of groups with one input and groups with two; at most
+ * three layers with weights) go NNF_HIP_MAX_GROUPS_PER_LAUNCH to a launch, whose grid is their tiles one after the other. Same results as group_count calls of nnf_hip_chain_forward with descs[i],
  * outputs[i], inputs[i], chunk_ptrs[i] (chunk_ptrs, or an entry of it, may be null where no layer has weights); what a
  * launch loses while the device fills and drains is paid once per launch instead of once per group. The groups run in
  * no particular order and possibly at the same time: the output of a group may overlap no other group's output or

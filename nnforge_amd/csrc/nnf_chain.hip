@@ -507,14 +507,16 @@ namespace nnf
 		// after the other, a workgroup finds its group by its index and then does what chain_kernel does. The time a
 		// launch loses while the device fills and drains is paid once for all of them (measured with 51 one-read-
 		// one-write tensors of the ResNet-50 stack's sizes: 915 us one by one, 831 us six per launch, at 64 entries;
-		// 214 against 121 us at 8 entries). All groups of a launch share NIN and the launch shape. DIRECT_MODE: how
+		// 214 against 121 us at 8 entries). All groups of a launch share NIN and the launch shape (groups of two kinds
+		// in one launch: chain_batch_mixed_kernel below). DIRECT_MODE: how
 		// they read their weights - all through LDS coefficients (0), all straight from memory (1), or each its own way
 		// (2: direct_mask says which; the workgroup takes one path or the other as a whole).
-		constexpr uint32_t max_batch = 11; // what 4 KB of kernel arguments hold
+		constexpr uint32_t max_batch = NNF_HIP_MAX_GROUPS_PER_LAUNCH; // what 4 KB of kernel arguments hold
 		struct chain_batch_args
 		{
 			uint32_t count;
 			uint32_t direct_mask;         // bit g: group g reads its weights straight from memory
+			uint32_t two_input_mask;      // bit g: group g has two inputs (chain_batch_mixed_kernel)
 			uint32_t tile_end[max_batch]; // running total of the groups' tile counts
 			chain_batch_group_args group[max_batch];
 		};
@@ -532,6 +534,36 @@ namespace nnf
 				chain_tile<NIN, BLOCK, U, true, 0>(b.group[g], tile_index, lds_raw);
 			else
 				chain_tile<NIN, BLOCK, U, false, 0>(b.group[g], tile_index, lds_raw);
+		}
+
+		// Groups with one input (four float4s per lane) and groups with two (two float4s per lane) in one launch: the
+		// tiles differ in size, the workgroups do not (BLOCK lanes), and a workgroup takes the body of its group's kind.
+		// What this buys: the groups of a residual network that wait for each other (the joins of a stage) are few
+		// per level of the graph, and each level can take a share of the groups that wait for nothing along, instead of
+		// being a small launch of its own.
+		template<int BLOCK, int DIRECT_MODE>
+		__global__ void __launch_bounds__(BLOCK) chain_batch_mixed_kernel(const chain_batch_args b)
+		{
+			extern __shared__ __align__(16) unsigned char lds_raw[];
+			uint32_t g = 0;
+			while ((g + 1 < b.count) && (blockIdx.x >= b.tile_end[g]))
+				++g;
+			const uint32_t tile_index = blockIdx.x - ((g == 0) ? 0u : b.tile_end[g - 1]);
+			const bool direct = (DIRECT_MODE == 1) || ((DIRECT_MODE == 2) && (((b.direct_mask >> g) & 1u) != 0));
+			if (((b.two_input_mask >> g) & 1u) != 0)
+			{
+				if (direct)
+					chain_tile<2, BLOCK, 2, true, 0>(b.group[g], tile_index, lds_raw);
+				else
+					chain_tile<2, BLOCK, 2, false, 0>(b.group[g], tile_index, lds_raw);
+			}
+			else
+			{
+				if (direct)
+					chain_tile<1, BLOCK, 4, true, 0>(b.group[g], tile_index, lds_raw);
+				else
+					chain_tile<1, BLOCK, 4, false, 0>(b.group[g], tile_index, lds_raw);
+			}
 		}
 
 		// The same group on a grid that stays put: as many workgroups as the device holds at once (or fewer), each
@@ -1012,6 +1044,22 @@ namespace nnf
 			}
 		}
 
+		chain_batch_kernel_fn pick_batch_mixed_kernel(int direct_mode)
+		{
+			switch (direct_mode)
+			{
+			case 0: return chain_batch_mixed_kernel<256, 0>;
+			case 1: return chain_batch_mixed_kernel<256, 1>;
+			default: return chain_batch_mixed_kernel<256, 2>;
+			}
+		}
+
+		// the two kinds of group chain_batch_mixed_kernel takes side by side
+		bool mixes(const prepared_group& g)
+		{
+			return ((g.input_count == 1) && (g.shape == 0)) || ((g.input_count == 2) && (g.shape == 1));
+		}
+
 		chain_batch_kernel_fn pick_batch_kernel(uint32_t input_count, int shape, int direct_mode)
 		{
 			switch (input_count)
@@ -1083,7 +1131,8 @@ namespace nnf
 				for(uint32_t j = first + 1; (j < group_count) && (members.size() < max_batch); ++j)
 				{
 					const prepared_group& g = groups[j];
-					if (!launched[j] && !g.nothing_to_do && (g.program == 0) && (g.input_count == lead.input_count) && (g.shape == lead.shape)
+					const bool same_kind = (g.input_count == lead.input_count) && (g.shape == lead.shape);
+					if (!launched[j] && !g.nothing_to_do && (g.program == 0) && (same_kind || (mixes(lead) && mixes(g)))
 						&& (g.a.slot_count <= static_cast<uint32_t>(batch_slots)))
 					{
 						members.push_back(j);
@@ -1106,16 +1155,18 @@ namespace nnf
 				const prepared_group& g = groups[members[m]];
 				b.group[m] = batch_group_args_of(g.a);
 				b.direct_mask |= g.direct ? (1u << m) : 0u;
+				b.two_input_mask |= (g.input_count == 2) ? (1u << m) : 0u;
 				tiles += g.tiles;
 				b.tile_end[m] = static_cast<uint32_t>(tiles);
 				lds_bytes = std::max(lds_bytes, g.lds_bytes);
 			}
 			if (tiles > 0x7FFFFFFFull)
 				return NNF_HIP_ETOOBIG;
-			const uint32_t all_direct = (1u << b.count) - 1u;
-			const int direct_mode = (b.direct_mask == all_direct) ? 1 : ((b.direct_mask == 0) ? 0 : 2);
-			hipLaunchKernelGGL(pick_batch_kernel(lead.input_count, lead.shape, direct_mode), dim3(static_cast<uint32_t>(tiles)), dim3(launch_shapes[lead.shape].block),
-				lds_bytes, stream, b);
+			const uint32_t all_groups = (1u << b.count) - 1u;
+			const int direct_mode = (b.direct_mask == all_groups) ? 1 : ((b.direct_mask == 0) ? 0 : 2);
+			const bool one_kind = (b.two_input_mask == 0) || (b.two_input_mask == all_groups) || !mixes(lead);
+			const chain_batch_kernel_fn kernel = one_kind ? pick_batch_kernel(lead.input_count, lead.shape, direct_mode) : pick_batch_mixed_kernel(direct_mode);
+			hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>(tiles)), dim3(launch_shapes[lead.shape].block), lds_bytes, stream, b);
 			const int rc = launch_status();
 			if (rc != NNF_HIP_OK)
 				return rc;

@@ -229,8 +229,8 @@ def test_plan_of_the_resnet50_post_convolution_graph_equals_the_benchmark_group_
     """Config 4 as a network: the graph examples/imagenet/imagenet_toolset.cpp:476-550, 729-831 builds, convolution outputs as
     data layers. With one launch per group the driver's fusion pass must arrive at the 49 groups nnforge_amd.workloads lists by
     hand (kind, shape, order), the last of them folded into the 7x7 average behind it, then the softmax; the residual of a block
-    that keeps its shape is the block before. By default the steps are ordered by depth in the graph and independent groups are
-    launched together."""
+    that keeps its shape is the block before. By default the steps are ordered so that groups which do not depend on each other
+    are launched together, in launches of about the same size."""
     from nnforge_amd import schemas, workloads as w
 
     layers, configs, outputs = schemas.resnet50_post_convolution()
@@ -290,8 +290,9 @@ def test_plan_of_the_resnet50_post_convolution_graph_equals_the_benchmark_group_
     assert [s["layers"] for s in single["steps"]] == [s["layers"] for s in steps]
     assert all(s["stream"] == 0 for s in single["steps"])
 
-    # the default: the same launches ordered by depth in the graph - everything that reads convolution outputs only comes
-    # first, the blocks that read the block before follow level by level - and every level's groups launched together
+    # the default: the same launches in six runs, as many as the longest chain of blocks that read the block before
+    # (res4a ... res4f); every run is one call for all its groups, at most eleven of them (one kernel launch), the groups
+    # nothing waits for spread over the runs so that each has about the same number of bytes to move
     batched = plan(layers, configs, outputs)["steps"]
     assert sorted(tuple(s["layers"]) for s in batched) == sorted(tuple(s["layers"]) for s in steps)
     assert all(s["stream"] == 0 for s in batched)
@@ -301,15 +302,22 @@ def test_plan_of_the_resnet50_post_convolution_graph_equals_the_benchmark_group_
             if source in position:
                 assert position[source] < i and batched[position[source]]["run"] != s["run"], (i, s)   # never in a run with its producer
     runs = [s["run"] for s in batched]
-    assert runs[:37] == [0] * 37 and batched[37]["layers"] == ["prob"] and runs[37] is None   # 1 + 16 + 16 + 4 groups, then the softmax
-    assert [batched[i]["layers"][-1] for i in range(38, 42)] == ["res2b_relu", "res3b_relu", "res4b_relu", "res5b_relu"] and runs[38:42] == [1] * 4
-    # the last block's group goes with the average: a launch of its own among the groups of its level
-    assert runs[42:45] == [2] * 3 and batched[45]["layers"][-1] == "pool5" and runs[45] is None and runs[46:] == [3, 3, 4, 5]
+    alone = [s["layers"][-1] for s in batched if s["run"] is None]
+    assert alone == ["prob", "pool5"]   # the softmax, and the last block's group with the average: launches of their own
+    in_runs = [r for r in runs if r is not None]
+    assert in_runs == sorted(in_runs) and sorted(set(in_runs)) == list(range(6))
+    run_bytes = [sum(floats(s["layers"][-1]) * (len(s["inputs"]) + 1) for s in batched if s["run"] == r) for r in range(6)]
+    run_sizes = [in_runs.count(r) for r in range(6)]
+    assert max(run_sizes) <= 11 and sum(run_sizes) == 48
+    assert max(run_bytes) < 1.2 * min(run_bytes), run_bytes
+    chain = [runs[position["res4%s_relu" % block]] for block in "abcdef"]
+    assert chain == list(range(6))
     # with the stem's pooling in the graph, batch norm and ReLU are applied on the way into the pooling kernel
     layers, configs, outputs = schemas.resnet50_post_convolution(with_pool1=True)
     rep = plan(layers, configs, outputs)
-    assert len(rep["steps"]) == 50 and rep["steps"][0]["layers"] == ["conv1_bn", "relu1", "pool1"] and rep["steps"][0]["fused"]
-    assert rep["steps"][0]["run"] is None and rep["steps"][1]["run"] == 0   # the pooling step is no fused group: it launches alone
+    stem = [s for s in rep["steps"] if s["layers"][-1] == "pool1"]
+    assert len(rep["steps"]) == 50 and len(stem) == 1 and stem[0]["layers"] == ["conv1_bn", "relu1", "pool1"] and stem[0]["fused"]
+    assert stem[0]["run"] is None and rep["steps"][0]["run"] == 0   # the pooling step is no fused group: it launches alone, behind the first run
 
 
 def stem_net(c=8):

@@ -453,6 +453,35 @@ def test_independent_groups_in_one_call_equal_the_groups_one_by_one(gpu, first_s
         check_exact(out, group[7], "group %d of the call (seed %d)" % (i, first_seed + i))
 
 
+@pytest.mark.parametrize("planes", [(784, 3136), (49, 9), (784, 49), (49, 196, 7, 3136)])
+def test_groups_of_one_and_of_two_inputs_share_launches(gpu, planes):
+    """A residual network's groups as the driver hands them over: BatchNorm -> ReLU over one tensor and BatchNorm
+    (-> BatchNorm on the shortcut) -> Add -> ReLU over two, thirteen of them in one call - more than one launch holds -
+    with planes whose weights are read straight from memory, planes that need staged coefficients, and both in one call."""
+    groups = []
+    for i in range(13):
+        gen = T.rng(17, 100 * len(planes) + i)
+        plane = planes[i % len(planes)]
+        n, c = 1 + i % 3, (5, 16, 64)[(i // 2) % 3]
+        x = T.normal(gen, (n, c, plane), 1.5)
+        g, b, m, s = T.bn_params(gen, c)
+        if i % 2 == 0:
+            groups.append(((n, c, plane), [[(BN, 0), (RELU, 0, 0.0)]], [], [x], [g, b, m, s], False, 1.0,
+                           oracle.rectified_linear(oracle.batch_norm(x, g, b, m, s))))
+        elif i % 4 == 1:
+            r = T.normal(gen, (n, c, plane))
+            groups.append(((n, c, plane), [[], [(BN, 0)]], [(RELU, 0, 0.0)], [r, x], [g, b, m, s], True, 1.0,
+                           oracle.rectified_linear(oracle.add([r, oracle.batch_norm(x, g, b, m, s)]))))
+        else:
+            y = T.normal(gen, (n, c, plane))
+            g2, b2, m2, s2 = T.bn_params(gen, c)
+            groups.append(((n, c, plane), [[(BN, 0)], [(BN, 4)]], [(RELU, 0, 0.0)], [y, x], [g2, b2, m2, s2, g, b, m, s], True, 1.0,
+                           oracle.rectified_linear(oracle.add([oracle.batch_norm(y, g2, b2, m2, s2), oracle.batch_norm(x, g, b, m, s)]))))
+    got = gpu.chain_batch([group[:7] for group in groups])
+    for i, (out, group) in enumerate(zip(got, groups)):
+        check_exact(out, group[7], "group %d of the call (plane %d, %d inputs)" % (i, group[0][2], len(group[3])))
+
+
 def test_groups_of_one_call_must_not_touch_each_other(gpu):
     x = gpu.to_device(T.normal(T.rng(16, 0), 4096))
     y = gpu.torch.empty(8192, dtype=gpu.torch.float32, device=gpu.device)
