@@ -363,6 +363,7 @@ namespace nnforge
 			std::vector<std::pair<std::string, pending_group> > groups; // materialized, in execution order
 			std::vector<std::pair<std::string, bool> > step_order;      // (layer name, is_group)
 			std::map<std::string, pending_group> prologues;             // subsampling layer -> the group it applies to its input
+			std::vector<unsigned int> step_slots;                       // with runs of groups launched together: the slot of every step of step_order
 
 			auto materialize = [&](const std::string& name)
 			{
@@ -592,7 +593,10 @@ namespace nnforge
 					{ return (slot[a] != slot[b]) ? (slot[a] < slot[b]) : (rank_in_slot[a] < rank_in_slot[b]); });
 				std::vector<std::pair<std::string, bool> > sorted;
 				for(size_t i : order)
+				{
 					sorted.push_back(step_order[i]);
+					step_slots.push_back(slot[i]);
+				}
 				step_order.swap(sorted);
 			}
 
@@ -746,11 +750,20 @@ namespace nnforge
 				for(const std::string& in : p->plans[i].info.input_names)
 					last_use[in] = i;
 
+			// With runs of groups launched together a buffer whose value dies in a slot is handed out again from the next slot
+			// on: given to a step of the same slot it would make that step wait for the buffer's readers, and the run would
+			// end there (device memory is not what this driver is short of).
 			std::vector<int> free_buffers;
+			std::vector<int> freed_in_this_slot;
 			std::set<int> shareable; // buffers that hold intermediate values
 			for(size_t i = 0; i < p->plans.size(); ++i)
 			{
 				step_plan& plan = p->plans[i];
+				if (!step_slots.empty() && (i > 0) && (step_slots[i] != step_slots[i - 1]))
+				{
+					free_buffers.insert(free_buffers.end(), freed_in_this_slot.begin(), freed_in_this_slot.end());
+					freed_in_this_slot.clear();
+				}
 				const std::string& out_name = plan.info.layer_names.back();
 				// per entry read: a layer behind a tiling layer holds several entries for each (nnforge/plain/forward_propagation_plain.cpp:281)
 				const size_t out_floats = static_cast<size_t>(layer_config_map[out_name].get_neuron_count()) * plan.entry_factor;
@@ -802,9 +815,10 @@ namespace nnforge
 				for(size_t j = 0; j < plan.info.input_names.size(); ++j)
 				{
 					const int b = plan.input_buffers[j];
+					std::vector<int>& released = step_slots.empty() ? free_buffers : freed_in_this_slot;
 					if ((last_use[plan.info.input_names[j]] == i) && (b != chosen) && (shareable.find(b) != shareable.end())
-						&& (std::find(free_buffers.begin(), free_buffers.end(), b) == free_buffers.end()))
-						free_buffers.push_back(b);
+						&& (std::find(released.begin(), released.end(), b) == released.end()))
+						released.push_back(b);
 				}
 			}
 

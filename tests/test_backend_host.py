@@ -320,6 +320,27 @@ def test_plan_of_the_resnet50_post_convolution_graph_equals_the_benchmark_group_
     assert stem[0]["run"] is None and rep["steps"][0]["run"] == 0   # the pooling step is no fused group: it launches alone, behind the first run
 
 
+def test_plan_keeps_independent_towers_in_the_same_runs():
+    """Two towers that share nothing, three groups deep, every group's result read twice (so nothing fuses across): the
+    groups of a depth form one run. A buffer whose value dies in a run is not handed to a later group of the same run -
+    that group would have to wait for the buffer's readers and the run would end there."""
+    layers, outputs = [], []
+    for k in "12":
+        layers += [S.L("Data", "d" + k), S.L("BatchNorm", "bn" + k, ["d" + k], feature_map_count=4), S.L("ReLU", "a" + k, ["bn" + k]),
+                   S.L("Absolute", "abs" + k, ["a" + k]), S.L("TanH", "t" + k, ["abs" + k], scale=1.0, steepness=1.0),
+                   S.L("Sigmoid", "sig" + k, ["a" + k]), S.L("Absolute", "s" + k, ["sig" + k]),
+                   S.L("ELU", "elu" + k, ["t" + k]), S.L("Absolute", "u" + k, ["elu" + k]),
+                   S.L("ReLU", "relu" + k, ["t" + k]), S.L("Sigmoid", "v" + k, ["relu" + k])]
+        outputs += ["s" + k, "u" + k, "v" + k]
+    rep = plan(layers, {"d1": (4, [6, 6]), "d2": (4, [6, 6])}, outputs)
+    runs = {s["layers"][-1]: s["run"] for s in rep["steps"]}
+    assert [runs[n] for n in ("a1", "a2")] == [0, 0]
+    assert [runs[n] for n in ("t1", "s1", "t2", "s2")] == [1, 1, 1, 1]
+    assert [runs[n] for n in ("u1", "v1", "u2", "v2")] == [2, 2, 2, 2]
+    # 2 inputs, 6 outputs, a1, a2, t1, t2 each in a buffer of its own (t2 not in a1's, which dies in the same run)
+    assert rep["per_entry_bytes"] == 4 * (12 * 4 * 36)
+
+
 def stem_net(c=8):
     """BatchNorm -> ReLU -> overlapping max pooling, then TanH -> Absolute -> 2x2 average pooling (the stage of
     nnForge's GTSRB example, examples/gtsrb/schema.txt), then a global average."""
