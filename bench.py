@@ -12,7 +12,7 @@ under "per_config" on the same JSON line.
 
 Prints ONE JSON line. `value` = algorithmic bytes per step / wall time per step (GB/s), where the
 wall time brackets exactly K steps with a device synchronisation on both sides. `roofline` is
-measured with HIP events on the launch stream around a second pass of the same K steps (recording
+measured with HIP events on the launch stream around three further passes of the same K steps, the median taken (recording
 the events inside the wall-clock region would add about 10 us of instrumentation to it). `cpu_baseline` is the CPU
 restatement of nnForge's plain backend (oracle/, layer by layer, unfused, OpenMP on all host
 cores) timed in this process on the same workload; `per_config[...].cpu` holds the same for every
@@ -153,8 +153,9 @@ class Runner:
 
     def time_steps(self, step, steps, warmup):
         """Returns (wall seconds per step, event seconds per step) for exactly `steps` steps: the wall clock around
-        `steps` steps with a device synchronisation on both sides, then HIP events on the launch stream around a second
-        pass of the same `steps` steps. Two passes, because recording the two events costs about 10 us of the
+        `steps` steps with a device synchronisation on both sides, then HIP events on the launch stream around further
+        passes of the same `steps` steps (three of them, the median reported: one pass of 20 launches of 10 us now and
+        then comes out 10 % long). Separate passes, because recording the two events costs about 10 us of the
         wall-clock region (measured: 20 launches of config 0 take 193 us without and 203 us with them), which is
         instrumentation and not the workload."""
         lib = self.lib
@@ -167,14 +168,17 @@ class Runner:
         self.sync()
         t1 = time.perf_counter()
         e0, e1 = self.event(), self.event()
-        lib.nnf_hip_event_record(e0, self.stream)
-        for i in range(steps):
-            step(warmup + steps + i)
-        lib.nnf_hip_event_record(e1, self.stream)
-        self.sync()
-        ms = ctypes.c_float()
-        self.capi.check(lib.nnf_hip_event_elapsed_ms(ctypes.byref(ms), e0, e1))
-        return (t1 - t0) / steps, ms.value * 1e-3 / steps
+        event_ms = []
+        for event_pass in range(1, 4):
+            lib.nnf_hip_event_record(e0, self.stream)
+            for i in range(steps):
+                step(warmup + event_pass * steps + i)
+            lib.nnf_hip_event_record(e1, self.stream)
+            self.sync()
+            ms = ctypes.c_float()
+            self.capi.check(lib.nnf_hip_event_elapsed_ms(ctypes.byref(ms), e0, e1))
+            event_ms.append(ms.value)
+        return (t1 - t0) / steps, sorted(event_ms)[1] * 1e-3 / steps
 
 
 def time_steps_queued(runner, step, steps, hold_ms=12.0):
@@ -957,7 +961,7 @@ def main():
             # achieved and frac: HIP events on the launch stream around the steps, launched one by one by the host.
             # queued_*: the same launches queued behind a spin kernel first (where measured), so that the host's launch
             # calls are out of the picture
-            "timing": "events around a second pass of the same steps, right after the wall-clock pass",
+            "timing": "events around three further passes of the same steps, right after the wall-clock pass; the median pass",
             "queued_achieved": main_entry.get("queued_event_gbps"),
             "queued_frac": (main_entry["queued_event_gbps"] / HBM_PEAK_GBPS) if main_entry.get("queued_event_gbps") else None,
             "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
