@@ -579,9 +579,13 @@ def test_plan_of_random_networks_keeps_every_layer_once_and_in_order(seed):
         seen = [n for s in rep["steps"] for n in s["layers"]]
         assert sorted(seen) == sorted(n for n in executed if n in needed), "every needed layer exactly once"
         produced = {"in0", "in1"}
+        run_of = {}
         for s in rep["steps"]:
             assert all(i in produced for i in s["inputs"]), "a step reads only what earlier steps wrote: %s" % s
             produced.add(s["layers"][-1])
+            # groups launched together do not wait for each other
+            assert s["run"] is None or all(run_of.get(i) != s["run"] for i in s["inputs"]), "a step in one run with its producer: %s" % s
+            run_of[s["layers"][-1]] = s["run"]
             # inside a step only the last layer's value exists afterwards: nobody outside may read the others
             for inner in s["layers"][:-1]:
                 readers = [l["name"] for l in layers if inner in l["inputs"] and l["name"] in needed]
