@@ -307,7 +307,7 @@ def bench_resnet50(runner, steps, warmup, n=64, kernel_stream_count=0, one_launc
                                max_entry_count=n, kernel_stream_count=kernel_stream_count, one_launch_per_group=one_launch_per_group)
     groups = w.resnet50_groups(n)
     assert rep["timed_entries"] == n and rep["launches"] == len(groups) + 1, rep["raw"]
-    # the driver orders the steps by depth in the graph: same groups as the hand-written list, not the same order; the step
+    # the driver orders the steps into the slots of its launch plan: same groups as the hand-written list, not the same order; the step
     # of the last group also holds the average behind it
     planned = sorted((len(step["inputs"]), len(step["layers"]) - (step["layers"][-1] == "pool5")) for step in rep["steps"] if step["fused"])
     listed = sorted((len(g.arms), sum(len(a) for a in g.arms) + len(g.tail) + (len(g.arms) > 1)) for g in groups)
