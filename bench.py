@@ -142,9 +142,9 @@ class Runner:
         stream = self.stream
         desc_ref = ctypes.byref(desc)
 
-        def launch(i):
+        def launch(i, on_stream=None):
             out_ptr, in_ptrs = calls[i % sets]
-            rc = fn(stream, desc_ref, out_ptr, in_ptrs, chunk_ptrs)
+            rc = fn(stream if on_stream is None else on_stream, desc_ref, out_ptr, in_ptrs, chunk_ptrs)
             if rc != 0:
                 raise RuntimeError(capi.error_string(rc))
 
@@ -200,6 +200,33 @@ def time_steps_queued(runner, step, steps, hold_ms=12.0):
     return ms.value * 1e-3 / steps
 
 
+def time_steps_on_streams(runner, step, steps, stream_count):
+    """Wall seconds per step with the steps - each on buffers of its own, none depending on another - dealt out to
+    `stream_count` streams in turn, a device synchronisation on both sides: the end of one launch overlaps the start
+    of the next, which one stream does not allow. What independent batches can reach; reported beside the one-stream
+    figure, never as it."""
+    lib = runner.lib
+    streams = []
+    for _ in range(stream_count):
+        s = ctypes.c_void_p()
+        runner.capi.check(lib.nnf_hip_stream_create(ctypes.byref(s)))
+        streams.append(s)
+    try:
+        for i in range(2 * stream_count):
+            step(i, streams[i % stream_count])
+        runner.sync()
+        t0 = time.perf_counter()
+        for i in range(steps):
+            step(2 * stream_count + i, streams[i % stream_count])
+        runner.sync()
+        t1 = time.perf_counter()
+    finally:
+        runner.sync()
+        for s in streams:
+            lib.nnf_hip_stream_destroy(s)
+    return (t1 - t0) / steps
+
+
 def result_entry(name, alg_bytes, elements, wall_s, event_s, launches, extra=None):
     entry = {
         "workload": name,
@@ -233,6 +260,10 @@ def bench_group(runner, label, group, steps, warmup, make_input=None):
     extra = {"buffer_sets": sets, "shape": [group.entry_count, group.feature_map_count, group.plane],
              "queued_event_ms_per_step": queued * 1e3, "queued_event_gbps": alg / queued / 1e9}
     if alg <= CACHE_HOT_LIMIT_BYTES:
+        # a launch this small spends a good part of its time filling and draining the device: independent steps on two and
+        # three streams, whose ends and starts overlap (wall clock, same number of steps)
+        spread = {str(n): time_steps_on_streams(runner, launch, steps, n) for n in (2, 3)}
+        extra["independent_steps_on_streams"] = {n: {"ms_per_step": sec * 1e3, "gbps": alg / sec / 1e9} for n, sec in spread.items()}
         # the same launch on one buffer set over and over: served by the 256 MB last-level cache, not by HBM - reported beside
         # the HBM-resident figure, never as it
         del launch
