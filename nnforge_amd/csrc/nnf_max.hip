@@ -82,9 +82,16 @@ namespace nnf
 		// PROLOGUE: the staged values go through the layers of pro first, with the weights of the feature
 		// map each value belongs to (a float4 may straddle two planes when several planes that are not
 		// a multiple of four floats long share a workgroup; the host declines planes of under 4 floats).
-		template<int OP, int WIN_W, int WIN_H, bool TRUNC, bool PROLOGUE, bool EXP, bool UNIFORM>
+		// PAIR: a lane takes two neighbouring outputs of a row at a time (stride_x == 2, WIN_W 2 or 3, rows that are a
+		// multiple of four floats long and an even number of outputs per row: the host checks). The four columns
+		// both windows start in are one 16-byte LDS read, aligned; with three columns per window the fifth is one more
+		// read - two LDS reads per window row and pair instead of six, none of them with lanes two words apart (which
+		// puts two lanes on every bank), and the two results leave as one 8-byte store. Each window is still folded
+		// in the reference's order (x fastest, then y).
+		template<int OP, int WIN_W, int WIN_H, bool TRUNC, bool PROLOGUE, bool EXP, bool UNIFORM, bool PAIR = false>
 		__device__ __forceinline__ void window2d_body(const window2d_args& a, const window_prologue& pro)
 		{
+			static_assert(!PAIR || (((WIN_W == 2) || (WIN_W == 3)) && (WIN_H > 0)), "pairs of outputs: windows 2 or 3 wide, height known");
 			extern __shared__ __align__(16) float lds_in[];
 			__shared__ uint64_t lds_exp[EXP ? exp_lds_entries : 1];
 			__shared__ float lds_coef[PROLOGUE ? prologue_coef_floats : 1];
@@ -237,24 +244,27 @@ namespace nnf
 			}
 			__syncthreads();
 
-			const uint32_t outputs_per_plane = rows_here * a.out_w;
+			// A lane's unit of work: one output, or (PAIR) two neighbouring outputs of a row
+			const uint32_t units_w = PAIR ? (a.out_w >> 1) : a.out_w;
+			const uint32_t unit_stride_x = PAIR ? 2 * a.stride_x : a.stride_x;
+			const uint32_t outputs_per_plane = rows_here * units_w;
 			const uint32_t outputs_here = planes_here * outputs_per_plane;
 			float* dst = a.out + (first_plane * a.out_h + first_row) * a.out_w;
 
-			// A lane takes outputs tid, tid + 256, ... of the workgroup's run. Where its window starts - column
+			// A lane takes units tid, tid + 256, ... of the workgroup's run. Where its window starts - column
 			// x0 and row y0 of the plane, float index win of the staged copy - is worked out once with
-			// divisions and then carried from one output to the next with additions: 256 outputs further is
+			// divisions and then carried from one unit to the next with additions: 256 units further is
 			// step_p planes, step_y rows and step_x columns further, with a carry from columns into rows
 			// and from rows into planes (integer multiplications run at a quarter of the rate of additions
 			// here, and the scan, not the memory, was what bounded this kernel).
 			const uint32_t step_p = max_block_size / outputs_per_plane;
 			const uint32_t step_rest = max_block_size - step_p * outputs_per_plane;
-			const uint32_t step_y = step_rest / a.out_w;
-			const uint32_t step_x = step_rest - step_y * a.out_w;
+			const uint32_t step_y = step_rest / units_w;
+			const uint32_t step_x = step_rest - step_y * units_w;
 			const uint32_t row_floats = a.stride_y * a.in_w;        // one output row further
-			const uint32_t x_limit = a.out_w * a.stride_x;          // x0 of the column behind the last one
+			const uint32_t x_limit = units_w * unit_stride_x;       // x0 of the column behind the last one
 			const uint32_t y_limit = (first_row + rows_here) * a.stride_y;
-			const uint32_t x_advance = step_x * a.stride_x;
+			const uint32_t x_advance = step_x * unit_stride_x;
 			const uint32_t y_advance = step_y * a.stride_y;
 			const uint32_t win_advance = step_p * in_plane + step_y * row_floats + x_advance;
 			const uint32_t x_carry_win = row_floats - x_limit;                 // back to column 0, one row down
@@ -265,11 +275,19 @@ namespace nnf
 			{
 				// rows_here differs from a.rows only in the last band, where planes_here == 1 and p is 0 anyway
 				const uint32_t o = threadIdx.x;
-				const uint32_t p = (planes_here > 1) ? fast_divide(o, outputs_per_plane, a.band_magic) : 0u;
-				const uint32_t r = o - p * outputs_per_plane;
-				const uint32_t oy = fast_divide(r, a.out_w, a.out_w_magic);
-				const uint32_t ox = r - oy * a.out_w;
-				x0 = ox * a.stride_x;
+				uint32_t p, oy;
+				if (PAIR)
+				{
+					p = (planes_here > 1) ? o / outputs_per_plane : 0u;
+					oy = (o - p * outputs_per_plane) / units_w;
+				}
+				else
+				{
+					p = (planes_here > 1) ? fast_divide(o, outputs_per_plane, a.band_magic) : 0u;
+					oy = fast_divide(o - p * outputs_per_plane, a.out_w, a.out_w_magic);
+				}
+				const uint32_t ox = o - p * outputs_per_plane - oy * units_w;
+				x0 = ox * unit_stride_x;
 				y0 = (first_row + oy) * a.stride_y;
 				win = shift + p * in_plane + (y0 - in_row0) * a.in_w + x0;
 			}
@@ -283,6 +301,41 @@ namespace nnf
 				const uint32_t last_y = TRUNC ? min(win_h, a.in_h - y0) - 1 : 0u;
 				static_assert(!(TRUNC && (OP == window_op_sum)), "a truncated window re-reads values");
 				float current = window_fold_start<OP>();
+				if (PAIR)
+				{
+					// columns x0 .. x0 + 3 lie inside the row (its length is a multiple of four, as is x0); the second
+					// window's third column, x0 + 4, may not
+					uint32_t row_offset[WIN_H > 0 ? WIN_H : 1];
+					row_offset[0] = 0;
+					#pragma unroll
+					for(int y = 1; y < WIN_H; ++y)
+						row_offset[y] = TRUNC ? row_offset[y - 1] + ((static_cast<uint32_t>(y) <= last_y) ? a.in_w : 0u) : static_cast<uint32_t>(y) * a.in_w;
+					const bool fifth_inside = !TRUNC || (x0 + 4 < a.in_w);
+					float second = window_fold_start<OP>();
+					#pragma unroll
+					for(int y = 0; y < WIN_H; ++y)
+					{
+						const float* row = src + row_offset[y];
+						const floatx4 v = *reinterpret_cast<const floatx4*>(row);
+						if (WIN_W == 2)
+						{
+							current = window_fold<OP>(window_fold<OP>(current, v.x), v.y);
+							second = window_fold<OP>(window_fold<OP>(second, v.z), v.w);
+						}
+						else
+						{
+							const float fifth = fifth_inside ? row[4] : v.w;
+							current = window_fold<OP>(window_fold<OP>(window_fold<OP>(current, v.x), v.y), v.z);
+							second = window_fold<OP>(window_fold<OP>(window_fold<OP>(second, v.z), v.w), fifth);
+						}
+					}
+					float2 both;
+					both.x = (OP == window_op_sum) ? current * a.mult : current;
+					both.y = (OP == window_op_sum) ? second * a.mult : second;
+					*reinterpret_cast<float2*>(dst + 2 * o) = both;
+				}
+				else
+				{
 				if ((WIN_W > 0) && (WIN_H > 0))
 				{
 					// min(y, last_y) * in_w and min(x, last_x) without multiplications
@@ -313,8 +366,9 @@ namespace nnf
 							current = window_fold<OP>(current, row[x]);
 				}
 				dst[o] = (OP == window_op_sum) ? current * a.mult : current;
+				}
 
-				// 256 outputs further
+				// 256 units further
 				x0 += x_advance;
 				y0 += y_advance;
 				win += win_advance;
@@ -332,20 +386,20 @@ namespace nnf
 			}
 		}
 
-		template<int OP, int WIN_W, int WIN_H, bool TRUNC>
+		template<int OP, int WIN_W, int WIN_H, bool TRUNC, bool PAIR = false>
 		__global__ void __launch_bounds__(max_block_size) max_window2d_kernel(const window2d_args a)
 		{
 			window_prologue none; // not read
-			window2d_body<OP, WIN_W, WIN_H, TRUNC, false, false, false>(a, none);
+			window2d_body<OP, WIN_W, WIN_H, TRUNC, false, false, false, PAIR>(a, none);
 		}
 
 		// UNIFORM: one plane per workgroup (a.planes == 1). Without expf the layers fit 96 registers per lane,
 		// which lets a compute unit hold five workgroups instead of four (measured: 10 % faster); with expf
 		// that would spill.
-		template<int OP, int WIN_W, int WIN_H, bool TRUNC, bool UNIFORM>
+		template<int OP, int WIN_W, int WIN_H, bool TRUNC, bool UNIFORM, bool PAIR = false>
 		__global__ void __launch_bounds__(max_block_size) __attribute__((amdgpu_waves_per_eu(5, 5))) max_window2d_prologue_kernel(const window2d_args a, const window_prologue pro)
 		{
-			window2d_body<OP, WIN_W, WIN_H, TRUNC, true, false, UNIFORM>(a, pro);
+			window2d_body<OP, WIN_W, WIN_H, TRUNC, true, false, UNIFORM, PAIR>(a, pro);
 		}
 
 		template<int OP, int WIN_W, int WIN_H, bool TRUNC, bool UNIFORM>
@@ -727,6 +781,13 @@ namespace nnf
 			return (pa < pb + b_bytes) && (pb < pa + a_bytes);
 		}
 
+		// Shapes the kernels take two outputs per lane at a time for (window2d_body's PAIR): every staged row starts on
+		// a 16-byte boundary of LDS and holds whole float4s, and a row's outputs pair up.
+		bool pairs_of_outputs(const window2d_args& a)
+		{
+			return (a.stride_x == 2) && ((a.in_w % 4) == 0) && ((a.out_w % 2) == 0) && (a.out_w >= 2);
+		}
+
 		template<int OP, bool TRUNC, bool UNIFORM>
 		void launch_window2d_prologue(hipStream_t stream, const window2d_args& a, uint32_t grid, size_t lds_bytes, const window_prologue& pro)
 		{
@@ -740,7 +801,10 @@ namespace nnf
 			}
 			else
 			{
-				if (w3) hipLaunchKernelGGL((max_window2d_prologue_kernel<OP, 3, 3, TRUNC, UNIFORM>), g, b, lds_bytes, stream, a, pro);
+				const bool pair = pairs_of_outputs(a);
+				if (w3 && pair) hipLaunchKernelGGL((max_window2d_prologue_kernel<OP, 3, 3, TRUNC, UNIFORM, true>), g, b, lds_bytes, stream, a, pro);
+				else if (w2 && pair) hipLaunchKernelGGL((max_window2d_prologue_kernel<OP, 2, 2, TRUNC, UNIFORM, true>), g, b, lds_bytes, stream, a, pro);
+				else if (w3) hipLaunchKernelGGL((max_window2d_prologue_kernel<OP, 3, 3, TRUNC, UNIFORM>), g, b, lds_bytes, stream, a, pro);
 				else if (w2) hipLaunchKernelGGL((max_window2d_prologue_kernel<OP, 2, 2, TRUNC, UNIFORM>), g, b, lds_bytes, stream, a, pro);
 				else hipLaunchKernelGGL((max_window2d_prologue_kernel<OP, 0, 0, TRUNC, UNIFORM>), g, b, lds_bytes, stream, a, pro);
 			}
@@ -757,7 +821,12 @@ namespace nnf
 					launch_window2d_prologue<OP, TRUNC, false>(stream, a, grid, lds_bytes, *pro);
 				return;
 			}
-			if ((a.win_w == 3) && (a.win_h == 3))
+			const bool pair = pairs_of_outputs(a);
+			if ((a.win_w == 3) && (a.win_h == 3) && pair)
+				hipLaunchKernelGGL((max_window2d_kernel<OP, 3, 3, TRUNC, true>), dim3(grid), dim3(max_block_size), lds_bytes, stream, a);
+			else if ((a.win_w == 2) && (a.win_h == 2) && pair)
+				hipLaunchKernelGGL((max_window2d_kernel<OP, 2, 2, TRUNC, true>), dim3(grid), dim3(max_block_size), lds_bytes, stream, a);
+			else if ((a.win_w == 3) && (a.win_h == 3))
 				hipLaunchKernelGGL((max_window2d_kernel<OP, 3, 3, TRUNC>), dim3(grid), dim3(max_block_size), lds_bytes, stream, a);
 			else if ((a.win_w == 2) && (a.win_h == 2))
 				hipLaunchKernelGGL((max_window2d_kernel<OP, 2, 2, TRUNC>), dim3(grid), dim3(max_block_size), lds_bytes, stream, a);

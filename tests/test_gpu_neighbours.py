@@ -138,6 +138,9 @@ POOL_CASES = [
     ((8, 96, 55, 55), [3, 3], [2, 2], None),                 # AlexNet-style overlapping pooling
     ((16, 32, 28, 28), [2, 2], None, None),                  # whole planes per workgroup
     ((7, 5, 13, 13), [3, 3], [2, 2], [True, True]),          # many small planes per workgroup, odd counts
+    ((6, 5, 10, 12), [3, 3], [2, 2], [True, True]),          # ... with rows of whole float4s: two outputs per lane at a time, the last pair's window cut off
+    ((3, 7, 9, 8), [2, 2], None, None),                      # ... 2x2 windows, an input row left over
+    ((2, 3, 6, 16), [3, 3], [2, 2], [True, False]),          # rounded up in x only
     ((3, 3, 9, 31), [5, 2], [3, 1], [True, False]),          # run-time window sizes
     ((2, 2, 300, 200), [4, 7], [4, 5], None),                # bands of a large plane
     ((2, 3, 4, 4000), [3, 2], [2, 2], None),                 # very wide rows: one output row per band
@@ -304,6 +307,8 @@ FUSED_MAX_CASES = [
     ((8, 96, 55, 55), [3, 3], [2, 2], None, "bn_relu"),                # planes of 3025 floats, several per workgroup
     ((16, 32, 28, 28), [2, 2], None, None, "tanh_abs"),                # several planes per workgroup
     ((9, 3, 12, 12), [2, 2], None, None, "bn_prelu_elu_sigmoid"),      # more planes per workgroup than feature maps
+    ((6, 5, 10, 12), [3, 3], [2, 2], [True, True], "bn_relu"),         # two outputs per lane at a time, small planes
+    ((2, 4, 57, 56), [3, 3], [2, 2], [True, True], "prelu_bn"),        # ... a plane per workgroup
     ((5, 7, 6, 10), [3, 2], [2, 2], [True, False], "bn_relu"),         # run-time window, odd plane counts
     ((6, 10, 7, 7), [3, 3], [2, 2], None, "bn_prelu_elu_sigmoid"),     # planes of 49 floats: float4s straddle planes
     ((4, 3, 13, 13), [3, 3], [2, 2], [True, True], "bn_relu"),         # ... with more planes per workgroup than feature maps
