@@ -551,18 +551,32 @@ namespace nnf
 			}
 			__syncthreads();
 
-			const uint32_t positions_per_plane = (oy1 - oy0) * a.out_w;
+			const uint32_t rows_here = oy1 - oy0;
+			const uint32_t positions_per_plane = rows_here * a.out_w;
 			const uint32_t positions = planes_here * positions_per_plane;
 			const size_t grid_stride = static_cast<size_t>(a.fm_count) * out_plane; // from one output entry to the next
+			// A lane takes positions tid, tid + 256, ...: plane, row and column of the first one by division, the following
+			// ones by addition with carries (256 positions further is step_p planes, step_y rows and step_x columns further)
+			// instead of three integer divisions per position.
+			const uint32_t step_p = max_block_size / positions_per_plane;
+			const uint32_t step_rest = max_block_size - step_p * positions_per_plane;
+			const uint32_t step_y = step_rest / a.out_w;
+			const uint32_t step_x = step_rest - step_y * a.out_w;
+			uint32_t p = (planes_here > 1) ? threadIdx.x / positions_per_plane : 0u;
+			uint32_t oy = (threadIdx.x - p * positions_per_plane) / a.out_w;
+			uint32_t ox = threadIdx.x - p * positions_per_plane - oy * a.out_w;
+			// a band: one plane for the whole workgroup
+			const uint32_t band_entry = first_plane / a.fm_count;
+			const uint32_t band_fm = first_plane - band_entry * a.fm_count;
 			for(uint32_t pos = threadIdx.x; pos < positions; pos += max_block_size)
 			{
-				const uint32_t p = pos / positions_per_plane;
-				const uint32_t rem = pos - p * positions_per_plane;
-				const uint32_t oy = rem / a.out_w;
-				const uint32_t ox = rem - oy * a.out_w;
-				const uint32_t plane_id = first_plane + p;
-				const uint32_t entry = plane_id / a.fm_count;
-				const uint32_t fm = plane_id - entry * a.fm_count;
+				uint32_t entry = band_entry, fm = band_fm;
+				if (planes_here > 1)
+				{
+					const uint32_t plane_id = first_plane + p;
+					entry = plane_id / a.fm_count;
+					fm = plane_id - entry * a.fm_count;
+				}
 				const float* corner = staged + p * in_plane + oy * win_h * a.in_w + ox * win_w;
 				float* dst = a.out + (static_cast<size_t>(entry) * (win_w * win_h) * a.fm_count + fm) * out_plane + (oy0 + oy) * a.out_w + ox;
 				// grids in the order of the window scan: x shift fastest
@@ -583,6 +597,20 @@ namespace nnf
 						*dst = current;
 						dst += grid_stride;
 					}
+				}
+				// 256 positions further
+				ox += step_x;
+				oy += step_y;
+				p += step_p;
+				if (ox >= a.out_w)
+				{
+					ox -= a.out_w;
+					++oy;
+				}
+				if (oy >= rows_here)
+				{
+					oy -= rows_here;
+					++p;
 				}
 			}
 		}
