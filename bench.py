@@ -43,7 +43,7 @@ MEASURED_TRAFFIC_BYTES = {
     "config1": 2117540,     # algorithmic 2,048,000 (profiles/softmax_and_resnet50_stack.md)
     "max_subsampling_tiling": 402617602,  # algorithmic 403,767,296 (profiles/tiling_and_entry_window_kernels.md)
     "entry_window": 256931085,            # algorithmic 256,901,120
-    "config4": 6313457776,  # per pass of the launch plan through the driver (50 plan steps in 8 kernel launches: independent groups
+    "config4": 6313391834,  # per pass of the launch plan through the driver (50 plan steps in 8 kernel launches: independent groups
                             # share launches, the last group is applied by the average's kernel and neither written nor read
                             # back), algorithmic 6,359,339,008 (profiles/chain_batch_kernel_config4_through_driver.md)
     "config4_direct": 6370619861,  # per step = the 51 launches of a pass (profiles/softmax_and_resnet50_stack.md)

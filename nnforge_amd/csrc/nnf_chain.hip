@@ -536,8 +536,10 @@ namespace nnf
 				chain_tile<NIN, BLOCK, U, false, 0>(b.group[g], tile_index, lds_raw);
 		}
 
-		// Groups with one input (four float4s per lane) and groups with two (two float4s per lane) in one launch: the
-		// tiles differ in size, the workgroups do not (BLOCK lanes), and a workgroup takes the body of its group's kind.
+		// Groups with one input (four float4s per lane; two where the weights go through LDS coefficients, which keeps
+		// the kernel at 60 registers per lane, eight wavefronts per SIMD) and groups with two (two float4s per lane) in one
+		// launch: the tiles differ in size, the workgroups do not (BLOCK lanes), and a workgroup takes the body of its
+		// group's kind.
 		// What this buys: the groups of a residual network that wait for each other (the joins of a stage) are few
 		// per level of the graph, and each level can take a share of the groups that wait for nothing along, instead of
 		// being a small launch of its own.
@@ -562,7 +564,7 @@ namespace nnf
 				if (direct)
 					chain_tile<1, BLOCK, 4, true, 0>(b.group[g], tile_index, lds_raw);
 				else
-					chain_tile<1, BLOCK, 4, false, 0>(b.group[g], tile_index, lds_raw);
+					chain_tile<1, BLOCK, 2, false, 0>(b.group[g], tile_index, lds_raw);
 			}
 		}
 
@@ -959,6 +961,10 @@ namespace nnf
 			}
 			if ((program > 0) && (shape == 0))
 				shape = 1; // the compile-time programs have no four-float4 instance (smaller tile: LDS still fits)
+			// as one of several groups of a launch, a group with one input whose weights go through LDS coefficients takes
+			// two float4s per lane: the body chain_batch_mixed_kernel has for it
+			if (automatic && !single_launch && (desc->input_count == 1) && (shape == 0) && !direct_of(0))
+				shape = 1;
 			// One input, four float4s per lane, and more tiles than the device holds workgroups at once (8 per compute
 			// unit: above 33 MB per tensor): a second, partial round of workgroups would follow the first and the time per
 			// byte jumps (32 MB: 11.0 us, 38.5 MB: 15.5 us). There the grid that stays put takes over, five workgroups
@@ -1057,7 +1063,7 @@ namespace nnf
 		// the two kinds of group chain_batch_mixed_kernel takes side by side
 		bool mixes(const prepared_group& g)
 		{
-			return ((g.input_count == 1) && (g.shape == 0)) || ((g.input_count == 2) && (g.shape == 1));
+			return ((g.input_count == 1) && (g.shape == (g.direct ? 0 : 1))) || ((g.input_count == 2) && (g.shape == 1));
 		}
 
 		chain_batch_kernel_fn pick_batch_kernel(uint32_t input_count, int shape, int direct_mode)
@@ -1127,6 +1133,7 @@ namespace nnf
 			// the groups behind it that can share its kernel instance, max_batch to a launch; the compile-time
 			// expf programs are bound by the vector ALU, not by launches: they keep their own kernels
 			std::vector<uint32_t> members(1, first);
+			bool one_kind = true; // all members share the lead's number of inputs and tile size
 			if ((lead.program == 0) && (lead.a.slot_count <= static_cast<uint32_t>(batch_slots)))
 				for(uint32_t j = first + 1; (j < group_count) && (members.size() < max_batch); ++j)
 				{
@@ -1137,6 +1144,7 @@ namespace nnf
 					{
 						members.push_back(j);
 						launched[j] = true;
+						one_kind = one_kind && same_kind;
 					}
 				}
 			if (members.size() == 1)
@@ -1164,7 +1172,6 @@ namespace nnf
 				return NNF_HIP_ETOOBIG;
 			const uint32_t all_groups = (1u << b.count) - 1u;
 			const int direct_mode = (b.direct_mask == all_groups) ? 1 : ((b.direct_mask == 0) ? 0 : 2);
-			const bool one_kind = (b.two_input_mask == 0) || (b.two_input_mask == all_groups) || !mixes(lead);
 			const chain_batch_kernel_fn kernel = one_kind ? pick_batch_kernel(lead.input_count, lead.shape, direct_mode) : pick_batch_mixed_kernel(direct_mode);
 			hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>(tiles)), dim3(launch_shapes[lead.shape].block), lds_bytes, stream, b);
 			const int rc = launch_status();
