@@ -235,7 +235,7 @@ namespace nnf
 		// coefficients and every value picks its own. JOIN: two inputs, each through its own layers, summed by the
 		// group's Add, the layers behind it applied to the sum.
 		// Measured on 64 x 2048 x 7 x 7 (25.7 MB): 6.2 us against 8.9 us for the kernel above; 64 planes per wavefront 6.8 us,
-		// all thirteen float4s of a lane loaded before the first LDS store 9.0 us. With BatchNorm + ReLU folded in 8.9 us, with a
+		// all thirteen float4s of a lane loaded before the first LDS store 9.0 us (all seven of 32 planes: 6.3 us, no change). With BatchNorm + ReLU folded in 8.9 us, with a
 		// joined block 14.0 us (16 planes per wavefront: 9.8 and 14.5 us; 64: 10.3 and 13.2 us).
 		constexpr uint32_t linear_planes_per_wave = 32;
 		constexpr int linear_waves = 4;
