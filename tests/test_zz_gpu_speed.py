@@ -2,7 +2,8 @@
 slower while it still computes the right bits - a load loop that serialises, a launch shape that leaves the machine empty.
 Every bound is a ratio: the kernel's time against the library's plain copy kernel moving the same number of bytes, timed in
 the same test on the same machine, with the launches of both queued behind a spin kernel so that neither the machine's
-clocks of the day nor the host's launch calls enter. Today's ratios are between 0.9 and 1.3 (the expf chain: 1.7)."""
+clocks of the day nor the host's launch calls enter. Today's ratios are between 0.9 and 1.3 (the expf chain: 1.7). The last test
+bounds the driver's launch plan the same way: against the same network with one launch per group."""
 
 import ctypes
 
@@ -171,3 +172,35 @@ def test_tiling_and_entry_windows_stay_on_their_own_kernels(gpu):
         assert rc == 0, capi.error_string(rc)
 
     assert_ratio(gpu, "the average over 4 entries", time_launches(gpu, entry_window, reps=30, warmup=3), 4 * (n * c * size * size * 5 // 4), 1.8, reps=30)
+
+
+def test_groups_launched_together_stay_ahead_of_one_launch_per_group(gpu):
+    """The ResNet-50 post-convolution stack through the driver at 8 entries per packet, where launches are what a pass
+    costs: the default plan (8 kernel launches for 50 steps) against one launch per group on one stream, both timed by the
+    driver on the same resident packet. Today's ratio is 1.5; a plan that fell back to a launch per group, or runs that
+    ended early, would bring it to 1."""
+    from nnforge_amd import backend, schemas
+
+    gen = np.random.Generator(np.random.MT19937(91))
+    layers, configs, outputs = schemas.resnet50_post_convolution()
+    weights = {}
+    for l in layers:
+        if l["type"] == "BatchNorm":
+            c = l["params"]["feature_map_count"]
+            weights[l["name"]] = [gen.random(c, dtype=np.float32) + np.float32(0.5), gen.standard_normal(c, dtype=np.float32) * np.float32(0.3),
+                                  gen.standard_normal(c, dtype=np.float32) * np.float32(0.3), gen.random(c, dtype=np.float32) + np.float32(0.6)]
+    text = schemas.schema_text(layers, "ResNet-50 post-convolution")
+    n = 8
+    largest = max(fm * dims[0] * dims[1] for fm, dims in configs.values())
+    pool = gen.standard_normal(n * largest, dtype=np.float32)
+
+    def seconds(**options):
+        rep = backend.time_kernels(text, weights, configs, outputs, warmup=3, passes=20, shared_input_pool=pool, entry_count=n, max_entry_count=n, **options)
+        assert rep["timed_entries"] == n
+        return rep["device_seconds_per_pass"], rep
+
+    together, rep = seconds()
+    one_by_one, _ = seconds(one_launch_per_group=True, kernel_stream_count=1)
+    runs = {s["run"] for s in rep["steps"] if s["run"] is not None}
+    assert len(runs) == 6, "the stack's groups in six runs, as many as its longest chain of blocks"
+    assert one_by_one > 1.25 * together, "groups launched together: %.1f us per pass, one launch per group: %.1f us" % (together * 1e6, one_by_one * 1e6)
