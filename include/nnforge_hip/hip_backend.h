@@ -286,6 +286,7 @@ namespace nnforge
 				unsigned int launch_count;     // launches per pass
 				float wall_seconds_per_pass;
 				float device_seconds_per_pass; // from events on the kernel stream
+				float host_seconds_per_pass;   // what the calling thread spends enqueuing a pass (the device runs behind it)
 			};
 			kernel_timing time_kernels(structured_data_bunch_reader& reader, unsigned int entry_count, unsigned int warmup, unsigned int passes);
 

@@ -128,8 +128,9 @@ NNF_BACKEND_API int nnf_backend_update_bn_weights(
 /* Times the launch plan of the schema alone, on one packet of entry_count entries that stays in device memory
  * (forward_propagation_hip::time_kernels): uploaded once, then `warmup` untimed and `passes` timed runs of the plan,
  * nothing copied back. The report lists the plan like nnf_backend_run_schema, then "launches: N", "timed_entries: N",
- * "wall_seconds_per_pass: S" (device synchronisation on both sides of the timed passes) and
- * "device_seconds_per_pass: S" (events on the kernel stream). Inputs whose data pointers are equal are fine: the
+ * "wall_seconds_per_pass: S" (device synchronisation on both sides of the timed passes),
+ * "device_seconds_per_pass: S" (events on the kernel stream) and "host_seconds_per_pass: S" (what the calling thread
+ * spends enqueuing a pass while the device runs behind it). Inputs whose data pointers are equal are fine: the
  * values do not matter for the time. */
 NNF_BACKEND_API int nnf_backend_time_kernels(
 	const char* schema_text,

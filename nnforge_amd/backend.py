@@ -156,7 +156,7 @@ def parse_report(text):
                                  "run": int(run) if run else None})
         elif key in ("per_entry_bytes", "max_entry_count", "entries", "writer_entries", "launches", "timed_entries"):
             res[key] = int(rest)
-        elif key in ("wall_seconds_per_pass", "device_seconds_per_pass"):
+        elif key in ("wall_seconds_per_pass", "device_seconds_per_pass", "host_seconds_per_pass"):
             res[key] = float(rest)
         elif key == "seconds":
             name, _, sec = rest.rpartition(" ")

@@ -480,6 +480,7 @@ extern "C"
 			out.precision(9);
 			out << "wall_seconds_per_pass: " << t.wall_seconds_per_pass << "\n";
 			out << "device_seconds_per_pass: " << t.device_seconds_per_pass << "\n";
+			out << "host_seconds_per_pass: " << t.host_seconds_per_pass << "\n";
 		}, report, report_capacity);
 	}
 

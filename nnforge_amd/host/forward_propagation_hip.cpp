@@ -1389,6 +1389,7 @@ namespace nnforge
 			for(unsigned int i = 0; i < passes; ++i)
 				one_pass();
 			hip_safe_call(nnf_hip_event_record(stop.ev, p->stream));
+			const std::chrono::duration<float> enqueued = std::chrono::high_resolution_clock::now() - t0;
 			hip_safe_call(nnf_hip_device_synchronize());
 			const std::chrono::duration<float> wall = std::chrono::high_resolution_clock::now() - t0;
 			float ms = 0.0F;
@@ -1396,6 +1397,7 @@ namespace nnforge
 			const float n = static_cast<float>(std::max(1U, passes));
 			res.wall_seconds_per_pass = wall.count() / n;
 			res.device_seconds_per_pass = ms * 1.0e-3F / n;
+			res.host_seconds_per_pass = enqueued.count() / n;
 			return res;
 		}
 
