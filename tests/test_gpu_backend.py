@@ -402,6 +402,34 @@ def test_resnet50_post_convolution_graph_layer_by_layer(mode):
             assert_bits(got[name], values[name], name)
 
 
+def test_resnet50_post_convolution_graph_at_64_entries():
+    """Config 4 at its full size through the driver, one packet of 64 entries, the default launch plan (six runs of
+    groups launched together, tiles of every ResNet-50 shape by the hundred thousand per launch): every output against
+    the oracle run layer by layer, bit for bit (softmax to 1e-5). Inputs are cut out of one pool of normal values at
+    offsets of their own (what is compared is arithmetic and indexing, not statistics)."""
+    from nnforge_amd import schemas
+
+    gen = T.rng(62, 64)
+    n = 64
+    layers, configs, outputs = schemas.resnet50_post_convolution()
+    weights = S.make_weights(layers, gen)
+    pool = T.normal(gen, 1 << 25, 1.5)
+    inputs = {}
+    for i, (name, (fm, dims)) in enumerate(sorted(configs.items())):
+        count = n * fm * dims[0] * dims[1]
+        start = (7919 * (i + 1)) % 65536
+        inputs[name] = np.resize(pool[start:], count).reshape(n, fm, dims[1], dims[0])
+    values = S.evaluate(layers, weights, inputs)
+    got, rep = run(layers, weights, inputs, outputs, values, max_entry_count=n)
+    assert rep["entries"] == n and rep["max_entry_count"] == n and len(rep["steps"]) == 50
+    assert len({s["run"] for s in rep["steps"]} - {None}) == 6
+    for name in outputs:
+        if name == "prob":
+            assert np.all(np.abs(got[name] - values[name]) <= 1e-5 * np.abs(values[name])), name
+        else:
+            assert_bits(got[name], values[name], name)
+
+
 def test_dropout_only_network():
     """Dropout straight from the data layer to the output: in place there is nothing to launch."""
     gen = T.rng(58, 0)
