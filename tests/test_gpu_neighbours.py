@@ -135,6 +135,7 @@ POOL_CASES = [
     # shape, windows (x first), strides, round_ups
     ((32, 64, 112, 112), [3, 3], [2, 2], None),              # ResNet pool1 as nnForge computes it: 55x55
     ((4, 64, 112, 112), [3, 3], [2, 2], [True, True]),       # 56x56, the last window cut off
+    ((64, 64, 112, 112), [3, 3], [2, 2], [True, True]),      # ... at the size of the ResNet-50 stem with 64 entries
     ((8, 96, 55, 55), [3, 3], [2, 2], None),                 # AlexNet-style overlapping pooling
     ((16, 32, 28, 28), [2, 2], None, None),                  # whole planes per workgroup
     ((7, 5, 13, 13), [3, 3], [2, 2], [True, True]),          # many small planes per workgroup, odd counts
@@ -303,6 +304,7 @@ def prologue_input(gen, shape):
 FUSED_MAX_CASES = [
     # shape, windows (x first), strides, round_ups, group
     ((4, 64, 112, 112), [3, 3], [2, 2], [True, True], "bn_relu"),       # ResNet stem: bands of a plane per workgroup
+    ((64, 64, 112, 112), [3, 3], [2, 2], [True, True], "bn_relu"),      # ... with 64 entries
     ((2, 6, 112, 112), [3, 3], [2, 2], None, "bn_prelu_elu_sigmoid"),
     ((8, 96, 55, 55), [3, 3], [2, 2], None, "bn_relu"),                # planes of 3025 floats, several per workgroup
     ((16, 32, 28, 28), [2, 2], None, None, "tanh_abs"),                # several planes per workgroup
@@ -417,6 +419,7 @@ def test_average_subsampling_with_group_folded_in(gpu, shape, ww, wh, group):
 JOINED_POOL_CASES = [
     # shape, arms ("bn": BatchNorm, "-": nothing, "leaky": ReLU 0.1, "elu"), alpha, tail
     ((64, 128, 7, 7), ("-", "bn"), 1.0, "relu"),        # residual + BatchNorm(main) -> Add -> ReLU: the last block of a ResNet
+    ((64, 2048, 7, 7), ("-", "bn"), 1.0, "relu"),       # ... at ResNet-50's size with 64 entries
     ((5, 24, 7, 7), ("bn", "bn"), 1.0, "relu"),         # BatchNorm on both arms (a block with a projection shortcut)
     ((3, 5, 7, 7), ("bn", "elu"), 0.5, "sigmoid"),      # 15 planes in the last workgroup, three floats behind the last float4
     ((9, 70, 8, 8), ("leaky", "-"), 2.0, "none"),       # planes that are multiples of 4 floats, nothing behind the Add
