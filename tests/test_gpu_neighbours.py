@@ -102,6 +102,7 @@ def run_maxout(gpu, x, k, expect=0):
 
 @pytest.mark.parametrize("shape,k", [
     ((32, 256, 14, 14), 2),
+    ((64, 512, 14, 14), 2),    # the benchmark's shape
     ((8, 96, 7, 7), 3),        # group 32*49 is a multiple of 4
     ((5, 15, 3, 3), 5),        # scalar path
     ((1, 2, 1), 2),
@@ -184,6 +185,7 @@ TILING_CASES = [
     ((7, 37, 6, 5), [2, 2]),              # 259 small planes: 256 in the first workgroup, 3 in the second
     ((1, 2, 200, 300), [3, 2]),           # bands of a large plane
     ((2, 3, 112, 112), [3, 3]),           # a whole plane per workgroup
+    ((64, 64, 112, 112), [2, 2]),         # the benchmark's shape: 256 output entries of 55 x 55
     ((2, 1, 5, 20000), [2, 2]),           # rows too wide to stage: one lane per output
     ((3, 2, 40000), [3]),                 # 1-D, wide
 ]
