@@ -2,6 +2,8 @@
 host tensors go in through factory_generator_hip -> forward_propagation_hip; the outputs must equal
 the CPU oracle run layer by layer the way the plain backend drives its testers."""
 
+import os
+
 import numpy as np
 import pytest
 
@@ -255,7 +257,11 @@ def test_groups_folded_into_the_subsampling_layers_behind_them(fuse, size):
         assert len(names) == 8
 
 
-@pytest.mark.parametrize("seed", list(range(12)) + [-s for s in range(1, 13)])
+# NNF_EXHAUSTIVE=1: 395 more networks (a few seconds on the device)
+MORE_NETWORK_SEEDS = (list(range(12, 260)) + [-s for s in range(13, 160)]) if os.environ.get("NNF_EXHAUSTIVE") == "1" else []
+
+
+@pytest.mark.parametrize("seed", list(range(12)) + [-s for s in range(1, 13)] + MORE_NETWORK_SEEDS)
 def test_random_networks_equal_the_oracle_layer_by_layer(seed):
     """Random DAGs of every layer type the backend runs (the generator of the planner tests), in packets, with
     fusion and buffer sharing on: every output equals the oracle run layer by layer, bit for bit; the same

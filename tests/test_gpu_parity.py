@@ -7,6 +7,7 @@ kernel except the row softmax, whose sum is a tree instead of a left-to-right lo
 """
 
 import ctypes
+import os
 
 import numpy as np
 import pytest
@@ -427,7 +428,8 @@ def random_group(seed, allow_exp=True):
     return (n, c, plane), arms, tail, inputs, chunks, has_add, alpha, want
 
 
-@pytest.mark.parametrize("seed", range(40))
+# NNF_EXHAUSTIVE=1: 360 more groups
+@pytest.mark.parametrize("seed", range(400 if os.environ.get("NNF_EXHAUSTIVE") == "1" else 40))
 def test_random_groups_equal_the_layers_one_by_one(gpu, seed):
     """Random groups against the oracle run layer by layer, bit for bit."""
     shape3, arms, tail, inputs, chunks, has_add, alpha, want = random_group(seed)
