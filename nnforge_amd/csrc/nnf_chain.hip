@@ -692,26 +692,6 @@ namespace nnf
 			return chain_kernel_persistent<1, 256, 4>; // one input only: see persistent_max_inputs
 		}
 
-		// compute units of the current device (asked once per device)
-		uint32_t compute_unit_count()
-		{
-			constexpr int max_devices = 64;
-			static std::atomic<uint32_t> known[max_devices];
-			int device = 0;
-			if ((hipGetDevice(&device) != hipSuccess) || (device < 0) || (device >= max_devices))
-				return 256;
-			uint32_t count = known[device].load(std::memory_order_relaxed);
-			if (count == 0)
-			{
-				int value = 0;
-				if ((hipDeviceGetAttribute(&value, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess) || (value <= 0))
-					value = 256;
-				count = static_cast<uint32_t>(value);
-				known[device].store(count, std::memory_order_relaxed);
-			}
-			return count;
-		}
-
 		// index into known_programs of a single-input group without Add, 0 when it is not one of them
 		int match_known_program(const nnf_hip_chain_desc& desc, uint32_t op_count)
 		{

@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "../../include/nnforge_hip.h"
 #include "nnf_math.h"
 
@@ -81,6 +83,26 @@ namespace nnf
 	inline int hip_status(hipError_t e)
 	{
 		return static_cast<int>(e);
+	}
+
+	// compute units of the current device (asked once per device)
+	inline uint32_t compute_unit_count()
+	{
+		constexpr int max_devices = 64;
+		static std::atomic<uint32_t> known[max_devices];
+		int device = 0;
+		if ((hipGetDevice(&device) != hipSuccess) || (device < 0) || (device >= max_devices))
+			return 256;
+		uint32_t count = known[device].load(std::memory_order_relaxed);
+		if (count == 0)
+		{
+			int value = 0;
+			if ((hipDeviceGetAttribute(&value, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess) || (value <= 0))
+				value = 256;
+			count = static_cast<uint32_t>(value);
+			known[device].store(count, std::memory_order_relaxed);
+		}
+		return count;
 	}
 
 	// Launch errors are reported by hipGetLastError right after the launch; asynchronous faults

@@ -2,8 +2,10 @@
 //
 // Both reference testers fold the values of a window in a fixed order with std::max / std::min,
 // whose result for equal values (+0.0 and -0.0) and for NaN depends on the argument order, and
-// max subsampling starts the fold at -1.0e37F / 1.0e37F. The kernels keep the order, the argument
-// order and the start value, so results equal the reference's bit for bit:
+// max subsampling starts the fold at -1.0e37F / 1.0e37F. The kernels' results equal the reference's bit
+// for bit: the staged 2-D kernels take the hardware's maximum of a window and fold it again in the
+// reference's order where only that order decides (a result of zero), the others keep the order, the
+// argument order and the start value throughout:
 //   nnforge/plain/max_subsampling_layer_tester_plain.cpp:175-290  std::max<float>(current, new), x fastest
 //   nnforge/plain/maxout_layer_tester_plain.cpp:56-80             std::max(new, current), starts at the first value
 #include "nnf_common.h"
@@ -49,6 +51,106 @@ namespace nnf
 			if (OP == window_op_sum)
 				return 0.0f;
 			return (OP == window_op_min) ? 1.0e37f : -1.0e37f;
+		}
+
+		// ---- the hardware's maximum / minimum, with the reference's result ------------------------
+		// std::max<float>(current, new) from a finite start value never holds a NaN (current < NaN is false), so a
+		// window's result is the largest of the start value and the window's numbers - whatever the order of
+		// the fold - with one exception: when that largest value is a zero, the fold keeps the first zero it met,
+		// -0.0 or +0.0, while v_max_f32 ranks +0.0 above -0.0. The kernels therefore fold with v_max3_f32 /
+		// v_min3_f32 (two values per instruction instead of a compare and a select per value) and a lane whose
+		// result is a zero folds its window again the reference's way. v_max_f32 passes over a quiet NaN operand but
+		// answers a signalling one with a NaN, which the next fold would then pass over together with everything
+		// folded so far: the values are made quiet (canonical) once, on their way into LDS.
+		__device__ __forceinline__ float quiet(float v)
+		{
+			return __builtin_canonicalizef(v);
+		}
+
+		__device__ __forceinline__ floatx4 quiet(floatx4 v)
+		{
+			floatx4 q;
+			q.x = quiet(v.x); q.y = quiet(v.y); q.z = quiet(v.z); q.w = quiet(v.w);
+			return q;
+		}
+
+		template<bool IS_MIN>
+		__device__ __forceinline__ float hw_fold(float a, float b)
+		{
+			float d;
+			if (IS_MIN)
+				asm("v_min_f32 %0, %1, %2" : "=v"(d) : "v"(a), "v"(b));
+			else
+				asm("v_max_f32 %0, %1, %2" : "=v"(d) : "v"(a), "v"(b));
+			return d;
+		}
+
+		template<bool IS_MIN>
+		__device__ __forceinline__ float hw_fold3(float a, float b, float c)
+		{
+			float d;
+			if (IS_MIN)
+				asm("v_min3_f32 %0, %1, %2, %3" : "=v"(d) : "v"(a), "v"(b), "v"(c));
+			else
+				asm("v_max3_f32 %0, %1, %2, %3" : "=v"(d) : "v"(a), "v"(b), "v"(c));
+			return d;
+		}
+
+		// The largest (smallest) of the start value and COUNT quiet values: the window's result, unless it is a zero.
+		template<int OP, int COUNT>
+		__device__ __forceinline__ float fold_values_hw(const float (&v)[COUNT])
+		{
+			constexpr bool is_min = (OP == window_op_min);
+			float current = window_fold_start<OP>();
+			#pragma unroll
+			for(int i = 0; i + 1 < COUNT; i += 2)
+				current = hw_fold3<is_min>(current, v[i], v[i + 1]);
+			if (COUNT % 2 != 0)
+				current = hw_fold<is_min>(current, v[COUNT - 1]);
+			return current;
+		}
+
+		// The reference's fold of COUNT values in the order given.
+		template<int OP, int COUNT>
+		__device__ __forceinline__ float fold_values_in_order(const float (&v)[COUNT])
+		{
+			float current = window_fold_start<OP>();
+			#pragma unroll
+			for(int i = 0; i < COUNT; ++i)
+				current = window_fold<OP>(current, v[i]);
+			return current;
+		}
+
+		// One window: the values in scan order (quiet ones, for maximum and minimum).
+		template<int OP, int COUNT>
+		__device__ __forceinline__ float fold_values(const float (&v)[COUNT])
+		{
+			if (OP == window_op_sum)
+				return fold_values_in_order<OP>(v);
+			float current = fold_values_hw<OP>(v);
+			if (current == 0.0f)
+				current = fold_values_in_order<OP>(v); // which zero: the first one in scan order
+			return current;
+		}
+
+		// Two windows behind one test, so that the lanes without a zero jump over one block of code instead of
+		// stepping through two short ones.
+		template<int OP, int COUNT>
+		__device__ __forceinline__ void fold_values_twice(float& first_result, float& second_result, const float (&first)[COUNT], const float (&second)[COUNT])
+		{
+			if (OP == window_op_sum)
+			{
+				first_result = fold_values_in_order<OP>(first);
+				second_result = fold_values_in_order<OP>(second);
+				return;
+			}
+			first_result = fold_values_hw<OP>(first);
+			second_result = fold_values_hw<OP>(second);
+			if ((first_result == 0.0f) || (second_result == 0.0f))
+			{
+				first_result = fold_values_in_order<OP>(first);
+				second_result = fold_values_in_order<OP>(second);
+			}
 		}
 
 		// ---- 2-D windows, staged through LDS ------------------------------------------------------
@@ -117,6 +219,10 @@ namespace nnf
 			const uint32_t g0_aligned = g0 & ~3u;
 			const uint32_t shift = g0 - g0_aligned;
 			const uint32_t vectors = (g1 - g0_aligned + 3) / 4;
+			// Only the tensor's last float4 can be partial, so only the launch's last workgroup can meet it. The others
+			// take a loop without that case: with it in, every load had to wait for the one before (the compiler
+			// reused a load's destination registers for the next load's address).
+			const bool whole_vectors = g0_aligned + vectors * 4 <= a.total_in;
 			// all loads of a round are issued before the first one is stored to LDS
 			constexpr int STAGE = stage_vectors_per_lane;
 			// the weights are requested first and looked at once the first round's tensor loads are out
@@ -134,22 +240,35 @@ namespace nnf
 			for(uint32_t base = 0; base < vectors; base += STAGE * max_block_size)
 			{
 				floatx4 t[STAGE];
-				#pragma unroll
-				for(int k = 0; k < STAGE; ++k)
+				if (whole_vectors)
 				{
-					const uint32_t i = base + k * max_block_size + threadIdx.x;
-					const uint32_t g = g0_aligned + i * 4;
-					if (i < vectors)
+					#pragma unroll
+					for(int k = 0; k < STAGE; ++k)
 					{
-						if (g + 4 <= a.total_in)
-							t[k] = load_stream(reinterpret_cast<const floatx4*>(a.in + g));
-						else
+						const uint32_t i = base + k * max_block_size + threadIdx.x;
+						if (i < vectors)
+							t[k] = load_stream(reinterpret_cast<const floatx4*>(a.in + g0_aligned + i * 4));
+					}
+				}
+				else
+				{
+					#pragma unroll
+					for(int k = 0; k < STAGE; ++k)
+					{
+						const uint32_t i = base + k * max_block_size + threadIdx.x;
+						const uint32_t g = g0_aligned + i * 4;
+						if (i < vectors)
 						{
-							// the last, partial vector of the tensor
-							t[k].x = a.in[g];
-							t[k].y = (g + 1 < a.total_in) ? a.in[g + 1] : 0.0f;
-							t[k].z = (g + 2 < a.total_in) ? a.in[g + 2] : 0.0f;
-							t[k].w = 0.0f;
+							if (g + 4 <= a.total_in)
+								t[k] = load_stream(reinterpret_cast<const floatx4*>(a.in + g));
+							else
+							{
+								// the last, partial vector of the tensor
+								t[k].x = a.in[g];
+								t[k].y = (g + 1 < a.total_in) ? a.in[g + 1] : 0.0f;
+								t[k].z = (g + 2 < a.total_in) ? a.in[g + 2] : 0.0f;
+								t[k].w = 0.0f;
+							}
 						}
 					}
 				}
@@ -239,7 +358,7 @@ namespace nnf
 				{
 					const uint32_t i = base + k * max_block_size + threadIdx.x;
 					if (i < vectors)
-						*reinterpret_cast<floatx4*>(lds_in + i * 4) = t[k];
+						*reinterpret_cast<floatx4*>(lds_in + i * 4) = (OP == window_op_sum) ? t[k] : quiet(t[k]);
 				}
 			}
 			__syncthreads();
@@ -300,7 +419,6 @@ namespace nnf
 				const uint32_t last_x = TRUNC ? min(win_w, a.in_w - x0) - 1 : 0u;
 				const uint32_t last_y = TRUNC ? min(win_h, a.in_h - y0) - 1 : 0u;
 				static_assert(!(TRUNC && (OP == window_op_sum)), "a truncated window re-reads values");
-				float current = window_fold_start<OP>();
 				if (PAIR)
 				{
 					// columns x0 .. x0 + 3 lie inside the row (its length is a multiple of four, as is x0); the second
@@ -311,7 +429,8 @@ namespace nnf
 					for(int y = 1; y < WIN_H; ++y)
 						row_offset[y] = TRUNC ? row_offset[y - 1] + ((static_cast<uint32_t>(y) <= last_y) ? a.in_w : 0u) : static_cast<uint32_t>(y) * a.in_w;
 					const bool fifth_inside = !TRUNC || (x0 + 4 < a.in_w);
-					float second = window_fold_start<OP>();
+					constexpr int count = ((WIN_W > 0) && (WIN_H > 0)) ? WIN_W * WIN_H : 1;
+					float first[count], second[count];
 					#pragma unroll
 					for(int y = 0; y < WIN_H; ++y)
 					{
@@ -319,23 +438,28 @@ namespace nnf
 						const floatx4 v = *reinterpret_cast<const floatx4*>(row);
 						if (WIN_W == 2)
 						{
-							current = window_fold<OP>(window_fold<OP>(current, v.x), v.y);
-							second = window_fold<OP>(window_fold<OP>(second, v.z), v.w);
+							first[y * WIN_W] = v.x; first[y * WIN_W + 1] = v.y;
+							second[y * WIN_W] = v.z; second[y * WIN_W + 1] = v.w;
 						}
 						else
 						{
 							const float fifth = fifth_inside ? row[4] : v.w;
-							current = window_fold<OP>(window_fold<OP>(window_fold<OP>(current, v.x), v.y), v.z);
-							second = window_fold<OP>(window_fold<OP>(window_fold<OP>(second, v.z), v.w), fifth);
+							first[y * WIN_W] = v.x; first[y * WIN_W + 1] = v.y; first[y * WIN_W + 2] = v.z;
+							second[y * WIN_W] = v.z; second[y * WIN_W + 1] = v.w; second[y * WIN_W + 2] = fifth;
 						}
 					}
 					float2 both;
-					both.x = (OP == window_op_sum) ? current * a.mult : current;
-					both.y = (OP == window_op_sum) ? second * a.mult : second;
+					fold_values_twice<OP>(both.x, both.y, first, second);
+					if (OP == window_op_sum)
+					{
+						both.x *= a.mult;
+						both.y *= a.mult;
+					}
 					*reinterpret_cast<float2*>(dst + 2 * o) = both;
 				}
 				else
 				{
+				float current;
 				if ((WIN_W > 0) && (WIN_H > 0))
 				{
 					// min(y, last_y) * in_w and min(x, last_x) without multiplications
@@ -347,23 +471,46 @@ namespace nnf
 					#pragma unroll
 					for(int x = 0; x < WIN_W; ++x)
 						column_offset[x] = TRUNC ? min(static_cast<uint32_t>(x), last_x) : static_cast<uint32_t>(x);
+					constexpr int count = ((WIN_W > 0) && (WIN_H > 0)) ? WIN_W * WIN_H : 1;
+					float values[count];
 					#pragma unroll
 					for(int y = 0; y < WIN_H; ++y)
 					{
 						const float* row = src + row_offset[y];
 						#pragma unroll
 						for(int x = 0; x < WIN_W; ++x)
-							current = window_fold<OP>(current, row[column_offset[x]]);
+							values[y * WIN_W + x] = row[column_offset[x]];
 					}
+					current = fold_values<OP>(values);
 				}
 				else
 				{
 					const uint32_t fit_w = TRUNC ? last_x + 1 : win_w;
 					const uint32_t fit_h = TRUNC ? last_y + 1 : win_h;
+					current = window_fold_start<OP>();
 					const float* row = src;
-					for(uint32_t y = 0; y < fit_h; ++y, row += a.in_w)
-						for(uint32_t x = 0; x < fit_w; ++x)
-							current = window_fold<OP>(current, row[x]);
+					if (OP == window_op_sum)
+					{
+						for(uint32_t y = 0; y < fit_h; ++y, row += a.in_w)
+							for(uint32_t x = 0; x < fit_w; ++x)
+								current += row[x];
+					}
+					else
+					{
+						constexpr bool is_min = (OP == window_op_min);
+						for(uint32_t y = 0; y < fit_h; ++y, row += a.in_w)
+							for(uint32_t x = 0; x < fit_w; ++x)
+								current = hw_fold<is_min>(current, row[x]);
+						if (current == 0.0f)
+						{
+							// which zero: the first one in scan order, as the reference's fold keeps it
+							current = window_fold_start<OP>();
+							row = src;
+							for(uint32_t y = 0; y < fit_h; ++y, row += a.in_w)
+								for(uint32_t x = 0; x < fit_w; ++x)
+									current = fold<is_min>(current, row[x]);
+						}
+					}
 				}
 				dst[o] = (OP == window_op_sum) ? current * a.mult : current;
 				}
@@ -485,194 +632,372 @@ namespace nnf
 		// ---- tiling in 1 or 2 dimensions, staged through LDS ---------------------------------------
 		// A workgroup stages whole planes (small ones, several) or the input rows of a band of output rows, once, and
 		// every lane then takes output positions of that range: at a position it folds the window of each of the
-		// win_w * win_h shifted grids out of LDS and stores it to that grid's output entry. The input is read from
-		// memory once (twice where bands overlap) instead of once per grid.
+		// win_w * win_h shifted grids out of LDS. The input is read from memory once (twice where bands overlap)
+		// instead of once per grid. A band's results are contiguous in every grid's output plane: they are collected
+		// in LDS, one run per grid, and leave as aligned float4s (a wavefront's 64 single floats at an odd address,
+		// which is what a position per lane gives, cost the write path more than the staging costs: the planes of
+		// 55 x 55 outputs that 112 x 112 inputs give start on any 4-byte boundary). Several small planes per
+		// workgroup are stored from the lanes directly.
 		struct tiling2d_args
 		{
 			float* out;
 			const float* in;
+			uint32_t total_in;              // floats in the input tensor
 			uint32_t in_w, in_h, out_w, out_h, win_w, win_h;
 			uint32_t fm_count, plane_count; // planes = entries * feature maps
 			uint32_t planes;                // whole planes per workgroup; 1: bands of `rows` output rows, `bands` per plane
 			uint32_t rows, bands;
+			uint32_t in_area;               // bands: LDS floats in front of the grids' output runs
+			uint32_t out_pitch;             // bands: LDS floats from one grid's run to the next (a multiple of 4)
 		};
 
-		template<int OP, int WIN_W, int WIN_H>
-		__global__ void __launch_bounds__(max_block_size) tiling2d_kernel(const tiling2d_args a)
+		// What a workgroup stages: planes [first_plane, first_plane + planes_here), output rows [oy0, oy1) of them
+		struct tiling_range
 		{
-			extern __shared__ __attribute__((aligned(16))) float staged[];
-			const uint32_t win_w = (WIN_W > 0) ? WIN_W : a.win_w, win_h = (WIN_H > 0) ? WIN_H : a.win_h;
-			const uint32_t in_plane = a.in_w * a.in_h, out_plane = a.out_w * a.out_h;
 			uint32_t first_plane, planes_here, oy0, oy1;
+			uint32_t g0_aligned;   // first float of the aligned float4s around the staged input
+			uint32_t shift;        // floats of the first float4 in front of the range
+			uint32_t vectors;      // float4s to stage
+		};
+
+		__device__ __forceinline__ tiling_range tiling_range_of(const tiling2d_args& a, uint32_t work_id, uint32_t win_h)
+		{
+			tiling_range r;
+			const uint32_t in_plane = a.in_w * a.in_h;
 			if (a.planes > 1)
 			{
-				first_plane = blockIdx.x * a.planes;
-				planes_here = min(a.planes, a.plane_count - first_plane);
-				oy0 = 0;
-				oy1 = a.out_h;
+				r.first_plane = work_id * a.planes;
+				r.planes_here = min(a.planes, a.plane_count - r.first_plane);
+				r.oy0 = 0;
+				r.oy1 = a.out_h;
 			}
 			else
 			{
-				first_plane = blockIdx.x / a.bands;
-				planes_here = 1;
-				oy0 = (blockIdx.x - first_plane * a.bands) * a.rows;
-				oy1 = min(oy0 + a.rows, a.out_h);
+				r.first_plane = work_id / a.bands;
+				r.planes_here = 1;
+				r.oy0 = (work_id - r.first_plane * a.bands) * a.rows;
+				r.oy1 = min(r.oy0 + a.rows, a.out_h);
 			}
 			// input rows oy0 * win_h .. oy1 * win_h + win_h - 2 of every plane: the last grid's last window ends there
 			// (out_h * win_h + win_h - 1 <= in_h by the layer's output size); several planes are staged whole
-			const uint32_t first_row = oy0 * win_h;
-			const uint32_t staged_floats = (a.planes > 1) ? planes_here * in_plane : (oy1 * win_h + win_h - 1 - first_row) * a.in_w;
-			const float* src = a.in + static_cast<size_t>(first_plane) * in_plane + first_row * a.in_w;
-			if (((reinterpret_cast<uintptr_t>(src) & 15) == 0) && (staged_floats % 4 == 0))
-			{
-				// the usual case (even sizes): float4, four loads in flight per lane before the first LDS store
-				constexpr uint32_t in_flight = 4;
-				const floatx4* src4 = reinterpret_cast<const floatx4*>(src);
-				floatx4* staged4 = reinterpret_cast<floatx4*>(staged);
-				const uint32_t vectors = staged_floats / 4;
-				for(uint32_t base = threadIdx.x; base < vectors; base += max_block_size * in_flight)
-				{
-					floatx4 t[in_flight];
-					#pragma unroll
-					for(uint32_t k = 0; k < in_flight; ++k)
-						if (base + k * max_block_size < vectors)
-							t[k] = load_stream(src4 + base + k * max_block_size);
-					#pragma unroll
-					for(uint32_t k = 0; k < in_flight; ++k)
-						if (base + k * max_block_size < vectors)
-							staged4[base + k * max_block_size] = t[k];
-				}
-			}
-			else
-			{
-				#pragma unroll 8
-				for(uint32_t i = threadIdx.x; i < staged_floats; i += max_block_size)
-					staged[i] = src[i];
-			}
-			__syncthreads();
+			const uint32_t first_row = r.oy0 * win_h;
+			const uint32_t staged_floats = (a.planes > 1) ? r.planes_here * in_plane : (r.oy1 * win_h + win_h - 1 - first_row) * a.in_w;
+			const uint32_t g0 = r.first_plane * in_plane + first_row * a.in_w;
+			r.g0_aligned = g0 & ~3u;
+			r.shift = g0 - r.g0_aligned;
+			r.vectors = (staged_floats + r.shift + 3) / 4;
+			return r;
+		}
 
-			const uint32_t rows_here = oy1 - oy0;
+		// The staged input is in LDS (behind a barrier): every lane folds its positions. Bands put their results
+		// into the grids' runs in LDS, several planes store them.
+		template<int OP, int WIN_W, int WIN_H, int BLOCK>
+		__device__ __forceinline__ void tiling_scan(const tiling2d_args& a, const tiling_range& r, float* staged_area)
+		{
+			const uint32_t win_w = (WIN_W > 0) ? WIN_W : a.win_w, win_h = (WIN_H > 0) ? WIN_H : a.win_h;
+			const uint32_t in_plane = a.in_w * a.in_h, out_plane = a.out_w * a.out_h;
+			const bool band = a.planes == 1;
+			const uint32_t first_plane = r.first_plane, planes_here = r.planes_here;
+			const float* staged = staged_area + r.shift;
+			const uint32_t rows_here = r.oy1 - r.oy0;
 			const uint32_t positions_per_plane = rows_here * a.out_w;
 			const uint32_t positions = planes_here * positions_per_plane;
-			const size_t grid_stride = static_cast<size_t>(a.fm_count) * out_plane; // from one output entry to the next
-			// A lane takes positions tid, tid + 256, ...: plane, row and column of the first one by division, the following
-			// ones by addition with carries (256 positions further is step_p planes, step_y rows and step_x columns further)
-			// instead of three integer divisions per position.
-			const uint32_t step_p = max_block_size / positions_per_plane;
-			const uint32_t step_rest = max_block_size - step_p * positions_per_plane;
+			const uint32_t tiles = win_w * win_h;
+			const uint32_t grid_stride = a.fm_count * out_plane; // from one output entry to the next (tensors are indexed with 32 bits)
+			// A lane takes positions tid, tid + BLOCK, ...: plane, row and column of the first one by division, the following
+			// ones by addition with carries (BLOCK positions further is step_p planes, step_y rows and step_x columns further)
+			// instead of divisions and multiplications per position; the same for where its windows start in LDS.
+			const uint32_t step_p = BLOCK / positions_per_plane;
+			const uint32_t step_rest = BLOCK - step_p * positions_per_plane;
 			const uint32_t step_y = step_rest / a.out_w;
 			const uint32_t step_x = step_rest - step_y * a.out_w;
+			const uint32_t row_floats = win_h * a.in_w;                        // one output row further
+			const uint32_t corner_advance = step_p * in_plane + step_y * row_floats + step_x * win_w;
+			const uint32_t x_carry_corner = row_floats - a.out_w * win_w;      // back to column 0, one row down
+			const uint32_t y_carry_corner = in_plane - rows_here * row_floats; // back to row 0, one plane on
 			uint32_t p = (planes_here > 1) ? threadIdx.x / positions_per_plane : 0u;
 			uint32_t oy = (threadIdx.x - p * positions_per_plane) / a.out_w;
 			uint32_t ox = threadIdx.x - p * positions_per_plane - oy * a.out_w;
-			// a band: one plane for the whole workgroup
+			uint32_t corner_offset = p * in_plane + oy * row_floats + ox * win_w;
+			// a band: one plane for the whole workgroup, and its positions lie in the output plane one after the other.
+			// Grid g's run starts at band_out_index + g * grid_stride; in LDS it is kept at the same offset from a 16-byte
+			// boundary as in memory, so that an aligned float4 of the one is an aligned float4 of the other.
 			const uint32_t band_entry = first_plane / a.fm_count;
 			const uint32_t band_fm = first_plane - band_entry * a.fm_count;
-			for(uint32_t pos = threadIdx.x; pos < positions; pos += max_block_size)
+			const uint32_t band_out_index = (band_entry * tiles * a.fm_count + band_fm) * out_plane + r.oy0 * a.out_w;
+			float* const runs = staged_area + a.in_area;
+			// With the window size known a lane works on several positions at a time: the LDS reads of all of them are
+			// out before the first is folded.
+			constexpr bool sized = (WIN_W > 0) && (WIN_H > 0);
+			constexpr int batch = !sized ? 1 : ((WIN_W * WIN_H <= 4) ? 4 : 2);
+			constexpr bool is_min = (OP == window_op_min);
+			for(uint32_t pos = threadIdx.x; pos < positions; pos += BLOCK * batch)
 			{
-				uint32_t entry = band_entry, fm = band_fm;
-				if (planes_here > 1)
-				{
-					const uint32_t plane_id = first_plane + p;
-					entry = plane_id / a.fm_count;
-					fm = plane_id - entry * a.fm_count;
-				}
-				const float* corner = staged + p * in_plane + oy * win_h * a.in_w + ox * win_w;
-				float* dst = a.out + (static_cast<size_t>(entry) * (win_w * win_h) * a.fm_count + fm) * out_plane + (oy0 + oy) * a.out_w + ox;
-				// grids in the order of the window scan: x shift fastest
+				uint32_t out_index[batch], corner_of[batch];
+				bool valid[batch];
 				#pragma unroll
-				for(uint32_t sy = 0; sy < win_h; ++sy)
+				for(int b = 0; b < batch; ++b)
 				{
-					#pragma unroll
-					for(uint32_t sx = 0; sx < win_w; ++sx)
+					valid[b] = pos + b * BLOCK < positions;
+					out_index[b] = pos + b * BLOCK; // bands: inside the run
+					if (!band)
 					{
-						float current = window_fold_start<OP>();
-						#pragma unroll
-						for(uint32_t y = 0; y < win_h; ++y)
-						{
-							#pragma unroll
-							for(uint32_t x = 0; x < win_w; ++x)
-								current = window_fold<OP>(current, corner[(sy + y) * a.in_w + sx + x]);
-						}
-						*dst = current;
-						dst += grid_stride;
+						const uint32_t plane_id = first_plane + p;
+						const uint32_t entry = plane_id / a.fm_count;
+						const uint32_t fm = plane_id - entry * a.fm_count;
+						out_index[b] = (entry * tiles * a.fm_count + fm) * out_plane + oy * a.out_w + ox;
+					}
+					corner_of[b] = valid[b] ? corner_offset : 0u;
+					// BLOCK positions further
+					ox += step_x;
+					oy += step_y;
+					p += step_p;
+					corner_offset += corner_advance;
+					if (ox >= a.out_w)
+					{
+						ox -= a.out_w;
+						++oy;
+						corner_offset += x_carry_corner;
+					}
+					if (oy >= rows_here)
+					{
+						oy -= rows_here;
+						++p;
+						corner_offset += y_carry_corner;
 					}
 				}
-				// 256 positions further
-				ox += step_x;
-				oy += step_y;
-				p += step_p;
-				if (ox >= a.out_w)
+				// grids in the order of the window scan: x shift fastest
+				if (sized)
 				{
-					ox -= a.out_w;
-					++oy;
+					// the (2 * height - 1) x (2 * width - 1) values the grids' windows at a position cover
+					constexpr int span_w = sized ? 2 * WIN_W - 1 : 1, span_h = sized ? 2 * WIN_H - 1 : 1;
+					constexpr int grids = sized ? WIN_W * WIN_H : 1;
+					float near[batch][span_h][span_w];
+					#pragma unroll
+					for(int b = 0; b < batch; ++b)
+					{
+						const float* corner = staged + corner_of[b];
+						#pragma unroll
+						for(int y = 0; y < span_h; ++y)
+						{
+							#pragma unroll
+							for(int x = 0; x < span_w; ++x)
+								near[b][y][x] = corner[y * a.in_w + x];
+						}
+					}
+					#pragma unroll
+					for(int b = 0; b < batch; ++b)
+					{
+						float values[grids][grids], result[grids];
+						bool any_zero = false;
+						#pragma unroll
+						for(int g = 0; g < grids; ++g)
+						{
+							#pragma unroll
+							for(int y = 0; y < WIN_H; ++y)
+							{
+								#pragma unroll
+								for(int x = 0; x < WIN_W; ++x)
+									values[g][y * WIN_W + x] = near[b][g / WIN_W + y][g % WIN_W + x];
+							}
+							result[g] = fold_values_hw<OP>(values[g]);
+							any_zero = any_zero || (result[g] == 0.0f);
+						}
+						// which zero: the first one in scan order, as the reference's fold keeps it
+						if (any_zero)
+						{
+							#pragma unroll
+							for(int g = 0; g < grids; ++g)
+								result[g] = fold_values_in_order<OP>(values[g]);
+						}
+						if (valid[b])
+						{
+							#pragma unroll
+							for(int g = 0; g < grids; ++g)
+							{
+								if (band)
+									runs[g * a.out_pitch + ((band_out_index + g * grid_stride) & 3u) + out_index[b]] = result[g];
+								else
+									a.out[out_index[b] + g * grid_stride] = result[g];
+							}
+						}
+					}
 				}
-				if (oy >= rows_here)
+				else if (valid[0])
 				{
-					oy -= rows_here;
-					++p;
+					const float* corner = staged + corner_of[0];
+					uint32_t g = 0;
+					for(uint32_t sy = 0; sy < win_h; ++sy)
+					{
+						for(uint32_t sx = 0; sx < win_w; ++sx, ++g)
+						{
+							float current = window_fold_start<OP>();
+							for(uint32_t y = 0; y < win_h; ++y)
+								for(uint32_t x = 0; x < win_w; ++x)
+									current = hw_fold<is_min>(current, corner[(sy + y) * a.in_w + sx + x]);
+							if (current == 0.0f)
+							{
+								current = window_fold_start<OP>();
+								for(uint32_t y = 0; y < win_h; ++y)
+									for(uint32_t x = 0; x < win_w; ++x)
+										current = fold<is_min>(current, corner[(sy + y) * a.in_w + sx + x]);
+							}
+							if (band)
+								runs[g * a.out_pitch + ((band_out_index + g * grid_stride) & 3u) + out_index[0]] = current;
+							else
+								a.out[out_index[0] + g * grid_stride] = current;
+						}
+					}
 				}
 			}
 		}
 
+		// A band's runs are in LDS (behind a barrier) and leave: aligned float4s, and single floats where a run starts
+		// or ends inside one.
+		template<int BLOCK>
+		__device__ __forceinline__ void tiling_write_runs(const tiling2d_args& a, const tiling_range& r, const float* staged_area, uint32_t tiles)
+		{
+			const uint32_t out_plane = a.out_w * a.out_h;
+			const uint32_t grid_stride = a.fm_count * out_plane;
+			const uint32_t band_entry = r.first_plane / a.fm_count;
+			const uint32_t band_fm = r.first_plane - band_entry * a.fm_count;
+			const uint32_t band_out_index = (band_entry * tiles * a.fm_count + band_fm) * out_plane + r.oy0 * a.out_w;
+			const uint32_t positions = (r.oy1 - r.oy0) * a.out_w;
+			const float* runs = staged_area + a.in_area;
+			for(uint32_t g = 0; g < tiles; ++g)
+			{
+				const uint32_t run_index = band_out_index + g * grid_stride;   // first float of the run in the output tensor
+				const uint32_t lead = run_index & 3u;                          // floats of the first float4 in front of it
+				const float* from = runs + g * a.out_pitch;                    // from[lead + i]: float i of the run
+				float* to = a.out + (run_index - lead);                        // 16-byte aligned: the tensor's base is
+				const uint32_t end = lead + positions;
+				for(uint32_t k = threadIdx.x * 4; k < end; k += BLOCK * 4)
+				{
+					const floatx4 v = *reinterpret_cast<const floatx4*>(from + k);
+					if ((k >= lead) && (k + 4 <= end))
+						store_stream(reinterpret_cast<floatx4*>(to + k), v);
+					else
+					{
+						if ((k >= lead) && (k < end)) to[k] = v.x;
+						if ((k + 1 >= lead) && (k + 1 < end)) to[k + 1] = v.y;
+						if ((k + 2 >= lead) && (k + 2 < end)) to[k + 2] = v.z;
+						if ((k + 3 >= lead) && (k + 3 < end)) to[k + 3] = v.w;
+					}
+				}
+			}
+		}
+
+		template<int OP, int WIN_W, int WIN_H, int BLOCK>
+		__global__ void __launch_bounds__(BLOCK) tiling2d_kernel(const tiling2d_args a)
+		{
+			extern __shared__ __attribute__((aligned(16))) float staged_area[];
+			const uint32_t win_w = (WIN_W > 0) ? WIN_W : a.win_w, win_h = (WIN_H > 0) ? WIN_H : a.win_h;
+			const tiling_range r = tiling_range_of(a, blockIdx.x, win_h);
+			// Eight loads in flight per lane before the first LDS store. A band of the usual size is two or three float4s per
+			// lane; with sixteen the kernel holds 73 registers per lane and 64 x 64 planes of 112 x 112 with 2 x 2 windows
+			// take 78-80 us instead of 73.5.
+			constexpr uint32_t in_flight = 8;
+			floatx4* staged4 = reinterpret_cast<floatx4*>(staged_area);
+			// only the tensor's last float4 can be partial (in the launch's last workgroup): it is staged by one lane, float by float
+			const uint32_t whole_vectors = min(r.vectors, (a.total_in - r.g0_aligned) / 4);
+			for(uint32_t base = threadIdx.x; base < whole_vectors; base += BLOCK * in_flight)
+			{
+				floatx4 t[in_flight];
+				#pragma unroll
+				for(uint32_t k = 0; k < in_flight; ++k)
+					if (base + k * BLOCK < whole_vectors)
+						t[k] = *reinterpret_cast<const floatx4*>(a.in + r.g0_aligned + (base + k * BLOCK) * 4); // rows shared by two bands are wanted twice: no streaming hint
+				#pragma unroll
+				for(uint32_t k = 0; k < in_flight; ++k)
+					if (base + k * BLOCK < whole_vectors)
+						staged4[base + k * BLOCK] = quiet(t[k]);
+			}
+			if ((whole_vectors < r.vectors) && (threadIdx.x == 0))
+			{
+				for(uint32_t g = r.g0_aligned + whole_vectors * 4; g < a.total_in; ++g)
+					staged_area[g - r.g0_aligned] = quiet(a.in[g]);
+			}
+			__syncthreads();
+			tiling_scan<OP, WIN_W, WIN_H, BLOCK>(a, r, staged_area);
+			if (a.planes > 1)
+				return;
+			__syncthreads();
+			tiling_write_runs<BLOCK>(a, r, staged_area, win_w * win_h);
+		}
+
 		// -> true when the staged kernel took the work
-		bool launch_tiling2d(hipStream_t stream, bool is_min, float* output, const float* input, uint32_t plane_count, uint32_t fm_count,
+		bool launch_tiling2d(hipStream_t stream, bool is_min, float* output, const float* input, uint32_t total_in, uint32_t plane_count, uint32_t fm_count,
 			uint32_t in_w, uint32_t in_h, uint32_t out_w, uint32_t out_h, uint32_t win_w, uint32_t win_h)
 		{
-			constexpr uint32_t lds_floats_max = 15 * 1024;
+			constexpr uint32_t lds_floats_max = 15 * 1024;  // what a workgroup may use
+			constexpr uint32_t lds_floats_band = 6 * 1024;  // what a band and its output runs should stay under: six workgroups or more to a compute unit
 			tiling2d_args a = {};
 			a.out = output;
 			a.in = input;
+			a.total_in = total_in;
 			a.in_w = in_w; a.in_h = in_h; a.out_w = out_w; a.out_h = out_h; a.win_w = win_w; a.win_h = win_h;
 			a.fm_count = fm_count;
 			a.plane_count = plane_count;
 			const uint64_t in_plane = static_cast<uint64_t>(in_w) * in_h;
-			const uint64_t band_floats_min = static_cast<uint64_t>(2 * win_h - 1) * in_w; // one output row
-			if (band_floats_min > lds_floats_max)
+			const uint32_t tiles = win_w * win_h;
+			// a band of `rows` output rows: (rows * win_h + win_h - 1) input rows (+ 3 floats in front of an unaligned start),
+			// and a run of rows * out_w floats (+ up to 3 in front, rounded up to float4s) per grid
+			auto band_floats = [&](uint32_t rows, uint32_t& in_area, uint32_t& out_pitch) -> uint64_t
+			{
+				const uint64_t in_floats = static_cast<uint64_t>(rows * win_h + win_h - 1) * in_w + 3;
+				in_area = static_cast<uint32_t>((in_floats + 3) & ~static_cast<uint64_t>(3));
+				out_pitch = (rows * out_w + 3 + 3) & ~3u;
+				return static_cast<uint64_t>(in_area) + static_cast<uint64_t>(tiles) * out_pitch;
+			};
+			uint32_t in_area_one, out_pitch_one;
+			if (band_floats(1, in_area_one, out_pitch_one) > lds_floats_max)
 				return false;
-			uint32_t grid, staged_floats;
-			if (in_plane * 2 <= lds_floats_max)
+			uint32_t grid;
+			size_t lds_floats;
+			a.planes = 1;
+			if (in_plane * 2 + 3 <= lds_floats_max)
 			{
 				// small planes: enough of them for four positions per lane, as far as LDS holds them
 				const uint32_t wanted = (4 * max_block_size + out_w * out_h - 1) / (out_w * out_h);
-				a.planes = max(1u, min(min(wanted, static_cast<uint32_t>(lds_floats_max / in_plane)), plane_count));
+				a.planes = max(1u, min(min(wanted, static_cast<uint32_t>((lds_floats_max - 3) / in_plane)), plane_count));
 			}
-			else
-				a.planes = 1;
 			if (a.planes > 1)
 			{
 				a.rows = out_h;
 				a.bands = 1;
 				grid = (plane_count + a.planes - 1) / a.planes;
-				staged_floats = a.planes * static_cast<uint32_t>(in_plane);
+				lds_floats = a.planes * static_cast<size_t>(in_plane) + 8;
 			}
 			else
 			{
-				// (rows * win_h + win_h - 1) * in_w <= lds_floats_max
-				a.rows = min(out_h, static_cast<uint32_t>((lds_floats_max / in_w - (win_h - 1)) / win_h));
-				a.bands = (out_h + a.rows - 1) / a.rows;
+				// the highest band within the budget (any band that fits, if none does)
+				uint32_t rows = out_h;
+				while ((rows > 1) && (band_floats(rows, a.in_area, a.out_pitch) > lds_floats_band))
+					rows = (band_floats(rows, a.in_area, a.out_pitch) > 2 * static_cast<uint64_t>(lds_floats_band)) ? (rows + 1) / 2 : rows - 1;
+				a.bands = (out_h + rows - 1) / rows;
 				// few planes: more, lower bands (not below 4 output rows) until about 1024 workgroups share the work
 				const uint32_t bands_wanted = (1024 + plane_count - 1) / plane_count;
 				a.bands = max(a.bands, min(bands_wanted, max(1u, out_h / 4)));
 				a.rows = (out_h + a.bands - 1) / a.bands; // bands of equal height
 				a.bands = (out_h + a.rows - 1) / a.rows;
 				grid = plane_count * a.bands;
-				staged_floats = (a.rows * win_h + win_h - 1) * in_w;
+				lds_floats = band_floats(a.rows, a.in_area, a.out_pitch);
 			}
-			const size_t lds_bytes = static_cast<size_t>(staged_floats) * sizeof(float);
-			const dim3 g(grid), b(max_block_size);
+			const size_t lds_bytes = lds_floats * sizeof(float);
+			constexpr int block = max_block_size;
 			const bool w2 = (win_w == 2) && (win_h == 2), w3 = (win_w == 3) && (win_h == 3);
+			const dim3 g(grid), b(block);
 			if (is_min)
 			{
-				if (w2) hipLaunchKernelGGL((tiling2d_kernel<window_op_min, 2, 2>), g, b, lds_bytes, stream, a);
-				else if (w3) hipLaunchKernelGGL((tiling2d_kernel<window_op_min, 3, 3>), g, b, lds_bytes, stream, a);
-				else hipLaunchKernelGGL((tiling2d_kernel<window_op_min, 0, 0>), g, b, lds_bytes, stream, a);
+				if (w2) hipLaunchKernelGGL((tiling2d_kernel<window_op_min, 2, 2, block>), g, b, lds_bytes, stream, a);
+				else if (w3) hipLaunchKernelGGL((tiling2d_kernel<window_op_min, 3, 3, block>), g, b, lds_bytes, stream, a);
+				else hipLaunchKernelGGL((tiling2d_kernel<window_op_min, 0, 0, block>), g, b, lds_bytes, stream, a);
 			}
 			else
 			{
-				if (w2) hipLaunchKernelGGL((tiling2d_kernel<window_op_max, 2, 2>), g, b, lds_bytes, stream, a);
-				else if (w3) hipLaunchKernelGGL((tiling2d_kernel<window_op_max, 3, 3>), g, b, lds_bytes, stream, a);
-				else hipLaunchKernelGGL((tiling2d_kernel<window_op_max, 0, 0>), g, b, lds_bytes, stream, a);
+				if (w2) hipLaunchKernelGGL((tiling2d_kernel<window_op_max, 2, 2, block>), g, b, lds_bytes, stream, a);
+				else if (w3) hipLaunchKernelGGL((tiling2d_kernel<window_op_max, 3, 3, block>), g, b, lds_bytes, stream, a);
+				else hipLaunchKernelGGL((tiling2d_kernel<window_op_max, 0, 0, block>), g, b, lds_bytes, stream, a);
 			}
 			return true;
 		}
@@ -1109,7 +1434,7 @@ namespace nnf
 			return NNF_HIP_ETOOBIG;
 		if (overlap(output, output_total * sizeof(float), input, input_total * sizeof(float)))
 			return NNF_HIP_EOVERLAP;
-		if ((dimension_count <= 2) && launch_tiling2d(stream, is_min != 0, output, input, input_entry_count * feature_map_count, feature_map_count,
+		if ((dimension_count <= 2) && launch_tiling2d(stream, is_min != 0, output, input, static_cast<uint32_t>(input_total), input_entry_count * feature_map_count, feature_map_count,
 			nd.in_size[0], nd.in_size[1], nd.out_size[0], nd.out_size[1], nd.window[0], nd.window[1]))
 			return launch_status();
 		nd.out = output;

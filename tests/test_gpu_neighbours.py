@@ -269,6 +269,72 @@ def test_neighbour_entry_points_reject_bad_arguments(gpu):
 # subsampling with the element-wise layers in front of it folded in
 # ---------------------------------------------------------------------------------------------
 
+def zero_heavy(gen, shape, negative_share=0.0):
+    """Data on which the hardware's maximum and the reference's fold part ways unless the kernels repair it: most
+    windows hold nothing above zero, so which zero comes first decides the sign of the result; signalling and
+    negative NaNs, denormals (a flushed one would be a zero), values under the fold's start value and infinities
+    are mixed in. negative_share: that part of the values is drawn negative normal instead (for data in front of
+    a rectified_linear with slope 0, whose results are the -0.0s)."""
+    zeros = [0x00000000, 0x80000000]
+    nans = [0x7FA00000, 0xFFA00000, 0x7FC00000, 0xFFC00001]                 # signalling and quiet, both signs
+    below = [0x80000001, 0x807FFFFF, 0xBF800000, 0xFF800000, 0xFE967699,    # negative denormals, -1.0, -inf, -1.0e38,
+             0xFCF0BDC2, 0xFCF0BDC3]                                        # the start value -1.0e37F and one step under it
+    above = [0x00000001, 0x007FFFFF, 0x7CF0BDC2, 0x7E967699, 0x7F800000]    # denormals, 1.0e37F, 1.0e38, +inf
+    count = int(np.prod(shape))
+    kind = gen.random(count)
+    pick = lambda values: np.array(values, np.uint32)[gen.integers(0, len(values), size=count)]
+    bits = np.where(kind < 0.5, pick(zeros), np.where(kind < 0.65, pick(nans), np.where(kind < 0.92, pick(below), pick(above))))
+    x = bits.view(F).copy()
+    rare = gen.random(count) < 0.02
+    x[rare] = T.normal(gen, (count,), 2.0)[rare]
+    if negative_share > 0.0:
+        negative = gen.random(count) < negative_share
+        x[negative] = -np.abs(T.normal(gen, (count,), 2.0))[negative] - F(1.0e-3)
+    return x.reshape(shape)
+
+
+ZERO_HEAVY_POOL_CASES = [
+    ((8, 64, 112, 112), [3, 3], [2, 2], [True, True]),       # two outputs per lane at a time, bands of a plane
+    ((8, 16, 55, 55), [3, 3], [2, 2], None),                 # one output per lane, window size known
+    ((16, 32, 28, 28), [2, 2], None, None),                  # whole planes per workgroup, pairs of 2x2 windows
+    ((3, 3, 9, 31), [5, 2], [3, 1], [True, False]),          # run-time window sizes
+    ((5, 6, 37), [4], [3], [True]),                          # 1-D
+]
+
+
+@pytest.mark.parametrize("is_min", [False, True])
+@pytest.mark.parametrize("shape,windows,strides,round_ups", ZERO_HEAVY_POOL_CASES)
+def test_max_subsampling_where_the_first_zero_decides(gpu, shape, windows, strides, round_ups, is_min):
+    """The kernels fold with the hardware's maximum and fold a window again in the reference's order when its result
+    is a zero: here most windows need that, and signalling NaNs and denormals lie in between."""
+    x = zero_heavy(T.rng(71, sum(shape)), shape)
+    if is_min:
+        x = -x
+    got = run_max_subsampling(gpu, x, windows, strides, round_ups, is_min=is_min)
+    want = oracle.max_subsampling(x, windows, strides=strides, round_ups=round_ups, is_min=is_min)
+    zeros = float(np.mean(want == 0.0))
+    assert zeros > 0.2, zeros  # the case is what it says
+    assert T.bit_mismatches(got, want) == 0
+
+
+@pytest.mark.parametrize("is_min", [False, True])
+@pytest.mark.parametrize("shape,windows", [((4, 16, 112, 112), [2, 2]), ((2, 3, 60, 60), [3, 3]), ((7, 37, 6, 5), [2, 2]),
+                                           ((3, 4, 9, 11), [2, 3]), ((5, 2, 23), [4])])
+def test_max_subsampling_with_tiling_where_the_first_zero_decides(gpu, shape, windows, is_min):
+    x = zero_heavy(T.rng(72, sum(shape)), shape)
+    if is_min:
+        x = -x
+    want = oracle.max_subsampling(x, windows, tiling=True, is_min=is_min)
+    assert float(np.mean(want == 0.0)) > 0.2
+    dims = list(shape[2:])[::-1]
+    d_in = gpu.to_device(x)
+    d_out = gpu.torch.full((want.size,), float("nan"), dtype=gpu.torch.float32, device=gpu.device)
+    rc = gpu.lib.nnf_hip_max_subsampling_tiling_forward(gpu.stream, d_out.data_ptr(), d_in.data_ptr(), shape[0], shape[1], len(dims),
+                                                        u32(dims), u32(windows), int(is_min))
+    assert rc == 0, capi.error_string(rc)
+    assert T.bit_mismatches(gpu.to_host(d_out, want.shape), want) == 0
+
+
 def prologue_case(kind, gen, c):
     """-> (ops of the single arm, weight chunks, oracle steps) of a group in front of a subsampling layer"""
     if kind == "bn_relu":
@@ -359,6 +425,35 @@ def test_max_subsampling_with_group_folded_in(gpu, shape, windows, strides, roun
     want = oracle.max_subsampling(v, windows, strides=strides, round_ups=round_ups, is_min=is_min)
     got = run_fused_max(gpu, x, ops, chunks, windows, strides, round_ups, is_min=is_min)
     assert got.shape == want.shape
+    assert T.bit_mismatches(got, want) == 0
+
+
+@pytest.mark.parametrize("shape,windows,strides,round_ups,group", [
+    ((8, 64, 112, 112), [3, 3], [2, 2], [True, True], "relu"),      # a ResNet stem's pooling behind ReLU: all-negative windows give -0.0
+    ((8, 64, 112, 112), [3, 3], [2, 2], [True, True], "bn_relu"),
+    ((16, 32, 28, 28), [2, 2], None, None, "relu"),
+    ((6, 10, 7, 7), [3, 3], [2, 2], None, "bn_relu"),
+    ((5, 7, 6, 10), [3, 2], [2, 2], [True, False], "relu"),
+])
+def test_max_subsampling_behind_relu_where_many_windows_hold_only_zeros(gpu, shape, windows, strides, round_ups, group):
+    """rectified_linear with slope 0 turns every negative value into -0.0 and keeps +0.0: with three values in four
+    negative about one window in eight (3x3) holds nothing but zeros and the first of them decides the sign."""
+    gen = T.rng(73, sum(shape))
+    if group == "relu":
+        ops, chunks, steps = [(capi.OP_RELU, 0, 0.0)], [], [lambda v: oracle.rectified_linear(v, 0.0)]
+        x = zero_heavy(gen, shape, negative_share=0.75)
+    else:
+        ops, chunks, steps = prologue_case("bn_relu", gen, shape[1])
+        x = T.normal(gen, shape, 1.0) - F(0.9)
+        flat = x.reshape(-1)
+        idx = gen.integers(0, flat.size, size=flat.size // 20)
+        flat[idx] = chunks[2][(idx // int(np.prod(shape[2:]))) % shape[1]]  # the feature map's mean: BatchNorm gives beta, often +-0 after ReLU
+    v = x
+    for step in steps:
+        v = step(v)
+    want = oracle.max_subsampling(v, windows, strides=strides, round_ups=round_ups)
+    assert float(np.mean(want == 0.0)) > 0.03
+    got = run_fused_max(gpu, x, ops, chunks, windows, strides, round_ups)
     assert T.bit_mismatches(got, want) == 0
 
 
