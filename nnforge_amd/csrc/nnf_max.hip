@@ -13,6 +13,7 @@
 
 #include <algorithm>
 #include <cstdlib>
+#include <type_traits>
 
 namespace nnf
 {
@@ -219,10 +220,6 @@ namespace nnf
 			const uint32_t g0_aligned = g0 & ~3u;
 			const uint32_t shift = g0 - g0_aligned;
 			const uint32_t vectors = (g1 - g0_aligned + 3) / 4;
-			// Only the tensor's last float4 can be partial, so only the launch's last workgroup can meet it. The others
-			// take a loop without that case: with it in, every load had to wait for the one before (the compiler
-			// reused a load's destination registers for the next load's address).
-			const bool whole_vectors = g0_aligned + vectors * 4 <= a.total_in;
 			// all loads of a round are issued before the first one is stored to LDS
 			constexpr int STAGE = stage_vectors_per_lane;
 			// the weights are requested first and looked at once the first round's tensor loads are out
@@ -237,43 +234,38 @@ namespace nnf
 				else
 					weights = load_prologue_weights(first_plane % pro.fm_count, planes_here, pro);
 			}
-			for(uint32_t base = 0; base < vectors; base += STAGE * max_block_size)
+			// A round: COUNT float4s per lane from float4 `base` of the range on, up to float4 `limit`. PARTIAL: the
+			// round is the tensor's last float4, which ends inside it.
+			bool first_round = true;
+			auto stage_round = [&](auto count_tag, auto partial_tag, const uint32_t base, const uint32_t limit)
 			{
-				floatx4 t[STAGE];
-				if (whole_vectors)
+				constexpr int COUNT = decltype(count_tag)::value;
+				constexpr bool PARTIAL = decltype(partial_tag)::value;
+				floatx4 t[COUNT];
+				#pragma unroll
+				for(int k = 0; k < COUNT; ++k)
 				{
-					#pragma unroll
-					for(int k = 0; k < STAGE; ++k)
+					const uint32_t i = base + k * max_block_size + threadIdx.x;
+					if (!PARTIAL)
 					{
-						const uint32_t i = base + k * max_block_size + threadIdx.x;
-						if (i < vectors)
-							t[k] = load_stream(reinterpret_cast<const floatx4*>(a.in + g0_aligned + i * 4));
+						// Lanes past the end load the last float4 once more (and do not stage it): without a branch
+						// around every load the loads of a round are issued one behind the other. With the branches
+						// the compiler formed a load's address in the registers an earlier load was to arrive in,
+						// and every load waited for the ones before it.
+						t[k] = load_stream(reinterpret_cast<const floatx4*>(a.in + g0_aligned) + min(i, limit - 1));
 					}
-				}
-				else
-				{
-					#pragma unroll
-					for(int k = 0; k < STAGE; ++k)
+					else if (i < limit)
 					{
-						const uint32_t i = base + k * max_block_size + threadIdx.x;
 						const uint32_t g = g0_aligned + i * 4;
-						if (i < vectors)
-						{
-							if (g + 4 <= a.total_in)
-								t[k] = load_stream(reinterpret_cast<const floatx4*>(a.in + g));
-							else
-							{
-								// the last, partial vector of the tensor
-								t[k].x = a.in[g];
-								t[k].y = (g + 1 < a.total_in) ? a.in[g + 1] : 0.0f;
-								t[k].z = (g + 2 < a.total_in) ? a.in[g + 2] : 0.0f;
-								t[k].w = 0.0f;
-							}
-						}
+						t[k].x = a.in[g];
+						t[k].y = (g + 1 < a.total_in) ? a.in[g + 1] : 0.0f;
+						t[k].z = (g + 2 < a.total_in) ? a.in[g + 2] : 0.0f;
+						t[k].w = 0.0f;
 					}
 				}
-				if (PROLOGUE && (base == 0))
+				if (PROLOGUE && first_round)
 				{
+					first_round = false;
 					if (uniform)
 						uniform_coefficients(own_coef, plane_weights, pro);
 					else
@@ -287,8 +279,8 @@ namespace nnf
 				}
 				if (PROLOGUE)
 				{
-					float v[STAGE][4];
-					uint32_t off[STAGE];
+					float v[COUNT][4];
+					uint32_t off[COUNT];
 					// Planes that are not a multiple of four floats long: a float4 may straddle two of them (never
 					// three: the host declines planes of under 4 floats). Bit k: vector k does.
 					// which plane a value belongs to matters only to layers with weights, and only with several planes here
@@ -296,10 +288,10 @@ namespace nnf
 					const bool straddle = per_plane && ((in_plane & 3u) != 0);
 					uint32_t straddling = 0;
 					#pragma unroll
-					for(int k = 0; k < STAGE; ++k)
+					for(int k = 0; k < COUNT; ++k)
 					{
 						const uint32_t i = base + k * max_block_size + threadIdx.x;
-						const bool valid = i < vectors;
+						const bool valid = i < limit;
 						// lanes past the end put zeros through the layers
 						v[k][0] = valid ? t[k].x : 0.0f; v[k][1] = valid ? t[k].y : 0.0f; v[k][2] = valid ? t[k].z : 0.0f; v[k][3] = valid ? t[k].w : 0.0f;
 						// plane, inside the workgroup's range, of the first float of this float4 (floats in front
@@ -313,9 +305,9 @@ namespace nnf
 							straddling |= 1u << k;
 					}
 					if (uniform)
-						apply_prologue<STAGE, EXP, true>(v, off, lds_coef, own_coef, pro, exp_ctx, 0, pro.op_count);
+						apply_prologue<COUNT, EXP, true>(v, off, lds_coef, own_coef, pro, exp_ctx, 0, pro.op_count);
 					else
-						apply_prologue<STAGE, EXP, false>(v, off, lds_coef, own_coef, pro, exp_ctx, 0, pro.op_count);
+						apply_prologue<COUNT, EXP, false>(v, off, lds_coef, own_coef, pro, exp_ctx, 0, pro.op_count);
 					// The floats of the second plane of a straddling float4 were given the first plane's
 					// coefficients: they are fetched again and go through the layers with their own.
 					while (__any(straddling != 0))
@@ -336,7 +328,7 @@ namespace nnf
 						const uint32_t off_next[1] = { p_next * (2 * pro.weighted_count) };
 						apply_prologue<1, EXP, false>(w, off_next, lds_coef, own_coef, pro, exp_ctx, 0, pro.op_count);
 						#pragma unroll
-						for(int k = 0; k < STAGE; ++k)
+						for(int k = 0; k < COUNT; ++k)
 						{
 							#pragma unroll
 							for(uint32_t e = 1; e < 4; ++e)
@@ -348,19 +340,26 @@ namespace nnf
 						straddling &= straddling - 1;
 					}
 					#pragma unroll
-					for(int k = 0; k < STAGE; ++k)
+					for(int k = 0; k < COUNT; ++k)
 					{
 						t[k].x = v[k][0]; t[k].y = v[k][1]; t[k].z = v[k][2]; t[k].w = v[k][3];
 					}
 				}
 				#pragma unroll
-				for(int k = 0; k < STAGE; ++k)
+				for(int k = 0; k < COUNT; ++k)
 				{
 					const uint32_t i = base + k * max_block_size + threadIdx.x;
-					if (i < vectors)
+					if (i < limit)
 						*reinterpret_cast<floatx4*>(lds_in + i * 4) = (OP == window_op_sum) ? t[k] : quiet(t[k]);
 				}
-			}
+			};
+			// whole float4s first; only the tensor's last float4 can be partial (in the launch's last workgroup) and gets a
+			// round of its own, so that the rounds all others take carry no such case
+			const uint32_t whole_vectors = min(vectors, (a.total_in - g0_aligned) / 4);
+			for(uint32_t base = 0; base < whole_vectors; base += STAGE * max_block_size)
+				stage_round(std::integral_constant<int, STAGE>(), std::false_type(), base, whole_vectors);
+			if (whole_vectors < vectors)
+				stage_round(std::integral_constant<int, 1>(), std::true_type(), whole_vectors, vectors);
 			__syncthreads();
 
 			// A lane's unit of work: one output, or (PAIR) two neighbouring outputs of a row
@@ -540,11 +539,13 @@ namespace nnf
 			window2d_body<OP, WIN_W, WIN_H, TRUNC, false, false, false, PAIR>(a, none);
 		}
 
-		// UNIFORM: one plane per workgroup (a.planes == 1). Without expf the layers fit 96 registers per lane,
-		// which lets a compute unit hold five workgroups instead of four (measured: 10 % faster); with expf
-		// that would spill.
+		// UNIFORM: one plane per workgroup (a.planes == 1). Without expf the layers fit 80 registers per lane,
+		// which lets a compute unit hold six workgroups instead of four where their LDS allows it (the two bands of a
+		// 112 x 112 plane are 25.6 KB each; BatchNorm + ReLU + 3x3/2 pooling of 64 x 64 such planes: 54 us at four,
+		// 46-47 us at five, 43.7 us at six); with expf that would spill, and so would the kernels for several planes per
+		// workgroup, which stay at five.
 		template<int OP, int WIN_W, int WIN_H, bool TRUNC, bool UNIFORM, bool PAIR = false>
-		__global__ void __launch_bounds__(max_block_size) __attribute__((amdgpu_waves_per_eu(5, 5))) max_window2d_prologue_kernel(const window2d_args a, const window_prologue pro)
+		__global__ void __launch_bounds__(max_block_size) __attribute__((amdgpu_waves_per_eu(UNIFORM ? 6 : 5, UNIFORM ? 6 : 5))) max_window2d_prologue_kernel(const window2d_args a, const window_prologue pro)
 		{
 			window2d_body<OP, WIN_W, WIN_H, TRUNC, true, false, UNIFORM, PAIR>(a, pro);
 		}
@@ -900,17 +901,20 @@ namespace nnf
 			floatx4* staged4 = reinterpret_cast<floatx4*>(staged_area);
 			// only the tensor's last float4 can be partial (in the launch's last workgroup): it is staged by one lane, float by float
 			const uint32_t whole_vectors = min(r.vectors, (a.total_in - r.g0_aligned) / 4);
-			for(uint32_t base = threadIdx.x; base < whole_vectors; base += BLOCK * in_flight)
+			for(uint32_t base = 0; base < whole_vectors; base += BLOCK * in_flight)
 			{
+				// A stripe of BLOCK float4s is skipped as a whole when it lies past the end (the same for all lanes), and inside
+				// the last stripe the lanes past the end load the last float4 once more: no lane-dependent branch around a load,
+				// so the loads are issued one behind the other. Rows shared by two bands are wanted twice: no streaming hint.
 				floatx4 t[in_flight];
 				#pragma unroll
 				for(uint32_t k = 0; k < in_flight; ++k)
 					if (base + k * BLOCK < whole_vectors)
-						t[k] = *reinterpret_cast<const floatx4*>(a.in + r.g0_aligned + (base + k * BLOCK) * 4); // rows shared by two bands are wanted twice: no streaming hint
+						t[k] = reinterpret_cast<const floatx4*>(a.in + r.g0_aligned)[min(base + k * BLOCK + threadIdx.x, whole_vectors - 1)];
 				#pragma unroll
 				for(uint32_t k = 0; k < in_flight; ++k)
-					if (base + k * BLOCK < whole_vectors)
-						staged4[base + k * BLOCK] = quiet(t[k]);
+					if (base + k * BLOCK + threadIdx.x < whole_vectors)
+						staged4[base + k * BLOCK + threadIdx.x] = quiet(t[k]);
 			}
 			if ((whole_vectors < r.vectors) && (threadIdx.x == 0))
 			{
