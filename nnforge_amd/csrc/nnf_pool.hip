@@ -34,18 +34,16 @@ namespace nnf
 			const float* src = in + static_cast<size_t>(first_plane) * plane; // 16-byte aligned: first_plane is a multiple of 4
 
 			const uint32_t vectors = floats_here / 4;
-			// eight loads in flight per lane before the first value goes to LDS
-			constexpr int stage = 8;
+			// four loads in flight per lane before the first value goes to LDS (a workgroup stages about 4096 floats)
+			constexpr int stage = 4;
 			for(uint32_t base = 0; base < vectors; base += stage * pool_block_size)
 			{
+				// No branch around a load (lanes past the end load the last float4 once more and do not stage it): with one,
+				// every load of a round waited for the one before it.
 				floatx4 t[stage];
 				#pragma unroll
 				for(int k = 0; k < stage; ++k)
-				{
-					const uint32_t i = base + k * pool_block_size + threadIdx.x;
-					if (i < vectors)
-						t[k] = load_stream(reinterpret_cast<const floatx4*>(src) + i);
-				}
+					t[k] = load_stream(reinterpret_cast<const floatx4*>(src) + min(base + k * pool_block_size + threadIdx.x, vectors - 1));
 				#pragma unroll
 				for(int k = 0; k < stage; ++k)
 				{

@@ -165,14 +165,13 @@ namespace nnf
 				#pragma unroll
 				for(int k = 0; k < stat_unroll; ++k)
 				{
-					const uint32_t t = first + k * stat_block_size + threadIdx.x;
-					if (t < units)
-					{
-						// element t of the run lies t * VEC floats into it plus the other feature maps of the
-						// entries before it: e * (entry_stride - plane); the tensor has fewer than 2^32 floats
-						const uint32_t e = (entries_here == 1) ? 0u : ((units_per_plane == 1) ? t : __umulhi(t, unit_magic));
-						v[k] = __builtin_nontemporal_load(reinterpret_cast<const vec_t*>(base + (t * VEC + e * entry_gap)));
-					}
+					// No branch around a load (lanes past the end load the run's last unit once more and leave it out of
+					// the sums): with one, every load of a round waited for the one before it.
+					const uint32_t t = min(first + k * stat_block_size + threadIdx.x, units - 1);
+					// element t of the run lies t * VEC floats into it plus the other feature maps of the
+					// entries before it: e * (entry_stride - plane); the tensor has fewer than 2^32 floats
+					const uint32_t e = (entries_here == 1) ? 0u : ((units_per_plane == 1) ? t : __umulhi(t, unit_magic));
+					v[k] = __builtin_nontemporal_load(reinterpret_cast<const vec_t*>(base + (t * VEC + e * entry_gap)));
 				}
 				#pragma unroll
 				for(int k = 0; k < stat_unroll; ++k)
