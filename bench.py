@@ -339,7 +339,7 @@ def bench_resnet50(runner, steps, warmup, n=64, kernel_stream_count=0, one_launc
     rep = backend.time_kernels(text, weights, configs, outputs, warmup=warmup, passes=steps, shared_input_pool=pool, entry_count=n,
                                max_entry_count=n, kernel_stream_count=kernel_stream_count, one_launch_per_group=one_launch_per_group)
     groups = w.resnet50_groups(n)
-    assert rep["timed_entries"] == n and rep["launches"] == len(groups) + 1, rep["raw"]
+    assert rep["timed_entries"] == n and rep["plan_steps"] == len(groups) + 1, rep["raw"]
     # the driver orders the steps into the slots of its launch plan: same groups as the hand-written list, not the same order; the step
     # of the last group also holds the average behind it
     planned = sorted((len(step["inputs"]), len(step["layers"]) - (step["layers"][-1] == "pool5")) for step in rep["steps"] if step["fused"])
@@ -351,7 +351,7 @@ def bench_resnet50(runner, steps, warmup, n=64, kernel_stream_count=0, one_launc
     assert sum(step["layers"][-1] == "pool5" and step["fused"] for step in rep["steps"]) == 1, rep["raw"]
     return result_entry("config4: ResNet-50 post-convolution stack N=%d (49 fused groups + 7x7 average + softmax) through forward_propagation_hip" % n,
                         g_bytes + p_bytes + s_bytes, elements, rep["wall_seconds_per_pass"], rep["device_seconds_per_pass"], 1,
-                        {"plan_steps_per_pass": rep["launches"], "host_enqueue_ms_per_pass": rep["host_seconds_per_pass"] * 1e3, "kernel_streams": len({st["stream"] for st in rep["steps"]}),
+                        {"plan_steps_per_pass": rep["plan_steps"], "kernel_launches_per_pass": rep["launches"], "host_enqueue_ms_per_pass": rep["host_seconds_per_pass"] * 1e3, "kernel_streams": len({st["stream"] for st in rep["steps"]}),
                          "runs_of_groups_launched_together": len({st["run"] for st in rep["steps"] if st["run"] is not None}),
                          "note": "a step is one pass of the launch plan, timed inside the C++ driver (forward_propagation_hip::time_kernels): "
                                  "one resident packet, the plan enqueued on the driver's kernel streams (independent groups share kernel "

@@ -364,6 +364,11 @@ NNF_HIP_API int nnf_hip_copy_kernel(void* stream, void* device_dst, const void* 
  * and nnforge/plain/hyperbolic_tangent_layer_tester_plain.cpp:55-56 rests on it. */
 NNF_HIP_API int nnf_hip_check_division_sequences(void* stream, uint64_t* device_mismatch_counts);
 
+/* Kernels the library has launched from the calling thread since it was loaded. The driver reads it on both sides of a
+ * pass of its plan to report how many launches a pass is (a call that takes several groups decides by itself how many
+ * kernels they share). No counterpart in the reference. */
+NNF_HIP_API int nnf_hip_launch_count(uint64_t* count);
+
 NNF_HIP_API const char* nnf_hip_error_string(int code);
 NNF_HIP_API const char* nnf_hip_version(void);
 

@@ -96,6 +96,12 @@ namespace nnforge
 			// 8 entries 243 -> 172 us.
 			bool batch_independent_groups;
 			unsigned int reserved_thread_count;
+			// run() makes its packets no larger than this much pinned staging (input + output entries) per I/O slot, so that
+			// reading, copying, computing and writing of neighbouring packets overlap; 0: no bound. It never pushes a
+			// packet under min_packet_entries_under_staging_bound entries (a network with many or large data layers would
+			// otherwise run its plan entry by entry).
+			size_t max_io_staging_bytes = static_cast<size_t>(64) << 20;
+			static constexpr unsigned int min_packet_entries_under_staging_bound = 8;
 			std::string device_name;
 			unsigned long long global_memory_size;
 			unsigned int compute_unit_count;
@@ -272,23 +278,30 @@ namespace nnforge
 			// device bytes per entry of the current buffer plan, and the packet size derived from it
 			size_t get_per_entry_buffer_bytes() const { return per_entry_bytes; }
 			unsigned int get_max_entry_count() const { return max_entry_count; }
-			// run() makes its packets no larger than this much pinned staging (input + output entries) per I/O slot
-			static constexpr size_t max_io_staging_bytes_per_slot = static_cast<size_t>(64) << 20;
+			// entries per packet of the latest run() (0 before the first): max_entry_count, the reader's entry count and the
+			// configuration's staging bound decide it
+			unsigned int get_packet_entry_count() const { return packet_entry_count; }
 
 			// Times the launch plan alone, on data that stays in device memory: reads one packet of up to entry_count
-			// entries from the reader and uploads it, runs the plan warmup times untimed, then `passes` times bracketed
-			// by a device synchronisation on both sides (wall clock) and by events on the kernel stream. Nothing is
-			// copied back and the writer's role is empty: this is the figure of merit of the kernels and of the way
-			// the driver enqueues them, without the host link. No counterpart in the reference.
+			// entries from the reader and uploads it, runs the plan once and warmup times more untimed, then `passes`
+			// times bracketed by a device synchronisation on both sides (wall clock) and by events on the kernel stream.
+			// resident_packets > 1: the data and output layers get that many sets of device buffers (every set holds
+			// the same packet) and the passes go round them, so that a small network's tensors come from memory and
+			// not from the last-level cache; buffers in between are shared by all sets. Nothing is copied back and
+			// the writer's role is empty: this is the figure of merit of the kernels and of the way the driver
+			// enqueues them, without the host link. No counterpart in the reference.
 			struct kernel_timing
 			{
 				unsigned int entry_count;      // entries the packet held
-				unsigned int launch_count;     // launches per pass
+				unsigned int resident_packets; // buffer sets the passes went round
+				unsigned int plan_step_count;  // steps of the plan that launch something
+				unsigned int launch_count;     // kernels one pass launches (steps that go to the kernels in one call share launches)
 				float wall_seconds_per_pass;
 				float device_seconds_per_pass; // from events on the kernel stream
 				float host_seconds_per_pass;   // what the calling thread spends enqueuing a pass (the device runs behind it)
 			};
-			kernel_timing time_kernels(structured_data_bunch_reader& reader, unsigned int entry_count, unsigned int warmup, unsigned int passes);
+			kernel_timing time_kernels(structured_data_bunch_reader& reader, unsigned int entry_count, unsigned int warmup, unsigned int passes,
+				unsigned int resident_packets = 1);
 
 		protected:
 			void actual_set_data(network_data::const_ptr data) override;
@@ -307,13 +320,15 @@ namespace nnforge
 			struct run_buffers;
 			// streams, device buffers for packets of `packet` entries (data and output layers once per I/O slot), pinned
 			// staging, weight pointers; what the run before left is used again when it was made for the same sizes
-			run_buffers& prepare_run(unsigned int packet, int slot_count, bool with_output_staging, bool stats_on_device);
+			// (staging_slot_count <= 0: as many as slot_count)
+			run_buffers& prepare_run(unsigned int packet, int slot_count, bool with_output_staging, bool stats_on_device, int staging_slot_count = 0);
 			std::unique_ptr<impl> p;
 			std::unique_ptr<run_buffers> kept_run; // released when the weights, the shapes or the packet size change
 			hip_running_configuration::const_ptr hip_config;
 			std::vector<forward_step> steps;
 			size_t per_entry_bytes;
 			unsigned int max_entry_count;
+			unsigned int packet_entry_count = 0;
 		};
 
 		// nnforge/cuda/forward_propagation_cuda_factory.h
@@ -334,7 +349,7 @@ namespace nnforge
 		// nnforge/cuda/factory_generator_cuda.h: options hip_device_id, hip_max_global_memory_usage_ratio,
 		// hip_fuse, hip_dont_share_buffers, hip_single_command_stream (as cuda_single_command_stream,
 		// nnforge/cuda/factory_generator_cuda.cpp:105-106), hip_batch_independent_groups, hip_kernel_stream_count, hip_max_entry_count,
-		// hip_reserved_thread_count (as cuda_reserved_thread_count, nnforge/cuda/factory_generator_cuda.cpp:95)
+		// hip_reserved_thread_count (as cuda_reserved_thread_count, nnforge/cuda/factory_generator_cuda.cpp:95), hip_max_io_staging_mb
 		class factory_generator_hip : public factory_generator
 		{
 		public:
@@ -356,6 +371,7 @@ namespace nnforge
 			int hip_kernel_stream_count;
 			int hip_max_entry_count;
 			int hip_reserved_thread_count;
+			int hip_max_io_staging_mb;
 
 		private:
 			hip_running_configuration::const_ptr hip_config;

@@ -44,8 +44,12 @@ typedef struct nnf_backend_output
 	size_t written_floats;         /* set by the call */
 } nnf_backend_output;
 
+/* struct_size: sizeof(nnf_backend_options) as the caller's header declares it. The library reads that many bytes and
+ * takes the members added since as zero (each member's default), so a caller built against an older header keeps
+ * working; a size of zero is refused. Zero the structure, set struct_size, then the members wanted. */
 typedef struct nnf_backend_options
 {
+	uint32_t struct_size;
 	int32_t fuse;                  /* hip_fuse */
 	int32_t dont_share_buffers;    /* hip_dont_share_buffers */
 	int32_t max_entry_count;       /* hip_max_entry_count; <= 0: default */
@@ -59,6 +63,9 @@ typedef struct nnf_backend_options
 	int32_t one_launch_per_group;  /* 1: hip_batch_independent_groups off (every fused group gets a launch of its own) */
 	int32_t host_thread_count;     /* threads that read input entries (sets hip_reserved_thread_count to the processors beyond
 	                                  them; at most 16 are used); <= 0: default, all processors but one */
+	int32_t max_io_staging_mb;     /* hip_max_io_staging_mb: pinned staging (input + output entries) per I/O slot that bounds a
+	                                  packet of run(); 0: default (64), < 0: no bound */
+	int32_t resident_packets;      /* nnf_backend_time_kernels: sets of data / output buffers the timed passes go round; <= 0: 1 */
 } nnf_backend_options;
 
 /* Runs the schema on device 0. The report lists one line per launch ("step: ..."), the buffer plan
@@ -127,7 +134,10 @@ NNF_BACKEND_API int nnf_backend_update_bn_weights(
 
 /* Times the launch plan of the schema alone, on one packet of entry_count entries that stays in device memory
  * (forward_propagation_hip::time_kernels): uploaded once, then `warmup` untimed and `passes` timed runs of the plan,
- * nothing copied back. The report lists the plan like nnf_backend_run_schema, then "launches: N", "timed_entries: N",
+ * nothing copied back. With options->resident_packets = R > 1 the data and output layers have R sets of device buffers and
+ * the passes go round them (a small network then reads memory, not the last-level cache). The report lists the plan like
+ * nnf_backend_run_schema, then "launches: N" (kernels one pass launches), "plan_steps: N" (steps of the plan that launch
+ * something; steps handed to the kernels together share launches), "resident_packets: R", "timed_entries: N",
  * "wall_seconds_per_pass: S" (device synchronisation on both sides of the timed passes),
  * "device_seconds_per_pass: S" (events on the kernel stream) and "host_seconds_per_pass: S" (what the calling thread
  * spends enqueuing a pass while the device runs behind it). Inputs whose data pointers are equal are fine: the

@@ -29,10 +29,11 @@ class Output(ctypes.Structure):
 
 
 class Options(ctypes.Structure):
-    _fields_ = [("fuse", ctypes.c_int32), ("dont_share_buffers", ctypes.c_int32), ("max_entry_count", ctypes.c_int32),
+    _fields_ = [("struct_size", ctypes.c_uint32), ("fuse", ctypes.c_int32), ("dont_share_buffers", ctypes.c_int32), ("max_entry_count", ctypes.c_int32),
                 ("profile", ctypes.c_int32), ("weights_from_folder", ctypes.c_int32), ("weights_folder", ctypes.c_char_p),
                 ("profile_folder", ctypes.c_char_p), ("stat_on_host", ctypes.c_int32), ("kernel_stream_count", ctypes.c_int32),
-                ("one_launch_per_group", ctypes.c_int32), ("host_thread_count", ctypes.c_int32)]
+                ("one_launch_per_group", ctypes.c_int32), ("host_thread_count", ctypes.c_int32), ("max_io_staging_mb", ctypes.c_int32),
+                ("resident_packets", ctypes.c_int32)]
 
 
 class DatasetFile(ctypes.Structure):
@@ -86,8 +87,12 @@ def load():
 
 
 def _options(fuse=True, dont_share_buffers=False, max_entry_count=0, profile=False, weights_folder=None,
-             profile_folder=None, stat_on_host=False, kernel_stream_count=0, one_launch_per_group=False, host_thread_count=0):
+             profile_folder=None, stat_on_host=False, kernel_stream_count=0, one_launch_per_group=False, host_thread_count=0,
+             max_io_staging_mb=0, resident_packets=0):
     o = Options()
+    o.struct_size = ctypes.sizeof(Options)
+    o.max_io_staging_mb = int(max_io_staging_mb)
+    o.resident_packets = int(resident_packets)
     o.fuse = int(fuse)
     o.dont_share_buffers = int(dont_share_buffers)
     o.max_entry_count = int(max_entry_count)
@@ -154,7 +159,7 @@ def parse_report(text):
             layers, _, sources = desc.partition(" <- ")
             res["steps"].append({"fused": kind == "fused", "layers": layers.split("+"), "inputs": sources.split(", "), "stream": int(stream),
                                  "run": int(run) if run else None})
-        elif key in ("per_entry_bytes", "max_entry_count", "entries", "writer_entries", "launches", "timed_entries"):
+        elif key in ("per_entry_bytes", "max_entry_count", "entries", "writer_entries", "launches", "timed_entries", "packet_entries", "plan_steps", "resident_packets"):
             res[key] = int(rest)
         elif key in ("wall_seconds_per_pass", "device_seconds_per_pass", "host_seconds_per_pass"):
             res[key] = float(rest)

@@ -111,7 +111,7 @@ namespace nnf
 			return NNF_HIP_ETOOBIG;
 		const uint32_t vectors = static_cast<uint32_t>(bytes / 16);
 		const uint32_t per_block = copy_block_size * copy_unroll;
-		hipLaunchKernelGGL(copy_kernel_impl, dim3((vectors + per_block - 1) / per_block), dim3(copy_block_size), 0, stream,
+		NNF_LAUNCH(copy_kernel_impl, dim3((vectors + per_block - 1) / per_block), dim3(copy_block_size), 0, stream,
 			static_cast<floatx4*>(dst), static_cast<const floatx4*>(src), vectors);
 		return launch_status();
 	}
@@ -304,7 +304,7 @@ extern "C"
 		if (device_mismatch_counts == nullptr)
 			return NNF_HIP_EINVAL;
 		static_assert(sizeof(unsigned long long) == sizeof(uint64_t), "counter width");
-		hipLaunchKernelGGL(division_check_kernel, dim3(4096), dim3(256), 0, static_cast<hipStream_t>(stream),
+		NNF_LAUNCH(division_check_kernel, dim3(4096), dim3(256), 0, static_cast<hipStream_t>(stream),
 			reinterpret_cast<unsigned long long*>(device_mismatch_counts));
 		return launch_status();
 	}
@@ -589,8 +589,16 @@ extern "C"
 		}
 	}
 
+	int nnf_hip_launch_count(uint64_t* count)
+	{
+		if (count == nullptr)
+			return NNF_HIP_EINVAL;
+		*count = launches_of_this_thread();
+		return NNF_HIP_OK;
+	}
+
 	const char* nnf_hip_version(void)
 	{
-		return "nnforge_hip 0.1 (gfx950)";
+		return "nnforge_hip 0.2 (gfx950)";
 	}
 }

@@ -971,10 +971,10 @@ namespace nnf
 			if (shape.persistent)
 			{
 				const uint32_t grid = std::min(p.tiles, compute_unit_count() * persistent_workgroups_per_compute_unit);
-				hipLaunchKernelGGL(pick_persistent_kernel(p.input_count), dim3(grid), dim3(shape.block), p.lds_bytes, stream, p.a, p.tiles);
+				NNF_LAUNCH(pick_persistent_kernel(p.input_count), dim3(grid), dim3(shape.block), p.lds_bytes, stream, p.a, p.tiles);
 				return launch_status();
 			}
-			hipLaunchKernelGGL(pick_kernel(p.input_count, p.shape, p.direct, p.program), dim3(p.tiles), dim3(shape.block), p.lds_bytes, stream, p.a);
+			NNF_LAUNCH(pick_kernel(p.input_count, p.shape, p.direct, p.program), dim3(p.tiles), dim3(shape.block), p.lds_bytes, stream, p.a);
 			return launch_status();
 		}
 
@@ -1153,7 +1153,7 @@ namespace nnf
 			const uint32_t all_groups = (1u << b.count) - 1u;
 			const int direct_mode = (b.direct_mask == all_groups) ? 1 : ((b.direct_mask == 0) ? 0 : 2);
 			const chain_batch_kernel_fn kernel = one_kind ? pick_batch_kernel(lead.input_count, lead.shape, direct_mode) : pick_batch_mixed_kernel(direct_mode);
-			hipLaunchKernelGGL(kernel, dim3(static_cast<uint32_t>(tiles)), dim3(launch_shapes[lead.shape].block), lds_bytes, stream, b);
+			NNF_LAUNCH(kernel, dim3(static_cast<uint32_t>(tiles)), dim3(launch_shapes[lead.shape].block), lds_bytes, stream, b);
 			const int rc = launch_status();
 			if (rc != NNF_HIP_OK)
 				return rc;

@@ -105,6 +105,15 @@ namespace nnf
 		return count;
 	}
 
+	// Kernels the library has launched from the calling thread (nnf_hip_launch_count): every launch goes through NNF_LAUNCH.
+	inline uint64_t& launches_of_this_thread()
+	{
+		static thread_local uint64_t count = 0;
+		return count;
+	}
+
+#define NNF_LAUNCH(...) do { ++::nnf::launches_of_this_thread(); hipLaunchKernelGGL(__VA_ARGS__); } while (0)
+
 	// Launch errors are reported by hipGetLastError right after the launch; asynchronous faults
 	// surface at the caller's next synchronising call, as with any HIP work.
 	inline int launch_status()

@@ -141,9 +141,9 @@ namespace nnf
 				continue;
 			const dim3 grid(blocks, std::min(entry_count, 65535u));
 			if (vector)
-				hipLaunchKernelGGL(concat_kernel<4>, grid, dim3(concat_block_size), 0, stream, a);
+				NNF_LAUNCH(concat_kernel<4>, grid, dim3(concat_block_size), 0, stream, a);
 			else
-				hipLaunchKernelGGL(concat_kernel<1>, grid, dim3(concat_block_size), 0, stream, a);
+				NNF_LAUNCH(concat_kernel<1>, grid, dim3(concat_block_size), 0, stream, a);
 			const int status = launch_status();
 			if (status != NNF_HIP_OK)
 				return status;

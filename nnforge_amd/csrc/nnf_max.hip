@@ -993,15 +993,15 @@ namespace nnf
 			const dim3 g(grid), b(block);
 			if (is_min)
 			{
-				if (w2) hipLaunchKernelGGL((tiling2d_kernel<window_op_min, 2, 2, block>), g, b, lds_bytes, stream, a);
-				else if (w3) hipLaunchKernelGGL((tiling2d_kernel<window_op_min, 3, 3, block>), g, b, lds_bytes, stream, a);
-				else hipLaunchKernelGGL((tiling2d_kernel<window_op_min, 0, 0, block>), g, b, lds_bytes, stream, a);
+				if (w2) NNF_LAUNCH((tiling2d_kernel<window_op_min, 2, 2, block>), g, b, lds_bytes, stream, a);
+				else if (w3) NNF_LAUNCH((tiling2d_kernel<window_op_min, 3, 3, block>), g, b, lds_bytes, stream, a);
+				else NNF_LAUNCH((tiling2d_kernel<window_op_min, 0, 0, block>), g, b, lds_bytes, stream, a);
 			}
 			else
 			{
-				if (w2) hipLaunchKernelGGL((tiling2d_kernel<window_op_max, 2, 2, block>), g, b, lds_bytes, stream, a);
-				else if (w3) hipLaunchKernelGGL((tiling2d_kernel<window_op_max, 3, 3, block>), g, b, lds_bytes, stream, a);
-				else hipLaunchKernelGGL((tiling2d_kernel<window_op_max, 0, 0, block>), g, b, lds_bytes, stream, a);
+				if (w2) NNF_LAUNCH((tiling2d_kernel<window_op_max, 2, 2, block>), g, b, lds_bytes, stream, a);
+				else if (w3) NNF_LAUNCH((tiling2d_kernel<window_op_max, 3, 3, block>), g, b, lds_bytes, stream, a);
+				else NNF_LAUNCH((tiling2d_kernel<window_op_max, 0, 0, block>), g, b, lds_bytes, stream, a);
 			}
 			return true;
 		}
@@ -1079,11 +1079,11 @@ namespace nnf
 			a.mult = mult;
 			const dim3 grid((a.row_vectors + max_block_size - 1) / max_block_size, min(a.out_rows, 65535u));
 			if (op == window_op_sum)
-				hipLaunchKernelGGL(window_rows_kernel<window_op_sum>, grid, dim3(max_block_size), 0, stream, a);
+				NNF_LAUNCH(window_rows_kernel<window_op_sum>, grid, dim3(max_block_size), 0, stream, a);
 			else if (op == window_op_min)
-				hipLaunchKernelGGL(window_rows_kernel<window_op_min>, grid, dim3(max_block_size), 0, stream, a);
+				NNF_LAUNCH(window_rows_kernel<window_op_min>, grid, dim3(max_block_size), 0, stream, a);
 			else
-				hipLaunchKernelGGL(window_rows_kernel<window_op_max>, grid, dim3(max_block_size), 0, stream, a);
+				NNF_LAUNCH(window_rows_kernel<window_op_max>, grid, dim3(max_block_size), 0, stream, a);
 			return true;
 		}
 
@@ -1152,18 +1152,18 @@ namespace nnf
 			const bool w3 = (a.win_w == 3) && (a.win_h == 3), w2 = (a.win_w == 2) && (a.win_h == 2);
 			if (pro.need_exp)
 			{
-				if (w3) hipLaunchKernelGGL((max_window2d_exp_prologue_kernel<OP, 3, 3, TRUNC, UNIFORM>), g, b, lds_bytes, stream, a, pro);
-				else if (w2) hipLaunchKernelGGL((max_window2d_exp_prologue_kernel<OP, 2, 2, TRUNC, UNIFORM>), g, b, lds_bytes, stream, a, pro);
-				else hipLaunchKernelGGL((max_window2d_exp_prologue_kernel<OP, 0, 0, TRUNC, UNIFORM>), g, b, lds_bytes, stream, a, pro);
+				if (w3) NNF_LAUNCH((max_window2d_exp_prologue_kernel<OP, 3, 3, TRUNC, UNIFORM>), g, b, lds_bytes, stream, a, pro);
+				else if (w2) NNF_LAUNCH((max_window2d_exp_prologue_kernel<OP, 2, 2, TRUNC, UNIFORM>), g, b, lds_bytes, stream, a, pro);
+				else NNF_LAUNCH((max_window2d_exp_prologue_kernel<OP, 0, 0, TRUNC, UNIFORM>), g, b, lds_bytes, stream, a, pro);
 			}
 			else
 			{
 				const bool pair = pairs_of_outputs(a);
-				if (w3 && pair) hipLaunchKernelGGL((max_window2d_prologue_kernel<OP, 3, 3, TRUNC, UNIFORM, true>), g, b, lds_bytes, stream, a, pro);
-				else if (w2 && pair) hipLaunchKernelGGL((max_window2d_prologue_kernel<OP, 2, 2, TRUNC, UNIFORM, true>), g, b, lds_bytes, stream, a, pro);
-				else if (w3) hipLaunchKernelGGL((max_window2d_prologue_kernel<OP, 3, 3, TRUNC, UNIFORM>), g, b, lds_bytes, stream, a, pro);
-				else if (w2) hipLaunchKernelGGL((max_window2d_prologue_kernel<OP, 2, 2, TRUNC, UNIFORM>), g, b, lds_bytes, stream, a, pro);
-				else hipLaunchKernelGGL((max_window2d_prologue_kernel<OP, 0, 0, TRUNC, UNIFORM>), g, b, lds_bytes, stream, a, pro);
+				if (w3 && pair) NNF_LAUNCH((max_window2d_prologue_kernel<OP, 3, 3, TRUNC, UNIFORM, true>), g, b, lds_bytes, stream, a, pro);
+				else if (w2 && pair) NNF_LAUNCH((max_window2d_prologue_kernel<OP, 2, 2, TRUNC, UNIFORM, true>), g, b, lds_bytes, stream, a, pro);
+				else if (w3) NNF_LAUNCH((max_window2d_prologue_kernel<OP, 3, 3, TRUNC, UNIFORM>), g, b, lds_bytes, stream, a, pro);
+				else if (w2) NNF_LAUNCH((max_window2d_prologue_kernel<OP, 2, 2, TRUNC, UNIFORM>), g, b, lds_bytes, stream, a, pro);
+				else NNF_LAUNCH((max_window2d_prologue_kernel<OP, 0, 0, TRUNC, UNIFORM>), g, b, lds_bytes, stream, a, pro);
 			}
 		}
 
@@ -1180,15 +1180,15 @@ namespace nnf
 			}
 			const bool pair = pairs_of_outputs(a);
 			if ((a.win_w == 3) && (a.win_h == 3) && pair)
-				hipLaunchKernelGGL((max_window2d_kernel<OP, 3, 3, TRUNC, true>), dim3(grid), dim3(max_block_size), lds_bytes, stream, a);
+				NNF_LAUNCH((max_window2d_kernel<OP, 3, 3, TRUNC, true>), dim3(grid), dim3(max_block_size), lds_bytes, stream, a);
 			else if ((a.win_w == 2) && (a.win_h == 2) && pair)
-				hipLaunchKernelGGL((max_window2d_kernel<OP, 2, 2, TRUNC, true>), dim3(grid), dim3(max_block_size), lds_bytes, stream, a);
+				NNF_LAUNCH((max_window2d_kernel<OP, 2, 2, TRUNC, true>), dim3(grid), dim3(max_block_size), lds_bytes, stream, a);
 			else if ((a.win_w == 3) && (a.win_h == 3))
-				hipLaunchKernelGGL((max_window2d_kernel<OP, 3, 3, TRUNC>), dim3(grid), dim3(max_block_size), lds_bytes, stream, a);
+				NNF_LAUNCH((max_window2d_kernel<OP, 3, 3, TRUNC>), dim3(grid), dim3(max_block_size), lds_bytes, stream, a);
 			else if ((a.win_w == 2) && (a.win_h == 2))
-				hipLaunchKernelGGL((max_window2d_kernel<OP, 2, 2, TRUNC>), dim3(grid), dim3(max_block_size), lds_bytes, stream, a);
+				NNF_LAUNCH((max_window2d_kernel<OP, 2, 2, TRUNC>), dim3(grid), dim3(max_block_size), lds_bytes, stream, a);
 			else
-				hipLaunchKernelGGL((max_window2d_kernel<OP, 0, 0, TRUNC>), dim3(grid), dim3(max_block_size), lds_bytes, stream, a);
+				NNF_LAUNCH((max_window2d_kernel<OP, 0, 0, TRUNC>), dim3(grid), dim3(max_block_size), lds_bytes, stream, a);
 		}
 
 		// LDS floats a workgroup of the 2-D kernel stages (measured best of 2048 ... 12288 on the ResNet stem's pooling)
@@ -1388,9 +1388,9 @@ namespace nnf
 		nd.in_plane = static_cast<uint32_t>(in_plane);
 		const dim3 grid((nd.output_count + max_block_size - 1) / max_block_size);
 		if (is_min)
-			hipLaunchKernelGGL(window_nd_kernel<window_op_min>, grid, dim3(max_block_size), 0, stream, nd);
+			NNF_LAUNCH(window_nd_kernel<window_op_min>, grid, dim3(max_block_size), 0, stream, nd);
 		else
-			hipLaunchKernelGGL(window_nd_kernel<window_op_max>, grid, dim3(max_block_size), 0, stream, nd);
+			NNF_LAUNCH(window_nd_kernel<window_op_max>, grid, dim3(max_block_size), 0, stream, nd);
 		return launch_status();
 	}
 
@@ -1450,9 +1450,9 @@ namespace nnf
 		nd.tile_count = static_cast<uint32_t>(tile_count);
 		const dim3 grid((nd.output_count + max_block_size - 1) / max_block_size);
 		if (is_min)
-			hipLaunchKernelGGL((window_nd_kernel<window_op_min, true>), grid, dim3(max_block_size), 0, stream, nd);
+			NNF_LAUNCH((window_nd_kernel<window_op_min, true>), grid, dim3(max_block_size), 0, stream, nd);
 		else
-			hipLaunchKernelGGL((window_nd_kernel<window_op_max, true>), grid, dim3(max_block_size), 0, stream, nd);
+			NNF_LAUNCH((window_nd_kernel<window_op_max, true>), grid, dim3(max_block_size), 0, stream, nd);
 		return launch_status();
 	}
 
@@ -1520,7 +1520,7 @@ namespace nnf
 			input_feature_map_count, out_fm, in_plane, feature_map_subsampling_size, entry_subsampling_size))
 			return launch_status();
 		const dim3 grid((nd.output_count + max_block_size - 1) / max_block_size);
-		hipLaunchKernelGGL(window_nd_kernel<window_op_sum>, grid, dim3(max_block_size), 0, stream, nd);
+		NNF_LAUNCH(window_nd_kernel<window_op_sum>, grid, dim3(max_block_size), 0, stream, nd);
 		return launch_status();
 	}
 
@@ -1558,12 +1558,12 @@ namespace nnf
 		if ((group % 4) == 0)
 		{
 			const dim3 grid((group / 4 + max_block_size - 1) / max_block_size, rows);
-			hipLaunchKernelGGL(maxout_vec4_kernel, grid, dim3(max_block_size), 0, stream, output, input, entry_count, group, feature_map_subsampling_size);
+			NNF_LAUNCH(maxout_vec4_kernel, grid, dim3(max_block_size), 0, stream, output, input, entry_count, group, feature_map_subsampling_size);
 		}
 		else
 		{
 			const dim3 grid((group + max_block_size - 1) / max_block_size, rows);
-			hipLaunchKernelGGL(maxout_scalar_kernel, grid, dim3(max_block_size), 0, stream, output, input, entry_count, group, feature_map_subsampling_size);
+			NNF_LAUNCH(maxout_scalar_kernel, grid, dim3(max_block_size), 0, stream, output, input, entry_count, group, feature_map_subsampling_size);
 		}
 		return launch_status();
 	}

@@ -407,7 +407,7 @@ namespace nnf
 			if (pro == nullptr)
 			{
 				const window_prologue none = {};
-				hipLaunchKernelGGL((global_pool_linear_kernel<false, false, false>), grid, block, lds_bytes, stream, output, input, input2, plane_count, plane, plane_magic, mult, none);
+				NNF_LAUNCH((global_pool_linear_kernel<false, false, false>), grid, block, lds_bytes, stream, output, input, input2, plane_count, plane, plane_magic, mult, none);
 				return;
 			}
 			auto kernel = global_pool_linear_kernel<true, false, false>;
@@ -415,7 +415,7 @@ namespace nnf
 				kernel = join ? global_pool_linear_kernel<true, true, true> : global_pool_linear_kernel<true, true, false>;
 			else if (join)
 				kernel = global_pool_linear_kernel<true, false, true>;
-			hipLaunchKernelGGL(kernel, grid, block, lds_bytes, stream, output, input, input2, plane_count, plane, plane_magic, mult, *pro);
+			NNF_LAUNCH(kernel, grid, block, lds_bytes, stream, output, input, input2, plane_count, plane, plane_magic, mult, *pro);
 		}
 
 		// 64 planes of 7x7; fewer of larger planes, so that a compute unit holds several workgroups
@@ -530,7 +530,7 @@ namespace nnf
 					kernel = join ? global_pool_prologue_kernel<true, true> : global_pool_prologue_kernel<true, false>;
 				else if (join)
 					kernel = global_pool_prologue_kernel<false, true>;
-				hipLaunchKernelGGL(kernel, grid, dim3(pool_block_size), lds_bytes, stream, output, input, input2, plane_count, plane, plane_magic, mult, planes_per_group, pro);
+				NNF_LAUNCH(kernel, grid, dim3(pool_block_size), lds_bytes, stream, output, input, input2, plane_count, plane, plane_magic, mult, planes_per_group, pro);
 				return launch_status();
 			}
 			if (join)
@@ -552,7 +552,7 @@ namespace nnf
 			const dim3 grid((plane_count + planes_per_group - 1) / planes_per_group);
 			// plane >= 2 here: a 1x1 window over a 1x1 plane takes the general kernel
 			const uint32_t plane_magic = static_cast<uint32_t>(((1ull << 32) + plane - 1) / plane);
-			hipLaunchKernelGGL(global_pool_kernel, grid, dim3(pool_block_size), lds_bytes, stream, output, input, plane_count, plane, plane_magic, mult, planes_per_group);
+			NNF_LAUNCH(global_pool_kernel, grid, dim3(pool_block_size), lds_bytes, stream, output, input, plane_count, plane, plane_magic, mult, planes_per_group);
 		}
 		else if (window2d_launch(stream, 4, mult, output, input, static_cast<uint32_t>(input_total), plane_count,
 			input_width, input_height, output_width, output_height, window_width, window_height, window_width, window_height))
@@ -562,7 +562,7 @@ namespace nnf
 		else
 		{
 			const dim3 grid((output_count + pool_block_size - 1) / pool_block_size);
-			hipLaunchKernelGGL(window_pool_kernel, grid, dim3(pool_block_size), 0, stream, output, input, output_count,
+			NNF_LAUNCH(window_pool_kernel, grid, dim3(pool_block_size), 0, stream, output, input, output_count,
 				input_width, input_height, output_width, output_height, window_width, window_height, mult);
 		}
 		return launch_status();

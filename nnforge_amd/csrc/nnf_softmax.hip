@@ -534,19 +534,19 @@ namespace nnf
 			const uint32_t rows_per_block = block / THREADS;
 			const dim3 grid((rows + rows_per_block - 1) / rows_per_block);
 			if (vectors_per_lane <= 1)
-				hipLaunchKernelGGL((softmax_rows_kernel<THREADS, 1, W>), grid, dim3(block), 0, stream, out, in, rows, fm_count);
+				NNF_LAUNCH((softmax_rows_kernel<THREADS, 1, W>), grid, dim3(block), 0, stream, out, in, rows, fm_count);
 			else if (vectors_per_lane <= 2)
-				hipLaunchKernelGGL((softmax_rows_kernel<THREADS, 2, W>), grid, dim3(block), 0, stream, out, in, rows, fm_count);
+				NNF_LAUNCH((softmax_rows_kernel<THREADS, 2, W>), grid, dim3(block), 0, stream, out, in, rows, fm_count);
 			else if (vectors_per_lane <= 4)
-				hipLaunchKernelGGL((softmax_rows_kernel<THREADS, 4, W>), grid, dim3(block), 0, stream, out, in, rows, fm_count);
+				NNF_LAUNCH((softmax_rows_kernel<THREADS, 4, W>), grid, dim3(block), 0, stream, out, in, rows, fm_count);
 			else
-				hipLaunchKernelGGL((softmax_rows_kernel<THREADS, 8, W>), grid, dim3(block), 0, stream, out, in, rows, fm_count);
+				NNF_LAUNCH((softmax_rows_kernel<THREADS, 8, W>), grid, dim3(block), 0, stream, out, in, rows, fm_count);
 		}
 
 		template<int THREADS, int W>
 		void launch_one_vector_per_lane(hipStream_t stream, float* out, const float* in, uint32_t rows, uint32_t fm_count)
 		{
-			hipLaunchKernelGGL((softmax_rows_kernel<THREADS, 1, W>), dim3(rows), dim3(THREADS), 0, stream, out, in, rows, fm_count);
+			NNF_LAUNCH((softmax_rows_kernel<THREADS, 1, W>), dim3(rows), dim3(THREADS), 0, stream, out, in, rows, fm_count);
 		}
 
 		// Few rows cannot fill the machine with one wavefront each, and what a launch then costs is
@@ -620,7 +620,7 @@ namespace nnf
 			else
 				launched = try_launch_rows<1>(stream, output, input, entry_count, feature_map_count);
 			if (!launched)
-				hipLaunchKernelGGL(softmax_long_rows_kernel, dim3(entry_count), dim3(1024), 0, stream, output, input, feature_map_count);
+				NNF_LAUNCH(softmax_long_rows_kernel, dim3(entry_count), dim3(1024), 0, stream, output, input, feature_map_count);
 		}
 		else
 		{
@@ -637,23 +637,23 @@ namespace nnf
 				if (staged_bytes <= staged_bytes_limit)
 				{
 					if (positions == 64)
-						hipLaunchKernelGGL((softmax_columns_sliced_kernel<64, true>), sliced_grid, dim3(256), staged_bytes, stream,
+						NNF_LAUNCH((softmax_columns_sliced_kernel<64, true>), sliced_grid, dim3(256), staged_bytes, stream,
 							output, input, columns, feature_map_count, neuron_count_per_feature_map);
 					else if (positions == 32)
-						hipLaunchKernelGGL((softmax_columns_sliced_kernel<32, true>), sliced_grid, dim3(256), staged_bytes, stream,
+						NNF_LAUNCH((softmax_columns_sliced_kernel<32, true>), sliced_grid, dim3(256), staged_bytes, stream,
 							output, input, columns, feature_map_count, neuron_count_per_feature_map);
 					else
-						hipLaunchKernelGGL((softmax_columns_sliced_kernel<16, true>), sliced_grid, dim3(256), staged_bytes, stream,
+						NNF_LAUNCH((softmax_columns_sliced_kernel<16, true>), sliced_grid, dim3(256), staged_bytes, stream,
 							output, input, columns, feature_map_count, neuron_count_per_feature_map);
 					return launch_status();
 				}
 				if (columns <= sliced_columns_limit)
 				{
 					if (columns >= 64u * 512u)
-						hipLaunchKernelGGL((softmax_columns_sliced_kernel<64, false>), dim3((columns + 63) / 64), dim3(256), 0, stream,
+						NNF_LAUNCH((softmax_columns_sliced_kernel<64, false>), dim3((columns + 63) / 64), dim3(256), 0, stream,
 							output, input, columns, feature_map_count, neuron_count_per_feature_map);
 					else
-						hipLaunchKernelGGL((softmax_columns_sliced_kernel<16, false>), dim3((columns + 15) / 16), dim3(256), 0, stream,
+						NNF_LAUNCH((softmax_columns_sliced_kernel<16, false>), dim3((columns + 15) / 16), dim3(256), 0, stream,
 							output, input, columns, feature_map_count, neuron_count_per_feature_map);
 					return launch_status();
 				}
@@ -668,29 +668,29 @@ namespace nnf
 				const uint32_t quads = columns / 4;
 				const dim3 quad_grid((quads + 255) / 256);
 				if (feature_map_count <= 2)
-					hipLaunchKernelGGL(softmax_columns_vec4_kernel<2>, quad_grid, dim3(256), 0, stream, output, input, quads, feature_map_count, neuron_count_per_feature_map);
+					NNF_LAUNCH(softmax_columns_vec4_kernel<2>, quad_grid, dim3(256), 0, stream, output, input, quads, feature_map_count, neuron_count_per_feature_map);
 				else if (feature_map_count <= 4)
-					hipLaunchKernelGGL(softmax_columns_vec4_kernel<4>, quad_grid, dim3(256), 0, stream, output, input, quads, feature_map_count, neuron_count_per_feature_map);
+					NNF_LAUNCH(softmax_columns_vec4_kernel<4>, quad_grid, dim3(256), 0, stream, output, input, quads, feature_map_count, neuron_count_per_feature_map);
 				else if (feature_map_count <= 8)
-					hipLaunchKernelGGL(softmax_columns_vec4_kernel<8>, quad_grid, dim3(256), 0, stream, output, input, quads, feature_map_count, neuron_count_per_feature_map);
+					NNF_LAUNCH(softmax_columns_vec4_kernel<8>, quad_grid, dim3(256), 0, stream, output, input, quads, feature_map_count, neuron_count_per_feature_map);
 				else
-					hipLaunchKernelGGL(softmax_columns_vec4_kernel<16>, quad_grid, dim3(256), 0, stream, output, input, quads, feature_map_count, neuron_count_per_feature_map);
+					NNF_LAUNCH(softmax_columns_vec4_kernel<16>, quad_grid, dim3(256), 0, stream, output, input, quads, feature_map_count, neuron_count_per_feature_map);
 				return launch_status();
 			}
 			if (feature_map_count <= 2)
-				hipLaunchKernelGGL(softmax_columns_kernel<2>, grid, block, 0, stream, output, input, columns, feature_map_count, neuron_count_per_feature_map);
+				NNF_LAUNCH(softmax_columns_kernel<2>, grid, block, 0, stream, output, input, columns, feature_map_count, neuron_count_per_feature_map);
 			else if (feature_map_count <= 4)
-				hipLaunchKernelGGL(softmax_columns_kernel<4>, grid, block, 0, stream, output, input, columns, feature_map_count, neuron_count_per_feature_map);
+				NNF_LAUNCH(softmax_columns_kernel<4>, grid, block, 0, stream, output, input, columns, feature_map_count, neuron_count_per_feature_map);
 			else if (feature_map_count <= 8)
-				hipLaunchKernelGGL(softmax_columns_kernel<8>, grid, block, 0, stream, output, input, columns, feature_map_count, neuron_count_per_feature_map);
+				NNF_LAUNCH(softmax_columns_kernel<8>, grid, block, 0, stream, output, input, columns, feature_map_count, neuron_count_per_feature_map);
 			else if (feature_map_count <= 16)
-				hipLaunchKernelGGL(softmax_columns_kernel<16>, grid, block, 0, stream, output, input, columns, feature_map_count, neuron_count_per_feature_map);
+				NNF_LAUNCH(softmax_columns_kernel<16>, grid, block, 0, stream, output, input, columns, feature_map_count, neuron_count_per_feature_map);
 			else if (feature_map_count <= 32)
-				hipLaunchKernelGGL(softmax_columns_kernel<32>, grid, block, 0, stream, output, input, columns, feature_map_count, neuron_count_per_feature_map);
+				NNF_LAUNCH(softmax_columns_kernel<32>, grid, block, 0, stream, output, input, columns, feature_map_count, neuron_count_per_feature_map);
 			else if (feature_map_count <= 64)
-				hipLaunchKernelGGL(softmax_columns_kernel<64>, grid, block, 0, stream, output, input, columns, feature_map_count, neuron_count_per_feature_map);
+				NNF_LAUNCH(softmax_columns_kernel<64>, grid, block, 0, stream, output, input, columns, feature_map_count, neuron_count_per_feature_map);
 			else
-				hipLaunchKernelGGL(softmax_columns_kernel<0>, grid, block, 0, stream, output, input, columns, feature_map_count, neuron_count_per_feature_map);
+				NNF_LAUNCH(softmax_columns_kernel<0>, grid, block, 0, stream, output, input, columns, feature_map_count, neuron_count_per_feature_map);
 		}
 		return launch_status();
 	}

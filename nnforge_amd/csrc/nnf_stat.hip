@@ -281,7 +281,7 @@ namespace nnf
 			return NNF_HIP_EINVAL;
 		if (!is_aligned16(device_stats))
 			return NNF_HIP_EALIGN;
-		hipLaunchKernelGGL(stat_init_kernel, dim3((feature_map_count + stat_block_size - 1) / stat_block_size), dim3(stat_block_size), 0, stream,
+		NNF_LAUNCH(stat_init_kernel, dim3((feature_map_count + stat_block_size - 1) / stat_block_size), dim3(stat_block_size), 0, stream,
 			device_stats, feature_map_count);
 		const int status = launch_status();
 		// Set-up of the statistics path on this device: the address of its static scratch array is looked up here,
@@ -349,20 +349,20 @@ namespace nnf
 			{
 				const uint32_t units = neuron_count_per_feature_map / 4;
 				const uint32_t magic = (units >= 2) ? static_cast<uint32_t>(((1ull << 32) + units - 1) / units) : 0u;
-				hipLaunchKernelGGL(stat_runs_kernel<4>, grid, dim3(stat_block_size), 0, stream, partial, input, entry_count, feature_map_count,
+				NNF_LAUNCH(stat_runs_kernel<4>, grid, dim3(stat_block_size), 0, stream, partial, input, entry_count, feature_map_count,
 					neuron_count_per_feature_map, p.entries_per_run, magic, p.segments, p.units_per_segment);
 			}
 			else
 			{
 				const uint32_t units = neuron_count_per_feature_map;
 				const uint32_t magic = (units >= 2) ? static_cast<uint32_t>(((1ull << 32) + units - 1) / units) : 0u;
-				hipLaunchKernelGGL(stat_runs_kernel<1>, grid, dim3(stat_block_size), 0, stream, partial, input, entry_count, feature_map_count,
+				NNF_LAUNCH(stat_runs_kernel<1>, grid, dim3(stat_block_size), 0, stream, partial, input, entry_count, feature_map_count,
 					neuron_count_per_feature_map, p.entries_per_run, magic, p.segments, p.units_per_segment);
 			}
 			int status = launch_status();
 			if (status != NNF_HIP_OK)
 				return status;
-			hipLaunchKernelGGL(stat_merge_kernel, dim3((feature_map_count + stat_block_size - 1) / stat_block_size), dim3(stat_block_size), 0, stream,
+			NNF_LAUNCH(stat_merge_kernel, dim3((feature_map_count + stat_block_size - 1) / stat_block_size), dim3(stat_block_size), 0, stream,
 				device_stats, partial, feature_map_count, p.runs * p.segments);
 			return launch_status();
 		}

@@ -57,6 +57,22 @@ namespace
 		}
 		out << "per_entry_bytes: " << fp.get_per_entry_buffer_bytes() << "\n";
 		out << "max_entry_count: " << fp.get_max_entry_count() << "\n";
+		if (fp.get_packet_entry_count() > 0)
+			out << "packet_entries: " << fp.get_packet_entry_count() << "\n"; // of the latest run()
+	}
+
+	// The caller's options as this library's structure: struct_size bytes of it are the caller's, the members behind
+	// them (added since the caller was built) are zero, which is every member's "default" value.
+	const nnf_backend_options * checked_options(const nnf_backend_options * caller_options, nnf_backend_options& storage)
+	{
+		if (caller_options == nullptr)
+			return nullptr;
+		if ((caller_options->struct_size < 2 * sizeof(uint32_t)) || (caller_options->struct_size > 4096))
+			throw neural_network_exception("nnf_backend_options.struct_size is " + std::to_string(caller_options->struct_size)
+				+ ": set it to sizeof(nnf_backend_options) of the header the caller was built with");
+		std::memset(&storage, 0, sizeof(storage));
+		std::memcpy(&storage, caller_options, std::min<size_t>(caller_options->struct_size, sizeof(storage)));
+		return &storage;
 	}
 
 	void apply_options(hip::factory_generator_hip& generator, const nnf_backend_options * options)
@@ -64,6 +80,8 @@ namespace
 		generator.apply_default_options();
 		if (options != nullptr)
 		{
+			if (options->max_io_staging_mb != 0)
+				generator.hip_max_io_staging_mb = std::max(0, options->max_io_staging_mb);
 			generator.hip_fuse = options->fuse != 0;
 			generator.hip_dont_share_buffers = options->dont_share_buffers != 0;
 			if (options->max_entry_count > 0)
@@ -169,11 +187,13 @@ extern "C"
 		const nnf_backend_input* inputs, uint32_t input_count,
 		uint32_t entry_count,
 		nnf_backend_output* outputs, uint32_t output_count,
-		const nnf_backend_options* options,
+		const nnf_backend_options* caller_options,
 		char* report, size_t report_capacity)
 	{
 		return guarded([&](std::ostream& out)
 		{
+			nnf_backend_options option_storage;
+			const nnf_backend_options * const options = checked_options(caller_options, option_storage);
 			const network_schema schema = parse_schema(schema_text);
 			if ((outputs == nullptr) || (output_count == 0))
 				throw neural_network_exception("No output layers specified for forward_propagation");
@@ -229,11 +249,13 @@ extern "C"
 		const nnf_backend_dataset_file* inputs, uint32_t input_count,
 		const nnf_backend_dataset_file* outputs, uint32_t output_count,
 		uint32_t compact_samples,
-		const nnf_backend_options* options,
+		const nnf_backend_options* caller_options,
 		char* report, size_t report_capacity)
 	{
 		return guarded([&](std::ostream& out)
 		{
+			nnf_backend_options option_storage;
+			const nnf_backend_options * const options = checked_options(caller_options, option_storage);
 			const network_schema schema = parse_schema(schema_text);
 			if ((outputs == nullptr) || (output_count == 0))
 				throw neural_network_exception("No output layers specified for forward_propagation");
@@ -340,11 +362,13 @@ extern "C"
 		uint32_t entry_count,
 		const char* layer_name, uint32_t feature_map_count,
 		float* min_values, float* max_values, float* averages, float* std_devs,
-		const nnf_backend_options* options,
+		const nnf_backend_options* caller_options,
 		char* report, size_t report_capacity)
 	{
 		return guarded([&](std::ostream& out)
 		{
+			nnf_backend_options option_storage;
+			const nnf_backend_options * const options = checked_options(caller_options, option_storage);
 			const network_schema schema = parse_schema(schema_text);
 			if (layer_name == nullptr)
 				throw neural_network_exception("No output layers specified for forward_propagation");
@@ -391,12 +415,14 @@ extern "C"
 		const nnf_backend_weights* weights, uint32_t weights_count,
 		const nnf_backend_input* inputs, uint32_t input_count,
 		uint32_t entry_count,
-		const nnf_backend_options* options,
+		const nnf_backend_options* caller_options,
 		const char* out_folder,
 		char* report, size_t report_capacity)
 	{
 		return guarded([&](std::ostream& out)
 		{
+			nnf_backend_options option_storage;
+			const nnf_backend_options * const options = checked_options(caller_options, option_storage);
 			const network_schema schema = parse_schema(schema_text);
 			if (out_folder == nullptr)
 				throw neural_network_exception("No folder given for the refreshed weights");
@@ -420,12 +446,14 @@ extern "C"
 		const char* schema_text,
 		const nnf_backend_input* inputs, uint32_t input_count,
 		const char* const* output_layer_names, uint32_t output_count,
-		const nnf_backend_options* options,
+		const nnf_backend_options* caller_options,
 		uint64_t memory_bytes,
 		char* report, size_t report_capacity)
 	{
 		return guarded([&](std::ostream& out)
 		{
+			nnf_backend_options option_storage;
+			const nnf_backend_options * const options = checked_options(caller_options, option_storage);
 			const network_schema schema = parse_schema(schema_text);
 			std::vector<std::string> output_names;
 			for(uint32_t i = 0; i < output_count; ++i)
@@ -448,12 +476,14 @@ extern "C"
 		const nnf_backend_input* inputs, uint32_t input_count,
 		uint32_t entry_count,
 		const char* const* output_layer_names, uint32_t output_count,
-		const nnf_backend_options* options,
+		const nnf_backend_options* caller_options,
 		uint32_t warmup, uint32_t passes,
 		char* report, size_t report_capacity)
 	{
 		return guarded([&](std::ostream& out)
 		{
+			nnf_backend_options option_storage;
+			const nnf_backend_options * const options = checked_options(caller_options, option_storage);
 			const network_schema schema = parse_schema(schema_text);
 			std::vector<std::string> output_names;
 			for(uint32_t i = 0; i < output_count; ++i)
@@ -473,9 +503,12 @@ extern "C"
 			hip::forward_propagation_hip * hfp = dynamic_cast<hip::forward_propagation_hip *>(fp.get());
 			if (hfp == nullptr)
 				throw neural_network_exception("The factory did not make a forward_propagation_hip");
-			const hip::forward_propagation_hip::kernel_timing t = hfp->time_kernels(reader, entry_count, warmup, passes);
+			const unsigned int resident_packets = ((options != nullptr) && (options->resident_packets > 0)) ? static_cast<unsigned int>(options->resident_packets) : 1U;
+			const hip::forward_propagation_hip::kernel_timing t = hfp->time_kernels(reader, entry_count, warmup, passes, resident_packets);
 			describe_plan(*hfp, out);
 			out << "launches: " << t.launch_count << "\n";
+			out << "plan_steps: " << t.plan_step_count << "\n";
+			out << "resident_packets: " << t.resident_packets << "\n";
 			out << "timed_entries: " << t.entry_count << "\n";
 			out.precision(9);
 			out << "wall_seconds_per_pass: " << t.wall_seconds_per_pass << "\n";

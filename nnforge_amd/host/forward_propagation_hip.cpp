@@ -117,12 +117,13 @@ namespace nnforge
 		{
 			unsigned int packet = 0;
 			int slot_count = 0;
+			int staging_slot_count = 0;
 			bool with_output_staging = false;
 			bool stats_on_device = false;
-			std::vector<hip_linear_buffer_device::ptr> buffers[2];
+			std::vector<std::vector<hip_linear_buffer_device::ptr> > buffers; // per slot
 			std::vector<std::pair<hip_linear_buffer_device::ptr, hip_linear_buffer_device::ptr> > temporary;
 			std::vector<std::vector<const float *> > chunk_ptrs; // weight pointers of the fused steps
-			std::map<std::string, std::unique_ptr<pinned_buffer> > staging[2];
+			std::vector<std::map<std::string, std::unique_ptr<pinned_buffer> > > staging; // per staging slot
 			std::map<std::string, hip_linear_buffer_device::ptr> stat_states, stat_workspaces;
 			std::map<std::string, size_t> stat_workspace_bytes;
 		};
@@ -995,10 +996,13 @@ namespace nnforge
 			};
 		}
 
-		forward_propagation_hip::run_buffers& forward_propagation_hip::prepare_run(unsigned int packet, int slot_count, bool with_output_staging, bool stats_on_device)
+		forward_propagation_hip::run_buffers& forward_propagation_hip::prepare_run(unsigned int packet, int slot_count, bool with_output_staging, bool stats_on_device,
+			int staging_slot_count)
 		{
 			hip_config->set_device();
-			if (kept_run && (kept_run->packet == packet) && (kept_run->slot_count == slot_count)
+			if (staging_slot_count <= 0)
+				staging_slot_count = slot_count;
+			if (kept_run && (kept_run->packet == packet) && (kept_run->slot_count == slot_count) && (kept_run->staging_slot_count == staging_slot_count)
 				&& (kept_run->with_output_staging == with_output_staging) && (kept_run->stats_on_device == stats_on_device))
 				return *kept_run;
 			kept_run.reset(); // what the run before held goes first: both sets need not fit side by side
@@ -1006,6 +1010,9 @@ namespace nnforge
 			run_buffers& r = *fresh;
 			r.packet = packet;
 			r.slot_count = slot_count;
+			r.staging_slot_count = staging_slot_count;
+			r.buffers.resize(static_cast<size_t>(slot_count));
+			r.staging.resize(static_cast<size_t>(staging_slot_count));
 			r.with_output_staging = with_output_staging;
 			r.stats_on_device = stats_on_device;
 			unsigned int stream_count = 1;
@@ -1025,10 +1032,13 @@ namespace nnforge
 			{
 				const size_t bytes = p->buffer_floats_per_entry[b] * sizeof(float) * packet;
 				r.buffers[0].push_back(hip_linear_buffer_device::ptr(new hip_linear_buffer_device(bytes)));
-				if ((slot_count > 1) && (io_buffers.find(static_cast<int>(b)) != io_buffers.end()))
-					r.buffers[1].push_back(hip_linear_buffer_device::ptr(new hip_linear_buffer_device(bytes)));
-				else
-					r.buffers[1].push_back(r.buffers[0].back());
+				for(int s = 1; s < slot_count; ++s)
+				{
+					if (io_buffers.find(static_cast<int>(b)) != io_buffers.end())
+						r.buffers[s].push_back(hip_linear_buffer_device::ptr(new hip_linear_buffer_device(bytes)));
+					else
+						r.buffers[s].push_back(r.buffers[0].back());
+				}
 			}
 			for(const step_plan& plan : p->plans)
 			{
@@ -1051,7 +1061,7 @@ namespace nnforge
 						r.chunk_ptrs[i].push_back(static_cast<const float *>(*b));
 
 			// pinned staging per I/O slot: the data layers, and the output layers unless only their statistics are wanted
-			for(int s = 0; s < slot_count; ++s)
+			for(int s = 0; s < staging_slot_count; ++s)
 			{
 				for(const std::string& n : data_layer_names)
 					r.staging[s][n].reset(new pinned_buffer(static_cast<size_t>(layer_config_map[n].get_neuron_count()) * sizeof(float) * packet));
@@ -1111,7 +1121,10 @@ namespace nnforge
 			// with them (reading, writing) bounds the run, not the kernels: packets are kept small enough for reading,
 			// copying, computing and writing of neighbouring packets to overlap. Measured with BatchNorm -> ReLU on
 			// 64 x 56 x 56 entries (0.8 MB in, 0.8 MB out per entry), 1024 entries: 12.6 GB/s of input + output with 51 MB of
-			// staging per slot, 13.3 with 103 MB, 8.8 with 205 MB, 3.7 with all 1024 entries as one packet.
+			// staging per slot, 13.3 with 103 MB, 8.8 with 205 MB, 3.7 with all 1024 entries as one packet. The bound
+			// (hip_max_io_staging_mb) never makes a packet smaller than a few entries: a network with many or large data
+			// layers would otherwise run its launch plan entry by entry, where launches are what a pass costs.
+			if (hip_config->max_io_staging_bytes > 0)
 			{
 				size_t io_bytes_per_entry = 0;
 				for(const std::string& n : data_layer_names)
@@ -1119,12 +1132,15 @@ namespace nnforge
 				if (!stats_on_device)
 					for(const std::string& n : output_layer_names)
 						io_bytes_per_entry += static_cast<size_t>(layer_config_map[n].get_neuron_count()) * sizeof(float) * output_layers_tiling_factor;
-				packet = std::min(packet, static_cast<unsigned int>(std::max<size_t>(1, max_io_staging_bytes_per_slot / std::max<size_t>(1, io_bytes_per_entry))));
+				const size_t fit = hip_config->max_io_staging_bytes / std::max<size_t>(1, io_bytes_per_entry);
+				const unsigned int floor_entries = std::min(packet, hip_running_configuration::min_packet_entries_under_staging_bound);
+				packet = std::max(floor_entries, std::min(packet, static_cast<unsigned int>(std::min<size_t>(fit, 0xFFFFFFFFu))));
 			}
+			packet_entry_count = packet;
 
 			constexpr int slot_count = 2;
 			run_buffers& r = prepare_run(packet, slot_count, !stats_on_device, stats_on_device);
-			std::map<std::string, std::unique_ptr<pinned_buffer> > (&staging)[2] = r.staging;
+			std::vector<std::map<std::string, std::unique_ptr<pinned_buffer> > >& staging = r.staging;
 			std::map<std::string, hip_linear_buffer_device::ptr>& stat_states = r.stat_states;
 			std::map<std::string, hip_linear_buffer_device::ptr>& stat_workspaces = r.stat_workspaces;
 			std::map<std::string, size_t>& stat_workspace_bytes = r.stat_workspace_bytes;
@@ -1216,9 +1232,27 @@ namespace nnforge
 					to_read = std::min(packet, static_cast<unsigned int>(reader_entry_count) - std::min(read_total, static_cast<unsigned int>(reader_entry_count)));
 				reads.entry_read.assign(to_read, 0);
 				reads.errors.assign(to_read, std::exception_ptr());
-				reads.pending = to_read;
 				for(unsigned int i = 0; i < to_read; ++i)
 				{
+					// counted before it is posted and taken back if posting fails: the destructor of `reads` waits for
+					// exactly the jobs that exist
+					{
+						std::lock_guard<std::mutex> lock(reads.m);
+						++reads.pending;
+					}
+					struct uncount_unless_posted
+					{
+						packet_reads& reads;
+						bool posted = false;
+						~uncount_unless_posted()
+						{
+							if (!posted)
+							{
+								std::lock_guard<std::mutex> lock(reads.m);
+								--reads.pending;
+							}
+						}
+					} guard{reads};
 					job_runner->post([this, &reads, &reader, &staging, slot, i, read_total]()
 					{
 						try
@@ -1236,6 +1270,7 @@ namespace nnforge
 						if (--reads.pending == 0)
 							reads.done.notify_all();
 					});
+					guard.posted = true;
 				}
 
 				// while the entries are read, the packet before goes to the writer
@@ -1336,17 +1371,18 @@ namespace nnforge
 		}
 
 		forward_propagation_hip::kernel_timing forward_propagation_hip::time_kernels(
-			structured_data_bunch_reader& reader, unsigned int entry_count, unsigned int warmup, unsigned int passes)
+			structured_data_bunch_reader& reader, unsigned int entry_count, unsigned int warmup, unsigned int passes, unsigned int resident_packets)
 		{
 			if (hip_config->is_offline())
 				throw neural_network_exception("This forward_propagation_hip was created for planning only (offline configuration): it cannot run");
 			set_input_configuration_specific(reader.get_config_map());
 			const unsigned int packet = std::min(std::max(1U, entry_count), max_entry_count);
-			run_buffers& r = prepare_run(packet, 1, false, false);
+			const int slot_count = static_cast<int>(std::max(1U, std::min(resident_packets, 64U)));
+			run_buffers& r = prepare_run(packet, slot_count, false, false, 1);
 			drain_streams drain_on_exit;
 			drain_on_exit.streams = p->kernel_streams;
 
-			// one packet, read and uploaded once
+			// one packet, read once and uploaded to every slot
 			unsigned int entries_read = 0;
 			{
 				std::map<std::string, std::unique_ptr<pinned_buffer> >& staging = r.staging[0];
@@ -1360,28 +1396,38 @@ namespace nnforge
 				}
 				if (entries_read == 0)
 					throw neural_network_exception("time_kernels: the reader holds no entries");
-				for(const std::string& n : data_layer_names)
-					hip_safe_call(nnf_hip_memcpy_h2d(*r.buffers[0][p->value_to_buffer[n]], staging[n]->ptr,
-						static_cast<size_t>(layer_config_map[n].get_neuron_count()) * sizeof(float) * entries_read, nullptr));
+				for(int slot = 0; slot < slot_count; ++slot)
+					for(const std::string& n : data_layer_names)
+						hip_safe_call(nnf_hip_memcpy_h2d(*r.buffers[slot][p->value_to_buffer[n]], staging[n]->ptr,
+							static_cast<size_t>(layer_config_map[n].get_neuron_count()) * sizeof(float) * entries_read, nullptr));
 			}
 
 			hip_event start, stop;
 			// A pass after a pass needs no wait between them: all steps that touch a buffer share a kernel stream,
 			// which runs in order. (Every pass still ends with the main stream waiting for the others, as a packet does.)
+			unsigned int pass_id = 0;
 			auto one_pass = [&]()
 			{
-				p->enqueue_plan(r.buffers[0], entries_read, r.chunk_ptrs, r.temporary, nullptr);
+				p->enqueue_plan(r.buffers[pass_id % static_cast<unsigned int>(slot_count)], entries_read, r.chunk_ptrs, r.temporary, nullptr);
+				++pass_id;
 			};
 			hip_safe_call(nnf_hip_device_synchronize());
+			kernel_timing res;
+			res.entry_count = entries_read;
+			res.resident_packets = static_cast<unsigned int>(slot_count);
+			res.plan_step_count = 0;
+			for(const step_plan& plan : p->plans)
+				res.plan_step_count += plan.launches_nothing() ? 0 : 1;
+			// what a pass launches: the kernels the library starts from this thread while one pass is enqueued
+			uint64_t launches_before = 0, launches_after = 0;
+			hip_safe_call(nnf_hip_launch_count(&launches_before));
+			one_pass();
+			hip_safe_call(nnf_hip_launch_count(&launches_after));
+			res.launch_count = static_cast<unsigned int>(launches_after - launches_before);
 			for(unsigned int i = 0; i < warmup; ++i)
 				one_pass();
 			hip_safe_call(nnf_hip_device_synchronize());
 
-			kernel_timing res;
-			res.entry_count = entries_read;
-			res.launch_count = 0;
-			for(const step_plan& plan : p->plans)
-				res.launch_count += plan.launches_nothing() ? 0 : 1;
 			const std::chrono::high_resolution_clock::time_point t0 = std::chrono::high_resolution_clock::now();
 			hip_safe_call(nnf_hip_event_record(start.ev, p->stream));
 			for(size_t ks = 1; ks < p->kernel_streams.size(); ++ks)
@@ -1427,16 +1473,19 @@ namespace nnforge
 			, hip_kernel_stream_count(hip_running_configuration::default_kernel_stream_count)
 			, hip_max_entry_count(4096)
 			, hip_reserved_thread_count(1)
+			, hip_max_io_staging_mb(64)
 		{
 		}
 
 		void factory_generator_hip::initialize()
 		{
 			hip::init();
-			hip_config = hip_running_configuration::const_ptr(new hip_running_configuration(
+			std::shared_ptr<hip_running_configuration> config(new hip_running_configuration(
 				hip_device_id, hip_max_global_memory_usage_ratio, hip_fuse, hip_dont_share_buffers, hip_max_entry_count,
 				hip_single_command_stream ? 1 : std::max(1, hip_kernel_stream_count), hip_batch_independent_groups,
 				static_cast<unsigned int>(std::max(0, hip_reserved_thread_count))));
+			config->max_io_staging_bytes = static_cast<size_t>(std::max(0, hip_max_io_staging_mb)) << 20;
+			hip_config = config;
 		}
 
 		forward_propagation_factory::ptr factory_generator_hip::create_forward_propagation_factory() const
@@ -1481,6 +1530,7 @@ namespace nnforge
 			res.push_back(int_option("hip_max_entry_count", &hip_max_entry_count, 4096, "Upper bound of entries processed per packet"));
 			res.push_back(int_option("hip_kernel_stream_count", &hip_kernel_stream_count, hip_running_configuration::default_kernel_stream_count, "Streams the kernels of independent layers are spread over"));
 			res.push_back(int_option("hip_reserved_thread_count", &hip_reserved_thread_count, 1, "The number of hw threads not used for input data processing"));
+			res.push_back(int_option("hip_max_io_staging_mb", &hip_max_io_staging_mb, 64, "Pinned staging per I/O slot, in MB, that bounds the entries of a packet (0: no bound)"));
 			return res;
 		}
 	}

@@ -7,6 +7,7 @@
 
 #include <atomic>
 #include <cstdio>
+#include <cstddef>
 #include <cstring>
 #include <string>
 #include <vector>
@@ -56,6 +57,7 @@ layer { type: "Softmax" name: "prob" input_layer_name: "sig" }
 		const char * outputs[1] = { "prob" };
 		nnf_backend_options options;
 		std::memset(&options, 0, sizeof(options));
+		options.struct_size = sizeof(options);
 		options.fuse = fuse;
 		std::vector<char> buffer(1 << 16);
 		const int rc = nnf_backend_plan_schema(text.c_str(), &input, 1, outputs, 1, &options, 1ull << 30, buffer.data(), buffer.size());
@@ -76,6 +78,25 @@ int main(int argc, char ** argv)
 		expect(plan(good, size, size, report, 1) == 0, "plan with fusion: " + report);
 		expect(report.find("bn+relu+pool1") != std::string::npos, "the pooling layer takes the group in front of it along: " + report);
 		expect(plan(good, size, size, report, 0) == 0, "plan without fusion: " + report);
+	}
+	// options without their size are refused; options of an older, shorter header are taken with the later members at their defaults
+	{
+		const uint32_t dims[2] = { 28, 28 };
+		nnf_backend_input input = { "conv1", 8, 2, dims, nullptr };
+		const char * outputs[1] = { "prob" };
+		std::vector<char> buffer(1 << 16);
+		nnf_backend_options options;
+		std::memset(&options, 0xFF, sizeof(options)); // whatever lies behind a shorter structure must not be read
+		options.struct_size = 0;
+		expect(nnf_backend_plan_schema(good.c_str(), &input, 1, outputs, 1, &options, 1ull << 30, buffer.data(), buffer.size()) != 0, "options with struct_size 0 are refused");
+		expect(std::string(buffer.data()).find("struct_size") != std::string::npos, std::string("the refusal names struct_size: ") + buffer.data());
+		options.struct_size = offsetof(nnf_backend_options, max_entry_count) + sizeof(options.max_entry_count);
+		options.fuse = 1;
+		options.dont_share_buffers = 0;
+		options.max_entry_count = 7;
+		expect(nnf_backend_plan_schema(good.c_str(), &input, 1, outputs, 1, &options, 1ull << 30, buffer.data(), buffer.size()) == 0, std::string("options of a shorter header: ") + buffer.data());
+		expect(std::string(buffer.data()).find("max_entry_count: 7") != std::string::npos, std::string("... are honoured as far as they go: ") + buffer.data());
+		expect(std::string(buffer.data()).find(" #") != std::string::npos, std::string("... and the members behind them take their defaults (groups launched together): ") + buffer.data());
 	}
 	// sizes the layers reject
 	expect(plan(good, 2, 2, report) != 0, "an input smaller than the windows is refused");

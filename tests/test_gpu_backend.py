@@ -408,11 +408,28 @@ def test_resnet50_post_convolution_graph_layer_by_layer(mode):
             assert_bits(got[name], values[name], name)
 
 
+def test_packets_under_the_staging_bound_keep_a_few_entries():
+    """hip_max_io_staging_mb bounds the pinned staging of a packet, but not below eight entries: entries of 12.6 MB in and
+    12.6 MB out would fit 64 MB two at a time. Twelve entries then go as packets of eight and four; with the bound lifted
+    as one packet of twelve; with hip_max_entry_count = 5 as packets of five (the bound never raises a packet)."""
+    gen = T.rng(63, 1)
+    n, c, size = 12, 3, 1024
+    layers = [S.L("Data", "x"), S.L("BatchNorm", "bn", ["x"], feature_map_count=c), S.L("ReLU", "act", ["bn"])]
+    weights = S.make_weights(layers, gen)
+    inputs = {"x": T.normal(gen, (n, c, size, size))}
+    values = S.evaluate(layers, weights, inputs)
+    for options, packet in (({}, 8), ({"max_io_staging_mb": -1}, 12), ({"max_entry_count": 5}, 5), ({"max_io_staging_mb": 1024}, 12)):
+        got, rep = run(layers, weights, inputs, ["act"], values, **options)
+        assert rep["packet_entries"] == packet, (options, rep["raw"])
+        assert_bits(got["act"], values["act"], str(options))
+
+
 def test_resnet50_post_convolution_graph_at_64_entries():
-    """Config 4 at its full size through the driver, one packet of 64 entries, the default launch plan (six runs of
-    groups launched together, tiles of every ResNet-50 shape by the hundred thousand per launch): every output against
-    the oracle run layer by layer, bit for bit (softmax to 1e-5). Inputs are cut out of one pool of normal values at
-    offsets of their own (what is compared is arithmetic and indexing, not statistics)."""
+    """Config 4 at its full size through the driver, one packet of 64 entries (the bound on a packet's pinned staging is
+    lifted for it: 54 data layers of 44 MB of input per entry would otherwise make packets of 8), the default launch
+    plan (six runs of groups launched together, tiles of every ResNet-50 shape by the hundred thousand per launch):
+    every output against the oracle run layer by layer, bit for bit (softmax to 1e-5). Inputs are cut out of one pool
+    of normal values at offsets of their own (what is compared is arithmetic and indexing, not statistics)."""
     from nnforge_amd import schemas
 
     gen = T.rng(62, 64)
@@ -426,8 +443,9 @@ def test_resnet50_post_convolution_graph_at_64_entries():
         start = (7919 * (i + 1)) % 65536
         inputs[name] = np.resize(pool[start:], count).reshape(n, fm, dims[1], dims[0])
     values = S.evaluate(layers, weights, inputs)
-    got, rep = run(layers, weights, inputs, outputs, values, max_entry_count=n)
+    got, rep = run(layers, weights, inputs, outputs, values, max_entry_count=n, max_io_staging_mb=-1)
     assert rep["entries"] == n and rep["max_entry_count"] == n and len(rep["steps"]) == 50
+    assert rep["packet_entries"] == n  # the launches compared below are the launches of 64 entries, not 64 times those of one
     assert len({s["run"] for s in rep["steps"]} - {None}) == 6
     for name in outputs:
         if name == "prob":
