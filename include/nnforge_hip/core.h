@@ -155,6 +155,7 @@ namespace nnforge
 	{
 		std::map<std::string, std::string> scalars;
 		std::vector<std::string> scalar_order; // the keys in the order set() received them: the order a writer emits
+		std::set<std::string> quoted;          // scalars that stood in quotes in the text a reader parsed (the values are kept without them)
 		std::vector<std::pair<std::string, schema_param_block> > blocks;
 
 		// the first nested message of that name, null when there is none

@@ -19,6 +19,31 @@ namespace nnforge
 		static const std::string layer_type_name;
 	};
 
+	// A layer of a type this backend has no class for (convolution, local contrast subtraction, error functions ...).
+	// It keeps the type name, the inputs and the parameter messages as the schema file states them, so that such a
+	// schema can be read, planned around and written back. It computes nothing: in a forward_propagation its output
+	// arrives as data under the layer's own name, like a data layer's (the reference's own example does this by hand:
+	// examples/gtsrb/working_data/schema_tail.txt:10-13 declares "tanh_3_layer" as a Data layer), with the configuration
+	// the reader states for it; what only such layers read is not computed. network_schema::read_proto makes these
+	// for unregistered types when asked to; by default an unregistered type is an error, as in the reference.
+	class external_layer : public layer
+	{
+	public:
+		explicit external_layer(const std::string& type_name);
+		layer::ptr clone() const override;
+		std::string get_type_name() const override;
+		// throws: the configuration of an external layer's output is the caller's to state
+		layer_configuration_specific get_output_layer_configuration_specific(
+			const std::vector<layer_configuration_specific>& input_configuration_specific_list) const override;
+		float get_forward_flops_per_entry(const std::vector<layer_configuration_specific>&) const override { return 0.0F; }
+		void read_proto(const void * layer_proto) override;  // keeps every nested message of the layer's block
+		void write_proto(void * layer_proto) const override; // and writes them back
+		std::vector<std::string> get_parameter_strings() const override;
+
+		std::string type_name;
+		schema_param_block params; // the "<type>_param { ... }" messages, verbatim
+	};
+
 	// Four weight chunks of feature_map_count floats: gamma, beta, mean, inverse standard
 	// deviation (nnforge/batch_norm_layer.h:26, batch_norm_layer.cpp:96-106). epsilon is carried
 	// for schema round trips only; inference never reads it.

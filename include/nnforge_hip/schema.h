@@ -23,14 +23,20 @@ namespace nnforge
 
 		// protobuf text format of nnforge/proto/nnforge.proto:5-42 (NetworkSchema { name, layer { type,
 		// name, input_layer_name*, <type>_param { ... } } }); the sample file of the reference is
-		// examples/gtsrb/working_data/schema.txt. Layer types not registered in layer_factory throw.
-		void read_proto(std::istream& stream_to_read_from);
+		// examples/gtsrb/working_data/schema.txt. Layer types not registered in layer_factory throw ("No layer is
+		// registered with type ...", nnforge/layer_factory.cpp) unless keep_unregistered_layers is set: then such a
+		// layer becomes an external_layer, which keeps its block of the file and computes nothing.
+		void read_proto(std::istream& stream_to_read_from, bool keep_unregistered_layers = false);
 		void write_proto(std::ostream& stream_to_write_to) const;
 
-		// layers needed to compute the given outputs, in forward propagation order
+		// Layers needed to compute the given outputs, in forward propagation order. The search stops at external layers:
+		// their output comes from outside, so what they read is not needed on their account, and they appear in the
+		// result without inputs - as sources of data beside the data layers.
 		std::vector<layer::const_ptr> get_required_layers(const std::vector<std::string>& output_layer_names) const;
+		bool has_external_layers() const;
 
 		std::vector<layer::const_ptr> get_layers() const { return layers; }
+		// layers without inputs: their values come from the reader
 		std::vector<layer::const_ptr> get_data_layers() const;
 		// inputs always precede their consumers; data layers included
 		std::vector<layer::const_ptr> get_layers_in_forward_propagation_order() const;

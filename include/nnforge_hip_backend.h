@@ -66,6 +66,11 @@ typedef struct nnf_backend_options
 	int32_t max_io_staging_mb;     /* hip_max_io_staging_mb: pinned staging (input + output entries) per I/O slot that bounds a
 	                                  packet of run(); 0: default (64), < 0: no bound */
 	int32_t resident_packets;      /* nnf_backend_time_kernels: sets of data / output buffers the timed passes go round; <= 0: 1 */
+	int32_t keep_unregistered_layers; /* 1: a layer of a type this backend has no class for (Convolution, LCS, LError ...) does not
+	                                  make the schema an error: it is kept as it stands in the file and computes nothing - its
+	                                  output comes in as an input under the layer's own name, with the configuration given for
+	                                  it, and what only such layers read is neither wanted nor computed. 0: such a type is an
+	                                  error ("No layer is registered with type ..."), as in the reference */
 } nnf_backend_options;
 
 /* Runs the schema on device 0. The report lists one line per launch ("step: ..."), the buffer plan
@@ -163,8 +168,13 @@ NNF_BACKEND_API int nnf_backend_plan_schema(
 	char* report, size_t report_capacity);
 
 /* Parses a schema and writes it back in text format (round trip of the reader/writer). A buffer too
- * small for the whole text is an error (the message says how many bytes are needed). */
-NNF_BACKEND_API int nnf_backend_rewrite_schema(const char* schema_text, char* out_text, size_t out_capacity);
+ * small for the whole text is an error (the message says how many bytes are needed). keep_unregistered_layers: as in
+ * nnf_backend_options; the layers kept that way are written back with the parameter messages they were read with. */
+NNF_BACKEND_API int nnf_backend_rewrite_schema(const char* schema_text, int32_t keep_unregistered_layers, char* out_text, size_t out_capacity);
+
+/* Parses a schema and lists its layers in forward propagation order, a line each:
+ * "layer: <type>\t<name>\t<input names, comma separated>\t<the layer's parameter strings, joined by '; '>\t<own|external>". */
+NNF_BACKEND_API int nnf_backend_list_layers(const char* schema_text, int32_t keep_unregistered_layers, char* report, size_t report_capacity);
 
 /* Writes / reads <layer>.data files in nnForge's format (weights in, weights out through `weights`
  * arrays owned by the caller; reading fills caller-provided chunks and checks their sizes). */

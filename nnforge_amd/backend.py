@@ -33,7 +33,7 @@ class Options(ctypes.Structure):
                 ("profile", ctypes.c_int32), ("weights_from_folder", ctypes.c_int32), ("weights_folder", ctypes.c_char_p),
                 ("profile_folder", ctypes.c_char_p), ("stat_on_host", ctypes.c_int32), ("kernel_stream_count", ctypes.c_int32),
                 ("one_launch_per_group", ctypes.c_int32), ("host_thread_count", ctypes.c_int32), ("max_io_staging_mb", ctypes.c_int32),
-                ("resident_packets", ctypes.c_int32)]
+                ("resident_packets", ctypes.c_int32), ("keep_unregistered_layers", ctypes.c_int32)]
 
 
 class DatasetFile(ctypes.Structure):
@@ -67,7 +67,8 @@ def load():
         lib.nnf_backend_time_kernels.argtypes = [ctypes.c_char_p, ctypes.POINTER(Weights), ctypes.c_uint32, ctypes.POINTER(Input),
                                                  ctypes.c_uint32, ctypes.c_uint32, ctypes.POINTER(ctypes.c_char_p), ctypes.c_uint32,
                                                  ctypes.POINTER(Options), ctypes.c_uint32, ctypes.c_uint32, ctypes.c_char_p, ctypes.c_size_t]
-        lib.nnf_backend_rewrite_schema.argtypes = [ctypes.c_char_p, ctypes.c_char_p, ctypes.c_size_t]
+        lib.nnf_backend_rewrite_schema.argtypes = [ctypes.c_char_p, ctypes.c_int32, ctypes.c_char_p, ctypes.c_size_t]
+        lib.nnf_backend_list_layers.argtypes = [ctypes.c_char_p, ctypes.c_int32, ctypes.c_char_p, ctypes.c_size_t]
         lib.nnf_backend_write_weights.argtypes = [ctypes.c_char_p, ctypes.POINTER(Weights), ctypes.c_uint32, ctypes.c_char_p, ctypes.c_size_t]
         lib.nnf_backend_read_weights.argtypes = [ctypes.c_char_p, ctypes.c_char_p, ctypes.c_uint32, _UP, ctypes.POINTER(_FP),
                                                  ctypes.c_char_p, ctypes.c_size_t]
@@ -88,8 +89,9 @@ def load():
 
 def _options(fuse=True, dont_share_buffers=False, max_entry_count=0, profile=False, weights_folder=None,
              profile_folder=None, stat_on_host=False, kernel_stream_count=0, one_launch_per_group=False, host_thread_count=0,
-             max_io_staging_mb=0, resident_packets=0):
+             max_io_staging_mb=0, resident_packets=0, keep_unregistered_layers=False):
     o = Options()
+    o.keep_unregistered_layers = int(keep_unregistered_layers)
     o.struct_size = ctypes.sizeof(Options)
     o.max_io_staging_mb = int(max_io_staging_mb)
     o.resident_packets = int(resident_packets)
@@ -274,13 +276,27 @@ def time_kernels(schema_text, weights, inputs, output_names, warmup=2, passes=5,
     return parse_report(report.value.decode())
 
 
-def rewrite_schema(schema_text):
+def rewrite_schema(schema_text, keep_unregistered_layers=False):
     lib = load()
     out = ctypes.create_string_buffer(REPORT_CAPACITY)
-    rc = lib.nnf_backend_rewrite_schema(schema_text.encode(), out, REPORT_CAPACITY)
+    rc = lib.nnf_backend_rewrite_schema(schema_text.encode(), int(keep_unregistered_layers), out, REPORT_CAPACITY)
     if rc != 0:
         raise BackendError(rc, out.value.decode(errors="replace"))
     return out.value.decode()
+
+
+def list_layers(schema_text, keep_unregistered_layers=False):
+    """-> [{"type", "name", "inputs", "parameters", "external"}] in forward propagation order"""
+    lib = load()
+    out = ctypes.create_string_buffer(REPORT_CAPACITY)
+    rc = lib.nnf_backend_list_layers(schema_text.encode(), int(keep_unregistered_layers), out, REPORT_CAPACITY)
+    if rc != 0:
+        raise BackendError(rc, out.value.decode(errors="replace"))
+    res = []
+    for line in out.value.decode().splitlines():
+        kind, name, inputs, params, origin = line[len("layer: "):].split("\t")
+        res.append({"type": kind, "name": name, "inputs": inputs.split(",") if inputs else [], "parameters": params, "external": origin == "external"})
+    return res
 
 
 def write_weights(folder, weights):

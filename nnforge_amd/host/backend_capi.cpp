@@ -23,14 +23,14 @@ namespace
 		dst[n] = '\0';
 	}
 
-	network_schema parse_schema(const char * schema_text)
+	network_schema parse_schema(const char * schema_text, bool keep_unregistered_layers)
 	{
 		hip::init(); // idempotent: registration ignores duplicates
 		if (schema_text == nullptr)
 			throw neural_network_exception("schema text is null");
 		std::istringstream in(schema_text);
 		network_schema schema;
-		schema.read_proto(in);
+		schema.read_proto(in, keep_unregistered_layers);
 		return schema;
 	}
 
@@ -194,7 +194,7 @@ extern "C"
 		{
 			nnf_backend_options option_storage;
 			const nnf_backend_options * const options = checked_options(caller_options, option_storage);
-			const network_schema schema = parse_schema(schema_text);
+			const network_schema schema = parse_schema(schema_text, (options != nullptr) && (options->keep_unregistered_layers != 0));
 			if ((outputs == nullptr) || (output_count == 0))
 				throw neural_network_exception("No output layers specified for forward_propagation");
 
@@ -256,7 +256,7 @@ extern "C"
 		{
 			nnf_backend_options option_storage;
 			const nnf_backend_options * const options = checked_options(caller_options, option_storage);
-			const network_schema schema = parse_schema(schema_text);
+			const network_schema schema = parse_schema(schema_text, (options != nullptr) && (options->keep_unregistered_layers != 0));
 			if ((outputs == nullptr) || (output_count == 0))
 				throw neural_network_exception("No output layers specified for forward_propagation");
 			std::vector<std::string> output_names;
@@ -369,7 +369,7 @@ extern "C"
 		{
 			nnf_backend_options option_storage;
 			const nnf_backend_options * const options = checked_options(caller_options, option_storage);
-			const network_schema schema = parse_schema(schema_text);
+			const network_schema schema = parse_schema(schema_text, (options != nullptr) && (options->keep_unregistered_layers != 0));
 			if (layer_name == nullptr)
 				throw neural_network_exception("No output layers specified for forward_propagation");
 			hip::factory_generator_hip generator;
@@ -423,7 +423,7 @@ extern "C"
 		{
 			nnf_backend_options option_storage;
 			const nnf_backend_options * const options = checked_options(caller_options, option_storage);
-			const network_schema schema = parse_schema(schema_text);
+			const network_schema schema = parse_schema(schema_text, (options != nullptr) && (options->keep_unregistered_layers != 0));
 			if (out_folder == nullptr)
 				throw neural_network_exception("No folder given for the refreshed weights");
 			hip::factory_generator_hip generator;
@@ -454,7 +454,7 @@ extern "C"
 		{
 			nnf_backend_options option_storage;
 			const nnf_backend_options * const options = checked_options(caller_options, option_storage);
-			const network_schema schema = parse_schema(schema_text);
+			const network_schema schema = parse_schema(schema_text, (options != nullptr) && (options->keep_unregistered_layers != 0));
 			std::vector<std::string> output_names;
 			for(uint32_t i = 0; i < output_count; ++i)
 				output_names.push_back(output_layer_names[i]);
@@ -484,7 +484,7 @@ extern "C"
 		{
 			nnf_backend_options option_storage;
 			const nnf_backend_options * const options = checked_options(caller_options, option_storage);
-			const network_schema schema = parse_schema(schema_text);
+			const network_schema schema = parse_schema(schema_text, (options != nullptr) && (options->keep_unregistered_layers != 0));
 			std::vector<std::string> output_names;
 			for(uint32_t i = 0; i < output_count; ++i)
 				output_names.push_back(output_layer_names[i]);
@@ -517,11 +517,30 @@ extern "C"
 		}, report, report_capacity);
 	}
 
-	int nnf_backend_rewrite_schema(const char* schema_text, char* out_text, size_t out_capacity)
+	int nnf_backend_list_layers(const char* schema_text, int32_t keep_unregistered_layers, char* report, size_t report_capacity)
 	{
 		return guarded([&](std::ostream& out)
 		{
-			const network_schema schema = parse_schema(schema_text);
+			const network_schema schema = parse_schema(schema_text, keep_unregistered_layers != 0);
+			for(const layer::const_ptr& l : schema.get_layers_in_forward_propagation_order())
+			{
+				out << "layer: " << l->get_type_name() << "\t" << l->instance_name << "\t";
+				for(size_t i = 0; i < l->input_layer_instance_names.size(); ++i)
+					out << (i == 0 ? "" : ",") << l->input_layer_instance_names[i];
+				out << "\t";
+				const std::vector<std::string> params = l->get_parameter_strings();
+				for(size_t i = 0; i < params.size(); ++i)
+					out << (i == 0 ? "" : "; ") << params[i];
+				out << "\t" << ((dynamic_cast<const external_layer *>(l.get()) != nullptr) ? "external" : "own") << "\n";
+			}
+		}, report, report_capacity);
+	}
+
+	int nnf_backend_rewrite_schema(const char* schema_text, int32_t keep_unregistered_layers, char* out_text, size_t out_capacity)
+	{
+		return guarded([&](std::ostream& out)
+		{
+			const network_schema schema = parse_schema(schema_text, keep_unregistered_layers != 0);
 			std::ostringstream text;
 			schema.write_proto(text);
 			// the text is the result: cut short it would be a different schema

@@ -290,7 +290,9 @@ namespace nnforge
 			{
 				if (l->input_layer_instance_names.empty())
 				{
-					if (l->get_type_name() != data_layer::layer_type_name)
+					// a data layer, or a layer computed elsewhere (the base class hands those over without inputs):
+					// either way the reader supplies its values
+					if ((l->get_type_name() != data_layer::layer_type_name) && (dynamic_cast<const external_layer *>(l.get()) == nullptr))
 						throw neural_network_exception("Layer " + l->instance_name + " of type " + l->get_type_name() + " has no inputs");
 					continue;
 				}

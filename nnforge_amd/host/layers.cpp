@@ -545,6 +545,37 @@ namespace nnforge
 		return std::vector<std::string>(1, res);
 	}
 
+	// ---- layers computed elsewhere -------------------------------------------------------------
+
+	external_layer::external_layer(const std::string& type_name) : type_name(type_name) {}
+	layer::ptr external_layer::clone() const { return layer::ptr(new external_layer(*this)); }
+	std::string external_layer::get_type_name() const { return type_name; }
+
+	layer_configuration_specific external_layer::get_output_layer_configuration_specific(const std::vector<layer_configuration_specific>&) const
+	{
+		throw neural_network_exception("Layer " + instance_name + " of type " + type_name
+			+ " is computed outside this backend: its output configuration has to be supplied like a data layer's");
+	}
+
+	void external_layer::read_proto(const void * layer_proto)
+	{
+		params = schema_param_block();
+		for(const std::pair<std::string, schema_param_block>& b : static_cast<const schema_param_block *>(layer_proto)->blocks)
+			if (b.first != "input_layer_name")
+				params.blocks.push_back(b);
+	}
+
+	void external_layer::write_proto(void * layer_proto) const
+	{
+		for(const std::pair<std::string, schema_param_block>& b : params.blocks)
+			static_cast<schema_param_block *>(layer_proto)->blocks.push_back(b);
+	}
+
+	std::vector<std::string> external_layer::get_parameter_strings() const
+	{
+		return std::vector<std::string>(1, "computed elsewhere");
+	}
+
 	// ---- Concat ------------------------------------------------------------------------------
 
 	const std::string concat_layer::layer_type_name = "Concat";

@@ -1,4 +1,5 @@
 #include "nnforge_hip/schema.h"
+#include "nnforge_hip/layers.h"
 
 #include <algorithm>
 #include <cctype>
@@ -138,7 +139,11 @@ namespace nnforge
 						block.blocks.back().second.scalars["value"] = v.text;
 					}
 					else
-						block.scalars[field] = v.text;
+					{
+						block.set(field, v.text);
+						if (v.kind == token::string_literal)
+							block.quoted.insert(field);
+					}
 				}
 				else
 					throw neural_network_exception("Value expected for field " + field + " in schema at line " + std::to_string(v.line));
@@ -217,7 +222,7 @@ namespace nnforge
 			name_to_index[layers[i]->instance_name] = i;
 	}
 
-	void network_schema::read_proto(std::istream& stream_to_read_from)
+	void network_schema::read_proto(std::istream& stream_to_read_from, bool keep_unregistered_layers)
 	{
 		tokenizer tk(stream_to_read_from);
 		schema_param_block root;
@@ -232,7 +237,8 @@ namespace nnforge
 			if (!lb->has("name"))
 				throw neural_network_exception("Layer without name in schema");
 			const std::string type = lb->scalars.find("type")->second;
-			layer::ptr l = layer_factory::get_singleton().create_layer(type);
+			layer::ptr l = (keep_unregistered_layers && !layer_factory::get_singleton().is_registered(type))
+				? layer::ptr(new external_layer(type)) : layer_factory::get_singleton().create_layer(type);
 			l->instance_name = lb->scalars.find("name")->second;
 			for(const schema_param_block * in : lb->children("input_layer_name"))
 				l->input_layer_instance_names.push_back(in->scalars.find("value")->second);
@@ -244,10 +250,17 @@ namespace nnforge
 
 	namespace
 	{
+		// a scalar as the text format wants it: strings (what a reader found in quotes) in quotes again
+		std::string scalar_text(const schema_param_block& block, const std::string& key)
+		{
+			const std::string& value = block.scalars.find(key)->second;
+			return (block.quoted.find(key) != block.quoted.end()) ? "\"" + value + "\"" : value;
+		}
+
 		void write_inline(std::ostream& out, const schema_param_block& block)
 		{
 			for(const std::string& key : block.scalar_order)
-				out << key << ": " << block.scalars.find(key)->second << " ";
+				out << key << ": " << scalar_text(block, key) << " ";
 			for(const std::pair<std::string, schema_param_block>& nested : block.blocks)
 			{
 				out << nested.first << " { ";
@@ -267,7 +280,7 @@ namespace nnforge
 				out << "}\n";
 			}
 			for(const std::string& key : block.scalar_order)
-				out << indent << key << ": " << block.scalars.find(key)->second << "\n";
+				out << indent << key << ": " << scalar_text(block, key) << "\n";
 		}
 	}
 
@@ -313,14 +326,34 @@ namespace nnforge
 			if (needed[cur])
 				continue;
 			needed[cur] = true;
+			if (dynamic_cast<const external_layer *>(layers[cur].get()) != nullptr)
+				continue; // its output comes from outside
 			for(const std::string& input : layers[cur]->input_layer_instance_names)
 				todo.push_back(name_to_index.find(input)->second);
 		}
 		std::vector<layer::const_ptr> res;
 		for(size_t i = 0; i < layers.size(); ++i)
-			if (needed[i])
+		{
+			if (!needed[i])
+				continue;
+			if ((dynamic_cast<const external_layer *>(layers[i].get()) != nullptr) && !layers[i]->input_layer_instance_names.empty())
+			{
+				layer::ptr source = layers[i]->clone();
+				source->input_layer_instance_names.clear();
+				res.push_back(source);
+			}
+			else
 				res.push_back(layers[i]);
+		}
 		return res;
+	}
+
+	bool network_schema::has_external_layers() const
+	{
+		for(const layer::const_ptr& l : layers)
+			if (dynamic_cast<const external_layer *>(l.get()) != nullptr)
+				return true;
+		return false;
 	}
 
 	std::vector<layer::const_ptr> network_schema::get_data_layers() const

@@ -11,6 +11,75 @@ import oracle
 from nnforge_amd.schemas import L, PARAM_BLOCK, schema_text  # noqa: F401 (re-exported: the tests build their networks with these)
 
 
+def parse_schema_text(text):
+    """A reader of nnForge's text-format schema written for the tests alone (the backend's C++ reader is what is under
+    test): -> (name, [{"type", "name", "inputs", "blocks": {message name: [fields]}}]) with fields = {field: value or
+    [values]}; repeated nested messages keep their order."""
+    import re
+
+    tokens = re.findall(r'"[^"]*"|[{}]|[^\s{}:"]+:?', text)
+    pos = 0
+
+    def message(top):
+        nonlocal pos
+        fields = []
+        while pos < len(tokens):
+            tok = tokens[pos]
+            pos += 1
+            if tok == "}":
+                assert not top
+                return fields
+            key = tok.rstrip(":")
+            if tokens[pos] == "{":
+                pos += 1
+                fields.append((key, message(False)))
+            else:
+                fields.append((key, tokens[pos].strip('"')))
+                pos += 1
+        assert top
+        return fields
+
+    root = message(True)
+    layers = []
+    for key, value in root:
+        if key != "layer":
+            continue
+        layer = {"type": None, "name": None, "inputs": [], "blocks": {}}
+        for k, v in value:
+            if k == "type":
+                layer["type"] = v
+            elif k == "name":
+                layer["name"] = v
+            elif k == "input_layer_name":
+                layer["inputs"].append(v)
+            else:
+                layer["blocks"].setdefault(k, []).append(v)
+        layers.append(layer)
+    return dict((k, v) for k, v in root if k == "name").get("name"), layers
+
+
+def layers_for_the_oracle(parsed_layers):
+    """The layers of parse_schema_text as the L(...) records evaluate() takes; layers of other types become Data layers
+    (their values are supplied, as for the backend)."""
+    out = []
+    for l in parsed_layers:
+        t, blocks = l["type"], l["blocks"]
+        first = lambda name: dict((k, v) for k, v in blocks[name][0] if not isinstance(v, list)) if name in blocks else {}
+        if t == "TanH":
+            f = first("tanh_param")
+            out.append(L(t, l["name"], l["inputs"], scale=float(f.get("scale", 1.0)), steepness=float(f.get("steepness", 1.0))))
+        elif t == "AverageSubsampling":
+            dims = [dict(v) for k, v in blocks["average_subsampling_param"][0] if k == "dimension_param"]
+            out.append(L(t, l["name"], l["inputs"], windows=[int(d["subsampling_size"]) for d in dims]))
+        elif t == "Dropout":
+            out.append(L(t, l["name"], l["inputs"], dropout_rate=float(first("dropout_param").get("dropout_rate", 0.5))))
+        elif t in ("Absolute", "ReLU", "Sigmoid", "ELU", "Softmax"):
+            out.append(L(t, l["name"], l["inputs"]))
+        else:
+            out.append(L("Data", l["name"]))
+    return out
+
+
 def make_weights(layers, gen):
     weights = {}
     for l in layers:

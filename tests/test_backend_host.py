@@ -62,6 +62,96 @@ layer { type: "AverageSubsampling" name: "avg_0_layer" input_layer_name: "tanh_0
     assert rep["per_entry_bytes"] == 4 * (3 * 48 + 3 * 12)
 
 
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def golden_text(name):
+    # byte for byte as the reference holds it: CR LF line ends, tabs, and two lines indented with spaces
+    with open(os.path.join(GOLDEN, name), "rb") as f:
+        return f.read().decode("ascii")
+
+
+def test_the_reference_example_schema_reads_with_its_convolutions_kept_as_external_layers():
+    """examples/gtsrb/working_data/schema.txt of the reference, verbatim. Its LCS, Convolution, SparseConvolution, LError
+    and Accuracy layers are types this backend has no class for: by default that is the reference's error, with
+    keep_unregistered_layers they stay in the schema as they stand in the file."""
+    text = golden_text("gtsrb_schema.txt")
+    assert "\r\n" in text and "        dimension_param" in text  # the fixture is the file, not a cleaned-up copy
+    with pytest.raises(backend.BackendError, match="No layer is registered with type LCS"):
+        backend.list_layers(text)
+    layers = backend.list_layers(text, keep_unregistered_layers=True)
+    name, want = S.parse_schema_text(text)
+    assert name == "GTSRB"
+    assert [(l["type"], l["name"], l["inputs"]) for l in layers] == [(l["type"], l["name"], l["inputs"]) for l in want]
+    assert len(layers) == 19
+    by_name = {l["name"]: l for l in layers}
+    assert {l["name"] for l in layers if l["external"]} == {"lcs_layer", "parameters_0", "parameters_1", "parameters_2", "parameters_3", "L2_error", "Accuracy"}
+    for i in range(4):
+        assert by_name["tanh_%d_layer" % i]["parameters"] == "scale 1.716, steepness 0.667"
+    for i in range(2):
+        assert by_name["avg_%d_layer" % i]["parameters"] == "2x2"
+    assert by_name["dropout_2_layer"]["parameters"] == "dropout rate 0.100"
+    assert by_name["L2_error"]["inputs"] == ["tanh_3_layer", "labels"]
+
+    # written back and read again: the same layers; the parameters of the layers the backend knows with the values of
+    # the file, the external layers with the messages they came with (fields in the writer's order: messages first)
+    again = backend.rewrite_schema(text, keep_unregistered_layers=True)
+    assert backend.list_layers(again, keep_unregistered_layers=True) == layers
+    _, rewritten = S.parse_schema_text(again)
+    canonical = lambda blocks: {name: [sorted(repr(field) for field in message) for message in messages] for name, messages in blocks.items()}
+    for l_in, l_out in zip(want, rewritten):
+        if by_name[l_in["name"]]["external"]:
+            assert canonical(l_out["blocks"]) == canonical(l_in["blocks"]), l_in["name"]
+        elif l_in["type"] == "TanH":
+            got = dict(l_out["blocks"]["tanh_param"][0])
+            assert F(got["scale"]) == F(1.7159) and F(got["steepness"]) == F(0.666666)
+        elif l_in["type"] == "AverageSubsampling":
+            assert [dict(v)["subsampling_size"] for k, v in l_out["blocks"]["average_subsampling_param"][0] if k == "dimension_param"] == ["2", "2"]
+        elif l_in["type"] == "Dropout":
+            assert F(dict(l_out["blocks"]["dropout_param"][0])["dropout_rate"]) == F(0.1)
+    sparse = [l for l in rewritten if l["name"] == "parameters_2"][0]["blocks"]["sparse_convolution_param"][0]
+    assert dict(f for f in sparse if not isinstance(f[1], list)) == {
+        "input_feature_map_count": "96", "output_feature_map_count": "200", "feature_map_connection_sparsity_ratio": "0.3"}
+    assert backend.rewrite_schema(again, keep_unregistered_layers=True) == again
+
+
+def test_the_reference_example_schema_plans_around_its_convolutions():
+    """What the backend computes of that network, given the convolutions' results: every TanH -> Absolute -> AverageSubsampling
+    stretch is one launch (the two element-wise layers are applied by the subsampling kernel to what it reads), TanH ->
+    Absolute -> Dropout is one, the last TanH one. Layers that only the convolutions read (the images, the contrast layer)
+    are neither asked for nor computed."""
+    text = golden_text("gtsrb_schema.txt")
+    configs = {"parameters_0": (38, [28, 28]), "parameters_1": (96, [10, 10]), "parameters_2": (200, [1, 1]), "parameters_3": (43, [1, 1])}
+    outputs = ["avg_0_layer", "avg_1_layer", "dropout_2_layer", "tanh_3_layer"]
+    rep = backend.plan_schema(text, configs, outputs, keep_unregistered_layers=True)
+    steps = {"+".join(s["layers"]): s["inputs"] for s in rep["steps"]}
+    assert steps == {"tanh_0_layer+abs_0_layer+avg_0_layer": ["parameters_0"], "tanh_1_layer+abs_1_layer+avg_1_layer": ["parameters_1"],
+                     "tanh_2_layer+abs_2_layer+dropout_2_layer": ["parameters_2"], "tanh_3_layer": ["parameters_3"]}
+    # device bytes per entry: the four inputs and the four outputs, nothing in between
+    assert rep["per_entry_bytes"] == 4 * (38 * 28 * 28 + 96 * 10 * 10 + 200 + 43 + 38 * 14 * 14 + 96 * 5 * 5 + 200 + 43)
+    # without the switch the schema is refused; an external layer's configuration has to be given
+    with pytest.raises(backend.BackendError, match="No layer is registered with type"):
+        backend.plan_schema(text, configs, outputs)
+    with pytest.raises(backend.BackendError, match="parameters_3"):
+        backend.plan_schema(text, {k: v for k, v in configs.items() if k != "parameters_3"}, outputs, keep_unregistered_layers=True)
+    # the whole error function hangs on external layers: asked for, it is a source of data like them
+    rep = backend.plan_schema(text, {"L2_error": (1, [1, 1])}, ["L2_error"], keep_unregistered_layers=True)
+    assert rep["steps"] == []
+
+
+def test_the_reference_example_tail_schema_reads():
+    """examples/gtsrb/working_data/schema_tail.txt: the reference itself feeds a network's result to the error layers as a
+    Data layer named like the layer that made it."""
+    text = golden_text("gtsrb_schema_tail.txt")
+    layers = backend.list_layers(text, keep_unregistered_layers=True)
+    assert [(l["type"], l["name"], l["inputs"], l["external"]) for l in layers] == [
+        ("Data", "images", [], False), ("Data", "labels", [], False), ("Data", "tanh_3_layer", [], False),
+        ("LError", "L2_error", ["tanh_3_layer", "labels"], True), ("Accuracy", "Accuracy", ["tanh_3_layer", "labels"], True)]
+    again = backend.rewrite_schema(text, keep_unregistered_layers=True)
+    assert "lerror_param" in again and "scale: 0.5" in again
+    assert backend.list_layers(again, keep_unregistered_layers=True) == layers
+
+
 def test_schema_errors():
     with pytest.raises(backend.BackendError, match="No layer is registered with type Convolution"):
         backend.rewrite_schema('layer { type: "Convolution" name: "c" }')

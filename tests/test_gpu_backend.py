@@ -408,6 +408,37 @@ def test_resnet50_post_convolution_graph_layer_by_layer(mode):
             assert_bits(got[name], values[name], name)
 
 
+def test_the_reference_example_schema_runs_around_its_convolutions(tmp_path):
+    """examples/gtsrb/working_data/schema.txt of the reference, as it stands in the file, with keep_unregistered_layers: the
+    results of its four convolutions come in as inputs (seeded values), and every layer the backend computes is compared
+    with the oracle layer by layer, bit for bit - TanH -> Absolute -> AverageSubsampling as one launch each, the average
+    being the plain tester's window sum (no alpha in the file)."""
+    import os
+
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "gtsrb_schema.txt"), "rb") as f:
+        text = f.read().decode("ascii")
+    _, parsed = S.parse_schema_text(text)
+    layers = S.layers_for_the_oracle(parsed)
+    gen = T.rng(64, 1)
+    n = 37
+    shapes = {"parameters_0": (n, 38, 28, 28), "parameters_1": (n, 96, 10, 10), "parameters_2": (n, 200, 1, 1), "parameters_3": (n, 43, 1, 1)}
+    inputs = {name: T.normal(gen, shape, 1.5) for name, shape in shapes.items()}
+    inputs["parameters_0"].reshape(-1)[::97] = np.array([0.0, -0.0, 70.0, -70.0, np.inf, -np.inf, 1.0e-40], np.float32)[np.arange(inputs["parameters_0"].size)[::97] % 7]
+    # the oracle's turn: only what hangs on the supplied values (the other data layers are never looked at)
+    needed = [l for l in layers if l["type"] == "Data" or all(i in inputs or i.startswith(("tanh", "abs", "avg", "dropout")) for i in l["inputs"])]
+    values = S.evaluate([l for l in needed if l["name"] in inputs or l["type"] != "Data"], {}, inputs)
+    outputs = ["avg_0_layer", "abs_0_layer", "avg_1_layer", "dropout_2_layer", "tanh_3_layer"]
+    shapes_out = {name: values[name].shape for name in outputs}
+    got, rep = backend.run_schema(text, {}, inputs, shapes_out, keep_unregistered_layers=True, max_entry_count=16)
+    assert rep["entries"] == n
+    # abs_0_layer is wanted as well here, so the first stretch cannot go into the average's kernel whole
+    assert sorted("+".join(st["layers"]) for st in rep["steps"]) == sorted([
+        "tanh_0_layer+abs_0_layer", "avg_0_layer", "tanh_1_layer+abs_1_layer+avg_1_layer", "tanh_2_layer+abs_2_layer+dropout_2_layer", "tanh_3_layer"])
+    for name in outputs:
+        assert_bits(got[name], values[name], name)
+    assert got["avg_0_layer"].shape == (n, 38, 14, 14) and got["avg_1_layer"].shape == (n, 96, 5, 5)
+
+
 def test_packets_under_the_staging_bound_keep_a_few_entries():
     """hip_max_io_staging_mb bounds the pinned staging of a packet, but not below eight entries: entries of 12.6 MB in and
     12.6 MB out would fit 64 MB two at a time. Twelve entries then go as packets of eight and four; with the bound lifted
