@@ -144,6 +144,11 @@ namespace nnforge
 		return x.action < y.action;
 	}
 
+	inline bool operator ==(const layer_name_with_action& x, const layer_name_with_action& y)
+	{
+		return !(x < y) && !(y < x);
+	}
+
 	typedef std::vector<unsigned int> data_config;
 	typedef std::vector<unsigned int> data_custom_config;
 

@@ -172,6 +172,45 @@ namespace nnforge
 		unsigned int index;
 	};
 
+	// The actions of a propagation and what each one waits for (nnforge/network_action_schema.h:35-126), as far as
+	// forward propagation uses it: one forward action per layer that computes something, depending on the forward
+	// actions of the layers it reads. The reference's scheduling helpers on top of the graph (streams, buffer sets,
+	// flops-driven ordering, Graphviz output) belong to its own backends and are not restated: this backend plans
+	// launches and buffers on its fused steps (forward_propagation_hip).
+	class network_action_schema
+	{
+	public:
+		typedef std::shared_ptr<network_action_schema> ptr;
+		typedef std::shared_ptr<const network_action_schema> const_ptr;
+
+		network_action_schema() = default;
+
+		// throws when the action exists already or a dependency does not
+		void add_action(layer::const_ptr l, layer_action action, const std::vector<layer_name_with_action>& dependencies = std::vector<layer_name_with_action>());
+		bool action_exists(const layer_name_with_action& layer_and_action) const;
+		void add_dependencies(const layer_name_with_action& source_layer_and_action, const std::vector<layer_name_with_action>& dependencies);
+		void add_dependency(const layer_name_with_action& source_layer_and_action, const layer_name_with_action& destination_layer_and_action);
+		bool dependency_exists(const layer_name_with_action& source_layer_and_action, const layer_name_with_action& destination_layer_and_action) const;
+		// what the action waits for directly
+		std::vector<layer_name_with_action> get_dependencies(const layer_name_with_action& action) const;
+		// every action behind the actions it waits for; among those free to go, the one added first comes first
+		std::vector<layer_name_with_action> get_actions_in_execution_order() const;
+		std::vector<layer_name_with_action> get_actions() const; // in the order they were added
+		layer::const_ptr get_layer(const layer_name_with_action& action) const;
+		// keeps the target actions and everything they wait for, directly or not
+		void drop_actions_not_required_to_do(const std::set<layer_name_with_action>& target_action_set);
+
+	private:
+		struct node
+		{
+			layer::const_ptr l;
+			layer_name_with_action key;
+			std::vector<layer_name_with_action> dependencies;
+		};
+		const node& find(const layer_name_with_action& action) const;
+		std::vector<node> nodes; // in the order of add_action
+	};
+
 	// nnforge/forward_propagation.h:39-115
 	class forward_propagation
 	{
@@ -233,6 +272,9 @@ namespace nnforge
 
 	protected:
 		network_schema::const_ptr schema; // reduced to what the outputs need
+		// one forward action per layer of `schema` that computes something (nnforge/forward_propagation.h:97,
+		// network_schema::get_actions_for_forward_propagation, nnforge/network_schema.cpp:242-300)
+		network_action_schema::ptr action_schema;
 		std::vector<std::string> output_layer_names;
 		debug_state::ptr debug;
 		profile_state::ptr profile;
@@ -316,6 +358,16 @@ namespace nnforge
 	typedef config_option<bool> bool_option;
 	typedef config_option<float> float_option;
 	typedef config_option<int> int_option;
+	// a path as text where the reference has boost::filesystem::path (nnforge/config_options.h:62-80)
+	typedef config_option<std::string> path_option;
+	// an option that may be given several times (nnforge/config_options.h:45-60): no default
+	struct multi_string_option
+	{
+		multi_string_option(const char * name, std::vector<std::string> * var, const char * description) : name(name), var(var), description(description) {}
+		std::string name;
+		std::vector<std::string> * var;
+		std::string description;
+	};
 
 	// nnforge/factory_generator.h:27-56
 	class factory_generator
@@ -328,6 +380,8 @@ namespace nnforge
 		virtual backward_propagation_factory::ptr create_backward_propagation_factory() const = 0;
 		virtual void info() const = 0;
 		virtual std::vector<string_option> get_string_options() { return std::vector<string_option>(); }
+		virtual std::vector<multi_string_option> get_multi_string_options() { return std::vector<multi_string_option>(); }
+		virtual std::vector<path_option> get_path_options() { return std::vector<path_option>(); }
 		virtual std::vector<bool_option> get_bool_options() { return std::vector<bool_option>(); }
 		virtual std::vector<float_option> get_float_options() { return std::vector<float_option>(); }
 		virtual std::vector<int_option> get_int_options() { return std::vector<int_option>(); }

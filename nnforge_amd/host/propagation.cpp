@@ -351,6 +351,23 @@ namespace nnforge
 		network_schema::ptr reduced(new network_schema(full_schema.get_required_layers(output_layer_names)));
 		reduced->name = full_schema.name;
 		schema = reduced;
+		// a forward action per layer with inputs, waiting for the forward actions of the layers it reads (layers
+		// without inputs - data layers, layers computed elsewhere - have no action: their values are there)
+		action_schema.reset(new network_action_schema());
+		for(const layer::const_ptr& l : schema->get_layers_in_forward_propagation_order())
+		{
+			if (l->input_layer_instance_names.empty())
+				continue;
+			std::vector<layer_name_with_action> dependencies;
+			for(const std::string& input : l->input_layer_instance_names)
+			{
+				const layer_name_with_action source(input, layer_action(layer_action::forward));
+				if (!schema->get_layer(input)->input_layer_instance_names.empty()
+					&& (std::find(dependencies.begin(), dependencies.end(), source) == dependencies.end()))
+					dependencies.push_back(source);
+			}
+			action_schema->add_action(l, layer_action(layer_action::forward), dependencies);
+		}
 		for(const layer::const_ptr& l : schema->get_data_layers())
 			data_layer_names.insert(l->instance_name);
 
@@ -360,6 +377,125 @@ namespace nnforge
 			if (cumulative_tiling_factor_map.at(n) != output_layers_tiling_factor)
 				throw neural_network_exception("Inconsistent tiling factors across output layers: "
 					+ std::to_string(output_layers_tiling_factor) + " and " + std::to_string(cumulative_tiling_factor_map.at(n)));
+	}
+
+	// ---- network_action_schema ---------------------------------------------------------------
+
+	const network_action_schema::node& network_action_schema::find(const layer_name_with_action& action) const
+	{
+		for(const node& n : nodes)
+			if (n.key == action)
+				return n;
+		throw neural_network_exception("Action not found in action schema: " + action.get_name() + " " + action.get_action().str());
+	}
+
+	bool network_action_schema::action_exists(const layer_name_with_action& layer_and_action) const
+	{
+		for(const node& n : nodes)
+			if (n.key == layer_and_action)
+				return true;
+		return false;
+	}
+
+	void network_action_schema::add_action(layer::const_ptr l, layer_action action, const std::vector<layer_name_with_action>& dependencies)
+	{
+		const layer_name_with_action key(l->instance_name, action);
+		if (action_exists(key))
+			throw neural_network_exception("Action already exists in action schema: " + key.get_name() + " " + action.str());
+		for(const layer_name_with_action& d : dependencies)
+			find(d);
+		node n;
+		n.l = l;
+		n.key = key;
+		nodes.push_back(n);
+		add_dependencies(key, dependencies);
+	}
+
+	void network_action_schema::add_dependencies(const layer_name_with_action& source_layer_and_action, const std::vector<layer_name_with_action>& dependencies)
+	{
+		for(const layer_name_with_action& d : dependencies)
+			add_dependency(source_layer_and_action, d);
+	}
+
+	void network_action_schema::add_dependency(const layer_name_with_action& source_layer_and_action, const layer_name_with_action& destination_layer_and_action)
+	{
+		find(destination_layer_and_action);
+		node& n = const_cast<node&>(find(source_layer_and_action));
+		if (std::find(n.dependencies.begin(), n.dependencies.end(), destination_layer_and_action) == n.dependencies.end())
+			n.dependencies.push_back(destination_layer_and_action);
+	}
+
+	bool network_action_schema::dependency_exists(const layer_name_with_action& source_layer_and_action, const layer_name_with_action& destination_layer_and_action) const
+	{
+		if (!action_exists(source_layer_and_action))
+			return false;
+		const node& n = find(source_layer_and_action);
+		return std::find(n.dependencies.begin(), n.dependencies.end(), destination_layer_and_action) != n.dependencies.end();
+	}
+
+	std::vector<layer_name_with_action> network_action_schema::get_dependencies(const layer_name_with_action& action) const
+	{
+		return find(action).dependencies;
+	}
+
+	std::vector<layer_name_with_action> network_action_schema::get_actions() const
+	{
+		std::vector<layer_name_with_action> res;
+		for(const node& n : nodes)
+			res.push_back(n.key);
+		return res;
+	}
+
+	layer::const_ptr network_action_schema::get_layer(const layer_name_with_action& action) const
+	{
+		return find(action).l;
+	}
+
+	std::vector<layer_name_with_action> network_action_schema::get_actions_in_execution_order() const
+	{
+		std::vector<layer_name_with_action> res;
+		std::vector<bool> done(nodes.size(), false);
+		while (res.size() < nodes.size())
+		{
+			bool progressed = false;
+			for(size_t i = 0; i < nodes.size(); ++i)
+			{
+				if (done[i])
+					continue;
+				bool ready = true;
+				for(const layer_name_with_action& d : nodes[i].dependencies)
+					ready = ready && (std::find(res.begin(), res.end(), d) != res.end());
+				if (ready)
+				{
+					res.push_back(nodes[i].key);
+					done[i] = true;
+					progressed = true;
+				}
+			}
+			if (!progressed)
+				throw neural_network_exception("The action schema has a cycle");
+		}
+		return res;
+	}
+
+	void network_action_schema::drop_actions_not_required_to_do(const std::set<layer_name_with_action>& target_action_set)
+	{
+		std::set<layer_name_with_action> needed;
+		std::vector<layer_name_with_action> todo(target_action_set.begin(), target_action_set.end());
+		while (!todo.empty())
+		{
+			const layer_name_with_action cur = todo.back();
+			todo.pop_back();
+			if (!needed.insert(cur).second)
+				continue;
+			for(const layer_name_with_action& d : find(cur).dependencies)
+				todo.push_back(d);
+		}
+		std::vector<node> kept;
+		for(const node& n : nodes)
+			if (needed.find(n.key) != needed.end())
+				kept.push_back(n);
+		nodes = kept;
 	}
 
 	bool forward_propagation::is_schema_with_weights() const
@@ -468,6 +604,8 @@ namespace nnforge
 	void factory_generator::apply_default_options()
 	{
 		for(string_option& o : get_string_options()) *o.var = o.default_value;
+		for(multi_string_option& o : get_multi_string_options()) o.var->clear();
+		for(path_option& o : get_path_options()) *o.var = o.default_value;
 		for(bool_option& o : get_bool_options()) *o.var = o.default_value;
 		for(float_option& o : get_float_options()) *o.var = o.default_value;
 		for(int_option& o : get_int_options()) *o.var = o.default_value;

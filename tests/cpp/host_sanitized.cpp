@@ -9,6 +9,9 @@
 #include <cstdio>
 #include <cstddef>
 #include <cstring>
+#include <map>
+#include <set>
+#include <sstream>
 #include <string>
 #include <vector>
 
@@ -98,18 +101,79 @@ int main(int argc, char ** argv)
 		expect(std::string(buffer.data()).find("max_entry_count: 7") != std::string::npos, std::string("... are honoured as far as they go: ") + buffer.data());
 		expect(std::string(buffer.data()).find(" #") != std::string::npos, std::string("... and the members behind them take their defaults (groups launched together): ") + buffer.data());
 	}
+	// what a subclass of the reference's base classes may touch: the action schema of a forward_propagation, every kind of
+	// option list of a factory_generator
+	{
+		struct probe : public nnforge::forward_propagation
+		{
+			probe(const nnforge::network_schema& schema, const std::vector<std::string>& outputs)
+				: nnforge::forward_propagation(schema, outputs, nnforge::debug_state::ptr(), nnforge::profile_state::ptr()) {}
+			void actual_set_data(nnforge::network_data::const_ptr) override {}
+			void actual_clear_data() override {}
+			void actual_run(nnforge::structured_data_bunch_reader&, nnforge::structured_data_bunch_writer&, unsigned int&,
+				std::map<nnforge::layer_name_with_action, float>&, float&) override {}
+			void layer_config_map_modified() override {}
+			const nnforge::network_action_schema& actions() const { return *action_schema; }
+		};
+		nnforge::init();
+		std::istringstream in(good);
+		nnforge::network_schema schema;
+		schema.read_proto(in);
+		probe fp(schema, std::vector<std::string>(1, "cat"));
+		const nnforge::layer_action forward(nnforge::layer_action::forward);
+		const std::vector<nnforge::layer_name_with_action> order = fp.actions().get_actions_in_execution_order();
+		expect(order.size() == 12, "a forward action for each of the twelve layers between the data layer and cat, none for what cat does not need: " + std::to_string(order.size()));
+		expect(!fp.actions().action_exists(nnforge::layer_name_with_action("conv1", forward)), "a data layer has no action");
+		expect(!fp.actions().action_exists(nnforge::layer_name_with_action("prob", forward)), "a layer the outputs do not need has no action");
+		expect(fp.actions().get_dependencies(nnforge::layer_name_with_action("bn", forward)).empty(), "the first layer waits for nothing");
+		const std::vector<nnforge::layer_name_with_action> of_sum = fp.actions().get_dependencies(nnforge::layer_name_with_action("sum", forward));
+		expect((of_sum.size() == 2) && (of_sum[0].get_name() == "drop") && (of_sum[1].get_name() == "pool2"), "the Add waits for both layers it reads");
+		expect(fp.actions().dependency_exists(nnforge::layer_name_with_action("cat", forward), nnforge::layer_name_with_action("pool2", forward)), "cat waits for pool2");
+		std::map<std::string, size_t> position;
+		for(size_t i = 0; i < order.size(); ++i)
+			position[order[i].get_name()] = i;
+		bool ordered = true;
+		for(const nnforge::layer_name_with_action& a : order)
+			for(const nnforge::layer_name_with_action& d : fp.actions().get_dependencies(a))
+				ordered = ordered && (position[d.get_name()] < position[a.get_name()]);
+		expect(ordered, "execution order puts every action behind what it waits for");
+		nnforge::network_action_schema copy(fp.actions());
+		copy.drop_actions_not_required_to_do(std::set<nnforge::layer_name_with_action>{ nnforge::layer_name_with_action("abs", forward) });
+		expect(copy.get_actions().size() == 5, "bn, relu, pool1, tanh, abs are what abs needs: " + std::to_string(copy.get_actions().size()));
+
+		struct generator : public nnforge::factory_generator
+		{
+			void initialize() override {}
+			nnforge::forward_propagation_factory::ptr create_forward_propagation_factory() const override { return nnforge::forward_propagation_factory::ptr(); }
+			nnforge::backward_propagation_factory::ptr create_backward_propagation_factory() const override { return nnforge::backward_propagation_factory::ptr(); }
+			void info() const override {}
+			std::vector<nnforge::multi_string_option> get_multi_string_options() override
+			{
+				return std::vector<nnforge::multi_string_option>(1, nnforge::multi_string_option("device", &devices, "devices to use"));
+			}
+			std::vector<nnforge::path_option> get_path_options() override
+			{
+				return std::vector<nnforge::path_option>(1, nnforge::path_option("cache_folder", &cache, "/tmp/cache", "where to keep things"));
+			}
+			std::vector<std::string> devices = std::vector<std::string>(2, "stale");
+			std::string cache = "stale";
+		} g;
+		expect(static_cast<nnforge::factory_generator&>(g).get_string_options().empty(), "option lists default to empty");
+		g.apply_default_options();
+		expect(g.devices.empty() && (g.cache == "/tmp/cache"), "defaults reach path options, and options that may repeat start empty");
+	}
 	// sizes the layers reject
 	expect(plan(good, 2, 2, report) != 0, "an input smaller than the windows is refused");
 	expect(plan(good, 0, 5, report) != 0, "an empty dimension is refused");
 
 	// the text written back parses again to the same text
 	std::vector<char> once(1 << 16), twice(1 << 16);
-	expect(nnf_backend_rewrite_schema(good.c_str(), once.data(), once.size()) == 0, "rewrite");
-	expect(nnf_backend_rewrite_schema(once.data(), twice.data(), twice.size()) == 0, "rewrite of the rewritten text");
+	expect(nnf_backend_rewrite_schema(good.c_str(), 0, once.data(), once.size()) == 0, "rewrite");
+	expect(nnf_backend_rewrite_schema(once.data(), 0, twice.data(), twice.size()) == 0, "rewrite of the rewritten text");
 	expect(std::strcmp(once.data(), twice.data()) == 0, "the writer's output is a fixed point of reader + writer");
 	// a buffer that is too small is reported, not overrun
 	std::vector<char> tiny(16);
-	expect(nnf_backend_rewrite_schema(good.c_str(), tiny.data(), tiny.size()) != 0, "a short output buffer is an error");
+	expect(nnf_backend_rewrite_schema(good.c_str(), 0, tiny.data(), tiny.size()) != 0, "a short output buffer is an error");
 
 	// damaged text: every prefix of the schema, single characters replaced, blocks doubled
 	int accepted = 0, refused = 0;
