@@ -53,6 +53,12 @@ MEASURED_TRAFFIC_BYTES = {
 }
 
 
+# Configuration 3 is bound by the vector ALU, not by HBM (three bit-exact expf and two exact divisions per element): what
+# the counters of profiles/chain_kernel_config3_activation_chain.md say about that bound, reported beside the HBM figure.
+# frac = SQ_ACTIVE_INST_VALU x 4 / (SIMDs x GRBM_GUI_ACTIVE per die): the share of cycles the vector ALUs issue in.
+CONFIG3_VALU_ROOFLINE = {"bound": "valu", "frac": 0.90, "instr_per_element": 65.9, "fp64_instr_per_element": 45.0, "clock_ghz_under_load": 2.16,
+                         "source": "profiles/chain_kernel_config3_activation_chain.md (rocprofv3 --pmc SQ_INSTS_VALU, SQ_ACTIVE_INST_VALU, SQ_BUSY_CYCLES, GRBM_GUI_ACTIVE)"}
+
 # groups at most this large are also timed on a single buffer set (cache-hot), beside the rotation through HBM
 CACHE_HOT_LIMIT_BYTES = 128 << 20
 
@@ -356,6 +362,49 @@ def bench_resnet50(runner, steps, warmup, n=64, kernel_stream_count=0, one_launc
                          "note": "a step is one pass of the launch plan, timed inside the C++ driver (forward_propagation_hip::time_kernels): "
                                  "one resident packet, the plan enqueued on the driver's kernel streams (independent groups share kernel "
                                  "launches, so a pass is fewer launches than plan steps), nothing copied to or from the host in the timed region"})
+
+
+def bench_through_driver(runner, config, c_abi_entry, steps, warmup):
+    """Configurations 0 to 3 as two-to-five-layer networks through the product driver: forward_propagation_hip fuses the layers
+    into the one group the C ABI figure launches by hand, and time_kernels runs that plan on packets resident in device
+    memory, going round enough sets of data / output buffers that the tensors come from HBM, not from the last-level cache
+    (the intermediate buffers of a plan are shared by all sets; these plans have none). The reference reports per-run
+    seconds from its driver too (nnforge/forward_propagation.cpp:137-190)."""
+    from nnforge_amd import backend, schemas
+
+    layers, configs, outputs, n = schemas.config_network(config)
+    gen = np.random.Generator(np.random.MT19937(SEED + 0x100 + config))
+    weights = {}
+    for l in layers:
+        if l["type"] == "BatchNorm":
+            c = l["params"]["feature_map_count"]
+            variance = gen.random(c, dtype=np.float32) * np.float32(1.5) + np.float32(0.5)
+            weights[l["name"]] = [gen.random(c, dtype=np.float32) + np.float32(0.5), gen.standard_normal(c, dtype=np.float32) * np.float32(0.316),
+                                  gen.standard_normal(c, dtype=np.float32) * np.float32(0.316), (1.0 / np.sqrt(variance + np.float32(1e-5))).astype(np.float32)]
+        elif l["type"] == "PReLU":
+            weights[l["name"]] = [gen.random(l["params"]["feature_map_count"], dtype=np.float32) * np.float32(0.25)]
+    largest = max(fm * dims[0] * dims[1] for fm, dims in configs.values())
+    pool = gen.standard_normal(n * largest, dtype=np.float32)
+    if config == 1:
+        pool *= np.float32(2.0)
+        pool[gen.random(pool.size) < 0.01] = np.float32(30.0)
+    if config == 3:
+        pool *= np.float32(np.sqrt(2.0))
+        outliers = gen.random(pool.size) < 0.001
+        pool[outliers] = np.where(gen.random(int(outliers.sum())) < 0.5, np.float32(50.0), np.float32(-50.0))
+    io_bytes = 4 * n * (sum(fm * dims[0] * dims[1] for fm, dims in configs.values()) + largest)
+    resident = int(max(1, min(64, -(-(768 << 20) // io_bytes))))
+    rep = backend.time_kernels(schemas.schema_text(layers), weights, configs, outputs, warmup=warmup, passes=steps, shared_input_pool=pool,
+                               entry_count=n, max_entry_count=n, resident_packets=resident)
+    assert rep["timed_entries"] == n and rep["launches"] == 1 and rep["plan_steps"] == 1 and rep["resident_packets"] == resident, rep["raw"]
+    alg = c_abi_entry["algorithmic_bytes_per_step"]
+    device_s, wall_s = rep["device_seconds_per_pass"], rep["wall_seconds_per_pass"]
+    return {"what": "the same workload as a network through forward_propagation_hip::time_kernels (one fused launch per pass, "
+                    "%d resident packets gone round)" % resident,
+            "event_ms_per_step": device_s * 1e3, "event_gbps": alg / device_s / 1e9, "event_pct_of_hbm_peak": 100.0 * alg / device_s / 1e9 / HBM_PEAK_GBPS,
+            "ms_per_step": wall_s * 1e3, "gbps": alg / wall_s / 1e9, "host_enqueue_ms_per_step": rep["host_seconds_per_pass"] * 1e3,
+            "resident_packets": resident, "steps": steps,
+            "event_time_vs_c_abi": device_s * 1e3 / c_abi_entry["event_ms_per_step"]}
 
 
 def bench_resnet50_direct(runner, steps, warmup, n=64):
@@ -948,12 +997,31 @@ def main():
 
     main_entry = run(args.workload, args.steps, args.warmup)
     per_config[args.workload] = main_entry
+
+    def annotate(name, entry):
+        if name == "config3":
+            entry["roofline_valu"] = CONFIG3_VALU_ROOFLINE
+        if (name == "config4") and (args.entries == 64):
+            # gbps credits the algorithmic bytes; the last group's result is neither written nor read back (it is applied by
+            # the average's kernel), so fewer bytes move: the rate of those beside it
+            moved = MEASURED_TRAFFIC_BYTES["config4"]
+            entry["moved_bytes_per_step"] = moved
+            entry["moved_gbps"] = moved / (entry["ms_per_step"] * 1e-3) / 1e9
+            entry["moved_pct_of_hbm_peak"] = 100.0 * entry["moved_gbps"] / HBM_PEAK_GBPS
+            entry["moved_event_gbps"] = moved / (entry["event_ms_per_step"] * 1e-3) / 1e9
+
+    annotate(args.workload, main_entry)
     cpu = None
     if not args.only:
         side_steps = {"config0": (200, 20), "config1": (400, 40), "config2": (20, 3), "config3": (60, 6), "config4": (10, 3)}
         for name in ("config0", "config1", "config2", "config3", "config4"):
             if name not in per_config:
                 per_config[name] = run(name, *side_steps[name])
+                annotate(name, per_config[name])
+        # the product driver's own timing of configurations 0 to 3 beside the C ABI figures (config 4 is timed through it anyway)
+        for number, name in enumerate(("config0", "config1", "config2", "config3")):
+            k, wu = side_steps[name] if name != args.workload else (args.steps, args.warmup)
+            per_config[name]["through_driver"] = bench_through_driver(runner, number, per_config[name], k, wu)
         per_config["copy_kernel"] = bench_copy(runner, 40, 5)
         # the neighbouring layers of the same chains
         for name, (k, wu) in (("global_average", (100, 10)), ("joined_global_average", (100, 10)), ("max_subsampling", (40, 5)), ("bn_relu_max_subsampling", (40, 5)),

@@ -55,6 +55,29 @@ def schema_text(layers, name="test_net"):
     return "\n".join(out) + "\n"
 
 
+def config_network(config):
+    """Configurations 0 to 3 of the benchmark as networks for forward_propagation_hip: the tensors the fused group reads are
+    data layers, its last layer is the output. -> (layers, {data layer: (feature maps, [width, height])}, output names, entries)"""
+    if config == 0:
+        n, c, hw = 32, 64, 56
+        return ([L("Data", "x"), L("BatchNorm", "bn", ["x"], feature_map_count=c), L("ReLU", "relu", ["bn"])],
+                {"x": (c, [hw, hw])}, ["relu"], n)
+    if config == 1:
+        n, c, _ = workloads.CONFIG1_SHAPE
+        return [L("Data", "logits"), L("Softmax", "prob", ["logits"])], {"logits": (c, [1, 1])}, ["prob"], n
+    if config == 2:
+        n, c, hw = 128, 256, 56
+        return ([L("Data", "main"), L("Data", "residual"), L("BatchNorm", "bn", ["main"], feature_map_count=c),
+                 L("Add", "sum", ["residual", "bn"]), L("PReLU", "prelu", ["sum"], feature_map_count=c)],
+                {"main": (c, [hw, hw]), "residual": (c, [hw, hw])}, ["prelu"], n)
+    if config == 3:
+        n, c, hw = 64, 512, 28
+        return ([L("Data", "x"), L("BatchNorm", "bn", ["x"], feature_map_count=c), L("ELU", "elu", ["bn"]), L("Sigmoid", "sigmoid", ["elu"]),
+                 L("TanH", "tanh", ["sigmoid"], scale=workloads.TANH_SCALE, steepness=workloads.TANH_STEEPNESS)],
+                {"x": (c, [hw, hw])}, ["tanh"], n)
+    raise ValueError(config)
+
+
 def resnet50_post_convolution(with_pool1=False):
     """Everything behind the convolutions of ResNet-50 as examples/imagenet/imagenet_toolset.cpp:476-550 and 729-831 build it,
     with the layer names used there; every convolution's output is a data layer of the same name (conv1, resNx_shortcut,
