@@ -349,6 +349,13 @@ NNF_HIP_API int nnf_hip_event_record(void* event, void* stream);
 NNF_HIP_API int nnf_hip_event_synchronize(void* event);
 NNF_HIP_API int nnf_hip_event_elapsed_ms(float* milliseconds, void* start_event, void* stop_event);
 NNF_HIP_API int nnf_hip_stream_wait_event(void* stream, void* event);
+/* A recorded sequence of launches (a HIP graph): what is enqueued on `stream` between begin and end is recorded instead
+ * of run (kernel launches only: no memory is set or copied by this library's entry points), end hands back an executable
+ * graph that nnf_hip_graph_launch replays on a stream. The pointers and sizes of the recorded launches are fixed. */
+NNF_HIP_API int nnf_hip_stream_begin_capture(void* stream);
+NNF_HIP_API int nnf_hip_stream_end_capture(void* stream, void** graph_exec);
+NNF_HIP_API int nnf_hip_graph_launch(void* graph_exec, void* stream);
+NNF_HIP_API int nnf_hip_graph_destroy(void* graph_exec);
 
 /* Plain device-to-device streaming copy kernel (float4 loads and stores, same launch shape as the
  * chain kernel). Used as the yardstick for achievable HBM bandwidth and for scaling profiler

@@ -300,8 +300,10 @@ namespace nnforge
 				float device_seconds_per_pass; // from events on the kernel stream
 				float host_seconds_per_pass;   // what the calling thread spends enqueuing a pass (the device runs behind it)
 			};
+			// replay_recorded_plan: the launches of a pass are recorded once (a HIP graph per set of buffers) and the timed
+			// passes replay the recordings - what the calling thread spends per pass is then one call per pass.
 			kernel_timing time_kernels(structured_data_bunch_reader& reader, unsigned int entry_count, unsigned int warmup, unsigned int passes,
-				unsigned int resident_packets = 1);
+				unsigned int resident_packets = 1, bool replay_recorded_plan = false);
 
 		protected:
 			void actual_set_data(network_data::const_ptr data) override;

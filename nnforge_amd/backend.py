@@ -33,7 +33,7 @@ class Options(ctypes.Structure):
                 ("profile", ctypes.c_int32), ("weights_from_folder", ctypes.c_int32), ("weights_folder", ctypes.c_char_p),
                 ("profile_folder", ctypes.c_char_p), ("stat_on_host", ctypes.c_int32), ("kernel_stream_count", ctypes.c_int32),
                 ("one_launch_per_group", ctypes.c_int32), ("host_thread_count", ctypes.c_int32), ("max_io_staging_mb", ctypes.c_int32),
-                ("resident_packets", ctypes.c_int32), ("keep_unregistered_layers", ctypes.c_int32)]
+                ("resident_packets", ctypes.c_int32), ("replay_recorded_plan", ctypes.c_int32), ("keep_unregistered_layers", ctypes.c_int32)]
 
 
 class DatasetFile(ctypes.Structure):
@@ -89,8 +89,9 @@ def load():
 
 def _options(fuse=True, dont_share_buffers=False, max_entry_count=0, profile=False, weights_folder=None,
              profile_folder=None, stat_on_host=False, kernel_stream_count=0, one_launch_per_group=False, host_thread_count=0,
-             max_io_staging_mb=0, resident_packets=0, keep_unregistered_layers=False):
+             max_io_staging_mb=0, resident_packets=0, keep_unregistered_layers=False, replay_recorded_plan=False):
     o = Options()
+    o.replay_recorded_plan = int(replay_recorded_plan)
     o.keep_unregistered_layers = int(keep_unregistered_layers)
     o.struct_size = ctypes.sizeof(Options)
     o.max_io_staging_mb = int(max_io_staging_mb)

@@ -571,6 +571,43 @@ extern "C"
 		return hip_status(hipStreamWaitEvent(static_cast<hipStream_t>(stream), static_cast<hipEvent_t>(event), 0));
 	}
 
+	int nnf_hip_stream_begin_capture(void* stream)
+	{
+		return hip_status(hipStreamBeginCapture(static_cast<hipStream_t>(stream), hipStreamCaptureModeThreadLocal));
+	}
+
+	int nnf_hip_stream_end_capture(void* stream, void** graph_exec)
+	{
+		if (graph_exec == nullptr)
+			return NNF_HIP_EINVAL;
+		*graph_exec = nullptr;
+		hipGraph_t graph = nullptr;
+		hipError_t e = hipStreamEndCapture(static_cast<hipStream_t>(stream), &graph);
+		if (e != hipSuccess)
+			return hip_status(e);
+		hipGraphExec_t exec = nullptr;
+		e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+		hipGraphDestroy(graph);
+		if (e != hipSuccess)
+			return hip_status(e);
+		*graph_exec = exec;
+		return NNF_HIP_OK;
+	}
+
+	int nnf_hip_graph_launch(void* graph_exec, void* stream)
+	{
+		if (graph_exec == nullptr)
+			return NNF_HIP_EINVAL;
+		return hip_status(hipGraphLaunch(static_cast<hipGraphExec_t>(graph_exec), static_cast<hipStream_t>(stream)));
+	}
+
+	int nnf_hip_graph_destroy(void* graph_exec)
+	{
+		if (graph_exec == nullptr)
+			return NNF_HIP_OK;
+		return hip_status(hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph_exec)));
+	}
+
 	const char* nnf_hip_error_string(int code)
 	{
 		switch (code)

@@ -504,7 +504,8 @@ extern "C"
 			if (hfp == nullptr)
 				throw neural_network_exception("The factory did not make a forward_propagation_hip");
 			const unsigned int resident_packets = ((options != nullptr) && (options->resident_packets > 0)) ? static_cast<unsigned int>(options->resident_packets) : 1U;
-			const hip::forward_propagation_hip::kernel_timing t = hfp->time_kernels(reader, entry_count, warmup, passes, resident_packets);
+			const hip::forward_propagation_hip::kernel_timing t = hfp->time_kernels(reader, entry_count, warmup, passes, resident_packets,
+				(options != nullptr) && (options->replay_recorded_plan != 0));
 			describe_plan(*hfp, out);
 			out << "launches: " << t.launch_count << "\n";
 			out << "plan_steps: " << t.plan_step_count << "\n";

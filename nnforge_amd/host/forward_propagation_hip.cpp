@@ -1373,7 +1373,8 @@ namespace nnforge
 		}
 
 		forward_propagation_hip::kernel_timing forward_propagation_hip::time_kernels(
-			structured_data_bunch_reader& reader, unsigned int entry_count, unsigned int warmup, unsigned int passes, unsigned int resident_packets)
+			structured_data_bunch_reader& reader, unsigned int entry_count, unsigned int warmup, unsigned int passes, unsigned int resident_packets,
+			bool replay_recorded_plan)
 		{
 			if (hip_config->is_offline())
 				throw neural_network_exception("This forward_propagation_hip was created for planning only (offline configuration): it cannot run");
@@ -1381,6 +1382,16 @@ namespace nnforge
 			const unsigned int packet = std::min(std::max(1U, entry_count), max_entry_count);
 			const int slot_count = static_cast<int>(std::max(1U, std::min(resident_packets, 64U)));
 			run_buffers& r = prepare_run(packet, slot_count, false, false, 1);
+			// recordings of the plan, released after the streams have drained (declared first, destroyed last)
+			struct recorded_plans
+			{
+				std::vector<void *> graphs;
+				~recorded_plans()
+				{
+					for(void * g : graphs)
+						nnf_hip_graph_destroy(g);
+				}
+			} recorded;
 			drain_streams drain_on_exit;
 			drain_on_exit.streams = p->kernel_streams;
 
@@ -1410,7 +1421,11 @@ namespace nnforge
 			unsigned int pass_id = 0;
 			auto one_pass = [&]()
 			{
-				p->enqueue_plan(r.buffers[pass_id % static_cast<unsigned int>(slot_count)], entries_read, r.chunk_ptrs, r.temporary, nullptr);
+				const unsigned int slot = pass_id % static_cast<unsigned int>(slot_count);
+				if (!recorded.graphs.empty())
+					hip_safe_call(nnf_hip_graph_launch(recorded.graphs[slot], p->stream));
+				else
+					p->enqueue_plan(r.buffers[slot], entries_read, r.chunk_ptrs, r.temporary, nullptr);
 				++pass_id;
 			};
 			hip_safe_call(nnf_hip_device_synchronize());
@@ -1426,6 +1441,20 @@ namespace nnforge
 			one_pass();
 			hip_safe_call(nnf_hip_launch_count(&launches_after));
 			res.launch_count = static_cast<unsigned int>(launches_after - launches_before);
+			if (replay_recorded_plan)
+			{
+				if (p->kernel_streams.size() != 1)
+					throw neural_network_exception("time_kernels: a recorded plan takes one kernel stream");
+				hip_safe_call(nnf_hip_device_synchronize());
+				for(int slot = 0; slot < slot_count; ++slot)
+				{
+					hip_safe_call(nnf_hip_stream_begin_capture(p->stream));
+					p->enqueue_plan(r.buffers[slot], entries_read, r.chunk_ptrs, r.temporary, nullptr);
+					void * graph = nullptr;
+					hip_safe_call(nnf_hip_stream_end_capture(p->stream, &graph));
+					recorded.graphs.push_back(graph);
+				}
+			}
 			for(unsigned int i = 0; i < warmup; ++i)
 				one_pass();
 			hip_safe_call(nnf_hip_device_synchronize());

@@ -455,6 +455,50 @@ def test_independent_groups_in_one_call_equal_the_groups_one_by_one(gpu, first_s
         check_exact(out, group[7], "group %d of the call (seed %d)" % (i, first_seed + i))
 
 
+def test_recorded_launches_replay_with_the_results_of_launching(gpu):
+    """nnf_hip_stream_begin_capture / nnf_hip_stream_end_capture / nnf_hip_graph_launch: a fused group, a softmax and a whole-plane
+    average recorded once on a stream of their own, then replayed four times with new values in the same input
+    buffers each time and the program's ordinary work (copies, synchronisations) in between: every replay gives the
+    bits the oracle gives (softmax to 1e-5)."""
+    lib, torch = gpu.lib, gpu.torch
+    n, c, plane = 5, 24, 49
+    gamma, beta, mean, inv_sigma = T.bn_params(T.rng(16, 1), c)
+    d_chunks = [gpu.to_device(a) for a in (gamma, beta, mean, inv_sigma)]
+    chk = capi.pointer_array([t.data_ptr() for t in d_chunks])
+    desc = capi.make_desc(n, c, plane, [[], [(BN, 0)]], [(RELU, 0, 0.0)])
+    d_x, d_r = gpu.to_device(np.zeros((n, c, plane), np.float32)), gpu.to_device(np.zeros((n, c, plane), np.float32))
+    d_y = torch.empty_like(d_x)
+    d_pool = torch.empty(n * c, dtype=torch.float32, device=gpu.device)
+    d_prob = torch.empty(n * c, dtype=torch.float32, device=gpu.device)
+    ins = capi.pointer_array([d_r.data_ptr(), d_x.data_ptr()])
+    stream = ctypes.c_void_p()
+    capi.check(lib.nnf_hip_stream_create(ctypes.byref(stream)))
+    torch.cuda.synchronize()
+    capi.check(lib.nnf_hip_stream_begin_capture(stream))
+    capi.check(lib.nnf_hip_chain_forward(stream, ctypes.byref(desc), d_y.data_ptr(), ins, chk))
+    capi.check(lib.nnf_hip_average_subsampling_forward(stream, d_pool.data_ptr(), d_y.data_ptr(), n, c, 7, 7, 7, 7, 1.0 / 49.0))
+    capi.check(lib.nnf_hip_softmax_forward(stream, d_prob.data_ptr(), d_pool.data_ptr(), n, c, 1))
+    graph = ctypes.c_void_p()
+    capi.check(lib.nnf_hip_stream_end_capture(stream, ctypes.byref(graph)))
+    assert graph.value
+    for replay in range(4):
+        gen = T.rng(17, replay)
+        x, r = T.normal(gen, (n, c, plane), 2.0), T.normal(gen, (n, c, plane), 2.0)
+        d_x.copy_(torch.from_numpy(x).reshape(d_x.shape))
+        d_r.copy_(torch.from_numpy(r).reshape(d_r.shape))
+        d_y.fill_(float("nan"))
+        torch.cuda.synchronize()
+        capi.check(lib.nnf_hip_graph_launch(graph, stream))
+        capi.check(lib.nnf_hip_stream_synchronize(stream))
+        want_y = oracle.rectified_linear(oracle.add([r, oracle.batch_norm(x, gamma, beta, mean, inv_sigma)]).reshape(x.shape))
+        want_pool = oracle.average_subsampling(want_y.reshape(n, c, 7, 7), [7, 7], mult=1.0 / 49.0)
+        check_exact(gpu.to_host(d_y, x.shape), want_y, "replay %d: group" % replay)
+        check_exact(gpu.to_host(d_pool, want_pool.shape), want_pool, "replay %d: average" % replay)
+        assert_softmax_close(gpu.to_host(d_prob, (n, c, 1)), oracle.softmax(want_pool.reshape(n, c, 1)), "replay %d: softmax" % replay)
+    capi.check(lib.nnf_hip_graph_destroy(graph))
+    capi.check(lib.nnf_hip_stream_destroy(stream))
+
+
 @pytest.mark.parametrize("planes", [(784, 3136), (49, 9), (784, 49), (49, 196, 7, 3136)])
 def test_groups_of_one_and_of_two_inputs_share_launches(gpu, planes):
     """A residual network's groups as the driver hands them over: BatchNorm -> ReLU over one tensor and BatchNorm
