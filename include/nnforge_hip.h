@@ -129,6 +129,17 @@ NNF_HIP_API int nnf_hip_chain_forward(void* stream, const nnf_hip_chain_desc* de
 NNF_HIP_API int nnf_hip_chain_forward_batch(void* stream, uint32_t group_count, const nnf_hip_chain_desc* descs,
 	float* const* outputs, const float* const* const* inputs, const float* const* const* chunk_ptrs);
 
+/* A fused group whose result is a part of a wider tensor: entry e of the result is written output_entry_stride floats behind
+ * entry e - 1 (the inputs are ordinary tensors, entry behind entry). With `output` pointing at the group's feature maps
+ * inside the first entry of a Concat layer's output and output_entry_stride that layer's neuron count, the group writes
+ * where nnforge/plain/concat_layer_tester_plain.cpp:45-58 would copy its result to, and the copy is not needed. Same bits as
+ * nnf_hip_chain_forward followed by that copy. One or two inputs; the neuron count of an entry and the stride must be
+ * multiples of 4 (every entry then starts on a 16-byte boundary): NNF_HIP_EUNSUPPORTED otherwise, and
+ * nnf_hip_chain_forward_strided_status tells so from the shapes alone. The written range may overlap no input. */
+NNF_HIP_API int nnf_hip_chain_forward_strided(void* stream, const nnf_hip_chain_desc* desc, float* output, uint32_t output_entry_stride,
+	const float* const* inputs, const float* const* chunk_ptrs);
+NNF_HIP_API int nnf_hip_chain_forward_strided_status(const nnf_hip_chain_desc* desc, uint32_t output_entry_stride);
+
 /* Single-layer entry points, one per reference tester (same arithmetic as the chain kernel). */
 NNF_HIP_API int nnf_hip_batch_norm_forward(void* stream, float* output, const float* input,
 	const float* gamma, const float* beta, const float* mean, const float* inverse_sigma,

@@ -111,6 +111,8 @@ SIGNATURES = {
     "nnf_hip_average_subsampling_joined_forward": [_VP, _VP, _PP, ctypes.POINTER(ChainDesc), _PP, _U32, _U32, _U32, _U32, _U32, _U32, _F],
     "nnf_hip_average_subsampling_joinable": [_U32, _U32, _U32, _U32, _U32, _U32],
     "nnf_hip_launch_count": [ctypes.POINTER(_U64)],
+    "nnf_hip_chain_forward_strided": [_VP, ctypes.POINTER(ChainDesc), _VP, _U32, _PP, _PP],
+    "nnf_hip_chain_forward_strided_status": [ctypes.POINTER(ChainDesc), _U32],
     "nnf_hip_stream_begin_capture": [_VP],
     "nnf_hip_stream_end_capture": [_VP, _PP],
     "nnf_hip_graph_launch": [_VP, _VP],

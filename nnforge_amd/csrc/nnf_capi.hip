@@ -133,6 +133,17 @@ extern "C"
 		return chain_forward_batch(static_cast<hipStream_t>(stream), group_count, descs, outputs, inputs, chunk_ptrs);
 	}
 
+	int nnf_hip_chain_forward_strided(void* stream, const nnf_hip_chain_desc* desc, float* output, uint32_t output_entry_stride,
+		const float* const* inputs, const float* const* chunk_ptrs)
+	{
+		return chain_forward_strided(static_cast<hipStream_t>(stream), desc, output, output_entry_stride, inputs, chunk_ptrs);
+	}
+
+	int nnf_hip_chain_forward_strided_status(const nnf_hip_chain_desc* desc, uint32_t output_entry_stride)
+	{
+		return chain_forward_strided_status(desc, output_entry_stride);
+	}
+
 	int nnf_hip_batch_norm_forward(void* stream, float* output, const float* input,
 		const float* gamma, const float* beta, const float* mean, const float* inverse_sigma,
 		uint32_t entry_count, uint32_t feature_map_count, uint32_t neuron_count_per_feature_map)

@@ -503,6 +503,46 @@ namespace nnf
 			chain_tile<NIN, BLOCK, U, DIRECT, PROGRAM>(a, blockIdx.x, lds_raw);
 		}
 
+		// A group whose result goes to a part of a wider tensor: entry e of the result starts out_entry_stride floats
+		// behind entry e - 1 instead of right behind it (the group writes its feature maps into the tensor of the Concat
+		// layer that would otherwise copy them there). The grid is (tiles of one entry) x (entries): a workgroup sees
+		// the arguments of a group of one entry, with the tensors' addresses moved to its entry, and does what
+		// chain_kernel does. The arguments' a.total is the number of elements of one entry.
+		template<int SLOTS>
+		struct chain_entry_view
+		{
+			const float* in[NNF_HIP_MAX_INPUTS];
+			float* out;
+			uint32_t total, fm_count, plane, plane_magic, span, has_add;
+			float alpha;
+			uint32_t arm_ops[NNF_HIP_MAX_INPUTS];
+			uint32_t tail_ops, slot_count, need_exp;
+			const chain_op (&ops)[NNF_HIP_MAX_OPS];
+			const chain_slot (&slots)[SLOTS];
+		};
+
+		template<int NIN, int BLOCK, int U, bool DIRECT>
+		__global__ void __launch_bounds__(BLOCK) chain_entries_kernel(const chain_args a, const uint32_t entry_count, const uint32_t out_entry_stride)
+		{
+			extern __shared__ __align__(16) unsigned char lds_raw[];
+			for(uint32_t entry = blockIdx.y; entry < entry_count; entry += gridDim.y)
+			{
+				chain_entry_view<max_slots> v = {
+					{}, a.out + static_cast<size_t>(entry) * out_entry_stride,
+					a.total, a.fm_count, a.plane, a.plane_magic, a.span, a.has_add, a.alpha,
+					{}, a.tail_ops, a.slot_count, a.need_exp, a.ops, a.slots };
+				#pragma unroll
+				for(int j = 0; j < NNF_HIP_MAX_INPUTS; ++j)
+				{
+					v.in[j] = (j < NIN) ? a.in[j] + static_cast<size_t>(entry) * a.total : nullptr;
+					v.arm_ops[j] = a.arm_ops[j];
+				}
+				chain_tile<NIN, BLOCK, U, DIRECT, 0>(v, blockIdx.x, lds_raw);
+				if (entry + gridDim.y < entry_count)
+					__syncthreads(); // the next entry's coefficients go where this one's are still being read
+			}
+		}
+
 		// Several groups that have nothing to do with each other in one launch: the grid is the groups' tiles one
 		// after the other, a workgroup finds its group by its index and then does what chain_kernel does. The time a
 		// launch loses while the device fills and drains is paid once for all of them (measured with 51 one-read-
@@ -768,8 +808,10 @@ namespace nnf
 
 		// Checks the call's arguments and fills p. single_launch: the group gets a launch of its own, so the grid
 		// that stays put is a candidate; as one of several groups of a launch it is not.
+		// wanted_shape >= 0: that launch shape and the interpreted layer list, whatever the size suggests (the launch over
+		// entries has instances for one shape).
 		int prepare_group(const nnf_hip_chain_desc* desc, float* output, const float* const* inputs, const float* const* chunk_ptrs,
-			bool single_launch, prepared_group& p)
+			bool single_launch, prepared_group& p, int wanted_shape = -1)
 		{
 			if ((desc == nullptr) || (output == nullptr) || (inputs == nullptr))
 				return NNF_HIP_EINVAL;
@@ -898,15 +940,17 @@ namespace nnf
 				return (a.total + tile - 1) / tile;
 			};
 
-			const int program = match_known_program(*desc, op_count);
+			const int program = (wanted_shape >= 0) ? 0 : match_known_program(*desc, op_count);
 			// the grid that stays put exists for the interpreted layer list with weights read straight from memory
 			auto persistent_possible = [&]() -> bool
 			{
 				return single_launch && (program == 0) && (desc->input_count <= persistent_max_inputs) && direct_of(persistent_shape);
 			};
-			int shape = forced_shape();
+			int shape = (wanted_shape >= 0) ? wanted_shape : forced_shape();
 			if ((shape == persistent_shape) && !persistent_possible())
 				shape = -1;
+			if ((wanted_shape >= 0) && (lds_bytes_of(shape) > max_dynamic_lds))
+				return NNF_HIP_EUNSUPPORTED;
 			const bool automatic = (shape < 0) || (lds_bytes_of(shape) > max_dynamic_lds);
 			if (automatic)
 			{
@@ -1064,6 +1108,62 @@ namespace nnf
 		prepared_group p;
 		const int rc = prepare_group(desc, output, inputs, chunk_ptrs, true, p);
 		return (rc != NNF_HIP_OK) ? rc : launch_group(stream, p);
+	}
+
+	// The launch over entries has instances for one or two inputs and 256 lanes x 2 float4s.
+	constexpr int strided_shape = 1;
+
+	int chain_forward_strided_status(const nnf_hip_chain_desc* desc, uint32_t output_entry_stride)
+	{
+		if (desc == nullptr)
+			return NNF_HIP_EINVAL;
+		const uint64_t per_entry = static_cast<uint64_t>(desc->feature_map_count) * desc->neuron_count_per_feature_map;
+		if ((per_entry == 0) || (desc->input_count < 1))
+			return NNF_HIP_EINVAL;
+		if (output_entry_stride < per_entry)
+			return NNF_HIP_EINVAL;
+		// every entry of the tensors starts on a 16-byte boundary, and at most two inputs
+		if (((per_entry % 4) != 0) || ((output_entry_stride % 4) != 0) || (desc->input_count > 2))
+			return NNF_HIP_EUNSUPPORTED;
+		if (static_cast<uint64_t>(desc->entry_count) * output_entry_stride > NNF_HIP_MAX_ELEMENT_COUNT)
+			return NNF_HIP_ETOOBIG;
+		return NNF_HIP_OK;
+	}
+
+	int chain_forward_strided(hipStream_t stream, const nnf_hip_chain_desc* desc, float* output, uint32_t output_entry_stride,
+		const float* const* inputs, const float* const* chunk_ptrs)
+	{
+		int rc = chain_forward_strided_status(desc, output_entry_stride);
+		if (rc != NNF_HIP_OK)
+			return rc;
+		if (desc->entry_count == 0)
+			return NNF_HIP_OK;
+		// planned as a group of one entry
+		nnf_hip_chain_desc one = *desc;
+		one.entry_count = 1;
+		prepared_group p;
+		rc = prepare_group(&one, output, inputs, chunk_ptrs, false, p, strided_shape);
+		if (rc != NNF_HIP_OK)
+			return rc;
+		// the whole of what is written and read
+		const size_t per_entry_bytes = p.bytes;
+		const size_t out_bytes = (static_cast<size_t>(desc->entry_count - 1) * output_entry_stride) * sizeof(float) + per_entry_bytes;
+		for(uint32_t j = 0; j < desc->input_count; ++j)
+			if (ranges_overlap(output, out_bytes, inputs[j], per_entry_bytes * desc->entry_count))
+				return NNF_HIP_EOVERLAP;
+		const dim3 grid(p.tiles, std::min(desc->entry_count, 65535u));
+		const dim3 block(launch_shapes[strided_shape].block);
+		if (desc->input_count == 1)
+		{
+			if (p.direct) NNF_LAUNCH((chain_entries_kernel<1, 256, 2, true>), grid, block, p.lds_bytes, stream, p.a, desc->entry_count, output_entry_stride);
+			else NNF_LAUNCH((chain_entries_kernel<1, 256, 2, false>), grid, block, p.lds_bytes, stream, p.a, desc->entry_count, output_entry_stride);
+		}
+		else
+		{
+			if (p.direct) NNF_LAUNCH((chain_entries_kernel<2, 256, 2, true>), grid, block, p.lds_bytes, stream, p.a, desc->entry_count, output_entry_stride);
+			else NNF_LAUNCH((chain_entries_kernel<2, 256, 2, false>), grid, block, p.lds_bytes, stream, p.a, desc->entry_count, output_entry_stride);
+		}
+		return launch_status();
 	}
 
 	int chain_forward_batch(hipStream_t stream, uint32_t group_count, const nnf_hip_chain_desc* descs, float* const* outputs,

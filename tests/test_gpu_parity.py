@@ -455,6 +455,70 @@ def test_independent_groups_in_one_call_equal_the_groups_one_by_one(gpu, first_s
         check_exact(out, group[7], "group %d of the call (seed %d)" % (i, first_seed + i))
 
 
+@pytest.mark.parametrize("n,c,plane,before,after,kind", [
+    (5, 64, 784, 32 * 784, 96 * 784, "bn_relu"),        # an Inception branch among others: weights straight from memory
+    (3, 8, 49, 12 * 49, 0, "bn_relu"),                  # planes of 49 floats: coefficients through LDS, last part of the wide tensor
+    (4, 16, 196, 0, 4 * 196, "bn_add_relu"),            # two inputs joined by an Add, first part
+    (70000, 4, 1, 8, 4, "prelu"),                       # more entries than the grid has rows: workgroups take several
+    (2, 6, 1000, 6000, 2000, "elu_tanh"),               # expf layers, one partly filled tile per entry
+    (0, 8, 16, 64, 64, "bn_relu"),                      # no entries
+])
+def test_group_written_into_a_wider_tensor(gpu, n, c, plane, before, after, kind):
+    """nnf_hip_chain_forward_strided: the group's result lands where a Concat layer would copy it, entry by entry, and
+    nothing around it is touched."""
+    gen = T.rng(18, n % 97 + c + plane)
+    per_entry = c * plane
+    stride = before + per_entry + after
+    x = config3_input((n, c, plane)) if kind == "elu_tanh" else T.normal(gen, (n, c, plane), 1.5)
+    inputs, chunks = [x], []
+    if kind == "bn_relu":
+        g, b, m, s = T.bn_params(gen, c)
+        arms, tail, chunks = [[(BN, 0), (RELU, 0, 0.0)]], [], [g, b, m, s]
+        want = oracle.rectified_linear(oracle.batch_norm(x, g, b, m, s))
+    elif kind == "bn_add_relu":
+        g, b, m, s = T.bn_params(gen, c)
+        r = T.normal(gen, (n, c, plane), 1.5)
+        inputs = [r, x]
+        arms, tail, chunks = [[], [(BN, 0)]], [(RELU, 0, 0.1)], [g, b, m, s]
+        want = oracle.rectified_linear(oracle.add([r, oracle.batch_norm(x, g, b, m, s)]).reshape(x.shape), 0.1)
+    elif kind == "prelu":
+        a = T.uniform(gen, c, -0.5, 0.5)
+        arms, tail, chunks = [[(PRELU, 0)]], [], [a]
+        want = oracle.parametric_rectified_linear(x, a)
+    else:
+        arms, tail = [[(ELU,), (TANH, 0, T.TANH_SCALE, T.TANH_STEEPNESS)]], []
+        want = oracle.hyperbolic_tangent(oracle.exponential_linear(x), T.TANH_SCALE, T.TANH_STEEPNESS)
+    desc = capi.make_desc(n, c, plane, arms, tail)
+    assert gpu.lib.nnf_hip_chain_forward_strided_status(ctypes.byref(desc), stride) == 0
+    sentinel = np.float32(-12345.5)
+    wide = gpu.torch.full((max(1, n * stride),), float(sentinel), dtype=gpu.torch.float32, device=gpu.device)
+    d_in = [gpu.to_device(a if a.size else np.zeros(4, np.float32)) for a in inputs]
+    d_chunks = [gpu.to_device(a) for a in chunks]
+    ins = capi.pointer_array([t.data_ptr() for t in d_in])
+    chk = capi.pointer_array([t.data_ptr() for t in d_chunks])
+    rc = gpu.lib.nnf_hip_chain_forward_strided(gpu.stream, ctypes.byref(desc), wide.data_ptr() + 4 * before, stride, ins, chk if d_chunks else None)
+    assert rc == 0, capi.error_string(rc)
+    got = gpu.to_host(wide)[:n * stride].reshape(n, stride)
+    check_exact(got[:, before:before + per_entry], want, "the group's part of the wide tensor")
+    assert (got[:, :before] == sentinel).all() and (got[:, before + per_entry:] == sentinel).all(), "the rest of the wide tensor is untouched"
+
+
+def test_group_written_into_a_wider_tensor_refuses_what_it_cannot_do(gpu):
+    desc = capi.make_desc(2, 3, 5, [[(RELU, 0, 0.0)]], [])           # 15 floats per entry: entries would not start on 16 bytes
+    assert gpu.lib.nnf_hip_chain_forward_strided_status(ctypes.byref(desc), 32) == capi.E_UNSUPPORTED
+    desc = capi.make_desc(2, 4, 4, [[(RELU, 0, 0.0)]], [])
+    assert gpu.lib.nnf_hip_chain_forward_strided_status(ctypes.byref(desc), 18) == capi.E_UNSUPPORTED   # stride not a multiple of 4
+    assert gpu.lib.nnf_hip_chain_forward_strided_status(ctypes.byref(desc), 12) == capi.E_INVAL         # narrower than the group
+    desc = capi.make_desc(2, 4, 4, [[], [], []], [(RELU, 0, 0.0)])
+    assert gpu.lib.nnf_hip_chain_forward_strided_status(ctypes.byref(desc), 32) == capi.E_UNSUPPORTED   # three inputs
+    # the written range may not reach into an input
+    desc = capi.make_desc(2, 4, 4, [[(RELU, 0, 0.0)]], [])
+    buf = gpu.torch.zeros(256, dtype=gpu.torch.float32, device=gpu.device)
+    ins = capi.pointer_array([buf.data_ptr() + 4 * 40])
+    assert gpu.lib.nnf_hip_chain_forward_strided(gpu.stream, ctypes.byref(desc), buf.data_ptr(), 32, ins, None) == capi.E_OVERLAP
+    gpu.torch.cuda.synchronize()
+
+
 def test_recorded_launches_replay_with_the_results_of_launching(gpu):
     """nnf_hip_stream_begin_capture / nnf_hip_stream_end_capture / nnf_hip_graph_launch: a fused group, a softmax and a whole-plane
     average recorded once on a stream of their own, then replayed four times with new values in the same input
