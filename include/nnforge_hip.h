@@ -189,6 +189,11 @@ NNF_HIP_API int nnf_hip_average_subsampling_forward(void* stream, float* output,
  * per feature map of input i. */
 NNF_HIP_API int nnf_hip_concat_forward(void* stream, float* output, const float* const* inputs,
 	const uint32_t* input_neuron_counts, uint32_t input_count, uint32_t entry_count);
+/* The same with some inputs already where they belong: input i with inputs_in_place[i] != 0 was written into its part of
+ * `output` by whoever made it (nnf_hip_chain_forward_strided) and is not copied - its pointer is not looked at; the others
+ * are copied to their parts as above. With every input in place nothing is launched. */
+NNF_HIP_API int nnf_hip_concat_forward_partial(void* stream, float* output, const float* const* inputs,
+	const uint32_t* input_neuron_counts, const uint8_t* inputs_in_place, uint32_t input_count, uint32_t entry_count);
 
 /* Maxout: output feature map o = maximum over the input feature maps o, o + output_feature_map_count,
  * o + 2*output_feature_map_count, ... (feature_map_subsampling_size of them), folded with

@@ -95,6 +95,9 @@ namespace nnforge
 			// on the 49 groups of the ResNet-50 post-convolution stack, all in one call: 64 entries 1091 -> 1042 us,
 			// 8 entries 243 -> 172 us.
 			bool batch_independent_groups;
+			// A fused group that only a Concat layer reads writes its result into that layer's output instead of a
+			// tensor of its own that the Concat would copy (measured in DESIGN.md); switch off to have every Concat copy
+			bool concat_in_place = true;
 			unsigned int reserved_thread_count;
 			// run() makes its packets no larger than this much pinned staging (input + output entries) per I/O slot, so that
 			// reading, copying, computing and writing of neighbouring packets overlap; 0: no bound. It never pushes a
@@ -184,6 +187,18 @@ namespace nnforge
 				const float * const * chunk_ptrs,
 				unsigned int entry_count);
 
+			// A tester that only puts its inputs side by side (Concat) need not copy an input that was written to its
+			// place in the output buffer by the step that made it. can_take_inputs_in_place: whether this tester can
+			// leave inputs out; enqueue_forward_propagation_with_inputs_in_place: the forward pass for the inputs
+			// whose flag is false (the buffers of the others are not looked at).
+			virtual bool can_take_inputs_in_place() const { return false; }
+			virtual void enqueue_forward_propagation_with_inputs_in_place(
+				void * stream_id,
+				hip_linear_buffer_device::ptr output_buffer,
+				const std::vector<hip_linear_buffer_device::const_ptr>& input_buffers,
+				const std::vector<bool>& inputs_in_place,
+				unsigned int entry_count);
+
 		protected:
 			layer_tester_hip() = default;
 			virtual void tester_configured() {}
@@ -258,6 +273,11 @@ namespace nnforge
 			// Consecutive fused groups that do not depend on each other are handed to the kernels in one call
 			// (nnf_hip_chain_forward_batch): steps with the same index >= 0 form such a run; -1: launched on its own.
 			int batch_index = -1;
+			// A fused group that writes its result straight into the output of the Concat layer behind it (entry by entry,
+			// at its feature maps' place): the name of that layer, empty otherwise. For the Concat step itself: the inputs
+			// it finds in place and does not copy.
+			std::string writes_into;
+			std::vector<std::string> inputs_in_place;
 			std::string description() const;       // e.g. "bn1+add1+relu1 <- conv_a, conv_b"
 		};
 
@@ -374,6 +394,7 @@ namespace nnforge
 			int hip_max_entry_count;
 			int hip_reserved_thread_count;
 			int hip_max_io_staging_mb;
+			bool hip_concat_in_place;
 
 		private:
 			hip_running_configuration::const_ptr hip_config;

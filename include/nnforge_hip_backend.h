@@ -66,6 +66,8 @@ typedef struct nnf_backend_options
 	int32_t max_io_staging_mb;     /* hip_max_io_staging_mb: pinned staging (input + output entries) per I/O slot that bounds a
 	                                  packet of run(); 0: default (64), < 0: no bound */
 	int32_t resident_packets;      /* nnf_backend_time_kernels: sets of data / output buffers the timed passes go round; <= 0: 1 */
+	int32_t concat_copies_every_input; /* 1: hip_concat_in_place off (every Concat layer copies all its inputs; by default fused groups
+	                                  that only a Concat reads write their results into its output) */
 	int32_t replay_recorded_plan;  /* nnf_backend_time_kernels: 1: the launches of a pass are recorded once as a HIP graph and the
 	                                  timed passes replay it (one kernel stream) */
 	int32_t keep_unregistered_layers; /* 1: a layer of a type this backend has no class for (Convolution, LCS, LError ...) does not

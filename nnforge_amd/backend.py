@@ -33,7 +33,7 @@ class Options(ctypes.Structure):
                 ("profile", ctypes.c_int32), ("weights_from_folder", ctypes.c_int32), ("weights_folder", ctypes.c_char_p),
                 ("profile_folder", ctypes.c_char_p), ("stat_on_host", ctypes.c_int32), ("kernel_stream_count", ctypes.c_int32),
                 ("one_launch_per_group", ctypes.c_int32), ("host_thread_count", ctypes.c_int32), ("max_io_staging_mb", ctypes.c_int32),
-                ("resident_packets", ctypes.c_int32), ("replay_recorded_plan", ctypes.c_int32), ("keep_unregistered_layers", ctypes.c_int32)]
+                ("resident_packets", ctypes.c_int32), ("concat_copies_every_input", ctypes.c_int32), ("replay_recorded_plan", ctypes.c_int32), ("keep_unregistered_layers", ctypes.c_int32)]
 
 
 class DatasetFile(ctypes.Structure):
@@ -89,8 +89,10 @@ def load():
 
 def _options(fuse=True, dont_share_buffers=False, max_entry_count=0, profile=False, weights_folder=None,
              profile_folder=None, stat_on_host=False, kernel_stream_count=0, one_launch_per_group=False, host_thread_count=0,
-             max_io_staging_mb=0, resident_packets=0, keep_unregistered_layers=False, replay_recorded_plan=False):
+             max_io_staging_mb=0, resident_packets=0, keep_unregistered_layers=False, replay_recorded_plan=False,
+             concat_copies_every_input=False):
     o = Options()
+    o.concat_copies_every_input = int(concat_copies_every_input)
     o.replay_recorded_plan = int(replay_recorded_plan)
     o.keep_unregistered_layers = int(keep_unregistered_layers)
     o.struct_size = ctypes.sizeof(Options)
@@ -158,10 +160,13 @@ def parse_report(text):
             # "fused|single <layers> <- <inputs> @<kernel stream>[ #<run of groups launched together>]"
             kind, _, desc = rest.partition(" ")
             desc, _, placement = desc.rpartition(" @")
+            placement, _, in_place = placement.partition(" =")
+            placement, _, writes_into = placement.partition(" >")
             stream, _, run = placement.partition(" #")
             layers, _, sources = desc.partition(" <- ")
             res["steps"].append({"fused": kind == "fused", "layers": layers.split("+"), "inputs": sources.split(", "), "stream": int(stream),
-                                 "run": int(run) if run else None})
+                                 "run": int(run) if run else None, "writes_into": writes_into or None,
+                                 "inputs_in_place": in_place.split(",") if in_place else []})
         elif key in ("per_entry_bytes", "max_entry_count", "entries", "writer_entries", "launches", "timed_entries", "packet_entries", "plan_steps", "resident_packets"):
             res[key] = int(rest)
         elif key in ("wall_seconds_per_pass", "device_seconds_per_pass", "host_seconds_per_pass"):

@@ -198,7 +198,13 @@ extern "C"
 	int nnf_hip_concat_forward(void* stream, float* output, const float* const* inputs,
 		const uint32_t* input_neuron_counts, uint32_t input_count, uint32_t entry_count)
 	{
-		return concat_forward(static_cast<hipStream_t>(stream), output, inputs, input_neuron_counts, input_count, entry_count);
+		return concat_forward(static_cast<hipStream_t>(stream), output, inputs, input_neuron_counts, nullptr, input_count, entry_count);
+	}
+
+	int nnf_hip_concat_forward_partial(void* stream, float* output, const float* const* inputs,
+		const uint32_t* input_neuron_counts, const uint8_t* inputs_in_place, uint32_t input_count, uint32_t entry_count)
+	{
+		return concat_forward(static_cast<hipStream_t>(stream), output, inputs, input_neuron_counts, inputs_in_place, input_count, entry_count);
 	}
 
 	int nnf_hip_maxout_forward(void* stream, float* output, const float* input,
@@ -598,7 +604,7 @@ extern "C"
 			return hip_status(e);
 		hipGraphExec_t exec = nullptr;
 		e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
-		hipGraphDestroy(graph);
+		(void)hipGraphDestroy(graph);
 		if (e != hipSuccess)
 			return hip_status(e);
 		*graph_exec = exec;

@@ -135,7 +135,7 @@ namespace nnf
 		uint32_t entry_count, uint32_t feature_map_count, uint32_t input_width, uint32_t input_height,
 		uint32_t window_width, uint32_t window_height, float mult);
 	int concat_forward(hipStream_t stream, float* output, const float* const* inputs, const uint32_t* input_neuron_counts,
-		uint32_t input_count, uint32_t entry_count);
+		const uint8_t* inputs_in_place, uint32_t input_count, uint32_t entry_count);
 	int maxout_forward(hipStream_t stream, float* output, const float* input,
 		uint32_t entry_count, uint32_t output_feature_map_count, uint32_t neuron_count_per_feature_map,
 		uint32_t feature_map_subsampling_size);

@@ -83,9 +83,11 @@ namespace nnf
 		}
 	}
 
+	// inputs_in_place (may be null): inputs that lie in their part of the output already; they take their room and no copy
 	int concat_forward(hipStream_t stream, float* output, const float* const* inputs, const uint32_t* input_neuron_counts,
-		uint32_t input_count, uint32_t entry_count)
+		const uint8_t* inputs_in_place, uint32_t input_count, uint32_t entry_count)
 	{
+		const auto in_place = [inputs_in_place] (uint32_t i) { return (inputs_in_place != nullptr) && (inputs_in_place[i] != 0); };
 		if ((output == nullptr) || (inputs == nullptr) || (input_neuron_counts == nullptr) || (input_count == 0))
 			return NNF_HIP_EINVAL;
 		if (!is_aligned16(output))
@@ -94,7 +96,7 @@ namespace nnf
 		bool vector = true;
 		for(uint32_t i = 0; i < input_count; ++i)
 		{
-			if (input_neuron_counts[i] != 0) // an input without neurons is never read
+			if ((input_neuron_counts[i] != 0) && !in_place(i)) // an input without neurons is never read
 			{
 				if (inputs[i] == nullptr)
 					return NNF_HIP_EINVAL;
@@ -112,7 +114,7 @@ namespace nnf
 		for(uint32_t i = 0; i < input_count; ++i)
 		{
 			const uintptr_t a = reinterpret_cast<uintptr_t>(output), b = reinterpret_cast<uintptr_t>(inputs[i]);
-			const uint64_t b_bytes = static_cast<uint64_t>(input_neuron_counts[i]) * entry_count * sizeof(float);
+			const uint64_t b_bytes = in_place(i) ? 0 : static_cast<uint64_t>(input_neuron_counts[i]) * entry_count * sizeof(float);
 			if ((b_bytes != 0) && (a < b + b_bytes) && (b < a + output_total * sizeof(float)))
 				return NNF_HIP_EOVERLAP;
 		}
@@ -129,12 +131,12 @@ namespace nnf
 			uint32_t blocks = 0;
 			for(uint32_t i = 0; i < a.input_count; ++i)
 			{
-				a.in[i] = inputs[first + i];
+				a.in[i] = in_place(first + i) ? nullptr : inputs[first + i];
 				a.length[i] = input_neuron_counts[first + i];
 				a.offset[i] = offset;
 				a.first_block[i] = blocks;
 				offset += a.length[i];
-				blocks += (a.length[i] + per_block - 1) / per_block;
+				blocks += in_place(first + i) ? 0 : (a.length[i] + per_block - 1) / per_block;
 			}
 			a.first_block[a.input_count] = blocks;
 			if (blocks == 0)

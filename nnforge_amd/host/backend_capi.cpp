@@ -47,12 +47,21 @@ namespace
 
 	void describe_plan(const hip::forward_propagation_hip& fp, std::ostream& out)
 	{
-		// "step: fused|single <layers> <- <inputs> @<kernel stream>[ #<run of groups launched together>]"
+		// "step: fused|single <layers> <- <inputs> @<kernel stream>[ #<run of groups launched together>][ ><Concat layer the
+		// group writes into>][ =<inputs the Concat finds in place, comma separated>]"
 		for(const hip::forward_step& s : fp.get_steps())
 		{
 			out << "step: " << (s.fused ? "fused " : "single ") << s.description() << " @" << s.stream_index;
 			if (s.batch_index >= 0)
 				out << " #" << s.batch_index;
+			if (!s.writes_into.empty())
+				out << " >" << s.writes_into;
+			if (!s.inputs_in_place.empty())
+			{
+				out << " =";
+				for(size_t i = 0; i < s.inputs_in_place.size(); ++i)
+					out << (i == 0 ? "" : ",") << s.inputs_in_place[i];
+			}
 			out << "\n";
 		}
 		out << "per_entry_bytes: " << fp.get_per_entry_buffer_bytes() << "\n";
@@ -80,6 +89,7 @@ namespace
 		generator.apply_default_options();
 		if (options != nullptr)
 		{
+			generator.hip_concat_in_place = options->concat_copies_every_input == 0;
 			if (options->max_io_staging_mb != 0)
 				generator.hip_max_io_staging_mb = std::max(0, options->max_io_staging_mb);
 			generator.hip_fuse = options->fuse != 0;
@@ -463,7 +473,10 @@ extern "C"
 			const int max_entries = ((options != nullptr) && (options->max_entry_count > 0)) ? options->max_entry_count : 4096;
 			const int kernel_streams = ((options != nullptr) && (options->kernel_stream_count > 0)) ? options->kernel_stream_count : hip::hip_running_configuration::default_kernel_stream_count;
 			const bool batch = (options == nullptr) || (options->one_launch_per_group == 0);
-			hip::hip_running_configuration::const_ptr config = hip::hip_running_configuration::create_offline(memory_bytes, 0.9F, fuse, dont_share, max_entries, kernel_streams, batch);
+			std::shared_ptr<hip::hip_running_configuration> offline = std::const_pointer_cast<hip::hip_running_configuration>(
+				hip::hip_running_configuration::create_offline(memory_bytes, 0.9F, fuse, dont_share, max_entries, kernel_streams, batch));
+			offline->concat_in_place = (options == nullptr) || (options->concat_copies_every_input == 0);
+			hip::hip_running_configuration::const_ptr config = offline;
 			hip::forward_propagation_hip fp(schema, output_names, debug_state::ptr(new debug_state(false)), profile_state::ptr(new profile_state(false)), config);
 			fp.set_input_configuration_specific(input_configs(inputs, input_count));
 			describe_plan(fp, out);

@@ -66,9 +66,15 @@ namespace nnforge
 				std::vector<int> input_buffers;
 				bool passes_input_on = false;        // every layer of the step is a Dropout
 				bool prologue = false;               // desc holds element-wise layers that the tester (a subsampling layer) applies to its input
+				// a fused group that writes into the output of the Concat layer behind it: where its feature maps start inside
+				// an entry of that output, and how long such an entry is (floats); stride 0: an ordinary step
+				uint32_t view_offset = 0, view_stride = 0;
+				std::vector<bool> inputs_in_place;   // a Concat step: the inputs that lie in its output already
 				unsigned int entry_factor = 1;       // entries of the step's output per entry read (the cumulative tiling factor of its last layer)
-				bool launches_nothing() const        // Dropout layers only, in place: nothing to do at inference
+				bool launches_nothing() const        // Dropout layers only, in place: nothing to do at inference; a Concat with every input in place
 				{
+					if (!inputs_in_place.empty())
+						return std::find(inputs_in_place.begin(), inputs_in_place.end(), false) == inputs_in_place.end();
 					return passes_input_on && (output_buffer == input_buffers.at(0));
 				}
 			};
@@ -246,9 +252,15 @@ namespace nnforge
 					std::vector<const float *> in_ptrs;
 					for(const hip_linear_buffer_device::const_ptr& b : inputs)
 						in_ptrs.push_back(static_cast<const float *>(*b));
-					hip_safe_call(nnf_hip_chain_forward(step_stream, &plan.desc, *buffers[plan.output_buffer], in_ptrs.data(),
-						chunk_ptrs[i].empty() ? nullptr : chunk_ptrs[i].data()));
+					if (plan.view_stride != 0)
+						hip_safe_call(nnf_hip_chain_forward_strided(step_stream, &plan.desc, static_cast<float *>(*buffers[plan.output_buffer]) + plan.view_offset,
+							plan.view_stride, in_ptrs.data(), chunk_ptrs[i].empty() ? nullptr : chunk_ptrs[i].data()));
+					else
+						hip_safe_call(nnf_hip_chain_forward(step_stream, &plan.desc, *buffers[plan.output_buffer], in_ptrs.data(),
+							chunk_ptrs[i].empty() ? nullptr : chunk_ptrs[i].data()));
 				}
+				else if (!plan.inputs_in_place.empty())
+					plan.tester->enqueue_forward_propagation_with_inputs_in_place(step_stream, buffers[plan.output_buffer], inputs, plan.inputs_in_place, step_entries);
 				else
 				{
 					const std::string& layer_name = plan.info.layer_names[0];
@@ -488,6 +500,68 @@ namespace nnforge
 			while (!pending.empty())
 				materialize(pending.begin()->first);
 
+			// ---- groups that write into the Concat layer behind them -----------------------------------------
+			// A Concat layer only puts its inputs side by side, entry by entry (nnforge/plain/concat_layer_tester_plain.cpp:
+			// 45-58). A fused group that nothing else reads can write its result there itself: its launch goes over
+			// (tiles of an entry) x (entries) and steps from entry to entry by the Concat's neuron count
+			// (nnf_hip_chain_forward_strided), the group's own tensor is never made, and the Concat copies only the inputs
+			// that are not such groups - nothing at all when every input is one. What qualifies: a group with at most two
+			// inputs, read by the Concat alone and no output itself, whose entries and whose place in the Concat's entry
+			// start on 16-byte boundaries, and large enough per entry for a launch over entries to be worth it.
+			struct concat_view
+			{
+				std::string concat;
+				uint32_t offset, stride;
+			};
+			std::map<std::string, concat_view> view_of;                        // by the group's name (its last layer)
+			std::map<std::string, std::vector<bool> > concat_inputs_in_place;  // by the Concat layer's name
+			if (hip_config->fuse_layers && hip_config->concat_in_place)
+			{
+				constexpr unsigned int min_view_floats_per_entry = 1024;
+				std::map<std::string, const pending_group *> group_named;
+				for(const std::pair<std::string, pending_group>& g : groups)
+					group_named[g.first] = &g.second;
+				for(const std::pair<std::string, bool>& so : step_order)
+				{
+					if (so.second || (prologues.find(so.first) != prologues.end()))
+						continue;
+					layer::const_ptr l = this->schema->get_layer(so.first);
+					if ((l->get_type_name() != concat_layer::layer_type_name) || !p->testers[so.first]->can_take_inputs_in_place())
+						continue;
+					const uint32_t stride = layer_config_map[so.first].get_neuron_count();
+					std::vector<bool> flags;
+					uint32_t offset = 0;
+					bool any = false;
+					for(const std::string& input : l->input_layer_instance_names)
+					{
+						const layer_configuration_specific& input_config = layer_config_map[input];
+						const uint32_t count = input_config.get_neuron_count();
+						bool in_place = false;
+						std::map<std::string, const pending_group *>::const_iterator g = group_named.find(input);
+						if ((g != group_named.end()) && (this->schema->get_consumer_count(input) == 1) && (outputs.find(input) == outputs.end())
+							&& (view_of.find(input) == view_of.end()) && (count >= min_view_floats_per_entry) && ((offset % 4) == 0))
+						{
+							nnf_hip_chain_desc shape;
+							std::memset(&shape, 0, sizeof(shape));
+							shape.entry_count = 1;
+							shape.feature_map_count = input_config.feature_map_count;
+							shape.neuron_count_per_feature_map = input_config.get_neuron_count_per_feature_map();
+							shape.input_count = static_cast<uint32_t>(g->second->arms.size());
+							in_place = nnf_hip_chain_forward_strided_status(&shape, stride) == NNF_HIP_OK;
+						}
+						if (in_place)
+						{
+							view_of[input] = concat_view{ so.first, offset, stride };
+							any = true;
+						}
+						flags.push_back(in_place);
+						offset += count;
+					}
+					if (any)
+						concat_inputs_in_place[so.first] = flags;
+				}
+			}
+
 			// ---- order: which steps share a launch ---------------------------------------------------------
 			// With independent groups launched together (see below) a run of such groups ends where a step depends on
 			// one of them, so the order of the steps decides how many launches there are and how large each is. Every
@@ -521,7 +595,8 @@ namespace nnforge
 						const pending_group& g = *group_of[name];
 						for(const pending_arm& a : g.arms)
 							sources.push_back(a.source);
-						joins_launches[i] = (g.op_count() + (g.add_layer_name.empty() ? 0 : 1)) > 1; // a single layer is its tester's launch
+						// a single layer is its tester's launch; a group that writes into a Concat's output has a launch of its own
+						joins_launches[i] = ((g.op_count() + (g.add_layer_name.empty() ? 0 : 1)) > 1) && (view_of.find(name) == view_of.end());
 						bytes[i] = static_cast<double>(layer_config_map[name].get_neuron_count()) * static_cast<double>(g.arms.size() + 1);
 					}
 					else if (prologues.find(name) != prologues.end())
@@ -696,7 +771,8 @@ namespace nnforge
 						plan.info.layer_names.push_back(g.add_layer_name);
 					for(const std::string& op : g.tail)
 						plan.info.layer_names.push_back(op);
-					if (single_layer)
+					std::map<std::string, concat_view>::const_iterator view = view_of.find(name);
+					if (single_layer && (view == view_of.end()))
 					{
 						// a group of one layer is that layer's own tester
 						plan.info.fused = false;
@@ -707,6 +783,19 @@ namespace nnforge
 						plan.info.fused = true;
 						fill_desc(g, config);
 					}
+					if (view != view_of.end())
+					{
+						plan.view_offset = view->second.offset;
+						plan.view_stride = view->second.stride;
+						plan.info.writes_into = view->second.concat;
+					}
+				}
+				if (!so.second && (concat_inputs_in_place.find(name) != concat_inputs_in_place.end()))
+				{
+					plan.inputs_in_place = concat_inputs_in_place[name];
+					for(size_t j = 0; j < plan.inputs_in_place.size(); ++j)
+						if (plan.inputs_in_place[j])
+							plan.info.inputs_in_place.push_back(plan.info.input_names[j]);
 				}
 				// report bookkeeping: name, layer types, flops (the reference's model) and memory traffic per entry
 				std::string types;
@@ -727,6 +816,9 @@ namespace nnforge
 				float step_bytes = static_cast<float>(config.get_neuron_count()) * sizeof(float) * static_cast<float>(plan.entry_factor);
 				for(const std::string& input : plan.info.input_names)
 					step_bytes += static_cast<float>(layer_config_map[input].get_neuron_count()) * sizeof(float) * static_cast<float>(cumulative_tiling_factor_map.at(input));
+				// what a Concat finds in place it neither reads nor writes
+				for(const std::string& input : plan.info.inputs_in_place)
+					step_bytes -= 2.0F * static_cast<float>(layer_config_map[input].get_neuron_count()) * sizeof(float) * static_cast<float>(cumulative_tiling_factor_map.at(input));
 				plan.action = layer_name_with_action(plan.info.layer_names.back(), layer_action(layer_action::forward));
 				action_flops_per_entry[plan.action] = step_flops;
 				action_bytes_per_entry[plan.action] = step_bytes;
@@ -768,17 +860,23 @@ namespace nnforge
 					freed_in_this_slot.clear();
 				}
 				const std::string& out_name = plan.info.layer_names.back();
+				// the value whose buffer the step writes: its own, or the output of the Concat layer it writes into
+				const std::string& buffer_owner = plan.info.writes_into.empty() ? out_name : plan.info.writes_into;
 				// per entry read: a layer behind a tiling layer holds several entries for each (nnforge/plain/forward_propagation_plain.cpp:281)
-				const size_t out_floats = static_cast<size_t>(layer_config_map[out_name].get_neuron_count()) * plan.entry_factor;
+				const size_t out_floats = static_cast<size_t>(layer_config_map[buffer_owner].get_neuron_count()) * plan.entry_factor;
 				for(const std::string& in : plan.info.input_names)
 					plan.input_buffers.push_back(p->value_to_buffer.at(in));
 
-				const bool dedicated = (outputs.find(out_name) != outputs.end()) || hip_config->dont_share_buffers;
+				const bool dedicated = (outputs.find(buffer_owner) != outputs.end()) || hip_config->dont_share_buffers;
 				int chosen = -1;
-				if (!dedicated)
+				// a Concat's buffer exists from the first group that writes into it
+				const std::map<std::string, int>::const_iterator planned = p->value_to_buffer.find(buffer_owner);
+				if (planned != p->value_to_buffer.end())
+					chosen = planned->second;
+				if (!dedicated && (chosen < 0))
 				{
 					// in place: the first input dies here, nothing else reads its buffer in this step, same size
-					const int can_write = plan.prologue ? -1 : (plan.info.fused ? 0 : plan.tester->get_input_index_layer_can_write());
+					const int can_write = (plan.prologue || (plan.view_stride != 0)) ? -1 : (plan.info.fused ? 0 : plan.tester->get_input_index_layer_can_write());
 					if (can_write == 0)
 					{
 						const int b0 = plan.input_buffers[0];
@@ -813,6 +911,7 @@ namespace nnforge
 				}
 				plan.output_buffer = chosen;
 				p->value_to_buffer[out_name] = chosen;
+				p->value_to_buffer[buffer_owner] = chosen;
 
 				// inputs that die here return to the pool (unless just reused in place)
 				for(size_t j = 0; j < plan.info.input_names.size(); ++j)
@@ -904,7 +1003,7 @@ namespace nnforge
 					plan.info.batch_index = -1;
 					if (plan.launches_nothing())
 						continue; // no launch: neither joins a run nor ends one
-					const bool can_join = batching && plan.info.fused && !plan.prologue;
+					const bool can_join = batching && plan.info.fused && !plan.prologue && (plan.view_stride == 0);
 					bool depends_on_run = false;
 					for(int member : run)
 						depends_on_run = depends_on_run || (depends_directly_on[i].find(member) != depends_directly_on[i].end());
@@ -1505,6 +1604,7 @@ namespace nnforge
 			, hip_max_entry_count(4096)
 			, hip_reserved_thread_count(1)
 			, hip_max_io_staging_mb(64)
+			, hip_concat_in_place(true)
 		{
 		}
 
@@ -1516,6 +1616,7 @@ namespace nnforge
 				hip_single_command_stream ? 1 : std::max(1, hip_kernel_stream_count), hip_batch_independent_groups,
 				static_cast<unsigned int>(std::max(0, hip_reserved_thread_count))));
 			config->max_io_staging_bytes = static_cast<size_t>(std::max(0, hip_max_io_staging_mb)) << 20;
+			config->concat_in_place = hip_concat_in_place;
 			hip_config = config;
 		}
 
@@ -1543,6 +1644,7 @@ namespace nnforge
 			res.push_back(bool_option("hip_fuse", &hip_fuse, true, "Fuse runs of element-wise layers (BatchNorm, activations, Add) into single kernel launches"));
 			res.push_back(bool_option("hip_dont_share_buffers", &hip_dont_share_buffers, false, "Don't share buffers between layers. Switch it on if you suspect a bug in there"));
 			res.push_back(bool_option("hip_single_command_stream", &hip_single_command_stream, false, "Use single stream for kernels. Switch it on if you suspect a bug in there"));
+			res.push_back(bool_option("hip_concat_in_place", &hip_concat_in_place, true, "Fused groups that only a Concat layer reads write their results into its output instead of having them copied there"));
 			res.push_back(bool_option("hip_batch_independent_groups", &hip_batch_independent_groups, true, "Launch consecutive fused groups that do not depend on each other together (takes one kernel stream)"));
 			return res;
 		}

@@ -184,6 +184,12 @@ namespace nnforge
 			throw neural_network_exception("Layer " + layer_schema->instance_name + " of type " + layer_schema->get_type_name() + " cannot apply other layers to its input");
 		}
 
+		void layer_tester_hip::enqueue_forward_propagation_with_inputs_in_place(void *, hip_linear_buffer_device::ptr, const std::vector<hip_linear_buffer_device::const_ptr>&,
+			const std::vector<bool>&, unsigned int)
+		{
+			throw neural_network_exception("Layer " + layer_schema->instance_name + " of type " + layer_schema->get_type_name() + " reads all its inputs: none of them can be taken as being in place");
+		}
+
 		layer_testing_schema::ptr layer_testing_schema::create(layer::const_ptr layer_schema) const
 		{
 			layer_testing_schema::ptr res = create_specific();
@@ -631,6 +637,26 @@ namespace nnforge
 						counts.push_back(input_elem_count_per_entry_list[i]);
 					}
 					hip_safe_call(nnf_hip_concat_forward(stream_id, *output_buffer, inputs.data(), counts.data(), static_cast<uint32_t>(inputs.size()), entry_count));
+				}
+
+				bool can_take_inputs_in_place() const override { return true; }
+
+				void enqueue_forward_propagation_with_inputs_in_place(void * stream_id, hip_linear_buffer_device::ptr output_buffer,
+					const std::vector<hip_linear_buffer_device::const_ptr>& input_buffers, const std::vector<bool>& inputs_in_place, unsigned int entry_count) override
+				{
+					require_inputs(input_buffers, input_elem_count_per_entry_list.size(), "Concat");
+					if (inputs_in_place.size() != input_buffers.size())
+						throw neural_network_exception("Concat: " + std::to_string(inputs_in_place.size()) + " flags for " + std::to_string(input_buffers.size()) + " inputs");
+					std::vector<const float *> inputs;
+					std::vector<uint32_t> counts;
+					std::vector<uint8_t> flags;
+					for(size_t i = 0; i < input_elem_count_per_entry_list.size(); ++i)
+					{
+						inputs.push_back(inputs_in_place[i] ? nullptr : float_ptr(input_buffers[i]));
+						counts.push_back(input_elem_count_per_entry_list[i]);
+						flags.push_back(inputs_in_place[i] ? 1 : 0);
+					}
+					hip_safe_call(nnf_hip_concat_forward_partial(stream_id, *output_buffer, inputs.data(), counts.data(), flags.data(), static_cast<uint32_t>(inputs.size()), entry_count));
 				}
 			};
 

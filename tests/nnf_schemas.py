@@ -182,6 +182,22 @@ def inception_like(c=8):
     ]
 
 
+def inception_block(c=16):
+    """Four branches behind one input, each ending in a fused group that only the Concat reads - BatchNorm -> ReLU twice
+    (different widths), a PReLU on its own, and BatchNorm + a second input joined by an Add -> ReLU - then Concat, Maxout
+    and an activation: the block whose Concat has nothing to copy."""
+    return [
+        L("Data", "conv_a"), L("Data", "conv_b"), L("Data", "conv_c"), L("Data", "conv_d"), L("Data", "conv_e"),
+        L("BatchNorm", "a_bn", ["conv_a"], feature_map_count=c), L("ReLU", "a_relu", ["a_bn"]),
+        L("BatchNorm", "b_bn", ["conv_b"], feature_map_count=2 * c), L("ReLU", "b_relu", ["b_bn"], negative_slope=0.125),
+        L("PReLU", "c_prelu", ["conv_c"], feature_map_count=c),
+        L("BatchNorm", "d_bn", ["conv_d"], feature_map_count=c), L("Add", "d_sum", ["conv_e", "d_bn"]), L("ReLU", "d_relu", ["d_sum"]),
+        L("Concat", "join", ["a_relu", "b_relu", "c_prelu", "d_relu"]),
+        L("Maxout", "mo", ["join"], feature_map_subsampling_size=5),
+        L("TanH", "out", ["mo"], scale=1.7159, steepness=0.6666),
+    ]
+
+
 def random_network(gen, layer_count=14, c=6, size=12, with_entry_factors=False):
     """A random DAG of the layer types the backend runs: chains of element-wise layers, Adds and Concats of values of
     equal shape, Maxout, max / min / average pooling, with some values consumed more than once. with_entry_factors:

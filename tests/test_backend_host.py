@@ -315,6 +315,73 @@ def test_plan_of_the_inception_like_block():
     assert rep["steps"][4]["inputs"] == ["b1_relu", "b2_abs", "b3_prelu", "pool1"]
 
 
+def test_groups_that_only_a_concat_reads_are_planned_into_its_output():
+    """The three element-wise branches of the block write into the Concat's output themselves; pool1, which three other layers
+    read as well, is what is left for the Concat to copy. With hip_concat_in_place off (concat_copies_every_input) the plan
+    is the one of before, with a buffer for every branch."""
+    configs = {"stem": (8, [29, 29])}
+    rep = plan(S.inception_like(8), configs, ["out"])
+    by_name = {"+".join(s["layers"]): s for s in rep["steps"]}
+    for branch in ("b1_bn+b1_relu", "b2_drop+b2_abs", "b3_prelu"):
+        assert by_name[branch]["writes_into"] == "join" and by_name[branch]["fused"] and by_name[branch]["run"] is None, branch
+    assert by_name["join"]["inputs_in_place"] == ["b1_relu", "b2_abs", "b3_prelu"]
+    plain = plan(S.inception_like(8), configs, ["out"], concat_copies_every_input=True)
+    assert all(s["writes_into"] is None and s["inputs_in_place"] == [] for s in plain["steps"])
+    assert step_names(plain) == step_names(rep)
+    # three tensors of 8 x 15 x 15 fewer to hold
+    assert plain["per_entry_bytes"] - rep["per_entry_bytes"] >= 4 * 8 * 15 * 15
+
+    # every input a group of its own: nothing left to copy
+    block = S.inception_block(16)
+    block_configs = {"conv_a": (16, [14, 14]), "conv_b": (32, [14, 14]), "conv_c": (16, [14, 14]), "conv_d": (16, [14, 14]), "conv_e": (16, [14, 14])}
+    rep = plan(block, block_configs, ["out"])
+    join = [s for s in rep["steps"] if s["layers"] == ["join"]][0]
+    assert join["inputs_in_place"] == ["a_relu", "b_relu", "c_prelu", "d_relu"]
+    assert sorted(s["layers"][-1] for s in rep["steps"] if s["writes_into"] == "join") == ["a_relu", "b_relu", "c_prelu", "d_relu"]
+    # conv inputs, the Concat's output, Maxout's, the result: no buffer for any branch
+    assert rep["per_entry_bytes"] == 4 * 196 * (16 + 32 + 16 + 16 + 16 + 80 + 16 + 16)
+
+
+def test_what_a_concat_cannot_take_in_place_is_copied():
+    L = S.L
+    branch = lambda name, source, c: [L("BatchNorm", name + "_bn", [source], feature_map_count=c), L("ReLU", name, [name + "_bn"])]
+
+    def in_place(layers, configs, outputs, concat="join"):
+        rep = plan(layers, configs, outputs)
+        return [s for s in rep["steps"] if s["layers"][-1] == concat][0]["inputs_in_place"]
+
+    two = [L("Data", "x"), L("Data", "y")]
+    configs = {"x": (8, [16, 16]), "y": (8, [16, 16])}
+    base = two + branch("a", "x", 8) + branch("b", "y", 8) + [L("Concat", "join", ["a", "b"]), L("ReLU", "out", ["join"])]
+    assert in_place(base, configs, ["out"]) == ["a", "b"]
+    # a branch that is wanted as an output keeps its own tensor
+    assert in_place(base, configs, ["out", "a"]) == ["b"]
+    # a branch that something else reads as well
+    assert in_place(base + [L("Sigmoid", "side", ["b"])], configs, ["out", "side"]) == ["a"]
+    # data layers and layers that are no fused groups (a pooling layer) are copied
+    mixed = two + branch("a", "x", 8) + [L("MaxSubsampling", "p", ["y"], windows=[1, 1]), L("Concat", "join", ["x", "a", "p"]), L("ReLU", "out", ["join"])]
+    assert in_place(mixed, configs, ["out"]) == ["a"]
+    # entries that would not start on 16 bytes: 5 x 9 x 9 floats; what follows such an input is off the boundary too
+    odd = {"x": (5, [9, 9]), "y": (8, [9, 9])}
+    odd_net = two + branch("a", "x", 5) + branch("b", "y", 8) + [L("Concat", "join", ["b", "a"]), L("ReLU", "out", ["join"])]
+    assert in_place(odd_net, odd, ["out"]) == []
+    odd_net = two + branch("a", "x", 5) + branch("b", "y", 8) + [L("Concat", "join", ["a", "b"]), L("ReLU", "out", ["join"])]
+    assert in_place(odd_net, odd, ["out"]) == []
+    # small entries stay with the copy: a launch over entries would be all launch
+    small = {"x": (8, [4, 4]), "y": (8, [4, 4])}
+    assert in_place(base, small, ["out"]) == []
+    # a group with three inputs
+    three = two + [L("Data", "z")] + branch("a", "x", 8) + [L("Add", "sum", ["x", "y", "z"]), L("ReLU", "b", ["sum"]), L("Concat", "join", ["a", "b"]), L("ReLU", "out", ["join"])]
+    assert in_place(three, dict(configs, z=(8, [16, 16])), ["out"]) == ["a"]
+    # the same value twice
+    twice = two[:1] + branch("a", "x", 8) + [L("Concat", "join", ["a", "a"]), L("ReLU", "out", ["join"])]
+    assert in_place(twice, {"x": (8, [16, 16])}, ["out"]) == []
+    # a Concat of Concats: the inner one is no fused group
+    nested = base[:-1] + [L("Data", "w")] + branch("c", "w", 8) + [L("Concat", "outer", ["join", "c"]), L("ReLU", "out", ["outer"])]
+    assert in_place(nested, dict(configs, w=(8, [16, 16])), ["out"], concat="outer") == ["c"]
+    assert in_place(nested, dict(configs, w=(8, [16, 16])), ["out"], concat="join") == ["a", "b"]
+
+
 def test_plan_of_the_resnet50_post_convolution_graph_equals_the_benchmark_group_list():
     """Config 4 as a network: the graph examples/imagenet/imagenet_toolset.cpp:476-550, 729-831 builds, convolution outputs as
     data layers. With one launch per group the driver's fusion pass must arrive at the 49 groups nnforge_amd.workloads lists by

@@ -228,6 +228,46 @@ def test_inception_like_block_with_the_neighbouring_layers(fuse):
     assert_bits(got["out"], values["out"], "output")
 
 
+@pytest.mark.parametrize("c,size,n,packet", [(16, 14, 23, 8), (32, 7, 9, 4), (16, 28, 5, 5)])
+def test_inception_block_whose_concat_has_nothing_to_copy(c, size, n, packet):
+    """Four branches that end in fused groups only the Concat reads: every group writes its feature maps into the Concat's
+    output (a launch over tiles x entries, entry to entry by the Concat's neuron count) and the Concat launches nothing.
+    Against the oracle layer by layer, bit for bit, in packets (the last one short); and the same bits with every input
+    copied (hip_concat_in_place off). 7 x 7 planes take their weights through LDS coefficients."""
+    gen = T.rng(65, size)
+    layers = S.inception_block(c)
+    weights = S.make_weights(layers, gen)
+    inputs = {name: T.normal(gen, (n, fm, size, size), 1.5) for name, fm in (("conv_a", c), ("conv_b", 2 * c), ("conv_c", c), ("conv_d", c), ("conv_e", c))}
+    values = S.evaluate(layers, weights, inputs)
+    assert values["join"].shape == (n, 5 * c, size, size)
+    got, rep = run(layers, weights, inputs, ["out", "mo"], values, max_entry_count=packet)
+    join = [s for s in rep["steps"] if s["layers"] == ["join"]][0]
+    assert join["inputs_in_place"] == ["a_relu", "b_relu", "c_prelu", "d_relu"], rep["raw"]
+    assert_bits(got["mo"], values["mo"], "maxout behind the concat")
+    assert_bits(got["out"], values["out"], "output")
+    # the Concat's output as an output of the network: the groups write into the buffer that is copied back
+    got, rep = run(layers, weights, inputs, ["join"], values, max_entry_count=packet)
+    assert_bits(got["join"], values["join"], "concat as output")
+    copied, rep = run(layers, weights, inputs, ["out", "join"], values, max_entry_count=packet, concat_copies_every_input=True)
+    assert all(s["inputs_in_place"] == [] for s in rep["steps"])
+    assert_bits(copied["join"], values["join"], "concat, every input copied")
+    assert_bits(copied["out"], values["out"], "output, every input copied")
+
+
+def test_concat_launches_nothing_when_every_input_is_in_place():
+    gen = T.rng(66, 1)
+    c, size, n = 16, 14, 6
+    layers = S.inception_block(c)
+    weights = S.make_weights(layers, gen)
+    inputs = {name: T.normal(gen, (n, fm, size, size), 1.5) for name, fm in (("conv_a", c), ("conv_b", 2 * c), ("conv_c", c), ("conv_d", c), ("conv_e", c))}
+    in_place = backend.time_kernels(S.schema_text(layers), weights, inputs, ["out"], warmup=1, passes=2, max_entry_count=n)
+    copying = backend.time_kernels(S.schema_text(layers), weights, inputs, ["out"], warmup=1, passes=2, max_entry_count=n, concat_copies_every_input=True)
+    # four groups, maxout, tanh: six steps, six kernels - the Concat is a step that launches nothing. Copying, it is a
+    # seventh step with a kernel of its own (and the three groups of several layers share launches)
+    assert in_place["launches"] == 6 and in_place["plan_steps"] == 6, in_place["raw"]
+    assert copying["plan_steps"] == 7 and 4 <= copying["launches"] <= 7, copying["raw"]
+
+
 @pytest.mark.parametrize("fuse", [True, False])
 @pytest.mark.parametrize("size", [28, 57])
 def test_groups_folded_into_the_subsampling_layers_behind_them(fuse, size):
