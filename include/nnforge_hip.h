@@ -42,6 +42,8 @@ extern "C" {
 #define NNF_HIP_MAX_ELEMENT_COUNT 0xFFFF0000ull
 
 #define NNF_HIP_MAX_OPS 8
+/* nnf_hip_chain_forward_strided_batch: most groups one kernel launch takes */
+#define NNF_HIP_MAX_STRIDED_GROUPS_PER_LAUNCH 6
 #define NNF_HIP_MAX_INPUTS 4
 /* nnf_hip_chain_forward_batch: most groups one kernel launch takes (what fits into 4 KB of kernel arguments) */
 #define NNF_HIP_MAX_GROUPS_PER_LAUNCH 11
@@ -139,6 +141,12 @@ NNF_HIP_API int nnf_hip_chain_forward_batch(void* stream, uint32_t group_count, 
 NNF_HIP_API int nnf_hip_chain_forward_strided(void* stream, const nnf_hip_chain_desc* desc, float* output, uint32_t output_entry_stride,
 	const float* const* inputs, const float* const* chunk_ptrs);
 NNF_HIP_API int nnf_hip_chain_forward_strided_status(const nnf_hip_chain_desc* desc, uint32_t output_entry_stride);
+/* group_count such groups over the same number of entries - the branches in front of one Concat layer, say - in one launch per
+ * NNF_HIP_MAX_STRIDED_GROUPS_PER_LAUNCH groups. Same results as group_count calls of nnf_hip_chain_forward_strided. What one group
+ * writes may touch no input of the call and no other group's result (NNF_HIP_EOVERLAP, nothing launched); results that step
+ * alike may lie side by side inside one step, as the parts of one wider tensor do. */
+NNF_HIP_API int nnf_hip_chain_forward_strided_batch(void* stream, uint32_t group_count, const nnf_hip_chain_desc* descs,
+	float* const* outputs, const uint32_t* output_entry_strides, const float* const* const* inputs, const float* const* const* chunk_ptrs);
 
 /* Single-layer entry points, one per reference tester (same arithmetic as the chain kernel). */
 NNF_HIP_API int nnf_hip_batch_norm_forward(void* stream, float* output, const float* input,

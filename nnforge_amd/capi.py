@@ -113,6 +113,7 @@ SIGNATURES = {
     "nnf_hip_launch_count": [ctypes.POINTER(_U64)],
     "nnf_hip_chain_forward_strided": [_VP, ctypes.POINTER(ChainDesc), _VP, _U32, _PP, _PP],
     "nnf_hip_chain_forward_strided_status": [ctypes.POINTER(ChainDesc), _U32],
+    "nnf_hip_chain_forward_strided_batch": [_VP, _U32, ctypes.POINTER(ChainDesc), ctypes.POINTER(_VP), ctypes.POINTER(_U32), ctypes.POINTER(ctypes.POINTER(_VP)), ctypes.POINTER(ctypes.POINTER(_VP))],
     "nnf_hip_stream_begin_capture": [_VP],
     "nnf_hip_stream_end_capture": [_VP, _PP],
     "nnf_hip_graph_launch": [_VP, _VP],

@@ -139,6 +139,12 @@ extern "C"
 		return chain_forward_strided(static_cast<hipStream_t>(stream), desc, output, output_entry_stride, inputs, chunk_ptrs);
 	}
 
+	int nnf_hip_chain_forward_strided_batch(void* stream, uint32_t group_count, const nnf_hip_chain_desc* descs,
+		float* const* outputs, const uint32_t* output_entry_strides, const float* const* const* inputs, const float* const* const* chunk_ptrs)
+	{
+		return chain_forward_strided_batch(static_cast<hipStream_t>(stream), group_count, descs, outputs, output_entry_strides, inputs, chunk_ptrs);
+	}
+
 	int nnf_hip_chain_forward_strided_status(const nnf_hip_chain_desc* desc, uint32_t output_entry_stride)
 	{
 		return chain_forward_strided_status(desc, output_entry_stride);

@@ -521,24 +521,64 @@ namespace nnf
 			const chain_slot (&slots)[SLOTS];
 		};
 
-		template<int NIN, int BLOCK, int U, bool DIRECT>
-		__global__ void __launch_bounds__(BLOCK) chain_entries_kernel(const chain_args a, const uint32_t entry_count, const uint32_t out_entry_stride)
+		// Up to max_strided_batch such groups in one launch (the branches in front of one Concat layer): along x the
+		// tiles of one entry of every group, one group after the other, along y the entries. A workgroup finds its group
+		// by its x index and takes the body of the group's kind (one input or two, weights straight from memory or
+		// through LDS coefficients), 256 lanes x 2 float4s each.
+		constexpr uint32_t max_strided_batch = NNF_HIP_MAX_STRIDED_GROUPS_PER_LAUNCH;
+		struct chain_strided_batch_args
+		{
+			uint32_t count;
+			uint32_t direct_mask;     // bit g: group g reads its weights straight from memory
+			uint32_t two_input_mask;  // bit g: group g has two inputs
+			uint32_t entry_count;
+			uint32_t tile_end[max_strided_batch];         // running total of the groups' tiles per entry
+			uint32_t out_entry_stride[max_strided_batch]; // floats from one entry of the group's result to the next
+			chain_args group[max_strided_batch];          // total: the elements of one entry
+		};
+		static_assert(sizeof(chain_strided_batch_args) <= 4096, "kernel arguments of a strided batch beyond 4 KB");
+
+		// ALL_DIRECT: every group of the launch reads its weights straight from memory; ONE_INPUT: every group has one
+		// input. The launch whose groups are all of one kind holds one body instead of four and half the registers
+		// (48 against 102 per lane: four Inception branches of 512 entries 135 against 172 us).
+		template<int BLOCK, bool ALL_DIRECT, bool ONE_INPUT>
+		__global__ void __launch_bounds__(BLOCK) chain_entries_batch_kernel(const chain_strided_batch_args b)
 		{
 			extern __shared__ __align__(16) unsigned char lds_raw[];
-			for(uint32_t entry = blockIdx.y; entry < entry_count; entry += gridDim.y)
+			uint32_t g = 0;
+			while ((g + 1 < b.count) && (blockIdx.x >= b.tile_end[g]))
+				++g;
+			const uint32_t tile_index = blockIdx.x - ((g == 0) ? 0u : b.tile_end[g - 1]);
+			const chain_args& a = b.group[g];
+			const bool direct = ALL_DIRECT || (((b.direct_mask >> g) & 1u) != 0);
+			const bool two_inputs = !ONE_INPUT && (((b.two_input_mask >> g) & 1u) != 0);
+			for(uint32_t entry = blockIdx.y; entry < b.entry_count; entry += gridDim.y)
 			{
 				chain_entry_view<max_slots> v = {
-					{}, a.out + static_cast<size_t>(entry) * out_entry_stride,
+					{}, a.out + static_cast<size_t>(entry) * b.out_entry_stride[g],
 					a.total, a.fm_count, a.plane, a.plane_magic, a.span, a.has_add, a.alpha,
 					{}, a.tail_ops, a.slot_count, a.need_exp, a.ops, a.slots };
 				#pragma unroll
 				for(int j = 0; j < NNF_HIP_MAX_INPUTS; ++j)
 				{
-					v.in[j] = (j < NIN) ? a.in[j] + static_cast<size_t>(entry) * a.total : nullptr;
+					v.in[j] = ((j == 0) || ((j == 1) && two_inputs)) ? a.in[j] + static_cast<size_t>(entry) * a.total : nullptr;
 					v.arm_ops[j] = a.arm_ops[j];
 				}
-				chain_tile<NIN, BLOCK, U, DIRECT, 0>(v, blockIdx.x, lds_raw);
-				if (entry + gridDim.y < entry_count)
+				if (two_inputs)
+				{
+					if (direct)
+						chain_tile<2, BLOCK, 2, true, 0>(v, tile_index, lds_raw);
+					else
+						chain_tile<2, BLOCK, 2, false, 0>(v, tile_index, lds_raw);
+				}
+				else
+				{
+					if (direct)
+						chain_tile<1, BLOCK, 2, true, 0>(v, tile_index, lds_raw);
+					else
+						chain_tile<1, BLOCK, 2, false, 0>(v, tile_index, lds_raw);
+				}
+				if (entry + gridDim.y < b.entry_count)
 					__syncthreads(); // the next entry's coefficients go where this one's are still being read
 			}
 		}
@@ -1130,40 +1170,104 @@ namespace nnf
 		return NNF_HIP_OK;
 	}
 
+	int chain_forward_strided_batch(hipStream_t stream, uint32_t group_count, const nnf_hip_chain_desc* descs, float* const* outputs,
+		const uint32_t* output_entry_strides, const float* const* const* inputs, const float* const* const* chunk_ptrs)
+	{
+		if (group_count == 0)
+			return NNF_HIP_OK;
+		if ((descs == nullptr) || (outputs == nullptr) || (output_entry_strides == nullptr) || (inputs == nullptr))
+			return NNF_HIP_EINVAL;
+		// everything is checked before anything is launched
+		const uint32_t entry_count = descs[0].entry_count;
+		for(uint32_t i = 0; i < group_count; ++i)
+		{
+			const int rc = chain_forward_strided_status(&descs[i], output_entry_strides[i]);
+			if (rc != NNF_HIP_OK)
+				return rc;
+			if (descs[i].entry_count != entry_count)
+				return NNF_HIP_EINVAL; // the groups of a call go entry by entry together
+		}
+		if (entry_count == 0)
+			return NNF_HIP_OK; // as the reference's loops over zero entries
+		std::vector<prepared_group> groups(group_count);
+		for(uint32_t i = 0; i < group_count; ++i)
+		{
+			int rc;
+			// planned as a group of one entry
+			nnf_hip_chain_desc one = descs[i];
+			one.entry_count = 1;
+			rc = prepare_group(&one, outputs[i], inputs[i], (chunk_ptrs == nullptr) ? nullptr : chunk_ptrs[i], false, groups[i], strided_shape);
+			if (rc != NNF_HIP_OK)
+				return rc;
+		}
+		// What group i writes: entry_count pieces of its entry size, output_entry_strides[i] floats apart. No input of the
+		// call may lie inside the span they cover, and the pieces of two groups may not meet: either their spans are
+		// apart, or they step alike and their pieces lie side by side inside one step (the parts of one wider tensor).
+		for(uint32_t i = 0; i < group_count; ++i)
+		{
+			const size_t piece_i = groups[i].bytes;
+			const size_t span_i = static_cast<size_t>(entry_count - 1) * output_entry_strides[i] * sizeof(float) + piece_i;
+			for(uint32_t j = 0; j < group_count; ++j)
+			{
+				for(uint32_t k = 0; k < groups[j].input_count; ++k)
+					if (ranges_overlap(outputs[i], span_i, groups[j].a.in[k], groups[j].bytes * entry_count))
+						return NNF_HIP_EOVERLAP;
+				if (j <= i)
+					continue;
+				const size_t piece_j = groups[j].bytes;
+				const size_t span_j = static_cast<size_t>(entry_count - 1) * output_entry_strides[j] * sizeof(float) + piece_j;
+				if (!ranges_overlap(outputs[i], span_i, outputs[j], span_j))
+					continue;
+				if (output_entry_strides[i] != output_entry_strides[j])
+					return NNF_HIP_EOVERLAP;
+				const uintptr_t pi = reinterpret_cast<uintptr_t>(outputs[i]), pj = reinterpret_cast<uintptr_t>(outputs[j]);
+				const size_t step = static_cast<size_t>(output_entry_strides[i]) * sizeof(float);
+				const size_t low_piece = (pi < pj) ? piece_i : piece_j, high_piece = (pi < pj) ? piece_j : piece_i;
+				const size_t gap = (pi < pj) ? (pj - pi) : (pi - pj);
+				if ((gap < low_piece) || (gap + high_piece > step))
+					return NNF_HIP_EOVERLAP;
+			}
+		}
+		for(uint32_t first = 0; first < group_count; first += max_strided_batch)
+		{
+			chain_strided_batch_args b = {};
+			b.count = std::min(max_strided_batch, group_count - first);
+			b.entry_count = entry_count;
+			size_t lds_bytes = 0;
+			uint32_t tiles = 0;
+			for(uint32_t m = 0; m < b.count; ++m)
+			{
+				const prepared_group& g = groups[first + m];
+				b.group[m] = g.a;
+				b.direct_mask |= g.direct ? (1u << m) : 0u;
+				b.two_input_mask |= (g.input_count == 2) ? (1u << m) : 0u;
+				b.out_entry_stride[m] = output_entry_strides[first + m];
+				tiles += g.tiles;
+				b.tile_end[m] = tiles;
+				lds_bytes = std::max(lds_bytes, g.lds_bytes);
+			}
+			const dim3 grid(tiles, std::min(entry_count, 65535u)), block(launch_shapes[strided_shape].block);
+			const bool all_direct = b.direct_mask == ((1u << b.count) - 1u), one_input = b.two_input_mask == 0;
+			if (all_direct && one_input) NNF_LAUNCH((chain_entries_batch_kernel<256, true, true>), grid, block, lds_bytes, stream, b);
+			else if (all_direct) NNF_LAUNCH((chain_entries_batch_kernel<256, true, false>), grid, block, lds_bytes, stream, b);
+			else if (one_input) NNF_LAUNCH((chain_entries_batch_kernel<256, false, true>), grid, block, lds_bytes, stream, b);
+			else NNF_LAUNCH((chain_entries_batch_kernel<256, false, false>), grid, block, lds_bytes, stream, b);
+			const int rc = launch_status();
+			if (rc != NNF_HIP_OK)
+				return rc;
+		}
+		return NNF_HIP_OK;
+	}
+
 	int chain_forward_strided(hipStream_t stream, const nnf_hip_chain_desc* desc, float* output, uint32_t output_entry_stride,
 		const float* const* inputs, const float* const* chunk_ptrs)
 	{
-		int rc = chain_forward_strided_status(desc, output_entry_stride);
-		if (rc != NNF_HIP_OK)
-			return rc;
-		if (desc->entry_count == 0)
-			return NNF_HIP_OK;
-		// planned as a group of one entry
-		nnf_hip_chain_desc one = *desc;
-		one.entry_count = 1;
-		prepared_group p;
-		rc = prepare_group(&one, output, inputs, chunk_ptrs, false, p, strided_shape);
-		if (rc != NNF_HIP_OK)
-			return rc;
-		// the whole of what is written and read
-		const size_t per_entry_bytes = p.bytes;
-		const size_t out_bytes = (static_cast<size_t>(desc->entry_count - 1) * output_entry_stride) * sizeof(float) + per_entry_bytes;
-		for(uint32_t j = 0; j < desc->input_count; ++j)
-			if (ranges_overlap(output, out_bytes, inputs[j], per_entry_bytes * desc->entry_count))
-				return NNF_HIP_EOVERLAP;
-		const dim3 grid(p.tiles, std::min(desc->entry_count, 65535u));
-		const dim3 block(launch_shapes[strided_shape].block);
-		if (desc->input_count == 1)
-		{
-			if (p.direct) NNF_LAUNCH((chain_entries_kernel<1, 256, 2, true>), grid, block, p.lds_bytes, stream, p.a, desc->entry_count, output_entry_stride);
-			else NNF_LAUNCH((chain_entries_kernel<1, 256, 2, false>), grid, block, p.lds_bytes, stream, p.a, desc->entry_count, output_entry_stride);
-		}
-		else
-		{
-			if (p.direct) NNF_LAUNCH((chain_entries_kernel<2, 256, 2, true>), grid, block, p.lds_bytes, stream, p.a, desc->entry_count, output_entry_stride);
-			else NNF_LAUNCH((chain_entries_kernel<2, 256, 2, false>), grid, block, p.lds_bytes, stream, p.a, desc->entry_count, output_entry_stride);
-		}
-		return launch_status();
+		if (desc == nullptr)
+			return NNF_HIP_EINVAL;
+		float* outputs[1] = { output };
+		const float* const* input_lists[1] = { inputs };
+		const float* const* chunk_lists[1] = { chunk_ptrs };
+		return chain_forward_strided_batch(stream, 1, desc, outputs, &output_entry_stride, input_lists, chunk_lists);
 	}
 
 	int chain_forward_batch(hipStream_t stream, uint32_t group_count, const nnf_hip_chain_desc* descs, float* const* outputs,

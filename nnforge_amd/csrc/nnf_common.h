@@ -125,6 +125,8 @@ namespace nnf
 	int chain_forward(hipStream_t stream, const nnf_hip_chain_desc* desc, float* output,
 		const float* const* inputs, const float* const* chunk_ptrs);
 	int chain_forward_strided_status(const nnf_hip_chain_desc* desc, uint32_t output_entry_stride);
+	int chain_forward_strided_batch(hipStream_t stream, uint32_t group_count, const nnf_hip_chain_desc* descs, float* const* outputs,
+		const uint32_t* output_entry_strides, const float* const* const* inputs, const float* const* const* chunk_ptrs);
 	int chain_forward_strided(hipStream_t stream, const nnf_hip_chain_desc* desc, float* output, uint32_t output_entry_stride,
 		const float* const* inputs, const float* const* chunk_ptrs);
 	int chain_forward_batch(hipStream_t stream, uint32_t group_count, const nnf_hip_chain_desc* descs, float* const* outputs,

@@ -246,18 +246,47 @@ namespace nnforge
 					plan.tester->enqueue_forward_propagation_with_prologue(step_stream, buffers[plan.output_buffer], inputs, plan.desc,
 						chunk_ptrs[i].empty() ? nullptr : chunk_ptrs[i].data(), step_entries);
 				}
+				else if (plan.info.fused && (plan.view_stride != 0))
+				{
+					// The groups that write into one Concat's output and follow one another in the plan go to the kernels in
+					// one call: none of them reads what another writes (only the Concat reads them), their parts of the
+					// output lie side by side. The first of them launches all; with per-action times wanted, each its own.
+					if ((profile_events == nullptr) && (i > 0) && (plans[i - 1].view_stride != 0) && (plans[i - 1].info.writes_into == plan.info.writes_into)
+						&& (plans[i - 1].info.stream_index == plan.info.stream_index) && (plans[i - 1].entry_factor == plan.entry_factor))
+						continue;
+					std::vector<nnf_hip_chain_desc> descs;
+					std::vector<float *> outputs;
+					std::vector<uint32_t> strides;
+					std::vector<std::vector<const float *> > in_ptrs;
+					std::vector<const float * const *> in_ptr_ptrs, chunk_ptr_ptrs;
+					for(size_t m = i; m < plans.size(); ++m)
+					{
+						step_plan& member = plans[m];
+						if ((m > i) && ((profile_events != nullptr) || (member.view_stride == 0) || (member.info.writes_into != plan.info.writes_into)
+							|| (member.info.stream_index != plan.info.stream_index) || (member.entry_factor != plan.entry_factor)))
+							break;
+						member.desc.entry_count = step_entries;
+						descs.push_back(member.desc);
+						outputs.push_back(static_cast<float *>(*buffers[member.output_buffer]) + member.view_offset);
+						strides.push_back(member.view_stride);
+						in_ptrs.push_back(std::vector<const float *>());
+						for(int b : member.input_buffers)
+							in_ptrs.back().push_back(static_cast<const float *>(*static_cast<hip_linear_buffer_device::const_ptr>(buffers[b])));
+						chunk_ptr_ptrs.push_back(chunk_ptrs[m].empty() ? nullptr : chunk_ptrs[m].data());
+					}
+					for(const std::vector<const float *>& v : in_ptrs)
+						in_ptr_ptrs.push_back(v.data());
+					hip_safe_call(nnf_hip_chain_forward_strided_batch(step_stream, static_cast<uint32_t>(descs.size()), descs.data(), outputs.data(),
+						strides.data(), in_ptr_ptrs.data(), chunk_ptr_ptrs.data()));
+				}
 				else if (plan.info.fused)
 				{
 					plan.desc.entry_count = step_entries;
 					std::vector<const float *> in_ptrs;
 					for(const hip_linear_buffer_device::const_ptr& b : inputs)
 						in_ptrs.push_back(static_cast<const float *>(*b));
-					if (plan.view_stride != 0)
-						hip_safe_call(nnf_hip_chain_forward_strided(step_stream, &plan.desc, static_cast<float *>(*buffers[plan.output_buffer]) + plan.view_offset,
-							plan.view_stride, in_ptrs.data(), chunk_ptrs[i].empty() ? nullptr : chunk_ptrs[i].data()));
-					else
-						hip_safe_call(nnf_hip_chain_forward(step_stream, &plan.desc, *buffers[plan.output_buffer], in_ptrs.data(),
-							chunk_ptrs[i].empty() ? nullptr : chunk_ptrs[i].data()));
+					hip_safe_call(nnf_hip_chain_forward(step_stream, &plan.desc, *buffers[plan.output_buffer], in_ptrs.data(),
+						chunk_ptrs[i].empty() ? nullptr : chunk_ptrs[i].data()));
 				}
 				else if (!plan.inputs_in_place.empty())
 					plan.tester->enqueue_forward_propagation_with_inputs_in_place(step_stream, buffers[plan.output_buffer], inputs, plan.inputs_in_place, step_entries);

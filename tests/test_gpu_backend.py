@@ -262,9 +262,9 @@ def test_concat_launches_nothing_when_every_input_is_in_place():
     inputs = {name: T.normal(gen, (n, fm, size, size), 1.5) for name, fm in (("conv_a", c), ("conv_b", 2 * c), ("conv_c", c), ("conv_d", c), ("conv_e", c))}
     in_place = backend.time_kernels(S.schema_text(layers), weights, inputs, ["out"], warmup=1, passes=2, max_entry_count=n)
     copying = backend.time_kernels(S.schema_text(layers), weights, inputs, ["out"], warmup=1, passes=2, max_entry_count=n, concat_copies_every_input=True)
-    # four groups, maxout, tanh: six steps, six kernels - the Concat is a step that launches nothing. Copying, it is a
-    # seventh step with a kernel of its own (and the three groups of several layers share launches)
-    assert in_place["launches"] == 6 and in_place["plan_steps"] == 6, in_place["raw"]
+    # four groups, maxout, tanh: six steps, and three kernels - the four groups go to the kernels in one call (one launch),
+    # the Concat is a step that launches nothing. Copying, it is a seventh step with a kernel of its own
+    assert in_place["launches"] == 3 and in_place["plan_steps"] == 6, in_place["raw"]
     assert copying["plan_steps"] == 7 and 4 <= copying["launches"] <= 7, copying["raw"]
 
 
