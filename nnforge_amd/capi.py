@@ -69,6 +69,7 @@ SIGNATURES = {
     "nnf_hip_absolute_forward": [_VP, _VP, _VP, _U64],
     "nnf_hip_dropout_forward": [_VP, _VP, _VP, _U64],
     "nnf_hip_concat_forward": [_VP, _VP, _PP, ctypes.POINTER(_U32), _U32, _U32],
+    "nnf_hip_concat_forward_partial": [_VP, _VP, _PP, ctypes.POINTER(_U32), ctypes.POINTER(ctypes.c_uint8), _U32, _U32],
     "nnf_hip_maxout_forward": [_VP, _VP, _VP, _U32, _U32, _U32, _U32],
     "nnf_hip_max_subsampling_forward": [_VP, _VP, _VP, _U32, _U32, _U32, ctypes.POINTER(_U32), ctypes.POINTER(_U32),
                                         ctypes.POINTER(_U32), ctypes.POINTER(_U32), _U32, _U32, ctypes.c_int32],
