@@ -89,6 +89,30 @@ def test_concat(gpu, n, fms, spatial):
     assert T.bit_mismatches(got, want) == 0
 
 
+@pytest.mark.parametrize("flags", [(1, 0, 1, 0), (0, 0, 0, 1), (1, 1, 1, 1), (0, 0, 0, 0), (0, 1, 1, 0, 1, 0, 1, 1, 0, 1)])
+def test_concat_with_inputs_already_in_place(gpu, flags):
+    """nnf_hip_concat_forward_partial: the inputs flagged as in place are not copied (their pointers are null here) and keep
+    what lies in their parts of the output; the others are copied to theirs."""
+    gen = T.rng(62, sum(flags) + len(flags))
+    n, plane = 7, 36
+    fms = [int(gen.integers(1, 9)) for _ in flags]
+    parts = [spiced(gen, (n, c, plane)) for c in fms]
+    want = oracle.concat(parts)
+    there = np.full_like(want, np.float32(-3.5))
+    offset = 0
+    for part, flag, c in zip(parts, flags, fms):
+        if flag:
+            there[:, offset:offset + c] = part
+        offset += c
+    d_out = gpu.to_device(there)
+    d_parts = [gpu.to_device(p) for p in parts]
+    ptrs = capi.pointer_array([0 if flag else t.data_ptr() for t, flag in zip(d_parts, flags)])
+    rc = gpu.lib.nnf_hip_concat_forward_partial(gpu.stream, d_out.data_ptr(), ptrs, u32([c * plane for c in fms]),
+                                                (ctypes.c_uint8 * len(flags))(*flags), len(flags), n)
+    assert rc == 0, capi.error_string(rc)
+    assert T.bit_mismatches(gpu.to_host(d_out, want.shape), want) == 0
+
+
 def run_maxout(gpu, x, k, expect=0):
     n, c = x.shape[:2]
     plane = int(np.prod(x.shape[2:], dtype=np.int64))

@@ -503,6 +503,65 @@ def test_group_written_into_a_wider_tensor(gpu, n, c, plane, before, after, kind
     assert (got[:, :before] == sentinel).all() and (got[:, before + per_entry:] == sentinel).all(), "the rest of the wide tensor is untouched"
 
 
+def test_groups_written_side_by_side_into_a_wider_tensor_in_one_call(gpu):
+    """nnf_hip_chain_forward_strided_batch: the branches in front of a Concat - a two-input group, a group on 7 x 7 planes
+    (coefficients through LDS), two plain ones, eight groups in all so that the call takes two launches - write their parts
+    of the wide tensor; the result is the oracle's groups concatenated, the room left between two parts stays untouched."""
+    gen = T.rng(19, 1)
+    n, plane = 6, 49
+    widths = [8, 12, 4, 16, 8, 4, 8, 12]
+    gap_after = 3   # leave 16 floats unused behind the third part
+    parts, descs, keep, outs, ins_list, chk_list, offsets = [], [], [], [], [], [], []
+    stride = sum(widths) * plane + 16
+    wide = gpu.torch.full((n * stride,), -777.25, dtype=gpu.torch.float32, device=gpu.device)
+    offset = 0
+    for i, c in enumerate(widths):
+        x = T.normal(gen, (n, c, plane), 1.5)
+        g, b, m, s_ = T.bn_params(gen, c)
+        if i == 1:
+            r = T.normal(gen, (n, c, plane), 1.5)
+            arms, tail, inputs = [[], [(BN, 0)]], [(RELU, 0, 0.0)], [r, x]
+            want = oracle.rectified_linear(oracle.add([r, oracle.batch_norm(x, g, b, m, s_)]).reshape(x.shape))
+        else:
+            arms, tail, inputs = [[(BN, 0), (RELU, 0, 0.125)]], [], [x]
+            want = oracle.rectified_linear(oracle.batch_norm(x, g, b, m, s_), 0.125)
+        descs.append(capi.make_desc(n, c, plane, arms, tail))
+        d_in = [gpu.to_device(a) for a in inputs]
+        d_chunks = [gpu.to_device(a) for a in (g, b, m, s_)]
+        keep += d_in + d_chunks
+        ins_list.append(capi.pointer_array([t.data_ptr() for t in d_in]))
+        chk_list.append(capi.pointer_array([t.data_ptr() for t in d_chunks]))
+        outs.append(wide.data_ptr() + 4 * offset)
+        offsets.append(offset)
+        parts.append(want.reshape(n, -1))
+        offset += c * plane + (16 if i == gap_after - 1 else 0)
+    count = len(widths)
+    desc_array = (capi.ChainDesc * count)(*descs)
+    out_array = (ctypes.c_void_p * count)(*outs)
+    strides = (ctypes.c_uint32 * count)(*([stride] * count))
+    in_array = (ctypes.POINTER(ctypes.c_void_p) * count)(*[ctypes.cast(p, ctypes.POINTER(ctypes.c_void_p)) for p in ins_list])
+    chk_array = (ctypes.POINTER(ctypes.c_void_p) * count)(*[ctypes.cast(p, ctypes.POINTER(ctypes.c_void_p)) for p in chk_list])
+    before = ctypes.c_uint64()
+    after = ctypes.c_uint64()
+    gpu.lib.nnf_hip_launch_count(ctypes.byref(before))
+    rc = gpu.lib.nnf_hip_chain_forward_strided_batch(gpu.stream, count, desc_array, out_array, strides, in_array, chk_array)
+    assert rc == 0, capi.error_string(rc)
+    gpu.lib.nnf_hip_launch_count(ctypes.byref(after))
+    assert after.value - before.value == 2   # six groups to a launch
+    got = gpu.to_host(wide).reshape(n, stride)
+    for i, c in enumerate(widths):
+        check_exact(got[:, offsets[i]:offsets[i] + c * plane], parts[i], "part %d" % i)
+    gap = offsets[gap_after] - 16
+    assert (got[:, gap:gap + 16] == np.float32(-777.25)).all()
+    # parts that meet are refused, whichever way: the second group moved 4 floats into the first one's part
+    out_array[1] = outs[1] - 16
+    assert gpu.lib.nnf_hip_chain_forward_strided_batch(gpu.stream, count, desc_array, out_array, strides, in_array, chk_array) == capi.E_OVERLAP
+    out_array[1] = outs[1]
+    strides[2] = stride + 4
+    assert gpu.lib.nnf_hip_chain_forward_strided_batch(gpu.stream, count, desc_array, out_array, strides, in_array, chk_array) == capi.E_OVERLAP
+    gpu.torch.cuda.synchronize()
+
+
 def test_group_written_into_a_wider_tensor_refuses_what_it_cannot_do(gpu):
     desc = capi.make_desc(2, 3, 5, [[(RELU, 0, 0.0)]], [])           # 15 floats per entry: entries would not start on 16 bytes
     assert gpu.lib.nnf_hip_chain_forward_strided_status(ctypes.byref(desc), 32) == capi.E_UNSUPPORTED
