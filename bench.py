@@ -407,6 +407,40 @@ def bench_through_driver(runner, config, c_abi_entry, steps, warmup):
             "event_time_vs_c_abi": device_s * 1e3 / c_abi_entry["event_ms_per_step"]}
 
 
+def bench_inception_block(runner, steps, warmup, n=128, copies=False):
+    """An Inception 3a-like block through the driver: BatchNorm -> ReLU behind four convolutions of 64, 128, 32 and 32 maps of 28 x 28,
+    then the Concat of the four. By default every group writes into the Concat's output (one launch for the four, none for the
+    Concat); with copies (hip_concat_in_place off) the groups have tensors of their own and the Concat copies them. The
+    algorithmic bytes are those of the first form: every convolution output read once, the Concat's output written once."""
+    from nnforge_amd import backend, schemas
+
+    fms = (64, 128, 32, 32)
+    layers = []
+    for i, c in enumerate(fms):
+        layers += [schemas.L("Data", "conv%d" % i), schemas.L("BatchNorm", "bn%d" % i, ["conv%d" % i], feature_map_count=c),
+                   schemas.L("ReLU", "relu%d" % i, ["bn%d" % i])]
+    layers.append(schemas.L("Concat", "join", ["relu%d" % i for i in range(len(fms))]))
+    configs = {"conv%d" % i: (c, [28, 28]) for i, c in enumerate(fms)}
+    gen = np.random.Generator(np.random.MT19937(SEED + 0x200))
+    weights = {}
+    for l in layers:
+        if l["type"] == "BatchNorm":
+            c = l["params"]["feature_map_count"]
+            weights[l["name"]] = [gen.random(c, dtype=np.float32) + np.float32(0.5), gen.standard_normal(c, dtype=np.float32) * np.float32(0.3),
+                                  gen.standard_normal(c, dtype=np.float32) * np.float32(0.3), gen.random(c, dtype=np.float32) + np.float32(0.6)]
+    elements = n * sum(fms) * 28 * 28
+    alg = 2 * 4 * elements
+    resident = int(max(1, min(32, -(-(768 << 20) // alg))))
+    pool = gen.standard_normal(n * max(fms) * 28 * 28, dtype=np.float32)
+    rep = backend.time_kernels(schemas.schema_text(layers), weights, configs, ["join"], warmup=warmup, passes=steps, shared_input_pool=pool, entry_count=n,
+                               max_entry_count=n, resident_packets=resident, concat_copies_every_input=copies)
+    assert rep["timed_entries"] == n and rep["plan_steps"] == (5 if copies else 4) and rep["launches"] == (2 if copies else 1), rep["raw"]
+    return result_entry("Inception-like block N=%d: batch_norm -> rectified_linear on 64+128+32+32 maps of 28x28, concat (%s)" % (
+                            n, "every input copied" if copies else "the groups write into the concat's output"),
+                        alg, elements, rep["wall_seconds_per_pass"], rep["device_seconds_per_pass"], rep["launches"],
+                        {"resident_packets": resident, "moved_bytes_per_step": alg * (2 if copies else 1)})
+
+
 def bench_resnet50_direct(runner, steps, warmup, n=64):
     """The same 51 launches issued one by one at the C ABI from this script, one stream: the cross-check beside the driver's figure."""
     from nnforge_amd import workloads as w
@@ -938,7 +972,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--workload", default="config0", choices=["config0", "config1", "config2", "config3", "config4", "copy", "max_subsampling", "bn_relu_max_subsampling", "max_subsampling_tiling",
                              "entry_window", "concat", "maxout", "feature_map_stat", "config4_direct", "yardsticks", "walking_grid",
-                             "global_average", "joined_global_average"],
+                             "global_average", "joined_global_average", "inception_block", "inception_block_copies"],
                     help="'copy' times the plain copy kernel (profiler-counter calibration and bandwidth yardstick); 'yardsticks' the runtime's and "
                          "torch's copy routines beside the library's kernels; 'config4_direct' the launches of config4 issued at the C ABI from this script")
     ap.add_argument("--entries", type=int, default=64, help="config4: entries per packet (BASELINE.json's configuration has 64)")
@@ -991,6 +1025,8 @@ def main():
             return bench_group(runner, "batch_norm -> rectified_linear N=64 C=64 56x56 (51 MB per tensor: the grid that stays put)", w.bn_relu("bn_relu", 64, 64, 56 * 56), steps, warmup)
         if name == "config4_direct":
             return bench_resnet50_direct(runner, steps, warmup)
+        if name in ("inception_block", "inception_block_copies"):
+            return bench_inception_block(runner, steps, warmup, n=args.entries if args.entries != 64 else 128, copies=name.endswith("copies"))
         if name == "yardsticks":
             return bench_yardsticks(runner, steps, warmup)
         return bench_resnet50(runner, steps, warmup, n=args.entries, kernel_stream_count=args.kernel_streams, one_launch_per_group=args.one_launch_per_group)
@@ -1025,7 +1061,8 @@ def main():
         per_config["copy_kernel"] = bench_copy(runner, 40, 5)
         # the neighbouring layers of the same chains
         for name, (k, wu) in (("global_average", (100, 10)), ("joined_global_average", (100, 10)), ("max_subsampling", (40, 5)), ("bn_relu_max_subsampling", (40, 5)),
-                              ("max_subsampling_tiling", (40, 5)), ("entry_window", (40, 5)), ("concat", (100, 10)), ("maxout", (100, 10)), ("feature_map_stat", (20, 3))):
+                              ("max_subsampling_tiling", (40, 5)), ("entry_window", (40, 5)), ("concat", (100, 10)), ("maxout", (100, 10)), ("feature_map_stat", (20, 3)),
+                              ("inception_block", (100, 10)), ("inception_block_copies", (100, 10))):
             if name not in per_config:
                 per_config[name] = run(name, k, wu)
         if args.workload == "config0":
@@ -1071,6 +1108,7 @@ def main():
                        "concat": "nnf::concat_kernel", "maxout": "nnf::maxout_vec4_kernel",
                        "feature_map_stat": "nnf::stat_runs_kernel", "walking_grid": "nnf::chain_kernel_persistent",
                        "global_average": "nnf::global_pool_linear_kernel", "joined_global_average": "nnf::global_pool_linear_kernel",
+                       "inception_block": "nnf::chain_entries_batch_kernel", "inception_block_copies": "nnf::chain_batch_kernel + nnf::concat_kernel",
                        "config4": "all kernels of one pass of the launch plan (nnf::chain_batch_mixed_kernel, nnf::chain_batch_kernel, nnf::chain_kernel, nnf::global_pool_linear_kernel, nnf::softmax_rows_kernel)",
                        "config4_direct": "all kernels of one pass (nnf::chain_kernel x 49, nnf::global_pool_kernel, nnf::softmax_rows_kernel)"}.get(args.workload, "nnf::chain_kernel"),
             "algorithmic_bytes_per_launch": main_entry["algorithmic_bytes_per_step"] / launches,
