@@ -329,7 +329,7 @@ def resnet50_network(n, gen):
     return schemas.schema_text(layers, "ResNet-50 post-convolution"), weights, configs, outputs
 
 
-def bench_resnet50(runner, steps, warmup, n=64, kernel_stream_count=0, one_launch_per_group=False):
+def bench_resnet50(runner, steps, warmup, n=64, kernel_stream_count=0, one_launch_per_group=False, replay_recorded_plan=False):
     """Config 4 through the product driver: the ResNet-50 post-convolution graph (convolution outputs as data layers) handed to
     forward_propagation_hip, whose fusion pass makes the 49 groups + average + softmax (the last group applied by the average's
     kernel on the way in, so that its result is neither written nor read back) and enqueues them on its kernel streams;
@@ -343,7 +343,8 @@ def bench_resnet50(runner, steps, warmup, n=64, kernel_stream_count=0, one_launc
     largest = max(fm * dims[0] * dims[1] for fm, dims in configs.values())
     pool = gen.standard_normal(n * largest, dtype=np.float32)
     rep = backend.time_kernels(text, weights, configs, outputs, warmup=warmup, passes=steps, shared_input_pool=pool, entry_count=n,
-                               max_entry_count=n, kernel_stream_count=kernel_stream_count, one_launch_per_group=one_launch_per_group)
+                               max_entry_count=n, kernel_stream_count=kernel_stream_count, one_launch_per_group=one_launch_per_group,
+                               replay_recorded_plan=replay_recorded_plan)
     groups = w.resnet50_groups(n)
     assert rep["timed_entries"] == n and rep["plan_steps"] == len(groups) + 1, rep["raw"]
     # the driver orders the steps into the slots of its launch plan: same groups as the hand-written list, not the same order; the step
@@ -357,7 +358,7 @@ def bench_resnet50(runner, steps, warmup, n=64, kernel_stream_count=0, one_launc
     assert sum(step["layers"][-1] == "pool5" and step["fused"] for step in rep["steps"]) == 1, rep["raw"]
     return result_entry("config4: ResNet-50 post-convolution stack N=%d (49 fused groups + 7x7 average + softmax) through forward_propagation_hip" % n,
                         g_bytes + p_bytes + s_bytes, elements, rep["wall_seconds_per_pass"], rep["device_seconds_per_pass"], 1,
-                        {"plan_steps_per_pass": rep["plan_steps"], "kernel_launches_per_pass": rep["launches"], "host_enqueue_ms_per_pass": rep["host_seconds_per_pass"] * 1e3, "kernel_streams": len({st["stream"] for st in rep["steps"]}),
+                        {"plan_steps_per_pass": rep["plan_steps"], "kernel_launches_per_pass": rep["launches"], "replayed_from_a_recorded_graph": bool(replay_recorded_plan), "host_enqueue_ms_per_pass": rep["host_seconds_per_pass"] * 1e3, "kernel_streams": len({st["stream"] for st in rep["steps"]}),
                          "runs_of_groups_launched_together": len({st["run"] for st in rep["steps"] if st["run"] is not None}),
                          "note": "a step is one pass of the launch plan, timed inside the C++ driver (forward_propagation_hip::time_kernels): "
                                  "one resident packet, the plan enqueued on the driver's kernel streams (independent groups share kernel "
@@ -978,6 +979,7 @@ def main():
     ap.add_argument("--entries", type=int, default=64, help="config4: entries per packet (BASELINE.json's configuration has 64)")
     ap.add_argument("--one-launch-per-group", action="store_true", help="config4: switch the driver's hip_batch_independent_groups off")
     ap.add_argument("--kernel-streams", type=int, default=0, help="config4: kernel streams of the driver (hip_kernel_stream_count); 0 = its default")
+    ap.add_argument("--replay-recorded-plan", action="store_true", help="config4: the timed passes replay a HIP graph recorded from the plan's launches")
     ap.add_argument("--only", action="store_true", help="time only the chosen workload (no per_config survey, no CPU baseline)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -1029,7 +1031,8 @@ def main():
             return bench_inception_block(runner, steps, warmup, n=args.entries if args.entries != 64 else 128, copies=name.endswith("copies"))
         if name == "yardsticks":
             return bench_yardsticks(runner, steps, warmup)
-        return bench_resnet50(runner, steps, warmup, n=args.entries, kernel_stream_count=args.kernel_streams, one_launch_per_group=args.one_launch_per_group)
+        return bench_resnet50(runner, steps, warmup, n=args.entries, kernel_stream_count=args.kernel_streams, one_launch_per_group=args.one_launch_per_group,
+                              replay_recorded_plan=args.replay_recorded_plan)
 
     main_entry = run(args.workload, args.steps, args.warmup)
     per_config[args.workload] = main_entry
