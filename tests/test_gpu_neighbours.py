@@ -210,6 +210,11 @@ TILING_CASES = [
     ((1, 2, 200, 300), [3, 2]),           # bands of a large plane
     ((2, 3, 112, 112), [3, 3]),           # a whole plane per workgroup
     ((64, 64, 112, 112), [2, 2]),         # the benchmark's shape: 256 output entries of 55 x 55
+    ((2, 5, 112, 112), [2, 2]),           # ten planes in five bands each: 40 workgroups regrouped by die, the last 10 in plain order
+    ((1, 3, 100, 96), [2, 2]),            # strips of four columns, bands of unequal height
+    ((3, 7, 90, 120), [2, 2]),
+    ((1, 1, 5000, 4), [2, 2]),            # rows of one strip
+    ((2, 9, 200, 300), [3, 2]),           # bands regrouped by die in the general kernel
     ((2, 1, 5, 20000), [2, 2]),           # rows too wide to stage: one lane per output
     ((3, 2, 40000), [3]),                 # 1-D, wide
 ]
@@ -342,7 +347,7 @@ def test_max_subsampling_where_the_first_zero_decides(gpu, shape, windows, strid
 
 
 @pytest.mark.parametrize("is_min", [False, True])
-@pytest.mark.parametrize("shape,windows", [((4, 16, 112, 112), [2, 2]), ((2, 3, 60, 60), [3, 3]), ((7, 37, 6, 5), [2, 2]),
+@pytest.mark.parametrize("shape,windows", [((4, 16, 112, 112), [2, 2]), ((1, 3, 100, 96), [2, 2]), ((2, 3, 60, 60), [3, 3]), ((7, 37, 6, 5), [2, 2]),
                                            ((3, 4, 9, 11), [2, 3]), ((5, 2, 23), [4])])
 def test_max_subsampling_with_tiling_where_the_first_zero_decides(gpu, shape, windows, is_min):
     x = zero_heavy(T.rng(72, sum(shape)), shape)
