@@ -207,7 +207,8 @@ namespace nnf
 		// read - two LDS reads per window row and pair instead of six, none of them with lanes two words apart (which
 		// puts two lanes on every bank), and the two results leave as one 8-byte store. Each window is still folded
 		// in the reference's order (x fastest, then y).
-		template<int OP, int WIN_W, int WIN_H, bool TRUNC, bool PROLOGUE, bool EXP, bool UNIFORM, bool PAIR = false>
+		// BN_RELU: the layers are BatchNorm -> ReLU and nothing else (with UNIFORM; apply_known_group)
+		template<int OP, int WIN_W, int WIN_H, bool TRUNC, bool PROLOGUE, bool EXP, bool UNIFORM, bool PAIR = false, bool BN_RELU = false>
 		__device__ __forceinline__ void window2d_body(const window2d_args& a, const window_prologue& pro)
 		{
 			static_assert(!PAIR || (((WIN_W == 2) || (WIN_W == 3)) && (WIN_H > 0)), "pairs of outputs: windows 2 or 3 wide, height known");
@@ -270,13 +271,16 @@ namespace nnf
 						// and every load waited for the ones before it.
 						t[k] = load_stream(reinterpret_cast<const floatx4*>(a.in + g0_aligned) + min(i, limit - 1));
 					}
-					else if (i < limit)
+					else
 					{
-						const uint32_t g = g0_aligned + i * 4;
-						t[k].x = a.in[g];
-						t[k].y = (g + 1 < a.total_in) ? a.in[g + 1] : 0.0f;
-						t[k].z = (g + 2 < a.total_in) ? a.in[g + 2] : 0.0f;
-						t[k].w = 0.0f;
+						t[k].x = t[k].y = t[k].z = t[k].w = 0.0f;
+						if (i < limit)
+						{
+							const uint32_t g = g0_aligned + i * 4;
+							t[k].x = a.in[g];
+							t[k].y = (g + 1 < a.total_in) ? a.in[g + 1] : 0.0f;
+							t[k].z = (g + 2 < a.total_in) ? a.in[g + 2] : 0.0f;
+						}
 					}
 				}
 				if (PROLOGUE && first_round)
@@ -308,8 +312,9 @@ namespace nnf
 					{
 						const uint32_t i = base + k * max_block_size + threadIdx.x;
 						const bool valid = i < limit;
-						// lanes past the end put zeros through the layers
-						v[k][0] = valid ? t[k].x : 0.0f; v[k][1] = valid ? t[k].y : 0.0f; v[k][2] = valid ? t[k].z : 0.0f; v[k][3] = valid ? t[k].w : 0.0f;
+						// lanes past the end put the values they hold through the layers with the others (whole float4s: the
+						// last float4 once more; the partial one: zeros) and store nothing
+						v[k][0] = t[k].x; v[k][1] = t[k].y; v[k][2] = t[k].z; v[k][3] = t[k].w;
 						// plane, inside the workgroup's range, of the first float of this float4 (floats in front
 						// of the range count as plane 0: they are staged but not read)
 						const uint32_t first_pos = max(i * 4, shift) - shift;
@@ -320,7 +325,9 @@ namespace nnf
 						if (straddle && valid && (p + 1 < planes_here) && (i * 4 + 3 >= (p + 1) * in_plane + shift))
 							straddling |= 1u << k;
 					}
-					if (uniform)
+					if (BN_RELU)
+						apply_known_group<COUNT, known_group_batch_norm_relu, true>(v, v, off, lds_coef, own_coef, pro, exp_ctx);
+					else if (uniform)
 						apply_prologue<COUNT, EXP, true>(v, off, lds_coef, own_coef, pro, exp_ctx, 0, pro.op_count);
 					else
 						apply_prologue<COUNT, EXP, false>(v, off, lds_coef, own_coef, pro, exp_ctx, 0, pro.op_count);
@@ -564,6 +571,13 @@ namespace nnf
 		__global__ void __launch_bounds__(max_block_size) __attribute__((amdgpu_waves_per_eu(UNIFORM ? 6 : 5, UNIFORM ? 6 : 5))) max_window2d_prologue_kernel(const window2d_args a, const window_prologue pro)
 		{
 			window2d_body<OP, WIN_W, WIN_H, TRUNC, true, false, UNIFORM, PAIR>(a, pro);
+		}
+
+		// One plane per workgroup, BatchNorm -> ReLU in front of the windows: the layers as straight code
+		template<int OP, int WIN_W, int WIN_H, bool TRUNC, bool PAIR = false>
+		__global__ void __launch_bounds__(max_block_size) __attribute__((amdgpu_waves_per_eu(6, 6))) max_window2d_bn_relu_kernel(const window2d_args a, const window_prologue pro)
+		{
+			window2d_body<OP, WIN_W, WIN_H, TRUNC, true, false, true, PAIR, true>(a, pro);
 		}
 
 		template<int OP, int WIN_W, int WIN_H, bool TRUNC, bool UNIFORM>
@@ -1270,6 +1284,15 @@ namespace nnf
 				if (w3) NNF_LAUNCH((max_window2d_exp_prologue_kernel<OP, 3, 3, TRUNC, UNIFORM>), g, b, lds_bytes, stream, a, pro);
 				else if (w2) NNF_LAUNCH((max_window2d_exp_prologue_kernel<OP, 2, 2, TRUNC, UNIFORM>), g, b, lds_bytes, stream, a, pro);
 				else NNF_LAUNCH((max_window2d_exp_prologue_kernel<OP, 0, 0, TRUNC, UNIFORM>), g, b, lds_bytes, stream, a, pro);
+			}
+			else if (UNIFORM && (known_group_of(pro) == known_group_batch_norm_relu))
+			{
+				const bool pair = pairs_of_outputs(a);
+				if (w3 && pair) NNF_LAUNCH((max_window2d_bn_relu_kernel<OP, 3, 3, TRUNC, true>), g, b, lds_bytes, stream, a, pro);
+				else if (w2 && pair) NNF_LAUNCH((max_window2d_bn_relu_kernel<OP, 2, 2, TRUNC, true>), g, b, lds_bytes, stream, a, pro);
+				else if (w3) NNF_LAUNCH((max_window2d_bn_relu_kernel<OP, 3, 3, TRUNC>), g, b, lds_bytes, stream, a, pro);
+				else if (w2) NNF_LAUNCH((max_window2d_bn_relu_kernel<OP, 2, 2, TRUNC>), g, b, lds_bytes, stream, a, pro);
+				else NNF_LAUNCH((max_window2d_bn_relu_kernel<OP, 0, 0, TRUNC>), g, b, lds_bytes, stream, a, pro);
 			}
 			else
 			{

@@ -174,6 +174,201 @@ namespace nnf
 
 		// UNIFORM: every value belongs to the same plane, whose coefficients are in own (registers)
 		// instead of coef (LDS). SPLIT: a vector's values may belong to two planes (two says which).
+		// One layer (kind, the slot of its coefficients, its two constants) over the values of a round.
+		template<int VECTORS, bool EXP, bool UNIFORM, bool SPLIT = false>
+		__device__ __forceinline__ void apply_prologue_layer(float (&v)[VECTORS][4], const uint32_t (&off)[VECTORS],
+			const float* coef, const float (&own)[prologue_weighted_max][2], const exp_context& exp_ctx, const two_plane_offsets<VECTORS>* two,
+			const int32_t kind, const uint32_t slot, const float f0, const float f1)
+		{
+			switch (kind)
+			{
+			case NNF_HIP_OP_BATCH_NORM:
+				if (UNIFORM)
+				{
+					static_assert(prologue_weighted_max == 2, "the coefficients of a layer are picked from two sets");
+					const float mult = (slot == 0) ? own[0][0] : own[1][0];
+					const float add = (slot == 0) ? own[0][1] : own[1][1];
+					#pragma unroll
+					for(int k = 0; k < VECTORS; ++k)
+					{
+						#pragma unroll
+						for(int e = 0; e < 4; ++e)
+							v[k][e] = nnf_batch_norm(v[k][e], mult, add);
+					}
+					break;
+				}
+				if (SPLIT)
+				{
+					float mult[VECTORS][2], add[VECTORS][2];
+					#pragma unroll
+					for(int k = 0; k < VECTORS; ++k)
+					{
+						mult[k][0] = coef[off[k] + slot];
+						add[k][0] = coef[off[k] + slot + 1];
+						mult[k][1] = coef[two->off2[k] + slot];
+						add[k][1] = coef[two->off2[k] + slot + 1];
+					}
+					#pragma unroll
+					for(int k = 0; k < VECTORS; ++k)
+					{
+						#pragma unroll
+						for(int e = 0; e < 4; ++e)
+						{
+							const bool first_plane = static_cast<uint32_t>(e) < two->split[k];
+							v[k][e] = nnf_batch_norm(v[k][e], first_plane ? mult[k][0] : mult[k][1], first_plane ? add[k][0] : add[k][1]);
+						}
+					}
+					break;
+				}
+				#pragma unroll
+				for(int k0 = 0; k0 < VECTORS; k0 += coef_batch)
+				{
+					float mult[coef_batch], add[coef_batch];
+					#pragma unroll
+					for(int k = 0; (k < coef_batch) && (k0 + k < VECTORS); ++k)
+					{
+						mult[k] = coef[off[k0 + k] + slot];
+						add[k] = coef[off[k0 + k] + slot + 1];
+					}
+					#pragma unroll
+					for(int k = 0; (k < coef_batch) && (k0 + k < VECTORS); ++k)
+					{
+						#pragma unroll
+						for(int e = 0; e < 4; ++e)
+							v[k0 + k][e] = nnf_batch_norm(v[k0 + k][e], mult[k], add[k]);
+					}
+				}
+				break;
+			case NNF_HIP_OP_PRELU:
+				if (UNIFORM)
+				{
+					const float slope = (slot == 0) ? own[0][0] : own[1][0];
+					#pragma unroll
+					for(int k = 0; k < VECTORS; ++k)
+					{
+						#pragma unroll
+						for(int e = 0; e < 4; ++e)
+							v[k][e] = nnf_parametric_rectified_linear(v[k][e], slope);
+					}
+				}
+				else if (SPLIT)
+				{
+					float slope[VECTORS][2];
+					#pragma unroll
+					for(int k = 0; k < VECTORS; ++k)
+					{
+						slope[k][0] = coef[off[k] + slot];
+						slope[k][1] = coef[two->off2[k] + slot];
+					}
+					#pragma unroll
+					for(int k = 0; k < VECTORS; ++k)
+					{
+						#pragma unroll
+						for(int e = 0; e < 4; ++e)
+							v[k][e] = nnf_parametric_rectified_linear(v[k][e], (static_cast<uint32_t>(e) < two->split[k]) ? slope[k][0] : slope[k][1]);
+					}
+				}
+				else
+				{
+					float slope[VECTORS];
+					#pragma unroll
+					for(int k = 0; k < VECTORS; ++k)
+						slope[k] = coef[off[k] + slot];
+					#pragma unroll
+					for(int k = 0; k < VECTORS; ++k)
+					{
+						#pragma unroll
+						for(int e = 0; e < 4; ++e)
+							v[k][e] = nnf_parametric_rectified_linear(v[k][e], slope[k]);
+					}
+				}
+				break;
+			case NNF_HIP_OP_RELU:
+				#pragma unroll
+				for(int k = 0; k < VECTORS; ++k)
+				{
+					#pragma unroll
+					for(int e = 0; e < 4; ++e)
+						v[k][e] = nnf_rectified_linear(v[k][e], f0);
+				}
+				break;
+			case NNF_HIP_OP_ABSOLUTE:
+				#pragma unroll
+				for(int k = 0; k < VECTORS; ++k)
+				{
+					#pragma unroll
+					for(int e = 0; e < 4; ++e)
+						v[k][e] = nnf_absolute(v[k][e]);
+				}
+				break;
+			case NNF_HIP_OP_ELU:
+			case NNF_HIP_OP_SIGMOID:
+			case NNF_HIP_OP_TANH:
+				if (EXP)
+				{
+					#pragma unroll
+					for(int k = 0; k < VECTORS; ++k)
+					{
+						if (kind == NNF_HIP_OP_ELU)
+							nnf_exponential_linear<4>(v[k], exp_ctx);
+						else if (kind == NNF_HIP_OP_SIGMOID)
+							nnf_sigmoid<4>(v[k], exp_ctx);
+						else
+							nnf_hyperbolic_tangent<4>(v[k], f1, f0, exp_ctx);
+					}
+				}
+				break;
+			default: // NNF_HIP_OP_DROPOUT: the value passes through
+				break;
+			}
+		}
+
+		// The two groups a residual network puts in front of its subsampling layers, as straight code for kernels compiled for
+		// just them: BatchNorm -> ReLU (between the first convolution and its pooling) and BatchNorm + shortcut -> Add -> ReLU
+		// (the last block in front of the global average). The loop of apply_prologue keeps the values of a round in fixed
+		// registers and copies every one of them once per layer (64 x 64 planes of 112 x 112 through BatchNorm, ReLU and 3 x 3
+		// pooling: 20.3 M vector instructions per launch with the loop, of which the two layers need a third). As a second
+		// path beside the loop in one kernel the straight code costs that kernel 40 spilled registers, hence kernels of its own:
+		// the pooling kernels have them for the first group (44.2 -> 42.1 us on those planes); the whole-plane average with the
+		// second group folded in does not wait for its vector instructions (14.1 us either way) and keeps the loop.
+		constexpr int known_group_none = 0;
+		constexpr int known_group_batch_norm_relu = 1;
+		constexpr int known_group_batch_norm_shortcut_add_relu = 2;
+
+		inline int known_group_of(const window_prologue& pro)
+		{
+			if ((pro.op_count != 2) || (pro.kind[0] != NNF_HIP_OP_BATCH_NORM) || (pro.kind[1] != NNF_HIP_OP_RELU))
+				return known_group_none;
+			if (pro.join == 0)
+				return known_group_batch_norm_relu;
+			return ((pro.arm_ops[0] == 1) && (pro.arm_ops[1] == 0)) ? known_group_batch_norm_shortcut_add_relu : known_group_none;
+		}
+
+		template<int VECTORS, int GROUP, bool UNIFORM, bool SPLIT = false>
+		__device__ __forceinline__ void apply_known_group(float (&v)[VECTORS][4], float (&u)[VECTORS][4], const uint32_t (&off)[VECTORS],
+			const float* coef, const float (&own)[prologue_weighted_max][2], const window_prologue& pro, const exp_context& exp_ctx,
+			const two_plane_offsets<VECTORS>* two = nullptr)
+		{
+			static_assert((GROUP == known_group_batch_norm_relu) || (GROUP == known_group_batch_norm_shortcut_add_relu), "one of the known groups");
+			apply_prologue_layer<VECTORS, false, UNIFORM, SPLIT>(v, off, coef, own, exp_ctx, two, NNF_HIP_OP_BATCH_NORM, 0u, 0.0f, 0.0f);
+			if (GROUP == known_group_batch_norm_shortcut_add_relu)
+			{
+				// nnforge/plain/add_layer_tester_plain.cpp:56-59: the sum starts at 0.0F, inputs in order, times alpha
+				#pragma unroll
+				for(int k = 0; k < VECTORS; ++k)
+				{
+					#pragma unroll
+					for(int e = 0; e < 4; ++e)
+					{
+						float sum = 0.0f + v[k][e];
+						sum = sum + u[k][e];
+						v[k][e] = sum * pro.alpha;
+					}
+				}
+			}
+			apply_prologue_layer<VECTORS, false, UNIFORM, SPLIT>(v, off, coef, own, exp_ctx, two, NNF_HIP_OP_RELU, 0u, pro.f0[1], 0.0f);
+		}
+
 		// Applies the layers first_op .. end_op - 1.
 		template<int VECTORS, bool EXP, bool UNIFORM, bool SPLIT = false>
 		__device__ __forceinline__ void apply_prologue(float (&v)[VECTORS][4], const uint32_t (&off)[VECTORS],
@@ -181,152 +376,7 @@ namespace nnf
 			uint32_t first_op, uint32_t end_op, const two_plane_offsets<VECTORS>* two = nullptr)
 		{
 			for(uint32_t i = first_op; i < end_op; ++i)
-			{
-				const int32_t kind = pro.kind[i];
-				const uint32_t slot = pro.slot[i];
-				const float f0 = pro.f0[i], f1 = pro.f1[i];
-				switch (kind)
-				{
-				case NNF_HIP_OP_BATCH_NORM:
-					if (UNIFORM)
-					{
-						static_assert(prologue_weighted_max == 2, "the coefficients of a layer are picked from two sets");
-						const float mult = (slot == 0) ? own[0][0] : own[1][0];
-						const float add = (slot == 0) ? own[0][1] : own[1][1];
-						#pragma unroll
-						for(int k = 0; k < VECTORS; ++k)
-						{
-							#pragma unroll
-							for(int e = 0; e < 4; ++e)
-								v[k][e] = nnf_batch_norm(v[k][e], mult, add);
-						}
-						break;
-					}
-					if (SPLIT)
-					{
-						float mult[VECTORS][2], add[VECTORS][2];
-						#pragma unroll
-						for(int k = 0; k < VECTORS; ++k)
-						{
-							mult[k][0] = coef[off[k] + slot];
-							add[k][0] = coef[off[k] + slot + 1];
-							mult[k][1] = coef[two->off2[k] + slot];
-							add[k][1] = coef[two->off2[k] + slot + 1];
-						}
-						#pragma unroll
-						for(int k = 0; k < VECTORS; ++k)
-						{
-							#pragma unroll
-							for(int e = 0; e < 4; ++e)
-							{
-								const bool first_plane = static_cast<uint32_t>(e) < two->split[k];
-								v[k][e] = nnf_batch_norm(v[k][e], first_plane ? mult[k][0] : mult[k][1], first_plane ? add[k][0] : add[k][1]);
-							}
-						}
-						break;
-					}
-					#pragma unroll
-					for(int k0 = 0; k0 < VECTORS; k0 += coef_batch)
-					{
-						float mult[coef_batch], add[coef_batch];
-						#pragma unroll
-						for(int k = 0; (k < coef_batch) && (k0 + k < VECTORS); ++k)
-						{
-							mult[k] = coef[off[k0 + k] + slot];
-							add[k] = coef[off[k0 + k] + slot + 1];
-						}
-						#pragma unroll
-						for(int k = 0; (k < coef_batch) && (k0 + k < VECTORS); ++k)
-						{
-							#pragma unroll
-							for(int e = 0; e < 4; ++e)
-								v[k0 + k][e] = nnf_batch_norm(v[k0 + k][e], mult[k], add[k]);
-						}
-					}
-					break;
-				case NNF_HIP_OP_PRELU:
-					if (UNIFORM)
-					{
-						const float slope = (slot == 0) ? own[0][0] : own[1][0];
-						#pragma unroll
-						for(int k = 0; k < VECTORS; ++k)
-						{
-							#pragma unroll
-							for(int e = 0; e < 4; ++e)
-								v[k][e] = nnf_parametric_rectified_linear(v[k][e], slope);
-						}
-					}
-					else if (SPLIT)
-					{
-						float slope[VECTORS][2];
-						#pragma unroll
-						for(int k = 0; k < VECTORS; ++k)
-						{
-							slope[k][0] = coef[off[k] + slot];
-							slope[k][1] = coef[two->off2[k] + slot];
-						}
-						#pragma unroll
-						for(int k = 0; k < VECTORS; ++k)
-						{
-							#pragma unroll
-							for(int e = 0; e < 4; ++e)
-								v[k][e] = nnf_parametric_rectified_linear(v[k][e], (static_cast<uint32_t>(e) < two->split[k]) ? slope[k][0] : slope[k][1]);
-						}
-					}
-					else
-					{
-						float slope[VECTORS];
-						#pragma unroll
-						for(int k = 0; k < VECTORS; ++k)
-							slope[k] = coef[off[k] + slot];
-						#pragma unroll
-						for(int k = 0; k < VECTORS; ++k)
-						{
-							#pragma unroll
-							for(int e = 0; e < 4; ++e)
-								v[k][e] = nnf_parametric_rectified_linear(v[k][e], slope[k]);
-						}
-					}
-					break;
-				case NNF_HIP_OP_RELU:
-					#pragma unroll
-					for(int k = 0; k < VECTORS; ++k)
-					{
-						#pragma unroll
-						for(int e = 0; e < 4; ++e)
-							v[k][e] = nnf_rectified_linear(v[k][e], f0);
-					}
-					break;
-				case NNF_HIP_OP_ABSOLUTE:
-					#pragma unroll
-					for(int k = 0; k < VECTORS; ++k)
-					{
-						#pragma unroll
-						for(int e = 0; e < 4; ++e)
-							v[k][e] = nnf_absolute(v[k][e]);
-					}
-					break;
-				case NNF_HIP_OP_ELU:
-				case NNF_HIP_OP_SIGMOID:
-				case NNF_HIP_OP_TANH:
-					if (EXP)
-					{
-						#pragma unroll
-						for(int k = 0; k < VECTORS; ++k)
-						{
-							if (kind == NNF_HIP_OP_ELU)
-								nnf_exponential_linear<4>(v[k], exp_ctx);
-							else if (kind == NNF_HIP_OP_SIGMOID)
-								nnf_sigmoid<4>(v[k], exp_ctx);
-							else
-								nnf_hyperbolic_tangent<4>(v[k], f1, f0, exp_ctx);
-						}
-					}
-					break;
-				default: // NNF_HIP_OP_DROPOUT: the value passes through
-					break;
-				}
-			}
+				apply_prologue_layer<VECTORS, EXP, UNIFORM, SPLIT>(v, off, coef, own, exp_ctx, two, pro.kind[i], pro.slot[i], pro.f0[i], pro.f1[i]);
 		}
 
 
