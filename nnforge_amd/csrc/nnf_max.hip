@@ -678,8 +678,10 @@ namespace nnf
 			uint32_t fm_count, plane_count; // planes = entries * feature maps
 			uint32_t planes;                // whole planes per workgroup; 1: bands of `rows` output rows, `bands` per plane
 			uint32_t rows, bands;
-			uint32_t in_area;               // bands: LDS floats in front of the grids' output runs
-			uint32_t out_pitch;             // bands: LDS floats from one grid's run to the next (a multiple of 4)
+			uint32_t runs;                  // results leave as one run per grid (bands, or planes of one entry); 0: stored from the scan
+			uint32_t in_area;               // runs: LDS floats in front of the grids' output runs
+			uint32_t out_pitch;             // runs: LDS floats from one grid's run to the next (a multiple of 4)
+			uint32_t together;              // runs: consecutive work items that go to workgroups of one XCD (xcd_grouped)
 		};
 
 		// What a workgroup stages: planes [first_plane, first_plane + planes_here), output rows [oy0, oy1) of them
@@ -727,7 +729,7 @@ namespace nnf
 		{
 			const uint32_t win_w = (WIN_W > 0) ? WIN_W : a.win_w, win_h = (WIN_H > 0) ? WIN_H : a.win_h;
 			const uint32_t in_plane = a.in_w * a.in_h, out_plane = a.out_w * a.out_h;
-			const bool band = a.planes == 1;
+			const bool band = a.runs != 0; // positions of the workgroup lie in every grid's output one after the other
 			const uint32_t first_plane = r.first_plane, planes_here = r.planes_here;
 			const float* staged = staged_area + r.shift;
 			const uint32_t rows_here = r.oy1 - r.oy0;
@@ -983,7 +985,7 @@ namespace nnf
 			const uint32_t band_entry = r.first_plane / a.fm_count;
 			const uint32_t band_fm = r.first_plane - band_entry * a.fm_count;
 			const uint32_t band_out_index = (band_entry * tiles * a.fm_count + band_fm) * out_plane + r.oy0 * a.out_w;
-			const uint32_t positions = (r.oy1 - r.oy0) * a.out_w;
+			const uint32_t positions = r.planes_here * (r.oy1 - r.oy0) * a.out_w;
 			const float* runs = staged_area + a.in_area;
 			for(uint32_t g = 0; g < tiles; ++g)
 			{
@@ -1014,7 +1016,7 @@ namespace nnf
 		{
 			extern __shared__ __attribute__((aligned(16))) float staged_area[];
 			const uint32_t win_w = (WIN_W > 0) ? WIN_W : a.win_w, win_h = (WIN_H > 0) ? WIN_H : a.win_h;
-			const uint32_t work_id = (a.planes == 1) ? xcd_grouped(blockIdx.x, a.bands, gridDim.x) : blockIdx.x;
+			const uint32_t work_id = a.runs ? xcd_grouped(blockIdx.x, a.together, gridDim.x) : blockIdx.x;
 			const tiling_range r = tiling_range_of(a, work_id, win_h);
 			// Eight loads in flight per lane before the first LDS store. A band of the usual size is two or three float4s per
 			// lane; with sixteen the kernel holds 73 registers per lane and 64 x 64 planes of 112 x 112 with 2 x 2 windows
@@ -1048,7 +1050,7 @@ namespace nnf
 				tiling_scan_strips<OP, BLOCK>(a, r, staged_area);
 			else
 				tiling_scan<OP, WIN_W, WIN_H, BLOCK>(a, r, staged_area);
-			if (a.planes > 1)
+			if (!a.runs)
 				return;
 			__syncthreads();
 			tiling_write_runs<BLOCK>(a, r, staged_area, win_w * win_h);
@@ -1083,20 +1085,37 @@ namespace nnf
 				return false;
 			uint32_t grid;
 			size_t lds_floats;
-			bool strips = false;
 			a.planes = 1;
+			a.runs = 1;
+			const uint32_t out_plane = out_w * out_h;
+			// several whole planes of one entry: their input (+ 3 floats in front of an unaligned start) and a run of their outputs per grid
+			auto planes_floats = [&](uint32_t planes, uint32_t& in_area, uint32_t& out_pitch) -> uint64_t
+			{
+				in_area = static_cast<uint32_t>((planes * in_plane + 3 + 3) & ~static_cast<uint64_t>(3));
+				out_pitch = (planes * out_plane + 3 + 3) & ~3u;
+				return static_cast<uint64_t>(in_area) + static_cast<uint64_t>(tiles) * out_pitch;
+			};
+			// planes of any entries with results stored from the scan: what remains when runs would leave the lanes with too little
+			uint32_t planes_without_runs = 1;
 			if (in_plane * 2 + 3 <= lds_floats_max)
 			{
-				// small planes: enough of them for four positions per lane, as far as LDS holds them
-				const uint32_t wanted = (4 * max_block_size + out_w * out_h - 1) / (out_w * out_h);
-				a.planes = max(1u, min(min(wanted, static_cast<uint32_t>((lds_floats_max - 3) / in_plane)), plane_count));
+				const uint32_t wanted = (4 * max_block_size + out_plane - 1) / out_plane;
+				planes_without_runs = max(1u, min(min(wanted, static_cast<uint32_t>((lds_floats_max - 3) / in_plane)), plane_count));
 			}
-			if (a.planes > 1)
+			constexpr uint32_t positions_worth_runs = 2 * max_block_size;
+			if (planes_floats(1, a.in_area, a.out_pitch) <= lds_floats_band)
 			{
+				// Planes that fit the budget whole: as many of one entry (so that their outputs are one run in every grid: a
+				// divisor of the number of feature maps) as stay within it, until the lanes have four positions each.
+				uint32_t in_area, out_pitch;
+				for(uint32_t planes = 2; (planes <= fm_count) && ((planes - 1) * out_plane < 4 * max_block_size); ++planes)
+				{
+					if ((fm_count % planes == 0) && (planes_floats(planes, in_area, out_pitch) <= lds_floats_band))
+						a.planes = planes;
+				}
 				a.rows = out_h;
 				a.bands = 1;
-				grid = (plane_count + a.planes - 1) / a.planes;
-				lds_floats = a.planes * static_cast<size_t>(in_plane) + 8;
+				a.together = 4; // neighbouring workgroups' runs meet in cache lines, as the bands of a plane do
 			}
 			else
 			{
@@ -1109,11 +1128,29 @@ namespace nnf
 				const uint32_t bands_wanted = (1024 + plane_count - 1) / plane_count;
 				a.bands = max(a.bands, min(bands_wanted, max(1u, out_h / 4)));
 				a.rows = (out_h + a.bands - 1) / a.bands; // bands of equal height
-				strips = (win_w == 2) && (win_h == 2) && (in_w % 4 == 0);
 				a.bands = (out_h + a.rows - 1) / a.rows;
+				a.together = a.bands;
+			}
+			if ((a.planes * a.rows * out_w < positions_worth_runs) && (planes_without_runs > 1))
+			{
+				a.planes = planes_without_runs;
+				a.runs = 0;
+				a.rows = out_h;
+				a.bands = 1;
+				grid = (plane_count + a.planes - 1) / a.planes;
+				lds_floats = a.planes * static_cast<size_t>(in_plane) + 8;
+			}
+			else if (a.bands == 1)
+			{
+				grid = (plane_count + a.planes - 1) / a.planes;
+				lds_floats = planes_floats(a.planes, a.in_area, a.out_pitch);
+			}
+			else
+			{
 				grid = plane_count * a.bands;
 				lds_floats = band_floats(a.rows, a.in_area, a.out_pitch);
 			}
+			const bool strips = a.runs && (a.planes == 1) && (win_w == 2) && (win_h == 2) && (in_w % 4 == 0);
 			const size_t lds_bytes = lds_floats * sizeof(float);
 			constexpr int block = max_block_size;
 			const bool w2 = (win_w == 2) && (win_h == 2), w3 = (win_w == 3) && (win_h == 3);

@@ -204,7 +204,10 @@ TILING_CASES = [
     ((5, 2, 23), [4]),                    # 1-D
     ((2, 2, 5, 6, 9), [3, 2, 2]),         # 3-D
     ((1, 2, 3, 5, 4, 7), [2, 2, 2, 1]),   # 4-D, a window of 1 in one dimension
-    ((4, 8, 28, 28), [2, 2]),
+    ((4, 8, 28, 28), [2, 2]),             # four planes of an entry per workgroup, one run per grid
+    ((2, 6, 30, 30), [2, 2]),             # three of six
+    ((3, 4, 21, 19), [3, 2]),             # planes of an odd number of floats: staged from an unaligned start
+    ((5, 12, 56, 56), [2, 2]),            # one plane per workgroup, neighbouring planes on one die
     ((2, 1, 3, 3), [1, 1]),               # one tile: plain copy
     ((7, 37, 6, 5), [2, 2]),              # 259 small planes: 256 in the first workgroup, 3 in the second
     ((1, 2, 200, 300), [3, 2]),           # bands of a large plane
@@ -348,6 +351,7 @@ def test_max_subsampling_where_the_first_zero_decides(gpu, shape, windows, strid
 
 @pytest.mark.parametrize("is_min", [False, True])
 @pytest.mark.parametrize("shape,windows", [((4, 16, 112, 112), [2, 2]), ((1, 3, 100, 96), [2, 2]), ((2, 3, 60, 60), [3, 3]), ((7, 37, 6, 5), [2, 2]),
+                                           ((4, 8, 28, 28), [2, 2]), ((3, 4, 21, 19), [3, 2]),
                                            ((3, 4, 9, 11), [2, 3]), ((5, 2, 23), [4])])
 def test_max_subsampling_with_tiling_where_the_first_zero_decides(gpu, shape, windows, is_min):
     x = zero_heavy(T.rng(72, sum(shape)), shape)
