@@ -239,8 +239,12 @@ namespace nnf
 		constexpr int linear_waves = 4;
 		constexpr size_t linear_lds_bytes_max = 64 * 1024;
 
+		// (Four wavefronts per SIMD for every instance: 64 x 2048 planes are 1024 workgroups, which 256 compute units hold all
+		// at once at four each - every load of the launch is then requested in its first microsecond. The instance with two
+		// inputs and no expf took 132 registers, three workgroups per compute unit and a second round for the last quarter;
+		// with two inputs and expf it takes 152 and would spill 45 of them, so that one stays at three.)
 		template<bool PROLOGUE, bool EXP, bool JOIN>
-		__global__ void __launch_bounds__(linear_waves * wave_size) global_pool_linear_kernel(float* out, const float* in, const float* in2,
+		__global__ void __launch_bounds__(linear_waves * wave_size) __attribute__((amdgpu_waves_per_eu((EXP && JOIN) ? 3 : 4))) global_pool_linear_kernel(float* out, const float* in, const float* in2,
 			uint32_t plane_count, uint32_t plane, uint32_t plane_magic, float mult, const window_prologue pro)
 		{
 			extern __shared__ __align__(16) float lds_planes[];

@@ -330,7 +330,8 @@ namespace nnf
 		// pooling: 20.3 M vector instructions per launch with the loop, of which the two layers need a third). As a second
 		// path beside the loop in one kernel the straight code costs that kernel 40 spilled registers, hence kernels of its own:
 		// the pooling kernels have them for the first group (44.2 -> 42.1 us on those planes); the whole-plane average with the
-		// second group folded in does not wait for its vector instructions (14.1 us either way) and keeps the loop.
+		// second group folded in gains nothing from it (13.3 us with the loop, 13.4 - 13.6 us with straight code on 64 x 2048
+		// planes of 7 x 7, all loads of a wavefront in one round or in two) and keeps the loop.
 		constexpr int known_group_none = 0;
 		constexpr int known_group_batch_norm_relu = 1;
 		constexpr int known_group_batch_norm_shortcut_add_relu = 2;
