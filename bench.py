@@ -1053,14 +1053,16 @@ def main():
     cpu = None
     if not args.only:
         side_steps = {"config0": (200, 20), "config1": (400, 40), "config2": (20, 3), "config3": (60, 6), "config4": (10, 3)}
-        for name in ("config0", "config1", "config2", "config3", "config4"):
+        for number, name in enumerate(("config0", "config1", "config2", "config3", "config4")):
             if name not in per_config:
                 per_config[name] = run(name, *side_steps[name])
                 annotate(name, per_config[name])
-        # the product driver's own timing of configurations 0 to 3 beside the C ABI figures (config 4 is timed through it anyway)
-        for number, name in enumerate(("config0", "config1", "config2", "config3")):
-            k, wu = side_steps[name] if name != args.workload else (args.steps, args.warmup)
-            per_config[name]["through_driver"] = bench_through_driver(runner, number, per_config[name], k, wu)
+            # the product driver's own timing of configurations 0 to 3 right behind the C ABI figure it is compared with (the
+            # device's clocks drift over a run of this script: measured minutes apart the two differ by 3 %, alternating in one
+            # process by under 1 %); config 4 is timed through the driver anyway
+            if number < 4:
+                k, wu = side_steps[name] if name != args.workload else (args.steps, args.warmup)
+                per_config[name]["through_driver"] = bench_through_driver(runner, number, per_config[name], k, wu)
         per_config["copy_kernel"] = bench_copy(runner, 40, 5)
         # the neighbouring layers of the same chains
         for name, (k, wu) in (("global_average", (100, 10)), ("joined_global_average", (100, 10)), ("max_subsampling", (40, 5)), ("bn_relu_max_subsampling", (40, 5)),
