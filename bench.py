@@ -41,7 +41,7 @@ MEASURED_TRAFFIC_BYTES = {
     "config2": 1233228800,  # algorithmic 1,233,130,496
     "config3": 205650944,   # algorithmic 205,529,088
     "config1": 2117540,     # algorithmic 2,048,000 (profiles/softmax_and_resnet50_stack.md)
-    "max_subsampling_tiling": 402617602,  # algorithmic 403,767,296 (profiles/tiling_and_entry_window_kernels.md)
+    "max_subsampling_tiling": 405866496,  # algorithmic 403,767,296 (profiles/tiling_and_entry_window_kernels.md)
     "entry_window": 256931085,            # algorithmic 256,901,120
     "config4": 6313391834,  # per pass of the launch plan through the driver (50 plan steps in 8 kernel launches: independent groups
                             # share launches, the last group is applied by the average's kernel and neither written nor read
@@ -115,7 +115,7 @@ class Runner:
         self.torch.cuda.synchronize()
 
     def config3_input(self, count):
-        """x ~ N(0, 2) (variance) with 0.1 % of the entries at +-50, as BASELINE.json states config 3."""
+        """x ~ N(0, 2) (variance) with 0.1 % of the entries at +-50, the benchmark's configuration 3."""
         t = self.randn(count, 2.0 ** 0.5)
         spikes = self.torch.rand(count, generator=self.gen, device=self.device) < 0.001
         signs = self.torch.rand(count, generator=self.gen, device=self.device) < 0.5
@@ -782,7 +782,7 @@ def cpu_baseline_config0(runner, group, seconds=8.0):
 class CpuPlainBackend:
     """nnForge's plain backend restated in oracle/, driven the way forward_propagation_plain drives its testers: one
     OpenMP pass per layer, in place where the tester allows it. Inputs are views of one pool of random floats (the
-    values do not matter for the time; expf-heavy layers get the spread BASELINE.json states through `scale`)."""
+    values do not matter for the time; expf-heavy layers get the spread the benchmark's configurations state through `scale`)."""
 
     def __init__(self, max_elements):
         import oracle
@@ -976,7 +976,7 @@ def main():
                              "global_average", "joined_global_average", "inception_block", "inception_block_copies"],
                     help="'copy' times the plain copy kernel (profiler-counter calibration and bandwidth yardstick); 'yardsticks' the runtime's and "
                          "torch's copy routines beside the library's kernels; 'config4_direct' the launches of config4 issued at the C ABI from this script")
-    ap.add_argument("--entries", type=int, default=64, help="config4: entries per packet (BASELINE.json's configuration has 64)")
+    ap.add_argument("--entries", type=int, default=64, help="config4: entries per packet (the benchmark's configuration has 64)")
     ap.add_argument("--one-launch-per-group", action="store_true", help="config4: switch the driver's hip_batch_independent_groups off")
     ap.add_argument("--kernel-streams", type=int, default=0, help="config4: kernel streams of the driver (hip_kernel_stream_count); 0 = its default")
     ap.add_argument("--replay-recorded-plan", action="store_true", help="config4: the timed passes replay a HIP graph recorded from the plan's launches")

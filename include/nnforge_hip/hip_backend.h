@@ -96,7 +96,8 @@ namespace nnforge
 			// 8 entries 243 -> 172 us.
 			bool batch_independent_groups;
 			// A fused group that only a Concat layer reads writes its result into that layer's output instead of a
-			// tensor of its own that the Concat would copy (measured in DESIGN.md); switch off to have every Concat copy
+			// tensor of its own that the Concat would copy (four branches of 64 + 128 + 32 + 32 maps of 28 x 28 at 128 entries:
+			// 37 us against 75 us); switch off to have every Concat copy
 			bool concat_in_place = true;
 			unsigned int reserved_thread_count;
 			// run() makes its packets no larger than this much pinned staging (input + output entries) per I/O slot, so that

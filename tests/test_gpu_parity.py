@@ -1,6 +1,6 @@
 """GPU parity: the HIP kernels, called through the C ABI, against the CPU oracle on identical seeded inputs.
 
-Bars (BASELINE north_star): batch norm and element-wise layers within max(2 ULP, 1e-6 relative) of
+Bars: batch norm and element-wise layers within max(2 ULP, 1e-6 relative) of
 the plain CPU tester; softmax within 1e-5 relative. On top of that the tests demand what the
 design promises: bit-for-bit equality wherever the operation order is the reference's own (every
 kernel except the row softmax, whose sum is a tree instead of a left-to-right loop).
