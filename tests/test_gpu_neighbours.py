@@ -685,3 +685,69 @@ def test_subsampling_that_cannot_fold_a_group_in_says_so(gpu):
     assert call(gpu.stream, out.data_ptr(), x.data_ptr(), ctypes.byref(two), chk, *shape_args) == 0
     assert call(gpu.stream, out.data_ptr(), x.data_ptr(), ctypes.byref(three), chk, *shape_args) == capi.E_UNSUPPORTED
     gpu.torch.cuda.synchronize()
+
+
+class Guarded:
+    """An output of `count` floats with 256 sentinel floats on either side of it (the inner pointer keeps the 1 KB
+    alignment of the allocation): a kernel that stores in front of its output or behind it changes a sentinel."""
+
+    margin = 256
+    sentinel = F(-123456.0)
+
+    def __init__(self, gpu, count):
+        self.gpu, self.count = gpu, count
+        self.whole = gpu.torch.full((count + 2 * self.margin,), float(self.sentinel), dtype=gpu.torch.float32, device=gpu.device)
+        self.ptr = self.whole.data_ptr() + 4 * self.margin
+
+    def check(self, want, what):
+        host = self.gpu.to_host(self.whole, (self.count + 2 * self.margin,))
+        assert np.all(host[:self.margin] == self.sentinel), what + ": stores in front of the output"
+        assert np.all(host[self.margin + self.count:] == self.sentinel), what + ": stores behind the output"
+        assert T.bit_mismatches(host[self.margin:self.margin + self.count].reshape(want.shape), want) == 0, what
+
+
+@pytest.mark.parametrize("shape,windows", [
+    ((2, 5, 112, 112), [2, 2]), ((1, 3, 100, 96), [2, 2]), ((4, 8, 28, 28), [2, 2]), ((3, 4, 21, 19), [3, 2]), ((7, 37, 6, 5), [2, 2]),
+    ((5, 12, 56, 56), [2, 2]), ((2, 3, 57, 57), [3, 3]), ((1, 2, 200, 300), [3, 2]), ((5, 2, 23), [4]), ((1, 1, 5000, 4), [2, 2])])
+def test_tiling_kernels_store_nothing_outside_their_output(gpu, shape, windows):
+    """Every way the tiling kernel leaves its results - runs of bands, runs of whole planes (one or several to a workgroup),
+    stores from the scan loop - with the output between sentinels: the runs' scalar heads and tails stop where the output does."""
+    x = spiced(T.rng(90, sum(shape)), shape)
+    want = oracle.max_subsampling(x, windows, tiling=True)
+    dims = list(shape[2:])[::-1]
+    out = Guarded(gpu, want.size)
+    rc = gpu.lib.nnf_hip_max_subsampling_tiling_forward(gpu.stream, out.ptr, gpu.to_device(x).data_ptr(), shape[0], shape[1], len(dims), u32(dims), u32(windows), 0)
+    assert rc == 0, capi.error_string(rc)
+    out.check(want, "tiling %r %r" % (shape, windows))
+
+
+@pytest.mark.parametrize("shape,windows,strides,round_ups", [
+    ((3, 5, 112, 112), [3, 3], [2, 2], [True, True]), ((2, 7, 55, 55), [3, 3], [2, 2], None), ((5, 3, 28, 28), [2, 2], None, None),
+    ((7, 5, 13, 13), [3, 3], [2, 2], [True, True]), ((6, 5, 10, 12), [3, 3], [2, 2], [True, True]), ((1, 3, 4, 4000), [3, 2], [2, 2], None)])
+def test_pooling_kernels_store_nothing_outside_their_output(gpu, shape, windows, strides, round_ups):
+    """The staged pooling kernels - alone, and with BatchNorm -> ReLU folded in (the kernel of its own for one plane per
+    workgroup and the general one) - with the output between sentinels."""
+    gen = T.rng(91, sum(shape))
+    x = spiced(gen, shape)
+    dims = list(shape[2:])[::-1]
+    want = oracle.max_subsampling(x, windows, strides=strides, round_ups=round_ups)
+    out = Guarded(gpu, want.size)
+    d_in = gpu.to_device(x)
+    args = (shape[0], shape[1], len(dims), u32(dims), u32(windows), u32(strides) if strides else None,
+            u32([int(r) for r in round_ups]) if round_ups else None, 1, 1, 0)
+    rc = gpu.lib.nnf_hip_max_subsampling_forward(gpu.stream, out.ptr, d_in.data_ptr(), *args)
+    assert rc == 0, capi.error_string(rc)
+    out.check(want, "pooling %r" % (shape,))
+    # the same with BatchNorm -> ReLU in front (values without NaN: ReLU of NaN is the reference's own matter)
+    c = shape[1]
+    y = T.normal(gen, shape, 2.0)
+    gamma, beta, mean, inv_sigma = T.bn_params(gen, c)
+    chunks = [gpu.to_device(a) for a in (gamma, beta, mean, inv_sigma)]
+    chk = capi.pointer_array([t.data_ptr() for t in chunks])
+    desc = capi.make_desc(shape[0], c, int(np.prod(dims)), [[(capi.OP_BATCH_NORM, 0), (capi.OP_RELU, 0, 0.0)]], [])
+    staged = oracle.rectified_linear(oracle.batch_norm(y.reshape(shape[0], c, -1), gamma, beta, mean, inv_sigma)).reshape(shape)
+    want = oracle.max_subsampling(staged, windows, strides=strides, round_ups=round_ups)
+    out = Guarded(gpu, want.size)
+    rc = gpu.lib.nnf_hip_max_subsampling_fused_forward(gpu.stream, out.ptr, gpu.to_device(y).data_ptr(), ctypes.byref(desc), chk, *args)
+    assert rc == 0, capi.error_string(rc)
+    out.check(want, "BatchNorm -> ReLU -> pooling %r" % (shape,))
