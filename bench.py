@@ -1108,7 +1108,7 @@ def main():
             "queued_achieved": main_entry.get("queued_event_gbps"),
             "queued_frac": (main_entry["queued_event_gbps"] / HBM_PEAK_GBPS) if main_entry.get("queued_event_gbps") else None,
             "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
-            "kernel": {"config1": "nnf::softmax_rows_kernel", "copy": "nnf::copy_kernel_impl", "max_subsampling": "nnf::max_window2d_kernel", "bn_relu_max_subsampling": "nnf::max_window2d_prologue_kernel",
+            "kernel": {"config1": "nnf::softmax_rows_kernel", "copy": "nnf::copy_kernel_impl", "max_subsampling": "nnf::max_window2d_kernel", "bn_relu_max_subsampling": "nnf::max_window2d_bn_relu_kernel",
                        "max_subsampling_tiling": "nnf::tiling2d_kernel", "entry_window": "nnf::window_rows_kernel",
                        "concat": "nnf::concat_kernel", "maxout": "nnf::maxout_vec4_kernel",
                        "feature_map_stat": "nnf::stat_runs_kernel", "walking_grid": "nnf::chain_kernel_persistent",
