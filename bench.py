@@ -278,6 +278,14 @@ def bench_group(runner, label, group, steps, warmup, make_input=None, overlapped
         launch = runner.prepare_group(group, 1, make_input)
         hot = time_steps_queued(runner, launch, min(max(steps, 50), 400), hold_ms=8.0)
         extra.update({"cache_hot_event_ms_per_step": hot * 1e3, "cache_hot_event_gbps": alg / hot / 1e9})
+    if alg >= (768 << 20):
+        # One buffer set alone is several times the last-level cache: the same launch on one set over and over, which is what
+        # the driver does with a resident packet. Faster than going round two sets by 2 to 3.5 us per launch whatever the size
+        # (1.23 / 2.47 / 3.70 GB per set: 188.6 against 192.3, 388.0 against 390.1, 585.4 against 588.0 us) - reported beside
+        # the rotating figure, which stays the configuration's.
+        _, one_set = runner.time_steps(lambda i: launch(0), steps, warmup)
+        extra.update({"one_buffer_set_event_ms_per_step": one_set * 1e3, "one_buffer_set_event_gbps": alg / one_set / 1e9,
+                      "one_buffer_set_pct_of_hbm_peak": 100.0 * alg / one_set / 1e9 / HBM_PEAK_GBPS})
     entry = result_entry(label, alg, w.group_elements(group), wall, ev, 1, extra)
     del launch
     runner.torch.cuda.empty_cache()
