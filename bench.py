@@ -280,9 +280,9 @@ def bench_group(runner, label, group, steps, warmup, make_input=None, overlapped
         extra.update({"cache_hot_event_ms_per_step": hot * 1e3, "cache_hot_event_gbps": alg / hot / 1e9})
     if alg >= (768 << 20):
         # One buffer set alone is several times the last-level cache: the same launch on one set over and over, which is what
-        # the driver does with a resident packet. Faster than going round two sets by 2 to 3.5 us per launch whatever the size
-        # (1.23 / 2.47 / 3.70 GB per set: 188.6 against 192.3, 388.0 against 390.1, 585.4 against 588.0 us) - reported beside
-        # the rotating figure, which stays the configuration's.
+        # the driver does with a resident packet - reported beside the rotating figure, which stays the configuration's. (In a
+        # process of its own one set came out 2 to 3.5 us per launch ahead at 1.23, 2.47 and 3.70 GB per set; at the end of this
+        # script's survey it has also come out 2 us behind: where the allocations lie matters more than how many there are.)
         _, one_set = runner.time_steps(lambda i: launch(0), steps, warmup)
         extra.update({"one_buffer_set_event_ms_per_step": one_set * 1e3, "one_buffer_set_event_gbps": alg / one_set / 1e9,
                       "one_buffer_set_pct_of_hbm_peak": 100.0 * alg / one_set / 1e9 / HBM_PEAK_GBPS})
