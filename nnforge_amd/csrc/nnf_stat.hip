@@ -23,10 +23,10 @@ namespace nnf
 	{
 		constexpr int stat_block_size = 256;
 		constexpr int stat_unroll = 4;                    // loads a lane has in flight
-		// Workgroups of this kernel an MI355X holds at once: 256 compute units x 7 workgroups of 256
-		// lanes (the kernel needs 70 vector registers, which leaves room for 7 wavefronts per SIMD).
+		// Workgroups of this kernel an MI355X holds at once: 256 compute units x 8 workgroups of 256
+		// lanes (the kernel needs 32 vector registers: 8 wavefronts per SIMD).
 		// The grid is cut so that it fills whole rounds of that many.
-		constexpr uint32_t stat_resident_blocks = 1792;
+		constexpr uint32_t stat_resident_blocks = 2048;
 		// what starting and finishing a workgroup costs, in floats of streaming (wavefront and LDS
 		// reductions, the partial state)
 		constexpr uint64_t stat_block_overhead_floats = 8192;
