@@ -575,7 +575,7 @@ namespace nnf
 
 		// One plane per workgroup, BatchNorm -> ReLU in front of the windows: the layers as straight code
 		template<int OP, int WIN_W, int WIN_H, bool TRUNC, bool PAIR = false>
-		__global__ void __launch_bounds__(max_block_size) __attribute__((amdgpu_waves_per_eu(6, 6))) max_window2d_bn_relu_kernel(const window2d_args a, const window_prologue pro)
+		__global__ void __launch_bounds__(max_block_size) __attribute__((amdgpu_waves_per_eu(6))) max_window2d_bn_relu_kernel(const window2d_args a, const window_prologue pro)
 		{
 			window2d_body<OP, WIN_W, WIN_H, TRUNC, true, false, true, PAIR, true>(a, pro);
 		}
