@@ -105,6 +105,34 @@ namespace nnf
 		return count;
 	}
 
+	// One round of resident workgroups whose loads are all requested in the launch's first half microsecond: memory serves
+	// a stream of reads followed by a stream of writes faster than the two mixed (a kernel that only reads gets 7.0 TB/s, one
+	// that only writes 6.8, a copy 6.1 to 6.3), so a kernel whose values are ready early keeps them in registers until the
+	// launch's reads have had their time and stores then. (Kernels that need per-feature-map weights have that wait
+	// by themselves: the weights come back behind the tensor. Measured on 25.7 MB in, 25.7 MB out: a copy of four inputs
+	// 10.0 -> 9.5 us (12.8 MB: 7.2 -> 6.7 us, 19.3 MB: 8.3 -> 7.6 us); a bare BatchNorm -> ReLU 10.5 -> 8.9 us; held 20 % longer
+	// than needed: + 2.5 %. The fused-group kernel does not use it: the few instructions it takes there cost the groups that
+	// do not need it 4 to 13 %.)
+	// -> 10 ns ticks from a workgroup's start to its first store, 0 when the launch is not of that kind.
+	inline uint32_t read_phase_ticks(uint64_t workgroups, uint32_t workgroups_per_compute_unit, uint64_t bytes_read)
+	{
+		constexpr uint64_t least_bytes = 12u << 20;       // below this a launch is over before a wait could pay (9.6 MB: a loss)
+		constexpr uint64_t bytes_per_tick = 68000;        // 6.8 TB/s
+		constexpr uint32_t start_ticks = 30;              // the workgroups of a launch start within 0.3 to 0.5 us
+		if ((workgroups > static_cast<uint64_t>(workgroups_per_compute_unit) * compute_unit_count()) || (bytes_read < least_bytes))
+			return 0;
+		return start_ticks + static_cast<uint32_t>(bytes_read / bytes_per_tick);
+	}
+
+#ifdef __HIPCC__
+	// started: wall_clock64() at the workgroup's start (100 MHz). The wait ends by the clock alone.
+	__device__ __forceinline__ void hold_until(uint64_t started, uint32_t ticks)
+	{
+		while (wall_clock64() - started < ticks)
+			__builtin_amdgcn_s_sleep(8);
+	}
+#endif
+
 	// Kernels the library has launched from the calling thread (nnf_hip_launch_count): every launch goes through NNF_LAUNCH.
 	inline uint64_t& launches_of_this_thread()
 	{

@@ -23,6 +23,7 @@ namespace nnf
 			uint32_t input_count;
 			uint32_t output_length;                  // neurons per output entry
 			uint32_t entry_count;
+			uint32_t hold_ticks;                     // stores wait until this many 10 ns ticks after the workgroup's start (0: no wait)
 		};
 
 		// VEC: floats per access; 4 when every length is a multiple of 4 (then every offset is as well)
@@ -35,6 +36,7 @@ namespace nnf
 				++i;
 			const uint32_t tile = (blockIdx.x - a.first_block[i]) * (concat_block_size * concat_unroll * VEC);
 			const uint32_t length = a.length[i];
+			const uint64_t started = (a.hold_ticks != 0) ? wall_clock64() : 0;
 			for(uint32_t entry = blockIdx.y; entry < a.entry_count; entry += gridDim.y)
 			{
 				const float* src = a.in[i] + static_cast<size_t>(entry) * length;
@@ -49,6 +51,14 @@ namespace nnf
 					const uint32_t r = tile + (k * concat_block_size + threadIdx.x) * VEC;
 					if (r < length)
 						v[k] = __builtin_nontemporal_load(reinterpret_cast<const vec_t*>(src + r));
+				}
+				if (a.hold_ticks != 0)
+				{
+					// the values wait in their registers until the launch's reads have had their time (read_phase_ticks)
+					#pragma unroll
+					for(int k = 0; k < concat_unroll; ++k)
+						asm volatile("" : "+v"(v[k]));
+					hold_until(started, a.hold_ticks);
 				}
 				#pragma unroll
 				for(int k = 0; k < concat_unroll; ++k)
@@ -142,6 +152,11 @@ namespace nnf
 			if (blocks == 0)
 				continue;
 			const dim3 grid(blocks, std::min(entry_count, 65535u));
+			// one round of resident workgroups: the stores wait for the launch's reads (read_phase_ticks)
+			uint64_t copied = 0;
+			for(uint32_t i = 0; i < a.input_count; ++i)
+				copied += (a.in[i] != nullptr) ? static_cast<uint64_t>(a.length[i]) * entry_count * sizeof(float) : 0;
+			a.hold_ticks = vector ? read_phase_ticks(static_cast<uint64_t>(grid.x) * grid.y, 8, copied) : 0;
 			if (vector)
 				NNF_LAUNCH(concat_kernel<4>, grid, dim3(concat_block_size), 0, stream, a);
 			else
