@@ -1118,7 +1118,7 @@ def main():
             "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
             "kernel": {"config1": "nnf::softmax_rows_kernel", "copy": "nnf::copy_kernel_impl", "max_subsampling": "nnf::max_window2d_kernel", "bn_relu_max_subsampling": "nnf::max_window2d_bn_relu_kernel",
                        "max_subsampling_tiling": "nnf::tiling2d_kernel", "entry_window": "nnf::window_rows_kernel",
-                       "concat": "nnf::concat_kernel", "maxout": "nnf::maxout_vec4_kernel",
+                       "concat": "nnf::concat_kernel", "maxout": "nnf::maxout_pairs_kernel",
                        "feature_map_stat": "nnf::stat_runs_kernel", "walking_grid": "nnf::chain_kernel_persistent",
                        "global_average": "nnf::global_pool_linear_kernel", "joined_global_average": "nnf::global_pool_linear_kernel",
                        "inception_block": "nnf::chain_entries_batch_kernel", "inception_block_copies": "nnf::chain_batch_kernel + nnf::concat_kernel",
