@@ -541,7 +541,9 @@ namespace nnf
 		// ALL_DIRECT: every group of the launch reads its weights straight from memory; ONE_INPUT: every group has one
 		// input. The launch whose groups are all of one kind holds one body instead of four and half the registers
 		// (48 against 102 per lane: four Inception branches of 512 entries 135 against 172 us).
-		template<int BLOCK, bool ALL_DIRECT, bool ONE_INPUT>
+		// U: float4s per lane - 2, or 4 for the launch of one kind whose workgroups then make one round of the machine
+		// (four branches of 32 entries, 51 MB moved: 11.7 -> 10.7 us; at 128 entries no difference, at 512 entries 3 % slower)
+		template<int BLOCK, bool ALL_DIRECT, bool ONE_INPUT, int U = 2>
 		__global__ void __launch_bounds__(BLOCK) chain_entries_batch_kernel(const chain_strided_batch_args b)
 		{
 			extern __shared__ __align__(16) unsigned char lds_raw[];
@@ -567,16 +569,16 @@ namespace nnf
 				if (two_inputs)
 				{
 					if (direct)
-						chain_tile<2, BLOCK, 2, true, 0>(v, tile_index, lds_raw);
+						chain_tile<2, BLOCK, U, true, 0>(v, tile_index, lds_raw);
 					else
-						chain_tile<2, BLOCK, 2, false, 0>(v, tile_index, lds_raw);
+						chain_tile<2, BLOCK, U, false, 0>(v, tile_index, lds_raw);
 				}
 				else
 				{
 					if (direct)
-						chain_tile<1, BLOCK, 2, true, 0>(v, tile_index, lds_raw);
+						chain_tile<1, BLOCK, U, true, 0>(v, tile_index, lds_raw);
 					else
-						chain_tile<1, BLOCK, 2, false, 0>(v, tile_index, lds_raw);
+						chain_tile<1, BLOCK, U, false, 0>(v, tile_index, lds_raw);
 				}
 				if (entry + gridDim.y < b.entry_count)
 					__syncthreads(); // the next entry's coefficients go where this one's are still being read
@@ -1150,8 +1152,10 @@ namespace nnf
 		return (rc != NNF_HIP_OK) ? rc : launch_group(stream, p);
 	}
 
-	// The launch over entries has instances for one or two inputs and 256 lanes x 2 float4s.
+	// The launch over entries has instances for one or two inputs and 256 lanes x 2 float4s, and one for groups of one
+	// input with weights straight from memory and 4 float4s.
 	constexpr int strided_shape = 1;
+	constexpr int strided_wide_shape = 0;
 
 	int chain_forward_strided_status(const nnf_hip_chain_desc* desc, uint32_t output_entry_stride)
 	{
@@ -1190,15 +1194,30 @@ namespace nnf
 		if (entry_count == 0)
 			return NNF_HIP_OK; // as the reference's loops over zero entries
 		std::vector<prepared_group> groups(group_count);
-		for(uint32_t i = 0; i < group_count; ++i)
+		// planned as groups of one entry: with the wide tiles where all groups of the call are of the one kind that has them
+		// and the launch is then one round of workgroups that still covers the machine, with the narrow ones otherwise
+		bool wide = group_count <= max_strided_batch;
+		for(;;)
 		{
-			int rc;
-			// planned as a group of one entry
-			nnf_hip_chain_desc one = descs[i];
-			one.entry_count = 1;
-			rc = prepare_group(&one, outputs[i], inputs[i], (chunk_ptrs == nullptr) ? nullptr : chunk_ptrs[i], false, groups[i], strided_shape);
-			if (rc != NNF_HIP_OK)
-				return rc;
+			uint64_t tiles = 0;
+			bool of_the_kind = true;
+			for(uint32_t i = 0; i < group_count; ++i)
+			{
+				nnf_hip_chain_desc one = descs[i];
+				one.entry_count = 1;
+				const int rc = prepare_group(&one, outputs[i], inputs[i], (chunk_ptrs == nullptr) ? nullptr : chunk_ptrs[i], false, groups[i],
+					wide ? strided_wide_shape : strided_shape);
+				if ((rc != NNF_HIP_OK) && !wide)
+					return rc;
+				of_the_kind = of_the_kind && (rc == NNF_HIP_OK) && groups[i].direct && (groups[i].input_count == 1);
+				tiles += groups[i].tiles;
+			}
+			if (!wide)
+				break;
+			const uint64_t workgroups = tiles * entry_count;
+			if (of_the_kind && (workgroups >= 2ull * compute_unit_count()) && (workgroups <= static_cast<uint64_t>(resident_workgroups_per_compute_unit) * compute_unit_count()))
+				break;
+			wide = false; // once more, with the narrow tiles
 		}
 		// What group i writes: entry_count pieces of its entry size, output_entry_strides[i] floats apart. No input of the
 		// call may lie inside the span they cover, and the pieces of two groups may not meet: either their spans are
@@ -1248,7 +1267,8 @@ namespace nnf
 			}
 			const dim3 grid(tiles, std::min(entry_count, 65535u)), block(launch_shapes[strided_shape].block);
 			const bool all_direct = b.direct_mask == ((1u << b.count) - 1u), one_input = b.two_input_mask == 0;
-			if (all_direct && one_input) NNF_LAUNCH((chain_entries_batch_kernel<256, true, true>), grid, block, lds_bytes, stream, b);
+			if (wide) NNF_LAUNCH((chain_entries_batch_kernel<256, true, true, 4>), grid, block, lds_bytes, stream, b);
+			else if (all_direct && one_input) NNF_LAUNCH((chain_entries_batch_kernel<256, true, true>), grid, block, lds_bytes, stream, b);
 			else if (all_direct) NNF_LAUNCH((chain_entries_batch_kernel<256, true, false>), grid, block, lds_bytes, stream, b);
 			else if (one_input) NNF_LAUNCH((chain_entries_batch_kernel<256, false, true>), grid, block, lds_bytes, stream, b);
 			else NNF_LAUNCH((chain_entries_batch_kernel<256, false, false>), grid, block, lds_bytes, stream, b);
