@@ -9,6 +9,7 @@
 
 #include <algorithm>
 #include <cstdlib>
+#include <type_traits>
 
 namespace nnf
 {
@@ -235,6 +236,11 @@ namespace nnf
 		// Measured on 64 x 2048 x 7 x 7 (25.7 MB): 6.2 us against 8.9 us for the kernel above; 64 planes per wavefront 6.8 us,
 		// all thirteen float4s of a lane loaded before the first LDS store 9.0 us (all seven of 32 planes: 6.3 us, no change). With BatchNorm + ReLU folded in 8.9 us, with a
 		// joined block 14.0 us (16 planes per wavefront: 9.8 and 14.5 us; 64: 10.3 and 13.2 us).
+		// GROUP: the folded layers are one of the groups of nnf_prologue.h's apply_known_group, compiled as straight code
+		// (68 registers per lane instead of 127), with rounds of two float4s per lane and input and the next round requested
+		// before the layers are applied to this one. Same shape: BatchNorm -> ReLU folded in 8.6 -> 7.2 us, the joined
+		// block 13.2 -> 10.8 us (128 entries: 21.7 -> 18.1 us; 32 x 1024 planes of 11 x 11: 12.6 -> 8.8 us). Rounds of
+		// one, three and four float4s: 10.8 / 11.7 / 11.7 us for the joined block, 7.4 / 8.1 / 7.6 us for BatchNorm -> ReLU.
 		constexpr uint32_t linear_planes_per_wave = 32;
 		constexpr int linear_waves = 4;
 		constexpr size_t linear_lds_bytes_max = 64 * 1024;
@@ -243,7 +249,7 @@ namespace nnf
 		// at once at four each - every load of the launch is then requested in its first microsecond. The instance with two
 		// inputs and no expf took 132 registers, three workgroups per compute unit and a second round for the last quarter;
 		// with two inputs and expf it takes 152 and would spill 45 of them, so that one stays at three.)
-		template<bool PROLOGUE, bool EXP, bool JOIN>
+		template<bool PROLOGUE, bool EXP, bool JOIN, int GROUP = known_group_none>
 		__global__ void __launch_bounds__(linear_waves * wave_size) __attribute__((amdgpu_waves_per_eu((EXP && JOIN) ? 3 : 4))) global_pool_linear_kernel(float* out, const float* in, const float* in2,
 			uint32_t plane_count, uint32_t plane, uint32_t plane_magic, float mult, const window_prologue pro)
 		{
@@ -292,10 +298,11 @@ namespace nnf
 			exp_context exp_ctx = make_exp_context(lds_exp);
 
 			const uint32_t vectors = floats_here / 4;
-			constexpr int stage = 4;
-			for(uint32_t base = 0; base < vectors; base += stage * wave_size)
+			constexpr int stage = (GROUP != known_group_none) ? 2 : 4; // float4s per lane, input and round
+			constexpr uint32_t step = stage * wave_size;
+			// a round of a lane's float4s: requested ...
+			auto request = [&](floatx4 (&t)[stage], floatx4 (&t2)[stage], const uint32_t base)
 			{
-				floatx4 t[stage], t2[stage];
 				#pragma unroll
 				for(int k = 0; k < stage; ++k)
 				{
@@ -305,41 +312,46 @@ namespace nnf
 					if (JOIN)
 						t2[k] = load_stream(reinterpret_cast<const floatx4*>(src2) + i);
 				}
+			};
+			// the coefficient table and the expf table of this wavefront, while the first loads are in flight
+			auto prepare_tables = [&]()
+			{
+				#pragma unroll
+				for(uint32_t j = 0; j < prologue_weighted_max; ++j)
+				{
+					#pragma unroll
+					for(int c = 0; c < 4; ++c)
+						asm volatile("" : "+v"(w[j][c])); // not looked at (nor waited for) before this point
+				}
+				#pragma unroll
+				for(uint32_t j = 0; j < prologue_weighted_max; ++j)
+				{
+					if ((j < pro.weighted_count) && (lane < planes_here))
+					{
+						float* dst = my_coef + (lane * pro.weighted_count + j) * 2;
+						if (pro.weighted_kind[j] == NNF_HIP_OP_BATCH_NORM)
+							nnf_batch_norm_coefficients(w[j][0], w[j][1], w[j][2], w[j][3], dst[0], dst[1]);
+						else
+							dst[0] = w[j][0];
+					}
+				}
+				if (EXP)
+					exp_ctx = stage_exp2_table_per_wavefront(lds_exp, exp_entry);
+				__builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+				__builtin_amdgcn_wave_barrier();
+				__builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+			};
+			// ... and the first COUNT of them taken through the layers into LDS
+			auto through_layers = [&](auto count, floatx4 (&t)[stage], floatx4 (&t2)[stage], const uint32_t base)
+			{
+				constexpr int COUNT = decltype(count)::value;
 				if (PROLOGUE)
 				{
-					if (base == 0)
-					{
-						// the coefficient table and the expf table of this wavefront, while the first loads are in flight
-						#pragma unroll
-						for(uint32_t j = 0; j < prologue_weighted_max; ++j)
-						{
-							#pragma unroll
-							for(int c = 0; c < 4; ++c)
-								asm volatile("" : "+v"(w[j][c])); // not looked at (nor waited for) before this point
-						}
-						#pragma unroll
-						for(uint32_t j = 0; j < prologue_weighted_max; ++j)
-						{
-							if ((j < pro.weighted_count) && (lane < planes_here))
-							{
-								float* dst = my_coef + (lane * pro.weighted_count + j) * 2;
-								if (pro.weighted_kind[j] == NNF_HIP_OP_BATCH_NORM)
-									nnf_batch_norm_coefficients(w[j][0], w[j][1], w[j][2], w[j][3], dst[0], dst[1]);
-								else
-									dst[0] = w[j][0];
-							}
-						}
-						if (EXP)
-							exp_ctx = stage_exp2_table_per_wavefront(lds_exp, exp_entry);
-						__builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-						__builtin_amdgcn_wave_barrier();
-						__builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-					}
-					float v[stage][4], u[stage][4];
-					uint32_t off[stage];
-					two_plane_offsets<stage> two;
+					float v[COUNT][4], u[COUNT][4];
+					uint32_t off[COUNT];
+					two_plane_offsets<COUNT> two;
 					#pragma unroll
-					for(int k = 0; k < stage; ++k)
+					for(int k = 0; k < COUNT; ++k)
 					{
 						const uint32_t i = min(base + k * wave_size + lane, vectors - 1);
 						v[k][0] = t[k].x; v[k][1] = t[k].y; v[k][2] = t[k].z; v[k][3] = t[k].w;
@@ -350,19 +362,69 @@ namespace nnf
 						two.off2[k] = min(p + 1, planes_here - 1) * coef_stride; // behind the last plane: values nobody stores
 						two.split[k] = (p + 1) * plane - i * 4;                  // >= 4: the whole float4 lies in plane p
 					}
-					apply_prologue_group<stage, EXP, JOIN, false, true>(v, u, off, my_coef, none, pro, exp_ctx, &two);
+					if (GROUP != known_group_none)
+						apply_known_group<COUNT, (GROUP != known_group_none) ? GROUP : known_group_batch_norm_relu, false, true>(v, u, off, my_coef, none, pro, exp_ctx, &two);
+					else
+						apply_prologue_group<COUNT, EXP, JOIN, false, true>(v, u, off, my_coef, none, pro, exp_ctx, &two);
 					#pragma unroll
-					for(int k = 0; k < stage; ++k)
+					for(int k = 0; k < COUNT; ++k)
 					{
 						t[k].x = v[k][0]; t[k].y = v[k][1]; t[k].z = v[k][2]; t[k].w = v[k][3];
 					}
 				}
 				#pragma unroll
-				for(int k = 0; k < stage; ++k)
+				for(int k = 0; k < COUNT; ++k)
 				{
 					const uint32_t i = base + k * wave_size + lane;
 					if (i < vectors)
 						reinterpret_cast<floatx4*>(mine)[i] = t[k];
+				}
+			};
+			auto finish = [&](floatx4 (&t)[stage], floatx4 (&t2)[stage], const uint32_t base)
+			{
+				if (PROLOGUE && (base == 0))
+					prepare_tables();
+				if (GROUP == known_group_none)
+				{
+					through_layers(std::integral_constant<int, stage>(), t, t2, base);
+					return;
+				}
+				// the wavefront's last round: only as many float4s per lane as some lane has left
+				static_assert((GROUP == known_group_none) || (stage == 2), "a round of the known groups is whole or half");
+				if (__builtin_amdgcn_readfirstlane(vectors - base) > wave_size)
+					through_layers(std::integral_constant<int, stage>(), t, t2, base);
+				else
+					through_layers(std::integral_constant<int, 1>(), t, t2, base);
+			};
+			if (GROUP != known_group_none)
+			{
+				// Two sets of registers take turns: the next round is on its way while the layers are applied to this one
+				// (every request unconditional and clamped: no join of two paths between a request and the wait for an
+				// earlier one, where the compiler would wait for everything outstanding). The request behind the last
+				// round asks for the wavefront's last float4 in every lane and is looked at by nobody.
+				floatx4 a[stage], a2[stage], b[stage], b2[stage];
+				request(a, a2, 0);
+				for(uint32_t base = 0; ; )
+				{
+					request(b, b2, base + step);
+					finish(a, a2, base);
+					base += step;
+					if (base >= vectors)
+						break;
+					request(a, a2, base + step);
+					finish(b, b2, base);
+					base += step;
+					if (base >= vectors)
+						break;
+				}
+			}
+			else
+			{
+				for(uint32_t base = 0; base < vectors; base += step)
+				{
+					floatx4 t[stage], t2[stage];
+					request(t, t2, base);
+					finish(t, t2, base);
 				}
 			}
 			// the up to three floats behind the last whole float4 (last wavefront of a plane count that is no multiple of 4)
@@ -415,8 +477,15 @@ namespace nnf
 				return;
 			}
 			auto kernel = global_pool_linear_kernel<true, false, false>;
+			const int group = known_group_of(*pro);
 			if (pro->need_exp)
 				kernel = join ? global_pool_linear_kernel<true, true, true> : global_pool_linear_kernel<true, true, false>;
+			else if (group == known_group_batch_norm_relu)
+				kernel = global_pool_linear_kernel<true, false, false, known_group_batch_norm_relu>;
+			else if (group == known_group_batch_norm_shortcut_add_relu)
+				kernel = global_pool_linear_kernel<true, false, true, known_group_batch_norm_shortcut_add_relu>;
+			else if (group == known_group_shortcut_batch_norm_add_relu)
+				kernel = global_pool_linear_kernel<true, false, true, known_group_shortcut_batch_norm_add_relu>;
 			else if (join)
 				kernel = global_pool_linear_kernel<true, false, true>;
 			NNF_LAUNCH(kernel, grid, block, lds_bytes, stream, output, input, input2, plane_count, plane, plane_magic, mult, *pro);

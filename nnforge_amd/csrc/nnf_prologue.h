@@ -329,12 +329,13 @@ namespace nnf
 		// registers and copies every one of them once per layer (64 x 64 planes of 112 x 112 through BatchNorm, ReLU and 3 x 3
 		// pooling: 20.3 M vector instructions per launch with the loop, of which the two layers need a third). As a second
 		// path beside the loop in one kernel the straight code costs that kernel 40 spilled registers, hence kernels of its own:
-		// the pooling kernels have them for the first group (44.2 -> 42.1 us on those planes); the whole-plane average with the
-		// second group folded in gains nothing from it (13.3 us with the loop, 13.4 - 13.6 us with straight code on 64 x 2048
-		// planes of 7 x 7, all loads of a wavefront in one round or in two) and keeps the loop.
+		// the pooling kernels have one for the first group (44.2 -> 42.1 us on those planes), the whole-plane average over
+		// planes of an odd size for both (64 x 2048 planes of 7 x 7 with the second group folded in: 13.2 -> 10.8 us, the
+		// registers set free going to a second round of loads in flight).
 		constexpr int known_group_none = 0;
 		constexpr int known_group_batch_norm_relu = 1;
-		constexpr int known_group_batch_norm_shortcut_add_relu = 2;
+		constexpr int known_group_batch_norm_shortcut_add_relu = 2; // BatchNorm on input 0, input 1 as it is
+		constexpr int known_group_shortcut_batch_norm_add_relu = 3; // input 0 as it is, BatchNorm on input 1
 
 		inline int known_group_of(const window_prologue& pro)
 		{
@@ -342,7 +343,9 @@ namespace nnf
 				return known_group_none;
 			if (pro.join == 0)
 				return known_group_batch_norm_relu;
-			return ((pro.arm_ops[0] == 1) && (pro.arm_ops[1] == 0)) ? known_group_batch_norm_shortcut_add_relu : known_group_none;
+			if ((pro.arm_ops[0] == 1) && (pro.arm_ops[1] == 0))
+				return known_group_batch_norm_shortcut_add_relu;
+			return ((pro.arm_ops[0] == 0) && (pro.arm_ops[1] == 1)) ? known_group_shortcut_batch_norm_add_relu : known_group_none;
 		}
 
 		template<int VECTORS, int GROUP, bool UNIFORM, bool SPLIT = false>
@@ -350,9 +353,9 @@ namespace nnf
 			const float* coef, const float (&own)[prologue_weighted_max][2], const window_prologue& pro, const exp_context& exp_ctx,
 			const two_plane_offsets<VECTORS>* two = nullptr)
 		{
-			static_assert((GROUP == known_group_batch_norm_relu) || (GROUP == known_group_batch_norm_shortcut_add_relu), "one of the known groups");
-			apply_prologue_layer<VECTORS, false, UNIFORM, SPLIT>(v, off, coef, own, exp_ctx, two, NNF_HIP_OP_BATCH_NORM, 0u, 0.0f, 0.0f);
-			if (GROUP == known_group_batch_norm_shortcut_add_relu)
+			static_assert((GROUP >= known_group_batch_norm_relu) && (GROUP <= known_group_shortcut_batch_norm_add_relu), "one of the known groups");
+			apply_prologue_layer<VECTORS, false, UNIFORM, SPLIT>((GROUP == known_group_shortcut_batch_norm_add_relu) ? u : v, off, coef, own, exp_ctx, two, NNF_HIP_OP_BATCH_NORM, 0u, 0.0f, 0.0f);
+			if (GROUP != known_group_batch_norm_relu)
 			{
 				// nnforge/plain/add_layer_tester_plain.cpp:56-59: the sum starts at 0.0F, inputs in order, times alpha
 				#pragma unroll

@@ -531,6 +531,14 @@ def run_fused_pool(gpu, x, ops, chunks, ww, wh, mult, expect=0):
     ((3, 7, 9, 9), 9, 9, "tanh_abs"),
     ((2, 3, 11, 11), 11, 11, "bn_prelu_elu_sigmoid"),  # 121 floats per plane: 62 KB of LDS per workgroup
     ((2, 5, 13, 13), 13, 13, "bn_relu"),               # 169 floats per plane: beyond that kernel, odd all the same
+    # BatchNorm -> ReLU on odd planes: straight code, rounds of two float4s per lane with the next round in flight
+    ((1, 37, 7, 7), 7, 7, "bn_relu"),                  # a wavefront with 5 planes: one round and a half, one float behind
+    ((3, 5, 7, 7), 7, 7, "bn_relu"),                   # 15 planes: 183 float4s (three rounds, the last one half) and three floats
+    ((5, 33, 5, 5), 5, 5, "bn_relu"),
+    ((3, 7, 9, 9), 9, 9, "bn_relu"),
+    ((2, 3, 11, 11), 11, 11, "bn_relu"),
+    ((1, 2, 3, 3), 3, 3, "bn_relu"),                   # 18 floats: four float4s and two floats in one wavefront
+    ((7, 96, 7, 7), 7, 7, "bn_relu"),                  # 672 planes: 21 whole wavefronts
 ])
 def test_average_subsampling_with_group_folded_in(gpu, shape, ww, wh, group):
     gen = T.rng(67, sum(shape) + ww)
@@ -559,6 +567,18 @@ JOINED_POOL_CASES = [
     ((70, 3, 3, 3), ("bn", "leaky"), 1.0, "relu"),      # 210 planes of 9 floats
     ((4, 9, 5, 5), ("-", "bn"), 0.25, "prelu"),
     ((2, 3, 11, 11), ("bn", "-"), 1.0, "relu"),         # 121 floats per plane: two staged tensors do not fit the odd-plane kernel
+    # the two residual groups compiled as straight code (BatchNorm on either input, ReLU behind the Add), ragged ends
+    ((5, 24, 7, 7), ("bn", "-"), 1.0, "relu"),
+    ((1, 37, 7, 7), ("bn", "-"), 0.5, "relu"),
+    ((3, 5, 7, 7), ("bn", "-"), 1.0, "relu"),
+    ((70, 3, 3, 3), ("bn", "-"), 1.0, "relu"),
+    ((3, 7, 9, 9), ("bn", "-"), 2.0, "relu"),
+    ((7, 96, 7, 7), ("bn", "-"), 1.0, "relu"),
+    ((1, 37, 7, 7), ("-", "bn"), 1.0, "relu"),
+    ((3, 5, 7, 7), ("-", "bn"), 0.25, "relu"),
+    ((70, 3, 3, 3), ("-", "bn"), 1.0, "relu"),
+    ((2, 5, 5, 5), ("-", "bn"), 1.0, "relu"),
+    ((1, 2, 3, 3), ("-", "bn"), 1.0, "relu"),
 ]
 
 
