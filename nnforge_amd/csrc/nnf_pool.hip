@@ -92,7 +92,12 @@ namespace nnf
 		// (planes of 49 floats): then it goes through the layers twice, once with each plane's
 		// coefficients, and every float keeps the result that is its own.
 		// JOIN: the group has two inputs (in, in2: same shape) that an Add sums after each one's own layers.
-		template<bool EXP, bool JOIN>
+		// GROUP: one of the groups of apply_known_group (nnf_prologue.h), compiled as straight code (77 to 92 registers per
+		// lane instead of 107 to 124). With the loads of a round issued without a branch around each as well: BatchNorm -> ReLU
+		// in front of the average over 64 x 2048 planes of 8 x 8 11.7 -> 8.2 us, 64 x 1024 of 14 x 14 16.6 -> 11.9 us,
+		// 256 x 1024 of 4 x 4 13.2 -> 7.7 us; the residual block (two inputs) 16.1 -> 12.8 us, 24.0 -> 19.6 us and
+		// 8.9 -> 6.6 us (256 x 512 of 4 x 4). The loads alone, any group: 16.0 -> 13.5 us and 23.9 -> 20.3 us.
+		template<bool EXP, bool JOIN, int GROUP = known_group_none>
 		__global__ void __launch_bounds__(pool_block_size) global_pool_prologue_kernel(float* out, const float* in, const float* in2, uint32_t plane_count, uint32_t plane,
 			uint32_t plane_magic, float mult, uint32_t planes_per_group, const window_prologue pro)
 		{
@@ -119,16 +124,11 @@ namespace nnf
 				#pragma unroll
 				for(int k = 0; k < stage; ++k)
 				{
-					const uint32_t i = base + k * pool_block_size + threadIdx.x;
-					t[k] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+					// no branch around a load: lanes past the end take the last float4 through the layers once more and do not stage it
+					const uint32_t i = min(base + k * pool_block_size + threadIdx.x, vectors - 1);
+					t[k] = load_stream(reinterpret_cast<const floatx4*>(src) + i);
 					if (JOIN)
-						t2[k] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
-					if (i < vectors)
-					{
-						t[k] = load_stream(reinterpret_cast<const floatx4*>(src) + i);
-						if (JOIN)
-							t2[k] = load_stream(reinterpret_cast<const floatx4*>(src2) + i);
-					}
+						t2[k] = load_stream(reinterpret_cast<const floatx4*>(src2) + i);
 				}
 				if (base == 0)
 				{
@@ -156,7 +156,10 @@ namespace nnf
 					off[k] = first_plane_of[k] * coef_stride;
 					straddles = straddles || (i * 4 + 3 >= (first_plane_of[k] + 1) * plane);
 				}
-				apply_prologue_group<stage, EXP, JOIN>(v, u, off, lds_coef, none, pro, exp_ctx);
+				if (GROUP != known_group_none)
+					apply_known_group<stage, (GROUP != known_group_none) ? GROUP : known_group_batch_norm_relu, false>(v, u, off, lds_coef, none, pro, exp_ctx);
+				else
+					apply_prologue_group<stage, EXP, JOIN>(v, u, off, lds_coef, none, pro, exp_ctx);
 				if (__any(straddles))
 				{
 					// one float4 at a time: the copies that go through the layers a second time stay few
@@ -171,7 +174,10 @@ namespace nnf
 							w2[0][0] = t2[k].x; w2[0][1] = t2[k].y; w2[0][2] = t2[k].z; w2[0][3] = t2[k].w;
 						}
 						const uint32_t next_off[1] = { min(first_plane_of[k] + 1, planes_here - 1) * coef_stride }; // beyond the last plane: not stored
-						apply_prologue_group<1, EXP, JOIN>(w, w2, next_off, lds_coef, none, pro, exp_ctx);
+						if (GROUP != known_group_none)
+							apply_known_group<1, (GROUP != known_group_none) ? GROUP : known_group_batch_norm_relu, false>(w, w2, next_off, lds_coef, none, pro, exp_ctx);
+						else
+							apply_prologue_group<1, EXP, JOIN>(w, w2, next_off, lds_coef, none, pro, exp_ctx);
 						#pragma unroll
 						for(uint32_t e = 1; e < 4; ++e)
 						{
@@ -208,7 +214,10 @@ namespace nnf
 				float one[1][4] = { { src[f], 0.0f, 0.0f, 0.0f } };
 				float one2[1][4] = { { JOIN ? src2[f] : 0.0f, 0.0f, 0.0f, 0.0f } };
 				const uint32_t one_off[1] = { p * coef_stride };
-				apply_prologue_group<1, EXP, JOIN>(one, one2, one_off, lds_coef, none, pro, exp_ctx);
+				if (GROUP != known_group_none)
+					apply_known_group<1, (GROUP != known_group_none) ? GROUP : known_group_batch_norm_relu, false>(one, one2, one_off, lds_coef, none, pro, exp_ctx);
+				else
+					apply_prologue_group<1, EXP, JOIN>(one, one2, one_off, lds_coef, none, pro, exp_ctx);
 				lds_planes[p * stride + (f - p * plane)] = one[0][0];
 			}
 			__syncthreads();
@@ -599,8 +608,15 @@ namespace nnf
 				const dim3 grid((plane_count + planes_per_group - 1) / planes_per_group);
 				const uint32_t plane_magic = static_cast<uint32_t>(((1ull << 32) + plane - 1) / plane);
 				auto kernel = global_pool_prologue_kernel<false, false>;
+				const int group = known_group_of(pro);
 				if (pro.need_exp)
 					kernel = join ? global_pool_prologue_kernel<true, true> : global_pool_prologue_kernel<true, false>;
+				else if (group == known_group_batch_norm_relu)
+					kernel = global_pool_prologue_kernel<false, false, known_group_batch_norm_relu>;
+				else if (group == known_group_batch_norm_shortcut_add_relu)
+					kernel = global_pool_prologue_kernel<false, true, known_group_batch_norm_shortcut_add_relu>;
+				else if (group == known_group_shortcut_batch_norm_add_relu)
+					kernel = global_pool_prologue_kernel<false, true, known_group_shortcut_batch_norm_add_relu>;
 				else if (join)
 					kernel = global_pool_prologue_kernel<false, true>;
 				NNF_LAUNCH(kernel, grid, dim3(pool_block_size), lds_bytes, stream, output, input, input2, plane_count, plane, plane_magic, mult, planes_per_group, pro);

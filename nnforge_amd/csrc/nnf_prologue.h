@@ -329,9 +329,9 @@ namespace nnf
 		// registers and copies every one of them once per layer (64 x 64 planes of 112 x 112 through BatchNorm, ReLU and 3 x 3
 		// pooling: 20.3 M vector instructions per launch with the loop, of which the two layers need a third). As a second
 		// path beside the loop in one kernel the straight code costs that kernel 40 spilled registers, hence kernels of its own:
-		// the pooling kernels have one for the first group (44.2 -> 42.1 us on those planes), the whole-plane average over
-		// planes of an odd size for both (64 x 2048 planes of 7 x 7 with the second group folded in: 13.2 -> 10.8 us, the
-		// registers set free going to a second round of loads in flight).
+		// the pooling kernels have one for the first group (44.2 -> 42.1 us on those planes), the whole-plane averages for
+		// both (64 x 2048 planes of 7 x 7 with the second group folded in: 13.2 -> 10.8 us, the registers set free going to
+		// a second round of loads in flight; planes of 8 x 8 with the first: 11.7 -> 8.2 us).
 		constexpr int known_group_none = 0;
 		constexpr int known_group_batch_norm_relu = 1;
 		constexpr int known_group_batch_norm_shortcut_add_relu = 2; // BatchNorm on input 0, input 1 as it is

@@ -539,6 +539,12 @@ def run_fused_pool(gpu, x, ops, chunks, ww, wh, mult, expect=0):
     ((2, 3, 11, 11), 11, 11, "bn_relu"),
     ((1, 2, 3, 3), 3, 3, "bn_relu"),                   # 18 floats: four float4s and two floats in one wavefront
     ((7, 96, 7, 7), 7, 7, "bn_relu"),                  # 672 planes: 21 whole wavefronts
+    # ... and on the planes the workgroup-wide kernel takes (even sizes, odd ones beyond 127 floats): straight code there too
+    ((9, 70, 8, 8), 8, 8, "bn_relu"),
+    ((5, 33, 14, 14), 14, 14, "bn_relu"),
+    ((3, 5, 4, 4), 4, 4, "bn_relu"),
+    ((2, 9, 6, 3), 3, 6, "bn_relu"),                   # 18 floats per plane: float4s that straddle two planes
+    ((1, 3, 2, 3), 3, 2, "bn_relu"),                   # 18 floats in all: four float4s and two floats behind them
 ])
 def test_average_subsampling_with_group_folded_in(gpu, shape, ww, wh, group):
     gen = T.rng(67, sum(shape) + ww)
@@ -579,6 +585,13 @@ JOINED_POOL_CASES = [
     ((70, 3, 3, 3), ("-", "bn"), 1.0, "relu"),
     ((2, 5, 5, 5), ("-", "bn"), 1.0, "relu"),
     ((1, 2, 3, 3), ("-", "bn"), 1.0, "relu"),
+    # ... on the planes of the workgroup-wide kernel
+    ((9, 70, 8, 8), ("bn", "-"), 1.0, "relu"),
+    ((5, 33, 14, 14), ("-", "bn"), 1.0, "relu"),
+    ((3, 5, 4, 4), ("bn", "-"), 0.5, "relu"),
+    ((2, 7, 15, 15), ("-", "bn"), 1.0, "relu"),         # 225 floats per plane, float4s that straddle two planes
+    ((2, 9, 3, 6), ("bn", "-"), 1.0, "relu"),
+    ((1, 3, 2, 3), ("-", "bn"), 2.0, "relu"),
 ]
 
 
