@@ -326,7 +326,7 @@ namespace nnf
 							straddling |= 1u << k;
 					}
 					if (BN_RELU)
-						apply_known_group<COUNT, known_group_batch_norm_relu, true>(v, v, off, lds_coef, own_coef, pro, exp_ctx);
+						apply_known_group<COUNT, known_group_batch_norm_relu, UNIFORM>(v, v, off, lds_coef, own_coef, pro, exp_ctx);
 					else if (uniform)
 						apply_prologue<COUNT, EXP, true>(v, off, lds_coef, own_coef, pro, exp_ctx, 0, pro.op_count);
 					else
@@ -349,7 +349,10 @@ namespace nnf
 							w[0][e] = (mine && (e >= split) && (g < a.total_in)) ? a.in[g] : 0.0f;
 						}
 						const uint32_t off_next[1] = { p_next * (2 * pro.weighted_count) };
-						apply_prologue<1, EXP, false>(w, off_next, lds_coef, own_coef, pro, exp_ctx, 0, pro.op_count);
+						if (BN_RELU)
+							apply_known_group<1, known_group_batch_norm_relu, false>(w, w, off_next, lds_coef, own_coef, pro, exp_ctx);
+						else
+							apply_prologue<1, EXP, false>(w, off_next, lds_coef, own_coef, pro, exp_ctx, 0, pro.op_count);
 						#pragma unroll
 						for(int k = 0; k < COUNT; ++k)
 						{
@@ -573,11 +576,12 @@ namespace nnf
 			window2d_body<OP, WIN_W, WIN_H, TRUNC, true, false, UNIFORM, PAIR>(a, pro);
 		}
 
-		// One plane per workgroup, BatchNorm -> ReLU in front of the windows: the layers as straight code
-		template<int OP, int WIN_W, int WIN_H, bool TRUNC, bool PAIR = false>
-		__global__ void __launch_bounds__(max_block_size) __attribute__((amdgpu_waves_per_eu(6))) max_window2d_bn_relu_kernel(const window2d_args a, const window_prologue pro)
+		// BatchNorm -> ReLU in front of the windows: the layers as straight code (several planes per workgroup: 96 registers
+		// either way; 64 x 256 planes of 27 x 27 20.9 -> 19.3 us, 64 x 128 of 28 x 28 10.2 -> 9.5 us)
+		template<int OP, int WIN_W, int WIN_H, bool TRUNC, bool PAIR = false, bool UNIFORM = true>
+		__global__ void __launch_bounds__(max_block_size) __attribute__((amdgpu_waves_per_eu(UNIFORM ? 6 : 4))) max_window2d_bn_relu_kernel(const window2d_args a, const window_prologue pro)
 		{
-			window2d_body<OP, WIN_W, WIN_H, TRUNC, true, false, true, PAIR, true>(a, pro);
+			window2d_body<OP, WIN_W, WIN_H, TRUNC, true, false, UNIFORM, PAIR, true>(a, pro);
 		}
 
 		template<int OP, int WIN_W, int WIN_H, bool TRUNC, bool UNIFORM>
@@ -1366,14 +1370,14 @@ namespace nnf
 				else if (w2) NNF_LAUNCH((max_window2d_exp_prologue_kernel<OP, 2, 2, TRUNC, UNIFORM>), g, b, lds_bytes, stream, a, pro);
 				else NNF_LAUNCH((max_window2d_exp_prologue_kernel<OP, 0, 0, TRUNC, UNIFORM>), g, b, lds_bytes, stream, a, pro);
 			}
-			else if (UNIFORM && (known_group_of(pro) == known_group_batch_norm_relu))
+			else if (known_group_of(pro) == known_group_batch_norm_relu)
 			{
 				const bool pair = pairs_of_outputs(a);
-				if (w3 && pair) NNF_LAUNCH((max_window2d_bn_relu_kernel<OP, 3, 3, TRUNC, true>), g, b, lds_bytes, stream, a, pro);
-				else if (w2 && pair) NNF_LAUNCH((max_window2d_bn_relu_kernel<OP, 2, 2, TRUNC, true>), g, b, lds_bytes, stream, a, pro);
-				else if (w3) NNF_LAUNCH((max_window2d_bn_relu_kernel<OP, 3, 3, TRUNC>), g, b, lds_bytes, stream, a, pro);
-				else if (w2) NNF_LAUNCH((max_window2d_bn_relu_kernel<OP, 2, 2, TRUNC>), g, b, lds_bytes, stream, a, pro);
-				else NNF_LAUNCH((max_window2d_bn_relu_kernel<OP, 0, 0, TRUNC>), g, b, lds_bytes, stream, a, pro);
+				if (w3 && pair) NNF_LAUNCH((max_window2d_bn_relu_kernel<OP, 3, 3, TRUNC, true, UNIFORM>), g, b, lds_bytes, stream, a, pro);
+				else if (w2 && pair) NNF_LAUNCH((max_window2d_bn_relu_kernel<OP, 2, 2, TRUNC, true, UNIFORM>), g, b, lds_bytes, stream, a, pro);
+				else if (w3) NNF_LAUNCH((max_window2d_bn_relu_kernel<OP, 3, 3, TRUNC, false, UNIFORM>), g, b, lds_bytes, stream, a, pro);
+				else if (w2) NNF_LAUNCH((max_window2d_bn_relu_kernel<OP, 2, 2, TRUNC, false, UNIFORM>), g, b, lds_bytes, stream, a, pro);
+				else NNF_LAUNCH((max_window2d_bn_relu_kernel<OP, 0, 0, TRUNC, false, UNIFORM>), g, b, lds_bytes, stream, a, pro);
 			}
 			else
 			{
@@ -1493,6 +1497,12 @@ namespace nnf
 				return false;
 			// the planes of a workgroup keep their coefficients in LDS
 			a.planes = std::min(a.planes, std::min(prologue_planes_max, prologue_coef_floats / (2 * prologue_weighted_max)));
+			// Layers with weights over planes this large: one plane per workgroup, whose coefficients come through the scalar
+			// cache into registers - no table in LDS, no barrier in front of the layers, no float4 between two planes
+			// (BatchNorm -> ReLU -> 3 x 3 every 2 on 64 x 96 planes of 55 x 55: 24.7 -> 20.5 us, of 51 x 51 22.0 -> 17.8 us,
+			// 2 x 2 on 56 x 56 14.0 -> 13.2 us; 64 x 128 planes of 40 x 40 the other way, 15.3 -> 17.8 us, 35 x 35 22.0 -> 23.9 us).
+			if ((a.planes > 1) && (pro.weighted_count != 0) && (plane >= (((plane & 3u) != 0) ? 2000u : 2304u)))
+				a.planes = 1;
 		}
 		if (plan_only)
 			return true;

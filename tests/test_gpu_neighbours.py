@@ -420,6 +420,17 @@ FUSED_MAX_CASES = [
     ((2, 3, 112, 112), [3, 3], [2, 2], None, "prelu_bn"),
     ((2, 2, 300, 200), [4, 7], [4, 5], None, "leaky"),
     ((1, 3, 4, 4000), [3, 2], [2, 2], None, "bn_relu"),                # one output row per band
+    # BatchNorm -> ReLU as straight code with several planes per workgroup (coefficients in LDS, float4s between planes) ...
+    ((5, 12, 27, 27), [3, 3], [2, 2], [True, True], "bn_relu"),
+    ((3, 10, 35, 35), [3, 3], [2, 2], [True, True], "bn_relu"),
+    ((4, 9, 28, 28), [2, 2], None, None, "bn_relu"),
+    ((2, 7, 40, 40), [2, 2], None, None, "bn_relu"),
+    ((7, 5, 9, 11), [2, 3], [1, 2], [False, True], "bn_relu"),
+    # ... and planes large enough to get a workgroup each although several would fit (weights through the scalar cache)
+    ((3, 5, 51, 51), [3, 3], [2, 2], [True, True], "bn_relu"),
+    ((2, 3, 45, 45), [3, 3], [2, 2], None, "prelu_bn"),
+    ((2, 7, 48, 48), [2, 2], None, None, "bn_prelu_elu_sigmoid"),
+    ((2, 6, 56, 56), [2, 2], None, None, "bn_relu"),
 ]
 
 
