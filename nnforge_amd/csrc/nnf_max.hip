@@ -208,7 +208,8 @@ namespace nnf
 		// puts two lanes on every bank), and the two results leave as one 8-byte store. Each window is still folded
 		// in the reference's order (x fastest, then y).
 		// BN_RELU: the layers are BatchNorm -> ReLU and nothing else (with UNIFORM; apply_known_group)
-		template<int OP, int WIN_W, int WIN_H, bool TRUNC, bool PROLOGUE, bool EXP, bool UNIFORM, bool PAIR = false, bool BN_RELU = false>
+		// CHUNKED (with BN_RELU): the layers go over the staged float4s two at a time and skip those no lane holds
+		template<int OP, int WIN_W, int WIN_H, bool TRUNC, bool PROLOGUE, bool EXP, bool UNIFORM, bool PAIR = false, bool BN_RELU = false, bool CHUNKED = false>
 		__device__ __forceinline__ void window2d_body(const window2d_args& a, const window_prologue& pro)
 		{
 			static_assert(!PAIR || (((WIN_W == 2) || (WIN_W == 3)) && (WIN_H > 0)), "pairs of outputs: windows 2 or 3 wide, height known");
@@ -297,7 +298,51 @@ namespace nnf
 					if (EXP)
 						exp_ctx = exp_context_from_lds(lds_exp);
 				}
-				if (PROLOGUE)
+				static_assert(!BN_RELU || UNIFORM || CHUNKED, "several planes per workgroup: the chunked form knows about float4s between planes");
+				if (PROLOGUE && BN_RELU && CHUNKED)
+				{
+					// Straight code, two float4s at a time, and only those the round holds for some lane (a workgroup
+					// with a plane of 3025 floats has three float4s per lane to stage, not the eight of a round). A
+					// float4 between two planes: every value picks its own plane's coefficients. Not for the bands of
+					// large planes, which fill their rounds: 64 x 64 planes of 112 x 112 42.7 us all eight at once,
+					// 43.5 us two at a time.
+					constexpr int CHUNK = (COUNT >= 2) ? 2 : 1;
+					const bool per_plane = !uniform && (planes_here > 1);
+					#pragma unroll
+					for(int k0 = 0; k0 < COUNT; k0 += CHUNK)
+					{
+						if (base + k0 * max_block_size < limit)
+						{
+							float v[CHUNK][4];
+							uint32_t off[CHUNK];
+							two_plane_offsets<CHUNK> two;
+							#pragma unroll
+							for(int k = 0; k < CHUNK; ++k)
+							{
+								const uint32_t i = base + (k0 + k) * max_block_size + threadIdx.x;
+								const bool valid = i < limit;
+								v[k][0] = t[k0 + k].x; v[k][1] = t[k0 + k].y; v[k][2] = t[k0 + k].z; v[k][3] = t[k0 + k].w;
+								// plane, inside the workgroup's range, of the first float of this float4 (floats in front
+								// of the range count as plane 0: they are staged but not read)
+								const uint32_t first_pos = max(i * 4, shift) - shift;
+								const uint32_t p = (per_plane && valid) ? fast_divide(first_pos, in_plane, pro.in_plane_magic) : 0u;
+								off[k] = p * (2 * pro.weighted_count);
+								two.off2[k] = min(p + 1, planes_here - 1) * (2 * pro.weighted_count); // behind the last plane: values nobody reads
+								two.split[k] = (p + 1) * in_plane + shift - i * 4;                    // >= 4: the whole float4 lies in plane p
+							}
+							if (UNIFORM)
+								apply_known_group<CHUNK, known_group_batch_norm_relu, true>(v, v, off, lds_coef, own_coef, pro, exp_ctx);
+							else
+								apply_known_group<CHUNK, known_group_batch_norm_relu, false, true>(v, v, off, lds_coef, own_coef, pro, exp_ctx, &two);
+							#pragma unroll
+							for(int k = 0; k < CHUNK; ++k)
+							{
+								t[k0 + k].x = v[k][0]; t[k0 + k].y = v[k][1]; t[k0 + k].z = v[k][2]; t[k0 + k].w = v[k][3];
+							}
+						}
+					}
+				}
+				else if (PROLOGUE)
 				{
 					float v[COUNT][4];
 					uint32_t off[COUNT];
@@ -326,7 +371,7 @@ namespace nnf
 							straddling |= 1u << k;
 					}
 					if (BN_RELU)
-						apply_known_group<COUNT, known_group_batch_norm_relu, UNIFORM>(v, v, off, lds_coef, own_coef, pro, exp_ctx);
+						apply_known_group<COUNT, known_group_batch_norm_relu, true>(v, v, off, lds_coef, own_coef, pro, exp_ctx);
 					else if (uniform)
 						apply_prologue<COUNT, EXP, true>(v, off, lds_coef, own_coef, pro, exp_ctx, 0, pro.op_count);
 					else
@@ -349,10 +394,7 @@ namespace nnf
 							w[0][e] = (mine && (e >= split) && (g < a.total_in)) ? a.in[g] : 0.0f;
 						}
 						const uint32_t off_next[1] = { p_next * (2 * pro.weighted_count) };
-						if (BN_RELU)
-							apply_known_group<1, known_group_batch_norm_relu, false>(w, w, off_next, lds_coef, own_coef, pro, exp_ctx);
-						else
-							apply_prologue<1, EXP, false>(w, off_next, lds_coef, own_coef, pro, exp_ctx, 0, pro.op_count);
+						apply_prologue<1, EXP, false>(w, off_next, lds_coef, own_coef, pro, exp_ctx, 0, pro.op_count);
 						#pragma unroll
 						for(int k = 0; k < COUNT; ++k)
 						{
@@ -576,12 +618,14 @@ namespace nnf
 			window2d_body<OP, WIN_W, WIN_H, TRUNC, true, false, UNIFORM, PAIR>(a, pro);
 		}
 
-		// BatchNorm -> ReLU in front of the windows: the layers as straight code (several planes per workgroup: 96 registers
-		// either way; 64 x 256 planes of 27 x 27 20.9 -> 19.3 us, 64 x 128 of 28 x 28 10.2 -> 9.5 us)
-		template<int OP, int WIN_W, int WIN_H, bool TRUNC, bool PAIR = false, bool UNIFORM = true>
+		// BatchNorm -> ReLU in front of the windows: the layers as straight code (several planes per workgroup: 77 to 80
+		// registers instead of 96; 64 x 256 planes of 27 x 27 20.9 -> 16.6 us, 64 x 128 of 28 x 28 10.2 -> 9.4 us)
+		// FILLED: one plane (or band) per workgroup that holds more than four float4s per lane
+		template<int OP, int WIN_W, int WIN_H, bool TRUNC, bool PAIR = false, bool UNIFORM = true, bool FILLED = true>
 		__global__ void __launch_bounds__(max_block_size) __attribute__((amdgpu_waves_per_eu(UNIFORM ? 6 : 4))) max_window2d_bn_relu_kernel(const window2d_args a, const window_prologue pro)
 		{
-			window2d_body<OP, WIN_W, WIN_H, TRUNC, true, false, UNIFORM, PAIR, true>(a, pro);
+			static_assert(UNIFORM || !FILLED, "several planes per workgroup go two float4s at a time");
+			window2d_body<OP, WIN_W, WIN_H, TRUNC, true, false, UNIFORM, PAIR, true, !FILLED>(a, pro);
 		}
 
 		template<int OP, int WIN_W, int WIN_H, bool TRUNC, bool UNIFORM>
@@ -1373,11 +1417,21 @@ namespace nnf
 			else if (known_group_of(pro) == known_group_batch_norm_relu)
 			{
 				const bool pair = pairs_of_outputs(a);
-				if (w3 && pair) NNF_LAUNCH((max_window2d_bn_relu_kernel<OP, 3, 3, TRUNC, true, UNIFORM>), g, b, lds_bytes, stream, a, pro);
-				else if (w2 && pair) NNF_LAUNCH((max_window2d_bn_relu_kernel<OP, 2, 2, TRUNC, true, UNIFORM>), g, b, lds_bytes, stream, a, pro);
-				else if (w3) NNF_LAUNCH((max_window2d_bn_relu_kernel<OP, 3, 3, TRUNC, false, UNIFORM>), g, b, lds_bytes, stream, a, pro);
-				else if (w2) NNF_LAUNCH((max_window2d_bn_relu_kernel<OP, 2, 2, TRUNC, false, UNIFORM>), g, b, lds_bytes, stream, a, pro);
-				else NNF_LAUNCH((max_window2d_bn_relu_kernel<OP, 0, 0, TRUNC, false, UNIFORM>), g, b, lds_bytes, stream, a, pro);
+				// the floats a workgroup stages, as lds_bytes counts them
+				const bool filled = UNIFORM && (lds_bytes / sizeof(float) > 4u * 4u * max_block_size);
+				if (filled)
+				{
+					if (w3 && pair) NNF_LAUNCH((max_window2d_bn_relu_kernel<OP, 3, 3, TRUNC, true>), g, b, lds_bytes, stream, a, pro);
+					else if (w2 && pair) NNF_LAUNCH((max_window2d_bn_relu_kernel<OP, 2, 2, TRUNC, true>), g, b, lds_bytes, stream, a, pro);
+					else if (w3) NNF_LAUNCH((max_window2d_bn_relu_kernel<OP, 3, 3, TRUNC>), g, b, lds_bytes, stream, a, pro);
+					else if (w2) NNF_LAUNCH((max_window2d_bn_relu_kernel<OP, 2, 2, TRUNC>), g, b, lds_bytes, stream, a, pro);
+					else NNF_LAUNCH((max_window2d_bn_relu_kernel<OP, 0, 0, TRUNC>), g, b, lds_bytes, stream, a, pro);
+				}
+				else if (w3 && pair) NNF_LAUNCH((max_window2d_bn_relu_kernel<OP, 3, 3, TRUNC, true, UNIFORM, false>), g, b, lds_bytes, stream, a, pro);
+				else if (w2 && pair) NNF_LAUNCH((max_window2d_bn_relu_kernel<OP, 2, 2, TRUNC, true, UNIFORM, false>), g, b, lds_bytes, stream, a, pro);
+				else if (w3) NNF_LAUNCH((max_window2d_bn_relu_kernel<OP, 3, 3, TRUNC, false, UNIFORM, false>), g, b, lds_bytes, stream, a, pro);
+				else if (w2) NNF_LAUNCH((max_window2d_bn_relu_kernel<OP, 2, 2, TRUNC, false, UNIFORM, false>), g, b, lds_bytes, stream, a, pro);
+				else NNF_LAUNCH((max_window2d_bn_relu_kernel<OP, 0, 0, TRUNC, false, UNIFORM, false>), g, b, lds_bytes, stream, a, pro);
 			}
 			else
 			{
@@ -1499,9 +1553,10 @@ namespace nnf
 			a.planes = std::min(a.planes, std::min(prologue_planes_max, prologue_coef_floats / (2 * prologue_weighted_max)));
 			// Layers with weights over planes this large: one plane per workgroup, whose coefficients come through the scalar
 			// cache into registers - no table in LDS, no barrier in front of the layers, no float4 between two planes
-			// (BatchNorm -> ReLU -> 3 x 3 every 2 on 64 x 96 planes of 55 x 55: 24.7 -> 20.5 us, of 51 x 51 22.0 -> 17.8 us,
-			// 2 x 2 on 56 x 56 14.0 -> 13.2 us; 64 x 128 planes of 40 x 40 the other way, 15.3 -> 17.8 us, 35 x 35 22.0 -> 23.9 us).
-			if ((a.planes > 1) && (pro.weighted_count != 0) && (plane >= (((plane & 3u) != 0) ? 2000u : 2304u)))
+			// (BatchNorm -> ReLU -> 3 x 3 every 2 on 64 x 96 planes of 55 x 55: 21.6 -> 19.8 us, of 51 x 51 19.5 -> 18.6 us,
+			// 2 x 2 on 56 x 56 14.9 -> 13.4 us; equal on 45 x 45 and 48 x 48; 64 x 128 planes of 40 x 40 the other way,
+			// 15.4 -> 18.2 us, 35 x 35 18.9 -> 24.1 us).
+			if ((a.planes > 1) && (pro.weighted_count != 0) && (plane >= 2500u))
 				a.planes = 1;
 		}
 		if (plan_only)
