@@ -1558,6 +1558,12 @@ namespace nnf
 			// 15.4 -> 18.2 us, 35 x 35 18.9 -> 24.1 us).
 			if ((a.planes > 1) && (pro.weighted_count != 0) && (plane >= 2500u))
 				a.planes = 1;
+			// Layers that call expf are what such a launch waits for, and a workgroup takes every round of eight float4s per
+			// lane through them whole: as many small planes as fill the rounds, not as few as give every lane four outputs
+			// (TanH -> Absolute -> average over 2 x 2 on 1024 x 38 planes of 28 x 28: six planes, 4.6 float4s per lane,
+			// 63.2 us; ten planes, 7.7 per lane, 46.6 us; 1024 x 96 planes of 10 x 10 26.9 -> 19.2 us).
+			if (pro.need_exp && (plane <= lds_floats_wanted))
+				a.planes = std::max(1u, std::min(lds_floats_wanted / plane, std::min(prologue_planes_max, prologue_coef_floats / (2 * prologue_weighted_max))));
 		}
 		if (plan_only)
 			return true;
