@@ -410,7 +410,8 @@ namespace nnf
 				// Two sets of registers take turns: the next round is on its way while the layers are applied to this one
 				// (every request unconditional and clamped: no join of two paths between a request and the wait for an
 				// earlier one, where the compiler would wait for everything outstanding). The request behind the last
-				// round asks for the wavefront's last float4 in every lane and is looked at by nobody.
+				// round asks for the wavefront's last float4 in every lane and is looked at by nobody. (vectors >= 1: the
+				// host folds a group in over planes of four floats or more only.)
 				floatx4 a[stage], a2[stage], b[stage], b2[stage];
 				request(a, a2, 0);
 				for(uint32_t base = 0; ; )
