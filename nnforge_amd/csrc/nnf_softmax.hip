@@ -630,8 +630,19 @@ namespace nnf
 				// a whole wavefront along the positions (256-byte accesses) once that still gives every
 				// compute unit a few workgroups; fewer positions when that is what lets the values fit LDS
 				uint32_t positions = (columns >= 64u * 512u) ? 64u : 16u;
+				// half a wavefront along the positions when that lets a compute unit hold twice the workgroups
+				// (256 x 128 feature maps of 28 x 28: 52.7 us with 64 positions and 32 KB, 46.3 us with 32)
+				if ((positions == 64u) && (static_cast<size_t>(feature_map_count) * positions * sizeof(float) > 24u * 1024u))
+					positions = 32u;
 				while ((positions > 16u) && (static_cast<size_t>(feature_map_count) * positions * sizeof(float) > staged_bytes_limit))
 					positions /= 2;
+				// eight positions for small tensors whose values then fit: 1000 feature maps of 7 x 7 in one read and one
+				// write, 22 us for 64 entries against 36 us in three passes with sixteen (large tensors: 32-byte accesses
+				// cost more than the passes, 315 against 137 us on 32 x 150 feature maps of 128 x 128)
+				if ((positions == 16u) && (columns <= sliced_columns_limit)
+					&& (static_cast<size_t>(feature_map_count) * 16u * sizeof(float) > staged_bytes_limit)
+					&& (static_cast<size_t>(feature_map_count) * 8u * sizeof(float) <= staged_bytes_limit))
+					positions = 8u;
 				const size_t staged_bytes = static_cast<size_t>(feature_map_count) * positions * sizeof(float);
 				const dim3 sliced_grid((columns + positions - 1) / positions);
 				if (staged_bytes <= staged_bytes_limit)
@@ -642,8 +653,11 @@ namespace nnf
 					else if (positions == 32)
 						NNF_LAUNCH((softmax_columns_sliced_kernel<32, true>), sliced_grid, dim3(256), staged_bytes, stream,
 							output, input, columns, feature_map_count, neuron_count_per_feature_map);
-					else
+					else if (positions == 16)
 						NNF_LAUNCH((softmax_columns_sliced_kernel<16, true>), sliced_grid, dim3(256), staged_bytes, stream,
+							output, input, columns, feature_map_count, neuron_count_per_feature_map);
+					else
+						NNF_LAUNCH((softmax_columns_sliced_kernel<8, true>), sliced_grid, dim3(256), staged_bytes, stream,
 							output, input, columns, feature_map_count, neuron_count_per_feature_map);
 					return launch_status();
 				}

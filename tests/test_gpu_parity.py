@@ -760,9 +760,12 @@ def test_softmax_columns_bit_exact(gpu, n, c, plane):
 @pytest.mark.parametrize("n,c,plane", [(1, 150, 333), (4, 1000, 49), (2, 65, 7), (3, 257, 100), (1, 4100, 3), (1, 66, 65536),
                                        # values staged in LDS: 64 positions x up to 240 feature maps, 32 x up to 480, 16 x up to 960
                                        (1, 70, 70001), (2, 150, 40000), (1, 240, 33000), (1, 241, 33000), (3, 960, 50), (3, 961, 50),
-                                       (1, 300, 65536), (1, 300, 65537), (1, 480, 33000), (1, 481, 33000)])
+                                       (1, 300, 65536), (1, 300, 65537), (1, 480, 33000), (1, 481, 33000),
+                                       # up to 65536 columns: 8 positions x up to 1920 feature maps staged; 32 positions from 97 feature maps on in large tensors
+                                       (64, 1000, 49), (2, 1920, 70), (2, 1921, 70), (3, 1500, 9), (1, 1100, 65536),
+                                       (1, 96, 33000), (1, 97, 33000), (2, 128, 20000)])
 def test_softmax_columns_sliced(gpu, n, c, plane):
-    """More than 64 feature maps: a column is shared out over 4 or 16 lanes whose partial sums are
+    """More than 64 feature maps: a column is shared out over 4 to 32 lanes whose partial sums are
     added in slice order, so the bar is the one stated for softmax, 1e-5 relative."""
     gen = T.rng(15, n * 100000 + c * 100 + plane)
     x = T.normal(gen, (n, c, plane), 4.0)
