@@ -539,8 +539,10 @@ namespace nnf
 				NNF_LAUNCH((softmax_rows_kernel<THREADS, 2, W>), grid, dim3(block), 0, stream, out, in, rows, fm_count);
 			else if (vectors_per_lane <= 4)
 				NNF_LAUNCH((softmax_rows_kernel<THREADS, 4, W>), grid, dim3(block), 0, stream, out, in, rows, fm_count);
-			else
+			else if (vectors_per_lane <= 8)
 				NNF_LAUNCH((softmax_rows_kernel<THREADS, 8, W>), grid, dim3(block), 0, stream, out, in, rows, fm_count);
+			else
+				NNF_LAUNCH((softmax_rows_kernel<THREADS, (W == 1) ? 16 : 8, W>), grid, dim3(block), 0, stream, out, in, rows, fm_count);
 		}
 
 		template<int THREADS, int W>
@@ -578,7 +580,9 @@ namespace nnf
 					launch_one_vector_per_lane<1024, W>(stream, out, in, rows, fm_count);
 				return true;
 			}
-			if (vectors <= wave_size * 8)
+			// (single floats - rows that are no multiple of four floats long, 1001 classes - up to sixteen per lane: a
+			// wavefront per row and no barrier, 8192 rows of 1001 37.5 us as one workgroup of 1024 lanes per row)
+			if (vectors <= wave_size * ((W == 1) ? 16 : 8))
 			{
 				launch_rows<wave_size, W>(stream, out, in, rows, fm_count, (vectors + wave_size - 1) / wave_size);
 				return true;
