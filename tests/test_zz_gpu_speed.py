@@ -147,6 +147,12 @@ def test_softmax_and_global_average_stay_fast(gpu):
     us = time_launches(gpu, lambda i: gpu.lib.nnf_hip_softmax_forward(gpu.stream, rows_out.data_ptr(), rows[i % 32].data_ptr(), 256, 1000, 1), reps=200, warmup=20)
     # 2 MB: both the softmax and the copy are bound by what a launch costs, about 2.7 against 2.2 us
     assert_ratio(gpu, "softmax 256 x 1000", us, 2 * 4 * 256 * 1000, 1.5, reps=200)
+    # many rows: bound by memory, 1.02 times the copy with non-temporal accesses (1.2 with ordinary ones)
+    many = [gpu.torch.randn(8192 * 1000, dtype=gpu.torch.float32, device=gpu.device) for _ in range(12)]
+    many_out = [gpu.torch.empty_like(many[0]) for _ in range(12)]
+    us = time_launches(gpu, lambda i: gpu.lib.nnf_hip_softmax_forward(gpu.stream, many_out[i % 12].data_ptr(), many[i % 12].data_ptr(), 8192, 1000, 1), reps=100, warmup=10)
+    assert_ratio(gpu, "softmax 8192 x 1000", us, 2 * 4 * 8192 * 1000, 1.25, reps=100)
+    del many, many_out
     planes = [gpu.torch.randn(64 * 2048 * 49, dtype=gpu.torch.float32, device=gpu.device) for _ in range(8)]
     sums = gpu.torch.empty(64 * 2048, dtype=gpu.torch.float32, device=gpu.device)
     us = time_launches(gpu, lambda i: gpu.lib.nnf_hip_average_subsampling_forward(gpu.stream, sums.data_ptr(), planes[i % 8].data_ptr(), 64, 2048, 7, 7, 7, 7, 1.0 / 49.0),
