@@ -41,13 +41,17 @@ namespace nnf
 		struct max_op { __device__ __forceinline__ float operator()(float a, float b) const { return ref_max(a, b); } };
 		struct sum_op { __device__ __forceinline__ float operator()(float a, float b) const { return a + b; } };
 
-		template<class OP>
+		// GROUP 16: every row of 16 lanes keeps its own result (four rows of a tensor to a wavefront).
+		template<int GROUP = 64, class OP>
 		__device__ __forceinline__ float wave_all_reduce(float v, OP op)
 		{
+			static_assert((GROUP == 64) || (GROUP == 16), "a wavefront, or one of its rows of 16 lanes");
 			v = op(v, dpp_move<0xB1>(v));
 			v = op(v, dpp_move<0x4E>(v));
 			v = op(v, dpp_move<0x141>(v));
 			v = op(v, dpp_move<0x140>(v));
+			if (GROUP == 16)
+				return v;
 			const float r0 = read_lane(v, 0);
 			const float r1 = read_lane(v, 16);
 			const float r2 = read_lane(v, 32);
@@ -93,7 +97,8 @@ namespace nnf
 			}
 		};
 
-		// One row per group of THREADS lanes (THREADS = 64: a wavefront; larger: a whole workgroup).
+		// One row per group of THREADS lanes (THREADS = 64: a wavefront; larger: a whole workgroup; 16: a quarter of a
+		// wavefront, for many short rows - 65536 rows of 100 floats keep 25 of a wavefront's 64 lanes busy, of 32 lanes 25).
 		// Lane t holds vectors t, t + THREADS, ... of its row: VPT vectors of W floats.
 		// Rows per workgroup = blockDim.x / THREADS. Requires fm_count <= THREADS * VPT * W and,
 		// for W == 4, fm_count % 4 == 0 (then every row start is 16-byte aligned).
@@ -136,7 +141,7 @@ namespace nnf
 						m = ref_max(m, v[k][e]);
 				}
 			}
-			m = wave_all_reduce(m, max_op());
+			m = wave_all_reduce<(THREADS == 16) ? 16 : 64>(m, max_op());
 			if (THREADS > wave_size)
 			{
 				const uint32_t wave = threadIdx.x / wave_size;
@@ -165,7 +170,7 @@ namespace nnf
 						sum += v[k][e];
 				}
 			}
-			sum = wave_all_reduce(sum, sum_op());
+			sum = wave_all_reduce<(THREADS == 16) ? 16 : 64>(sum, sum_op());
 			if (THREADS > wave_size)
 			{
 				const uint32_t wave = threadIdx.x / wave_size;
@@ -622,6 +627,11 @@ namespace nnf
 					launch_one_vector_per_lane<512, W>(stream, out, in, rows, fm_count);
 				else
 					launch_one_vector_per_lane<1024, W>(stream, out, in, rows, fm_count);
+				return true;
+			}
+			if ((rows >= 4096) && (vectors <= 32))
+			{
+				launch_rows<16, W>(stream, out, in, rows, fm_count, (vectors + 15) / 16);
 				return true;
 			}
 			// (single floats - rows that are no multiple of four floats long, 1001 classes - up to sixteen per lane: a

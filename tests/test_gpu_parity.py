@@ -730,7 +730,9 @@ def test_argument_errors(gpu):
 @pytest.mark.parametrize("n,c", [(1, 1), (3, 2), (5, 3), (2, 4), (7, 10), (4, 64), (9, 255), (3, 256), (2, 257), (5, 1000), (64, 1000),
                                  (3, 1001), (2, 2048), (2, 2049), (3, 4096), (2, 8200), (2, 32768), (1, 40000), (2, 33001), (5000, 12),
                                  # many rows that are no multiple of four floats long: a wavefront per row, up to sixteen floats per lane
-                                 (2048, 1001), (2100, 1023), (2049, 513), (2500, 999), (4099, 1021), (2048, 1025), (3000, 130)])
+                                 (2048, 1001), (2100, 1023), (2049, 513), (2500, 999), (4099, 1021), (2048, 1025), (3000, 130),
+                                 # 4096 rows or more of up to 32 vectors: four rows to a wavefront
+                                 (4096, 100), (4097, 128), (5000, 10), (4500, 31), (4100, 33), (4099, 1), (4111, 5), (70000, 100), (4096, 124)])
 def test_softmax_rows(gpu, n, c):
     gen = T.rng(13, n * 100000 + c)
     x = T.normal(gen, (n, c, 1), 4.0)
