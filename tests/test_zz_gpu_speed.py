@@ -147,19 +147,19 @@ def test_softmax_and_global_average_stay_fast(gpu):
     us = time_launches(gpu, lambda i: gpu.lib.nnf_hip_softmax_forward(gpu.stream, rows_out.data_ptr(), rows[i % 32].data_ptr(), 256, 1000, 1), reps=200, warmup=20)
     # 2 MB: both the softmax and the copy are bound by what a launch costs, about 2.7 against 2.2 us
     assert_ratio(gpu, "softmax 256 x 1000", us, 2 * 4 * 256 * 1000, 1.5, reps=200)
-    # many rows: bound by memory, 1.02 times the copy with non-temporal accesses (1.2 with ordinary ones)
+    # many rows: bound by memory, 1.02 to 1.2 times the copy depending on where the process's allocations lie
     many = [gpu.torch.randn(8192 * 1000, dtype=gpu.torch.float32, device=gpu.device) for _ in range(12)]
     many_out = [gpu.torch.empty_like(many[0]) for _ in range(12)]
     us = time_launches(gpu, lambda i: gpu.lib.nnf_hip_softmax_forward(gpu.stream, many_out[i % 12].data_ptr(), many[i % 12].data_ptr(), 8192, 1000, 1), reps=100, warmup=10)
-    assert_ratio(gpu, "softmax 8192 x 1000", us, 2 * 4 * 8192 * 1000, 1.25, reps=100)
+    assert_ratio(gpu, "softmax 8192 x 1000", us, 2 * 4 * 8192 * 1000, 1.5, reps=100)
     del many, many_out
     planes = [gpu.torch.randn(64 * 2048 * 49, dtype=gpu.torch.float32, device=gpu.device) for _ in range(8)]
     sums = gpu.torch.empty(64 * 2048, dtype=gpu.torch.float32, device=gpu.device)
     us = time_launches(gpu, lambda i: gpu.lib.nnf_hip_average_subsampling_forward(gpu.stream, sums.data_ptr(), planes[i % 8].data_ptr(), 64, 2048, 7, 7, 7, 7, 1.0 / 49.0),
                        reps=100, warmup=10)
     assert_ratio(gpu, "the 7x7 global average", us, 4 * (64 * 2048 * 49 + 64 * 2048), 1.5, reps=100)
-    # the last block of a residual network folded into it: 1.1 times the copy as straight code with the next round of loads
-    # in flight, 1.3 times through the kernel's loop over the layer list (either order of the Add's inputs must take the former)
+    # the last block of a residual network folded into it: 1.07 to 1.15 times the copy as straight code with the next round of
+    # loads in flight, 1.4 times through the kernel's loop over the layer list (either order of the Add's inputs must take the former)
     shortcuts = [gpu.torch.randn(64 * 2048 * 49, dtype=gpu.torch.float32, device=gpu.device) for _ in range(8)]
     chunks = [gpu.torch.rand(2048, dtype=gpu.torch.float32, device=gpu.device) + 0.5 for _ in range(4)]
     chk = capi.pointer_array([t.data_ptr() for t in chunks])
@@ -172,7 +172,7 @@ def test_softmax_and_global_average_stay_fast(gpu):
             assert rc == 0, capi.error_string(rc)
 
         assert_ratio(gpu, "the residual block and the 7x7 global average in one launch", time_launches(gpu, joined, reps=100, warmup=10),
-                     4 * (2 * 64 * 2048 * 49 + 64 * 2048), 1.25, reps=100)
+                     4 * (2 * 64 * 2048 * 49 + 64 * 2048), 1.35, reps=100)
 
 
 def test_tiling_and_entry_windows_stay_on_their_own_kernels(gpu):
