@@ -323,6 +323,36 @@ def bench_softmax(runner, steps, warmup):
                                  "queued behind a spin kernel"})
 
 
+SOFTMAX_SHAPES = {
+    # name -> (entries, feature maps, neurons per feature map)
+    "softmax_many_rows": (8192, 1000, 1),          # a large packet of classifier outputs: a wavefront per row
+    "softmax_rows_1001": (8192, 1001, 1),          # rows that are no multiple of four floats long
+    "softmax_short_rows": (65536, 100, 1),         # four rows to a wavefront
+    "softmax_columns": (64, 21, 64 * 64),          # per-position classes of a segmentation map: one lane per position
+    "softmax_wide_columns": (64, 1000, 7 * 7),     # more than 64 feature maps: a column shared out over lanes
+}
+
+
+def bench_softmax_shape(runner, steps, warmup, name):
+    """nnf_hip_softmax_forward at shapes other than configuration 1's, N(0, 2) inputs, buffers rotating through HBM."""
+    n, c, plane = SOFTMAX_SHAPES[name]
+    total = n * c * plane
+    sets = rotation_sets(8 * total)
+    ins = [runner.randn(total, 2.0) for _ in range(sets)]
+    outs = [runner.empty(total) for _ in range(sets)]
+    fn, stream = runner.lib.nnf_hip_softmax_forward, runner.stream
+
+    def launch(i):
+        rc = fn(stream, outs[i % sets].data_ptr(), ins[i % sets].data_ptr(), n, c, plane)
+        if rc != 0:
+            raise RuntimeError(runner.capi.error_string(rc))
+
+    wall, ev = runner.time_steps(launch, steps, warmup)
+    queued = time_steps_queued(runner, launch, min(steps, 400))
+    return result_entry("softmax over %d feature maps, N=%d, %d neurons per feature map" % (c, n, plane), 8 * total, total, wall, ev, 1,
+                        {"buffer_sets": sets, "queued_event_ms_per_step": queued * 1e3, "queued_event_gbps": 8 * total / queued / 1e9})
+
+
 def resnet50_network(n, gen):
     """Config 4 as a network for the hip backend: schema text, weights, data layer shapes, output names."""
     from nnforge_amd import schemas
@@ -981,7 +1011,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--workload", default="config0", choices=["config0", "config1", "config2", "config3", "config4", "copy", "max_subsampling", "bn_relu_max_subsampling", "max_subsampling_tiling",
                              "entry_window", "concat", "maxout", "feature_map_stat", "config4_direct", "yardsticks", "walking_grid",
-                             "global_average", "joined_global_average", "inception_block", "inception_block_copies"],
+                             "global_average", "joined_global_average", "inception_block", "inception_block_copies"] + sorted(SOFTMAX_SHAPES),
                     help="'copy' times the plain copy kernel (profiler-counter calibration and bandwidth yardstick); 'yardsticks' the runtime's and "
                          "torch's copy routines beside the library's kernels; 'config4_direct' the launches of config4 issued at the C ABI from this script")
     ap.add_argument("--entries", type=int, default=64, help="config4: entries per packet (the benchmark's configuration has 64)")
@@ -1007,6 +1037,8 @@ def main():
             return bench_group(runner, "config0: batch_norm -> rectified_linear N=32 C=64 56x56", w.config0(), steps, warmup, overlapped_steps=not args.only)
         if name == "config1":
             return bench_softmax(runner, steps, warmup)
+        if name in SOFTMAX_SHAPES:
+            return bench_softmax_shape(runner, steps, warmup, name)
         if name == "config2":
             return bench_group(runner, "config2: batch_norm -> add(residual) -> parametric_rectified_linear N=128 C=256 56x56", w.config2(), steps, warmup)
         if name == "config3":
@@ -1121,6 +1153,8 @@ def main():
                        "concat": "nnf::concat_kernel", "maxout": "nnf::maxout_pairs_kernel",
                        "feature_map_stat": "nnf::stat_runs_kernel", "walking_grid": "nnf::chain_kernel_persistent",
                        "global_average": "nnf::global_pool_linear_kernel", "joined_global_average": "nnf::global_pool_linear_kernel",
+                       "softmax_many_rows": "nnf::softmax_rows_kernel", "softmax_rows_1001": "nnf::softmax_rows_kernel", "softmax_short_rows": "nnf::softmax_rows_kernel",
+                       "softmax_columns": "nnf::softmax_columns_kernel", "softmax_wide_columns": "nnf::softmax_columns_sliced_kernel",
                        "inception_block": "nnf::chain_entries_batch_kernel", "inception_block_copies": "nnf::chain_batch_kernel + nnf::concat_kernel",
                        "config4": "all kernels of one pass of the launch plan (nnf::chain_batch_mixed_kernel, nnf::chain_batch_kernel, nnf::chain_kernel, nnf::global_pool_linear_kernel, nnf::softmax_rows_kernel)",
                        "config4_direct": "all kernels of one pass (nnf::chain_kernel x 49, nnf::global_pool_kernel, nnf::softmax_rows_kernel)"}.get(args.workload, "nnf::chain_kernel"),
