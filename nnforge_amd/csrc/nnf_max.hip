@@ -22,22 +22,6 @@ namespace nnf
 		constexpr int max_block_size = 256;
 		constexpr uint32_t max_dims = NNF_HIP_MAX_SUBSAMPLING_DIMENSIONS;
 
-		// Consecutive workgroups are handed to consecutive XCDs (eight dies, an L2 each). Work items that touch common memory -
-		// the bands of a plane: the input rows two of them stage, the output cache line two of them write - are `together`
-		// consecutive work items; of every 8 * together workgroups the ones with the same index modulo 8 take them, so that
-		// they meet in one die's L2 (what is left over at the end of the grid keeps its order). Measured on the tiling
-		// kernel, 64 x 64 planes of 112 x 112 in five bands each: 72.7 -> 67.7 us. The pooling kernels, whose bands share
-		// an input row but no output cache line, gain nothing from it (3 x 3 every 2 on the same planes, two bands each:
-		// 40.9 -> 40.7 us, with BatchNorm and ReLU folded in 44.1 -> 45.3 us) and keep the plain order.
-		__device__ __forceinline__ uint32_t xcd_grouped(uint32_t block, uint32_t together, uint32_t blocks)
-		{
-			const uint32_t chunk = 8 * together;
-			const uint32_t in_chunk = block % chunk;
-			if ((together < 2) || (block - in_chunk + chunk > blocks))
-				return block;
-			return block - in_chunk + (in_chunk % 8) * together + in_chunk / 8;
-		}
-
 		// std::max<float>(current, new_val) / std::min<float>(current, new_val)
 		template<bool IS_MIN>
 		__device__ __forceinline__ float fold(float current, float new_val)

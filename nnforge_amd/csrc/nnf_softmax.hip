@@ -469,7 +469,10 @@ namespace nnf
 
 			const uint32_t p = threadIdx.x % P;
 			const uint32_t slice = threadIdx.x / P;
-			const uint32_t column = blockIdx.x * P + p;
+			// Neighbouring blocks of positions lie in the same cache lines (P positions are P * 4 bytes of every feature
+			// map's row): sixteen of them (four of the wide ones) go to workgroups of one XCD, where the lines meet in one
+			// L2 (64 x 1000 feature maps of 7 x 7: 22.0 -> 17.2 us; 256 x 128 of 28 x 28: 45.8 -> 43.8 us).
+			const uint32_t column = xcd_grouped(blockIdx.x, (P < 32) ? 16u : 4u, gridDim.x) * P + p;
 			const bool valid = column < columns;
 			const uint32_t col = valid ? column : columns - 1; // lanes past the end shadow the last column and store nothing
 			const uint32_t entry = col / plane;
