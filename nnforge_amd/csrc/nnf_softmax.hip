@@ -258,7 +258,10 @@ namespace nnf
 		__global__ void __launch_bounds__(256) softmax_columns_kernel(float* out, const float* in, uint32_t columns, uint32_t fm_count, uint32_t plane)
 		{
 			__shared__ uint64_t lds_exp[exp_lds_entries];
-			const uint32_t column = blockIdx.x * blockDim.x + threadIdx.x;
+			// a feature map's row of a workgroup's columns starts anywhere in a cache line when the plane is no multiple of
+			// 32 floats: eight neighbouring workgroups to one XCD, whose L2 then holds the lines they share (256 x 64 feature
+			// maps of 28 x 28: 24.5 -> 21.3 us; planes that are multiples of 32 floats unchanged)
+			const uint32_t column = xcd_grouped(blockIdx.x, 8u, gridDim.x) * blockDim.x + threadIdx.x;
 			const bool valid = column < columns;
 			const uint32_t col = valid ? column : columns - 1; // lanes past the end shadow the last column and store nothing
 			const uint32_t entry = col / plane;
